@@ -1,0 +1,176 @@
+/*
+ * mcn_hip.h -- C ABI of the MI355X (gfx950) back-end for MatConvNet's convolution, batch-normalisation
+ * and pooling operators.
+ *
+ * This is the layer the reference's device structs call into: where MatConvNet's
+ * `ConvolutionBackward<VLDT_GPU,T>`, `BatchNormBackward<VLDT_GPU,T>` and `PoolingBackward<VLDT_GPU,T>`
+ * launch CUDA kernels / cuBLAS / cuDNN, the replacement `VLDT_GPU` branch calls the functions below.
+ *
+ * Conventions
+ *   - every tensor is fp32, MATLAB column-major H x W x C x N: element (h,w,c,n) at
+ *     h + H*(w + W*(c + C*n)); filters FH x FW x FC x K likewise (bits/nnpooling.cu:131, nnconv.cu:132);
+ *   - all pointers are DEVICE pointers on the current HIP device; `stream` is a hipStream_t passed as
+ *     void* (NULL = the default stream); calls only enqueue work, they never synchronise;
+ *   - scratch memory is supplied by the caller (the role of vl::Context::getWorkspace,
+ *     bits/data.cu:395-404): ask mcn_*_workspace_bytes, pass a buffer of at least that many bytes,
+ *     256-byte aligned; contents need not be preserved between calls;
+ *   - return value: 0 on success, otherwise a code numerically equal to the matching vl::ErrorCode
+ *     (bits/data.hpp:38-52); mcn_last_error_message() gives the text for the calling thread;
+ *   - shapes are validated on the host before any launch; nothing is launched on error.
+ */
+#ifndef MCN_HIP_H
+#define MCN_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define MCN_API __attribute__((visibility("default")))
+#else
+#define MCN_API
+#endif
+
+typedef void* mcn_stream_t;
+
+/* numerically equal to vl::ErrorCode (bits/data.hpp:38-52) */
+enum {
+  MCN_SUCCESS = 0,
+  MCN_UNSUPPORTED = 1,
+  MCN_DEVICE_ERROR = 2, /* VLE_Cuda: a HIP runtime call or launch failed */
+  MCN_OUT_OF_MEMORY = 5,
+  MCN_OUT_OF_GPU_MEMORY = 6,
+  MCN_ILLEGAL_ARGUMENT = 7,
+  MCN_UNKNOWN = 8
+};
+
+/* vl::nn::Convolution's public members (bits/nnconv.hpp:43-51) plus the tensor extents the MEX driver
+   checks (vl_nnconv.cu:269-342).  groups = C / FC; K must be a multiple of groups. */
+typedef struct mcn_conv_geom {
+  int H, W, C, N;    /* input x */
+  int FH, FW, FC, K; /* filters */
+  int strideY, strideX;
+  int padTop, padBottom, padLeft, padRight;
+  int dilateY, dilateX;
+} mcn_conv_geom;
+
+/* vl::nn::Pooling's public members (bits/nnpooling.hpp:39-48) plus the input extents. */
+typedef struct mcn_pool_geom {
+  int H, W, C, N;
+  int poolH, poolW;
+  int strideY, strideX;
+  int padTop, padBottom, padLeft, padRight;
+  int method; /* 0 = vl::nn::Pooling::Max, 1 = Average */
+} mcn_pool_geom;
+
+enum { MCN_POOL_MAX = 0, MCN_POOL_AVERAGE = 1 };
+
+/* which convolution product a workspace query is for */
+enum { MCN_CONV_FORWARD = 0, MCN_CONV_BACKWARD_DATA = 1, MCN_CONV_BACKWARD_FILTER = 2, MCN_CONV_BACKWARD_BIAS = 3 };
+
+/* ------------------------------------------------------------------------------------------------
+ * library
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Text of the last error raised on the calling thread (never NULL).  Replaces the message path of
+   vl::Context::setError / getLastErrorMessage (bits/data.cu:332-377) below the operator layer. */
+MCN_API const char* mcn_last_error_message(void);
+
+/* Generic name of an error code; same strings as vl::getErrorMessage (bits/data.cu:83-96). */
+MCN_API const char* mcn_error_name(int code);
+
+/* Compute units of the current device (for sizing grids / reporting); <0 on error. */
+MCN_API int mcn_device_compute_units(void);
+
+/* Name/value knobs for experiments (tile budgets, split factors).  Unknown names are rejected.
+   Not part of the reference interface. */
+MCN_API int mcn_set_tunable(const char* name, int value);
+MCN_API int mcn_get_tunable(const char* name, int* value);
+
+/* ------------------------------------------------------------------------------------------------
+ * convolution -- replaces ConvolutionForward/Backward<VLDT_GPU,T> (bits/nnconv.cu:71-157,163-317),
+ * i.e. im2row_gpu + cublasSgemm per image, and the cuDNN variant (bits/nnconv_cudnn.cu:40-540).
+ * ---------------------------------------------------------------------------------------------- */
+
+MCN_API int mcn_conv_output_size(const mcn_conv_geom* g, int* outH, int* outW);
+
+/* scratch bytes needed by one of the four products below (may be 0) */
+MCN_API size_t mcn_conv_workspace_bytes(const mcn_conv_geom* g, int product);
+
+/* y = outMult*y + inMult*conv(x,f) + b   (bits/nnconv.cu:71-157).  bias may be NULL.  When outMult is
+   0 the previous contents of y are ignored (BLAS beta = 0 rule). */
+MCN_API int mcn_conv_forward(mcn_stream_t stream, const mcn_conv_geom* g, float* y, float outMult,
+                             const float* x, float inMult, const float* filters, const float* bias,
+                             void* workspace, size_t workspaceBytes);
+
+/* dzdx: H x W x C x N, fully overwritten  (bits/nnconv.cu:247-277: gemm 'n','t' + im2row::backward) */
+MCN_API int mcn_conv_backward_data(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput,
+                                   const float* filters, const float* derOutput, void* workspace,
+                                   size_t workspaceBytes);
+
+/* dzdf: FH x FW x FC x K, fully overwritten  (bits/nnconv.cu:280-311: im2row::forward + gemm 't','n'
+   accumulated over images) */
+MCN_API int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters,
+                                     const float* x, const float* derOutput, void* workspace,
+                                     size_t workspaceBytes);
+
+/* dzdb: K values, fully overwritten  (bits/nnconv.cu:230-244: gemv with the all-ones vector) */
+MCN_API int mcn_conv_backward_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* derBias,
+                                   const float* derOutput, void* workspace, size_t workspaceBytes);
+
+/* ------------------------------------------------------------------------------------------------
+ * batch normalisation -- replaces BatchNorm*<VLDT_GPU,T> (bits/nnbnorm_gpu.cu:818-1188).
+ * `moments` is C x 2: C means followed by C sigmas, sigma = sqrt(var + epsilon) (bits/nnbnorm.cu:65-70).
+ * ---------------------------------------------------------------------------------------------- */
+
+MCN_API size_t mcn_bnorm_workspace_bytes(int H, int W, int C, int N);
+
+/* givenMoments == 0: moments are computed from the batch and, if `moments` is non-NULL, written there
+   (BatchNorm::forward, bits/nnbnorm.cu:201-256).  givenMoments != 0: `moments` is an input
+   (forwardWithMoment, :170-199). */
+MCN_API int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float* x,
+                              const float* multipliers, const float* biases, int H, int W, int C, int N,
+                              double epsilon, int givenMoments, void* workspace, size_t workspaceBytes);
+
+/* dzdx (H x W x C x N), dzdg (C), dzdb (C), all fully overwritten.  givenMoments == 0: BatchNorm::backward
+   (bits/nnbnorm.cu:307-365), moments written if non-NULL.  givenMoments != 0: backwardWithMoment (:263-305). */
+MCN_API int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers,
+                               float* derBiases, float* moments, const float* x,
+                               const float* multipliers, const float* derOutput, int H, int W, int C,
+                               int N, double epsilon, int givenMoments, void* workspace,
+                               size_t workspaceBytes);
+
+/* ------------------------------------------------------------------------------------------------
+ * pooling -- replaces PoolingForward/Backward<VLDT_GPU,T> (bits/nnpooling_gpu.cu:270-415).
+ * ---------------------------------------------------------------------------------------------- */
+
+MCN_API int mcn_pool_output_size(const mcn_pool_geom* g, int* outH, int* outW);
+
+MCN_API int mcn_pool_forward(mcn_stream_t stream, const mcn_pool_geom* g, float* y, const float* x);
+
+/* accumulate != 0: derInput += pooling'(derOutput), the contract of vl::nn::Pooling::backward, whose
+   caller zero-fills derInput first (vl_nnpool.cu:255-259).  accumulate == 0: derInput is write-only and
+   receives exactly what the reference produces from a zero-filled buffer, so the separate fill pass
+   can be dropped.  Either way the result is deterministic and, for max pooling, bit-identical to the
+   reference CPU loop (first maximum in memory order wins, bits/nnpooling.cu:47-53,190-206). */
+MCN_API int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInput,
+                              const float* x, const float* derOutput, int accumulate);
+
+/* ------------------------------------------------------------------------------------------------
+ * element-wise companions used between the operators above
+ * ---------------------------------------------------------------------------------------------- */
+
+/* y = max(x, 0); dzdx = dzdy .* (x > 0)   (matlab/vl_nnrelu.m:43-48, leak = 0) */
+MCN_API int mcn_relu_forward(mcn_stream_t stream, float* y, const float* x, size_t n);
+MCN_API int mcn_relu_backward(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, size_t n);
+/* y = a + b   (matlab/+dagnn/Sum.m:11-17; also the fan-out derivative sum of +dagnn/Layer.m:127-135) */
+MCN_API int mcn_add(mcn_stream_t stream, float* y, const float* a, const float* b, size_t n);
+/* y[i] = value   (bits/impl/copy_gpu.cu:17-33 fill) */
+MCN_API int mcn_fill(mcn_stream_t stream, float* y, float value, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MCN_HIP_H */

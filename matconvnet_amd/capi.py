@@ -1,0 +1,294 @@
+"""ctypes binding of the C ABI in include/mcn_hip.h (libmcn_hip.so).
+
+Fails loudly when the library is missing: there is no fallback path.  Tensors are torch CUDA tensors used
+purely as device buffers; a MATLAB array H x W x C x N (column-major) is a contiguous torch tensor of
+shape (N, C, W, H).
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmcn_hip.so")
+
+SUCCESS, UNSUPPORTED, DEVICE_ERROR, OUT_OF_MEMORY, OUT_OF_GPU_MEMORY, ILLEGAL_ARGUMENT, UNKNOWN = 0, 1, 2, 5, 6, 7, 8
+CONV_FORWARD, CONV_BACKWARD_DATA, CONV_BACKWARD_FILTER, CONV_BACKWARD_BIAS = 0, 1, 2, 3
+POOL_MAX, POOL_AVERAGE = 0, 1
+
+
+class ConvGeom(C.Structure):
+    _fields_ = [(n, C.c_int) for n in (
+        "H", "W", "C", "N", "FH", "FW", "FC", "K", "strideY", "strideX",
+        "padTop", "padBottom", "padLeft", "padRight", "dilateY", "dilateX")]
+
+
+class PoolGeom(C.Structure):
+    _fields_ = [(n, C.c_int) for n in (
+        "H", "W", "C", "N", "poolH", "poolW", "strideY", "strideX",
+        "padTop", "padBottom", "padLeft", "padRight", "method")]
+
+
+class McnError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("mcn error %d: %s" % (code, message))
+        self.code = code
+        self.message = message
+
+
+# every exported symbol of include/mcn_hip.h: (restype, argtypes)
+_vp, _sz, _i, _f, _d = C.c_void_p, C.c_size_t, C.c_int, C.c_float, C.c_double
+PROTOTYPES = {
+    "mcn_last_error_message": (C.c_char_p, []),
+    "mcn_error_name": (C.c_char_p, [_i]),
+    "mcn_device_compute_units": (_i, []),
+    "mcn_set_tunable": (_i, [C.c_char_p, _i]),
+    "mcn_get_tunable": (_i, [C.c_char_p, C.POINTER(_i)]),
+    "mcn_conv_output_size": (_i, [C.POINTER(ConvGeom), C.POINTER(_i), C.POINTER(_i)]),
+    "mcn_conv_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _i]),
+    "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),
+    "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
+    "mcn_conv_backward_filter": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
+    "mcn_conv_backward_bias": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _sz]),
+    "mcn_bnorm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "mcn_bnorm_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
+    "mcn_bnorm_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
+    "mcn_pool_output_size": (_i, [C.POINTER(PoolGeom), C.POINTER(_i), C.POINTER(_i)]),
+    "mcn_pool_forward": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp]),
+    "mcn_pool_backward": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp, _vp, _i]),
+    "mcn_relu_forward": (_i, [_vp, _vp, _vp, _sz]),
+    "mcn_relu_backward": (_i, [_vp, _vp, _vp, _vp, _sz]),
+    "mcn_add": (_i, [_vp, _vp, _vp, _vp, _sz]),
+    "mcn_fill": (_i, [_vp, _vp, _f, _sz]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built: no fallback exists."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -m matconvnet_amd.build` (hipcc, gfx950)" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise McnError(rc, lib().mcn_last_error_message().decode())
+
+
+def set_tunable(name, value):
+    check(lib().mcn_set_tunable(name.encode(), int(value)))
+
+
+def get_tunable(name):
+    v = C.c_int(0)
+    check(lib().mcn_get_tunable(name.encode(), C.byref(v)))
+    return v.value
+
+
+def _pair(v):
+    v = np.atleast_1d(v).astype(int).ravel()
+    return (int(v[0]), int(v[0])) if v.size == 1 else (int(v[0]), int(v[1]))
+
+
+def _quad(v):
+    v = np.atleast_1d(v).astype(int).ravel()
+    return (int(v[0]),) * 4 if v.size == 1 else tuple(int(t) for t in v[:4])
+
+
+def conv_geom(xshape, fshape, stride=1, pad=0, dilate=1):
+    """Shapes are MATLAB-style (H, W, C, N) / (FH, FW, FC, K)."""
+    H, W, Cc, N = (list(xshape) + [1, 1, 1])[:4]
+    FH, FW, FC, K = (list(fshape) + [1, 1, 1])[:4]
+    sy, sx = _pair(stride)
+    pt, pb, pl, pr = _quad(pad)
+    dy, dx = _pair(dilate)
+    return ConvGeom(H, W, Cc, N, FH, FW, FC, K, sy, sx, pt, pb, pl, pr, dy, dx)
+
+
+def pool_geom(xshape, pool, stride=1, pad=0, method="max"):
+    H, W, Cc, N = (list(xshape) + [1, 1, 1])[:4]
+    ph, pw = _pair(pool)
+    sy, sx = _pair(stride)
+    pt, pb, pl, pr = _quad(pad)
+    return PoolGeom(H, W, Cc, N, ph, pw, sy, sx, pt, pb, pl, pr, POOL_MAX if method == "max" else POOL_AVERAGE)
+
+
+def conv_out_shape(g):
+    oh, ow = C.c_int(0), C.c_int(0)
+    check(lib().mcn_conv_output_size(C.byref(g), C.byref(oh), C.byref(ow)))
+    return (oh.value, ow.value, g.K, g.N)
+
+
+def pool_out_shape(g):
+    oh, ow = C.c_int(0), C.c_int(0)
+    check(lib().mcn_pool_output_size(C.byref(g), C.byref(oh), C.byref(ow)))
+    return (oh.value, ow.value, g.C, g.N)
+
+
+# ---------------------------------------------------------------------------------------------------
+# device-buffer helpers (torch is plumbing: allocation, host<->device copies, the stream handle)
+# ---------------------------------------------------------------------------------------------------
+
+def _torch():
+    import torch
+    return torch
+
+
+def to_device(a):
+    """numpy (H,W,C,N) array in any order -> contiguous float32 CUDA tensor of shape reversed(a.shape)."""
+    torch = _torch()
+    f = np.asfortranarray(a, dtype=np.float32)
+    return torch.from_numpy(np.ascontiguousarray(f.T)).cuda()
+
+
+def to_host(t, dtype=None):
+    """CUDA tensor of shape (N,C,W,H) -> Fortran-ordered numpy array (H,W,C,N)."""
+    a = t.detach().cpu().numpy().T
+    return np.asfortranarray(a, dtype=dtype or a.dtype)
+
+
+def empty(mshape, fill=None):
+    """Device buffer for a MATLAB-shaped array (H,W,C,N,...)."""
+    torch = _torch()
+    shape = tuple(reversed([int(s) for s in mshape]))
+    if fill is None:
+        return torch.empty(shape, dtype=torch.float32, device="cuda")
+    return torch.full(shape, float(fill), dtype=torch.float32, device="cuda")
+
+
+def ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def stream():
+    return C.c_void_p(_torch().cuda.current_stream().cuda_stream)
+
+
+class Workspace:
+    """Grow-only device scratch buffer, the role of vl::Context::getWorkspace."""
+
+    def __init__(self):
+        self.buf = None
+
+    def get(self, nbytes):
+        torch = _torch()
+        nbytes = int(nbytes)
+        if nbytes == 0:
+            return None, 0
+        if self.buf is None or self.buf.numel() < nbytes:
+            self.buf = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        return C.c_void_p(self.buf.data_ptr()), self.buf.numel()
+
+
+_ws = Workspace()
+
+
+# ---------------------------------------------------------------------------------------------------
+# thin call wrappers (device tensors in, device tensors out)
+# ---------------------------------------------------------------------------------------------------
+
+def conv_forward(x, f, b, g, y=None, out_mult=0.0, in_mult=1.0, ws=None):
+    ws = ws or _ws
+    if y is None:
+        y = empty(conv_out_shape(g))
+    wp, wn = ws.get(lib().mcn_conv_workspace_bytes(C.byref(g), CONV_FORWARD))
+    check(lib().mcn_conv_forward(stream(), C.byref(g), ptr(y), out_mult, ptr(x), in_mult, ptr(f), ptr(b), wp, wn))
+    return y
+
+
+def conv_backward(x, f, dy, g, want=(True, True, True), ws=None):
+    ws = ws or _ws
+    L = lib()
+    dx = df = db = None
+    if want[0]:
+        dx = empty((g.H, g.W, g.C, g.N))
+        wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_DATA))
+        check(L.mcn_conv_backward_data(stream(), C.byref(g), ptr(dx), ptr(f), ptr(dy), wp, wn))
+    if want[1]:
+        df = empty((g.FH, g.FW, g.FC, g.K))
+        wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_FILTER))
+        check(L.mcn_conv_backward_filter(stream(), C.byref(g), ptr(df), ptr(x), ptr(dy), wp, wn))
+    if want[2]:
+        db = empty((g.K,))
+        wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_BIAS))
+        check(L.mcn_conv_backward_bias(stream(), C.byref(g), ptr(db), ptr(dy), wp, wn))
+    return dx, df, db
+
+
+def _hwcn(t):
+    s = list(reversed(t.shape))
+    return (s + [1, 1, 1])[:4]
+
+
+def bnorm_forward(x, g, b, eps=1e-4, moments=None, ws=None):
+    ws = ws or _ws
+    H, W, Cc, N = _hwcn(x)
+    y = empty((H, W, Cc, N))
+    given = moments is not None
+    mom = moments if given else empty((Cc, 2))
+    wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
+    check(lib().mcn_bnorm_forward(stream(), ptr(y), ptr(mom), ptr(x), ptr(g), ptr(b), H, W, Cc, N, eps, int(given), wp, wn))
+    return y, mom
+
+
+def bnorm_backward(x, g, dy, eps=1e-4, moments=None, ws=None, want_moments=True):
+    ws = ws or _ws
+    H, W, Cc, N = _hwcn(x)
+    dx = empty((H, W, Cc, N))
+    dg = empty((Cc,))
+    db = empty((Cc,))
+    given = moments is not None
+    mom = moments if given else (empty((Cc, 2)) if want_moments else None)
+    wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
+    check(lib().mcn_bnorm_backward(stream(), ptr(dx), ptr(dg), ptr(db), ptr(mom), ptr(x), ptr(g), ptr(dy),
+                                   H, W, Cc, N, eps, int(given), wp, wn))
+    return dx, dg, db, mom
+
+
+def pool_forward(x, g):
+    y = empty(pool_out_shape(g))
+    check(lib().mcn_pool_forward(stream(), C.byref(g), ptr(y), ptr(x)))
+    return y
+
+
+def pool_backward(x, dy, g, dx=None):
+    """dx given: accumulate into it (vl::nn::Pooling::backward contract); else a fresh write-only output."""
+    acc = dx is not None
+    if dx is None:
+        dx = empty((g.H, g.W, g.C, g.N))
+    check(lib().mcn_pool_backward(stream(), C.byref(g), ptr(dx), ptr(x), ptr(dy), int(acc)))
+    return dx
+
+
+def relu_forward(x):
+    y = _torch().empty_like(x)
+    check(lib().mcn_relu_forward(stream(), ptr(y), ptr(x), x.numel()))
+    return y
+
+
+def relu_backward(x, dy):
+    dx = _torch().empty_like(x)
+    check(lib().mcn_relu_backward(stream(), ptr(dx), ptr(x), ptr(dy), x.numel()))
+    return dx
+
+
+def add(a, b):
+    y = _torch().empty_like(a)
+    check(lib().mcn_add(stream(), ptr(y), ptr(a), ptr(b), a.numel()))
+    return y
+
+
+def fill(t, value):
+    check(lib().mcn_fill(stream(), ptr(t), float(value), t.numel()))
+    return t

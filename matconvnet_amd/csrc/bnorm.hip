@@ -1,0 +1,365 @@
+// Batch normalisation forward / backward for gfx950.
+//
+// Two launches per call:
+//   1. bnorm_sums  -- grid (channel, image-group).  Each workgroup streams its planes of x (and dzdy)
+//      once with 16-byte loads, keeps fp32 running sums per lane for one plane at a time, folds them into
+//      fp64 per plane, reduces across the wavefront with shuffles and across wavefronts through LDS, and
+//      writes one fp64 partial per (channel, group): sum x, sum x^2, sum x*dzdy, sum dzdy.
+//   2. bnorm_apply -- same grid.  Each workgroup re-reduces its channel's partials in a fixed order
+//      (deterministic), derives mean / sigma / dzdg / dzdb in fp64 exactly as the reference formulas
+//      (bits/nnbnorm.cu:101-164), and streams the elementwise result
+//      dzdx = G1*(dzdy - dzdb/m) - G2*(x - mean), written as two fused multiply-adds.
+//      The first group of each channel also stores dzdg, dzdb and the moments.
+//   The apply pass can walk the planes in the reverse order of the sums pass so that it starts on the
+//   data most recently pulled through the caches.
+//
+// Accuracy: the reference sums ~1e5 terms sequentially in float; here at most one plane-slice per lane
+// is summed in fp32 and everything above is fp64, so results sit close to the reference's own
+// double-precision instantiation.
+#include "mcn_internal.hpp"
+
+#include <algorithm>
+
+namespace mcn {
+namespace {
+
+struct BnormP {
+  int WH, C, N;
+  int groups;        // image groups per channel (grid = C * groups)
+  int reverse;       // apply pass walks logical ids backwards
+  double mass;       // WH * N
+  double epsilon;
+};
+
+__device__ __forceinline__ void image_range(const BnormP& p, int grp, int* n0, int* n1) {
+  *n0 = (int)(((long long)p.N * grp) / p.groups);
+  *n1 = (int)(((long long)p.N * (grp + 1)) / p.groups);
+}
+
+// Block-wide sum of NV doubles held per thread; result valid in thread 0.
+template <int NV>
+__device__ __forceinline__ void block_sum(double (&v)[NV], double* lds /* [4][NV] */) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) v[i] = wave_sum(v[i]);
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) lds[wave * NV + i] = v[i];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) v[i] = (lds[i] + lds[NV + i]) + (lds[2 * NV + i] + lds[3 * NV + i]);
+  }
+}
+
+// MODE 0: sum x, sum x^2               (forward, moments from the batch)
+// MODE 1: sum x*dy, sum dy             (backward, moments given)
+// MODE 2: all four                     (backward, moments from the batch)
+template <int MODE, bool VEC4>
+__global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
+                                                  const float* __restrict__ dy,
+                                                  double* __restrict__ partials, BnormP p) {
+  __shared__ double lds[16];
+  const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int c = logical / p.groups;
+  const int grp = logical - c * p.groups;
+  int n0, n1;
+  image_range(p, grp, &n0, &n1);
+  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  for (int n = n0; n < n1; ++n) {
+    const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
+    float sx = 0.f, sxx = 0.f, sxd = 0.f, sd = 0.f;
+    if (VEC4) {
+      const float4* x4 = (const float4*)(x + base);
+      const float4* d4 = (const float4*)(MODE != 0 ? dy + base : x + base);
+      for (int i = threadIdx.x; i < p.WH / 4; i += 256) {
+        const float4 a = x4[i];
+        if (MODE != 1) {
+          sx += (a.x + a.y) + (a.z + a.w);
+          sxx += (a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w);
+        }
+        if (MODE != 0) {
+          const float4 d = d4[i];
+          sxd += (a.x * d.x + a.y * d.y) + (a.z * d.z + a.w * d.w);
+          sd += (d.x + d.y) + (d.z + d.w);
+        }
+      }
+    } else {
+      for (int i = threadIdx.x; i < p.WH; i += 256) {
+        const float a = x[base + i];
+        if (MODE != 1) {
+          sx += a;
+          sxx += a * a;
+        }
+        if (MODE != 0) {
+          const float d = dy[base + i];
+          sxd += a * d;
+          sd += d;
+        }
+      }
+    }
+    acc[0] += (double)sx;
+    acc[1] += (double)sxx;
+    acc[2] += (double)sxd;
+    acc[3] += (double)sd;
+  }
+  block_sum<4>(acc, lds);
+  if (threadIdx.x == 0) {
+    double* out = partials + ((size_t)c * p.groups + grp) * 4;
+    out[0] = acc[0];
+    out[1] = acc[1];
+    out[2] = acc[2];
+    out[3] = acc[3];
+  }
+}
+
+// Sum of a channel's partials in a fixed order: lane i owns groups i, i+64, ...; then a wave tree.
+// Every lane of wave 0 ends with the totals; other waves read them from LDS.
+__device__ __forceinline__ void channel_totals(const double* __restrict__ partials, const BnormP& p,
+                                               int c, double* lds, double (&tot)[4]) {
+  if (threadIdx.x < kWave) {
+    double v[4] = {0.0, 0.0, 0.0, 0.0};
+    for (int g = threadIdx.x; g < p.groups; g += kWave) {
+      const double* in = partials + ((size_t)c * p.groups + g) * 4;
+      v[0] += in[0];
+      v[1] += in[1];
+      v[2] += in[2];
+      v[3] += in[3];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = wave_sum(v[i]);
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) lds[i] = v[i];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) tot[i] = lds[i];
+}
+
+// out = a*in1 + b*in2 + k over this workgroup's planes (in2 optional)
+template <bool TWO, bool VEC4>
+__device__ __forceinline__ void stream_planes(float* __restrict__ out, const float* __restrict__ in1,
+                                              const float* __restrict__ in2, float a, float b, float k,
+                                              const BnormP& p, int c, int n0, int n1) {
+  for (int nn = n0; nn < n1; ++nn) {
+    const int n = p.reverse ? (n1 - 1 - (nn - n0)) : nn;
+    const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
+    if (VEC4) {
+      const float4* s1 = (const float4*)(in1 + base);
+      const float4* s2 = (const float4*)(TWO ? in2 + base : in1 + base);
+      float4* o4 = (float4*)(out + base);
+      for (int i = threadIdx.x; i < p.WH / 4; i += 256) {
+        const float4 u = s1[i];
+        float4 r;
+        if (TWO) {
+          const float4 v = s2[i];
+          r.x = fmaf(a, u.x, fmaf(b, v.x, k));
+          r.y = fmaf(a, u.y, fmaf(b, v.y, k));
+          r.z = fmaf(a, u.z, fmaf(b, v.z, k));
+          r.w = fmaf(a, u.w, fmaf(b, v.w, k));
+        } else {
+          r.x = fmaf(a, u.x, k);
+          r.y = fmaf(a, u.y, k);
+          r.z = fmaf(a, u.z, k);
+          r.w = fmaf(a, u.w, k);
+        }
+        o4[i] = r;
+      }
+    } else {
+      for (int i = threadIdx.x; i < p.WH; i += 256) {
+        const float u = in1[base + i];
+        out[base + i] = TWO ? fmaf(a, u, fmaf(b, in2[base + i], k)) : fmaf(a, u, k);
+      }
+    }
+  }
+}
+
+// Backward apply.  GIVEN: mean/sigma come from `moments` (input); otherwise from the partial sums and
+// `moments` (if non-null) is written.
+template <bool GIVEN, bool VEC4>
+__global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ dx,
+                                                            float* __restrict__ dmult,
+                                                            float* __restrict__ dbias,
+                                                            float* __restrict__ moments,
+                                                            const float* __restrict__ x,
+                                                            const float* __restrict__ mult,
+                                                            const float* __restrict__ dy,
+                                                            const double* __restrict__ partials,
+                                                            BnormP p) {
+  __shared__ double lds[4];
+  int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  if (p.reverse) logical = (int)gridDim.x - 1 - logical;
+  const int c = logical / p.groups;
+  const int grp = logical - c * p.groups;
+  double tot[4];
+  channel_totals(partials, p, c, lds, tot);
+
+  double mean, sigma;
+  if (GIVEN) {
+    mean = (double)moments[c];
+    sigma = (double)moments[c + p.C];
+  } else {
+    mean = tot[0] / p.mass;
+    const double var = fmax(0.0, tot[1] / p.mass - mean * mean);
+    sigma = sqrt(var + p.epsilon);
+  }
+  const double dB = tot[3];
+  const double dG = (tot[2] - mean * dB) / sigma;
+  const double muz = dB / p.mass;
+  const double G1 = (double)mult[c] / sigma;
+  const double G2 = G1 * dG / (p.mass * sigma);
+  if (grp == 0 && threadIdx.x == 0) {
+    dmult[c] = (float)dG;
+    dbias[c] = (float)dB;
+    if (!GIVEN && moments) {
+      moments[c] = (float)mean;
+      moments[c + p.C] = (float)sigma;
+    }
+  }
+  // dzdx = G1*(dy - muz) - G2*(x - mean) = G1*dy + (-G2)*x + (G2*mean - G1*muz)
+  int n0, n1;
+  image_range(p, grp, &n0, &n1);
+  stream_planes<true, VEC4>(dx, dy, x, (float)G1, (float)(-G2), (float)(G2 * mean - G1 * muz), p, c, n0, n1);
+}
+
+// Forward apply: y = (g/sigma)*(x - mean) + b  (bits/nnbnorm.cu:190-199)
+template <bool GIVEN, bool VEC4>
+__global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y,
+                                                           float* __restrict__ moments,
+                                                           const float* __restrict__ x,
+                                                           const float* __restrict__ mult,
+                                                           const float* __restrict__ bias,
+                                                           const double* __restrict__ partials,
+                                                           BnormP p) {
+  __shared__ double lds[4];
+  int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  if (p.reverse) logical = (int)gridDim.x - 1 - logical;
+  const int c = logical / p.groups;
+  const int grp = logical - c * p.groups;
+  double mean, sigma;
+  if (GIVEN) {
+    mean = (double)moments[c];
+    sigma = (double)moments[c + p.C];
+  } else {
+    double tot[4];
+    channel_totals(partials, p, c, lds, tot);
+    mean = tot[0] / p.mass;
+    const double var = fmax(0.0, tot[1] / p.mass - mean * mean);
+    sigma = sqrt(var + p.epsilon);
+    if (grp == 0 && threadIdx.x == 0 && moments) {
+      moments[c] = (float)mean;
+      moments[c + p.C] = (float)sigma;
+    }
+  }
+  const double coef = (double)mult[c] / sigma;
+  int n0, n1;
+  image_range(p, grp, &n0, &n1);
+  stream_planes<false, VEC4>(y, x, nullptr, (float)coef, 0.f, (float)((double)bias[c] - coef * mean), p, c, n0, n1);
+}
+
+int image_groups(int WH, int N) {
+  // one plane per workgroup unless planes are small; then enough planes to own ~bnorm_block_elems
+  const int want = std::max(tunable("bnorm_block_elems", 4096), 1);
+  const int perBlock = std::max(1, want / std::max(WH, 1));
+  return std::max(1, (N + perBlock - 1) / perBlock);
+}
+
+int setup(const char* who, int H, int W, int C, int N, double epsilon, BnormP* p) {
+  if (H < 0 || W < 0 || C < 0 || N < 0) return fail(MCN_ILLEGAL_ARGUMENT, "%s: negative tensor extent", who);
+  if ((long long)H * W >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: plane too large", who);
+  p->WH = H * W;
+  p->C = C;
+  p->N = N;
+  p->groups = image_groups(p->WH, N);
+  p->reverse = tunable("bnorm_reverse_apply", 1) ? 1 : 0;
+  p->mass = (double)p->WH * (double)N;
+  p->epsilon = epsilon;
+  if ((long long)C * p->groups >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: too many channels", who);
+  return MCN_SUCCESS;
+}
+
+}  // namespace
+}  // namespace mcn
+
+using namespace mcn;
+
+extern "C" {
+
+size_t mcn_bnorm_workspace_bytes(int H, int W, int C, int N) {
+  if (H <= 0 || W <= 0 || C <= 0 || N <= 0) return 0;
+  return (size_t)C * image_groups(H * W, N) * 4 * sizeof(double);
+}
+
+int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,
+                      const float* biases, int H, int W, int C, int N, double epsilon, int givenMoments,
+                      void* workspace, size_t workspaceBytes) {
+  BnormP p;
+  int rc = setup("mcn_bnorm_forward", H, W, C, N, epsilon, &p);
+  if (rc) return rc;
+  if ((size_t)p.WH * C * N == 0) return MCN_SUCCESS;
+  if (!y || !x || !multipliers || !biases) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward: null tensor");
+  if (givenMoments && !moments) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward: moments are required");
+  hipStream_t s = as_stream(stream);
+  const bool vec = (p.WH % 4 == 0) && aligned16(y) && aligned16(x);
+  const dim3 grid((unsigned)(C * p.groups)), block(256);
+  double* partials = (double*)workspace;
+  if (!givenMoments) {
+    if (!workspace || workspaceBytes < mcn_bnorm_workspace_bytes(H, W, C, N))
+      return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward: workspace too small");
+    if (vec) hipLaunchKernelGGL((bnorm_sums<0, true>), grid, block, 0, s, x, x, partials, p);
+    else hipLaunchKernelGGL((bnorm_sums<0, false>), grid, block, 0, s, x, x, partials, p);
+    if ((rc = check_launch("mcn_bnorm_forward(sums)"))) return rc;
+    if (vec) hipLaunchKernelGGL((bnorm_forward_apply<false, true>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
+    else hipLaunchKernelGGL((bnorm_forward_apply<false, false>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
+  } else {
+    p.reverse = 0;
+    if (vec) hipLaunchKernelGGL((bnorm_forward_apply<true, true>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
+    else hipLaunchKernelGGL((bnorm_forward_apply<true, false>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
+  }
+  return check_launch("mcn_bnorm_forward");
+}
+
+int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases, float* moments,
+                       const float* x, const float* multipliers, const float* derOutput, int H, int W, int C,
+                       int N, double epsilon, int givenMoments, void* workspace, size_t workspaceBytes) {
+  BnormP p;
+  int rc = setup("mcn_bnorm_backward", H, W, C, N, epsilon, &p);
+  if (rc) return rc;
+  if (C == 0) return MCN_SUCCESS;
+  if (!derMultipliers || !derBiases || !multipliers)
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward: null parameter tensor");
+  if ((size_t)p.WH * N == 0) {
+    // nothing to sum over: the reference leaves dzdg = 0/sigma-related garbage; define zeros
+    if ((rc = mcn_fill(stream, derMultipliers, 0.f, (size_t)C))) return rc;
+    return mcn_fill(stream, derBiases, 0.f, (size_t)C);
+  }
+  if (!derInput || !x || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward: null tensor");
+  if (givenMoments && !moments) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward: moments are required");
+  if (!workspace || workspaceBytes < mcn_bnorm_workspace_bytes(H, W, C, N))
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward: workspace too small");
+  hipStream_t s = as_stream(stream);
+  const bool vec = (p.WH % 4 == 0) && aligned16(derInput) && aligned16(x) && aligned16(derOutput);
+  const dim3 grid((unsigned)(C * p.groups)), block(256);
+  double* partials = (double*)workspace;
+  if (givenMoments) {
+    if (vec) hipLaunchKernelGGL((bnorm_sums<1, true>), grid, block, 0, s, x, derOutput, partials, p);
+    else hipLaunchKernelGGL((bnorm_sums<1, false>), grid, block, 0, s, x, derOutput, partials, p);
+  } else {
+    if (vec) hipLaunchKernelGGL((bnorm_sums<2, true>), grid, block, 0, s, x, derOutput, partials, p);
+    else hipLaunchKernelGGL((bnorm_sums<2, false>), grid, block, 0, s, x, derOutput, partials, p);
+  }
+  if ((rc = check_launch("mcn_bnorm_backward(sums)"))) return rc;
+  if (givenMoments) {
+    if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
+    else hipLaunchKernelGGL((bnorm_backward_apply<true, false>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
+  } else {
+    if (vec) hipLaunchKernelGGL((bnorm_backward_apply<false, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
+    else hipLaunchKernelGGL((bnorm_backward_apply<false, false>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
+  }
+  return check_launch("mcn_bnorm_backward");
+}
+
+}  // extern "C"

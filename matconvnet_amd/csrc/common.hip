@@ -1,0 +1,103 @@
+// Error state, tunables and device queries of the gfx950 back-end.
+#include "mcn_internal.hpp"
+
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+
+namespace mcn {
+
+namespace {
+thread_local char g_message[512] = "";
+std::mutex g_tunable_mutex;
+
+struct Tunable {
+  const char* name;
+  int value;
+};
+// Defaults are the values chosen from on-device sweeps; see the per-kernel comments where each is read.
+Tunable g_tunables[] = {
+    {"pool_lds_bytes", 24 * 1024},     // LDS tile budget of the pooling-backward kernel
+    {"bnorm_block_elems", 4096},       // minimum elements a bnorm reduction block should own
+    {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)
+    {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels
+    {"conv_wgrad_blocks", 0},          // target workgroups for filter-gradient split (0 = 2 per CU)
+    {"conv_bias_blocks", 0},           // target workgroups for the bias-gradient reduction
+};
+}  // namespace
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_message, sizeof(g_message), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void clear_error() { g_message[0] = 0; }
+
+int check_launch(const char* what) {
+  hipError_t e = hipPeekAtLastError();
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(MCN_DEVICE_ERROR, "%s: %s", what, hipGetErrorString(e));
+  }
+  return MCN_SUCCESS;
+}
+
+int tunable(const char* name, int fallback) {
+  std::lock_guard<std::mutex> lock(g_tunable_mutex);
+  for (auto& t : g_tunables)
+    if (std::strcmp(t.name, name) == 0) return t.value;
+  return fallback;
+}
+
+}  // namespace mcn
+
+extern "C" {
+
+const char* mcn_last_error_message(void) { return mcn::g_message; }
+
+const char* mcn_error_name(int code) {
+  switch (code) {
+    case MCN_SUCCESS: return "success";
+    case MCN_UNSUPPORTED: return "unsupported feature error";
+    case MCN_DEVICE_ERROR: return "HIP error";
+    case MCN_OUT_OF_MEMORY: return "out of memory error";
+    case MCN_OUT_OF_GPU_MEMORY: return "out of GPU memory error";
+    case MCN_ILLEGAL_ARGUMENT: return "illegal argument error";
+    default: return "unknown error";
+  }
+}
+
+int mcn_device_compute_units(void) {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return -1;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
+  return cus;
+}
+
+int mcn_set_tunable(const char* name, int value) {
+  if (!name) return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_set_tunable: null name");
+  std::lock_guard<std::mutex> lock(mcn::g_tunable_mutex);
+  for (auto& t : mcn::g_tunables)
+    if (std::strcmp(t.name, name) == 0) {
+      t.value = value;
+      return MCN_SUCCESS;
+    }
+  return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_set_tunable: unknown tunable '%s'", name);
+}
+
+int mcn_get_tunable(const char* name, int* value) {
+  if (!name || !value) return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_get_tunable: null argument");
+  std::lock_guard<std::mutex> lock(mcn::g_tunable_mutex);
+  for (auto& t : mcn::g_tunables)
+    if (std::strcmp(t.name, name) == 0) {
+      *value = t.value;
+      return MCN_SUCCESS;
+    }
+  return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_get_tunable: unknown tunable '%s'", name);
+}
+
+}  // extern "C"

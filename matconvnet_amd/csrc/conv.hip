@@ -1,0 +1,178 @@
+// Convolution entry points: validation, dispatch between the MFMA implicit-GEMM kernels and the direct
+// kernels, and the bias-gradient reduction.
+#include "conv_common.hpp"
+
+#include <algorithm>
+
+namespace mcn {
+
+int conv_setup(const mcn_conv_geom* g, const char* who, ConvP* p) {
+  if (!g) return fail(MCN_ILLEGAL_ARGUMENT, "%s: null geometry", who);
+  if (g->H < 0 || g->W < 0 || g->C < 0 || g->N < 0) return fail(MCN_ILLEGAL_ARGUMENT, "%s: negative tensor extent", who);
+  if (g->strideY < 1 || g->strideX < 1)
+    return fail(MCN_ILLEGAL_ARGUMENT, "%s: at least one element of STRIDE is smaller than one", who);
+  if (g->padTop < 0 || g->padBottom < 0 || g->padLeft < 0 || g->padRight < 0)
+    return fail(MCN_ILLEGAL_ARGUMENT, "%s: an element of PAD is negative", who);
+  if (g->dilateY < 1 || g->dilateX < 1) return fail(MCN_ILLEGAL_ARGUMENT, "%s: an element of DILATE is less than one", who);
+  if (g->FH < 1 || g->FW < 1 || g->FC < 1 || g->K < 1) return fail(MCN_ILLEGAL_ARGUMENT, "%s: a dimension of FILTERS is void", who);
+  const int extY = (g->FH - 1) * g->dilateY + 1, extX = (g->FW - 1) * g->dilateX + 1;
+  if (g->H + g->padTop + g->padBottom < extY || g->W + g->padLeft + g->padRight < extX)
+    return fail(MCN_ILLEGAL_ARGUMENT, "%s: FILTERS are larger than the DATA (including padding)", who);
+  const int groups = g->C / g->FC;
+  if (groups * g->FC != g->C) return fail(MCN_ILLEGAL_ARGUMENT, "%s: the FILTERS depth does not divide the DATA depth", who);
+  if (groups < 1 || g->K % groups != 0)
+    return fail(MCN_ILLEGAL_ARGUMENT, "%s: the number of filter groups does not divide the number of filters", who);
+  p->H = g->H; p->W = g->W; p->C = g->C; p->N = g->N;
+  p->FH = g->FH; p->FW = g->FW; p->FC = g->FC; p->K = g->K;
+  p->sy = g->strideY; p->sx = g->strideX; p->pt = g->padTop; p->pl = g->padLeft;
+  p->dy = g->dilateY; p->dx = g->dilateX;
+  p->outH = (g->H + g->padTop + g->padBottom - extY) / g->strideY + 1;
+  p->outW = (g->W + g->padLeft + g->padRight - extX) / g->strideX + 1;
+  p->groups = groups;
+  p->Kg = g->K / groups;
+  const long long lim = 1ll << 31;
+  if ((long long)g->H * g->W * g->C >= lim || (long long)p->outH * p->outW * g->K >= lim ||
+      (long long)g->FH * g->FW * g->FC * g->K >= lim)
+    return fail(MCN_UNSUPPORTED, "%s: an image or the filter bank exceeds 2^31 elements", who);
+  return MCN_SUCCESS;
+}
+
+namespace {
+
+// ---- bias gradient: db[k] = sum_{n,p} dy[p,k,n].
+// Stage 1: grid (k, image group); lanes stream planes with 16-byte loads, fp32 per plane per lane, fp64
+// above, wavefront shuffle reduction + LDS across the four wavefronts.  Stage 2: one lane per filter adds
+// the image-group partials in a fixed order.
+template <bool VEC4>
+__global__ __launch_bounds__(256) void conv_bias_partial(double* __restrict__ partials,
+                                                         const float* __restrict__ dy, int P, int K, int N,
+                                                         int groups) {
+  __shared__ double lds[4];
+  const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int k = logical / groups, grp = logical - k * groups;
+  const int n0 = (int)(((long long)N * grp) / groups), n1 = (int)(((long long)N * (grp + 1)) / groups);
+  double acc = 0.0;
+  for (int n = n0; n < n1; ++n) {
+    const float* src = dy + (size_t)P * (k + (size_t)K * n);
+    float s = 0.f;
+    if (VEC4) {
+      const float4* s4 = (const float4*)src;
+      for (int i = threadIdx.x; i < P / 4; i += 256) {
+        const float4 v = s4[i];
+        s += (v.x + v.y) + (v.z + v.w);
+      }
+    } else {
+      for (int i = threadIdx.x; i < P; i += 256) s += src[i];
+    }
+    acc += (double)s;
+  }
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) partials[(size_t)k * groups + grp] = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+}
+
+__global__ __launch_bounds__(256) void conv_bias_finish(float* __restrict__ db, const double* __restrict__ partials,
+                                                        int K, int groups) {
+  const int k = blockIdx.x * 256 + threadIdx.x;
+  if (k >= K) return;
+  double s = 0.0;
+  for (int g = 0; g < groups; ++g) s += partials[(size_t)k * groups + g];
+  db[k] = (float)s;
+}
+
+int bias_groups(const ConvP& p) {
+  int target = tunable("conv_bias_blocks", 0);
+  if (target <= 0) target = 2048;
+  const int P = p.outH * p.outW;
+  const int perBlock = std::max(1, 4096 / std::max(P, 1));  // at least ~4096 elements per workgroup
+  const int maxGroups = std::max(1, (p.N + perBlock - 1) / perBlock);
+  return std::max(1, std::min(maxGroups, (target + p.K - 1) / p.K));
+}
+
+}  // namespace
+}  // namespace mcn
+
+using namespace mcn;
+
+extern "C" {
+
+int mcn_conv_output_size(const mcn_conv_geom* g, int* outH, int* outW) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_output_size", &p);
+  if (rc) return rc;
+  if (outH) *outH = p.outH;
+  if (outW) *outW = p.outW;
+  return MCN_SUCCESS;
+}
+
+size_t mcn_conv_workspace_bytes(const mcn_conv_geom* g, int product) {
+  ConvP p;
+  if (conv_setup(g, "mcn_conv_workspace_bytes", &p)) return 0;
+  if (p.N == 0) return 0;
+  if (product == MCN_CONV_BACKWARD_BIAS) return (size_t)p.K * bias_groups(p) * sizeof(double);
+  return conv_mfma_workspace_bytes(p, product);
+}
+
+int mcn_conv_forward(mcn_stream_t stream, const mcn_conv_geom* g, float* y, float outMult, const float* x,
+                     float inMult, const float* filters, const float* bias, void* workspace, size_t workspaceBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_forward", &p);
+  if (rc) return rc;
+  if ((size_t)p.outH * p.outW * p.K * p.N == 0) return MCN_SUCCESS;
+  if (!y || !x || !filters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_forward: null tensor");
+  if (!tunable("conv_force_direct", 0) && conv_mfma_forward_supported(p))
+    return conv_forward_mfma(as_stream(stream), p, y, outMult, x, inMult, filters, bias, workspace, workspaceBytes);
+  return conv_forward_direct(as_stream(stream), p, y, outMult, x, inMult, filters, bias);
+}
+
+int mcn_conv_backward_data(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, const float* filters,
+                           const float* derOutput, void* workspace, size_t workspaceBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_data", &p);
+  if (rc) return rc;
+  if ((size_t)p.H * p.W * p.C * p.N == 0) return MCN_SUCCESS;
+  if (!derInput || !filters || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data: null tensor");
+  if (!tunable("conv_force_direct", 0) && conv_mfma_backward_data_supported(p))
+    return conv_backward_data_mfma(as_stream(stream), p, derInput, filters, derOutput, workspace, workspaceBytes);
+  return conv_backward_data_direct(as_stream(stream), p, derInput, filters, derOutput);
+}
+
+int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters, const float* x,
+                             const float* derOutput, void* workspace, size_t workspaceBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_filter", &p);
+  if (rc) return rc;
+  if (!derFilters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: null tensor");
+  const size_t nf = (size_t)p.FH * p.FW * p.FC * p.K;
+  if ((size_t)p.outH * p.outW * p.N == 0) return mcn_fill(stream, derFilters, 0.f, nf);
+  if (!x || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: null tensor");
+  if (!tunable("conv_force_direct", 0) && conv_mfma_backward_filter_supported(p))
+    return conv_backward_filter_mfma(as_stream(stream), p, derFilters, x, derOutput, workspace, workspaceBytes);
+  return conv_backward_filter_direct(as_stream(stream), p, derFilters, x, derOutput);
+}
+
+int mcn_conv_backward_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* derBias, const float* derOutput,
+                           void* workspace, size_t workspaceBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_bias", &p);
+  if (rc) return rc;
+  if (!derBias) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_bias: null tensor");
+  const int P = p.outH * p.outW;
+  if ((size_t)P * p.N == 0) return mcn_fill(stream, derBias, 0.f, (size_t)p.K);
+  if (!derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_bias: null tensor");
+  const int groups = bias_groups(p);
+  if (!workspace || workspaceBytes < (size_t)p.K * groups * sizeof(double))
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_bias: workspace too small");
+  double* partials = (double*)workspace;
+  hipStream_t s = as_stream(stream);
+  const bool vec = (P % 4 == 0) && aligned16(derOutput);
+  const dim3 grid((unsigned)(p.K * groups)), block(256);
+  if (vec) hipLaunchKernelGGL(conv_bias_partial<true>, grid, block, 0, s, partials, derOutput, P, p.K, p.N, groups);
+  else hipLaunchKernelGGL(conv_bias_partial<false>, grid, block, 0, s, partials, derOutput, P, p.K, p.N, groups);
+  if ((rc = check_launch("mcn_conv_backward_bias(partial)"))) return rc;
+  hipLaunchKernelGGL(conv_bias_finish, dim3((unsigned)((p.K + 255) / 256)), block, 0, s, derBias, partials, p.K, groups);
+  return check_launch("mcn_conv_backward_bias");
+}
+
+}  // extern "C"

@@ -1,0 +1,89 @@
+// Element-wise companions of the operators: ReLU, sum of two tensors, fill.  Pure streaming kernels:
+// 16-byte accesses, grid-stride, enough workgroups to cover the chip several times.
+#include "mcn_internal.hpp"
+
+#include <algorithm>
+
+namespace mcn {
+namespace {
+
+enum { OP_RELU_FWD, OP_RELU_BWD, OP_ADD, OP_FILL };
+
+template <int OP>
+__device__ __forceinline__ float apply1(float a, float b, float k) {
+  switch (OP) {
+    case OP_RELU_FWD: return a > 0.f ? a : 0.f;          // max(x, 0)
+    case OP_RELU_BWD: return a > 0.f ? b : b * 0.f;      // dzdy .* (x > 0): keeps NaN/inf*0 semantics
+    case OP_ADD: return __fadd_rn(a, b);
+    default: return k;
+  }
+}
+
+// y = op(a, b).  The vector body covers n/4 float4s; the tail (n % 4) is handled by the first threads.
+template <int OP, bool VEC4>
+__global__ __launch_bounds__(256) void eltwise_kernel(float* __restrict__ y, const float* __restrict__ a,
+                                                      const float* __restrict__ b, float k, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (VEC4) {
+    const size_t n4 = n / 4;
+    for (size_t i = t; i < n4; i += stride) {
+      float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u, r;
+      if (OP != OP_FILL) u = ((const float4*)a)[i];
+      if (OP == OP_RELU_BWD || OP == OP_ADD) v = ((const float4*)b)[i];
+      r.x = apply1<OP>(u.x, v.x, k);
+      r.y = apply1<OP>(u.y, v.y, k);
+      r.z = apply1<OP>(u.z, v.z, k);
+      r.w = apply1<OP>(u.w, v.w, k);
+      ((float4*)y)[i] = r;
+    }
+    for (size_t i = n4 * 4 + t; i < n; i += stride) {
+      const float u = (OP != OP_FILL) ? a[i] : 0.f;
+      const float v = (OP == OP_RELU_BWD || OP == OP_ADD) ? b[i] : 0.f;
+      y[i] = apply1<OP>(u, v, k);
+    }
+  } else {
+    for (size_t i = t; i < n; i += stride) {
+      const float u = (OP != OP_FILL) ? a[i] : 0.f;
+      const float v = (OP == OP_RELU_BWD || OP == OP_ADD) ? b[i] : 0.f;
+      y[i] = apply1<OP>(u, v, k);
+    }
+  }
+}
+
+template <int OP>
+int launch(const char* who, mcn_stream_t stream, float* y, const float* a, const float* b, float k, size_t n) {
+  if (n == 0) return MCN_SUCCESS;
+  if (!y || (OP != OP_FILL && !a) || ((OP == OP_RELU_BWD || OP == OP_ADD) && !b))
+    return fail(MCN_ILLEGAL_ARGUMENT, "%s: null tensor", who);
+  const bool vec = aligned16(y) && (OP == OP_FILL || aligned16(a)) &&
+                   (!(OP == OP_RELU_BWD || OP == OP_ADD) || aligned16(b));
+  // each thread handles a few float4s; cap the grid at 32 workgroups per CU-equivalent (256 CUs)
+  const size_t work = vec ? (n + 3) / 4 : n;
+  const unsigned blocks = (unsigned)std::min<size_t>((work + 255) / 256, 256u * 32u);
+  if (vec) hipLaunchKernelGGL((eltwise_kernel<OP, true>), dim3(blocks), dim3(256), 0, as_stream(stream), y, a, b, k, n);
+  else hipLaunchKernelGGL((eltwise_kernel<OP, false>), dim3(blocks), dim3(256), 0, as_stream(stream), y, a, b, k, n);
+  return check_launch(who);
+}
+
+}  // namespace
+}  // namespace mcn
+
+using namespace mcn;
+
+extern "C" {
+
+int mcn_relu_forward(mcn_stream_t stream, float* y, const float* x, size_t n) {
+  return launch<OP_RELU_FWD>("mcn_relu_forward", stream, y, x, nullptr, 0.f, n);
+}
+int mcn_relu_backward(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, size_t n) {
+  return launch<OP_RELU_BWD>("mcn_relu_backward", stream, derInput, x, derOutput, 0.f, n);
+}
+int mcn_add(mcn_stream_t stream, float* y, const float* a, const float* b, size_t n) {
+  return launch<OP_ADD>("mcn_add", stream, y, a, b, 0.f, n);
+}
+int mcn_fill(mcn_stream_t stream, float* y, float value, size_t n) {
+  return launch<OP_FILL>("mcn_fill", stream, y, nullptr, nullptr, value, n);
+}
+
+}  // extern "C"

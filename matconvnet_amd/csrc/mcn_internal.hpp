@@ -1,0 +1,54 @@
+// Shared host/device helpers of the gfx950 back-end: error reporting, launch checks, index helpers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/mcn_hip.h"
+
+namespace mcn {
+
+// Records a message for the calling thread and returns `code` (numerically a vl::ErrorCode).
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+// Looks at the launch status without synchronising (the reference peeks the same way,
+// bits/datacu.cu:356-371): a failed launch becomes MCN_DEVICE_ERROR with the HIP text.
+int check_launch(const char* what);
+
+int tunable(const char* name, int fallback);
+
+inline hipStream_t as_stream(mcn_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int div_up(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+constexpr int kWave = 64;      // CDNA wavefront width
+constexpr int kNumXcd = 8;     // MI355X: 8 accelerator dies, each with its own L2
+
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs.  This maps a hardware block id to a
+// logical id such that each XCD walks one contiguous range of logical ids, so neighbouring tiles
+// (which share halos / operands) meet in the same L2.
+__device__ __forceinline__ int xcd_contiguous_id(int bid, int nblocks) {
+  const int q = nblocks / kNumXcd, r = nblocks % kNumXcd;
+  const int xcd = bid % kNumXcd, i = bid / kNumXcd;
+  return xcd * q + (xcd < r ? xcd : r) + i;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+}  // namespace mcn
