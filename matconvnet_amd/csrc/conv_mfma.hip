@@ -1,11 +1,561 @@
-// placeholder: MFMA kernels not yet enabled
+// Implicit-GEMM convolution on the fp32 matrix cores of gfx950 (v_mfma_f32_32x32x2_f32), filter groups = 1.
+//
+// No im2row buffer exists anywhere: the gather of shifted, zero-padded pixels happens while tiles are
+// loaded from global memory into LDS.
+//
+// Two kernels:
+//
+//   conv_pix_mfma    out[co, m] = sum_R wt[R][co] * in[ci(R), pixel(m) shifted by tap(R)]
+//       m runs over (output pixel, image) with pixels fastest -- the memory-contiguous axis of every tensor
+//       here -- and sits on the MFMA "B / column" side, so each accumulator register of a lane is one
+//       channel and 32 consecutive lanes are 32 consecutive pixels: stores are 128-byte runs.
+//       Forward:        in = x,    R = (i,j,c), out = y,    tap shift = (i*dilate - pad) on a strided grid.
+//       Backward-data:  in = dzdy, R = (i,j,k), out = dzdx, tap shift = (pad - i*dilate), stride 1.
+//       The filter bank is first rewritten as wt[R][co] (co contiguous, zero padded to tile multiples) by a
+//       small prologue kernel so weight tiles load as 16-byte vectors with no bounds tests.
+//
+//   conv_wgrad_mfma  dF[R, k] = sum_m xg[R, m] * dzdy[k, m],  xg = the (never materialised) patch matrix.
+//       The reduction axis m (pixels x images) is split across workgroups; each writes a partial filter
+//       bank and a second kernel adds the partials in a fixed order (deterministic, no atomics).
+//       R sits on the MFMA column side, so stores run along the contiguous axis of dF.
+//
+// Work decomposition: 256 threads = 4 wavefronts; a wavefront owns WA x WB blocks of 32 x 32 accumulators;
+// LDS tiles are double buffered with one barrier per reduction step; global loads for step i+1 are issued
+// before the MFMAs of step i and parked in registers.
 #include "conv_common.hpp"
+
+#include <algorithm>
+
 namespace mcn {
-bool conv_mfma_forward_supported(const ConvP&) { return false; }
-bool conv_mfma_backward_data_supported(const ConvP&) { return false; }
-bool conv_mfma_backward_filter_supported(const ConvP&) { return false; }
-size_t conv_mfma_workspace_bytes(const ConvP&, int) { return 0; }
-int conv_forward_mfma(hipStream_t, const ConvP&, float*, float, const float*, float, const float*, const float*, void*, size_t) { return fail(MCN_UNSUPPORTED, "n/a"); }
-int conv_backward_data_mfma(hipStream_t, const ConvP&, float*, const float*, const float*, void*, size_t) { return fail(MCN_UNSUPPORTED, "n/a"); }
-int conv_backward_filter_mfma(hipStream_t, const ConvP&, float*, const float*, const float*, void*, size_t) { return fail(MCN_UNSUPPORTED, "n/a"); }
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kMaxTaps = 128;
+
+// ------------------------------------------------------------------------------------------------
+// pixel-major kernel (forward / backward-data)
+// ------------------------------------------------------------------------------------------------
+
+struct PixP {
+  int IH, IW, Cin;    // grid and channels of the gathered tensor
+  int OH, OW, Cout;   // grid and channels of the produced tensor
+  int N;
+  int FH, T;          // filter height, taps = FH*FW
+  int sy, sx;         // gathered row = oh*sy + dh(tap)
+  int dhBase, dhStep, dwBase, dwStep;
+  int R;              // reduction length = T*Cin
+  int coutPad;        // row pitch of wt
+  long long M;        // OH*OW*N
+  float alpha, beta;
+};
+
+// wt[R][co] from the MATLAB filter bank f[i,j,c,k] (FV x K, column-major).
+//   forward:        R = t + T*c, co = k : f[R + FV*k]
+//   backward-data:  R = t + T*k, co = c : f[t + T*(c + C*k)]
+__global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt, const float* __restrict__ f,
+                                                         int T, int Cin, int Cout, int rPad, int coutPad,
+                                                         int backward) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)rPad * coutPad) return;
+  const int r = (int)(idx / coutPad), co = (int)(idx - (size_t)r * coutPad);
+  float v = 0.f;
+  if (r < T * Cin && co < Cout) {
+    if (!backward) {
+      v = f[(size_t)r + (size_t)T * Cin * co];
+    } else {
+      const int k = r / T, t = r - k * T;
+      v = f[(size_t)t + (size_t)T * (co + (size_t)Cout * k)];
+    }
+  }
+  wt[idx] = v;
 }
+
+template <int WA, int WB, int NWA, int NWB>
+__global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out, const float* __restrict__ in,
+                                                        const float* __restrict__ wt,
+                                                        const float* __restrict__ bias, PixP p) {
+  static_assert(NWA * NWB == 4, "four wavefronts per workgroup");
+  constexpr int BA = WA * 32 * NWA;  // output channels per workgroup
+  constexpr int BB = WB * 32 * NWB;  // pixels per workgroup
+  constexpr int BK = 16;             // reduction rows per step
+  constexpr int PIXG = 256 / BB;     // thread groups sharing the pixel tile rows
+  constexpr int RPT = BK / PIXG;     // gathered rows per thread and step
+  constexpr int A4 = BK * BA / 4;    // float4s in a weight tile
+  constexpr int APT = (A4 + 255) / 256;
+
+  __shared__ float As[2][BK * BA];
+  __shared__ float Bs[2][BK * BB];
+  __shared__ int2 tapTab[kMaxTaps];  // .x = dh + IH*dw, .y = (dh & 0xffff) | (dw << 16)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, kh = lane >> 5;
+  const int wa = wave / NWB, wb = wave - wa * NWB;
+
+  const int tilesA = (p.Cout + BA - 1) / BA;
+  const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int mt = logical / tilesA;
+  const int co0 = (logical - mt * tilesA) * BA;
+  const long long m0 = (long long)mt * BB;
+
+  const int IHW = p.IH * p.IW;
+  const int Q = p.OH * p.OW;
+
+  if (tid < p.T) {
+    const int j = tid / p.FH, i = tid - j * p.FH;
+    const int dh = p.dhBase + i * p.dhStep, dw = p.dwBase + j * p.dwStep;
+    tapTab[tid] = make_int2(dh + p.IH * dw, (int)((unsigned)(dh & 0xffff) | ((unsigned)dw << 16)));
+  }
+
+  // ---- this thread's pixel (fixed for the whole kernel)
+  const int mm = tid % BB, pg = tid / BB;
+  const long long m = m0 + mm;
+  const bool mvalid = m < p.M;
+  int ihB = 0, iwB = 0;
+  const float* inN = in;
+  {
+    const long long mc = mvalid ? m : 0;
+    const int n = (int)(mc / Q);
+    const int q = (int)(mc - (long long)n * Q);
+    const int ow = q / p.OH, oh = q - ow * p.OH;
+    ihB = oh * p.sy;
+    iwB = ow * p.sx;
+    inN = in + (size_t)n * p.Cin * IHW + ihB + p.IH * iwB;
+  }
+  // first gathered row of this thread: R = pg*RPT -> (tap, channel); advanced by BK per step
+  int tapS = (pg * RPT) % p.T, ciS = (pg * RPT) / p.T;
+  const int advC = BK / p.T, advT = BK % p.T;
+
+  floatx16 acc[WA][WB];
+#pragma unroll
+  for (int a = 0; a < WA; ++a)
+#pragma unroll
+    for (int b = 0; b < WB; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  float pb[RPT];
+  float4 pa[APT];
+  const int nSteps = (p.R + BK - 1) / BK;
+
+  auto fetch = [&](int step) {
+    int t = tapS, ci = ciS;
+#pragma unroll
+    for (int e = 0; e < RPT; ++e) {
+      const int2 tp = tapTab[t];
+      const int ih = ihB + (int)(short)(tp.y & 0xffff);
+      const int iw = iwB + (tp.y >> 16);
+      const bool ok = mvalid && ci < p.Cin && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
+      pb[e] = ok ? inN[ci * IHW + tp.x] : 0.f;
+      if (++t == p.T) {
+        t = 0;
+        ++ci;
+      }
+    }
+    ciS += advC;
+    tapS += advT;
+    if (tapS >= p.T) {
+      tapS -= p.T;
+      ++ciS;
+    }
+    const float* wrow = wt + (size_t)step * BK * p.coutPad + co0;
+#pragma unroll
+    for (int e = 0; e < APT; ++e) {
+      const int idx = tid + 256 * e;
+      if (A4 % 256 == 0 || idx < A4) {
+        const int row = idx / (BA / 4), c4 = idx - row * (BA / 4);
+        pa[e] = *(const float4*)(wrow + (size_t)row * p.coutPad + c4 * 4);
+      }
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int e = 0; e < RPT; ++e) Bs[buf][(pg * RPT + e) * BB + mm] = pb[e];
+#pragma unroll
+    for (int e = 0; e < APT; ++e) {
+      const int idx = tid + 256 * e;
+      if (A4 % 256 == 0 || idx < A4) *(float4*)&As[buf][idx * 4] = pa[e];
+    }
+  };
+
+  __syncthreads();  // tapTab ready
+  fetch(0);
+  stash(0);
+  __syncthreads();
+
+  for (int step = 0; step < nSteps; ++step) {
+    const int buf = step & 1;
+    if (step + 1 < nSteps) fetch(step + 1);
+    const float* Ab = As[buf] + wa * WA * 32 + l32;
+    const float* Bb = Bs[buf] + wb * WB * 32 + l32;
+#pragma unroll
+    for (int s = 0; s < BK / 2; ++s) {
+      float a[WA], b[WB];
+#pragma unroll
+      for (int ii = 0; ii < WA; ++ii) a[ii] = Ab[(2 * s + kh) * BA + ii * 32];
+#pragma unroll
+      for (int jj = 0; jj < WB; ++jj) b[jj] = Bb[(2 * s + kh) * BB + jj * 32];
+#pragma unroll
+      for (int ii = 0; ii < WA; ++ii)
+#pragma unroll
+        for (int jj = 0; jj < WB; ++jj)
+          acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii], b[jj], acc[ii][jj], 0, 0, 0);
+    }
+    if (step + 1 < nSteps) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane = pixel, register = channel
+#pragma unroll
+  for (int jj = 0; jj < WB; ++jj) {
+    const long long mo = m0 + wb * WB * 32 + jj * 32 + l32;
+    if (mo >= p.M) continue;
+    const int n = (int)(mo / Q);
+    const int q = (int)(mo - (long long)n * Q);
+    float* o = out + (size_t)n * p.Cout * Q + q;
+#pragma unroll
+    for (int ii = 0; ii < WA; ++ii)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int co = co0 + wa * WA * 32 + ii * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
+        if (co < p.Cout) {
+          float v = p.alpha * acc[ii][jj][r];
+          if (p.beta != 0.f) v = fmaf(p.beta, o[(size_t)co * Q], v);
+          if (bias) v += bias[co];
+          o[(size_t)co * Q] = v;
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// filter-gradient kernel
+// ------------------------------------------------------------------------------------------------
+
+struct WgP {
+  int H, W, C, K;
+  int OH, OW;
+  int FH, T;
+  int sy, sx, pt, pl, dly, dlx;
+  int FV;
+  long long M;           // OH*OW*N
+  long long chunkSpan;   // pixels per split (multiple of 32)
+  int splits;
+};
+
+template <int WA, int WB, int NWA, int NWB>
+__global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ out, const float* __restrict__ x,
+                                                          const float* __restrict__ dy, WgP p) {
+  static_assert(NWA * NWB == 4, "four wavefronts per workgroup");
+  constexpr int BA = WA * 32 * NWA;  // filters (k) per workgroup
+  constexpr int BB = WB * 32 * NWB;  // filter-volume rows (R) per workgroup
+  constexpr int BP = 32;             // pixels per reduction step
+  constexpr int LD = BP + 1;         // padded LDS pitch: column reads hit 32 distinct banks
+  constexpr int APT = BA / 8, BPT = BB / 8;
+
+  // dynamic LDS (the 128 x 128 configuration needs 67 KB, above the 64 KB static limit)
+  extern __shared__ float smem[];
+  float(*As)[BA * LD] = (float(*)[BA * LD])smem;                  // [2][BA*LD]
+  float(*Bs)[BB * LD] = (float(*)[BB * LD])(smem + 2 * BA * LD);  // [2][BB*LD]
+  int2* rowTab = (int2*)(smem + 2 * (BA + BB) * LD);              // [BB] .x = c*H*W + dh + H*dw, .y = dh | dw << 16
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, kh = lane >> 5;
+  const int wa = wave / NWB, wb = wave - wa * NWB;
+
+  const int tilesK = (p.K + BA - 1) / BA, tilesR = (p.FV + BB - 1) / BB;
+  const int tiles = tilesK * tilesR;
+  const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int split = logical / tiles;
+  const int tile = logical - split * tiles;
+  const int rt = tile / tilesK;
+  const int k0 = (tile - rt * tilesK) * BA;
+  const int r0 = rt * BB;
+
+  const int HW = p.H * p.W;
+  const int Q = p.OH * p.OW;
+
+  if (tid < BB) {
+    const int R = r0 + tid;
+    int2 e = make_int2(0, 0x8000);  // dh = -32768: never inside the image
+    if (R < p.FV) {
+      const int c = R / p.T, t = R - c * p.T;
+      const int j = t / p.FH, i = t - j * p.FH;
+      const int dh = i * p.dly - p.pt, dw = j * p.dlx - p.pl;
+      e = make_int2(c * HW + dh + p.H * dw, (int)((unsigned)(dh & 0xffff) | ((unsigned)dw << 16)));
+    }
+    rowTab[tid] = e;
+  }
+
+  const long long mBegin = (long long)split * p.chunkSpan;
+  const long long mEnd = min(mBegin + p.chunkSpan, p.M);
+  const int nSteps = mEnd > mBegin ? (int)((mEnd - mBegin + BP - 1) / BP) : 0;
+
+  const int px = tid & 31, rg = tid >> 5;
+
+  floatx16 acc[WA][WB];
+#pragma unroll
+  for (int a = 0; a < WA; ++a)
+#pragma unroll
+    for (int b = 0; b < WB; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  float pa[APT], pb[BPT];
+
+  auto fetch = [&](int step) {
+    const long long m = mBegin + (long long)step * BP + px;
+    const bool valid = m < mEnd;
+    const long long mc = valid ? m : mBegin;
+    const int n = (int)(mc / Q);
+    const int q = (int)(mc - (long long)n * Q);
+    const int ow = q / p.OH, oh = q - ow * p.OH;
+    const int ihB = oh * p.sy, iwB = ow * p.sx;
+    const float* xN = x + (size_t)n * p.C * HW + ihB + p.H * iwB;
+    const float* dyN = dy + (size_t)n * p.K * Q + q;
+#pragma unroll
+    for (int e = 0; e < BPT; ++e) {
+      const int2 tp = rowTab[rg + 8 * e];
+      const int ih = ihB + (int)(short)(tp.y & 0xffff);
+      const int iw = iwB + (tp.y >> 16);
+      const bool ok = valid && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+      pb[e] = ok ? xN[tp.x] : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < APT; ++e) {
+      const int k = k0 + rg + 8 * e;
+      pa[e] = (valid && k < p.K) ? dyN[(size_t)k * Q] : 0.f;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int e = 0; e < BPT; ++e) Bs[buf][(rg + 8 * e) * LD + px] = pb[e];
+#pragma unroll
+    for (int e = 0; e < APT; ++e) As[buf][(rg + 8 * e) * LD + px] = pa[e];
+  };
+
+  __syncthreads();  // rowTab ready
+  if (nSteps > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+
+  for (int step = 0; step < nSteps; ++step) {
+    const int buf = step & 1;
+    if (step + 1 < nSteps) fetch(step + 1);
+    const float* Ab = As[buf] + (wa * WA * 32 + l32) * LD + kh;
+    const float* Bb = Bs[buf] + (wb * WB * 32 + l32) * LD + kh;
+#pragma unroll
+    for (int s = 0; s < BP / 2; ++s) {
+      float a[WA], b[WB];
+#pragma unroll
+      for (int ii = 0; ii < WA; ++ii) a[ii] = Ab[ii * 32 * LD + 2 * s];
+#pragma unroll
+      for (int jj = 0; jj < WB; ++jj) b[jj] = Bb[jj * 32 * LD + 2 * s];
+#pragma unroll
+      for (int ii = 0; ii < WA; ++ii)
+#pragma unroll
+        for (int jj = 0; jj < WB; ++jj)
+          acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii], b[jj], acc[ii][jj], 0, 0, 0);
+    }
+    if (step + 1 < nSteps) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane = filter-volume row R (contiguous in dF), register = filter k
+  float* o = out + (size_t)split * p.FV * p.K;
+#pragma unroll
+  for (int jj = 0; jj < WB; ++jj) {
+    const int R = r0 + wb * WB * 32 + jj * 32 + l32;
+    if (R >= p.FV) continue;
+#pragma unroll
+    for (int ii = 0; ii < WA; ++ii)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int k = k0 + wa * WA * 32 + ii * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
+        if (k < p.K) o[(size_t)R + (size_t)p.FV * k] = acc[ii][jj][r];
+      }
+  }
+}
+
+// dF[e] = sum over splits, in ascending split order
+__global__ __launch_bounds__(256) void conv_wgrad_reduce(float* __restrict__ df, const float* __restrict__ partials,
+                                                         size_t n, int splits) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float s = partials[i];
+  for (int k = 1; k < splits; ++k) s += partials[(size_t)k * n + i];
+  df[i] = s;
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+
+int pick_channels_tile(int cout) { return cout > 64 ? 128 : (cout > 32 ? 64 : 32); }
+
+bool common_ok(const ConvP& p) {
+  // tap offsets are packed as 16-bit fields and "row absent" is encoded as offset -32768
+  const long long spanH = (long long)p.H + p.pt + (long long)p.FH * p.dy, spanW = (long long)p.W + p.pl + (long long)p.FW * p.dx;
+  return p.groups == 1 && p.FH * p.FW <= kMaxTaps && spanH < 32768 && spanW < 32768 &&
+         (long long)p.outH * p.outW * p.N < (1ll << 40);
+}
+
+int wgrad_splits(const ConvP& p, int* tilesOut) {
+  const int BA = pick_channels_tile(p.K), BB = 128;
+  const int tiles = ((p.K + BA - 1) / BA) * ((p.FH * p.FW * p.FC + BB - 1) / BB);
+  int target = tunable("conv_wgrad_blocks", 0);
+  if (target <= 0) target = 512;
+  const long long chunks = ((long long)p.outH * p.outW * p.N + 31) / 32;
+  long long s = std::max<long long>(1, target / tiles);
+  s = std::min<long long>(s, std::max<long long>(1, chunks / 4));  // at least 4 reduction steps per split
+  if (tilesOut) *tilesOut = tiles;
+  return (int)s;
+}
+
+template <int WA, int WB, int NWA, int NWB>
+void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, const PixP& p) {
+  constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB;
+  const long long mTiles = (p.M + BB - 1) / BB;
+  const int tilesA = (p.Cout + BA - 1) / BA;
+  hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB>), dim3((unsigned)(mTiles * tilesA)), dim3(256), 0, s, out, in,
+                     wt, bias, p);
+}
+
+template <int WA, int WB, int NWA, int NWB>
+int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const float* dy, const WgP& p) {
+  constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB, LD = 33;
+  constexpr size_t lds = (size_t)2 * (BA + BB) * LD * sizeof(float) + BB * sizeof(int2);
+  static bool raised = false;  // one-time opt-in to more than 64 KB of LDS per workgroup
+  if (lds > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(MCN_DEVICE_ERROR, "mcn_conv_backward_filter: cannot reserve %zu bytes of LDS", lds);
+    }
+    raised = true;
+  }
+  hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB>), grid, dim3(256), lds, s, out, x, dy, p);
+  return MCN_SUCCESS;
+}
+
+int run_pix(hipStream_t s, const char* who, float* out, const float* in, const float* f, const float* bias, PixP p,
+            int backward, void* ws, size_t wsBytes) {
+  const int BA = pick_channels_tile(p.Cout);
+  const int rPad = (p.R + 15) / 16 * 16;
+  p.coutPad = (p.Cout + BA - 1) / BA * BA;
+  const size_t need = (size_t)rPad * p.coutPad * sizeof(float);
+  if (!ws || wsBytes < need) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small (%zu < %zu bytes)", who, wsBytes, need);
+  if (!aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
+  float* wt = (float*)ws;
+  const size_t nW = (size_t)rPad * p.coutPad;
+  hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, wt, f, p.T, p.Cin, p.Cout,
+                     rPad, p.coutPad, backward);
+  int rc = check_launch(who);
+  if (rc) return rc;
+  const long long blocks = ((p.M + (BA == 128 ? 127 : 255)) / (BA == 128 ? 128 : 256)) * (p.coutPad / BA);
+  if (blocks >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
+  if (BA == 128) launch_pix<2, 2, 2, 2>(s, out, in, wt, bias, p);
+  else if (BA == 64) launch_pix<2, 2, 1, 4>(s, out, in, wt, bias, p);
+  else launch_pix<1, 2, 1, 4>(s, out, in, wt, bias, p);
+  return check_launch(who);
+}
+
+}  // namespace
+
+bool conv_mfma_forward_supported(const ConvP& p) { return common_ok(p); }
+bool conv_mfma_backward_data_supported(const ConvP& p) { return common_ok(p) && p.sy == 1 && p.sx == 1; }
+bool conv_mfma_backward_filter_supported(const ConvP& p) { return common_ok(p); }
+
+size_t conv_mfma_workspace_bytes(const ConvP& p, int product) {
+  const size_t FV = (size_t)p.FH * p.FW * p.FC;
+  switch (product) {
+    case MCN_CONV_FORWARD: {
+      if (!conv_mfma_forward_supported(p)) return 0;
+      const int BA = pick_channels_tile(p.K);
+      return ((FV + 15) / 16 * 16) * (size_t)((p.K + BA - 1) / BA * BA) * sizeof(float);
+    }
+    case MCN_CONV_BACKWARD_DATA: {
+      if (!conv_mfma_backward_data_supported(p)) return 0;
+      const int BA = pick_channels_tile(p.C);
+      const size_t R = (size_t)p.FH * p.FW * p.K;
+      return ((R + 15) / 16 * 16) * (size_t)((p.C + BA - 1) / BA * BA) * sizeof(float);
+    }
+    case MCN_CONV_BACKWARD_FILTER: {
+      if (!conv_mfma_backward_filter_supported(p)) return 0;
+      const int s = wgrad_splits(p, nullptr);
+      return s > 1 ? (size_t)s * FV * p.K * sizeof(float) : 0;
+    }
+    default: return 0;
+  }
+}
+
+int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
+                      const float* f, const float* b, void* ws, size_t wsBytes) {
+  PixP q;
+  q.IH = p.H; q.IW = p.W; q.Cin = p.C;
+  q.OH = p.outH; q.OW = p.outW; q.Cout = p.K;
+  q.N = p.N;
+  q.FH = p.FH; q.T = p.FH * p.FW;
+  q.sy = p.sy; q.sx = p.sx;
+  q.dhBase = -p.pt; q.dhStep = p.dy; q.dwBase = -p.pl; q.dwStep = p.dx;
+  q.R = q.T * q.Cin;
+  q.coutPad = 0;
+  q.M = (long long)p.outH * p.outW * p.N;
+  q.alpha = inMult; q.beta = outMult;
+  return run_pix(s, "mcn_conv_forward", y, x, f, b, q, 0, ws, wsBytes);
+}
+
+int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, const float* f, const float* dy, void* ws,
+                            size_t wsBytes) {
+  PixP q;
+  q.IH = p.outH; q.IW = p.outW; q.Cin = p.K;
+  q.OH = p.H; q.OW = p.W; q.Cout = p.C;
+  q.N = p.N;
+  q.FH = p.FH; q.T = p.FH * p.FW;
+  q.sy = 1; q.sx = 1;
+  q.dhBase = p.pt; q.dhStep = -p.dy; q.dwBase = p.pl; q.dwStep = -p.dx;
+  q.R = q.T * q.Cin;
+  q.coutPad = 0;
+  q.M = (long long)p.H * p.W * p.N;
+  q.alpha = 1.f; q.beta = 0.f;
+  return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, 1, ws, wsBytes);
+}
+
+int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,
+                              size_t wsBytes) {
+  WgP q;
+  q.H = p.H; q.W = p.W; q.C = p.C; q.K = p.K;
+  q.OH = p.outH; q.OW = p.outW;
+  q.FH = p.FH; q.T = p.FH * p.FW;
+  q.sy = p.sy; q.sx = p.sx; q.pt = p.pt; q.pl = p.pl; q.dly = p.dy; q.dlx = p.dx;
+  q.FV = p.FH * p.FW * p.FC;
+  q.M = (long long)p.outH * p.outW * p.N;
+  int tiles = 0;
+  q.splits = wgrad_splits(p, &tiles);
+  const long long chunks = (q.M + 31) / 32;
+  q.chunkSpan = ((chunks + q.splits - 1) / q.splits) * 32;
+  const size_t nF = (size_t)q.FV * p.K;
+  float* target = df;
+  if (q.splits > 1) {
+    const size_t need = (size_t)q.splits * nF * sizeof(float);
+    if (!ws || wsBytes < need)
+      return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: workspace too small (%zu < %zu bytes)", wsBytes, need);
+    target = (float*)ws;
+  }
+  const dim3 grid((unsigned)(tiles * q.splits)), block(256);
+  const int BA = pick_channels_tile(p.K);
+  int rc;
+  if (BA == 128) rc = launch_wgrad<2, 2, 2, 2>(s, grid, target, x, dy, q);
+  else if (BA == 64) rc = launch_wgrad<2, 1, 1, 4>(s, grid, target, x, dy, q);
+  else rc = launch_wgrad<1, 1, 1, 4>(s, grid, target, x, dy, q);
+  if (!rc) rc = check_launch("mcn_conv_backward_filter");
+  if (rc || q.splits == 1) return rc;
+  hipLaunchKernelGGL(conv_wgrad_reduce, dim3((unsigned)((nF + 255) / 256)), block, 0, s, df, target, nF, q.splits);
+  return check_launch("mcn_conv_backward_filter(reduce)");
+}
+
+}  // namespace mcn

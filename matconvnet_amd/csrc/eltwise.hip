@@ -4,6 +4,10 @@
 
 #include <algorithm>
 
+// Every multiply and add below must stay a separate IEEE operation: results are compared bit for bit
+// with the reference CPU loops, so fused multiply-add contraction is switched off for this file.
+#pragma clang fp contract(off)
+
 namespace mcn {
 namespace {
 
@@ -14,7 +18,7 @@ __device__ __forceinline__ float apply1(float a, float b, float k) {
   switch (OP) {
     case OP_RELU_FWD: return a > 0.f ? a : 0.f;          // max(x, 0)
     case OP_RELU_BWD: return a > 0.f ? b : b * 0.f;      // dzdy .* (x > 0): keeps NaN/inf*0 semantics
-    case OP_ADD: return __fadd_rn(a, b);
+    case OP_ADD: return a + b;
     default: return k;
   }
 }

@@ -19,6 +19,10 @@
 
 #include <algorithm>
 
+// Every multiply and add below must stay a separate IEEE operation: results are compared bit for bit
+// with the reference CPU loops, so fused multiply-add contraction is switched off for this file.
+#pragma clang fp contract(off)
+
 namespace mcn {
 namespace {
 
@@ -37,7 +41,7 @@ __device__ __forceinline__ float avg_scale(const PoolP& p, int oh, int ow) {
   int h2 = min(h1 + p.poolH, p.H), w2 = min(w1 + p.poolW, p.W);
   h1 = max(h1, 0);
   w1 = max(w1, 0);
-  return __fdiv_rn(1.0f, (float)((h2 - h1) * (w2 - w1)));
+  return 1.0f / (float)((h2 - h1) * (w2 - w1));  // correctly rounded IEEE division
 }
 
 template <bool MAX, bool VEC4>
@@ -130,9 +134,12 @@ __global__ __launch_bounds__(256) void pool_backward_tiled(float* __restrict__ d
       const int base = (ow - owLo) * p.outH;
       for (int oh = ohA; oh <= ohB; ++oh) {
         if (MAX) {
-          if (win[base + oh] == me) acc = __fadd_rn(acc, dys[base + oh]);
+          if (win[base + oh] == me) acc = acc + dys[base + oh];
         } else {
-          acc = __fadd_rn(acc, __fmul_rn(dys[base + oh], avg_scale(p, oh, ow)));
+          {
+            const float term = dys[base + oh] * avg_scale(p, oh, ow);  // rounded product, then a separate add
+            acc = acc + term;
+          }
         }
       }
     }
@@ -204,9 +211,12 @@ __global__ __launch_bounds__(256) void pool_backward_direct(float* __restrict__ 
               bi = ww * p.H + hh;
             }
           }
-        if (bi == me) acc = __fadd_rn(acc, d);
+        if (bi == me) acc = acc + d;
       } else {
-        acc = __fadd_rn(acc, __fmul_rn(d, avg_scale(p, oh, ow)));
+        {
+        const float term = d * avg_scale(p, oh, ow);
+        acc = acc + term;
+      }
       }
     }
   dx[idx] = acc;
@@ -240,8 +250,8 @@ __global__ __launch_bounds__(256) void pool_forward_kernel(float* __restrict__ y
   } else {
     float s = 0.f;
     for (int w = c1; w < c2; ++w)
-      for (int h = h1; h < h2; ++h) s = __fadd_rn(s, xp[w * p.H + h]);
-    y[idx] = __fmul_rn(s, __fdiv_rn(1.0f, (float)((h2 - h1) * (c2 - c1))));
+      for (int h = h1; h < h2; ++h) s = s + xp[w * p.H + h];
+    y[idx] = s * (1.0f / (float)((h2 - h1) * (c2 - c1)));
   }
 }
 

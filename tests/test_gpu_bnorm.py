@@ -1,0 +1,114 @@
+"""GPU parity, batch normalisation.  Gate (max|diff|/max|ref| over each output): 1e-5 against the double
+instantiation of the reference algorithm fed the same float inputs.  The float instantiation sums ~1e5
+terms sequentially in float and is itself further than 1e-5 from the double one at BASELINE sizes, so the
+distance to it is asserted only to the looser bound it can support."""
+import os
+
+import numpy as np
+import pytest
+
+from matconvnet_amd import workloads
+from util import F, rel_max
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "bnorm_golden.npz")
+SHAPES = [(2, 2, 1, 2), (8, 8, 3, 2), (13, 17, 4, 7), (8, 2, 3, 7), (1, 1, 5, 9), (56, 56, 8, 4), (7, 7, 64, 5), (30, 30, 3, 70)]
+
+
+def _case(shape, seed):
+    w = workloads.bnorm_case(seed=seed, H=shape[0], W=shape[1], C=shape[2], N=shape[3])
+    return w["x"], w["g"], w["b"], w["dy"]
+
+
+def _d(a):
+    return F(a, np.float64) if a.ndim > 1 else a.astype(np.float64)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("eps", [1e-4, 1e-5])
+def test_backward_batch_moments(capi, ob, shape, eps):
+    x, g, b, dy = _case(shape, 7)
+    dx, dg, db, mom = [capi.to_host(t) for t in capi.bnorm_backward(capi.to_device(x), capi.to_device(g), capi.to_device(dy), eps)]
+    wdx, wdg, wdb, wmom = ob.bnorm_backward(_d(x), _d(g), _d(dy), eps)
+    assert rel_max(dx, wdx) < TOL and rel_max(dg, wdg) < TOL and rel_max(db, wdb) < TOL and rel_max(mom, wmom) < TOL
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_backward_given_moments(capi, ob, shape):
+    x, g, b, dy = _case(shape, 8)
+    C = shape[2]
+    given = F(np.stack([np.linspace(-1, 1, C), np.linspace(0.5, 2, C)], axis=1))
+    dx, dg, db, _ = [capi.to_host(t) for t in capi.bnorm_backward(capi.to_device(x), capi.to_device(g), capi.to_device(dy), 1e-4, moments=capi.to_device(given))]
+    wdx, wdg, wdb, _ = ob.bnorm_backward(_d(x), _d(g), _d(dy), 1e-4, moments=_d(given))
+    assert rel_max(dx, wdx) < TOL and rel_max(dg, wdg) < TOL and rel_max(db, wdb) < TOL
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_forward_both_modes(capi, ob, shape):
+    x, g, b, dy = _case(shape, 9)
+    y, mom = [capi.to_host(t) for t in capi.bnorm_forward(capi.to_device(x), capi.to_device(g), capi.to_device(b), 1e-4)]
+    wy, wmom = ob.bnorm_forward(_d(x), _d(g), _d(b), 1e-4)
+    assert rel_max(y, wy) < TOL and rel_max(mom, wmom) < TOL
+    y2, _ = capi.bnorm_forward(capi.to_device(x), capi.to_device(g), capi.to_device(b), 1e-4, moments=capi.to_device(wmom))
+    assert rel_max(capi.to_host(y2), wy) < TOL
+
+
+def test_moments_not_requested(capi, ob):
+    """vl_nnbnorm with three outputs: no moments tensor is passed (vl_nnbnorm.cu:105,210-213)."""
+    x, g, b, dy = _case((8, 8, 3, 2), 3)
+    dx, dg, db, mom = capi.bnorm_backward(capi.to_device(x), capi.to_device(g), capi.to_device(dy), 1e-4, want_moments=False)
+    assert mom is None
+    wdx, wdg, wdb, _ = ob.bnorm_backward(_d(x), _d(g), _d(dy), 1e-4)
+    assert rel_max(capi.to_host(dx), wdx) < TOL
+
+
+def test_golden_vectors_from_reference(capi):
+    """Outputs of the compiled reference (its double instantiation: entries with float64 dtype)."""
+    z = np.load(GOLDEN)
+    checked = 0
+    for k in range(int(z["count"])):
+        if z["x_%d" % k].dtype != np.float64:
+            continue
+        x, g, b, dy, eps = z["x_%d" % k], z["g_%d" % k], z["b_%d" % k], z["dy_%d" % k], float(z["eps_%d" % k])
+        xd, gd, bd, dyd = capi.to_device(x), capi.to_device(g), capi.to_device(b), capi.to_device(dy)
+        y, mom = [capi.to_host(t) for t in capi.bnorm_forward(xd, gd, bd, eps)]
+        assert rel_max(y, z["y_%d" % k]) < TOL and rel_max(mom, z["mom_%d" % k]) < TOL
+        dx, dg, db, mom2 = [capi.to_host(t) for t in capi.bnorm_backward(xd, gd, dyd, eps)]
+        assert rel_max(dx, z["dx_%d" % k]) < TOL and rel_max(dg, z["dg_%d" % k]) < TOL
+        assert rel_max(db, z["db_%d" % k]) < TOL and rel_max(mom2, z["mom2_%d" % k]) < TOL
+        given = capi.to_device(z["given_%d" % k])
+        dxg, dgg, dbg, _ = [capi.to_host(t) for t in capi.bnorm_backward(xd, gd, dyd, eps, moments=given)]
+        assert rel_max(dxg, z["dxg_%d" % k]) < TOL and rel_max(dgg, z["dgg_%d" % k]) < TOL and rel_max(dbg, z["dbg_%d" % k]) < TOL
+        checked += 1
+    assert checked >= 4
+
+
+def test_baseline_config_full_size(capi, ob):
+    """BASELINE config 2: 56x56x256x32, eps 1e-4, moments from the batch."""
+    w = workloads.bnorm_case()
+    x, g, dy = w["x"], w["g"], w["dy"]
+    dx, dg, db, mom = [capi.to_host(t) for t in capi.bnorm_backward(capi.to_device(x), capi.to_device(g), capi.to_device(dy), w["eps"])]
+    wdx, wdg, wdb, wmom = ob.bnorm_backward(_d(x), _d(g), _d(dy), w["eps"])
+    d = dict(dzdx=rel_max(dx, wdx), dzdg=rel_max(dg, wdg), dzdb=rel_max(db, wdb), moments=rel_max(mom, wmom))
+    print("bnorm cfg2 vs double oracle:", d)
+    assert max(d.values()) < TOL, d
+    # distance to the float instantiation (what the reference's float CPU path returns): reported, loosely bounded
+    fdx, fdg, fdb, fmom = ob.bnorm_backward(x, g, dy, w["eps"])
+    df = dict(dzdx=rel_max(dx, fdx), dzdg=rel_max(dg, fdg), dzdb=rel_max(db, fdb), moments=rel_max(mom, fmom))
+    print("bnorm cfg2 vs float oracle:", df)
+    assert max(df.values()) < 5e-4, df
+    # size-independent invariants of the gradient, per channel
+    s = dx.astype(np.float64).sum(axis=(0, 1, 3))
+    assert np.abs(s).max() / np.abs(dx).astype(np.float64).sum(axis=(0, 1, 3)).max() < 1e-5
+
+
+def test_bottleneck_shapes(capi, ob):
+    """The two bnorm shapes of BASELINE config 4 (eps 1e-5)."""
+    for C in (64, 256):
+        w = workloads.bnorm_case(seed=20 + C, C=C, N=8, eps=1e-5)
+        x, g, dy = w["x"], w["g"], w["dy"]
+        dx, dg, db, mom = [capi.to_host(t) for t in capi.bnorm_backward(capi.to_device(x), capi.to_device(g), capi.to_device(dy), 1e-5)]
+        wdx, wdg, wdb, wmom = ob.bnorm_backward(_d(x), _d(g), _d(dy), 1e-5)
+        assert rel_max(dx, wdx) < TOL and rel_max(dg, wdg) < TOL and rel_max(db, wdb) < TOL and rel_max(mom, wmom) < TOL

@@ -1,0 +1,164 @@
+"""GPU parity, convolution (forward, backward-data, backward-filter, backward-bias) through the C ABI.
+Gate from the task: max|diff|/max|ref| <= 2e-4 in fp32 against the CPU restatement of the reference
+(im2row + sgemm per image) on the same seeded inputs."""
+import numpy as np
+import pytest
+
+from matconvnet_amd import workloads
+from util import F, rel_max
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-4
+
+# H, W, C, N, FH, FW, FC, K, stride, pad, dilate
+CASES = [
+    (8, 9, 3, 2, 3, 3, 3, 4, 1, 1, 1),
+    (9, 8, 4, 3, 3, 2, 4, 6, (2, 1), (1, 0, 2, 1), 1),
+    (12, 11, 2, 2, 3, 3, 2, 3, (2, 3), (2, 2, 1, 1), (2, 1)),
+    (7, 7, 6, 2, 1, 1, 6, 5, 1, 0, 1),
+    (10, 10, 6, 2, 3, 3, 2, 9, 1, 1, 1),                    # 3 filter groups
+    (10, 9, 4, 2, 5, 3, 2, 4, (1, 2), (2, 1, 1, 3), 1),     # 2 groups, rectangular, asymmetric pad
+    (16, 16, 8, 3, 3, 3, 8, 8, 1, (0, 2, 1, 0), 1),         # asymmetric pad, stride 1
+    (14, 14, 16, 2, 3, 3, 16, 32, 1, 1, (2, 2)),            # dilation
+    (64, 64, 8, 2, 11, 11, 8, 10, (3, 2), (5, 5, 8, 8), 1), # nnconv.m:163-202 geometry (reduced N)
+    (28, 28, 32, 4, 3, 3, 32, 48, 1, 1, 1),
+    (28, 28, 48, 3, 1, 1, 48, 24, 1, 0, 1),
+    (17, 13, 5, 3, 5, 5, 5, 7, 1, 2, 1),                    # odd everything
+    (6, 6, 3, 2, 6, 6, 3, 4, 1, 0, 1),                      # 1x1 output (the reference's FC special case)
+]
+
+
+def _tensors(case, seed=5):
+    H, W, C, N, FH, FW, FC, K, stride, pad, dilate = case
+    r = np.random.default_rng(seed)
+    x = F(r.standard_normal((H, W, C, N)))
+    f = F(r.standard_normal((FH, FW, FC, K)) / np.sqrt(FH * FW * FC))
+    b = r.standard_normal(K).astype(np.float32)
+    return x, f, b
+
+
+def _check(capi, ob, x, f, b, dy, stride, pad, dilate, tol=TOL):
+    g = capi.conv_geom(x.shape, f.shape, stride, pad, dilate)
+    og = ob.conv_geom(x.shape, f.shape, stride, pad, dilate)
+    xd, fd, dyd = capi.to_device(x), capi.to_device(f), capi.to_device(dy)
+    dx, df, db = [capi.to_host(t) for t in capi.conv_backward(xd, fd, dyd, g)]
+    wdx, wdf, wdb = ob.conv_backward(x, f, dy, og)
+    errs = dict(dzdx=rel_max(dx, wdx), dzdf=rel_max(df, wdf), dzdb=rel_max(db, wdb))
+    assert max(errs.values()) <= tol, errs
+    return errs
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_backward_vs_oracle(capi, ob, case):
+    x, f, b = _tensors(case)
+    og = ob.conv_geom(x.shape, f.shape, *case[8:])
+    dy = F(np.random.default_rng(6).standard_normal(ob.conv_out_shape(og)))
+    _check(capi, ob, x, f, b, dy, *case[8:])
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_forward_vs_oracle(capi, ob, case):
+    x, f, b = _tensors(case)
+    g = capi.conv_geom(x.shape, f.shape, *case[8:])
+    og = ob.conv_geom(x.shape, f.shape, *case[8:])
+    y = capi.to_host(capi.conv_forward(capi.to_device(x), capi.to_device(f), capi.to_device(b), g))
+    assert rel_max(y, ob.conv_forward(x, f, b, og)) <= TOL
+    # no bias, and y = outMult*y + inMult*conv
+    base = F(np.random.default_rng(7).standard_normal(y.shape))
+    y2 = capi.to_host(capi.conv_forward(capi.to_device(x), capi.to_device(f), None, g, y=capi.to_device(base), out_mult=0.5, in_mult=2.0))
+    assert rel_max(y2, ob.conv_forward(x, f, None, og, y=base.copy(order="F"), out_mult=0.5, in_mult=2.0)) <= TOL
+
+
+def test_out_mult_zero_ignores_previous_output(capi, ob):
+    case = CASES[0]
+    x, f, b = _tensors(case)
+    g = capi.conv_geom(x.shape, f.shape, *case[8:])
+    y = capi.empty(capi.conv_out_shape(g), fill=float("nan"))
+    capi.conv_forward(capi.to_device(x), capi.to_device(f), capi.to_device(b), g, y=y, out_mult=0.0)
+    assert np.isfinite(capi.to_host(y)).all()
+
+
+def test_direct_and_mfma_paths_agree(capi, ob):
+    """The general direct kernels and the MFMA implicit-GEMM kernels compute the same thing."""
+    case = (28, 28, 32, 4, 3, 3, 32, 48, 1, 1, 1)
+    x, f, b = _tensors(case)
+    g = capi.conv_geom(x.shape, f.shape, *case[8:])
+    dy = F(np.random.default_rng(6).standard_normal(capi.conv_out_shape(g)))
+    xd, fd, dyd = capi.to_device(x), capi.to_device(f), capi.to_device(dy)
+    fast = [capi.to_host(t) for t in capi.conv_backward(xd, fd, dyd, g)]
+    try:
+        capi.set_tunable("conv_force_direct", 1)
+        slow = [capi.to_host(t) for t in capi.conv_backward(xd, fd, dyd, g)]
+    finally:
+        capi.set_tunable("conv_force_direct", 0)
+    for a, w in zip(fast, slow):
+        assert rel_max(a, w) <= TOL
+
+
+def test_baseline_config1_full(capi, ob):
+    """BASELINE config 1: x 32x32x3x100, f 5x5x3x32, stride 1, pad 2 (the reference's CPU-runnable case)."""
+    w = workloads.conv_single()
+    errs = _check(capi, ob, w["x"], w["f"], w["b"], w["dy"], w["stride"], w["pad"], w["dilate"])
+    print("conv cfg1:", errs)
+    g = capi.conv_geom(w["x"].shape, w["f"].shape, w["stride"], w["pad"], w["dilate"])
+    y = capi.to_host(capi.conv_forward(capi.to_device(w["x"]), capi.to_device(w["f"]), capi.to_device(w["b"]), g))
+    assert rel_max(y, ob.conv_forward(w["x"], w["f"], w["b"], ob.conv_geom(w["x"].shape, w["f"].shape, 1, 2, 1))) <= TOL
+
+
+@pytest.mark.parametrize("which", ["1x1_256_64", "3x3_64_64", "1x1_64_256"])
+def test_baseline_config4_conv_shapes_full(capi, ob, which):
+    """The three convolutions of the ResNet-50 bottleneck at N = 32, 56x56 (BASELINE config 4)."""
+    r = np.random.default_rng(40)
+    C, K, fs, pad = {"1x1_256_64": (256, 64, 1, 0), "3x3_64_64": (64, 64, 3, 1), "1x1_64_256": (64, 256, 1, 0)}[which]
+    x = F(r.standard_normal((56, 56, C, 32), dtype=np.float32))
+    f = workloads.he_normal(r, (fs, fs, C, K))
+    dy = F(r.standard_normal((56, 56, K, 32), dtype=np.float32))
+    print(which, _check(capi, ob, x, f, None, dy, 1, pad, 1))
+
+
+def test_baseline_config5_reduced_batch(capi, ob):
+    """BASELINE config 5 geometry (56x56x256, 3x3x256x256, pad 1) at N = 2 against the oracle."""
+    w = workloads.conv_vgg(N=2)
+    print("conv cfg5 (N=2):", _check(capi, ob, w["x"], w["f"], None, w["dy"], 1, 1, 1))
+
+
+def test_baseline_config5_full_size_properties(capi, ob):
+    """BASELINE config 5 at full size (N = 64): too big for the CPU oracle in a test, so
+    (1) dzdx of single images is compared with the oracle run on those images alone (images are
+        independent in backward-data),
+    (2) dzdf / dzdb are linear in the batch: the full-batch result must equal the sum of the results on the
+        two half batches, and the first half's dzdf is checked against the oracle on a 2-image slice via
+        the same linearity (full = slice + rest)."""
+    w = workloads.conv_vgg()
+    x, f, dy = w["x"], w["f"], w["dy"]
+    N = x.shape[3]
+    g = capi.conv_geom(x.shape, f.shape, 1, 1, 1)
+    xd, fd, dyd = capi.to_device(x), capi.to_device(f), capi.to_device(dy)
+    dx, df, db = capi.conv_backward(xd, fd, dyd, g)
+    dxh = capi.to_host(dx)
+    for n in (0, N - 1):
+        og = ob.conv_geom((56, 56, 256, 1), f.shape, 1, 1, 1)
+        wdx, _, _ = ob.conv_backward(None, f, F(dy[:, :, :, n:n + 1]), og, want=(True, False, False))
+        assert rel_max(dxh[:, :, :, n:n + 1], wdx) <= TOL
+    # linearity over the batch, and an oracle anchor on a 2-image slice
+    def part(lo, hi):
+        gp = capi.conv_geom((56, 56, 256, hi - lo), f.shape, 1, 1, 1)
+        _, dfp, dbp = capi.conv_backward(capi.to_device(x[:, :, :, lo:hi]), fd, capi.to_device(dy[:, :, :, lo:hi]), gp, want=(False, True, True))
+        return capi.to_host(dfp).astype(np.float64), capi.to_host(dbp).astype(np.float64)
+    dfa, dba = part(0, 2)
+    dfb, dbb = part(2, N)
+    assert rel_max(capi.to_host(df), dfa + dfb) <= TOL and rel_max(capi.to_host(db), dba + dbb) <= TOL
+    og2 = ob.conv_geom((56, 56, 256, 2), f.shape, 1, 1, 1)
+    _, wdf, wdb = ob.conv_backward(F(x[:, :, :, 0:2]), f, F(dy[:, :, :, 0:2]), og2, want=(False, True, True))
+    assert rel_max(dfa, wdf) <= TOL and rel_max(dba, wdb) <= TOL
+
+
+def test_errors(capi):
+    with pytest.raises(capi.McnError) as e:
+        capi.conv_out_shape(capi.conv_geom((8, 8, 3, 1), (3, 3, 2, 4)))
+    assert e.value.code == capi.ILLEGAL_ARGUMENT
+    with pytest.raises(capi.McnError):
+        capi.conv_out_shape(capi.conv_geom((2, 2, 3, 1), (3, 3, 3, 4)))
+    with pytest.raises(capi.McnError):
+        capi.conv_out_shape(capi.conv_geom((8, 8, 4, 1), (3, 3, 2, 3)))  # 2 groups do not divide 3 filters

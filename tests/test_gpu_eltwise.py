@@ -1,0 +1,35 @@
+"""GPU parity of the element-wise companions (ReLU, sum, fill): bit-exact against the oracle."""
+import numpy as np
+import pytest
+
+from util import F, bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 255, 1024, 100003])
+def test_relu_add_fill(capi, ob, n):
+    r = np.random.default_rng(n)
+    x = r.standard_normal(n).astype(np.float32)
+    x[::7] = 0.0
+    if n > 4:
+        x[3] = np.nan
+        x[4] = -0.0
+    dy = r.standard_normal(n).astype(np.float32)
+    xd, dyd = capi.to_device(x), capi.to_device(dy)
+    assert bits_equal(capi.to_host(capi.relu_forward(xd)), ob.relu_forward(x))
+    assert bits_equal(capi.to_host(capi.relu_backward(xd, dyd)), ob.relu_backward(x, dy))
+    assert bits_equal(capi.to_host(capi.add(xd, dyd)), ob.add(x, dy))
+    t = capi.empty((n,))
+    capi.fill(t, 1.5)
+    assert np.array_equal(capi.to_host(t), np.full(n, 1.5, np.float32))
+
+
+def test_unaligned_views(capi, ob):
+    """Pointers that are only 4-byte aligned take the scalar path."""
+    import torch
+    base = torch.randn(1001, device="cuda")
+    x = base[1:]
+    y = torch.empty(1001, device="cuda")[1:]
+    capi.check(capi.lib().mcn_relu_forward(capi.stream(), capi.ptr(y), capi.ptr(x), x.numel()))
+    assert torch.equal(y, torch.clamp_min(x, 0))

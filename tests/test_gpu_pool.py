@@ -1,0 +1,144 @@
+"""GPU parity, pooling: the HIP kernels (through the C ABI) against the CPU oracle and the golden vectors
+from the compiled reference.  Bar: bit-exact, max AND average (tolerance stated by the task for average is
+1e-5 relative; the gather order makes it exact, so exactness is what is asserted)."""
+import os
+
+import numpy as np
+import pytest
+
+from matconvnet_amd import workloads
+from util import F, bits_equal, count_bit_mismatches
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "pool_golden.npz")
+
+GEOMS = [
+    (5, 6, 2, 3, 2, 1, 0), (5, 6, 2, 3, 3, 2, 1), (8, 8, 1, 2, 3, 3, 2), (7, 9, 3, 1, (2, 3), (1, 2), (1, 0, 2, 1)),
+    (9, 7, 2, 2, (3, 2), (2, 1), (0, 1, 1, 0)), (4, 4, 1, 1, 4, 4, 3), (6, 6, 2, 2, 2, 2, (0, 1, 0, 1)),
+    (12, 12, 2, 2, 3, 2, 1), (5, 5, 1, 1, 1, 1, 0), (10, 3, 1, 2, (5, 3), (3, 1), (2, 2, 1, 1)),
+    (28, 28, 5, 3, 3, 2, 1), (56, 56, 4, 2, 2, 2, 0), (33, 47, 3, 2, (3, 5), (2, 3), (1, 2, 4, 0)),
+    (224, 8, 2, 1, 3, 2, 1), (8, 224, 2, 1, 3, 2, 1),
+]
+
+
+def _inputs(shape, seed, mode):
+    r = np.random.default_rng(seed)
+    n = int(np.prod(shape))
+    if mode == "distinct":
+        x = r.permutation(n).astype(np.float32).reshape(shape)
+    elif mode == "ties":
+        x = r.integers(0, 3, size=shape).astype(np.float32)
+    elif mode == "special":
+        x = r.integers(0, 3, size=shape).astype(np.float32)
+        flat = x.reshape(-1)
+        flat[r.random(n) < 0.25] = np.nan
+        flat[r.random(n) < 0.25] = -np.inf
+        flat[r.random(n) < 0.05] = np.inf
+    else:
+        x = r.standard_normal(shape).astype(np.float32)
+    return F(x)
+
+
+def _run(capi, ob, x, dy, shape, pool, stride, pad, method, accumulate_into=None):
+    g = capi.pool_geom(shape, pool, stride, pad, method)
+    og = ob.pool_geom(shape, pool, stride, pad, method)
+    xd, dyd = capi.to_device(x), capi.to_device(dy)
+    if accumulate_into is None:
+        got = capi.to_host(capi.pool_backward(xd, dyd, g))
+        want = ob.pool_backward(x, dy, og)
+    else:
+        got = capi.to_host(capi.pool_backward(xd, dyd, g, dx=capi.to_device(accumulate_into)))
+        want = ob.pool_backward(x, dy, og, dx=accumulate_into.copy(order="F"))
+    return got, want
+
+
+@pytest.mark.parametrize("geom", GEOMS)
+@pytest.mark.parametrize("method", ["max", "avg"])
+@pytest.mark.parametrize("mode", ["distinct", "ties", "special", "normal"])
+def test_backward_bit_exact_small(capi, ob, geom, method, mode):
+    H, W, C, N, pool, stride, pad = geom
+    shape = (H, W, C, N)
+    og = ob.pool_geom(shape, pool, stride, pad, method)
+    x = _inputs(shape, 11, mode)
+    dy = F(np.random.default_rng(12).standard_normal(ob.pool_out_shape(og)))
+    got, want = _run(capi, ob, x, dy, shape, pool, stride, pad, method)
+    assert bits_equal(got, want), count_bit_mismatches(got, want)
+
+
+@pytest.mark.parametrize("geom", GEOMS[:8])
+@pytest.mark.parametrize("method", ["max", "avg"])
+def test_forward_bit_exact_small(capi, ob, geom, method):
+    H, W, C, N, pool, stride, pad = geom
+    shape = (H, W, C, N)
+    x = _inputs(shape, 5, "special" if method == "max" else "normal")
+    g = capi.pool_geom(shape, pool, stride, pad, method)
+    got = capi.to_host(capi.pool_forward(capi.to_device(x), g))
+    want = ob.pool_forward(x, ob.pool_geom(shape, pool, stride, pad, method))
+    assert bits_equal(got, want)
+
+
+@pytest.mark.parametrize("method", ["max", "avg"])
+def test_backward_accumulate_mode(capi, ob, method):
+    """accumulate != 0 is the vl::nn::Pooling::backward contract: derInput += ..., same addition order."""
+    shape = (12, 12, 2, 2)
+    x = _inputs(shape, 3, "ties")
+    og = ob.pool_geom(shape, 3, 2, 1, method)
+    dy = F(np.random.default_rng(4).standard_normal(ob.pool_out_shape(og)))
+    base = F(np.random.default_rng(5).standard_normal(shape))
+    got, want = _run(capi, ob, x, dy, shape, 3, 2, 1, method, accumulate_into=base)
+    assert bits_equal(got, want)
+
+
+@pytest.mark.parametrize("budget", [1024, 4096, 65536])
+def test_tile_width_does_not_change_results(capi, ob, budget):
+    """Different LDS budgets -> different tile widths (and the non-tiled fallback): identical bits."""
+    old = capi.get_tunable("pool_lds_bytes")
+    try:
+        capi.set_tunable("pool_lds_bytes", budget)
+        for method in ("max", "avg"):
+            shape = (40, 36, 3, 2)
+            x = _inputs(shape, 8, "ties")
+            og = ob.pool_geom(shape, 3, 2, 1, method)
+            dy = F(np.random.default_rng(9).standard_normal(ob.pool_out_shape(og)))
+            got, want = _run(capi, ob, x, dy, shape, 3, 2, 1, method)
+            assert bits_equal(got, want)
+    finally:
+        capi.set_tunable("pool_lds_bytes", old)
+
+
+def test_golden_vectors_from_reference(capi):
+    z = np.load(GOLDEN)
+    for i in range(int(z["count"])):
+        v = [int(t) for t in z["geom_%d" % i]]
+        g = capi.PoolGeom(*v)
+        xd, dyd = capi.to_device(z["x_%d" % i]), capi.to_device(z["dy_%d" % i])
+        assert bits_equal(capi.to_host(capi.pool_forward(xd, g)), F(z["y_%d" % i])), i
+        assert bits_equal(capi.to_host(capi.pool_backward(xd, dyd, g)), F(z["dx_%d" % i])), i
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_baseline_max_pool_full_size_bit_exact(capi, ob, ties):
+    """BASELINE config 3a: 112x112x64x32, 3x3 stride 2 pad 1, and its 8-level tie-stress variant."""
+    w = workloads.pool_max_case(ties=ties)
+    got, want = _run(capi, ob, w["x"], w["dy"], w["x"].shape, w["pool"], w["stride"], w["pad"], "max")
+    assert bits_equal(got, want), count_bit_mismatches(got, want)
+    # size-independent property: every dzdy lands on exactly one input when the window has a finite max
+    assert np.isclose(got.astype(np.float64).sum(), w["dy"].astype(np.float64).sum(), rtol=1e-6)
+
+
+def test_baseline_avg_pool_full_size_bit_exact(capi, ob):
+    """BASELINE config 3b: 56x56x256x32, 2x2 stride 2."""
+    w = workloads.pool_avg_case()
+    got, want = _run(capi, ob, w["x"], w["dy"], w["x"].shape, w["pool"], w["stride"], w["pad"], "avg")
+    assert bits_equal(got, want), count_bit_mismatches(got, want)
+
+
+def test_errors(capi):
+    g = capi.pool_geom((8, 8, 1, 1), 3, 0, 0, "max")
+    with pytest.raises(capi.McnError) as e:
+        capi.pool_out_shape(g)
+    assert e.value.code == capi.ILLEGAL_ARGUMENT
+    g = capi.pool_geom((2, 2, 1, 1), 5, 1, 0, "max")
+    with pytest.raises(capi.McnError):
+        capi.pool_out_shape(g)
