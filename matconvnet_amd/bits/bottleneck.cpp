@@ -1,0 +1,139 @@
+#include "bottleneck.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include "../../include/mcn_hip.h"
+#include "hiphelper.hpp"
+#include "nnbnorm.hpp"
+#include "nnconv.hpp"
+
+namespace vl { namespace harness {
+
+Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon)
+    : H(H), W(W), C(C), M(M), N(N), epsilon(epsilon), error(VLE_Success), stageHook(NULL), hookUser(NULL) {
+  const TensorShape big(H, W, C, N), small(H, W, M, N);
+  // inputs and parameters
+  make("x", big); make("dzdy", big);
+  make("f1", TensorShape(1, 1, C, M)); make("f2", TensorShape(3, 3, M, M)); make("f3", TensorShape(1, 1, M, C));
+  make("g1", TensorShape(M, 1, 1, 1)); make("b1", TensorShape(M, 1, 1, 1));
+  make("g2", TensorShape(M, 1, 1, 1)); make("b2", TensorShape(M, 1, 1, 1));
+  make("g3", TensorShape(C, 1, 1, 1)); make("b3", TensorShape(C, 1, 1, 1));
+  // forward activations
+  make("a1", small); make("n1", small); make("r1", small);
+  make("a2", small); make("n2", small); make("r2", small);
+  make("a3", big); make("n3", big); make("s", big); make("y", big);
+  make("m1", TensorShape(M, 2, 1, 1)); make("m2", TensorShape(M, 2, 1, 1)); make("m3", TensorShape(C, 2, 1, 1));
+  // derivatives
+  make("ds", big); make("da3", big); make("dr2", small); make("dn2", small); make("da2", small);
+  make("dr1", small); make("dn1", small); make("da1", small); make("dxm", big); make("dzdx", big);
+  make("df1", TensorShape(1, 1, C, M)); make("df2", TensorShape(3, 3, M, M)); make("df3", TensorShape(1, 1, M, C));
+  make("dg1", TensorShape(M, 1, 1, 1)); make("db1", TensorShape(M, 1, 1, 1));
+  make("dg2", TensorShape(M, 1, 1, 1)); make("db2", TensorShape(M, 1, 1, 1));
+  make("dg3", TensorShape(C, 1, 1, 1)); make("db3", TensorShape(C, 1, 1, 1));
+}
+
+Bottleneck::~Bottleneck() {
+  for (std::size_t i = 0; i < slots.size(); ++i)
+    if (slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
+}
+
+Tensor Bottleneck::make(std::string const& name, TensorShape const& shape) {
+  void* memory = NULL;
+  const std::size_t bytes = shape.getNumElements() * sizeof(float);
+  if (error == VLE_Success && hipMalloc(&memory, bytes ? bytes : 4) != hipSuccess) {
+    (void)hipGetLastError();
+    error = VLE_OutOfGPUMemeory;
+    message = "cannot allocate buffer '" + name + "'";
+    memory = NULL;
+  }
+  Slot s;
+  s.name = name;
+  s.tensor = Tensor(shape, VLDT_Float, VLDT_GPU, memory, bytes);
+  slots.push_back(s);
+  return s.tensor;
+}
+
+Tensor& Bottleneck::slot(std::string const& name) {
+  for (std::size_t i = 0; i < slots.size(); ++i)
+    if (slots[i].name == name) return slots[i].tensor;
+  static Tensor none;
+  return none;
+}
+
+float* Bottleneck::buffer(std::string const& name, std::size_t* count) {
+  Tensor& t = slot(name);
+  if (count) *count = t.getNumElements();
+  return (float*)t.getMemory();
+}
+
+ErrorCode Bottleneck::setStream(void* stream) { return context.getHipHelper().setStream(stream); }
+
+ErrorCode Bottleneck::fail(ErrorCode e, char const* where) {
+  if (e != VLE_Success) {
+    error = e;
+    message = std::string(where) + ": " + context.getLastErrorMessage();
+  }
+  return e;
+}
+
+#define STEP(stage, call)                                   \
+  do {                                                      \
+    mark(stage, 1);                                         \
+    ErrorCode e_ = (call);                                  \
+    mark(stage, 0);                                         \
+    if (e_ != VLE_Success) return fail(e_, stage);          \
+  } while (0)
+
+#define ABI(stage, call)                                                                    \
+  do {                                                                                      \
+    mark(stage, 1);                                                                         \
+    int rc_ = (call);                                                                       \
+    mark(stage, 0);                                                                         \
+    if (rc_ != 0) {                                                                         \
+      context.setError((ErrorCode)rc_, mcn_last_error_message());                           \
+      return fail((ErrorCode)rc_, stage);                                                   \
+    }                                                                                       \
+  } while (0)
+
+ErrorCode Bottleneck::forward() {
+  if (error != VLE_Success) return error;
+  void* st = context.getHipHelper().getStream();
+  Tensor none;
+  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, 1, 1, 1, 1, 1, 1, 1, 1);
+  nn::BatchNorm bn(context, epsilon);
+  const std::size_t nSmall = slot("a1").getNumElements(), nBig = slot("a3").getNumElements();
+  STEP("conv1_fwd", c1.forward(slot("a1"), 0, slot("x"), 1, slot("f1"), none));
+  STEP("bn1_fwd", bn.forward(slot("n1"), slot("m1"), slot("a1"), slot("g1"), slot("b1")));
+  ABI("relu1_fwd", mcn_relu_forward(st, buffer("r1"), buffer("n1"), nSmall));
+  STEP("conv2_fwd", c2.forward(slot("a2"), 0, slot("r1"), 1, slot("f2"), none));
+  STEP("bn2_fwd", bn.forward(slot("n2"), slot("m2"), slot("a2"), slot("g2"), slot("b2")));
+  ABI("relu2_fwd", mcn_relu_forward(st, buffer("r2"), buffer("n2"), nSmall));
+  STEP("conv3_fwd", c1.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
+  STEP("bn3_fwd", bn.forward(slot("n3"), slot("m3"), slot("a3"), slot("g3"), slot("b3")));
+  ABI("sum_fwd", mcn_add(st, buffer("s"), buffer("n3"), buffer("x"), nBig));
+  ABI("relu3_fwd", mcn_relu_forward(st, buffer("y"), buffer("s"), nBig));
+  return VLE_Success;
+}
+
+ErrorCode Bottleneck::backward() {
+  if (error != VLE_Success) return error;
+  void* st = context.getHipHelper().getStream();
+  Tensor none;
+  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, 1, 1, 1, 1, 1, 1, 1, 1);
+  nn::BatchNorm bn(context, epsilon);
+  const std::size_t nSmall = slot("a1").getNumElements(), nBig = slot("a3").getNumElements();
+  ABI("relu3_bwd", mcn_relu_backward(st, buffer("ds"), buffer("s"), buffer("dzdy"), nBig));
+  // the sum passes ds to both of its inputs: the branch (n3) and the shortcut (x)
+  STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot("ds")));
+  STEP("conv3_bwd", c1.backward(slot("dr2"), slot("df3"), none, slot("r2"), slot("f3"), slot("da3")));
+  ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer("n2"), buffer("dr2"), nSmall));
+  STEP("bn2_bwd", bn.backwardWithMoment(slot("da2"), slot("dg2"), slot("db2"), slot("m2"), slot("a2"), slot("g2"), slot("b2"), slot("dn2")));
+  STEP("conv2_bwd", c2.backward(slot("dr1"), slot("df2"), none, slot("r1"), slot("f2"), slot("da2")));
+  ABI("relu1_bwd", mcn_relu_backward(st, buffer("dn1"), buffer("n1"), buffer("dr1"), nSmall));
+  STEP("bn1_bwd", bn.backwardWithMoment(slot("da1"), slot("dg1"), slot("db1"), slot("m1"), slot("a1"), slot("g1"), slot("b1"), slot("dn1")));
+  STEP("conv1_bwd", c1.backward(slot("dxm"), slot("df1"), none, slot("x"), slot("f1"), slot("da1")));
+  ABI("sum_bwd", mcn_add(st, buffer("dzdx"), buffer("dxm"), buffer("ds"), nBig));
+  return VLE_Success;
+}
+
+} }  // namespace vl::harness

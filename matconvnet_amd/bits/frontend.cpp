@@ -1,0 +1,414 @@
+// See frontend.hpp.  Error texts are the reference drivers' own, so callers that match on them keep working.
+#include "frontend.hpp"
+
+#include <cctype>
+#include <cstdio>
+
+#include "nnbnorm.hpp"
+#include "nnconv.hpp"
+#include "nnpooling.hpp"
+
+namespace vl { namespace frontend {
+
+Arg Arg::array(Tensor const& t) {
+  Arg a;
+  a.kind = Array;
+  a.tensor = t;
+  return a;
+}
+
+Arg Arg::string(std::string const& s) {
+  Arg a;
+  a.kind = String;
+  a.text = s;
+  return a;
+}
+
+Arg Arg::numeric(std::vector<double> const& values) {
+  Arg a;
+  a.kind = Array;
+  a.owned.reset(new std::vector<double>(values));
+  std::size_t dims[2] = {values.empty() ? 0u : 1u, values.size()};
+  a.tensor = Tensor(TensorShape(dims, 2), VLDT_Double, VLDT_CPU, values.empty() ? NULL : &(*a.owned)[0],
+                    values.size() * sizeof(double));
+  return a;
+}
+
+namespace {
+
+struct Failure {
+  ErrorCode code;
+  std::string text;
+};
+
+[[noreturn]] void raise(ErrorCode code, std::string const& text) {
+  Failure f = {code, text};
+  throw f;
+}
+
+bool sameTextNoCase(std::string const& a, char const* b) {
+  std::size_t i = 0;
+  for (; i < a.size() && b[i]; ++i)
+    if (std::tolower((unsigned char)a[i]) != std::tolower((unsigned char)b[i])) return false;
+  return i == a.size() && b[i] == 0;
+}
+
+struct OptionSpec {
+  char const* name;
+  bool hasArgument;
+  int code;
+};
+
+// Walks "name, value, name, ..." like vlmxNextOption (matlab/src/bits/mexutils.h:470-562): names are
+// matched without regard to case; unknown names and missing values are errors.
+int nextOption(Arg const* in, int nin, OptionSpec const* specs, int* next, Arg const** value) {
+  if (*next >= nin) return -1;
+  Arg const& nameArg = in[*next];
+  char buffer[160];
+  if (nameArg.kind != Arg::String) {
+    std::snprintf(buffer, sizeof(buffer), "The option name is not a string (argument number %d)", *next + 1);
+    raise(VLE_IllegalArgument, buffer);
+  }
+  ++*next;
+  for (int i = 0; specs[i].name; ++i) {
+    if (!sameTextNoCase(nameArg.text, specs[i].name)) continue;
+    if (!specs[i].hasArgument) {
+      *value = NULL;
+      return specs[i].code;
+    }
+    if (*next >= nin) {
+      std::snprintf(buffer, sizeof(buffer), "Option '%s' requires an argument.", specs[i].name);
+      raise(VLE_IllegalArgument, buffer);
+    }
+    *value = &in[*next];
+    ++*next;
+    return specs[i].code;
+  }
+  raise(VLE_IllegalArgument, "Unknown option '" + nameArg.text + "'.");
+}
+
+// "plain matrix": a real, full, double host array (vlmxIsPlainMatrix).
+bool isPlainMatrix(Arg const& a) {
+  return a.kind == Arg::Array && a.tensor.getDeviceType() == VLDT_CPU && a.tensor.getDataType() == VLDT_Double &&
+         a.tensor.getNumDimensions() <= 2 && (a.tensor.getNumElements() == 0 || !a.tensor.isNull());
+}
+
+double const* values(Arg const& a) { return (double const*)a.tensor.getMemory(); }
+
+void readPair(Arg const& a, char const* NAME, int* y, int* x) {
+  if (!isPlainMatrix(a)) raise(VLE_IllegalArgument, std::string(NAME) + " is not a plain matrix.");
+  switch (a.tensor.getNumElements()) {
+    case 1: *y = *x = (int)values(a)[0]; break;
+    case 2: *y = (int)values(a)[0]; *x = (int)values(a)[1]; break;
+    default: raise(VLE_IllegalArgument, std::string(NAME) + " has neither one nor two elements.");
+  }
+}
+
+void readPad(Arg const& a, int* top, int* bottom, int* left, int* right) {
+  if (!isPlainMatrix(a)) raise(VLE_IllegalArgument, "PAD is not a plain matrix.");
+  switch (a.tensor.getNumElements()) {
+    case 1: *top = *bottom = *left = *right = (int)values(a)[0]; break;
+    case 4:
+      *top = (int)values(a)[0]; *bottom = (int)values(a)[1]; *left = (int)values(a)[2]; *right = (int)values(a)[3];
+      break;
+    default: raise(VLE_IllegalArgument, "PAD has neither one nor four elements.");
+  }
+}
+
+// Data arguments: numeric arrays of class single or double (MexTensor::init, bits/datamex.cu:339-434).
+Tensor dataTensor(Arg const& a, char const* NAME, std::size_t rank) {
+  if (a.kind != Arg::Array) raise(VLE_IllegalArgument, std::string(NAME) + " is not a numeric array.");
+  if (a.tensor.getDataType() != VLDT_Float && a.tensor.getDataType() != VLDT_Double)
+    raise(VLE_IllegalArgument, std::string(NAME) + " is neither SINGLE nor DOUBLE.");
+  Tensor t(a.tensor);
+  t.reshape(rank);
+  return t;
+}
+
+Tensor emptyMatrix(DataType type) {
+  std::size_t dims[2] = {0, 0};
+  return Tensor(TensorShape(dims, 2), type, VLDT_CPU, NULL, 0);
+}
+
+// Uninitialised output of a given shape on the device/type of the data (MexTensor::init with a shape).
+Tensor newOutput(Allocator& allocator, DeviceType device, DataType type, TensorShape const& shape) {
+  const std::size_t bytes = shape.getNumElements() * getDataTypeSizeInBytes(type);
+  void* memory = NULL;
+  if (bytes > 0) {
+    memory = allocator.allocate(device, bytes);
+    if (!memory) raise(device == VLDT_GPU ? VLE_OutOfGPUMemeory : VLE_OutOfMemory, "Could not allocate an output array.");
+  }
+  return Tensor(shape, type, device, memory, bytes);
+}
+
+void failFromContext(Context& context, ErrorCode e) {
+  if (e != VLE_Success) raise(e, context.getLastErrorMessage());
+}
+
+// ------------------------------------------------------------------------------------------ vl_nnconv
+
+void nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in) {
+  enum { optStride, optPad, optDilate, optVerbose, optNoDerData, optNoDerFilters, optNoDerBiases, optCudnn, optNoCudnn, optCudnnWs };
+  static OptionSpec const specs[] = {
+      {"Stride", true, optStride}, {"Pad", true, optPad}, {"Dilate", true, optDilate}, {"Verbose", false, optVerbose},
+      {"NoDerData", false, optNoDerData}, {"NoDerFilters", false, optNoDerFilters}, {"NoderBiases", false, optNoDerBiases},
+      {"Cudnn", false, optCudnn}, {"NoCudnn", false, optNoCudnn}, {"CudnnWorkSpaceLimit", true, optCudnnWs}, {NULL, false, 0}};
+  int strideX = 1, strideY = 1, padLeft = 0, padRight = 0, padTop = 0, padBottom = 0, dilateX = 1, dilateY = 1;
+  bool wantDerData = true, wantDerFilters = true, wantDerBiases = true;
+
+  if (nin < 3) raise(VLE_IllegalArgument, "There are less than three arguments.");
+  int next = 4;
+  bool backMode;
+  if (nin > 3 && in[3].kind == Arg::String) {
+    next = 3;
+    backMode = false;
+  } else {
+    backMode = nin >= 4;
+  }
+  int opt;
+  Arg const* value = NULL;
+  while ((opt = nextOption(in, nin, specs, &next, &value)) >= 0) {
+    switch (opt) {
+      case optStride: readPair(*value, "STRIDE", &strideY, &strideX); break;
+      case optPad: readPad(*value, &padTop, &padBottom, &padLeft, &padRight); break;
+      case optDilate: readPair(*value, "DILATE", &dilateY, &dilateX); break;
+      case optNoDerData: wantDerData = false; break;
+      case optNoDerFilters: wantDerFilters = false; break;
+      case optNoDerBiases: wantDerBiases = false; break;
+      default: break;  // Verbose and the cuDNN switches have nothing to act on here
+    }
+  }
+
+  Tensor data = dataTensor(in[0], "DATA", 4);
+  Tensor filters = dataTensor(in[1], "FILTERS", 4);
+  Tensor biases = dataTensor(in[2], "BIASES", in[2].tensor.getNumDimensions());
+  Tensor derOutput;
+  if (backMode) derOutput = dataTensor(in[3], "DEROUTPUT", 4);
+  const bool hasFilters = !filters.isEmpty(), hasBiases = !biases.isEmpty();
+
+  if (hasFilters && !areCompatible(data, filters)) raise(VLE_IllegalArgument, "DATA and FILTERS do not have compatible formats.");
+  if (hasBiases && !areCompatible(data, biases)) raise(VLE_IllegalArgument, "DATA and BIASES do not have compatible formats.");
+  if (backMode && !areCompatible(data, derOutput)) raise(VLE_IllegalArgument, "DATA and DEROUTPUT do not have compatible formats.");
+  if (strideX < 1 || strideY < 1) raise(VLE_IllegalArgument, "At least one element of STRIDE is smaller than one.");
+  if (padLeft < 0 || padRight < 0 || padTop < 0 || padBottom < 0) raise(VLE_IllegalArgument, "An element of PAD is negative.");
+  if (dilateY < 1 || dilateX < 1) raise(VLE_IllegalArgument, "An element of DILATE is less than one.");
+  if (!hasFilters && (dilateY != 1 || dilateX != 1)) raise(VLE_IllegalArgument, "There are no filters and DILATE is not one.");
+  if (!hasFilters)
+    raise(VLE_Unsupported, "Empty FILTERS (subsampling with bias) are not implemented by this library.");
+
+  TensorShape filtersShape(filters);
+  if (filtersShape.getHeight() == 0 || filtersShape.getWidth() == 0 || filtersShape.getDepth() == 0)
+    raise(VLE_IllegalArgument, "A dimension of FILTERS is void.");
+  const long extentY = ((long)filters.getHeight() - 1) * dilateY + 1, extentX = ((long)filters.getWidth() - 1) * dilateX + 1;
+  if ((long)data.getHeight() + (padTop + padBottom) < extentY || (long)data.getWidth() + (padLeft + padRight) < extentX)
+    raise(VLE_IllegalArgument, "FILTERS are larger than the DATA (including padding).");
+  const std::size_t groups = data.getDepth() / filters.getDepth();
+  if (groups * filters.getDepth() != data.getDepth()) raise(VLE_IllegalArgument, "The FILTERS depth does not divide the DATA depth.");
+  if (groups == 0 || filters.getSize() % groups != 0)
+    raise(VLE_IllegalArgument, "The number of filter groups does not divide the number of filters.");
+
+  TensorShape outputShape(((long)data.getHeight() + (padTop + padBottom) - extentY) / strideY + 1,
+                          ((long)data.getWidth() + (padLeft + padRight) - extentX) / strideX + 1, filters.getSize(),
+                          data.getSize());
+  if (backMode && (TensorShape(derOutput) != outputShape))
+    raise(VLE_IllegalArgument, "DEROUTPUT dimensions are incompatible with X and FILTERS.");
+  if (hasBiases && biases.getNumElements() != filtersShape.getSize())
+    raise(VLE_IllegalArgument, "The number of elements of BIASES is not the same as the number of filters.");
+
+  const DeviceType device = data.getDeviceType();
+  const DataType type = data.getDataType();
+  nn::Convolution op(context, strideY, strideX, padTop, padBottom, padLeft, padRight, dilateY, dilateX);
+  if (!backMode) {
+    Tensor output = newOutput(allocator, device, type, outputShape);
+    Tensor noBias;
+    failFromContext(context, op.forward(output, 0, data, 1, filters, hasBiases ? biases : noBias));
+    out[0] = output;
+    return;
+  }
+  Tensor derData, derFilters, derBiases;
+  if (wantDerData) derData = newOutput(allocator, device, type, data.getShape());
+  if (wantDerFilters) derFilters = newOutput(allocator, device, type, filters.getShape());
+  if (wantDerBiases && hasBiases) derBiases = newOutput(allocator, device, type, biases.getShape());
+  failFromContext(context, op.backward(derData, derFilters, derBiases, data, filters, derOutput));
+  const DataType outType = derOutput.getDataType();
+  out[0] = wantDerData ? derData : emptyMatrix(outType);
+  if (nout > 1) out[1] = wantDerFilters ? derFilters : emptyMatrix(outType);
+  if (nout > 2) out[2] = (wantDerBiases && hasBiases) ? derBiases : emptyMatrix(outType);
+}
+
+// ----------------------------------------------------------------------------------------- vl_nnbnorm
+
+void nnbnorm(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in) {
+  enum { optVerbose, optEpsilon, optMoments, optCudnn, optNoCudnn };
+  static OptionSpec const specs[] = {{"Verbose", false, optVerbose}, {"Epsilon", true, optEpsilon}, {"Moments", true, optMoments},
+                                     {"Cudnn", false, optCudnn}, {"NoCudnn", false, optNoCudnn}, {NULL, false, 0}};
+  double epsilon = 1e-4;
+  if (nin < 3) raise(VLE_IllegalArgument, "The arguments are less than three.");
+  int next = 4;
+  bool backMode;
+  if (nin > 3 && in[3].kind == Arg::String) {
+    next = 3;
+    backMode = false;
+  } else {
+    backMode = nin >= 4;
+  }
+  const bool returnMoments = backMode ? (nout > 3) : (nout > 1);
+  Arg const* momentsArg = NULL;
+  int opt;
+  Arg const* value = NULL;
+  while ((opt = nextOption(in, nin, specs, &next, &value)) >= 0) {
+    switch (opt) {
+      case optEpsilon:
+        if (!isPlainMatrix(*value) || value->tensor.getNumElements() != 1) raise(VLE_IllegalArgument, "EPSILON is not a plain scalar.");
+        epsilon = values(*value)[0];
+        break;
+      case optMoments: momentsArg = value; break;
+      default: break;
+    }
+  }
+  const bool givenMoments = momentsArg != NULL;
+
+  Tensor data = dataTensor(in[0], "DATA", 4);
+  Tensor multipliers = dataTensor(in[1], "MULTIPLIERS", 1);
+  Tensor biases = dataTensor(in[2], "BIASES", 1);
+  Tensor derOutput, moments;
+  if (backMode) derOutput = dataTensor(in[3], "DEROUTPUT", 4);
+  if (givenMoments) moments = dataTensor(*momentsArg, "MOMENTS", 2);
+
+  if (!areCompatible(data, multipliers)) raise(VLE_IllegalArgument, "DATA and MULTIPLIERS do not have compatible formats.");
+  if (!areCompatible(data, biases)) raise(VLE_IllegalArgument, "DATA and BIASES do not have compatible formats.");
+  if (backMode && !areCompatible(data, derOutput)) raise(VLE_IllegalArgument, "DATA and DEROUTPUT do not have compatible formats.");
+  if (backMode && (data.getShape() != derOutput.getShape())) raise(VLE_IllegalArgument, "DATA and DEROUTPUT do not have the same size.");
+  if (givenMoments && !areCompatible(data, moments)) raise(VLE_IllegalArgument, "DATA and MOMENTS do not have compatible formats.");
+  if (multipliers.getHeight() != data.getDepth()) raise(VLE_IllegalArgument, "The MULTIPLIERS size does not match the DATA depth.");
+  if (biases.getHeight() != data.getDepth()) raise(VLE_IllegalArgument, "The BIASES size does not match the DATA depth.");
+  if (givenMoments && moments.getNumElements() != 2 * data.getDepth())
+    raise(VLE_IllegalArgument, "The MOMENTS size does not match the DATA depth.");
+
+  const DeviceType device = data.getDeviceType();
+  const DataType type = data.getDataType();
+  if (returnMoments && !givenMoments) moments = newOutput(allocator, device, type, TensorShape(data.getDepth(), 2, 1, 1));
+
+  nn::BatchNorm op(context, epsilon);
+  if (!backMode) {
+    Tensor output = newOutput(allocator, device, type, data.getShape());
+    failFromContext(context, givenMoments ? op.forwardWithMoment(output, moments, data, multipliers, biases)
+                                          : op.forward(output, moments, data, multipliers, biases));
+    out[0] = output;
+    if (nout > 1 && moments) out[1] = moments;
+    return;
+  }
+  // derivatives of the parameters keep the shape the parameters were passed with
+  Tensor derData = newOutput(allocator, device, type, data.getShape());
+  Tensor derMultipliers = newOutput(allocator, device, type, in[1].tensor.getShape());
+  Tensor derBiases = newOutput(allocator, device, type, in[2].tensor.getShape());
+  failFromContext(context, givenMoments
+                               ? op.backwardWithMoment(derData, derMultipliers, derBiases, moments, data, multipliers, biases, derOutput)
+                               : op.backward(derData, derMultipliers, derBiases, moments, data, multipliers, biases, derOutput));
+  out[0] = derData;
+  if (nout > 1) out[1] = derMultipliers;
+  if (nout > 2) out[2] = derBiases;
+  if (nout > 3 && moments) out[3] = moments;
+}
+
+// ------------------------------------------------------------------------------------------ vl_nnpool
+
+void nnpool(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in) {
+  enum { optStride, optPad, optMethod, optVerbose, optCudnn, optNoCudnn };
+  static OptionSpec const specs[] = {{"Stride", true, optStride}, {"Pad", true, optPad}, {"Method", true, optMethod},
+                                     {"Verbose", false, optVerbose}, {"CUDNN", false, optCudnn}, {"NoCUDNN", false, optNoCudnn},
+                                     {NULL, false, 0}};
+  int poolWidth = 0, poolHeight = 0, strideX = 1, strideY = 1, padLeft = 0, padRight = 0, padTop = 0, padBottom = 0;
+  nn::Pooling::Method method = nn::Pooling::Max;
+  if (nin < 2) raise(VLE_IllegalArgument, "The arguments are less than two.");
+  int next = 3;
+  bool backMode;
+  if (nin > 2 && in[2].kind == Arg::String) {
+    next = 2;
+    backMode = false;
+  } else {
+    backMode = nin >= 3;
+  }
+  int opt;
+  Arg const* value = NULL;
+  while ((opt = nextOption(in, nin, specs, &next, &value)) >= 0) {
+    switch (opt) {
+      case optStride: readPair(*value, "STRIDE", &strideY, &strideX); break;
+      case optPad: readPad(*value, &padTop, &padBottom, &padLeft, &padRight); break;
+      case optMethod:
+        if (value->kind != Arg::String) raise(VLE_IllegalArgument, "METHOD is not a string.");
+        if (sameTextNoCase(value->text, "max")) method = nn::Pooling::Max;
+        else if (sameTextNoCase(value->text, "avg")) method = nn::Pooling::Average;
+        else raise(VLE_IllegalArgument, "METHOD is not a supported method.");
+        break;
+      default: break;
+    }
+  }
+  Tensor data = dataTensor(in[0], "DATA", 4);
+  Tensor derOutput;
+  if (backMode) derOutput = dataTensor(in[2], "DEROUTPUT", 4);
+  if (backMode && !areCompatible(data, derOutput)) raise(VLE_IllegalArgument, "DATA and DEROUTPUT do not have compatible formats.");
+  if (!isPlainMatrix(in[1])) raise(VLE_IllegalArgument, "SIZE is not a plain matrix.");
+  switch (in[1].tensor.getNumElements()) {
+    case 1: poolHeight = poolWidth = (int)values(in[1])[0]; break;
+    case 2: poolHeight = (int)values(in[1])[0]; poolWidth = (int)values(in[1])[1]; break;
+    default: raise(VLE_IllegalArgument, "SIZE has neither one nor two elements.");
+  }
+  if (strideX < 1 || strideY < 1) raise(VLE_IllegalArgument, "At least one element of STRIDE is smaller than one.");
+  if (poolHeight == 0 || poolWidth == 0) raise(VLE_IllegalArgument, "A dimension of the pooling SIZE is void.");
+  if ((long)data.getHeight() + (padTop + padBottom) < poolHeight || (long)data.getWidth() + (padLeft + padRight) < poolWidth)
+    raise(VLE_IllegalArgument, "The pooling window is larger than the DATA (including padding).");
+  if (padLeft < 0 || padRight < 0 || padTop < 0 || padBottom < 0) raise(VLE_IllegalArgument, "An element of PAD is negative.");
+  if (padLeft >= poolWidth || padRight >= poolWidth || padTop >= poolHeight || padBottom >= poolHeight)
+    raise(VLE_IllegalArgument, "A padding value is larger or equal to the size of the pooling window.");
+  TensorShape outputShape(((long)data.getHeight() + (padTop + padBottom) - poolHeight) / strideY + 1,
+                          ((long)data.getWidth() + (padLeft + padRight) - poolWidth) / strideX + 1, data.getDepth(),
+                          data.getSize());
+  if (backMode && (TensorShape(derOutput) != outputShape))
+    raise(VLE_IllegalArgument, "DEROUTPUT dimensions are incompatible with X and POOL.");
+
+  const DeviceType device = data.getDeviceType();
+  const DataType type = data.getDataType();
+  nn::Pooling op(context, poolHeight, poolWidth, strideY, strideX, padTop, padBottom, padLeft, padRight, method);
+  if (!backMode) {
+    Tensor output = newOutput(allocator, device, type, outputShape);
+    failFromContext(context, op.forward(output, data));
+    out[0] = output;
+  } else {
+    // The MEX driver zero-fills dzdx and lets the operator add into it (vl_nnpool.cu:255-259); the gather
+    // kernel can write every element itself, which saves that pass over dzdx.
+    Tensor derData = newOutput(allocator, device, type, data.getShape());
+    failFromContext(context, op.backwardOverwrite(derData, data, derOutput));
+    out[0] = derData;
+  }
+  (void)nout;
+}
+
+typedef void (*Body)(Context&, Allocator&, int, Tensor*, int, Arg const*);
+
+ErrorCode guarded(Body body, Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
+                  std::string& message) {
+  message.clear();
+  context.resetLastError();
+  try {
+    body(context, allocator, nout, out, nin, in);
+  } catch (Failure const& f) {
+    message = f.text;
+    return f.code;
+  }
+  return VLE_Success;
+}
+
+}  // namespace
+
+ErrorCode vl_nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
+  return guarded(nnconv, context, allocator, nout, out, nin, in, message);
+}
+ErrorCode vl_nnbnorm(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
+  return guarded(nnbnorm, context, allocator, nout, out, nin, in, message);
+}
+ErrorCode vl_nnpool(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
+  return guarded(nnpool, context, allocator, nout, out, nin, in, message);
+}
+
+} }  // namespace vl::frontend

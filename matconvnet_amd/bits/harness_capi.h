@@ -1,0 +1,55 @@
+/* C entry points onto the C++ operator layer, for callers without a C++ compiler at hand (ctypes, other
+ * FFIs) and for the stand-alone bench.  Not part of the reference interface: it stands where MATLAB's
+ * mexFunction call mechanism stands in the reference. */
+#ifndef MCN_AMD_HARNESS_CAPI_H
+#define MCN_AMD_HARNESS_CAPI_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VLH_API __attribute__((visibility("default")))
+
+/* one argument / one result of a front-end call */
+typedef struct vlh_arg {
+  int kind;        /* 0 = numeric array, 1 = string */
+  void* data;      /* array memory (device or host) */
+  int device;      /* 0 = host (VLDT_CPU), 1 = HIP device (VLDT_GPU) */
+  int dtype;       /* 1 = float, 2 = double (vl::DataType) */
+  int ndims;
+  size_t dims[8];
+  const char* text; /* kind == 1 */
+} vlh_arg;
+
+typedef void* (*vlh_alloc_fn)(void* user, int device, size_t bytes);
+
+/* function: "vl_nnconv" | "vl_nnbnorm" | "vl_nnpool".  `out` must have room for 4 entries.  Returns a
+   vl::ErrorCode; vlh_last_message() has the text. */
+VLH_API int vlh_call(const char* function, int nout, vlh_arg* out, int nin, const vlh_arg* in, vlh_alloc_fn alloc,
+                     void* user, void* stream);
+VLH_API const char* vlh_last_message(void);
+
+/* direct calls of the operator classes (device fp32 tensors, MATLAB-shaped H x W x C x N) */
+VLH_API int vlh_pooling_backward(void* stream, float* derInput, const float* input, const float* derOutput, int H,
+                                 int W, int C, int N, int poolH, int poolW, int strideY, int strideX, int padTop,
+                                 int padBottom, int padLeft, int padRight, int method, int overwrite);
+VLH_API int vlh_cpu_tensor_is_refused(void);
+
+/* ResNet bottleneck block */
+VLH_API void* vlh_bottleneck_create(int H, int W, int C, int M, int N, double epsilon);
+VLH_API void vlh_bottleneck_destroy(void* block);
+VLH_API float* vlh_bottleneck_buffer(void* block, const char* name, size_t* count);
+VLH_API int vlh_bottleneck_set_stream(void* block, void* stream);
+VLH_API int vlh_bottleneck_forward(void* block);
+VLH_API int vlh_bottleneck_backward(void* block);
+/* runs `steps` forward+backward passes; if stage != NULL the launches of that stage are bracketed by HIP
+   events and *stage_ms receives their mean duration */
+VLH_API int vlh_bottleneck_run(void* block, int steps, const char* stage, float* stage_ms);
+VLH_API const char* vlh_bottleneck_message(void* block);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,193 @@
+// Stand-alone bench of the operator layer: no MATLAB, no Python.  Drives vl::nn::Convolution / BatchNorm /
+// Pooling (HIP device tensors) and the bottleneck block on the benchmark configurations with seeded
+// synthetic inputs, times them with HIP events and prints TFLOP/s, GB/s and images/s beside the
+// fraction of the MI355X rooflines (fp32 matrix 157.3 TFLOP/s, HBM 8 TB/s).
+//
+//   mcn_bench [--iters K] [--warmup W] [--only conv5|bnorm|maxpool|avgpool|block|conv1]
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include <hip/hip_runtime_api.h>
+
+#include "bottleneck.hpp"
+#include "hiphelper.hpp"
+#include "nnbnorm.hpp"
+#include "nnconv.hpp"
+#include "nnpooling.hpp"
+
+using namespace vl;
+
+static const double kPeakMfma = 157.3e12, kPeakHbm = 8.0e12;
+
+#define HIP_OK(call)                                                                  \
+  do {                                                                                \
+    hipError_t e_ = (call);                                                           \
+    if (e_ != hipSuccess) {                                                           \
+      std::fprintf(stderr, "%s failed: %s\n", #call, hipGetErrorString(e_));          \
+      std::exit(2);                                                                   \
+    }                                                                                 \
+  } while (0)
+
+struct DeviceTensor {
+  Tensor view;
+  DeviceTensor(TensorShape const& shape) {
+    void* p = NULL;
+    HIP_OK(hipMalloc(&p, std::max<size_t>(shape.getNumElements(), 1) * sizeof(float)));
+    view = Tensor(shape, VLDT_Float, VLDT_GPU, p, shape.getNumElements() * sizeof(float));
+  }
+  ~DeviceTensor() { (void)hipFree(view.getMemory()); }
+  void randn(unsigned seed, float scale = 1.f, float shift = 0.f) {
+    std::mt19937_64 gen(seed);
+    std::normal_distribution<float> dist(0.f, 1.f);
+    std::vector<float> host(view.getNumElements());
+    for (size_t i = 0; i < host.size(); ++i) host[i] = shift + scale * dist(gen);
+    HIP_OK(hipMemcpy(view.getMemory(), host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice));
+  }
+  void fill(float v) {
+    std::vector<float> host(view.getNumElements(), v);
+    HIP_OK(hipMemcpy(view.getMemory(), host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice));
+  }
+};
+
+template <typename F>
+static double medianMs(F&& body, int warmup, int iters) {
+  hipEvent_t a, b;
+  HIP_OK(hipEventCreate(&a));
+  HIP_OK(hipEventCreate(&b));
+  for (int i = 0; i < warmup; ++i) body();
+  HIP_OK(hipDeviceSynchronize());
+  std::vector<float> ms(iters);
+  for (int i = 0; i < iters; ++i) {
+    HIP_OK(hipEventRecord(a, 0));
+    body();
+    HIP_OK(hipEventRecord(b, 0));
+    HIP_OK(hipEventSynchronize(b));
+    HIP_OK(hipEventElapsedTime(&ms[i], a, b));
+  }
+  std::sort(ms.begin(), ms.end());
+  hipEventDestroy(a);
+  hipEventDestroy(b);
+  return ms[iters / 2];
+}
+
+static void check(Context& ctx, ErrorCode e, char const* what) {
+  if (e != VLE_Success) {
+    std::fprintf(stderr, "%s: %s\n", what, ctx.getLastErrorMessage().c_str());
+    std::exit(3);
+  }
+}
+
+static void benchConv(char const* name, int H, int W, int C, int N, int F, int K, int pad, int warmup, int iters) {
+  Context ctx;
+  DeviceTensor x(TensorShape(H, W, C, N)), f(TensorShape(F, F, C, K)), dy(TensorShape(H, W, K, N));
+  DeviceTensor dx(TensorShape(H, W, C, N)), df(TensorShape(F, F, C, K)), db(TensorShape(K, 1, 1, 1));
+  x.randn(1);
+  f.randn(2, std::sqrt(2.f / (F * F * C)));
+  dy.randn(3);
+  nn::Convolution op(ctx, 1, 1, pad, pad, pad, pad, 1, 1);
+  Tensor none;
+  const double flops = 2.0 * H * W * (double)F * F * C * K * N;
+  double tData = medianMs([&] { check(ctx, op.backward(dx.view, none, none, none, f.view, dy.view), name); }, warmup, iters);
+  double tFilt = medianMs([&] { check(ctx, op.backward(none, df.view, none, x.view, none, dy.view), name); }, warmup, iters);
+  double tBias = medianMs([&] { check(ctx, op.backward(none, none, db.view, none, none, dy.view), name); }, warmup, iters);
+  double tAll = medianMs([&] { check(ctx, op.backward(dx.view, df.view, db.view, x.view, f.view, dy.view), name); }, warmup, iters);
+  std::printf("%-28s bwd-data %8.3f ms %6.1f TFLOP/s (%4.1f%%) | bwd-filter %8.3f ms %6.1f TFLOP/s (%4.1f%%) | bias %6.1f us | all three %8.3f ms %6.1f TFLOP/s (%4.1f%% of fp32 MFMA peak)\n",
+              name, tData, flops / tData / 1e9, 100 * flops / (tData * 1e-3) / kPeakMfma, tFilt, flops / tFilt / 1e9,
+              100 * flops / (tFilt * 1e-3) / kPeakMfma, tBias * 1e3, tAll, 2 * flops / tAll / 1e9,
+              100 * 2 * flops / (tAll * 1e-3) / kPeakMfma);
+}
+
+static void benchBnorm(int warmup, int iters) {
+  const int H = 56, W = 56, C = 256, N = 32;
+  Context ctx;
+  DeviceTensor x(TensorShape(H, W, C, N)), dy(TensorShape(H, W, C, N)), dx(TensorShape(H, W, C, N));
+  DeviceTensor g(TensorShape(C, 1, 1, 1)), b(TensorShape(C, 1, 1, 1)), dg(TensorShape(C, 1, 1, 1)), db(TensorShape(C, 1, 1, 1)), m(TensorShape(C, 2, 1, 1));
+  x.randn(4, 1.3f, 0.5f);
+  dy.randn(5);
+  g.fill(1.f);
+  b.fill(0.f);
+  nn::BatchNorm op(ctx, 1e-4);
+  const double bytes = 5.0 * H * W * C * N * 4;
+  double t = medianMs([&] { check(ctx, op.backward(dx.view, dg.view, db.view, m.view, x.view, g.view, b.view, dy.view), "bnorm"); }, warmup, iters);
+  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; 5 tensor sweeps = %.1f MB)\n", "bnorm bwd 56x56x256x32", t * 1e3,
+              bytes / t / 1e6, 100 * bytes / (t * 1e-3) / kPeakHbm, bytes / 1e6);
+}
+
+static void benchPool(bool isMax, int warmup, int iters) {
+  const int H = isMax ? 112 : 56, C = isMax ? 64 : 256, N = 32, P = isMax ? 3 : 2, pad = isMax ? 1 : 0;
+  const int OH = (H + 2 * pad - P) / 2 + 1;
+  Context ctx;
+  DeviceTensor x(TensorShape(H, H, C, N)), dy(TensorShape(OH, OH, C, N)), dx(TensorShape(H, H, C, N));
+  x.randn(6);
+  dy.randn(7);
+  nn::Pooling op(ctx, P, P, 2, 2, pad, pad, pad, pad, isMax ? nn::Pooling::Max : nn::Pooling::Average);
+  const double e = (double)H * H * C * N * 4, o = (double)OH * OH * C * N * 4;
+  const double bytes = isMax ? (2 * e + o) : (e + o);
+  double t = medianMs([&] { check(ctx, op.backwardOverwrite(dx.view, x.view, dy.view), "pool"); }, warmup, iters);
+  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; %.1f MB)\n", isMax ? "max-pool bwd 112x112x64x32" : "avg-pool bwd 56x56x256x32",
+              t * 1e3, bytes / t / 1e6, 100 * bytes / (t * 1e-3) / kPeakHbm, bytes / 1e6);
+}
+
+static void benchBlock(int warmup, int iters) {
+  const int H = 56, W = 56, C = 256, M = 64, N = 32;
+  harness::Bottleneck block(H, W, C, M, N, 1e-5);
+  if (!block.ok()) {
+    std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
+    std::exit(3);
+  }
+  std::mt19937_64 gen(8);
+  std::normal_distribution<float> dist(0.f, 1.f);
+  auto upload = [&](char const* name, float scale, float constant, bool random) {
+    size_t n = 0;
+    float* p = block.buffer(name, &n);
+    std::vector<float> host(n);
+    for (size_t i = 0; i < n; ++i) host[i] = random ? scale * dist(gen) : constant;
+    HIP_OK(hipMemcpy(p, host.data(), n * sizeof(float), hipMemcpyHostToDevice));
+  };
+  upload("x", 1, 0, true);
+  upload("dzdy", 1, 0, true);
+  upload("f1", std::sqrt(2.f / C), 0, true);
+  upload("f2", std::sqrt(2.f / (9 * M)), 0, true);
+  upload("f3", std::sqrt(2.f / M), 0, true);
+  for (char const* g : {"g1", "g2", "g3"}) upload(g, 0, 1.f, false);
+  for (char const* b : {"b1", "b2", "b3"}) upload(b, 0, 0.f, false);
+  double t = medianMs([&] {
+    if (block.forward() != VLE_Success || block.backward() != VLE_Success) {
+      std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
+      std::exit(3);
+    }
+  }, warmup, iters);
+  std::printf("%-28s %8.3f ms/step %9.0f images/s (fwd+bwd, N = %d, 41.93 GFLOP of convolution per step)\n",
+              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N);
+}
+
+int main(int argc, char** argv) {
+  int iters = 20, warmup = 3;
+  std::string only;
+  for (int i = 1; i < argc; ++i) {
+    if (!std::strcmp(argv[i], "--iters") && i + 1 < argc) iters = std::atoi(argv[++i]);
+    else if (!std::strcmp(argv[i], "--warmup") && i + 1 < argc) warmup = std::atoi(argv[++i]);
+    else if (!std::strcmp(argv[i], "--only") && i + 1 < argc) only = argv[++i];
+    else {
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--only conv5|conv1|bnorm|maxpool|avgpool|block]\n");
+      return 1;
+    }
+  }
+  hipDeviceProp_t prop;
+  HIP_OK(hipGetDeviceProperties(&prop, 0));
+  std::printf("device: %s, %d CUs, %.0f MHz\n", prop.name, prop.multiProcessorCount, prop.clockRate / 1000.0);
+  auto want = [&](char const* k) { return only.empty() || only == k; };
+  if (want("conv1")) benchConv("conv 5x5x3x32 on 32x32x3x100", 32, 32, 3, 100, 5, 32, 2, warmup, iters);
+  if (want("bnorm")) benchBnorm(warmup, iters);
+  if (want("maxpool")) benchPool(true, warmup, iters);
+  if (want("avgpool")) benchPool(false, warmup, iters);
+  if (want("block")) benchBlock(warmup, iters);
+  if (want("conv5")) benchConv("conv 3x3x256x256 56x56 N=64", 56, 56, 256, 64, 3, 256, 1, warmup, iters);
+  return 0;
+}

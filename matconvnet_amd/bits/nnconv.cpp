@@ -1,0 +1,118 @@
+// vl::nn::Convolution on the HIP device.  Where the reference loops over images calling im2row and a BLAS
+// GEMM (matlab/src/bits/nnconv.cu:71-317), each product here is one call into the C ABI, which runs an
+// implicit-GEMM kernel over the whole batch.
+#include "nnconv.hpp"
+
+#include "impl/dispatcher.hpp"
+
+using namespace vl;
+using namespace vl::nn;
+using namespace vl::impl;
+
+Convolution::Convolution(Context& context, int strideY, int strideX, int padTop, int padBottom, int padLeft,
+                         int padRight, int dilateY, int dilateX)
+    : context(context), strideY(strideY), strideX(strideX), padTop(padTop), padBottom(padBottom), padLeft(padLeft),
+      padRight(padRight), dilateY(dilateY), dilateX(dilateX) {}
+
+namespace {
+
+mcn_conv_geom geometry(Convolution const& op, TensorShape const& data, TensorShape const& filter) {
+  mcn_conv_geom g;
+  g.H = asInt(data.getHeight()); g.W = asInt(data.getWidth()); g.C = asInt(data.getDepth()); g.N = asInt(data.getSize());
+  g.FH = asInt(filter.getHeight()); g.FW = asInt(filter.getWidth()); g.FC = asInt(filter.getDepth()); g.K = asInt(filter.getSize());
+  g.strideY = op.strideY; g.strideX = op.strideX;
+  g.padTop = op.padTop; g.padBottom = op.padBottom; g.padLeft = op.padLeft; g.padRight = op.padRight;
+  g.dilateY = op.dilateY; g.dilateX = op.dilateX;
+  return g;
+}
+
+// Scratch from the context, sized by the back-end; NULL with an error recorded when it cannot be had.
+bool scratch(Context& context, mcn_conv_geom const& g, int product, void** ws, size_t* bytes) {
+  *bytes = mcn_conv_workspace_bytes(&g, product);
+  *ws = NULL;
+  if (*bytes == 0) return true;
+  *ws = context.getWorkspace(VLDT_GPU, *bytes);
+  return *ws != NULL;
+}
+
+}  // namespace
+
+ErrorCode Convolution::forward(Tensor& output, double outputMult, Tensor const& input, double inputMult,
+                               Tensor const& filter, Tensor const& bias) {
+  tensor_type tt = findTensorType(output, input, filter, bias);
+  ErrorCode e = requireHipFloat(context, tt, "Convolution::forward");
+  if (e != VLE_Success) return e;
+  if (!output || !input || !filter)
+    return context.setError(VLE_IllegalArgument, "Convolution::forward: OUTPUT, INPUT and FILTER are required");
+  mcn_conv_geom g = geometry(*this, input, filter);
+  int oh = 0, ow = 0;
+  int rc = mcn_conv_output_size(&g, &oh, &ow);
+  if (rc) return fromAbi(context, rc, "Convolution::forward");
+  if ((int)output.getHeight() != oh || (int)output.getWidth() != ow || output.getDepth() != filter.getSize() ||
+      output.getSize() != input.getSize())
+    return context.setError(VLE_IllegalArgument, "Convolution::forward: OUTPUT dimensions are incompatible with X and FILTERS");
+  if (bias && bias.getNumElements() != filter.getSize())
+    return context.setError(VLE_IllegalArgument, "Convolution::forward: the number of elements of BIASES is not the number of filters");
+  void* ws;
+  size_t bytes;
+  if (!scratch(context, g, MCN_CONV_FORWARD, &ws, &bytes)) return context.getLastError();
+  rc = mcn_conv_forward(context.getHipHelper().getStream(), &g, (float*)output.getMemory(), (float)outputMult,
+                        (float const*)input.getMemory(), (float)inputMult, (float const*)filter.getMemory(),
+                        (float const*)bias.getMemory(), ws, bytes);
+  return fromAbi(context, rc, "Convolution::forward");
+}
+
+ErrorCode Convolution::backward(Tensor& derInput, Tensor& derFilter, Tensor& derBias, Tensor const& input,
+                                Tensor const& filter, Tensor const& derOutput) {
+  tensor_type tt = findTensorType(derInput, derFilter, derBias, input, filter, derOutput);
+  ErrorCode e = requireHipFloat(context, tt, "Convolution::backward");
+  if (e != VLE_Success) return e;
+  if (!derOutput) return context.setError(VLE_IllegalArgument, "Convolution::backward: DEROUTPUT is required");
+  void* stream = context.getHipHelper().getStream();
+  void* ws;
+  size_t bytes;
+  int rc;
+
+  if (derBias) {
+    // only the extent of DEROUTPUT matters: describe it as a 1x1 convolution over itself
+    TensorShape unit(1, 1, derOutput.getDepth(), derOutput.getDepth());
+    Convolution plain(context, 1, 1, 0, 0, 0, 0, 1, 1);
+    mcn_conv_geom g = geometry(plain, derOutput, unit);
+    if (derBias.getNumElements() != derOutput.getDepth())
+      return context.setError(VLE_IllegalArgument, "Convolution::backward: DERBIASES has the wrong number of elements");
+    if (!scratch(context, g, MCN_CONV_BACKWARD_BIAS, &ws, &bytes)) return context.getLastError();
+    rc = mcn_conv_backward_bias(stream, &g, (float*)derBias.getMemory(), (float const*)derOutput.getMemory(), ws, bytes);
+    if (rc) return fromAbi(context, rc, "Convolution::backward");
+  }
+
+  if (derInput) {
+    if (!filter) return context.setError(VLE_IllegalArgument, "Convolution::backward: FILTER is required for DERINPUT");
+    mcn_conv_geom g = geometry(*this, derInput, filter);
+    int oh = 0, ow = 0;
+    rc = mcn_conv_output_size(&g, &oh, &ow);
+    if (rc) return fromAbi(context, rc, "Convolution::backward");
+    if ((int)derOutput.getHeight() != oh || (int)derOutput.getWidth() != ow || derOutput.getDepth() != filter.getSize() ||
+        derOutput.getSize() != derInput.getSize())
+      return context.setError(VLE_IllegalArgument, "Convolution::backward: DEROUTPUT dimensions are incompatible with X and FILTERS");
+    if (!scratch(context, g, MCN_CONV_BACKWARD_DATA, &ws, &bytes)) return context.getLastError();
+    rc = mcn_conv_backward_data(stream, &g, (float*)derInput.getMemory(), (float const*)filter.getMemory(),
+                                (float const*)derOutput.getMemory(), ws, bytes);
+    if (rc) return fromAbi(context, rc, "Convolution::backward");
+  }
+
+  if (derFilter) {
+    if (!input) return context.setError(VLE_IllegalArgument, "Convolution::backward: INPUT is required for DERFILTER");
+    mcn_conv_geom g = geometry(*this, input, derFilter);
+    int oh = 0, ow = 0;
+    rc = mcn_conv_output_size(&g, &oh, &ow);
+    if (rc) return fromAbi(context, rc, "Convolution::backward");
+    if ((int)derOutput.getHeight() != oh || (int)derOutput.getWidth() != ow || derOutput.getDepth() != derFilter.getSize() ||
+        derOutput.getSize() != input.getSize())
+      return context.setError(VLE_IllegalArgument, "Convolution::backward: DEROUTPUT dimensions are incompatible with X and FILTERS");
+    if (!scratch(context, g, MCN_CONV_BACKWARD_FILTER, &ws, &bytes)) return context.getLastError();
+    rc = mcn_conv_backward_filter(stream, &g, (float*)derFilter.getMemory(), (float const*)input.getMemory(),
+                                  (float const*)derOutput.getMemory(), ws, bytes);
+    if (rc) return fromAbi(context, rc, "Convolution::backward");
+  }
+  return VLE_Success;
+}

@@ -1,0 +1,35 @@
+// vl::nn::Convolution -- same class interface as matlab/src/bits/nnconv.hpp:23-52.
+#ifndef MCN_AMD_BITS_NNCONV_HPP
+#define MCN_AMD_BITS_NNCONV_HPP
+
+#include "data.hpp"
+
+namespace vl { namespace nn {
+
+class Convolution {
+ public:
+  Convolution(Context& context, int strideY, int strideX, int padTop, int padBottom, int padLeft, int padRight,
+              int dilateY, int dilateX);
+
+  // output = outputMult*output + inputMult*conv(input, filter) + bias.  `bias` may be a null tensor.
+  vl::ErrorCode forward(vl::Tensor& output, double outputMult, vl::Tensor const& input, double inputMult,
+                        vl::Tensor const& filter, vl::Tensor const& bias);
+
+  // Any of derInput / derFilter / derBias may be a null tensor, meaning "do not compute".  The ones given
+  // are fully overwritten.  `input` is needed for derFilter, `filter` for derInput.
+  vl::ErrorCode backward(vl::Tensor& derInput, vl::Tensor& derFilter, vl::Tensor& derBias, vl::Tensor const& input,
+                         vl::Tensor const& filter, vl::Tensor const& derOutput);
+
+  Context& context;
+  int strideY;
+  int strideX;
+  int padTop;
+  int padBottom;
+  int padLeft;
+  int padRight;
+  int dilateY;
+  int dilateX;
+};
+
+} }  // namespace vl::nn
+#endif

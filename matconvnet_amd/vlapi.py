@@ -1,0 +1,218 @@
+"""ctypes binding of the C++ operator layer (libmcn_vl.so): the MATLAB-style entry points
+
+    y                        = vl_nnconv(x, f, b, 'pad', p, 'stride', s, ...)
+    dzdx, dzdf, dzdb         = vl_nnconv(x, f, b, dzdy, ...)
+    y[, moments]             = vl_nnbnorm(x, g, b, 'epsilon', e[, 'moments', m])
+    dzdx, dzdg, dzdb[, mom]  = vl_nnbnorm(x, g, b, dzdy, ...)
+    y / dzdx                 = vl_nnpool(x, pool[, dzdy], 'stride', s, 'pad', p, 'method', 'max'|'avg')
+
+Arguments follow the MEX drivers (matlab/src/vl_nnconv.cu, vl_nnbnorm.cu, vl_nnpool.cu): data arguments are
+torch CUDA tensors standing for MATLAB arrays -- a MATLAB array of size H x W x C x N is a contiguous
+tensor of shape (N, C, W, H) -- option names are case-insensitive strings, option values are numbers or
+sequences.  Errors raise VlError carrying the reference's message text.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmcn_vl.so")
+
+
+class VlError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("vl error %d: %s" % (code, message))
+        self.code = code
+        self.message = message
+
+
+class Arg(C.Structure):
+    _fields_ = [("kind", C.c_int), ("data", C.c_void_p), ("device", C.c_int), ("dtype", C.c_int),
+                ("ndims", C.c_int), ("dims", C.c_size_t * 8), ("text", C.c_char_p)]
+
+
+ALLOC_FN = C.CFUNCTYPE(C.c_void_p, C.c_void_p, C.c_int, C.c_size_t)
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("%s is missing: build it with `python -m matconvnet_amd.build`" % LIB_PATH)
+        L = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+        L.vlh_call.restype = C.c_int
+        L.vlh_call.argtypes = [C.c_char_p, C.c_int, C.POINTER(Arg), C.c_int, C.POINTER(Arg), ALLOC_FN, C.c_void_p, C.c_void_p]
+        L.vlh_last_message.restype = C.c_char_p
+        L.vlh_pooling_backward.restype = C.c_int
+        L.vlh_pooling_backward.argtypes = [C.c_void_p] * 4 + [C.c_int] * 14
+        L.vlh_cpu_tensor_is_refused.restype = C.c_int
+        L.vlh_bottleneck_create.restype = C.c_void_p
+        L.vlh_bottleneck_create.argtypes = [C.c_int] * 5 + [C.c_double]
+        L.vlh_bottleneck_destroy.argtypes = [C.c_void_p]
+        L.vlh_bottleneck_buffer.restype = C.c_void_p
+        L.vlh_bottleneck_buffer.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_size_t)]
+        L.vlh_bottleneck_set_stream.argtypes = [C.c_void_p, C.c_void_p]
+        L.vlh_bottleneck_forward.argtypes = [C.c_void_p]
+        L.vlh_bottleneck_backward.argtypes = [C.c_void_p]
+        L.vlh_bottleneck_run.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.POINTER(C.c_float)]
+        L.vlh_bottleneck_message.restype = C.c_char_p
+        L.vlh_bottleneck_message.argtypes = [C.c_void_p]
+        _lib = L
+    return _lib
+
+
+def _torch():
+    import torch
+    return torch
+
+
+def _array_arg(value, keep):
+    """torch tensor (device or host), numpy array or number(s) -> Arg."""
+    torch = _torch()
+    a = Arg()
+    a.kind = 0
+    a.text = None
+    if isinstance(value, torch.Tensor):
+        t = value.contiguous()
+        keep.append(t)
+        mshape = list(reversed(t.shape))
+        a.data = t.data_ptr() if t.numel() else None
+        a.device = 1 if t.is_cuda else 0
+        a.dtype = {torch.float32: 1, torch.float64: 2}.get(t.dtype, 0)
+    else:  # host option value: MATLAB passes double row vectors
+        v = np.atleast_1d(np.asarray(value, dtype=np.float64)).ravel()
+        keep.append(v)
+        mshape = [1, v.size] if v.size else [0, 0]
+        a.data = v.ctypes.data if v.size else None
+        a.device = 0
+        a.dtype = 2
+    a.ndims = len(mshape)
+    for i, d in enumerate(mshape):
+        a.dims[i] = int(d)
+    return a
+
+
+def _call(function, nout, args):
+    torch = _torch()
+    L = lib()
+    keep = []
+    cargs = (Arg * max(len(args), 1))()
+    for i, v in enumerate(args):
+        if isinstance(v, str):
+            cargs[i].kind = 1
+            b = v.encode()
+            keep.append(b)
+            cargs[i].text = b
+        else:
+            cargs[i] = _array_arg(v, keep)
+    allocated = {}
+
+    def alloc(user, device, nbytes):
+        try:
+            t = torch.empty(int(nbytes), dtype=torch.uint8, device="cuda" if device else "cpu")
+        except RuntimeError:
+            return None
+        allocated[t.data_ptr()] = t
+        return t.data_ptr()
+
+    cb = ALLOC_FN(alloc)
+    out = (Arg * 4)()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream) if torch.cuda.is_available() else None
+    rc = L.vlh_call(function.encode(), nout, out, len(args), cargs, cb, None, stream)
+    if rc != 0:
+        raise VlError(rc, L.vlh_last_message().decode())
+    results = []
+    for i in range(max(nout, 1)):
+        o = out[i]
+        mshape = [int(o.dims[k]) for k in range(o.ndims)]
+        while len(mshape) > 2 and mshape[-1] == 1:  # MATLAB drops trailing singleton dimensions
+            mshape.pop()
+        if not o.data:
+            results.append(torch.empty(tuple(reversed(mshape)) if mshape else (0,), dtype=torch.float32))
+            continue
+        raw = allocated[o.data]
+        dt = torch.float32 if o.dtype == 1 else torch.float64
+        results.append(raw.view(dt).view(tuple(reversed(mshape))))
+    return results
+
+
+def vl_nnconv(*args, nout=None):
+    back = len(args) > 3 and not isinstance(args[3], str)
+    n = nout if nout is not None else (3 if back else 1)
+    r = _call("vl_nnconv", n, list(args))
+    return r[0] if n == 1 else tuple(r[:n])
+
+
+def vl_nnbnorm(*args, nout=None):
+    back = len(args) > 3 and not isinstance(args[3], str)
+    n = nout if nout is not None else (3 if back else 1)
+    r = _call("vl_nnbnorm", n, list(args))
+    return r[0] if n == 1 else tuple(r[:n])
+
+
+def vl_nnpool(*args):
+    return _call("vl_nnpool", 1, list(args))[0]
+
+
+class Bottleneck:
+    """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
+
+    def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5):
+        self.L = lib()
+        self.shape = (H, W, Cc, M, N)
+        self.h = self.L.vlh_bottleneck_create(H, W, Cc, M, N, eps)
+        torch = _torch()
+        self.L.vlh_bottleneck_set_stream(self.h, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    def close(self):
+        if self.h:
+            self.L.vlh_bottleneck_destroy(self.h)
+            self.h = None
+
+    def _buf(self, name):
+        n = C.c_size_t(0)
+        p = self.L.vlh_bottleneck_buffer(self.h, name.encode(), C.byref(n))
+        if not p:
+            raise KeyError(name)
+        return p, n.value
+
+    def set(self, name, array):
+        """Upload a MATLAB-shaped numpy array (any order) into the named buffer."""
+        torch = _torch()
+        p, n = self._buf(name)
+        host = np.ascontiguousarray(np.asfortranarray(array, dtype=np.float32).T).ravel()
+        assert host.size == n, (name, host.size, n)
+        src = torch.from_numpy(host).cuda()
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        assert hip.hipMemcpy(p, src.data_ptr(), n * 4, 3) == 0  # device to device
+        torch.cuda.synchronize()
+
+    def get(self, name, mshape):
+        torch = _torch()
+        p, n = self._buf(name)
+        dst = torch.empty(n, dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        assert hip.hipMemcpy(dst.data_ptr(), p, n * 4, 3) == 0
+        torch.cuda.synchronize()
+        return np.asfortranarray(dst.cpu().numpy().reshape(tuple(reversed(mshape))).T)
+
+    def _check(self, rc):
+        if rc != 0:
+            raise VlError(rc, self.L.vlh_bottleneck_message(self.h).decode())
+
+    def forward(self):
+        self._check(self.L.vlh_bottleneck_forward(self.h))
+
+    def backward(self):
+        self._check(self.L.vlh_bottleneck_backward(self.h))
+
+    def run(self, steps, stage=None):
+        ms = C.c_float(0.0)
+        self._check(self.L.vlh_bottleneck_run(self.h, steps, stage.encode() if stage else None, C.byref(ms)))
+        return ms.value

@@ -1,0 +1,284 @@
+"""The C++ operator layer (vl::nn classes + MEX-convention front-end) on the GPU, driven the way the
+reference's own tests drive vl_nnconv / vl_nnbnorm / vl_nnpool (matlab/xtest/suite/nnconv.m, nnbnorm.m,
+nnpool.m), checked against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from matconvnet_amd import workloads
+from util import F, bits_equal, rel_max
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def vl():
+    from matconvnet_amd import vlapi
+    vlapi.lib()
+    return vlapi
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(np.asfortranarray(a, dtype=np.float32).T)).cuda()
+
+
+def host(t):
+    return np.asfortranarray(t.detach().cpu().numpy().T)
+
+
+def test_vl_nnconv_forward_backward(vl, ob):
+    r = np.random.default_rng(1)
+    x = F(r.standard_normal((14, 12, 6, 3)))
+    f = F(r.standard_normal((3, 3, 6, 8)) * 0.2)
+    b = r.standard_normal(8).astype(np.float32)
+    g = ob.conv_geom(x.shape, f.shape, (1, 1), (1, 0, 2, 1), 1)
+    y = vl.vl_nnconv(dev(x), dev(f), dev(b), "pad", [1, 0, 2, 1])
+    want = ob.conv_forward(x, f, b, g)
+    assert tuple(reversed(y.shape)) == want.shape
+    assert rel_max(host(y), want) < 2e-4
+    dy = F(r.standard_normal(want.shape))
+    dx, df, db = vl.vl_nnconv(dev(x), dev(f), dev(b), dev(dy), "Pad", [1, 0, 2, 1], "STRIDE", 1)
+    wdx, wdf, wdb = ob.conv_backward(x, f, dy, g)
+    assert rel_max(host(dx), wdx) < 2e-4 and rel_max(host(df), wdf) < 2e-4 and rel_max(host(db).ravel(), wdb) < 2e-4
+    assert tuple(reversed(df.shape)) == f.shape
+
+
+def test_vl_nnconv_skipped_outputs_and_empty_bias(vl, ob):
+    r = np.random.default_rng(2)
+    x = F(r.standard_normal((9, 9, 4, 2)))
+    f = F(r.standard_normal((3, 3, 4, 5)))
+    dy = F(r.standard_normal((7, 7, 5, 2)))
+    empty = torch.empty((0,), dtype=torch.float32, device="cuda")
+    dx, df, db = vl.vl_nnconv(dev(x), dev(f), empty, dev(dy), "NoDerData")
+    assert dx.numel() == 0 and db.numel() == 0 and df.numel() == f.size
+    g = ob.conv_geom(x.shape, f.shape, 1, 0, 1)
+    assert rel_max(host(df), ob.conv_backward(x, f, dy, g)[1]) < 2e-4
+
+
+def test_vl_nnconv_validation_messages(vl):
+    x = torch.zeros((2, 4, 8, 8), device="cuda")   # MATLAB 8x8x4x2
+    f = torch.zeros((5, 4, 3, 3), device="cuda")   # 3x3x4x5
+    b = torch.zeros((5,), device="cuda")
+    cases = [
+        (("stride", 0), "At least one element of STRIDE is smaller than one."),
+        (("pad", -1), "An element of PAD is negative."),
+        (("pad", [1, 2, 3]), "PAD has neither one nor four elements."),
+        (("dilate", 0), "An element of DILATE is less than one."),
+        (("bogus", 1), "Unknown option 'bogus'."),
+        (("stride",), "Option 'Stride' requires an argument."),
+    ]
+    for opts, message in cases:
+        with pytest.raises(vl.VlError) as e:
+            vl.vl_nnconv(x, f, b, *opts)
+        assert e.value.message == message, e.value.message
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(x, torch.zeros((5, 3, 3, 3), device="cuda"), b)
+    assert e.value.message == "The FILTERS depth does not divide the DATA depth."
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(x, torch.zeros((5, 4, 9, 9), device="cuda"), b)
+    assert e.value.message == "FILTERS are larger than the DATA (including padding)."
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(x, f, b, torch.zeros((2, 5, 5, 5), device="cuda"))
+    assert e.value.message == "DEROUTPUT dimensions are incompatible with X and FILTERS."
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(x, f, torch.zeros((4,), device="cuda"))
+    assert e.value.message == "The number of elements of BIASES is not the same as the number of filters."
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(x, f)
+    assert e.value.message == "There are less than three arguments."
+
+
+def test_cpu_tensors_are_refused_not_silently_computed(vl):
+    assert vl.lib().vlh_cpu_tensor_is_refused() == 1
+    assert b"HIP" in vl.lib().vlh_last_message()
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnpool(torch.zeros((1, 1, 4, 4)), 2)
+    assert e.value.code == 1  # VLE_Unsupported
+
+
+def test_vl_nnbnorm_modes(vl, ob):
+    w = workloads.bnorm_case(seed=3, H=13, W=17, C=4, N=7)
+    x, g, b, dy = w["x"], w["g"], w["b"], w["dy"]
+    d = lambda a: F(a, np.float64) if a.ndim > 1 else a.astype(np.float64)
+    y, mom = vl.vl_nnbnorm(dev(x), dev(g), dev(b), nout=2)
+    wy, wmom = ob.bnorm_forward(d(x), d(g), d(b), 1e-4)
+    assert tuple(reversed(mom.shape)) == (4, 2)
+    assert rel_max(host(y), wy) < 1e-5 and rel_max(host(mom), wmom) < 1e-5
+    dx, dg, db, mom2 = vl.vl_nnbnorm(dev(x), dev(g), dev(b), dev(dy), "epsilon", 1e-3, nout=4)
+    wdx, wdg, wdb, wmom2 = ob.bnorm_backward(d(x), d(g), d(dy), 1e-3)
+    assert rel_max(host(dx), wdx) < 1e-5 and rel_max(host(dg).ravel(), wdg) < 1e-5
+    assert rel_max(host(db).ravel(), wdb) < 1e-5 and rel_max(host(mom2), wmom2) < 1e-5
+    # 'moments' given = batch moments reproduces the batch mode (nnbnorm.m:53-79)
+    dx2, dg2, db2 = vl.vl_nnbnorm(dev(x), dev(g), dev(b), dev(dy), "epsilon", 1e-3, "moments", mom2)
+    assert rel_max(host(dx2), wdx) < 1e-5 and rel_max(host(dg2).ravel(), wdg) < 1e-5
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnbnorm(dev(x), dev(g[:3]), dev(b))
+    assert e.value.message == "The MULTIPLIERS size does not match the DATA depth."
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnbnorm(dev(x), dev(g), dev(b), dev(dy[:, :, :, :3]))
+    assert e.value.message == "DATA and DEROUTPUT do not have the same size."
+
+
+@pytest.mark.parametrize("method", ["max", "avg"])
+def test_vl_nnpool(vl, ob, method):
+    r = np.random.default_rng(4)
+    x = F(r.integers(0, 4, size=(12, 14, 3, 2)).astype(np.float32))
+    g = ob.pool_geom(x.shape, (3, 2), (2, 1), (1, 0, 0, 1), method)
+    y = vl.vl_nnpool(dev(x), [3, 2], "stride", [2, 1], "pad", [1, 0, 0, 1], "method", method)
+    assert bits_equal(host(y), ob.pool_forward(x, g))
+    dy = F(r.standard_normal(ob.pool_out_shape(g)))
+    dx = vl.vl_nnpool(dev(x), [3, 2], dev(dy), "stride", [2, 1], "pad", [1, 0, 0, 1], "METHOD", method.upper())
+    assert bits_equal(host(dx), ob.pool_backward(x, dy, g))
+
+
+def test_vl_nnpool_validation_messages(vl):
+    x = torch.zeros((1, 1, 8, 8), device="cuda")
+    for args, message in [
+        ((3, "pad", 3), "A padding value is larger or equal to the size of the pooling window."),
+        ((0,), "A dimension of the pooling SIZE is void."),
+        ((9,), "The pooling window is larger than the DATA (including padding)."),
+        ((2, "method", "median"), "METHOD is not a supported method."),
+        ((2, "stride", [1, 0]), "At least one element of STRIDE is smaller than one."),
+        (([1, 2, 3],), "SIZE has neither one nor two elements."),
+    ]:
+        with pytest.raises(vl.VlError) as e:
+            vl.vl_nnpool(x, *args)
+        assert e.value.message == message, e.value.message
+
+
+def test_pooling_class_accumulates_like_the_reference(vl, ob):
+    """vl::nn::Pooling::backward adds into derInput (callers zero it); backwardOverwrite does not read it."""
+    import ctypes as C
+    r = np.random.default_rng(5)
+    x = F(r.integers(0, 3, size=(10, 10, 2, 2)).astype(np.float32))
+    g = ob.pool_geom(x.shape, 3, 2, 1, "max")
+    dy = F(r.standard_normal(ob.pool_out_shape(g)))
+    base = F(r.standard_normal(x.shape))
+    xd, dyd = dev(x), dev(dy)
+    for overwrite in (0, 1):
+        dx = dev(base)
+        rc = vl.lib().vlh_pooling_backward(C.c_void_p(torch.cuda.current_stream().cuda_stream), C.c_void_p(dx.data_ptr()),
+                                           C.c_void_p(xd.data_ptr()), C.c_void_p(dyd.data_ptr()), 10, 10, 2, 2, 3, 3, 2, 2, 1, 1, 1, 1, 0, overwrite)
+        assert rc == 0
+        want = ob.pool_backward(x, dy, g) if overwrite else ob.pool_backward(x, dy, g, dx=base.copy(order="F"))
+        assert bits_equal(host(dx), want)
+
+
+def _oracle_bottleneck(ob, w, dtype):
+    """The block composed from oracle operators, DagNN order."""
+    c = lambda a: F(a, dtype) if a.ndim > 1 else a.astype(dtype)
+    x, dy = c(w["x"]), c(w["dy"])
+    f1, f2, f3 = c(w["f1"]), c(w["f2"]), c(w["f3"])
+    eps = w["eps"]
+    g1 = ob.conv_geom(x.shape, f1.shape, 1, 0, 1)
+    a1 = ob.conv_forward(x, f1, None, g1)
+    n1, m1 = ob.bnorm_forward(a1, c(w["g1"]), c(w["b1"]), eps)
+    r1 = ob.relu_forward(n1)
+    g2 = ob.conv_geom(r1.shape, f2.shape, 1, 1, 1)
+    a2 = ob.conv_forward(r1, f2, None, g2)
+    n2, m2 = ob.bnorm_forward(a2, c(w["g2"]), c(w["b2"]), eps)
+    r2 = ob.relu_forward(n2)
+    g3 = ob.conv_geom(r2.shape, f3.shape, 1, 0, 1)
+    a3 = ob.conv_forward(r2, f3, None, g3)
+    n3, m3 = ob.bnorm_forward(a3, c(w["g3"]), c(w["b3"]), eps)
+    s = ob.add(n3, x)
+    y = ob.relu_forward(s)
+    ds = ob.relu_backward(s, dy)
+    da3, dg3, db3, _ = ob.bnorm_backward(a3, c(w["g3"]), ds, eps, moments=m3)
+    dr2, df3, _ = ob.conv_backward(r2, f3, da3, g3, want=(True, True, False))
+    dn2 = ob.relu_backward(n2, dr2)
+    da2, dg2, db2, _ = ob.bnorm_backward(a2, c(w["g2"]), dn2, eps, moments=m2)
+    dr1, df2, _ = ob.conv_backward(r1, f2, da2, g2, want=(True, True, False))
+    dn1 = ob.relu_backward(n1, dr1)
+    da1, dg1, db1, _ = ob.bnorm_backward(a1, c(w["g1"]), dn1, eps, moments=m1)
+    dxm, df1, _ = ob.conv_backward(x, f1, da1, g1, want=(True, True, False))
+    dx = ob.add(dxm, ds)
+    return dict(y=y, dzdx=dx, df1=df1, df2=df2, df3=df3, dg1=dg1, db1=db1, dg2=dg2, db2=db2, dg3=dg3, db3=db3)
+
+
+def _load(blk, w):
+    for k in ("x", "f1", "f2", "f3", "g1", "b1", "g2", "b2", "g3", "b3"):
+        blk.set(k, w[k])
+    blk.set("dzdy", w["dy"])
+
+
+def test_bottleneck_block_end_to_end_small_batch(vl, ob):
+    """ResNet-50 bottleneck fwd+bwd at N = 2 against the block composed from oracle operators (double).
+    Block-level gate 5e-4 on every output (three stacked layers of 2e-4 / 1e-5 operators)."""
+    w = workloads.bottleneck_case(N=2)
+    blk = vl.Bottleneck(N=2, eps=w["eps"])
+    try:
+        _load(blk, w)
+        blk.forward()
+        blk.backward()
+        want = _oracle_bottleneck(ob, w, np.float64)
+        shapes = dict(y=w["x"].shape, dzdx=w["x"].shape, df1=w["f1"].shape, df2=w["f2"].shape, df3=w["f3"].shape,
+                      dg1=(64,), db1=(64,), dg2=(64,), db2=(64,), dg3=(256,), db3=(256,))
+        errs = {k: rel_max(blk.get(k, shapes[k]), want[k]) for k in shapes}
+        print("bottleneck N=2:", {k: "%.1e" % v for k, v in errs.items()})
+        assert max(errs.values()) < 5e-4, errs
+    finally:
+        blk.close()
+
+
+def test_bottleneck_block_full_config_stage_by_stage(vl, ob):
+    """BASELINE config 4 at its full size (N = 32, 56x56, 256/64 channels).  ReLU's derivative is
+    discontinuous, so an end-to-end comparison of gradients at this size flips a handful of masks between any
+    two float implementations and says nothing about either.  Instead every stage of the GPU block is
+    checked against the oracle applied to the SAME inputs (the GPU's own intermediate buffers): wiring,
+    shapes and each operator at its real size.  Gates: conv 2e-4 (float oracle), bnorm 1e-5 (double oracle on
+    the float inputs), relu / sum bit-exact.  The forward output y, which is continuous in everything, is
+    also compared end to end."""
+    N = 32
+    w = workloads.bottleneck_case(N=N)
+    blk = vl.Bottleneck(N=N, eps=w["eps"])
+    try:
+        _load(blk, w)
+        blk.forward()
+        blk.backward()
+        big, small = (56, 56, 256, N), (56, 56, 64, N)
+        shp = dict(a1=small, n1=small, r1=small, a2=small, n2=small, r2=small, a3=big, n3=big, s=big, y=big,
+                   m1=(64, 2), m2=(64, 2), m3=(256, 2), ds=big, da3=big, dr2=small, dn2=small, da2=small,
+                   dr1=small, dn1=small, da1=small, dxm=big, dzdx=big, df1=w["f1"].shape, df2=w["f2"].shape,
+                   df3=w["f3"].shape, dg1=(64,), db1=(64,), dg2=(64,), db2=(64,), dg3=(256,), db3=(256,))
+        G = {k: blk.get(k, v) for k, v in shp.items()}
+        x, dy, eps = w["x"], w["dy"], w["eps"]
+        d = lambda a: F(a, np.float64) if a.ndim > 1 else a.astype(np.float64)
+        g1 = ob.conv_geom(x.shape, w["f1"].shape, 1, 0, 1)
+        g2 = ob.conv_geom(small, w["f2"].shape, 1, 1, 1)
+        g3 = ob.conv_geom(small, w["f3"].shape, 1, 0, 1)
+        errs = {}
+        # forward
+        errs["a1"] = rel_max(G["a1"], ob.conv_forward(x, w["f1"], None, g1))
+        errs["a2"] = rel_max(G["a2"], ob.conv_forward(G["r1"], w["f2"], None, g2))
+        errs["a3"] = rel_max(G["a3"], ob.conv_forward(G["r2"], w["f3"], None, g3))
+        for i, (a, n, m, gk, bk) in enumerate([("a1", "n1", "m1", "g1", "b1"), ("a2", "n2", "m2", "g2", "b2"), ("a3", "n3", "m3", "g3", "b3")]):
+            wy, wm = ob.bnorm_forward(d(G[a]), d(w[gk]), d(w[bk]), eps)
+            errs[n] = rel_max(G[n], wy)
+            errs[m] = rel_max(G[m], wm)
+        assert bits_equal(G["r1"], ob.relu_forward(G["n1"])) and bits_equal(G["r2"], ob.relu_forward(G["n2"]))
+        assert bits_equal(G["s"], ob.add(G["n3"], x)) and bits_equal(G["y"], ob.relu_forward(G["s"]))
+        # backward
+        assert bits_equal(G["ds"], ob.relu_backward(G["s"], dy))
+        for (da, dg, db, a, m, gk, dyk) in [("da3", "dg3", "db3", "a3", "m3", "g3", "ds"), ("da2", "dg2", "db2", "a2", "m2", "g2", "dn2"),
+                                            ("da1", "dg1", "db1", "a1", "m1", "g1", "dn1")]:
+            wdx, wdg, wdb, _ = ob.bnorm_backward(d(G[a]), d(w[gk]), d(G[dyk]), eps, moments=d(G[m]))
+            errs[da], errs[dg], errs[db] = rel_max(G[da], wdx), rel_max(G[dg], wdg), rel_max(G[db], wdb)
+        wdx, wdf, _ = ob.conv_backward(G["r2"], w["f3"], G["da3"], g3, want=(True, True, False))
+        errs["dr2"], errs["df3"] = rel_max(G["dr2"], wdx), rel_max(G["df3"], wdf)
+        assert bits_equal(G["dn2"], ob.relu_backward(G["n2"], G["dr2"]))
+        wdx, wdf, _ = ob.conv_backward(G["r1"], w["f2"], G["da2"], g2, want=(True, True, False))
+        errs["dr1"], errs["df2"] = rel_max(G["dr1"], wdx), rel_max(G["df2"], wdf)
+        assert bits_equal(G["dn1"], ob.relu_backward(G["n1"], G["dr1"]))
+        wdx, wdf, _ = ob.conv_backward(x, w["f1"], G["da1"], g1, want=(True, True, False))
+        errs["dxm"], errs["df1"] = rel_max(G["dxm"], wdx), rel_max(G["df1"], wdf)
+        assert bits_equal(G["dzdx"], ob.add(G["dxm"], G["ds"]))
+        print("bottleneck N=32 stage errors:", {k: "%.1e" % v for k, v in errs.items()})
+        for k, v in errs.items():
+            gate = 1e-5 if k[0] in "nm" or k[:2] in ("da", "dg", "db") else 2e-4
+            assert v <= gate, (k, v, gate)
+        # end to end, forward only
+        want_y = _oracle_bottleneck(ob, w, np.float32)["y"]
+        assert rel_max(G["y"], want_y) < 2e-4
+    finally:
+        blk.close()
