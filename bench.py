@@ -1,0 +1,263 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X back-end on the reference's headline configurations.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one forward+backward pass of the ResNet-50 bottleneck block (BASELINE configs[3]: 56x56, 256/64
+channels, N = 32, fp32) through the C++ operator layer, with every tensor resident in HBM before the timed
+region.  `value` is images/s over exactly K steps.  The same line carries
+  roofline      the kernel that takes most of the step, timed live with HIP events on its launch stream,
+  rooflines     the graded kernels on their own configurations: conv backward (configs[4], fp32 MFMA),
+                batch-norm backward (configs[1], HBM), max/avg pooling backward (configs[2], HBM),
+  cpu_baseline  the CPU restatement of the reference path (oracle/) timed on this machine's host cores.
+One GPU only: nothing here shards.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_FP32 = 157.3e12  # FLOP/s, MI355X dense fp32 matrix
+PEAK_HBM = 8.0e12          # B/s
+
+
+def _sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def kernel_time(capi, kernel, launch, reps):
+    """Mean duration (s) of `kernel` over `reps` calls of `launch`, from HIP events bracketing each launch."""
+    capi.profile_begin(kernel)
+    for _ in range(reps):
+        launch()
+    n, ms = capi.profile_end()
+    return (ms / n) * 1e-3 if n else float("nan"), n
+
+
+def bench_block(vlapi, capi, workloads, steps, warmup):
+    w = workloads.bottleneck_case()
+    N = w["x"].shape[3]
+    blk = vlapi.Bottleneck(N=N, eps=w["eps"])
+    for k in ("x", "f1", "f2", "f3", "g1", "b1", "g2", "b2", "g3", "b3"):
+        blk.set(k, w[k])
+    blk.set("dzdy", w["dy"])
+    blk.run(warmup)
+    _sync()
+    t0 = time.perf_counter()
+    blk.run(steps)
+    _sync()
+    dt = time.perf_counter() - t0
+    # which kernel family dominates the step, and its live duration
+    P = 56 * 56
+    conv_flops = {  # per launch family per step: forward + backward-data launches of conv_pix_mfma
+        "conv_pix_mfma": 2.0 * (2.0 * P * N * (256 * 64 + 9 * 64 * 64 + 64 * 256)),
+        "conv_wgrad_mfma": 2.0 * P * N * (256 * 64 + 9 * 64 * 64 + 64 * 256),
+    }
+    eS, eB = 4.0 * P * 64 * N, 4.0 * P * 256 * N
+    hbm_bytes = {  # algorithmic bytes per step of the memory-bound families (reads + writes once each)
+        "bnorm_sums": (eS + eS + eB) + 2 * (eS + eS + eB),       # forward reads x; backward reads x and dzdy
+        "bnorm_forward_apply": 2 * (eS + eS + eB),
+        "bnorm_backward_apply": 3 * (eS + eS + eB),
+        "eltwise_kernel": (2 * eS) * 2 + 3 * eB + 2 * eB + 3 * eB + (3 * eS) * 2 + 3 * eB,
+    }
+    fam = {}
+    for name in list(conv_flops) + list(hbm_bytes) + ["conv_wgrad_reduce", "conv_pack_weights"]:
+        capi.profile_begin(name)
+        blk.run(steps)
+        n, ms = capi.profile_end()
+        fam[name] = (n, ms * 1e-3)
+    blk.close()
+    top = max(fam, key=lambda k: fam[k][1])
+    n, total = fam[top]
+    if top in conv_flops:
+        achieved = conv_flops[top] * steps / total
+        roof = dict(kernel=top, bound="mfma", achieved=achieved / 1e12, peak=PEAK_MFMA_FP32 / 1e12, unit="TFLOP/s",
+                    frac=achieved / PEAK_MFMA_FP32, traffic=None, launches_per_step=n // steps,
+                    avg_launch_us=total / n * 1e6)
+    else:
+        work = hbm_bytes.get(top, float("nan"))
+        achieved = work * steps / total
+        roof = dict(kernel=top, bound="hbm", achieved=achieved / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s",
+                    frac=achieved / PEAK_HBM, traffic=None, launches_per_step=n // steps, avg_launch_us=total / n * 1e6)
+    breakdown = {k: round(v[1] / steps * 1e3, 4) for k, v in fam.items()}  # ms per step by kernel family
+    return N * steps / dt, dt / steps * 1e3, roof, breakdown
+
+
+def bench_conv_bwd(capi, workloads, reps):
+    """BASELINE configs[4]: 3x3x256x256 on 56x56x256x64, stride 1, pad 1: dzdx + dzdf (+ dzdb)."""
+    import ctypes as C
+    import torch
+    L = capi.lib()
+    xs, fs = (56, 56, 256, 64), (3, 3, 256, 256)
+    g = capi.conv_geom(xs, fs, 1, 1, 1)
+    x = torch.randn(tuple(reversed(xs)), device="cuda")
+    f = torch.randn(tuple(reversed(fs)), device="cuda") * float(np.sqrt(2.0 / (9 * 256)))
+    dy = torch.randn(tuple(reversed(xs)), device="cuda")
+    dx, df, db = capi.empty(xs), capi.empty(fs), capi.empty((256,))
+    ws = capi.Workspace()
+    nbytes = max(L.mcn_conv_workspace_bytes(C.byref(g), k) for k in range(4))
+    wp, wn = ws.get(nbytes)
+    st = capi.stream()
+    flops = 2.0 * 56 * 56 * 9 * 256 * 256 * 64
+    data = lambda: capi.check(L.mcn_conv_backward_data(st, C.byref(g), capi.ptr(dx), capi.ptr(f), capi.ptr(dy), wp, wn))
+    filt = lambda: capi.check(L.mcn_conv_backward_filter(st, C.byref(g), capi.ptr(df), capi.ptr(x), capi.ptr(dy), wp, wn))
+    bias = lambda: capi.check(L.mcn_conv_backward_bias(st, C.byref(g), capi.ptr(db), capi.ptr(dy), wp, wn))
+    for fn in (data, filt, bias):
+        fn()
+    _sync()
+    t_data, _ = kernel_time(capi, "conv_pix_mfma", data, reps)
+    t_filt, _ = kernel_time(capi, "conv_wgrad_mfma", filt, reps)
+    t_red, _ = kernel_time(capi, "conv_wgrad_reduce", filt, reps)
+    # whole backward call (all launches incl. weight packing, partial-sum reduction and bias), wall clock
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        data(); filt(); bias()
+    _sync()
+    t_all = (time.perf_counter() - t0) / reps
+    out = []
+    for name, kern, t in (("conv backward-data", "conv_pix_mfma", t_data), ("conv backward-filter", "conv_wgrad_mfma", t_filt)):
+        out.append(dict(op=name, kernel=kern, workload="configs[4] 3x3x256x256 on 56x56x256x64", bound="mfma",
+                        achieved=flops / t / 1e12, peak=PEAK_MFMA_FP32 / 1e12, unit="TFLOP/s", frac=flops / t / PEAK_MFMA_FP32,
+                        avg_launch_us=t * 1e6, traffic=None))
+    whole = dict(tflops=2 * flops / t_all / 1e12, frac=2 * flops / t_all / PEAK_MFMA_FP32, ms=t_all * 1e3,
+                 wgrad_reduce_us=t_red * 1e6)
+    return out, whole
+
+
+def bench_bnorm_bwd(capi, workloads, reps):
+    """BASELINE configs[1]: 56x56x256x32, moments from the batch."""
+    import ctypes as C
+    import torch
+    L = capi.lib()
+    H, W, Cc, N = 56, 56, 256, 32
+    x = torch.randn((N, Cc, W, H), device="cuda") * 1.3 + 0.5
+    dy = torch.randn((N, Cc, W, H), device="cuda")
+    g = torch.rand(Cc, device="cuda") + 0.5
+    dx, dg, db, mom = capi.empty((H, W, Cc, N)), capi.empty((Cc,)), capi.empty((Cc,)), capi.empty((Cc, 2))
+    ws = capi.Workspace()
+    wp, wn = ws.get(L.mcn_bnorm_workspace_bytes(H, W, Cc, N))
+    st = capi.stream()
+    call = lambda: capi.check(L.mcn_bnorm_backward(st, capi.ptr(dx), capi.ptr(dg), capi.ptr(db), capi.ptr(mom), capi.ptr(x),
+                                                   capi.ptr(g), capi.ptr(dy), H, W, Cc, N, 1e-4, 0, wp, wn))
+    call()
+    _sync()
+    E = 4.0 * H * W * Cc * N
+    t_sums, _ = kernel_time(capi, "bnorm_sums", call, reps)
+    t_apply, _ = kernel_time(capi, "bnorm_backward_apply", call, reps)
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        call()
+    _sync()
+    t_all = (time.perf_counter() - t0) / reps
+    rows = [
+        dict(op="bnorm backward, pass 1 (sums)", kernel="bnorm_sums", workload="configs[1] 56x56x256x32", bound="hbm",
+             achieved=2 * E / t_sums / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=2 * E / t_sums / PEAK_HBM,
+             avg_launch_us=t_sums * 1e6, traffic=None),
+        dict(op="bnorm backward, pass 2 (apply)", kernel="bnorm_backward_apply", workload="configs[1] 56x56x256x32", bound="hbm",
+             achieved=3 * E / t_apply / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=3 * E / t_apply / PEAK_HBM,
+             avg_launch_us=t_apply * 1e6, traffic=None),
+    ]
+    whole = dict(gbs=5 * E / t_all / 1e9, frac=5 * E / t_all / PEAK_HBM, us=t_all * 1e6, gbs_compulsory=3 * E / t_all / 1e9)
+    return rows, whole
+
+
+def bench_pool_bwd(capi, workloads, reps):
+    """BASELINE configs[2]: (a) max 3x3 s2 p1 on 112x112x64x32, (b) avg 2x2 s2 on 56x56x256x32."""
+    import ctypes as C
+    import torch
+    L = capi.lib()
+    rows = []
+    for name, shape, pool, pad, method in (("max-pool backward", (112, 112, 64, 32), 3, 1, "max"),
+                                           ("avg-pool backward", (56, 56, 256, 32), 2, 0, "avg")):
+        g = capi.pool_geom(shape, pool, 2, pad, method)
+        oshape = capi.pool_out_shape(g)
+        x = torch.randn(tuple(reversed(shape)), device="cuda")
+        dy = torch.randn(tuple(reversed(oshape)), device="cuda")
+        dx = capi.empty(shape)
+        st = capi.stream()
+        call = lambda: capi.check(L.mcn_pool_backward(st, C.byref(g), capi.ptr(dx), capi.ptr(x), capi.ptr(dy), 0))
+        call()
+        _sync()
+        e, o = 4.0 * np.prod(shape), 4.0 * np.prod(oshape)
+        nbytes = (2 * e + o) if method == "max" else (e + o)
+        t, _ = kernel_time(capi, "pool_backward_tiled", call, reps)
+        rows.append(dict(op=name, kernel="pool_backward_tiled", workload="configs[2] %s on %s" % (method, "x".join(map(str, shape))),
+                         bound="hbm", achieved=nbytes / t / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=nbytes / t / PEAK_HBM,
+                         avg_launch_us=t * 1e6, traffic=None))
+    return rows
+
+
+def cpu_baseline(workloads):
+    """The CPU restatement of the reference path on this host: one forward+backward of the same block
+    (same N = 32 inputs), GEMMs threaded like the reference's BLAS, everything else serial."""
+    from oracle import binding as ob
+    from oracle import blocks
+    blas = ob.use_openblas(True)
+    w = workloads.bottleneck_case()
+    N = w["x"].shape[3]
+    blocks.bottleneck(workloads.bottleneck_case(N=2))  # warm the threads and pages
+    t0 = time.perf_counter()
+    reps = 0
+    while reps < 1 or (time.perf_counter() - t0 < 8.0 and reps < 4):
+        blocks.bottleneck(w)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    ob.use_openblas(False)
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    return dict(value=N / dt, unit="images/s", cores=cores, kind="port",
+                sample="%d full forward+backward passes of the same N=%d block; oracle/ (im2row + sgemm per image, serial "
+                       "bnorm/relu loops); sgemm = %s" % (reps, N, "OpenBLAS (numpy wheel), threaded" if blas else "built-in OpenMP kernel"),
+                ms_per_step=dt * 1e3)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.stderr.write("bench.py measures one GPU: this hot path does not shard in this build (run with --gpus 1)\n")
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py needs a GPU\n")
+        sys.exit(2)
+    from matconvnet_amd import capi, vlapi, workloads
+    capi.lib()
+    vlapi.lib()
+
+    images_per_s, ms_per_step, roof, breakdown = bench_block(vlapi, capi, workloads, args.steps, args.warmup)
+    conv_rows, conv_whole = bench_conv_bwd(capi, workloads, max(5, args.steps // 5))
+    bn_rows, bn_whole = bench_bnorm_bwd(capi, workloads, args.steps)
+    pool_rows = bench_pool_bwd(capi, workloads, args.steps)
+    line = {
+        "metric": "ResNet-50-block fwd+bwd images/s; conv-bwd TFLOP/s; bnorm/pool-bwd GB/s",
+        "value": images_per_s, "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[3]: ResNet-50 bottleneck fwd+bwd, 56x56, 256->64->64->256, N=32, via vl::nn operators"},
+        "roofline": roof,
+        "step_breakdown_ms": breakdown,
+        "conv_bwd_tflops": conv_whole["tflops"], "conv_bwd_frac_of_mfma_peak": conv_whole["frac"], "conv_bwd_ms": conv_whole["ms"],
+        "bnorm_bwd_gbs": bn_whole["gbs"], "bnorm_bwd_frac_of_hbm_peak": bn_whole["frac"], "bnorm_bwd_us": bn_whole["us"],
+        "maxpool_bwd_gbs": pool_rows[0]["achieved"], "avgpool_bwd_gbs": pool_rows[1]["achieved"],
+        "rooflines": conv_rows + bn_rows + pool_rows,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(workloads)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -89,6 +89,15 @@ MCN_API int mcn_device_compute_units(void);
 MCN_API int mcn_set_tunable(const char* name, int value);
 MCN_API int mcn_get_tunable(const char* name, int* value);
 
+/* Live per-kernel timing with HIP events on the stream the kernel is launched on.  After
+   mcn_profile_begin("name"), every launch of the kernel family whose name contains "name" (e.g.
+   "conv_pix_mfma", "conv_wgrad_mfma", "bnorm_sums", "bnorm_backward_apply", "pool_backward") is bracketed
+   by a pair of events.  mcn_profile_end waits for the last one and reports the number of bracketed
+   launches and the sum of their durations in milliseconds.  Not part of the reference interface (the
+   reference relies on nvprof brackets, matlab/src/vl_cudatool.cu:126-131). */
+MCN_API int mcn_profile_begin(const char* kernel_name);
+MCN_API int mcn_profile_end(int* launches, double* total_ms);
+
 /* ------------------------------------------------------------------------------------------------
  * convolution -- replaces ConvolutionForward/Backward<VLDT_GPU,T> (bits/nnconv.cu:71-157,163-317),
  * i.e. im2row_gpu + cublasSgemm per image, and the cuDNN variant (bits/nnconv_cudnn.cu:40-540).

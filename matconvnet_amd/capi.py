@@ -44,6 +44,8 @@ PROTOTYPES = {
     "mcn_device_compute_units": (_i, []),
     "mcn_set_tunable": (_i, [C.c_char_p, _i]),
     "mcn_get_tunable": (_i, [C.c_char_p, C.POINTER(_i)]),
+    "mcn_profile_begin": (_i, [C.c_char_p]),
+    "mcn_profile_end": (_i, [C.POINTER(_i), C.POINTER(_d)]),
     "mcn_conv_output_size": (_i, [C.POINTER(ConvGeom), C.POINTER(_i), C.POINTER(_i)]),
     "mcn_conv_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _i]),
     "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),
@@ -94,6 +96,17 @@ def get_tunable(name):
     v = C.c_int(0)
     check(lib().mcn_get_tunable(name.encode(), C.byref(v)))
     return v.value
+
+
+def profile_begin(kernel_name):
+    check(lib().mcn_profile_begin(kernel_name.encode()))
+
+
+def profile_end():
+    """(bracketed launches, sum of their durations in ms)"""
+    n, ms = C.c_int(0), C.c_double(0.0)
+    check(lib().mcn_profile_end(C.byref(n), C.byref(ms)))
+    return n.value, ms.value
 
 
 def _pair(v):

@@ -309,13 +309,18 @@ int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float
   if (!givenMoments) {
     if (!workspace || workspaceBytes < mcn_bnorm_workspace_bytes(H, W, C, N))
       return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward: workspace too small");
-    if (vec) hipLaunchKernelGGL((bnorm_sums<0, true>), grid, block, 0, s, x, x, partials, p);
-    else hipLaunchKernelGGL((bnorm_sums<0, false>), grid, block, 0, s, x, x, partials, p);
+    {
+      KernelTimer timer("bnorm_sums", s);
+      if (vec) hipLaunchKernelGGL((bnorm_sums<0, true>), grid, block, 0, s, x, x, partials, p);
+      else hipLaunchKernelGGL((bnorm_sums<0, false>), grid, block, 0, s, x, x, partials, p);
+    }
     if ((rc = check_launch("mcn_bnorm_forward(sums)"))) return rc;
+    KernelTimer timer("bnorm_forward_apply", s);
     if (vec) hipLaunchKernelGGL((bnorm_forward_apply<false, true>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
     else hipLaunchKernelGGL((bnorm_forward_apply<false, false>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
   } else {
     p.reverse = 0;
+    KernelTimer timer("bnorm_forward_apply", s);
     if (vec) hipLaunchKernelGGL((bnorm_forward_apply<true, true>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
     else hipLaunchKernelGGL((bnorm_forward_apply<true, false>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
   }
@@ -344,14 +349,18 @@ int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultiplie
   const bool vec = (p.WH % 4 == 0) && aligned16(derInput) && aligned16(x) && aligned16(derOutput);
   const dim3 grid((unsigned)(C * p.groups)), block(256);
   double* partials = (double*)workspace;
-  if (givenMoments) {
-    if (vec) hipLaunchKernelGGL((bnorm_sums<1, true>), grid, block, 0, s, x, derOutput, partials, p);
-    else hipLaunchKernelGGL((bnorm_sums<1, false>), grid, block, 0, s, x, derOutput, partials, p);
-  } else {
-    if (vec) hipLaunchKernelGGL((bnorm_sums<2, true>), grid, block, 0, s, x, derOutput, partials, p);
-    else hipLaunchKernelGGL((bnorm_sums<2, false>), grid, block, 0, s, x, derOutput, partials, p);
+  {
+    KernelTimer timer("bnorm_sums", s);
+    if (givenMoments) {
+      if (vec) hipLaunchKernelGGL((bnorm_sums<1, true>), grid, block, 0, s, x, derOutput, partials, p);
+      else hipLaunchKernelGGL((bnorm_sums<1, false>), grid, block, 0, s, x, derOutput, partials, p);
+    } else {
+      if (vec) hipLaunchKernelGGL((bnorm_sums<2, true>), grid, block, 0, s, x, derOutput, partials, p);
+      else hipLaunchKernelGGL((bnorm_sums<2, false>), grid, block, 0, s, x, derOutput, partials, p);
+    }
   }
   if ((rc = check_launch("mcn_bnorm_backward(sums)"))) return rc;
+  KernelTimer timer("bnorm_backward_apply", s);
   if (givenMoments) {
     if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
     else hipLaunchKernelGGL((bnorm_backward_apply<true, false>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);

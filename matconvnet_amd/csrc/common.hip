@@ -1,10 +1,12 @@
 // Error state, tunables and device queries of the gfx950 back-end.
 #include "mcn_internal.hpp"
 
+#include <atomic>
 #include <cstring>
 #include <map>
 #include <mutex>
 #include <string>
+#include <vector>
 
 namespace mcn {
 
@@ -46,6 +48,36 @@ int check_launch(const char* what) {
   return MCN_SUCCESS;
 }
 
+namespace {
+struct ProfileState {
+  std::mutex mutex;
+  std::atomic<bool> active{false};
+  std::string pattern;
+  std::vector<hipEvent_t> begin, end;
+  size_t used = 0;
+} g_profile;
+}  // namespace
+
+KernelTimer::KernelTimer(const char* kernel, hipStream_t s) : slot(-1), stream(s) {
+  if (!g_profile.active.load(std::memory_order_relaxed)) return;
+  std::lock_guard<std::mutex> lock(g_profile.mutex);
+  if (!g_profile.active || std::strstr(kernel, g_profile.pattern.c_str()) == nullptr) return;
+  if (g_profile.used == g_profile.begin.size()) {
+    hipEvent_t b, e;
+    if (hipEventCreate(&b) != hipSuccess || hipEventCreate(&e) != hipSuccess) return;
+    g_profile.begin.push_back(b);
+    g_profile.end.push_back(e);
+  }
+  slot = (int)g_profile.used++;
+  (void)hipEventRecord(g_profile.begin[slot], stream);
+}
+
+KernelTimer::~KernelTimer() {
+  if (slot < 0) return;
+  std::lock_guard<std::mutex> lock(g_profile.mutex);
+  (void)hipEventRecord(g_profile.end[slot], stream);
+}
+
 int tunable(const char* name, int fallback) {
   std::lock_guard<std::mutex> lock(g_tunable_mutex);
   for (auto& t : g_tunables)
@@ -76,6 +108,34 @@ int mcn_device_compute_units(void) {
   if (hipGetDevice(&dev) != hipSuccess) return -1;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
   return cus;
+}
+
+int mcn_profile_begin(const char* kernel_name) {
+  if (!kernel_name || !*kernel_name) return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_profile_begin: empty kernel name");
+  std::lock_guard<std::mutex> lock(mcn::g_profile.mutex);
+  mcn::g_profile.pattern = kernel_name;
+  mcn::g_profile.used = 0;
+  mcn::g_profile.active = true;
+  return MCN_SUCCESS;
+}
+
+int mcn_profile_end(int* launches, double* total_ms) {
+  std::lock_guard<std::mutex> lock(mcn::g_profile.mutex);
+  mcn::g_profile.active = false;
+  double total = 0.0;
+  const size_t n = mcn::g_profile.used;
+  if (n > 0 && hipEventSynchronize(mcn::g_profile.end[n - 1]) != hipSuccess)
+    return mcn::fail(MCN_DEVICE_ERROR, "mcn_profile_end: event synchronisation failed");
+  for (size_t i = 0; i < n; ++i) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, mcn::g_profile.begin[i], mcn::g_profile.end[i]) != hipSuccess)
+      return mcn::fail(MCN_DEVICE_ERROR, "mcn_profile_end: event %zu was not recorded", i);
+    total += ms;
+  }
+  if (launches) *launches = (int)n;
+  if (total_ms) *total_ms = total;
+  mcn::g_profile.used = 0;
+  return MCN_SUCCESS;
 }
 
 int mcn_set_tunable(const char* name, int value) {

@@ -168,6 +168,7 @@ int mcn_conv_backward_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* d
   hipStream_t s = as_stream(stream);
   const bool vec = (P % 4 == 0) && aligned16(derOutput);
   const dim3 grid((unsigned)(p.K * groups)), block(256);
+  KernelTimer timer("conv_bias_partial", s);
   if (vec) hipLaunchKernelGGL(conv_bias_partial<true>, grid, block, 0, s, partials, derOutput, P, p.K, p.N, groups);
   else hipLaunchKernelGGL(conv_bias_partial<false>, grid, block, 0, s, partials, derOutput, P, p.K, p.N, groups);
   if ((rc = check_launch("mcn_conv_backward_bias(partial)"))) return rc;

@@ -421,6 +421,7 @@ void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, con
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB;
   const long long mTiles = (p.M + BB - 1) / BB;
   const int tilesA = (p.Cout + BA - 1) / BA;
+  KernelTimer timer("conv_pix_mfma", s);
   hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB>), dim3((unsigned)(mTiles * tilesA)), dim3(256), 0, s, out, in,
                      wt, bias, p);
 }
@@ -438,6 +439,7 @@ int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const flo
     }
     raised = true;
   }
+  KernelTimer timer("conv_wgrad_mfma", s);
   hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB>), grid, dim3(256), lds, s, out, x, dy, p);
   return MCN_SUCCESS;
 }
@@ -452,9 +454,13 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   if (!aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
   float* wt = (float*)ws;
   const size_t nW = (size_t)rPad * p.coutPad;
-  hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, wt, f, p.T, p.Cin, p.Cout,
-                     rPad, p.coutPad, backward);
-  int rc = check_launch(who);
+  int rc;
+  {
+    KernelTimer timer("conv_pack_weights", s);
+    hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, wt, f, p.T, p.Cin, p.Cout,
+                       rPad, p.coutPad, backward);
+    rc = check_launch(who);
+  }
   if (rc) return rc;
   const long long blocks = ((p.M + (BA == 128 ? 127 : 255)) / (BA == 128 ? 128 : 256)) * (p.coutPad / BA);
   if (blocks >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
@@ -554,6 +560,7 @@ int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const fl
   else rc = launch_wgrad<1, 1, 1, 4>(s, grid, target, x, dy, q);
   if (!rc) rc = check_launch("mcn_conv_backward_filter");
   if (rc || q.splits == 1) return rc;
+  KernelTimer timer("conv_wgrad_reduce", s);
   hipLaunchKernelGGL(conv_wgrad_reduce, dim3((unsigned)((nF + 255) / 256)), block, 0, s, df, target, nF, q.splits);
   return check_launch("mcn_conv_backward_filter(reduce)");
 }

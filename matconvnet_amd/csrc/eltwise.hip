@@ -65,6 +65,7 @@ int launch(const char* who, mcn_stream_t stream, float* y, const float* a, const
   // each thread handles a few float4s; cap the grid at 32 workgroups per CU-equivalent (256 CUs)
   const size_t work = vec ? (n + 3) / 4 : n;
   const unsigned blocks = (unsigned)std::min<size_t>((work + 255) / 256, 256u * 32u);
+  KernelTimer timer("eltwise_kernel", as_stream(stream));
   if (vec) hipLaunchKernelGGL((eltwise_kernel<OP, true>), dim3(blocks), dim3(256), 0, as_stream(stream), y, a, b, k, n);
   else hipLaunchKernelGGL((eltwise_kernel<OP, false>), dim3(blocks), dim3(256), 0, as_stream(stream), y, a, b, k, n);
   return check_launch(who);

@@ -22,6 +22,18 @@ int check_launch(const char* what);
 
 int tunable(const char* name, int fallback);
 
+// Brackets one kernel launch with HIP events when live profiling of that kernel family is switched on
+// (mcn_profile_begin); costs one relaxed load otherwise.  Construct right before the launch, on its stream.
+class KernelTimer {
+ public:
+  KernelTimer(const char* kernel, hipStream_t stream);
+  ~KernelTimer();
+
+ private:
+  int slot;
+  hipStream_t stream;
+};
+
 inline hipStream_t as_stream(mcn_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

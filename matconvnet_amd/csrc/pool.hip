@@ -369,6 +369,7 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
     const bool vec = (p.H % 4 == 0) && (p.outH % 4 == 0) && aligned16(derInput) && aligned16(derOutput) &&
                      (!isMax || aligned16(x));
     const dim3 grid((unsigned)(planes * tiles)), block(256);
+    KernelTimer timer("pool_backward_tiled", s);
     if (isMax) {
       if (vec) hipLaunchKernelGGL((pool_backward_tiled<true, true>), grid, block, lds, s, derInput, x, derOutput, p);
       else hipLaunchKernelGGL((pool_backward_tiled<true, false>), grid, block, lds, s, derInput, x, derOutput, p);
