@@ -3,7 +3,7 @@
 // synthetic inputs, times them with HIP events and prints TFLOP/s, GB/s and images/s beside the
 // fraction of the MI355X rooflines (fp32 matrix 157.3 TFLOP/s, HBM 8 TB/s).
 //
-//   mcn_bench [--iters K] [--warmup W] [--only conv5|bnorm|maxpool|avgpool|block|conv1]
+//   mcn_bench [--iters K] [--warmup W] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy]
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
@@ -20,6 +20,7 @@
 #include "nnbnorm.hpp"
 #include "nnconv.hpp"
 #include "nnpooling.hpp"
+#include "../../include/mcn_hip.h"
 
 using namespace vl;
 
@@ -134,6 +135,17 @@ static void benchPool(bool isMax, int warmup, int iters) {
               t * 1e3, bytes / t / 1e6, 100 * bytes / (t * 1e-3) / kPeakHbm, bytes / 1e6);
 }
 
+// A plain streaming copy of known size (ReLU of positive data): the yardstick the HBM byte counters of the
+// other kernels are scaled by.
+static void benchCopy(int warmup, int iters) {
+  const size_t n = 64u << 20;  // 64 Mi floats: reads 256 MiB, writes 256 MiB
+  DeviceTensor a(TensorShape(n, 1, 1, 1)), b(TensorShape(n, 1, 1, 1));
+  a.fill(1.f);
+  double t = medianMs([&] { mcn_relu_forward(NULL, (float*)b.view.getMemory(), (float const*)a.view.getMemory(), n); }, warmup, iters);
+  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; reads %zu B, writes %zu B per launch)\n", "copy 256 MiB", t * 1e3,
+              2.0 * n * 4 / t / 1e6, 100 * 2.0 * n * 4 / (t * 1e-3) / kPeakHbm, n * 4, n * 4);
+}
+
 static void benchBlock(int warmup, int iters) {
   const int H = 56, W = 56, C = 256, M = 64, N = 32;
   harness::Bottleneck block(H, W, C, M, N, 1e-5);
@@ -175,7 +187,7 @@ int main(int argc, char** argv) {
     else if (!std::strcmp(argv[i], "--warmup") && i + 1 < argc) warmup = std::atoi(argv[++i]);
     else if (!std::strcmp(argv[i], "--only") && i + 1 < argc) only = argv[++i];
     else {
-      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--only conv5|conv1|bnorm|maxpool|avgpool|block]\n");
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy]\n");
       return 1;
     }
   }
@@ -183,6 +195,7 @@ int main(int argc, char** argv) {
   HIP_OK(hipGetDeviceProperties(&prop, 0));
   std::printf("device: %s, %d CUs, %.0f MHz\n", prop.name, prop.multiProcessorCount, prop.clockRate / 1000.0);
   auto want = [&](char const* k) { return only.empty() || only == k; };
+  if (only == "copy") benchCopy(warmup, iters);
   if (want("conv1")) benchConv("conv 5x5x3x32 on 32x32x3x100", 32, 32, 3, 100, 5, 32, 2, warmup, iters);
   if (want("bnorm")) benchBnorm(warmup, iters);
   if (want("maxpool")) benchPool(true, warmup, iters);
