@@ -40,6 +40,31 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 inline int div_up(long long a, long long b) { return (int)((a + b - 1) / b); }
 
+// Division of a non-negative 31-bit integer by a run-time constant without the ~35-instruction hardware
+// sequence: q = (mulhi(n, mul) + n) >> shift with mul = floor(2^32 (2^shift - d) / d) + 1, shift = ceil(log2 d).
+// Exact for 0 <= n < 2^31, 1 <= d < 2^31.  Built on the host, passed to kernels by value.
+struct FastDiv {
+  unsigned mul, shift;
+  int d;
+  FastDiv() : mul(0), shift(0), d(1) {}
+  explicit FastDiv(int divisor) : d(divisor < 1 ? 1 : divisor) {
+    shift = 0;
+    while ((1ll << shift) < d) ++shift;
+    mul = (unsigned)((((1ull << 32) * ((1ull << shift) - (unsigned long long)d)) / (unsigned long long)d) + 1ull);
+  }
+  __host__ __device__ __forceinline__ int div(int n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (int)((__umulhi((unsigned)n, mul) + (unsigned)n) >> shift);
+#else
+    return (int)(((((unsigned long long)(unsigned)n * mul) >> 32) + (unsigned)n) >> shift);
+#endif
+  }
+  __host__ __device__ __forceinline__ void divmod(int n, int* q, int* r) const {
+    *q = div(n);
+    *r = n - *q * d;
+  }
+};
+
 constexpr int kWave = 64;      // CDNA wavefront width
 constexpr int kNumXcd = 8;     // MI355X: 8 accelerator dies, each with its own L2
 
