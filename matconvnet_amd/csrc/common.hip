@@ -20,7 +20,7 @@ struct Tunable {
 };
 // Defaults are the values chosen from on-device sweeps; see the per-kernel comments where each is read.
 Tunable g_tunables[] = {
-    {"pool_lds_bytes", 24 * 1024},     // LDS tile budget of the pooling-backward kernels
+    {"pool_lds_bytes", 16 * 1024},     // LDS tile budget of the pooling-backward kernels
     {"pool_force_gather", 0},          // 1: skip the ordered-pass kernel, use the general tiled gather
     {"bnorm_block_elems", 4096},       // minimum elements a bnorm reduction block should own
     {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)

@@ -35,7 +35,7 @@ struct PoolP {
   // rankTab[i] = (pool - 1 - i) / stride   (windows up to 8 x 8)
   int rankH[8], rankW[8];
   // host-precomputed helpers of the ordered-pass kernel (no integer division on the device)
-  FastDiv byTiles, bySx, byOutH, byStageRow;  // stage row = H/4 (16-byte staging) or H
+  FastDiv byTiles, bySx, byOutH, byStageRow, byBorder;  // stage row = H/4 (16-byte staging) or H; border rows per column
   int outStepQ, outStepR;      // 256 = outStepQ * outH + outStepR
   int stageStepQ, stageStepR;  // 256 = stageStepQ * stageRow + stageStepR
   int KH, nPasses;
@@ -454,7 +454,8 @@ __global__ __launch_bounds__(256) void pool_backward_passes(float* __restrict__ 
   // framed staging area: frame column c <-> image column cLo + c, frame row r <-> image row r - pt
   const int cLo = owLo * p.sx - p.pl;
   const int nC = MAX && nOW > 0 ? (owHi - owLo) * p.sx + poolW : 0;
-  const int Hp = (p.outH - 1) * p.sy + poolH;
+  // frame pitch: every row a window can read, and never less than the rows the interior copy writes
+  const int Hp = max((p.outH - 1) * p.sy + poolH, p.pt + p.H);
 
   float* acc = smem;                    // [nIn] one accumulator per owned input element
   float* xs = acc + ((nIn + 3) & ~3);   // [nC*Hp] x inside a -inf frame (max only)
@@ -546,11 +547,14 @@ __global__ __launch_bounds__(256) void pool_backward_passes(float* __restrict__ 
         }
       }
     }
-    // border: rows above / below the image in every present column ...
-    const int below = Hp - p.pt - p.H;  // may be <= 0 when the last rows of x are read by no window
-    for (int c = ca - cLo; c < cb - cLo; ++c) {
-      if (tid < p.pt) xs[c * Hp + tid] = -INFINITY;
-      if (tid < below) xs[c * Hp + p.pt + p.H + tid] = -INFINITY;
+    // border cells (-inf): the rows above / below the image in every present column, one cell per thread ...
+    const int below = max(Hp - p.pt - p.H, 0), nb = p.pt + below;
+    if (nb > 0) {
+      for (int i = tid; i < (cb - ca) * nb; i += 256) {
+        int c, k;
+        p.byBorder.divmod(i, &c, &k);
+        xs[(ca - cLo + c) * Hp + (k < p.pt ? k : p.H + k)] = -INFINITY;
+      }
     }
     // ... and whole columns left / right of the image
     for (int c = 0; c < ca - cLo; ++c)
@@ -835,7 +839,7 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
   p.accumulate = accumulate ? 1 : 0;
   hipStream_t s = as_stream(stream);
 
-  const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 24 * 1024), 1024), 64 * 1024);
+  const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024), 64 * 1024);
   const int kh = (p.poolH + p.sy - 1) / p.sy, kw = (p.poolW + p.sx - 1) / p.sx;
   const int passes = isMax ? kh * kw : p.poolH * p.poolW;
   const bool vecIn = (p.H % 4 == 0) && aligned16(derInput);
@@ -859,7 +863,7 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
         size_t need = pad4((size_t)(w1 - w0) * p.H);
         if (isMax) {
           const size_t nC = nOW > 0 ? (size_t)(owHi - owLo) * p.sx + p.poolW : 0;
-          const size_t Hp = (size_t)(p.outH - 1) * p.sy + p.poolH;
+          const size_t Hp = (size_t)std::max((p.outH - 1) * p.sy + p.poolH, p.pt + p.H);
           need += nC * Hp;
         }
         worst = std::max(worst, need * sizeof(float));
@@ -880,6 +884,7 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
       p.bySx = FastDiv(p.sx);
       p.byOutH = FastDiv(p.outH);
       p.byStageRow = FastDiv(stageRow);
+      p.byBorder = FastDiv(std::max(p.pt + std::max((p.outH - 1) * p.sy + p.poolH - p.pt - p.H, 0), 1));  // = Hp - H
       p.outStepQ = 256 / p.outH;
       p.outStepR = 256 % p.outH;
       p.stageStepQ = 256 / stageRow;

@@ -107,6 +107,42 @@ def test_tile_width_does_not_change_results(capi, ob, budget):
         capi.set_tunable("pool_lds_bytes", old)
 
 
+@pytest.mark.parametrize("method", ["max", "avg"])
+@pytest.mark.parametrize("geom", [(20, 18, 2, 2, 3, 2, 1), (16, 16, 3, 1, 2, 2, 0), (15, 13, 2, 2, (3, 2), (1, 2), (1, 0, 0, 1))])
+def test_general_gather_kernels_agree(capi, ob, method, geom):
+    """The ordered-pass kernel is the default; the general tiled gather / flag kernels behind it give the
+    same bits."""
+    H, W, C, N, pool, stride, pad = geom
+    shape = (H, W, C, N)
+    x = _inputs(shape, 31, "ties")
+    og = ob.pool_geom(shape, pool, stride, pad, method)
+    dy = F(np.random.default_rng(32).standard_normal(ob.pool_out_shape(og)))
+    try:
+        capi.set_tunable("pool_force_gather", 1)
+        got, want = _run(capi, ob, x, dy, shape, pool, stride, pad, method)
+        assert bits_equal(got, want)
+        base = F(np.random.default_rng(33).standard_normal(shape))
+        got, want = _run(capi, ob, x, dy, shape, pool, stride, pad, method, accumulate_into=base)
+        assert bits_equal(got, want)
+    finally:
+        capi.set_tunable("pool_force_gather", 0)
+
+
+@pytest.mark.parametrize("method", ["max", "avg"])
+@pytest.mark.parametrize("geom", [(24, 20, 2, 2, 5, 1, 2), (30, 30, 1, 2, 9, 4, 4), (21, 17, 2, 1, (7, 3), (1, 1), (3, 3, 1, 1)),
+                                   (40, 40, 2, 1, 3, 5, 0)])
+def test_large_windows_and_sparse_strides(capi, ob, method, geom):
+    """Windows covered by many outputs (more than 16 passes), windows larger than 8, and strides larger than
+    the window (inputs no output covers) take the general paths."""
+    H, W, C, N, pool, stride, pad = geom
+    shape = (H, W, C, N)
+    x = _inputs(shape, 41, "ties")
+    og = ob.pool_geom(shape, pool, stride, pad, method)
+    dy = F(np.random.default_rng(42).standard_normal(ob.pool_out_shape(og)))
+    got, want = _run(capi, ob, x, dy, shape, pool, stride, pad, method)
+    assert bits_equal(got, want), count_bit_mismatches(got, want)
+
+
 def test_golden_vectors_from_reference(capi):
     z = np.load(GOLDEN)
     for i in range(int(z["count"])):
