@@ -25,6 +25,7 @@ Tunable g_tunables[] = {
     {"bnorm_block_elems", 4096},       // minimum elements a bnorm reduction block should own
     {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)
     {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels
+    {"conv_pix_tile", 0},              // force a tile shape of the pixel-major MFMA kernel (0 = automatic)
     {"conv_wgrad_blocks", 0},          // target workgroups for filter-gradient split (0 = 2 per CU)
     {"conv_bias_blocks", 0},           // target workgroups for the bias-gradient reduction
 };

@@ -46,8 +46,10 @@ struct PixP {
   int dhBase, dhStep, dwBase, dwStep;
   int R;              // reduction length = T*Cin
   int coutPad;        // row pitch of wt
-  long long M;        // OH*OW*N
+  int M;              // OH*OW*N (< 2^31)
   float alpha, beta;
+  FastDiv byQ, byOH, byT;  // Q = OH*OW; T = taps
+  int advC, advT;          // 16 = advC*T + advT (reduction rows per step)
 };
 
 // wt[R][co] from the MATLAB filter bank f[i,j,c,k] (FV x K, column-major).
@@ -97,7 +99,7 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int mt = logical / tilesA;
   const int co0 = (logical - mt * tilesA) * BA;
-  const long long m0 = (long long)mt * BB;
+  const int m0 = mt * BB;
 
   const int IHW = p.IH * p.IW;
   const int Q = p.OH * p.OW;
@@ -110,22 +112,22 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
 
   // ---- this thread's pixel (fixed for the whole kernel)
   const int mm = tid % BB, pg = tid / BB;
-  const long long m = m0 + mm;
+  const int m = m0 + mm;
   const bool mvalid = m < p.M;
   int ihB = 0, iwB = 0;
   const float* inN = in;
   {
-    const long long mc = mvalid ? m : 0;
-    const int n = (int)(mc / Q);
-    const int q = (int)(mc - (long long)n * Q);
-    const int ow = q / p.OH, oh = q - ow * p.OH;
+    int n, q, ow, oh;
+    p.byQ.divmod(mvalid ? m : 0, &n, &q);
+    p.byOH.divmod(q, &ow, &oh);
     ihB = oh * p.sy;
     iwB = ow * p.sx;
     inN = in + (size_t)n * p.Cin * IHW + ihB + p.IH * iwB;
   }
   // first gathered row of this thread: R = pg*RPT -> (tap, channel); advanced by BK per step
-  int tapS = (pg * RPT) % p.T, ciS = (pg * RPT) / p.T;
-  const int advC = BK / p.T, advT = BK % p.T;
+  int ciS, tapS;
+  p.byT.divmod(pg * RPT, &ciS, &tapS);
+  const int advC = p.advC, advT = p.advT;
 
   floatx16 acc[WA][WB];
 #pragma unroll
@@ -209,10 +211,10 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   // ---- epilogue: lane = pixel, register = channel
 #pragma unroll
   for (int jj = 0; jj < WB; ++jj) {
-    const long long mo = m0 + wb * WB * 32 + jj * 32 + l32;
+    const int mo = m0 + wb * WB * 32 + jj * 32 + l32;
     if (mo >= p.M) continue;
-    const int n = (int)(mo / Q);
-    const int q = (int)(mo - (long long)n * Q);
+    int n, q;
+    p.byQ.divmod(mo, &n, &q);
     float* o = out + (size_t)n * p.Cout * Q + q;
 #pragma unroll
     for (int ii = 0; ii < WA; ++ii)
@@ -239,9 +241,10 @@ struct WgP {
   int FH, T;
   int sy, sx, pt, pl, dly, dlx;
   int FV;
-  long long M;           // OH*OW*N
-  long long chunkSpan;   // pixels per split (multiple of 32)
+  int M;                 // OH*OW*N (< 2^31)
+  int chunkSpan;         // pixels per split (multiple of 32)
   int splits;
+  FastDiv byQ, byOH, byT, byFH, byTiles, byTilesK;
 };
 
 template <int WA, int WB, int NWA, int NWB>
@@ -265,13 +268,11 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   const int l32 = lane & 31, kh = lane >> 5;
   const int wa = wave / NWB, wb = wave - wa * NWB;
 
-  const int tilesK = (p.K + BA - 1) / BA, tilesR = (p.FV + BB - 1) / BB;
-  const int tiles = tilesK * tilesR;
   const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int split = logical / tiles;
-  const int tile = logical - split * tiles;
-  const int rt = tile / tilesK;
-  const int k0 = (tile - rt * tilesK) * BA;
+  int split, tile, rt, kt;
+  p.byTiles.divmod(logical, &split, &tile);
+  p.byTilesK.divmod(tile, &rt, &kt);
+  const int k0 = kt * BA;
   const int r0 = rt * BB;
 
   const int HW = p.H * p.W;
@@ -281,17 +282,18 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
     const int R = r0 + tid;
     int2 e = make_int2(0, 0x8000);  // dh = -32768: never inside the image
     if (R < p.FV) {
-      const int c = R / p.T, t = R - c * p.T;
-      const int j = t / p.FH, i = t - j * p.FH;
+      int c, t, j, i;
+      p.byT.divmod(R, &c, &t);
+      p.byFH.divmod(t, &j, &i);
       const int dh = i * p.dly - p.pt, dw = j * p.dlx - p.pl;
       e = make_int2(c * HW + dh + p.H * dw, (int)((unsigned)(dh & 0xffff) | ((unsigned)dw << 16)));
     }
     rowTab[tid] = e;
   }
 
-  const long long mBegin = (long long)split * p.chunkSpan;
-  const long long mEnd = min(mBegin + p.chunkSpan, p.M);
-  const int nSteps = mEnd > mBegin ? (int)((mEnd - mBegin + BP - 1) / BP) : 0;
+  const int mBegin = split * p.chunkSpan;
+  const int mEnd = min(mBegin + p.chunkSpan, p.M);
+  const int nSteps = mEnd > mBegin ? (mEnd - mBegin + BP - 1) / BP : 0;
 
   const int px = tid & 31, rg = tid >> 5;
 
@@ -306,12 +308,11 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   float pa[APT], pb[BPT];
 
   auto fetch = [&](int step) {
-    const long long m = mBegin + (long long)step * BP + px;
+    const int m = mBegin + step * BP + px;
     const bool valid = m < mEnd;
-    const long long mc = valid ? m : mBegin;
-    const int n = (int)(mc / Q);
-    const int q = (int)(mc - (long long)n * Q);
-    const int ow = q / p.OH, oh = q - ow * p.OH;
+    int n, q, ow, oh;
+    p.byQ.divmod(valid ? m : mBegin, &n, &q);
+    p.byOH.divmod(q, &ow, &oh);
     const int ihB = oh * p.sy, iwB = ow * p.sx;
     const float* xN = x + (size_t)n * p.C * HW + ihB + p.H * iwB;
     const float* dyN = dy + (size_t)n * p.K * Q + q;
@@ -381,14 +382,28 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   }
 }
 
-// dF[e] = sum over splits, in ascending split order
+// dF[e] = sum over splits.  A workgroup owns 64 consecutive elements; thread (e, g) adds the splits
+// g, g+4, g+8, ... (four independent load streams per element, each unrolled), then the four partial sums
+// are combined through LDS in a fixed order.  Deterministic; ~splits/4 dependent loads per thread.
 __global__ __launch_bounds__(256) void conv_wgrad_reduce(float* __restrict__ df, const float* __restrict__ partials,
                                                          size_t n, int splits) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  float s = partials[i];
-  for (int k = 1; k < splits; ++k) s += partials[(size_t)k * n + i];
-  df[i] = s;
+  __shared__ float part[4][64];
+  const int e = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const size_t i = (size_t)blockIdx.x * 64 + e;
+  float s = 0.f;
+  if (i < n) {
+    int k = g;
+#pragma unroll 1
+    for (; k + 12 < splits; k += 16) {
+      const float a = partials[(size_t)k * n + i], b = partials[(size_t)(k + 4) * n + i];
+      const float c = partials[(size_t)(k + 8) * n + i], d = partials[(size_t)(k + 12) * n + i];
+      s += (a + b) + (c + d);
+    }
+    for (; k < splits; k += 4) s += partials[(size_t)k * n + i];
+  }
+  part[g][e] = s;
+  __syncthreads();
+  if (g == 0 && i < n) df[i] = (part[0][e] + part[1][e]) + (part[2][e] + part[3][e]);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -401,7 +416,7 @@ bool common_ok(const ConvP& p) {
   // tap offsets are packed as 16-bit fields and "row absent" is encoded as offset -32768
   const long long spanH = (long long)p.H + p.pt + (long long)p.FH * p.dy, spanW = (long long)p.W + p.pl + (long long)p.FW * p.dx;
   return p.groups == 1 && p.FH * p.FW <= kMaxTaps && spanH < 32768 && spanW < 32768 &&
-         (long long)p.outH * p.outW * p.N < (1ll << 40);
+         (long long)p.outH * p.outW * p.N < (1ll << 31) && (long long)p.H * p.W * p.N < (1ll << 31);
 }
 
 int wgrad_splits(const ConvP& p, int* tilesOut) {
@@ -419,7 +434,7 @@ int wgrad_splits(const ConvP& p, int* tilesOut) {
 template <int WA, int WB, int NWA, int NWB>
 void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, const PixP& p) {
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB;
-  const long long mTiles = (p.M + BB - 1) / BB;
+  const long long mTiles = ((long long)p.M + BB - 1) / BB;
   const int tilesA = (p.Cout + BA - 1) / BA;
   KernelTimer timer("conv_pix_mfma", s);
   hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB>), dim3((unsigned)(mTiles * tilesA)), dim3(256), 0, s, out, in,
@@ -462,11 +477,34 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
     rc = check_launch(who);
   }
   if (rc) return rc;
-  const long long blocks = ((p.M + (BA == 128 ? 127 : 255)) / (BA == 128 ? 128 : 256)) * (p.coutPad / BA);
-  if (blocks >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
-  if (BA == 128) launch_pix<2, 2, 2, 2>(s, out, in, wt, bias, p);
-  else if (BA == 64) launch_pix<2, 2, 1, 4>(s, out, in, wt, bias, p);
-  else launch_pix<1, 2, 1, 4>(s, out, in, wt, bias, p);
+  if (((long long)p.M / 64 + 1) * (p.coutPad / 32) >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
+  p.byQ = FastDiv(p.OH * p.OW);
+  p.byOH = FastDiv(p.OH);
+  p.byT = FastDiv(p.T);
+  p.advC = 16 / p.T;
+  p.advT = 16 % p.T;
+  // Tile shape, channels x pixels per workgroup: the widest pixel tile that still yields >= 2048 workgroups
+  // (8 per CU), because short reduction loops hide their load latency only through occupancy.  The tunable
+  // forces a shape for experiments.
+  int shape = tunable("conv_pix_tile", 0);
+  if (shape == 0) {
+    const long long tilesA = p.coutPad / BA;
+    auto blocks = [&](int px) { return (((long long)p.M + px - 1) / px) * tilesA; };
+    if (BA == 128) shape = blocks(128) >= 2048 ? 1 : 5;
+    else if (BA == 64) shape = blocks(256) >= 2048 ? 2 : (blocks(128) >= 2048 ? 4 : 6);
+    else shape = 3;
+  }
+  if ((shape == 1 || shape == 5) && BA != 128) shape = BA == 64 ? 2 : 3;
+  if ((shape == 2 || shape == 4 || shape == 6) && BA != 64) shape = BA == 128 ? 1 : 3;
+  if (shape == 3 && BA != 32) shape = BA == 128 ? 1 : 2;
+  switch (shape) {
+    case 1: launch_pix<2, 2, 2, 2>(s, out, in, wt, bias, p); break;  // 128 x 128
+    case 2: launch_pix<2, 2, 1, 4>(s, out, in, wt, bias, p); break;  //  64 x 256
+    case 3: launch_pix<1, 2, 1, 4>(s, out, in, wt, bias, p); break;  //  32 x 256
+    case 4: launch_pix<1, 2, 2, 2>(s, out, in, wt, bias, p); break;  //  64 x 128
+    case 5: launch_pix<2, 1, 2, 2>(s, out, in, wt, bias, p); break;  // 128 x  64
+    default: launch_pix<1, 1, 2, 2>(s, out, in, wt, bias, p); break; //  64 x  64
+  }
   return check_launch(who);
 }
 
@@ -510,7 +548,7 @@ int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, co
   q.dhBase = -p.pt; q.dhStep = p.dy; q.dwBase = -p.pl; q.dwStep = p.dx;
   q.R = q.T * q.Cin;
   q.coutPad = 0;
-  q.M = (long long)p.outH * p.outW * p.N;
+  q.M = p.outH * p.outW * p.N;
   q.alpha = inMult; q.beta = outMult;
   return run_pix(s, "mcn_conv_forward", y, x, f, b, q, 0, ws, wsBytes);
 }
@@ -526,7 +564,7 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, const floa
   q.dhBase = p.pt; q.dhStep = -p.dy; q.dwBase = p.pl; q.dwStep = -p.dx;
   q.R = q.T * q.Cin;
   q.coutPad = 0;
-  q.M = (long long)p.H * p.W * p.N;
+  q.M = p.H * p.W * p.N;
   q.alpha = 1.f; q.beta = 0.f;
   return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, 1, ws, wsBytes);
 }
@@ -539,11 +577,20 @@ int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const fl
   q.FH = p.FH; q.T = p.FH * p.FW;
   q.sy = p.sy; q.sx = p.sx; q.pt = p.pt; q.pl = p.pl; q.dly = p.dy; q.dlx = p.dx;
   q.FV = p.FH * p.FW * p.FC;
-  q.M = (long long)p.outH * p.outW * p.N;
+  q.M = p.outH * p.outW * p.N;
   int tiles = 0;
   q.splits = wgrad_splits(p, &tiles);
-  const long long chunks = (q.M + 31) / 32;
+  const int chunks = (q.M + 31) / 32;
   q.chunkSpan = ((chunks + q.splits - 1) / q.splits) * 32;
+  {
+    const int BAk = pick_channels_tile(p.K);
+    q.byQ = FastDiv(p.outH * p.outW);
+    q.byOH = FastDiv(p.outH);
+    q.byT = FastDiv(q.T);
+    q.byFH = FastDiv(p.FH);
+    q.byTiles = FastDiv(tiles);
+    q.byTilesK = FastDiv((p.K + BAk - 1) / BAk);
+  }
   const size_t nF = (size_t)q.FV * p.K;
   float* target = df;
   if (q.splits > 1) {
@@ -561,7 +608,7 @@ int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const fl
   if (!rc) rc = check_launch("mcn_conv_backward_filter");
   if (rc || q.splits == 1) return rc;
   KernelTimer timer("conv_wgrad_reduce", s);
-  hipLaunchKernelGGL(conv_wgrad_reduce, dim3((unsigned)((nF + 255) / 256)), block, 0, s, df, target, nF, q.splits);
+  hipLaunchKernelGGL(conv_wgrad_reduce, dim3((unsigned)((nF + 63) / 64)), block, 0, s, df, target, nF, q.splits);
   return check_launch("mcn_conv_backward_filter(reduce)");
 }
 
