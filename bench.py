@@ -189,8 +189,8 @@ def bench_pool_bwd(capi, workloads, reps):
         _sync()
         e, o = 4.0 * np.prod(shape), 4.0 * np.prod(oshape)
         nbytes = (2 * e + o) if method == "max" else (e + o)
-        t, _ = kernel_time(capi, "pool_backward_tiled", call, reps)
-        rows.append(dict(op=name, kernel="pool_backward_tiled", workload="configs[2] %s on %s" % (method, "x".join(map(str, shape))),
+        t, _ = kernel_time(capi, "pool_backward", call, reps)
+        rows.append(dict(op=name, kernel="pool_backward_passes", workload="configs[2] %s on %s" % (method, "x".join(map(str, shape))),
                          bound="hbm", achieved=nbytes / t / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=nbytes / t / PEAK_HBM,
                          avg_launch_us=t * 1e6, traffic=None))
     return rows

@@ -26,6 +26,7 @@ Tunable g_tunables[] = {
     {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)
     {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels
     {"conv_pix_tile", 0},              // force a tile shape of the pixel-major MFMA kernel (0 = automatic)
+    {"conv_no_uniform_tap", 0},        // 1: disable the uniform-tap variant of the pixel-major kernel
     {"conv_wgrad_blocks", 0},          // target workgroups for filter-gradient split (0 = 2 per CU)
     {"conv_bias_blocks", 0},           // target workgroups for the bias-gradient reduction
 };

@@ -52,28 +52,31 @@ struct PixP {
   int advC, advT;          // 16 = advC*T + advT (reduction rows per step)
 };
 
-// wt[R][co] from the MATLAB filter bank f[i,j,c,k] (FV x K, column-major).
-//   forward:        R = t + T*c, co = k : f[R + FV*k]
-//   backward-data:  R = t + T*k, co = c : f[t + T*(c + C*k)]
+// wt[R][co] from the MATLAB filter bank f[i,j,c,k] (FV x K, column-major), t = i + FH*j.
+//   reduction row R = t + T*ci (channel-major) or, when tapMajor, R = ci + Cin*t
+//   forward:        ci = c, co = k : f[t + T*c + FV*k]
+//   backward-data:  ci = k, co = c : f[t + T*(c + C*k)]
 __global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt, const float* __restrict__ f,
                                                          int T, int Cin, int Cout, int rPad, int coutPad,
-                                                         int backward) {
+                                                         int backward, int tapMajor) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (size_t)rPad * coutPad) return;
   const int r = (int)(idx / coutPad), co = (int)(idx - (size_t)r * coutPad);
   float v = 0.f;
   if (r < T * Cin && co < Cout) {
-    if (!backward) {
-      v = f[(size_t)r + (size_t)T * Cin * co];
-    } else {
-      const int k = r / T, t = r - k * T;
-      v = f[(size_t)t + (size_t)T * (co + (size_t)Cout * k)];
-    }
+    const int ci = tapMajor ? r % Cin : r / T;
+    const int t = tapMajor ? r / Cin : r % T;
+    v = backward ? f[(size_t)t + (size_t)T * (co + (size_t)Cout * ci)] : f[(size_t)t + (size_t)T * ci + (size_t)T * Cin * co];
   }
   wt[idx] = v;
 }
 
-template <int WA, int WB, int NWA, int NWB>
+// UT ("uniform tap"): the reduction runs tap-major (R = ci + Cin*t) and Cin is a multiple of 16, so all 16
+// rows of a step share one tap: the tap's shift and the inside-the-image test are computed once per step and
+// thread, the step's base address is uniform (scalar registers), and every gathered row is a load at a
+// per-thread constant 32-bit offset from it.  This removes almost all vector-ALU work from the loop, and
+// vector-ALU work is what competes with the MFMAs for the SIMD.
+template <int WA, int WB, int NWA, int NWB, bool UT>
 __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out, const float* __restrict__ in,
                                                         const float* __restrict__ wt,
                                                         const float* __restrict__ bias, PixP p) {
@@ -128,6 +131,15 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   int ciS, tapS;
   p.byT.divmod(pg * RPT, &ciS, &tapS);
   const int advC = p.advC, advT = p.advT;
+  // UT: per-thread constant element offsets (relative to `in`) of this thread's RPT channels at tap shift 0,
+  // and the uniform (tap, first channel) of the step being fetched
+  int offE[RPT];
+  int utTap = 0, utCi = 0;
+  if (UT) {
+    const int pix = (int)(inN - in);
+#pragma unroll
+    for (int e = 0; e < RPT; ++e) offE[e] = pix + (pg * RPT + e) * IHW;
+  }
 
   floatx16 acc[WA][WB];
 #pragma unroll
@@ -138,47 +150,80 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
   float pb[RPT];
-  float4 pa[APT];
+  float4 pa0 = make_float4(0.f, 0.f, 0.f, 0.f), pa1 = pa0;  // parked weight vectors (APT <= 2)
+  static_assert(APT <= 2, "at most two weight vectors per thread and step");
+  unsigned okMask = 0;  // bit e: gathered row e of the parked step lies inside the image
   const int nSteps = (p.R + BK - 1) / BK;
 
+  // Issues the global loads of one step and parks them in registers.  Straight-line on purpose: the tap
+  // table reads go out together, and rows that fall outside the image load a dummy (the tensor's first
+  // element) instead of branching, so all loads are in flight before anything waits; the mask zeroes them
+  // when they are written to LDS.
   auto fetch = [&](int step) {
-    int t = tapS, ci = ciS;
+    if (UT) {
+      const int2 tp = tapTab[utTap];
+      const int shift = __builtin_amdgcn_readfirstlane(tp.x), packed = __builtin_amdgcn_readfirstlane(tp.y);
+      const int ih = ihB + (int)(short)(packed & 0xffff), iw = iwB + (packed >> 16);
+      const bool ok = mvalid && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
+      const float* base = in + (utCi * IHW + shift);  // uniform
+      if (ok) {
 #pragma unroll
-    for (int e = 0; e < RPT; ++e) {
-      const int2 tp = tapTab[t];
-      const int ih = ihB + (int)(short)(tp.y & 0xffff);
-      const int iw = iwB + (tp.y >> 16);
-      const bool ok = mvalid && ci < p.Cin && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
-      pb[e] = ok ? inN[ci * IHW + tp.x] : 0.f;
-      if (++t == p.T) {
-        t = 0;
-        ++ci;
+        for (int e = 0; e < RPT; ++e) pb[e] = base[offE[e]];
+      } else {
+#pragma unroll
+        for (int e = 0; e < RPT; ++e) pb[e] = 0.f;
       }
-    }
-    ciS += advC;
-    tapS += advT;
-    if (tapS >= p.T) {
-      tapS -= p.T;
-      ++ciS;
+      utCi += BK;
+      if (utCi >= p.Cin) {
+        utCi = 0;
+        ++utTap;
+      }
+    } else {
+      int2 tp[RPT];
+      int cix[RPT];
+      int t = tapS, ci = ciS;
+#pragma unroll
+      for (int e = 0; e < RPT; ++e) {
+        tp[e] = tapTab[t];
+        cix[e] = ci;
+        if (++t == p.T) {
+          t = 0;
+          ++ci;
+        }
+      }
+      okMask = 0;
+#pragma unroll
+      for (int e = 0; e < RPT; ++e) {
+        const int ih = ihB + (int)(short)(tp[e].y & 0xffff);
+        const int iw = iwB + (tp[e].y >> 16);
+        const bool ok = mvalid && cix[e] < p.Cin && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
+        const float* src = ok ? inN + (cix[e] * IHW + tp[e].x) : in;
+        pb[e] = *src;
+        okMask |= ok ? (1u << e) : 0u;
+      }
+      ciS += advC;
+      tapS += advT;
+      if (tapS >= p.T) {
+        tapS -= p.T;
+        ++ciS;
+      }
     }
     const float* wrow = wt + (size_t)step * BK * p.coutPad + co0;
-#pragma unroll
-    for (int e = 0; e < APT; ++e) {
-      const int idx = tid + 256 * e;
-      if (A4 % 256 == 0 || idx < A4) {
-        const int row = idx / (BA / 4), c4 = idx - row * (BA / 4);
-        pa[e] = *(const float4*)(wrow + (size_t)row * p.coutPad + c4 * 4);
-      }
+    if (A4 % 256 == 0 || tid < A4) {
+      const int row = tid / (BA / 4), c4 = tid - row * (BA / 4);
+      pa0 = *(const float4*)(wrow + (size_t)row * p.coutPad + c4 * 4);
+    }
+    if (APT == 2) {
+      const int idx = tid + 256;
+      const int row = idx / (BA / 4), c4 = idx - row * (BA / 4);
+      pa1 = *(const float4*)(wrow + (size_t)row * p.coutPad + c4 * 4);
     }
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int e = 0; e < RPT; ++e) Bs[buf][(pg * RPT + e) * BB + mm] = pb[e];
-#pragma unroll
-    for (int e = 0; e < APT; ++e) {
-      const int idx = tid + 256 * e;
-      if (A4 % 256 == 0 || idx < A4) *(float4*)&As[buf][idx * 4] = pa[e];
-    }
+    for (int e = 0; e < RPT; ++e) Bs[buf][(pg * RPT + e) * BB + mm] = (UT || ((okMask >> e) & 1u)) ? pb[e] : 0.f;
+    if (A4 % 256 == 0 || tid < A4) *(float4*)&As[buf][tid * 4] = pa0;
+    if (APT == 2) *(float4*)&As[buf][(tid + 256) * 4] = pa1;
   };
 
   __syncthreads();  // tapTab ready
@@ -189,20 +234,29 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   for (int step = 0; step < nSteps; ++step) {
     const int buf = step & 1;
     if (step + 1 < nSteps) fetch(step + 1);
-    const float* Ab = As[buf] + wa * WA * 32 + l32;
-    const float* Bb = Bs[buf] + wb * WB * 32 + l32;
+    const float* Ab = As[buf] + wa * WA * 32 + l32 + kh * BA;
+    const float* Bb = Bs[buf] + wb * WB * 32 + l32 + kh * BB;
+    // operand fragments are read one reduction pair ahead of the MFMAs that consume them
+    float a[2][WA], b[2][WB];
+#pragma unroll
+    for (int ii = 0; ii < WA; ++ii) a[0][ii] = Ab[ii * 32];
+#pragma unroll
+    for (int jj = 0; jj < WB; ++jj) b[0][jj] = Bb[jj * 32];
 #pragma unroll
     for (int s = 0; s < BK / 2; ++s) {
-      float a[WA], b[WB];
+      const int cur = s & 1, nxt = cur ^ 1;
+      if (s + 1 < BK / 2) {
 #pragma unroll
-      for (int ii = 0; ii < WA; ++ii) a[ii] = Ab[(2 * s + kh) * BA + ii * 32];
+        for (int ii = 0; ii < WA; ++ii) a[nxt][ii] = Ab[(2 * s + 2) * BA + ii * 32];
 #pragma unroll
-      for (int jj = 0; jj < WB; ++jj) b[jj] = Bb[(2 * s + kh) * BB + jj * 32];
+        for (int jj = 0; jj < WB; ++jj) b[nxt][jj] = Bb[(2 * s + 2) * BB + jj * 32];
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the look-ahead reads ahead of this pair's MFMAs
 #pragma unroll
       for (int ii = 0; ii < WA; ++ii)
 #pragma unroll
         for (int jj = 0; jj < WB; ++jj)
-          acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii], b[jj], acc[ii][jj], 0, 0, 0);
+          acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][ii], b[cur][jj], acc[ii][jj], 0, 0, 0);
     }
     if (step + 1 < nSteps) stash(buf ^ 1);
     __syncthreads();
@@ -306,7 +360,10 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
   float pa[APT], pb[BPT];
+  unsigned okA = 0, okB = 0;
 
+  // Straight-line like the pixel-major kernel's: table reads first, then every load (absent elements read a
+  // dummy and are zeroed by mask when written to LDS).
   auto fetch = [&](int step) {
     const int m = mBegin + step * BP + px;
     const bool valid = m < mEnd;
@@ -316,25 +373,34 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
     const int ihB = oh * p.sy, iwB = ow * p.sx;
     const float* xN = x + (size_t)n * p.C * HW + ihB + p.H * iwB;
     const float* dyN = dy + (size_t)n * p.K * Q + q;
+    int2 tp[BPT];
+#pragma unroll
+    for (int e = 0; e < BPT; ++e) tp[e] = rowTab[rg + 8 * e];
+    okB = 0;
 #pragma unroll
     for (int e = 0; e < BPT; ++e) {
-      const int2 tp = rowTab[rg + 8 * e];
-      const int ih = ihB + (int)(short)(tp.y & 0xffff);
-      const int iw = iwB + (tp.y >> 16);
+      const int ih = ihB + (int)(short)(tp[e].y & 0xffff);
+      const int iw = iwB + (tp[e].y >> 16);
       const bool ok = valid && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
-      pb[e] = ok ? xN[tp.x] : 0.f;
+      const float* src = ok ? xN + tp[e].x : x;
+      pb[e] = *src;
+      okB |= ok ? (1u << e) : 0u;
     }
+    okA = 0;
 #pragma unroll
     for (int e = 0; e < APT; ++e) {
       const int k = k0 + rg + 8 * e;
-      pa[e] = (valid && k < p.K) ? dyN[(size_t)k * Q] : 0.f;
+      const bool ok = valid && k < p.K;
+      const float* src = ok ? dyN + (size_t)k * Q : dy;
+      pa[e] = *src;
+      okA |= ok ? (1u << e) : 0u;
     }
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int e = 0; e < BPT; ++e) Bs[buf][(rg + 8 * e) * LD + px] = pb[e];
+    for (int e = 0; e < BPT; ++e) Bs[buf][(rg + 8 * e) * LD + px] = ((okB >> e) & 1u) ? pb[e] : 0.f;
 #pragma unroll
-    for (int e = 0; e < APT; ++e) As[buf][(rg + 8 * e) * LD + px] = pa[e];
+    for (int e = 0; e < APT; ++e) As[buf][(rg + 8 * e) * LD + px] = ((okA >> e) & 1u) ? pa[e] : 0.f;
   };
 
   __syncthreads();  // rowTab ready
@@ -349,18 +415,26 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
     if (step + 1 < nSteps) fetch(step + 1);
     const float* Ab = As[buf] + (wa * WA * 32 + l32) * LD + kh;
     const float* Bb = Bs[buf] + (wb * WB * 32 + l32) * LD + kh;
+    float a[2][WA], b[2][WB];
+#pragma unroll
+    for (int ii = 0; ii < WA; ++ii) a[0][ii] = Ab[ii * 32 * LD];
+#pragma unroll
+    for (int jj = 0; jj < WB; ++jj) b[0][jj] = Bb[jj * 32 * LD];
 #pragma unroll
     for (int s = 0; s < BP / 2; ++s) {
-      float a[WA], b[WB];
+      const int cur = s & 1, nxt = cur ^ 1;
+      if (s + 1 < BP / 2) {
 #pragma unroll
-      for (int ii = 0; ii < WA; ++ii) a[ii] = Ab[ii * 32 * LD + 2 * s];
+        for (int ii = 0; ii < WA; ++ii) a[nxt][ii] = Ab[ii * 32 * LD + 2 * s + 2];
 #pragma unroll
-      for (int jj = 0; jj < WB; ++jj) b[jj] = Bb[jj * 32 * LD + 2 * s];
+        for (int jj = 0; jj < WB; ++jj) b[nxt][jj] = Bb[jj * 32 * LD + 2 * s + 2];
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the look-ahead reads ahead of this pair's MFMAs
 #pragma unroll
       for (int ii = 0; ii < WA; ++ii)
 #pragma unroll
         for (int jj = 0; jj < WB; ++jj)
-          acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii], b[jj], acc[ii][jj], 0, 0, 0);
+          acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][ii], b[cur][jj], acc[ii][jj], 0, 0, 0);
     }
     if (step + 1 < nSteps) stash(buf ^ 1);
     __syncthreads();
@@ -432,13 +506,14 @@ int wgrad_splits(const ConvP& p, int* tilesOut) {
 }
 
 template <int WA, int WB, int NWA, int NWB>
-void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, const PixP& p) {
+void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, const PixP& p, bool ut) {
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB;
   const long long mTiles = ((long long)p.M + BB - 1) / BB;
   const int tilesA = (p.Cout + BA - 1) / BA;
+  const dim3 grid((unsigned)(mTiles * tilesA));
   KernelTimer timer("conv_pix_mfma", s);
-  hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB>), dim3((unsigned)(mTiles * tilesA)), dim3(256), 0, s, out, in,
-                     wt, bias, p);
+  if (ut) hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB, true>), grid, dim3(256), 0, s, out, in, wt, bias, p);
+  else hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB, false>), grid, dim3(256), 0, s, out, in, wt, bias, p);
 }
 
 template <int WA, int WB, int NWA, int NWB>
@@ -469,11 +544,13 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   if (!aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
   float* wt = (float*)ws;
   const size_t nW = (size_t)rPad * p.coutPad;
+  // uniform-tap variant: whole 16-row steps inside one tap, and 32-bit element offsets into the gathered tensor
+  const bool ut = p.Cin % 16 == 0 && (long long)p.IH * p.IW * p.Cin * p.N < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
   int rc;
   {
     KernelTimer timer("conv_pack_weights", s);
     hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, wt, f, p.T, p.Cin, p.Cout,
-                       rPad, p.coutPad, backward);
+                       rPad, p.coutPad, backward, ut ? 1 : 0);
     rc = check_launch(who);
   }
   if (rc) return rc;
@@ -498,12 +575,12 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   if ((shape == 2 || shape == 4 || shape == 6) && BA != 64) shape = BA == 128 ? 1 : 3;
   if (shape == 3 && BA != 32) shape = BA == 128 ? 1 : 2;
   switch (shape) {
-    case 1: launch_pix<2, 2, 2, 2>(s, out, in, wt, bias, p); break;  // 128 x 128
-    case 2: launch_pix<2, 2, 1, 4>(s, out, in, wt, bias, p); break;  //  64 x 256
-    case 3: launch_pix<1, 2, 1, 4>(s, out, in, wt, bias, p); break;  //  32 x 256
-    case 4: launch_pix<1, 2, 2, 2>(s, out, in, wt, bias, p); break;  //  64 x 128
-    case 5: launch_pix<2, 1, 2, 2>(s, out, in, wt, bias, p); break;  // 128 x  64
-    default: launch_pix<1, 1, 2, 2>(s, out, in, wt, bias, p); break; //  64 x  64
+    case 1: launch_pix<2, 2, 2, 2>(s, out, in, wt, bias, p, ut); break;  // 128 x 128
+    case 2: launch_pix<2, 2, 1, 4>(s, out, in, wt, bias, p, ut); break;  //  64 x 256
+    case 3: launch_pix<1, 2, 1, 4>(s, out, in, wt, bias, p, ut); break;  //  32 x 256
+    case 4: launch_pix<1, 2, 2, 2>(s, out, in, wt, bias, p, ut); break;  //  64 x 128
+    case 5: launch_pix<2, 1, 2, 2>(s, out, in, wt, bias, p, ut); break;  // 128 x  64
+    default: launch_pix<1, 1, 2, 2>(s, out, in, wt, bias, p, ut); break; //  64 x  64
   }
   return check_launch(who);
 }
