@@ -298,10 +298,14 @@ struct WgP {
   int M;                 // OH*OW*N (< 2^31)
   int chunkSpan;         // pixels per split (multiple of 32)
   int splits;
-  FastDiv byQ, byOH, byT, byFH, byTiles, byTilesK;
+  FastDiv byQ, byOH, byT, byFH, byTiles, byTilesK, byC;
 };
 
-template <int WA, int WB, int NWA, int NWB>
+// UT ("uniform tap"): rows are ordered tap-major (R' = c + C*t) and C is a multiple of 32, so each 32-row MFMA
+// block lies inside one tap.  A thread's sixteen patch rows then need four inside-the-image tests per step
+// instead of sixteen, and every load is a per-thread constant 32-bit offset from a per-step pixel offset.
+// The partial banks come out in R' order; conv_wgrad_reduce puts them back in MATLAB order.
+template <int WA, int WB, int NWA, int NWB, bool UT>
 __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ out, const float* __restrict__ x,
                                                           const float* __restrict__ dy, WgP p) {
   static_assert(NWA * NWB == 4, "four wavefronts per workgroup");
@@ -332,7 +336,7 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   const int HW = p.H * p.W;
   const int Q = p.OH * p.OW;
 
-  if (tid < BB) {
+  if (!UT && tid < BB) {
     const int R = r0 + tid;
     int2 e = make_int2(0, 0x8000);  // dh = -32768: never inside the image
     if (R < p.FV) {
@@ -362,6 +366,32 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   float pa[APT], pb[BPT];
   unsigned okA = 0, okB = 0;
 
+  // UT: per 32-row block its tap shift (uniform), per thread the constant offsets of its rows
+  constexpr int NBLK = BB / 32;
+  int blkDh[NBLK], blkDw[NBLK];
+  int xOff[BPT], yOff[APT];
+  unsigned kPresent = 0;
+  if (UT) {
+#pragma unroll
+    for (int jb = 0; jb < NBLK; ++jb) {
+      const int Rb = r0 + 32 * jb;
+      int t, cb, j, i;
+      p.byC.divmod(Rb < p.FV ? Rb : 0, &t, &cb);
+      p.byFH.divmod(t, &j, &i);
+      const int dh = i * p.dly - p.pt, dw = j * p.dlx - p.pl;
+      blkDh[jb] = Rb < p.FV ? dh : -32768;  // absent block: never inside the image
+      blkDw[jb] = dw;
+#pragma unroll
+      for (int e4 = 0; e4 < 4; ++e4) xOff[4 * jb + e4] = (cb + rg + 8 * e4) * HW + dh + p.H * dw;
+    }
+#pragma unroll
+    for (int e = 0; e < APT; ++e) {
+      const int k = k0 + rg + 8 * e;
+      yOff[e] = (k < p.K ? k : 0) * Q;
+      kPresent |= k < p.K ? (1u << e) : 0u;
+    }
+  }
+
   // Straight-line like the pixel-major kernel's: table reads first, then every load (absent elements read a
   // dummy and are zeroed by mask when written to LDS).
   auto fetch = [&](int step) {
@@ -371,6 +401,31 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
     p.byQ.divmod(valid ? m : mBegin, &n, &q);
     p.byOH.divmod(q, &ow, &oh);
     const int ihB = oh * p.sy, iwB = ow * p.sx;
+    if (UT) {
+      const int pixX = n * (p.C * HW) + ihB + p.H * iwB;
+      const int pixY = n * (p.K * Q) + q;
+#pragma unroll
+      for (int jb = 0; jb < NBLK; ++jb) {
+        const bool ok = valid && (unsigned)(ihB + blkDh[jb]) < (unsigned)p.H && (unsigned)(iwB + blkDw[jb]) < (unsigned)p.W;
+        if (ok) {
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) pb[4 * jb + e4] = x[pixX + xOff[4 * jb + e4]];
+        } else {
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) pb[4 * jb + e4] = 0.f;
+        }
+      }
+      if (valid) {
+#pragma unroll
+        for (int e = 0; e < APT; ++e) pa[e] = dy[pixY + yOff[e]];
+      } else {
+#pragma unroll
+        for (int e = 0; e < APT; ++e) pa[e] = 0.f;
+      }
+      okA = kPresent;
+      okB = 0xffffffffu;
+      return;
+    }
     const float* xN = x + (size_t)n * p.C * HW + ihB + p.H * iwB;
     const float* dyN = dy + (size_t)n * p.K * Q + q;
     int2 tp[BPT];
@@ -396,11 +451,17 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
       okA |= ok ? (1u << e) : 0u;
     }
   };
+  const bool allK = k0 + BA <= p.K;  // uniform: no filter row of this tile is absent
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int e = 0; e < BPT; ++e) Bs[buf][(rg + 8 * e) * LD + px] = ((okB >> e) & 1u) ? pb[e] : 0.f;
+    for (int e = 0; e < BPT; ++e) Bs[buf][(rg + 8 * e) * LD + px] = (UT || ((okB >> e) & 1u)) ? pb[e] : 0.f;
+    if (UT && allK) {
 #pragma unroll
-    for (int e = 0; e < APT; ++e) As[buf][(rg + 8 * e) * LD + px] = ((okA >> e) & 1u) ? pa[e] : 0.f;
+      for (int e = 0; e < APT; ++e) As[buf][(rg + 8 * e) * LD + px] = pa[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < APT; ++e) As[buf][(rg + 8 * e) * LD + px] = ((okA >> e) & 1u) ? pa[e] : 0.f;
+    }
   };
 
   __syncthreads();  // rowTab ready
@@ -460,7 +521,7 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
 // g, g+4, g+8, ... (four independent load streams per element, each unrolled), then the four partial sums
 // are combined through LDS in a fixed order.  Deterministic; ~splits/4 dependent loads per thread.
 __global__ __launch_bounds__(256) void conv_wgrad_reduce(float* __restrict__ df, const float* __restrict__ partials,
-                                                         size_t n, int splits) {
+                                                         size_t n, int splits, int tapMajor, int C, int T) {
   __shared__ float part[4][64];
   const int e = threadIdx.x & 63, g = threadIdx.x >> 6;
   const size_t i = (size_t)blockIdx.x * 64 + e;
@@ -477,7 +538,16 @@ __global__ __launch_bounds__(256) void conv_wgrad_reduce(float* __restrict__ df,
   }
   part[g][e] = s;
   __syncthreads();
-  if (g == 0 && i < n) df[i] = (part[0][e] + part[1][e]) + (part[2][e] + part[3][e]);
+  if (g == 0 && i < n) {
+    size_t o = i;
+    if (tapMajor) {  // partial banks are indexed c + C*t + FV*k; MATLAB order is t + T*c + FV*k
+      const size_t FV = (size_t)C * T;
+      const size_t k = i / FV, r = i - k * FV;
+      const size_t t = r / C, c = r - t * C;
+      o = t + (size_t)T * c + FV * k;
+    }
+    df[o] = (part[0][e] + part[1][e]) + (part[2][e] + part[3][e]);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -491,6 +561,12 @@ bool common_ok(const ConvP& p) {
   const long long spanH = (long long)p.H + p.pt + (long long)p.FH * p.dy, spanW = (long long)p.W + p.pl + (long long)p.FW * p.dx;
   return p.groups == 1 && p.FH * p.FW <= kMaxTaps && spanH < 32768 && spanW < 32768 &&
          (long long)p.outH * p.outW * p.N < (1ll << 31) && (long long)p.H * p.W * p.N < (1ll << 31);
+}
+
+// the tap-major variant of the filter-gradient kernel: 32-row blocks inside one tap, 32-bit element offsets
+bool wgrad_uniform_tap(const ConvP& p) {
+  return p.C % 32 == 0 && (long long)p.H * p.W * p.C * p.N < (1ll << 31) &&
+         (long long)p.outH * p.outW * p.K * p.N < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
 }
 
 int wgrad_splits(const ConvP& p, int* tilesOut) {
@@ -516,13 +592,13 @@ void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, con
   else hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB, false>), grid, dim3(256), 0, s, out, in, wt, bias, p);
 }
 
-template <int WA, int WB, int NWA, int NWB>
+template <int WA, int WB, int NWA, int NWB, bool UT>
 int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const float* dy, const WgP& p) {
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB, LD = 33;
   constexpr size_t lds = (size_t)2 * (BA + BB) * LD * sizeof(float) + BB * sizeof(int2);
   static bool raised = false;  // one-time opt-in to more than 64 KB of LDS per workgroup
   if (lds > 64 * 1024 && !raised) {
-    if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB, UT>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return fail(MCN_DEVICE_ERROR, "mcn_conv_backward_filter: cannot reserve %zu bytes of LDS", lds);
@@ -530,7 +606,7 @@ int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const flo
     raised = true;
   }
   KernelTimer timer("conv_wgrad_mfma", s);
-  hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB>), grid, dim3(256), lds, s, out, x, dy, p);
+  hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB, UT>), grid, dim3(256), lds, s, out, x, dy, p);
   return MCN_SUCCESS;
 }
 
@@ -608,7 +684,7 @@ size_t conv_mfma_workspace_bytes(const ConvP& p, int product) {
     case MCN_CONV_BACKWARD_FILTER: {
       if (!conv_mfma_backward_filter_supported(p)) return 0;
       const int s = wgrad_splits(p, nullptr);
-      return s > 1 ? (size_t)s * FV * p.K * sizeof(float) : 0;
+      return (s > 1 || wgrad_uniform_tap(p)) ? (size_t)s * FV * p.K * sizeof(float) : 0;
     }
     default: return 0;
   }
@@ -669,8 +745,10 @@ int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const fl
     q.byTilesK = FastDiv((p.K + BAk - 1) / BAk);
   }
   const size_t nF = (size_t)q.FV * p.K;
+  const bool ut = wgrad_uniform_tap(p);
+  q.byC = FastDiv(p.C);
   float* target = df;
-  if (q.splits > 1) {
+  if (q.splits > 1 || ut) {
     const size_t need = (size_t)q.splits * nF * sizeof(float);
     if (!ws || wsBytes < need)
       return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: workspace too small (%zu < %zu bytes)", wsBytes, need);
@@ -679,13 +757,20 @@ int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const fl
   const dim3 grid((unsigned)(tiles * q.splits)), block(256);
   const int BA = pick_channels_tile(p.K);
   int rc;
-  if (BA == 128) rc = launch_wgrad<2, 2, 2, 2>(s, grid, target, x, dy, q);
-  else if (BA == 64) rc = launch_wgrad<2, 1, 1, 4>(s, grid, target, x, dy, q);
-  else rc = launch_wgrad<1, 1, 1, 4>(s, grid, target, x, dy, q);
+  if (ut) {
+    if (BA == 128) rc = launch_wgrad<2, 2, 2, 2, true>(s, grid, target, x, dy, q);
+    else if (BA == 64) rc = launch_wgrad<2, 1, 1, 4, true>(s, grid, target, x, dy, q);
+    else rc = launch_wgrad<1, 1, 1, 4, true>(s, grid, target, x, dy, q);
+  } else {
+    if (BA == 128) rc = launch_wgrad<2, 2, 2, 2, false>(s, grid, target, x, dy, q);
+    else if (BA == 64) rc = launch_wgrad<2, 1, 1, 4, false>(s, grid, target, x, dy, q);
+    else rc = launch_wgrad<1, 1, 1, 4, false>(s, grid, target, x, dy, q);
+  }
   if (!rc) rc = check_launch("mcn_conv_backward_filter");
-  if (rc || q.splits == 1) return rc;
+  if (rc || target == df) return rc;
   KernelTimer timer("conv_wgrad_reduce", s);
-  hipLaunchKernelGGL(conv_wgrad_reduce, dim3((unsigned)((nF + 63) / 64)), block, 0, s, df, target, nF, q.splits);
+  hipLaunchKernelGGL(conv_wgrad_reduce, dim3((unsigned)((nF + 63) / 64)), block, 0, s, df, target, nF, q.splits, ut ? 1 : 0,
+                     p.C, q.T);
   return check_launch("mcn_conv_backward_filter(reduce)");
 }
 
