@@ -1,0 +1,115 @@
+"""Host-side logic of the C++ operator layer, no GPU needed: tensor-shape rules, option parsing and the
+validation order / message texts of the vl_nnconv, vl_nnbnorm, vl_nnpool front-ends (which run before any
+device work), and the refusal of CPU tensors by the operators (this library has no CPU compute path)."""
+import numpy as np
+import pytest
+import torch
+
+
+@pytest.fixture(scope="module")
+def vl():
+    from matconvnet_amd import vlapi
+    vlapi.lib()
+    return vlapi
+
+
+def z(*mshape):
+    """CPU float tensor standing for a MATLAB array of size mshape."""
+    return torch.zeros(tuple(reversed(mshape)), dtype=torch.float32)
+
+
+def test_library_exports_the_harness_entry_points(vl):
+    L = vl.lib()
+    for name in ("vlh_call", "vlh_last_message", "vlh_pooling_backward", "vlh_bottleneck_create", "vlh_bottleneck_forward",
+                 "vlh_bottleneck_backward", "vlh_bottleneck_run", "vlh_cpu_tensor_is_refused"):
+        assert hasattr(L, name), name
+
+
+def test_cpu_tensors_pass_validation_then_are_refused(vl):
+    """Valid arguments on the CPU reach the operator, which reports VLE_Unsupported: nothing is computed on the
+    host behind the caller's back."""
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "pad", 1)
+    assert e.value.code == 1 and "GPU" in e.value.message
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnbnorm(z(8, 8, 4, 2), z(4), z(4))
+    assert e.value.code == 1
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnpool(z(8, 8, 4, 2), 2, "stride", 2)
+    assert e.value.code == 1
+    assert vl.lib().vlh_cpu_tensor_is_refused() == 1
+
+
+CONV_ERRORS = [
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5)), "There are less than three arguments."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "stride", 0), "At least one element of STRIDE is smaller than one."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "stride", [1, 2, 3]), "STRIDE has neither one nor two elements."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "pad", -1), "An element of PAD is negative."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "pad", [1, 2]), "PAD has neither one nor four elements."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "dilate", [1, 0]), "An element of DILATE is less than one."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "DiLaTe", [1, 1, 1]), "DILATE has neither one nor two elements."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "nosuchoption"), "Unknown option 'nosuchoption'."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "pad"), "Option 'Pad' requires an argument."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), z(6, 6, 5, 2), 3.0), "The option name is not a string (argument number 5)"),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), 3.0), "DATA and DEROUTPUT do not have compatible formats."),
+    ((z(8, 8, 4, 2), z(3, 3, 3, 5), z(5)), "The FILTERS depth does not divide the DATA depth."),
+    ((z(8, 8, 4, 2), z(3, 3, 2, 5), z(5)), "The number of filter groups does not divide the number of filters."),
+    ((z(8, 8, 4, 2), z(9, 3, 4, 5), z(5)), "FILTERS are larger than the DATA (including padding)."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), "dilate", 4), "FILTERS are larger than the DATA (including padding)."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(4)), "The number of elements of BIASES is not the same as the number of filters."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), z(6, 6, 5, 3)), "DEROUTPUT dimensions are incompatible with X and FILTERS."),
+    ((z(8, 8, 4, 2), z(3, 3, 4, 5), z(5), z(7, 6, 5, 2)), "DEROUTPUT dimensions are incompatible with X and FILTERS."),
+    ((z(8, 8, 4, 2), torch.zeros((5, 4, 3, 3), dtype=torch.float64), z(5)), "DATA and FILTERS do not have compatible formats."),
+]
+
+
+@pytest.mark.parametrize("args,message", CONV_ERRORS)
+def test_vl_nnconv_validation(vl, args, message):
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(*args)
+    assert e.value.message == message
+
+
+def test_vl_nnconv_empty_filters_are_reported_unsupported(vl):
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(z(8, 8, 4, 2), torch.zeros((0,)), z(4))
+    assert e.value.code == 1 and "FILTERS" in e.value.message
+
+
+BNORM_ERRORS = [
+    ((z(8, 8, 4, 2), z(4)), "The arguments are less than three."),
+    ((z(8, 8, 4, 2), z(3), z(4)), "The MULTIPLIERS size does not match the DATA depth."),
+    ((z(8, 8, 4, 2), z(4), z(5)), "The BIASES size does not match the DATA depth."),
+    ((z(8, 8, 4, 2), z(4), z(4), z(8, 8, 4, 3)), "DATA and DEROUTPUT do not have the same size."),
+    ((z(8, 8, 4, 2), z(4), z(4), "epsilon", [1.0, 2.0]), "EPSILON is not a plain scalar."),
+    ((z(8, 8, 4, 2), z(4), z(4), "moments", z(4, 3)), "The MOMENTS size does not match the DATA depth."),
+    ((z(8, 8, 4, 2), z(4), z(4), "momentz", z(4, 2)), "Unknown option 'momentz'."),
+]
+
+
+@pytest.mark.parametrize("args,message", BNORM_ERRORS)
+def test_vl_nnbnorm_validation(vl, args, message):
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnbnorm(*args)
+    assert e.value.message == message
+
+
+POOL_ERRORS = [
+    ((z(8, 8, 1, 1),), "The arguments are less than two."),
+    ((z(8, 8, 1, 1), [1, 2, 3]), "SIZE has neither one nor two elements."),
+    ((z(8, 8, 1, 1), 0), "A dimension of the pooling SIZE is void."),
+    ((z(8, 8, 1, 1), 9), "The pooling window is larger than the DATA (including padding)."),
+    ((z(8, 8, 1, 1), 3, "pad", 3), "A padding value is larger or equal to the size of the pooling window."),
+    ((z(8, 8, 1, 1), 3, "pad", [0, 0, 0, -1]), "An element of PAD is negative."),
+    ((z(8, 8, 1, 1), 2, "stride", [0, 1]), "At least one element of STRIDE is smaller than one."),
+    ((z(8, 8, 1, 1), 2, "method", "median"), "METHOD is not a supported method."),
+    ((z(8, 8, 1, 1), 2, "method", 3), "METHOD is not a string."),
+    ((z(8, 8, 1, 1), 2, z(3, 3, 1, 1), "stride", 2), "DEROUTPUT dimensions are incompatible with X and POOL."),
+]
+
+
+@pytest.mark.parametrize("args,message", POOL_ERRORS)
+def test_vl_nnpool_validation(vl, args, message):
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnpool(*args)
+    assert e.value.message == message

@@ -26,6 +26,9 @@ CASES = [
     (28, 28, 48, 3, 1, 1, 48, 24, 1, 0, 1),
     (17, 13, 5, 3, 5, 5, 5, 7, 1, 2, 1),                    # odd everything
     (6, 6, 3, 2, 6, 6, 3, 4, 1, 0, 1),                      # 1x1 output (the reference's FC special case)
+    (20, 18, 32, 2, 3, 3, 32, 40, (2, 1), (1, 0, 2, 1), (1, 2)),  # 32 channels: tap-major kernels with stride + dilation
+    (13, 11, 64, 3, 2, 3, 64, 130, 1, (0, 1, 1, 1), 1),      # even-sized filter, 130 filters (partial channel tile)
+    (9, 9, 16, 2, 3, 3, 16, 16, (3, 3), 1, 1),               # 16 channels: tap-major forward only
 ]
 
 
@@ -93,6 +96,28 @@ def test_direct_and_mfma_paths_agree(capi, ob):
     finally:
         capi.set_tunable("conv_force_direct", 0)
     for a, w in zip(fast, slow):
+        assert rel_max(a, w) <= TOL
+
+
+@pytest.mark.parametrize("case", [(28, 28, 32, 4, 3, 3, 32, 48, 1, 1, 1), (20, 18, 32, 2, 3, 3, 32, 40, (2, 1), (1, 0, 2, 1), (1, 2)),
+                                  (14, 14, 64, 2, 1, 1, 64, 256, 1, 0, 1)])
+def test_tap_major_and_channel_major_kernels_agree(capi, ob, case):
+    """The uniform-tap (tap-major) MFMA kernels and the general channel-major ones are two orderings of the same
+    sums: both within the gate of the oracle and of each other."""
+    x, f, b = _tensors(case)
+    g = capi.conv_geom(x.shape, f.shape, *case[8:])
+    dy = F(np.random.default_rng(6).standard_normal(capi.conv_out_shape(g)))
+    xd, fd, dyd, bd = capi.to_device(x), capi.to_device(f), capi.to_device(dy), capi.to_device(b)
+    fast = [capi.to_host(t) for t in capi.conv_backward(xd, fd, dyd, g)] + [capi.to_host(capi.conv_forward(xd, fd, bd, g))]
+    try:
+        capi.set_tunable("conv_no_uniform_tap", 1)
+        slow = [capi.to_host(t) for t in capi.conv_backward(xd, fd, dyd, g)] + [capi.to_host(capi.conv_forward(xd, fd, bd, g))]
+    finally:
+        capi.set_tunable("conv_no_uniform_tap", 0)
+    for a, w in zip(fast, slow):
+        assert rel_max(a, w) <= TOL
+    og = ob.conv_geom(x.shape, f.shape, *case[8:])
+    for a, w in zip(slow[:3], ob.conv_backward(x, f, dy, og)):
         assert rel_max(a, w) <= TOL
 
 
