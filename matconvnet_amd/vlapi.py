@@ -42,7 +42,7 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise RuntimeError("%s is missing: build it with `python -m matconvnet_amd.build`" % LIB_PATH)
-        L = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+        L = C.CDLL(LIB_PATH)
         L.vlh_call.restype = C.c_int
         L.vlh_call.argtypes = [C.c_char_p, C.c_int, C.POINTER(Arg), C.c_int, C.POINTER(Arg), ALLOC_FN, C.c_void_p, C.c_void_p]
         L.vlh_last_message.restype = C.c_char_p
