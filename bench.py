@@ -44,7 +44,7 @@ def kernel_time(capi, kernel, launch, reps):
 def bench_block(vlapi, capi, workloads, steps, warmup):
     w = workloads.bottleneck_case()
     N = w["x"].shape[3]
-    blk = vlapi.Bottleneck(N=N, eps=w["eps"])
+    blk = vlapi.Bottleneck(N=N, eps=w["eps"], fused=True)
     for k in ("x", "f1", "f2", "f3", "g1", "b1", "g2", "b2", "g3", "b3"):
         blk.set(k, w[k])
     blk.set("dzdy", w["dy"])

@@ -143,6 +143,16 @@ MCN_API int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, con
                               const float* multipliers, const float* biases, int H, int W, int C, int N,
                               double epsilon, int givenMoments, void* workspace, size_t workspaceBytes);
 
+/* Same as mcn_bnorm_forward with the element-wise layers that usually follow folded into the output pass:
+   y = act(bnorm(x) [+ residual]), act = ReLU when relu != 0 (matlab/vl_nnrelu.m:43-48), residual added as
+   matlab/+dagnn/Sum.m:11-17 would.  Every element takes the same roundings as with separate calls, so the
+   result is bit-identical to mcn_bnorm_forward + mcn_add + mcn_relu_forward; two passes over the tensor are
+   saved per folded layer.  No counterpart in the reference, which runs these layers one by one. */
+MCN_API int mcn_bnorm_forward_fused(mcn_stream_t stream, float* y, float* moments, const float* x,
+                                    const float* multipliers, const float* biases, const float* residual,
+                                    int relu, int H, int W, int C, int N, double epsilon, int givenMoments,
+                                    void* workspace, size_t workspaceBytes);
+
 /* dzdx (H x W x C x N), dzdg (C), dzdb (C), all fully overwritten.  givenMoments == 0: BatchNorm::backward
    (bits/nnbnorm.cu:307-365), moments written if non-NULL.  givenMoments != 0: backwardWithMoment (:263-305). */
 MCN_API int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers,

@@ -10,7 +10,7 @@
 namespace vl { namespace harness {
 
 Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon)
-    : H(H), W(W), C(C), M(M), N(N), epsilon(epsilon), error(VLE_Success), stageHook(NULL), hookUser(NULL) {
+    : H(H), W(W), C(C), M(M), N(N), epsilon(epsilon), error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false) {
   const TensorShape big(H, W, C, N), small(H, W, M, N);
   // inputs and parameters
   make("x", big); make("dzdy", big);
@@ -102,6 +102,21 @@ ErrorCode Bottleneck::forward() {
   nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, 1, 1, 1, 1, 1, 1, 1, 1);
   nn::BatchNorm bn(context, epsilon);
   const std::size_t nSmall = slot("a1").getNumElements(), nBig = slot("a3").getNumElements();
+  if (fused) {
+    const size_t wsSmall = mcn_bnorm_workspace_bytes(H, W, M, N), wsBig = mcn_bnorm_workspace_bytes(H, W, C, N);
+    void* ws = context.getWorkspace(VLDT_GPU, wsBig > wsSmall ? wsBig : wsSmall);
+    if (!ws) return fail(context.getLastError(), "workspace");
+    STEP("conv1_fwd", c1.forward(slot("a1"), 0, slot("x"), 1, slot("f1"), none));
+    ABI("bn1_fwd", mcn_bnorm_forward_fused(st, buffer("r1"), buffer("m1"), buffer("a1"), buffer("g1"), buffer("b1"), NULL, 1,
+                                           H, W, M, N, epsilon, 0, ws, wsSmall));
+    STEP("conv2_fwd", c2.forward(slot("a2"), 0, slot("r1"), 1, slot("f2"), none));
+    ABI("bn2_fwd", mcn_bnorm_forward_fused(st, buffer("r2"), buffer("m2"), buffer("a2"), buffer("g2"), buffer("b2"), NULL, 1,
+                                           H, W, M, N, epsilon, 0, ws, wsSmall));
+    STEP("conv3_fwd", c1.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
+    ABI("bn3_fwd", mcn_bnorm_forward_fused(st, buffer("y"), buffer("m3"), buffer("a3"), buffer("g3"), buffer("b3"), buffer("x"), 1,
+                                           H, W, C, N, epsilon, 0, ws, wsBig));
+    return VLE_Success;
+  }
   STEP("conv1_fwd", c1.forward(slot("a1"), 0, slot("x"), 1, slot("f1"), none));
   STEP("bn1_fwd", bn.forward(slot("n1"), slot("m1"), slot("a1"), slot("g1"), slot("b1")));
   ABI("relu1_fwd", mcn_relu_forward(st, buffer("r1"), buffer("n1"), nSmall));
@@ -122,14 +137,18 @@ ErrorCode Bottleneck::backward() {
   nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, 1, 1, 1, 1, 1, 1, 1, 1);
   nn::BatchNorm bn(context, epsilon);
   const std::size_t nSmall = slot("a1").getNumElements(), nBig = slot("a3").getNumElements();
-  ABI("relu3_bwd", mcn_relu_backward(st, buffer("ds"), buffer("s"), buffer("dzdy"), nBig));
+  // ReLU masks: the layer's input, or (fused mode) its output -- max(v, 0) > 0 exactly when v > 0
+  char const* mask3 = fused ? "y" : "s";
+  char const* mask2 = fused ? "r2" : "n2";
+  char const* mask1 = fused ? "r1" : "n1";
+  ABI("relu3_bwd", mcn_relu_backward(st, buffer("ds"), buffer(mask3), buffer("dzdy"), nBig));
   // the sum passes ds to both of its inputs: the branch (n3) and the shortcut (x)
   STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot("ds")));
   STEP("conv3_bwd", c1.backward(slot("dr2"), slot("df3"), none, slot("r2"), slot("f3"), slot("da3")));
-  ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer("n2"), buffer("dr2"), nSmall));
+  ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer(mask2), buffer("dr2"), nSmall));
   STEP("bn2_bwd", bn.backwardWithMoment(slot("da2"), slot("dg2"), slot("db2"), slot("m2"), slot("a2"), slot("g2"), slot("b2"), slot("dn2")));
   STEP("conv2_bwd", c2.backward(slot("dr1"), slot("df2"), none, slot("r1"), slot("f2"), slot("da2")));
-  ABI("relu1_bwd", mcn_relu_backward(st, buffer("dn1"), buffer("n1"), buffer("dr1"), nSmall));
+  ABI("relu1_bwd", mcn_relu_backward(st, buffer("dn1"), buffer(mask1), buffer("dr1"), nSmall));
   STEP("bn1_bwd", bn.backwardWithMoment(slot("da1"), slot("dg1"), slot("db1"), slot("m1"), slot("a1"), slot("g1"), slot("b1"), slot("dn1")));
   STEP("conv1_bwd", c1.backward(slot("dxm"), slot("df1"), none, slot("x"), slot("f1"), slot("da1")));
   ABI("sum_bwd", mcn_add(st, buffer("dzdx"), buffer("dxm"), buffer("ds"), nBig));

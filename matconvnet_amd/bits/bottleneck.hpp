@@ -27,6 +27,10 @@ class Bottleneck {
   float* buffer(std::string const& name, std::size_t* count = NULL);
   ErrorCode setStream(void* stream);
 
+  // fused = true: batch-norm forward applies the ReLU (and, for the last one, the shortcut sum) in its output
+  // pass (mcn_bnorm_forward_fused); the un-activated tensors n1, n2, n3, s are then never written and the
+  // ReLU derivatives take their masks from r1, r2, y.  Results are bit-identical to the layer-by-layer mode.
+  void setFused(bool on) { fused = on; }
   ErrorCode forward();
   ErrorCode backward();
 
@@ -49,6 +53,7 @@ class Bottleneck {
   std::string message;
   StageHook stageHook;
   void* hookUser;
+  bool fused;
 };
 
 } }  // namespace vl::harness

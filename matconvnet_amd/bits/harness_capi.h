@@ -42,6 +42,8 @@ VLH_API void* vlh_bottleneck_create(int H, int W, int C, int M, int N, double ep
 VLH_API void vlh_bottleneck_destroy(void* block);
 VLH_API float* vlh_bottleneck_buffer(void* block, const char* name, size_t* count);
 VLH_API int vlh_bottleneck_set_stream(void* block, void* stream);
+/* fused != 0: batch-norm forward also applies the ReLU / shortcut sum that follows it (same bits, fewer passes) */
+VLH_API void vlh_bottleneck_set_fused(void* block, int fused);
 VLH_API int vlh_bottleneck_forward(void* block);
 VLH_API int vlh_bottleneck_backward(void* block);
 /* runs `steps` forward+backward passes; if stage != NULL the launches of that stage are bracketed by HIP

@@ -146,9 +146,10 @@ static void benchCopy(int warmup, int iters) {
               2.0 * n * 4 / t / 1e6, 100 * 2.0 * n * 4 / (t * 1e-3) / kPeakHbm, n * 4, n * 4);
 }
 
-static void benchBlock(int warmup, int iters) {
+static void benchBlock(int warmup, int iters, bool fused) {
   const int H = 56, W = 56, C = 256, M = 64, N = 32;
   harness::Bottleneck block(H, W, C, M, N, 1e-5);
+  block.setFused(fused);
   if (!block.ok()) {
     std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
     std::exit(3);
@@ -175,8 +176,8 @@ static void benchBlock(int warmup, int iters) {
       std::exit(3);
     }
   }, warmup, iters);
-  std::printf("%-28s %8.3f ms/step %9.0f images/s (fwd+bwd, N = %d, 41.93 GFLOP of convolution per step)\n",
-              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N);
+  std::printf("%-28s %8.3f ms/step %9.0f images/s (fwd+bwd, N = %d, 41.93 GFLOP of convolution per step; %s)\n",
+              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, fused ? "relu/sum folded into bnorm" : "layer by layer");
 }
 
 int main(int argc, char** argv) {
@@ -200,7 +201,10 @@ int main(int argc, char** argv) {
   if (want("bnorm")) benchBnorm(warmup, iters);
   if (want("maxpool")) benchPool(true, warmup, iters);
   if (want("avgpool")) benchPool(false, warmup, iters);
-  if (want("block")) benchBlock(warmup, iters);
+  if (want("block")) {
+    benchBlock(warmup, iters, false);
+    benchBlock(warmup, iters, true);
+  }
   if (want("conv5")) benchConv("conv 3x3x256x256 56x56 N=64", 56, 56, 256, 64, 3, 256, 1, warmup, iters);
   return 0;
 }

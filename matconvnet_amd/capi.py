@@ -54,6 +54,7 @@ PROTOTYPES = {
     "mcn_conv_backward_bias": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _sz]),
     "mcn_bnorm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mcn_bnorm_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
+    "mcn_bnorm_forward_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_bnorm_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_pool_output_size": (_i, [C.POINTER(PoolGeom), C.POINTER(_i), C.POINTER(_i)]),
     "mcn_pool_forward": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp]),
@@ -252,6 +253,17 @@ def bnorm_forward(x, g, b, eps=1e-4, moments=None, ws=None):
     mom = moments if given else empty((Cc, 2))
     wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
     check(lib().mcn_bnorm_forward(stream(), ptr(y), ptr(mom), ptr(x), ptr(g), ptr(b), H, W, Cc, N, eps, int(given), wp, wn))
+    return y, mom
+
+
+def bnorm_forward_fused(x, g, b, residual=None, relu=False, eps=1e-4, ws=None):
+    ws = ws or _ws
+    H, W, Cc, N = _hwcn(x)
+    y = empty((H, W, Cc, N))
+    mom = empty((Cc, 2))
+    wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
+    check(lib().mcn_bnorm_forward_fused(stream(), ptr(y), ptr(mom), ptr(x), ptr(g), ptr(b), ptr(residual), int(relu),
+                                        H, W, Cc, N, eps, 0, wp, wn))
     return y, mom
 
 

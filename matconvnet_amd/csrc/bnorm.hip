@@ -225,13 +225,47 @@ __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ 
   stream_planes<true, VEC4>(dx, dy, x, (float)G1, (float)(-G2), (float)(G2 * mean - G1 * muz), p, c, n0, n1);
 }
 
-// Forward apply: y = (g/sigma)*(x - mean) + b  (bits/nnbnorm.cu:190-199)
-template <bool GIVEN, bool VEC4>
+// out = act(a*in + k [+ res]) over this workgroup's planes: the forward apply with the element-wise layers
+// that follow it folded in.  Each element goes through the same roundings as the separate kernels would
+// give it: fma, then add, then max.
+template <bool RES, bool RELU, bool VEC4>
+__device__ __forceinline__ void stream_forward(float* __restrict__ out, const float* __restrict__ in,
+                                               const float* __restrict__ res, float a, float k, const BnormP& p,
+                                               int c, int n0, int n1) {
+  auto one = [&](float u, float r) -> float {
+    float v = fmaf(a, u, k);
+    if (RES) v = v + r;
+    if (RELU) v = v > 0.f ? v : 0.f;
+    return v;
+  };
+  for (int nn = n0; nn < n1; ++nn) {
+    const int n = p.reverse ? (n1 - 1 - (nn - n0)) : nn;
+    const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
+    if (VEC4) {
+      const float4* s1 = (const float4*)(in + base);
+      const float4* s2 = (const float4*)((RES ? res : in) + base);
+      float4* o4 = (float4*)(out + base);
+      for (int i = threadIdx.x; i < p.WH / 4; i += 256) {
+        const float4 u = s1[i];
+        float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (RES) r = s2[i];
+        o4[i] = make_float4(one(u.x, r.x), one(u.y, r.y), one(u.z, r.z), one(u.w, r.w));
+      }
+    } else {
+      for (int i = threadIdx.x; i < p.WH; i += 256) out[base + i] = one(in[base + i], RES ? res[base + i] : 0.f);
+    }
+  }
+}
+
+// Forward apply: y = (g/sigma)*(x - mean) + b  (bits/nnbnorm.cu:190-199), optionally followed by "+ residual"
+// (matlab/+dagnn/Sum.m) and ReLU (matlab/vl_nnrelu.m) in the same pass.
+template <bool GIVEN, bool VEC4, bool RES, bool RELU>
 __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y,
                                                            float* __restrict__ moments,
                                                            const float* __restrict__ x,
                                                            const float* __restrict__ mult,
                                                            const float* __restrict__ bias,
+                                                           const float* __restrict__ residual,
                                                            const double* __restrict__ partials,
                                                            BnormP p) {
   __shared__ double lds[4];
@@ -257,7 +291,7 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
   const double coef = (double)mult[c] / sigma;
   int n0, n1;
   image_range(p, grp, &n0, &n1);
-  stream_planes<false, VEC4>(y, x, nullptr, (float)coef, 0.f, (float)((double)bias[c] - coef * mean), p, c, n0, n1);
+  stream_forward<RES, RELU, VEC4>(y, x, residual, (float)coef, (float)((double)bias[c] - coef * mean), p, c, n0, n1);
 }
 
 int image_groups(int WH, int N) {
@@ -293,9 +327,9 @@ size_t mcn_bnorm_workspace_bytes(int H, int W, int C, int N) {
   return (size_t)C * image_groups(H * W, N) * 4 * sizeof(double);
 }
 
-int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,
-                      const float* biases, int H, int W, int C, int N, double epsilon, int givenMoments,
-                      void* workspace, size_t workspaceBytes) {
+int mcn_bnorm_forward_fused(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,
+                            const float* biases, const float* residual, int relu, int H, int W, int C, int N,
+                            double epsilon, int givenMoments, void* workspace, size_t workspaceBytes) {
   BnormP p;
   int rc = setup("mcn_bnorm_forward", H, W, C, N, epsilon, &p);
   if (rc) return rc;
@@ -303,7 +337,7 @@ int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float
   if (!y || !x || !multipliers || !biases) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward: null tensor");
   if (givenMoments && !moments) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward: moments are required");
   hipStream_t s = as_stream(stream);
-  const bool vec = (p.WH % 4 == 0) && aligned16(y) && aligned16(x);
+  const bool vec = (p.WH % 4 == 0) && aligned16(y) && aligned16(x) && (!residual || aligned16(residual));
   const dim3 grid((unsigned)(C * p.groups)), block(256);
   double* partials = (double*)workspace;
   if (!givenMoments) {
@@ -315,16 +349,37 @@ int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float
       else hipLaunchKernelGGL((bnorm_sums<0, false>), grid, block, 0, s, x, x, partials, p);
     }
     if ((rc = check_launch("mcn_bnorm_forward(sums)"))) return rc;
-    KernelTimer timer("bnorm_forward_apply", s);
-    if (vec) hipLaunchKernelGGL((bnorm_forward_apply<false, true>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
-    else hipLaunchKernelGGL((bnorm_forward_apply<false, false>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
   } else {
     p.reverse = 0;
-    KernelTimer timer("bnorm_forward_apply", s);
-    if (vec) hipLaunchKernelGGL((bnorm_forward_apply<true, true>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
-    else hipLaunchKernelGGL((bnorm_forward_apply<true, false>), grid, block, 0, s, y, moments, x, multipliers, biases, partials, p);
   }
+  KernelTimer timer("bnorm_forward_apply", s);
+#define MCN_BN_FWD(GIVENF, VECF, RESF, RELUF)                                                                      \
+  hipLaunchKernelGGL((bnorm_forward_apply<GIVENF, VECF, RESF, RELUF>), grid, block, 0, s, y, moments, x, multipliers, \
+                     biases, residual, partials, p)
+#define MCN_BN_FWD_EPI(GIVENF, VECF)                        \
+  do {                                                      \
+    if (residual && relu) MCN_BN_FWD(GIVENF, VECF, true, true);   \
+    else if (residual) MCN_BN_FWD(GIVENF, VECF, true, false);     \
+    else if (relu) MCN_BN_FWD(GIVENF, VECF, false, true);         \
+    else MCN_BN_FWD(GIVENF, VECF, false, false);                  \
+  } while (0)
+  if (givenMoments) {
+    if (vec) MCN_BN_FWD_EPI(true, true);
+    else MCN_BN_FWD_EPI(true, false);
+  } else {
+    if (vec) MCN_BN_FWD_EPI(false, true);
+    else MCN_BN_FWD_EPI(false, false);
+  }
+#undef MCN_BN_FWD_EPI
+#undef MCN_BN_FWD
   return check_launch("mcn_bnorm_forward");
+}
+
+int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,
+                      const float* biases, int H, int W, int C, int N, double epsilon, int givenMoments,
+                      void* workspace, size_t workspaceBytes) {
+  return mcn_bnorm_forward_fused(stream, y, moments, x, multipliers, biases, NULL, 0, H, W, C, N, epsilon,
+                                 givenMoments, workspace, workspaceBytes);
 }
 
 int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases, float* moments,

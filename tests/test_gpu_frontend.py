@@ -255,3 +255,36 @@ def test_bottleneck_block_full_config_stage_by_stage(vl, ob):
         assert rel_max(G["y"], want_y) < 2e-4
     finally:
         blk.close()
+
+
+def test_bottleneck_fused_mode_is_bit_identical(vl, ob):
+    """Folding ReLU and the shortcut sum into the batch-norm output pass changes no bit of any output."""
+    w = workloads.bottleneck_case(N=4)
+    outs = {}
+    shapes = dict(y=w["x"].shape, dzdx=w["x"].shape, df1=w["f1"].shape, df2=w["f2"].shape, df3=w["f3"].shape,
+                  dg1=(64,), db1=(64,), dg2=(64,), db2=(64,), dg3=(256,), db3=(256,), m1=(64, 2), m3=(256, 2))
+    for fused in (False, True):
+        blk = vl.Bottleneck(N=4, eps=w["eps"], fused=fused)
+        try:
+            _load(blk, w)
+            blk.forward()
+            blk.backward()
+            outs[fused] = {k: blk.get(k, v) for k, v in shapes.items()}
+        finally:
+            blk.close()
+    for k in shapes:
+        assert bits_equal(outs[False][k], outs[True][k]), k
+
+
+def test_bnorm_forward_fused_matches_separate_calls(capi, ob):
+    w = workloads.bnorm_case(seed=5, H=14, W=14, C=8, N=3)
+    res = F(np.random.default_rng(6).standard_normal(w["x"].shape))
+    xd, gd, bd, rd = capi.to_device(w["x"]), capi.to_device(w["g"]), capi.to_device(w["b"]), capi.to_device(res)
+    y0, m0 = capi.bnorm_forward(xd, gd, bd, 1e-4)
+    want = capi.relu_forward(capi.add(y0, rd))
+    got, m1 = capi.bnorm_forward_fused(xd, gd, bd, residual=rd, relu=True, eps=1e-4)
+    assert bits_equal(capi.to_host(got), capi.to_host(want)) and bits_equal(capi.to_host(m1), capi.to_host(m0))
+    got, _ = capi.bnorm_forward_fused(xd, gd, bd, relu=True, eps=1e-4)
+    assert bits_equal(capi.to_host(got), capi.to_host(capi.relu_forward(y0)))
+    got, _ = capi.bnorm_forward_fused(xd, gd, bd, residual=rd, eps=1e-4)
+    assert bits_equal(capi.to_host(got), capi.to_host(capi.add(y0, rd)))
