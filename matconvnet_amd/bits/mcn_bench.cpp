@@ -3,12 +3,18 @@
 // synthetic inputs, times them with HIP events and prints TFLOP/s, GB/s and images/s beside the
 // fraction of the MI355X rooflines (fp32 matrix 157.3 TFLOP/s, HBM 8 TB/s).
 //
-//   mcn_bench [--iters K] [--warmup W] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy]
+//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy]
+//
+// The bandwidth-bound operators (bnorm, pooling, copy) are timed over R independent sets of tensors used in
+// turn (default 4), so that no launch finds its inputs in the 256 MB memory-side cache because the previous
+// launch left them there: with R sets, more than 256 MB of other traffic passes between two uses of a buffer.
+// --rotate 1 gives the warm figure a loop over one set of buffers shows.
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <random>
 #include <string>
 #include <vector>
@@ -54,6 +60,23 @@ struct DeviceTensor {
     std::vector<float> host(view.getNumElements(), v);
     HIP_OK(hipMemcpy(view.getMemory(), host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice));
   }
+};
+
+static int gRotate = 4;
+
+// R device tensors of one shape holding the same values
+struct TensorSet {
+  std::vector<std::unique_ptr<DeviceTensor>> t;
+  TensorSet(TensorShape const& shape, int count) {
+    for (int i = 0; i < count; ++i) t.emplace_back(new DeviceTensor(shape));
+  }
+  void spread() {
+    for (size_t i = 1; i < t.size(); ++i)
+      HIP_OK(hipMemcpy(t[i]->view.getMemory(), t[0]->view.getMemory(), t[0]->view.getNumElements() * sizeof(float),
+                       hipMemcpyDeviceToDevice));
+  }
+  DeviceTensor& first() { return *t[0]; }
+  Tensor& operator[](int i) { return t[i % t.size()]->view; }
 };
 
 template <typename F>
@@ -107,43 +130,61 @@ static void benchConv(char const* name, int H, int W, int C, int N, int F, int K
 static void benchBnorm(int warmup, int iters) {
   const int H = 56, W = 56, C = 256, N = 32;
   Context ctx;
-  DeviceTensor x(TensorShape(H, W, C, N)), dy(TensorShape(H, W, C, N)), dx(TensorShape(H, W, C, N));
+  TensorSet x(TensorShape(H, W, C, N), gRotate), dy(TensorShape(H, W, C, N), gRotate), dx(TensorShape(H, W, C, N), gRotate);
   DeviceTensor g(TensorShape(C, 1, 1, 1)), b(TensorShape(C, 1, 1, 1)), dg(TensorShape(C, 1, 1, 1)), db(TensorShape(C, 1, 1, 1)), m(TensorShape(C, 2, 1, 1));
-  x.randn(4, 1.3f, 0.5f);
-  dy.randn(5);
+  x.first().randn(4, 1.3f, 0.5f);
+  dy.first().randn(5);
+  x.spread();
+  dy.spread();
   g.fill(1.f);
   b.fill(0.f);
   nn::BatchNorm op(ctx, 1e-4);
   const double bytes = 5.0 * H * W * C * N * 4;
-  double t = medianMs([&] { check(ctx, op.backward(dx.view, dg.view, db.view, m.view, x.view, g.view, b.view, dy.view), "bnorm"); }, warmup, iters);
-  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; 5 tensor sweeps = %.1f MB)\n", "bnorm bwd 56x56x256x32", t * 1e3,
-              bytes / t / 1e6, 100 * bytes / (t * 1e-3) / kPeakHbm, bytes / 1e6);
+  int turn = 0;
+  double t = medianMs([&] {
+    check(ctx, op.backward(dx[turn], dg.view, db.view, m.view, x[turn], g.view, b.view, dy[turn]), "bnorm");
+    ++turn;
+  }, warmup, iters);
+  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; 5 tensor sweeps = %.1f MB; %d buffer sets in turn)\n",
+              "bnorm bwd 56x56x256x32", t * 1e3, bytes / t / 1e6, 100 * bytes / (t * 1e-3) / kPeakHbm, bytes / 1e6, gRotate);
 }
 
 static void benchPool(bool isMax, int warmup, int iters) {
   const int H = isMax ? 112 : 56, C = isMax ? 64 : 256, N = 32, P = isMax ? 3 : 2, pad = isMax ? 1 : 0;
   const int OH = (H + 2 * pad - P) / 2 + 1;
   Context ctx;
-  DeviceTensor x(TensorShape(H, H, C, N)), dy(TensorShape(OH, OH, C, N)), dx(TensorShape(H, H, C, N));
-  x.randn(6);
-  dy.randn(7);
+  TensorSet x(TensorShape(H, H, C, N), gRotate), dy(TensorShape(OH, OH, C, N), gRotate), dx(TensorShape(H, H, C, N), gRotate);
+  x.first().randn(6);
+  dy.first().randn(7);
+  x.spread();
+  dy.spread();
   nn::Pooling op(ctx, P, P, 2, 2, pad, pad, pad, pad, isMax ? nn::Pooling::Max : nn::Pooling::Average);
   const double e = (double)H * H * C * N * 4, o = (double)OH * OH * C * N * 4;
   const double bytes = isMax ? (2 * e + o) : (e + o);
-  double t = medianMs([&] { check(ctx, op.backwardOverwrite(dx.view, x.view, dy.view), "pool"); }, warmup, iters);
-  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; %.1f MB)\n", isMax ? "max-pool bwd 112x112x64x32" : "avg-pool bwd 56x56x256x32",
-              t * 1e3, bytes / t / 1e6, 100 * bytes / (t * 1e-3) / kPeakHbm, bytes / 1e6);
+  int turn = 0;
+  double t = medianMs([&] {
+    check(ctx, op.backwardOverwrite(dx[turn], x[turn], dy[turn]), "pool");
+    ++turn;
+  }, warmup, iters);
+  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; %.1f MB; %d buffer sets in turn)\n",
+              isMax ? "max-pool bwd 112x112x64x32" : "avg-pool bwd 56x56x256x32", t * 1e3, bytes / t / 1e6,
+              100 * bytes / (t * 1e-3) / kPeakHbm, bytes / 1e6, gRotate);
 }
 
 // A plain streaming copy of known size (ReLU of positive data): the yardstick the HBM byte counters of the
 // other kernels are scaled by.
 static void benchCopy(int warmup, int iters) {
   const size_t n = 64u << 20;  // 64 Mi floats: reads 256 MiB, writes 256 MiB
-  DeviceTensor a(TensorShape(n, 1, 1, 1)), b(TensorShape(n, 1, 1, 1));
-  a.fill(1.f);
-  double t = medianMs([&] { mcn_relu_forward(NULL, (float*)b.view.getMemory(), (float const*)a.view.getMemory(), n); }, warmup, iters);
-  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; reads %zu B, writes %zu B per launch)\n", "copy 256 MiB", t * 1e3,
-              2.0 * n * 4 / t / 1e6, 100 * 2.0 * n * 4 / (t * 1e-3) / kPeakHbm, n * 4, n * 4);
+  TensorSet a(TensorShape(n, 1, 1, 1), gRotate), b(TensorShape(n, 1, 1, 1), gRotate);
+  a.first().fill(1.f);
+  a.spread();
+  int turn = 0;
+  double t = medianMs([&] {
+    mcn_relu_forward(NULL, (float*)b[turn].getMemory(), (float const*)a[turn].getMemory(), n);
+    ++turn;
+  }, warmup, iters);
+  std::printf("%-28s %8.1f us %7.0f GB/s (%4.1f%% of HBM peak; reads %zu B, writes %zu B per launch; %d buffer sets in turn)\n",
+              "copy 256 MiB", t * 1e3, 2.0 * n * 4 / t / 1e6, 100 * 2.0 * n * 4 / (t * 1e-3) / kPeakHbm, n * 4, n * 4, gRotate);
 }
 
 static void benchBlock(int warmup, int iters, bool fused) {
@@ -187,8 +228,9 @@ int main(int argc, char** argv) {
     if (!std::strcmp(argv[i], "--iters") && i + 1 < argc) iters = std::atoi(argv[++i]);
     else if (!std::strcmp(argv[i], "--warmup") && i + 1 < argc) warmup = std::atoi(argv[++i]);
     else if (!std::strcmp(argv[i], "--only") && i + 1 < argc) only = argv[++i];
+    else if (!std::strcmp(argv[i], "--rotate") && i + 1 < argc) gRotate = std::max(1, std::atoi(argv[++i]));
     else {
-      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy]\n");
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy]\n");
       return 1;
     }
   }

@@ -152,10 +152,10 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
       const float4* s2 = (const float4*)(TWO ? in2 + base : in1 + base);
       float4* o4 = (float4*)(out + base);
       for (int i = threadIdx.x; i < p.WH / 4; i += 256) {
-        const float4 u = s1[i];
+        const float4 u = stream_load4(s1 + i);
         float4 r;
         if (TWO) {
-          const float4 v = s2[i];
+          const float4 v = stream_load4(s2 + i);
           r.x = fmaf(a, u.x, fmaf(b, v.x, k));
           r.y = fmaf(a, u.y, fmaf(b, v.y, k));
           r.z = fmaf(a, u.z, fmaf(b, v.z, k));
@@ -166,7 +166,7 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
           r.z = fmaf(a, u.z, k);
           r.w = fmaf(a, u.w, k);
         }
-        o4[i] = r;
+        stream_store4(o4 + i, r);
       }
     } else {
       for (int i = threadIdx.x; i < p.WH; i += 256) {
@@ -246,10 +246,10 @@ __device__ __forceinline__ void stream_forward(float* __restrict__ out, const fl
       const float4* s2 = (const float4*)((RES ? res : in) + base);
       float4* o4 = (float4*)(out + base);
       for (int i = threadIdx.x; i < p.WH / 4; i += 256) {
-        const float4 u = s1[i];
+        const float4 u = stream_load4(s1 + i);
         float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (RES) r = s2[i];
-        o4[i] = make_float4(one(u.x, r.x), one(u.y, r.y), one(u.z, r.z), one(u.w, r.w));
+        if (RES) r = stream_load4(s2 + i);
+        stream_store4(o4 + i, make_float4(one(u.x, r.x), one(u.y, r.y), one(u.z, r.z), one(u.w, r.w)));
       }
     } else {
       for (int i = threadIdx.x; i < p.WH; i += 256) out[base + i] = one(in[base + i], RES ? res[base + i] : 0.f);

@@ -21,6 +21,9 @@ struct Tunable {
 // Defaults are the values chosen from on-device sweeps; see the per-kernel comments where each is read.
 Tunable g_tunables[] = {
     {"pool_lds_bytes", 16 * 1024},     // LDS tile budget of the pooling-backward kernels
+    {"pool_no_stream", 0},             // 1: max pooling skips the streaming kernel
+    {"pool_walk", 0},                  // streaming kernel's tile order: 0 round-robin, 1 contiguous runs, 2 round-robin per XCD
+    {"pool_blocks_per_cu", 3},         // persistent workgroups per compute unit of the streaming kernel
     {"pool_force_gather", 0},          // 1: skip the ordered-pass kernel, use the general tiled gather
     {"bnorm_block_elems", 4096},       // minimum elements a bnorm reduction block should own
     {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)

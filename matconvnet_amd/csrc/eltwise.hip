@@ -33,13 +33,13 @@ __global__ __launch_bounds__(256) void eltwise_kernel(float* __restrict__ y, con
     const size_t n4 = n / 4;
     for (size_t i = t; i < n4; i += stride) {
       float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u, r;
-      if (OP != OP_FILL) u = ((const float4*)a)[i];
-      if (OP == OP_RELU_BWD || OP == OP_ADD) v = ((const float4*)b)[i];
+      if (OP != OP_FILL) u = stream_load4((const float4*)a + i);
+      if (OP == OP_RELU_BWD || OP == OP_ADD) v = stream_load4((const float4*)b + i);
       r.x = apply1<OP>(u.x, v.x, k);
       r.y = apply1<OP>(u.y, v.y, k);
       r.z = apply1<OP>(u.z, v.z, k);
       r.w = apply1<OP>(u.w, v.w, k);
-      ((float4*)y)[i] = r;
+      stream_store4((float4*)y + i, r);
     }
     for (size_t i = n4 * 4 + t; i < n; i += stride) {
       const float u = (OP != OP_FILL) ? a[i] : 0.f;

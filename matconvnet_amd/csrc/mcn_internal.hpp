@@ -77,6 +77,32 @@ __device__ __forceinline__ int xcd_contiguous_id(int bid, int nblocks) {
   return xcd * q + (xcd < r ? xcd : r) + i;
 }
 
+// 16-byte accesses for data that is touched once per kernel: the non-temporal hint keeps such streams from
+// displacing re-used lines (halos, accumulators being merged) in the L2 of each XCD.
+#ifndef MCN_NT_STORE
+#define MCN_NT_STORE 1
+#endif
+#ifndef MCN_NT_LOAD
+#define MCN_NT_LOAD 0
+#endif
+typedef float v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void stream_store4(float4* p, const float4 v) {
+#if MCN_NT_STORE
+  v4f t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, (v4f*)p);
+#else
+  *p = v;
+#endif
+}
+__device__ __forceinline__ float4 stream_load4(const float4* p) {
+#if MCN_NT_LOAD
+  const v4f t = __builtin_nontemporal_load((const v4f*)p);
+  return make_float4(t.x, t.y, t.z, t.w);
+#else
+  return *p;
+#endif
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

@@ -24,6 +24,10 @@
 #pragma clang fp contract(off)
 
 namespace mcn {
+
+bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, float* derInput,
+                                     const float* x, const float* derOutput, int accumulate);  // pool_stream.hip
+
 namespace {
 
 struct PoolP {
@@ -651,7 +655,7 @@ __global__ __launch_bounds__(256) void pool_backward_passes(float* __restrict__ 
 
   // ---- stream the accumulators out
   if (VEC4) {
-    for (int i = tid; i < nIn / 4; i += 256) ((float4*)out)[i] = ((const float4*)acc)[i];
+    for (int i = tid; i < nIn / 4; i += 256) stream_store4((float4*)out + i, ((const float4*)acc)[i]);
   } else {
     for (int i = tid; i < nIn; i += 256) out[i] = acc[i];
   }
@@ -844,7 +848,11 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
   const int passes = isMax ? kh * kw : p.poolH * p.poolW;
   const bool vecIn = (p.H % 4 == 0) && aligned16(derInput);
 
-  // ---- fast path: ordered passes.  Widest tile whose LDS fits the budget and whose outputs fit 4 per thread.
+  // ---- max pooling, plane height a multiple of 4: streaming kernel
+  if (isMax && pool_max_backward_stream_launch(s, g, p.outH, p.outW, derInput, x, derOutput, accumulate))
+    return check_launch("mcn_pool_backward");
+
+  // ---- ordered passes.  Widest tile whose LDS fits the budget and whose outputs fit 4 per thread.
   if (passes <= 16 && p.poolH <= 8 && p.poolW <= 8 && !tunable("pool_force_gather", 0)) {
     int tiles = 0, maxOut = 0;
     size_t lds = 0;

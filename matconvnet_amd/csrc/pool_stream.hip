@@ -1,0 +1,447 @@
+// Max-pooling backward, streaming form (the fast path for planes whose height is a multiple of 4).
+//
+// Same arithmetic and visiting order as the ordered-pass kernel of pool.hip -- one fp32 accumulator per input
+// element, every output adds its dzdy to the first maximum of its window, outputs reach an accumulator in
+// ascending (output column, output row) order (bits/nnpooling.cu:33-66,190-206) -- organised so that HBM
+// never waits for the arithmetic:
+//   * persistent workgroups: workgroup b of G takes tiles b, b + G, ... (a tile = all rows of TW columns of one
+//     plane) and loads its NEXT tile's x and dzdy into registers before it works on the current one;
+//   * the x columns a tile's windows read live in LDS inside a -inf frame whose image rows start on a
+//     16-byte boundary, so staging is one 16-byte LDS write per 16-byte global load and windows need no
+//     clipping tests;
+//   * the winner search is straight-line compare/select code (no divergent branches), the rank tables are
+//     packed into two scalars;
+//   * accumulators are streamed out with non-temporal 16-byte stores and reset by the thread that read them.
+// No atomics; bit-identical to the CPU loops.
+#include "mcn_internal.hpp"
+
+#include <algorithm>
+
+#pragma clang fp contract(off)
+
+namespace mcn {
+namespace {
+
+struct PoolS {
+  int H, W, outH, outW, sy, sx, pt, pl, poolH, poolW;
+  int H4;        // H / 4
+  int top;       // frame row of image row 0: the padding rounded up to a multiple of 4
+  int Hp;        // frame pitch in floats (multiple of 4)
+  int maxC;      // widest frame over the tiles of a plane, in columns
+  int TW, tilesPerPlane, totalTiles;
+  int accumulate;
+  int walk;  // 0: tiles dealt round-robin to workgroups; 1: one contiguous run each; 2: round-robin inside each XCD's eighth
+  int KH, nPasses;
+  unsigned rankHpk, rankWpk;  // 4 bits per window offset: (pool - 1 - offset) / stride
+  FastDiv byTiles, bySx, byOutH, byH4, byBorder;  // byBorder: border rows per frame column (Hp - H)
+  int outStepQ, outStepR;    // 256 = outStepQ * outH + outStepR
+  int cellStepQ, cellStepR;  // 256 = cellStepQ * H4 + cellStepR
+};
+
+// Uniform description of one tile: all rows of the image columns [w0, w0 + nW) of one plane.
+struct Tile {
+  int w0, nW;          // owned columns
+  int owLo, nOut;      // first output column whose window touches the tile; outputs touching it
+  int cLo, nC;         // frame column 0 is image column cLo (may be negative: padding); frame columns
+  int ca;              // first image column present in the frame
+  int nCells;          // 16-byte cells of x to load: columns [ca, cb) x H/4
+  const float* xsrc;   // x at (row 0, column ca)
+  const float* dsrc;   // dzdy at (row 0, column owLo)
+  float* out;          // dzdx at (row 0, column w0)
+};
+
+__device__ __forceinline__ Tile tile_geometry(const PoolS& p, int tile, int poolW, const float* xPlane,
+                                              const float* dyPlane, float* dxPlane) {
+  Tile g;
+  g.w0 = tile * p.TW;
+  const int w1 = min(g.w0 + p.TW, p.W);
+  g.nW = w1 - g.w0;
+  const int loNum = g.w0 + p.pl - poolW + 1;
+  g.owLo = loNum <= 0 ? 0 : p.bySx.div(loNum + p.sx - 1);
+  const int owHi = min(p.outW - 1, p.bySx.div(w1 - 1 + p.pl));
+  const int nOW = max(owHi - g.owLo + 1, 0);
+  g.nOut = nOW * p.outH;
+  g.cLo = g.owLo * p.sx - p.pl;
+  g.nC = nOW > 0 ? (nOW - 1) * p.sx + poolW : 0;
+  g.ca = max(g.cLo, 0);
+  const int cb = min(g.cLo + g.nC, p.W);
+  g.nCells = max(cb - g.ca, 0) * p.H4;
+  g.xsrc = xPlane + g.ca * p.H;
+  g.dsrc = dyPlane + g.owLo * p.outH;
+  g.out = dxPlane + g.w0 * p.H;
+  return g;
+}
+
+// Issues the global loads of tile g: this thread's cells of x and its outputs' dzdy.
+template <int OPT, int XPT>
+__device__ __forceinline__ void prefetch_tile(v4f (&xr)[XPT], float (&dr)[OPT], const Tile& g, int tid) {
+  // Lanes past the end re-read the last element instead of being masked off (their copies are never used):
+  // a clamped index costs one instruction, a masked region four.
+  if (g.nCells > 0) {
+#pragma unroll
+    for (int u = 0; u < XPT; ++u) xr[u] = ((const v4f*)g.xsrc)[min(tid + 256 * u, g.nCells - 1)];
+  }
+  if (g.nOut > 0) {
+#pragma unroll
+    for (int k = 0; k < OPT; ++k) dr[k] = g.dsrc[min(tid + 256 * k, g.nOut - 1)];
+  }
+}
+
+// max(a, b) as the hardware instruction: returns the other operand when one is NaN.  (The library call would
+// add an instruction per operand to quieten signalling NaNs, which plays no role here.)
+__device__ __forceinline__ float hw_max(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// LDS-only barrier: waits for this wave's LDS traffic, not for the global loads of the next tile in flight
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// OPT outputs and XPT 16-byte cells of x per thread and tile; NP > 0: the number of passes, known at compile time.
+template <int PH, int PW, int NP, int OPT, int XPT>
+__global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restrict__ dx,
+                                                                const float* __restrict__ x,
+                                                                const float* __restrict__ dy, PoolS p) {
+  extern __shared__ float smem[];
+  float* acc = smem;                 // [TW * H] accumulators, all +0 between tiles
+  float* frame = smem + p.TW * p.H;  // [maxC * Hp] x inside its -inf frame; frame row r = image row r - top
+  // after the frame: one 16-byte cell that swallows the staging writes of idle lanes, and one float per lane
+  // that swallows the additions of lanes sitting out a pass
+  const int trashCell = p.maxC * p.Hp;                      // relative to frame
+  const int idleAcc = p.TW * p.H + p.maxC * p.Hp + 4 + threadIdx.x;  // relative to acc
+  const int tid = threadIdx.x;
+  const int poolH = PH > 0 ? PH : p.poolH, poolW = PW > 0 ? PW : p.poolW;
+
+  // Tiles are dealt so that the workgroups running at any moment cover one contiguous stretch of each tensor
+  // (DRAM rows are used up while they are open): workgroup b takes tiles b, b + G, b + 2G, ...  Measured on the
+  // 112x112x64x32 3x3/2 case, cold caches: 44 us, against 46.5 us when each XCD walks its own eighth of the
+  // tiles that way and 50 us when every workgroup owns one contiguous run of tiles.
+  const int G = (int)gridDim.x;
+  int t0, t1, step;
+  if (p.walk == 0) {
+    t0 = blockIdx.x;
+    t1 = p.totalTiles;
+    step = G;
+  } else if (p.walk == 1) {
+    const int lb = xcd_contiguous_id(blockIdx.x, G);
+    t0 = (int)(((long long)lb * p.totalTiles) / G);
+    t1 = (int)(((long long)(lb + 1) * p.totalTiles) / G);
+    step = 1;
+  } else {
+    const int nx = min(kNumXcd, G);  // groups of workgroups; with 8 or more workgroups, one group per XCD
+    const int xcd = blockIdx.x % nx, j = blockIdx.x / nx;
+    step = G / nx + (xcd < G % nx ? 1 : 0);
+    t0 = (int)(((long long)xcd * p.totalTiles) / nx) + j;
+    t1 = (int)(((long long)(xcd + 1) * p.totalTiles) / nx);
+  }
+  if (t0 >= t1) return;
+
+  // ---- once: accumulators at +0; the frame rows above and below the image at -inf (no tile writes them)
+  for (int i = tid; i < p.TW * p.H4; i += 256) ((float4*)acc)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  {
+    const int nb = p.Hp - p.H;
+    for (int i = tid; i < p.maxC * nb; i += 256) {
+      int c, k;
+      p.byBorder.divmod(i, &c, &k);
+      frame[c * p.Hp + (k < p.top ? k : k + p.H)] = -INFINITY;
+    }
+  }
+
+  // ---- per-thread constants that no tile changes
+  // outputs o = tid + 256 k of a tile: tile-relative output column oCol, output row oRow
+  int oRow[OPT], oCol[OPT], orgOff[OPT], locBase[OPT];
+  {
+    int owr, oh;
+    p.byOutH.divmod(tid, &owr, &oh);
+#pragma unroll
+    for (int k = 0; k < OPT; ++k) {
+      oRow[k] = oh;
+      oCol[k] = owr;
+      orgOff[k] = owr * p.sx * p.Hp + oh * p.sy + p.top - p.pt;  // window origin inside the frame
+      locBase[k] = owr * p.sx * p.H + oh * p.sy - p.pt;           // its accumulator, before the tile's column shift
+      owr += p.outStepQ;
+      oh += p.outStepR;
+      if (oh >= p.outH) {
+        oh -= p.outH;
+        ++owr;
+      }
+    }
+  }
+  // cells i = tid + 256 u of the tile's x: column i / H4 after the first present one, rows 4 (i % H4) ...
+  int cellDst[XPT];  // frame position when the first present column is frame column 0
+  {
+    int c, s;
+    p.byH4.divmod(tid, &c, &s);
+#pragma unroll
+    for (int u = 0; u < XPT; ++u) {
+      cellDst[u] = c * p.Hp + p.top + 4 * s;
+      c += p.cellStepQ;
+      s += p.cellStepR;
+      if (s >= p.H4) {
+        s -= p.H4;
+        ++c;
+      }
+    }
+  }
+
+  // ---- walk the tiles t0, t0 + step, ... < t1
+  const size_t planeIn = (size_t)p.H * p.W, planeOut = (size_t)p.outH * p.outW;
+  v4f xr[XPT];  // native vectors: these stay in registers under conditional assignment
+  float dr[OPT];
+  Tile cur;
+  {
+    int z, tile;
+    p.byTiles.divmod(t0, &z, &tile);
+    cur = tile_geometry(p, tile, poolW, x + z * planeIn, dy + z * planeOut, dx + z * planeIn);
+  }
+  prefetch_tile<OPT, XPT>(xr, dr, cur, tid);
+
+  // The accumulators of a finished tile are written to memory at the start of the next iteration, so their
+  // stores have a whole tile's worth of work to complete before this wave next waits on its memory counter.
+  float* prevOut = dx;
+  int prevIn4 = 0;
+
+  for (int t = t0; t < t1; t += step) {
+    const int nIn4 = cur.nW * p.H4;
+    // Everything this wave has in flight (this tile's loads, the previous tile's stores) is needed or long
+    // done by now.  Waiting here, outside any branch, also tells the compiler that nothing is pending on any
+    // path, so it places no memory waits of its own in the arithmetic below.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    // ---- registers -> LDS (image cells only; the -inf rows above and below are permanent)
+    {
+      const int colShift = (cur.ca - cur.cLo) * p.Hp;
+#pragma unroll
+      for (int u = 0; u < XPT; ++u)
+        *(v4f*)(frame + (tid + 256 * u < cur.nCells ? cellDst[u] + colShift : trashCell)) = xr[u];
+      // frame columns left / right of the image (first and last tiles of a plane only)
+      if (cur.cLo < 0)
+        for (int r = tid; r < colShift; r += 256) frame[r] = -INFINITY;
+      const int c0 = p.W - cur.cLo;
+      if (cur.nC > c0)
+        for (int r = tid; r < (cur.nC - c0) * p.Hp; r += 256) frame[c0 * p.Hp + r] = -INFINITY;
+    }
+    float dv[OPT];
+#pragma unroll
+    for (int k = 0; k < OPT; ++k) dv[k] = dr[k];
+    // ---- previous tile: stream its accumulators out, leaving +0 (or this tile's derInput when accumulating)
+    for (int i = tid; i < prevIn4; i += 256) {
+      const float4 a = ((const float4*)acc)[i];
+      ((float4*)acc)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      stream_store4((float4*)prevOut + i, a);
+    }
+    if (p.accumulate)
+      for (int i = tid; i < nIn4; i += 256) ((float4*)acc)[i] = ((const float4*)cur.out)[i];
+    lds_barrier();
+
+    // ---- next tile's loads go out now and land while this tile is computed
+    Tile nxt = cur;
+    if (t + step < t1) {
+      int z, tile;
+      p.byTiles.divmod(t + step, &z, &tile);
+      nxt = tile_geometry(p, tile, poolW, x + z * planeIn, dy + z * planeOut, dx + z * planeIn);
+      prefetch_tile<OPT, XPT>(xr, dr, nxt, tid);
+    }
+
+    // ---- winner of each owned output: first maximum of its window, scanning column by column
+    float best[OPT];
+    int code[OPT];  // 8 * column offset + row offset of the winner, -1 when nothing beats -inf
+    const float* org[OPT];
+#pragma unroll
+    for (int k = 0; k < OPT; ++k) {
+      org[k] = frame + (tid + 256 * k < cur.nOut ? orgOff[k] : 0);  // idle lanes read a valid window
+      best[k] = -INFINITY;
+      code[k] = -1;
+    }
+    if (PH > 0 && PW > 0) {
+      float v[OPT][PW > 0 ? PW : 1][PH > 0 ? PH : 1];
+#pragma unroll
+      for (int k = 0; k < OPT; ++k)
+#pragma unroll
+        for (int j = 0; j < PW; ++j)
+#pragma unroll
+          for (int i = 0; i < PH; ++i) v[k][j][i] = org[k][j * p.Hp + i];
+      // the OPT compare/select chains advance together, so no chain waits on its own previous compare
+#pragma unroll
+      for (int j = 0; j < PW; ++j)
+#pragma unroll
+        for (int i = 0; i < PH; ++i)
+#pragma unroll
+          for (int k = 0; k < OPT; ++k) {
+            code[k] = v[k][j][i] > best[k] ? (8 * j + i) : code[k];
+            best[k] = hw_max(best[k], v[k][j][i]);
+          }
+    } else {
+      for (int j = 0; j < poolW; ++j)
+        for (int i = 0; i < poolH; ++i)
+#pragma unroll
+          for (int k = 0; k < OPT; ++k) {
+            const float v = org[k][j * p.Hp + i];
+            code[k] = v > best[k] ? (8 * j + i) : code[k];
+            best[k] = hw_max(best[k], v);
+          }
+    }
+    // ---- the winner's accumulator and the output's rank among the outputs sharing that winner
+    int loc[OPT], rank[OPT];
+    const int shift = cur.cLo - cur.w0;  // frame column 0 relative to the tile's first column
+#pragma unroll
+    for (int k = 0; k < OPT; ++k) {
+      const int bj = code[k] >> 3, bi = code[k] & 7;
+      const int w = oCol[k] * p.sx + bj + shift;  // tile-relative column of the winner
+      const bool ok = code[k] >= 0 && tid + 256 * k < cur.nOut && (unsigned)w < (unsigned)cur.nW;
+      const int ra = (int)((p.rankHpk >> (4 * bi)) & 15u), rb = (int)((p.rankWpk >> (4 * bj)) & 15u);
+      rank[k] = (min(cur.owLo + oCol[k], rb) * p.KH + min(oRow[k], ra)) | (ok ? 0 : -1);  // -1: routes nothing
+      loc[k] = locBase[k] + (shift + bj) * p.H + bi;
+    }
+
+    // ---- ordered passes: in pass r the outputs of rank r add into their winner's accumulator
+    // (a lane sitting out a pass adds into its private idle slot: a select instead of a masked region)
+    if (NP > 0) {
+#pragma unroll
+      for (int r = 0; r < NP; ++r) {
+        float a[OPT];
+        int at[OPT];
+#pragma unroll
+        for (int k = 0; k < OPT; ++k) {
+          at[k] = rank[k] == r ? loc[k] : idleAcc;
+          a[k] = acc[at[k]];
+        }
+        // (outputs of equal rank never share a winner, so the real addresses of one pass are all distinct)
+#pragma unroll
+        for (int k = 0; k < OPT; ++k) acc[at[k]] = a[k] + dv[k];
+        lds_barrier();
+      }
+    } else {
+      for (int r = 0; r < p.nPasses; ++r) {
+#pragma unroll
+        for (int k = 0; k < OPT; ++k)
+          if (rank[k] == r) acc[loc[k]] = acc[loc[k]] + dv[k];
+        lds_barrier();
+      }
+    }
+    prevOut = cur.out;
+    prevIn4 = nIn4;
+    cur = nxt;
+  }
+  // ---- last tile
+  for (int i = tid; i < prevIn4; i += 256) stream_store4((float4*)prevOut + i, ((const float4*)acc)[i]);
+}
+
+}  // namespace
+
+// Launches the streaming kernel when the problem fits it.  Returns true when the work was enqueued.
+bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, float* derInput,
+                                     const float* x, const float* derOutput, int accumulate) {
+  if (g->H % 4 != 0 || !aligned16(derInput) || !aligned16(x)) return false;
+  if (g->poolH > 8 || g->poolW > 8) return false;
+  const int kh = (g->poolH + g->strideY - 1) / g->strideY, kw = (g->poolW + g->strideX - 1) / g->strideX;
+  if (kh * kw > 4) return false;  // windows overlapping more than 2 x 2 outputs: the ordered-pass kernel of pool.hip is faster
+  if (tunable("pool_force_gather", 0) || tunable("pool_no_stream", 0)) return false;
+  const size_t planes = (size_t)g->C * g->N;
+
+  PoolS p;
+  p.H = g->H; p.W = g->W; p.outH = outH; p.outW = outW;
+  p.sy = g->strideY; p.sx = g->strideX; p.pt = g->padTop; p.pl = g->padLeft;
+  p.poolH = g->poolH; p.poolW = g->poolW;
+  p.H4 = g->H / 4;
+  p.top = (g->padTop + 3) & ~3;
+  const int rows = std::max(p.top + g->H, p.top - g->padTop + (outH - 1) * g->strideY + g->poolH);
+  p.Hp = (rows + 3) & ~3;
+  p.accumulate = accumulate ? 1 : 0;
+  p.walk = tunable("pool_walk", 0);
+  p.KH = kh;
+  p.nPasses = kh * kw;
+  p.rankHpk = p.rankWpk = 0;
+  for (int i = 0; i < g->poolH; ++i) p.rankHpk |= (unsigned)((g->poolH - 1 - i) / g->strideY) << (4 * i);
+  for (int i = 0; i < g->poolW; ++i) p.rankWpk |= (unsigned)((g->poolW - 1 - i) / g->strideX) << (4 * i);
+
+  // widest tile whose LDS fits the budget and whose outputs and cells fit 4 per thread
+  const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024), 64 * 1024);
+  int TW = 0, maxOut = 0, maxCells = 0, maxC = 0;
+  size_t lds = 0;
+  for (int nT = 1; nT <= p.W; ++nT) {
+    const int cand = (p.W + nT - 1) / nT;
+    if (nT > 1 && cand == (p.W + nT - 2) / (nT - 1)) continue;
+    int worstOut = 0, worstCells = 0, worstC = 0;
+    for (int w0 = 0; w0 < p.W; w0 += cand) {
+      const int w1 = std::min(w0 + cand, p.W);
+      const int num = w0 + p.pl - p.poolW + 1;
+      const int owLo = num <= 0 ? 0 : (num + p.sx - 1) / p.sx;
+      const int owHi = std::min(p.outW - 1, (w1 - 1 + p.pl) / p.sx);
+      const int nOW = std::max(owHi - owLo + 1, 0);
+      const int cLo = owLo * p.sx - p.pl, nC = nOW > 0 ? (nOW - 1) * p.sx + p.poolW : 0;
+      const int ca = std::max(cLo, 0), cb = std::min(cLo + nC, p.W);
+      worstOut = std::max(worstOut, nOW * p.outH);
+      worstCells = std::max(worstCells, std::max(cb - ca, 0) * p.H4);
+      worstC = std::max(worstC, nC);
+    }
+    worstC = std::max(worstC, p.poolW);  // idle lanes read the window at the frame origin
+    const size_t need = ((size_t)cand * p.H + (size_t)worstC * p.Hp) * sizeof(float);
+    if (need <= budget && worstOut <= 4 * 256 && worstCells <= 4 * 256) {
+      TW = cand;
+      maxOut = worstOut;
+      maxCells = worstCells;
+      maxC = worstC;
+      lds = need;
+      break;
+    }
+  }
+  if (TW == 0) return false;
+  const size_t tilesPerPlane = (size_t)(p.W + TW - 1) / TW;
+  if (planes * tilesPerPlane >= (1ull << 31)) return false;
+  p.TW = TW;
+  p.maxC = maxC;
+  p.tilesPerPlane = (int)tilesPerPlane;
+  p.totalTiles = (int)(planes * tilesPerPlane);
+  p.byTiles = FastDiv((int)tilesPerPlane);
+  p.bySx = FastDiv(p.sx);
+  p.byOutH = FastDiv(p.outH);
+  p.byH4 = FastDiv(p.H4);
+  p.byBorder = FastDiv(std::max(p.Hp - p.H, 1));
+  p.outStepQ = 256 / p.outH;
+  p.outStepR = 256 % p.outH;
+  p.cellStepQ = 256 / p.H4;
+  p.cellStepR = 256 % p.H4;
+  const int opt = std::max((maxOut + 255) / 256, 1), xpt = std::max((maxCells + 255) / 256, 1);
+  lds += (4 + 256) * sizeof(float);  // the idle-lane cell and slots
+
+  int cus = 256;
+  {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+      cus = prop.multiProcessorCount;
+  }
+  const int perCu = std::min(std::max(tunable("pool_blocks_per_cu", 3), 1), (int)std::max<size_t>((160 * 1024) / std::max<size_t>(lds, 1), 1));
+  const int blocks = (int)std::min<long long>(p.totalTiles, (long long)cus * perCu);
+  const dim3 grid((unsigned)blocks), block(256);
+  KernelTimer timer("pool_backward_stream", s);
+#define MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, XPTF) \
+  hipLaunchKernelGGL((pool_max_backward_stream<PHF, PWF, NPF, OPTF, XPTF>), grid, block, lds, s, derInput, x, derOutput, p)
+#define MCN_POOL_STREAM_XPT(PHF, PWF, NPF, OPTF)               \
+  do {                                                         \
+    if (xpt == 1) MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, 1);      \
+    else if (xpt == 2) MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, 2); \
+    else if (xpt == 3) MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, 3); \
+    else MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, 4);               \
+  } while (0)
+#define MCN_POOL_STREAM_OPT(PHF, PWF, NPF)                   \
+  do {                                                       \
+    if (opt == 1) MCN_POOL_STREAM_XPT(PHF, PWF, NPF, 1);      \
+    else if (opt == 2) MCN_POOL_STREAM_XPT(PHF, PWF, NPF, 2); \
+    else if (opt == 3) MCN_POOL_STREAM_XPT(PHF, PWF, NPF, 3); \
+    else MCN_POOL_STREAM_XPT(PHF, PWF, NPF, 4);               \
+  } while (0)
+  // the common shapes get their window and pass count at compile time
+  if (p.poolH == 3 && p.poolW == 3 && p.nPasses == 4) MCN_POOL_STREAM_OPT(3, 3, 4);        // 3x3, stride 2
+  else if (p.poolH == 2 && p.poolW == 2 && p.nPasses == 1) MCN_POOL_STREAM_OPT(2, 2, 1);   // 2x2, stride 2
+  else if (p.poolH == 3 && p.poolW == 3) MCN_POOL_STREAM_OPT(3, 3, 0);
+  else if (p.poolH == 2 && p.poolW == 2) MCN_POOL_STREAM_OPT(2, 2, 0);
+  else MCN_POOL_STREAM_OPT(0, 0, 0);
+#undef MCN_POOL_STREAM_OPT
+#undef MCN_POOL_STREAM_XPT
+#undef MCN_POOL_STREAM
+  return true;
+}
+
+}  // namespace mcn
