@@ -8,7 +8,10 @@ channels, N = 32, fp32) through the C++ operator layer, with every tensor reside
 region.  `value` is images/s over exactly K steps.  The same line carries
   roofline      the kernel that takes most of the step, timed live with HIP events on its launch stream,
   rooflines     the graded kernels on their own configurations: conv backward (configs[4], fp32 MFMA),
-                batch-norm backward (configs[1], HBM), max/avg pooling backward (configs[2], HBM),
+                batch-norm backward (configs[1], HBM), max/avg pooling backward (configs[2], HBM).  The HBM-bound
+                ones are timed COLD: four sets of tensors used in turn, so that no launch finds its inputs in the
+                256 MB memory-side cache because the previous launch left them there (`achieved`); the figure a
+                loop over one set of buffers shows is reported beside it as `achieved_warm`,
   cpu_baseline  the CPU restatement of the reference path (oracle/) timed on this machine's host cores.
 One GPU only: nothing here shards.
 """
@@ -25,6 +28,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_FP32 = 157.3e12  # FLOP/s, MI355X dense fp32 matrix
 PEAK_HBM = 8.0e12          # B/s
+COLD_SETS = 4              # tensor sets used in turn by the HBM-bound measurements (> 256 MB between reuses)
 
 
 def _sync():
@@ -63,9 +67,9 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
     eS, eB = 4.0 * P * 64 * N, 4.0 * P * 256 * N
     hbm_bytes = {  # algorithmic bytes per step of the memory-bound families (reads + writes once each)
         "bnorm_sums": (eS + eS + eB) + 2 * (eS + eS + eB),       # forward reads x; backward reads x and dzdy
-        "bnorm_forward_apply": 2 * (eS + eS + eB),
+        "bnorm_forward_apply": 2 * eS + 2 * eS + 3 * eB,          # bn1, bn2 with ReLU; bn3 with shortcut sum and ReLU
         "bnorm_backward_apply": 3 * (eS + eS + eB),
-        "eltwise_kernel": (2 * eS) * 2 + 3 * eB + 2 * eB + 3 * eB + (3 * eS) * 2 + 3 * eB,
+        "eltwise_kernel": 3 * eB + 3 * eS + 3 * eS + 3 * eB,      # three ReLU derivatives, one fan-out sum
     }
     fam = {}
     for name in list(conv_flops) + list(hbm_bytes) + ["conv_wgrad_reduce", "conv_pack_weights"]:
@@ -138,35 +142,50 @@ def bench_bnorm_bwd(capi, workloads, reps):
     import torch
     L = capi.lib()
     H, W, Cc, N = 56, 56, 256, 32
-    x = torch.randn((N, Cc, W, H), device="cuda") * 1.3 + 0.5
-    dy = torch.randn((N, Cc, W, H), device="cuda")
+    xs = [torch.randn((N, Cc, W, H), device="cuda") * 1.3 + 0.5 for _ in range(COLD_SETS)]
+    dys = [torch.randn((N, Cc, W, H), device="cuda") for _ in range(COLD_SETS)]
+    dxs = [capi.empty((H, W, Cc, N)) for _ in range(COLD_SETS)]
     g = torch.rand(Cc, device="cuda") + 0.5
-    dx, dg, db, mom = capi.empty((H, W, Cc, N)), capi.empty((Cc,)), capi.empty((Cc,)), capi.empty((Cc, 2))
+    dg, db, mom = capi.empty((Cc,)), capi.empty((Cc,)), capi.empty((Cc, 2))
     ws = capi.Workspace()
     wp, wn = ws.get(L.mcn_bnorm_workspace_bytes(H, W, Cc, N))
     st = capi.stream()
-    call = lambda: capi.check(L.mcn_bnorm_backward(st, capi.ptr(dx), capi.ptr(dg), capi.ptr(db), capi.ptr(mom), capi.ptr(x),
-                                                   capi.ptr(g), capi.ptr(dy), H, W, Cc, N, 1e-4, 0, wp, wn))
-    call()
-    _sync()
+    turn = [0]
+
+    def make(sets):
+        def call():
+            i = turn[0] % sets
+            turn[0] += 1
+            capi.check(L.mcn_bnorm_backward(st, capi.ptr(dxs[i]), capi.ptr(dg), capi.ptr(db), capi.ptr(mom), capi.ptr(xs[i]),
+                                            capi.ptr(g), capi.ptr(dys[i]), H, W, Cc, N, 1e-4, 0, wp, wn))
+        return call
+
     E = 4.0 * H * W * Cc * N
-    t_sums, _ = kernel_time(capi, "bnorm_sums", call, reps)
-    t_apply, _ = kernel_time(capi, "bnorm_backward_apply", call, reps)
-    _sync()
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        call()
-    _sync()
-    t_all = (time.perf_counter() - t0) / reps
+    t = {}
+    for label, sets in (("cold", COLD_SETS), ("warm", 1)):
+        call = make(sets)
+        for _ in range(COLD_SETS):
+            call()
+        _sync()
+        t_sums, _ = kernel_time(capi, "bnorm_sums", call, reps)
+        t_apply, _ = kernel_time(capi, "bnorm_backward_apply", call, reps)
+        _sync()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            call()
+        _sync()
+        t[label] = (t_sums, t_apply, (time.perf_counter() - t0) / reps)
     rows = [
         dict(op="bnorm backward, pass 1 (sums)", kernel="bnorm_sums", workload="configs[1] 56x56x256x32", bound="hbm",
-             achieved=2 * E / t_sums / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=2 * E / t_sums / PEAK_HBM,
-             avg_launch_us=t_sums * 1e6, traffic=None),
+             achieved=2 * E / t["cold"][0] / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=2 * E / t["cold"][0] / PEAK_HBM,
+             avg_launch_us=t["cold"][0] * 1e6, achieved_warm=2 * E / t["warm"][0] / 1e9, traffic=None),
         dict(op="bnorm backward, pass 2 (apply)", kernel="bnorm_backward_apply", workload="configs[1] 56x56x256x32", bound="hbm",
-             achieved=3 * E / t_apply / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=3 * E / t_apply / PEAK_HBM,
-             avg_launch_us=t_apply * 1e6, traffic=None),
+             achieved=3 * E / t["cold"][1] / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=3 * E / t["cold"][1] / PEAK_HBM,
+             avg_launch_us=t["cold"][1] * 1e6, achieved_warm=3 * E / t["warm"][1] / 1e9, traffic=None),
     ]
-    whole = dict(gbs=5 * E / t_all / 1e9, frac=5 * E / t_all / PEAK_HBM, us=t_all * 1e6, gbs_compulsory=3 * E / t_all / 1e9)
+    t_all = t["cold"][2]
+    whole = dict(gbs=5 * E / t_all / 1e9, frac=5 * E / t_all / PEAK_HBM, us=t_all * 1e6, gbs_compulsory=3 * E / t_all / 1e9,
+                 gbs_warm=5 * E / t["warm"][2] / 1e9, us_warm=t["warm"][2] * 1e6)
     return rows, whole
 
 
@@ -180,19 +199,34 @@ def bench_pool_bwd(capi, workloads, reps):
                                            ("avg-pool backward", (56, 56, 256, 32), 2, 0, "avg")):
         g = capi.pool_geom(shape, pool, 2, pad, method)
         oshape = capi.pool_out_shape(g)
-        x = torch.randn(tuple(reversed(shape)), device="cuda")
-        dy = torch.randn(tuple(reversed(oshape)), device="cuda")
-        dx = capi.empty(shape)
+        xs = [torch.randn(tuple(reversed(shape)), device="cuda") for _ in range(COLD_SETS)]
+        dys = [torch.randn(tuple(reversed(oshape)), device="cuda") for _ in range(COLD_SETS)]
+        dxs = [capi.empty(shape) for _ in range(COLD_SETS)]
         st = capi.stream()
-        call = lambda: capi.check(L.mcn_pool_backward(st, C.byref(g), capi.ptr(dx), capi.ptr(x), capi.ptr(dy), 0))
-        call()
-        _sync()
+        turn = [0]
+
+        def make(sets):
+            def call():
+                i = turn[0] % sets
+                turn[0] += 1
+                capi.check(L.mcn_pool_backward(st, C.byref(g), capi.ptr(dxs[i]), capi.ptr(xs[i]), capi.ptr(dys[i]), 0))
+            return call
+
         e, o = 4.0 * np.prod(shape), 4.0 * np.prod(oshape)
         nbytes = (2 * e + o) if method == "max" else (e + o)
-        t, _ = kernel_time(capi, "pool_backward", call, reps)
-        rows.append(dict(op=name, kernel="pool_backward_passes", workload="configs[2] %s on %s" % (method, "x".join(map(str, shape))),
-                         bound="hbm", achieved=nbytes / t / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=nbytes / t / PEAK_HBM,
-                         avg_launch_us=t * 1e6, traffic=None))
+        t = {}
+        for label, sets in (("cold", COLD_SETS), ("warm", 1)):
+            call = make(sets)
+            for _ in range(COLD_SETS):
+                call()
+            _sync()
+            t[label], _ = kernel_time(capi, "pool_backward", call, reps)
+        rows.append(dict(op=name, kernel="pool_max_backward_stream" if method == "max" else "pool_backward_passes",
+                         workload="configs[2] %s on %s" % (method, "x".join(map(str, shape))),
+                         bound="hbm", achieved=nbytes / t["cold"] / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s",
+                         frac=nbytes / t["cold"] / PEAK_HBM, avg_launch_us=t["cold"] * 1e6,
+                         achieved_warm=nbytes / t["warm"] / 1e9, traffic=None))
+        del xs, dys, dxs
     return rows
 
 
@@ -251,7 +285,10 @@ def main():
         "step_breakdown_ms": breakdown,
         "conv_bwd_tflops": conv_whole["tflops"], "conv_bwd_frac_of_mfma_peak": conv_whole["frac"], "conv_bwd_ms": conv_whole["ms"],
         "bnorm_bwd_gbs": bn_whole["gbs"], "bnorm_bwd_frac_of_hbm_peak": bn_whole["frac"], "bnorm_bwd_us": bn_whole["us"],
+        "bnorm_bwd_gbs_warm": bn_whole["gbs_warm"],
         "maxpool_bwd_gbs": pool_rows[0]["achieved"], "avgpool_bwd_gbs": pool_rows[1]["achieved"],
+        "maxpool_bwd_gbs_warm": pool_rows[0]["achieved_warm"], "avgpool_bwd_gbs_warm": pool_rows[1]["achieved_warm"],
+        "hbm_timing": "cold: %d tensor sets in rotation; *_warm: one set reused" % COLD_SETS,
         "rooflines": conv_rows + bn_rows + pool_rows,
     }
     if not args.no_cpu_baseline:
