@@ -28,6 +28,18 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_FP32 = 157.3e12  # FLOP/s, MI355X dense fp32 matrix
 PEAK_HBM = 8.0e12          # B/s
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/*.txt), scaled by what the same counters
+# read for a 256 MiB streaming copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per unit).  Counters are not
+# readable from inside this process, so these are the profiled values of exactly these launches.
+TRAFFIC = {
+    "block/conv_pix_mfma": 1.039e8,    # mean of the 6 launches of a step (profiles/bottleneck_block_56x56_N32_fwd_bwd.txt)
+    "cfg5/conv_pix_mfma": 2.319e9,     # profiles/conv_vgg_3x3x256x256_N64_backward.txt (operands 2.08e8: tiles re-read through L2)
+    "cfg5/conv_wgrad_mfma": 9.08e8,
+    "cfg2/bnorm_sums": 2.058e8,        # profiles/bnorm_56x56x256x32_backward.txt
+    "cfg2/bnorm_backward_apply": 3.086e8,
+    "cfg3a/pool": 2.518e8,             # profiles/maxpool_112x112x64x32_backward.txt (halo columns fetched by two workgroups)
+    "cfg3b/pool": 1.286e8,             # profiles/avgpool_56x56x256x32_backward.txt
+}
 COLD_SETS = 4              # tensor sets used in turn by the HBM-bound measurements (> 256 MB between reuses)
 
 
@@ -83,13 +95,13 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
     if top in conv_flops:
         achieved = conv_flops[top] * steps / total
         roof = dict(kernel=top, bound="mfma", achieved=achieved / 1e12, peak=PEAK_MFMA_FP32 / 1e12, unit="TFLOP/s",
-                    frac=achieved / PEAK_MFMA_FP32, traffic=None, launches_per_step=n // steps,
+                    frac=achieved / PEAK_MFMA_FP32, traffic=TRAFFIC.get("block/" + top), launches_per_step=n // steps,
                     avg_launch_us=total / n * 1e6)
     else:
         work = hbm_bytes.get(top, float("nan"))
         achieved = work * steps / total
         roof = dict(kernel=top, bound="hbm", achieved=achieved / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s",
-                    frac=achieved / PEAK_HBM, traffic=None, launches_per_step=n // steps, avg_launch_us=total / n * 1e6)
+                    frac=achieved / PEAK_HBM, traffic=TRAFFIC.get("block/" + top), launches_per_step=n // steps, avg_launch_us=total / n * 1e6)
     breakdown = {k: round(v[1] / steps * 1e3, 4) for k, v in fam.items()}  # ms per step by kernel family
     return N * steps / dt, dt / steps * 1e3, roof, breakdown
 
@@ -130,7 +142,7 @@ def bench_conv_bwd(capi, workloads, reps):
     for name, kern, t in (("conv backward-data", "conv_pix_mfma", t_data), ("conv backward-filter", "conv_wgrad_mfma", t_filt)):
         out.append(dict(op=name, kernel=kern, workload="configs[4] 3x3x256x256 on 56x56x256x64", bound="mfma",
                         achieved=flops / t / 1e12, peak=PEAK_MFMA_FP32 / 1e12, unit="TFLOP/s", frac=flops / t / PEAK_MFMA_FP32,
-                        avg_launch_us=t * 1e6, traffic=None))
+                        avg_launch_us=t * 1e6, traffic=TRAFFIC["cfg5/" + kern]))
     whole = dict(tflops=2 * flops / t_all / 1e12, frac=2 * flops / t_all / PEAK_MFMA_FP32, ms=t_all * 1e3,
                  wgrad_reduce_us=t_red * 1e6)
     return out, whole
@@ -178,10 +190,10 @@ def bench_bnorm_bwd(capi, workloads, reps):
     rows = [
         dict(op="bnorm backward, pass 1 (sums)", kernel="bnorm_sums", workload="configs[1] 56x56x256x32", bound="hbm",
              achieved=2 * E / t["cold"][0] / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=2 * E / t["cold"][0] / PEAK_HBM,
-             avg_launch_us=t["cold"][0] * 1e6, achieved_warm=2 * E / t["warm"][0] / 1e9, traffic=None),
+             avg_launch_us=t["cold"][0] * 1e6, achieved_warm=2 * E / t["warm"][0] / 1e9, traffic=TRAFFIC["cfg2/bnorm_sums"]),
         dict(op="bnorm backward, pass 2 (apply)", kernel="bnorm_backward_apply", workload="configs[1] 56x56x256x32", bound="hbm",
              achieved=3 * E / t["cold"][1] / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s", frac=3 * E / t["cold"][1] / PEAK_HBM,
-             avg_launch_us=t["cold"][1] * 1e6, achieved_warm=3 * E / t["warm"][1] / 1e9, traffic=None),
+             avg_launch_us=t["cold"][1] * 1e6, achieved_warm=3 * E / t["warm"][1] / 1e9, traffic=TRAFFIC["cfg2/bnorm_backward_apply"]),
     ]
     t_all = t["cold"][2]
     whole = dict(gbs=5 * E / t_all / 1e9, frac=5 * E / t_all / PEAK_HBM, us=t_all * 1e6, gbs_compulsory=3 * E / t_all / 1e9,
@@ -225,7 +237,8 @@ def bench_pool_bwd(capi, workloads, reps):
                          workload="configs[2] %s on %s" % (method, "x".join(map(str, shape))),
                          bound="hbm", achieved=nbytes / t["cold"] / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s",
                          frac=nbytes / t["cold"] / PEAK_HBM, avg_launch_us=t["cold"] * 1e6,
-                         achieved_warm=nbytes / t["warm"] / 1e9, traffic=None))
+                         achieved_warm=nbytes / t["warm"] / 1e9,
+                         traffic=TRAFFIC["cfg3a/pool" if method == "max" else "cfg3b/pool"]))
         del xs, dys, dxs
     return rows
 
