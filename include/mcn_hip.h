@@ -130,6 +130,30 @@ MCN_API int mcn_conv_backward_bias(mcn_stream_t stream, const mcn_conv_geom* g, 
                                    const float* derOutput, void* workspace, size_t workspaceBytes);
 
 /* ------------------------------------------------------------------------------------------------
+ * subsampling with bias -- vl_nnconv with empty FILTERS (the identity filter bank, vl_nnconv.cu:316-321,432-441):
+ * replaces Subsample::forwardWithBias / backwardWithBias (bits/nnsubsample.cu:31-216, nnsubsample_gpu.cu).
+ * Output extent: (H + padTop + padBottom - 1)/strideY + 1, likewise for the width.
+ * ---------------------------------------------------------------------------------------------- */
+
+MCN_API int mcn_subsample_output_size(int H, int W, int strideY, int strideX, int padTop, int padBottom,
+                                      int padLeft, int padRight, int* outH, int* outW);
+
+/* y[oh,ow,c,n] = x[oh*strideY - padTop, ow*strideX - padLeft, c, n] (0 outside x) + bias[c]; bias may be NULL */
+MCN_API int mcn_subsample_forward(mcn_stream_t stream, float* y, const float* x, const float* bias, int H, int W,
+                                  int C, int N, int strideY, int strideX, int padTop, int padBottom, int padLeft,
+                                  int padRight);
+
+/* dzdx (H x W x C x N, fully overwritten): dzdy placed back on the sampled positions, 0 elsewhere.  The bias
+   derivative of this layer is mcn_conv_backward_bias on dzdy. */
+MCN_API int mcn_subsample_backward(mcn_stream_t stream, float* derInput, const float* derOutput, int H, int W,
+                                   int C, int N, int strideY, int strideX, int padTop, int padBottom, int padLeft,
+                                   int padRight);
+
+/* y[h,w,c,n] += bias[c] in place -- the bias step of ConvolutionTranspose forward (bits/nnconv.cu:369-371,
+   vl::nn::Bias::forward with both multipliers 1, bits/nnbias.cu) */
+MCN_API int mcn_bias_add(mcn_stream_t stream, float* y, const float* bias, int H, int W, int C, int N);
+
+/* ------------------------------------------------------------------------------------------------
  * batch normalisation -- replaces BatchNorm*<VLDT_GPU,T> (bits/nnbnorm_gpu.cu:818-1188).
  * `moments` is C x 2: C means followed by C sigmas, sigma = sqrt(var + epsilon) (bits/nnbnorm.cu:65-70).
  * ---------------------------------------------------------------------------------------------- */

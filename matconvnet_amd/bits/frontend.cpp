@@ -7,6 +7,7 @@
 #include "nnbnorm.hpp"
 #include "nnconv.hpp"
 #include "nnpooling.hpp"
+#include "nnsubsample.hpp"
 
 namespace vl { namespace frontend {
 
@@ -193,22 +194,28 @@ void nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int n
   if (padLeft < 0 || padRight < 0 || padTop < 0 || padBottom < 0) raise(VLE_IllegalArgument, "An element of PAD is negative.");
   if (dilateY < 1 || dilateX < 1) raise(VLE_IllegalArgument, "An element of DILATE is less than one.");
   if (!hasFilters && (dilateY != 1 || dilateX != 1)) raise(VLE_IllegalArgument, "There are no filters and DILATE is not one.");
-  if (!hasFilters)
-    raise(VLE_Unsupported, "Empty FILTERS (subsampling with bias) are not implemented by this library.");
-
+  // the filter shape; empty FILTERS stand for the identity filter bank (vl_nnconv.cu:296-321)
   TensorShape filtersShape(filters);
-  if (filtersShape.getHeight() == 0 || filtersShape.getWidth() == 0 || filtersShape.getDepth() == 0)
-    raise(VLE_IllegalArgument, "A dimension of FILTERS is void.");
-  const long extentY = ((long)filters.getHeight() - 1) * dilateY + 1, extentX = ((long)filters.getWidth() - 1) * dilateX + 1;
-  if ((long)data.getHeight() + (padTop + padBottom) < extentY || (long)data.getWidth() + (padLeft + padRight) < extentX)
-    raise(VLE_IllegalArgument, "FILTERS are larger than the DATA (including padding).");
-  const std::size_t groups = data.getDepth() / filters.getDepth();
-  if (groups * filters.getDepth() != data.getDepth()) raise(VLE_IllegalArgument, "The FILTERS depth does not divide the DATA depth.");
-  if (groups == 0 || filters.getSize() % groups != 0)
-    raise(VLE_IllegalArgument, "The number of filter groups does not divide the number of filters.");
+  std::size_t equivalentNumFilters;
+  if (hasFilters) {
+    if (filtersShape.getHeight() == 0 || filtersShape.getWidth() == 0 || filtersShape.getDepth() == 0)
+      raise(VLE_IllegalArgument, "A dimension of FILTERS is void.");
+    if ((long)data.getHeight() + (padTop + padBottom) < ((long)filters.getHeight() - 1) * dilateY + 1 ||
+        (long)data.getWidth() + (padLeft + padRight) < ((long)filters.getWidth() - 1) * dilateX + 1)
+      raise(VLE_IllegalArgument, "FILTERS are larger than the DATA (including padding).");
+    const std::size_t groups = data.getDepth() / filters.getDepth();
+    if (groups * filters.getDepth() != data.getDepth()) raise(VLE_IllegalArgument, "The FILTERS depth does not divide the DATA depth.");
+    if (groups == 0 || filters.getSize() % groups != 0)
+      raise(VLE_IllegalArgument, "The number of filter groups does not divide the number of filters.");
+    equivalentNumFilters = filters.getSize();
+  } else {
+    filtersShape = TensorShape(1, 1, data.getDepth(), data.getDepth());
+    equivalentNumFilters = data.getDepth();
+  }
+  const long extentY = ((long)filtersShape.getHeight() - 1) * dilateY + 1, extentX = ((long)filtersShape.getWidth() - 1) * dilateX + 1;
 
   TensorShape outputShape(((long)data.getHeight() + (padTop + padBottom) - extentY) / strideY + 1,
-                          ((long)data.getWidth() + (padLeft + padRight) - extentX) / strideX + 1, filters.getSize(),
+                          ((long)data.getWidth() + (padLeft + padRight) - extentX) / strideX + 1, equivalentNumFilters,
                           data.getSize());
   if (backMode && (TensorShape(derOutput) != outputShape))
     raise(VLE_IllegalArgument, "DEROUTPUT dimensions are incompatible with X and FILTERS.");
@@ -217,11 +224,124 @@ void nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int n
 
   const DeviceType device = data.getDeviceType();
   const DataType type = data.getDataType();
+  // (the reference's fully-connected special case, vl_nnconv.cu:343-358,424-433, is the same product: the general
+  // kernels below cover 1 x 1 outputs)
   nn::Convolution op(context, strideY, strideX, padTop, padBottom, padLeft, padRight, dilateY, dilateX);
+  nn::Subsample sub(context, strideY, strideX, padTop, padBottom, padLeft, padRight);  // no filters: subsample + bias
+  Tensor noBias;
   if (!backMode) {
     Tensor output = newOutput(allocator, device, type, outputShape);
-    Tensor noBias;
-    failFromContext(context, op.forward(output, 0, data, 1, filters, hasBiases ? biases : noBias));
+    failFromContext(context, hasFilters ? op.forward(output, 0, data, 1, filters, hasBiases ? biases : noBias)
+                                        : sub.forwardWithBias(output, data, hasBiases ? biases : noBias));
+    out[0] = output;
+    return;
+  }
+  Tensor derData, derFilters, derBiases;
+  if (wantDerData) derData = newOutput(allocator, device, type, data.getShape());
+  if (wantDerFilters && hasFilters) derFilters = newOutput(allocator, device, type, filters.getShape());
+  if (wantDerBiases && hasBiases) derBiases = newOutput(allocator, device, type, biases.getShape());
+  failFromContext(context, hasFilters ? op.backward(derData, derFilters, derBiases, data, filters, derOutput)
+                                      : sub.backwardWithBias(derData, derBiases, derOutput));
+  const DataType outType = derOutput.getDataType();
+  out[0] = wantDerData ? derData : emptyMatrix(outType);
+  if (nout > 1) out[1] = (wantDerFilters && hasFilters) ? derFilters : emptyMatrix(outType);
+  if (nout > 2) out[2] = (wantDerBiases && hasBiases) ? derBiases : emptyMatrix(outType);
+}
+
+// ----------------------------------------------------------------------------------------- vl_nnconvt
+
+void nnconvt(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in) {
+  enum { optUpsample, optCrop, optVerbose, optNumGroups, optNoDerData, optNoDerFilters, optNoDerBiases, optCudnn, optNoCudnn, optCudnnWs };
+  static OptionSpec const specs[] = {
+      {"Upsample", true, optUpsample}, {"Crop", true, optCrop}, {"Verbose", false, optVerbose}, {"NumGroups", true, optNumGroups},
+      {"NoDerData", false, optNoDerData}, {"NoDerFilters", false, optNoDerFilters}, {"NoDerBiases", false, optNoDerBiases},
+      {"CUDNN", false, optCudnn}, {"NoCUDNN", false, optNoCudnn}, {"CudnnWorkSpaceLimit", true, optCudnnWs}, {NULL, false, 0}};
+  int upsampleX = 1, upsampleY = 1, cropLeft = 0, cropRight = 0, cropTop = 0, cropBottom = 0, numFilterGroups = 1;
+  bool wantDerData = true, wantDerFilters = true, wantDerBiases = true;
+
+  if (nin < 3) raise(VLE_IllegalArgument, "There are less than three arguments.");
+  int next = 4;
+  bool backMode;
+  if (nin > 3 && in[3].kind == Arg::String) {
+    next = 3;
+    backMode = false;
+  } else {
+    backMode = nin >= 4;
+  }
+  int opt;
+  Arg const* value = NULL;
+  while ((opt = nextOption(in, nin, specs, &next, &value)) >= 0) {
+    switch (opt) {
+      case optUpsample:  // texts as in vl_nnconvt.cu:128-142
+        if (!isPlainMatrix(*value)) raise(VLE_IllegalArgument, "upsample is not a plain matrix.");
+        switch (value->tensor.getNumElements()) {
+          case 1: upsampleY = upsampleX = (int)values(*value)[0]; break;
+          case 2: upsampleY = (int)values(*value)[0]; upsampleX = (int)values(*value)[1]; break;
+          default: raise(VLE_IllegalArgument, "upsample has neither one nor two elements.");
+        }
+        break;
+      case optCrop:  // vl_nnconvt.cu:145-164
+        if (!isPlainMatrix(*value)) raise(VLE_IllegalArgument, "crop is not a plain matrix.");
+        switch (value->tensor.getNumElements()) {
+          case 1: cropLeft = cropRight = cropTop = cropBottom = (int)values(*value)[0]; break;
+          case 4:
+            cropTop = (int)values(*value)[0]; cropBottom = (int)values(*value)[1]; cropLeft = (int)values(*value)[2];
+            cropRight = (int)values(*value)[3];
+            break;
+          default: raise(VLE_IllegalArgument, "crop has neither one nor two elements.");
+        }
+        break;
+      case optNumGroups:
+        if (!isPlainMatrix(*value) || value->tensor.getNumElements() != 1) raise(VLE_IllegalArgument, "NUMGROUPS is not a plain scalar.");
+        numFilterGroups = (int)values(*value)[0];
+        break;
+      case optNoDerData: wantDerData = false; break;
+      case optNoDerFilters: wantDerFilters = false; break;
+      case optNoDerBiases: wantDerBiases = false; break;
+      default: break;
+    }
+  }
+
+  Tensor data = dataTensor(in[0], "DATA", 4);
+  Tensor filters = dataTensor(in[1], "FILTERS", 4);
+  Tensor biases = dataTensor(in[2], "BIASES", in[2].tensor.getNumDimensions());
+  Tensor derOutput;
+  if (backMode) derOutput = dataTensor(in[3], "DEROUTPUT", 4);
+  const bool hasBiases = !biases.isEmpty();
+
+  if (!areCompatible(data, filters)) raise(VLE_IllegalArgument, "DATA and FILTERS do not have compatible formats.");
+  if (hasBiases && !areCompatible(data, biases)) raise(VLE_IllegalArgument, "DATA and BIASES do not have compatible formats.");
+  if (backMode && !areCompatible(data, derOutput)) raise(VLE_IllegalArgument, "DATA and DEROUTPUT do not have compatible formats.");
+  if (upsampleX < 1 || upsampleY < 1) raise(VLE_IllegalArgument, "At least one element of UPSAMPLE is smaller than one.");
+  if (cropLeft < 0 || cropRight < 0 || cropTop < 0 || cropBottom < 0) raise(VLE_IllegalArgument, "An element of CROP is negative.");
+
+  TensorShape filtersShape(filters);
+  if (filtersShape.getHeight() == 0 || filtersShape.getWidth() == 0 || filtersShape.getDepth() == 0)
+    raise(VLE_IllegalArgument, "A dimension of FILTERS is void.");
+  if (numFilterGroups < 1) raise(VLE_IllegalArgument, "NUMGROUPS is less than 1.");
+  if (filters.getSize() % numFilterGroups != 0)
+    raise(VLE_IllegalArgument,
+          "The number of filter groups does not divide the filter bank depth (fourth dimension of FILTERS).");
+  if (filters.getSize() != data.getDepth())
+    raise(VLE_IllegalArgument,
+          "The filter bank depth (fourth dimension of FILTERS) is not the same as the data depth (third dimension of X).");
+
+  const long outH = ((long)data.getHeight() - 1) * upsampleY - (cropTop + cropBottom) + (long)filtersShape.getHeight();
+  const long outW = ((long)data.getWidth() - 1) * upsampleX - (cropLeft + cropRight) + (long)filtersShape.getWidth();
+  if (outH < 1 || outW < 1) raise(VLE_IllegalArgument, "The output array is empty due to CROP being too large.");
+  TensorShape outputShape(outH, outW, filtersShape.getDepth() * numFilterGroups, data.getSize());
+  if (backMode && (TensorShape(derOutput) != outputShape))
+    raise(VLE_IllegalArgument, "DEROUTPUT dimensions are incompatible with X and FILTERS.");
+  if (hasBiases && biases.getNumElements() != outputShape.getDepth())
+    raise(VLE_IllegalArgument, "The number of elements of BIASES is not the same as the dimenison of the filters.");
+
+  const DeviceType device = data.getDeviceType();
+  const DataType type = data.getDataType();
+  nn::ConvolutionTranspose op(context, upsampleY, upsampleX, cropTop, cropBottom, cropLeft, cropRight);
+  Tensor noBias;
+  if (!backMode) {
+    Tensor output = newOutput(allocator, device, type, outputShape);
+    failFromContext(context, op.forward(output, data, filters, hasBiases ? biases : noBias));
     out[0] = output;
     return;
   }
@@ -403,6 +523,9 @@ ErrorCode guarded(Body body, Context& context, Allocator& allocator, int nout, T
 
 ErrorCode vl_nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
   return guarded(nnconv, context, allocator, nout, out, nin, in, message);
+}
+ErrorCode vl_nnconvt(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
+  return guarded(nnconvt, context, allocator, nout, out, nin, in, message);
 }
 ErrorCode vl_nnbnorm(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
   return guarded(nnbnorm, context, allocator, nout, out, nin, in, message);

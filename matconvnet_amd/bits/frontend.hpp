@@ -2,7 +2,8 @@
 // C++ entry points (no MATLAB needed).  Each function takes what the MEX driver's mexFunction takes --
 // a list of inputs (arrays and strings) and a number of requested outputs -- and applies the same
 // parsing, validation, output-allocation and error rules:
-//   vl_nnconv (x, f, b [, dzdy], options...)   matlab/src/vl_nnconv.cu:87-502
+//   vl_nnconv (x, f, b [, dzdy], options...)   matlab/src/vl_nnconv.cu:87-502  (empty f: subsample + bias)
+//   vl_nnconvt(x, f, b [, dzdy], options...)   matlab/src/vl_nnconvt.cu:81-417
 //   vl_nnbnorm(x, g, b [, dzdy], options...)   matlab/src/vl_nnbnorm.cu:73-301
 //   vl_nnpool (x, pool [, dzdy], options...)   matlab/src/vl_nnpool.cu:72-314
 // Where the MEX drivers raise a MATLAB error these return a vl::ErrorCode and leave the reference's
@@ -42,10 +43,13 @@ class Allocator {
 // out[0..nout-1] receive views of freshly allocated outputs.  A skipped output is an empty 0 x 0 null
 // tensor, as the MEX drivers return empty matrices.  Outputs by position:
 //   vl_nnconv : forward [y]             backward [dzdx, dzdf, dzdb]
+//   vl_nnconvt: forward [y]             backward [dzdx, dzdf, dzdb]
 //   vl_nnbnorm: forward [y, moments]    backward [dzdx, dzdg, dzdb, moments]
 //   vl_nnpool : forward [y]             backward [dzdx]
 ErrorCode vl_nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                     std::string& message);
+ErrorCode vl_nnconvt(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
+                     std::string& message);
 ErrorCode vl_nnbnorm(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                      std::string& message);
 ErrorCode vl_nnpool(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,

@@ -25,7 +25,7 @@ typedef struct vlh_arg {
 
 typedef void* (*vlh_alloc_fn)(void* user, int device, size_t bytes);
 
-/* function: "vl_nnconv" | "vl_nnbnorm" | "vl_nnpool".  `out` must have room for 4 entries.  Returns a
+/* function: "vl_nnconv" | "vl_nnconvt" | "vl_nnbnorm" | "vl_nnpool".  `out` must have room for 4 entries.  Returns a
    vl::ErrorCode; vlh_last_message() has the text. */
 VLH_API int vlh_call(const char* function, int nout, vlh_arg* out, int nin, const vlh_arg* in, vlh_alloc_fn alloc,
                      void* user, void* stream);

@@ -116,3 +116,61 @@ ErrorCode Convolution::backward(Tensor& derInput, Tensor& derFilter, Tensor& der
   }
   return VLE_Success;
 }
+
+// ---------------------------------------------------------------------------------- ConvolutionTranspose
+//
+// The transpose of a convolution with stride = upsample and pad = crop (matlab/src/bits/nnconv.cu:323-421):
+// forward is that convolution's backward-data product with the roles of input and output exchanged, backward is
+// its forward and backward-filter products.  The reference loops over images in forward because its
+// per-image GEMM would otherwise fold the batch; the batched kernels here take the whole batch in one call.
+
+ConvolutionTranspose::ConvolutionTranspose(Context& context, int upsampleY, int upsampleX, int cropTop, int cropBottom,
+                                           int cropLeft, int cropRight)
+    : context(context), upsampleY(upsampleY), upsampleX(upsampleX), cropTop(cropTop), cropBottom(cropBottom),
+      cropLeft(cropLeft), cropRight(cropRight) {}
+
+ErrorCode ConvolutionTranspose::forward(Tensor& output, Tensor const& input, Tensor const& filter, Tensor const& bias) {
+  tensor_type tt = findTensorType(output, input, filter, bias);
+  ErrorCode e = requireHipFloat(context, tt, "ConvolutionTranspose::forward");
+  if (e != VLE_Success) return e;
+  if (!output || !input || !filter)
+    return context.setError(VLE_IllegalArgument, "ConvolutionTranspose::forward: OUTPUT, INPUT and FILTER are required");
+  if (bias && bias.getNumElements() != output.getDepth())
+    return context.setError(VLE_IllegalArgument, "ConvolutionTranspose::forward: the number of elements of BIASES is not the output depth");
+  Convolution opc(context, upsampleY, upsampleX, cropTop, cropBottom, cropLeft, cropRight, 1, 1);
+  Tensor null;
+  e = opc.backward(output, null, null, null, filter, input);
+  if (e != VLE_Success) return context.passError(e, "ConvolutionTranspose::forward");
+  if (bias) {
+    int rc = mcn_bias_add(context.getHipHelper().getStream(), (float*)output.getMemory(), (float const*)bias.getMemory(),
+                          asInt(output.getHeight()), asInt(output.getWidth()), asInt(output.getDepth()), asInt(output.getSize()));
+    return fromAbi(context, rc, "ConvolutionTranspose::forward");
+  }
+  return VLE_Success;
+}
+
+ErrorCode ConvolutionTranspose::backward(Tensor& derData, Tensor& derFilter, Tensor& derBias, Tensor const& input,
+                                         Tensor const& filter, Tensor const& derOutput) {
+  tensor_type tt = findTensorType(derData, derFilter, derBias, input, filter, derOutput);
+  ErrorCode e = requireHipFloat(context, tt, "ConvolutionTranspose::backward");
+  if (e != VLE_Success) return e;
+  if (!derOutput) return context.setError(VLE_IllegalArgument, "ConvolutionTranspose::backward: DEROUTPUT is required");
+  Convolution opc(context, upsampleY, upsampleX, cropTop, cropBottom, cropLeft, cropRight, 1, 1);
+  Tensor null;
+  if (derData) {
+    if (!filter) return context.setError(VLE_IllegalArgument, "ConvolutionTranspose::backward: FILTER is required for DERDATA");
+    e = opc.forward(derData, 0, derOutput, 1, filter, null);
+    if (e != VLE_Success) return context.passError(e, "ConvolutionTranspose::backward");
+  }
+  if (derFilter) {
+    if (!input) return context.setError(VLE_IllegalArgument, "ConvolutionTranspose::backward: INPUT is required for DERFILTER");
+    e = opc.backward(null, derFilter, null, derOutput, null, input);
+    if (e != VLE_Success) return context.passError(e, "ConvolutionTranspose::backward");
+  }
+  if (derBias) {
+    Tensor none1, none2;
+    e = opc.backward(none1, none2, derBias, null, null, derOutput);
+    if (e != VLE_Success) return context.passError(e, "ConvolutionTranspose::backward");
+  }
+  return VLE_Success;
+}

@@ -31,5 +31,28 @@ class Convolution {
   int dilateX;
 };
 
+// Same class interface as matlab/src/bits/nnconv.hpp:54-81.  FILTER is FH x FW x (output depth / groups) x (input
+// depth); output extent (H-1)*upsample - (cropA + cropB) + FH.
+class ConvolutionTranspose {
+ public:
+  ConvolutionTranspose(Context& context, int upsampleY, int upsampleX, int cropTop, int cropBottom, int cropLeft,
+                       int cropRight);
+
+  // output (fully overwritten) = convt(input, filter) + bias.  `bias` may be a null tensor.
+  vl::ErrorCode forward(vl::Tensor& output, vl::Tensor const& input, vl::Tensor const& filter, vl::Tensor const& bias);
+
+  // Any of derData / derFilter / derBias may be a null tensor, meaning "do not compute".
+  vl::ErrorCode backward(vl::Tensor& derData, vl::Tensor& derFilter, vl::Tensor& derBias, vl::Tensor const& input,
+                         vl::Tensor const& filter, vl::Tensor const& derOutput);
+
+  Context& context;
+  int upsampleY;
+  int upsampleX;
+  int cropTop;
+  int cropBottom;
+  int cropLeft;
+  int cropRight;
+};
+
 } }  // namespace vl::nn
 #endif

@@ -52,6 +52,10 @@ PROTOTYPES = {
     "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_filter": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_bias": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _sz]),
+    "mcn_subsample_output_size": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.POINTER(_i), C.POINTER(_i)]),
+    "mcn_subsample_forward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i]),
+    "mcn_subsample_backward": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i]),
+    "mcn_bias_add": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),
     "mcn_bnorm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "mcn_bnorm_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_bnorm_forward_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _d, _i, _vp, _sz]),

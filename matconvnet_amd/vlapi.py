@@ -1,7 +1,8 @@
 """ctypes binding of the C++ operator layer (libmcn_vl.so): the MATLAB-style entry points
 
     y                        = vl_nnconv(x, f, b, 'pad', p, 'stride', s, ...)
-    dzdx, dzdf, dzdb         = vl_nnconv(x, f, b, dzdy, ...)
+    dzdx, dzdf, dzdb         = vl_nnconv(x, f, b, dzdy, ...)            (f empty: subsample + bias)
+    y / dzdx, dzdf, dzdb     = vl_nnconvt(x, f, b[, dzdy], 'upsample', u, 'crop', c, 'numGroups', g)
     y[, moments]             = vl_nnbnorm(x, g, b, 'epsilon', e[, 'moments', m])
     dzdx, dzdg, dzdb[, mom]  = vl_nnbnorm(x, g, b, dzdy, ...)
     y / dzdx                 = vl_nnpool(x, pool[, dzdy], 'stride', s, 'pad', p, 'method', 'max'|'avg')
@@ -146,6 +147,13 @@ def vl_nnconv(*args, nout=None):
     n = nout if nout is not None else (3 if back else 1)
     r = _call("vl_nnconv", n, list(args))
     return r[0] if n == 1 else tuple(r[:n])
+
+
+def vl_nnconvt(*args, nout=None):
+    back = len(args) > 3 and not isinstance(args[3], str)
+    n = nout if nout is not None else (3 if back else 1)
+    r = _call("vl_nnconvt", n, list(args))
+    return r[0] if n == 1 else tuple(r)
 
 
 def vl_nnbnorm(*args, nout=None):

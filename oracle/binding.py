@@ -192,6 +192,77 @@ def conv_backward(x, f, dy, g, want=(True, True, True)):
     return dx, df, db
 
 
+def subsample_out_shape(xshape, stride=1, pad=0):
+    H, W, Cc, N = (list(xshape) + [1, 1, 1])[:4]
+    sy, sx = _pair(stride)
+    pt, pb, pl, pr = _quad(pad)
+    return ((H + pt + pb - 1) // sy + 1, (W + pl + pr - 1) // sx + 1, Cc, N)
+
+
+def subsample_forward(x, b, stride=1, pad=0):
+    """vl_nnconv(x, [], b, 'stride', s, 'pad', p): bits/nnsubsample.cu:36-117."""
+    s, _ = _sfx(x.dtype)
+    H, W, Cc, N = (list(x.shape) + [1, 1, 1])[:4]
+    sy, sx = _pair(stride)
+    pt, pb, pl, pr = _quad(pad)
+    y = fempty(subsample_out_shape(x.shape, stride, pad), x.dtype)
+    fn = getattr(lib(), "oracle_subsample_forward_" + s)
+    fn.argtypes = [C.c_void_p] * 3 + [C.c_int] * 10
+    fn(_p(y), _p(x), _p(b), H, W, Cc, N, sy, sx, pt, pb, pl, pr)
+    return y
+
+
+def subsample_backward(xshape, dy, stride=1, pad=0):
+    """dzdx of the same call (bits/nnsubsample.cu:125-165); dzdb is the per-channel sum of dzdy."""
+    s, _ = _sfx(dy.dtype)
+    H, W, Cc, N = (list(xshape) + [1, 1, 1])[:4]
+    sy, sx = _pair(stride)
+    pt, pb, pl, pr = _quad(pad)
+    dx = fempty((H, W, Cc, N), dy.dtype)
+    fn = getattr(lib(), "oracle_subsample_backward_" + s)
+    fn.argtypes = [C.c_void_p] * 2 + [C.c_int] * 10
+    fn(_p(dx), _p(dy), H, W, Cc, N, sy, sx, pt, pb, pl, pr)
+    return dx
+
+
+def convt_out_shape(xshape, fshape, upsample=1, crop=0, groups=1):
+    """vl_nnconvt.cu:296-299."""
+    H, W, Cc, N = (list(xshape) + [1, 1, 1])[:4]
+    FH, FW, FC, K = (list(fshape) + [1, 1, 1])[:4]
+    uy, ux = _pair(upsample)
+    ct, cb, cl, cr = _quad(crop)
+    return ((H - 1) * uy - (ct + cb) + FH, (W - 1) * ux - (cl + cr) + FW, FC * groups, N)
+
+
+def convt_forward(x, f, b, upsample=1, crop=0, groups=1):
+    """ConvolutionTransposeForward, bits/nnconv.cu:323-375: per image, the backward-data product of the
+    convolution with stride = upsample and pad = crop, taking x as the output derivative; then the bias."""
+    oshape = convt_out_shape(x.shape, f.shape, upsample, crop, groups)
+    x4 = farray(x).reshape((list(x.shape) + [1, 1, 1])[:4], order="F")
+    y = fempty(oshape, x.dtype)
+    for n in range(oshape[3]):
+        g = conv_geom(oshape[:3] + (1,), f.shape, upsample, crop, 1)
+        dx, _, _ = conv_backward(None, f, farray(x4[:, :, :, n:n + 1]), g, want=(True, False, False))
+        y[:, :, :, n] = dx[:, :, :, 0]
+    if b is not None:
+        y += np.asarray(b, dtype=x.dtype).reshape(1, 1, -1, 1)
+    return farray(y)
+
+
+def convt_backward(x, f, dy, upsample=1, crop=0, groups=1, want=(True, True, True)):
+    """ConvolutionTransposeBackward, bits/nnconv.cu:381-421: dzdx = forward convolution of dzdy, dzdf = the
+    filter derivative of that convolution with x in the role of its output derivative, dzdb = sums of dzdy."""
+    dy4 = farray(dy).reshape((list(dy.shape) + [1, 1, 1])[:4], order="F")
+    x4 = farray(x).reshape((list(x.shape) + [1, 1, 1])[:4], order="F")
+    g = conv_geom(dy4.shape, f.shape, upsample, crop, 1)
+    dx = conv_forward(dy4, f, None, g) if want[0] else None
+    df = conv_backward(dy4, None, x4, g, want=(False, True, False))[1] if want[1] else None
+    db = None
+    if want[2]:
+        db = conv_backward(None, None, dy4, conv_geom(dy4.shape, (1, 1, dy4.shape[2], dy4.shape[2])), want=(False, False, True))[2]
+    return dx, df, db
+
+
 def bnorm_forward(x, mult, bias, eps=1e-4, moments=None):
     s, ct = _sfx(x.dtype)
     H, W, Cc, N = (list(x.shape) + [1, 1, 1])[:4]

@@ -31,6 +31,17 @@
  *                                     matlab/xtest/suite/nnconv.m:88-161.  Only the
  *                                     summation order inside a GEMM is unpinned (it lives
  *                                     in MKL); the parity gate for conv is 2e-4 relative.
+ *   subsample_*                    -- bits/nnsubsample.cu needs the same <blas.h> (bias via
+ *                                     GEMM with a ones vector), so it cannot be built either.
+ *                                     Pinned by the reference's own definition -- empty
+ *                                     FILTERS "pretend the identity filter bank"
+ *                                     (vl_nnconv.cu:316-321): equal to oracle conv with
+ *                                     identity 1x1 filters, forward and backward, bit for bit
+ *                                     (tests/test_oracle_conv.py), plus brute force.
+ *   convolution transpose          -- composed in oracle/binding.py from conv_backward /
+ *                                     conv_forward exactly as bits/nnconv.cu:323-421 does;
+ *                                     pinned against torch conv_transpose2d autograd in
+ *                                     double (upsample, crop, groups).
  */
 #ifndef MCN_ORACLE_H
 #define MCN_ORACLE_H
@@ -106,7 +117,15 @@ void oracle_set_dgemm(void* fn);
   void oracle_relu_forward_##S(T* y, const T* x, size_t n);                               \
   void oracle_relu_backward_##S(T* dx, const T* x, const T* dy, size_t n);                \
   /* matlab/+dagnn/Sum.m:11-17 for two inputs */                                           \
-  void oracle_sum_##S(T* y, const T* a, const T* b, size_t n);
+  void oracle_sum_##S(T* y, const T* a, const T* b, size_t n);                            \
+  /* bits/nnsubsample.cu:36-117 (vl_nnconv with empty FILTERS); bias may be NULL */        \
+  void oracle_subsample_forward_##S(T* y, const T* x, const T* bias, int H, int W, int C, \
+                                    int N, int strideY, int strideX, int padTop,           \
+                                    int padBottom, int padLeft, int padRight);             \
+  /* bits/nnsubsample.cu:125-165 */                                                        \
+  void oracle_subsample_backward_##S(T* dx, const T* dy, int H, int W, int C, int N,      \
+                                     int strideY, int strideX, int padTop, int padBottom, \
+                                     int padLeft, int padRight);
 
 ORACLE_DECLARE(float, f32)
 ORACLE_DECLARE(double, f64)

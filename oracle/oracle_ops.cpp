@@ -363,6 +363,45 @@ void pool_backward(T* dx, const T* x, const T* dy, const oracle_pool_geom& g) {
 
 }  // namespace
 
+// ---------------------------------------------------------------------------------------------------
+// Subsampling with bias: what vl_nnconv computes for empty FILTERS (bits/nnsubsample.cu).
+// ---------------------------------------------------------------------------------------------------
+
+// bits/nnsubsample.cu:36-72 (sampling) and :88-117 (bias: output += ones * biases', one add per element)
+template <typename T>
+static void subsample_forward(T* y, const T* x, const T* bias, int H, int W, int Cc, int N, int sy, int sx, int pt,
+                              int pb, int pl, int pr) {
+  const int outW = (W + (pl + pr) - 1) / sx + 1, outH = (H + (pt + pb) - 1) / sy + 1;
+  for (long z = 0; z < (long)Cc * N; ++z) {
+    const T* in = x + z * (long)W * H;
+    T* out = y + z * (long)outW * outH;
+    for (int ox = 0; ox < outW; ++ox)
+      for (int oy = 0; oy < outH; ++oy) {
+        const int x1 = ox * sx - pl, y1 = oy * sy - pt;
+        T value = 0;
+        if (x1 >= 0 && x1 < W && y1 >= 0 && y1 < H) value = in[x1 * H + y1];
+        out[ox * outH + oy] = bias ? value + bias[z % Cc] : value;
+      }
+  }
+}
+
+// bits/nnsubsample.cu:125-165: zero-fill, then every sampled position receives its output's derivative
+template <typename T>
+static void subsample_backward(T* dx, const T* dy, int H, int W, int Cc, int N, int sy, int sx, int pt, int pb, int pl,
+                               int pr) {
+  const int outW = (W + (pl + pr) - 1) / sx + 1, outH = (H + (pt + pb) - 1) / sy + 1;
+  std::memset(dx, 0, sizeof(T) * (size_t)W * H * Cc * N);
+  for (long z = 0; z < (long)Cc * N; ++z) {
+    T* din = dx + z * (long)W * H;
+    const T* dout = dy + z * (long)outW * outH;
+    for (int px = 0; px < outW; ++px)
+      for (int py = 0; py < outH; ++py) {
+        const int x1 = px * sx - pl, y1 = py * sy - pt;
+        if (x1 >= 0 && x1 < W && y1 >= 0 && y1 < H) din[x1 * H + y1] = dout[px * outH + py];
+      }
+  }
+}
+
 extern "C" {
 
 int oracle_conv_out_h(const oracle_conv_geom* g) {
@@ -415,6 +454,14 @@ int oracle_pool_out_w(const oracle_pool_geom* g) {
   }                                                                                                \
   void oracle_sum_##S(T* y, const T* a, const T* b, size_t n) {                                    \
     for (size_t i = 0; i < n; ++i) y[i] = a[i] + b[i];                                             \
+  }                                                                                                \
+  void oracle_subsample_forward_##S(T* y, const T* x, const T* bias, int H, int W, int Cc, int N, \
+                                    int sy, int sx, int pt, int pb, int pl, int pr) {              \
+    subsample_forward<T>(y, x, bias, H, W, Cc, N, sy, sx, pt, pb, pl, pr);                         \
+  }                                                                                                \
+  void oracle_subsample_backward_##S(T* dx, const T* dy, int H, int W, int Cc, int N, int sy,     \
+                                     int sx, int pt, int pb, int pl, int pr) {                     \
+    subsample_backward<T>(dx, dy, H, W, Cc, N, sy, sx, pt, pb, pl, pr);                            \
   }
 
 ORACLE_DEFINE(float, f32)

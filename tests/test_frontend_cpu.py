@@ -70,12 +70,6 @@ def test_vl_nnconv_validation(vl, args, message):
     assert e.value.message == message
 
 
-def test_vl_nnconv_empty_filters_are_reported_unsupported(vl):
-    with pytest.raises(vl.VlError) as e:
-        vl.vl_nnconv(z(8, 8, 4, 2), torch.zeros((0,)), z(4))
-    assert e.value.code == 1 and "FILTERS" in e.value.message
-
-
 BNORM_ERRORS = [
     ((z(8, 8, 4, 2), z(4)), "The arguments are less than three."),
     ((z(8, 8, 4, 2), z(3), z(4)), "The MULTIPLIERS size does not match the DATA depth."),
@@ -113,3 +107,47 @@ def test_vl_nnpool_validation(vl, args, message):
     with pytest.raises(vl.VlError) as e:
         vl.vl_nnpool(*args)
     assert e.value.message == message
+
+
+CONVT_ERRORS = [
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4)), "There are less than three arguments."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(5), "upsample", 0), "At least one element of UPSAMPLE is smaller than one."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(5), "upsample", [1, 2, 3]), "upsample has neither one nor two elements."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(5), "crop", -1), "An element of CROP is negative."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(5), "crop", [1, 2]), "crop has neither one nor two elements."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(5), "numgroups", 0), "NUMGROUPS is less than 1."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(5), "numgroups", 3),
+     "The number of filter groups does not divide the filter bank depth (fourth dimension of FILTERS)."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 6), z(5)),
+     "The filter bank depth (fourth dimension of FILTERS) is not the same as the data depth (third dimension of X)."),
+    ((z(2, 2, 4, 2), z(3, 3, 5, 4), z(5), "crop", 2), "The output array is empty due to CROP being too large."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(5), z(9, 9, 5, 2)), "DEROUTPUT dimensions are incompatible with X and FILTERS."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(7)), "The number of elements of BIASES is not the same as the dimenison of the filters."),
+    ((z(8, 8, 4, 2), z(3, 3, 5, 4), z(5), "bogus", 1), "Unknown option 'bogus'."),
+]
+
+
+@pytest.mark.parametrize("args,message", CONVT_ERRORS)
+def test_vl_nnconvt_messages(vl, args, message):
+    """Texts and order of matlab/src/vl_nnconvt.cu:105-320."""
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconvt(*args)
+    assert e.value.message == message
+
+
+def test_vl_nnconv_empty_filters_follow_the_identity_bank_rules(vl):
+    """vl_nnconv.cu:293-295,316-321,337-341: no dilation without filters; BIASES sized by the data depth; the
+    output has the data's depth."""
+    e0 = torch.zeros((0,), dtype=torch.float32)
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(z(8, 8, 4, 2), e0, z(4), "dilate", 2)
+    assert e.value.message == "There are no filters and DILATE is not one."
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(z(8, 8, 4, 2), e0, z(5))
+    assert e.value.message == "The number of elements of BIASES is not the same as the number of filters."
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnconv(z(8, 8, 4, 2), e0, z(4), z(4, 4, 5, 2), "stride", 2)
+    assert e.value.message == "DEROUTPUT dimensions are incompatible with X and FILTERS."
+    with pytest.raises(vl.VlError) as e:  # valid arguments reach the operator, which has no CPU path
+        vl.vl_nnconv(z(8, 8, 4, 2), e0, z(4), "stride", 2)
+    assert e.value.code == 1
