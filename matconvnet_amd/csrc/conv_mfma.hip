@@ -37,20 +37,6 @@ constexpr int kMaxTaps = 128;
 // pixel-major kernel (forward / backward-data)
 // ------------------------------------------------------------------------------------------------
 
-struct PixP {
-  int IH, IW, Cin;    // grid and channels of the gathered tensor
-  int OH, OW, Cout;   // grid and channels of the produced tensor
-  int N;
-  int FH, T;          // filter height, taps = FH*FW
-  int sy, sx;         // gathered row = oh*sy + dh(tap)
-  int dhBase, dhStep, dwBase, dwStep;
-  int R;              // reduction length = T*Cin
-  int coutPad;        // row pitch of wt
-  int M;              // OH*OW*N (< 2^31)
-  float alpha, beta;
-  FastDiv byQ, byOH, byT;  // Q = OH*OW; T = taps
-  int advC, advT;          // 16 = advC*T + advT (reduction rows per step)
-};
 
 // wt[R][co] from the MATLAB filter bank f[i,j,c,k] (FV x K, column-major), t = i + FH*j.
 //   reduction row R = t + T*ci (channel-major) or, when tapMajor, R = ci + Cin*t
@@ -636,6 +622,12 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   p.byT = FastDiv(p.T);
   p.advC = 16 / p.T;
   p.advT = 16 % p.T;
+  // small filter banks: keep all the weights in LDS and stream the pixels past them (conv_ws.hip)
+  if (ut) {
+    int handled = 0;
+    rc = conv_ws_launch(s, who, out, in, wt, bias, p, &handled);
+    if (rc || handled) return rc;
+  }
   // Tile shape, channels x pixels per workgroup: the widest pixel tile that still yields >= 2048 workgroups
   // (8 per CU), because short reduction loops hide their load latency only through occupancy.  The tunable
   // forces a shape for experiments.

@@ -1,0 +1,330 @@
+// Weights-stationary implicit-GEMM convolution for small filter banks (forward and backward-data of layers whose
+// whole packed bank wt[R][co] fits in LDS: the 1x1 and 3x3 layers of a ResNet bottleneck, for instance).
+//
+// The tiled kernel of conv_mfma.hip stages both operands through LDS with a barrier per 16 reduction rows; with
+// short reductions (R = 64 ... 576) and 64-channel tiles its workgroups spend most of their time waiting for the
+// one step of loads they have in flight.  Here
+//   * a persistent workgroup copies the bank into LDS once (up to 150 KB; one or two workgroups per CU), laid out
+//     [channel block][R][32 WA] so that every weight-fragment read is "lane base + immediate";
+//   * each wavefront then works alone, with no barriers: it takes units of 32 pixels x (32 WA) output channels;
+//     the pixel operand of v_mfma_f32_32x32x2_f32 is exactly "lane = pixel (l32), half = reduction row (kh)", so it
+//     is loaded from global memory straight into the register the MFMA reads -- 32 consecutive pixels of one
+//     channel per half-wave, 128-byte runs;
+//   * those loads are buffer loads: the per-lane offset is the pixel (+ tap shift), the scalar offset is the
+//     channel, and a lane whose shifted pixel falls outside the image simply uses an offset beyond the tensor,
+//     for which the hardware returns 0 -- no masks, no selects, no branches, no out-of-bounds access possible;
+//   * three register buffers of 8 reduction pairs rotate, so two groups of loads are in flight behind the one
+//     being multiplied, and the first loads of a wave's next unit are issued before the stores of the finished one;
+//   * the loop carries about one vector-ALU instruction per 8 MFMAs (vector-ALU work is what competes with the
+//     matrix pipe for the SIMD: with 5 per MFMA an earlier form of this kernel reached only half the MFMA rate);
+//   * units are dealt so that every SIMD of the chip gets the same number of them to within one, and the channel
+//     blocks of one pixel block go to neighbouring wavefronts of one workgroup (the pixels come from HBM once).
+// Reduction order: tap-major (R = ci + Cin*t), pairs of rows per MFMA, sequential accumulation in fp32 like the
+// tiled kernel.
+#include "conv_common.hpp"
+
+#include <algorithm>
+
+namespace mcn {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kDepth = 8;       // reduction pairs per group: Cin must be a multiple of 16 so a group stays inside a tap
+constexpr int kMaxTapsWs = 128;
+constexpr unsigned kOutside = 0x80000000u;  // buffer offset no tensor reaches (tensors here are < 2 GiB): reads as 0
+
+struct WsP {
+  int nUnits;        // pixel blocks x channel blocks
+  int chanBlocks;    // coutPad / (32 WA)
+  int groups;        // R / (2 kDepth)
+  int groupsPerTap;  // Cin / (2 kDepth)
+  unsigned inBytes;  // size of the gathered tensor
+  FastDiv byCB, byRow;  // byRow: 8 WA = 16-byte vectors per bank row of one channel block
+};
+
+// A store the compiler's memory-wait bookkeeping does not see.  With ordinary stores in flight beside loads it
+// can no longer tell which of them the hardware counter is counting and waits for everything at every use of a
+// loaded value, which would drain the load pipeline at every MFMA of the next unit.  The hardware counter still
+// counts these stores; that only makes the compiler's waits for older loads (which return in order among
+// themselves) longer, never shorter.  Store data is read when the instruction issues, so the accumulators can be
+// cleared right after.
+__device__ __forceinline__ void store_untracked(float* ptr, float v) {
+  asm volatile("global_store_dword %0, %1, off" ::"v"(ptr), "v"(v) : "memory");
+}
+
+template <int WA, bool TAPS, int THREADS>
+__global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out, const float* __restrict__ in,
+                                                        const float* __restrict__ wt, const float* __restrict__ bias,
+                                                        PixP p, WsP w) {
+  extern __shared__ float smem[];
+  float* wtL = smem;                               // [chanBlocks][R][32 WA]
+  int2* tapTab = (int2*)(smem + p.R * p.coutPad);  // [T] .x = dh + IH*dw, .y = (dh & 0xffff) | (dw << 16)
+  constexpr int ROW = 32 * WA;                     // floats per bank row of one channel block
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  // (readfirstlane tells the compiler what it cannot see: a wavefront's index is the same in all its lanes, so
+  // everything derived from it -- the unit, the loop bounds, the scalar load offsets -- lives in scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, kh = lane >> 5;
+  const int IHW = p.IH * p.IW, Q = p.OH * p.OW;
+
+  // ---- once per workgroup: the bank, re-laid by channel block, and the tap table
+  {
+    const int perBlock = p.R * (ROW / 4);  // 16-byte vectors per channel block
+    const int n4 = perBlock * w.chanBlocks;
+    for (int i = tid; i < n4; i += THREADS) {
+      const int cbk = i / perBlock;  // (one-time code: a plain division)
+      const int rem = i - cbk * perBlock;
+      int r, v;
+      w.byRow.divmod(rem, &r, &v);
+      ((float4*)wtL)[i] = *(const float4*)(wt + (size_t)r * p.coutPad + cbk * ROW + v * 4);
+    }
+    if (TAPS && tid < p.T) {
+      const int j = tid / p.FH, i = tid - j * p.FH;
+      const int dh = p.dhBase + i * p.dhStep, dw = p.dwBase + j * p.dwStep;
+      tapTab[tid] = make_int2(dh + p.IH * dw, (int)((unsigned)(dh & 0xffff) | ((unsigned)dw << 16)));
+    }
+  }
+  __syncthreads();
+
+  // ---- units of this wavefront.  The channel blocks of one pixel block go to neighbouring wavefronts of one
+  // workgroup, which reach them at about the same time.  Pixel blocks are dealt slot-major (slot = wavefront /
+  // channel blocks), so that consecutive pixel blocks sit on different CUs and every SIMD of the chip gets the
+  // same number of units to within one.
+  constexpr int wavesPerGroup = THREADS / 64;
+  const int sib = w.chanBlocks <= wavesPerGroup ? w.chanBlocks : 1;  // siblings side by side (else one wave, all blocks in turn)
+  const int slots = wavesPerGroup / sib;
+  const int unitStep = (int)gridDim.x * slots * sib;
+  int unit = ((wave / sib) * (int)gridDim.x + (int)blockIdx.x) * sib + (wave % sib);
+  if (wave >= slots * sib || unit >= w.nUnits) return;
+
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, (int)w.inBytes, 0x00020000);
+  const int planeBytes = IHW * 4;
+
+  // per-unit, per-lane state
+  unsigned voff;   // byte offset of this lane's pixel and reduction half at tap shift 0 (kOutside for idle lanes)
+  int ihB, iwB;    // gathered coordinates at tap shift 0
+  int cb;          // channel block of the unit
+
+  auto setup = [&](int u) {
+    int pb;
+    w.byCB.divmod(u, &pb, &cb);
+    const int m = pb * 32 + l32;
+    const bool mvalid = m < p.M;
+    int n, q, ow, oh;
+    p.byQ.divmod(mvalid ? m : 0, &n, &q);
+    p.byOH.divmod(q, &ow, &oh);
+    ihB = oh * p.sy;
+    iwB = ow * p.sx;
+    voff = mvalid ? (unsigned)(n * (p.Cin * IHW) + ihB + p.IH * iwB + kh * IHW) * 4u : kOutside;
+  };
+
+  // per-lane offset of the pixels of tap `tap` (kOutside where the shifted pixel is not in the image)
+  auto tap_offset = [&](int tap) -> unsigned {
+    if (!TAPS) return voff;
+    const int2 tp = tapTab[tap];
+    const int shift = __builtin_amdgcn_readfirstlane(tp.x), packed = __builtin_amdgcn_readfirstlane(tp.y);
+    const int ih = ihB + (int)(short)(packed & 0xffff), iw = iwB + (packed >> 16);
+    const bool ok = voff != kOutside && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
+    return ok ? voff + (unsigned)(shift * 4) : kOutside;
+  };
+
+  typedef float vbuf __attribute__((ext_vector_type(kDepth)));
+  vbuf b0, b1, b2;
+  // the loader's position in the current unit: next group, its tap, its 16-channel chunk inside the tap, and the
+  // per-lane offset of that tap's pixels (kept in a register of its own for the whole tap: recomputing it per
+  // group let the register allocator hand its register to a load result, and every group then waited for all
+  // loads in flight before it could form the next offset)
+  int gLoad, tapL, giL;
+  unsigned voTap;
+
+  // Loads the loader's next group into DST and advances it.  Past the last group the loads still go out, with
+  // the "outside" offset (they fetch nothing and return 0): the instruction stream stays the same on every path,
+  // which lets the compiler count exactly how many younger loads may stay in flight at each MFMA.
+#define WS_LOAD_NEXT(DST)                                                                                 \
+  do {                                                                                                    \
+    const int sbase_ = giL * (2 * kDepth) * planeBytes;                                                   \
+    _Pragma("unroll") for (int d_ = 0; d_ < kDepth; ++d_) DST[d_] = __builtin_bit_cast(                   \
+        float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voTap, sbase_ + 2 * d_ * planeBytes, 0));  \
+    ++gLoad;                                                                                              \
+    if (++giL == w.groupsPerTap) {                                                                        \
+      giL = 0;                                                                                            \
+      ++tapL;                                                                                             \
+      voTap = gLoad < w.groups ? tap_offset(TAPS ? min(tapL, p.T - 1) : 0) : kOutside;                    \
+    }                                                                                                     \
+  } while (0)
+
+#define WS_PRIME()             \
+  do {                         \
+    gLoad = 0;                 \
+    tapL = 0;                  \
+    giL = 0;                   \
+    voTap = tap_offset(0);     \
+    WS_LOAD_NEXT(b0);          \
+    WS_LOAD_NEXT(b1);          \
+  } while (0)
+
+  // multiply group G (operands CUR) after putting the loader's next group (G + 2) in flight into FREE
+#define WS_STEP(G, CUR, FREE)                                                                                     \
+  if ((G) < w.groups) {                                                                                          \
+    WS_LOAD_NEXT(FREE);                                                                                          \
+    const float* aG_ = aLane + (G) * (2 * kDepth * ROW);                                                         \
+    constexpr int HALF_ = kDepth / 2;                                                                            \
+    _Pragma("unroll") for (int h_ = 0; h_ < 2; ++h_) {                                                           \
+      float av_[HALF_][WA];                                                                                      \
+      _Pragma("unroll") for (int d_ = 0; d_ < HALF_; ++d_)                                                       \
+        _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_) av_[d_][a_] = aG_[(2 * (h_ * HALF_ + d_)) * ROW + a_ * 32]; \
+      _Pragma("unroll") for (int d_ = 0; d_ < HALF_; ++d_)                                                       \
+        _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_)                                                        \
+          acc[a_] = __builtin_amdgcn_mfma_f32_32x32x2f32(av_[d_][a_], CUR[h_ * HALF_ + d_], acc[a_], 0, 0, 0);   \
+    }                                                                                                            \
+  }
+
+  setup(unit);
+  WS_PRIME();
+
+  while (true) {
+    floatx16 acc[WA];
+#pragma unroll
+    for (int a = 0; a < WA; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
+
+    const float* aLane = wtL + (size_t)cb * p.R * ROW + kh * ROW + l32;
+    for (int g0 = 0; g0 < w.groups; g0 += 3) {
+      WS_STEP(g0, b0, b2)
+      WS_STEP(g0 + 1, b1, b0)
+      WS_STEP(g0 + 2, b2, b1)
+    }
+
+    // ---- the finished unit's geometry, then the next unit's first loads, then the stores
+    const int doneCb = cb;
+    const int mo = w.byCB.div(unit) * 32 + l32;  // unit = pixel block * chanBlocks + channel block
+    const int next = unit + unitStep;
+    const bool more = next < w.nUnits;
+    if (more) {
+      setup(next);
+      WS_PRIME();
+    }
+    if (mo < p.M) {
+      int n, q;
+      p.byQ.divmod(mo, &n, &q);
+      float* o = out + (size_t)n * p.Cout * Q + q;
+#pragma unroll
+      for (int a = 0; a < WA; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int co = doneCb * ROW + a * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
+          if (co < p.Cout) {
+            float v = p.alpha * acc[a][r];
+            if (p.beta != 0.f) v = fmaf(p.beta, o[(size_t)co * Q], v);
+            if (bias) v += bias[co];
+            store_untracked(o + (size_t)co * Q, v);
+          }
+        }
+    }
+    if (!more) break;
+    unit = next;
+  }
+#undef WS_STEP
+#undef WS_PRIME
+#undef WS_LOAD_NEXT
+}
+
+template <int WA, bool TAPS, int THREADS>
+int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, const float* in, const float* wt,
+           const float* bias, const PixP& p, const WsP& w) {
+  static size_t raised = 0;  // largest dynamic LDS size this instantiation has been opted into
+  if (lds > 64 * 1024 && lds > raised) {
+    if (hipFuncSetAttribute((const void*)conv_ws_mfma<WA, TAPS, THREADS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(MCN_DEVICE_ERROR, "%s: cannot reserve %zu bytes of LDS", who, lds);
+    }
+    raised = lds;
+  }
+  KernelTimer timer("conv_ws_mfma", s);
+  hipLaunchKernelGGL((conv_ws_mfma<WA, TAPS, THREADS>), dim3((unsigned)blocks), dim3(THREADS), lds, s, out, in, wt, bias, p, w);
+  return check_launch(who);
+}
+
+// Wavefronts per CU: 16 (4 per SIMD, 128 registers each) for the narrow units; 8 for WA = 4, whose 64 accumulator
+// registers plus operands need more than 128.
+template <int WA, bool TAPS>
+int dispatch(hipStream_t s, const char* who, int cus, bool twoFit, size_t lds, float* out, const float* in, const float* wt,
+             const float* bias, const PixP& p, const WsP& w) {
+  if constexpr (WA == 4) {
+    return launch<WA, TAPS, 512>(s, who, cus, lds, out, in, wt, bias, p, w);
+  } else {
+    if (twoFit) return launch<WA, TAPS, 512>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
+    return launch<WA, TAPS, 1024>(s, who, cus, lds, out, in, wt, bias, p, w);
+  }
+}
+
+}  // namespace
+
+int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, const float* wt, const float* bias,
+                   const PixP& p, int* handled) {
+  *handled = 0;
+  if (tunable("conv_no_ws", 0)) return MCN_SUCCESS;
+  if (p.Cin % (2 * kDepth) != 0 || p.T > kMaxTapsWs || p.coutPad % 32 != 0) return MCN_SUCCESS;
+  const size_t lds = (size_t)p.R * p.coutPad * sizeof(float) + (size_t)p.T * sizeof(int2);
+  if (lds > 150 * 1024) return MCN_SUCCESS;
+  // byte offsets into the gathered tensor must stay below the "outside" offset
+  const long long inBytes = (long long)p.IH * p.IW * p.Cin * p.N * 4;
+  if (inBytes >= (long long)kOutside) return MCN_SUCCESS;
+
+  int cus = mcn_device_compute_units();
+  if (cus <= 0) cus = 256;
+  const bool twoFit = lds <= 78 * 1024;  // two workgroups per CU fit the 160 KB
+  const long long simds = (long long)cus * 4;
+  const long long pixelBlocks = ((long long)p.M + 31) / 32;
+
+  // channels per wavefront: the widest unit that still spreads evenly over the SIMDs (wider units amortise the
+  // pixel loads over more MFMAs; narrower ones balance better)
+  const int minUnits = tunable("conv_ws_min_units", 0);
+  // Measured on the 56x56 bottleneck shapes: with a short reduction (64 channels, one tap) a unit is 32 MFMAs
+  // between a prologue and 16 stores, and the tiled kernel's wider tiles win; from 128 rows up this kernel does.
+  if (minUnits <= 0 && p.R < 128) return MCN_SUCCESS;
+  int WA = tunable("conv_ws_wa", 0);
+  if (WA != 1 && WA != 2 && WA != 4 && p.T > 1 && p.coutPad % 64 == 0 && p.coutPad < 128) WA = 2;  // measured best for 3x3, 64 channels
+  if (WA != 1 && WA != 2 && WA != 4) {
+    double best = 0;
+    for (int cand : {4, 2, 1}) {
+      if (p.coutPad % (32 * cand) != 0) continue;
+      const long long units = pixelBlocks * (p.coutPad / (32 * cand));
+      const double balance = (double)units / (double)(((units + simds - 1) / simds) * simds);
+      const double issue = cand == 4 ? 0.96 : (cand == 2 ? 0.94 : 0.90);
+      if (balance * issue > best) {
+        best = balance * issue;
+        WA = cand;
+      }
+    }
+  }
+  if (p.coutPad % (32 * WA) != 0) return MCN_SUCCESS;
+  WsP w;
+  w.chanBlocks = p.coutPad / (32 * WA);
+  const long long units = pixelBlocks * w.chanBlocks;
+  // too little work to keep every SIMD busy: leave it to the tiled kernel
+  if (units >= (1ll << 31) || units < (minUnits > 0 ? (long long)minUnits : simds * 2)) return MCN_SUCCESS;
+  w.nUnits = (int)units;
+  w.groups = p.R / (2 * kDepth);
+  w.groupsPerTap = p.Cin / (2 * kDepth);
+  w.inBytes = (unsigned)inBytes;
+  w.byCB = FastDiv(w.chanBlocks);
+  w.byRow = FastDiv(8 * WA);
+  const bool taps = !(p.T == 1 && p.dhBase == 0 && p.dwBase == 0 && p.sy == 1 && p.sx == 1 && p.IH == p.OH && p.IW == p.OW);
+  int rc;
+  if (taps) rc = WA == 4 ? dispatch<4, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
+                 : (WA == 2 ? dispatch<2, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
+                            : dispatch<1, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w));
+  else rc = WA == 4 ? dispatch<4, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
+            : (WA == 2 ? dispatch<2, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
+                       : dispatch<1, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w));
+  *handled = 1;
+  return rc;
+}
+
+}  // namespace mcn

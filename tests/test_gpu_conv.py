@@ -187,3 +187,54 @@ def test_errors(capi):
         capi.conv_out_shape(capi.conv_geom((2, 2, 3, 1), (3, 3, 3, 4)))
     with pytest.raises(capi.McnError):
         capi.conv_out_shape(capi.conv_geom((8, 8, 4, 1), (3, 3, 2, 3)))  # 2 groups do not divide 3 filters
+
+
+WS_CASES = [  # (xshape, fshape, stride, pad, dilate): channel counts a multiple of 16, bank small enough for LDS
+    ((20, 18, 32, 3), (1, 1, 32, 64), 1, 0, 1),
+    ((20, 18, 64, 2), (1, 1, 64, 40), 1, 0, 1),          # output channels not a multiple of 32
+    ((13, 11, 16, 5), (3, 3, 16, 32), 1, 1, 1),          # pixels not a multiple of 32
+    ((17, 15, 32, 2), (3, 3, 32, 48), 1, (2, 0, 1, 3), 1),
+    ((19, 19, 16, 2), (3, 2, 16, 96), (2, 3), 1, 1),     # strided: forward only on this path
+    ((21, 20, 16, 2), (3, 3, 16, 32), 1, 2, 2),          # dilated
+    ((12, 12, 48, 4), (5, 5, 48, 16), 1, 2, 1),
+]
+
+
+@pytest.mark.parametrize("wa", [0, 1, 2, 4])
+@pytest.mark.parametrize("xs,fs,stride,pad,dilate", WS_CASES)
+def test_weights_stationary_kernel(capi, ob, xs, fs, stride, pad, dilate, wa):
+    """Forward and backward-data through the weights-stationary MFMA kernel (forced onto small problems),
+    every width of its units, against the oracle."""
+    r = np.random.default_rng(sum(xs) + sum(fs) + wa)
+    x = F(r.standard_normal(xs))
+    f = F(r.standard_normal(fs) * 0.2)
+    b = r.standard_normal(fs[3]).astype(np.float32)
+    g = ob.conv_geom(xs, fs, stride, pad, dilate)
+    cg = capi.conv_geom(xs, fs, stride, pad, dilate)
+    capi.set_tunable("conv_ws_min_units", 1)
+    capi.set_tunable("conv_ws_wa", wa)
+    try:
+        capi.profile_begin("conv_ws_mfma")
+        y = capi.conv_forward(capi.to_device(x), capi.to_device(f), capi.to_device(b), cg)
+        want = ob.conv_forward(x, f, b, g)
+        dy = F(r.standard_normal(want.shape))
+        dx, _, _ = capi.conv_backward(capi.to_device(x), capi.to_device(f), capi.to_device(dy), cg, want=(True, False, False))
+        launches, _ = capi.profile_end()
+    finally:
+        capi.set_tunable("conv_ws_min_units", 0)
+        capi.set_tunable("conv_ws_wa", 0)
+    strided = np.any(np.atleast_1d(stride) != 1)
+
+    def eligible(cin, cout):
+        """The kernel's own admission rule: reduction channels a multiple of 16, the packed bank (padded to the
+        channel tile) within 150 KB of LDS, the padded channel count a whole number of units."""
+        taps = fs[0] * fs[1]
+        tile = 128 if cout > 64 else (64 if cout > 32 else 32)
+        padded = -(-cout // tile) * tile
+        return (cin % 16 == 0 and taps * cin * padded * 4 + taps * 8 <= 150 * 1024 and
+                (wa == 0 or padded % (32 * wa) == 0))
+
+    expected = int(eligible(xs[2], fs[3])) + int(eligible(fs[3], xs[2]) and not strided)
+    assert launches == expected  # the kernel under test really ran
+    assert rel_max(capi.to_host(y), want) < 2e-4
+    assert rel_max(capi.to_host(dx), ob.conv_backward(x, f, dy, g, want=(True, False, False))[0]) < 2e-4
