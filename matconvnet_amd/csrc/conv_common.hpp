@@ -48,7 +48,82 @@ struct PixP {
   float alpha, beta;
   FastDiv byQ, byOH, byT;  // Q = OH*OW; T = taps
   int advC, advT;          // 16 = advC*T + advT (reduction rows per step)
+  unsigned outBytes;       // size of the produced tensor, or 0 when it does not fit a 2 GiB buffer descriptor
 };
+
+// ------------------------------------------------------------------------------------------------
+// Epilogue shared by the pixel-major MFMA kernels
+// ------------------------------------------------------------------------------------------------
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef int bufrsrc __attribute__((ext_vector_type(4)));
+
+constexpr unsigned kOutside = 0x80000000u;  // buffer offset no tensor handled here reaches (they are < 2 GiB)
+
+// Raw buffer descriptor over `bytes` bytes at `base` (uniform): accesses at offsets >= bytes are dropped (stores)
+// or return 0 (loads).
+__device__ __forceinline__ bufrsrc make_bufrsrc(const void* base, unsigned bytes) {
+  const unsigned long long a = (unsigned long long)base;
+  bufrsrc r;
+  r.x = (int)(unsigned)(a & 0xffffffffull);
+  r.y = (int)(unsigned)((a >> 32) & 0xffffull);
+  r.z = (int)bytes;
+  r.w = 0x00020000;
+  return r;
+}
+
+// A store the compiler's memory-wait bookkeeping does not see.  With ordinary stores in flight beside loads it
+// can no longer tell which of them the hardware counter is counting and waits for everything at every use of a
+// loaded value.  The hardware counter still counts these stores; that only makes the compiler's waits for older
+// loads (which return in order among themselves) longer, never shorter.  Store data is read when the
+// instruction issues, so the registers can be reused right after.
+__device__ __forceinline__ void buffer_store_untracked(float v, unsigned voffset, bufrsrc rsrc, int soffset) {
+  asm volatile("buffer_store_dword %0, %1, %2, %3 offen" ::"v"(v), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+
+// Writes one wavefront's 32 channels x 32 pixels accumulator block of v_mfma_f32_32x32x2_f32 (register r of lane
+// l holds channel 8(r/4) + 4(l/32) + r%4 of pixel l%32):  out = alpha*acc (+ beta*out) (+ bias).
+//   rsrc     descriptor of the whole output tensor
+//   voffset  byte offset of this lane's pixel in channel 4(l/32) of the block's image (kOutside: lane writes nothing)
+//   sblock   byte offset of the block's first channel plane (uniform)
+//   plane    bytes per channel plane (uniform)
+//   biasBlk  bias of the block's first channel, or null (uniform)
+// Straight-line: 16 stores at "lane offset + scalar offset", no per-store address arithmetic in vector registers,
+// no per-store branches.
+template <bool BETA, bool BIAS>
+__device__ __forceinline__ void store_block_as(floatx16 acc, bufrsrc rsrc, unsigned voffset, int sblock, int plane,
+                                               float alpha, float beta, const float* biasBlk, int kh) {
+  float old[16], bv[16];
+  if (BETA) {
+    const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(((unsigned long long)(unsigned)rsrc.x) | ((unsigned long long)(unsigned)rsrc.y << 32)), 0, rsrc.z, rsrc.w);
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      old[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rr, (int)voffset, sblock + (8 * (r / 4) + r % 4) * plane, 0));
+  }
+  if (BIAS) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) bv[r] = biasBlk[8 * (r / 4) + 4 * kh + r % 4];
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float v = alpha * acc[r];
+    if (BETA) v = fmaf(beta, old[r], v);
+    if (BIAS) v += bv[r];
+    buffer_store_untracked(v, voffset, rsrc, sblock + (8 * (r / 4) + r % 4) * plane);
+  }
+}
+
+__device__ __forceinline__ void store_block(floatx16 acc, bufrsrc rsrc, unsigned voffset, int sblock, int plane,
+                                            float alpha, float beta, const float* biasBlk, int kh) {
+  if (beta != 0.f) {
+    if (biasBlk) store_block_as<true, true>(acc, rsrc, voffset, sblock, plane, alpha, beta, biasBlk, kh);
+    else store_block_as<true, false>(acc, rsrc, voffset, sblock, plane, alpha, beta, biasBlk, kh);
+  } else if (biasBlk) {
+    store_block_as<false, true>(acc, rsrc, voffset, sblock, plane, alpha, beta, biasBlk, kh);
+  } else {
+    store_block_as<false, false>(acc, rsrc, voffset, sblock, plane, alpha, beta, biasBlk, kh);
+  }
+}
 
 // Weights-stationary variant (conv_ws.hip) for filter banks that fit in LDS: wt is the packed bank in tap-major
 // order (R = ci + Cin*t).  Sets *handled when it took the work.

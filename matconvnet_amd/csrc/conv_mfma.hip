@@ -29,7 +29,6 @@
 namespace mcn {
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kMaxTaps = 128;
 
@@ -249,6 +248,25 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   }
 
   // ---- epilogue: lane = pixel, register = channel
+  const int waU = __builtin_amdgcn_readfirstlane(wa);  // a wavefront's tile position is uniform
+  const int coW = co0 + waU * WA * 32;
+  if (p.outBytes != 0 && coW + WA * 32 <= p.Cout) {
+    // whole channel blocks inside the tensor: straight-line stores through a buffer descriptor
+    const bufrsrc rsrc = make_bufrsrc(out, p.outBytes);
+    const int plane = Q * 4;
+#pragma unroll
+    for (int jj = 0; jj < WB; ++jj) {
+      const int mo = m0 + wb * WB * 32 + jj * 32 + l32;
+      int n, q;
+      p.byQ.divmod(mo < p.M ? mo : 0, &n, &q);
+      const unsigned vo = mo < p.M ? (unsigned)(n * p.Cout * Q + q + 4 * kh * Q) * 4u : kOutside;
+#pragma unroll
+      for (int ii = 0; ii < WA; ++ii)
+        store_block(acc[ii][jj], rsrc, vo, (coW + ii * 32) * plane, plane, p.alpha, p.beta,
+                    bias ? bias + coW + ii * 32 : nullptr, kh);
+    }
+    return;
+  }
 #pragma unroll
   for (int jj = 0; jj < WB; ++jj) {
     const int mo = m0 + wb * WB * 32 + jj * 32 + l32;
@@ -617,6 +635,10 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   }
   if (rc) return rc;
   if (((long long)p.M / 64 + 1) * (p.coutPad / 32) >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
+  {
+    const long long ob = (long long)p.OH * p.OW * p.Cout * p.N * 4;
+    p.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
+  }
   p.byQ = FastDiv(p.OH * p.OW);
   p.byOH = FastDiv(p.OH);
   p.byT = FastDiv(p.T);

@@ -13,8 +13,11 @@
 //   * those loads are buffer loads: the per-lane offset is the pixel (+ tap shift), the scalar offset is the
 //     channel, and a lane whose shifted pixel falls outside the image simply uses an offset beyond the tensor,
 //     for which the hardware returns 0 -- no masks, no selects, no branches, no out-of-bounds access possible;
-//   * three register buffers of 8 reduction pairs rotate, so two groups of loads are in flight behind the one
-//     being multiplied, and the first loads of a wave's next unit are issued before the stores of the finished one;
+//   * four register buffers of 8 reduction pairs rotate, so three groups of loads are in flight behind the one
+//     being multiplied, and the stream of loads runs on from one unit of a wavefront into its next without
+//     draining (the per-unit address arithmetic is done beside the stores of the unit before);
+//   * a finished unit is written by 16 straight-line buffer stores per 32 channels ("lane offset + scalar
+//     offset"), invisible to the compiler's wait bookkeeping so that they do not drain the load stream;
 //   * the loop carries about one vector-ALU instruction per 8 MFMAs (vector-ALU work is what competes with the
 //     matrix pipe for the SIMD: with 5 per MFMA an earlier form of this kernel reached only half the MFMA rate);
 //   * units are dealt so that every SIMD of the chip gets the same number of them to within one, and the channel
@@ -28,11 +31,8 @@
 namespace mcn {
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
 constexpr int kDepth = 8;       // reduction pairs per group: Cin must be a multiple of 16 so a group stays inside a tap
 constexpr int kMaxTapsWs = 128;
-constexpr unsigned kOutside = 0x80000000u;  // buffer offset no tensor reaches (tensors here are < 2 GiB): reads as 0
 
 struct WsP {
   int nUnits;        // pixel blocks x channel blocks
@@ -42,16 +42,6 @@ struct WsP {
   unsigned inBytes;  // size of the gathered tensor
   FastDiv byCB, byRow;  // byRow: 8 WA = 16-byte vectors per bank row of one channel block
 };
-
-// A store the compiler's memory-wait bookkeeping does not see.  With ordinary stores in flight beside loads it
-// can no longer tell which of them the hardware counter is counting and waits for everything at every use of a
-// loaded value, which would drain the load pipeline at every MFMA of the next unit.  The hardware counter still
-// counts these stores; that only makes the compiler's waits for older loads (which return in order among
-// themselves) longer, never shorter.  Store data is read when the instruction issues, so the accumulators can be
-// cleared right after.
-__device__ __forceinline__ void store_untracked(float* ptr, float v) {
-  asm volatile("global_store_dword %0, %1, off" ::"v"(ptr), "v"(v) : "memory");
-}
 
 template <int WA, bool TAPS, int THREADS>
 __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out, const float* __restrict__ in,
@@ -74,12 +64,23 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   {
     const int perBlock = p.R * (ROW / 4);  // 16-byte vectors per channel block
     const int n4 = perBlock * w.chanBlocks;
-    for (int i = tid; i < n4; i += THREADS) {
-      const int cbk = i / perBlock;  // (one-time code: a plain division)
-      const int rem = i - cbk * perBlock;
-      int r, v;
-      w.byRow.divmod(rem, &r, &v);
-      ((float4*)wtL)[i] = *(const float4*)(wt + (size_t)r * p.coutPad + cbk * ROW + v * 4);
+    // (four vectors in flight per thread: one at a time, every round trip to L2 would be paid in full; the empty
+    // asm keeps the compiler from sinking each load into the branch that guards its store)
+    for (int i0 = tid; i0 < n4; i0 += 4 * THREADS) {
+      v4f v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int i = min(i0 + k * THREADS, n4 - 1);
+        const int cbk = i / perBlock;  // (one-time code: a plain division)
+        const int rem = i - cbk * perBlock;
+        int r, c4;
+        w.byRow.divmod(rem, &r, &c4);
+        v[k] = *(const v4f*)(wt + (size_t)r * p.coutPad + cbk * ROW + c4 * 4);
+      }
+      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
     }
     if (TAPS && tid < p.T) {
       const int j = tid / p.FH, i = tid - j * p.FH;
@@ -103,22 +104,27 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, (int)w.inBytes, 0x00020000);
   const int planeBytes = IHW * 4;
 
-  // per-unit, per-lane state
-  unsigned voff;   // byte offset of this lane's pixel and reduction half at tap shift 0 (kOutside for idle lanes)
-  int ihB, iwB;    // gathered coordinates at tap shift 0
-  int cb;          // channel block of the unit
+  // ---- the loader: a stream of groups (16 reduction rows x 32 pixels) that runs three groups ahead of the MFMAs
+  // and passes from one unit of this wavefront to the next without draining.  Its state:
+  unsigned voff;     // byte offset of this lane's pixel and reduction half at tap shift 0 (kOutside: idle lane)
+  int ihB, iwB;      // gathered coordinates at tap shift 0
+  unsigned voffN;    // the same three for the unit after the one being loaded: worked out beside the stores of a
+  int ihBN, iwBN;    // finished unit, so that the loop itself carries no address arithmetic
+  int tapL = 0, giL = 0;  // tap and 16-channel chunk inside the tap of the next group
+  unsigned voTap;    // per-lane offset of that tap's pixels (a register of its own for the whole tap: recomputed
+                     // per group, the register allocator handed its register to a load result, and every group
+                     // then waited for all loads in flight before it could form the next offset)
 
-  auto setup = [&](int u) {
-    int pb;
-    w.byCB.divmod(u, &pb, &cb);
-    const int m = pb * 32 + l32;
-    const bool mvalid = m < p.M;
+  // lane geometry of unit u (the pixels do not depend on the channel block); past the last unit every lane idles
+  auto setup_next = [&](int u) {
+    const int m = w.byCB.div(u) * 32 + l32;
+    const bool mvalid = u < w.nUnits && m < p.M;
     int n, q, ow, oh;
     p.byQ.divmod(mvalid ? m : 0, &n, &q);
     p.byOH.divmod(q, &ow, &oh);
-    ihB = oh * p.sy;
-    iwB = ow * p.sx;
-    voff = mvalid ? (unsigned)(n * (p.Cin * IHW) + ihB + p.IH * iwB + kh * IHW) * 4u : kOutside;
+    ihBN = oh * p.sy;
+    iwBN = ow * p.sx;
+    voffN = mvalid ? (unsigned)(n * (p.Cin * IHW) + ihBN + p.IH * iwBN + kh * IHW) * 4u : kOutside;
   };
 
   // per-lane offset of the pixels of tap `tap` (kOutside where the shifted pixel is not in the image)
@@ -132,83 +138,96 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   };
 
   typedef float vbuf __attribute__((ext_vector_type(kDepth)));
-  vbuf b0, b1, b2;
-  // the loader's position in the current unit: next group, its tap, its 16-channel chunk inside the tap, and the
-  // per-lane offset of that tap's pixels (kept in a register of its own for the whole tap: recomputing it per
-  // group let the register allocator hand its register to a load result, and every group then waited for all
-  // loads in flight before it could form the next offset)
-  int gLoad, tapL, giL;
-  unsigned voTap;
+  vbuf b0, b1, b2, b3;
 
-  // Loads the loader's next group into DST and advances it.  Past the last group the loads still go out, with
-  // the "outside" offset (they fetch nothing and return 0): the instruction stream stays the same on every path,
-  // which lets the compiler count exactly how many younger loads may stay in flight at each MFMA.
+  // Loads the stream's next group into DST and advances the loader.  Past this wavefront's last unit the loads
+  // still go out, with the "outside" offset (they fetch nothing and return 0): the instruction stream is the same
+  // on every path, which lets the compiler count exactly how many younger loads may stay in flight at each MFMA.
 #define WS_LOAD_NEXT(DST)                                                                                 \
   do {                                                                                                    \
     const int sbase_ = giL * (2 * kDepth) * planeBytes;                                                   \
     _Pragma("unroll") for (int d_ = 0; d_ < kDepth; ++d_) DST[d_] = __builtin_bit_cast(                   \
         float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voTap, sbase_ + 2 * d_ * planeBytes, 0));  \
-    ++gLoad;                                                                                              \
     if (++giL == w.groupsPerTap) {                                                                        \
       giL = 0;                                                                                            \
-      ++tapL;                                                                                             \
-      voTap = gLoad < w.groups ? tap_offset(TAPS ? min(tapL, p.T - 1) : 0) : kOutside;                    \
+      if (++tapL == p.T) {                                                                                \
+        tapL = 0;                                                                                         \
+        voff = voffN;                                                                                     \
+        ihB = ihBN;                                                                                       \
+        iwB = iwBN;                                                                                       \
+      }                                                                                                   \
+      voTap = tap_offset(tapL);                                                                           \
     }                                                                                                     \
   } while (0)
 
-#define WS_PRIME()             \
-  do {                         \
-    gLoad = 0;                 \
-    tapL = 0;                  \
-    giL = 0;                   \
-    voTap = tap_offset(0);     \
-    WS_LOAD_NEXT(b0);          \
-    WS_LOAD_NEXT(b1);          \
-  } while (0)
-
-  // multiply group G (operands CUR) after putting the loader's next group (G + 2) in flight into FREE
+  // multiplies the stream's oldest group (operands CUR, group G of the unit in hand) after putting one more
+  // group in flight into FREE
 #define WS_STEP(G, CUR, FREE)                                                                                     \
-  if ((G) < w.groups) {                                                                                          \
-    WS_LOAD_NEXT(FREE);                                                                                          \
-    const float* aG_ = aLane + (G) * (2 * kDepth * ROW);                                                         \
-    constexpr int HALF_ = kDepth / 2;                                                                            \
-    _Pragma("unroll") for (int h_ = 0; h_ < 2; ++h_) {                                                           \
-      float av_[HALF_][WA];                                                                                      \
-      _Pragma("unroll") for (int d_ = 0; d_ < HALF_; ++d_)                                                       \
+  {                                                                                                               \
+    WS_LOAD_NEXT(FREE);                                                                                           \
+    const float* aG_ = aG + (G) * (2 * kDepth * ROW);                                                             \
+    constexpr int HALF_ = kDepth / 2;                                                                             \
+    _Pragma("unroll") for (int h_ = 0; h_ < 2; ++h_) {                                                            \
+      float av_[HALF_][WA];                                                                                       \
+      _Pragma("unroll") for (int d_ = 0; d_ < HALF_; ++d_)                                                        \
         _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_) av_[d_][a_] = aG_[(2 * (h_ * HALF_ + d_)) * ROW + a_ * 32]; \
-      _Pragma("unroll") for (int d_ = 0; d_ < HALF_; ++d_)                                                       \
-        _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_)                                                        \
-          acc[a_] = __builtin_amdgcn_mfma_f32_32x32x2f32(av_[d_][a_], CUR[h_ * HALF_ + d_], acc[a_], 0, 0, 0);   \
-    }                                                                                                            \
+      _Pragma("unroll") for (int d_ = 0; d_ < HALF_; ++d_)                                                        \
+        _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_)                                                         \
+          acc[a_] = __builtin_amdgcn_mfma_f32_32x32x2f32(av_[d_][a_], CUR[h_ * HALF_ + d_], acc[a_], 0, 0, 0);    \
+    }                                                                                                             \
+    /* Pins the step's MFMAs before the next step's loads.  Left free, the compiler lifts those loads over the */ \
+    /* last MFMA, which still reads a register of the buffer they fill; the load then gets a fresh register    */ \
+    /* and the loop copies it back at its end, after waiting for every load in flight.                         */ \
+    _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_) asm volatile("" : "+v"(acc[a_])::"memory");                 \
   }
 
-  setup(unit);
-  WS_PRIME();
+  setup_next(unit);
+  voff = voffN;
+  ihB = ihBN;
+  iwB = iwBN;
+  setup_next(unit + unitStep);
+  voTap = tap_offset(0);
+  WS_LOAD_NEXT(b0);
+  WS_LOAD_NEXT(b1);
+  WS_LOAD_NEXT(b2);
 
+  const bufrsrc orsrc = make_bufrsrc(out, p.outBytes);
+  const int plane = Q * 4;
+
+  floatx16 acc[WA];
+#pragma unroll
+  for (int a = 0; a < WA; ++a)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
+  int pb, cb;
+  w.byCB.divmod(unit, &pb, &cb);  // unit = pixel block * chanBlocks + channel block
+  const float* aLane = wtL + (size_t)cb * p.R * ROW + kh * ROW + l32;
+  const float* aG = aLane;  // weight rows of the group in hand
+
+  // One flat loop over this wavefront's whole stream, four groups per turn (the host admits only reductions of
+  // a multiple of 4 groups, so a unit ends at the end of a turn with the four buffers back in place).
+  const int quadsPerUnit = w.groups >> 2;
+  int quadsLeft = quadsPerUnit;
   while (true) {
-    floatx16 acc[WA];
-#pragma unroll
-    for (int a = 0; a < WA; ++a)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
+    WS_STEP(0, b0, b3)
+    WS_STEP(1, b1, b0)
+    WS_STEP(2, b2, b1)
+    WS_STEP(3, b3, b2)
+    aG += 4 * (2 * kDepth * ROW);
+    if (--quadsLeft != 0) continue;
 
-    const float* aLane = wtL + (size_t)cb * p.R * ROW + kh * ROW + l32;
-    for (int g0 = 0; g0 < w.groups; g0 += 3) {
-      WS_STEP(g0, b0, b2)
-      WS_STEP(g0 + 1, b1, b0)
-      WS_STEP(g0 + 2, b2, b1)
-    }
-
-    // ---- the finished unit's geometry, then the next unit's first loads, then the stores
-    const int doneCb = cb;
-    const int mo = w.byCB.div(unit) * 32 + l32;  // unit = pixel block * chanBlocks + channel block
-    const int next = unit + unitStep;
-    const bool more = next < w.nUnits;
-    if (more) {
-      setup(next);
-      WS_PRIME();
-    }
-    if (mo < p.M) {
+    // ---- stores of the finished unit (the next unit's first three groups are already in flight)
+    const int mo = pb * 32 + l32;
+    if (p.outBytes != 0 && (cb + 1) * ROW <= p.Cout) {
+      // whole channel blocks inside the tensor: straight-line stores through a buffer descriptor
+      int n, q;
+      p.byQ.divmod(mo < p.M ? mo : 0, &n, &q);
+      const unsigned vo = mo < p.M ? (unsigned)(n * p.Cout * Q + q + 4 * kh * Q) * 4u : kOutside;
+#pragma unroll
+      for (int a = 0; a < WA; ++a)
+        store_block(acc[a], orsrc, vo, (cb * ROW + a * 32) * plane, plane, p.alpha, p.beta,
+                    bias ? bias + cb * ROW + a * 32 : nullptr, kh);
+    } else if (mo < p.M) {
       int n, q;
       p.byQ.divmod(mo, &n, &q);
       float* o = out + (size_t)n * p.Cout * Q + q;
@@ -216,20 +235,28 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
       for (int a = 0; a < WA; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int co = doneCb * ROW + a * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
+          const int co = cb * ROW + a * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
           if (co < p.Cout) {
             float v = p.alpha * acc[a][r];
             if (p.beta != 0.f) v = fmaf(p.beta, o[(size_t)co * Q], v);
             if (bias) v += bias[co];
-            store_untracked(o + (size_t)co * Q, v);
+            o[(size_t)co * Q] = v;
           }
         }
     }
-    if (!more) break;
-    unit = next;
+    unit += unitStep;
+    if (unit >= w.nUnits) break;
+    setup_next(unit + unitStep);  // (the loader is already inside `unit`)
+#pragma unroll
+    for (int a = 0; a < WA; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
+    w.byCB.divmod(unit, &pb, &cb);
+    aLane = wtL + (size_t)cb * p.R * ROW + kh * ROW + l32;
+    aG = aLane;
+    quadsLeft = quadsPerUnit;
   }
 #undef WS_STEP
-#undef WS_PRIME
 #undef WS_LOAD_NEXT
 }
 
@@ -269,7 +296,7 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
                    const PixP& p, int* handled) {
   *handled = 0;
   if (tunable("conv_no_ws", 0)) return MCN_SUCCESS;
-  if (p.Cin % (2 * kDepth) != 0 || p.T > kMaxTapsWs || p.coutPad % 32 != 0) return MCN_SUCCESS;
+  if (p.Cin % (2 * kDepth) != 0 || p.R % (8 * kDepth) != 0 || p.T > kMaxTapsWs || p.coutPad % 32 != 0) return MCN_SUCCESS;
   const size_t lds = (size_t)p.R * p.coutPad * sizeof(float) + (size_t)p.T * sizeof(int2);
   if (lds > 150 * 1024) return MCN_SUCCESS;
   // byte offsets into the gathered tensor must stay below the "outside" offset
@@ -285,11 +312,7 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
   // channels per wavefront: the widest unit that still spreads evenly over the SIMDs (wider units amortise the
   // pixel loads over more MFMAs; narrower ones balance better)
   const int minUnits = tunable("conv_ws_min_units", 0);
-  // Measured on the 56x56 bottleneck shapes: with a short reduction (64 channels, one tap) a unit is 32 MFMAs
-  // between a prologue and 16 stores, and the tiled kernel's wider tiles win; from 128 rows up this kernel does.
-  if (minUnits <= 0 && p.R < 128) return MCN_SUCCESS;
   int WA = tunable("conv_ws_wa", 0);
-  if (WA != 1 && WA != 2 && WA != 4 && p.T > 1 && p.coutPad % 64 == 0 && p.coutPad < 128) WA = 2;  // measured best for 3x3, 64 channels
   if (WA != 1 && WA != 2 && WA != 4) {
     double best = 0;
     for (int cand : {4, 2, 1}) {
@@ -308,7 +331,7 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
   w.chanBlocks = p.coutPad / (32 * WA);
   const long long units = pixelBlocks * w.chanBlocks;
   // too little work to keep every SIMD busy: leave it to the tiled kernel
-  if (units >= (1ll << 31) || units < (minUnits > 0 ? (long long)minUnits : simds * 2)) return MCN_SUCCESS;
+  if (units >= (1ll << 30) || units < (minUnits > 0 ? (long long)minUnits : simds * 2)) return MCN_SUCCESS;
   w.nUnits = (int)units;
   w.groups = p.R / (2 * kDepth);
   w.groupsPerTap = p.Cin / (2 * kDepth);

@@ -189,14 +189,16 @@ def test_errors(capi):
         capi.conv_out_shape(capi.conv_geom((8, 8, 4, 1), (3, 3, 2, 3)))  # 2 groups do not divide 3 filters
 
 
-WS_CASES = [  # (xshape, fshape, stride, pad, dilate): channel counts a multiple of 16, bank small enough for LDS
-    ((20, 18, 32, 3), (1, 1, 32, 64), 1, 0, 1),
+WS_CASES = [  # (xshape, fshape, stride, pad, dilate): reduction rows a multiple of 64, bank small enough for LDS
+    ((20, 18, 64, 3), (1, 1, 64, 64), 1, 0, 1),
     ((20, 18, 64, 2), (1, 1, 64, 40), 1, 0, 1),          # output channels not a multiple of 32
-    ((13, 11, 16, 5), (3, 3, 16, 32), 1, 1, 1),          # pixels not a multiple of 32
-    ((17, 15, 32, 2), (3, 3, 32, 48), 1, (2, 0, 1, 3), 1),
-    ((19, 19, 16, 2), (3, 2, 16, 96), (2, 3), 1, 1),     # strided: forward only on this path
-    ((21, 20, 16, 2), (3, 3, 16, 32), 1, 2, 2),          # dilated
-    ((12, 12, 48, 4), (5, 5, 48, 16), 1, 2, 1),
+    ((13, 11, 64, 5), (3, 3, 64, 32), 1, 1, 1),          # pixels not a multiple of 32
+    ((17, 15, 64, 2), (3, 3, 64, 64), 1, (2, 0, 1, 3), 1),
+    ((19, 19, 64, 2), (3, 2, 64, 96), (2, 3), 1, 1),     # strided: forward only on this path
+    ((21, 20, 64, 2), (3, 3, 64, 64), 1, 2, 2),          # dilated
+    ((12, 12, 64, 4), (2, 2, 64, 16), 1, (1, 0, 0, 1), 1),
+    ((10, 9, 64, 3), (1, 1, 64, 128), 1, 0, 1),          # wide enough for the 128-channel units
+    ((56, 56, 64, 3), (1, 1, 64, 64), 1, 0, 1),          # several units per wavefront: the load stream crosses units
 ]
 
 
@@ -226,15 +228,43 @@ def test_weights_stationary_kernel(capi, ob, xs, fs, stride, pad, dilate, wa):
     strided = np.any(np.atleast_1d(stride) != 1)
 
     def eligible(cin, cout):
-        """The kernel's own admission rule: reduction channels a multiple of 16, the packed bank (padded to the
-        channel tile) within 150 KB of LDS, the padded channel count a whole number of units."""
+        """The kernel's own admission rule: reduction channels a multiple of 16 and rows a multiple of 64, the
+        packed bank (padded to the channel tile) within 150 KB of LDS, the padded channel count a whole number
+        of units."""
         taps = fs[0] * fs[1]
         tile = 128 if cout > 64 else (64 if cout > 32 else 32)
         padded = -(-cout // tile) * tile
-        return (cin % 16 == 0 and taps * cin * padded * 4 + taps * 8 <= 150 * 1024 and
+        return (cin % 16 == 0 and (taps * cin) % 64 == 0 and taps * cin * padded * 4 + taps * 8 <= 150 * 1024 and
                 (wa == 0 or padded % (32 * wa) == 0))
 
     expected = int(eligible(xs[2], fs[3])) + int(eligible(fs[3], xs[2]) and not strided)
     assert launches == expected  # the kernel under test really ran
     assert rel_max(capi.to_host(y), want) < 2e-4
     assert rel_max(capi.to_host(dx), ob.conv_backward(x, f, dy, g, want=(True, False, False))[0]) < 2e-4
+
+
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_fast_epilogue_out_mult(capi, ob, with_bias, tiled):
+    """y = outMult*y + inMult*conv (+ bias) through the straight-line store path of both MFMA kernels."""
+    r = np.random.default_rng(11 + with_bias)
+    xs, fs = (20, 18, 64, 3), (3, 3, 64, 64)
+    x = F(r.standard_normal(xs))
+    f = F(r.standard_normal(fs) * 0.2)
+    b = r.standard_normal(fs[3]).astype(np.float32) if with_bias else None
+    g = ob.conv_geom(xs, fs, 1, 1, 1)
+    cg = capi.conv_geom(xs, fs, 1, 1, 1)
+    base = F(r.standard_normal(capi.conv_out_shape(cg)))
+    capi.set_tunable("conv_ws_min_units", 1)
+    capi.set_tunable("conv_no_ws", int(tiled))
+    try:
+        capi.profile_begin("conv_ws_mfma")
+        y = capi.conv_forward(capi.to_device(x), capi.to_device(f), None if b is None else capi.to_device(b), cg,
+                              y=capi.to_device(base), out_mult=0.5, in_mult=2.0)
+        launches, _ = capi.profile_end()
+    finally:
+        capi.set_tunable("conv_ws_min_units", 0)
+        capi.set_tunable("conv_no_ws", 0)
+    assert launches == (0 if tiled else 1)
+    want = ob.conv_forward(x, f, b, g, y=base.copy(order="F"), out_mult=0.5, in_mult=2.0)
+    assert rel_max(capi.to_host(y), want) < 2e-4
