@@ -32,7 +32,7 @@ PEAK_HBM = 8.0e12          # B/s
 # read for a 256 MiB streaming copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per unit).  Counters are not
 # readable from inside this process, so these are the profiled values of exactly these launches.
 TRAFFIC = {
-    "block/conv_pix_mfma": 1.039e8,    # mean of the 6 launches of a step (profiles/bottleneck_block_56x56_N32_fwd_bwd.txt)
+    "block/conv_ws_mfma": None,        # mean of the 6 launches of a step (profiles/bottleneck_block_56x56_N32_fwd_bwd.txt)
     "cfg5/conv_pix_mfma": 2.319e9,     # profiles/conv_vgg_3x3x256x256_N64_backward.txt (operands 2.08e8: tiles re-read through L2)
     "cfg5/conv_wgrad_mfma": 9.08e8,
     "cfg2/bnorm_sums": 2.058e8,        # profiles/bnorm_56x56x256x32_backward.txt
@@ -72,10 +72,11 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
     dt = time.perf_counter() - t0
     # which kernel family dominates the step, and its live duration
     P = 56 * 56
-    conv_flops = {  # per launch family per step: forward + backward-data launches of conv_pix_mfma
-        "conv_pix_mfma": 2.0 * (2.0 * P * N * (256 * 64 + 9 * 64 * 64 + 64 * 256)),
-        "conv_wgrad_mfma": 2.0 * P * N * (256 * 64 + 9 * 64 * 64 + 64 * 256),
-    }
+    # per launch family per step.  The six forward + backward-data launches go to the weights-stationary kernel
+    # (conv_ws_mfma) when the bank fits in LDS, else to the tiled one (conv_pix_mfma); if a step ever mixes them,
+    # they are reported as one family.
+    pix_flops = 2.0 * (2.0 * P * N * (256 * 64 + 9 * 64 * 64 + 64 * 256))
+    conv_flops = {"conv_wgrad_mfma": 2.0 * P * N * (256 * 64 + 9 * 64 * 64 + 64 * 256)}
     eS, eB = 4.0 * P * 64 * N, 4.0 * P * 256 * N
     hbm_bytes = {  # algorithmic bytes per step of the memory-bound families (reads + writes once each)
         "bnorm_sums": (eS + eS + eB) + 2 * (eS + eS + eB),       # forward reads x; backward reads x and dzdy
@@ -84,12 +85,16 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
         "eltwise_kernel": 3 * eB + 3 * eS + 3 * eS + 3 * eB,      # three ReLU derivatives, one fan-out sum
     }
     fam = {}
-    for name in list(conv_flops) + list(hbm_bytes) + ["conv_wgrad_reduce", "conv_pack_weights"]:
+    for name in ["conv_ws_mfma", "conv_pix_mfma"] + list(conv_flops) + list(hbm_bytes) + ["conv_wgrad_reduce", "conv_pack_weights"]:
         capi.profile_begin(name)
         blk.run(steps)
         n, ms = capi.profile_end()
         fam[name] = (n, ms * 1e-3)
     blk.close()
+    ws, pix = fam.pop("conv_ws_mfma"), fam.pop("conv_pix_mfma")
+    pix_name = "conv_ws_mfma" if pix[0] == 0 else ("conv_pix_mfma" if ws[0] == 0 else "conv_ws_mfma+conv_pix_mfma")
+    fam[pix_name] = (ws[0] + pix[0], ws[1] + pix[1])
+    conv_flops[pix_name] = pix_flops
     top = max(fam, key=lambda k: fam[k][1])
     n, total = fam[top]
     if top in conv_flops:

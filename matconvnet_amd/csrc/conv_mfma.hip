@@ -303,6 +303,7 @@ struct WgP {
   int chunkSpan;         // pixels per split (multiple of 32)
   int splits;
   FastDiv byQ, byOH, byT, byFH, byTiles, byTilesK, byC;
+  unsigned outBytes;     // size of the partial banks, or 0 when they do not fit a 2 GiB buffer descriptor
 };
 
 // UT ("uniform tap"): rows are ordered tap-major (R' = c + C*t) and C is a multiple of 32, so each 32-row MFMA
@@ -506,6 +507,23 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   }
 
   // ---- epilogue: lane = filter-volume row R (contiguous in dF), register = filter k
+  const int waU = __builtin_amdgcn_readfirstlane(wa);  // a wavefront's tile position is uniform
+  const int kW = k0 + waU * WA * 32;
+  if (p.outBytes != 0 && kW + WA * 32 <= p.K) {
+    // whole filter blocks present: straight-line stores through a buffer descriptor
+    const bufrsrc rsrc = make_bufrsrc(out, p.outBytes);
+    const int plane = p.FV * 4;
+    const int sbase = __builtin_amdgcn_readfirstlane(split) * p.K * plane;
+#pragma unroll
+    for (int jj = 0; jj < WB; ++jj) {
+      const int R = r0 + wb * WB * 32 + jj * 32 + l32;
+      const unsigned vo = R < p.FV ? (unsigned)(R + 4 * kh * p.FV) * 4u : kOutside;
+#pragma unroll
+      for (int ii = 0; ii < WA; ++ii)
+        store_block(acc[ii][jj], rsrc, vo, sbase + (kW + ii * 32) * plane, plane, 1.f, 0.f, nullptr, kh);
+    }
+    return;
+  }
   float* o = out + (size_t)split * p.FV * p.K;
 #pragma unroll
   for (int jj = 0; jj < WB; ++jj) {
@@ -573,8 +591,14 @@ bool wgrad_uniform_tap(const ConvP& p) {
          (long long)p.outH * p.outW * p.K * p.N < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
 }
 
+// filter-volume rows per workgroup of the filter-gradient kernel: 128, or 64 when the whole volume fits in 64
+// rows (a 1x1 layer with 64 input channels) and the filter tile leaves room for that shape
+int pick_rows_tile(const ConvP& p) {
+  return (p.FH * p.FW * p.FC <= 64 && pick_channels_tile(p.K) >= 64) ? 64 : 128;
+}
+
 int wgrad_splits(const ConvP& p, int* tilesOut) {
-  const int BA = pick_channels_tile(p.K), BB = 128;
+  const int BA = pick_channels_tile(p.K), BB = pick_rows_tile(p);
   const int tiles = ((p.K + BA - 1) / BA) * ((p.FH * p.FW * p.FC + BB - 1) / BB);
   int target = tunable("conv_wgrad_blocks", 0);
   if (target <= 0) target = 512;
@@ -768,16 +792,21 @@ int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const fl
       return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: workspace too small (%zu < %zu bytes)", wsBytes, need);
     target = (float*)ws;
   }
+  {
+    const unsigned long long ob = (unsigned long long)q.splits * nF * sizeof(float);
+    q.outBytes = ob < (1ull << 31) ? (unsigned)ob : 0u;
+  }
   const dim3 grid((unsigned)(tiles * q.splits)), block(256);
   const int BA = pick_channels_tile(p.K);
   int rc;
+  const bool narrow = pick_rows_tile(p) == 64;
   if (ut) {
-    if (BA == 128) rc = launch_wgrad<2, 2, 2, 2, true>(s, grid, target, x, dy, q);
-    else if (BA == 64) rc = launch_wgrad<2, 1, 1, 4, true>(s, grid, target, x, dy, q);
+    if (BA == 128) rc = narrow ? launch_wgrad<2, 1, 2, 2, true>(s, grid, target, x, dy, q) : launch_wgrad<2, 2, 2, 2, true>(s, grid, target, x, dy, q);
+    else if (BA == 64) rc = narrow ? launch_wgrad<1, 1, 2, 2, true>(s, grid, target, x, dy, q) : launch_wgrad<2, 1, 1, 4, true>(s, grid, target, x, dy, q);
     else rc = launch_wgrad<1, 1, 1, 4, true>(s, grid, target, x, dy, q);
   } else {
-    if (BA == 128) rc = launch_wgrad<2, 2, 2, 2, false>(s, grid, target, x, dy, q);
-    else if (BA == 64) rc = launch_wgrad<2, 1, 1, 4, false>(s, grid, target, x, dy, q);
+    if (BA == 128) rc = narrow ? launch_wgrad<2, 1, 2, 2, false>(s, grid, target, x, dy, q) : launch_wgrad<2, 2, 2, 2, false>(s, grid, target, x, dy, q);
+    else if (BA == 64) rc = narrow ? launch_wgrad<1, 1, 2, 2, false>(s, grid, target, x, dy, q) : launch_wgrad<2, 1, 1, 4, false>(s, grid, target, x, dy, q);
     else rc = launch_wgrad<1, 1, 1, 4, false>(s, grid, target, x, dy, q);
   }
   if (!rc) rc = check_launch("mcn_conv_backward_filter");
