@@ -119,6 +119,15 @@ MCN_API int mcn_conv_backward_data(mcn_stream_t stream, const mcn_conv_geom* g, 
                                    const float* filters, const float* derOutput, void* workspace,
                                    size_t workspaceBytes);
 
+/* dzdx accumulated: derInput = derInputMult*derInput + dzdx (derInputMult = 0: same as mcn_conv_backward_data,
+   previous contents ignored).  The reference has no such call: where a variable feeds several layers its
+   derivatives are added by the network wrapper afterwards (matlab/+dagnn/Layer.m:130-132,
+   "net.vars(v).der = net.vars(v).der + derInputs{i}"); this folds that addition into the convolution's output
+   pass. */
+MCN_API int mcn_conv_backward_data_acc(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput,
+                                       float derInputMult, const float* filters, const float* derOutput,
+                                       void* workspace, size_t workspaceBytes);
+
 /* dzdf: FH x FW x FC x K, fully overwritten  (bits/nnconv.cu:280-311: im2row::forward + gemm 't','n'
    accumulated over images) */
 MCN_API int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters,

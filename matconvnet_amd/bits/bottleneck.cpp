@@ -141,15 +141,21 @@ ErrorCode Bottleneck::backward() {
   char const* mask3 = fused ? "y" : "s";
   char const* mask2 = fused ? "r2" : "n2";
   char const* mask1 = fused ? "r1" : "n1";
-  ABI("relu3_bwd", mcn_relu_backward(st, buffer("ds"), buffer(mask3), buffer("dzdy"), nBig));
-  // the sum passes ds to both of its inputs: the branch (n3) and the shortcut (x)
-  STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot("ds")));
+  // the sum passes ds to both of its inputs: the branch (n3) and the shortcut (x).  Fused mode keeps ds in the
+  // output buffer and lets the first convolution add its derivative to it.
+  char const* dsName = fused ? "dzdx" : "ds";
+  ABI("relu3_bwd", mcn_relu_backward(st, buffer(dsName), buffer(mask3), buffer("dzdy"), nBig));
+  STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot(dsName)));
   STEP("conv3_bwd", c1.backward(slot("dr2"), slot("df3"), none, slot("r2"), slot("f3"), slot("da3")));
   ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer(mask2), buffer("dr2"), nSmall));
   STEP("bn2_bwd", bn.backwardWithMoment(slot("da2"), slot("dg2"), slot("db2"), slot("m2"), slot("a2"), slot("g2"), slot("b2"), slot("dn2")));
   STEP("conv2_bwd", c2.backward(slot("dr1"), slot("df2"), none, slot("r1"), slot("f2"), slot("da2")));
   ABI("relu1_bwd", mcn_relu_backward(st, buffer("dn1"), buffer(mask1), buffer("dr1"), nSmall));
   STEP("bn1_bwd", bn.backwardWithMoment(slot("da1"), slot("dg1"), slot("db1"), slot("m1"), slot("a1"), slot("g1"), slot("b1"), slot("dn1")));
+  if (fused) {
+    STEP("conv1_bwd", c1.backwardAccumulate(slot("dzdx"), 1, slot("df1"), none, slot("x"), slot("f1"), slot("da1")));
+    return VLE_Success;
+  }
   STEP("conv1_bwd", c1.backward(slot("dxm"), slot("df1"), none, slot("x"), slot("f1"), slot("da1")));
   ABI("sum_bwd", mcn_add(st, buffer("dzdx"), buffer("dxm"), buffer("ds"), nBig));
   return VLE_Success;

@@ -64,6 +64,11 @@ ErrorCode Convolution::forward(Tensor& output, double outputMult, Tensor const& 
 
 ErrorCode Convolution::backward(Tensor& derInput, Tensor& derFilter, Tensor& derBias, Tensor const& input,
                                 Tensor const& filter, Tensor const& derOutput) {
+  return backwardAccumulate(derInput, 0, derFilter, derBias, input, filter, derOutput);
+}
+
+ErrorCode Convolution::backwardAccumulate(Tensor& derInput, double derInputMult, Tensor& derFilter, Tensor& derBias,
+                                          Tensor const& input, Tensor const& filter, Tensor const& derOutput) {
   tensor_type tt = findTensorType(derInput, derFilter, derBias, input, filter, derOutput);
   ErrorCode e = requireHipFloat(context, tt, "Convolution::backward");
   if (e != VLE_Success) return e;
@@ -95,8 +100,8 @@ ErrorCode Convolution::backward(Tensor& derInput, Tensor& derFilter, Tensor& der
         derOutput.getSize() != derInput.getSize())
       return context.setError(VLE_IllegalArgument, "Convolution::backward: DEROUTPUT dimensions are incompatible with X and FILTERS");
     if (!scratch(context, g, MCN_CONV_BACKWARD_DATA, &ws, &bytes)) return context.getLastError();
-    rc = mcn_conv_backward_data(stream, &g, (float*)derInput.getMemory(), (float const*)filter.getMemory(),
-                                (float const*)derOutput.getMemory(), ws, bytes);
+    rc = mcn_conv_backward_data_acc(stream, &g, (float*)derInput.getMemory(), (float)derInputMult,
+                                    (float const*)filter.getMemory(), (float const*)derOutput.getMemory(), ws, bytes);
     if (rc) return fromAbi(context, rc, "Convolution::backward");
   }
 

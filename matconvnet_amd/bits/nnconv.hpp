@@ -20,6 +20,12 @@ class Convolution {
   vl::ErrorCode backward(vl::Tensor& derInput, vl::Tensor& derFilter, vl::Tensor& derBias, vl::Tensor const& input,
                          vl::Tensor const& filter, vl::Tensor const& derOutput);
 
+  // The same with derInput = derInputMult*derInput + dzdx: the sum a network wrapper makes where a variable
+  // feeds several layers (matlab/+dagnn/Layer.m:130-132), folded into the convolution's output pass.  Not part
+  // of the reference's class.
+  vl::ErrorCode backwardAccumulate(vl::Tensor& derInput, double derInputMult, vl::Tensor& derFilter, vl::Tensor& derBias,
+                                   vl::Tensor const& input, vl::Tensor const& filter, vl::Tensor const& derOutput);
+
   Context& context;
   int strideY;
   int strideX;

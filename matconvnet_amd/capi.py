@@ -50,6 +50,7 @@ PROTOTYPES = {
     "mcn_conv_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _i]),
     "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
+    "mcn_conv_backward_data_acc": (_i, [_vp, C.POINTER(ConvGeom), _vp, C.c_float, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_filter": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_bias": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _sz]),
     "mcn_subsample_output_size": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.POINTER(_i), C.POINTER(_i)]),
@@ -242,6 +243,15 @@ def conv_backward(x, f, dy, g, want=(True, True, True), ws=None):
         wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_BIAS))
         check(L.mcn_conv_backward_bias(stream(), C.byref(g), ptr(db), ptr(dy), wp, wn))
     return dx, df, db
+
+
+def conv_backward_data_acc(dx, mult, f, dy, g, ws=None):
+    """dx = mult*dx + dzdx, in place (include/mcn_hip.h: mcn_conv_backward_data_acc)."""
+    ws = ws or _ws
+    L = lib()
+    wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_DATA))
+    check(L.mcn_conv_backward_data_acc(stream(), C.byref(g), ptr(dx), float(mult), ptr(f), ptr(dy), wp, wn))
+    return dx
 
 
 def _hwcn(t):

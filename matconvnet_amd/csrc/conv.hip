@@ -126,16 +126,21 @@ int mcn_conv_forward(mcn_stream_t stream, const mcn_conv_geom* g, float* y, floa
   return conv_forward_direct(as_stream(stream), p, y, outMult, x, inMult, filters, bias);
 }
 
-int mcn_conv_backward_data(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, const float* filters,
-                           const float* derOutput, void* workspace, size_t workspaceBytes) {
+int mcn_conv_backward_data_acc(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, float derInputMult,
+                               const float* filters, const float* derOutput, void* workspace, size_t workspaceBytes) {
   ConvP p;
   int rc = conv_setup(g, "mcn_conv_backward_data", &p);
   if (rc) return rc;
   if ((size_t)p.H * p.W * p.C * p.N == 0) return MCN_SUCCESS;
   if (!derInput || !filters || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data: null tensor");
   if (!tunable("conv_force_direct", 0) && conv_mfma_backward_data_supported(p))
-    return conv_backward_data_mfma(as_stream(stream), p, derInput, filters, derOutput, workspace, workspaceBytes);
-  return conv_backward_data_direct(as_stream(stream), p, derInput, filters, derOutput);
+    return conv_backward_data_mfma(as_stream(stream), p, derInput, derInputMult, filters, derOutput, workspace, workspaceBytes);
+  return conv_backward_data_direct(as_stream(stream), p, derInput, derInputMult, filters, derOutput);
+}
+
+int mcn_conv_backward_data(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, const float* filters,
+                           const float* derOutput, void* workspace, size_t workspaceBytes) {
+  return mcn_conv_backward_data_acc(stream, g, derInput, 0.f, filters, derOutput, workspace, workspaceBytes);
 }
 
 int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters, const float* x,

@@ -19,7 +19,7 @@ int conv_setup(const mcn_conv_geom* g, const char* who, ConvP* p);
 // direct (one accumulator per output element) kernels: any stride / dilation / padding / groups
 int conv_forward_direct(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
                         const float* f, const float* b);
-int conv_backward_data_direct(hipStream_t s, const ConvP& p, float* dx, const float* f, const float* dy);
+int conv_backward_data_direct(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy);
 int conv_backward_filter_direct(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy);
 
 // MFMA implicit-GEMM kernels (groups == 1).  *_supported says whether the fast path covers `p`.
@@ -29,8 +29,8 @@ bool conv_mfma_backward_filter_supported(const ConvP& p);
 size_t conv_mfma_workspace_bytes(const ConvP& p, int product);
 int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
                       const float* f, const float* b, void* ws, size_t wsBytes);
-int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, const float* f, const float* dy, void* ws,
-                            size_t wsBytes);
+int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
+                            void* ws, size_t wsBytes);
 int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,
                               size_t wsBytes);
 

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void conv_fwd_direct(float* __restrict__ y, fl
   y[idx] = r0;
 }
 
-__global__ __launch_bounds__(256) void conv_bwd_data_direct(float* __restrict__ dx,
+__global__ __launch_bounds__(256) void conv_bwd_data_direct(float* __restrict__ dx, float dxMult,
                                                             const float* __restrict__ f,
                                                             const float* __restrict__ dy, ConvP p,
                                                             size_t total) {
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void conv_bwd_data_direct(float* __restrict__ 
       }
     }
   }
-  dx[idx] = acc;
+  dx[idx] = dxMult != 0.f ? fmaf(dxMult, dx[idx], acc) : acc;
 }
 
 // one workgroup per filter element
@@ -127,11 +127,11 @@ int conv_forward_direct(hipStream_t s, const ConvP& p, float* y, float outMult, 
   return check_launch("conv forward (direct)");
 }
 
-int conv_backward_data_direct(hipStream_t s, const ConvP& p, float* dx, const float* f, const float* dy) {
+int conv_backward_data_direct(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy) {
   const size_t total = (size_t)p.H * p.W * p.C * p.N;
   const size_t blocks = (total + 255) / 256;
   if (blocks >= (1ull << 31)) return fail(MCN_UNSUPPORTED, "conv backward-data: tensor too large");
-  hipLaunchKernelGGL(conv_bwd_data_direct, dim3((unsigned)blocks), dim3(256), 0, s, dx, f, dy, p, total);
+  hipLaunchKernelGGL(conv_bwd_data_direct, dim3((unsigned)blocks), dim3(256), 0, s, dx, dxMult, f, dy, p, total);
   return check_launch("conv backward-data (direct)");
 }
 

@@ -744,8 +744,8 @@ int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, co
   return run_pix(s, "mcn_conv_forward", y, x, f, b, q, 0, ws, wsBytes);
 }
 
-int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, const float* f, const float* dy, void* ws,
-                            size_t wsBytes) {
+int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
+                            void* ws, size_t wsBytes) {
   PixP q;
   q.IH = p.outH; q.IW = p.outW; q.Cin = p.K;
   q.OH = p.H; q.OW = p.W; q.Cout = p.C;
@@ -756,7 +756,7 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, const floa
   q.R = q.T * q.Cin;
   q.coutPad = 0;
   q.M = p.H * p.W * p.N;
-  q.alpha = 1.f; q.beta = 0.f;
+  q.alpha = 1.f; q.beta = dxMult;
   return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, 1, ws, wsBytes);
 }
 

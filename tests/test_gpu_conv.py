@@ -268,3 +268,29 @@ def test_fast_epilogue_out_mult(capi, ob, with_bias, tiled):
     assert launches == (0 if tiled else 1)
     want = ob.conv_forward(x, f, b, g, y=base.copy(order="F"), out_mult=0.5, in_mult=2.0)
     assert rel_max(capi.to_host(y), want) < 2e-4
+
+
+@pytest.mark.parametrize("path", ["ws", "tiled", "direct"])
+def test_backward_data_accumulate(capi, ob, path):
+    """derInput = mult*derInput + dzdx through each kernel family (and mult = 0 ignores what was there)."""
+    r = np.random.default_rng(23)
+    xs, fs = (20, 18, 64, 3), (3, 3, 64, 64)
+    x = F(r.standard_normal(xs))
+    f = F(r.standard_normal(fs) * 0.2)
+    g = ob.conv_geom(xs, fs, 1, 1, 1)
+    cg = capi.conv_geom(xs, fs, 1, 1, 1)
+    dy = F(r.standard_normal(capi.conv_out_shape(cg)))
+    base = F(r.standard_normal(xs))
+    want = ob.conv_backward(x, f, dy, g, want=(True, False, False))[0]
+    capi.set_tunable("conv_ws_min_units", 1)
+    capi.set_tunable("conv_no_ws", int(path != "ws"))
+    capi.set_tunable("conv_force_direct", int(path == "direct"))
+    try:
+        got = capi.to_host(capi.conv_backward_data_acc(capi.to_device(base), 0.75, capi.to_device(f), capi.to_device(dy), cg))
+        poisoned = capi.empty(xs, fill=float("nan"))
+        plain = capi.to_host(capi.conv_backward_data_acc(poisoned, 0.0, capi.to_device(f), capi.to_device(dy), cg))
+    finally:
+        for k in ("conv_ws_min_units", "conv_no_ws", "conv_force_direct"):
+            capi.set_tunable(k, 0)
+    assert rel_max(got, 0.75 * base + want) < 2e-4
+    assert rel_max(plain, want) < 2e-4
