@@ -186,6 +186,18 @@ MCN_API int mcn_bnorm_forward_fused(mcn_stream_t stream, float* y, float* moment
                                     int relu, int H, int W, int C, int N, double epsilon, int givenMoments,
                                     void* workspace, size_t workspaceBytes);
 
+/* The derivative of "batch normalisation, then ReLU" in one go: derOutput is dz/d(ReLU output), and it counts only
+   where the layer's own output g*(x - mean)/sigma + b was positive, which is recomputed from x and the moments the
+   forward pass stored (mcn_bnorm_forward* normalise with exactly those stored values, so the sign comes out the
+   same bit for bit).  Otherwise as mcn_bnorm_backward with givenMoments != 0; results are bit-identical to
+   mcn_relu_backward on the forward output followed by mcn_bnorm_backward, without writing and re-reading the
+   masked derivative.  No counterpart in the reference, which runs these layers one by one
+   (matlab/vl_nnrelu.m, bits/nnbnorm.cu:263-305). */
+MCN_API int mcn_bnorm_backward_relu(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
+                                    const float* moments, const float* x, const float* multipliers,
+                                    const float* biases, const float* derOutput, int H, int W, int C, int N,
+                                    double epsilon, void* workspace, size_t workspaceBytes);
+
 /* dzdx (H x W x C x N), dzdg (C), dzdb (C), all fully overwritten.  givenMoments == 0: BatchNorm::backward
    (bits/nnbnorm.cu:307-365), moments written if non-NULL.  givenMoments != 0: backwardWithMoment (:263-305). */
 MCN_API int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers,

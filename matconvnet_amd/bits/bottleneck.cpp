@@ -147,11 +147,29 @@ ErrorCode Bottleneck::backward() {
   ABI("relu3_bwd", mcn_relu_backward(st, buffer(dsName), buffer(mask3), buffer("dzdy"), nBig));
   STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot(dsName)));
   STEP("conv3_bwd", c1.backward(slot("dr2"), slot("df3"), none, slot("r2"), slot("f3"), slot("da3")));
-  ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer(mask2), buffer("dr2"), nSmall));
-  STEP("bn2_bwd", bn.backwardWithMoment(slot("da2"), slot("dg2"), slot("db2"), slot("m2"), slot("a2"), slot("g2"), slot("b2"), slot("dn2")));
+  const size_t wsSmall = mcn_bnorm_workspace_bytes(H, W, M, N);
+  void* wsBn = NULL;
+  if (fused) {
+    // ReLU's derivative folded into the batch-norm derivative that follows it: the mask is recomputed from the
+    // layer's input and stored moments, the masked derivative is never written out
+    wsBn = context.getWorkspace(VLDT_GPU, wsSmall);
+    if (!wsBn) return fail(context.getLastError(), "workspace");
+    ABI("bn2_bwd", mcn_bnorm_backward_relu(st, buffer("da2"), buffer("dg2"), buffer("db2"), buffer("m2"), buffer("a2"),
+                                           buffer("g2"), buffer("b2"), buffer("dr2"), H, W, M, N, epsilon, wsBn, wsSmall));
+  } else {
+    ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer(mask2), buffer("dr2"), nSmall));
+    STEP("bn2_bwd", bn.backwardWithMoment(slot("da2"), slot("dg2"), slot("db2"), slot("m2"), slot("a2"), slot("g2"), slot("b2"), slot("dn2")));
+  }
   STEP("conv2_bwd", c2.backward(slot("dr1"), slot("df2"), none, slot("r1"), slot("f2"), slot("da2")));
-  ABI("relu1_bwd", mcn_relu_backward(st, buffer("dn1"), buffer(mask1), buffer("dr1"), nSmall));
-  STEP("bn1_bwd", bn.backwardWithMoment(slot("da1"), slot("dg1"), slot("db1"), slot("m1"), slot("a1"), slot("g1"), slot("b1"), slot("dn1")));
+  if (fused) {
+    wsBn = context.getWorkspace(VLDT_GPU, wsSmall);  // (the convolution in between may have grown the workspace)
+    if (!wsBn) return fail(context.getLastError(), "workspace");
+    ABI("bn1_bwd", mcn_bnorm_backward_relu(st, buffer("da1"), buffer("dg1"), buffer("db1"), buffer("m1"), buffer("a1"),
+                                           buffer("g1"), buffer("b1"), buffer("dr1"), H, W, M, N, epsilon, wsBn, wsSmall));
+  } else {
+    ABI("relu1_bwd", mcn_relu_backward(st, buffer("dn1"), buffer(mask1), buffer("dr1"), nSmall));
+    STEP("bn1_bwd", bn.backwardWithMoment(slot("da1"), slot("dg1"), slot("db1"), slot("m1"), slot("a1"), slot("g1"), slot("b1"), slot("dn1")));
+  }
   if (fused) {
     STEP("conv1_bwd", c1.backwardAccumulate(slot("dzdx"), 1, slot("df1"), none, slot("x"), slot("f1"), slot("da1")));
     return VLE_Success;

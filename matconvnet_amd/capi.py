@@ -61,6 +61,7 @@ PROTOTYPES = {
     "mcn_bnorm_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_bnorm_forward_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_bnorm_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
+    "mcn_bnorm_backward_relu": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _vp, _sz]),
     "mcn_pool_output_size": (_i, [C.POINTER(PoolGeom), C.POINTER(_i), C.POINTER(_i)]),
     "mcn_pool_forward": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp]),
     "mcn_pool_backward": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp, _vp, _i]),
@@ -293,6 +294,19 @@ def bnorm_backward(x, g, dy, eps=1e-4, moments=None, ws=None, want_moments=True)
     check(lib().mcn_bnorm_backward(stream(), ptr(dx), ptr(dg), ptr(db), ptr(mom), ptr(x), ptr(g), ptr(dy),
                                    H, W, Cc, N, eps, int(given), wp, wn))
     return dx, dg, db, mom
+
+
+def bnorm_backward_relu(x, g, b, dy, moments, eps=1e-4, ws=None):
+    """Derivative of ReLU(bnorm(x)) given dz/d(ReLU output) and the forward pass's moments."""
+    ws = ws or _ws
+    H, W, Cc, N = _hwcn(x)
+    dx = empty((H, W, Cc, N))
+    dg = empty((Cc,))
+    db = empty((Cc,))
+    wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
+    check(lib().mcn_bnorm_backward_relu(stream(), ptr(dx), ptr(dg), ptr(db), ptr(moments), ptr(x), ptr(g), ptr(b),
+                                        ptr(dy), H, W, Cc, N, eps, wp, wn))
+    return dx, dg, db
 
 
 def pool_forward(x, g):

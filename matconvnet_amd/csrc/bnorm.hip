@@ -36,6 +36,15 @@ __device__ __forceinline__ void image_range(const BnormP& p, int grp, int* n0, i
   *n1 = (int)(((long long)p.N * (grp + 1)) / p.groups);
 }
 
+// y = a*x + k with the rounding of the forward pass: the moments as stored (float), everything else in double,
+// the two coefficients rounded to float once.  Forward and the ReLU-masked backward both go through here, so
+// that "a*x + k > 0" decides the same way in both.
+__device__ __forceinline__ void forward_coefficients(double mean, double sigma, float mult, float bias, float* a, float* k) {
+  const double coef = (double)mult / sigma;
+  *a = (float)coef;
+  *k = (float)((double)bias - coef * mean);
+}
+
 // Block-wide sum of NV doubles held per thread; result valid in thread 0.
 template <int NV>
 __device__ __forceinline__ void block_sum(double (&v)[NV], double* lds /* [4][NV] */) {
@@ -56,16 +65,25 @@ __device__ __forceinline__ void block_sum(double (&v)[NV], double* lds /* [4][NV
 // MODE 0: sum x, sum x^2               (forward, moments from the batch)
 // MODE 1: sum x*dy, sum dy             (backward, moments given)
 // MODE 2: all four                     (backward, moments from the batch)
-template <int MODE, bool VEC4>
+// RELU (MODE 1 only): dy is the derivative after a ReLU that followed this layer; it counts only where the
+// layer's output a*x + k was positive (a, k: the forward pass's own coefficients, see forward_coefficients).
+template <int MODE, bool VEC4, bool RELU = false>
 __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
                                                   const float* __restrict__ dy,
-                                                  double* __restrict__ partials, BnormP p) {
+                                                  double* __restrict__ partials, BnormP p,
+                                                  const float* __restrict__ moments = nullptr,
+                                                  const float* __restrict__ mult = nullptr,
+                                                  const float* __restrict__ bias = nullptr) {
+  static_assert(!RELU || MODE == 1, "the ReLU mask needs the moments of the forward pass");
   __shared__ double lds[16];
   const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int c = logical / p.groups;
   const int grp = logical - c * p.groups;
   int n0, n1;
   image_range(p, grp, &n0, &n1);
+  float ra = 0.f, rk = 0.f;
+  if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &ra, &rk);
+  auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv, rk) > 0.f ? dv : 0.f) : dv; };
   double acc[4] = {0.0, 0.0, 0.0, 0.0};
   for (int n = n0; n < n1; ++n) {
     const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
@@ -80,7 +98,8 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
           sxx += (a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w);
         }
         if (MODE != 0) {
-          const float4 d = d4[i];
+          float4 d = d4[i];
+          if (RELU) d = make_float4(gate(a.x, d.x), gate(a.y, d.y), gate(a.z, d.z), gate(a.w, d.w));
           sxd += (a.x * d.x + a.y * d.y) + (a.z * d.z + a.w * d.w);
           sd += (d.x + d.y) + (d.z + d.w);
         }
@@ -93,7 +112,7 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
           sxx += a * a;
         }
         if (MODE != 0) {
-          const float d = dy[base + i];
+          const float d = gate(a, dy[base + i]);
           sxd += a * d;
           sd += d;
         }
@@ -140,10 +159,13 @@ __device__ __forceinline__ void channel_totals(const double* __restrict__ partia
 }
 
 // out = a*in1 + b*in2 + k over this workgroup's planes (in2 optional)
-template <bool TWO, bool VEC4>
+// RELU: in1 counts only where ra*in2 + rk > 0 (in1 = derivative after the ReLU, in2 = the layer's input)
+template <bool TWO, bool VEC4, bool RELU = false>
 __device__ __forceinline__ void stream_planes(float* __restrict__ out, const float* __restrict__ in1,
                                               const float* __restrict__ in2, float a, float b, float k,
-                                              const BnormP& p, int c, int n0, int n1) {
+                                              const BnormP& p, int c, int n0, int n1, float ra = 0.f, float rk = 0.f) {
+  static_assert(!RELU || TWO, "the mask is computed from the second stream");
+  auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv, rk) > 0.f ? dv : 0.f) : dv; };
   for (int nn = n0; nn < n1; ++nn) {
     const int n = p.reverse ? (n1 - 1 - (nn - n0)) : nn;
     const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
@@ -156,10 +178,10 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
         float4 r;
         if (TWO) {
           const float4 v = stream_load4(s2 + i);
-          r.x = fmaf(a, u.x, fmaf(b, v.x, k));
-          r.y = fmaf(a, u.y, fmaf(b, v.y, k));
-          r.z = fmaf(a, u.z, fmaf(b, v.z, k));
-          r.w = fmaf(a, u.w, fmaf(b, v.w, k));
+          r.x = fmaf(a, gate(v.x, u.x), fmaf(b, v.x, k));
+          r.y = fmaf(a, gate(v.y, u.y), fmaf(b, v.y, k));
+          r.z = fmaf(a, gate(v.z, u.z), fmaf(b, v.z, k));
+          r.w = fmaf(a, gate(v.w, u.w), fmaf(b, v.w, k));
         } else {
           r.x = fmaf(a, u.x, k);
           r.y = fmaf(a, u.y, k);
@@ -171,7 +193,7 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
     } else {
       for (int i = threadIdx.x; i < p.WH; i += 256) {
         const float u = in1[base + i];
-        out[base + i] = TWO ? fmaf(a, u, fmaf(b, in2[base + i], k)) : fmaf(a, u, k);
+        out[base + i] = TWO ? fmaf(a, gate(in2[base + i], u), fmaf(b, in2[base + i], k)) : fmaf(a, u, k);
       }
     }
   }
@@ -179,7 +201,7 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
 
 // Backward apply.  GIVEN: mean/sigma come from `moments` (input); otherwise from the partial sums and
 // `moments` (if non-null) is written.
-template <bool GIVEN, bool VEC4>
+template <bool GIVEN, bool VEC4, bool RELU = false>
 __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ dx,
                                                             float* __restrict__ dmult,
                                                             float* __restrict__ dbias,
@@ -188,7 +210,8 @@ __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ 
                                                             const float* __restrict__ mult,
                                                             const float* __restrict__ dy,
                                                             const double* __restrict__ partials,
-                                                            BnormP p) {
+                                                            BnormP p, const float* __restrict__ bias = nullptr) {
+  static_assert(!RELU || GIVEN, "the ReLU mask needs the moments of the forward pass");
   __shared__ double lds[4];
   int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   if (p.reverse) logical = (int)gridDim.x - 1 - logical;
@@ -222,7 +245,9 @@ __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ 
   // dzdx = G1*(dy - muz) - G2*(x - mean) = G1*dy + (-G2)*x + (G2*mean - G1*muz)
   int n0, n1;
   image_range(p, grp, &n0, &n1);
-  stream_planes<true, VEC4>(dx, dy, x, (float)G1, (float)(-G2), (float)(G2 * mean - G1 * muz), p, c, n0, n1);
+  float ra = 0.f, rk = 0.f;
+  if (RELU) forward_coefficients(mean, sigma, mult[c], bias[c], &ra, &rk);
+  stream_planes<true, VEC4, RELU>(dx, dy, x, (float)G1, (float)(-G2), (float)(G2 * mean - G1 * muz), p, c, n0, n1, ra, rk);
 }
 
 // out = act(a*in + k [+ res]) over this workgroup's planes: the forward apply with the element-wise layers
@@ -287,11 +312,16 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
       moments[c] = (float)mean;
       moments[c + p.C] = (float)sigma;
     }
+    // normalise with the moments as they are stored (like the reference, whose moments are of the data type):
+    // a later pass that is given them reproduces this one bit for bit
+    mean = (double)(float)mean;
+    sigma = (double)(float)sigma;
   }
-  const double coef = (double)mult[c] / sigma;
+  float a, k;
+  forward_coefficients(mean, sigma, mult[c], bias[c], &a, &k);
   int n0, n1;
   image_range(p, grp, &n0, &n1);
-  stream_forward<RES, RELU, VEC4>(y, x, residual, (float)coef, (float)((double)bias[c] - coef * mean), p, c, n0, n1);
+  stream_forward<RES, RELU, VEC4>(y, x, residual, a, k, p, c, n0, n1);
 }
 
 int image_groups(int WH, int N) {
@@ -380,6 +410,40 @@ int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float
                       void* workspace, size_t workspaceBytes) {
   return mcn_bnorm_forward_fused(stream, y, moments, x, multipliers, biases, NULL, 0, H, W, C, N, epsilon,
                                  givenMoments, workspace, workspaceBytes);
+}
+
+int mcn_bnorm_backward_relu(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
+                            const float* moments, const float* x, const float* multipliers, const float* biases,
+                            const float* derOutput, int H, int W, int C, int N, double epsilon, void* workspace,
+                            size_t workspaceBytes) {
+  BnormP p;
+  int rc = setup("mcn_bnorm_backward_relu", H, W, C, N, epsilon, &p);
+  if (rc) return rc;
+  if (C == 0) return MCN_SUCCESS;
+  if (!derMultipliers || !derBiases || !multipliers || !biases || !moments)
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_relu: null parameter tensor");
+  if ((size_t)p.WH * N == 0) {
+    if ((rc = mcn_fill(stream, derMultipliers, 0.f, (size_t)C))) return rc;
+    return mcn_fill(stream, derBiases, 0.f, (size_t)C);
+  }
+  if (!derInput || !x || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_relu: null tensor");
+  if (!workspace || workspaceBytes < mcn_bnorm_workspace_bytes(H, W, C, N))
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_relu: workspace too small");
+  hipStream_t s = as_stream(stream);
+  const bool vec = (p.WH % 4 == 0) && aligned16(derInput) && aligned16(x) && aligned16(derOutput);
+  const dim3 grid((unsigned)(C * p.groups)), block(256);
+  double* partials = (double*)workspace;
+  float* mom = const_cast<float*>(moments);  // (the kernels only write moments when they are not given)
+  {
+    KernelTimer timer("bnorm_sums", s);
+    if (vec) hipLaunchKernelGGL((bnorm_sums<1, true, true>), grid, block, 0, s, x, derOutput, partials, p, moments, multipliers, biases);
+    else hipLaunchKernelGGL((bnorm_sums<1, false, true>), grid, block, 0, s, x, derOutput, partials, p, moments, multipliers, biases);
+  }
+  if ((rc = check_launch("mcn_bnorm_backward_relu(sums)"))) return rc;
+  KernelTimer timer("bnorm_backward_apply", s);
+  if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, derOutput, partials, p, biases);
+  else hipLaunchKernelGGL((bnorm_backward_apply<true, false, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, derOutput, partials, p, biases);
+  return check_launch("mcn_bnorm_backward_relu");
 }
 
 int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases, float* moments,

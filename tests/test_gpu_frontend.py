@@ -288,3 +288,25 @@ def test_bnorm_forward_fused_matches_separate_calls(capi, ob):
     assert bits_equal(capi.to_host(got), capi.to_host(capi.relu_forward(y0)))
     got, _ = capi.bnorm_forward_fused(xd, gd, bd, residual=rd, eps=1e-4)
     assert bits_equal(capi.to_host(got), capi.to_host(capi.add(y0, rd)))
+
+
+def test_bnorm_backward_relu_matches_separate_calls(capi, ob):
+    """ReLU's derivative folded into batch-norm's: bit-identical to the two calls, and right against the oracle."""
+    w = workloads.bnorm_case(seed=9, H=14, W=18, C=8, N=5)
+    d = lambda a: F(a, np.float64) if a.ndim > 1 else a.astype(np.float64)
+    xd, gd, bd, dyd = (capi.to_device(w[k]) for k in ("x", "g", "b", "dy"))
+    r, mom = capi.bnorm_forward_fused(xd, gd, bd, relu=True, eps=1e-4)
+    masked = capi.relu_backward(r, dyd)
+    want = capi.bnorm_backward(xd, gd, masked, 1e-4, moments=mom)
+    got = capi.bnorm_backward_relu(xd, gd, bd, dyd, mom, 1e-4)
+    for a, b_ in zip(got, want[:3]):
+        assert bits_equal(capi.to_host(a), capi.to_host(b_))
+    # against the oracle in double: forward, mask, backward
+    y64, _ = ob.bnorm_forward(d(w["x"]), d(w["g"]), d(w["b"]), 1e-4)
+    dy64 = d(w["dy"]) * (y64 > 0)
+    odx, odg, odb, _ = ob.bnorm_backward(d(w["x"]), d(w["g"]), dy64, 1e-4)
+    # (an element whose pre-activation is within rounding of 0 may be masked differently in float and double)
+    flips = np.sum((capi.to_host(r) > 0) != (y64 > 0))
+    if flips == 0:
+        assert rel_max(capi.to_host(got[0]), odx) < 1e-5
+        assert rel_max(capi.to_host(got[1]).ravel(), odg) < 1e-5 and rel_max(capi.to_host(got[2]).ravel(), odb) < 1e-5
