@@ -48,8 +48,22 @@ struct PixP {
   float alpha, beta;
   FastDiv byQ, byOH, byT;  // Q = OH*OW; T = taps
   int advC, advT;          // 16 = advC*T + advT (reduction rows per step)
-  unsigned outBytes;       // size of the produced tensor, or 0 when it does not fit a 2 GiB buffer descriptor
+  unsigned outBytes;       // bytes from `out` to the end of the produced tensor, or 0 when >= 2 GiB (no buffer descriptor)
+  // Where things lie, in elements.  The gathered tensor: image n, channel ci at in + n*inImg + ci*IH*IW.  The produced
+  // tensor: pixel (oh, ow) of image n, channel co at out + n*outImg + co*outPlane + outOff + oh*outSH + ow*outSW.
+  // A plain layer has inImg = Cin*IH*IW, outImg = Cout*OH*OW, outPlane = OH*OW, outOff = 0, outSH = 1, outSW = OH
+  // (dense = 1: the pixel offset is the pixel index itself); a filter group sees a slice of the channels of a
+  // wider tensor, a stride class of a strided layer's backward-data product a sub-grid of the pixels.
+  int inImg, outImg, outPlane, outOff, outSH, outSW, dense;
 };
+
+// the pixel's element offset inside its channel plane of the produced tensor
+__device__ __forceinline__ int out_pixel_offset(const PixP& p, int q) {
+  if (p.dense) return q;
+  int ow, oh;
+  p.byOH.divmod(q, &ow, &oh);
+  return p.outOff + oh * p.outSH + ow * p.outSW;
+}
 
 // ------------------------------------------------------------------------------------------------
 // Epilogue shared by the pixel-major MFMA kernels

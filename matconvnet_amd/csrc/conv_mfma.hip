@@ -41,17 +41,29 @@ constexpr int kMaxTaps = 128;
 //   reduction row R = t + T*ci (channel-major) or, when tapMajor, R = ci + Cin*t
 //   forward:        ci = c, co = k : f[t + T*c + FV*k]
 //   backward-data:  ci = k, co = c : f[t + T*(c + C*k)]
+// Only the taps (i0 + a*iStep, j0 + b*jStep), a < nI, b < nJ, of the FH x FW filter take part (all of them for a
+// plain layer; one stride class for the backward-data product of a strided layer); T = nI*nJ, t = a + nI*b.
+struct TapSet {
+  int FH, FW;            // the filter as stored
+  int i0, iStep, nI;
+  int j0, jStep, nJ;
+};
+
 __global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt, const float* __restrict__ f,
-                                                         int T, int Cin, int Cout, int rPad, int coutPad,
+                                                         TapSet ts, int Cin, int Cout, int rPad, int coutPad,
                                                          int backward, int tapMajor) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (size_t)rPad * coutPad) return;
+  const int T = ts.nI * ts.nJ;
   const int r = (int)(idx / coutPad), co = (int)(idx - (size_t)r * coutPad);
   float v = 0.f;
   if (r < T * Cin && co < Cout) {
     const int ci = tapMajor ? r % Cin : r / T;
     const int t = tapMajor ? r / Cin : r % T;
-    v = backward ? f[(size_t)t + (size_t)T * (co + (size_t)Cout * ci)] : f[(size_t)t + (size_t)T * ci + (size_t)T * Cin * co];
+    const int b = t / ts.nI, a = t - b * ts.nI;
+    const size_t Tf = (size_t)ts.FH * ts.FW;
+    const size_t tf = (size_t)(ts.i0 + a * ts.iStep) + (size_t)ts.FH * (ts.j0 + b * ts.jStep);
+    v = backward ? f[tf + Tf * (co + (size_t)Cout * ci)] : f[tf + Tf * ci + Tf * Cin * co];
   }
   wt[idx] = v;
 }
@@ -90,7 +102,6 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   const int m0 = mt * BB;
 
   const int IHW = p.IH * p.IW;
-  const int Q = p.OH * p.OW;
 
   if (tid < p.T) {
     const int j = tid / p.FH, i = tid - j * p.FH;
@@ -110,7 +121,7 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
     p.byOH.divmod(q, &ow, &oh);
     ihB = oh * p.sy;
     iwB = ow * p.sx;
-    inN = in + (size_t)n * p.Cin * IHW + ihB + p.IH * iwB;
+    inN = in + (size_t)n * p.inImg + ihB + p.IH * iwB;
   }
   // first gathered row of this thread: R = pg*RPT -> (tap, channel); advanced by BK per step
   int ciS, tapS;
@@ -253,13 +264,13 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   if (p.outBytes != 0 && coW + WA * 32 <= p.Cout) {
     // whole channel blocks inside the tensor: straight-line stores through a buffer descriptor
     const bufrsrc rsrc = make_bufrsrc(out, p.outBytes);
-    const int plane = Q * 4;
+    const int plane = p.outPlane * 4;
 #pragma unroll
     for (int jj = 0; jj < WB; ++jj) {
       const int mo = m0 + wb * WB * 32 + jj * 32 + l32;
       int n, q;
       p.byQ.divmod(mo < p.M ? mo : 0, &n, &q);
-      const unsigned vo = mo < p.M ? (unsigned)(n * p.Cout * Q + q + 4 * kh * Q) * 4u : kOutside;
+      const unsigned vo = mo < p.M ? (unsigned)(n * p.outImg + out_pixel_offset(p, q) + 4 * kh * p.outPlane) * 4u : kOutside;
 #pragma unroll
       for (int ii = 0; ii < WA; ++ii)
         store_block(acc[ii][jj], rsrc, vo, (coW + ii * 32) * plane, plane, p.alpha, p.beta,
@@ -273,7 +284,7 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
     if (mo >= p.M) continue;
     int n, q;
     p.byQ.divmod(mo, &n, &q);
-    float* o = out + (size_t)n * p.Cout * Q + q;
+    float* o = out + (size_t)n * p.outImg + out_pixel_offset(p, q);
 #pragma unroll
     for (int ii = 0; ii < WA; ++ii)
 #pragma unroll
@@ -281,9 +292,9 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
         const int co = co0 + wa * WA * 32 + ii * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
         if (co < p.Cout) {
           float v = p.alpha * acc[ii][jj][r];
-          if (p.beta != 0.f) v = fmaf(p.beta, o[(size_t)co * Q], v);
+          if (p.beta != 0.f) v = fmaf(p.beta, o[(size_t)co * p.outPlane], v);
           if (bias) v += bias[co];
-          o[(size_t)co * Q] = v;
+          o[(size_t)co * p.outPlane] = v;
         }
       }
   }
@@ -639,7 +650,7 @@ int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const flo
 }
 
 int run_pix(hipStream_t s, const char* who, float* out, const float* in, const float* f, const float* bias, PixP p,
-            int backward, void* ws, size_t wsBytes) {
+            const TapSet& taps, int backward, void* ws, size_t wsBytes) {
   const int BA = pick_channels_tile(p.Cout);
   const int rPad = (p.R + 15) / 16 * 16;
   p.coutPad = (p.Cout + BA - 1) / BA * BA;
@@ -649,18 +660,19 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   float* wt = (float*)ws;
   const size_t nW = (size_t)rPad * p.coutPad;
   // uniform-tap variant: whole 16-row steps inside one tap, and 32-bit element offsets into the gathered tensor
-  const bool ut = p.Cin % 16 == 0 && (long long)p.IH * p.IW * p.Cin * p.N < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
+  const long long inSpan = (long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW;  // elements from `in` to the end
+  const bool ut = p.Cin % 16 == 0 && inSpan < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
   int rc;
   {
     KernelTimer timer("conv_pack_weights", s);
-    hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, wt, f, p.T, p.Cin, p.Cout,
+    hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, wt, f, taps, p.Cin, p.Cout,
                        rPad, p.coutPad, backward, ut ? 1 : 0);
     rc = check_launch(who);
   }
   if (rc) return rc;
   if (((long long)p.M / 64 + 1) * (p.coutPad / 32) >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
   {
-    const long long ob = (long long)p.OH * p.OW * p.Cout * p.N * 4;
+    const long long ob = ((long long)(p.N - 1) * p.outImg + (long long)p.Cout * p.outPlane) * 4;
     p.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
   }
   p.byQ = FastDiv(p.OH * p.OW);
@@ -702,7 +714,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
 }  // namespace
 
 bool conv_mfma_forward_supported(const ConvP& p) { return common_ok(p); }
-bool conv_mfma_backward_data_supported(const ConvP& p) { return common_ok(p) && p.sy == 1 && p.sx == 1; }
+bool conv_mfma_backward_data_supported(const ConvP& p) { return common_ok(p); }
 bool conv_mfma_backward_filter_supported(const ConvP& p) { return common_ok(p); }
 
 size_t conv_mfma_workspace_bytes(const ConvP& p, int product) {
@@ -728,6 +740,27 @@ size_t conv_mfma_workspace_bytes(const ConvP& p, int product) {
   }
 }
 
+namespace {
+
+TapSet all_taps(const ConvP& p) {
+  TapSet t;
+  t.FH = p.FH; t.FW = p.FW;
+  t.i0 = 0; t.iStep = 1; t.nI = p.FH;
+  t.j0 = 0; t.jStep = 1; t.nJ = p.FW;
+  return t;
+}
+
+void dense_layout(PixP* q) {
+  q->inImg = q->Cin * q->IH * q->IW;
+  q->outPlane = q->OH * q->OW;
+  q->outImg = q->Cout * q->outPlane;
+  q->outOff = 0; q->outSH = 1; q->outSW = q->OH; q->dense = 1;
+}
+
+int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
+
+}  // namespace
+
 int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
                       const float* f, const float* b, void* ws, size_t wsBytes) {
   PixP q;
@@ -741,23 +774,80 @@ int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, co
   q.coutPad = 0;
   q.M = p.outH * p.outW * p.N;
   q.alpha = inMult; q.beta = outMult;
-  return run_pix(s, "mcn_conv_forward", y, x, f, b, q, 0, ws, wsBytes);
+  dense_layout(&q);
+  return run_pix(s, "mcn_conv_forward", y, x, f, b, q, all_taps(p), 0, ws, wsBytes);
 }
 
+// dzdx[h, w] = sum over taps (i, j) with (h + pt - i*dy) and (w + pl - j*dx) divisible by the strides of
+//   dzdy[(h + pt - i*dy)/sy, (w + pl - j*dx)/sx] * f[i, j]
+// With unit stride that is one gather product over all taps.  With a stride the pixels split into sy*sx classes
+// (h mod sy, w mod sx); inside a class the taps that take part form an arithmetic progression and the gathered
+// position moves by one per pixel of the class, so each class is the same gather product over a sub-grid of dzdx
+// with a subset of the taps.  Classes no tap reaches (1x1 filters with stride 2: three of four) are zeros.
 int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
                             void* ws, size_t wsBytes) {
   PixP q;
   q.IH = p.outH; q.IW = p.outW; q.Cin = p.K;
-  q.OH = p.H; q.OW = p.W; q.Cout = p.C;
   q.N = p.N;
-  q.FH = p.FH; q.T = p.FH * p.FW;
+  q.Cout = p.C;
   q.sy = 1; q.sx = 1;
-  q.dhBase = p.pt; q.dhStep = -p.dy; q.dwBase = p.pl; q.dwStep = -p.dx;
-  q.R = q.T * q.Cin;
   q.coutPad = 0;
-  q.M = p.H * p.W * p.N;
   q.alpha = 1.f; q.beta = dxMult;
-  return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, 1, ws, wsBytes);
+  if (p.sy == 1 && p.sx == 1) {
+    q.OH = p.H; q.OW = p.W;
+    q.FH = p.FH; q.T = p.FH * p.FW;
+    q.dhBase = p.pt; q.dhStep = -p.dy; q.dwBase = p.pl; q.dwStep = -p.dx;
+    q.R = q.T * q.Cin;
+    q.M = p.H * p.W * p.N;
+    dense_layout(&q);
+    return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, all_taps(p), 1, ws, wsBytes);
+  }
+  // one class at a time; first the taps of every class, to know whether any class is empty
+  struct Axis { int first, step, count, dBase, dStep; };
+  auto axis = [](int phase, int pad, int dil, int stride, int taps) {
+    Axis a;
+    a.step = stride / gcd_int(dil, stride);
+    a.first = -1;
+    for (int i = 0; i < taps && i < a.step; ++i)
+      if ((phase + pad - i * dil) % stride == 0) { a.first = i; break; }
+    a.count = a.first < 0 ? 0 : (taps - a.first + a.step - 1) / a.step;
+    a.dBase = a.first < 0 ? 0 : (phase + pad - a.first * dil) / stride;  // exact: the numerator is a multiple of stride
+    a.dStep = -(a.step * dil) / stride;                                   // exact likewise
+    return a;
+  };
+  bool anyEmpty = false;
+  for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
+    for (int ph = 0; ph < p.sy && ph < p.H; ++ph)
+      if (axis(ph, p.pt, p.dy, p.sy, p.FH).count == 0 || axis(pw, p.pl, p.dx, p.sx, p.FW).count == 0) anyEmpty = true;
+  if (anyEmpty && dxMult == 0.f) {
+    int rc = mcn_fill((mcn_stream_t)s, dx, 0.f, (size_t)p.H * p.W * p.C * p.N);
+    if (rc) return rc;
+  } else if (anyEmpty && dxMult != 1.f) {
+    return fail(MCN_UNSUPPORTED, "mcn_conv_backward_data: accumulation with a multiplier other than 1 is not available for this stride");
+  }
+  for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
+    for (int ph = 0; ph < p.sy && ph < p.H; ++ph) {
+      const Axis ai = axis(ph, p.pt, p.dy, p.sy, p.FH), aj = axis(pw, p.pl, p.dx, p.sx, p.FW);
+      if (ai.count == 0 || aj.count == 0) continue;
+      PixP c = q;
+      c.OH = (p.H - ph + p.sy - 1) / p.sy;
+      c.OW = (p.W - pw + p.sx - 1) / p.sx;
+      c.FH = ai.count; c.T = ai.count * aj.count;
+      c.dhBase = ai.dBase; c.dhStep = ai.dStep; c.dwBase = aj.dBase; c.dwStep = aj.dStep;
+      c.R = c.T * c.Cin;
+      c.M = c.OH * c.OW * p.N;
+      c.inImg = c.Cin * c.IH * c.IW;
+      c.outPlane = p.H * p.W;
+      c.outImg = p.C * c.outPlane;
+      c.outOff = ph + p.H * pw; c.outSH = p.sy; c.outSW = p.H * p.sx; c.dense = 0;
+      TapSet t;
+      t.FH = p.FH; t.FW = p.FW;
+      t.i0 = ai.first; t.iStep = ai.step; t.nI = ai.count;
+      t.j0 = aj.first; t.jStep = aj.step; t.nJ = aj.count;
+      int rc = run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, c, t, 1, ws, wsBytes);
+      if (rc) return rc;
+    }
+  return MCN_SUCCESS;
 }
 
 int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,

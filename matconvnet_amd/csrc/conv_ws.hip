@@ -58,7 +58,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   // everything derived from it -- the unit, the loop bounds, the scalar load offsets -- lives in scalar registers)
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, kh = lane >> 5;
-  const int IHW = p.IH * p.IW, Q = p.OH * p.OW;
+  const int IHW = p.IH * p.IW;
 
   // ---- once per workgroup: the bank, re-laid by channel block, and the tap table
   {
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     p.byOH.divmod(q, &ow, &oh);
     ihBN = oh * p.sy;
     iwBN = ow * p.sx;
-    voffN = mvalid ? (unsigned)(n * (p.Cin * IHW) + ihBN + p.IH * iwBN + kh * IHW) * 4u : kOutside;
+    voffN = mvalid ? (unsigned)(n * p.inImg + ihBN + p.IH * iwBN + kh * IHW) * 4u : kOutside;
   };
 
   // per-lane offset of the pixels of tap `tap` (kOutside where the shifted pixel is not in the image)
@@ -192,7 +192,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   WS_LOAD_NEXT(b2);
 
   const bufrsrc orsrc = make_bufrsrc(out, p.outBytes);
-  const int plane = Q * 4;
+  const int plane = p.outPlane * 4;
 
   floatx16 acc[WA];
 #pragma unroll
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
       // whole channel blocks inside the tensor: straight-line stores through a buffer descriptor
       int n, q;
       p.byQ.divmod(mo < p.M ? mo : 0, &n, &q);
-      const unsigned vo = mo < p.M ? (unsigned)(n * p.Cout * Q + q + 4 * kh * Q) * 4u : kOutside;
+      const unsigned vo = mo < p.M ? (unsigned)(n * p.outImg + out_pixel_offset(p, q) + 4 * kh * p.outPlane) * 4u : kOutside;
 #pragma unroll
       for (int a = 0; a < WA; ++a)
         store_block(acc[a], orsrc, vo, (cb * ROW + a * 32) * plane, plane, p.alpha, p.beta,
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     } else if (mo < p.M) {
       int n, q;
       p.byQ.divmod(mo, &n, &q);
-      float* o = out + (size_t)n * p.Cout * Q + q;
+      float* o = out + (size_t)n * p.outImg + out_pixel_offset(p, q);
 #pragma unroll
       for (int a = 0; a < WA; ++a)
 #pragma unroll
@@ -238,9 +238,9 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
           const int co = cb * ROW + a * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
           if (co < p.Cout) {
             float v = p.alpha * acc[a][r];
-            if (p.beta != 0.f) v = fmaf(p.beta, o[(size_t)co * Q], v);
+            if (p.beta != 0.f) v = fmaf(p.beta, o[(size_t)co * p.outPlane], v);
             if (bias) v += bias[co];
-            o[(size_t)co * Q] = v;
+            o[(size_t)co * p.outPlane] = v;
           }
         }
     }
@@ -300,7 +300,7 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
   const size_t lds = (size_t)p.R * p.coutPad * sizeof(float) + (size_t)p.T * sizeof(int2);
   if (lds > 150 * 1024) return MCN_SUCCESS;
   // byte offsets into the gathered tensor must stay below the "outside" offset
-  const long long inBytes = (long long)p.IH * p.IW * p.Cin * p.N * 4;
+  const long long inBytes = ((long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW) * 4;
   if (inBytes >= (long long)kOutside) return MCN_SUCCESS;
 
   int cus = mcn_device_compute_units();

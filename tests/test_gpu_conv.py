@@ -194,7 +194,9 @@ WS_CASES = [  # (xshape, fshape, stride, pad, dilate): reduction rows a multiple
     ((20, 18, 64, 2), (1, 1, 64, 40), 1, 0, 1),          # output channels not a multiple of 32
     ((13, 11, 64, 5), (3, 3, 64, 32), 1, 1, 1),          # pixels not a multiple of 32
     ((17, 15, 64, 2), (3, 3, 64, 64), 1, (2, 0, 1, 3), 1),
-    ((19, 19, 64, 2), (3, 2, 64, 96), (2, 3), 1, 1),     # strided: forward only on this path
+    ((19, 19, 64, 2), (3, 2, 64, 96), (2, 3), 1, 1),     # strided: backward-data runs once per stride class
+    ((22, 21, 64, 2), (1, 1, 64, 64), 2, 0, 1),          # 1x1, stride 2: three of four classes are zeros
+    ((23, 20, 64, 2), (5, 3, 64, 64), (2, 2), (2, 1, 1, 0), (2, 1)),  # stride and dilation together
     ((21, 20, 64, 2), (3, 3, 64, 64), 1, 2, 2),          # dilated
     ((12, 12, 64, 4), (2, 2, 64, 16), 1, (1, 0, 0, 1), 1),
     ((10, 9, 64, 3), (1, 1, 64, 128), 1, 0, 1),          # wide enough for the 128-channel units
@@ -237,8 +239,12 @@ def test_weights_stationary_kernel(capi, ob, xs, fs, stride, pad, dilate, wa):
         return (cin % 16 == 0 and (taps * cin) % 64 == 0 and taps * cin * padded * 4 + taps * 8 <= 150 * 1024 and
                 (wa == 0 or padded % (32 * wa) == 0))
 
-    expected = int(eligible(xs[2], fs[3])) + int(eligible(fs[3], xs[2]) and not strided)
-    assert launches == expected  # the kernel under test really ran
+    # the kernel under test really ran (a strided layer's backward-data product is one launch per stride class
+    # whose tap subset is eligible, so only a lower bound is fixed there)
+    if strided:
+        assert launches >= int(eligible(xs[2], fs[3]))
+    else:
+        assert launches == int(eligible(xs[2], fs[3])) + int(eligible(fs[3], xs[2]))
     assert rel_max(capi.to_host(y), want) < 2e-4
     assert rel_max(capi.to_host(dx), ob.conv_backward(x, f, dy, g, want=(True, False, False))[0]) < 2e-4
 
