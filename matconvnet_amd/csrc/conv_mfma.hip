@@ -315,6 +315,7 @@ struct WgP {
   int splits;
   FastDiv byQ, byOH, byT, byFH, byTiles, byTilesK, byC;
   unsigned outBytes;     // size of the partial banks, or 0 when they do not fit a 2 GiB buffer descriptor
+  int xImg, dyImg;       // elements between images of x and of dzdy (wider than C*H*W, K*OH*OW for a filter group)
 };
 
 // UT ("uniform tap"): rows are ordered tap-major (R' = c + C*t) and C is a multiple of 32, so each 32-row MFMA
@@ -418,8 +419,8 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
     p.byOH.divmod(q, &ow, &oh);
     const int ihB = oh * p.sy, iwB = ow * p.sx;
     if (UT) {
-      const int pixX = n * (p.C * HW) + ihB + p.H * iwB;
-      const int pixY = n * (p.K * Q) + q;
+      const int pixX = n * p.xImg + ihB + p.H * iwB;
+      const int pixY = n * p.dyImg + q;
 #pragma unroll
       for (int jb = 0; jb < NBLK; ++jb) {
         const bool ok = valid && (unsigned)(ihB + blkDh[jb]) < (unsigned)p.H && (unsigned)(iwB + blkDw[jb]) < (unsigned)p.W;
@@ -442,8 +443,8 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
       okB = 0xffffffffu;
       return;
     }
-    const float* xN = x + (size_t)n * p.C * HW + ihB + p.H * iwB;
-    const float* dyN = dy + (size_t)n * p.K * Q + q;
+    const float* xN = x + (size_t)n * p.xImg + ihB + p.H * iwB;
+    const float* dyN = dy + (size_t)n * p.dyImg + q;
     int2 tp[BPT];
 #pragma unroll
     for (int e = 0; e < BPT; ++e) tp[e] = rowTab[rg + 8 * e];
@@ -592,13 +593,31 @@ int pick_channels_tile(int cout) { return cout > 64 ? 128 : (cout > 32 ? 64 : 32
 bool common_ok(const ConvP& p) {
   // tap offsets are packed as 16-bit fields and "row absent" is encoded as offset -32768
   const long long spanH = (long long)p.H + p.pt + (long long)p.FH * p.dy, spanW = (long long)p.W + p.pl + (long long)p.FW * p.dx;
-  return p.groups == 1 && p.FH * p.FW <= kMaxTaps && spanH < 32768 && spanW < 32768 &&
-         (long long)p.outH * p.outW * p.N < (1ll << 31) && (long long)p.H * p.W * p.N < (1ll << 31);
+  return p.FH * p.FW <= kMaxTaps && spanH < 32768 && spanW < 32768 &&
+         (long long)p.outH * p.outW * p.N < (1ll << 31) && (long long)p.H * p.W * p.N < (1ll << 31) &&
+         (long long)p.H * p.W * p.C < (1ll << 31) && (long long)p.outH * p.outW * p.K < (1ll << 31);
 }
 
+// One filter group of a layer as a layer of its own: FC input channels, K/groups filters.  Its tensors are slices
+// of the layer's (the image strides stay those of the whole layer: struct Wide).
+ConvP group_view(const ConvP& p) {
+  ConvP g = p;
+  g.C = p.FC;
+  g.K = p.Kg;
+  g.groups = 1;
+  return g;
+}
+
+struct Wide {
+  int xImg, yImg;  // elements between images of the layer's input and output tensors
+};
+
+Wide wide_of(const ConvP& p) { return Wide{p.C * p.H * p.W, p.K * p.outH * p.outW}; }
+
 // the tap-major variant of the filter-gradient kernel: 32-row blocks inside one tap, 32-bit element offsets
+// (takes the whole layer, not a group view: the offsets span the whole tensors)
 bool wgrad_uniform_tap(const ConvP& p) {
-  return p.C % 32 == 0 && (long long)p.H * p.W * p.C * p.N < (1ll << 31) &&
+  return p.FC % 32 == 0 && (long long)p.H * p.W * p.C * p.N < (1ll << 31) &&
          (long long)p.outH * p.outW * p.K * p.N < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
 }
 
@@ -717,24 +736,25 @@ bool conv_mfma_forward_supported(const ConvP& p) { return common_ok(p); }
 bool conv_mfma_backward_data_supported(const ConvP& p) { return common_ok(p); }
 bool conv_mfma_backward_filter_supported(const ConvP& p) { return common_ok(p); }
 
-size_t conv_mfma_workspace_bytes(const ConvP& p, int product) {
+size_t conv_mfma_workspace_bytes(const ConvP& layer, int product) {
+  const ConvP p = group_view(layer);  // the groups run one after the other through the same workspace
   const size_t FV = (size_t)p.FH * p.FW * p.FC;
   switch (product) {
     case MCN_CONV_FORWARD: {
-      if (!conv_mfma_forward_supported(p)) return 0;
+      if (!conv_mfma_forward_supported(layer)) return 0;
       const int BA = pick_channels_tile(p.K);
       return ((FV + 15) / 16 * 16) * (size_t)((p.K + BA - 1) / BA * BA) * sizeof(float);
     }
     case MCN_CONV_BACKWARD_DATA: {
-      if (!conv_mfma_backward_data_supported(p)) return 0;
+      if (!conv_mfma_backward_data_supported(layer)) return 0;
       const int BA = pick_channels_tile(p.C);
       const size_t R = (size_t)p.FH * p.FW * p.K;
       return ((R + 15) / 16 * 16) * (size_t)((p.C + BA - 1) / BA * BA) * sizeof(float);
     }
     case MCN_CONV_BACKWARD_FILTER: {
-      if (!conv_mfma_backward_filter_supported(p)) return 0;
+      if (!conv_mfma_backward_filter_supported(layer)) return 0;
       const int s = wgrad_splits(p, nullptr);
-      return (s > 1 || wgrad_uniform_tap(p)) ? (size_t)s * FV * p.K * sizeof(float) : 0;
+      return (s > 1 || wgrad_uniform_tap(layer)) ? (size_t)s * FV * p.K * sizeof(float) : 0;
     }
     default: return 0;
   }
@@ -761,8 +781,9 @@ int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
 
 }  // namespace
 
-int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
-                      const float* f, const float* b, void* ws, size_t wsBytes) {
+namespace {
+int forward_group(hipStream_t s, const ConvP& p, Wide wd, float* y, float outMult, const float* x, float inMult,
+                  const float* f, const float* b, void* ws, size_t wsBytes) {
   PixP q;
   q.IH = p.H; q.IW = p.W; q.Cin = p.C;
   q.OH = p.outH; q.OW = p.outW; q.Cout = p.K;
@@ -775,7 +796,23 @@ int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, co
   q.M = p.outH * p.outW * p.N;
   q.alpha = inMult; q.beta = outMult;
   dense_layout(&q);
+  q.inImg = wd.xImg;
+  q.outImg = wd.yImg;
   return run_pix(s, "mcn_conv_forward", y, x, f, b, q, all_taps(p), 0, ws, wsBytes);
+}
+}  // namespace
+
+int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
+                      const float* f, const float* b, void* ws, size_t wsBytes) {
+  const ConvP g = group_view(p);
+  const Wide wd = wide_of(p);
+  const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
+  for (int i = 0; i < p.groups; ++i) {
+    int rc = forward_group(s, g, wd, y + i * p.Kg * Q, outMult, x + i * p.FC * HW, inMult, f + i * p.Kg * FV,
+                           b ? b + i * p.Kg : nullptr, ws, wsBytes);
+    if (rc) return rc;
+  }
+  return MCN_SUCCESS;
 }
 
 // dzdx[h, w] = sum over taps (i, j) with (h + pt - i*dy) and (w + pl - j*dx) divisible by the strides of
@@ -784,8 +821,22 @@ int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, co
 // (h mod sy, w mod sx); inside a class the taps that take part form an arithmetic progression and the gathered
 // position moves by one per pixel of the class, so each class is the same gather product over a sub-grid of dzdx
 // with a subset of the taps.  Classes no tap reaches (1x1 filters with stride 2: three of four) are zeros.
-int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
-                            void* ws, size_t wsBytes) {
+namespace {
+struct Axis { int first, step, count, dBase, dStep; };
+Axis stride_axis(int phase, int pad, int dil, int stride, int taps) {
+  Axis a;
+  a.step = stride / gcd_int(dil, stride);
+  a.first = -1;
+  for (int i = 0; i < taps && i < a.step; ++i)
+    if ((phase + pad - i * dil) % stride == 0) { a.first = i; break; }
+  a.count = a.first < 0 ? 0 : (taps - a.first + a.step - 1) / a.step;
+  a.dBase = a.first < 0 ? 0 : (phase + pad - a.first * dil) / stride;  // exact: the numerator is a multiple of stride
+  a.dStep = -(a.step * dil) / stride;                                   // exact likewise
+  return a;
+}
+
+int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float dxMult, const float* f, const float* dy,
+                        void* ws, size_t wsBytes) {
   PixP q;
   q.IH = p.outH; q.IW = p.outW; q.Cin = p.K;
   q.N = p.N;
@@ -800,34 +851,14 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMu
     q.R = q.T * q.Cin;
     q.M = p.H * p.W * p.N;
     dense_layout(&q);
+    q.inImg = wd.yImg;
+    q.outImg = wd.xImg;
     return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, all_taps(p), 1, ws, wsBytes);
   }
-  // one class at a time; first the taps of every class, to know whether any class is empty
-  struct Axis { int first, step, count, dBase, dStep; };
-  auto axis = [](int phase, int pad, int dil, int stride, int taps) {
-    Axis a;
-    a.step = stride / gcd_int(dil, stride);
-    a.first = -1;
-    for (int i = 0; i < taps && i < a.step; ++i)
-      if ((phase + pad - i * dil) % stride == 0) { a.first = i; break; }
-    a.count = a.first < 0 ? 0 : (taps - a.first + a.step - 1) / a.step;
-    a.dBase = a.first < 0 ? 0 : (phase + pad - a.first * dil) / stride;  // exact: the numerator is a multiple of stride
-    a.dStep = -(a.step * dil) / stride;                                   // exact likewise
-    return a;
-  };
-  bool anyEmpty = false;
-  for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
-    for (int ph = 0; ph < p.sy && ph < p.H; ++ph)
-      if (axis(ph, p.pt, p.dy, p.sy, p.FH).count == 0 || axis(pw, p.pl, p.dx, p.sx, p.FW).count == 0) anyEmpty = true;
-  if (anyEmpty && dxMult == 0.f) {
-    int rc = mcn_fill((mcn_stream_t)s, dx, 0.f, (size_t)p.H * p.W * p.C * p.N);
-    if (rc) return rc;
-  } else if (anyEmpty && dxMult != 1.f) {
-    return fail(MCN_UNSUPPORTED, "mcn_conv_backward_data: accumulation with a multiplier other than 1 is not available for this stride");
-  }
+  // one class at a time (the caller has dealt with the classes no tap reaches)
   for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
     for (int ph = 0; ph < p.sy && ph < p.H; ++ph) {
-      const Axis ai = axis(ph, p.pt, p.dy, p.sy, p.FH), aj = axis(pw, p.pl, p.dx, p.sx, p.FW);
+      const Axis ai = stride_axis(ph, p.pt, p.dy, p.sy, p.FH), aj = stride_axis(pw, p.pl, p.dx, p.sx, p.FW);
       if (ai.count == 0 || aj.count == 0) continue;
       PixP c = q;
       c.OH = (p.H - ph + p.sy - 1) / p.sy;
@@ -836,9 +867,9 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMu
       c.dhBase = ai.dBase; c.dhStep = ai.dStep; c.dwBase = aj.dBase; c.dwStep = aj.dStep;
       c.R = c.T * c.Cin;
       c.M = c.OH * c.OW * p.N;
-      c.inImg = c.Cin * c.IH * c.IW;
+      c.inImg = wd.yImg;
       c.outPlane = p.H * p.W;
-      c.outImg = p.C * c.outPlane;
+      c.outImg = wd.xImg;
       c.outOff = ph + p.H * pw; c.outSH = p.sy; c.outSW = p.H * p.sx; c.dense = 0;
       TapSet t;
       t.FH = p.FH; t.FW = p.FW;
@@ -849,10 +880,37 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMu
     }
   return MCN_SUCCESS;
 }
+}  // namespace
 
-int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,
-                              size_t wsBytes) {
+int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
+                            void* ws, size_t wsBytes) {
+  // stride classes no tap reaches get no launch: they are zeros (or keep what is there, when accumulating)
+  bool anyEmpty = false;
+  for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
+    for (int ph = 0; ph < p.sy && ph < p.H; ++ph)
+      if (stride_axis(ph, p.pt, p.dy, p.sy, p.FH).count == 0 || stride_axis(pw, p.pl, p.dx, p.sx, p.FW).count == 0) anyEmpty = true;
+  if (anyEmpty && dxMult == 0.f) {
+    int rc = mcn_fill((mcn_stream_t)s, dx, 0.f, (size_t)p.H * p.W * p.C * p.N);
+    if (rc) return rc;
+  } else if (anyEmpty && dxMult != 1.f) {
+    return fail(MCN_UNSUPPORTED, "mcn_conv_backward_data: accumulation with a multiplier other than 1 is not available for this stride");
+  }
+  const ConvP g = group_view(p);
+  const Wide wd = wide_of(p);
+  const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
+  for (int i = 0; i < p.groups; ++i) {
+    int rc = backward_data_group(s, g, wd, dx + i * p.FC * HW, dxMult, f + i * p.Kg * FV, dy + i * p.Kg * Q, ws, wsBytes);
+    if (rc) return rc;
+  }
+  return MCN_SUCCESS;
+}
+
+namespace {
+int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float* df, const float* x, const float* dy,
+                          void* ws, size_t wsBytes) {
   WgP q;
+  q.xImg = wd.xImg;
+  q.dyImg = wd.yImg;
   q.H = p.H; q.W = p.W; q.C = p.C; q.K = p.K;
   q.OH = p.outH; q.OW = p.outW;
   q.FH = p.FH; q.T = p.FH * p.FW;
@@ -873,7 +931,6 @@ int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const fl
     q.byTilesK = FastDiv((p.K + BAk - 1) / BAk);
   }
   const size_t nF = (size_t)q.FV * p.K;
-  const bool ut = wgrad_uniform_tap(p);
   q.byC = FastDiv(p.C);
   float* target = df;
   if (q.splits > 1 || ut) {
@@ -905,6 +962,20 @@ int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const fl
   hipLaunchKernelGGL(conv_wgrad_reduce, dim3((unsigned)((nF + 63) / 64)), block, 0, s, df, target, nF, q.splits, ut ? 1 : 0,
                      p.C, q.T);
   return check_launch("mcn_conv_backward_filter(reduce)");
+}
+}  // namespace
+
+int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,
+                              size_t wsBytes) {
+  const ConvP g = group_view(p);
+  const Wide wd = wide_of(p);
+  const bool ut = wgrad_uniform_tap(p);
+  const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
+  for (int i = 0; i < p.groups; ++i) {
+    int rc = backward_filter_group(s, g, wd, ut, df + i * p.Kg * FV, x + i * p.FC * HW, dy + i * p.Kg * Q, ws, wsBytes);
+    if (rc) return rc;
+  }
+  return MCN_SUCCESS;
 }
 
 }  // namespace mcn

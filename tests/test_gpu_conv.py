@@ -29,6 +29,9 @@ CASES = [
     (20, 18, 32, 2, 3, 3, 32, 40, (2, 1), (1, 0, 2, 1), (1, 2)),  # 32 channels: tap-major kernels with stride + dilation
     (13, 11, 64, 3, 2, 3, 64, 130, 1, (0, 1, 1, 1), 1),      # even-sized filter, 130 filters (partial channel tile)
     (9, 9, 16, 2, 3, 3, 16, 16, (3, 3), 1, 1),               # 16 channels: tap-major forward only
+    (14, 14, 64, 2, 3, 3, 32, 64, 1, 1, 1),                  # 2 groups of 32 channels: tap-major kernels per group
+    (15, 14, 64, 2, 3, 3, 16, 96, (2, 2), 1, 1),             # 4 groups, strided: stride classes inside every group
+    (12, 12, 96, 2, 1, 1, 32, 48, 2, 0, 1),                  # 3 groups, 1x1 stride 2
 ]
 
 
@@ -300,3 +303,18 @@ def test_backward_data_accumulate(capi, ob, path):
             capi.set_tunable(k, 0)
     assert rel_max(got, 0.75 * base + want) < 2e-4
     assert rel_max(plain, want) < 2e-4
+
+
+def test_groups_and_strides_run_on_the_mfma_kernels(capi, ob):
+    """Filter groups and strided backward-data are served by the MFMA kernels (one launch per group and stride
+    class), not by the one-thread-per-output fallback."""
+    case = (15, 14, 64, 2, 3, 3, 16, 96, (2, 2), 1, 1)
+    x, f, b = _tensors(case)
+    cg = capi.conv_geom(x.shape, f.shape, *case[8:])
+    dy = F(np.random.default_rng(3).standard_normal(capi.conv_out_shape(cg)))
+    capi.profile_begin("_mfma")
+    capi.conv_forward(capi.to_device(x), capi.to_device(f), capi.to_device(b), cg)
+    capi.conv_backward(capi.to_device(x), capi.to_device(f), capi.to_device(dy), cg)
+    launches, _ = capi.profile_end()
+    # 4 groups: forward 4, backward-filter 4, backward-data 4 groups x 4 stride classes
+    assert launches == 4 + 4 + 16
