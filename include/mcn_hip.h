@@ -231,6 +231,10 @@ MCN_API int mcn_relu_forward(mcn_stream_t stream, float* y, const float* x, size
 MCN_API int mcn_relu_backward(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, size_t n);
 /* y = a + b   (matlab/+dagnn/Sum.m:11-17; also the fan-out derivative sum of +dagnn/Layer.m:127-135) */
 MCN_API int mcn_add(mcn_stream_t stream, float* y, const float* a, const float* b, size_t n);
+/* y = alpha*a + beta*b, the momentum / weight update of SGD (matlab/src/vl_taccummex.cu:48-78: copy, BLAS scal, then
+   BLAS axpy; examples/cnn_train_dag.m:316-378).  y may be a (the MEX's 'InPlace' mode).  Each element goes through
+   the roundings of that pair: t = fl(alpha*a), y = fl(t + fl(beta*b)). */
+MCN_API int mcn_taccum(mcn_stream_t stream, float* y, float alpha, const float* a, float beta, const float* b, size_t n);
 /* y[i] = value   (bits/impl/copy_gpu.cu:17-33 fill) */
 MCN_API int mcn_fill(mcn_stream_t stream, float* y, float value, size_t n);
 

@@ -1,6 +1,8 @@
 // See frontend.hpp.  Error texts are the reference drivers' own, so callers that match on them keep working.
 #include "frontend.hpp"
 
+#include "accumulate.hpp"
+
 #include <cctype>
 #include <cstdio>
 
@@ -504,6 +506,30 @@ void nnpool(Context& context, Allocator& allocator, int nout, Tensor* out, int n
   (void)nout;
 }
 
+// ------------------------------------------------------------------------------------------ vl_taccum
+// matlab/src/vl_taccummex.cu:151-224 (the MEX behind matlab/vl_taccum.m): (alpha, A, beta, B [, 'InPlace'])
+
+void taccum(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in) {
+  enum { optInPlace, optVerbose };
+  static OptionSpec const specs[] = {{"InPlace", false, optInPlace}, {"Verbose", false, optVerbose}, {NULL, false, 0}};
+  bool inplace = false;
+  if (nin < 4) raise(VLE_IllegalArgument, "There are less than four arguments.");
+  int next = 4, opt;
+  Arg const* value = NULL;
+  while ((opt = nextOption(in, nin, specs, &next, &value)) >= 0)
+    if (opt == optInPlace) inplace = true;
+  if (!(isPlainMatrix(in[0]) && in[0].tensor.getNumElements() == 1)) raise(VLE_IllegalArgument, "ALPHA is not a plain scalar.");
+  if (!(isPlainMatrix(in[2]) && in[2].tensor.getNumElements() == 1)) raise(VLE_IllegalArgument, "BETA is not a plain scalar.");
+  Tensor a = dataTensor(in[1], "A", 4), b = dataTensor(in[3], "B", 4);
+  if (!areCompatible(a, b)) raise(VLE_IllegalArgument, "A and B do not have compatible formats.");
+  if (a.getNumElements() != b.getNumElements()) raise(VLE_IllegalArgument, "A and B do not have the same number of elements.");
+  const double alpha = values(in[0])[0], beta = values(in[2])[0];
+  Tensor output = inplace ? a : newOutput(allocator, a.getDeviceType(), a.getDataType(), in[1].tensor.getShape());
+  failFromContext(context, vl::accumulate(context, output, alpha, a, beta, b));
+  if (!inplace) out[0] = output;
+  (void)nout;
+}
+
 typedef void (*Body)(Context&, Allocator&, int, Tensor*, int, Arg const*);
 
 ErrorCode guarded(Body body, Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
@@ -532,6 +558,9 @@ ErrorCode vl_nnbnorm(Context& context, Allocator& allocator, int nout, Tensor* o
 }
 ErrorCode vl_nnpool(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
   return guarded(nnpool, context, allocator, nout, out, nin, in, message);
+}
+ErrorCode vl_taccum(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
+  return guarded(taccum, context, allocator, nout, out, nin, in, message);
 }
 
 } }  // namespace vl::frontend

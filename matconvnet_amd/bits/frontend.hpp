@@ -6,6 +6,7 @@
 //   vl_nnconvt(x, f, b [, dzdy], options...)   matlab/src/vl_nnconvt.cu:81-417
 //   vl_nnbnorm(x, g, b [, dzdy], options...)   matlab/src/vl_nnbnorm.cu:73-301
 //   vl_nnpool (x, pool [, dzdy], options...)   matlab/src/vl_nnpool.cu:72-314
+//   vl_taccum (alpha, a, beta, b [, 'InPlace']) matlab/src/vl_taccummex.cu:151-224
 // Where the MEX drivers raise a MATLAB error these return a vl::ErrorCode and leave the reference's
 // message text in `message`.
 #ifndef MCN_AMD_BITS_FRONTEND_HPP
@@ -46,6 +47,7 @@ class Allocator {
 //   vl_nnconvt: forward [y]             backward [dzdx, dzdf, dzdb]
 //   vl_nnbnorm: forward [y, moments]    backward [dzdx, dzdg, dzdb, moments]
 //   vl_nnpool : forward [y]             backward [dzdx]
+//   vl_taccum : [alpha*a + beta*b]; nothing with 'InPlace' (a itself is updated)
 ErrorCode vl_nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                     std::string& message);
 ErrorCode vl_nnconvt(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
@@ -53,6 +55,8 @@ ErrorCode vl_nnconvt(Context& context, Allocator& allocator, int nout, Tensor* o
 ErrorCode vl_nnbnorm(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                      std::string& message);
 ErrorCode vl_nnpool(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
+                    std::string& message);
+ErrorCode vl_taccum(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                     std::string& message);
 
 } }  // namespace vl::frontend

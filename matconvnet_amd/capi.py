@@ -50,6 +50,7 @@ PROTOTYPES = {
     "mcn_conv_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _i]),
     "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
+    "mcn_taccum": (_i, [_vp, _vp, C.c_float, _vp, C.c_float, _vp, _sz]),
     "mcn_conv_backward_data_acc": (_i, [_vp, C.POINTER(ConvGeom), _vp, C.c_float, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_filter": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_bias": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _sz]),
@@ -334,6 +335,13 @@ def relu_backward(x, dy):
     dx = _torch().empty_like(x)
     check(lib().mcn_relu_backward(stream(), ptr(dx), ptr(x), ptr(dy), x.numel()))
     return dx
+
+
+def taccum(alpha, a, beta, b, out=None):
+    """alpha*a + beta*b (include/mcn_hip.h: mcn_taccum); out may be a."""
+    y = _torch().empty_like(a) if out is None else out
+    check(lib().mcn_taccum(stream(), ptr(y), float(alpha), ptr(a), float(beta), ptr(b), a.numel()))
+    return y
 
 
 def add(a, b):

@@ -1,4 +1,4 @@
-// Element-wise companions of the operators: ReLU, sum of two tensors, fill.  Pure streaming kernels:
+// Element-wise companions of the operators: ReLU, sum of two tensors, scaled sum (the SGD update), fill.  Pure streaming kernels:
 // 16-byte accesses, grid-stride, enough workgroups to cover the chip several times.
 #include "mcn_internal.hpp"
 
@@ -11,11 +11,21 @@
 namespace mcn {
 namespace {
 
-enum { OP_RELU_FWD, OP_RELU_BWD, OP_ADD, OP_FILL };
+enum { OP_RELU_FWD, OP_RELU_BWD, OP_ADD, OP_FILL, OP_AXPBY };
 
 template <int OP>
-__device__ __forceinline__ float apply1(float a, float b, float k) {
+struct Reads {
+  static constexpr bool a = OP != OP_FILL;
+  static constexpr bool b = OP == OP_RELU_BWD || OP == OP_ADD || OP == OP_AXPBY;
+};
+
+template <int OP>
+__device__ __forceinline__ float apply1(float a, float b, float k, float k2) {
   switch (OP) {
+    case OP_AXPBY: {                                     // scal, then axpy: three roundings like the BLAS pair
+      const float t = k * a;
+      return t + k2 * b;
+    }
     case OP_RELU_FWD: return a > 0.f ? a : 0.f;          // max(x, 0)
     case OP_RELU_BWD: return a > 0.f ? b : b * 0.f;      // dzdy .* (x > 0): keeps NaN/inf*0 semantics
     case OP_ADD: return a + b;
@@ -26,48 +36,47 @@ __device__ __forceinline__ float apply1(float a, float b, float k) {
 // y = op(a, b).  The vector body covers n/4 float4s; the tail (n % 4) is handled by the first threads.
 template <int OP, bool VEC4>
 __global__ __launch_bounds__(256) void eltwise_kernel(float* __restrict__ y, const float* __restrict__ a,
-                                                      const float* __restrict__ b, float k, size_t n) {
+                                                      const float* __restrict__ b, float k, float k2, size_t n) {
   const size_t stride = (size_t)gridDim.x * 256;
   const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (VEC4) {
     const size_t n4 = n / 4;
     for (size_t i = t; i < n4; i += stride) {
       float4 u = make_float4(0.f, 0.f, 0.f, 0.f), v = u, r;
-      if (OP != OP_FILL) u = stream_load4((const float4*)a + i);
-      if (OP == OP_RELU_BWD || OP == OP_ADD) v = stream_load4((const float4*)b + i);
-      r.x = apply1<OP>(u.x, v.x, k);
-      r.y = apply1<OP>(u.y, v.y, k);
-      r.z = apply1<OP>(u.z, v.z, k);
-      r.w = apply1<OP>(u.w, v.w, k);
+      if (Reads<OP>::a) u = stream_load4((const float4*)a + i);
+      if (Reads<OP>::b) v = stream_load4((const float4*)b + i);
+      r.x = apply1<OP>(u.x, v.x, k, k2);
+      r.y = apply1<OP>(u.y, v.y, k, k2);
+      r.z = apply1<OP>(u.z, v.z, k, k2);
+      r.w = apply1<OP>(u.w, v.w, k, k2);
       stream_store4((float4*)y + i, r);
     }
     for (size_t i = n4 * 4 + t; i < n; i += stride) {
-      const float u = (OP != OP_FILL) ? a[i] : 0.f;
-      const float v = (OP == OP_RELU_BWD || OP == OP_ADD) ? b[i] : 0.f;
-      y[i] = apply1<OP>(u, v, k);
+      const float u = Reads<OP>::a ? a[i] : 0.f;
+      const float v = Reads<OP>::b ? b[i] : 0.f;
+      y[i] = apply1<OP>(u, v, k, k2);
     }
   } else {
     for (size_t i = t; i < n; i += stride) {
-      const float u = (OP != OP_FILL) ? a[i] : 0.f;
-      const float v = (OP == OP_RELU_BWD || OP == OP_ADD) ? b[i] : 0.f;
-      y[i] = apply1<OP>(u, v, k);
+      const float u = Reads<OP>::a ? a[i] : 0.f;
+      const float v = Reads<OP>::b ? b[i] : 0.f;
+      y[i] = apply1<OP>(u, v, k, k2);
     }
   }
 }
 
 template <int OP>
-int launch(const char* who, mcn_stream_t stream, float* y, const float* a, const float* b, float k, size_t n) {
+int launch(const char* who, mcn_stream_t stream, float* y, const float* a, const float* b, float k, size_t n,
+           float k2 = 0.f) {
   if (n == 0) return MCN_SUCCESS;
-  if (!y || (OP != OP_FILL && !a) || ((OP == OP_RELU_BWD || OP == OP_ADD) && !b))
-    return fail(MCN_ILLEGAL_ARGUMENT, "%s: null tensor", who);
-  const bool vec = aligned16(y) && (OP == OP_FILL || aligned16(a)) &&
-                   (!(OP == OP_RELU_BWD || OP == OP_ADD) || aligned16(b));
+  if (!y || (Reads<OP>::a && !a) || (Reads<OP>::b && !b)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: null tensor", who);
+  const bool vec = aligned16(y) && (!Reads<OP>::a || aligned16(a)) && (!Reads<OP>::b || aligned16(b));
   // each thread handles a few float4s; cap the grid at 32 workgroups per CU-equivalent (256 CUs)
   const size_t work = vec ? (n + 3) / 4 : n;
   const unsigned blocks = (unsigned)std::min<size_t>((work + 255) / 256, 256u * 32u);
   KernelTimer timer("eltwise_kernel", as_stream(stream));
-  if (vec) hipLaunchKernelGGL((eltwise_kernel<OP, true>), dim3(blocks), dim3(256), 0, as_stream(stream), y, a, b, k, n);
-  else hipLaunchKernelGGL((eltwise_kernel<OP, false>), dim3(blocks), dim3(256), 0, as_stream(stream), y, a, b, k, n);
+  if (vec) hipLaunchKernelGGL((eltwise_kernel<OP, true>), dim3(blocks), dim3(256), 0, as_stream(stream), y, a, b, k, k2, n);
+  else hipLaunchKernelGGL((eltwise_kernel<OP, false>), dim3(blocks), dim3(256), 0, as_stream(stream), y, a, b, k, k2, n);
   return check_launch(who);
 }
 
@@ -86,6 +95,9 @@ int mcn_relu_backward(mcn_stream_t stream, float* derInput, const float* x, cons
 }
 int mcn_add(mcn_stream_t stream, float* y, const float* a, const float* b, size_t n) {
   return launch<OP_ADD>("mcn_add", stream, y, a, b, 0.f, n);
+}
+int mcn_taccum(mcn_stream_t stream, float* y, float alpha, const float* a, float beta, const float* b, size_t n) {
+  return launch<OP_AXPBY>("mcn_taccum", stream, y, a, b, alpha, n, beta);
 }
 int mcn_fill(mcn_stream_t stream, float* y, float value, size_t n) {
   return launch<OP_FILL>("mcn_fill", stream, y, nullptr, nullptr, value, n);

@@ -167,6 +167,14 @@ def vl_nnpool(*args):
     return _call("vl_nnpool", 1, list(args))[0]
 
 
+def vl_taccum(*args):
+    """vl_taccum(alpha, a, beta, b [, 'inplace']): alpha*a + beta*b (matlab/vl_taccum.m); with 'inplace', `a` itself
+    is updated and returned."""
+    inplace = any(isinstance(o, str) and o.lower() == "inplace" for o in args[4:])
+    r = _call("vl_taccum", 0 if inplace else 1, list(args))
+    return args[1] if inplace else r[0]
+
+
 class Bottleneck:
     """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
 

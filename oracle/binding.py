@@ -212,6 +212,16 @@ def subsample_forward(x, b, stride=1, pad=0):
     return y
 
 
+def taccum(alpha, a, beta, b):
+    """vl_taccum(alpha, a, beta, b): matlab/src/vl_taccummex.cu:48-78."""
+    s, ct = _sfx(a.dtype)
+    y = fempty(a.shape, a.dtype)
+    fn = getattr(lib(), "oracle_taccum_" + s)
+    fn.argtypes = [C.c_void_p, ct, C.c_void_p, ct, C.c_void_p, C.c_size_t]
+    fn(_p(y), alpha, _p(a), beta, _p(b), a.size)
+    return y
+
+
 def subsample_backward(xshape, dy, stride=1, pad=0):
     """dzdx of the same call (bits/nnsubsample.cu:125-165); dzdb is the per-channel sum of dzdy."""
     s, _ = _sfx(dy.dtype)

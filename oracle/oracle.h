@@ -125,7 +125,10 @@ void oracle_set_dgemm(void* fn);
   /* bits/nnsubsample.cu:125-165 */                                                        \
   void oracle_subsample_backward_##S(T* dx, const T* dy, int H, int W, int C, int N,      \
                                      int strideY, int strideX, int padTop, int padBottom, \
-                                     int padLeft, int padRight);
+                                     int padLeft, int padRight);                                \
+  /* matlab/src/vl_taccummex.cu:48-78: y = a (copy), BLAS scal y *= alpha, BLAS axpy       \
+     y += beta*b, as the reference-BLAS loops; y may be a */                               \
+  void oracle_taccum_##S(T* y, T alpha, const T* a, T beta, const T* b, size_t n);
 
 ORACLE_DECLARE(float, f32)
 ORACLE_DECLARE(double, f64)

@@ -462,6 +462,11 @@ int oracle_pool_out_w(const oracle_pool_geom* g) {
   void oracle_subsample_backward_##S(T* dx, const T* dy, int H, int W, int Cc, int N, int sy,     \
                                      int sx, int pt, int pb, int pl, int pr) {                     \
     subsample_backward<T>(dx, dy, H, W, Cc, N, sy, sx, pt, pb, pl, pr);                            \
+  }                                                                                                \
+  void oracle_taccum_##S(T* y, T alpha, const T* a, T beta, const T* b, size_t n) {                \
+    for (size_t i = 0; i < n; ++i) y[i] = a[i];               /* copy  */                          \
+    for (size_t i = 0; i < n; ++i) y[i] = alpha * y[i];       /* scal  */                          \
+    for (size_t i = 0; i < n; ++i) y[i] = y[i] + beta * b[i]; /* axpy  */                          \
   }
 
 ORACLE_DEFINE(float, f32)

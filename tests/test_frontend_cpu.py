@@ -151,3 +151,27 @@ def test_vl_nnconv_empty_filters_follow_the_identity_bank_rules(vl):
     with pytest.raises(vl.VlError) as e:  # valid arguments reach the operator, which has no CPU path
         vl.vl_nnconv(z(8, 8, 4, 2), e0, z(4), "stride", 2)
     assert e.value.code == 1
+
+
+TACCUM_ERRORS = [
+    ((1.0, z(4, 4, 2, 1), 2.0), "There are less than four arguments."),
+    (([1.0, 2.0], z(4, 4, 2, 1), 2.0, z(4, 4, 2, 1)), "ALPHA is not a plain scalar."),
+    ((1.0, z(4, 4, 2, 1), [], z(4, 4, 2, 1)), "BETA is not a plain scalar."),
+    ((1.0, z(4, 4, 2, 1), 2.0, z(4, 4, 2, 1).double()), "A and B do not have compatible formats."),
+    ((1.0, z(4, 4, 2, 1), 2.0, z(4, 4, 3, 1)), "A and B do not have the same number of elements."),
+    ((1.0, z(4, 4, 2, 1), 2.0, z(4, 4, 2, 1), "bogus"), "Unknown option 'bogus'."),
+]
+
+
+@pytest.mark.parametrize("args,message", TACCUM_ERRORS)
+def test_vl_taccum_messages(vl, args, message):
+    """Texts and order of matlab/src/vl_taccummex.cu:165-194."""
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_taccum(*args)
+    assert e.value.message == message
+
+
+def test_vl_taccum_reaches_the_operator_which_has_no_cpu_path(vl):
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_taccum(0.9, z(4, 4, 2, 1), -0.1, z(4, 4, 2, 1))
+    assert e.value.code == 1  # VLE_Unsupported

@@ -112,3 +112,19 @@ def test_convt_upsample_is_zero_insertion(ob):
     stuffed = np.zeros(((4 - 1) * uy + 1, (5 - 1) * ux + 1, 3, 2), order="F")
     stuffed[::uy, ::ux] = x
     assert rel_max(ob.convt_forward(x, f, None, (uy, ux), 0), ob.convt_forward(F(stuffed, np.float64), f, None, 1, 0)) < 1e-13
+
+
+def test_taccum_is_the_scal_axpy_pair(ob):
+    """vl_taccummex.cu:57-74: every element is fl(fl(alpha*a) + fl(beta*b)); numpy's float32 arithmetic rounds each
+    operation separately, so the restatement must agree with it bit for bit; and the SGD momentum update it serves
+    (cnn_train_dag.m:350-366) comes out as the closed form in double."""
+    r = np.random.default_rng(2)
+    a = F(r.standard_normal((7, 5, 3, 2)))
+    b = F(r.standard_normal((7, 5, 3, 2)))
+    alpha, beta = np.float32(0.9), np.float32(-0.0123)
+    got = ob.taccum(float(alpha), a, float(beta), b)
+    want = (alpha * a) + (beta * b)
+    assert got.dtype == np.float32 and np.array_equal(got, want)
+    got64 = ob.taccum(0.9, F(a, np.float64), -0.0123, F(b, np.float64))
+    assert np.allclose(got64, 0.9 * a.astype(np.float64) - 0.0123 * b.astype(np.float64), rtol=1e-15, atol=0)
+    assert np.array_equal(ob.taccum(1.0, a, 0.0, b), a) and np.array_equal(ob.taccum(0.0, a, 1.0, b), b)
