@@ -139,8 +139,8 @@ __device__ __forceinline__ void store_block(floatx16 acc, bufrsrc rsrc, unsigned
   }
 }
 
-// Weights-stationary variant (conv_ws.hip) for filter banks that fit in LDS: wt is the packed bank in tap-major
-// order (R = ci + Cin*t).  Sets *handled when it took the work.
+// Weights-stationary variant (conv_ws.hip) for filter banks that fit in LDS: wt is the packed bank in the
+// 16-channel-chunk order of conv_pack_weights.  Sets *handled when it took the work.
 int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, const float* wt, const float* bias,
                    const PixP& p, int* handled);
 

@@ -38,7 +38,11 @@ constexpr int kMaxTaps = 128;
 
 
 // wt[R][co] from the MATLAB filter bank f[i,j,c,k] (FV x K, column-major), t = i + FH*j.
-//   reduction row R = t + T*ci (channel-major) or, when tapMajor, R = ci + Cin*t
+//   reduction row R = t + T*ci (channel-major) or, when tapMajor (Cin a multiple of 16), in chunks of 16 channels
+//   with the taps inside a chunk: R = c16 + 16*(t + T*chunk), ci = 16*chunk + c16.  Walking the taps of a few
+//   channels before moving to the next channels re-reads the same pixels (shifted by a tap) back to back, while
+//   they are still in L1 / L2; tap-outermost order re-read the whole channel range between two visits, which sent
+//   3x3 layers through the memory fabric 8 times over.
 //   forward:        ci = c, co = k : f[t + T*c + FV*k]
 //   backward-data:  ci = k, co = c : f[t + T*(c + C*k)]
 // Only the taps (i0 + a*iStep, j0 + b*jStep), a < nI, b < nJ, of the FH x FW filter take part (all of them for a
@@ -58,8 +62,15 @@ __global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt,
   const int r = (int)(idx / coutPad), co = (int)(idx - (size_t)r * coutPad);
   float v = 0.f;
   if (r < T * Cin && co < Cout) {
-    const int ci = tapMajor ? r % Cin : r / T;
-    const int t = tapMajor ? r / Cin : r % T;
+    int ci, t;
+    if (tapMajor) {
+      const int chunk = r / (16 * T), rem = r - chunk * 16 * T;
+      t = rem / 16;
+      ci = chunk * 16 + (rem - t * 16);
+    } else {
+      ci = r / T;
+      t = r - ci * T;
+    }
     const int b = t / ts.nI, a = t - b * ts.nI;
     const size_t Tf = (size_t)ts.FH * ts.FW;
     const size_t tf = (size_t)(ts.i0 + a * ts.iStep) + (size_t)ts.FH * (ts.j0 + b * ts.jStep);
@@ -68,8 +79,8 @@ __global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt,
   wt[idx] = v;
 }
 
-// UT ("uniform tap"): the reduction runs tap-major (R = ci + Cin*t) and Cin is a multiple of 16, so all 16
-// rows of a step share one tap: the tap's shift and the inside-the-image test are computed once per step and
+// UT ("uniform tap"): Cin is a multiple of 16 and the reduction runs in chunks of 16 channels, tap by tap inside
+// a chunk (see conv_pack_weights), so all 16 rows of a step share one tap: the tap's shift and the inside-the-image test are computed once per step and
 // thread, the step's base address is uniform (scalar registers), and every gathered row is a load at a
 // per-thread constant 32-bit offset from it.  This removes almost all vector-ALU work from the loop, and
 // vector-ALU work is what competes with the MFMAs for the SIMD.
@@ -169,10 +180,9 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
 #pragma unroll
         for (int e = 0; e < RPT; ++e) pb[e] = 0.f;
       }
-      utCi += BK;
-      if (utCi >= p.Cin) {
-        utCi = 0;
-        ++utTap;
+      if (++utTap == p.T) {  // the taps of these 16 channels, then the next 16 channels
+        utTap = 0;
+        utCi += BK;
       }
     } else {
       int2 tp[RPT];

@@ -22,7 +22,7 @@
 //     matrix pipe for the SIMD: with 5 per MFMA an earlier form of this kernel reached only half the MFMA rate);
 //   * units are dealt so that every SIMD of the chip gets the same number of them to within one, and the channel
 //     blocks of one pixel block go to neighbouring wavefronts of one workgroup (the pixels come from HBM once).
-// Reduction order: tap-major (R = ci + Cin*t), pairs of rows per MFMA, sequential accumulation in fp32 like the
+// Reduction order: chunks of 16 channels, the taps inside a chunk (the packed bank's order), pairs of rows per MFMA, sequential accumulation in fp32 like the
 // tiled kernel.
 #include "conv_common.hpp"
 
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   int ihB, iwB;      // gathered coordinates at tap shift 0
   unsigned voffN;    // the same three for the unit after the one being loaded: worked out beside the stores of a
   int ihBN, iwBN;    // finished unit, so that the loop itself carries no address arithmetic
-  int tapL = 0, giL = 0;  // tap and 16-channel chunk inside the tap of the next group
+  int tapL = 0, giL = 0;  // tap and 16-channel chunk of the next group (taps innermost: see conv_pack_weights)
   unsigned voTap;    // per-lane offset of that tap's pixels (a register of its own for the whole tap: recomputed
                      // per group, the register allocator handed its register to a load result, and every group
                      // then waited for all loads in flight before it could form the next offset)
@@ -148,16 +148,17 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     const int sbase_ = giL * (2 * kDepth) * planeBytes;                                                   \
     _Pragma("unroll") for (int d_ = 0; d_ < kDepth; ++d_) DST[d_] = __builtin_bit_cast(                   \
         float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voTap, sbase_ + 2 * d_ * planeBytes, 0));  \
-    if (++giL == w.groupsPerTap) {                                                                        \
-      giL = 0;                                                                                            \
-      if (++tapL == p.T) {                                                                                \
-        tapL = 0;                                                                                         \
+    if (++tapL == p.T) {                                                                                  \
+      tapL = 0;                                                                                           \
+      if (++giL == w.groupsPerTap) {                                                                      \
+        giL = 0;                                                                                          \
         voff = voffN;                                                                                     \
         ihB = ihBN;                                                                                       \
         iwB = iwBN;                                                                                       \
+        if (!TAPS) voTap = voff;                                                                          \
       }                                                                                                   \
-      voTap = tap_offset(tapL);                                                                           \
     }                                                                                                     \
+    if (TAPS) voTap = tap_offset(tapL);                                                                   \
   } while (0)
 
   // multiplies the stream's oldest group (operands CUR, group G of the unit in hand) after putting one more
