@@ -30,6 +30,8 @@ Tunable g_tunables[] = {
     {"conv_no_ws", 0},                 // 1: never use the weights-stationary kernel
     {"conv_ws_min_units", 0},          // least number of units for the weights-stationary kernel; 0 = two per SIMD
     {"conv_ws_wa", 0},                 // 1, 2, 4: force its channels-per-wavefront (in units of 32); 0 = choose
+    {"conv_no_split", 0},              // 1: the tiled kernel never splits its reduction over workgroups
+    {"conv_no_fc_view", 0},            // 1: fully-connected layers are not recast as 1x1 layers
     {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels
     {"conv_pix_tile", 0},              // force a tile shape of the pixel-major MFMA kernel (0 = automatic)
     {"conv_no_uniform_tap", 0},        // 1: disable the uniform-tap variant of the pixel-major kernel

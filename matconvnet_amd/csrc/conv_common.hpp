@@ -55,6 +55,12 @@ struct PixP {
   // (dense = 1: the pixel offset is the pixel index itself); a filter group sees a slice of the channels of a
   // wider tensor, a stride class of a strided layer's backward-data product a sub-grid of the pixels.
   int inImg, outImg, outPlane, outOff, outSH, outSW, dense;
+  // Split reduction (tiled kernel only; 1 = none): workgroup `split` multiplies steps [split*stepsPerSplit, ...) of
+  // 16 rows and writes its partial result to out + split*partStride (dense layout, alpha = 1, beta = 0, no bias);
+  // conv_pix_reduce then adds the partials up.  For layers with few output pixels and a long reduction
+  // (fully-connected layers above all), which would otherwise keep a handful of workgroups busy for a long time.
+  int rSplits, stepsPerSplit;
+  long long partStride;
 };
 
 // the pixel's element offset inside its channel plane of the produced tensor

@@ -79,6 +79,21 @@ __global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt,
   wt[idx] = v;
 }
 
+// out = alpha * (sum of the partial results of a split reduction) + beta*out + bias, element by element of a dense
+// output tensor [n][co][q].  The partials are added in split order: deterministic.
+__global__ __launch_bounds__(256) void conv_pix_reduce(float* __restrict__ out, const float* __restrict__ partials,
+                                                       const float* __restrict__ bias, size_t n, long long partStride,
+                                                       int splits, float alpha, float beta, int Q, int Cout) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float s = partials[i];
+  for (int k = 1; k < splits; ++k) s += partials[(size_t)k * partStride + i];
+  float v = alpha * s;
+  if (beta != 0.f) v = fmaf(beta, out[i], v);
+  if (bias) v += bias[(i / Q) % Cout];
+  out[i] = v;
+}
+
 // UT ("uniform tap"): Cin is a multiple of 16 and the reduction runs in chunks of 16 channels, tap by tap inside
 // a chunk (see conv_pack_weights), so all 16 rows of a step share one tap: the tap's shift and the inside-the-image test are computed once per step and
 // thread, the step's base address is uniform (scalar registers), and every gathered row is a load at a
@@ -107,7 +122,14 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   const int wa = wave / NWB, wb = wave - wa * NWB;
 
   const int tilesA = (p.Cout + BA - 1) / BA;
-  const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  int split = 0;
+  if (p.rSplits > 1) {  // (split-major: the workgroups of one split are neighbours)
+    const int tiles = (int)gridDim.x / p.rSplits;
+    split = logical / tiles;
+    logical -= split * tiles;
+    out += (size_t)split * p.partStride;
+  }
   const int mt = logical / tilesA;
   const int co0 = (logical - mt * tilesA) * BA;
   const int m0 = mt * BB;
@@ -135,13 +157,16 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
     inN = in + (size_t)n * p.inImg + ihB + p.IH * iwB;
   }
   // first gathered row of this thread: R = pg*RPT -> (tap, channel); advanced by BK per step
+  const int nStepsAll = (p.R + BK - 1) / BK;
+  const int sBegin = split * p.stepsPerSplit;
+  const int sEnd = p.rSplits > 1 ? min(nStepsAll, sBegin + p.stepsPerSplit) : nStepsAll;
   int ciS, tapS;
-  p.byT.divmod(pg * RPT, &ciS, &tapS);
+  p.byT.divmod(pg * RPT + sBegin * BK, &ciS, &tapS);
   const int advC = p.advC, advT = p.advT;
   // UT: per-thread constant element offsets (relative to `in`) of this thread's RPT channels at tap shift 0,
   // and the uniform (tap, first channel) of the step being fetched
   int offE[RPT];
-  int utTap = 0, utCi = 0;
+  int utTap = 0, utCi = 0;  // step s of the chunked order: tap s % T of channels 16*(s / T) ...
   if (UT) {
     const int pix = (int)(inN - in);
 #pragma unroll
@@ -160,7 +185,11 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   float4 pa0 = make_float4(0.f, 0.f, 0.f, 0.f), pa1 = pa0;  // parked weight vectors (APT <= 2)
   static_assert(APT <= 2, "at most two weight vectors per thread and step");
   unsigned okMask = 0;  // bit e: gathered row e of the parked step lies inside the image
-  const int nSteps = (p.R + BK - 1) / BK;
+  if (UT && sBegin > 0) {
+    const int chunk = p.byT.div(sBegin);
+    utTap = sBegin - chunk * p.T;
+    utCi = chunk * BK;
+  }
 
   // Issues the global loads of one step and parks them in registers.  Straight-line on purpose: the tap
   // table reads go out together, and rows that fall outside the image load a dummy (the tensor's first
@@ -233,13 +262,15 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   };
 
   __syncthreads();  // tapTab ready
-  fetch(0);
-  stash(0);
+  if (sBegin < sEnd) {
+    fetch(sBegin);
+    stash(0);
+  }
   __syncthreads();
 
-  for (int step = 0; step < nSteps; ++step) {
-    const int buf = step & 1;
-    if (step + 1 < nSteps) fetch(step + 1);
+  for (int step = sBegin; step < sEnd; ++step) {
+    const int buf = (step - sBegin) & 1;
+    if (step + 1 < sEnd) fetch(step + 1);
     const float* Ab = As[buf] + wa * WA * 32 + l32 + kh * BA;
     const float* Bb = Bs[buf] + wb * WB * 32 + l32 + kh * BB;
     // operand fragments are read one reduction pair ahead of the MFMAs that consume them
@@ -264,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
         for (int jj = 0; jj < WB; ++jj)
           acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][ii], b[cur][jj], acc[ii][jj], 0, 0, 0);
     }
-    if (step + 1 < nSteps) stash(buf ^ 1);
+    if (step + 1 < sEnd) stash(buf ^ 1);
     __syncthreads();
   }
 
@@ -618,6 +649,23 @@ ConvP group_view(const ConvP& p) {
   return g;
 }
 
+// A layer whose filters cover its whole (unpadded) input makes one output pixel per image: a fully-connected
+// layer.  In memory x is then the matrix (H*W*C) x N and the bank (H*W*C) x K, which is exactly a 1x1 layer over a
+// 1x1 image with H*W*C channels -- the reference's special case too (bits/nnfullyconnected.cu:30-185: plain GEMMs).
+// Seen that way the reduction has one tap and H*W*C rows instead of H*W taps of which each output pixel of the
+// backward-data product uses one.
+ConvP fc_view(const ConvP& p) {
+  if (!(p.groups == 1 && p.FH == p.H && p.FW == p.W && p.pt == 0 && p.pl == 0 && p.outH == 1 && p.outW == 1 &&
+        p.dy == 1 && p.dx == 1) || (p.H == 1 && p.W == 1) || (long long)p.H * p.W * p.C >= (1ll << 31) ||
+      tunable("conv_no_fc_view", 0))
+    return p;
+  ConvP v = p;
+  v.C = v.FC = p.H * p.W * p.C;
+  v.H = v.W = v.FH = v.FW = 1;
+  v.sy = v.sx = 1;
+  return v;
+}
+
 struct Wide {
   int xImg, yImg;  // elements between images of the layer's input and output tensors
 };
@@ -654,10 +702,30 @@ void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, con
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB;
   const long long mTiles = ((long long)p.M + BB - 1) / BB;
   const int tilesA = (p.Cout + BA - 1) / BA;
-  const dim3 grid((unsigned)(mTiles * tilesA));
+  const dim3 grid((unsigned)(mTiles * tilesA * p.rSplits));
   KernelTimer timer("conv_pix_mfma", s);
   if (ut) hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB, true>), grid, dim3(256), 0, s, out, in, wt, bias, p);
   else hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB, false>), grid, dim3(256), 0, s, out, in, wt, bias, p);
+}
+
+// `shape` as in PixPlan; the tunable forces one for experiments (it must fit the channel tile)
+void launch_shape(hipStream_t s, int shape, float* out, const float* in, const float* wt, const float* bias, const PixP& p,
+                  bool ut) {
+  const int BA = pick_channels_tile(p.Cout);
+  const int forced = tunable("conv_pix_tile", 0);
+  if (forced) shape = forced;
+  if ((shape == 1 || shape == 5 || shape == 7) && BA != 128) shape = BA == 64 ? 2 : 3;
+  if ((shape == 2 || shape == 4 || shape == 6) && BA != 64) shape = BA == 128 ? 1 : 3;
+  if (shape == 3 && BA != 32) shape = BA == 128 ? 1 : 2;
+  switch (shape) {
+    case 1: launch_pix<2, 2, 2, 2>(s, out, in, wt, bias, p, ut); break;  // 128 x 128
+    case 2: launch_pix<2, 2, 1, 4>(s, out, in, wt, bias, p, ut); break;  //  64 x 256
+    case 3: launch_pix<1, 2, 1, 4>(s, out, in, wt, bias, p, ut); break;  //  32 x 256
+    case 4: launch_pix<1, 2, 2, 2>(s, out, in, wt, bias, p, ut); break;  //  64 x 128
+    case 5: launch_pix<2, 1, 2, 2>(s, out, in, wt, bias, p, ut); break;  // 128 x  64
+    case 7: launch_pix<1, 1, 4, 1>(s, out, in, wt, bias, p, ut); break;  // 128 x  32
+    default: launch_pix<1, 1, 2, 2>(s, out, in, wt, bias, p, ut); break; //  64 x  64
+  }
 }
 
 template <int WA, int WB, int NWA, int NWB, bool UT>
@@ -678,12 +746,46 @@ int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const flo
   return MCN_SUCCESS;
 }
 
+// Tile shape of the tiled kernel (channels x pixels per workgroup) and how many ways the reduction is split.
+struct PixPlan {
+  int shape;   // 1: 128x128  2: 64x256  3: 32x256  4: 64x128  5: 128x64  6: 64x64  7: 128x32
+  int splits;
+};
+
+PixPlan plan_pix(int Cout, long long M, int R, bool dense) {
+  PixPlan plan;
+  const int BA = pick_channels_tile(Cout);
+  const long long tilesA = (Cout + BA - 1) / BA;
+  auto blocks = [&](int px) { return ((M + px - 1) / px) * tilesA; };
+  // the widest pixel tile that still yields >= 2048 workgroups (8 per CU), because short reduction loops hide
+  // their load latency only through occupancy
+  int px;
+  if (BA == 128) { plan.shape = M <= 32 ? 7 : (blocks(128) >= 2048 ? 1 : 5); px = plan.shape == 7 ? 32 : (plan.shape == 1 ? 128 : 64); }
+  else if (BA == 64) { plan.shape = blocks(256) >= 2048 ? 2 : (blocks(128) >= 2048 ? 4 : 6); px = plan.shape == 2 ? 256 : (plan.shape == 4 ? 128 : 64); }
+  else { plan.shape = 3; px = 256; }
+  // few workgroups with a long reduction each: split it, down to 8 steps of 16 rows per workgroup, until about two
+  // workgroups per CU exist
+  plan.splits = 1;
+  const long long nb = blocks(px);
+  const int nSteps = (R + 15) / 16;
+  if (dense && nb <= 128 && nSteps >= 32 && !tunable("conv_no_split", 0)) {
+    long long want = (512 + nb - 1) / nb;
+    plan.splits = (int)std::max<long long>(1, std::min<long long>(want, nSteps / 8));
+  }
+  return plan;
+}
+
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
 int run_pix(hipStream_t s, const char* who, float* out, const float* in, const float* f, const float* bias, PixP p,
             const TapSet& taps, int backward, void* ws, size_t wsBytes) {
   const int BA = pick_channels_tile(p.Cout);
   const int rPad = (p.R + 15) / 16 * 16;
   p.coutPad = (p.Cout + BA - 1) / BA * BA;
-  const size_t need = (size_t)rPad * p.coutPad * sizeof(float);
+  const PixPlan plan = plan_pix(p.Cout, p.M, p.R, p.dense != 0 && p.outImg == p.Cout * p.outPlane);
+  const size_t nOut = (size_t)p.N * p.Cout * p.OH * p.OW;
+  const size_t needW = (size_t)rPad * p.coutPad * sizeof(float);
+  const size_t need = plan.splits > 1 ? align256(needW) + (size_t)plan.splits * nOut * sizeof(float) : needW;
   if (!ws || wsBytes < need) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small (%zu < %zu bytes)", who, wsBytes, need);
   if (!aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
   float* wt = (float*)ws;
@@ -709,57 +811,65 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   p.byT = FastDiv(p.T);
   p.advC = 16 / p.T;
   p.advT = 16 % p.T;
+  p.rSplits = 1;
+  p.stepsPerSplit = 0;
+  p.partStride = 0;
   // small filter banks: keep all the weights in LDS and stream the pixels past them (conv_ws.hip)
   if (ut) {
     int handled = 0;
     rc = conv_ws_launch(s, who, out, in, wt, bias, p, &handled);
     if (rc || handled) return rc;
   }
-  // Tile shape, channels x pixels per workgroup: the widest pixel tile that still yields >= 2048 workgroups
-  // (8 per CU), because short reduction loops hide their load latency only through occupancy.  The tunable
-  // forces a shape for experiments.
-  int shape = tunable("conv_pix_tile", 0);
-  if (shape == 0) {
-    const long long tilesA = p.coutPad / BA;
-    auto blocks = [&](int px) { return (((long long)p.M + px - 1) / px) * tilesA; };
-    if (BA == 128) shape = blocks(128) >= 2048 ? 1 : 5;
-    else if (BA == 64) shape = blocks(256) >= 2048 ? 2 : (blocks(128) >= 2048 ? 4 : 6);
-    else shape = 3;
+  if (plan.splits > 1) {
+    // every workgroup a slice of the reduction into its own partial tensor, then one pass to add them up
+    float* partials = (float*)((char*)ws + align256(needW));
+    PixP q = p;
+    const int nSteps = rPad / 16;
+    q.stepsPerSplit = (nSteps + plan.splits - 1) / plan.splits;
+    q.rSplits = (nSteps + q.stepsPerSplit - 1) / q.stepsPerSplit;
+    q.partStride = (long long)nOut;
+    q.alpha = 1.f;
+    q.beta = 0.f;
+    {
+      const long long ob = (long long)nOut * 4;
+      q.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
+    }
+    launch_shape(s, plan.shape, partials, in, wt, nullptr, q, ut);
+    if ((rc = check_launch(who))) return rc;
+    KernelTimer timer("conv_pix_reduce", s);
+    hipLaunchKernelGGL(conv_pix_reduce, dim3((unsigned)((nOut + 255) / 256)), dim3(256), 0, s, out, partials, bias, nOut,
+                       q.partStride, q.rSplits, p.alpha, p.beta, p.OH * p.OW, p.Cout);
+    return check_launch(who);
   }
-  if ((shape == 1 || shape == 5) && BA != 128) shape = BA == 64 ? 2 : 3;
-  if ((shape == 2 || shape == 4 || shape == 6) && BA != 64) shape = BA == 128 ? 1 : 3;
-  if (shape == 3 && BA != 32) shape = BA == 128 ? 1 : 2;
-  switch (shape) {
-    case 1: launch_pix<2, 2, 2, 2>(s, out, in, wt, bias, p, ut); break;  // 128 x 128
-    case 2: launch_pix<2, 2, 1, 4>(s, out, in, wt, bias, p, ut); break;  //  64 x 256
-    case 3: launch_pix<1, 2, 1, 4>(s, out, in, wt, bias, p, ut); break;  //  32 x 256
-    case 4: launch_pix<1, 2, 2, 2>(s, out, in, wt, bias, p, ut); break;  //  64 x 128
-    case 5: launch_pix<2, 1, 2, 2>(s, out, in, wt, bias, p, ut); break;  // 128 x  64
-    default: launch_pix<1, 1, 2, 2>(s, out, in, wt, bias, p, ut); break; //  64 x  64
-  }
+  launch_shape(s, plan.shape, out, in, wt, bias, p, ut);
   return check_launch(who);
 }
 
 }  // namespace
 
-bool conv_mfma_forward_supported(const ConvP& p) { return common_ok(p); }
-bool conv_mfma_backward_data_supported(const ConvP& p) { return common_ok(p); }
-bool conv_mfma_backward_filter_supported(const ConvP& p) { return common_ok(p); }
+bool conv_mfma_forward_supported(const ConvP& p) { return common_ok(fc_view(p)); }
+bool conv_mfma_backward_data_supported(const ConvP& p) { return common_ok(fc_view(p)); }
+bool conv_mfma_backward_filter_supported(const ConvP& p) { return common_ok(fc_view(p)); }
 
-size_t conv_mfma_workspace_bytes(const ConvP& layer, int product) {
+size_t conv_mfma_workspace_bytes(const ConvP& original, int product) {
+  const ConvP layer = fc_view(original);
   const ConvP p = group_view(layer);  // the groups run one after the other through the same workspace
   const size_t FV = (size_t)p.FH * p.FW * p.FC;
+  // packed bank, plus the partial results when the tiled kernel splits the reduction (plan_pix)
+  auto pix_need = [&](int Cout, long long M, int R, bool dense) {
+    const int BA = pick_channels_tile(Cout);
+    const size_t needW = ((size_t)(R + 15) / 16 * 16) * (size_t)((Cout + BA - 1) / BA * BA) * sizeof(float);
+    const PixPlan plan = plan_pix(Cout, M, R, dense);
+    return plan.splits > 1 ? align256(needW) + (size_t)plan.splits * (size_t)M * Cout * sizeof(float) : needW;
+  };
   switch (product) {
     case MCN_CONV_FORWARD: {
       if (!conv_mfma_forward_supported(layer)) return 0;
-      const int BA = pick_channels_tile(p.K);
-      return ((FV + 15) / 16 * 16) * (size_t)((p.K + BA - 1) / BA * BA) * sizeof(float);
+      return pix_need(p.K, (long long)p.outH * p.outW * p.N, (int)FV, layer.groups == 1);
     }
     case MCN_CONV_BACKWARD_DATA: {
       if (!conv_mfma_backward_data_supported(layer)) return 0;
-      const int BA = pick_channels_tile(p.C);
-      const size_t R = (size_t)p.FH * p.FW * p.K;
-      return ((R + 15) / 16 * 16) * (size_t)((p.C + BA - 1) / BA * BA) * sizeof(float);
+      return pix_need(p.C, (long long)p.H * p.W * p.N, p.FH * p.FW * p.K, layer.groups == 1 && p.sy == 1 && p.sx == 1);
     }
     case MCN_CONV_BACKWARD_FILTER: {
       if (!conv_mfma_backward_filter_supported(layer)) return 0;
@@ -812,8 +922,9 @@ int forward_group(hipStream_t s, const ConvP& p, Wide wd, float* y, float outMul
 }
 }  // namespace
 
-int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
+int conv_forward_mfma(hipStream_t s, const ConvP& original, float* y, float outMult, const float* x, float inMult,
                       const float* f, const float* b, void* ws, size_t wsBytes) {
+  const ConvP p = fc_view(original);
   const ConvP g = group_view(p);
   const Wide wd = wide_of(p);
   const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
@@ -892,8 +1003,9 @@ int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float
 }
 }  // namespace
 
-int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
+int conv_backward_data_mfma(hipStream_t s, const ConvP& original, float* dx, float dxMult, const float* f, const float* dy,
                             void* ws, size_t wsBytes) {
+  const ConvP p = fc_view(original);
   // stride classes no tap reaches get no launch: they are zeros (or keep what is there, when accumulating)
   bool anyEmpty = false;
   for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
@@ -975,8 +1087,9 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
 }
 }  // namespace
 
-int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,
+int conv_backward_filter_mfma(hipStream_t s, const ConvP& original, float* df, const float* x, const float* dy, void* ws,
                               size_t wsBytes) {
+  const ConvP p = fc_view(original);
   const ConvP g = group_view(p);
   const Wide wd = wide_of(p);
   const bool ut = wgrad_uniform_tap(p);

@@ -32,6 +32,9 @@ CASES = [
     (14, 14, 64, 2, 3, 3, 32, 64, 1, 1, 1),                  # 2 groups of 32 channels: tap-major kernels per group
     (15, 14, 64, 2, 3, 3, 16, 96, (2, 2), 1, 1),             # 4 groups, strided: stride classes inside every group
     (12, 12, 96, 2, 1, 1, 32, 48, 2, 0, 1),                  # 3 groups, 1x1 stride 2
+    (6, 6, 32, 8, 6, 6, 32, 200, 1, 0, 1),                   # fully connected, 1152 rows: forward splits the reduction
+    (4, 4, 16, 4, 4, 4, 16, 640, 1, 0, 1),                   # fully connected, 640 filters: backward-data splits it
+    (13, 13, 2, 3, 13, 13, 2, 5, 1, 0, 1),                   # fully connected with 169 taps: only the 1x1 view fits the MFMA kernels
 ]
 
 
@@ -318,3 +321,27 @@ def test_groups_and_strides_run_on_the_mfma_kernels(capi, ob):
     launches, _ = capi.profile_end()
     # 4 groups: forward 4, backward-filter 4, backward-data 4 groups x 4 stride classes
     assert launches == 4 + 4 + 16
+
+
+def test_fully_connected_split_reduction(capi, ob):
+    """A filter bank that covers the whole input runs as a 1x1 layer over H*W*C channels with the reduction split
+    over workgroups; y = outMult*y + inMult*conv + bias through the pass that adds the partial results."""
+    r = np.random.default_rng(31)
+    xs, fs = (6, 6, 32, 8), (6, 6, 32, 200)
+    x = F(r.standard_normal(xs))
+    f = F(r.standard_normal(fs) * 0.05)
+    b = r.standard_normal(fs[3]).astype(np.float32)
+    g = ob.conv_geom(xs, fs, 1, 0, 1)
+    cg = capi.conv_geom(xs, fs, 1, 0, 1)
+    base = F(r.standard_normal(capi.conv_out_shape(cg)))
+    capi.profile_begin("conv_pix_reduce")
+    y = capi.conv_forward(capi.to_device(x), capi.to_device(f), capi.to_device(b), cg, y=capi.to_device(base), out_mult=0.5, in_mult=2.0)
+    launches, _ = capi.profile_end()
+    assert launches == 1
+    assert rel_max(capi.to_host(y), ob.conv_forward(x, f, b, g, y=base.copy(order="F"), out_mult=0.5, in_mult=2.0)) < 2e-4
+    capi.set_tunable("conv_no_split", 1)
+    try:
+        y1 = capi.conv_forward(capi.to_device(x), capi.to_device(f), capi.to_device(b), cg)
+    finally:
+        capi.set_tunable("conv_no_split", 0)
+    assert rel_max(capi.to_host(y1), ob.conv_forward(x, f, b, g)) < 2e-4
