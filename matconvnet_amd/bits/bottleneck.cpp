@@ -10,7 +10,9 @@
 namespace vl { namespace harness {
 
 Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon)
-    : H(H), W(W), C(C), M(M), N(N), epsilon(epsilon), error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false) {
+    : H(H), W(W), C(C), M(M), N(N), epsilon(epsilon), error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false),
+      overlap(false), sideStream(NULL) {
+  for (int i = 0; i < 4; ++i) events[i] = NULL;
   const TensorShape big(H, W, C, N), small(H, W, M, N);
   // inputs and parameters
   make("x", big); make("dzdy", big);
@@ -32,7 +34,38 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon)
   make("dg3", TensorShape(C, 1, 1, 1)); make("db3", TensorShape(C, 1, 1, 1));
 }
 
+ErrorCode Bottleneck::setOverlap(bool on) {
+  if (on && !sideStream) {
+    hipStream_t st = NULL;
+    if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) {
+      (void)hipGetLastError();
+      message = "cannot create the second stream";
+      return error = VLE_Cuda;
+    }
+    sideStream = st;
+    for (int i = 0; i < 4; ++i) {
+      hipEvent_t e = NULL;
+      if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError();
+        message = "cannot create an event";
+        return error = VLE_Cuda;
+      }
+      events[i] = e;
+    }
+    sideContext.getHipHelper().setStream(sideStream);
+  }
+  overlap = on;
+  return VLE_Success;
+}
+
 Bottleneck::~Bottleneck() {
+  if (sideStream) {
+    (void)hipStreamSynchronize((hipStream_t)sideStream);
+    sideContext.clear();
+    for (int i = 0; i < 4; ++i)
+      if (events[i]) (void)hipEventDestroy((hipEvent_t)events[i]);
+    (void)hipStreamDestroy((hipStream_t)sideStream);
+  }
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
 }
@@ -146,7 +179,31 @@ ErrorCode Bottleneck::backward() {
   char const* dsName = fused ? "dzdx" : "ds";
   ABI("relu3_bwd", mcn_relu_backward(st, buffer(dsName), buffer(mask3), buffer("dzdy"), nBig));
   STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot(dsName)));
-  STEP("conv3_bwd", c1.backward(slot("dr2"), slot("df3"), none, slot("r2"), slot("f3"), slot("da3")));
+  // A convolution's backward: the input gradient on the caller's stream; the filter gradient beside it on the
+  // second stream when overlapping (enqueued after it, so the persistent input-gradient kernel takes its CUs
+  // first and the filter-gradient workgroups fill in beside and behind it).
+  nn::Convolution c1s(sideContext, 1, 1, 0, 0, 0, 0, 1, 1), c2s(sideContext, 1, 1, 1, 1, 1, 1, 1, 1);
+  Tensor none2, none3;
+  auto convBackward = [&](nn::Convolution& onMain, nn::Convolution& onSide, int k, Tensor& derIn, double derInMult,
+                          Tensor& derFilter, Tensor const& in, Tensor const& filter, Tensor const& derOut) -> ErrorCode {
+    if (!overlap) return onMain.backwardAccumulate(derIn, derInMult, derFilter, none, in, filter, derOut);
+    if (hipEventRecord((hipEvent_t)events[k], (hipStream_t)st) != hipSuccess ||
+        hipStreamWaitEvent((hipStream_t)sideStream, (hipEvent_t)events[k], 0) != hipSuccess)
+      return context.setError(VLE_Cuda, "cannot order the second stream");
+    ErrorCode e = onMain.backwardAccumulate(derIn, derInMult, none2, none, in, filter, derOut);
+    if (e != VLE_Success) return e;
+    e = onSide.backwardAccumulate(none3, 0, derFilter, none, in, filter, derOut);
+    if (e != VLE_Success) context.setError(e, sideContext.getLastErrorMessage().c_str());
+    return e;
+  };
+  auto joinSide = [&]() -> ErrorCode {
+    if (!overlap) return VLE_Success;
+    if (hipEventRecord((hipEvent_t)events[3], (hipStream_t)sideStream) != hipSuccess ||
+        hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)events[3], 0) != hipSuccess)
+      return context.setError(VLE_Cuda, "cannot join the second stream");
+    return VLE_Success;
+  };
+  STEP("conv3_bwd", convBackward(c1, c1s, 0, slot("dr2"), 0, slot("df3"), slot("r2"), slot("f3"), slot("da3")));
   const size_t wsSmall = mcn_bnorm_workspace_bytes(H, W, M, N);
   void* wsBn = NULL;
   if (fused) {
@@ -160,7 +217,7 @@ ErrorCode Bottleneck::backward() {
     ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer(mask2), buffer("dr2"), nSmall));
     STEP("bn2_bwd", bn.backwardWithMoment(slot("da2"), slot("dg2"), slot("db2"), slot("m2"), slot("a2"), slot("g2"), slot("b2"), slot("dn2")));
   }
-  STEP("conv2_bwd", c2.backward(slot("dr1"), slot("df2"), none, slot("r1"), slot("f2"), slot("da2")));
+  STEP("conv2_bwd", convBackward(c2, c2s, 1, slot("dr1"), 0, slot("df2"), slot("r1"), slot("f2"), slot("da2")));
   if (fused) {
     wsBn = context.getWorkspace(VLDT_GPU, wsSmall);  // (the convolution in between may have grown the workspace)
     if (!wsBn) return fail(context.getLastError(), "workspace");
@@ -171,11 +228,13 @@ ErrorCode Bottleneck::backward() {
     STEP("bn1_bwd", bn.backwardWithMoment(slot("da1"), slot("dg1"), slot("db1"), slot("m1"), slot("a1"), slot("g1"), slot("b1"), slot("dn1")));
   }
   if (fused) {
-    STEP("conv1_bwd", c1.backwardAccumulate(slot("dzdx"), 1, slot("df1"), none, slot("x"), slot("f1"), slot("da1")));
+    STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dzdx"), 1, slot("df1"), slot("x"), slot("f1"), slot("da1")));
+    STEP("join", joinSide());
     return VLE_Success;
   }
-  STEP("conv1_bwd", c1.backward(slot("dxm"), slot("df1"), none, slot("x"), slot("f1"), slot("da1")));
+  STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dxm"), 0, slot("df1"), slot("x"), slot("f1"), slot("da1")));
   ABI("sum_bwd", mcn_add(st, buffer("dzdx"), buffer("dxm"), buffer("ds"), nBig));
+  STEP("join", joinSide());
   return VLE_Success;
 }
 

@@ -31,6 +31,11 @@ class Bottleneck {
   // pass (mcn_bnorm_forward_fused); the un-activated tensors n1, n2, n3, s are then never written and the
   // ReLU derivatives take their masks from r1, r2, y.  Results are bit-identical to the layer-by-layer mode.
   void setFused(bool on) { fused = on; }
+  // overlap = true: in the backward pass each convolution's filter gradient runs on a second stream (with a
+  // context and workspace of its own) beside the same layer's input gradient, which is all the following layers
+  // wait for; the second stream is joined before backward() returns its work to the caller's stream.  Results are
+  // the same bits; only the schedule changes.
+  ErrorCode setOverlap(bool on);
   ErrorCode forward();
   ErrorCode backward();
 
@@ -54,6 +59,10 @@ class Bottleneck {
   StageHook stageHook;
   void* hookUser;
   bool fused;
+  bool overlap;
+  Context sideContext;
+  void* sideStream;     // hipStream_t
+  void* events[4];      // hipEvent_t: "derivative ready" for the three convolutions, "second stream done"
 };
 
 } }  // namespace vl::harness

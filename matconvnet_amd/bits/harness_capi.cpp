@@ -174,6 +174,8 @@ int vlh_bottleneck_set_stream(void* block, void* stream) {
 
 void vlh_bottleneck_set_fused(void* block, int fused) { ((BlockHandle*)block)->block->setFused(fused != 0); }
 
+int vlh_bottleneck_set_overlap(void* block, int overlap) { return (int)((BlockHandle*)block)->block->setOverlap(overlap != 0); }
+
 int vlh_bottleneck_forward(void* block) { return (int)((BlockHandle*)block)->block->forward(); }
 int vlh_bottleneck_backward(void* block) { return (int)((BlockHandle*)block)->block->backward(); }
 const char* vlh_bottleneck_message(void* block) { return ((BlockHandle*)block)->block->lastMessage().c_str(); }

@@ -44,6 +44,9 @@ VLH_API float* vlh_bottleneck_buffer(void* block, const char* name, size_t* coun
 VLH_API int vlh_bottleneck_set_stream(void* block, void* stream);
 /* fused != 0: batch-norm forward also applies the ReLU / shortcut sum that follows it (same bits, fewer passes) */
 VLH_API void vlh_bottleneck_set_fused(void* block, int fused);
+/* overlap != 0: backward runs each convolution's filter gradient on a second stream beside its input gradient
+   (same bits; the second stream is joined before vlh_bottleneck_backward's work is complete on the block's stream) */
+VLH_API int vlh_bottleneck_set_overlap(void* block, int overlap);
 VLH_API int vlh_bottleneck_forward(void* block);
 VLH_API int vlh_bottleneck_backward(void* block);
 /* runs `steps` forward+backward passes; if stage != NULL the launches of that stage are bracketed by HIP

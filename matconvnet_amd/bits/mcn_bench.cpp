@@ -187,10 +187,11 @@ static void benchCopy(int warmup, int iters) {
               "copy 256 MiB", t * 1e3, 2.0 * n * 4 / t / 1e6, 100 * 2.0 * n * 4 / (t * 1e-3) / kPeakHbm, n * 4, n * 4, gRotate);
 }
 
-static void benchBlock(int warmup, int iters, bool fused) {
+static void benchBlock(int warmup, int iters, bool fused, bool overlap = false) {
   const int H = 56, W = 56, C = 256, M = 64, N = 32;
   harness::Bottleneck block(H, W, C, M, N, 1e-5);
   block.setFused(fused);
+  if (overlap) block.setOverlap(true);
   if (!block.ok()) {
     std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
     std::exit(3);
@@ -218,7 +219,7 @@ static void benchBlock(int warmup, int iters, bool fused) {
     }
   }, warmup, iters);
   std::printf("%-28s %8.3f ms/step %9.0f images/s (fwd+bwd, N = %d, 41.93 GFLOP of convolution per step; %s)\n",
-              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, fused ? "relu/sum folded into bnorm" : "layer by layer");
+              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, overlap ? "folded, filter gradients on a second stream" : (fused ? "relu/sum folded into bnorm" : "layer by layer"));
 }
 
 int main(int argc, char** argv) {
@@ -246,6 +247,7 @@ int main(int argc, char** argv) {
   if (want("block")) {
     benchBlock(warmup, iters, false);
     benchBlock(warmup, iters, true);
+    benchBlock(warmup, iters, true, true);
   }
   if (want("conv5")) benchConv("conv 3x3x256x256 56x56 N=64", 56, 56, 256, 64, 3, 256, 1, warmup, iters);
   return 0;

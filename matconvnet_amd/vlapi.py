@@ -58,6 +58,7 @@ def lib():
         L.vlh_bottleneck_set_stream.argtypes = [C.c_void_p, C.c_void_p]
         L.vlh_bottleneck_set_fused.argtypes = [C.c_void_p, C.c_int]
         L.vlh_bottleneck_set_fused.restype = None
+        L.vlh_bottleneck_set_overlap.argtypes = [C.c_void_p, C.c_int]
         L.vlh_bottleneck_forward.argtypes = [C.c_void_p]
         L.vlh_bottleneck_backward.argtypes = [C.c_void_p]
         L.vlh_bottleneck_run.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.POINTER(C.c_float)]
@@ -178,13 +179,15 @@ def vl_taccum(*args):
 class Bottleneck:
     """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
 
-    def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False):
+    def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False, overlap=False):
         self.L = lib()
         self.shape = (H, W, Cc, M, N)
         self.h = self.L.vlh_bottleneck_create(H, W, Cc, M, N, eps)
         torch = _torch()
         self.L.vlh_bottleneck_set_stream(self.h, C.c_void_p(torch.cuda.current_stream().cuda_stream))
         self.L.vlh_bottleneck_set_fused(self.h, int(fused))
+        if overlap and self.L.vlh_bottleneck_set_overlap(self.h, 1) != 0:
+            raise VlError(2, self.L.vlh_bottleneck_message(self.h).decode())
 
     def close(self):
         if self.h:

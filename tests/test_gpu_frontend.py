@@ -263,17 +263,19 @@ def test_bottleneck_fused_mode_is_bit_identical(vl, ob):
     outs = {}
     shapes = dict(y=w["x"].shape, dzdx=w["x"].shape, df1=w["f1"].shape, df2=w["f2"].shape, df3=w["f3"].shape,
                   dg1=(64,), db1=(64,), dg2=(64,), db2=(64,), dg3=(256,), db3=(256,), m1=(64, 2), m3=(256, 2))
-    for fused in (False, True):
-        blk = vl.Bottleneck(N=4, eps=w["eps"], fused=fused)
+    for fused in (False, True, "overlap"):
+        blk = vl.Bottleneck(N=4, eps=w["eps"], fused=bool(fused), overlap=(fused == "overlap"))
         try:
             _load(blk, w)
-            blk.forward()
-            blk.backward()
+            for _ in range(3 if fused == "overlap" else 1):  # (several steps: the second stream must be joined each time)
+                blk.forward()
+                blk.backward()
             outs[fused] = {k: blk.get(k, v) for k, v in shapes.items()}
         finally:
             blk.close()
     for k in shapes:
         assert bits_equal(outs[False][k], outs[True][k]), k
+        assert bits_equal(outs[False][k], outs["overlap"][k]), k  # filter gradients on a second stream: same bits
 
 
 def test_bnorm_forward_fused_matches_separate_calls(capi, ob):
