@@ -345,3 +345,35 @@ def test_fully_connected_split_reduction(capi, ob):
     finally:
         capi.set_tunable("conv_no_split", 0)
     assert rel_max(capi.to_host(y1), ob.conv_forward(x, f, b, g)) < 2e-4
+
+
+def _random_case(r):
+    """A valid layer geometry: groups, strides, dilation, asymmetric padding, channel counts on both sides of the
+    kernels' 16 / 32-channel thresholds, sometimes a filter that covers the whole input."""
+    groups = int(r.choice([1, 1, 2, 4]))
+    FC = int(r.choice([1, 3, 8, 16, 32]))
+    Kg = int(r.choice([1, 5, 16, 32, 40]))
+    FH, FW = int(r.integers(1, 6)), int(r.integers(1, 6))
+    dil = (int(r.integers(1, 3)), int(r.integers(1, 3)))
+    stride = (int(r.integers(1, 4)), int(r.integers(1, 4)))
+    pad = tuple(int(v) for v in r.integers(0, 3, size=4))
+    eh, ew = (FH - 1) * dil[0] + 1, (FW - 1) * dil[1] + 1
+    H = max(1, eh - pad[0] - pad[1]) + int(r.integers(0, 12))
+    W = max(1, ew - pad[2] - pad[3]) + int(r.integers(0, 12))
+    if r.random() < 0.15:  # fully connected
+        FH, FW, dil, pad = H, W, (1, 1), (0, 0, 0, 0)
+    return (H, W, FC * groups, int(r.integers(1, 5)), FH, FW, FC, Kg * groups, stride, pad, dil)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_geometries_vs_oracle(capi, ob, seed):
+    """Forward and all three derivatives on seeded random geometries (whatever kernel the dispatch picks)."""
+    r = np.random.default_rng(1000 + seed)
+    case = _random_case(r)
+    x, f, b = _tensors(case, seed=seed)
+    og = ob.conv_geom(x.shape, f.shape, *case[8:])
+    cg = capi.conv_geom(x.shape, f.shape, *case[8:])
+    y = capi.to_host(capi.conv_forward(capi.to_device(x), capi.to_device(f), capi.to_device(b), cg))
+    assert rel_max(y, ob.conv_forward(x, f, b, og)) <= TOL, case
+    dy = F(r.standard_normal(ob.conv_out_shape(og)))
+    _check(capi, ob, x, f, b, dy, *case[8:])
