@@ -79,10 +79,12 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
     conv_flops = {"conv_wgrad_mfma": 2.0 * P * N * (256 * 64 + 9 * 64 * 64 + 64 * 256)}
     eS, eB = 4.0 * P * 64 * N, 4.0 * P * 256 * N
     hbm_bytes = {  # algorithmic bytes per step of the memory-bound families (reads + writes once each)
-        "bnorm_sums": (eS + eS + eB) + 2 * (eS + eS + eB),       # forward reads x; backward reads x and dzdy
+        # forward reads x; backward reads x and dzdy; bn3's backward also reads the block output (mask) and writes
+        # the masked derivative
+        "bnorm_sums": (eS + eS + eB) + 2 * (eS + eS + eB) + 2 * eB,
         "bnorm_forward_apply": 2 * eS + 2 * eS + 3 * eB,          # bn1, bn2 with ReLU; bn3 with shortcut sum and ReLU
         "bnorm_backward_apply": 3 * (eS + eS + eB),
-        "eltwise_kernel": 3 * eB + 3 * eS + 3 * eS + 3 * eB,      # three ReLU derivatives, one fan-out sum
+        "eltwise_kernel": 0.0,                                    # (nothing left: every element-wise layer is folded)
     }
     fam = {}
     for name in ["conv_ws_mfma", "conv_pix_mfma"] + list(conv_flops) + list(hbm_bytes) + ["conv_wgrad_reduce", "conv_pack_weights"]:

@@ -198,6 +198,18 @@ MCN_API int mcn_bnorm_backward_relu(mcn_stream_t stream, float* derInput, float*
                                     const float* biases, const float* derOutput, int H, int W, int C, int N,
                                     double epsilon, void* workspace, size_t workspaceBytes);
 
+/* Batch-norm derivative (given moments) whose incoming derivative first passes the derivative of a ReLU that sits
+   later in the network, behind other layers (in a residual block: behind the shortcut sum), so that the mask cannot
+   be recomputed from x: maskedDerOutput = derOutput where maskSource > 0, else derOutput*0 (maskSource: that ReLU's
+   output or input; as mcn_relu_backward), written out because the other consumers of that ReLU's derivative need it
+   too, and summed in the same pass over the data.  Bit-identical to mcn_relu_backward followed by
+   mcn_bnorm_backward with givenMoments != 0; one sweep of the tensor less.  No counterpart in the reference. */
+MCN_API int mcn_bnorm_backward_masked(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
+                                      const float* moments, const float* x, const float* multipliers,
+                                      const float* derOutput, const float* maskSource, float* maskedDerOutput,
+                                      int H, int W, int C, int N, double epsilon, void* workspace,
+                                      size_t workspaceBytes);
+
 /* dzdx (H x W x C x N), dzdg (C), dzdb (C), all fully overwritten.  givenMoments == 0: BatchNorm::backward
    (bits/nnbnorm.cu:307-365), moments written if non-NULL.  givenMoments != 0: backwardWithMoment (:263-305). */
 MCN_API int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers,

@@ -177,8 +177,19 @@ ErrorCode Bottleneck::backward() {
   // the sum passes ds to both of its inputs: the branch (n3) and the shortcut (x).  Fused mode keeps ds in the
   // output buffer and lets the first convolution add its derivative to it.
   char const* dsName = fused ? "dzdx" : "ds";
-  ABI("relu3_bwd", mcn_relu_backward(st, buffer(dsName), buffer(mask3), buffer("dzdy"), nBig));
-  STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot(dsName)));
+  if (fused) {
+    // the block's last ReLU sits behind the shortcut sum: its derivative is taken and written (for the shortcut
+    // branch) in the summing pass of the batch-norm derivative
+    const size_t wsBig = mcn_bnorm_workspace_bytes(H, W, C, N);
+    void* wsB = context.getWorkspace(VLDT_GPU, wsBig);
+    if (!wsB) return fail(context.getLastError(), "workspace");
+    ABI("bn3_bwd", mcn_bnorm_backward_masked(st, buffer("da3"), buffer("dg3"), buffer("db3"), buffer("m3"), buffer("a3"),
+                                             buffer("g3"), buffer("dzdy"), buffer(mask3), buffer(dsName), H, W, C, N, epsilon,
+                                             wsB, wsBig));
+  } else {
+    ABI("relu3_bwd", mcn_relu_backward(st, buffer(dsName), buffer(mask3), buffer("dzdy"), nBig));
+    STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot(dsName)));
+  }
   // A convolution's backward: the input gradient on the caller's stream; the filter gradient beside it on the
   // second stream when overlapping (enqueued after it, so the persistent input-gradient kernel takes its CUs
   // first and the filter-gradient workgroups fill in beside and behind it).

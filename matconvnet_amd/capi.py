@@ -62,6 +62,7 @@ PROTOTYPES = {
     "mcn_bnorm_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_bnorm_forward_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_bnorm_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
+    "mcn_bnorm_backward_masked": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _vp, _sz]),
     "mcn_bnorm_backward_relu": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _vp, _sz]),
     "mcn_pool_output_size": (_i, [C.POINTER(PoolGeom), C.POINTER(_i), C.POINTER(_i)]),
     "mcn_pool_forward": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp]),
@@ -308,6 +309,18 @@ def bnorm_backward_relu(x, g, b, dy, moments, eps=1e-4, ws=None):
     check(lib().mcn_bnorm_backward_relu(stream(), ptr(dx), ptr(dg), ptr(db), ptr(moments), ptr(x), ptr(g), ptr(b),
                                         ptr(dy), H, W, Cc, N, eps, wp, wn))
     return dx, dg, db
+
+
+def bnorm_backward_masked(x, g, dy, mask_source, moments, eps=1e-4, ws=None):
+    """bnorm derivative of dy*[mask_source > 0]; also returns that masked derivative."""
+    ws = ws or _ws
+    H, W, Cc, N = _hwcn(x)
+    dx, masked = empty((H, W, Cc, N)), empty((H, W, Cc, N))
+    dg, db = empty((Cc,)), empty((Cc,))
+    wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
+    check(lib().mcn_bnorm_backward_masked(stream(), ptr(dx), ptr(dg), ptr(db), ptr(moments), ptr(x), ptr(g), ptr(dy),
+                                          ptr(mask_source), ptr(masked), H, W, Cc, N, eps, wp, wn))
+    return dx, dg, db, masked
 
 
 def pool_forward(x, g):

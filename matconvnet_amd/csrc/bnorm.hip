@@ -67,14 +67,20 @@ __device__ __forceinline__ void block_sum(double (&v)[NV], double* lds /* [4][NV
 // MODE 2: all four                     (backward, moments from the batch)
 // RELU (MODE 1 only): dy is the derivative after a ReLU that followed this layer; it counts only where the
 // layer's output a*x + k was positive (a, k: the forward pass's own coefficients, see forward_coefficients).
-template <int MODE, bool VEC4, bool RELU = false>
+// YMASK (MODE 1 only): dy first passes the derivative of a ReLU whose *output* is ymask (dy counts where
+// ymask > 0, else dy*0 like mcn_relu_backward), and the masked derivative is also written to `masked` for the
+// passes that follow (this layer's apply pass, and whoever else consumes it).
+template <int MODE, bool VEC4, bool RELU = false, bool YMASK = false>
 __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
                                                   const float* __restrict__ dy,
                                                   double* __restrict__ partials, BnormP p,
                                                   const float* __restrict__ moments = nullptr,
                                                   const float* __restrict__ mult = nullptr,
-                                                  const float* __restrict__ bias = nullptr) {
+                                                  const float* __restrict__ bias = nullptr,
+                                                  const float* __restrict__ ymask = nullptr,
+                                                  float* __restrict__ masked = nullptr) {
   static_assert(!RELU || MODE == 1, "the ReLU mask needs the moments of the forward pass");
+  static_assert(!YMASK || (MODE == 1 && !RELU), "one kind of mask at a time, with given moments");
   __shared__ double lds[16];
   const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int c = logical / p.groups;
@@ -100,6 +106,12 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
         if (MODE != 0) {
           float4 d = d4[i];
           if (RELU) d = make_float4(gate(a.x, d.x), gate(a.y, d.y), gate(a.z, d.z), gate(a.w, d.w));
+          if (YMASK) {
+            const float4 m = ((const float4*)(ymask + base))[i];
+            d = make_float4(m.x > 0.f ? d.x : d.x * 0.f, m.y > 0.f ? d.y : d.y * 0.f, m.z > 0.f ? d.z : d.z * 0.f,
+                            m.w > 0.f ? d.w : d.w * 0.f);
+            ((float4*)(masked + base))[i] = d;
+          }
           sxd += (a.x * d.x + a.y * d.y) + (a.z * d.z + a.w * d.w);
           sd += (d.x + d.y) + (d.z + d.w);
         }
@@ -112,7 +124,11 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
           sxx += a * a;
         }
         if (MODE != 0) {
-          const float d = gate(a, dy[base + i]);
+          float d = gate(a, dy[base + i]);
+          if (YMASK) {
+            d = ymask[base + i] > 0.f ? d : d * 0.f;
+            masked[base + i] = d;
+          }
           sxd += a * d;
           sd += d;
         }
@@ -444,6 +460,42 @@ int mcn_bnorm_backward_relu(mcn_stream_t stream, float* derInput, float* derMult
   if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, derOutput, partials, p, biases);
   else hipLaunchKernelGGL((bnorm_backward_apply<true, false, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, derOutput, partials, p, biases);
   return check_launch("mcn_bnorm_backward_relu");
+}
+
+int mcn_bnorm_backward_masked(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
+                              const float* moments, const float* x, const float* multipliers, const float* derOutput,
+                              const float* maskSource, float* maskedDerOutput, int H, int W, int C, int N,
+                              double epsilon, void* workspace, size_t workspaceBytes) {
+  BnormP p;
+  int rc = setup("mcn_bnorm_backward_masked", H, W, C, N, epsilon, &p);
+  if (rc) return rc;
+  if (C == 0) return MCN_SUCCESS;
+  if (!derMultipliers || !derBiases || !multipliers || !moments)
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_masked: null parameter tensor");
+  if ((size_t)p.WH * N == 0) {
+    if ((rc = mcn_fill(stream, derMultipliers, 0.f, (size_t)C))) return rc;
+    return mcn_fill(stream, derBiases, 0.f, (size_t)C);
+  }
+  if (!derInput || !x || !derOutput || !maskSource || !maskedDerOutput)
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_masked: null tensor");
+  if (!workspace || workspaceBytes < mcn_bnorm_workspace_bytes(H, W, C, N))
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_masked: workspace too small");
+  hipStream_t s = as_stream(stream);
+  const bool vec = (p.WH % 4 == 0) && aligned16(derInput) && aligned16(x) && aligned16(derOutput) && aligned16(maskSource) &&
+                   aligned16(maskedDerOutput);
+  const dim3 grid((unsigned)(C * p.groups)), block(256);
+  double* partials = (double*)workspace;
+  float* mom = const_cast<float*>(moments);  // (the kernels only write moments when they are not given)
+  {
+    KernelTimer timer("bnorm_sums", s);
+    if (vec) hipLaunchKernelGGL((bnorm_sums<1, true, false, true>), grid, block, 0, s, x, derOutput, partials, p, nullptr, nullptr, nullptr, maskSource, maskedDerOutput);
+    else hipLaunchKernelGGL((bnorm_sums<1, false, false, true>), grid, block, 0, s, x, derOutput, partials, p, nullptr, nullptr, nullptr, maskSource, maskedDerOutput);
+  }
+  if ((rc = check_launch("mcn_bnorm_backward_masked(sums)"))) return rc;
+  KernelTimer timer("bnorm_backward_apply", s);
+  if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, maskedDerOutput, partials, p);
+  else hipLaunchKernelGGL((bnorm_backward_apply<true, false>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, maskedDerOutput, partials, p);
+  return check_launch("mcn_bnorm_backward_masked");
 }
 
 int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases, float* moments,

@@ -312,3 +312,19 @@ def test_bnorm_backward_relu_matches_separate_calls(capi, ob):
     if flips == 0:
         assert rel_max(capi.to_host(got[0]), odx) < 1e-5
         assert rel_max(capi.to_host(got[1]).ravel(), odg) < 1e-5 and rel_max(capi.to_host(got[2]).ravel(), odb) < 1e-5
+
+
+def test_bnorm_backward_masked_matches_separate_calls(capi, ob):
+    """A later ReLU's derivative taken (and written out) inside batch-norm's summing pass: same bits as the two calls."""
+    w = workloads.bnorm_case(seed=12, H=14, W=18, C=8, N=5)
+    r = np.random.default_rng(13)
+    later = F(r.standard_normal(w["x"].shape))   # output of the later ReLU's layer: zeros, negatives, positives
+    later[::3] = 0.0
+    xd, gd, bd, dyd, ld = (capi.to_device(v) for v in (w["x"], w["g"], w["b"], w["dy"], later))
+    _, mom = capi.bnorm_forward(xd, gd, bd, 1e-4)
+    masked = capi.relu_backward(ld, dyd)
+    want = capi.bnorm_backward(xd, gd, masked, 1e-4, moments=mom)
+    got = capi.bnorm_backward_masked(xd, gd, dyd, ld, mom, 1e-4)
+    for a, b_ in zip(got[:3], want[:3]):
+        assert bits_equal(capi.to_host(a), capi.to_host(b_))
+    assert bits_equal(capi.to_host(got[3]), capi.to_host(masked))
