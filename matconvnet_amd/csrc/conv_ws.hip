@@ -98,7 +98,12 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   const int sib = w.chanBlocks <= wavesPerGroup ? w.chanBlocks : 1;  // siblings side by side (else one wave, all blocks in turn)
   const int slots = wavesPerGroup / sib;
   const int unitStep = (int)gridDim.x * slots * sib;
-  int unit = ((wave / sib) * (int)gridDim.x + (int)blockIdx.x) * sib + (wave % sib);
+  // (workgroup ids are dealt round-robin to the 8 XCDs; with taps, numbering them XCD by XCD puts neighbouring
+  // pixel blocks, whose taps reach into each other's columns, behind the same L2: the 3x3 layer of the block then
+  // fetches 30 MB per launch through the fabric instead of 128 MB.  Without taps nothing is shared and spreading
+  // neighbours over the XCDs measured 5% faster.)
+  const int wg = TAPS ? xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x) : (int)blockIdx.x;
+  int unit = ((wave / sib) * (int)gridDim.x + wg) * sib + (wave % sib);
   if (wave >= slots * sib || unit >= w.nUnits) return;
 
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, (int)w.inBytes, 0x00020000);
