@@ -32,7 +32,7 @@ PEAK_HBM = 8.0e12          # B/s
 # read for a 256 MiB streaming copy (FETCH_SIZE: 2 KiB per unit, WRITE_SIZE: 1 KiB per unit).  Counters are not
 # readable from inside this process, so these are the profiled values of exactly these launches.
 TRAFFIC = {
-    "block/conv_ws_mfma": 1.459e8,     # mean of the 6 launches of a step (profiles/bottleneck_block_56x56_N32_fwd_bwd.txt; operands 1.028e8)
+    "block/conv_ws_mfma": 1.161e8,     # mean of the 6 launches of a step (profiles/bottleneck_block_56x56_N32_fwd_bwd.txt; operands 1.028e8)
     "cfg5/conv_pix_mfma": 5.579e8,     # profiles/conv_vgg_3x3x256x256_N64_backward.txt (operands 4.13e8: dzdy in, dzdx out, bank)
     "cfg5/conv_wgrad_mfma": 9.06e8,    # (operands 4.13e8: x and dzdy are both re-read by the filter-volume tiles)
     "cfg2/bnorm_sums": 2.058e8,        # profiles/bnorm_56x56x256x32_backward.txt
