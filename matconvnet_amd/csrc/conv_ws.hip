@@ -48,8 +48,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
                                                         const float* __restrict__ wt, const float* __restrict__ bias,
                                                         PixP p, WsP w) {
   extern __shared__ float smem[];
-  float* wtL = smem;                               // [chanBlocks][R][32 WA]
-  int2* tapTab = (int2*)(smem + p.R * p.coutPad);  // [T] .x = dh + IH*dw, .y = (dh & 0xffff) | (dw << 16)
+  float* wtL = smem;  // [chanBlocks][R][32 WA]
   constexpr int ROW = 32 * WA;                     // floats per bank row of one channel block
 
   const int tid = threadIdx.x;
@@ -60,7 +59,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   const int l32 = lane & 31, kh = lane >> 5;
   const int IHW = p.IH * p.IW;
 
-  // ---- once per workgroup: the bank, re-laid by channel block, and the tap table
+  // ---- once per workgroup: the bank, re-laid by channel block
   {
     const int perBlock = p.R * (ROW / 4);  // 16-byte vectors per channel block
     const int n4 = perBlock * w.chanBlocks;
@@ -81,11 +80,6 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
 #pragma unroll
       for (int k = 0; k < 4; ++k)
         if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
-    }
-    if (TAPS && tid < p.T) {
-      const int j = tid / p.FH, i = tid - j * p.FH;
-      const int dh = p.dhBase + i * p.dhStep, dw = p.dwBase + j * p.dwStep;
-      tapTab[tid] = make_int2(dh + p.IH * dw, (int)((unsigned)(dh & 0xffff) | ((unsigned)dw << 16)));
     }
   }
   __syncthreads();
@@ -127,19 +121,20 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     int n, q, ow, oh;
     p.byQ.divmod(mvalid ? m : 0, &n, &q);
     p.byOH.divmod(q, &ow, &oh);
-    ihBN = oh * p.sy;
+    ihBN = mvalid ? oh * p.sy : -0x40000000;  // (an idle lane fails every "row inside the image" test)
     iwBN = ow * p.sx;
-    voffN = mvalid ? (unsigned)(n * p.inImg + ihBN + p.IH * iwBN + kh * IHW) * 4u : kOutside;
+    voffN = mvalid ? (unsigned)(n * p.inImg + oh * p.sy + p.IH * iwBN + kh * IHW) * 4u : kOutside;
   };
 
-  // per-lane offset of the pixels of tap `tap` (kOutside where the shifted pixel is not in the image)
-  auto tap_offset = [&](int tap) -> unsigned {
+  // The loader's tap, as scalars kept up to date by additions: row index inside the filter column and the tap's
+  // shift (dh, dw) of the gathered position.  (A table in LDS cost a read, two readfirstlanes and the wait for
+  // them in every group.)
+  int tapRow = 0, dhL = p.dhBase, dwL = p.dwBase;
+  // per-lane offset of the pixels at shift (dh, dw): kOutside where the shifted pixel is not in the image
+  auto tap_offset = [&](int dh, int dw) -> unsigned {
     if (!TAPS) return voff;
-    const int2 tp = tapTab[tap];
-    const int shift = __builtin_amdgcn_readfirstlane(tp.x), packed = __builtin_amdgcn_readfirstlane(tp.y);
-    const int ih = ihB + (int)(short)(packed & 0xffff), iw = iwB + (packed >> 16);
-    const bool ok = voff != kOutside && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
-    return ok ? voff + (unsigned)(shift * 4) : kOutside;
+    const bool ok = (unsigned)(ihB + dh) < (unsigned)p.IH && (unsigned)(iwB + dw) < (unsigned)p.IW;
+    return ok ? voff + (unsigned)((dh + p.IH * dw) * 4) : kOutside;
   };
 
   typedef float vbuf __attribute__((ext_vector_type(kDepth)));
@@ -153,8 +148,17 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     const int sbase_ = giL * (2 * kDepth) * planeBytes;                                                   \
     _Pragma("unroll") for (int d_ = 0; d_ < kDepth; ++d_) DST[d_] = __builtin_bit_cast(                   \
         float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voTap, sbase_ + 2 * d_ * planeBytes, 0));  \
+    if (TAPS) {                                                                                           \
+      dhL += p.dhStep;                                                                                    \
+      if (++tapRow == p.FH) {                                                                             \
+        tapRow = 0;                                                                                       \
+        dhL = p.dhBase;                                                                                   \
+        dwL += p.dwStep;                                                                                  \
+      }                                                                                                   \
+    }                                                                                                     \
     if (++tapL == p.T) {                                                                                  \
       tapL = 0;                                                                                           \
+      dwL = p.dwBase;                                                                                     \
       if (++giL == w.groupsPerTap) {                                                                      \
         giL = 0;                                                                                          \
         voff = voffN;                                                                                     \
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
         if (!TAPS) voTap = voff;                                                                          \
       }                                                                                                   \
     }                                                                                                     \
-    if (TAPS) voTap = tap_offset(tapL);                                                                   \
+    if (TAPS) voTap = tap_offset(dhL, dwL);                                                               \
   } while (0)
 
   // multiplies the stream's oldest group (operands CUR, group G of the unit in hand) after putting one more
@@ -192,7 +196,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   ihB = ihBN;
   iwB = iwBN;
   setup_next(unit + unitStep);
-  voTap = tap_offset(0);
+  voTap = tap_offset(dhL, dwL);
   WS_LOAD_NEXT(b0);
   WS_LOAD_NEXT(b1);
   WS_LOAD_NEXT(b2);
@@ -303,7 +307,7 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
   *handled = 0;
   if (tunable("conv_no_ws", 0)) return MCN_SUCCESS;
   if (p.Cin % (2 * kDepth) != 0 || p.R % (8 * kDepth) != 0 || p.T > kMaxTapsWs || p.coutPad % 32 != 0) return MCN_SUCCESS;
-  const size_t lds = (size_t)p.R * p.coutPad * sizeof(float) + (size_t)p.T * sizeof(int2);
+  const size_t lds = (size_t)p.R * p.coutPad * sizeof(float);
   if (lds > 150 * 1024) return MCN_SUCCESS;
   // byte offsets into the gathered tensor must stay below the "outside" offset
   const long long inBytes = ((long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW) * 4;

@@ -242,7 +242,7 @@ def test_weights_stationary_kernel(capi, ob, xs, fs, stride, pad, dilate, wa):
         taps = fs[0] * fs[1]
         tile = 128 if cout > 64 else (64 if cout > 32 else 32)
         padded = -(-cout // tile) * tile
-        return (cin % 16 == 0 and (taps * cin) % 64 == 0 and taps * cin * padded * 4 + taps * 8 <= 150 * 1024 and
+        return (cin % 16 == 0 and (taps * cin) % 64 == 0 and taps * cin * padded * 4 <= 150 * 1024 and
                 (wa == 0 or padded % (32 * wa) == 0))
 
     # the kernel under test really ran (a strided layer's backward-data product is one launch per stride class
