@@ -377,3 +377,23 @@ def test_random_geometries_vs_oracle(capi, ob, seed):
     assert rel_max(y, ob.conv_forward(x, f, b, og)) <= TOL, case
     dy = F(r.standard_normal(ob.conv_out_shape(og)))
     _check(capi, ob, x, f, b, dy, *case[8:])
+
+
+def test_tensors_over_2_gib_match_small_batches(capi):
+    """Tensors beyond 2^31 bytes leave the 32-bit-offset fast paths (buffer descriptors, uniform-tap offsets): the
+    same layer on the whole batch and on its first / last images must agree (images are independent)."""
+    import torch
+    H, W, Cc, N = 64, 64, 64, 2100            # 2.2 GB per tensor
+    fs = (3, 3, Cc, Cc)
+    torch.manual_seed(5)
+    x = torch.randn((N, Cc, W, H), device="cuda")
+    f = torch.randn(tuple(reversed(fs)), device="cuda") * 0.05
+    g = capi.conv_geom((H, W, Cc, N), fs, 1, 1, 1)
+    y = capi.conv_forward(x, f, None, g)
+    dx, _, _ = capi.conv_backward(x, f, y, g, want=(True, False, False))
+    for sl in (slice(0, 3), slice(N - 3, N)):
+        gs = capi.conv_geom((H, W, Cc, 3), fs, 1, 1, 1)
+        ys = capi.conv_forward(x[sl].contiguous(), f, None, gs)
+        assert float((ys - y[sl]).abs().max()) <= 2e-4 * float(ys.abs().max())
+        dxs, _, _ = capi.conv_backward(x[sl].contiguous(), f, ys, gs, want=(True, False, False))
+        assert float((dxs - dx[sl]).abs().max()) <= 2e-4 * float(dxs.abs().max())
