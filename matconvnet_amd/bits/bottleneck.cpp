@@ -9,29 +9,42 @@
 
 namespace vl { namespace harness {
 
-Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon)
-    : H(H), W(W), C(C), M(M), N(N), epsilon(epsilon), error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false),
-      overlap(false), sideStream(NULL) {
-  for (int i = 0; i < 4; ++i) events[i] = NULL;
-  const TensorShape big(H, W, C, N), small(H, W, M, N);
+Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int CoutArg, int stride, bool adapter,
+                       Context* shared)
+    : H(H), W(W), C(C), M(M), N(N), Cout(CoutArg > 0 ? CoutArg : C), stride(stride), Ho((H - 1) / stride + 1),
+      Wo((W - 1) / stride + 1), adapter(adapter), epsilon(epsilon), context(shared ? *shared : ownContext),
+      error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), sideStream(NULL) {
+  for (int i = 0; i < 5; ++i) events[i] = NULL;
+  if (!adapter && (Cout != C || stride != 1)) {
+    error = VLE_IllegalArgument;
+    message = "a unit that changes the number of channels or the resolution needs the adapter on its shortcut";
+    return;
+  }
+  const TensorShape in(H, W, C, N), mid(H, W, M, N), midOut(Ho, Wo, M, N), out(Ho, Wo, Cout, N);
   // inputs and parameters
-  make("x", big); make("dzdy", big);
-  make("f1", TensorShape(1, 1, C, M)); make("f2", TensorShape(3, 3, M, M)); make("f3", TensorShape(1, 1, M, C));
+  make("x", in); make("dzdy", out);
+  make("f1", TensorShape(1, 1, C, M)); make("f2", TensorShape(3, 3, M, M)); make("f3", TensorShape(1, 1, M, Cout));
   make("g1", TensorShape(M, 1, 1, 1)); make("b1", TensorShape(M, 1, 1, 1));
   make("g2", TensorShape(M, 1, 1, 1)); make("b2", TensorShape(M, 1, 1, 1));
-  make("g3", TensorShape(C, 1, 1, 1)); make("b3", TensorShape(C, 1, 1, 1));
+  make("g3", TensorShape(Cout, 1, 1, 1)); make("b3", TensorShape(Cout, 1, 1, 1));
   // forward activations
-  make("a1", small); make("n1", small); make("r1", small);
-  make("a2", small); make("n2", small); make("r2", small);
-  make("a3", big); make("n3", big); make("s", big); make("y", big);
-  make("m1", TensorShape(M, 2, 1, 1)); make("m2", TensorShape(M, 2, 1, 1)); make("m3", TensorShape(C, 2, 1, 1));
+  make("a1", mid); make("n1", mid); make("r1", mid);
+  make("a2", midOut); make("n2", midOut); make("r2", midOut);
+  make("a3", out); make("n3", out); make("s", out); make("y", out);
+  make("m1", TensorShape(M, 2, 1, 1)); make("m2", TensorShape(M, 2, 1, 1)); make("m3", TensorShape(Cout, 2, 1, 1));
   // derivatives
-  make("ds", big); make("da3", big); make("dr2", small); make("dn2", small); make("da2", small);
-  make("dr1", small); make("dn1", small); make("da1", small); make("dxm", big); make("dzdx", big);
-  make("df1", TensorShape(1, 1, C, M)); make("df2", TensorShape(3, 3, M, M)); make("df3", TensorShape(1, 1, M, C));
+  make("ds", out); make("da3", out); make("dr2", midOut); make("dn2", midOut); make("da2", midOut);
+  make("dr1", mid); make("dn1", mid); make("da1", mid); make("dxm", in); make("dzdx", in);
+  make("df1", TensorShape(1, 1, C, M)); make("df2", TensorShape(3, 3, M, M)); make("df3", TensorShape(1, 1, M, Cout));
   make("dg1", TensorShape(M, 1, 1, 1)); make("db1", TensorShape(M, 1, 1, 1));
   make("dg2", TensorShape(M, 1, 1, 1)); make("db2", TensorShape(M, 1, 1, 1));
-  make("dg3", TensorShape(C, 1, 1, 1)); make("db3", TensorShape(C, 1, 1, 1));
+  make("dg3", TensorShape(Cout, 1, 1, 1)); make("db3", TensorShape(Cout, 1, 1, 1));
+  if (adapter) {
+    make("fs", TensorShape(1, 1, C, Cout)); make("gs", TensorShape(Cout, 1, 1, 1)); make("bs", TensorShape(Cout, 1, 1, 1));
+    make("as", out); make("ns", out); make("ms", TensorShape(Cout, 2, 1, 1));
+    make("das", out); make("dfs", TensorShape(1, 1, C, Cout));
+    make("dgs", TensorShape(Cout, 1, 1, 1)); make("dbs", TensorShape(Cout, 1, 1, 1));
+  }
 }
 
 ErrorCode Bottleneck::setOverlap(bool on) {
@@ -43,7 +56,7 @@ ErrorCode Bottleneck::setOverlap(bool on) {
       return error = VLE_Cuda;
     }
     sideStream = st;
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 5; ++i) {
       hipEvent_t e = NULL;
       if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
         (void)hipGetLastError();
@@ -62,12 +75,12 @@ Bottleneck::~Bottleneck() {
   if (sideStream) {
     (void)hipStreamSynchronize((hipStream_t)sideStream);
     sideContext.clear();
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 5; ++i)
       if (events[i]) (void)hipEventDestroy((hipEvent_t)events[i]);
     (void)hipStreamDestroy((hipStream_t)sideStream);
   }
   for (std::size_t i = 0; i < slots.size(); ++i)
-    if (slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
+    if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
 }
 
 Tensor Bottleneck::make(std::string const& name, TensorShape const& shape) {
@@ -82,6 +95,7 @@ Tensor Bottleneck::make(std::string const& name, TensorShape const& shape) {
   Slot s;
   s.name = name;
   s.tensor = Tensor(shape, VLDT_Float, VLDT_GPU, memory, bytes);
+  s.owned = true;
   slots.push_back(s);
   return s.tensor;
 }
@@ -97,6 +111,19 @@ float* Bottleneck::buffer(std::string const& name, std::size_t* count) {
   Tensor& t = slot(name);
   if (count) *count = t.getNumElements();
   return (float*)t.getMemory();
+}
+
+ErrorCode Bottleneck::alias(std::string const& name, float* memory) {
+  for (std::size_t i = 0; i < slots.size(); ++i) {
+    if (slots[i].name != name) continue;
+    if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
+    const TensorShape shape = slots[i].tensor.getShape();
+    slots[i].tensor = Tensor(shape, VLDT_Float, VLDT_GPU, memory, shape.getNumElements() * sizeof(float));
+    slots[i].owned = false;
+    return VLE_Success;
+  }
+  message = "no buffer '" + name + "'";
+  return error = VLE_IllegalArgument;
 }
 
 ErrorCode Bottleneck::setStream(void* stream) { return context.getHipHelper().setStream(stream); }
@@ -132,34 +159,47 @@ ErrorCode Bottleneck::forward() {
   if (error != VLE_Success) return error;
   void* st = context.getHipHelper().getStream();
   Tensor none;
-  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, 1, 1, 1, 1, 1, 1, 1, 1);
+  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),
+      cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
   nn::BatchNorm bn(context, epsilon);
-  const std::size_t nSmall = slot("a1").getNumElements(), nBig = slot("a3").getNumElements();
+  const std::size_t nMid = slot("a1").getNumElements(), nMidOut = slot("a2").getNumElements(),
+                    nOut = slot("a3").getNumElements();
+  // the shortcut: the input, or its adapted version (matlab: Conv([name '_adapt_conv'], 1, ..., 'relu', false))
+  char const* shortcut = "x";
+  if (adapter) {
+    STEP("convs_fwd", cs.forward(slot("as"), 0, slot("x"), 1, slot("fs"), none));
+    STEP("bns_fwd", bn.forward(slot("ns"), slot("ms"), slot("as"), slot("gs"), slot("bs")));
+    shortcut = "ns";
+  }
   if (fused) {
-    const size_t wsSmall = mcn_bnorm_workspace_bytes(H, W, M, N), wsBig = mcn_bnorm_workspace_bytes(H, W, C, N);
-    void* ws = context.getWorkspace(VLDT_GPU, wsBig > wsSmall ? wsBig : wsSmall);
-    if (!ws) return fail(context.getLastError(), "workspace");
+    const size_t wsMid = mcn_bnorm_workspace_bytes(H, W, M, N), wsOut = mcn_bnorm_workspace_bytes(Ho, Wo, Cout, N);
     STEP("conv1_fwd", c1.forward(slot("a1"), 0, slot("x"), 1, slot("f1"), none));
+    void* ws = context.getWorkspace(VLDT_GPU, wsMid > wsOut ? wsMid : wsOut);
+    if (!ws) return fail(context.getLastError(), "workspace");
     ABI("bn1_fwd", mcn_bnorm_forward_fused(st, buffer("r1"), buffer("m1"), buffer("a1"), buffer("g1"), buffer("b1"), NULL, 1,
-                                           H, W, M, N, epsilon, 0, ws, wsSmall));
+                                           H, W, M, N, epsilon, 0, ws, wsMid));
     STEP("conv2_fwd", c2.forward(slot("a2"), 0, slot("r1"), 1, slot("f2"), none));
+    ws = context.getWorkspace(VLDT_GPU, wsMid > wsOut ? wsMid : wsOut);  // (a convolution may have grown it)
+    if (!ws) return fail(context.getLastError(), "workspace");
     ABI("bn2_fwd", mcn_bnorm_forward_fused(st, buffer("r2"), buffer("m2"), buffer("a2"), buffer("g2"), buffer("b2"), NULL, 1,
-                                           H, W, M, N, epsilon, 0, ws, wsSmall));
+                                           Ho, Wo, M, N, epsilon, 0, ws, wsMid));
     STEP("conv3_fwd", c1.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
-    ABI("bn3_fwd", mcn_bnorm_forward_fused(st, buffer("y"), buffer("m3"), buffer("a3"), buffer("g3"), buffer("b3"), buffer("x"), 1,
-                                           H, W, C, N, epsilon, 0, ws, wsBig));
+    ws = context.getWorkspace(VLDT_GPU, wsMid > wsOut ? wsMid : wsOut);
+    if (!ws) return fail(context.getLastError(), "workspace");
+    ABI("bn3_fwd", mcn_bnorm_forward_fused(st, buffer("y"), buffer("m3"), buffer("a3"), buffer("g3"), buffer("b3"),
+                                           buffer(shortcut), 1, Ho, Wo, Cout, N, epsilon, 0, ws, wsOut));
     return VLE_Success;
   }
   STEP("conv1_fwd", c1.forward(slot("a1"), 0, slot("x"), 1, slot("f1"), none));
   STEP("bn1_fwd", bn.forward(slot("n1"), slot("m1"), slot("a1"), slot("g1"), slot("b1")));
-  ABI("relu1_fwd", mcn_relu_forward(st, buffer("r1"), buffer("n1"), nSmall));
+  ABI("relu1_fwd", mcn_relu_forward(st, buffer("r1"), buffer("n1"), nMid));
   STEP("conv2_fwd", c2.forward(slot("a2"), 0, slot("r1"), 1, slot("f2"), none));
   STEP("bn2_fwd", bn.forward(slot("n2"), slot("m2"), slot("a2"), slot("g2"), slot("b2")));
-  ABI("relu2_fwd", mcn_relu_forward(st, buffer("r2"), buffer("n2"), nSmall));
+  ABI("relu2_fwd", mcn_relu_forward(st, buffer("r2"), buffer("n2"), nMidOut));
   STEP("conv3_fwd", c1.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
   STEP("bn3_fwd", bn.forward(slot("n3"), slot("m3"), slot("a3"), slot("g3"), slot("b3")));
-  ABI("sum_fwd", mcn_add(st, buffer("s"), buffer("n3"), buffer("x"), nBig));
-  ABI("relu3_fwd", mcn_relu_forward(st, buffer("y"), buffer("s"), nBig));
+  ABI("sum_fwd", mcn_add(st, buffer("s"), buffer("n3"), buffer(shortcut), nOut));
+  ABI("relu3_fwd", mcn_relu_forward(st, buffer("y"), buffer("s"), nOut));
   return VLE_Success;
 }
 
@@ -167,33 +207,24 @@ ErrorCode Bottleneck::backward() {
   if (error != VLE_Success) return error;
   void* st = context.getHipHelper().getStream();
   Tensor none;
-  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, 1, 1, 1, 1, 1, 1, 1, 1);
+  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),
+      cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
   nn::BatchNorm bn(context, epsilon);
-  const std::size_t nSmall = slot("a1").getNumElements(), nBig = slot("a3").getNumElements();
+  const std::size_t nMid = slot("a1").getNumElements(), nMidOut = slot("a2").getNumElements(),
+                    nIn = slot("x").getNumElements(), nOut = slot("a3").getNumElements();
   // ReLU masks: the layer's input, or (fused mode) its output -- max(v, 0) > 0 exactly when v > 0
   char const* mask3 = fused ? "y" : "s";
   char const* mask2 = fused ? "r2" : "n2";
   char const* mask1 = fused ? "r1" : "n1";
-  // the sum passes ds to both of its inputs: the branch (n3) and the shortcut (x).  Fused mode keeps ds in the
-  // output buffer and lets the first convolution add its derivative to it.
-  char const* dsName = fused ? "dzdx" : "ds";
-  if (fused) {
-    // the block's last ReLU sits behind the shortcut sum: its derivative is taken and written (for the shortcut
-    // branch) in the summing pass of the batch-norm derivative
-    const size_t wsBig = mcn_bnorm_workspace_bytes(H, W, C, N);
-    void* wsB = context.getWorkspace(VLDT_GPU, wsBig);
-    if (!wsB) return fail(context.getLastError(), "workspace");
-    ABI("bn3_bwd", mcn_bnorm_backward_masked(st, buffer("da3"), buffer("dg3"), buffer("db3"), buffer("m3"), buffer("a3"),
-                                             buffer("g3"), buffer("dzdy"), buffer(mask3), buffer(dsName), H, W, C, N, epsilon,
-                                             wsB, wsBig));
-  } else {
-    ABI("relu3_bwd", mcn_relu_backward(st, buffer(dsName), buffer(mask3), buffer("dzdy"), nBig));
-    STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot(dsName)));
-  }
+  // The sum passes ds to both of its inputs: the branch (n3) and the shortcut.  With an identity shortcut the fused
+  // mode keeps ds in the output buffer and lets the first convolution add its derivative to it.
+  char const* dsName = (fused && !adapter) ? "dzdx" : "ds";
+
   // A convolution's backward: the input gradient on the caller's stream; the filter gradient beside it on the
   // second stream when overlapping (enqueued after it, so the persistent input-gradient kernel takes its CUs
   // first and the filter-gradient workgroups fill in beside and behind it).
-  nn::Convolution c1s(sideContext, 1, 1, 0, 0, 0, 0, 1, 1), c2s(sideContext, 1, 1, 1, 1, 1, 1, 1, 1);
+  nn::Convolution c1s(sideContext, 1, 1, 0, 0, 0, 0, 1, 1), c2s(sideContext, stride, stride, 1, 1, 1, 1, 1, 1),
+      css(sideContext, stride, stride, 0, 0, 0, 0, 1, 1);
   Tensor none2, none3;
   auto convBackward = [&](nn::Convolution& onMain, nn::Convolution& onSide, int k, Tensor& derIn, double derInMult,
                           Tensor& derFilter, Tensor const& in, Tensor const& filter, Tensor const& derOut) -> ErrorCode {
@@ -209,34 +240,62 @@ ErrorCode Bottleneck::backward() {
   };
   auto joinSide = [&]() -> ErrorCode {
     if (!overlap) return VLE_Success;
-    if (hipEventRecord((hipEvent_t)events[3], (hipStream_t)sideStream) != hipSuccess ||
-        hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)events[3], 0) != hipSuccess)
+    if (hipEventRecord((hipEvent_t)events[4], (hipStream_t)sideStream) != hipSuccess ||
+        hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)events[4], 0) != hipSuccess)
       return context.setError(VLE_Cuda, "cannot join the second stream");
     return VLE_Success;
   };
-  STEP("conv3_bwd", convBackward(c1, c1s, 0, slot("dr2"), 0, slot("df3"), slot("r2"), slot("f3"), slot("da3")));
-  const size_t wsSmall = mcn_bnorm_workspace_bytes(H, W, M, N);
+
+  const size_t wsMid = mcn_bnorm_workspace_bytes(H, W, M, N), wsOut = mcn_bnorm_workspace_bytes(Ho, Wo, Cout, N);
+  const size_t wsBnBytes = wsMid > wsOut ? wsMid : wsOut;
   void* wsBn = NULL;
+  if (fused) {
+    // the unit's last ReLU sits behind the shortcut sum: its derivative is taken and written (for the shortcut
+    // branch) in the summing pass of the batch-norm derivative
+    wsBn = context.getWorkspace(VLDT_GPU, wsBnBytes);
+    if (!wsBn) return fail(context.getLastError(), "workspace");
+    ABI("bn3_bwd", mcn_bnorm_backward_masked(st, buffer("da3"), buffer("dg3"), buffer("db3"), buffer("m3"), buffer("a3"),
+                                             buffer("g3"), buffer("dzdy"), buffer(mask3), buffer(dsName), Ho, Wo, Cout, N,
+                                             epsilon, wsBn, wsOut));
+  } else {
+    ABI("relu3_bwd", mcn_relu_backward(st, buffer(dsName), buffer(mask3), buffer("dzdy"), nOut));
+    STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot(dsName)));
+  }
+  STEP("conv3_bwd", convBackward(c1, c1s, 0, slot("dr2"), 0, slot("df3"), slot("r2"), slot("f3"), slot("da3")));
   if (fused) {
     // ReLU's derivative folded into the batch-norm derivative that follows it: the mask is recomputed from the
     // layer's input and stored moments, the masked derivative is never written out
-    wsBn = context.getWorkspace(VLDT_GPU, wsSmall);
+    wsBn = context.getWorkspace(VLDT_GPU, wsBnBytes);  // (the convolution in between may have grown the workspace)
     if (!wsBn) return fail(context.getLastError(), "workspace");
     ABI("bn2_bwd", mcn_bnorm_backward_relu(st, buffer("da2"), buffer("dg2"), buffer("db2"), buffer("m2"), buffer("a2"),
-                                           buffer("g2"), buffer("b2"), buffer("dr2"), H, W, M, N, epsilon, wsBn, wsSmall));
+                                           buffer("g2"), buffer("b2"), buffer("dr2"), Ho, Wo, M, N, epsilon, wsBn, wsMid));
   } else {
-    ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer(mask2), buffer("dr2"), nSmall));
+    ABI("relu2_bwd", mcn_relu_backward(st, buffer("dn2"), buffer(mask2), buffer("dr2"), nMidOut));
     STEP("bn2_bwd", bn.backwardWithMoment(slot("da2"), slot("dg2"), slot("db2"), slot("m2"), slot("a2"), slot("g2"), slot("b2"), slot("dn2")));
   }
   STEP("conv2_bwd", convBackward(c2, c2s, 1, slot("dr1"), 0, slot("df2"), slot("r1"), slot("f2"), slot("da2")));
   if (fused) {
-    wsBn = context.getWorkspace(VLDT_GPU, wsSmall);  // (the convolution in between may have grown the workspace)
+    wsBn = context.getWorkspace(VLDT_GPU, wsBnBytes);
     if (!wsBn) return fail(context.getLastError(), "workspace");
     ABI("bn1_bwd", mcn_bnorm_backward_relu(st, buffer("da1"), buffer("dg1"), buffer("db1"), buffer("m1"), buffer("a1"),
-                                           buffer("g1"), buffer("b1"), buffer("dr1"), H, W, M, N, epsilon, wsBn, wsSmall));
+                                           buffer("g1"), buffer("b1"), buffer("dr1"), H, W, M, N, epsilon, wsBn, wsMid));
   } else {
-    ABI("relu1_bwd", mcn_relu_backward(st, buffer("dn1"), buffer(mask1), buffer("dr1"), nSmall));
+    ABI("relu1_bwd", mcn_relu_backward(st, buffer("dn1"), buffer(mask1), buffer("dr1"), nMid));
     STEP("bn1_bwd", bn.backwardWithMoment(slot("da1"), slot("dg1"), slot("db1"), slot("m1"), slot("a1"), slot("g1"), slot("b1"), slot("dn1")));
+  }
+  if (adapter) {
+    // the shortcut branch: bnorm (no ReLU) and the strided 1x1 convolution, whose input gradient opens dzdx
+    STEP("bns_bwd", bn.backwardWithMoment(slot("das"), slot("dgs"), slot("dbs"), slot("ms"), slot("as"), slot("gs"), slot("bs"), slot("ds")));
+    if (fused) {
+      STEP("convs_bwd", convBackward(cs, css, 3, slot("dzdx"), 0, slot("dfs"), slot("x"), slot("fs"), slot("das")));
+      STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dzdx"), 1, slot("df1"), slot("x"), slot("f1"), slot("da1")));
+    } else {
+      STEP("convs_bwd", convBackward(cs, css, 3, slot("dxm"), 0, slot("dfs"), slot("x"), slot("fs"), slot("das")));
+      STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dzdx"), 0, slot("df1"), slot("x"), slot("f1"), slot("da1")));
+      ABI("sum_bwd", mcn_add(st, buffer("dzdx"), buffer("dzdx"), buffer("dxm"), nIn));
+    }
+    STEP("join", joinSide());
+    return VLE_Success;
   }
   if (fused) {
     STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dzdx"), 1, slot("df1"), slot("x"), slot("f1"), slot("da1")));
@@ -244,7 +303,7 @@ ErrorCode Bottleneck::backward() {
     return VLE_Success;
   }
   STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dxm"), 0, slot("df1"), slot("x"), slot("f1"), slot("da1")));
-  ABI("sum_bwd", mcn_add(st, buffer("dzdx"), buffer("dxm"), buffer("ds"), nBig));
+  ABI("sum_bwd", mcn_add(st, buffer("dzdx"), buffer("dxm"), buffer("ds"), nIn));
   STEP("join", joinSide());
   return VLE_Success;
 }

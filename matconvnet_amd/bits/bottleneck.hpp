@@ -1,9 +1,11 @@
-// ResNet-50 bottleneck block (forward + backward) wired directly onto the vl::nn operators, the way the
-// reference's DagNN would drive them for the block built by examples/imagenet/cnn_imagenet_init_resnet.m:16-48:
-//   conv1x1 C->M, bnorm, relu, conv3x3 M->M (pad 1), bnorm, relu, conv1x1 M->C, bnorm, + identity, relu
-// Convolutions have no bias.  Batch-norm backward uses the moments cached by the forward pass
-// (matlab/+dagnn/BatchNorm.m:27-34); the shortcut's derivative is added to the branch's as
-// matlab/+dagnn/Layer.m:127-135 does for variables with fan-out > 1.
+// ResNet bottleneck unit (forward + backward) wired directly onto the vl::nn operators, the way the reference's
+// DagNN would drive them for one segment of examples/imagenet/cnn_imagenet_init_resnet.m:86-118:
+//   conv1x1 C->M, bnorm, relu, conv3x3 M->M (pad 1, stride s), bnorm, relu, conv1x1 M->Cout, bnorm,
+//   + shortcut, relu
+// where the shortcut is the input itself, or (first segment of a section: `adapter`) conv1x1 C->Cout with
+// stride s followed by bnorm.  Convolutions have no bias.  Batch-norm backward uses the moments cached by the
+// forward pass (matlab/+dagnn/BatchNorm.m:27-34); derivatives of a variable with two consumers are added as
+// matlab/+dagnn/Layer.m:127-135 does.
 // All buffers are allocated once; a step performs no allocation.
 #ifndef MCN_AMD_BITS_BOTTLENECK_HPP
 #define MCN_AMD_BITS_BOTTLENECK_HPP
@@ -17,19 +19,30 @@ namespace vl { namespace harness {
 
 class Bottleneck {
  public:
-  Bottleneck(int H, int W, int C, int M, int N, double epsilon);
+  // H x W x C x N input, M channels inside, Cout channels out (0: same as C), stride 1 or 2 on the 3x3 layer and
+  // the adapter.  `shared`: use this context (stream, workspace) instead of one of the unit's own.
+  Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Cout = 0, int stride = 1, bool adapter = false,
+             Context* shared = NULL);
   ~Bottleneck();
   bool ok() const { return error == VLE_Success; }
   ErrorCode lastError() const { return error; }
   std::string const& lastMessage() const { return message; }
 
-  // named device buffers: inputs "x","dzdy","f1","f2","f3","g1","b1",...; outputs "y","dzdx","df1","dg1","db1",...
+  // named device buffers: inputs "x","dzdy","f1","f2","f3","g1","b1",... (adapter: "fs","gs","bs");
+  // outputs "y","dzdx","df1","dg1","db1",...
   float* buffer(std::string const& name, std::size_t* count = NULL);
+  // makes a named buffer a view of memory owned by someone else (the previous unit's output, say); the unit's own
+  // allocation for it is released
+  ErrorCode alias(std::string const& name, float* memory);
   ErrorCode setStream(void* stream);
+  int outHeight() const { return Ho; }
+  int outWidth() const { return Wo; }
+  int outDepth() const { return Cout; }
 
   // fused = true: batch-norm forward applies the ReLU (and, for the last one, the shortcut sum) in its output
-  // pass (mcn_bnorm_forward_fused); the un-activated tensors n1, n2, n3, s are then never written and the
-  // ReLU derivatives take their masks from r1, r2, y.  Results are bit-identical to the layer-by-layer mode.
+  // pass (mcn_bnorm_forward_fused), so the un-activated tensors n1, n2, n3, s are never written; in the backward
+  // pass ReLU's derivatives are taken inside the batch-norm derivatives and the shortcut's fan-out sum inside the
+  // first convolution's.  Results are bit-identical to the layer-by-layer mode.
   void setFused(bool on) { fused = on; }
   // overlap = true: in the backward pass each convolution's filter gradient runs on a second stream (with a
   // context and workspace of its own) beside the same layer's input gradient, which is all the following layers
@@ -44,15 +57,17 @@ class Bottleneck {
   void setStageHook(StageHook hook, void* user) { stageHook = hook; hookUser = user; }
 
  private:
-  struct Slot { std::string name; Tensor tensor; };
+  struct Slot { std::string name; Tensor tensor; bool owned; };
   Tensor& slot(std::string const& name);
   Tensor make(std::string const& name, TensorShape const& shape);
   ErrorCode fail(ErrorCode e, char const* where);
   void mark(char const* stage, int begin) { if (stageHook) stageHook(hookUser, stage, begin); }
 
-  int H, W, C, M, N;
+  int H, W, C, M, N, Cout, stride, Ho, Wo;
+  bool adapter;
   double epsilon;
-  Context context;
+  Context ownContext;
+  Context& context;
   std::vector<Slot> slots;
   ErrorCode error;
   std::string message;
@@ -62,7 +77,7 @@ class Bottleneck {
   bool overlap;
   Context sideContext;
   void* sideStream;     // hipStream_t
-  void* events[4];      // hipEvent_t: "derivative ready" for the three convolutions, "second stream done"
+  void* events[5];      // hipEvent_t: "derivative ready" for the convolutions, "second stream done"
 };
 
 } }  // namespace vl::harness

@@ -155,6 +155,13 @@ void* vlh_bottleneck_create(int H, int W, int C, int M, int N, double epsilon) {
   return h;
 }
 
+void* vlh_unit_create(int H, int W, int C, int M, int N, double epsilon, int Cout, int stride, int adapter) {
+  BlockHandle* h = new BlockHandle;
+  h->block = new harness::Bottleneck(H, W, C, M, N, epsilon, Cout, stride, adapter != 0);
+  h->stream = NULL;
+  return h;
+}
+
 void vlh_bottleneck_destroy(void* block) {
   BlockHandle* h = (BlockHandle*)block;
   if (!h) return;

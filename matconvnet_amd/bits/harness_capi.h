@@ -39,6 +39,9 @@ VLH_API int vlh_cpu_tensor_is_refused(void);
 
 /* ResNet bottleneck block */
 VLH_API void* vlh_bottleneck_create(int H, int W, int C, int M, int N, double epsilon);
+/* the general unit: Cout output channels, stride 1 or 2 on the 3x3 layer, adapter != 0: conv1x1 (same stride) +
+   bnorm on the shortcut (buffers "fs", "gs", "bs", "dfs", "dgs", "dbs"); same handle functions as above */
+VLH_API void* vlh_unit_create(int H, int W, int C, int M, int N, double epsilon, int Cout, int stride, int adapter);
 VLH_API void vlh_bottleneck_destroy(void* block);
 VLH_API float* vlh_bottleneck_buffer(void* block, const char* name, size_t* count);
 VLH_API int vlh_bottleneck_set_stream(void* block, void* stream);

@@ -52,6 +52,8 @@ def lib():
         L.vlh_cpu_tensor_is_refused.restype = C.c_int
         L.vlh_bottleneck_create.restype = C.c_void_p
         L.vlh_bottleneck_create.argtypes = [C.c_int] * 5 + [C.c_double]
+        L.vlh_unit_create.restype = C.c_void_p
+        L.vlh_unit_create.argtypes = [C.c_int] * 5 + [C.c_double] + [C.c_int] * 3
         L.vlh_bottleneck_destroy.argtypes = [C.c_void_p]
         L.vlh_bottleneck_buffer.restype = C.c_void_p
         L.vlh_bottleneck_buffer.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_size_t)]
@@ -179,10 +181,11 @@ def vl_taccum(*args):
 class Bottleneck:
     """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
 
-    def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False, overlap=False):
+    def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False, overlap=False, Cout=0, stride=1,
+                 adapter=False):
         self.L = lib()
         self.shape = (H, W, Cc, M, N)
-        self.h = self.L.vlh_bottleneck_create(H, W, Cc, M, N, eps)
+        self.h = self.L.vlh_unit_create(H, W, Cc, M, N, eps, Cout, stride, int(adapter))
         torch = _torch()
         self.L.vlh_bottleneck_set_stream(self.h, C.c_void_p(torch.cuda.current_stream().cuda_stream))
         self.L.vlh_bottleneck_set_fused(self.h, int(fused))

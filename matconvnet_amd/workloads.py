@@ -55,19 +55,27 @@ def he_normal(r, shape):
     return _f(r.standard_normal(shape, dtype=np.float32) * np.float32(np.sqrt(2.0 / (fh * fw * fc))))
 
 
-def bottleneck_case(seed=5, H=56, W=56, C=256, M=64, N=32, eps=1e-5):
-    """ResNet-50 bottleneck: conv1x1 C->M, bn, relu, conv3x3 M->M pad 1, bn, relu, conv1x1 M->C, bn,
-    + identity, relu.  He-normal weights, no conv bias, bnorm gain 1 / bias 0."""
+def bottleneck_case(seed=5, H=56, W=56, C=256, M=64, N=32, eps=1e-5, Cout=None, stride=1, adapter=False):
+    """ResNet-50 bottleneck unit: conv1x1 C->M, bn, relu, conv3x3 M->M pad 1 (stride), bn, relu, conv1x1 M->Cout,
+    bn, + shortcut, relu; shortcut = identity, or (adapter) conv1x1 C->Cout (stride) + bn.  He-normal weights, no
+    conv bias, bnorm gain 1 / bias 0 (gains and biases of the adapter unit are randomised a little so that they
+    matter)."""
     r = np.random.default_rng(seed)
+    Cout = C if Cout is None else Cout
+    Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
     x = _f(r.standard_normal((H, W, C, N), dtype=np.float32))
-    dy = _f(r.standard_normal((H, W, C, N), dtype=np.float32))
+    dy = _f(r.standard_normal((Ho, Wo, Cout, N), dtype=np.float32))
     f1 = he_normal(r, (1, 1, C, M))
     f2 = he_normal(r, (3, 3, M, M))
-    f3 = he_normal(r, (1, 1, M, C))
+    f3 = he_normal(r, (1, 1, M, Cout))
     ones = lambda n: np.ones((n,), np.float32)
     zeros = lambda n: np.zeros((n,), np.float32)
-    return dict(x=x, dy=dy, f1=f1, f2=f2, f3=f3, g1=ones(M), b1=zeros(M), g2=ones(M), b2=zeros(M),
-                g3=ones(C), b3=zeros(C), eps=eps)
+    w = dict(x=x, dy=dy, f1=f1, f2=f2, f3=f3, g1=ones(M), b1=zeros(M), g2=ones(M), b2=zeros(M),
+             g3=ones(Cout), b3=zeros(Cout), eps=eps, stride=stride, adapter=adapter)
+    if adapter:
+        w.update(fs=he_normal(r, (1, 1, C, Cout)), gs=(1 + 0.1 * r.standard_normal(Cout)).astype(np.float32),
+                 bs=(0.1 * r.standard_normal(Cout)).astype(np.float32))
+    return w
 
 
 def conv_vgg(seed=6, H=56, W=56, C=256, K=256, N=64):

@@ -328,3 +328,45 @@ def test_bnorm_backward_masked_matches_separate_calls(capi, ob):
     for a, b_ in zip(got[:3], want[:3]):
         assert bits_equal(capi.to_host(a), capi.to_host(b_))
     assert bits_equal(capi.to_host(got[3]), capi.to_host(masked))
+
+
+UNITS = [  # (H, W, C, M, Cout, stride, adapter): the kinds of segment ResNet-50 is made of, at reduced size
+    (14, 14, 64, 16, 64, 1, False),     # plain segment, identity shortcut
+    (14, 14, 32, 16, 64, 1, True),      # first segment of section 2: adapter, no downsampling
+    (14, 14, 64, 32, 128, 2, True),     # first segment of sections 3-5: adapter and 3x3 layer with stride 2
+    (13, 11, 64, 32, 128, 2, True),     # odd extents: the stride classes differ in size
+]
+
+
+@pytest.mark.parametrize("H,W,Cc,M,Cout,stride,adapter", UNITS)
+def test_residual_unit_against_oracle_and_across_modes(vl, ob, H, W, Cc, M, Cout, stride, adapter):
+    """Each kind of ResNet-50 segment, N = 3: against the unit composed from oracle operators (double), and the fused
+    and two-stream schedules bit for bit against the layer-by-layer one."""
+    w = workloads.bottleneck_case(seed=9, H=H, W=W, C=Cc, M=M, N=3, Cout=Cout, stride=stride, adapter=adapter)
+    Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
+    shapes = dict(y=(Ho, Wo, Cout, 3), dzdx=w["x"].shape, df1=w["f1"].shape, df2=w["f2"].shape, df3=w["f3"].shape,
+                  dg1=(M,), db1=(M,), dg2=(M,), db2=(M,), dg3=(Cout,), db3=(Cout,))
+    names = ["x", "f1", "f2", "f3", "g1", "b1", "g2", "b2", "g3", "b3"]
+    if adapter:
+        shapes.update(dfs=w["fs"].shape, dgs=(Cout,), dbs=(Cout,))
+        names += ["fs", "gs", "bs"]
+    outs = {}
+    for mode in ("plain", "fused", "overlap"):
+        blk = vl.Bottleneck(H=H, W=W, Cc=Cc, M=M, N=3, eps=w["eps"], fused=mode != "plain", overlap=mode == "overlap",
+                            Cout=Cout, stride=stride, adapter=adapter)
+        try:
+            for k in names:
+                blk.set(k, w[k])
+            blk.set("dzdy", w["dy"])
+            for _ in range(2):
+                blk.forward()
+                blk.backward()
+            outs[mode] = {k: blk.get(k, v) for k, v in shapes.items()}
+        finally:
+            blk.close()
+    want = _oracle_bottleneck(ob, w, np.float64)
+    errs = {k: rel_max(outs["plain"][k], want[k]) for k in shapes}
+    assert max(errs.values()) < 5e-4, errs
+    for k in shapes:
+        assert bits_equal(outs["plain"][k], outs["fused"][k]), k
+        assert bits_equal(outs["plain"][k], outs["overlap"][k]), k
