@@ -7,6 +7,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include "bottleneck.hpp"
+#include "resnet.hpp"
 #include "frontend.hpp"
 #include "hiphelper.hpp"
 #include "nnpooling.hpp"
@@ -221,5 +222,21 @@ int vlh_bottleneck_run(void* block, int steps, const char* stage, float* stage_m
   }
   return rc;
 }
+
+void* vlh_resnet50_create(int N, double epsilon, int imageSize, int classes) {
+  return new harness::ResNet50(N, epsilon, imageSize, classes);
+}
+void vlh_resnet50_destroy(void* net) { delete (harness::ResNet50*)net; }
+int vlh_resnet50_units(void* net) { return ((harness::ResNet50*)net)->numUnits(); }
+float* vlh_resnet50_buffer(void* net, const char* name, size_t* count) {
+  return ((harness::ResNet50*)net)->buffer(name, count);
+}
+int vlh_resnet50_set_stream(void* net, void* stream) { return (int)((harness::ResNet50*)net)->setStream(stream); }
+void vlh_resnet50_set_fused(void* net, int fused) { ((harness::ResNet50*)net)->setFused(fused != 0); }
+int vlh_resnet50_init(void* net, unsigned long long seed) { return (int)((harness::ResNet50*)net)->initParameters(seed); }
+int vlh_resnet50_forward(void* net) { return (int)((harness::ResNet50*)net)->forward(); }
+int vlh_resnet50_backward(void* net) { return (int)((harness::ResNet50*)net)->backward(); }
+double vlh_resnet50_forward_flops(void* net) { return ((harness::ResNet50*)net)->convForwardFlopsPerImage(); }
+const char* vlh_resnet50_message(void* net) { return ((harness::ResNet50*)net)->lastMessage().c_str(); }
 
 }  // extern "C"

@@ -57,6 +57,23 @@ VLH_API int vlh_bottleneck_backward(void* block);
 VLH_API int vlh_bottleneck_run(void* block, int steps, const char* stage, float* stage_ms);
 VLH_API const char* vlh_bottleneck_message(void* block);
 
+/* ResNet-50 (examples/imagenet/cnn_imagenet_init_resnet.m:52-134 without the loss layers): imageSize x imageSize x 3 x N
+   input, `classes` outputs.  Buffers: "input", "prediction", "dprediction", "stem.f|g|b|df|dg|db", "fc.f|b|df|db",
+   "unit<i>.<name>" for the i-th bottleneck unit (names as for vlh_bottleneck_buffer). */
+VLH_API void* vlh_resnet50_create(int N, double epsilon, int imageSize, int classes);
+VLH_API void vlh_resnet50_destroy(void* net);
+VLH_API int vlh_resnet50_units(void* net);
+VLH_API float* vlh_resnet50_buffer(void* net, const char* name, size_t* count);
+VLH_API int vlh_resnet50_set_stream(void* net, void* stream);
+VLH_API void vlh_resnet50_set_fused(void* net, int fused);
+/* He-normal filters, gains 1, biases 0 from a seeded host generator */
+VLH_API int vlh_resnet50_init(void* net, unsigned long long seed);
+VLH_API int vlh_resnet50_forward(void* net);
+VLH_API int vlh_resnet50_backward(void* net);
+/* forward FLOPs of the convolutions for one image */
+VLH_API double vlh_resnet50_forward_flops(void* net);
+VLH_API const char* vlh_resnet50_message(void* net);
+
 #ifdef __cplusplus
 }
 #endif

@@ -3,7 +3,7 @@
 // synthetic inputs, times them with HIP events and prints TFLOP/s, GB/s and images/s beside the
 // fraction of the MI355X rooflines (fp32 matrix 157.3 TFLOP/s, HBM 8 TB/s).
 //
-//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy]
+//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|resnet50] [--batch N]
 //
 // The bandwidth-bound operators (bnorm, pooling, copy) are timed over R independent sets of tensors used in
 // turn (default 4), so that no launch finds its inputs in the 256 MB memory-side cache because the previous
@@ -26,6 +26,7 @@
 #include "nnbnorm.hpp"
 #include "nnconv.hpp"
 #include "nnpooling.hpp"
+#include "resnet.hpp"
 #include "../../include/mcn_hip.h"
 
 using namespace vl;
@@ -222,16 +223,50 @@ static void benchBlock(int warmup, int iters, bool fused, bool overlap = false) 
               "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, overlap ? "folded, filter gradients on a second stream" : (fused ? "relu/sum folded into bnorm" : "layer by layer"));
 }
 
+// Whole ResNet-50 (224 x 224 images, 1000 classes): forward alone (training-mode batch normalisation: moments are
+// computed, nothing is merged into the filters) and forward + backward.
+static void benchResNet(int warmup, int iters, int N, bool fused) {
+  harness::ResNet50 net(N, 1e-5, 224, 1000);
+  if (!net.ok() || net.initParameters(11) != VLE_Success) {
+    std::fprintf(stderr, "resnet-50: %s\n", net.lastMessage().c_str());
+    std::exit(3);
+  }
+  net.setFused(fused);
+  {
+    std::mt19937_64 gen(12);
+    std::normal_distribution<float> dist(0.f, 1.f);
+    for (char const* name : {"input", "dprediction"}) {
+      size_t n = 0;
+      float* p = net.buffer(name, &n);
+      std::vector<float> host(n);
+      for (size_t i = 0; i < n; ++i) host[i] = dist(gen);
+      HIP_OK(hipMemcpy(p, host.data(), n * sizeof(float), hipMemcpyHostToDevice));
+    }
+  }
+  auto stop = [&] {
+    std::fprintf(stderr, "resnet-50: %s\n", net.lastMessage().c_str());
+    std::exit(3);
+  };
+  double tf = medianMs([&] { if (net.forward() != VLE_Success) stop(); }, warmup, iters);
+  double t = medianMs([&] { if (net.forward() != VLE_Success || net.backward() != VLE_Success) stop(); }, warmup, iters);
+  const double gf = net.convForwardFlopsPerImage() * 1e-9;
+  std::printf("%-28s %8.2f ms forward  %8.0f images/s %6.1f TFLOP/s | %8.2f ms fwd+bwd %8.0f images/s %6.1f TFLOP/s "
+              "(N = %d, %.2f GFLOP of convolution per image forward; %s)\n",
+              "resnet-50 224x224", tf, N / (tf * 1e-3), gf * N / tf, t, N / (t * 1e-3), 3 * gf * N / t, N, gf,
+              fused ? "relu/sum folded into bnorm" : "layer by layer");
+}
+
 int main(int argc, char** argv) {
-  int iters = 20, warmup = 3;
+  int iters = 20, warmup = 3, batch = 32;
   std::string only;
   for (int i = 1; i < argc; ++i) {
     if (!std::strcmp(argv[i], "--iters") && i + 1 < argc) iters = std::atoi(argv[++i]);
     else if (!std::strcmp(argv[i], "--warmup") && i + 1 < argc) warmup = std::atoi(argv[++i]);
     else if (!std::strcmp(argv[i], "--only") && i + 1 < argc) only = argv[++i];
+    else if (!std::strcmp(argv[i], "--batch") && i + 1 < argc) batch = std::max(1, std::atoi(argv[++i]));
     else if (!std::strcmp(argv[i], "--rotate") && i + 1 < argc) gRotate = std::max(1, std::atoi(argv[++i]));
     else {
-      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy]\n");
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|resnet50] [--batch N]\n");
       return 1;
     }
   }
@@ -240,6 +275,10 @@ int main(int argc, char** argv) {
   std::printf("device: %s, %d CUs, %.0f MHz\n", prop.name, prop.multiProcessorCount, prop.clockRate / 1000.0);
   auto want = [&](char const* k) { return only.empty() || only == k; };
   if (only == "copy") benchCopy(warmup, iters);
+  if (only == "resnet50") {
+    benchResNet(warmup, iters, batch, false);
+    benchResNet(warmup, iters, batch, true);
+  }
   if (want("conv1")) benchConv("conv 5x5x3x32 on 32x32x3x100", 32, 32, 3, 100, 5, 32, 2, warmup, iters);
   if (want("bnorm")) benchBnorm(warmup, iters);
   if (want("maxpool")) benchPool(true, warmup, iters);

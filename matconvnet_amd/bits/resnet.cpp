@@ -1,0 +1,280 @@
+#include "resnet.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdlib>
+#include <random>
+
+#include "../../include/mcn_hip.h"
+#include "hiphelper.hpp"
+#include "nnbnorm.hpp"
+#include "nnconv.hpp"
+#include "nnpooling.hpp"
+
+namespace vl { namespace harness {
+
+namespace {
+double conv_flops(int outH, int outW, int fh, int fw, int cin, int cout) {
+  return 2.0 * outH * outW * fh * fw * cin * cout;
+}
+}  // namespace
+
+ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
+    : N(N), S(imageSize), classes(classes), epsilon(epsilon), fused(true), error(VLE_Success), flops(0) {
+  if (S < 32 || S % 32 != 0) {
+    error = VLE_IllegalArgument;
+    message = "the image size must be a multiple of 32";
+    return;
+  }
+  const int S2 = S / 2, S4 = S / 4;
+  make("input", TensorShape(S, S, 3, N));
+  make("stem.f", TensorShape(7, 7, 3, 64)); make("stem.g", TensorShape(64, 1, 1, 1)); make("stem.b", TensorShape(64, 1, 1, 1));
+  make("stem.a", TensorShape(S2, S2, 64, N)); make("stem.n", TensorShape(S2, S2, 64, N)); make("stem.r", TensorShape(S2, S2, 64, N));
+  make("stem.m", TensorShape(64, 2, 1, 1));
+  make("stem.p", TensorShape(S4, S4, 64, N));
+  make("stem.dp", TensorShape(S4, S4, 64, N)); make("stem.dr", TensorShape(S2, S2, 64, N)); make("stem.dn", TensorShape(S2, S2, 64, N));
+  make("stem.da", TensorShape(S2, S2, 64, N));
+  make("stem.df", TensorShape(7, 7, 3, 64)); make("stem.dg", TensorShape(64, 1, 1, 1)); make("stem.db", TensorShape(64, 1, 1, 1));
+  flops += conv_flops(S2, S2, 7, 7, 3, 64);
+
+  // sections 2..5 (cnn_imagenet_init_resnet.m:73-118)
+  static const int sectionLen[4] = {3, 4, 6, 3};
+  int H = S4, C = 64;
+  for (int s = 0; s < 4 && error == VLE_Success; ++s) {
+    const int depth = 64 << s, out = 256 << s;
+    for (int l = 0; l < sectionLen[s] && error == VLE_Success; ++l) {
+      const bool first = l == 0;
+      const int stride = (first && s >= 1) ? 2 : 1;
+      Bottleneck* u = new Bottleneck(H, H, C, depth, N, epsilon, out, stride, first, &context);
+      units.push_back(u);
+      if (!u->ok()) {
+        error = u->lastError();
+        message = u->lastMessage();
+        break;
+      }
+      const int Ho = u->outHeight();
+      flops += conv_flops(H, H, 1, 1, C, depth) + conv_flops(Ho, Ho, 3, 3, depth, depth) + conv_flops(Ho, Ho, 1, 1, depth, out);
+      if (first) flops += conv_flops(Ho, Ho, 1, 1, C, out);
+      H = Ho;
+      C = out;
+    }
+  }
+  if (error != VLE_Success) return;
+  // wiring: a unit's input is the previous unit's output; the derivative it receives is the next unit's dzdx
+  units[0]->alias("x", (float*)slot("stem.p").getMemory());
+  for (std::size_t i = 1; i < units.size(); ++i) units[i]->alias("x", units[i - 1]->buffer("y"));
+  for (std::size_t i = 0; i + 1 < units.size(); ++i) units[i]->alias("dzdy", units[i + 1]->buffer("dzdx"));
+  units[0]->alias("dzdx", (float*)slot("stem.dp").getMemory());
+
+  make("avg", TensorShape(1, 1, C, N)); make("davg", TensorShape(1, 1, C, N));
+  make("fc.f", TensorShape(1, 1, C, classes)); make("fc.b", TensorShape(classes, 1, 1, 1));
+  make("fc.df", TensorShape(1, 1, C, classes)); make("fc.db", TensorShape(classes, 1, 1, 1));
+  make("prediction", TensorShape(1, 1, classes, N)); make("dprediction", TensorShape(1, 1, classes, N));
+  flops += conv_flops(1, 1, 1, 1, C, classes);
+  setFused(true);
+}
+
+ResNet50::~ResNet50() {
+  for (std::size_t i = 0; i < units.size(); ++i) delete units[i];
+  for (std::size_t i = 0; i < slots.size(); ++i)
+    if (slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
+}
+
+Tensor ResNet50::make(std::string const& name, TensorShape const& shape) {
+  void* memory = NULL;
+  const std::size_t bytes = shape.getNumElements() * sizeof(float);
+  if (error == VLE_Success && hipMalloc(&memory, bytes ? bytes : 4) != hipSuccess) {
+    (void)hipGetLastError();
+    error = VLE_OutOfGPUMemeory;
+    message = "cannot allocate buffer '" + name + "'";
+    memory = NULL;
+  }
+  Slot s;
+  s.name = name;
+  s.tensor = Tensor(shape, VLDT_Float, VLDT_GPU, memory, bytes);
+  slots.push_back(s);
+  return s.tensor;
+}
+
+Tensor& ResNet50::slot(std::string const& name) {
+  for (std::size_t i = 0; i < slots.size(); ++i)
+    if (slots[i].name == name) return slots[i].tensor;
+  static Tensor none;
+  return none;
+}
+
+float* ResNet50::buffer(std::string const& name, std::size_t* count) {
+  if (name.compare(0, 4, "unit") == 0) {
+    const std::size_t dot = name.find('.');
+    if (dot == std::string::npos) return NULL;
+    const int i = std::atoi(name.substr(4, dot - 4).c_str());
+    if (i < 0 || i >= (int)units.size()) return NULL;
+    return units[i]->buffer(name.substr(dot + 1), count);
+  }
+  Tensor& t = slot(name);
+  if (count) *count = t.getNumElements();
+  return (float*)t.getMemory();
+}
+
+ErrorCode ResNet50::setStream(void* stream) { return context.getHipHelper().setStream(stream); }
+
+void ResNet50::setFused(bool on) {
+  fused = on;
+  for (std::size_t i = 0; i < units.size(); ++i) units[i]->setFused(on);
+}
+
+ErrorCode ResNet50::fail(ErrorCode e, char const* where) {
+  if (e != VLE_Success) {
+    error = e;
+    message = std::string(where) + ": " + context.getLastErrorMessage();
+  }
+  return e;
+}
+
+ErrorCode ResNet50::initParameters(unsigned long long seed) {
+  if (error != VLE_Success) return error;
+  std::mt19937_64 gen(seed);
+  std::normal_distribution<float> dist(0.f, 1.f);
+  std::vector<float> host;
+  auto upload = [&](float* dst, std::size_t n, float scale, float constant, bool random) -> bool {
+    host.resize(n);
+    for (std::size_t i = 0; i < n; ++i) host[i] = random ? scale * dist(gen) : constant;
+    return hipMemcpy(dst, host.data(), n * sizeof(float), hipMemcpyHostToDevice) == hipSuccess;
+  };
+  auto filter = [&](std::string const& name) -> bool {
+    std::size_t n = 0;
+    float* p = buffer(name, &n);
+    if (!p) return true;  // (a unit without adapter has no "fs")
+    // fan-in = elements per filter: the last extent of the bank is the number of filters
+    Tensor* t = NULL;
+    if (name.compare(0, 4, "unit") != 0) t = &slot(name);
+    std::size_t filters = t ? t->getSize() : 0;
+    if (!t) {
+      // bank shapes of a unit follow from its name
+      const std::size_t dot = name.find('.');
+      Bottleneck* u = units[std::atoi(name.substr(4, dot - 4).c_str())];
+      const std::string leaf = name.substr(dot + 1);
+      std::size_t m = 0, c3 = 0;
+      u->buffer("g1", &m);
+      u->buffer("g3", &c3);
+      filters = (leaf == "f1" || leaf == "f2") ? m : c3;
+    }
+    const float scale = std::sqrt(2.f / (float)(n / filters));
+    return upload(p, n, scale, 0.f, true);
+  };
+  auto constant = [&](std::string const& name, float value) -> bool {
+    std::size_t n = 0;
+    float* p = buffer(name, &n);
+    return !p || upload(p, n, 0.f, value, false);
+  };
+  bool good = filter("stem.f") && constant("stem.g", 1.f) && constant("stem.b", 0.f);
+  for (std::size_t i = 0; i < units.size() && good; ++i) {
+    const std::string u = "unit" + std::to_string(i) + ".";
+    good = filter(u + "f1") && filter(u + "f2") && filter(u + "f3") && filter(u + "fs");
+    for (char const* g : {"g1", "g2", "g3", "gs"}) good = good && constant(u + g, 1.f);
+    for (char const* b : {"b1", "b2", "b3", "bs"}) good = good && constant(u + b, 0.f);
+  }
+  good = good && filter("fc.f") && constant("fc.b", 0.f);
+  if (!good) {
+    (void)hipGetLastError();
+    message = "cannot upload the parameters";
+    return error = VLE_Cuda;
+  }
+  return VLE_Success;
+}
+
+#define STEP(stage, call)                                   \
+  do {                                                      \
+    ErrorCode e_ = (call);                                  \
+    if (e_ != VLE_Success) return fail(e_, stage);          \
+  } while (0)
+
+#define ABI(stage, call)                                                                    \
+  do {                                                                                      \
+    int rc_ = (call);                                                                       \
+    if (rc_ != 0) {                                                                         \
+      context.setError((ErrorCode)rc_, mcn_last_error_message());                           \
+      return fail((ErrorCode)rc_, stage);                                                   \
+    }                                                                                       \
+  } while (0)
+
+ErrorCode ResNet50::forward() {
+  if (error != VLE_Success) return error;
+  void* st = context.getHipHelper().getStream();
+  Tensor none;
+  const int S2 = S / 2;
+  nn::Convolution stem(context, 2, 2, 3, 3, 3, 3, 1, 1), fc(context, 1, 1, 0, 0, 0, 0, 1, 1);
+  nn::BatchNorm bn(context, epsilon);
+  nn::Pooling maxPool(context, 3, 3, 2, 2, 1, 1, 1, 1, nn::Pooling::Max);
+  STEP("stem conv", stem.forward(slot("stem.a"), 0, slot("input"), 1, slot("stem.f"), none));
+  if (fused) {
+    const size_t wsBytes = mcn_bnorm_workspace_bytes(S2, S2, 64, N);
+    void* ws = context.getWorkspace(VLDT_GPU, wsBytes);
+    if (!ws) return fail(context.getLastError(), "workspace");
+    ABI("stem bnorm", mcn_bnorm_forward_fused(st, (float*)slot("stem.r").getMemory(), (float*)slot("stem.m").getMemory(),
+                                              (float const*)slot("stem.a").getMemory(), (float const*)slot("stem.g").getMemory(),
+                                              (float const*)slot("stem.b").getMemory(), NULL, 1, S2, S2, 64, N, epsilon, 0, ws, wsBytes));
+  } else {
+    STEP("stem bnorm", bn.forward(slot("stem.n"), slot("stem.m"), slot("stem.a"), slot("stem.g"), slot("stem.b")));
+    ABI("stem relu", mcn_relu_forward(st, (float*)slot("stem.r").getMemory(), (float const*)slot("stem.n").getMemory(),
+                                      slot("stem.n").getNumElements()));
+  }
+  STEP("stem pool", maxPool.forward(slot("stem.p"), slot("stem.r")));
+  for (std::size_t i = 0; i < units.size(); ++i)
+    if (units[i]->forward() != VLE_Success) {
+      message = "unit " + std::to_string(i) + ": " + units[i]->lastMessage();
+      return error = units[i]->lastError();
+    }
+  Bottleneck* last = units.back();
+  const int Hf = last->outHeight(), Cf = last->outDepth();
+  Tensor features(TensorShape(Hf, Hf, Cf, N), VLDT_Float, VLDT_GPU, last->buffer("y"), sizeof(float) * (size_t)Hf * Hf * Cf * N);
+  nn::Pooling avgPool(context, Hf, Hf, 1, 1, 0, 0, 0, 0, nn::Pooling::Average);
+  STEP("average pool", avgPool.forward(slot("avg"), features));
+  STEP("classifier", fc.forward(slot("prediction"), 0, slot("avg"), 1, slot("fc.f"), slot("fc.b")));
+  return VLE_Success;
+}
+
+ErrorCode ResNet50::backward() {
+  if (error != VLE_Success) return error;
+  void* st = context.getHipHelper().getStream();
+  Tensor none;
+  const int S2 = S / 2;
+  nn::Convolution stem(context, 2, 2, 3, 3, 3, 3, 1, 1), fc(context, 1, 1, 0, 0, 0, 0, 1, 1);
+  nn::BatchNorm bn(context, epsilon);
+  nn::Pooling maxPool(context, 3, 3, 2, 2, 1, 1, 1, 1, nn::Pooling::Max);
+  Bottleneck* last = units.back();
+  const int Hf = last->outHeight(), Cf = last->outDepth();
+  const size_t nFeatures = (size_t)Hf * Hf * Cf * N;
+  Tensor features(TensorShape(Hf, Hf, Cf, N), VLDT_Float, VLDT_GPU, last->buffer("y"), sizeof(float) * nFeatures);
+  Tensor derFeatures(TensorShape(Hf, Hf, Cf, N), VLDT_Float, VLDT_GPU, last->buffer("dzdy"), sizeof(float) * nFeatures);
+  nn::Pooling avgPool(context, Hf, Hf, 1, 1, 0, 0, 0, 0, nn::Pooling::Average);
+  STEP("classifier", fc.backward(slot("davg"), slot("fc.df"), slot("fc.db"), slot("avg"), slot("fc.f"), slot("dprediction")));
+  STEP("average pool", avgPool.backwardOverwrite(derFeatures, features, slot("davg")));
+  for (std::size_t i = units.size(); i-- > 0;)
+    if (units[i]->backward() != VLE_Success) {
+      message = "unit " + std::to_string(i) + ": " + units[i]->lastMessage();
+      return error = units[i]->lastError();
+    }
+  STEP("stem pool", maxPool.backwardOverwrite(slot("stem.dr"), slot("stem.r"), slot("stem.dp")));
+  if (fused) {
+    const size_t wsBytes = mcn_bnorm_workspace_bytes(S2, S2, 64, N);
+    void* ws = context.getWorkspace(VLDT_GPU, wsBytes);
+    if (!ws) return fail(context.getLastError(), "workspace");
+    ABI("stem bnorm", mcn_bnorm_backward_relu(st, (float*)slot("stem.da").getMemory(), (float*)slot("stem.dg").getMemory(),
+                                              (float*)slot("stem.db").getMemory(), (float const*)slot("stem.m").getMemory(),
+                                              (float const*)slot("stem.a").getMemory(), (float const*)slot("stem.g").getMemory(),
+                                              (float const*)slot("stem.b").getMemory(), (float const*)slot("stem.dr").getMemory(),
+                                              S2, S2, 64, N, epsilon, ws, wsBytes));
+  } else {
+    ABI("stem relu", mcn_relu_backward(st, (float*)slot("stem.dn").getMemory(), (float const*)slot("stem.n").getMemory(),
+                                       (float const*)slot("stem.dr").getMemory(), slot("stem.dn").getNumElements()));
+    STEP("stem bnorm", bn.backwardWithMoment(slot("stem.da"), slot("stem.dg"), slot("stem.db"), slot("stem.m"), slot("stem.a"),
+                                             slot("stem.g"), slot("stem.b"), slot("stem.dn")));
+  }
+  // the network's input needs no derivative: filter gradient only
+  STEP("stem conv", stem.backward(none, slot("stem.df"), none, slot("input"), slot("stem.f"), slot("stem.da")));
+  return VLE_Success;
+}
+
+} }  // namespace vl::harness

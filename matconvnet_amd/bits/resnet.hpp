@@ -1,0 +1,60 @@
+// ResNet-50 forward + backward on the vl::nn operators: the network that
+// examples/imagenet/cnn_imagenet_init_resnet.m:52-134 builds (without the loss layers: the derivative with respect
+// to the prediction is an input).
+//   conv 7x7/2 3->64, bnorm, relu, max-pool 3x3/2 pad 1
+//   sections 2..5 of 3, 4, 6, 3 bottleneck segments, 64/128/256/512 channels inside and 4x that out; the first
+//   segment of a section has the conv + bnorm adapter on its shortcut and, from section 3 on, stride 2
+//   average pooling over the remaining extent (7x7 for 224x224 images), 1x1 convolution 2048 -> classes with bias
+// All buffers are allocated at construction; a step performs no allocation.
+#ifndef MCN_AMD_BITS_RESNET_HPP
+#define MCN_AMD_BITS_RESNET_HPP
+
+#include <string>
+#include <vector>
+
+#include "bottleneck.hpp"
+#include "data.hpp"
+
+namespace vl { namespace harness {
+
+class ResNet50 {
+ public:
+  // imageSize: input height = width (a multiple of 32); 224 gives the reference network
+  ResNet50(int N, double epsilon, int imageSize = 224, int classes = 1000);
+  ~ResNet50();
+  bool ok() const { return error == VLE_Success; }
+  std::string const& lastMessage() const { return message; }
+
+  // "input" (S x S x 3 x N), "prediction" / "dprediction" (1 x 1 x classes x N), the stem's "stem.f", "stem.g",
+  // "stem.b" and their derivatives "stem.df", ..., the classifier's "fc.f", "fc.b", "fc.df", "fc.db", and every
+  // buffer of segment i (0-based, in network order) as "unit<i>.<name>" (see Bottleneck::buffer)
+  float* buffer(std::string const& name, std::size_t* count = NULL);
+  int numUnits() const { return (int)units.size(); }
+  ErrorCode setStream(void* stream);
+  void setFused(bool on);
+  // He-normal filters (matlab/+dagnn/Conv.m:40 style), gains 1, biases 0, from a seeded generator on the host
+  ErrorCode initParameters(unsigned long long seed);
+  ErrorCode forward();
+  ErrorCode backward();
+  // forward FLOPs of all convolutions per image (2 per multiply-add); backward is twice that, minus the stem's dzdx
+  double convForwardFlopsPerImage() const { return flops; }
+
+ private:
+  struct Slot { std::string name; Tensor tensor; };
+  Tensor& slot(std::string const& name);
+  Tensor make(std::string const& name, TensorShape const& shape);
+  ErrorCode fail(ErrorCode e, char const* where);
+
+  int N, S, classes;
+  double epsilon;
+  bool fused;
+  Context context;
+  std::vector<Slot> slots;
+  std::vector<Bottleneck*> units;
+  ErrorCode error;
+  std::string message;
+  double flops;
+};
+
+} }  // namespace vl::harness
+#endif

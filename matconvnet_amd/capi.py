@@ -83,6 +83,9 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(
                 "%s is missing: build it with `python -m matconvnet_amd.build` (hipcc, gfx950)" % LIB_PATH)
+        # torch first: it brings a HIP runtime of its own, and device tensors are shared with it only when that
+        # runtime is the one already in the process when this library's dependency on libamdhip64 is resolved
+        import torch  # noqa: F401
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in PROTOTYPES.items():
             fn = getattr(L, name)

@@ -43,6 +43,9 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise RuntimeError("%s is missing: build it with `python -m matconvnet_amd.build`" % LIB_PATH)
+        # torch first: it brings a HIP runtime of its own, and device tensors are shared with it only when that
+        # runtime is the one already in the process when this library's dependency on libamdhip64 is resolved
+        import torch  # noqa: F401
         L = C.CDLL(LIB_PATH)
         L.vlh_call.restype = C.c_int
         L.vlh_call.argtypes = [C.c_char_p, C.c_int, C.POINTER(Arg), C.c_int, C.POINTER(Arg), ALLOC_FN, C.c_void_p, C.c_void_p]
@@ -66,6 +69,23 @@ def lib():
         L.vlh_bottleneck_run.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.POINTER(C.c_float)]
         L.vlh_bottleneck_message.restype = C.c_char_p
         L.vlh_bottleneck_message.argtypes = [C.c_void_p]
+        L.vlh_resnet50_create.restype = C.c_void_p
+        L.vlh_resnet50_create.argtypes = [C.c_int, C.c_double, C.c_int, C.c_int]
+        L.vlh_resnet50_destroy.argtypes = [C.c_void_p]
+        L.vlh_resnet50_destroy.restype = None
+        L.vlh_resnet50_units.argtypes = [C.c_void_p]
+        L.vlh_resnet50_buffer.restype = C.c_void_p
+        L.vlh_resnet50_buffer.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_size_t)]
+        L.vlh_resnet50_set_stream.argtypes = [C.c_void_p, C.c_void_p]
+        L.vlh_resnet50_set_fused.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_resnet50_set_fused.restype = None
+        L.vlh_resnet50_init.argtypes = [C.c_void_p, C.c_ulonglong]
+        L.vlh_resnet50_forward.argtypes = [C.c_void_p]
+        L.vlh_resnet50_backward.argtypes = [C.c_void_p]
+        L.vlh_resnet50_forward_flops.argtypes = [C.c_void_p]
+        L.vlh_resnet50_forward_flops.restype = C.c_double
+        L.vlh_resnet50_message.restype = C.c_char_p
+        L.vlh_resnet50_message.argtypes = [C.c_void_p]
         _lib = L
     return _lib
 
@@ -178,7 +198,90 @@ def vl_taccum(*args):
     return args[1] if inplace else r[0]
 
 
-class Bottleneck:
+class _NamedBuffers:
+    """Upload / download of the named device buffers a C++ harness object owns."""
+
+    def set(self, name, array):
+        """Upload a MATLAB-shaped numpy array (any order) into the named buffer."""
+        torch = _torch()
+        p, n = self._buf(name)
+        host = np.ascontiguousarray(np.asfortranarray(array, dtype=np.float32).T).ravel()
+        assert host.size == n, (name, host.size, n)
+        src = torch.from_numpy(host).cuda()
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        assert hip.hipMemcpy(p, src.data_ptr(), n * 4, 3) == 0  # device to device
+        torch.cuda.synchronize()
+
+    def get(self, name, mshape=None):
+        """Download the named buffer as a MATLAB-shaped array (flat when no shape is given)."""
+        torch = _torch()
+        p, n = self._buf(name)
+        dst = torch.empty(n, dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        assert hip.hipMemcpy(dst.data_ptr(), p, n * 4, 3) == 0
+        torch.cuda.synchronize()
+        if mshape is None:
+            return dst.cpu().numpy()
+        return np.asfortranarray(dst.cpu().numpy().reshape(tuple(reversed(mshape))).T)
+
+
+class ResNet50(_NamedBuffers):
+    """ResNet-50 forward + backward of the C++ harness (examples/imagenet/cnn_imagenet_init_resnet.m:52-134 without
+    the loss layers); buffers are owned by the C++ side and named "input", "prediction", "dprediction",
+    "stem.f", "fc.f", "unit<i>.<name>", ..."""
+
+    def __init__(self, N=32, eps=1e-5, image_size=224, classes=1000, fused=True, seed=None):
+        self.L = lib()
+        self.N, self.image_size, self.classes = N, image_size, classes
+        self.h = self.L.vlh_resnet50_create(N, eps, image_size, classes)
+        msg = self.L.vlh_resnet50_message(self.h).decode()
+        if msg:
+            self.close()
+            raise VlError(2, msg)
+        torch = _torch()
+        self._check(self.L.vlh_resnet50_set_stream(self.h, C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        self.L.vlh_resnet50_set_fused(self.h, int(fused))
+        if seed is not None:
+            self._check(self.L.vlh_resnet50_init(self.h, seed))
+
+    def close(self):
+        if self.h:
+            self.L.vlh_resnet50_destroy(self.h)
+            self.h = None
+
+    @property
+    def units(self):
+        return self.L.vlh_resnet50_units(self.h)
+
+    @property
+    def forward_flops_per_image(self):
+        return self.L.vlh_resnet50_forward_flops(self.h)
+
+    def set_fused(self, on):
+        self.L.vlh_resnet50_set_fused(self.h, int(on))
+
+    def _buf(self, name):
+        n = C.c_size_t(0)
+        p = self.L.vlh_resnet50_buffer(self.h, name.encode(), C.byref(n))
+        if not p:
+            raise KeyError(name)
+        return p, n.value
+
+    def _check(self, rc):
+        if rc != 0:
+            raise VlError(rc, self.L.vlh_resnet50_message(self.h).decode())
+
+    def forward(self):
+        self._check(self.L.vlh_resnet50_forward(self.h))
+
+    def backward(self):
+        self._check(self.L.vlh_resnet50_backward(self.h))
+
+
+class Bottleneck(_NamedBuffers):
     """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
 
     def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False, overlap=False, Cout=0, stride=1,
@@ -203,29 +306,6 @@ class Bottleneck:
         if not p:
             raise KeyError(name)
         return p, n.value
-
-    def set(self, name, array):
-        """Upload a MATLAB-shaped numpy array (any order) into the named buffer."""
-        torch = _torch()
-        p, n = self._buf(name)
-        host = np.ascontiguousarray(np.asfortranarray(array, dtype=np.float32).T).ravel()
-        assert host.size == n, (name, host.size, n)
-        src = torch.from_numpy(host).cuda()
-        hip = C.CDLL("libamdhip64.so")
-        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
-        assert hip.hipMemcpy(p, src.data_ptr(), n * 4, 3) == 0  # device to device
-        torch.cuda.synchronize()
-
-    def get(self, name, mshape):
-        torch = _torch()
-        p, n = self._buf(name)
-        dst = torch.empty(n, dtype=torch.float32, device="cuda")
-        torch.cuda.synchronize()
-        hip = C.CDLL("libamdhip64.so")
-        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
-        assert hip.hipMemcpy(dst.data_ptr(), p, n * 4, 3) == 0
-        torch.cuda.synchronize()
-        return np.asfortranarray(dst.cpu().numpy().reshape(tuple(reversed(mshape))).T)
 
     def _check(self, rc):
         if rc != 0:

@@ -78,6 +78,31 @@ def bottleneck_case(seed=5, H=56, W=56, C=256, M=64, N=32, eps=1e-5, Cout=None, 
     return w
 
 
+def resnet50_case(seed=9, image_size=64, N=4, classes=10, eps=1e-5):
+    """Parameters and inputs of ResNet-50 (examples/imagenet/cnn_imagenet_init_resnet.m:52-134): He-normal filters,
+    gains and biases a little away from 1 and 0 so that they matter, N(0,1) images and prediction derivative."""
+    r = np.random.default_rng(seed)
+    gain = lambda n: (1 + 0.1 * r.standard_normal(n)).astype(np.float32)
+    bias = lambda n: (0.1 * r.standard_normal(n)).astype(np.float32)
+    w = dict(eps=eps, input=_f(r.standard_normal((image_size, image_size, 3, N), dtype=np.float32)),
+             dprediction=_f(r.standard_normal((1, 1, classes, N), dtype=np.float32)),
+             stem=dict(f=he_normal(r, (7, 7, 3, 64)), g=gain(64), b=bias(64)), units=[])
+    C = 64
+    for s, length in enumerate((3, 4, 6, 3)):
+        M, Cout = 64 << s, 256 << s
+        for l in range(length):
+            first = l == 0
+            u = dict(f1=he_normal(r, (1, 1, C, M)), f2=he_normal(r, (3, 3, M, M)), f3=he_normal(r, (1, 1, M, Cout)),
+                     g1=gain(M), b1=bias(M), g2=gain(M), b2=bias(M), g3=gain(Cout), b3=bias(Cout), eps=eps,
+                     stride=2 if first and s >= 1 else 1, adapter=first)
+            if first:
+                u.update(fs=he_normal(r, (1, 1, C, Cout)), gs=gain(Cout), bs=bias(Cout))
+            w["units"].append(u)
+            C = Cout
+    w["fc"] = dict(f=he_normal(r, (1, 1, C, classes)), b=bias(classes))
+    return w
+
+
 def conv_vgg(seed=6, H=56, W=56, C=256, K=256, N=64):
     """VGG-style wide 3x3 conv backward: x N(0,1), f He-normal 3x3xCxK, stride 1, pad 1."""
     r = np.random.default_rng(seed)

@@ -43,3 +43,10 @@ def capi():
     from matconvnet_amd import capi as c
     c.lib()  # raises if the HIP library is missing: there is no fallback
     return c
+
+
+@pytest.fixture(scope="session")
+def vl():
+    from matconvnet_amd import vlapi
+    vlapi.lib()  # raises if the C++ operator library is missing: there is no fallback
+    return vlapi

@@ -11,13 +11,6 @@ from util import F, bits_equal, rel_max
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def vl():
-    from matconvnet_amd import vlapi
-    vlapi.lib()
-    return vlapi
-
-
 def dev(a):
     return torch.from_numpy(np.ascontiguousarray(np.asfortranarray(a, dtype=np.float32).T)).cuda()
 

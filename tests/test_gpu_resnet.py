@@ -1,0 +1,185 @@
+"""ResNet-50 forward + backward driven through the C++ operator classes (examples/imagenet/cnn_imagenet_init_resnet.m:
+52-134), at reduced image size, against the network composed from oracle operators."""
+import numpy as np
+import pytest
+
+from matconvnet_amd import workloads
+from util import bits_equal, rel_max
+
+pytestmark = pytest.mark.gpu
+
+S, N, CLASSES = 64, 4, 10
+UNIT_PARAMS = ("f1", "f2", "f3", "g1", "b1", "g2", "b2", "g3", "b3")
+ADAPTER_PARAMS = ("fs", "gs", "bs")
+
+
+def _load(net, w):
+    net.set("input", w["input"])
+    net.set("dprediction", w["dprediction"])
+    for k in "fgb":
+        net.set("stem." + k, w["stem"][k])
+    for i, u in enumerate(w["units"]):
+        for k in UNIT_PARAMS + (ADAPTER_PARAMS if u["adapter"] else ()):
+            net.set("unit%d.%s" % (i, k), u[k])
+    net.set("fc.f", w["fc"]["f"])
+    net.set("fc.b", w["fc"]["b"])
+
+
+def _gradient_names(w):
+    names = ["prediction", "fc.df", "fc.db", "stem.df", "stem.dg", "stem.db"]
+    for i, u in enumerate(w["units"]):
+        names += ["unit%d.d%s" % (i, k) for k in UNIT_PARAMS + (ADAPTER_PARAMS if u["adapter"] else ())]
+        names += ["unit%d.y" % i, "unit%d.dzdx" % i]
+    return names
+
+
+@pytest.fixture(scope="module")
+def case():
+    return workloads.resnet50_case(seed=9, image_size=S, N=N, classes=CLASSES)
+
+
+@pytest.fixture(scope="module")
+def runs(vl, case):
+    """Every output buffer of the network after two forward + backward passes, layer by layer and fused."""
+    out = {}
+    for mode in ("plain", "fused"):
+        net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=mode == "fused")
+        try:
+            assert net.units == 16
+            _load(net, case)
+            for _ in range(2):
+                net.forward()
+                net.backward()
+            got = {k: net.get(k) for k in _gradient_names(case)}
+            got["stem.p"] = net.get("stem.p")
+            got["stem.dp"] = net.get("stem.dp")
+            got["unit15.dzdy"] = net.get("unit15.dzdy")
+            if mode == "plain":   # the tensors ReLU and max pooling take their masks from
+                got["stem.n"], got["stem.r"] = net.get("stem.n"), net.get("stem.r")
+                for i in range(net.units):
+                    for k in ("n1", "n2", "s"):
+                        got["unit%d.%s" % (i, k)] = net.get("unit%d.%s" % (i, k))
+            out[mode] = got
+        finally:
+            net.close()
+    return out
+
+
+def test_fused_schedule_is_bit_identical(runs, case):
+    for k in _gradient_names(case):
+        assert bits_equal(runs["plain"][k], runs["fused"][k]), k
+
+
+def test_prediction_end_to_end(runs, case, ob):
+    """Forward pass of the whole network against the oracle network (float and double)."""
+    from oracle import blocks
+    want = blocks.resnet50(case, np.float64)
+    got = runs["plain"]["prediction"].reshape(want["prediction"].shape, order="F")
+    assert np.isfinite(got).all()
+    assert rel_max(got, want["prediction"]) < 1e-3
+
+
+def test_stage_by_stage_against_oracle(runs, case, ob):
+    """ReLU's derivative is discontinuous and the deepest sections normalise over few samples, so the gradients of
+    the whole network are not a continuous function of rounding error (the oracle in float and in double differ by
+    several percent there).  Each stage is therefore checked on the inputs the device network actually gave it: the
+    stage's input and incoming derivative are read back from the device, the oracle stage runs on them in double, and
+    every output of the device's stage is compared.  A stage's input buffer is its predecessor's output buffer, so the
+    chain of checks covers the wiring as well.  Inside a stage the tensors that ReLU and max pooling derive their masks
+    from are compared with the oracle's and then taken from the device, so that a value within rounding of zero (or
+    of its neighbour in a pooling window) selects the same elements on both sides."""
+    from oracle import binding
+    from oracle import blocks
+    G = runs["plain"]
+    f64 = lambda a: np.asfortranarray(a, dtype=np.float64) if a.ndim > 1 else a.astype(np.float64)
+    shaped = lambda name, like: G[name].reshape(like.shape, order="F")
+    errs = {}
+
+    # stem: input -> pooled map; pooled derivative -> parameter derivatives
+    st, eps = case["stem"], case["eps"]
+    x = f64(case["input"])
+    g0 = binding.conv_geom(x.shape, st["f"].shape, 2, 3, 1)
+    a0 = binding.conv_forward(x, f64(st["f"]), None, g0)
+    n0, m0 = binding.bnorm_forward(a0, f64(st["g"]), f64(st["b"]), eps)
+    r0 = binding.relu_forward(n0)
+    gp = binding.pool_geom(r0.shape, 3, 2, 1, "max")
+    p0 = binding.pool_forward(r0, gp)
+    assert p0.shape == (S // 4, S // 4, 64, N)
+    errs["stem.p"] = rel_max(shaped("stem.p", p0), p0)
+    errs["stem.n"] = rel_max(shaped("stem.n", n0), n0)
+    errs["stem.r"] = rel_max(shaped("stem.r", r0), r0)
+    n0, r0 = f64(shaped("stem.n", n0)), f64(shaped("stem.r", r0))
+    dp = f64(shaped("stem.dp", p0))
+    dr0 = binding.pool_backward(r0, dp, gp)
+    dn0 = binding.relu_backward(n0, dr0)
+    da0, dg0, db0, _ = binding.bnorm_backward(a0, f64(st["g"]), dn0, eps, moments=m0)
+    _, df0, _ = binding.conv_backward(x, f64(st["f"]), da0, g0, want=(False, True, False))
+    errs["stem.df"] = rel_max(shaped("stem.df", df0), df0)
+    errs["stem.dg"] = rel_max(G["stem.dg"], dg0)
+    errs["stem.db"] = rel_max(G["stem.db"], db0)
+
+    # units: input = the device's previous output, incoming derivative = the device's next dzdx
+    h = f64(shaped("stem.p", p0))
+    states = []
+    for i, u in enumerate(case["units"]):
+        t = blocks.unit_forward(u, h, np.float64)
+        states.append(t)
+        errs["unit%d.y" % i] = rel_max(shaped("unit%d.y" % i, t["y"]), t["y"])
+        for k in ("n1", "n2", "s"):
+            name = "unit%d.%s" % (i, k)
+            errs[name] = rel_max(shaped(name, t[k]), t[k])
+            t[k] = f64(shaped(name, t[k]))
+        h = f64(shaped("unit%d.y" % i, t["y"]))
+    last = states[-1]["y"]
+    assert last.shape == (S // 32, S // 32, 2048, N)
+    for i, u in enumerate(case["units"]):
+        nxt = "unit%d.dzdx" % (i + 1) if i + 1 < len(case["units"]) else "unit15.dzdy"
+        dy = f64(G[nxt].reshape(states[i]["y"].shape, order="F"))
+        g = blocks.unit_backward(u, states[i], dy, np.float64)
+        for k, v in g.items():
+            name = "unit%d.%s" % (i, k)
+            errs[name] = rel_max(G[name].reshape(v.shape, order="F"), v)
+    # the first unit's dzdx is the buffer the stem reads
+    assert bits_equal(G["unit0.dzdx"], G["stem.dp"])
+
+    # head: average pooling over the whole map, 1x1 convolution with bias
+    ga = binding.pool_geom(h.shape, (h.shape[0], h.shape[1]), 1, 0, "avg")
+    avg = binding.pool_forward(h, ga)
+    ff, fb = f64(case["fc"]["f"]), f64(case["fc"]["b"])
+    gf = binding.conv_geom(avg.shape, ff.shape, 1, 0, 1)
+    pred = binding.conv_forward(avg, ff, fb, gf)
+    errs["prediction"] = rel_max(shaped("prediction", pred), pred)
+    davg, dff, dfb = binding.conv_backward(avg, ff, f64(case["dprediction"]), gf)
+    dlast = binding.pool_backward(h, davg, ga)
+    errs["fc.df"] = rel_max(shaped("fc.df", dff), dff)
+    errs["fc.db"] = rel_max(G["fc.db"], dfb)
+    errs["unit15.dzdy"] = rel_max(shaped("unit15.dzdy", dlast), dlast)
+
+    worst = sorted(errs.items(), key=lambda kv: -kv[1])[:6]
+    print("ResNet-50 %dx%d N=%d, worst stage errors:" % (S, S, N), {k: "%.1e" % v for k, v in worst})
+    assert all(np.isfinite(v) for v in errs.values())
+    assert max(errs.values()) < 1e-4, worst
+
+
+def test_seeded_initialisation_runs_at_full_image_size(vl):
+    """224 x 224 images, 1000 classes, N = 2: the reference geometry end to end (7 x 7 average pooling, finite outputs,
+    gradients that are not identically zero)."""
+    net = vl.ResNet50(N=2, eps=1e-5, image_size=224, classes=1000, fused=True, seed=3)
+    try:
+        r = np.random.default_rng(4)
+        net.set("input", np.asfortranarray(r.standard_normal((224, 224, 3, 2), dtype=np.float32)))
+        net.set("dprediction", np.asfortranarray(r.standard_normal((1, 1, 1000, 2), dtype=np.float32)))
+        net.forward()
+        net.backward()
+        assert abs(net.forward_flops_per_image / 1e9 - 8.178) < 0.001   # 4.09 G multiply-adds
+        for name in ("prediction", "stem.df", "unit0.dfs", "unit7.df2", "unit15.dg3", "fc.df", "fc.db"):
+            v = net.get(name)
+            assert np.isfinite(v).all() and np.abs(v).max() > 0, name
+    finally:
+        net.close()
+
+
+def test_image_size_must_be_a_multiple_of_32(vl):
+    from matconvnet_amd.vlapi import VlError
+    with pytest.raises(VlError, match="multiple of 32"):
+        vl.ResNet50(N=1, image_size=100)
