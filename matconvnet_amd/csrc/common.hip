@@ -31,6 +31,9 @@ Tunable g_tunables[] = {
     {"conv_ws_min_units", 0},          // least number of units for the weights-stationary kernel; 0 = two per SIMD
     {"conv_ws_wa", 0},                 // 1, 2, 4: force its channels-per-wavefront (in units of 32); 0 = choose
     {"conv_no_split", 0},              // 1: the tiled kernel never splits its reduction over workgroups
+    {"conv_split_max_blocks", 512},    // ... it splits when the unsplit launch has at most this many workgroups,
+    {"conv_split_target", 1024},       // aiming at this many workgroups in all,
+    {"conv_split_min_steps", 16},      // with at least this many 16-row steps left to each
     {"conv_no_fc_view", 0},            // 1: fully-connected layers are not recast as 1x1 layers
     {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels
     {"conv_pix_tile", 0},              // force a tile shape of the pixel-major MFMA kernel (0 = automatic)

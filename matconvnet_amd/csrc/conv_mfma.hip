@@ -79,19 +79,24 @@ __global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt,
   wt[idx] = v;
 }
 
-// out = alpha * (sum of the partial results of a split reduction) + beta*out + bias, element by element of a dense
-// output tensor [n][co][q].  The partials are added in split order: deterministic.
+// out = alpha * (sum of the partial results of a split reduction) + beta*out + bias.  The partials are dense tensors
+// [n][co][q]; the destination is the layout the PixP describes (a dense tensor, one group's channels of a wider
+// tensor, or one stride class of a backward-data product).  The partials are added in split order: deterministic.
 __global__ __launch_bounds__(256) void conv_pix_reduce(float* __restrict__ out, const float* __restrict__ partials,
-                                                       const float* __restrict__ bias, size_t n, long long partStride,
-                                                       int splits, float alpha, float beta, int Q, int Cout) {
+                                                       const float* __restrict__ bias, size_t n, PixP p) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float s = partials[i];
-  for (int k = 1; k < splits; ++k) s += partials[(size_t)k * partStride + i];
-  float v = alpha * s;
-  if (beta != 0.f) v = fmaf(beta, out[i], v);
-  if (bias) v += bias[(i / Q) % Cout];
-  out[i] = v;
+  for (int k = 1; k < p.rSplits; ++k) s += partials[(size_t)k * p.partStride + i];
+  const int Q = p.OH * p.OW;
+  const size_t plane = i / Q;
+  const int q = (int)(i - plane * Q), co = (int)(plane % p.Cout);
+  const size_t img = plane / p.Cout;
+  float* dst = out + img * (size_t)p.outImg + (size_t)co * p.outPlane + out_pixel_offset(p, q);
+  float v = p.alpha * s;
+  if (p.beta != 0.f) v = fmaf(p.beta, *dst, v);
+  if (bias) v += bias[co];
+  *dst = v;
 }
 
 // UT ("uniform tap"): Cin is a multiple of 16 and the reduction runs in chunks of 16 channels, tap by tap inside
@@ -752,7 +757,7 @@ struct PixPlan {
   int splits;
 };
 
-PixPlan plan_pix(int Cout, long long M, int R, bool dense) {
+PixPlan plan_pix(int Cout, long long M, int R) {
   PixPlan plan;
   const int BA = pick_channels_tile(Cout);
   const long long tilesA = (Cout + BA - 1) / BA;
@@ -763,14 +768,17 @@ PixPlan plan_pix(int Cout, long long M, int R, bool dense) {
   if (BA == 128) { plan.shape = M <= 32 ? 7 : (blocks(128) >= 2048 ? 1 : 5); px = plan.shape == 7 ? 32 : (plan.shape == 1 ? 128 : 64); }
   else if (BA == 64) { plan.shape = blocks(256) >= 2048 ? 2 : (blocks(128) >= 2048 ? 4 : 6); px = plan.shape == 2 ? 256 : (plan.shape == 4 ? 128 : 64); }
   else { plan.shape = 3; px = 256; }
-  // few workgroups with a long reduction each: split it, down to 8 steps of 16 rows per workgroup, until about two
-  // workgroups per CU exist
+  // fewer than two workgroups per CU with a long reduction each: split it, down to 16 steps of 16 rows per
+  // workgroup, until about four workgroups per CU exist (values from a sweep over the 14x14 and 7x7 layers of
+  // ResNet-50 at 32 images: 126 -> 89 us for 3x3x256x256)
   plan.splits = 1;
   const long long nb = blocks(px);
   const int nSteps = (R + 15) / 16;
-  if (dense && nb <= 128 && nSteps >= 32 && !tunable("conv_no_split", 0)) {
-    long long want = (512 + nb - 1) / nb;
-    plan.splits = (int)std::max<long long>(1, std::min<long long>(want, nSteps / 8));
+  const int maxBlocks = tunable("conv_split_max_blocks", 512), target = tunable("conv_split_target", 1024),
+            minSteps = tunable("conv_split_min_steps", 16);
+  if (nb <= maxBlocks && nSteps >= 4 * minSteps && !tunable("conv_no_split", 0)) {
+    long long want = (target + nb - 1) / nb;
+    plan.splits = (int)std::max<long long>(1, std::min<long long>(want, nSteps / minSteps));
   }
   return plan;
 }
@@ -782,7 +790,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   const int BA = pick_channels_tile(p.Cout);
   const int rPad = (p.R + 15) / 16 * 16;
   p.coutPad = (p.Cout + BA - 1) / BA * BA;
-  const PixPlan plan = plan_pix(p.Cout, p.M, p.R, p.dense != 0 && p.outImg == p.Cout * p.outPlane);
+  const PixPlan plan = plan_pix(p.Cout, p.M, p.R);
   const size_t nOut = (size_t)p.N * p.Cout * p.OH * p.OW;
   const size_t needW = (size_t)rPad * p.coutPad * sizeof(float);
   const size_t need = plan.splits > 1 ? align256(needW) + (size_t)plan.splits * nOut * sizeof(float) : needW;
@@ -830,19 +838,41 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
     q.partStride = (long long)nOut;
     q.alpha = 1.f;
     q.beta = 0.f;
+    // the partial tensors are dense whatever the destination's layout is
+    q.outPlane = q.OH * q.OW;
+    q.outImg = q.Cout * q.outPlane;
+    q.outOff = 0; q.outSH = 1; q.outSW = q.OH; q.dense = 1;
     {
       const long long ob = (long long)nOut * 4;
       q.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
     }
     launch_shape(s, plan.shape, partials, in, wt, nullptr, q, ut);
     if ((rc = check_launch(who))) return rc;
+    p.rSplits = q.rSplits;
+    p.partStride = q.partStride;
     KernelTimer timer("conv_pix_reduce", s);
-    hipLaunchKernelGGL(conv_pix_reduce, dim3((unsigned)((nOut + 255) / 256)), dim3(256), 0, s, out, partials, bias, nOut,
-                       q.partStride, q.rSplits, p.alpha, p.beta, p.OH * p.OW, p.Cout);
+    hipLaunchKernelGGL(conv_pix_reduce, dim3((unsigned)((nOut + 255) / 256)), dim3(256), 0, s, out, partials, bias, nOut, p);
     return check_launch(who);
   }
   launch_shape(s, plan.shape, out, in, wt, bias, p, ut);
   return check_launch(who);
+}
+
+int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
+
+// One axis of a stride class of the backward-data product (see backward_data_group): the taps that take part are
+// first, first + step, ... (count of them); the gathered position starts at dBase and moves by dStep per tap.
+struct Axis { int first, step, count, dBase, dStep; };
+Axis stride_axis(int phase, int pad, int dil, int stride, int taps) {
+  Axis a;
+  a.step = stride / gcd_int(dil, stride);
+  a.first = -1;
+  for (int i = 0; i < taps && i < a.step; ++i)
+    if ((phase + pad - i * dil) % stride == 0) { a.first = i; break; }
+  a.count = a.first < 0 ? 0 : (taps - a.first + a.step - 1) / a.step;
+  a.dBase = a.first < 0 ? 0 : (phase + pad - a.first * dil) / stride;  // exact: the numerator is a multiple of stride
+  a.dStep = -(a.step * dil) / stride;                                   // exact likewise
+  return a;
 }
 
 }  // namespace
@@ -856,20 +886,29 @@ size_t conv_mfma_workspace_bytes(const ConvP& original, int product) {
   const ConvP p = group_view(layer);  // the groups run one after the other through the same workspace
   const size_t FV = (size_t)p.FH * p.FW * p.FC;
   // packed bank, plus the partial results when the tiled kernel splits the reduction (plan_pix)
-  auto pix_need = [&](int Cout, long long M, int R, bool dense) {
+  auto pix_need = [&](int Cout, long long M, int R) {
     const int BA = pick_channels_tile(Cout);
     const size_t needW = ((size_t)(R + 15) / 16 * 16) * (size_t)((Cout + BA - 1) / BA * BA) * sizeof(float);
-    const PixPlan plan = plan_pix(Cout, M, R, dense);
+    const PixPlan plan = plan_pix(Cout, M, R);
     return plan.splits > 1 ? align256(needW) + (size_t)plan.splits * (size_t)M * Cout * sizeof(float) : needW;
   };
   switch (product) {
     case MCN_CONV_FORWARD: {
       if (!conv_mfma_forward_supported(layer)) return 0;
-      return pix_need(p.K, (long long)p.outH * p.outW * p.N, (int)FV, layer.groups == 1);
+      return pix_need(p.K, (long long)p.outH * p.outW * p.N, (int)FV);
     }
     case MCN_CONV_BACKWARD_DATA: {
       if (!conv_mfma_backward_data_supported(layer)) return 0;
-      return pix_need(p.C, (long long)p.H * p.W * p.N, p.FH * p.FW * p.K, layer.groups == 1 && p.sy == 1 && p.sx == 1);
+      // the largest need of any stride class (one class, all taps, when the strides are 1)
+      size_t need = 0;
+      for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
+        for (int ph = 0; ph < p.sy && ph < p.H; ++ph) {
+          const Axis ai = stride_axis(ph, p.pt, p.dy, p.sy, p.FH), aj = stride_axis(pw, p.pl, p.dx, p.sx, p.FW);
+          if (ai.count == 0 || aj.count == 0) continue;
+          const long long M = (long long)((p.H - ph + p.sy - 1) / p.sy) * ((p.W - pw + p.sx - 1) / p.sx) * p.N;
+          need = std::max(need, pix_need(p.C, M, ai.count * aj.count * p.K));
+        }
+      return need;
     }
     case MCN_CONV_BACKWARD_FILTER: {
       if (!conv_mfma_backward_filter_supported(layer)) return 0;
@@ -897,7 +936,6 @@ void dense_layout(PixP* q) {
   q->outOff = 0; q->outSH = 1; q->outSW = q->OH; q->dense = 1;
 }
 
-int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
 
 }  // namespace
 
@@ -943,19 +981,6 @@ int conv_forward_mfma(hipStream_t s, const ConvP& original, float* y, float outM
 // position moves by one per pixel of the class, so each class is the same gather product over a sub-grid of dzdx
 // with a subset of the taps.  Classes no tap reaches (1x1 filters with stride 2: three of four) are zeros.
 namespace {
-struct Axis { int first, step, count, dBase, dStep; };
-Axis stride_axis(int phase, int pad, int dil, int stride, int taps) {
-  Axis a;
-  a.step = stride / gcd_int(dil, stride);
-  a.first = -1;
-  for (int i = 0; i < taps && i < a.step; ++i)
-    if ((phase + pad - i * dil) % stride == 0) { a.first = i; break; }
-  a.count = a.first < 0 ? 0 : (taps - a.first + a.step - 1) / a.step;
-  a.dBase = a.first < 0 ? 0 : (phase + pad - a.first * dil) / stride;  // exact: the numerator is a multiple of stride
-  a.dStep = -(a.step * dil) / stride;                                   // exact likewise
-  return a;
-}
-
 int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float dxMult, const float* f, const float* dy,
                         void* ws, size_t wsBytes) {
   PixP q;
