@@ -801,8 +801,12 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   // uniform-tap variant: whole 16-row steps inside one tap, and 32-bit element offsets into the gathered tensor
   const long long inSpan = (long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW;  // elements from `in` to the end
   const bool ut = p.Cin % 16 == 0 && inSpan < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
-  int rc;
-  {
+  int rc = MCN_SUCCESS;
+  // The backward-data product of a 1x1 bank whose extents need no padding reads it as it is stored: rows = filters,
+  // columns = the filters' channels, which is the packed order.
+  if (backward && taps.FH * taps.FW == 1 && rPad == p.R && p.coutPad == p.Cout && aligned16(f)) {
+    wt = const_cast<float*>(f);
+  } else {
     KernelTimer timer("conv_pack_weights", s);
     hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, wt, f, taps, p.Cin, p.Cout,
                        rPad, p.coutPad, backward, ut ? 1 : 0);

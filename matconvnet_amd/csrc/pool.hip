@@ -99,6 +99,16 @@ __device__ __forceinline__ int cover_range(int h, int pad, int pool, int stride,
   return (lo & 0xffff) | (hi << 16);
 }
 
+// Average pooling whose single window covers the whole plane: dx = [dx +] dy[plane] * (1 / (H*W)).
+__global__ __launch_bounds__(256) void pool_avg_backward_whole(float* __restrict__ dx, const float* __restrict__ dy,
+                                                               unsigned total, unsigned planeSize, int accumulate) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= total) return;
+  const float scale = 1.0f / (float)planeSize;  // as avg_scale: correctly rounded IEEE division
+  const float v = dy[i / planeSize] * scale;
+  dx[i] = (accumulate ? dx[i] : 0.0f) + v;  // (0 + v, as the general kernels' sum starts: -0 becomes +0)
+}
+
 // KH, KW: upper bounds on the number of output rows / columns covering one input element
 // (ceil(pool/stride)); 0 selects run-time loops.  With compile-time bounds the candidate loads are issued
 // together and the adds are predicated, which keeps the reference's addition order.
@@ -851,6 +861,16 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
   // ---- max pooling, plane height a multiple of 4: streaming kernel
   if (isMax && pool_max_backward_stream_launch(s, g, p.outH, p.outW, derInput, x, derOutput, accumulate))
     return check_launch("mcn_pool_backward");
+
+  // ---- average over one window that covers the whole plane (the pooling before a network's classifier): every
+  //      element receives its plane's dzdy / (H*W), the single contribution the general kernels would add
+  if (!isMax && p.outH == 1 && p.outW == 1 && p.poolH - p.pt >= p.H && p.poolW - p.pl >= p.W && total < (1ull << 32) &&
+      !tunable("pool_force_gather", 0)) {
+    KernelTimer timer("pool_avg_backward_whole", s);
+    hipLaunchKernelGGL(pool_avg_backward_whole, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, derInput, derOutput,
+                       (unsigned)total, (unsigned)(p.H * p.W), p.accumulate);
+    return check_launch("mcn_pool_backward");
+  }
 
   // ---- ordered passes.  Widest tile whose LDS fits the budget and whose outputs fit 4 per thread.
   if (passes <= 16 && p.poolH <= 8 && p.poolW <= 8 && !tunable("pool_force_gather", 0)) {

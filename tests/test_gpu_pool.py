@@ -143,6 +143,33 @@ def test_large_windows_and_sparse_strides(capi, ob, method, geom):
     assert bits_equal(got, want), count_bit_mismatches(got, want)
 
 
+@pytest.mark.parametrize("geom", [(7, 7, 5, 3, 7, 1, 0), (6, 9, 3, 2, (6, 9), (1, 1), 0), (5, 4, 2, 2, (7, 6), (2, 3), (1, 1, 1, 1)),
+                                  (4, 4, 2, 2, (5, 5), (1, 1), (0, 1, 0, 1))])
+def test_average_over_the_whole_plane(capi, ob, geom):
+    """One window covering the plane (the pooling before a classifier) has a kernel of its own: same bits as the
+    oracle and as the general kernel, overwriting and accumulating, zeros of either sign included."""
+    H, W, C, N, pool, stride, pad = geom
+    shape = (H, W, C, N)
+    x = _inputs(shape, 41, "normal")
+    og = ob.pool_geom(shape, pool, stride, pad, "avg")
+    assert ob.pool_out_shape(og)[:2] == (1, 1)
+    dy = F(np.random.default_rng(42).standard_normal(ob.pool_out_shape(og)))
+    dy[0, 0, 0, 0] = -0.0
+    base = F(np.random.default_rng(43).standard_normal(shape))
+    outs = []
+    for force in (0, 1):
+        try:
+            capi.set_tunable("pool_force_gather", force)
+            got, want = _run(capi, ob, x, dy, shape, pool, stride, pad, "avg")
+            assert bits_equal(got, want)
+            got2, want2 = _run(capi, ob, x, dy, shape, pool, stride, pad, "avg", accumulate_into=base)
+            assert bits_equal(got2, want2)
+            outs.append((got, got2))
+        finally:
+            capi.set_tunable("pool_force_gather", 0)
+    assert bits_equal(outs[0][0], outs[1][0]) and bits_equal(outs[0][1], outs[1][1])
+
+
 def test_golden_vectors_from_reference(capi):
     z = np.load(GOLDEN)
     for i in range(int(z["count"])):
