@@ -247,6 +247,21 @@ MCN_API int mcn_add(mcn_stream_t stream, float* y, const float* a, const float* 
    BLAS axpy; examples/cnn_train_dag.m:316-378).  y may be a (the MEX's 'InPlace' mode).  Each element goes through
    the roundings of that pair: t = fl(alpha*a), y = fl(t + fl(beta*b)). */
 MCN_API int mcn_taccum(mcn_stream_t stream, float* y, float alpha, const float* a, float beta, const float* b, size_t n);
+/* SGD with momentum, the default solver of examples/cnn_train_dag.m:335-364, over all parameters of a network in one
+   launch instead of three vl_taccum calls per parameter.  value / state / der are arenas of `chunks` chunks of
+   MCN_SGD_CHUNK floats; each parameter occupies whole chunks (padded with zeros), chunk c belongs to parameter
+   chunkParam[c] (device array), and rates[2p], rates[2p+1] (device array of doubles) are that parameter's learningRate
+   and weightDecay multipliers (net.params(p).learningRate / .weightDecay).  Per element, with
+   thisLR = (float)(learningRate*rates[2p]), thisDecay = (float)(weightDecay*rates[2p+1]) and the roundings of the
+   reference's calls (each vl_taccum is t = fl(alpha*a), y = fl(t + fl(beta*b))):
+     d     = vl_taccum(derScale, der, thisDecay, value)        derScale = 1/numWorkers (:344)
+     state = vl_taccum(momentum, state, -1, d)                 (:350)
+     value = vl_taccum(1, value, thisLR, nesterov ? fl(fl(momentum*state) - d) : state)   (:355-362)
+   Parameters with thisLR = thisDecay = 0 are left alone (:342).  der is not modified. */
+#define MCN_SGD_CHUNK 1024
+MCN_API int mcn_sgd_momentum(mcn_stream_t stream, float* value, float* state, const float* der, size_t chunks,
+                             const unsigned short* chunkParam, const double* rates, double learningRate,
+                             double weightDecay, double momentum, double derScale, int nesterov);
 /* y[i] = value   (bits/impl/copy_gpu.cu:17-33 fill) */
 MCN_API int mcn_fill(mcn_stream_t stream, float* y, float value, size_t n);
 

@@ -236,6 +236,10 @@ void vlh_resnet50_set_fused(void* net, int fused) { ((harness::ResNet50*)net)->s
 int vlh_resnet50_init(void* net, unsigned long long seed) { return (int)((harness::ResNet50*)net)->initParameters(seed); }
 int vlh_resnet50_forward(void* net) { return (int)((harness::ResNet50*)net)->forward(); }
 int vlh_resnet50_backward(void* net) { return (int)((harness::ResNet50*)net)->backward(); }
+int vlh_resnet50_sgd_step(void* net, double learningRate, double momentum, double weightDecay) {
+  return (int)((harness::ResNet50*)net)->sgdStep(learningRate, momentum, weightDecay);
+}
+size_t vlh_resnet50_parameters(void* net) { return ((harness::ResNet50*)net)->numParameters(); }
 double vlh_resnet50_forward_flops(void* net) { return ((harness::ResNet50*)net)->convForwardFlopsPerImage(); }
 const char* vlh_resnet50_message(void* net) { return ((harness::ResNet50*)net)->lastMessage().c_str(); }
 

@@ -70,6 +70,11 @@ VLH_API void vlh_resnet50_set_fused(void* net, int fused);
 VLH_API int vlh_resnet50_init(void* net, unsigned long long seed);
 VLH_API int vlh_resnet50_forward(void* net);
 VLH_API int vlh_resnet50_backward(void* net);
+/* SGD with momentum and weight decay on all parameters (one worker) and the moving average of the batch moments, as
+   examples/cnn_train_dag.m:316-364 with the rates of cnn_imagenet_init_resnet.m:178-195; buffers "momentum.<parameter>"
+   and "running.<moments>" hold the solver state */
+VLH_API int vlh_resnet50_sgd_step(void* net, double learningRate, double momentum, double weightDecay);
+VLH_API size_t vlh_resnet50_parameters(void* net);
 /* forward FLOPs of the convolutions for one image */
 VLH_API double vlh_resnet50_forward_flops(void* net);
 VLH_API const char* vlh_resnet50_message(void* net);

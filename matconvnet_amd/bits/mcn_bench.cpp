@@ -249,11 +249,15 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
   };
   double tf = medianMs([&] { if (net.forward() != VLE_Success) stop(); }, warmup, iters);
   double t = medianMs([&] { if (net.forward() != VLE_Success || net.backward() != VLE_Success) stop(); }, warmup, iters);
+  double ts = medianMs([&] {
+    if (net.forward() != VLE_Success || net.backward() != VLE_Success || net.sgdStep(1e-3, 0.9, 1e-4) != VLE_Success) stop();
+  }, warmup, iters);
   const double gf = net.convForwardFlopsPerImage() * 1e-9;
-  std::printf("%-28s %8.2f ms forward  %8.0f images/s %6.1f TFLOP/s | %8.2f ms fwd+bwd %8.0f images/s %6.1f TFLOP/s "
+  std::printf("%-28s %8.2f ms forward  %8.0f images/s %6.1f TFLOP/s | %8.2f ms fwd+bwd %8.0f images/s %6.1f TFLOP/s | "
+              "%8.2f ms training step (with the SGD update of %.1f M parameters) %8.0f images/s "
               "(N = %d, %.2f GFLOP of convolution per image forward; %s)\n",
-              "resnet-50 224x224", tf, N / (tf * 1e-3), gf * N / tf, t, N / (t * 1e-3), 3 * gf * N / t, N, gf,
-              fused ? "relu/sum folded into bnorm" : "layer by layer");
+              "resnet-50 224x224", tf, N / (tf * 1e-3), gf * N / tf, t, N / (t * 1e-3), 3 * gf * N / t, ts,
+              net.numParameters() * 1e-6, N / (ts * 1e-3), N, gf, fused ? "relu/sum folded into bnorm" : "layer by layer");
 }
 
 int main(int argc, char** argv) {

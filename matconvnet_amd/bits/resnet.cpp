@@ -20,8 +20,25 @@ double conv_flops(int outH, int outW, int fh, int fw, int cin, int cout) {
 }
 }  // namespace
 
+#define STEP(stage, call)                                   \
+  do {                                                      \
+    ErrorCode e_ = (call);                                  \
+    if (e_ != VLE_Success) return fail(e_, stage);          \
+  } while (0)
+
+#define ABI(stage, call)                                                                    \
+  do {                                                                                      \
+    int rc_ = (call);                                                                       \
+    if (rc_ != 0) {                                                                         \
+      context.setError((ErrorCode)rc_, mcn_last_error_message());                           \
+      return fail((ErrorCode)rc_, stage);                                                   \
+    }                                                                                       \
+  } while (0)
+
 ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
-    : N(N), S(imageSize), classes(classes), epsilon(epsilon), fused(true), error(VLE_Success), flops(0) {
+    : N(N), S(imageSize), classes(classes), epsilon(epsilon), fused(true), error(VLE_Success), flops(0), values(NULL),
+      ders(NULL), state(NULL), batchMoments(NULL), runningMoments(NULL), chunkParam(NULL), rates(NULL), chunks(0),
+      momentsCount(0), parameterCount(0) {
   if (S < 32 || S % 32 != 0) {
     error = VLE_IllegalArgument;
     message = "the image size must be a multiple of 32";
@@ -29,13 +46,10 @@ ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
   }
   const int S2 = S / 2, S4 = S / 4;
   make("input", TensorShape(S, S, 3, N));
-  make("stem.f", TensorShape(7, 7, 3, 64)); make("stem.g", TensorShape(64, 1, 1, 1)); make("stem.b", TensorShape(64, 1, 1, 1));
   make("stem.a", TensorShape(S2, S2, 64, N)); make("stem.n", TensorShape(S2, S2, 64, N)); make("stem.r", TensorShape(S2, S2, 64, N));
-  make("stem.m", TensorShape(64, 2, 1, 1));
   make("stem.p", TensorShape(S4, S4, 64, N));
   make("stem.dp", TensorShape(S4, S4, 64, N)); make("stem.dr", TensorShape(S2, S2, 64, N)); make("stem.dn", TensorShape(S2, S2, 64, N));
   make("stem.da", TensorShape(S2, S2, 64, N));
-  make("stem.df", TensorShape(7, 7, 3, 64)); make("stem.dg", TensorShape(64, 1, 1, 1)); make("stem.db", TensorShape(64, 1, 1, 1));
   flops += conv_flops(S2, S2, 7, 7, 3, 64);
 
   // sections 2..5 (cnn_imagenet_init_resnet.m:73-118)
@@ -68,17 +82,141 @@ ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
   units[0]->alias("dzdx", (float*)slot("stem.dp").getMemory());
 
   make("avg", TensorShape(1, 1, C, N)); make("davg", TensorShape(1, 1, C, N));
-  make("fc.f", TensorShape(1, 1, C, classes)); make("fc.b", TensorShape(classes, 1, 1, 1));
-  make("fc.df", TensorShape(1, 1, C, classes)); make("fc.db", TensorShape(classes, 1, 1, 1));
   make("prediction", TensorShape(1, 1, classes, N)); make("dprediction", TensorShape(1, 1, classes, N));
   flops += conv_flops(1, 1, 1, 1, C, classes);
+  if (error == VLE_Success) buildArenas();
   setFused(true);
+}
+
+// Lays all parameters out in the arenas (each parameter whole chunks of MCN_SGD_CHUNK floats, zero padded) and points
+// the layers' parameter, derivative and moments buffers into them.
+ErrorCode ResNet50::buildArenas() {
+  const int finalDepth = units.back()->outDepth();
+  struct Shape { std::string name; TensorShape shape; double lr; };
+  std::vector<Shape> own;
+  // the first filter bank learns 100^2 times slower (cnn_imagenet_init_resnet.m:186-188)
+  own.push_back({"stem.f", TensorShape(7, 7, 3, 64), 1.0 / (100.0 * 100.0)});
+  own.push_back({"stem.g", TensorShape(64, 1, 1, 1), 1.0});
+  own.push_back({"stem.b", TensorShape(64, 1, 1, 1), 1.0});
+  auto add = [&](std::string const& name, std::string const& der, std::size_t count, double lr) {
+    Param p;
+    p.name = name; p.der = der; p.count = count; p.learningRate = lr; p.weightDecay = 1.0;
+    p.offset = chunks * MCN_SGD_CHUNK;
+    chunks += (count + MCN_SGD_CHUNK - 1) / MCN_SGD_CHUNK;
+    parameterCount += count;
+    params.push_back(p);
+  };
+  auto addMoments = [&](std::string const& name, std::size_t count) {
+    Moments m;
+    m.name = name; m.count = count; m.offset = momentsCount;
+    momentsCount += count;
+    moments.push_back(m);
+  };
+  for (std::size_t i = 0; i < own.size(); ++i)
+    add(own[i].name, "stem.d" + own[i].name.substr(5), own[i].shape.getNumElements(), own[i].lr);
+  addMoments("stem.m", 128);
+  for (std::size_t u = 0; u < units.size(); ++u) {
+    const std::string prefix = "unit" + std::to_string(u) + ".";
+    for (char const* layer : {"1", "2", "3", "s"}) {
+      std::size_t n = 0;
+      if (!units[u]->buffer(std::string("f") + layer, &n)) continue;  // (no adapter)
+      add(prefix + "f" + layer, prefix + "df" + layer, n, 1.0);
+      units[u]->buffer(std::string("g") + layer, &n);
+      add(prefix + "g" + layer, prefix + "dg" + layer, n, 1.0);
+      add(prefix + "b" + layer, prefix + "db" + layer, n, 1.0);
+      addMoments(prefix + "m" + layer, 2 * n);
+    }
+  }
+  add("fc.f", "fc.df", (std::size_t)finalDepth * classes, 1.0);
+  add("fc.b", "fc.db", (std::size_t)classes, 1.0);
+  if (params.size() >= 65536) {
+    message = "too many parameters";
+    return error = VLE_Unsupported;
+  }
+
+  const std::size_t arenaBytes = chunks * MCN_SGD_CHUNK * sizeof(float), momentsBytes = momentsCount * sizeof(float);
+  std::vector<unsigned short> hostChunks;
+  std::vector<double> hostRates;
+  for (std::size_t p = 0; p < params.size(); ++p) {
+    hostChunks.insert(hostChunks.end(), (params[p].count + MCN_SGD_CHUNK - 1) / MCN_SGD_CHUNK, (unsigned short)p);
+    hostRates.push_back(params[p].learningRate);
+    hostRates.push_back(params[p].weightDecay);
+  }
+  bool good = hipMalloc((void**)&values, arenaBytes) == hipSuccess && hipMalloc((void**)&ders, arenaBytes) == hipSuccess &&
+              hipMalloc((void**)&state, arenaBytes) == hipSuccess &&
+              hipMalloc((void**)&batchMoments, momentsBytes) == hipSuccess &&
+              hipMalloc((void**)&runningMoments, momentsBytes) == hipSuccess &&
+              hipMalloc((void**)&chunkParam, hostChunks.size() * sizeof(unsigned short)) == hipSuccess &&
+              hipMalloc((void**)&rates, hostRates.size() * sizeof(double)) == hipSuccess;
+  good = good && hipMemset(values, 0, arenaBytes) == hipSuccess && hipMemset(ders, 0, arenaBytes) == hipSuccess &&
+         hipMemset(state, 0, arenaBytes) == hipSuccess && hipMemset(batchMoments, 0, momentsBytes) == hipSuccess &&
+         hipMemset(runningMoments, 0, momentsBytes) == hipSuccess &&
+         hipMemcpy(chunkParam, hostChunks.data(), hostChunks.size() * sizeof(unsigned short), hipMemcpyHostToDevice) == hipSuccess &&
+         hipMemcpy(rates, hostRates.data(), hostRates.size() * sizeof(double), hipMemcpyHostToDevice) == hipSuccess;
+  if (!good) {
+    (void)hipGetLastError();
+    message = "cannot allocate the parameter arenas";
+    return error = VLE_OutOfGPUMemeory;
+  }
+
+  // views
+  for (std::size_t i = 0; i < own.size(); ++i) {
+    view(own[i].name, own[i].shape, values + params[i].offset);
+    view(params[i].der, own[i].shape, ders + params[i].offset);
+  }
+  view("stem.m", TensorShape(64, 2, 1, 1), batchMoments + moments[0].offset);
+  for (std::size_t p = own.size(); p + 2 < params.size(); ++p) {
+    const std::size_t dot = params[p].name.find('.');
+    Bottleneck* u = units[std::atoi(params[p].name.substr(4, dot - 4).c_str())];
+    if (u->alias(params[p].name.substr(dot + 1), values + params[p].offset) != VLE_Success ||
+        u->alias(params[p].der.substr(dot + 1), ders + params[p].offset) != VLE_Success) {
+      message = u->lastMessage();
+      return error = u->lastError();
+    }
+  }
+  for (std::size_t m = 1; m < moments.size(); ++m) {
+    const std::size_t dot = moments[m].name.find('.');
+    Bottleneck* u = units[std::atoi(moments[m].name.substr(4, dot - 4).c_str())];
+    if (u->alias(moments[m].name.substr(dot + 1), batchMoments + moments[m].offset) != VLE_Success) {
+      message = u->lastMessage();
+      return error = u->lastError();
+    }
+  }
+  const Param& ff = params[params.size() - 2];
+  const Param& fb = params[params.size() - 1];
+  view("fc.f", TensorShape(1, 1, finalDepth, classes), values + ff.offset);
+  view("fc.df", TensorShape(1, 1, finalDepth, classes), ders + ff.offset);
+  view("fc.b", TensorShape(classes, 1, 1, 1), values + fb.offset);
+  view("fc.db", TensorShape(classes, 1, 1, 1), ders + fb.offset);
+  return VLE_Success;
+}
+
+void ResNet50::view(std::string const& name, TensorShape const& shape, float* memory) {
+  Slot s;
+  s.name = name;
+  s.tensor = Tensor(shape, VLDT_Float, VLDT_GPU, memory, shape.getNumElements() * sizeof(float));
+  s.owned = false;
+  slots.push_back(s);
+}
+
+ErrorCode ResNet50::sgdStep(double learningRate, double momentum, double weightDecay) {
+  if (error != VLE_Success) return error;
+  void* st = context.getHipHelper().getStream();
+  // gradient-trained parameters: the default solver of examples/cnn_train_dag.m:340-364, one worker
+  ABI("sgd", mcn_sgd_momentum(st, values, state, ders, chunks, chunkParam, rates, learningRate, weightDecay, momentum, 1.0, 0));
+  // moments: trainMethod 'average' (:331-335) with the rate cnn_imagenet_init_resnet.m:190-195 sets, fan-out 1
+  const double rate = 0.3;
+  ABI("moments", mcn_taccum(st, runningMoments, (float)(1.0 - rate), runningMoments, (float)rate, batchMoments, momentsCount));
+  return VLE_Success;
 }
 
 ResNet50::~ResNet50() {
   for (std::size_t i = 0; i < units.size(); ++i) delete units[i];
   for (std::size_t i = 0; i < slots.size(); ++i)
-    if (slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
+    if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
+  void* arenas[] = {values, ders, state, batchMoments, runningMoments, chunkParam, rates};
+  for (void* a : arenas)
+    if (a) (void)hipFree(a);
 }
 
 Tensor ResNet50::make(std::string const& name, TensorShape const& shape) {
@@ -93,6 +231,7 @@ Tensor ResNet50::make(std::string const& name, TensorShape const& shape) {
   Slot s;
   s.name = name;
   s.tensor = Tensor(shape, VLDT_Float, VLDT_GPU, memory, bytes);
+  s.owned = true;
   slots.push_back(s);
   return s.tensor;
 }
@@ -111,6 +250,22 @@ float* ResNet50::buffer(std::string const& name, std::size_t* count) {
     const int i = std::atoi(name.substr(4, dot - 4).c_str());
     if (i < 0 || i >= (int)units.size()) return NULL;
     return units[i]->buffer(name.substr(dot + 1), count);
+  }
+  if (name.compare(0, 9, "momentum.") == 0) {
+    for (std::size_t p = 0; p < params.size(); ++p)
+      if (params[p].name == name.substr(9)) {
+        if (count) *count = params[p].count;
+        return state + params[p].offset;
+      }
+    return NULL;
+  }
+  if (name.compare(0, 8, "running.") == 0) {
+    for (std::size_t m = 0; m < moments.size(); ++m)
+      if (moments[m].name == name.substr(8)) {
+        if (count) *count = moments[m].count;
+        return runningMoments + moments[m].offset;
+      }
+    return NULL;
   }
   Tensor& t = slot(name);
   if (count) *count = t.getNumElements();
@@ -183,21 +338,6 @@ ErrorCode ResNet50::initParameters(unsigned long long seed) {
   }
   return VLE_Success;
 }
-
-#define STEP(stage, call)                                   \
-  do {                                                      \
-    ErrorCode e_ = (call);                                  \
-    if (e_ != VLE_Success) return fail(e_, stage);          \
-  } while (0)
-
-#define ABI(stage, call)                                                                    \
-  do {                                                                                      \
-    int rc_ = (call);                                                                       \
-    if (rc_ != 0) {                                                                         \
-      context.setError((ErrorCode)rc_, mcn_last_error_message());                           \
-      return fail((ErrorCode)rc_, stage);                                                   \
-    }                                                                                       \
-  } while (0)
 
 ErrorCode ResNet50::forward() {
   if (error != VLE_Success) return error;

@@ -5,6 +5,10 @@
 //   sections 2..5 of 3, 4, 6, 3 bottleneck segments, 64/128/256/512 channels inside and 4x that out; the first
 //   segment of a section has the conv + bnorm adapter on its shortcut and, from section 3 on, stride 2
 //   average pooling over the remaining extent (7x7 for 224x224 images), 1x1 convolution 2048 -> classes with bias
+// Training follows examples/cnn_train_dag.m:316-364: SGD with momentum and weight decay on filters, gains and biases
+// (rates of examples/imagenet/cnn_imagenet_init_resnet.m:178-192), a moving average of the batch moments.  All
+// parameters live in one arena (values), their derivatives in a second, the momentum in a third, so that the update is
+// one launch over everything instead of three per parameter.
 // All buffers are allocated at construction; a step performs no allocation.
 #ifndef MCN_AMD_BITS_RESNET_HPP
 #define MCN_AMD_BITS_RESNET_HPP
@@ -27,7 +31,9 @@ class ResNet50 {
 
   // "input" (S x S x 3 x N), "prediction" / "dprediction" (1 x 1 x classes x N), the stem's "stem.f", "stem.g",
   // "stem.b" and their derivatives "stem.df", ..., the classifier's "fc.f", "fc.b", "fc.df", "fc.db", and every
-  // buffer of segment i (0-based, in network order) as "unit<i>.<name>" (see Bottleneck::buffer)
+  // buffer of segment i (0-based, in network order) as "unit<i>.<name>" (see Bottleneck::buffer); the momentum of a
+  // parameter as "momentum.<parameter>" ("momentum.unit3.f2") and the moving average of a batch normalisation's
+  // moments as "running.<moments>" ("running.stem.m", "running.unit3.m1")
   float* buffer(std::string const& name, std::size_t* count = NULL);
   int numUnits() const { return (int)units.size(); }
   ErrorCode setStream(void* stream);
@@ -36,11 +42,19 @@ class ResNet50 {
   ErrorCode initParameters(unsigned long long seed);
   ErrorCode forward();
   ErrorCode backward();
+  // one update of all parameters from the derivatives backward() left (numWorkers = 1), and of the moving averages of
+  // the moments from those forward() left
+  ErrorCode sgdStep(double learningRate, double momentum, double weightDecay);
+  std::size_t numParameters() const { return parameterCount; }
   // forward FLOPs of all convolutions per image (2 per multiply-add); backward is twice that, minus the stem's dzdx
   double convForwardFlopsPerImage() const { return flops; }
 
  private:
-  struct Slot { std::string name; Tensor tensor; };
+  struct Slot { std::string name; Tensor tensor; bool owned; };
+  struct Param { std::string name, der; std::size_t count, offset; double learningRate, weightDecay; };
+  struct Moments { std::string name; std::size_t count, offset; };
+  void view(std::string const& name, TensorShape const& shape, float* memory);
+  ErrorCode buildArenas();
   Tensor& slot(std::string const& name);
   Tensor make(std::string const& name, TensorShape const& shape);
   ErrorCode fail(ErrorCode e, char const* where);
@@ -54,6 +68,12 @@ class ResNet50 {
   ErrorCode error;
   std::string message;
   double flops;
+  std::vector<Param> params;
+  std::vector<Moments> moments;
+  float *values, *ders, *state, *batchMoments, *runningMoments;
+  unsigned short* chunkParam;   // device
+  double* rates;                // device
+  std::size_t chunks, momentsCount, parameterCount;
 };
 
 } }  // namespace vl::harness

@@ -51,6 +51,7 @@ PROTOTYPES = {
     "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_taccum": (_i, [_vp, _vp, C.c_float, _vp, C.c_float, _vp, _sz]),
+    "mcn_sgd_momentum": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _vp] + [C.c_double] * 4 + [C.c_int]),
     "mcn_conv_backward_data_acc": (_i, [_vp, C.POINTER(ConvGeom), _vp, C.c_float, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_filter": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_bias": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _sz]),
@@ -351,6 +352,34 @@ def relu_backward(x, dy):
     dx = _torch().empty_like(x)
     check(lib().mcn_relu_backward(stream(), ptr(dx), ptr(x), ptr(dy), x.numel()))
     return dx
+
+
+SGD_CHUNK = 1024   # MCN_SGD_CHUNK of include/mcn_hip.h
+
+
+def sgd_arena_layout(counts):
+    """Offsets (in floats) of parameters of the given element counts inside an arena whose parameters occupy whole
+    chunks, the total number of chunks, and the chunk -> parameter table (numpy int16)."""
+    offsets, chunk_param, at = [], [], 0
+    for p, n in enumerate(counts):
+        offsets.append(at)
+        k = (n + SGD_CHUNK - 1) // SGD_CHUNK
+        chunk_param += [p] * k
+        at += k * SGD_CHUNK
+    assert len(counts) < 32768
+    return offsets, len(chunk_param), np.asarray(chunk_param, dtype=np.int16)
+
+
+def sgd_momentum(value, state, der, chunk_param, rates, learning_rate, weight_decay, momentum, der_scale=1.0,
+                 nesterov=False):
+    """In-place SGD step over parameter arenas (include/mcn_hip.h: mcn_sgd_momentum).  value, state, der: float32
+    device tensors of chunks*SGD_CHUNK elements; chunk_param: int16 device tensor; rates: float64 device tensor
+    [params][2] of (learningRate, weightDecay) multipliers."""
+    chunks = chunk_param.numel()
+    assert value.numel() == state.numel() == der.numel() == chunks * SGD_CHUNK
+    check(lib().mcn_sgd_momentum(stream(), ptr(value), ptr(state), ptr(der), chunks, ptr(chunk_param), ptr(rates),
+                                 float(learning_rate), float(weight_decay), float(momentum), float(der_scale),
+                                 int(bool(nesterov))))
 
 
 def taccum(alpha, a, beta, b, out=None):

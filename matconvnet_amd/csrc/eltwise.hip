@@ -1,4 +1,4 @@
-// Element-wise companions of the operators: ReLU, sum of two tensors, scaled sum (the SGD update), fill.  Pure streaming kernels:
+// Element-wise companions of the operators: ReLU, sum of two tensors, scaled sum and the SGD step built from it, fill.  Pure streaming kernels:
 // 16-byte accesses, grid-stride, enough workgroups to cover the chip several times.
 #include "mcn_internal.hpp"
 
@@ -65,6 +65,40 @@ __global__ __launch_bounds__(256) void eltwise_kernel(float* __restrict__ y, con
   }
 }
 
+// SGD with momentum over an arena of parameters: one workgroup per chunk of 1024 elements, every chunk inside one
+// parameter, whose rates come from a table.  Each element goes through the roundings of the three scaled sums the
+// reference performs one parameter at a time.
+__global__ __launch_bounds__(256) void sgd_momentum_kernel(float* __restrict__ value, float* __restrict__ state,
+                                                           const float* __restrict__ der,
+                                                           const unsigned short* __restrict__ chunkParam,
+                                                           const double* __restrict__ rates, double learningRate,
+                                                           double weightDecay, float momentum, float derScale, int nesterov) {
+  const int p = chunkParam[blockIdx.x];
+  const float lr = (float)(learningRate * rates[2 * p]), decay = (float)(weightDecay * rates[2 * p + 1]);
+  if (!(lr > 0.f || decay > 0.f)) return;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const float4 v = stream_load4((const float4*)value + i), g = stream_load4((const float4*)der + i);
+  const float4 m = stream_load4((const float4*)state + i);
+  float4 vo, mo;
+  auto one = [&](float v1, float g1, float m1, float& vOut, float& mOut) {
+    const float t = derScale * g1;
+    const float d = t + decay * v1;      // gradient, normalised, plus weight decay
+    const float u = momentum * m1;
+    const float mNew = u + (-1.f) * d;   // momentum
+    float delta = mNew;
+    if (nesterov) delta = momentum * mNew - d;
+    const float w = 1.f * v1;
+    vOut = w + lr * delta;
+    mOut = mNew;
+  };
+  one(v.x, g.x, m.x, vo.x, mo.x);
+  one(v.y, g.y, m.y, vo.y, mo.y);
+  one(v.z, g.z, m.z, vo.z, mo.z);
+  one(v.w, g.w, m.w, vo.w, mo.w);
+  stream_store4((float4*)state + i, mo);
+  stream_store4((float4*)value + i, vo);
+}
+
 template <int OP>
 int launch(const char* who, mcn_stream_t stream, float* y, const float* a, const float* b, float k, size_t n,
            float k2 = 0.f) {
@@ -98,6 +132,19 @@ int mcn_add(mcn_stream_t stream, float* y, const float* a, const float* b, size_
 }
 int mcn_taccum(mcn_stream_t stream, float* y, float alpha, const float* a, float beta, const float* b, size_t n) {
   return launch<OP_AXPBY>("mcn_taccum", stream, y, a, b, alpha, n, beta);
+}
+int mcn_sgd_momentum(mcn_stream_t stream, float* value, float* state, const float* der, size_t chunks,
+                     const unsigned short* chunkParam, const double* rates, double learningRate, double weightDecay,
+                     double momentum, double derScale, int nesterov) {
+  if (chunks == 0) return MCN_SUCCESS;
+  if (!value || !state || !der || !chunkParam || !rates) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_sgd_momentum: null argument");
+  if (!aligned16(value) || !aligned16(state) || !aligned16(der))
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_sgd_momentum: the arenas must be 16-byte aligned");
+  if (chunks >= (1ull << 31)) return fail(MCN_UNSUPPORTED, "mcn_sgd_momentum: arena too large");
+  KernelTimer timer("sgd_momentum_kernel", as_stream(stream));
+  hipLaunchKernelGGL(sgd_momentum_kernel, dim3((unsigned)chunks), dim3(256), 0, as_stream(stream), value, state, der,
+                     chunkParam, rates, learningRate, weightDecay, (float)momentum, (float)derScale, nesterov ? 1 : 0);
+  return check_launch("mcn_sgd_momentum");
 }
 int mcn_fill(mcn_stream_t stream, float* y, float value, size_t n) {
   return launch<OP_FILL>("mcn_fill", stream, y, nullptr, nullptr, value, n);

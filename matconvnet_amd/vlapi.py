@@ -82,6 +82,9 @@ def lib():
         L.vlh_resnet50_init.argtypes = [C.c_void_p, C.c_ulonglong]
         L.vlh_resnet50_forward.argtypes = [C.c_void_p]
         L.vlh_resnet50_backward.argtypes = [C.c_void_p]
+        L.vlh_resnet50_sgd_step.argtypes = [C.c_void_p, C.c_double, C.c_double, C.c_double]
+        L.vlh_resnet50_parameters.argtypes = [C.c_void_p]
+        L.vlh_resnet50_parameters.restype = C.c_size_t
         L.vlh_resnet50_forward_flops.argtypes = [C.c_void_p]
         L.vlh_resnet50_forward_flops.restype = C.c_double
         L.vlh_resnet50_message.restype = C.c_char_p
@@ -279,6 +282,13 @@ class ResNet50(_NamedBuffers):
 
     def backward(self):
         self._check(self.L.vlh_resnet50_backward(self.h))
+
+    def sgd_step(self, learning_rate, momentum=0.9, weight_decay=1e-4):
+        self._check(self.L.vlh_resnet50_sgd_step(self.h, learning_rate, momentum, weight_decay))
+
+    @property
+    def parameters(self):
+        return self.L.vlh_resnet50_parameters(self.h)
 
 
 class Bottleneck(_NamedBuffers):

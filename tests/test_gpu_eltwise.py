@@ -63,3 +63,46 @@ def test_vl_taccum_driver(ob):
     assert bits_equal(host(y), want) and bits_equal(host(ad), a)
     same = vl.vl_taccum(0.5, ad, 2.0, bd, "inplace")
     assert same is ad and bits_equal(host(ad), want)
+
+
+@pytest.mark.parametrize("nesterov", [False, True])
+def test_sgd_momentum_arena_matches_the_reference_call_sequence(capi, ob, nesterov):
+    """One launch over all parameters against the three vl_taccum calls per parameter of
+    examples/cnn_train_dag.m:335-364 (oracle, float): same bits, for parameters with their own learning-rate and
+    weight-decay multipliers, one of them frozen (both rates 0), sizes that are not multiples of the chunk."""
+    import torch
+    counts = [7 * 7 * 3 * 64, 64, 64, 1024, 3 * 3 * 16 * 16, 1, 5000]
+    mults = [(0.0001, 1.0), (1.0, 1.0), (1.0, 0.0), (0.0, 0.0), (1.0, 1.0), (2.0, 0.5), (1.0, 1.0)]
+    lr, wd, mom, workers = 0.1, 1e-4, 0.9, 4
+    offsets, chunks, chunk_param = capi.sgd_arena_layout(counts)
+    r = np.random.default_rng(21)
+    n = chunks * capi.SGD_CHUNK
+    value, state, der = (np.zeros(n, np.float32) for _ in range(3))
+    for off, c in zip(offsets, counts):
+        value[off:off + c] = r.standard_normal(c)
+        state[off:off + c] = 0.1 * r.standard_normal(c)
+        der[off:off + c] = r.standard_normal(c)
+    vd, sd, dd = (torch.from_numpy(a.copy()).cuda() for a in (value, state, der))
+    capi.sgd_momentum(vd, sd, dd, torch.from_numpy(chunk_param).cuda(),
+                      torch.tensor(mults, dtype=torch.float64).cuda(), lr, wd, mom, der_scale=1.0 / workers,
+                      nesterov=nesterov)
+    got_v, got_s = vd.cpu().numpy(), sd.cpu().numpy()
+    assert bits_equal(dd.cpu().numpy(), der)
+    f32 = np.float32
+    for off, c, (lm, dm) in zip(offsets, counts, mults):
+        v, s_, d = value[off:off + c], state[off:off + c], der[off:off + c]
+        this_lr, this_decay = lr * lm, wd * dm
+        if this_lr > 0 or this_decay > 0:
+            g = ob.taccum(1.0 / workers, d, this_decay, v)
+            s_new = ob.taccum(mom, s_, -1.0, g)
+            delta = (f32(mom) * s_new - g).astype(f32) if nesterov else s_new
+            v_new = ob.taccum(1.0, v, this_lr, delta)
+        else:
+            s_new, v_new = s_, v
+        assert bits_equal(got_s[off:off + c], s_new), (off, c)
+        assert bits_equal(got_v[off:off + c], v_new), (off, c)
+    # padding stays zero
+    pad = np.ones(n, bool)
+    for off, c in zip(offsets, counts):
+        pad[off:off + c] = False
+    assert not got_v[pad].any() and not got_s[pad].any()

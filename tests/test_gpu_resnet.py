@@ -179,6 +179,46 @@ def test_seeded_initialisation_runs_at_full_image_size(vl):
         net.close()
 
 
+def test_sgd_step_follows_the_reference_solver(vl, ob, case):
+    """Two training steps (forward, backward, update).  After each, every parameter, its momentum and the moving
+    averages of the moments equal, bit for bit, what the three vl_taccum calls per parameter of
+    examples/cnn_train_dag.m:335-364 (oracle, float) give from the state before the step and the derivatives the
+    device computed; rates as examples/imagenet/cnn_imagenet_init_resnet.m:178-195 sets them."""
+    lr, mom, wd = 0.1, 0.9, 1e-4
+    net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=True)
+    try:
+        _load(net, case)
+        names = [("stem." + k, "stem.d" + k) for k in "fgb"]
+        moments = ["stem.m"]
+        for i, u in enumerate(case["units"]):
+            names += [("unit%d.%s" % (i, k), "unit%d.d%s" % (i, k)) for k in UNIT_PARAMS + (ADAPTER_PARAMS if u["adapter"] else ())]
+            moments += ["unit%d.m%s" % (i, k) for k in ("1", "2", "3") + (("s",) if u["adapter"] else ())]
+        names += [("fc.f", "fc.df"), ("fc.b", "fc.db")]
+        assert net.parameters == sum(net.get(v).size for v, _ in names)
+        f32 = np.float32
+        for step in range(2):
+            before = {v: (net.get(v), net.get("momentum." + v)) for v, _ in names}
+            running = {m: net.get("running." + m) for m in moments}
+            net.forward()
+            net.backward()
+            net.sgd_step(lr, mom, wd)
+            for v, d in names:
+                value, state = before[v]
+                der = net.get(d)
+                this_lr = lr / 100.0 ** 2 if v == "stem.f" else lr
+                g = ob.taccum(1.0, der, wd, value)
+                s_new = ob.taccum(mom, state, -1.0, g)
+                v_new = ob.taccum(1.0, value, this_lr, s_new)
+                assert bits_equal(net.get("momentum." + v), s_new), (step, v)
+                assert bits_equal(net.get(v), v_new), (step, v)
+                assert np.abs(v_new - value).max() > 0, v
+            for m in moments:
+                want = ob.taccum(1.0 - 0.3, running[m], 0.3, net.get(m))
+                assert bits_equal(net.get("running." + m), want), (step, m)
+    finally:
+        net.close()
+
+
 def test_image_size_must_be_a_multiple_of_32(vl):
     from matconvnet_amd.vlapi import VlError
     with pytest.raises(VlError, match="multiple of 32"):
