@@ -12,6 +12,8 @@ region.  `value` is images/s over exactly K steps.  The same line carries
                 ones are timed COLD: four sets of tensors used in turn, so that no launch finds its inputs in the
                 256 MB memory-side cache because the previous launch left them there (`achieved`); the figure a
                 loop over one set of buffers shows is reported beside it as `achieved_warm`,
+  resnet50      the whole ResNet-50 (224 x 224) through the same operator classes: forward and whole training steps
+                (forward, backward, SGD update) at 32 and 128 images,
   cpu_baseline  the CPU restatement of the reference path (oracle/) timed on this machine's host cores.
 One GPU only: nothing here shards.
 """
@@ -250,6 +252,43 @@ def bench_pool_bwd(capi, workloads, reps):
     return rows
 
 
+def bench_resnet50(vlapi, batch, steps, warmup):
+    """Whole ResNet-50 (224 x 224, 1000 classes; examples/imagenet/cnn_imagenet_init_resnet.m) through the same
+    operator classes: forward alone (training-mode batch normalisation) and the training step forward + backward +
+    SGD update, images/s."""
+    import torch
+    net = vlapi.ResNet50(N=batch, eps=1e-5, image_size=224, classes=1000, fused=True, seed=11)
+    try:
+        r = np.random.default_rng(12)
+        net.set("input", np.asfortranarray(r.standard_normal((224, 224, 3, batch), dtype=np.float32)))
+        net.set("dprediction", np.asfortranarray(r.standard_normal((1, 1, 1000, batch), dtype=np.float32)))
+
+        def timed(fn):
+            for _ in range(warmup):
+                fn()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            _sync()
+            a.record()
+            for _ in range(steps):
+                fn()
+            b.record()
+            _sync()
+            return a.elapsed_time(b) / steps
+
+        def train():
+            net.forward()
+            net.backward()
+            net.sgd_step(1e-3, 0.9, 1e-4)
+
+        fwd_ms, step_ms = timed(net.forward), timed(train)
+        flops = net.forward_flops_per_image * batch
+        return {"batch": batch, "forward_ms": fwd_ms, "forward_images_per_s": batch / fwd_ms * 1e3,
+                "train_step_ms": step_ms, "train_images_per_s": batch / step_ms * 1e3,
+                "train_conv_tflops": 3 * flops / step_ms / 1e9, "parameters": net.parameters}
+    finally:
+        net.close()
+
+
 def cpu_baseline(workloads):
     """The CPU restatement of the reference path on this host: one forward+backward of the same block
     (same N = 32 inputs), GEMMs threaded like the reference's BLAS, everything else serial."""
@@ -310,6 +349,8 @@ def main():
         "maxpool_bwd_gbs_warm": pool_rows[0]["achieved_warm"], "avgpool_bwd_gbs_warm": pool_rows[1]["achieved_warm"],
         "hbm_timing": "cold: %d tensor sets in rotation; *_warm: one set reused" % COLD_SETS,
         "rooflines": conv_rows + bn_rows + pool_rows,
+        # beyond the headline block: the whole network the block comes from, per-image rates of whole training steps
+        "resnet50": [bench_resnet50(vlapi, b, max(3, args.steps // 10), 2) for b in (32, 128)],
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(workloads)
