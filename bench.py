@@ -254,8 +254,9 @@ def bench_pool_bwd(capi, workloads, reps):
 
 def bench_resnet50(vlapi, batch, steps, warmup):
     """Whole ResNet-50 (224 x 224, 1000 classes; examples/imagenet/cnn_imagenet_init_resnet.m) through the same
-    operator classes: forward alone (training-mode batch normalisation) and the training step forward + backward +
-    SGD update, images/s."""
+    operator classes: forward alone (training-mode batch normalisation), the training step forward + backward +
+    SGD update, and evaluation (stored moments; the mode of the reference's published 396 images/s,
+    doc/site/docs/pretrained.md:233, measured there on other hardware), images/s."""
     import torch
     net = vlapi.ResNet50(N=batch, eps=1e-5, image_size=224, classes=1000, fused=True, seed=11)
     try:
@@ -281,8 +282,12 @@ def bench_resnet50(vlapi, batch, steps, warmup):
             net.sgd_step(1e-3, 0.9, 1e-4)
 
         fwd_ms, step_ms = timed(net.forward), timed(train)
+        net.set_test_mode(True)     # evaluation: batch normalisation with the moving averages of the steps above
+        eval_ms = timed(net.forward)
+        net.set_test_mode(False)
         flops = net.forward_flops_per_image * batch
-        return {"batch": batch, "forward_ms": fwd_ms, "forward_images_per_s": batch / fwd_ms * 1e3,
+        return {"batch": batch, "eval_ms": eval_ms, "eval_images_per_s": batch / eval_ms * 1e3,
+                "forward_ms": fwd_ms, "forward_images_per_s": batch / fwd_ms * 1e3,
                 "train_step_ms": step_ms, "train_images_per_s": batch / step_ms * 1e3,
                 "train_conv_tflops": 3 * flops / step_ms / 1e9, "parameters": net.parameters}
     finally:

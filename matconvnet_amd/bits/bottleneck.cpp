@@ -13,7 +13,7 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
                        Context* shared)
     : H(H), W(W), C(C), M(M), N(N), Cout(CoutArg > 0 ? CoutArg : C), stride(stride), Ho((H - 1) / stride + 1),
       Wo((W - 1) / stride + 1), adapter(adapter), epsilon(epsilon), context(shared ? *shared : ownContext),
-      error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), sideStream(NULL) {
+      error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), testMode(false), sideStream(NULL) {
   for (int i = 0; i < 5; ++i) events[i] = NULL;
   if (!adapter && (Cout != C || stride != 1)) {
     error = VLE_IllegalArgument;
@@ -32,6 +32,7 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
   make("a2", midOut); make("n2", midOut); make("r2", midOut);
   make("a3", out); make("n3", out); make("s", out); make("y", out);
   make("m1", TensorShape(M, 2, 1, 1)); make("m2", TensorShape(M, 2, 1, 1)); make("m3", TensorShape(Cout, 2, 1, 1));
+  make("rm1", TensorShape(M, 2, 1, 1)); make("rm2", TensorShape(M, 2, 1, 1)); make("rm3", TensorShape(Cout, 2, 1, 1));
   // derivatives
   make("ds", out); make("da3", out); make("dr2", midOut); make("dn2", midOut); make("da2", midOut);
   make("dr1", mid); make("dn1", mid); make("da1", mid); make("dxm", in); make("dzdx", in);
@@ -42,6 +43,7 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
   if (adapter) {
     make("fs", TensorShape(1, 1, C, Cout)); make("gs", TensorShape(Cout, 1, 1, 1)); make("bs", TensorShape(Cout, 1, 1, 1));
     make("as", out); make("ns", out); make("ms", TensorShape(Cout, 2, 1, 1));
+    make("rms", TensorShape(Cout, 2, 1, 1));
     make("das", out); make("dfs", TensorShape(1, 1, C, Cout));
     make("dgs", TensorShape(Cout, 1, 1, 1)); make("dbs", TensorShape(Cout, 1, 1, 1));
   }
@@ -164,11 +166,22 @@ ErrorCode Bottleneck::forward() {
   nn::BatchNorm bn(context, epsilon);
   const std::size_t nMid = slot("a1").getNumElements(), nMidOut = slot("a2").getNumElements(),
                     nOut = slot("a3").getNumElements();
+  // training: moments from the batch, kept for the backward pass; test mode: the stored moments "rm*"
+  // (matlab/+dagnn/BatchNorm.m:12-24)
+  const int given = testMode ? 1 : 0;
+  char const* m1 = testMode ? "rm1" : "m1";
+  char const* m2 = testMode ? "rm2" : "m2";
+  char const* m3 = testMode ? "rm3" : "m3";
+  char const* ms = testMode ? "rms" : "ms";
+  auto bnForward = [&](char const* out, char const* moments, char const* in, char const* g, char const* b) -> ErrorCode {
+    return testMode ? bn.forwardWithMoment(slot(out), slot(moments), slot(in), slot(g), slot(b))
+                    : bn.forward(slot(out), slot(moments), slot(in), slot(g), slot(b));
+  };
   // the shortcut: the input, or its adapted version (matlab: Conv([name '_adapt_conv'], 1, ..., 'relu', false))
   char const* shortcut = "x";
   if (adapter) {
     STEP("convs_fwd", cs.forward(slot("as"), 0, slot("x"), 1, slot("fs"), none));
-    STEP("bns_fwd", bn.forward(slot("ns"), slot("ms"), slot("as"), slot("gs"), slot("bs")));
+    STEP("bns_fwd", bnForward("ns", ms, "as", "gs", "bs"));
     shortcut = "ns";
   }
   if (fused) {
@@ -176,28 +189,28 @@ ErrorCode Bottleneck::forward() {
     STEP("conv1_fwd", c1.forward(slot("a1"), 0, slot("x"), 1, slot("f1"), none));
     void* ws = context.getWorkspace(VLDT_GPU, wsMid > wsOut ? wsMid : wsOut);
     if (!ws) return fail(context.getLastError(), "workspace");
-    ABI("bn1_fwd", mcn_bnorm_forward_fused(st, buffer("r1"), buffer("m1"), buffer("a1"), buffer("g1"), buffer("b1"), NULL, 1,
-                                           H, W, M, N, epsilon, 0, ws, wsMid));
+    ABI("bn1_fwd", mcn_bnorm_forward_fused(st, buffer("r1"), buffer(m1), buffer("a1"), buffer("g1"), buffer("b1"), NULL, 1,
+                                           H, W, M, N, epsilon, given, ws, wsMid));
     STEP("conv2_fwd", c2.forward(slot("a2"), 0, slot("r1"), 1, slot("f2"), none));
     ws = context.getWorkspace(VLDT_GPU, wsMid > wsOut ? wsMid : wsOut);  // (a convolution may have grown it)
     if (!ws) return fail(context.getLastError(), "workspace");
-    ABI("bn2_fwd", mcn_bnorm_forward_fused(st, buffer("r2"), buffer("m2"), buffer("a2"), buffer("g2"), buffer("b2"), NULL, 1,
-                                           Ho, Wo, M, N, epsilon, 0, ws, wsMid));
+    ABI("bn2_fwd", mcn_bnorm_forward_fused(st, buffer("r2"), buffer(m2), buffer("a2"), buffer("g2"), buffer("b2"), NULL, 1,
+                                           Ho, Wo, M, N, epsilon, given, ws, wsMid));
     STEP("conv3_fwd", c1.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
     ws = context.getWorkspace(VLDT_GPU, wsMid > wsOut ? wsMid : wsOut);
     if (!ws) return fail(context.getLastError(), "workspace");
-    ABI("bn3_fwd", mcn_bnorm_forward_fused(st, buffer("y"), buffer("m3"), buffer("a3"), buffer("g3"), buffer("b3"),
-                                           buffer(shortcut), 1, Ho, Wo, Cout, N, epsilon, 0, ws, wsOut));
+    ABI("bn3_fwd", mcn_bnorm_forward_fused(st, buffer("y"), buffer(m3), buffer("a3"), buffer("g3"), buffer("b3"),
+                                           buffer(shortcut), 1, Ho, Wo, Cout, N, epsilon, given, ws, wsOut));
     return VLE_Success;
   }
   STEP("conv1_fwd", c1.forward(slot("a1"), 0, slot("x"), 1, slot("f1"), none));
-  STEP("bn1_fwd", bn.forward(slot("n1"), slot("m1"), slot("a1"), slot("g1"), slot("b1")));
+  STEP("bn1_fwd", bnForward("n1", m1, "a1", "g1", "b1"));
   ABI("relu1_fwd", mcn_relu_forward(st, buffer("r1"), buffer("n1"), nMid));
   STEP("conv2_fwd", c2.forward(slot("a2"), 0, slot("r1"), 1, slot("f2"), none));
-  STEP("bn2_fwd", bn.forward(slot("n2"), slot("m2"), slot("a2"), slot("g2"), slot("b2")));
+  STEP("bn2_fwd", bnForward("n2", m2, "a2", "g2", "b2"));
   ABI("relu2_fwd", mcn_relu_forward(st, buffer("r2"), buffer("n2"), nMidOut));
   STEP("conv3_fwd", c1.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
-  STEP("bn3_fwd", bn.forward(slot("n3"), slot("m3"), slot("a3"), slot("g3"), slot("b3")));
+  STEP("bn3_fwd", bnForward("n3", m3, "a3", "g3", "b3"));
   ABI("sum_fwd", mcn_add(st, buffer("s"), buffer("n3"), buffer(shortcut), nOut));
   ABI("relu3_fwd", mcn_relu_forward(st, buffer("y"), buffer("s"), nOut));
   return VLE_Success;
@@ -205,6 +218,10 @@ ErrorCode Bottleneck::forward() {
 
 ErrorCode Bottleneck::backward() {
   if (error != VLE_Success) return error;
+  if (testMode) {
+    message = "backward needs the batch moments of a training-mode forward pass";
+    return VLE_IllegalArgument;
+  }
   void* st = context.getHipHelper().getStream();
   Tensor none;
   nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),

@@ -29,7 +29,7 @@ class Bottleneck {
   std::string const& lastMessage() const { return message; }
 
   // named device buffers: inputs "x","dzdy","f1","f2","f3","g1","b1",... (adapter: "fs","gs","bs");
-  // outputs "y","dzdx","df1","dg1","db1",...
+  // outputs "y","dzdx","df1","dg1","db1",...; batch moments "m1",..., stored moments "rm1",...
   float* buffer(std::string const& name, std::size_t* count = NULL);
   // makes a named buffer a view of memory owned by someone else (the previous unit's output, say); the unit's own
   // allocation for it is released
@@ -49,6 +49,9 @@ class Bottleneck {
   // wait for; the second stream is joined before backward() returns its work to the caller's stream.  Results are
   // the same bits; only the schedule changes.
   ErrorCode setOverlap(bool on);
+  // test mode: batch normalisation uses the stored moments "rm1", "rm2", "rm3" ("rms") instead of the batch's
+  // (matlab/+dagnn/BatchNorm.m:12-17); forward only
+  void setTestMode(bool on) { testMode = on; }
   ErrorCode forward();
   ErrorCode backward();
 
@@ -75,6 +78,7 @@ class Bottleneck {
   void* hookUser;
   bool fused;
   bool overlap;
+  bool testMode;
   Context sideContext;
   void* sideStream;     // hipStream_t
   void* events[5];      // hipEvent_t: "derivative ready" for the convolutions, "second stream done"

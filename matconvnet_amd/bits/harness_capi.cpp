@@ -233,6 +233,7 @@ float* vlh_resnet50_buffer(void* net, const char* name, size_t* count) {
 }
 int vlh_resnet50_set_stream(void* net, void* stream) { return (int)((harness::ResNet50*)net)->setStream(stream); }
 void vlh_resnet50_set_fused(void* net, int fused) { ((harness::ResNet50*)net)->setFused(fused != 0); }
+void vlh_resnet50_set_test_mode(void* net, int test) { ((harness::ResNet50*)net)->setTestMode(test != 0); }
 int vlh_resnet50_init(void* net, unsigned long long seed) { return (int)((harness::ResNet50*)net)->initParameters(seed); }
 int vlh_resnet50_forward(void* net) { return (int)((harness::ResNet50*)net)->forward(); }
 int vlh_resnet50_backward(void* net) { return (int)((harness::ResNet50*)net)->backward(); }

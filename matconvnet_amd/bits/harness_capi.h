@@ -66,6 +66,8 @@ VLH_API int vlh_resnet50_units(void* net);
 VLH_API float* vlh_resnet50_buffer(void* net, const char* name, size_t* count);
 VLH_API int vlh_resnet50_set_stream(void* net, void* stream);
 VLH_API void vlh_resnet50_set_fused(void* net, int fused);
+/* test != 0: batch normalisation uses the moving averages "running.*" (evaluation of a trained network); forward only */
+VLH_API void vlh_resnet50_set_test_mode(void* net, int test);
 /* He-normal filters, gains 1, biases 0 from a seeded host generator */
 VLH_API int vlh_resnet50_init(void* net, unsigned long long seed);
 VLH_API int vlh_resnet50_forward(void* net);

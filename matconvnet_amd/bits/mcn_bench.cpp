@@ -252,7 +252,13 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
   double ts = medianMs([&] {
     if (net.forward() != VLE_Success || net.backward() != VLE_Success || net.sgdStep(1e-3, 0.9, 1e-4) != VLE_Success) stop();
   }, warmup, iters);
+  // evaluation: batch normalisation with the moving averages the training steps above have produced
+  net.setTestMode(true);
+  double te = medianMs([&] { if (net.forward() != VLE_Success) stop(); }, warmup, iters);
+  net.setTestMode(false);
   const double gf = net.convForwardFlopsPerImage() * 1e-9;
+  std::printf("%-28s %8.2f ms evaluation (stored moments) %8.0f images/s %6.1f TFLOP/s\n", "resnet-50 224x224", te,
+              N / (te * 1e-3), gf * N / te);
   std::printf("%-28s %8.2f ms forward  %8.0f images/s %6.1f TFLOP/s | %8.2f ms fwd+bwd %8.0f images/s %6.1f TFLOP/s | "
               "%8.2f ms training step (with the SGD update of %.1f M parameters) %8.0f images/s "
               "(N = %d, %.2f GFLOP of convolution per image forward; %s)\n",

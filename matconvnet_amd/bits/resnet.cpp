@@ -36,7 +36,7 @@ double conv_flops(int outH, int outW, int fh, int fw, int cin, int cout) {
   } while (0)
 
 ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
-    : N(N), S(imageSize), classes(classes), epsilon(epsilon), fused(true), error(VLE_Success), flops(0), values(NULL),
+    : N(N), S(imageSize), classes(classes), epsilon(epsilon), fused(true), testMode(false), error(VLE_Success), flops(0), values(NULL),
       ders(NULL), state(NULL), batchMoments(NULL), runningMoments(NULL), chunkParam(NULL), rates(NULL), chunks(0),
       momentsCount(0), parameterCount(0) {
   if (S < 32 || S % 32 != 0) {
@@ -177,7 +177,8 @@ ErrorCode ResNet50::buildArenas() {
   for (std::size_t m = 1; m < moments.size(); ++m) {
     const std::size_t dot = moments[m].name.find('.');
     Bottleneck* u = units[std::atoi(moments[m].name.substr(4, dot - 4).c_str())];
-    if (u->alias(moments[m].name.substr(dot + 1), batchMoments + moments[m].offset) != VLE_Success) {
+    if (u->alias(moments[m].name.substr(dot + 1), batchMoments + moments[m].offset) != VLE_Success ||
+        u->alias("r" + moments[m].name.substr(dot + 1), runningMoments + moments[m].offset) != VLE_Success) {
       message = u->lastMessage();
       return error = u->lastError();
     }
@@ -279,6 +280,11 @@ void ResNet50::setFused(bool on) {
   for (std::size_t i = 0; i < units.size(); ++i) units[i]->setFused(on);
 }
 
+void ResNet50::setTestMode(bool on) {
+  testMode = on;
+  for (std::size_t i = 0; i < units.size(); ++i) units[i]->setTestMode(on);
+}
+
 ErrorCode ResNet50::fail(ErrorCode e, char const* where) {
   if (e != VLE_Success) {
     error = e;
@@ -352,11 +358,18 @@ ErrorCode ResNet50::forward() {
     const size_t wsBytes = mcn_bnorm_workspace_bytes(S2, S2, 64, N);
     void* ws = context.getWorkspace(VLDT_GPU, wsBytes);
     if (!ws) return fail(context.getLastError(), "workspace");
-    ABI("stem bnorm", mcn_bnorm_forward_fused(st, (float*)slot("stem.r").getMemory(), (float*)slot("stem.m").getMemory(),
+    float* stemMoments = testMode ? runningMoments + moments[0].offset : (float*)slot("stem.m").getMemory();
+    ABI("stem bnorm", mcn_bnorm_forward_fused(st, (float*)slot("stem.r").getMemory(), stemMoments,
                                               (float const*)slot("stem.a").getMemory(), (float const*)slot("stem.g").getMemory(),
-                                              (float const*)slot("stem.b").getMemory(), NULL, 1, S2, S2, 64, N, epsilon, 0, ws, wsBytes));
+                                              (float const*)slot("stem.b").getMemory(), NULL, 1, S2, S2, 64, N, epsilon,
+                                              testMode ? 1 : 0, ws, wsBytes));
   } else {
-    STEP("stem bnorm", bn.forward(slot("stem.n"), slot("stem.m"), slot("stem.a"), slot("stem.g"), slot("stem.b")));
+    if (testMode) {
+      Tensor running(TensorShape(64, 2, 1, 1), VLDT_Float, VLDT_GPU, runningMoments + moments[0].offset, 128 * sizeof(float));
+      STEP("stem bnorm", bn.forwardWithMoment(slot("stem.n"), running, slot("stem.a"), slot("stem.g"), slot("stem.b")));
+    } else {
+      STEP("stem bnorm", bn.forward(slot("stem.n"), slot("stem.m"), slot("stem.a"), slot("stem.g"), slot("stem.b")));
+    }
     ABI("stem relu", mcn_relu_forward(st, (float*)slot("stem.r").getMemory(), (float const*)slot("stem.n").getMemory(),
                                       slot("stem.n").getNumElements()));
   }
@@ -377,6 +390,10 @@ ErrorCode ResNet50::forward() {
 
 ErrorCode ResNet50::backward() {
   if (error != VLE_Success) return error;
+  if (testMode) {
+    message = "backward needs the batch moments of a training-mode forward pass";
+    return VLE_IllegalArgument;
+  }
   void* st = context.getHipHelper().getStream();
   Tensor none;
   const int S2 = S / 2;

@@ -38,6 +38,9 @@ class ResNet50 {
   int numUnits() const { return (int)units.size(); }
   ErrorCode setStream(void* stream);
   void setFused(bool on);
+  // test mode: every batch normalisation uses the moving averages "running.*" instead of the batch's moments
+  // (matlab/+dagnn/BatchNorm.m:12-17), as evaluation of a trained network does; forward only
+  void setTestMode(bool on);
   // He-normal filters (matlab/+dagnn/Conv.m:40 style), gains 1, biases 0, from a seeded generator on the host
   ErrorCode initParameters(unsigned long long seed);
   ErrorCode forward();
@@ -61,7 +64,7 @@ class ResNet50 {
 
   int N, S, classes;
   double epsilon;
-  bool fused;
+  bool fused, testMode;
   Context context;
   std::vector<Slot> slots;
   std::vector<Bottleneck*> units;

@@ -79,6 +79,8 @@ def lib():
         L.vlh_resnet50_set_stream.argtypes = [C.c_void_p, C.c_void_p]
         L.vlh_resnet50_set_fused.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_fused.restype = None
+        L.vlh_resnet50_set_test_mode.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_resnet50_set_test_mode.restype = None
         L.vlh_resnet50_init.argtypes = [C.c_void_p, C.c_ulonglong]
         L.vlh_resnet50_forward.argtypes = [C.c_void_p]
         L.vlh_resnet50_backward.argtypes = [C.c_void_p]
@@ -265,6 +267,10 @@ class ResNet50(_NamedBuffers):
 
     def set_fused(self, on):
         self.L.vlh_resnet50_set_fused(self.h, int(on))
+
+    def set_test_mode(self, on):
+        """Batch normalisation with the moving averages ("running.*") instead of the batch's moments; forward only."""
+        self.L.vlh_resnet50_set_test_mode(self.h, int(on))
 
     def _buf(self, name):
         n = C.c_size_t(0)

@@ -219,6 +219,40 @@ def test_sgd_step_follows_the_reference_solver(vl, ob, case):
         net.close()
 
 
+def test_test_mode_uses_the_stored_moments(vl, case):
+    """Evaluation mode (matlab/+dagnn/BatchNorm.m:12-17): with the moving averages set to the batch's own moments the
+    prediction is the training-mode one; with other moments it is not; fused and layer-by-layer agree bit for bit;
+    backward is refused."""
+    from matconvnet_amd.vlapi import VlError
+    outs = {}
+    for fused in (False, True):
+        net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=fused)
+        try:
+            _load(net, case)
+            net.forward()
+            train = net.get("prediction")
+            moments = ["stem.m"]
+            for i, u in enumerate(case["units"]):
+                moments += ["unit%d.m%s" % (i, k) for k in ("1", "2", "3") + (("s",) if u["adapter"] else ())]
+            net.set_test_mode(True)
+            net.forward()
+            zero_moments = net.get("prediction")          # running moments still zero: mean 0, sigma 0
+            assert not np.allclose(zero_moments, train, rtol=1e-3, atol=1e-3)
+            for m in moments:
+                net.set("running." + m, net.get(m))
+            net.forward()
+            outs[fused] = net.get("prediction")
+            assert rel_max(outs[fused], train) < 1e-6
+            with pytest.raises(VlError, match="training-mode"):
+                net.backward()
+            net.set_test_mode(False)
+            net.forward()
+            net.backward()
+        finally:
+            net.close()
+    assert bits_equal(outs[False], outs[True])
+
+
 def test_image_size_must_be_a_multiple_of_32(vl):
     from matconvnet_amd.vlapi import VlError
     with pytest.raises(VlError, match="multiple of 32"):
