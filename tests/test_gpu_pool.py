@@ -66,7 +66,7 @@ def test_backward_bit_exact_small(capi, ob, geom, method, mode):
     assert bits_equal(got, want), count_bit_mismatches(got, want)
 
 
-@pytest.mark.parametrize("geom", GEOMS[:8])
+@pytest.mark.parametrize("geom", GEOMS)
 @pytest.mark.parametrize("method", ["max", "avg"])
 def test_forward_bit_exact_small(capi, ob, geom, method):
     H, W, C, N, pool, stride, pad = geom
@@ -76,6 +76,20 @@ def test_forward_bit_exact_small(capi, ob, geom, method):
     got = capi.to_host(capi.pool_forward(capi.to_device(x), g))
     want = ob.pool_forward(x, ob.pool_geom(shape, pool, stride, pad, method))
     assert bits_equal(got, want)
+
+
+@pytest.mark.parametrize("method", ["max", "avg"])
+@pytest.mark.parametrize("geom", [(40, 36, 3, 2, 3, 2, 1), (112, 112, 4, 2, 3, 2, 1), (21, 17, 2, 1, (7, 3), (1, 1), (3, 3, 1, 1)),
+                                  (30, 30, 1, 2, 9, 4, 4), (7, 7, 5, 3, 7, 1, 0), (300, 9, 2, 1, (2, 5), (2, 1), 0)])
+def test_forward_bit_exact_larger_planes(capi, ob, method, geom):
+    """Forward pass on planes of several hundred elements, wide windows and whole-plane windows: the oracle's bits
+    (ties, NaN, infinities and zeros of both signs included)."""
+    H, W, C, N, pool, stride, pad = geom
+    shape = (H, W, C, N)
+    x = _inputs(shape, 51, "special" if method == "max" else "normal")
+    g = capi.pool_geom(shape, pool, stride, pad, method)
+    want = ob.pool_forward(x, ob.pool_geom(shape, pool, stride, pad, method))
+    assert bits_equal(capi.to_host(capi.pool_forward(capi.to_device(x), g)), want)
 
 
 @pytest.mark.parametrize("method", ["max", "avg"])
