@@ -240,6 +240,10 @@ int vlh_resnet50_backward(void* net) { return (int)((harness::ResNet50*)net)->ba
 int vlh_resnet50_sgd_step(void* net, double learningRate, double momentum, double weightDecay) {
   return (int)((harness::ResNet50*)net)->sgdStep(learningRate, momentum, weightDecay);
 }
+int vlh_resnet50_capture(void* net, int training, double learningRate, double momentum, double weightDecay) {
+  return (int)((harness::ResNet50*)net)->capture(training != 0, learningRate, momentum, weightDecay);
+}
+int vlh_resnet50_replay(void* net) { return (int)((harness::ResNet50*)net)->replay(); }
 size_t vlh_resnet50_parameters(void* net) { return ((harness::ResNet50*)net)->numParameters(); }
 double vlh_resnet50_forward_flops(void* net) { return ((harness::ResNet50*)net)->convForwardFlopsPerImage(); }
 const char* vlh_resnet50_message(void* net) { return ((harness::ResNet50*)net)->lastMessage().c_str(); }

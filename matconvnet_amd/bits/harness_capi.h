@@ -77,6 +77,11 @@ VLH_API int vlh_resnet50_backward(void* net);
    and "running.<moments>" hold the solver state */
 VLH_API int vlh_resnet50_sgd_step(void* net, double learningRate, double momentum, double weightDecay);
 VLH_API size_t vlh_resnet50_parameters(void* net);
+/* records forward (training == 0) or a whole training step (forward, backward, SGD update with these rates) on the
+   network's stream -- which must not be the default stream -- into a HIP graph; vlh_resnet50_replay launches it.  The
+   recorded work must have run once eagerly before; capture again after changing rates, modes or the stream. */
+VLH_API int vlh_resnet50_capture(void* net, int training, double learningRate, double momentum, double weightDecay);
+VLH_API int vlh_resnet50_replay(void* net);
 /* forward FLOPs of the convolutions for one image */
 VLH_API double vlh_resnet50_forward_flops(void* net);
 VLH_API const char* vlh_resnet50_message(void* net);

@@ -81,7 +81,7 @@ struct TensorSet {
 };
 
 template <typename F>
-static double medianMs(F&& body, int warmup, int iters) {
+static double medianMs(F&& body, int warmup, int iters, hipStream_t stream = 0) {
   hipEvent_t a, b;
   HIP_OK(hipEventCreate(&a));
   HIP_OK(hipEventCreate(&b));
@@ -89,9 +89,9 @@ static double medianMs(F&& body, int warmup, int iters) {
   HIP_OK(hipDeviceSynchronize());
   std::vector<float> ms(iters);
   for (int i = 0; i < iters; ++i) {
-    HIP_OK(hipEventRecord(a, 0));
+    HIP_OK(hipEventRecord(a, stream));
     body();
-    HIP_OK(hipEventRecord(b, 0));
+    HIP_OK(hipEventRecord(b, stream));
     HIP_OK(hipEventSynchronize(b));
     HIP_OK(hipEventElapsedTime(&ms[i], a, b));
   }
@@ -252,13 +252,27 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
   double ts = medianMs([&] {
     if (net.forward() != VLE_Success || net.backward() != VLE_Success || net.sgdStep(1e-3, 0.9, 1e-4) != VLE_Success) stop();
   }, warmup, iters);
+  // the same training step and evaluation pass replayed from HIP graphs (recorded on a stream of the network's own)
+  hipStream_t own = NULL;
+  HIP_OK(hipStreamCreateWithFlags(&own, hipStreamNonBlocking));
+  HIP_OK(hipDeviceSynchronize());
+  net.setStream(own);
+  double tsg = 0, teg = 0;
+  if (net.forward() != VLE_Success || net.backward() != VLE_Success || net.sgdStep(1e-3, 0.9, 1e-4) != VLE_Success ||
+      net.capture(true, 1e-3, 0.9, 1e-4) != VLE_Success) stop();
+  tsg = medianMs([&] { if (net.replay() != VLE_Success) stop(); }, warmup, iters, own);
   // evaluation: batch normalisation with the moving averages the training steps above have produced
   net.setTestMode(true);
-  double te = medianMs([&] { if (net.forward() != VLE_Success) stop(); }, warmup, iters);
+  double te = medianMs([&] { if (net.forward() != VLE_Success) stop(); }, warmup, iters, own);
+  if (net.capture(false) != VLE_Success) stop();
+  teg = medianMs([&] { if (net.replay() != VLE_Success) stop(); }, warmup, iters, own);
   net.setTestMode(false);
+  HIP_OK(hipStreamSynchronize(own));
+  net.setStream(NULL);
   const double gf = net.convForwardFlopsPerImage() * 1e-9;
-  std::printf("%-28s %8.2f ms evaluation (stored moments) %8.0f images/s %6.1f TFLOP/s\n", "resnet-50 224x224", te,
-              N / (te * 1e-3), gf * N / te);
+  std::printf("%-28s %8.2f ms evaluation (stored moments) %8.0f images/s %6.1f TFLOP/s | replayed from a HIP graph: evaluation "
+              "%8.2f ms %8.0f images/s, training step %8.2f ms %8.0f images/s\n", "resnet-50 224x224", te,
+              N / (te * 1e-3), gf * N / te, teg, N / (teg * 1e-3), tsg, N / (tsg * 1e-3));
   std::printf("%-28s %8.2f ms forward  %8.0f images/s %6.1f TFLOP/s | %8.2f ms fwd+bwd %8.0f images/s %6.1f TFLOP/s | "
               "%8.2f ms training step (with the SGD update of %.1f M parameters) %8.0f images/s "
               "(N = %d, %.2f GFLOP of convolution per image forward; %s)\n",

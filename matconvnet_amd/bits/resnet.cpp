@@ -38,7 +38,7 @@ double conv_flops(int outH, int outW, int fh, int fw, int cin, int cout) {
 ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
     : N(N), S(imageSize), classes(classes), epsilon(epsilon), fused(true), testMode(false), error(VLE_Success), flops(0), values(NULL),
       ders(NULL), state(NULL), batchMoments(NULL), runningMoments(NULL), chunkParam(NULL), rates(NULL), chunks(0),
-      momentsCount(0), parameterCount(0) {
+      momentsCount(0), parameterCount(0), graph(NULL), graphExec(NULL) {
   if (S < 32 || S % 32 != 0) {
     error = VLE_IllegalArgument;
     message = "the image size must be a multiple of 32";
@@ -211,7 +211,69 @@ ErrorCode ResNet50::sgdStep(double learningRate, double momentum, double weightD
   return VLE_Success;
 }
 
+void ResNet50::dropGraph() {
+  if (graphExec) (void)hipGraphExecDestroy((hipGraphExec_t)graphExec);
+  if (graph) (void)hipGraphDestroy((hipGraph_t)graph);
+  graph = graphExec = NULL;
+}
+
+ErrorCode ResNet50::capture(bool training, double learningRate, double momentum, double weightDecay) {
+  if (error != VLE_Success) return error;
+  hipStream_t st = (hipStream_t)context.getHipHelper().getStream();
+  if (!st) {
+    message = "capture needs a stream of its own (the default stream cannot be captured)";
+    return VLE_IllegalArgument;
+  }
+  dropGraph();
+  if (hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+    (void)hipGetLastError();
+    message = "cannot begin the stream capture";
+    return VLE_Cuda;
+  }
+  ErrorCode e = forward();
+  if (e == VLE_Success && training) e = backward();
+  if (e == VLE_Success && training) e = sgdStep(learningRate, momentum, weightDecay);
+  hipGraph_t g = NULL;
+  const hipError_t ended = hipStreamEndCapture(st, &g);
+  if (e != VLE_Success) {
+    if (g) (void)hipGraphDestroy(g);
+    (void)hipGetLastError();
+    return e;
+  }
+  if (ended != hipSuccess || !g) {
+    (void)hipGetLastError();
+    message = std::string("the stream capture failed: ") + hipGetErrorString(ended) +
+              " (run the step once eagerly first: capture cannot grow the workspace)";
+    return VLE_Cuda;
+  }
+  hipGraphExec_t x = NULL;
+  if (hipGraphInstantiate(&x, g, NULL, NULL, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipGraphDestroy(g);
+    message = "cannot instantiate the graph";
+    return VLE_Cuda;
+  }
+  graph = g;
+  graphExec = x;
+  return VLE_Success;
+}
+
+ErrorCode ResNet50::replay() {
+  if (error != VLE_Success) return error;
+  if (!graphExec) {
+    message = "nothing has been captured";
+    return VLE_IllegalArgument;
+  }
+  if (hipGraphLaunch((hipGraphExec_t)graphExec, (hipStream_t)context.getHipHelper().getStream()) != hipSuccess) {
+    (void)hipGetLastError();
+    message = "cannot launch the graph";
+    return VLE_Cuda;
+  }
+  return VLE_Success;
+}
+
 ResNet50::~ResNet50() {
+  dropGraph();
   for (std::size_t i = 0; i < units.size(); ++i) delete units[i];
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());

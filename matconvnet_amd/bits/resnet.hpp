@@ -49,6 +49,13 @@ class ResNet50 {
   // the moments from those forward() left
   ErrorCode sgdStep(double learningRate, double momentum, double weightDecay);
   std::size_t numParameters() const { return parameterCount; }
+  // Records forward() -- and, when `training`, backward() and sgdStep(...) behind it -- on the network's stream into a
+  // HIP graph; replay() launches that graph, which saves the host's per-launch work (several hundred launches per
+  // step, many of them a few microseconds long).  The network's stream must not be the default stream; the recorded
+  // work must have run once eagerly beforehand (so that the workspace has its final size: capture cannot allocate);
+  // rates, modes (fused, test) and buffers are those at capture time -- capture again after changing any.
+  ErrorCode capture(bool training, double learningRate = 0, double momentum = 0, double weightDecay = 0);
+  ErrorCode replay();
   // forward FLOPs of all convolutions per image (2 per multiply-add); backward is twice that, minus the stem's dzdx
   double convForwardFlopsPerImage() const { return flops; }
 
@@ -77,6 +84,8 @@ class ResNet50 {
   unsigned short* chunkParam;   // device
   double* rates;                // device
   std::size_t chunks, momentsCount, parameterCount;
+  void *graph, *graphExec;      // hipGraph_t, hipGraphExec_t
+  void dropGraph();
 };
 
 } }  // namespace vl::harness

@@ -86,6 +86,8 @@ def lib():
         L.vlh_resnet50_backward.argtypes = [C.c_void_p]
         L.vlh_resnet50_sgd_step.argtypes = [C.c_void_p, C.c_double, C.c_double, C.c_double]
         L.vlh_resnet50_parameters.argtypes = [C.c_void_p]
+        L.vlh_resnet50_capture.argtypes = [C.c_void_p, C.c_int, C.c_double, C.c_double, C.c_double]
+        L.vlh_resnet50_replay.argtypes = [C.c_void_p]
         L.vlh_resnet50_parameters.restype = C.c_size_t
         L.vlh_resnet50_forward_flops.argtypes = [C.c_void_p]
         L.vlh_resnet50_forward_flops.restype = C.c_double
@@ -295,6 +297,17 @@ class ResNet50(_NamedBuffers):
     @property
     def parameters(self):
         return self.L.vlh_resnet50_parameters(self.h)
+
+    def set_stream(self, torch_stream):
+        self._check(self.L.vlh_resnet50_set_stream(self.h, C.c_void_p(torch_stream.cuda_stream)))
+
+    def capture(self, training, learning_rate=0.0, momentum=0.0, weight_decay=0.0):
+        """Record forward (or the whole training step) on the network's stream into a HIP graph; `replay` launches it.
+        Needs a stream other than the default one (`set_stream`) and one eager run of the same work beforehand."""
+        self._check(self.L.vlh_resnet50_capture(self.h, int(training), learning_rate, momentum, weight_decay))
+
+    def replay(self):
+        self._check(self.L.vlh_resnet50_replay(self.h))
 
 
 class Bottleneck(_NamedBuffers):

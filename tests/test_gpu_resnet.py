@@ -253,6 +253,72 @@ def test_test_mode_uses_the_stored_moments(vl, case):
     assert bits_equal(outs[False], outs[True])
 
 
+def test_graph_replays_match_eager_steps(vl, case):
+    """A training step and an evaluation pass recorded into HIP graphs: every replay -- with uploads, downloads and
+    device synchronisations of the program between them, and the input changed from one to the next -- leaves the same
+    bits in the parameters, the momentum, the moving averages and the prediction as the same calls made eagerly."""
+    import torch
+    from matconvnet_amd.vlapi import VlError
+    lr, mom, wd = 0.05, 0.9, 1e-4
+    r = np.random.default_rng(77)
+    inputs = [np.asfortranarray(r.standard_normal((S, S, 3, N), dtype=np.float32)) for _ in range(3)]
+    watch = ["prediction", "stem.f", "momentum.stem.f", "running.stem.m", "unit0.fs", "unit7.g2", "momentum.unit7.f2",
+             "running.unit15.m3", "unit15.f3", "fc.f", "fc.b", "momentum.fc.b"]
+    stream = torch.cuda.Stream()
+    history = {}
+    with torch.cuda.stream(stream):
+        for mode in ("eager", "graph"):
+            net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=True)
+            try:
+                _load(net, case)
+                if mode == "graph":
+                    with pytest.raises(VlError, match="nothing has been captured"):
+                        net.replay()
+                net.forward(); net.backward(); net.sgd_step(lr, mom, wd)     # (also sizes the workspace)
+                if mode == "graph":
+                    net.capture(True, lr, mom, wd)
+                seen = []
+                for x in inputs:
+                    net.set("input", x)
+                    if mode == "graph":
+                        net.replay()
+                    else:
+                        net.forward(); net.backward(); net.sgd_step(lr, mom, wd)
+                    seen.append({k: net.get(k) for k in watch})
+                # evaluation with the moving averages the steps above left
+                net.set_test_mode(True)
+                net.forward()
+                if mode == "graph":
+                    net.capture(False)
+                for x in inputs:
+                    net.set("input", x)
+                    if mode == "graph":
+                        net.replay()
+                    else:
+                        net.forward()
+                    seen.append({"prediction": net.get("prediction")})
+                history[mode] = seen
+            finally:
+                net.close()
+    for i, (a, b) in enumerate(zip(history["eager"], history["graph"])):
+        for k in a:
+            assert np.isfinite(a[k]).all(), (i, k)
+            assert bits_equal(a[k], b[k]), (i, k)
+    assert not bits_equal(history["eager"][0]["fc.f"], history["eager"][2]["fc.f"])
+    assert not bits_equal(history["eager"][3]["prediction"], history["eager"][4]["prediction"])
+
+
+def test_capture_needs_a_stream_of_its_own(vl):
+    from matconvnet_amd.vlapi import VlError
+    net = vl.ResNet50(N=1, image_size=32, classes=4, seed=1)
+    try:
+        net.forward()
+        with pytest.raises(VlError, match="default stream"):
+            net.capture(False)
+    finally:
+        net.close()
+
+
 def test_image_size_must_be_a_multiple_of_32(vl):
     from matconvnet_amd.vlapi import VlError
     with pytest.raises(VlError, match="multiple of 32"):
