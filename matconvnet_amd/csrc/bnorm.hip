@@ -27,6 +27,8 @@ struct BnormP {
   int WH, C, N;
   int groups;        // image groups per channel (grid = C * groups)
   int reverse;       // apply pass walks logical ids backwards
+  int teamShift[2];  // log2 of the threads that share one plane, for scalar [0] and 16-byte [1] accesses: planes
+                     // smaller than a workgroup's 256 accesses are walked several at a time, one per team
   double mass;       // WH * N
   double epsilon;
 };
@@ -91,13 +93,15 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
   if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &ra, &rk);
   auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv, rk) > 0.f ? dv : 0.f) : dv; };
   double acc[4] = {0.0, 0.0, 0.0, 0.0};
-  for (int n = n0; n < n1; ++n) {
+  const int shift = p.teamShift[VEC4 ? 1 : 0], TS = 1 << shift, teams = 256 >> shift;
+  const int team = threadIdx.x >> shift, j0 = threadIdx.x & (TS - 1);
+  for (int n = n0 + team; n < n1; n += teams) {
     const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
     float sx = 0.f, sxx = 0.f, sxd = 0.f, sd = 0.f;
     if (VEC4) {
       const float4* x4 = (const float4*)(x + base);
       const float4* d4 = (const float4*)(MODE != 0 ? dy + base : x + base);
-      for (int i = threadIdx.x; i < p.WH / 4; i += 256) {
+      for (int i = j0; i < p.WH / 4; i += TS) {
         const float4 a = x4[i];
         if (MODE != 1) {
           sx += (a.x + a.y) + (a.z + a.w);
@@ -117,7 +121,7 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
         }
       }
     } else {
-      for (int i = threadIdx.x; i < p.WH; i += 256) {
+      for (int i = j0; i < p.WH; i += TS) {
         const float a = x[base + i];
         if (MODE != 1) {
           sx += a;
@@ -182,14 +186,16 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
                                               const BnormP& p, int c, int n0, int n1, float ra = 0.f, float rk = 0.f) {
   static_assert(!RELU || TWO, "the mask is computed from the second stream");
   auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv, rk) > 0.f ? dv : 0.f) : dv; };
-  for (int nn = n0; nn < n1; ++nn) {
+  const int shift = p.teamShift[VEC4 ? 1 : 0], TS = 1 << shift, teams = 256 >> shift;
+  const int team = threadIdx.x >> shift, j0 = threadIdx.x & (TS - 1);
+  for (int nn = n0 + team; nn < n1; nn += teams) {
     const int n = p.reverse ? (n1 - 1 - (nn - n0)) : nn;
     const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
     if (VEC4) {
       const float4* s1 = (const float4*)(in1 + base);
       const float4* s2 = (const float4*)(TWO ? in2 + base : in1 + base);
       float4* o4 = (float4*)(out + base);
-      for (int i = threadIdx.x; i < p.WH / 4; i += 256) {
+      for (int i = j0; i < p.WH / 4; i += TS) {
         const float4 u = stream_load4(s1 + i);
         float4 r;
         if (TWO) {
@@ -207,7 +213,7 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
         stream_store4(o4 + i, r);
       }
     } else {
-      for (int i = threadIdx.x; i < p.WH; i += 256) {
+      for (int i = j0; i < p.WH; i += TS) {
         const float u = in1[base + i];
         out[base + i] = TWO ? fmaf(a, gate(in2[base + i], u), fmaf(b, in2[base + i], k)) : fmaf(a, u, k);
       }
@@ -279,21 +285,23 @@ __device__ __forceinline__ void stream_forward(float* __restrict__ out, const fl
     if (RELU) v = v > 0.f ? v : 0.f;
     return v;
   };
-  for (int nn = n0; nn < n1; ++nn) {
+  const int shift = p.teamShift[VEC4 ? 1 : 0], TS = 1 << shift, teams = 256 >> shift;
+  const int team = threadIdx.x >> shift, j0 = threadIdx.x & (TS - 1);
+  for (int nn = n0 + team; nn < n1; nn += teams) {
     const int n = p.reverse ? (n1 - 1 - (nn - n0)) : nn;
     const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
     if (VEC4) {
       const float4* s1 = (const float4*)(in + base);
       const float4* s2 = (const float4*)((RES ? res : in) + base);
       float4* o4 = (float4*)(out + base);
-      for (int i = threadIdx.x; i < p.WH / 4; i += 256) {
+      for (int i = j0; i < p.WH / 4; i += TS) {
         const float4 u = stream_load4(s1 + i);
         float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
         if (RES) r = stream_load4(s2 + i);
         stream_store4(o4 + i, make_float4(one(u.x, r.x), one(u.y, r.y), one(u.z, r.z), one(u.w, r.w)));
       }
     } else {
-      for (int i = threadIdx.x; i < p.WH; i += 256) out[base + i] = one(in[base + i], RES ? res[base + i] : 0.f);
+      for (int i = j0; i < p.WH; i += TS) out[base + i] = one(in[base + i], RES ? res[base + i] : 0.f);
     }
   }
 }
@@ -355,6 +363,12 @@ int setup(const char* who, int H, int W, int C, int N, double epsilon, BnormP* p
   p->N = N;
   p->groups = image_groups(p->WH, N);
   p->reverse = tunable("bnorm_reverse_apply", 1) ? 1 : 0;
+  for (int v = 0; v < 2; ++v) {
+    const int accesses = v ? p->WH / 4 : p->WH;  // per plane
+    int shift = 4;                               // teams of 16 ... 256 threads
+    while (shift < 8 && (1 << shift) < accesses) ++shift;
+    p->teamShift[v] = shift;
+  }
   p->mass = (double)p->WH * (double)N;
   p->epsilon = epsilon;
   if ((long long)C * p->groups >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: too many channels", who);
