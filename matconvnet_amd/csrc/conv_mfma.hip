@@ -82,16 +82,53 @@ __global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt,
 // out = alpha * (sum of the partial results of a split reduction) + beta*out + bias.  The partials are dense tensors
 // [n][co][q]; the destination is the layout the PixP describes (a dense tensor, one group's channels of a wider
 // tensor, or one stride class of a backward-data product).  The partials are added in split order: deterministic.
+// FLAT: the destination is the dense tensor itself (element i goes to element i) and n is a multiple of 4: 16-byte
+// accesses, no index arithmetic beyond the bias channel.  Otherwise 32-bit indices with multiply-shift divisions
+// (WIDE: tensors of 2^31 elements or more, plain 64-bit arithmetic).
+template <bool FLAT, bool WIDE>
 __global__ __launch_bounds__(256) void conv_pix_reduce(float* __restrict__ out, const float* __restrict__ partials,
-                                                       const float* __restrict__ bias, size_t n, PixP p) {
+                                                       const float* __restrict__ bias, size_t n, PixP p, FastDiv byCout) {
+  if (FLAT) {
+    const unsigned i4 = blockIdx.x * 256u + threadIdx.x;  // float4 index
+    if ((size_t)i4 * 4 >= n) return;
+    const v4f* src = (const v4f*)partials + i4;
+    const size_t stride4 = (size_t)p.partStride / 4;
+    v4f s = src[0];
+    for (int k = 1; k < p.rSplits; ++k) s += src[(size_t)k * stride4];
+    v4f v = p.alpha * s;
+    if (p.beta != 0.f) {
+      const v4f o = ((const v4f*)out)[i4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = fmaf(p.beta, o[j], v[j]);
+    }
+    if (bias) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int plane = p.byQ.div((int)(i4 * 4 + j));
+        v[j] += bias[plane - byCout.div(plane) * p.Cout];
+      }
+    }
+    ((v4f*)out)[i4] = v;
+    return;
+  }
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float s = partials[i];
   for (int k = 1; k < p.rSplits; ++k) s += partials[(size_t)k * p.partStride + i];
-  const int Q = p.OH * p.OW;
-  const size_t plane = i / Q;
-  const int q = (int)(i - plane * Q), co = (int)(plane % p.Cout);
-  const size_t img = plane / p.Cout;
+  int q, co;
+  size_t img;
+  if (WIDE) {
+    const int Q = p.OH * p.OW;
+    const size_t plane = i / Q;
+    q = (int)(i - plane * Q);
+    co = (int)(plane % p.Cout);
+    img = plane / p.Cout;
+  } else {
+    int plane, im;
+    p.byQ.divmod((int)i, &plane, &q);
+    byCout.divmod(plane, &im, &co);
+    img = (size_t)im;
+  }
   float* dst = out + img * (size_t)p.outImg + (size_t)co * p.outPlane + out_pixel_offset(p, q);
   float v = p.alpha * s;
   if (p.beta != 0.f) v = fmaf(p.beta, *dst, v);
@@ -855,7 +892,18 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
     p.rSplits = q.rSplits;
     p.partStride = q.partStride;
     KernelTimer timer("conv_pix_reduce", s);
-    hipLaunchKernelGGL(conv_pix_reduce, dim3((unsigned)((nOut + 255) / 256)), dim3(256), 0, s, out, partials, bias, nOut, p);
+    const FastDiv byCout(p.Cout);
+    const bool flat = p.dense != 0 && p.outImg == p.Cout * p.outPlane && nOut % 4 == 0 && nOut < (1ull << 31) &&
+                      aligned16(out) && aligned16(partials);
+    if (flat)
+      hipLaunchKernelGGL((conv_pix_reduce<true, false>), dim3((unsigned)((nOut / 4 + 255) / 256)), dim3(256), 0, s, out,
+                         partials, bias, nOut, p, byCout);
+    else if (nOut < (1ull << 31))
+      hipLaunchKernelGGL((conv_pix_reduce<false, false>), dim3((unsigned)((nOut + 255) / 256)), dim3(256), 0, s, out,
+                         partials, bias, nOut, p, byCout);
+    else
+      hipLaunchKernelGGL((conv_pix_reduce<false, true>), dim3((unsigned)((nOut + 255) / 256)), dim3(256), 0, s, out,
+                         partials, bias, nOut, p, byCout);
     return check_launch(who);
   }
   launch_shape(s, plan.shape, out, in, wt, bias, p, ut);
