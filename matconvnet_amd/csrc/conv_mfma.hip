@@ -805,6 +805,10 @@ PixPlan plan_pix(int Cout, long long M, int R) {
   if (BA == 128) { plan.shape = M <= 32 ? 7 : (blocks(128) >= 2048 ? 1 : 5); px = plan.shape == 7 ? 32 : (plan.shape == 1 ? 128 : 64); }
   else if (BA == 64) { plan.shape = blocks(256) >= 2048 ? 2 : (blocks(128) >= 2048 ? 4 : 6); px = plan.shape == 2 ? 256 : (plan.shape == 4 ? 128 : 64); }
   else { plan.shape = 3; px = 256; }
+  if (const int forced = tunable("conv_pix_tile", 0)) {  // (experiments: a shape that fits the channel tile)
+    static const int pxOf[8] = {0, 128, 256, 256, 128, 64, 64, 32}, baOf[8] = {0, 128, 64, 32, 64, 128, 64, 128};
+    if (forced >= 1 && forced <= 7 && baOf[forced] == BA) { plan.shape = forced; px = pxOf[forced]; }
+  }
   // fewer than two workgroups per CU with a long reduction each: split it, down to 16 steps of 16 rows per
   // workgroup, until about four workgroups per CU exist (values from a sweep over the 14x14 and 7x7 layers of
   // ResNet-50 at 32 images: 126 -> 89 us for 3x3x256x256)
@@ -817,6 +821,7 @@ PixPlan plan_pix(int Cout, long long M, int R) {
     long long want = (target + nb - 1) / nb;
     plan.splits = (int)std::max<long long>(1, std::min<long long>(want, nSteps / minSteps));
   }
+  if (const int forcedSplits = tunable("conv_split_force", 0)) plan.splits = std::max(1, std::min(forcedSplits, nSteps));
   return plan;
 }
 
