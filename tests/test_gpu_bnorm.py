@@ -1,6 +1,6 @@
 """GPU parity, batch normalisation.  Gate (max|diff|/max|ref| over each output): 1e-5 against the double
 instantiation of the reference algorithm fed the same float inputs.  The float instantiation sums ~1e5
-terms sequentially in float and is itself further than 1e-5 from the double one at BASELINE sizes, so the
+terms sequentially in float and is itself further than 1e-5 from the double one at the benchmark sizes, so the
 distance to it is asserted only to the looser bound it can support."""
 import os
 
@@ -86,7 +86,7 @@ def test_golden_vectors_from_reference(capi):
 
 
 def test_baseline_config_full_size(capi, ob):
-    """BASELINE config 2: 56x56x256x32, eps 1e-4, moments from the batch."""
+    """benchmark configuration 2: 56x56x256x32, eps 1e-4, moments from the batch."""
     w = workloads.bnorm_case()
     x, g, dy = w["x"], w["g"], w["dy"]
     dx, dg, db, mom = [capi.to_host(t) for t in capi.bnorm_backward(capi.to_device(x), capi.to_device(g), capi.to_device(dy), w["eps"])]
@@ -105,7 +105,7 @@ def test_baseline_config_full_size(capi, ob):
 
 
 def test_bottleneck_shapes(capi, ob):
-    """The two bnorm shapes of BASELINE config 4 (eps 1e-5)."""
+    """The two bnorm shapes of benchmark configuration 4 (eps 1e-5)."""
     for C in (64, 256):
         w = workloads.bnorm_case(seed=20 + C, C=C, N=8, eps=1e-5)
         x, g, dy = w["x"], w["g"], w["dy"]

@@ -128,7 +128,7 @@ def test_tap_major_and_channel_major_kernels_agree(capi, ob, case):
 
 
 def test_baseline_config1_full(capi, ob):
-    """BASELINE config 1: x 32x32x3x100, f 5x5x3x32, stride 1, pad 2 (the reference's CPU-runnable case)."""
+    """benchmark configuration 1: x 32x32x3x100, f 5x5x3x32, stride 1, pad 2 (the reference's CPU-runnable case)."""
     w = workloads.conv_single()
     errs = _check(capi, ob, w["x"], w["f"], w["b"], w["dy"], w["stride"], w["pad"], w["dilate"])
     print("conv cfg1:", errs)
@@ -139,7 +139,7 @@ def test_baseline_config1_full(capi, ob):
 
 @pytest.mark.parametrize("which", ["1x1_256_64", "3x3_64_64", "1x1_64_256"])
 def test_baseline_config4_conv_shapes_full(capi, ob, which):
-    """The three convolutions of the ResNet-50 bottleneck at N = 32, 56x56 (BASELINE config 4)."""
+    """The three convolutions of the ResNet-50 bottleneck at N = 32, 56x56 (benchmark configuration 4)."""
     r = np.random.default_rng(40)
     C, K, fs, pad = {"1x1_256_64": (256, 64, 1, 0), "3x3_64_64": (64, 64, 3, 1), "1x1_64_256": (64, 256, 1, 0)}[which]
     x = F(r.standard_normal((56, 56, C, 32), dtype=np.float32))
@@ -149,13 +149,13 @@ def test_baseline_config4_conv_shapes_full(capi, ob, which):
 
 
 def test_baseline_config5_reduced_batch(capi, ob):
-    """BASELINE config 5 geometry (56x56x256, 3x3x256x256, pad 1) at N = 2 against the oracle."""
+    """benchmark configuration 5 geometry (56x56x256, 3x3x256x256, pad 1) at N = 2 against the oracle."""
     w = workloads.conv_vgg(N=2)
     print("conv cfg5 (N=2):", _check(capi, ob, w["x"], w["f"], None, w["dy"], 1, 1, 1))
 
 
 def test_baseline_config5_full_size_properties(capi, ob):
-    """BASELINE config 5 at full size (N = 64): too big for the CPU oracle in a test, so
+    """benchmark configuration 5 at full size (N = 64): too big for the CPU oracle in a test, so
     (1) dzdx of single images is compared with the oracle run on those images alone (images are
         independent in backward-data),
     (2) dzdf / dzdb are linear in the batch: the full-batch result must equal the sum of the results on the

@@ -188,7 +188,7 @@ def test_bottleneck_block_end_to_end_small_batch(vl, ob):
 
 
 def test_bottleneck_block_full_config_stage_by_stage(vl, ob):
-    """BASELINE config 4 at its full size (N = 32, 56x56, 256/64 channels).  ReLU's derivative is
+    """benchmark configuration 4 at its full size (N = 32, 56x56, 256/64 channels).  ReLU's derivative is
     discontinuous, so an end-to-end comparison of gradients at this size flips a handful of masks between any
     two float implementations and says nothing about either.  Instead every stage of the GPU block is
     checked against the oracle applied to the SAME inputs (the GPU's own intermediate buffers): wiring,

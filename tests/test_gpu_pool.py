@@ -196,7 +196,7 @@ def test_golden_vectors_from_reference(capi):
 
 @pytest.mark.parametrize("ties", [False, True])
 def test_baseline_max_pool_full_size_bit_exact(capi, ob, ties):
-    """BASELINE config 3a: 112x112x64x32, 3x3 stride 2 pad 1, and its 8-level tie-stress variant."""
+    """benchmark configuration 3a: 112x112x64x32, 3x3 stride 2 pad 1, and its 8-level tie-stress variant."""
     w = workloads.pool_max_case(ties=ties)
     got, want = _run(capi, ob, w["x"], w["dy"], w["x"].shape, w["pool"], w["stride"], w["pad"], "max")
     assert bits_equal(got, want), count_bit_mismatches(got, want)
@@ -205,7 +205,7 @@ def test_baseline_max_pool_full_size_bit_exact(capi, ob, ties):
 
 
 def test_baseline_avg_pool_full_size_bit_exact(capi, ob):
-    """BASELINE config 3b: 56x56x256x32, 2x2 stride 2."""
+    """benchmark configuration 3b: 56x56x256x32, 2x2 stride 2."""
     w = workloads.pool_avg_case()
     got, want = _run(capi, ob, w["x"], w["dy"], w["x"].shape, w["pool"], w["stride"], w["pad"], "avg")
     assert bits_equal(got, want), count_bit_mismatches(got, want)

@@ -76,7 +76,7 @@ TORCH_CASES = [
     (7, 7, 6, 2, 1, 1, 6, 5, 1, 0, 1),
     (10, 10, 6, 2, 3, 3, 2, 9, 1, 1, 1),           # 3 filter groups (nnconv.m:144-161)
     (10, 9, 4, 2, 5, 3, 2, 4, (1, 2), (2, 2, 1, 1), 1),  # 2 groups, rectangular filter
-    (32, 32, 3, 2, 5, 5, 3, 8, 1, 2, 1),           # BASELINE config 1 geometry, reduced N and K
+    (32, 32, 3, 2, 5, 5, 3, 8, 1, 2, 1),           # benchmark configuration 1 geometry, reduced N and K
 ]
 
 
