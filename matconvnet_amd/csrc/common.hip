@@ -24,6 +24,7 @@ Tunable g_tunables[] = {
     {"pool_no_stream", 0},             // 1: max pooling skips the streaming kernel
     {"pool_walk", 0},                  // streaming kernel's tile order: 0 round-robin, 1 contiguous runs, 2 round-robin per XCD
     {"pool_blocks_per_cu", 3},         // persistent workgroups per compute unit of the streaming kernel
+    {"pool_forward_threads_k", 2048},  // threads (in 1024s) the four-rows-per-thread forward kernel aims at
     {"pool_force_gather", 0},          // 1: skip the ordered-pass kernel, use the general tiled gather
     {"bnorm_block_elems", 4096},       // minimum elements a bnorm reduction block should own
     {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)

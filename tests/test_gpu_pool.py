@@ -80,10 +80,13 @@ def test_forward_bit_exact_small(capi, ob, geom, method):
 
 @pytest.mark.parametrize("method", ["max", "avg"])
 @pytest.mark.parametrize("geom", [(40, 36, 3, 2, 3, 2, 1), (112, 112, 4, 2, 3, 2, 1), (21, 17, 2, 1, (7, 3), (1, 1), (3, 3, 1, 1)),
-                                  (30, 30, 1, 2, 9, 4, 4), (7, 7, 5, 3, 7, 1, 0), (300, 9, 2, 1, (2, 5), (2, 1), 0)])
+                                  (30, 30, 1, 2, 9, 4, 4), (7, 7, 5, 3, 7, 1, 0), (300, 9, 2, 1, (2, 5), (2, 1), 0),
+                                  (56, 56, 4, 2, 2, 2, 0), (8, 6, 3, 2, 3, 2, (1, 0, 1, 0)), (4, 2, 2, 1, 3, 2, 1),
+                                  (12, 10, 2, 3, 2, 2, (0, 1, 0, 1)), (42, 36, 2, 2, 3, 2, 1), (40, 35, 2, 2, 3, 2, 1)])
 def test_forward_bit_exact_larger_planes(capi, ob, method, geom):
-    """Forward pass on planes of several hundred elements, wide windows and whole-plane windows: the oracle's bits
-    (ties, NaN, infinities and zeros of both signs included)."""
+    """Forward pass on planes of several hundred elements, wide windows and whole-plane windows, and the
+    down-sampling cases that have a kernel of their own (3x3 / 2x2 windows, stride 2, heights that are and are not
+    multiples of 4): the oracle's bits (ties, NaN, infinities and zeros of both signs included)."""
     H, W, C, N, pool, stride, pad = geom
     shape = (H, W, C, N)
     x = _inputs(shape, 51, "special" if method == "max" else "normal")
