@@ -128,6 +128,39 @@ MCN_API int mcn_conv_backward_data_acc(mcn_stream_t stream, const mcn_conv_geom*
                                        float derInputMult, const float* filters, const float* derOutput,
                                        void* workspace, size_t workspaceBytes);
 
+/* Filter banks packed ahead.  The matrix kernels read the filters re-laid ("packed": rows = reduction index in the
+   order the kernel walks it, columns = output channels, padded to the tile).  mcn_conv_forward / mcn_conv_backward_data
+   pack into their workspace on every call -- a launch of a few microseconds that a 53-layer network pays 80 times per
+   step.  A caller whose filters stay put between calls (a network between two parameter updates, or for good when
+   it only evaluates) can pack once into a buffer of its own and hand it to the *_packed calls.  No counterpart in
+   the reference, whose GEMMs read the bank as stored (bits/nnconv.cu:126-134,256-264).
+     mcn_conv_packed_bytes   size of that buffer for one product (MCN_CONV_FORWARD or MCN_CONV_BACKWARD_DATA) of one
+                             geometry; 0 when the product reads no packed bank (direct kernels; 1x1 banks that
+                             backward-data reads as stored).  The layout depends on the whole geometry, N included.
+     mcn_conv_pack_filters   fills it (one launch per bank: one per filter group and stride class).
+     mcn_conv_pack_plan / _layout / _batch   the same for many layers in one launch: _plan appends the jobs of one
+                             product to a host array (filters and packed are the device addresses the jobs will
+                             read and write), _layout numbers the workgroups of all jobs and returns their total,
+                             and _batch, given a copy of the array in device memory, runs them all.
+     mcn_conv_forward_packed, mcn_conv_backward_data_packed   as mcn_conv_forward / mcn_conv_backward_data_acc, reading
+                             the banks from `packed` (NULL: pack on the fly as usual).  `filters` is still needed (banks
+                             that are read as stored).  The packed buffer must have been filled from these filters
+                             for this geometry and product: a stale buffer gives stale results. */
+typedef struct { unsigned long long opaque[10]; } mcn_conv_pack_job;
+MCN_API size_t mcn_conv_packed_bytes(const mcn_conv_geom* g, int product);
+MCN_API int mcn_conv_pack_filters(mcn_stream_t stream, const mcn_conv_geom* g, int product, const float* filters,
+                                  void* packed, size_t packedBytes);
+MCN_API int mcn_conv_pack_plan(const mcn_conv_geom* g, int product, const float* filters, void* packed, size_t packedBytes,
+                               mcn_conv_pack_job* jobs, int maxJobs, int* nJobs);
+MCN_API unsigned mcn_conv_pack_layout(mcn_conv_pack_job* jobs, int nJobs);
+MCN_API int mcn_conv_pack_batch(mcn_stream_t stream, const mcn_conv_pack_job* deviceJobs, int nJobs, unsigned totalBlocks);
+MCN_API int mcn_conv_forward_packed(mcn_stream_t stream, const mcn_conv_geom* g, float* y, float outMult, const float* x,
+                                    float inMult, const float* filters, const void* packed, size_t packedBytes,
+                                    const float* bias, void* workspace, size_t workspaceBytes);
+MCN_API int mcn_conv_backward_data_packed(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, float derInputMult,
+                                          const float* filters, const void* packed, size_t packedBytes,
+                                          const float* derOutput, void* workspace, size_t workspaceBytes);
+
 /* dzdf: FH x FW x FC x K, fully overwritten  (bits/nnconv.cu:280-311: im2row::forward + gemm 't','n'
    accumulated over images) */
 MCN_API int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters,

@@ -51,6 +51,13 @@ PROTOTYPES = {
     "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_taccum": (_i, [_vp, _vp, C.c_float, _vp, C.c_float, _vp, _sz]),
+    "mcn_conv_packed_bytes": (_sz, [_vp, _i]),
+    "mcn_conv_pack_filters": (_i, [_vp, _vp, _i, _vp, _vp, _sz]),
+    "mcn_conv_pack_plan": (_i, [_vp, _i, _vp, _vp, _sz, _vp, _i, _vp]),
+    "mcn_conv_pack_layout": (C.c_uint, [_vp, _i]),
+    "mcn_conv_pack_batch": (_i, [_vp, _vp, _i, C.c_uint]),
+    "mcn_conv_forward_packed": (_i, [_vp, _vp, _vp, C.c_float, _vp, C.c_float, _vp, _vp, _sz, _vp, _vp, _sz]),
+    "mcn_conv_backward_data_packed": (_i, [_vp, _vp, _vp, C.c_float, _vp, _vp, _sz, _vp, _vp, _sz]),
     "mcn_sgd_momentum": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _vp] + [C.c_double] * 4 + [C.c_int]),
     "mcn_conv_backward_data_acc": (_i, [_vp, C.POINTER(ConvGeom), _vp, C.c_float, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_filter": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
@@ -258,6 +265,71 @@ def conv_backward_data_acc(dx, mult, f, dy, g, ws=None):
     L = lib()
     wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_DATA))
     check(L.mcn_conv_backward_data_acc(stream(), C.byref(g), ptr(dx), float(mult), ptr(f), ptr(dy), wp, wn))
+    return dx
+
+
+class PackJob(C.Structure):
+    """mcn_conv_pack_job of include/mcn_hip.h (opaque)."""
+    _fields_ = [("opaque", C.c_ulonglong * 10)]
+
+
+def conv_packed_bytes(g, product):
+    return lib().mcn_conv_packed_bytes(C.byref(g), product)
+
+
+def conv_pack_filters(f, g, product):
+    """The filters packed ahead for one product (a uint8 device tensor; None when the product reads none)."""
+    n = conv_packed_bytes(g, product)
+    if n == 0:
+        return None
+    packed = _torch().empty(n, dtype=_torch().uint8, device="cuda")
+    check(lib().mcn_conv_pack_filters(stream(), C.byref(g), product, ptr(f), ptr(packed), n))
+    return packed
+
+
+def conv_pack_many(layers):
+    """layers: [(f, g, product)].  One buffer and ONE launch for all of them (mcn_conv_pack_plan / _layout / _batch);
+    returns the views [(packed or None)] in the same order."""
+    torch = _torch()
+    L = lib()
+    sizes = [conv_packed_bytes(g, product) for _, g, product in layers]
+    total = sum(sizes)
+    arena = torch.empty(max(total, 16), dtype=torch.uint8, device="cuda")
+    jobs = (PackJob * 256)()
+    n_jobs, at, views = 0, 0, []
+    for (f, g, product), size in zip(layers, sizes):
+        view = arena[at:at + size] if size else None
+        views.append(view)
+        if size:
+            got = C.c_int(0)
+            check(L.mcn_conv_pack_plan(C.byref(g), product, ptr(f), ptr(view), size,
+                                       C.byref(jobs, n_jobs * C.sizeof(PackJob)), 256 - n_jobs, C.byref(got)))
+            n_jobs += got.value
+        at += size
+    blocks = L.mcn_conv_pack_layout(jobs, n_jobs)
+    host = np.frombuffer(jobs, dtype=np.uint8, count=n_jobs * C.sizeof(PackJob)).copy()
+    device_jobs = torch.from_numpy(host).cuda() if n_jobs else None
+    check(L.mcn_conv_pack_batch(stream(), ptr(device_jobs), n_jobs, blocks))
+    torch.cuda.synchronize()   # (device_jobs must outlive the launch)
+    return views
+
+
+def conv_forward_packed(x, f, packed, b, g, y=None, out_mult=0.0, in_mult=1.0, ws=None):
+    ws = ws or _ws
+    if y is None:
+        y = empty(conv_out_shape(g))
+    wp, wn = ws.get(lib().mcn_conv_workspace_bytes(C.byref(g), CONV_FORWARD))
+    check(lib().mcn_conv_forward_packed(stream(), C.byref(g), ptr(y), out_mult, ptr(x), in_mult, ptr(f), ptr(packed),
+                                        packed.numel() if packed is not None else 0, ptr(b), wp, wn))
+    return y
+
+
+def conv_backward_data_packed(dx, mult, f, packed, dy, g, ws=None):
+    ws = ws or _ws
+    L = lib()
+    wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_DATA))
+    check(L.mcn_conv_backward_data_packed(stream(), C.byref(g), ptr(dx), float(mult), ptr(f), ptr(packed),
+                                          packed.numel() if packed is not None else 0, ptr(dy), wp, wn))
     return dx
 
 

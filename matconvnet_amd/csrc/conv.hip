@@ -2,6 +2,9 @@
 // kernels, and the bias-gradient reduction.
 #include "conv_common.hpp"
 
+#include <cstring>
+#include <vector>
+
 #include <algorithm>
 
 namespace mcn {
@@ -135,6 +138,116 @@ int mcn_conv_backward_data_acc(mcn_stream_t stream, const mcn_conv_geom* g, floa
   if (!derInput || !filters || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data: null tensor");
   if (!tunable("conv_force_direct", 0) && conv_mfma_backward_data_supported(p))
     return conv_backward_data_mfma(as_stream(stream), p, derInput, derInputMult, filters, derOutput, workspace, workspaceBytes);
+  return conv_backward_data_direct(as_stream(stream), p, derInput, derInputMult, filters, derOutput);
+}
+
+namespace {
+// the three uses of a packed-ahead buffer share the walk over a product's banks
+int walk_packed(hipStream_t s, const ConvP& p, int product, const float* filters, PackCtx* pk) {
+  float* dummy = const_cast<float*>(filters);  // (no tensor is touched when planning or packing)
+  if (product == MCN_CONV_FORWARD) {
+    if (!conv_mfma_forward_supported(p) || tunable("conv_force_direct", 0)) return MCN_SUCCESS;
+    return conv_forward_mfma(s, p, dummy, 0.f, dummy, 1.f, filters, nullptr, nullptr, 0, pk);
+  }
+  if (product == MCN_CONV_BACKWARD_DATA) {
+    if (!conv_mfma_backward_data_supported(p) || tunable("conv_force_direct", 0)) return MCN_SUCCESS;
+    return conv_backward_data_mfma(s, p, dummy, 0.f, filters, dummy, nullptr, 0, pk);
+  }
+  return fail(MCN_ILLEGAL_ARGUMENT, "packed filters exist for the forward and the backward-data product only");
+}
+static_assert(sizeof(PackJob) <= sizeof(mcn_conv_pack_job), "mcn_conv_pack_job must hold a PackJob");
+}  // namespace
+
+size_t mcn_conv_packed_bytes(const mcn_conv_geom* g, int product) {
+  ConvP p;
+  if (conv_setup(g, "mcn_conv_packed_bytes", &p) || p.N == 0) return 0;
+  PackCtx pk = {PackCtx::kPlan, nullptr, 0, 0, nullptr};
+  if (walk_packed(nullptr, p, product, nullptr, &pk)) return 0;
+  return pk.offset;
+}
+
+int mcn_conv_pack_filters(mcn_stream_t stream, const mcn_conv_geom* g, int product, const float* filters, void* packed,
+                          size_t packedBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_pack_filters", &p);
+  if (rc) return rc;
+  if (p.N == 0) return MCN_SUCCESS;
+  if (!filters || (!packed && packedBytes)) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_pack_filters: null argument");
+  if (!aligned16(packed)) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_pack_filters: the buffer must be 16-byte aligned");
+  PackCtx pk = {PackCtx::kPack, (char*)packed, packedBytes, 0, nullptr};
+  return walk_packed(as_stream(stream), p, product, filters, &pk);
+}
+
+int mcn_conv_pack_plan(const mcn_conv_geom* g, int product, const float* filters, void* packed, size_t packedBytes,
+                       mcn_conv_pack_job* jobs, int maxJobs, int* nJobs) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_pack_plan", &p);
+  if (rc) return rc;
+  if (!nJobs) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_pack_plan: null argument");
+  *nJobs = 0;
+  if (p.N == 0) return MCN_SUCCESS;
+  std::vector<PackJob> found;
+  PackCtx pk = {PackCtx::kPlan, (char*)packed, packedBytes, 0, &found};
+  if ((rc = walk_packed(nullptr, p, product, filters, &pk))) return rc;
+  if (pk.offset > packedBytes) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_pack_plan: packed filter buffer too small");
+  if ((int)found.size() > maxJobs) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_pack_plan: more than %d jobs", maxJobs);
+  for (size_t i = 0; i < found.size(); ++i) {
+    std::memset(&jobs[i], 0, sizeof(jobs[i]));
+    std::memcpy(&jobs[i], &found[i], sizeof(PackJob));
+  }
+  *nJobs = (int)found.size();
+  return MCN_SUCCESS;
+}
+
+unsigned mcn_conv_pack_layout(mcn_conv_pack_job* jobs, int nJobs) {
+  unsigned at = 0;
+  for (int i = 0; i < nJobs; ++i) {
+    PackJob j;
+    std::memcpy(&j, &jobs[i], sizeof(PackJob));
+    j.firstBlock = at;
+    at += j.blocks;
+    std::memcpy(&jobs[i], &j, sizeof(PackJob));
+  }
+  return at;
+}
+
+int mcn_conv_pack_batch(mcn_stream_t stream, const mcn_conv_pack_job* deviceJobs, int nJobs, unsigned totalBlocks) {
+  if (nJobs > 0 && !deviceJobs) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_pack_batch: null argument");
+  static_assert(sizeof(mcn_conv_pack_job) == sizeof(PackJob), "a device array of mcn_conv_pack_job is read as PackJob[]");
+  return conv_pack_batch(as_stream(stream), (const PackJob*)deviceJobs, nJobs, totalBlocks);
+}
+
+int mcn_conv_forward_packed(mcn_stream_t stream, const mcn_conv_geom* g, float* y, float outMult, const float* x,
+                            float inMult, const float* filters, const void* packed, size_t packedBytes, const float* bias,
+                            void* workspace, size_t workspaceBytes) {
+  if (!packed) return mcn_conv_forward(stream, g, y, outMult, x, inMult, filters, bias, workspace, workspaceBytes);
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_forward", &p);
+  if (rc) return rc;
+  if ((size_t)p.outH * p.outW * p.K * p.N == 0) return MCN_SUCCESS;
+  if (!y || !x || !filters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_forward: null tensor");
+  if (!tunable("conv_force_direct", 0) && conv_mfma_forward_supported(p)) {
+    PackCtx pk = {PackCtx::kUse, (char*)const_cast<void*>(packed), packedBytes, 0, nullptr};
+    return conv_forward_mfma(as_stream(stream), p, y, outMult, x, inMult, filters, bias, workspace, workspaceBytes, &pk);
+  }
+  return conv_forward_direct(as_stream(stream), p, y, outMult, x, inMult, filters, bias);
+}
+
+int mcn_conv_backward_data_packed(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, float derInputMult,
+                                  const float* filters, const void* packed, size_t packedBytes, const float* derOutput,
+                                  void* workspace, size_t workspaceBytes) {
+  if (!packed)
+    return mcn_conv_backward_data_acc(stream, g, derInput, derInputMult, filters, derOutput, workspace, workspaceBytes);
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_data", &p);
+  if (rc) return rc;
+  if ((size_t)p.H * p.W * p.C * p.N == 0) return MCN_SUCCESS;
+  if (!derInput || !filters || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data: null tensor");
+  if (!tunable("conv_force_direct", 0) && conv_mfma_backward_data_supported(p)) {
+    PackCtx pk = {PackCtx::kUse, (char*)const_cast<void*>(packed), packedBytes, 0, nullptr};
+    return conv_backward_data_mfma(as_stream(stream), p, derInput, derInputMult, filters, derOutput, workspace,
+                                   workspaceBytes, &pk);
+  }
   return conv_backward_data_direct(as_stream(stream), p, derInput, derInputMult, filters, derOutput);
 }
 

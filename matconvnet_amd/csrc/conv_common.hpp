@@ -3,6 +3,8 @@
 
 #include "mcn_internal.hpp"
 
+#include <vector>
+
 namespace mcn {
 
 struct ConvP {
@@ -22,15 +24,45 @@ int conv_forward_direct(hipStream_t s, const ConvP& p, float* y, float outMult, 
 int conv_backward_data_direct(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy);
 int conv_backward_filter_direct(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy);
 
+// The taps of a stored FH x FW filter that take part in one product: (i0 + a*iStep, j0 + b*jStep), a < nI, b < nJ
+// (all of them for a plain layer; one stride class for the backward-data product of a strided layer).
+struct TapSet {
+  int FH, FW;            // the filter as stored
+  int i0, iStep, nI;
+  int j0, jStep, nJ;
+};
+
+// One re-laying of (part of) a filter bank into the order the MFMA kernels read: a launch of conv_pack_weights, or
+// one entry of a batched launch.  Plain data: it crosses the C ABI as mcn_conv_pack_job.
+struct PackJob {
+  float* wt;
+  const float* f;
+  TapSet taps;
+  int Cin, Cout, rPad, coutPad, backward, tapMajor;
+  unsigned firstBlock, blocks;  // workgroups [firstBlock, firstBlock + blocks) of a batched launch
+};
+
+// Filter banks packed ahead of the calls that use them.  The products of a layer visit their banks in a fixed
+// order (groups, then stride classes); every bank takes a 256-byte aligned slot of the caller's buffer in that
+// order, so planning, packing and using agree on where each one lies.
+struct PackCtx {
+  enum Mode { kPlan, kPack, kUse };
+  Mode mode;
+  char* base;                  // the caller's buffer (null when only the size is wanted)
+  size_t capacity, offset;
+  std::vector<PackJob>* jobs;  // kPlan: the jobs are appended here instead of being launched
+};
+
 // MFMA implicit-GEMM kernels (groups == 1).  *_supported says whether the fast path covers `p`.
 bool conv_mfma_forward_supported(const ConvP& p);
 bool conv_mfma_backward_data_supported(const ConvP& p);
 bool conv_mfma_backward_filter_supported(const ConvP& p);
 size_t conv_mfma_workspace_bytes(const ConvP& p, int product);
 int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
-                      const float* f, const float* b, void* ws, size_t wsBytes);
+                      const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk = nullptr);
 int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
-                            void* ws, size_t wsBytes);
+                            void* ws, size_t wsBytes, PackCtx* pk = nullptr);
+int conv_pack_batch(hipStream_t s, const PackJob* deviceJobs, int nJobs, unsigned totalBlocks);
 int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,
                               size_t wsBytes);
 

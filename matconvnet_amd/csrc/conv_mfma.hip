@@ -45,18 +45,9 @@ constexpr int kMaxTaps = 128;
 //   3x3 layers through the memory fabric 8 times over.
 //   forward:        ci = c, co = k : f[t + T*c + FV*k]
 //   backward-data:  ci = k, co = c : f[t + T*(c + C*k)]
-// Only the taps (i0 + a*iStep, j0 + b*jStep), a < nI, b < nJ, of the FH x FW filter take part (all of them for a
-// plain layer; one stride class for the backward-data product of a strided layer); T = nI*nJ, t = a + nI*b.
-struct TapSet {
-  int FH, FW;            // the filter as stored
-  int i0, iStep, nI;
-  int j0, jStep, nJ;
-};
-
-__global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt, const float* __restrict__ f,
-                                                         TapSet ts, int Cin, int Cout, int rPad, int coutPad,
-                                                         int backward, int tapMajor) {
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+// Only the taps of the TapSet take part; T = nI*nJ, t = a + nI*b.
+__device__ __forceinline__ void pack_element(float* __restrict__ wt, const float* __restrict__ f, const TapSet& ts, int Cin,
+                                             int Cout, int rPad, int coutPad, int backward, int tapMajor, size_t idx) {
   if (idx >= (size_t)rPad * coutPad) return;
   const int T = ts.nI * ts.nJ;
   const int r = (int)(idx / coutPad), co = (int)(idx - (size_t)r * coutPad);
@@ -77,6 +68,25 @@ __global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt,
     v = backward ? f[tf + Tf * (co + (size_t)Cout * ci)] : f[tf + Tf * ci + Tf * Cin * co];
   }
   wt[idx] = v;
+}
+
+__global__ __launch_bounds__(256) void conv_pack_weights(float* __restrict__ wt, const float* __restrict__ f,
+                                                         TapSet ts, int Cin, int Cout, int rPad, int coutPad,
+                                                         int backward, int tapMajor) {
+  pack_element(wt, f, ts, Cin, Cout, rPad, coutPad, backward, tapMajor, (size_t)blockIdx.x * 256 + threadIdx.x);
+}
+
+// Many banks in one launch: workgroup b belongs to the job whose [firstBlock, firstBlock + blocks) holds b.
+__global__ __launch_bounds__(256) void conv_pack_many(const PackJob* __restrict__ jobs, int nJobs) {
+  int lo = 0, hi = nJobs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) / 2;
+    if (jobs[mid].firstBlock <= blockIdx.x) lo = mid;
+    else hi = mid - 1;
+  }
+  const PackJob j = jobs[lo];
+  pack_element(j.wt, j.f, j.taps, j.Cin, j.Cout, j.rPad, j.coutPad, j.backward, j.tapMajor,
+               (size_t)(blockIdx.x - j.firstBlock) * 256 + threadIdx.x);
 }
 
 // out = alpha * (sum of the partial results of a split reduction) + beta*out + bias.  The partials are dense tensors
@@ -828,26 +838,53 @@ PixPlan plan_pix(int Cout, long long M, int R) {
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 int run_pix(hipStream_t s, const char* who, float* out, const float* in, const float* f, const float* bias, PixP p,
-            const TapSet& taps, int backward, void* ws, size_t wsBytes) {
+            const TapSet& taps, int backward, void* ws, size_t wsBytes, PackCtx* pk) {
   const int BA = pick_channels_tile(p.Cout);
   const int rPad = (p.R + 15) / 16 * 16;
   p.coutPad = (p.Cout + BA - 1) / BA * BA;
   const PixPlan plan = plan_pix(p.Cout, p.M, p.R);
   const size_t nOut = (size_t)p.N * p.Cout * p.OH * p.OW;
   const size_t needW = (size_t)rPad * p.coutPad * sizeof(float);
-  const size_t need = plan.splits > 1 ? align256(needW) + (size_t)plan.splits * nOut * sizeof(float) : needW;
-  if (!ws || wsBytes < need) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small (%zu < %zu bytes)", who, wsBytes, need);
-  if (!aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
-  float* wt = (float*)ws;
   const size_t nW = (size_t)rPad * p.coutPad;
   // uniform-tap variant: whole 16-row steps inside one tap, and 32-bit element offsets into the gathered tensor
   const long long inSpan = (long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW;  // elements from `in` to the end
   const bool ut = p.Cin % 16 == 0 && inSpan < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
-  int rc = MCN_SUCCESS;
   // The backward-data product of a 1x1 bank whose extents need no padding reads it as it is stored: rows = filters,
   // columns = the filters' channels, which is the packed order.
-  if (backward && taps.FH * taps.FW == 1 && rPad == p.R && p.coutPad == p.Cout && aligned16(f)) {
+  const bool asStored = backward && taps.FH * taps.FW == 1 && rPad == p.R && p.coutPad == p.Cout && aligned16(f);
+  float* slot = nullptr;  // this bank's place in a buffer packed ahead
+  if (pk && !asStored) {
+    slot = pk->base ? (float*)(pk->base + pk->offset) : nullptr;
+    pk->offset += align256(needW);
+    if (pk->mode != PackCtx::kPlan && pk->offset > pk->capacity)
+      return fail(MCN_ILLEGAL_ARGUMENT, "%s: packed filter buffer too small (%zu < %zu bytes)", who, pk->capacity, pk->offset);
+  }
+  if (pk && pk->mode != PackCtx::kUse) {
+    if (asStored) return MCN_SUCCESS;
+    if (pk->mode == PackCtx::kPlan) {
+      if (pk->jobs) {
+        PackJob j;
+        j.wt = slot; j.f = f; j.taps = taps;
+        j.Cin = p.Cin; j.Cout = p.Cout; j.rPad = rPad; j.coutPad = p.coutPad; j.backward = backward; j.tapMajor = ut ? 1 : 0;
+        j.firstBlock = 0; j.blocks = (unsigned)((nW + 255) / 256);
+        pk->jobs->push_back(j);
+      }
+      return MCN_SUCCESS;
+    }
+    KernelTimer timer("conv_pack_weights", s);
+    hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, slot, f, taps, p.Cin, p.Cout,
+                       rPad, p.coutPad, backward, ut ? 1 : 0);
+    return check_launch(who);
+  }
+  const size_t need = plan.splits > 1 ? align256(needW) + (size_t)plan.splits * nOut * sizeof(float) : (slot || asStored ? 0 : needW);
+  if (need && (!ws || wsBytes < need)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small (%zu < %zu bytes)", who, wsBytes, need);
+  if (need && !aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
+  float* wt = (float*)ws;
+  int rc = MCN_SUCCESS;
+  if (asStored) {
     wt = const_cast<float*>(f);
+  } else if (slot) {
+    wt = slot;
   } else {
     KernelTimer timer("conv_pack_weights", s);
     hipLaunchKernelGGL(conv_pack_weights, dim3((unsigned)((nW + 255) / 256)), dim3(256), 0, s, wt, f, taps, p.Cin, p.Cout,
@@ -998,7 +1035,7 @@ void dense_layout(PixP* q) {
 
 namespace {
 int forward_group(hipStream_t s, const ConvP& p, Wide wd, float* y, float outMult, const float* x, float inMult,
-                  const float* f, const float* b, void* ws, size_t wsBytes) {
+                  const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk) {
   PixP q;
   q.IH = p.H; q.IW = p.W; q.Cin = p.C;
   q.OH = p.outH; q.OW = p.outW; q.Cout = p.K;
@@ -1013,19 +1050,26 @@ int forward_group(hipStream_t s, const ConvP& p, Wide wd, float* y, float outMul
   dense_layout(&q);
   q.inImg = wd.xImg;
   q.outImg = wd.yImg;
-  return run_pix(s, "mcn_conv_forward", y, x, f, b, q, all_taps(p), 0, ws, wsBytes);
+  return run_pix(s, "mcn_conv_forward", y, x, f, b, q, all_taps(p), 0, ws, wsBytes, pk);
 }
 }  // namespace
 
+int conv_pack_batch(hipStream_t s, const PackJob* deviceJobs, int nJobs, unsigned totalBlocks) {
+  if (nJobs <= 0 || totalBlocks == 0) return MCN_SUCCESS;
+  KernelTimer timer("conv_pack_many", s);
+  hipLaunchKernelGGL(conv_pack_many, dim3(totalBlocks), dim3(256), 0, s, deviceJobs, nJobs);
+  return check_launch("mcn_conv_pack_batch");
+}
+
 int conv_forward_mfma(hipStream_t s, const ConvP& original, float* y, float outMult, const float* x, float inMult,
-                      const float* f, const float* b, void* ws, size_t wsBytes) {
+                      const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk) {
   const ConvP p = fc_view(original);
   const ConvP g = group_view(p);
   const Wide wd = wide_of(p);
   const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
   for (int i = 0; i < p.groups; ++i) {
     int rc = forward_group(s, g, wd, y + i * p.Kg * Q, outMult, x + i * p.FC * HW, inMult, f + i * p.Kg * FV,
-                           b ? b + i * p.Kg : nullptr, ws, wsBytes);
+                           b ? b + i * p.Kg : nullptr, ws, wsBytes, pk);
     if (rc) return rc;
   }
   return MCN_SUCCESS;
@@ -1039,7 +1083,7 @@ int conv_forward_mfma(hipStream_t s, const ConvP& original, float* y, float outM
 // with a subset of the taps.  Classes no tap reaches (1x1 filters with stride 2: three of four) are zeros.
 namespace {
 int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float dxMult, const float* f, const float* dy,
-                        void* ws, size_t wsBytes) {
+                        void* ws, size_t wsBytes, PackCtx* pk) {
   PixP q;
   q.IH = p.outH; q.IW = p.outW; q.Cin = p.K;
   q.N = p.N;
@@ -1056,7 +1100,7 @@ int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float
     dense_layout(&q);
     q.inImg = wd.yImg;
     q.outImg = wd.xImg;
-    return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, all_taps(p), 1, ws, wsBytes);
+    return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, all_taps(p), 1, ws, wsBytes, pk);
   }
   // one class at a time (the caller has dealt with the classes no tap reaches)
   for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
@@ -1078,7 +1122,7 @@ int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float
       t.FH = p.FH; t.FW = p.FW;
       t.i0 = ai.first; t.iStep = ai.step; t.nI = ai.count;
       t.j0 = aj.first; t.jStep = aj.step; t.nJ = aj.count;
-      int rc = run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, c, t, 1, ws, wsBytes);
+      int rc = run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, c, t, 1, ws, wsBytes, pk);
       if (rc) return rc;
     }
   return MCN_SUCCESS;
@@ -1086,14 +1130,16 @@ int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float
 }  // namespace
 
 int conv_backward_data_mfma(hipStream_t s, const ConvP& original, float* dx, float dxMult, const float* f, const float* dy,
-                            void* ws, size_t wsBytes) {
+                            void* ws, size_t wsBytes, PackCtx* pk) {
   const ConvP p = fc_view(original);
+  const bool compute = !pk || pk->mode == PackCtx::kUse;
   // stride classes no tap reaches get no launch: they are zeros (or keep what is there, when accumulating)
   bool anyEmpty = false;
   for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
     for (int ph = 0; ph < p.sy && ph < p.H; ++ph)
       if (stride_axis(ph, p.pt, p.dy, p.sy, p.FH).count == 0 || stride_axis(pw, p.pl, p.dx, p.sx, p.FW).count == 0) anyEmpty = true;
-  if (anyEmpty && dxMult == 0.f) {
+  if (!compute) {
+  } else if (anyEmpty && dxMult == 0.f) {
     int rc = mcn_fill((mcn_stream_t)s, dx, 0.f, (size_t)p.H * p.W * p.C * p.N);
     if (rc) return rc;
   } else if (anyEmpty && dxMult != 1.f) {
@@ -1103,7 +1149,7 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& original, float* dx, flo
   const Wide wd = wide_of(p);
   const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
   for (int i = 0; i < p.groups; ++i) {
-    int rc = backward_data_group(s, g, wd, dx + i * p.FC * HW, dxMult, f + i * p.Kg * FV, dy + i * p.Kg * Q, ws, wsBytes);
+    int rc = backward_data_group(s, g, wd, dx + i * p.FC * HW, dxMult, f + i * p.Kg * FV, dy + i * p.Kg * Q, ws, wsBytes, pk);
     if (rc) return rc;
   }
   return MCN_SUCCESS;

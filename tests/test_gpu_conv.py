@@ -397,3 +397,60 @@ def test_tensors_over_2_gib_match_small_batches(capi):
         assert float((ys - y[sl]).abs().max()) <= 2e-4 * float(ys.abs().max())
         dxs, _, _ = capi.conv_backward(x[sl].contiguous(), f, ys, gs, want=(True, False, False))
         assert float((dxs - dx[sl]).abs().max()) <= 2e-4 * float(dxs.abs().max())
+
+
+PACKED_CASES = [  # (H, W, C, N, FH, FW, K, stride, pad, dilate, groups)
+    (14, 14, 64, 3, 1, 1, 128, 1, 0, 1, 1),     # 1x1: backward-data reads the bank as stored
+    (14, 14, 48, 3, 1, 1, 72, 1, 0, 1, 1),      # 1x1 whose extents need padding
+    (12, 10, 32, 2, 3, 3, 64, 1, 1, 1, 1),      # 3x3
+    (13, 11, 32, 2, 3, 3, 64, 2, 1, 1, 1),      # stride 2: four stride classes, each its own bank
+    (12, 12, 64, 2, 1, 1, 128, 2, 0, 1, 1),     # strided 1x1: one class
+    (9, 9, 3, 2, 5, 5, 16, 1, 2, 1, 1),         # 3 channels: the general (not uniform-tap) order
+    (10, 10, 32, 2, 3, 3, 32, 1, 1, 1, 2),      # two filter groups
+    (6, 6, 16, 4, 6, 6, 40, 1, 0, 1, 1),        # fully connected
+    (14, 14, 256, 4, 3, 3, 256, 1, 1, 1, 1),    # split reduction
+]
+
+
+@pytest.mark.parametrize("case", PACKED_CASES)
+def test_filters_packed_ahead_give_the_same_bits(capi, case):
+    """Forward and backward-data (overwriting and accumulating) with the banks packed ahead, one layer at a time and
+    several layers in one batched launch, against the calls that pack on the fly."""
+    import torch
+    H, W, Cc, N, FH, FW, K, stride, pad, dilate, groups = case
+    r = np.random.default_rng(5)
+    xs, fs = (H, W, Cc, N), (FH, FW, Cc // groups, K)
+    g = capi.conv_geom(xs, fs, stride, pad, dilate)
+    x, f = capi.to_device(F(r.standard_normal(xs))), capi.to_device(F(r.standard_normal(fs)))
+    b = capi.to_device(r.standard_normal(K).astype(np.float32))
+    dy = capi.to_device(F(r.standard_normal(capi.conv_out_shape(g))))
+    base = capi.to_device(F(r.standard_normal(xs)))
+    want_y = capi.conv_forward(x, f, b, g)
+    want_dx = capi.conv_backward_data_acc(capi.empty(xs), 0.0, f, dy, g)
+    want_acc = capi.conv_backward_data_acc(base.clone(), 1.0, f, dy, g)
+    # a second layer packed in the same batch
+    g2 = capi.conv_geom((8, 8, 32, 2), (3, 3, 32, 32), 1, 1, 1)
+    f2 = capi.to_device(F(r.standard_normal((3, 3, 32, 32))))
+    for how in ("single", "batch"):
+        if how == "single":
+            pf, pb = capi.conv_pack_filters(f, g, capi.CONV_FORWARD), capi.conv_pack_filters(f, g, capi.CONV_BACKWARD_DATA)
+        else:
+            _, pf, pb, _ = capi.conv_pack_many([(f2, g2, capi.CONV_FORWARD), (f, g, capi.CONV_FORWARD),
+                                                (f, g, capi.CONV_BACKWARD_DATA), (f2, g2, capi.CONV_BACKWARD_DATA)])
+        assert (pf is None) == (capi.conv_packed_bytes(g, capi.CONV_FORWARD) == 0)
+        assert torch.equal(capi.conv_forward_packed(x, f, pf, b, g), want_y), how
+        assert torch.equal(capi.conv_backward_data_packed(capi.empty(xs), 0.0, f, pb, dy, g), want_dx), how
+        assert torch.equal(capi.conv_backward_data_packed(base.clone(), 1.0, f, pb, dy, g), want_acc), how
+    # the first case reads the 1x1 bank as stored: nothing to pack for backward-data
+    if case == PACKED_CASES[0]:
+        assert capi.conv_packed_bytes(g, capi.CONV_BACKWARD_DATA) == 0 and capi.conv_packed_bytes(g, capi.CONV_FORWARD) > 0
+
+
+def test_packed_buffer_too_small_is_refused(capi):
+    import ctypes as C
+    g = capi.conv_geom((8, 8, 32, 2), (3, 3, 32, 32), 1, 1, 1)
+    f = capi.to_device(F(np.ones((3, 3, 32, 32))))
+    n = capi.conv_packed_bytes(g, capi.CONV_FORWARD)
+    small = capi.to_device(np.zeros(n // 8, np.float32))
+    rc = capi.lib().mcn_conv_pack_filters(capi.stream(), C.byref(g), capi.CONV_FORWARD, capi.ptr(f), capi.ptr(small), n // 2)
+    assert rc != 0 and b"too small" in capi.lib().mcn_last_error_message()
