@@ -62,7 +62,9 @@ def kernel_time(capi, kernel, launch, reps):
 def bench_block(vlapi, capi, workloads, steps, warmup):
     w = workloads.bottleneck_case()
     N = w["x"].shape[3]
-    blk = vlapi.Bottleneck(N=N, eps=w["eps"], fused=True)
+    # fused: ReLU / shortcut sum folded into batch normalisation; packed: the filter banks are re-laid for the matrix
+    # kernels by ONE launch at the start of every step (as after an update of the filters) instead of one per product
+    blk = vlapi.Bottleneck(N=N, eps=w["eps"], fused=True, packed=True)
     for k in ("x", "f1", "f2", "f3", "g1", "b1", "g2", "b2", "g3", "b3"):
         blk.set(k, w[k])
     blk.set("dzdy", w["dy"])
@@ -89,7 +91,7 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
         "eltwise_kernel": 0.0,                                    # (nothing left: every element-wise layer is folded)
     }
     fam = {}
-    for name in ["conv_ws_mfma", "conv_pix_mfma"] + list(conv_flops) + list(hbm_bytes) + ["conv_wgrad_reduce", "conv_pack_weights"]:
+    for name in ["conv_ws_mfma", "conv_pix_mfma"] + list(conv_flops) + list(hbm_bytes) + ["conv_wgrad_reduce", "conv_pack_weights", "conv_pack_many"]:
         capi.profile_begin(name)
         blk.run(steps)
         n, ms = capi.profile_end()

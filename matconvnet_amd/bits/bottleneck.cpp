@@ -13,7 +13,7 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
                        Context* shared)
     : H(H), W(W), C(C), M(M), N(N), Cout(CoutArg > 0 ? CoutArg : C), stride(stride), Ho((H - 1) / stride + 1),
       Wo((W - 1) / stride + 1), adapter(adapter), epsilon(epsilon), context(shared ? *shared : ownContext),
-      error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), testMode(false), sideStream(NULL) {
+      error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), testMode(false), packed(false), packedArena(NULL), packedJobs(NULL), packedBlocks(0), sideStream(NULL) {
   for (int i = 0; i < 5; ++i) events[i] = NULL;
   if (!adapter && (Cout != C || stride != 1)) {
     error = VLE_IllegalArgument;
@@ -83,6 +83,91 @@ Bottleneck::~Bottleneck() {
   }
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
+  if (packedArena) (void)hipFree(packedArena);
+  if (packedJobs) (void)hipFree(packedJobs);
+}
+
+#define STEP(stage, call)                                   \
+  do {                                                      \
+    mark(stage, 1);                                         \
+    ErrorCode e_ = (call);                                  \
+    mark(stage, 0);                                         \
+    if (e_ != VLE_Success) return fail(e_, stage);          \
+  } while (0)
+
+#define ABI(stage, call)                                                                    \
+  do {                                                                                      \
+    mark(stage, 1);                                                                         \
+    int rc_ = (call);                                                                       \
+    mark(stage, 0);                                                                         \
+    if (rc_ != 0) {                                                                         \
+      context.setError((ErrorCode)rc_, mcn_last_error_message());                           \
+      return fail((ErrorCode)rc_, stage);                                                   \
+    }                                                                                       \
+  } while (0)
+
+// The four convolutions in a fixed order: 1x1 in, 3x3, 1x1 out, adapter.
+ErrorCode Bottleneck::setPacked(bool on) {
+  if (packedArena) (void)hipFree(packedArena);
+  if (packedJobs) (void)hipFree(packedJobs);
+  packedArena = NULL;
+  packedJobs = NULL;
+  jobs.clear();
+  packed = false;
+  if (!on || error != VLE_Success) return error;
+  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),
+      cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
+  struct Layer { nn::Convolution* op; char const* data; char const* filter; };
+  const Layer layers[4] = {{&c1, "x", "f1"}, {&c2, "r1", "f2"}, {&c1, "r2", "f3"}, {&cs, "x", "fs"}};
+  const int count = adapter ? 4 : 3;
+  std::size_t total = 0;
+  for (int l = 0; l < count; ++l)
+    for (int product = 0; product < 2; ++product) {  // MCN_CONV_FORWARD, MCN_CONV_BACKWARD_DATA
+      banks[l][product].offset = total;
+      banks[l][product].bytes = layers[l].op->packedBytes(product, slot(layers[l].data).getShape(), slot(layers[l].filter).getShape());
+      total += banks[l][product].bytes;
+    }
+  if (hipMalloc(&packedArena, total ? total : 16) != hipSuccess) {
+    (void)hipGetLastError();
+    packedArena = NULL;
+    message = "cannot allocate the packed filter banks";
+    return VLE_OutOfGPUMemeory;
+  }
+  for (int l = 0; l < count; ++l)
+    for (int product = 0; product < 2; ++product) {
+      if (banks[l][product].bytes == 0) continue;
+      ErrorCode e = layers[l].op->planPack(product, slot(layers[l].data).getShape(), slot(layers[l].filter),
+                                           (char*)packedArena + banks[l][product].offset, banks[l][product].bytes, jobs);
+      if (e != VLE_Success) return fail(e, "planPack");
+    }
+  packed = true;
+  return VLE_Success;
+}
+
+void Bottleneck::attachPacked(nn::Convolution& c1, nn::Convolution& c2, nn::Convolution& c3, nn::Convolution& cs) {
+  if (!packed) return;
+  nn::Convolution* ops[4] = {&c1, &c2, &c3, &cs};
+  for (int l = 0; l < (adapter ? 4 : 3); ++l)
+    ops[l]->usePacked(banks[l][0].bytes ? (char*)packedArena + banks[l][0].offset : NULL, banks[l][0].bytes,
+                      banks[l][1].bytes ? (char*)packedArena + banks[l][1].offset : NULL, banks[l][1].bytes);
+}
+
+ErrorCode Bottleneck::pack() {
+  if (!packed) return VLE_Success;
+  if (!packedJobs && !jobs.empty()) {
+    std::vector<mcn_conv_pack_job> numbered(jobs);
+    packedBlocks = mcn_conv_pack_layout(numbered.data(), (int)numbered.size());
+    const std::size_t bytes = numbered.size() * sizeof(mcn_conv_pack_job);
+    if (hipMalloc(&packedJobs, bytes) != hipSuccess ||
+        hipMemcpy(packedJobs, numbered.data(), bytes, hipMemcpyHostToDevice) != hipSuccess) {
+      (void)hipGetLastError();
+      message = "cannot upload the packing jobs";
+      return VLE_Cuda;
+    }
+  }
+  ABI("pack", mcn_conv_pack_batch(context.getHipHelper().getStream(), (mcn_conv_pack_job const*)packedJobs, (int)jobs.size(),
+                                  packedBlocks));
+  return VLE_Success;
 }
 
 Tensor Bottleneck::make(std::string const& name, TensorShape const& shape) {
@@ -116,6 +201,7 @@ float* Bottleneck::buffer(std::string const& name, std::size_t* count) {
 }
 
 ErrorCode Bottleneck::alias(std::string const& name, float* memory) {
+  if (packed) setPacked(false);  // (the packing jobs hold the old addresses)
   for (std::size_t i = 0; i < slots.size(); ++i) {
     if (slots[i].name != name) continue;
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
@@ -138,31 +224,13 @@ ErrorCode Bottleneck::fail(ErrorCode e, char const* where) {
   return e;
 }
 
-#define STEP(stage, call)                                   \
-  do {                                                      \
-    mark(stage, 1);                                         \
-    ErrorCode e_ = (call);                                  \
-    mark(stage, 0);                                         \
-    if (e_ != VLE_Success) return fail(e_, stage);          \
-  } while (0)
-
-#define ABI(stage, call)                                                                    \
-  do {                                                                                      \
-    mark(stage, 1);                                                                         \
-    int rc_ = (call);                                                                       \
-    mark(stage, 0);                                                                         \
-    if (rc_ != 0) {                                                                         \
-      context.setError((ErrorCode)rc_, mcn_last_error_message());                           \
-      return fail((ErrorCode)rc_, stage);                                                   \
-    }                                                                                       \
-  } while (0)
-
 ErrorCode Bottleneck::forward() {
   if (error != VLE_Success) return error;
   void* st = context.getHipHelper().getStream();
   Tensor none;
   nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),
-      cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
+      c3(context, 1, 1, 0, 0, 0, 0, 1, 1), cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
+  attachPacked(c1, c2, c3, cs);
   nn::BatchNorm bn(context, epsilon);
   const std::size_t nMid = slot("a1").getNumElements(), nMidOut = slot("a2").getNumElements(),
                     nOut = slot("a3").getNumElements();
@@ -196,7 +264,7 @@ ErrorCode Bottleneck::forward() {
     if (!ws) return fail(context.getLastError(), "workspace");
     ABI("bn2_fwd", mcn_bnorm_forward_fused(st, buffer("r2"), buffer(m2), buffer("a2"), buffer("g2"), buffer("b2"), NULL, 1,
                                            Ho, Wo, M, N, epsilon, given, ws, wsMid));
-    STEP("conv3_fwd", c1.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
+    STEP("conv3_fwd", c3.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
     ws = context.getWorkspace(VLDT_GPU, wsMid > wsOut ? wsMid : wsOut);
     if (!ws) return fail(context.getLastError(), "workspace");
     ABI("bn3_fwd", mcn_bnorm_forward_fused(st, buffer("y"), buffer(m3), buffer("a3"), buffer("g3"), buffer("b3"),
@@ -209,7 +277,7 @@ ErrorCode Bottleneck::forward() {
   STEP("conv2_fwd", c2.forward(slot("a2"), 0, slot("r1"), 1, slot("f2"), none));
   STEP("bn2_fwd", bnForward("n2", m2, "a2", "g2", "b2"));
   ABI("relu2_fwd", mcn_relu_forward(st, buffer("r2"), buffer("n2"), nMidOut));
-  STEP("conv3_fwd", c1.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
+  STEP("conv3_fwd", c3.forward(slot("a3"), 0, slot("r2"), 1, slot("f3"), none));
   STEP("bn3_fwd", bnForward("n3", m3, "a3", "g3", "b3"));
   ABI("sum_fwd", mcn_add(st, buffer("s"), buffer("n3"), buffer(shortcut), nOut));
   ABI("relu3_fwd", mcn_relu_forward(st, buffer("y"), buffer("s"), nOut));
@@ -225,7 +293,8 @@ ErrorCode Bottleneck::backward() {
   void* st = context.getHipHelper().getStream();
   Tensor none;
   nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),
-      cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
+      c3(context, 1, 1, 0, 0, 0, 0, 1, 1), cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
+  attachPacked(c1, c2, c3, cs);
   nn::BatchNorm bn(context, epsilon);
   const std::size_t nMid = slot("a1").getNumElements(), nMidOut = slot("a2").getNumElements(),
                     nIn = slot("x").getNumElements(), nOut = slot("a3").getNumElements();
@@ -278,7 +347,7 @@ ErrorCode Bottleneck::backward() {
     ABI("relu3_bwd", mcn_relu_backward(st, buffer(dsName), buffer(mask3), buffer("dzdy"), nOut));
     STEP("bn3_bwd", bn.backwardWithMoment(slot("da3"), slot("dg3"), slot("db3"), slot("m3"), slot("a3"), slot("g3"), slot("b3"), slot(dsName)));
   }
-  STEP("conv3_bwd", convBackward(c1, c1s, 0, slot("dr2"), 0, slot("df3"), slot("r2"), slot("f3"), slot("da3")));
+  STEP("conv3_bwd", convBackward(c3, c1s, 0, slot("dr2"), 0, slot("df3"), slot("r2"), slot("f3"), slot("da3")));
   if (fused) {
     // ReLU's derivative folded into the batch-norm derivative that follows it: the mask is recomputed from the
     // layer's input and stored moments, the masked derivative is never written out

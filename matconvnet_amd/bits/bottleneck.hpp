@@ -13,7 +13,9 @@
 #include <string>
 #include <vector>
 
+#include "../../include/mcn_hip.h"
 #include "data.hpp"
+#include "nnconv.hpp"
 
 namespace vl { namespace harness {
 
@@ -52,6 +54,13 @@ class Bottleneck {
   // test mode: batch normalisation uses the stored moments "rm1", "rm2", "rm3" ("rms") instead of the batch's
   // (matlab/+dagnn/BatchNorm.m:12-17); forward only
   void setTestMode(bool on) { testMode = on; }
+  // packed = true: the convolutions read filter banks packed ahead (mcn_conv_pack_* of the C ABI) instead of
+  // packing them on every call; pack() refreshes all of the unit's banks in one launch and must be called after
+  // every change of the filters (setPacked does not pack).  packJobs(): the unit's jobs, for a caller that packs
+  // several units in one launch of its own.  Same bits either way.
+  ErrorCode setPacked(bool on);
+  ErrorCode pack();
+  std::vector<mcn_conv_pack_job> const& packJobs() const { return jobs; }
   ErrorCode forward();
   ErrorCode backward();
 
@@ -79,6 +88,14 @@ class Bottleneck {
   bool fused;
   bool overlap;
   bool testMode;
+  void attachPacked(nn::Convolution& c1, nn::Convolution& c2, nn::Convolution& c3, nn::Convolution& cs);
+  struct Bank { std::size_t offset, bytes; };
+  bool packed;
+  Bank banks[4][2];              // [convolution][forward, backward-data]
+  void* packedArena;
+  void* packedJobs;              // device copy of `jobs`, numbered for the unit's own launch
+  unsigned packedBlocks;
+  std::vector<mcn_conv_pack_job> jobs;
   Context sideContext;
   void* sideStream;     // hipStream_t
   void* events[5];      // hipEvent_t: "derivative ready" for the convolutions, "second stream done"

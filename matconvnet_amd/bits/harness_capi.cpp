@@ -184,6 +184,8 @@ void vlh_bottleneck_set_fused(void* block, int fused) { ((BlockHandle*)block)->b
 
 int vlh_bottleneck_set_overlap(void* block, int overlap) { return (int)((BlockHandle*)block)->block->setOverlap(overlap != 0); }
 
+int vlh_bottleneck_set_packed(void* block, int packed) { return (int)((BlockHandle*)block)->block->setPacked(packed != 0); }
+int vlh_bottleneck_pack(void* block) { return (int)((BlockHandle*)block)->block->pack(); }
 int vlh_bottleneck_forward(void* block) { return (int)((BlockHandle*)block)->block->forward(); }
 int vlh_bottleneck_backward(void* block) { return (int)((BlockHandle*)block)->block->backward(); }
 const char* vlh_bottleneck_message(void* block) { return ((BlockHandle*)block)->block->lastMessage().c_str(); }
@@ -199,7 +201,8 @@ int vlh_bottleneck_run(void* block, int steps, const char* stage, float* stage_m
   }
   int rc = 0;
   for (int i = 0; i < steps && rc == 0; ++i) {
-    rc = (int)h->block->forward();
+    rc = (int)h->block->pack();  // (packed mode: the filters may have changed since the last step; else nothing)
+    if (rc == 0) rc = (int)h->block->forward();
     if (rc == 0) rc = (int)h->block->backward();
   }
   h->block->setStageHook(NULL, NULL);
@@ -234,6 +237,8 @@ float* vlh_resnet50_buffer(void* net, const char* name, size_t* count) {
 int vlh_resnet50_set_stream(void* net, void* stream) { return (int)((harness::ResNet50*)net)->setStream(stream); }
 void vlh_resnet50_set_fused(void* net, int fused) { ((harness::ResNet50*)net)->setFused(fused != 0); }
 void vlh_resnet50_set_test_mode(void* net, int test) { ((harness::ResNet50*)net)->setTestMode(test != 0); }
+int vlh_resnet50_set_packed(void* net, int packed) { return (int)((harness::ResNet50*)net)->setPacked(packed != 0); }
+int vlh_resnet50_pack(void* net) { return (int)((harness::ResNet50*)net)->pack(); }
 int vlh_resnet50_init(void* net, unsigned long long seed) { return (int)((harness::ResNet50*)net)->initParameters(seed); }
 int vlh_resnet50_forward(void* net) { return (int)((harness::ResNet50*)net)->forward(); }
 int vlh_resnet50_backward(void* net) { return (int)((harness::ResNet50*)net)->backward(); }

@@ -50,6 +50,10 @@ VLH_API void vlh_bottleneck_set_fused(void* block, int fused);
 /* overlap != 0: backward runs each convolution's filter gradient on a second stream beside its input gradient
    (same bits; the second stream is joined before vlh_bottleneck_backward's work is complete on the block's stream) */
 VLH_API int vlh_bottleneck_set_overlap(void* block, int overlap);
+/* packed != 0: the convolutions read filter banks packed ahead; vlh_bottleneck_pack refreshes them (one launch) and
+   must follow every change of the filters */
+VLH_API int vlh_bottleneck_set_packed(void* block, int packed);
+VLH_API int vlh_bottleneck_pack(void* block);
 VLH_API int vlh_bottleneck_forward(void* block);
 VLH_API int vlh_bottleneck_backward(void* block);
 /* runs `steps` forward+backward passes; if stage != NULL the launches of that stage are bracketed by HIP
@@ -69,6 +73,11 @@ VLH_API void vlh_resnet50_set_fused(void* net, int fused);
 /* test != 0: batch normalisation uses the moving averages "running.*" (evaluation of a trained network); forward only */
 VLH_API void vlh_resnet50_set_test_mode(void* net, int test);
 /* He-normal filters, gains 1, biases 0 from a seeded host generator */
+/* packed != 0: all convolutions read filter banks packed ahead, refreshed by ONE launch: by vlh_resnet50_pack, and at the
+   end of vlh_resnet50_sgd_step and vlh_resnet50_init.  Call vlh_resnet50_pack after writing filters through
+   vlh_resnet50_buffer.  Same bits as packing on every call (the default). */
+VLH_API int vlh_resnet50_set_packed(void* net, int packed);
+VLH_API int vlh_resnet50_pack(void* net);
 VLH_API int vlh_resnet50_init(void* net, unsigned long long seed);
 VLH_API int vlh_resnet50_forward(void* net);
 VLH_API int vlh_resnet50_backward(void* net);

@@ -188,7 +188,7 @@ static void benchCopy(int warmup, int iters) {
               "copy 256 MiB", t * 1e3, 2.0 * n * 4 / t / 1e6, 100 * 2.0 * n * 4 / (t * 1e-3) / kPeakHbm, n * 4, n * 4, gRotate);
 }
 
-static void benchBlock(int warmup, int iters, bool fused, bool overlap = false) {
+static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, bool packed = false) {
   const int H = 56, W = 56, C = 256, M = 64, N = 32;
   harness::Bottleneck block(H, W, C, M, N, 1e-5);
   block.setFused(fused);
@@ -213,14 +213,20 @@ static void benchBlock(int warmup, int iters, bool fused, bool overlap = false) 
   upload("f3", std::sqrt(2.f / M), 0, true);
   for (char const* g : {"g1", "g2", "g3"}) upload(g, 0, 1.f, false);
   for (char const* b : {"b1", "b2", "b3"}) upload(b, 0, 0.f, false);
+  if (packed && block.setPacked(true) != VLE_Success) {
+    std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
+    std::exit(3);
+  }
   double t = medianMs([&] {
-    if (block.forward() != VLE_Success || block.backward() != VLE_Success) {
+    // (packed: the banks are re-packed every step, as they would be after an update of the filters: one launch)
+    if (block.pack() != VLE_Success || block.forward() != VLE_Success || block.backward() != VLE_Success) {
       std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
       std::exit(3);
     }
   }, warmup, iters);
   std::printf("%-28s %8.3f ms/step %9.0f images/s (fwd+bwd, N = %d, 41.93 GFLOP of convolution per step; %s)\n",
-              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, overlap ? "folded, filter gradients on a second stream" : (fused ? "relu/sum folded into bnorm" : "layer by layer"));
+              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, packed ? "folded, filter banks packed by one launch per step"
+                     : (overlap ? "folded, filter gradients on a second stream" : (fused ? "relu/sum folded into bnorm" : "layer by layer")));
 }
 
 // Whole ResNet-50 (224 x 224 images, 1000 classes): forward alone (training-mode batch normalisation: moments are
@@ -232,6 +238,10 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
     std::exit(3);
   }
   net.setFused(fused);
+  if (fused && net.setPacked(true) != VLE_Success) {  // (the folded run also packs the filter banks ahead, once per update)
+    std::fprintf(stderr, "resnet-50: %s\n", net.lastMessage().c_str());
+    std::exit(3);
+  }
   {
     std::mt19937_64 gen(12);
     std::normal_distribution<float> dist(0.f, 1.f);
@@ -277,7 +287,7 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
               "%8.2f ms training step (with the SGD update of %.1f M parameters) %8.0f images/s "
               "(N = %d, %.2f GFLOP of convolution per image forward; %s)\n",
               "resnet-50 224x224", tf, N / (tf * 1e-3), gf * N / tf, t, N / (t * 1e-3), 3 * gf * N / t, ts,
-              net.numParameters() * 1e-6, N / (ts * 1e-3), N, gf, fused ? "relu/sum folded into bnorm" : "layer by layer");
+              net.numParameters() * 1e-6, N / (ts * 1e-3), N, gf, fused ? "relu/sum folded into bnorm, filter banks packed once per update" : "layer by layer");
 }
 
 int main(int argc, char** argv) {
@@ -311,6 +321,7 @@ int main(int argc, char** argv) {
     benchBlock(warmup, iters, false);
     benchBlock(warmup, iters, true);
     benchBlock(warmup, iters, true, true);
+    benchBlock(warmup, iters, true, false, true);
   }
   if (want("conv5")) benchConv("conv 3x3x256x256 56x56 N=64", 56, 56, 256, 64, 3, 256, 1, warmup, iters);
   return 0;

@@ -12,7 +12,8 @@ using namespace vl::impl;
 Convolution::Convolution(Context& context, int strideY, int strideX, int padTop, int padBottom, int padLeft,
                          int padRight, int dilateY, int dilateX)
     : context(context), strideY(strideY), strideX(strideX), padTop(padTop), padBottom(padBottom), padLeft(padLeft),
-      padRight(padRight), dilateY(dilateY), dilateX(dilateX) {}
+      padRight(padRight), dilateY(dilateY), dilateX(dilateX), packedForward(NULL), packedForwardBytes(0),
+      packedBackward(NULL), packedBackwardBytes(0) {}
 
 namespace {
 
@@ -56,10 +57,26 @@ ErrorCode Convolution::forward(Tensor& output, double outputMult, Tensor const& 
   void* ws;
   size_t bytes;
   if (!scratch(context, g, MCN_CONV_FORWARD, &ws, &bytes)) return context.getLastError();
-  rc = mcn_conv_forward(context.getHipHelper().getStream(), &g, (float*)output.getMemory(), (float)outputMult,
-                        (float const*)input.getMemory(), (float)inputMult, (float const*)filter.getMemory(),
-                        (float const*)bias.getMemory(), ws, bytes);
+  rc = mcn_conv_forward_packed(context.getHipHelper().getStream(), &g, (float*)output.getMemory(), (float)outputMult,
+                               (float const*)input.getMemory(), (float)inputMult, (float const*)filter.getMemory(),
+                               packedForward, packedForwardBytes, (float const*)bias.getMemory(), ws, bytes);
   return fromAbi(context, rc, "Convolution::forward");
+}
+
+std::size_t Convolution::packedBytes(int product, TensorShape const& data, TensorShape const& filter) const {
+  mcn_conv_geom g = geometry(*this, data, filter);
+  return mcn_conv_packed_bytes(&g, product);
+}
+
+ErrorCode Convolution::planPack(int product, TensorShape const& data, Tensor const& filter, void* packed, std::size_t bytes,
+                                std::vector<mcn_conv_pack_job>& jobs) {
+  mcn_conv_geom g = geometry(*this, data, filter);
+  mcn_conv_pack_job found[64];
+  int n = 0;
+  int rc = mcn_conv_pack_plan(&g, product, (float const*)filter.getMemory(), packed, bytes, found, 64, &n);
+  if (rc) return fromAbi(context, rc, "Convolution::planPack");
+  jobs.insert(jobs.end(), found, found + n);
+  return VLE_Success;
 }
 
 ErrorCode Convolution::backward(Tensor& derInput, Tensor& derFilter, Tensor& derBias, Tensor const& input,
@@ -100,8 +117,9 @@ ErrorCode Convolution::backwardAccumulate(Tensor& derInput, double derInputMult,
         derOutput.getSize() != derInput.getSize())
       return context.setError(VLE_IllegalArgument, "Convolution::backward: DEROUTPUT dimensions are incompatible with X and FILTERS");
     if (!scratch(context, g, MCN_CONV_BACKWARD_DATA, &ws, &bytes)) return context.getLastError();
-    rc = mcn_conv_backward_data_acc(stream, &g, (float*)derInput.getMemory(), (float)derInputMult,
-                                    (float const*)filter.getMemory(), (float const*)derOutput.getMemory(), ws, bytes);
+    rc = mcn_conv_backward_data_packed(stream, &g, (float*)derInput.getMemory(), (float)derInputMult,
+                                       (float const*)filter.getMemory(), packedBackward, packedBackwardBytes,
+                                       (float const*)derOutput.getMemory(), ws, bytes);
     if (rc) return fromAbi(context, rc, "Convolution::backward");
   }
 

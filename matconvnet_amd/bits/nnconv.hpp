@@ -2,6 +2,9 @@
 #ifndef MCN_AMD_BITS_NNCONV_HPP
 #define MCN_AMD_BITS_NNCONV_HPP
 
+#include <vector>
+
+#include "../../include/mcn_hip.h"
 #include "data.hpp"
 
 namespace vl { namespace nn {
@@ -26,6 +29,20 @@ class Convolution {
   vl::ErrorCode backwardAccumulate(vl::Tensor& derInput, double derInputMult, vl::Tensor& derFilter, vl::Tensor& derBias,
                                    vl::Tensor const& input, vl::Tensor const& filter, vl::Tensor const& derOutput);
 
+  // Filter banks packed ahead (mcn_conv_pack_filters and friends, include/mcn_hip.h), for callers whose filters stay
+  // put between calls.  Not part of the reference's class.
+  //   packedBytes   size of the packed bank of a product (MCN_CONV_FORWARD / MCN_CONV_BACKWARD_DATA) for data of
+  //                 this shape (the layer's input) and this filter bank; 0: the product reads none
+  //   planPack      appends the product's packing jobs (filter bank -> `packed`) to `jobs`, for one batched launch
+  //   usePacked     the banks forward / backward[Accumulate] read from now on (null: pack on the fly, the default)
+  std::size_t packedBytes(int product, vl::TensorShape const& data, vl::TensorShape const& filter) const;
+  vl::ErrorCode planPack(int product, vl::TensorShape const& data, vl::Tensor const& filter, void* packed, std::size_t bytes,
+                         std::vector<mcn_conv_pack_job>& jobs);
+  void usePacked(void const* forwardBank, std::size_t forwardBytes, void const* backwardBank, std::size_t backwardBytes) {
+    packedForward = forwardBank; packedForwardBytes = forwardBytes;
+    packedBackward = backwardBank; packedBackwardBytes = backwardBytes;
+  }
+
   Context& context;
   int strideY;
   int strideX;
@@ -35,6 +52,10 @@ class Convolution {
   int padRight;
   int dilateY;
   int dilateX;
+  void const* packedForward;
+  std::size_t packedForwardBytes;
+  void const* packedBackward;
+  std::size_t packedBackwardBytes;
 };
 
 // Same class interface as matlab/src/bits/nnconv.hpp:54-81.  FILTER is FH x FW x (output depth / groups) x (input

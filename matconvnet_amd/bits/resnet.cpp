@@ -38,7 +38,9 @@ double conv_flops(int outH, int outW, int fh, int fw, int cin, int cout) {
 ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
     : N(N), S(imageSize), classes(classes), epsilon(epsilon), fused(true), testMode(false), error(VLE_Success), flops(0), values(NULL),
       ders(NULL), state(NULL), batchMoments(NULL), runningMoments(NULL), chunkParam(NULL), rates(NULL), chunks(0),
-      momentsCount(0), parameterCount(0), graph(NULL), graphExec(NULL) {
+      momentsCount(0), parameterCount(0), packed(false), packedArena(NULL), packedJobs(NULL), stemBytes(0),
+      fcForwardBytes(0), fcBackwardBytes(0), fcBackwardOffset(0), packedJobCount(0), packedBlocks(0), graph(NULL),
+      graphExec(NULL) {
   if (S < 32 || S % 32 != 0) {
     error = VLE_IllegalArgument;
     message = "the image size must be a multiple of 32";
@@ -208,13 +210,67 @@ ErrorCode ResNet50::sgdStep(double learningRate, double momentum, double weightD
   // moments: trainMethod 'average' (:331-335) with the rate cnn_imagenet_init_resnet.m:190-195 sets, fan-out 1
   const double rate = 0.3;
   ABI("moments", mcn_taccum(st, runningMoments, (float)(1.0 - rate), runningMoments, (float)rate, batchMoments, momentsCount));
-  return VLE_Success;
+  return pack();  // (the filters have changed)
 }
 
 void ResNet50::dropGraph() {
   if (graphExec) (void)hipGraphExecDestroy((hipGraphExec_t)graphExec);
   if (graph) (void)hipGraphDestroy((hipGraph_t)graph);
   graph = graphExec = NULL;
+}
+
+ErrorCode ResNet50::setPacked(bool on) {
+  if (error != VLE_Success) return error;
+  dropGraph();
+  if (packedArena) (void)hipFree(packedArena);
+  if (packedJobs) (void)hipFree(packedJobs);
+  packedArena = packedJobs = NULL;
+  packed = false;
+  for (std::size_t i = 0; i < units.size(); ++i)
+    if (units[i]->setPacked(on) != VLE_Success) {
+      message = units[i]->lastMessage();
+      return VLE_OutOfGPUMemeory;
+    }
+  if (!on) return VLE_Success;
+  nn::Convolution stem(context, 2, 2, 3, 3, 3, 3, 1, 1), fc(context, 1, 1, 0, 0, 0, 0, 1, 1);
+  const TensorShape inputShape = slot("input").getShape(), avgShape = slot("avg").getShape();
+  stemBytes = stem.packedBytes(MCN_CONV_FORWARD, inputShape, slot("stem.f").getShape());
+  fcForwardBytes = fc.packedBytes(MCN_CONV_FORWARD, avgShape, slot("fc.f").getShape());
+  fcBackwardBytes = fc.packedBytes(MCN_CONV_BACKWARD_DATA, avgShape, slot("fc.f").getShape());
+  fcBackwardOffset = stemBytes + fcForwardBytes;
+  const std::size_t total = stemBytes + fcForwardBytes + fcBackwardBytes;
+  if (hipMalloc(&packedArena, total ? total : 16) != hipSuccess) {
+    (void)hipGetLastError();
+    packedArena = NULL;
+    message = "cannot allocate the packed filter banks";
+    return VLE_OutOfGPUMemeory;
+  }
+  std::vector<mcn_conv_pack_job> jobs;
+  char* arena = (char*)packedArena;
+  if ((stemBytes && stem.planPack(MCN_CONV_FORWARD, inputShape, slot("stem.f"), arena, stemBytes, jobs) != VLE_Success) ||
+      (fcForwardBytes && fc.planPack(MCN_CONV_FORWARD, avgShape, slot("fc.f"), arena + stemBytes, fcForwardBytes, jobs) != VLE_Success) ||
+      (fcBackwardBytes && fc.planPack(MCN_CONV_BACKWARD_DATA, avgShape, slot("fc.f"), arena + fcBackwardOffset, fcBackwardBytes, jobs) != VLE_Success))
+    return fail(context.getLastError(), "planPack");
+  for (std::size_t i = 0; i < units.size(); ++i) jobs.insert(jobs.end(), units[i]->packJobs().begin(), units[i]->packJobs().end());
+  packedJobCount = (int)jobs.size();
+  packedBlocks = mcn_conv_pack_layout(jobs.data(), packedJobCount);
+  const std::size_t bytes = jobs.size() * sizeof(mcn_conv_pack_job);
+  if (hipMalloc(&packedJobs, bytes ? bytes : 16) != hipSuccess ||
+      hipMemcpy(packedJobs, jobs.data(), bytes, hipMemcpyHostToDevice) != hipSuccess) {
+    (void)hipGetLastError();
+    message = "cannot upload the packing jobs";
+    return VLE_Cuda;
+  }
+  packed = true;
+  return pack();
+}
+
+ErrorCode ResNet50::pack() {
+  if (error != VLE_Success) return error;
+  if (!packed) return VLE_Success;
+  ABI("pack", mcn_conv_pack_batch(context.getHipHelper().getStream(), (mcn_conv_pack_job const*)packedJobs, packedJobCount,
+                                  packedBlocks));
+  return VLE_Success;
 }
 
 ErrorCode ResNet50::capture(bool training, double learningRate, double momentum, double weightDecay) {
@@ -277,7 +333,7 @@ ResNet50::~ResNet50() {
   for (std::size_t i = 0; i < units.size(); ++i) delete units[i];
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
-  void* arenas[] = {values, ders, state, batchMoments, runningMoments, chunkParam, rates};
+  void* arenas[] = {values, ders, state, batchMoments, runningMoments, chunkParam, rates, packedArena, packedJobs};
   for (void* a : arenas)
     if (a) (void)hipFree(a);
 }
@@ -404,7 +460,7 @@ ErrorCode ResNet50::initParameters(unsigned long long seed) {
     message = "cannot upload the parameters";
     return error = VLE_Cuda;
   }
-  return VLE_Success;
+  return pack();
 }
 
 ErrorCode ResNet50::forward() {
@@ -415,6 +471,10 @@ ErrorCode ResNet50::forward() {
   nn::Convolution stem(context, 2, 2, 3, 3, 3, 3, 1, 1), fc(context, 1, 1, 0, 0, 0, 0, 1, 1);
   nn::BatchNorm bn(context, epsilon);
   nn::Pooling maxPool(context, 3, 3, 2, 2, 1, 1, 1, 1, nn::Pooling::Max);
+  if (packed) {
+    stem.usePacked(stemBytes ? packedArena : NULL, stemBytes, NULL, 0);
+    fc.usePacked(fcForwardBytes ? (char*)packedArena + stemBytes : NULL, fcForwardBytes, NULL, 0);
+  }
   STEP("stem conv", stem.forward(slot("stem.a"), 0, slot("input"), 1, slot("stem.f"), none));
   if (fused) {
     const size_t wsBytes = mcn_bnorm_workspace_bytes(S2, S2, 64, N);
@@ -468,6 +528,7 @@ ErrorCode ResNet50::backward() {
   Tensor features(TensorShape(Hf, Hf, Cf, N), VLDT_Float, VLDT_GPU, last->buffer("y"), sizeof(float) * nFeatures);
   Tensor derFeatures(TensorShape(Hf, Hf, Cf, N), VLDT_Float, VLDT_GPU, last->buffer("dzdy"), sizeof(float) * nFeatures);
   nn::Pooling avgPool(context, Hf, Hf, 1, 1, 0, 0, 0, 0, nn::Pooling::Average);
+  if (packed) fc.usePacked(NULL, 0, fcBackwardBytes ? (char*)packedArena + fcBackwardOffset : NULL, fcBackwardBytes);
   STEP("classifier", fc.backward(slot("davg"), slot("fc.df"), slot("fc.db"), slot("avg"), slot("fc.f"), slot("dprediction")));
   STEP("average pool", avgPool.backwardOverwrite(derFeatures, features, slot("davg")));
   for (std::size_t i = units.size(); i-- > 0;)

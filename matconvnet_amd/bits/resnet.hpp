@@ -43,6 +43,10 @@ class ResNet50 {
   void setTestMode(bool on);
   // He-normal filters (matlab/+dagnn/Conv.m:40 style), gains 1, biases 0, from a seeded generator on the host
   ErrorCode initParameters(unsigned long long seed);
+  // packed = true: every convolution reads filter banks packed ahead; pack() refreshes them all in ONE launch.
+  // sgdStep() and initParameters() end with pack(); a caller that writes filters itself (through buffer()) calls it.
+  ErrorCode setPacked(bool on);
+  ErrorCode pack();
   ErrorCode forward();
   ErrorCode backward();
   // one update of all parameters from the derivatives backward() left (numWorkers = 1), and of the moving averages of
@@ -84,6 +88,11 @@ class ResNet50 {
   unsigned short* chunkParam;   // device
   double* rates;                // device
   std::size_t chunks, momentsCount, parameterCount;
+  bool packed;
+  void *packedArena, *packedJobs;   // banks of the stem and the classifier; device table of all the network's jobs
+  std::size_t stemBytes, fcForwardBytes, fcBackwardBytes, fcBackwardOffset;
+  int packedJobCount;
+  unsigned packedBlocks;
   void *graph, *graphExec;      // hipGraph_t, hipGraphExec_t
   void dropGraph();
 };

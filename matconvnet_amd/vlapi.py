@@ -81,6 +81,10 @@ def lib():
         L.vlh_resnet50_set_fused.restype = None
         L.vlh_resnet50_set_test_mode.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_test_mode.restype = None
+        L.vlh_resnet50_set_packed.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_resnet50_pack.argtypes = [C.c_void_p]
+        L.vlh_bottleneck_set_packed.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_bottleneck_pack.argtypes = [C.c_void_p]
         L.vlh_resnet50_init.argtypes = [C.c_void_p, C.c_ulonglong]
         L.vlh_resnet50_forward.argtypes = [C.c_void_p]
         L.vlh_resnet50_backward.argtypes = [C.c_void_p]
@@ -240,8 +244,11 @@ class ResNet50(_NamedBuffers):
     the loss layers); buffers are owned by the C++ side and named "input", "prediction", "dprediction",
     "stem.f", "fc.f", "unit<i>.<name>", ..."""
 
-    def __init__(self, N=32, eps=1e-5, image_size=224, classes=1000, fused=True, seed=None):
+    def __init__(self, N=32, eps=1e-5, image_size=224, classes=1000, fused=True, seed=None, packed=True):
+        """packed: the convolutions read filter banks packed ahead, refreshed in one launch after every update (and by
+        `set` of a parameter here); False: every call packs its own, as the plain operator calls do."""
         self.L = lib()
+        self.packed = False
         self.N, self.image_size, self.classes = N, image_size, classes
         self.h = self.L.vlh_resnet50_create(N, eps, image_size, classes)
         msg = self.L.vlh_resnet50_message(self.h).decode()
@@ -251,8 +258,20 @@ class ResNet50(_NamedBuffers):
         torch = _torch()
         self._check(self.L.vlh_resnet50_set_stream(self.h, C.c_void_p(torch.cuda.current_stream().cuda_stream)))
         self.L.vlh_resnet50_set_fused(self.h, int(fused))
+        if packed:
+            self._check(self.L.vlh_resnet50_set_packed(self.h, 1))
+            self.packed = True
         if seed is not None:
             self._check(self.L.vlh_resnet50_init(self.h, seed))
+
+    def set(self, name, array):
+        super().set(name, array)
+        if self.packed and name.rsplit(".", 1)[-1] in ("f", "f1", "f2", "f3", "fs"):
+            self.pack()
+
+    def pack(self):
+        """Refresh the packed filter banks (one launch); needed after writing filters by other means than `set`."""
+        self._check(self.L.vlh_resnet50_pack(self.h))
 
     def close(self):
         if self.h:
@@ -314,8 +333,11 @@ class Bottleneck(_NamedBuffers):
     """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
 
     def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False, overlap=False, Cout=0, stride=1,
-                 adapter=False):
+                 adapter=False, packed=False):
+        """packed: the convolutions read filter banks packed ahead; `set` of a filter and every step of `run` refresh
+        them with one launch (`pack`)."""
         self.L = lib()
+        self.packed = False
         self.shape = (H, W, Cc, M, N)
         self.h = self.L.vlh_unit_create(H, W, Cc, M, N, eps, Cout, stride, int(adapter))
         torch = _torch()
@@ -323,6 +345,17 @@ class Bottleneck(_NamedBuffers):
         self.L.vlh_bottleneck_set_fused(self.h, int(fused))
         if overlap and self.L.vlh_bottleneck_set_overlap(self.h, 1) != 0:
             raise VlError(2, self.L.vlh_bottleneck_message(self.h).decode())
+        if packed:
+            self._check(self.L.vlh_bottleneck_set_packed(self.h, 1))
+            self.packed = True
+
+    def set(self, name, array):
+        super().set(name, array)
+        if self.packed and name in ("f1", "f2", "f3", "fs"):
+            self.pack()
+
+    def pack(self):
+        self._check(self.L.vlh_bottleneck_pack(self.h))
 
     def close(self):
         if self.h:

@@ -253,6 +253,30 @@ def test_test_mode_uses_the_stored_moments(vl, case):
     assert bits_equal(outs[False], outs[True])
 
 
+def test_filters_packed_ahead_change_no_bit(vl, case):
+    """All convolutions reading banks packed ahead by one launch (after uploads, and after every update) against every
+    call packing its own: predictions, gradients, and the parameters after two training steps."""
+    lr, mom, wd = 0.05, 0.9, 1e-4
+    watch = _gradient_names(case) + ["stem.f", "unit0.f1", "unit3.f2", "unit3.fs", "unit15.f3", "fc.f", "momentum.unit7.f2"]
+    seen = {}
+    for packed in (False, True):
+        net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=True, packed=packed)
+        try:
+            _load(net, case)
+            for _ in range(2):
+                net.forward()
+                net.backward()
+                net.sgd_step(lr, mom, wd)
+            net.forward()
+            net.backward()
+            seen[packed] = {k: net.get(k) for k in watch}
+        finally:
+            net.close()
+    for k in watch:
+        assert bits_equal(seen[False][k], seen[True][k]), k
+    assert not bits_equal(seen[True]["unit3.f2"], np.asfortranarray(case["units"][3]["f2"]).ravel(order="F"))
+
+
 def test_graph_replays_match_eager_steps(vl, case):
     """A training step and an evaluation pass recorded into HIP graphs: every replay -- with uploads, downloads and
     device synchronisations of the program between them, and the input changed from one to the next -- leaves the same
