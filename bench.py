@@ -13,7 +13,7 @@ region.  `value` is images/s over exactly K steps.  The same line carries
                 256 MB memory-side cache because the previous launch left them there (`achieved`); the figure a
                 loop over one set of buffers shows is reported beside it as `achieved_warm`,
   resnet50      the whole ResNet-50 (224 x 224) through the same operator classes: forward and whole training steps
-                (forward, backward, SGD update) at 32 and 128 images,
+                (forward, backward, SGD update) at 32, 64 and 128 images,
   cpu_baseline  the CPU restatement of the reference path (oracle/) timed on this machine's host cores.
 One GPU only: nothing here shards.
 """
@@ -357,7 +357,9 @@ def main():
         "hbm_timing": "cold: %d tensor sets in rotation; *_warm: one set reused" % COLD_SETS,
         "rooflines": conv_rows + bn_rows + pool_rows,
         # beyond the headline block: the whole network the block comes from, per-image rates of whole training steps
-        "resnet50": [bench_resnet50(vlapi, b, max(3, args.steps // 10), 2) for b in (32, 128)],
+        # (64 is the reference's own sub-batch for this network: batchSize 256 in 4 sub-batches,
+        # examples/imagenet/cnn_imagenet_init_resnet.m:170-171)
+        "resnet50": [bench_resnet50(vlapi, b, max(3, args.steps // 10), 2) for b in (32, 64, 128)],
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(workloads)
