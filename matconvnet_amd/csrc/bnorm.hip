@@ -29,6 +29,7 @@ struct BnormP {
   int reverse;       // apply pass walks logical ids backwards
   int teamShift[2];  // log2 of the threads that share one plane, for scalar [0] and 16-byte [1] accesses: planes
                      // smaller than a workgroup's 256 accesses are walked several at a time, one per team
+  int oneLaunch;     // groups == 1 and the apply kernels compute the sums themselves (small channels): no sums launch
   double mass;       // WH * N
   double epsilon;
 };
@@ -72,27 +73,12 @@ __device__ __forceinline__ void block_sum(double (&v)[NV], double* lds /* [4][NV
 // YMASK (MODE 1 only): dy first passes the derivative of a ReLU whose *output* is ymask (dy counts where
 // ymask > 0, else dy*0 like mcn_relu_backward), and the masked derivative is also written to `masked` for the
 // passes that follow (this layer's apply pass, and whoever else consumes it).
-template <int MODE, bool VEC4, bool RELU = false, bool YMASK = false>
-__global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
-                                                  const float* __restrict__ dy,
-                                                  double* __restrict__ partials, BnormP p,
-                                                  const float* __restrict__ moments = nullptr,
-                                                  const float* __restrict__ mult = nullptr,
-                                                  const float* __restrict__ bias = nullptr,
-                                                  const float* __restrict__ ymask = nullptr,
-                                                  float* __restrict__ masked = nullptr) {
-  static_assert(!RELU || MODE == 1, "the ReLU mask needs the moments of the forward pass");
-  static_assert(!YMASK || (MODE == 1 && !RELU), "one kind of mask at a time, with given moments");
-  __shared__ double lds[16];
-  const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int c = logical / p.groups;
-  const int grp = logical - c * p.groups;
-  int n0, n1;
-  image_range(p, grp, &n0, &n1);
-  float ra = 0.f, rk = 0.f;
-  if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &ra, &rk);
+template <int MODE, bool VEC4, bool RELU, bool YMASK>
+__device__ __forceinline__ void sums_of_planes(double (&acc)[4], const float* __restrict__ x, const float* __restrict__ dy,
+                                               const BnormP& p, int c, int n0, int n1, float ra, float rk,
+                                               const float* __restrict__ ymask, float* __restrict__ masked, double* lds) {
   auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv, rk) > 0.f ? dv : 0.f) : dv; };
-  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  acc[0] = acc[1] = acc[2] = acc[3] = 0.0;
   const int shift = p.teamShift[VEC4 ? 1 : 0], TS = 1 << shift, teams = 256 >> shift;
   const int team = threadIdx.x >> shift, j0 = threadIdx.x & (TS - 1);
   for (int n = n0 + team; n < n1; n += teams) {
@@ -144,6 +130,29 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
     acc[3] += (double)sd;
   }
   block_sum<4>(acc, lds);
+}
+
+template <int MODE, bool VEC4, bool RELU = false, bool YMASK = false>
+__global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
+                                                  const float* __restrict__ dy,
+                                                  double* __restrict__ partials, BnormP p,
+                                                  const float* __restrict__ moments = nullptr,
+                                                  const float* __restrict__ mult = nullptr,
+                                                  const float* __restrict__ bias = nullptr,
+                                                  const float* __restrict__ ymask = nullptr,
+                                                  float* __restrict__ masked = nullptr) {
+  static_assert(!RELU || MODE == 1, "the ReLU mask needs the moments of the forward pass");
+  static_assert(!YMASK || (MODE == 1 && !RELU), "one kind of mask at a time, with given moments");
+  __shared__ double lds[16];
+  const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int c = logical / p.groups;
+  const int grp = logical - c * p.groups;
+  int n0, n1;
+  image_range(p, grp, &n0, &n1);
+  float ra = 0.f, rk = 0.f;
+  if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &ra, &rk);
+  double acc[4];
+  sums_of_planes<MODE, VEC4, RELU, YMASK>(acc, x, dy, p, c, n0, n1, ra, rk, ymask, masked, lds);
   if (threadIdx.x == 0) {
     double* out = partials + ((size_t)c * p.groups + grp) * 4;
     out[0] = acc[0];
@@ -151,6 +160,23 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
     out[2] = acc[2];
     out[3] = acc[3];
   }
+}
+
+// The totals of channel c when its single workgroup computes them itself (oneLaunch): the sums over all its
+// planes, handed to every thread.  `lds`: 20 doubles.
+template <int MODE, bool VEC4, bool RELU, bool YMASK>
+__device__ __forceinline__ void own_totals(double (&tot)[4], const float* __restrict__ x, const float* __restrict__ dy,
+                                           const BnormP& p, int c, float ra, float rk, const float* __restrict__ ymask,
+                                           float* __restrict__ masked, double* lds) {
+  double acc[4];
+  sums_of_planes<MODE, VEC4, RELU, YMASK>(acc, x, dy, p, c, 0, p.N, ra, rk, ymask, masked, lds);
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds[16 + i] = acc[i];
+  }
+  __syncthreads();  // (also orders the masked derivative written above before the apply pass reads it)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) tot[i] = lds[16 + i];
 }
 
 // Sum of a channel's partials in a fixed order: lane i owns groups i, i+64, ...; then a wave tree.
@@ -223,7 +249,10 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
 
 // Backward apply.  GIVEN: mean/sigma come from `moments` (input); otherwise from the partial sums and
 // `moments` (if non-null) is written.
-template <bool GIVEN, bool VEC4, bool RELU = false>
+// ONE: 0 = totals from the partials of a sums launch; 1 = this workgroup sums its channel itself first (oneLaunch);
+// 2 = the same with the mask of a later ReLU (dy = the raw derivative, ymask that ReLU's output, masked = where the
+// masked derivative goes: the apply pass then reads it back).
+template <bool GIVEN, bool VEC4, bool RELU = false, int ONE = 0>
 __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ dx,
                                                             float* __restrict__ dmult,
                                                             float* __restrict__ dbias,
@@ -232,15 +261,25 @@ __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ 
                                                             const float* __restrict__ mult,
                                                             const float* __restrict__ dy,
                                                             const double* __restrict__ partials,
-                                                            BnormP p, const float* __restrict__ bias = nullptr) {
+                                                            BnormP p, const float* __restrict__ bias = nullptr,
+                                                            const float* __restrict__ ymask = nullptr,
+                                                            float* __restrict__ masked = nullptr) {
   static_assert(!RELU || GIVEN, "the ReLU mask needs the moments of the forward pass");
-  __shared__ double lds[4];
+  static_assert(ONE != 2 || (GIVEN && !RELU), "one kind of mask at a time, with given moments");
+  __shared__ double lds[20];
   int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   if (p.reverse) logical = (int)gridDim.x - 1 - logical;
   const int c = logical / p.groups;
   const int grp = logical - c * p.groups;
   double tot[4];
-  channel_totals(partials, p, c, lds, tot);
+  if (ONE) {
+    float sa = 0.f, sk = 0.f;
+    if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &sa, &sk);
+    own_totals<GIVEN ? 1 : 2, VEC4, RELU, ONE == 2>(tot, x, dy, p, c, sa, sk, ymask, masked, lds);
+    if (ONE == 2) dy = masked;
+  } else {
+    channel_totals(partials, p, c, lds, tot);
+  }
 
   double mean, sigma;
   if (GIVEN) {
@@ -308,7 +347,7 @@ __device__ __forceinline__ void stream_forward(float* __restrict__ out, const fl
 
 // Forward apply: y = (g/sigma)*(x - mean) + b  (bits/nnbnorm.cu:190-199), optionally followed by "+ residual"
 // (matlab/+dagnn/Sum.m) and ReLU (matlab/vl_nnrelu.m) in the same pass.
-template <bool GIVEN, bool VEC4, bool RES, bool RELU>
+template <bool GIVEN, bool VEC4, bool RES, bool RELU, bool ONE = false>
 __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y,
                                                            float* __restrict__ moments,
                                                            const float* __restrict__ x,
@@ -317,7 +356,7 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
                                                            const float* __restrict__ residual,
                                                            const double* __restrict__ partials,
                                                            BnormP p) {
-  __shared__ double lds[4];
+  __shared__ double lds[20];
   int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   if (p.reverse) logical = (int)gridDim.x - 1 - logical;
   const int c = logical / p.groups;
@@ -328,7 +367,8 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
     sigma = (double)moments[c + p.C];
   } else {
     double tot[4];
-    channel_totals(partials, p, c, lds, tot);
+    if (ONE) own_totals<0, VEC4, false, false>(tot, x, x, p, c, 0.f, 0.f, nullptr, nullptr, lds);
+    else channel_totals(partials, p, c, lds, tot);
     mean = tot[0] / p.mass;
     const double var = fmax(0.0, tot[1] / p.mass - mean * mean);
     sigma = sqrt(var + p.epsilon);
@@ -362,6 +402,13 @@ int setup(const char* who, int H, int W, int C, int N, double epsilon, BnormP* p
   p->C = C;
   p->N = N;
   p->groups = image_groups(p->WH, N);
+  // small channels (the 14x14 and 7x7 layers of a network at a few dozen images): one workgroup per channel sums
+  // and applies in the same launch; the second pass over the channel's few KB comes out of the caches
+  p->oneLaunch = 0;
+  if ((long long)p->WH * N <= tunable("bnorm_one_launch_elems", 8192) && C >= 128) {
+    p->groups = 1;
+    p->oneLaunch = 1;
+  }
   p->reverse = tunable("bnorm_reverse_apply", 1) ? 1 : 0;
   for (int v = 0; v < 2; ++v) {
     const int accesses = v ? p->WH / 4 : p->WH;  // per plane
@@ -400,7 +447,8 @@ int mcn_bnorm_forward_fused(mcn_stream_t stream, float* y, float* moments, const
   const bool vec = (p.WH % 4 == 0) && aligned16(y) && aligned16(x) && (!residual || aligned16(residual));
   const dim3 grid((unsigned)(C * p.groups)), block(256);
   double* partials = (double*)workspace;
-  if (!givenMoments) {
+  const bool one = p.oneLaunch && !givenMoments;
+  if (!givenMoments && !one) {
     if (!workspace || workspaceBytes < mcn_bnorm_workspace_bytes(H, W, C, N))
       return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward: workspace too small");
     {
@@ -413,9 +461,15 @@ int mcn_bnorm_forward_fused(mcn_stream_t stream, float* y, float* moments, const
     p.reverse = 0;
   }
   KernelTimer timer("bnorm_forward_apply", s);
-#define MCN_BN_FWD(GIVENF, VECF, RESF, RELUF)                                                                      \
-  hipLaunchKernelGGL((bnorm_forward_apply<GIVENF, VECF, RESF, RELUF>), grid, block, 0, s, y, moments, x, multipliers, \
-                     biases, residual, partials, p)
+#define MCN_BN_FWD(GIVENF, VECF, RESF, RELUF)                                                                          \
+  do {                                                                                                                  \
+    if (!GIVENF && one)                                                                                                 \
+      hipLaunchKernelGGL((bnorm_forward_apply<false, VECF, RESF, RELUF, true>), grid, block, 0, s, y, moments, x,       \
+                         multipliers, biases, residual, partials, p);                                                   \
+    else                                                                                                                \
+      hipLaunchKernelGGL((bnorm_forward_apply<GIVENF, VECF, RESF, RELUF>), grid, block, 0, s, y, moments, x, multipliers, \
+                         biases, residual, partials, p);                                                                \
+  } while (0)
 #define MCN_BN_FWD_EPI(GIVENF, VECF)                        \
   do {                                                      \
     if (residual && relu) MCN_BN_FWD(GIVENF, VECF, true, true);   \
@@ -464,6 +518,12 @@ int mcn_bnorm_backward_relu(mcn_stream_t stream, float* derInput, float* derMult
   const dim3 grid((unsigned)(C * p.groups)), block(256);
   double* partials = (double*)workspace;
   float* mom = const_cast<float*>(moments);  // (the kernels only write moments when they are not given)
+  if (p.oneLaunch) {
+    KernelTimer timer("bnorm_backward_apply", s);
+    if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true, true, 1>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, derOutput, partials, p, biases);
+    else hipLaunchKernelGGL((bnorm_backward_apply<true, false, true, 1>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, derOutput, partials, p, biases);
+    return check_launch("mcn_bnorm_backward_relu");
+  }
   {
     KernelTimer timer("bnorm_sums", s);
     if (vec) hipLaunchKernelGGL((bnorm_sums<1, true, true>), grid, block, 0, s, x, derOutput, partials, p, moments, multipliers, biases);
@@ -500,6 +560,12 @@ int mcn_bnorm_backward_masked(mcn_stream_t stream, float* derInput, float* derMu
   const dim3 grid((unsigned)(C * p.groups)), block(256);
   double* partials = (double*)workspace;
   float* mom = const_cast<float*>(moments);  // (the kernels only write moments when they are not given)
+  if (p.oneLaunch) {
+    KernelTimer timer("bnorm_backward_apply", s);
+    if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true, false, 2>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, derOutput, partials, p, nullptr, maskSource, maskedDerOutput);
+    else hipLaunchKernelGGL((bnorm_backward_apply<true, false, false, 2>), grid, block, 0, s, derInput, derMultipliers, derBiases, mom, x, multipliers, derOutput, partials, p, nullptr, maskSource, maskedDerOutput);
+    return check_launch("mcn_bnorm_backward_masked");
+  }
   {
     KernelTimer timer("bnorm_sums", s);
     if (vec) hipLaunchKernelGGL((bnorm_sums<1, true, false, true>), grid, block, 0, s, x, derOutput, partials, p, nullptr, nullptr, nullptr, maskSource, maskedDerOutput);
@@ -534,6 +600,17 @@ int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultiplie
   const bool vec = (p.WH % 4 == 0) && aligned16(derInput) && aligned16(x) && aligned16(derOutput);
   const dim3 grid((unsigned)(C * p.groups)), block(256);
   double* partials = (double*)workspace;
+  if (p.oneLaunch) {
+    KernelTimer timer("bnorm_backward_apply", s);
+    if (givenMoments) {
+      if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true, false, 1>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
+      else hipLaunchKernelGGL((bnorm_backward_apply<true, false, false, 1>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
+    } else {
+      if (vec) hipLaunchKernelGGL((bnorm_backward_apply<false, true, false, 1>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
+      else hipLaunchKernelGGL((bnorm_backward_apply<false, false, false, 1>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
+    }
+    return check_launch("mcn_bnorm_backward");
+  }
   {
     KernelTimer timer("bnorm_sums", s);
     if (givenMoments) {

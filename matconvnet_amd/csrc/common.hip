@@ -27,6 +27,7 @@ Tunable g_tunables[] = {
     {"pool_forward_threads_k", 2048},  // threads (in 1024s) the four-rows-per-thread forward kernel aims at
     {"pool_force_gather", 0},          // 1: skip the ordered-pass kernel, use the general tiled gather
     {"bnorm_block_elems", 4096},       // minimum elements a bnorm reduction block should own
+    {"bnorm_one_launch_elems", 8192},  // channels of at most this many elements (and >= 128 of them): sums and apply in one launch
     {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)
     {"conv_no_ws", 0},                 // 1: never use the weights-stationary kernel
     {"conv_ws_min_units", 0},          // least number of units for the weights-stationary kernel; 0 = two per SIMD

@@ -14,7 +14,8 @@ pytestmark = pytest.mark.gpu
 
 TOL = 1e-5
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "bnorm_golden.npz")
-SHAPES = [(2, 2, 1, 2), (8, 8, 3, 2), (13, 17, 4, 7), (8, 2, 3, 7), (1, 1, 5, 9), (56, 56, 8, 4), (7, 7, 64, 5), (30, 30, 3, 70)]
+SHAPES = [(2, 2, 1, 2), (8, 8, 3, 2), (13, 17, 4, 7), (8, 2, 3, 7), (1, 1, 5, 9), (56, 56, 8, 4), (7, 7, 64, 5), (30, 30, 3, 70),
+          (7, 7, 130, 6), (14, 14, 256, 4)]   # the last two: many small channels (one launch per call)
 
 
 def _case(shape, seed):
@@ -112,3 +113,37 @@ def test_bottleneck_shapes(capi, ob):
         dx, dg, db, mom = [capi.to_host(t) for t in capi.bnorm_backward(capi.to_device(x), capi.to_device(g), capi.to_device(dy), 1e-5)]
         wdx, wdg, wdb, wmom = ob.bnorm_backward(_d(x), _d(g), _d(dy), 1e-5)
         assert rel_max(dx, wdx) < TOL and rel_max(dg, wdg) < TOL and rel_max(db, wdb) < TOL and rel_max(mom, wmom) < TOL
+
+
+@pytest.mark.parametrize("shape", [(7, 7, 130, 6), (14, 14, 256, 4), (2, 2, 128, 9), (4, 6, 192, 32)])
+def test_small_channels_in_one_launch_give_the_same_bits(capi, shape):
+    """Channels of a few thousand elements are summed and normalised by one launch (one workgroup per channel does
+    both); with that switched off the usual two launches run: every output of every entry point has the same bits."""
+    from util import bits_equal
+    H, W, C, N = shape
+    w = workloads.bnorm_case(seed=21, H=H, W=W, C=C, N=N)
+    r = np.random.default_rng(22)
+    later = F(r.standard_normal(w["x"].shape))
+    later[::3] = 0.0
+    res = F(r.standard_normal(w["x"].shape))
+    xd, gd, bd, dyd, ld, rd = (capi.to_device(v) for v in (w["x"], w["g"], w["b"], w["dy"], later, res))
+    old = capi.get_tunable("bnorm_one_launch_elems")
+    outs = []
+    try:
+        for limit in (old, 0):
+            capi.set_tunable("bnorm_one_launch_elems", limit)
+            got = []
+            y, mom = capi.bnorm_forward(xd, gd, bd, 1e-5)
+            got += [y, mom]
+            got += list(capi.bnorm_forward_fused(xd, gd, bd, residual=rd, relu=True, eps=1e-5))
+            got += list(capi.bnorm_forward_fused(xd, gd, bd, relu=True, eps=1e-5))
+            got += list(capi.bnorm_backward(xd, gd, dyd, 1e-5))
+            got += list(capi.bnorm_backward(xd, gd, dyd, 1e-5, moments=mom))
+            got += list(capi.bnorm_backward_relu(xd, gd, bd, dyd, mom, 1e-5))
+            got += list(capi.bnorm_backward_masked(xd, gd, dyd, ld, mom, 1e-5))
+            outs.append([capi.to_host(t) for t in got if t is not None])
+    finally:
+        capi.set_tunable("bnorm_one_launch_elems", old)
+    assert len(outs[0]) == len(outs[1]) and len(outs[0]) >= 20
+    for a, b_ in zip(*outs):
+        assert bits_equal(a, b_)
