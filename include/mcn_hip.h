@@ -167,6 +167,27 @@ MCN_API int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g
                                      const float* x, const float* derOutput, void* workspace,
                                      size_t workspaceBytes);
 
+/* Filter gradients whose final sum is deferred.  mcn_conv_backward_filter is two launches: the matrix kernel, which
+   leaves one partial bank per reduction split in the workspace, and a sum over the splits of a few microseconds --
+   which a network pays once per layer.  A caller that needs the gradients only at the end of its backward pass can
+   keep each layer's partial banks in a buffer of its own and sum all layers in ONE launch.  No counterpart in the
+   reference (its GEMM accumulates over images with beta = 1, bits/nnconv.cu:300-308).
+     mcn_conv_backward_filter_partial_bytes   size of the buffer of partial banks for this geometry (0: the deferred
+                                              form is not available; use mcn_conv_backward_filter)
+     mcn_conv_backward_filter_plan            the jobs (one per filter group) that will sum `partials` into derFilters
+     mcn_conv_backward_filter_partial         the matrix kernel alone; derFilters is written only by the later sum
+                                              (or at once, when the geometry needs no sum at all: then no job exists)
+     mcn_conv_reduce_layout / _batch          number the workgroups of many jobs; run them all, given the array in
+                                              device memory.  Same bits as mcn_conv_backward_filter. */
+typedef struct { unsigned long long opaque[6]; } mcn_conv_reduce_job;
+MCN_API size_t mcn_conv_backward_filter_partial_bytes(const mcn_conv_geom* g);
+MCN_API int mcn_conv_backward_filter_plan(const mcn_conv_geom* g, float* derFilters, void* partials, size_t partialBytes,
+                                          mcn_conv_reduce_job* jobs, int maxJobs, int* nJobs);
+MCN_API int mcn_conv_backward_filter_partial(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters, const float* x,
+                                             const float* derOutput, void* partials, size_t partialBytes);
+MCN_API unsigned mcn_conv_reduce_layout(mcn_conv_reduce_job* jobs, int nJobs);
+MCN_API int mcn_conv_reduce_batch(mcn_stream_t stream, const mcn_conv_reduce_job* deviceJobs, int nJobs, unsigned totalBlocks);
+
 /* dzdb: K values, fully overwritten  (bits/nnconv.cu:230-244: gemv with the all-ones vector) */
 MCN_API int mcn_conv_backward_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* derBias,
                                    const float* derOutput, void* workspace, size_t workspaceBytes);

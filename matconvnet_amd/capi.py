@@ -51,6 +51,11 @@ PROTOTYPES = {
     "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_taccum": (_i, [_vp, _vp, C.c_float, _vp, C.c_float, _vp, _sz]),
+    "mcn_conv_backward_filter_partial_bytes": (_sz, [_vp]),
+    "mcn_conv_backward_filter_plan": (_i, [_vp, _vp, _vp, _sz, _vp, _i, _vp]),
+    "mcn_conv_backward_filter_partial": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz]),
+    "mcn_conv_reduce_layout": (C.c_uint, [_vp, _i]),
+    "mcn_conv_reduce_batch": (_i, [_vp, _vp, _i, C.c_uint]),
     "mcn_conv_packed_bytes": (_sz, [_vp, _i]),
     "mcn_conv_pack_filters": (_i, [_vp, _vp, _i, _vp, _vp, _sz]),
     "mcn_conv_pack_plan": (_i, [_vp, _i, _vp, _vp, _sz, _vp, _i, _vp]),
@@ -312,6 +317,42 @@ def conv_pack_many(layers):
     check(L.mcn_conv_pack_batch(stream(), ptr(device_jobs), n_jobs, blocks))
     torch.cuda.synchronize()   # (device_jobs must outlive the launch)
     return views
+
+
+class ReduceJob(C.Structure):
+    """mcn_conv_reduce_job of include/mcn_hip.h (opaque)."""
+    _fields_ = [("opaque", C.c_ulonglong * 6)]
+
+
+def conv_backward_filter_deferred(layers):
+    """layers: [(x, dy, g)].  The filter gradients of all of them with ONE launch for the sums over reduction splits
+    (mcn_conv_backward_filter_partial + mcn_conv_reduce_layout / _batch); layers whose geometry has no deferred form
+    go through mcn_conv_backward_filter.  Returns the gradients in order."""
+    torch = _torch()
+    L = lib()
+    jobs = (ReduceJob * 256)()
+    n_jobs, outs, keep = 0, [], []
+    for x, dy, g in layers:
+        df = empty((g.FH, g.FW, g.FC, g.K))
+        outs.append(df)
+        size = L.mcn_conv_backward_filter_partial_bytes(C.byref(g))
+        if size == 0:
+            wp, wn = _ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_FILTER))
+            check(L.mcn_conv_backward_filter(stream(), C.byref(g), ptr(df), ptr(x), ptr(dy), wp, wn))
+            continue
+        partials = torch.empty(size, dtype=torch.uint8, device="cuda")
+        keep.append(partials)
+        got = C.c_int(0)
+        check(L.mcn_conv_backward_filter_plan(C.byref(g), ptr(df), ptr(partials), size,
+                                              C.byref(jobs, n_jobs * C.sizeof(ReduceJob)), 256 - n_jobs, C.byref(got)))
+        n_jobs += got.value
+        check(L.mcn_conv_backward_filter_partial(stream(), C.byref(g), ptr(df), ptr(x), ptr(dy), ptr(partials), size))
+    blocks = L.mcn_conv_reduce_layout(jobs, n_jobs)
+    host = np.frombuffer(jobs, dtype=np.uint8, count=n_jobs * C.sizeof(ReduceJob)).copy()
+    device_jobs = torch.from_numpy(host).cuda() if n_jobs else None
+    check(L.mcn_conv_reduce_batch(stream(), ptr(device_jobs), n_jobs, blocks))
+    torch.cuda.synchronize()   # (device_jobs and the partial banks must outlive the launch)
+    return outs
 
 
 def conv_forward_packed(x, f, packed, b, g, y=None, out_mult=0.0, in_mult=1.0, ws=None):

@@ -270,6 +270,69 @@ int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float*
   return conv_backward_filter_direct(as_stream(stream), p, derFilters, x, derOutput);
 }
 
+namespace {
+static_assert(sizeof(ReduceJob) == sizeof(mcn_conv_reduce_job), "a device array of mcn_conv_reduce_job is read as ReduceJob[]");
+bool deferred_available(const ConvP& p) {
+  return !tunable("conv_force_direct", 0) && conv_mfma_backward_filter_supported(p) && (size_t)p.outH * p.outW * p.N != 0;
+}
+}  // namespace
+
+size_t mcn_conv_backward_filter_partial_bytes(const mcn_conv_geom* g) {
+  ConvP p;
+  if (conv_setup(g, "mcn_conv_backward_filter_partial_bytes", &p) || !deferred_available(p)) return 0;
+  ReduceCtx ctx = {nullptr, 0, 0, nullptr, false};
+  float* dummy = nullptr;
+  if (conv_backward_filter_mfma(nullptr, p, dummy, dummy, dummy, nullptr, 0, &ctx)) return 0;
+  return ctx.offset;
+}
+
+int mcn_conv_backward_filter_plan(const mcn_conv_geom* g, float* derFilters, void* partials, size_t partialBytes,
+                                  mcn_conv_reduce_job* jobs, int maxJobs, int* nJobs) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_filter_plan", &p);
+  if (rc) return rc;
+  if (!nJobs || !derFilters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_plan: null argument");
+  *nJobs = 0;
+  if (!deferred_available(p)) return fail(MCN_UNSUPPORTED, "mcn_conv_backward_filter_plan: this geometry has no deferred sum");
+  std::vector<ReduceJob> found;
+  ReduceCtx ctx = {(char*)partials, partialBytes, 0, &found, false};
+  if ((rc = conv_backward_filter_mfma(nullptr, p, derFilters, derFilters, derFilters, nullptr, 0, &ctx))) return rc;
+  if (ctx.offset > partialBytes) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_plan: buffer of partial banks too small");
+  if ((int)found.size() > maxJobs) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_plan: more than %d jobs", maxJobs);
+  for (size_t i = 0; i < found.size(); ++i) std::memcpy(&jobs[i], &found[i], sizeof(ReduceJob));
+  *nJobs = (int)found.size();
+  return MCN_SUCCESS;
+}
+
+int mcn_conv_backward_filter_partial(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters, const float* x,
+                                     const float* derOutput, void* partials, size_t partialBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_filter_partial", &p);
+  if (rc) return rc;
+  if (!derFilters || !x || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_partial: null tensor");
+  if (!deferred_available(p)) return fail(MCN_UNSUPPORTED, "mcn_conv_backward_filter_partial: this geometry has no deferred sum");
+  if (!aligned16(partials)) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_partial: the buffer must be 16-byte aligned");
+  ReduceCtx ctx = {(char*)partials, partialBytes, 0, nullptr, true};
+  return conv_backward_filter_mfma(as_stream(stream), p, derFilters, x, derOutput, nullptr, 0, &ctx);
+}
+
+unsigned mcn_conv_reduce_layout(mcn_conv_reduce_job* jobs, int nJobs) {
+  unsigned at = 0;
+  for (int i = 0; i < nJobs; ++i) {
+    ReduceJob j;
+    std::memcpy(&j, &jobs[i], sizeof(ReduceJob));
+    j.firstBlock = at;
+    at += j.blocks;
+    std::memcpy(&jobs[i], &j, sizeof(ReduceJob));
+  }
+  return at;
+}
+
+int mcn_conv_reduce_batch(mcn_stream_t stream, const mcn_conv_reduce_job* deviceJobs, int nJobs, unsigned totalBlocks) {
+  if (nJobs > 0 && !deviceJobs) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_reduce_batch: null argument");
+  return conv_reduce_batch(as_stream(stream), (const ReduceJob*)deviceJobs, nJobs, totalBlocks);
+}
+
 int mcn_conv_backward_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* derBias, const float* derOutput,
                            void* workspace, size_t workspaceBytes) {
   ConvP p;

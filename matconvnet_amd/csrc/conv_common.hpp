@@ -53,6 +53,25 @@ struct PackCtx {
   std::vector<PackJob>* jobs;  // kPlan: the jobs are appended here instead of being launched
 };
 
+// The sum over reduction splits that finishes a filter gradient (conv_wgrad_reduce), as data: one entry of a batched
+// launch.  Plain data: it crosses the C ABI as mcn_conv_reduce_job.
+struct ReduceJob {
+  float* df;
+  const float* partials;
+  size_t n;               // elements of the bank
+  int splits, tapMajor, C, T;
+  unsigned firstBlock, blocks;
+};
+
+// Filter gradients whose final sum is deferred: the matrix kernel leaves its partial banks in the caller's buffer
+// (one 256-byte aligned slot per filter group, in group order) and the sums of many layers run in one launch later.
+struct ReduceCtx {
+  char* base;
+  size_t capacity, offset;
+  std::vector<ReduceJob>* jobs;  // not null: the jobs are appended here
+  bool launch;                   // false: plan only (sizes and jobs), nothing is launched
+};
+
 // MFMA implicit-GEMM kernels (groups == 1).  *_supported says whether the fast path covers `p`.
 bool conv_mfma_forward_supported(const ConvP& p);
 bool conv_mfma_backward_data_supported(const ConvP& p);
@@ -64,7 +83,8 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMu
                             void* ws, size_t wsBytes, PackCtx* pk = nullptr);
 int conv_pack_batch(hipStream_t s, const PackJob* deviceJobs, int nJobs, unsigned totalBlocks);
 int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,
-                              size_t wsBytes);
+                              size_t wsBytes, ReduceCtx* deferred = nullptr);
+int conv_reduce_batch(hipStream_t s, const ReduceJob* deviceJobs, int nJobs, unsigned totalBlocks);
 
 // Parameters of the pixel-major products (forward / backward-data): out[co, m] = sum_R wt[R][co] * in[ci(R), pixel(m) + tap(R)]
 struct PixP {

@@ -647,11 +647,10 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
 // dF[e] = sum over splits.  A workgroup owns 64 consecutive elements; thread (e, g) adds the splits
 // g, g+4, g+8, ... (four independent load streams per element, each unrolled), then the four partial sums
 // are combined through LDS in a fixed order.  Deterministic; ~splits/4 dependent loads per thread.
-__global__ __launch_bounds__(256) void conv_wgrad_reduce(float* __restrict__ df, const float* __restrict__ partials,
-                                                         size_t n, int splits, int tapMajor, int C, int T) {
-  __shared__ float part[4][64];
+__device__ __forceinline__ void wgrad_reduce_block(float* __restrict__ df, const float* __restrict__ partials, size_t n,
+                                                   int splits, int tapMajor, int C, int T, unsigned block, float (*part)[64]) {
   const int e = threadIdx.x & 63, g = threadIdx.x >> 6;
-  const size_t i = (size_t)blockIdx.x * 64 + e;
+  const size_t i = (size_t)block * 64 + e;
   float s = 0.f;
   if (i < n) {
     int k = g;
@@ -675,6 +674,26 @@ __global__ __launch_bounds__(256) void conv_wgrad_reduce(float* __restrict__ df,
     }
     df[o] = (part[0][e] + part[1][e]) + (part[2][e] + part[3][e]);
   }
+}
+
+__global__ __launch_bounds__(256) void conv_wgrad_reduce(float* __restrict__ df, const float* __restrict__ partials,
+                                                         size_t n, int splits, int tapMajor, int C, int T) {
+  __shared__ float part[4][64];
+  wgrad_reduce_block(df, partials, n, splits, tapMajor, C, T, blockIdx.x, part);
+}
+
+// The sums of many filter gradients in one launch: workgroup b belongs to the job whose [firstBlock, firstBlock +
+// blocks) holds b.
+__global__ __launch_bounds__(256) void conv_wgrad_reduce_many(const ReduceJob* __restrict__ jobs, int nJobs) {
+  __shared__ float part[4][64];
+  int lo = 0, hi = nJobs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) / 2;
+    if (jobs[mid].firstBlock <= blockIdx.x) lo = mid;
+    else hi = mid - 1;
+  }
+  const ReduceJob j = jobs[lo];
+  wgrad_reduce_block(j.df, j.partials, j.n, j.splits, j.tapMajor, j.C, j.T, blockIdx.x - j.firstBlock, part);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1157,7 +1176,7 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& original, float* dx, flo
 
 namespace {
 int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float* df, const float* x, const float* dy,
-                          void* ws, size_t wsBytes) {
+                          void* ws, size_t wsBytes, ReduceCtx* deferred) {
   WgP q;
   q.xImg = wd.xImg;
   q.dyImg = wd.yImg;
@@ -1185,10 +1204,26 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
   float* target = df;
   if (q.splits > 1 || ut) {
     const size_t need = (size_t)q.splits * nF * sizeof(float);
-    if (!ws || wsBytes < need)
-      return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: workspace too small (%zu < %zu bytes)", wsBytes, need);
-    target = (float*)ws;
+    if (deferred) {
+      // the partial banks stay in the caller's buffer until the deferred sum
+      target = deferred->base ? (float*)(deferred->base + deferred->offset) : nullptr;
+      deferred->offset += align256(need);
+      if (deferred->launch && deferred->offset > deferred->capacity)
+        return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: buffer of partial banks too small (%zu < %zu bytes)",
+                    deferred->capacity, deferred->offset);
+      if (deferred->jobs) {
+        ReduceJob j;
+        j.df = df; j.partials = target; j.n = nF; j.splits = q.splits; j.tapMajor = ut ? 1 : 0; j.C = p.C; j.T = q.T;
+        j.firstBlock = 0; j.blocks = (unsigned)((nF + 63) / 64);
+        deferred->jobs->push_back(j);
+      }
+    } else {
+      if (!ws || wsBytes < need)
+        return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: workspace too small (%zu < %zu bytes)", wsBytes, need);
+      target = (float*)ws;
+    }
   }
+  if (deferred && !deferred->launch) return MCN_SUCCESS;
   {
     const unsigned long long ob = (unsigned long long)q.splits * nF * sizeof(float);
     q.outBytes = ob < (1ull << 31) ? (unsigned)ob : 0u;
@@ -1207,7 +1242,7 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
     else rc = launch_wgrad<1, 1, 1, 4, false>(s, grid, target, x, dy, q);
   }
   if (!rc) rc = check_launch("mcn_conv_backward_filter");
-  if (rc || target == df) return rc;
+  if (rc || target == df || deferred) return rc;
   KernelTimer timer("conv_wgrad_reduce", s);
   hipLaunchKernelGGL(conv_wgrad_reduce, dim3((unsigned)((nF + 63) / 64)), block, 0, s, df, target, nF, q.splits, ut ? 1 : 0,
                      p.C, q.T);
@@ -1215,15 +1250,22 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
 }
 }  // namespace
 
+int conv_reduce_batch(hipStream_t s, const ReduceJob* deviceJobs, int nJobs, unsigned totalBlocks) {
+  if (nJobs <= 0 || totalBlocks == 0) return MCN_SUCCESS;
+  KernelTimer timer("conv_wgrad_reduce_many", s);
+  hipLaunchKernelGGL(conv_wgrad_reduce_many, dim3(totalBlocks), dim3(256), 0, s, deviceJobs, nJobs);
+  return check_launch("mcn_conv_reduce_batch");
+}
+
 int conv_backward_filter_mfma(hipStream_t s, const ConvP& original, float* df, const float* x, const float* dy, void* ws,
-                              size_t wsBytes) {
+                              size_t wsBytes, ReduceCtx* deferred) {
   const ConvP p = fc_view(original);
   const ConvP g = group_view(p);
   const Wide wd = wide_of(p);
   const bool ut = wgrad_uniform_tap(p);
   const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
   for (int i = 0; i < p.groups; ++i) {
-    int rc = backward_filter_group(s, g, wd, ut, df + i * p.Kg * FV, x + i * p.FC * HW, dy + i * p.Kg * Q, ws, wsBytes);
+    int rc = backward_filter_group(s, g, wd, ut, df + i * p.Kg * FV, x + i * p.FC * HW, dy + i * p.Kg * Q, ws, wsBytes, deferred);
     if (rc) return rc;
   }
   return MCN_SUCCESS;

@@ -454,3 +454,22 @@ def test_packed_buffer_too_small_is_refused(capi):
     small = capi.to_device(np.zeros(n // 8, np.float32))
     rc = capi.lib().mcn_conv_pack_filters(capi.stream(), C.byref(g), capi.CONV_FORWARD, capi.ptr(f), capi.ptr(small), n // 2)
     assert rc != 0 and b"too small" in capi.lib().mcn_last_error_message()
+
+
+def test_filter_gradients_with_one_deferred_sum(capi):
+    """The filter gradients of several layers (1x1, 3x3, strided, grouped, 3-channel, fully connected) from the matrix
+    kernels alone plus ONE launch that sums all their reduction splits, against mcn_conv_backward_filter per layer."""
+    import torch
+    r = np.random.default_rng(6)
+    layers, want = [], []
+    for H, W, Cc, N, FH, FW, K, stride, pad, dilate, groups in PACKED_CASES:
+        xs, fs = (H, W, Cc, N), (FH, FW, Cc // groups, K)
+        g = capi.conv_geom(xs, fs, stride, pad, dilate)
+        x = capi.to_device(F(r.standard_normal(xs)))
+        dy = capi.to_device(F(r.standard_normal(capi.conv_out_shape(g))))
+        layers.append((x, dy, g))
+        want.append(capi.conv_backward(x, None, dy, g, want=(False, True, False))[1])
+    got = capi.conv_backward_filter_deferred(layers)
+    assert sum(capi.lib().mcn_conv_backward_filter_partial_bytes(__import__("ctypes").byref(g)) > 0 for _, _, g in layers) >= 6
+    for a, b_, case in zip(got, want, PACKED_CASES):
+        assert torch.equal(a, b_), case
