@@ -13,7 +13,8 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
                        Context* shared)
     : H(H), W(W), C(C), M(M), N(N), Cout(CoutArg > 0 ? CoutArg : C), stride(stride), Ho((H - 1) / stride + 1),
       Wo((W - 1) / stride + 1), adapter(adapter), epsilon(epsilon), context(shared ? *shared : ownContext),
-      error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), testMode(false), packed(false), packedArena(NULL), packedJobs(NULL), packedBlocks(0), sideStream(NULL) {
+      error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), testMode(false), packed(false), packedArena(NULL), packedJobs(NULL), packedBlocks(0), deferred(false), externalSums(false),
+      partialArena(NULL), sumJobsDevice(NULL), sumBlocks(0), sideStream(NULL) {
   for (int i = 0; i < 5; ++i) events[i] = NULL;
   if (!adapter && (Cout != C || stride != 1)) {
     error = VLE_IllegalArgument;
@@ -85,6 +86,8 @@ Bottleneck::~Bottleneck() {
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
   if (packedArena) (void)hipFree(packedArena);
   if (packedJobs) (void)hipFree(packedJobs);
+  if (partialArena) (void)hipFree(partialArena);
+  if (sumJobsDevice) (void)hipFree(sumJobsDevice);
 }
 
 #define STEP(stage, call)                                   \
@@ -141,6 +144,53 @@ ErrorCode Bottleneck::setPacked(bool on) {
       if (e != VLE_Success) return fail(e, "planPack");
     }
   packed = true;
+  return VLE_Success;
+}
+
+ErrorCode Bottleneck::setDeferred(bool on, bool external) {
+  if (partialArena) (void)hipFree(partialArena);
+  if (sumJobsDevice) (void)hipFree(sumJobsDevice);
+  partialArena = sumJobsDevice = NULL;
+  sumJobs.clear();
+  deferred = false;
+  if (!on || error != VLE_Success) return error;
+  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),
+      cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
+  struct Layer { nn::Convolution* op; char const* data; char const* der; };
+  const Layer layers[4] = {{&c1, "x", "df1"}, {&c2, "r1", "df2"}, {&c1, "r2", "df3"}, {&cs, "x", "dfs"}};
+  const int count = adapter ? 4 : 3;
+  std::size_t total = 0;
+  for (int l = 0; l < 4; ++l) partialBank[l].offset = partialBank[l].bytes = 0;
+  for (int l = 0; l < count; ++l) {
+    partialBank[l].offset = total;
+    partialBank[l].bytes = layers[l].op->filterPartialBytes(slot(layers[l].data).getShape(), slot(layers[l].der).getShape());
+    total += partialBank[l].bytes;
+  }
+  if (hipMalloc(&partialArena, total ? total : 16) != hipSuccess) {
+    (void)hipGetLastError();
+    partialArena = NULL;
+    message = "cannot allocate the partial filter gradients";
+    return VLE_OutOfGPUMemeory;
+  }
+  for (int l = 0; l < count; ++l) {
+    if (partialBank[l].bytes == 0) continue;
+    ErrorCode e = layers[l].op->planFilterPartial(slot(layers[l].data).getShape(), slot(layers[l].der),
+                                                  (char*)partialArena + partialBank[l].offset, partialBank[l].bytes, sumJobs);
+    if (e != VLE_Success) return fail(e, "planFilterPartial");
+  }
+  if (!external && !sumJobs.empty()) {
+    std::vector<mcn_conv_reduce_job> numbered(sumJobs);
+    sumBlocks = mcn_conv_reduce_layout(numbered.data(), (int)numbered.size());
+    const std::size_t bytes = numbered.size() * sizeof(mcn_conv_reduce_job);
+    if (hipMalloc(&sumJobsDevice, bytes) != hipSuccess ||
+        hipMemcpy(sumJobsDevice, numbered.data(), bytes, hipMemcpyHostToDevice) != hipSuccess) {
+      (void)hipGetLastError();
+      message = "cannot upload the summing jobs";
+      return VLE_Cuda;
+    }
+  }
+  deferred = true;
+  externalSums = external;
   return VLE_Success;
 }
 
@@ -202,6 +252,7 @@ float* Bottleneck::buffer(std::string const& name, std::size_t* count) {
 
 ErrorCode Bottleneck::alias(std::string const& name, float* memory) {
   if (packed) setPacked(false);  // (the packing jobs hold the old addresses)
+  if (deferred) setDeferred(false);
   for (std::size_t i = 0; i < slots.size(); ++i) {
     if (slots[i].name != name) continue;
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
@@ -312,8 +363,16 @@ ErrorCode Bottleneck::backward() {
   nn::Convolution c1s(sideContext, 1, 1, 0, 0, 0, 0, 1, 1), c2s(sideContext, stride, stride, 1, 1, 1, 1, 1, 1),
       css(sideContext, stride, stride, 0, 0, 0, 0, 1, 1);
   Tensor none2, none3;
+  // (k: the event of the two-stream schedule; 3 - k = the layer's place in {conv1, conv2, conv3, adapter} for k < 3)
   auto convBackward = [&](nn::Convolution& onMain, nn::Convolution& onSide, int k, Tensor& derIn, double derInMult,
                           Tensor& derFilter, Tensor const& in, Tensor const& filter, Tensor const& derOut) -> ErrorCode {
+    const int layer = k == 3 ? 3 : 2 - k;
+    if (!overlap && deferred && partialBank[layer].bytes) {
+      ErrorCode ed = onMain.backwardAccumulate(derIn, derInMult, none2, none, in, filter, derOut);
+      if (ed != VLE_Success) return ed;
+      return onMain.backwardFilterPartial(derFilter, in, derOut, (char*)partialArena + partialBank[layer].offset,
+                                          partialBank[layer].bytes);
+    }
     if (!overlap) return onMain.backwardAccumulate(derIn, derInMult, derFilter, none, in, filter, derOut);
     if (hipEventRecord((hipEvent_t)events[k], (hipStream_t)st) != hipSuccess ||
         hipStreamWaitEvent((hipStream_t)sideStream, (hipEvent_t)events[k], 0) != hipSuccess)
@@ -325,6 +384,10 @@ ErrorCode Bottleneck::backward() {
     return e;
   };
   auto joinSide = [&]() -> ErrorCode {
+    if (!overlap && deferred && !externalSums && !sumJobs.empty()) {
+      int rcSum = mcn_conv_reduce_batch(st, (mcn_conv_reduce_job const*)sumJobsDevice, (int)sumJobs.size(), sumBlocks);
+      if (rcSum) return context.setError((ErrorCode)rcSum, mcn_last_error_message());
+    }
     if (!overlap) return VLE_Success;
     if (hipEventRecord((hipEvent_t)events[4], (hipStream_t)sideStream) != hipSuccess ||
         hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)events[4], 0) != hipSuccess)

@@ -61,6 +61,12 @@ class Bottleneck {
   ErrorCode setPacked(bool on);
   ErrorCode pack();
   std::vector<mcn_conv_pack_job> const& packJobs() const { return jobs; }
+  // deferred = true: backward() runs only the matrix kernels of the filter gradients and keeps their partial banks;
+  // the sums over reduction splits of all the unit's layers run in one launch at the end of backward() -- or, with
+  // `external`, in a launch of the caller's that covers several units (reduceJobs()).  Same bits.  Not combined with
+  // setOverlap.
+  ErrorCode setDeferred(bool on, bool external = false);
+  std::vector<mcn_conv_reduce_job> const& reduceJobs() const { return sumJobs; }
   ErrorCode forward();
   ErrorCode backward();
 
@@ -96,6 +102,12 @@ class Bottleneck {
   void* packedJobs;              // device copy of `jobs`, numbered for the unit's own launch
   unsigned packedBlocks;
   std::vector<mcn_conv_pack_job> jobs;
+  bool deferred, externalSums;
+  Bank partialBank[4];           // [convolution]: its partial banks inside partialArena (bytes 0: no deferred form)
+  void* partialArena;
+  void* sumJobsDevice;
+  unsigned sumBlocks;
+  std::vector<mcn_conv_reduce_job> sumJobs;
   Context sideContext;
   void* sideStream;     // hipStream_t
   void* events[5];      // hipEvent_t: "derivative ready" for the convolutions, "second stream done"

@@ -52,6 +52,8 @@ VLH_API void vlh_bottleneck_set_fused(void* block, int fused);
 VLH_API int vlh_bottleneck_set_overlap(void* block, int overlap);
 /* packed != 0: the convolutions read filter banks packed ahead; vlh_bottleneck_pack refreshes them (one launch) and
    must follow every change of the filters */
+/* deferred != 0: one launch sums the reduction splits of all the unit's filter gradients at the end of backward */
+VLH_API int vlh_bottleneck_set_deferred(void* block, int deferred);
 VLH_API int vlh_bottleneck_set_packed(void* block, int packed);
 VLH_API int vlh_bottleneck_pack(void* block);
 VLH_API int vlh_bottleneck_forward(void* block);
@@ -76,6 +78,9 @@ VLH_API void vlh_resnet50_set_test_mode(void* net, int test);
 /* packed != 0: all convolutions read filter banks packed ahead, refreshed by ONE launch: by vlh_resnet50_pack, and at the
    end of vlh_resnet50_sgd_step and vlh_resnet50_init.  Call vlh_resnet50_pack after writing filters through
    vlh_resnet50_buffer.  Same bits as packing on every call (the default). */
+/* deferred != 0: the sums over reduction splits that finish the filter gradients run in ONE launch at the end of
+   vlh_resnet50_backward instead of one per layer (same bits) */
+VLH_API int vlh_resnet50_set_deferred(void* net, int deferred);
 VLH_API int vlh_resnet50_set_packed(void* net, int packed);
 VLH_API int vlh_resnet50_pack(void* net);
 VLH_API int vlh_resnet50_init(void* net, unsigned long long seed);

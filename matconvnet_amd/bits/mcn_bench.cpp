@@ -213,7 +213,7 @@ static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, 
   upload("f3", std::sqrt(2.f / M), 0, true);
   for (char const* g : {"g1", "g2", "g3"}) upload(g, 0, 1.f, false);
   for (char const* b : {"b1", "b2", "b3"}) upload(b, 0, 0.f, false);
-  if (packed && block.setPacked(true) != VLE_Success) {
+  if (packed && (block.setPacked(true) != VLE_Success || block.setDeferred(true) != VLE_Success)) {
     std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
     std::exit(3);
   }
@@ -225,7 +225,7 @@ static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, 
     }
   }, warmup, iters);
   std::printf("%-28s %8.3f ms/step %9.0f images/s (fwd+bwd, N = %d, 41.93 GFLOP of convolution per step; %s)\n",
-              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, packed ? "folded, filter banks packed by one launch per step"
+              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, packed ? "folded, filter banks packed by one launch per step, filter gradients summed by one"
                      : (overlap ? "folded, filter gradients on a second stream" : (fused ? "relu/sum folded into bnorm" : "layer by layer")));
 }
 
@@ -238,7 +238,8 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
     std::exit(3);
   }
   net.setFused(fused);
-  if (fused && net.setPacked(true) != VLE_Success) {  // (the folded run also packs the filter banks ahead, once per update)
+  // (the folded run also packs the filter banks ahead, once per update)
+  if (fused && net.setPacked(true) != VLE_Success) {
     std::fprintf(stderr, "resnet-50: %s\n", net.lastMessage().c_str());
     std::exit(3);
   }

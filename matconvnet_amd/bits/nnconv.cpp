@@ -79,6 +79,41 @@ ErrorCode Convolution::planPack(int product, TensorShape const& data, Tensor con
   return VLE_Success;
 }
 
+std::size_t Convolution::filterPartialBytes(TensorShape const& data, TensorShape const& filter) const {
+  mcn_conv_geom g = geometry(*this, data, filter);
+  return mcn_conv_backward_filter_partial_bytes(&g);
+}
+
+ErrorCode Convolution::planFilterPartial(TensorShape const& data, Tensor& derFilter, void* partials, std::size_t bytes,
+                                         std::vector<mcn_conv_reduce_job>& jobs) {
+  mcn_conv_geom g = geometry(*this, data, derFilter);
+  mcn_conv_reduce_job found[64];
+  int n = 0;
+  int rc = mcn_conv_backward_filter_plan(&g, (float*)derFilter.getMemory(), partials, bytes, found, 64, &n);
+  if (rc) return fromAbi(context, rc, "Convolution::planFilterPartial");
+  jobs.insert(jobs.end(), found, found + n);
+  return VLE_Success;
+}
+
+ErrorCode Convolution::backwardFilterPartial(Tensor& derFilter, Tensor const& input, Tensor const& derOutput, void* partials,
+                                             std::size_t bytes) {
+  tensor_type tt = findTensorType(derFilter, input, derOutput);
+  ErrorCode e = requireHipFloat(context, tt, "Convolution::backwardFilterPartial");
+  if (e != VLE_Success) return e;
+  if (!derFilter || !input || !derOutput)
+    return context.setError(VLE_IllegalArgument, "Convolution::backwardFilterPartial: DERFILTER, INPUT and DEROUTPUT are required");
+  mcn_conv_geom g = geometry(*this, input, derFilter);
+  int oh = 0, ow = 0;
+  int rc = mcn_conv_output_size(&g, &oh, &ow);
+  if (rc) return fromAbi(context, rc, "Convolution::backwardFilterPartial");
+  if ((int)derOutput.getHeight() != oh || (int)derOutput.getWidth() != ow || derOutput.getDepth() != derFilter.getSize() ||
+      derOutput.getSize() != input.getSize())
+    return context.setError(VLE_IllegalArgument, "Convolution::backwardFilterPartial: DEROUTPUT dimensions are incompatible with X and FILTERS");
+  rc = mcn_conv_backward_filter_partial(context.getHipHelper().getStream(), &g, (float*)derFilter.getMemory(),
+                                        (float const*)input.getMemory(), (float const*)derOutput.getMemory(), partials, bytes);
+  return fromAbi(context, rc, "Convolution::backwardFilterPartial");
+}
+
 ErrorCode Convolution::backward(Tensor& derInput, Tensor& derFilter, Tensor& derBias, Tensor const& input,
                                 Tensor const& filter, Tensor const& derOutput) {
   return backwardAccumulate(derInput, 0, derFilter, derBias, input, filter, derOutput);

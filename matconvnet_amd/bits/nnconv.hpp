@@ -43,6 +43,16 @@ class Convolution {
     packedBackward = backwardBank; packedBackwardBytes = backwardBytes;
   }
 
+  // Filter gradient with its final sum deferred (mcn_conv_backward_filter_partial and friends): the matrix kernel
+  // leaves the partial banks in `partials`; the jobs planned once sum them into derFilter in a launch the caller
+  // makes for many layers at once.  filterPartialBytes == 0: this geometry has no deferred form (use backward).
+  // Not part of the reference's class.
+  std::size_t filterPartialBytes(vl::TensorShape const& data, vl::TensorShape const& filter) const;
+  vl::ErrorCode planFilterPartial(vl::TensorShape const& data, vl::Tensor& derFilter, void* partials, std::size_t bytes,
+                                  std::vector<mcn_conv_reduce_job>& jobs);
+  vl::ErrorCode backwardFilterPartial(vl::Tensor& derFilter, vl::Tensor const& input, vl::Tensor const& derOutput,
+                                      void* partials, std::size_t bytes);
+
   Context& context;
   int strideY;
   int strideX;

@@ -38,7 +38,8 @@ double conv_flops(int outH, int outW, int fh, int fw, int cin, int cout) {
 ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
     : N(N), S(imageSize), classes(classes), epsilon(epsilon), fused(true), testMode(false), error(VLE_Success), flops(0), values(NULL),
       ders(NULL), state(NULL), batchMoments(NULL), runningMoments(NULL), chunkParam(NULL), rates(NULL), chunks(0),
-      momentsCount(0), parameterCount(0), packed(false), packedArena(NULL), packedJobs(NULL), stemBytes(0),
+      momentsCount(0), parameterCount(0), deferred(false), partialArena(NULL), sumJobsDevice(NULL), stemPartialBytes(0),
+      fcPartialBytes(0), sumJobCount(0), sumBlocks(0), packed(false), packedArena(NULL), packedJobs(NULL), stemBytes(0),
       fcForwardBytes(0), fcBackwardBytes(0), fcBackwardOffset(0), packedJobCount(0), packedBlocks(0), graph(NULL),
       graphExec(NULL) {
   if (S < 32 || S % 32 != 0) {
@@ -265,6 +266,50 @@ ErrorCode ResNet50::setPacked(bool on) {
   return pack();
 }
 
+ErrorCode ResNet50::setDeferred(bool on) {
+  if (error != VLE_Success) return error;
+  dropGraph();
+  if (partialArena) (void)hipFree(partialArena);
+  if (sumJobsDevice) (void)hipFree(sumJobsDevice);
+  partialArena = sumJobsDevice = NULL;
+  deferred = false;
+  for (std::size_t i = 0; i < units.size(); ++i)
+    if (units[i]->setDeferred(on, true) != VLE_Success) {
+      message = units[i]->lastMessage();
+      return VLE_OutOfGPUMemeory;
+    }
+  if (!on) return VLE_Success;
+  nn::Convolution stem(context, 2, 2, 3, 3, 3, 3, 1, 1), fc(context, 1, 1, 0, 0, 0, 0, 1, 1);
+  const TensorShape inputShape = slot("input").getShape(), avgShape = slot("avg").getShape();
+  stemPartialBytes = stem.filterPartialBytes(inputShape, slot("stem.df").getShape());
+  fcPartialBytes = fc.filterPartialBytes(avgShape, slot("fc.df").getShape());
+  const std::size_t total = stemPartialBytes + fcPartialBytes;
+  if (hipMalloc(&partialArena, total ? total : 16) != hipSuccess) {
+    (void)hipGetLastError();
+    partialArena = NULL;
+    message = "cannot allocate the partial filter gradients";
+    return VLE_OutOfGPUMemeory;
+  }
+  std::vector<mcn_conv_reduce_job> jobs;
+  char* arena = (char*)partialArena;
+  if ((stemPartialBytes && stem.planFilterPartial(inputShape, slot("stem.df"), arena, stemPartialBytes, jobs) != VLE_Success) ||
+      (fcPartialBytes && fc.planFilterPartial(avgShape, slot("fc.df"), arena + stemPartialBytes, fcPartialBytes, jobs) != VLE_Success))
+    return fail(context.getLastError(), "planFilterPartial");
+  for (std::size_t i = 0; i < units.size(); ++i)
+    jobs.insert(jobs.end(), units[i]->reduceJobs().begin(), units[i]->reduceJobs().end());
+  sumJobCount = (int)jobs.size();
+  sumBlocks = mcn_conv_reduce_layout(jobs.data(), sumJobCount);
+  const std::size_t bytes = jobs.size() * sizeof(mcn_conv_reduce_job);
+  if (hipMalloc(&sumJobsDevice, bytes ? bytes : 16) != hipSuccess ||
+      hipMemcpy(sumJobsDevice, jobs.data(), bytes, hipMemcpyHostToDevice) != hipSuccess) {
+    (void)hipGetLastError();
+    message = "cannot upload the summing jobs";
+    return VLE_Cuda;
+  }
+  deferred = true;
+  return VLE_Success;
+}
+
 ErrorCode ResNet50::pack() {
   if (error != VLE_Success) return error;
   if (!packed) return VLE_Success;
@@ -333,7 +378,8 @@ ResNet50::~ResNet50() {
   for (std::size_t i = 0; i < units.size(); ++i) delete units[i];
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
-  void* arenas[] = {values, ders, state, batchMoments, runningMoments, chunkParam, rates, packedArena, packedJobs};
+  void* arenas[] = {values, ders, state, batchMoments, runningMoments, chunkParam, rates, packedArena, packedJobs,
+                    partialArena, sumJobsDevice};
   for (void* a : arenas)
     if (a) (void)hipFree(a);
 }
@@ -529,7 +575,13 @@ ErrorCode ResNet50::backward() {
   Tensor derFeatures(TensorShape(Hf, Hf, Cf, N), VLDT_Float, VLDT_GPU, last->buffer("dzdy"), sizeof(float) * nFeatures);
   nn::Pooling avgPool(context, Hf, Hf, 1, 1, 0, 0, 0, 0, nn::Pooling::Average);
   if (packed) fc.usePacked(NULL, 0, fcBackwardBytes ? (char*)packedArena + fcBackwardOffset : NULL, fcBackwardBytes);
-  STEP("classifier", fc.backward(slot("davg"), slot("fc.df"), slot("fc.db"), slot("avg"), slot("fc.f"), slot("dprediction")));
+  if (deferred && fcPartialBytes) {
+    STEP("classifier", fc.backward(slot("davg"), none, slot("fc.db"), slot("avg"), slot("fc.f"), slot("dprediction")));
+    STEP("classifier", fc.backwardFilterPartial(slot("fc.df"), slot("avg"), slot("dprediction"),
+                                                (char*)partialArena + stemPartialBytes, fcPartialBytes));
+  } else {
+    STEP("classifier", fc.backward(slot("davg"), slot("fc.df"), slot("fc.db"), slot("avg"), slot("fc.f"), slot("dprediction")));
+  }
   STEP("average pool", avgPool.backwardOverwrite(derFeatures, features, slot("davg")));
   for (std::size_t i = units.size(); i-- > 0;)
     if (units[i]->backward() != VLE_Success) {
@@ -553,7 +605,13 @@ ErrorCode ResNet50::backward() {
                                              slot("stem.g"), slot("stem.b"), slot("stem.dn")));
   }
   // the network's input needs no derivative: filter gradient only
-  STEP("stem conv", stem.backward(none, slot("stem.df"), none, slot("input"), slot("stem.f"), slot("stem.da")));
+  if (deferred && stemPartialBytes) {
+    STEP("stem conv", stem.backwardFilterPartial(slot("stem.df"), slot("input"), slot("stem.da"), partialArena, stemPartialBytes));
+  } else {
+    STEP("stem conv", stem.backward(none, slot("stem.df"), none, slot("input"), slot("stem.f"), slot("stem.da")));
+  }
+  if (deferred)  // the sums over the reduction splits of every filter gradient of the network
+    ABI("filter sums", mcn_conv_reduce_batch(st, (mcn_conv_reduce_job const*)sumJobsDevice, sumJobCount, sumBlocks));
   return VLE_Success;
 }
 

@@ -47,6 +47,9 @@ class ResNet50 {
   // sgdStep() and initParameters() end with pack(); a caller that writes filters itself (through buffer()) calls it.
   ErrorCode setPacked(bool on);
   ErrorCode pack();
+  // deferred = true: backward() runs the matrix kernels of all filter gradients and sums their reduction splits in ONE
+  // launch at its end instead of one per layer.  Same bits.
+  ErrorCode setDeferred(bool on);
   ErrorCode forward();
   ErrorCode backward();
   // one update of all parameters from the derivatives backward() left (numWorkers = 1), and of the moving averages of
@@ -88,6 +91,11 @@ class ResNet50 {
   unsigned short* chunkParam;   // device
   double* rates;                // device
   std::size_t chunks, momentsCount, parameterCount;
+  bool deferred;
+  void *partialArena, *sumJobsDevice;   // partial banks of the stem and the classifier; device table of all summing jobs
+  std::size_t stemPartialBytes, fcPartialBytes;
+  int sumJobCount;
+  unsigned sumBlocks;
   bool packed;
   void *packedArena, *packedJobs;   // banks of the stem and the classifier; device table of all the network's jobs
   std::size_t stemBytes, fcForwardBytes, fcBackwardBytes, fcBackwardOffset;

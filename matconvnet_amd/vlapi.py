@@ -81,6 +81,8 @@ def lib():
         L.vlh_resnet50_set_fused.restype = None
         L.vlh_resnet50_set_test_mode.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_test_mode.restype = None
+        L.vlh_resnet50_set_deferred.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_bottleneck_set_deferred.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_packed.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_pack.argtypes = [C.c_void_p]
         L.vlh_bottleneck_set_packed.argtypes = [C.c_void_p, C.c_int]
@@ -244,9 +246,12 @@ class ResNet50(_NamedBuffers):
     the loss layers); buffers are owned by the C++ side and named "input", "prediction", "dprediction",
     "stem.f", "fc.f", "unit<i>.<name>", ..."""
 
-    def __init__(self, N=32, eps=1e-5, image_size=224, classes=1000, fused=True, seed=None, packed=True):
+    def __init__(self, N=32, eps=1e-5, image_size=224, classes=1000, fused=True, seed=None, packed=True, deferred=False):
         """packed: the convolutions read filter banks packed ahead, refreshed in one launch after every update (and by
-        `set` of a parameter here); False: every call packs its own, as the plain operator calls do."""
+        `set` of a parameter here); False: every call packs its own, as the plain operator calls do.
+        deferred: the sums that finish the filter gradients run in one launch at the end of backward (off by
+        default: for a whole network the partial banks, about 33 MB per layer, have left the caches by then, and
+        reading them back from memory costs what the 54 saved launches gain)."""
         self.L = lib()
         self.packed = False
         self.N, self.image_size, self.classes = N, image_size, classes
@@ -261,6 +266,8 @@ class ResNet50(_NamedBuffers):
         if packed:
             self._check(self.L.vlh_resnet50_set_packed(self.h, 1))
             self.packed = True
+        if deferred:
+            self._check(self.L.vlh_resnet50_set_deferred(self.h, 1))
         if seed is not None:
             self._check(self.L.vlh_resnet50_init(self.h, seed))
 
@@ -333,9 +340,10 @@ class Bottleneck(_NamedBuffers):
     """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
 
     def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False, overlap=False, Cout=0, stride=1,
-                 adapter=False, packed=False):
+                 adapter=False, packed=False, deferred=False):
         """packed: the convolutions read filter banks packed ahead; `set` of a filter and every step of `run` refresh
-        them with one launch (`pack`)."""
+        them with one launch (`pack`).  deferred: one launch at the end of backward sums the reduction splits of all
+        the unit's filter gradients."""
         self.L = lib()
         self.packed = False
         self.shape = (H, W, Cc, M, N)
@@ -348,6 +356,8 @@ class Bottleneck(_NamedBuffers):
         if packed:
             self._check(self.L.vlh_bottleneck_set_packed(self.h, 1))
             self.packed = True
+        if deferred:
+            self._check(self.L.vlh_bottleneck_set_deferred(self.h, 1))
 
     def set(self, name, array):
         super().set(name, array)

@@ -334,7 +334,7 @@ UNITS = [  # (H, W, C, M, Cout, stride, adapter): the kinds of segment ResNet-50
 @pytest.mark.parametrize("H,W,Cc,M,Cout,stride,adapter", UNITS)
 def test_residual_unit_against_oracle_and_across_modes(vl, ob, H, W, Cc, M, Cout, stride, adapter):
     """Each kind of ResNet-50 segment, N = 3: against the unit composed from oracle operators (double), and the fused,
-    two-stream and packed-ahead schedules bit for bit against the layer-by-layer one."""
+    two-stream and packed-ahead / deferred-sum schedules bit for bit against the layer-by-layer one."""
     w = workloads.bottleneck_case(seed=9, H=H, W=W, C=Cc, M=M, N=3, Cout=Cout, stride=stride, adapter=adapter)
     Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
     shapes = dict(y=(Ho, Wo, Cout, 3), dzdx=w["x"].shape, df1=w["f1"].shape, df2=w["f2"].shape, df3=w["f3"].shape,
@@ -346,7 +346,7 @@ def test_residual_unit_against_oracle_and_across_modes(vl, ob, H, W, Cc, M, Cout
     outs = {}
     for mode in ("plain", "fused", "overlap", "packed"):
         blk = vl.Bottleneck(H=H, W=W, Cc=Cc, M=M, N=3, eps=w["eps"], fused=mode != "plain", overlap=mode == "overlap",
-                            Cout=Cout, stride=stride, adapter=adapter, packed=mode == "packed")
+                            Cout=Cout, stride=stride, adapter=adapter, packed=mode == "packed", deferred=mode == "packed")
         try:
             for k in names:
                 blk.set(k, w[k])

@@ -253,14 +253,15 @@ def test_test_mode_uses_the_stored_moments(vl, case):
     assert bits_equal(outs[False], outs[True])
 
 
-def test_filters_packed_ahead_change_no_bit(vl, case):
-    """All convolutions reading banks packed ahead by one launch (after uploads, and after every update) against every
-    call packing its own: predictions, gradients, and the parameters after two training steps."""
+def test_filters_packed_ahead_and_deferred_sums_change_no_bit(vl, case):
+    """All convolutions reading banks packed ahead by one launch (after uploads, and after every update), and all
+    filter gradients finished by one summing launch at the end of backward, against every call packing and summing
+    for itself: predictions, gradients, and the parameters after two training steps."""
     lr, mom, wd = 0.05, 0.9, 1e-4
     watch = _gradient_names(case) + ["stem.f", "unit0.f1", "unit3.f2", "unit3.fs", "unit15.f3", "fc.f", "momentum.unit7.f2"]
     seen = {}
     for packed in (False, True):
-        net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=True, packed=packed)
+        net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=True, packed=packed, deferred=packed)  # (deferred is off by default)
         try:
             _load(net, case)
             for _ in range(2):
