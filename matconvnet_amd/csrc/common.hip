@@ -30,7 +30,9 @@ Tunable g_tunables[] = {
     {"bnorm_one_launch_elems", 8192},  // channels of at most this many elements (and >= 128 of them): sums and apply in one launch
     {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)
     {"conv_no_ws", 0},                 // 1: never use the weights-stationary kernel
-    {"conv_ws_min_units", 0},          // least number of units for the weights-stationary kernel; 0 = two per SIMD
+    {"conv_ws_min_units", 0},          // least number of units for the weights-stationary kernel; 0 = one per two SIMDs
+    {"conv_ws_max_slices", 8},         // most slices of output channels its bank may be cut into (1: whole banks only)
+    {"conv_ws_sliced_strided", 0},     // 1: sliced banks also for strided gathers (slower than the tiled kernel)
     {"conv_ws_wa", 0},                 // 1, 2, 4: force its channels-per-wavefront (in units of 32); 0 = choose
     {"conv_no_split", 0},              // 1: the tiled kernel never splits its reduction over workgroups
     {"conv_split_max_blocks", 512},    // ... it splits when the unsplit launch has at most this many workgroups,

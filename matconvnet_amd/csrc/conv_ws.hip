@@ -35,8 +35,9 @@ constexpr int kDepth = 8;       // reduction pairs per group: Cin must be a mult
 constexpr int kMaxTapsWs = 128;
 
 struct WsP {
-  int nUnits;        // pixel blocks x channel blocks
-  int chanBlocks;    // coutPad / (32 WA)
+  int nUnits;        // pixel blocks x channel blocks, of one slice
+  int slices;        // the bank is cut into this many slices of output channels; a workgroup holds one of them
+  int chanBlocks;    // channel blocks of 32 WA channels per slice: coutPad / (32 WA slices)
   int groups;        // R / (2 kDepth)
   int groupsPerTap;  // Cin / (2 kDepth)
   unsigned inBytes;  // size of the gathered tensor
@@ -59,6 +60,14 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   const int l32 = lane & 31, kh = lane >> 5;
   const int IHW = p.IH * p.IW;
 
+  // Banks too large for LDS are cut into slices of output channels: workgroup w holds slice w % slices and works
+  // through all the pixels for those channels (the pixels are then read once per slice, from L2 after the first).
+  const int wgAll = TAPS ? xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x) : (int)blockIdx.x;
+  const int slice = w.slices > 1 ? wgAll % w.slices : 0;
+  const int wg = w.slices > 1 ? wgAll / w.slices : wgAll;          // this workgroup's place among those of its slice
+  const int nWg = (int)gridDim.x / w.slices;
+  const int cbBase = slice * w.chanBlocks;                         // first channel block of the slice
+
   // ---- once per workgroup: the bank, re-laid by channel block
   {
     const int perBlock = p.R * (ROW / 4);  // 16-byte vectors per channel block
@@ -74,7 +83,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
         const int rem = i - cbk * perBlock;
         int r, c4;
         w.byRow.divmod(rem, &r, &c4);
-        v[k] = *(const v4f*)(wt + (size_t)r * p.coutPad + cbk * ROW + c4 * 4);
+        v[k] = *(const v4f*)(wt + (size_t)r * p.coutPad + (cbBase + cbk) * ROW + c4 * 4);
       }
       asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
 #pragma unroll
@@ -91,13 +100,12 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   constexpr int wavesPerGroup = THREADS / 64;
   const int sib = w.chanBlocks <= wavesPerGroup ? w.chanBlocks : 1;  // siblings side by side (else one wave, all blocks in turn)
   const int slots = wavesPerGroup / sib;
-  const int unitStep = (int)gridDim.x * slots * sib;
+  const int unitStep = nWg * slots * sib;
   // (workgroup ids are dealt round-robin to the 8 XCDs; with taps, numbering them XCD by XCD puts neighbouring
   // pixel blocks, whose taps reach into each other's columns, behind the same L2: the 3x3 layer of the block then
   // fetches 30 MB per launch through the fabric instead of 128 MB.  Without taps nothing is shared and spreading
   // neighbours over the XCDs measured 5% faster.)
-  const int wg = TAPS ? xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x) : (int)blockIdx.x;
-  int unit = ((wave / sib) * (int)gridDim.x + wg) * sib + (wave % sib);
+  int unit = ((wave / sib) * nWg + wg) * sib + (wave % sib);
   if (wave >= slots * sib || unit >= w.nUnits) return;
 
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, (int)w.inBytes, 0x00020000);
@@ -228,15 +236,16 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
 
     // ---- stores of the finished unit (the next unit's first three groups are already in flight)
     const int mo = pb * 32 + l32;
-    if (p.outBytes != 0 && (cb + 1) * ROW <= p.Cout) {
+    const int cbOut = cbBase + cb;  // the channel block's place in the whole bank
+    if (p.outBytes != 0 && (cbOut + 1) * ROW <= p.Cout) {
       // whole channel blocks inside the tensor: straight-line stores through a buffer descriptor
       int n, q;
       p.byQ.divmod(mo < p.M ? mo : 0, &n, &q);
       const unsigned vo = mo < p.M ? (unsigned)(n * p.outImg + out_pixel_offset(p, q) + 4 * kh * p.outPlane) * 4u : kOutside;
 #pragma unroll
       for (int a = 0; a < WA; ++a)
-        store_block(acc[a], orsrc, vo, (cb * ROW + a * 32) * plane, plane, p.alpha, p.beta,
-                    bias ? bias + cb * ROW + a * 32 : nullptr, kh);
+        store_block(acc[a], orsrc, vo, (cbOut * ROW + a * 32) * plane, plane, p.alpha, p.beta,
+                    bias ? bias + cbOut * ROW + a * 32 : nullptr, kh);
     } else if (mo < p.M) {
       int n, q;
       p.byQ.divmod(mo, &n, &q);
@@ -245,7 +254,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
       for (int a = 0; a < WA; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int co = cb * ROW + a * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
+          const int co = cbOut * ROW + a * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
           if (co < p.Cout) {
             float v = p.alpha * acc[a][r];
             if (p.beta != 0.f) v = fmaf(p.beta, o[(size_t)co * p.outPlane], v);
@@ -307,14 +316,26 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
   *handled = 0;
   if (tunable("conv_no_ws", 0)) return MCN_SUCCESS;
   if (p.Cin % (2 * kDepth) != 0 || p.R % (8 * kDepth) != 0 || p.T > kMaxTapsWs || p.coutPad % 32 != 0) return MCN_SUCCESS;
-  const size_t lds = (size_t)p.R * p.coutPad * sizeof(float);
-  if (lds > 150 * 1024) return MCN_SUCCESS;
+  // the bank, or the smallest power-of-two number of slices of it (each a multiple of 32 output channels), in 150 KB
+  const int maxSlices = std::max(1, tunable("conv_ws_max_slices", 8));
+  int slices = 1;
+  while (slices <= maxSlices && ((size_t)p.R * (p.coutPad / slices) * sizeof(float) > 150 * 1024 || p.coutPad % (32 * slices) != 0)) {
+    if (p.coutPad % (32 * slices * 2) != 0) return MCN_SUCCESS;
+    slices *= 2;
+  }
+  if (slices > maxSlices) return MCN_SUCCESS;
+  // every slice gathers all the pixels again: with a strided gather (half of each line fetched unused) the tiled
+  // kernel, which gathers once, is the faster one
+  if (slices > 1 && (p.sy > 1 || p.sx > 1) && !tunable("conv_ws_sliced_strided", 0)) return MCN_SUCCESS;
+  const int coutSlice = p.coutPad / slices;
+  const size_t lds = (size_t)p.R * coutSlice * sizeof(float);
   // byte offsets into the gathered tensor must stay below the "outside" offset
   const long long inBytes = ((long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW) * 4;
   if (inBytes >= (long long)kOutside) return MCN_SUCCESS;
 
   int cus = mcn_device_compute_units();
   if (cus <= 0) cus = 256;
+  if (cus % slices != 0) return MCN_SUCCESS;  // (every slice gets the same number of workgroups)
   const bool twoFit = lds <= 78 * 1024;  // two workgroups per CU fit the 160 KB
   const long long simds = (long long)cus * 4;
   const long long pixelBlocks = ((long long)p.M + 31) / 32;
@@ -326,7 +347,7 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
   if (WA != 1 && WA != 2 && WA != 4) {
     double best = 0;
     for (int cand : {4, 2, 1}) {
-      if (p.coutPad % (32 * cand) != 0) continue;
+      if (coutSlice % (32 * cand) != 0) continue;
       const long long units = pixelBlocks * (p.coutPad / (32 * cand));
       const double balance = (double)units / (double)(((units + simds - 1) / simds) * simds);
       const double issue = cand == 4 ? 0.96 : (cand == 2 ? 0.94 : 0.90);
@@ -336,12 +357,13 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
       }
     }
   }
-  if (p.coutPad % (32 * WA) != 0) return MCN_SUCCESS;
+  if (coutSlice % (32 * WA) != 0) return MCN_SUCCESS;
   WsP w;
-  w.chanBlocks = p.coutPad / (32 * WA);
-  const long long units = pixelBlocks * w.chanBlocks;
-  // too little work to keep every SIMD busy: leave it to the tiled kernel
-  if (units >= (1ll << 30) || units < (minUnits > 0 ? (long long)minUnits : simds * 2)) return MCN_SUCCESS;
+  w.slices = slices;
+  w.chanBlocks = coutSlice / (32 * WA);
+  const long long units = pixelBlocks * w.chanBlocks;  // per slice
+  // too little work to occupy even half of the SIMDs: leave it to the tiled kernel, which can split its reduction
+  if (units >= (1ll << 30) || units * slices < (minUnits > 0 ? (long long)minUnits : simds / 2)) return MCN_SUCCESS;
   w.nUnits = (int)units;
   w.groups = p.R / (2 * kDepth);
   w.groupsPerTap = p.Cin / (2 * kDepth);

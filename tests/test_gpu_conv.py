@@ -207,6 +207,11 @@ WS_CASES = [  # (xshape, fshape, stride, pad, dilate): reduction rows a multiple
     ((12, 12, 64, 4), (2, 2, 64, 16), 1, (1, 0, 0, 1), 1),
     ((10, 9, 64, 3), (1, 1, 64, 128), 1, 0, 1),          # wide enough for the 128-channel units
     ((56, 56, 64, 3), (1, 1, 64, 64), 1, 0, 1),          # several units per wavefront: the load stream crosses units
+    # banks larger than LDS, cut into slices of output channels (one slice per workgroup)
+    ((28, 28, 128, 2), (1, 1, 128, 512), 1, 0, 1),       # 2 slices forward; backward-data (512 -> 128) 2 slices too
+    ((14, 14, 256, 3), (1, 1, 256, 1000), 1, 0, 1),      # 8 slices, output channels not a multiple of the slice
+    ((14, 13, 128, 3), (3, 3, 128, 128), 1, 1, 1),       # 3x3: 4 slices of 32 channels
+    ((15, 14, 64, 2), (3, 3, 64, 192), 2, 1, 1),         # strided, sliced
 ]
 
 
@@ -223,6 +228,7 @@ def test_weights_stationary_kernel(capi, ob, xs, fs, stride, pad, dilate, wa):
     cg = capi.conv_geom(xs, fs, stride, pad, dilate)
     capi.set_tunable("conv_ws_min_units", 1)
     capi.set_tunable("conv_ws_wa", wa)
+    capi.set_tunable("conv_ws_sliced_strided", 1)   # (by default a sliced bank is not used for a strided gather)
     try:
         capi.profile_begin("conv_ws_mfma")
         y = capi.conv_forward(capi.to_device(x), capi.to_device(f), capi.to_device(b), cg)
@@ -233,17 +239,24 @@ def test_weights_stationary_kernel(capi, ob, xs, fs, stride, pad, dilate, wa):
     finally:
         capi.set_tunable("conv_ws_min_units", 0)
         capi.set_tunable("conv_ws_wa", 0)
+        capi.set_tunable("conv_ws_sliced_strided", 0)
     strided = np.any(np.atleast_1d(stride) != 1)
 
     def eligible(cin, cout):
         """The kernel's own admission rule: reduction channels a multiple of 16 and rows a multiple of 64, the
-        packed bank (padded to the channel tile) within 150 KB of LDS, the padded channel count a whole number
-        of units."""
+        packed bank (padded to the channel tile) -- or one of 2, 4 or 8 equal slices of its output channels, each a
+        multiple of 32 -- within 150 KB of LDS, a slice a whole number of units."""
         taps = fs[0] * fs[1]
         tile = 128 if cout > 64 else (64 if cout > 32 else 32)
         padded = -(-cout // tile) * tile
-        return (cin % 16 == 0 and (taps * cin) % 64 == 0 and taps * cin * padded * 4 <= 150 * 1024 and
-                (wa == 0 or padded % (32 * wa) == 0))
+        if cin % 16 != 0 or (taps * cin) % 64 != 0:
+            return False
+        for slices in (1, 2, 4, 8):
+            if padded % (32 * slices) != 0:
+                return False
+            if taps * cin * (padded // slices) * 4 <= 150 * 1024:
+                return wa == 0 or (padded // slices) % (32 * wa) == 0
+        return False
 
     # the kernel under test really ran (a strided layer's backward-data product is one launch per stride class
     # whose tap subset is eligible, so only a lower bound is fixed there)
@@ -253,6 +266,24 @@ def test_weights_stationary_kernel(capi, ob, xs, fs, stride, pad, dilate, wa):
         assert launches == int(eligible(xs[2], fs[3])) + int(eligible(fs[3], xs[2]))
     assert rel_max(capi.to_host(y), want) < 2e-4
     assert rel_max(capi.to_host(dx), ob.conv_backward(x, f, dy, g, want=(True, False, False))[0]) < 2e-4
+
+
+def test_sliced_bank_not_used_for_strided_gather(capi, ob):
+    """A bank cut into slices makes every slice gather the pixels again; for a strided forward gather the tiled
+    kernel is chosen instead (same result either way)."""
+    xs, fs = (15, 14, 64, 2), (3, 3, 64, 192)
+    r = np.random.default_rng(5)
+    x, f = F(r.standard_normal(xs)), F(r.standard_normal(fs) * 0.2)
+    cg = capi.conv_geom(xs, fs, 2, 1, 1)
+    capi.set_tunable("conv_ws_min_units", 1)
+    try:
+        capi.profile_begin("conv_ws_mfma")
+        y = capi.conv_forward(capi.to_device(x), capi.to_device(f), None, cg)
+        launches, _ = capi.profile_end()
+    finally:
+        capi.set_tunable("conv_ws_min_units", 0)
+    assert launches == 0
+    assert rel_max(capi.to_host(y), ob.conv_forward(x, f, None, ob.conv_geom(xs, fs, 2, 1, 1))) < 2e-4
 
 
 @pytest.mark.parametrize("with_bias", [False, True])
