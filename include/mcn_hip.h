@@ -319,6 +319,33 @@ MCN_API int mcn_sgd_momentum(mcn_stream_t stream, float* value, float* state, co
 /* y[i] = value   (bits/impl/copy_gpu.cu:17-33 fill) */
 MCN_API int mcn_fill(mcn_stream_t stream, float* y, float value, size_t n);
 
+/* ------------------------------------------------------------------------------------------------
+ * double precision -- the operators' VLDT_Double instantiation (bits/impl/dispatcher.hpp:60-98 switches on the
+ * tensors' data type; bits/nnconv.cu:444-469, bits/nnbnorm.cu:388-442, bits/nnpooling.cu:270-282 instantiate
+ * every product for float and double).  Same arguments and meaning as the single-precision calls above; general
+ * kernels (any geometry, one accumulator per output element), not tuned ones.  Pooling results have the bits of
+ * the reference's sequential CPU loops.  The convolution calls need no workspace; the batch-normalisation calls
+ * need 2*C doubles of workspace only when `moments` is NULL.
+ * ---------------------------------------------------------------------------------------------- */
+MCN_API int mcn_conv_forward_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* y, double outMult, const double* x,
+                                 double inMult, const double* filters, const double* bias);
+MCN_API int mcn_conv_backward_data_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* derInput, const double* filters,
+                                       const double* derOutput);
+MCN_API int mcn_conv_backward_filter_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* derFilters, const double* x,
+                                         const double* derOutput);
+MCN_API int mcn_conv_backward_bias_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* derBias,
+                                       const double* derOutput);
+MCN_API int mcn_bnorm_forward_f64(mcn_stream_t stream, double* y, double* moments, const double* x,
+                                  const double* multipliers, const double* biases, int H, int W, int C, int N,
+                                  double epsilon, int givenMoments, void* workspace, size_t workspaceBytes);
+MCN_API int mcn_bnorm_backward_f64(mcn_stream_t stream, double* derInput, double* derMultipliers, double* derBiases,
+                                   double* moments, const double* x, const double* multipliers, const double* derOutput,
+                                   int H, int W, int C, int N, double epsilon, int givenMoments, void* workspace,
+                                   size_t workspaceBytes);
+MCN_API int mcn_pool_forward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* y, const double* x);
+MCN_API int mcn_pool_backward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* derInput, const double* x,
+                                  const double* derOutput, int accumulate);
+
 #ifdef __cplusplus
 }
 #endif

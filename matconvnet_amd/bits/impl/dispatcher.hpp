@@ -1,7 +1,9 @@
 // Picks the back-end of an operator call from its tensor arguments.  Same rule as the reference
 // (matlab/src/bits/impl/dispatcher.hpp:30-53): the LAST non-null tensor argument decides device and
-// element type.  This library holds one back-end only -- single precision on the HIP device; any other
-// combination is reported as VLE_Unsupported with a message instead of silently running elsewhere.
+// element type.  This library holds one back-end only -- the HIP device, single precision everywhere and double
+// precision for the three operators the reference instantiates for both (convolution, batch normalisation,
+// pooling); any other combination is reported as VLE_Unsupported with a message instead of silently running
+// elsewhere.
 #ifndef MCN_AMD_BITS_IMPL_DISPATCHER_HPP
 #define MCN_AMD_BITS_IMPL_DISPATCHER_HPP
 
@@ -50,6 +52,17 @@ inline ErrorCode requireHipFloat(Context& context, tensor_type const& tt, char c
   if (tt.dataType != VLDT_Float)
     return context.setError(VLE_Unsupported, (std::string(op) + ": only single precision is implemented on the HIP device").c_str());
   return VLE_Success;
+}
+
+// The same for operators that also have double precision kernels; *isDouble tells which to call.
+inline ErrorCode requireHip(Context& context, tensor_type const& tt, char const* op, bool* isDouble) {
+  *isDouble = false;
+  if (tt.deviceType != VLDT_GPU) return requireHipFloat(context, tt, op);
+  if (tt.dataType == VLDT_Double) {
+    *isDouble = true;
+    return VLE_Success;
+  }
+  return requireHipFloat(context, tt, op);
 }
 
 // Turns a C-ABI return code into a vl::ErrorCode recorded in the context (codes are numerically equal).

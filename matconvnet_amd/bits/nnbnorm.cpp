@@ -35,11 +35,22 @@ ErrorCode forwardAny(BatchNorm& op, char const* name, Tensor& output, Tensor con
                      Tensor const& multiplier, Tensor const& bias, bool given) {
   Context& context = op.context;
   tensor_type tt = findTensorType(output, moment, input, multiplier, bias);
-  ErrorCode e = requireHipFloat(context, tt, name);
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, name, &isDouble);
   if (e != VLE_Success) return e;
   if (!output || !input || !bias) return context.setError(VLE_IllegalArgument, (std::string(name) + ": OUTPUT, INPUT and BIASES are required").c_str());
   Extents x = extentsOf(input);
   if ((e = checkParameters(context, name, x, multiplier, bias, moment, given)) != VLE_Success) return e;
+  if (isDouble) {
+    const size_t need = moment ? 0 : 2 * (size_t)x.C * sizeof(double);
+    void* scratch = need ? context.getWorkspace(VLDT_GPU, need) : NULL;
+    if (need && !scratch) return context.getLastError();
+    int rc64 = mcn_bnorm_forward_f64(context.getHipHelper().getStream(), (double*)output.getMemory(),
+                                     (double*)const_cast<void*>(moment.getMemory()), (double const*)input.getMemory(),
+                                     (double const*)multiplier.getMemory(), (double const*)bias.getMemory(), x.H, x.W, x.C,
+                                     x.N, op.epsilon, given ? 1 : 0, scratch, need);
+    return fromAbi(context, rc64, name);
+  }
   const size_t bytes = mcn_bnorm_workspace_bytes(x.H, x.W, x.C, x.N);
   void* ws = bytes ? context.getWorkspace(VLDT_GPU, bytes) : NULL;
   if (bytes && !ws) return context.getLastError();
@@ -55,7 +66,8 @@ ErrorCode backwardAny(BatchNorm& op, char const* name, Tensor& derInput, Tensor&
                       Tensor const& derOutput, bool given) {
   Context& context = op.context;
   tensor_type tt = findTensorType(derInput, derMultiplier, derBias, moment, input, multiplier, bias, derOutput);
-  ErrorCode e = requireHipFloat(context, tt, name);
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, name, &isDouble);
   if (e != VLE_Success) return e;
   if (!derInput || !derMultiplier || !derBias || !input || !derOutput)
     return context.setError(VLE_IllegalArgument, (std::string(name) + ": DERINPUT, DERMULTIPLIERS, DERBIASES, INPUT and DEROUTPUT are required").c_str());
@@ -63,6 +75,17 @@ ErrorCode backwardAny(BatchNorm& op, char const* name, Tensor& derInput, Tensor&
   if ((e = checkParameters(context, name, x, multiplier, bias, moment, given)) != VLE_Success) return e;
   if (derOutput.getNumElements() != input.getNumElements() || derInput.getNumElements() != input.getNumElements())
     return context.setError(VLE_IllegalArgument, (std::string(name) + ": DEROUTPUT and DERINPUT must have the size of INPUT").c_str());
+  if (isDouble) {
+    const size_t need = moment ? 0 : 2 * (size_t)x.C * sizeof(double);
+    void* scratch = need ? context.getWorkspace(VLDT_GPU, need) : NULL;
+    if (need && !scratch) return context.getLastError();
+    int rc64 = mcn_bnorm_backward_f64(context.getHipHelper().getStream(), (double*)derInput.getMemory(),
+                                      (double*)derMultiplier.getMemory(), (double*)derBias.getMemory(),
+                                      (double*)const_cast<void*>(moment.getMemory()), (double const*)input.getMemory(),
+                                      (double const*)multiplier.getMemory(), (double const*)derOutput.getMemory(), x.H,
+                                      x.W, x.C, x.N, op.epsilon, given ? 1 : 0, scratch, need);
+    return fromAbi(context, rc64, name);
+  }
   const size_t bytes = mcn_bnorm_workspace_bytes(x.H, x.W, x.C, x.N);
   void* ws = bytes ? context.getWorkspace(VLDT_GPU, bytes) : NULL;
   if (bytes && !ws) return context.getLastError();

@@ -41,7 +41,8 @@ bool scratch(Context& context, mcn_conv_geom const& g, int product, void** ws, s
 ErrorCode Convolution::forward(Tensor& output, double outputMult, Tensor const& input, double inputMult,
                                Tensor const& filter, Tensor const& bias) {
   tensor_type tt = findTensorType(output, input, filter, bias);
-  ErrorCode e = requireHipFloat(context, tt, "Convolution::forward");
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, "Convolution::forward", &isDouble);
   if (e != VLE_Success) return e;
   if (!output || !input || !filter)
     return context.setError(VLE_IllegalArgument, "Convolution::forward: OUTPUT, INPUT and FILTER are required");
@@ -54,6 +55,12 @@ ErrorCode Convolution::forward(Tensor& output, double outputMult, Tensor const& 
     return context.setError(VLE_IllegalArgument, "Convolution::forward: OUTPUT dimensions are incompatible with X and FILTERS");
   if (bias && bias.getNumElements() != filter.getSize())
     return context.setError(VLE_IllegalArgument, "Convolution::forward: the number of elements of BIASES is not the number of filters");
+  if (isDouble) {
+    rc = mcn_conv_forward_f64(context.getHipHelper().getStream(), &g, (double*)output.getMemory(), outputMult,
+                              (double const*)input.getMemory(), inputMult, (double const*)filter.getMemory(),
+                              (double const*)bias.getMemory());
+    return fromAbi(context, rc, "Convolution::forward");
+  }
   void* ws;
   size_t bytes;
   if (!scratch(context, g, MCN_CONV_FORWARD, &ws, &bytes)) return context.getLastError();
@@ -122,9 +129,12 @@ ErrorCode Convolution::backward(Tensor& derInput, Tensor& derFilter, Tensor& der
 ErrorCode Convolution::backwardAccumulate(Tensor& derInput, double derInputMult, Tensor& derFilter, Tensor& derBias,
                                           Tensor const& input, Tensor const& filter, Tensor const& derOutput) {
   tensor_type tt = findTensorType(derInput, derFilter, derBias, input, filter, derOutput);
-  ErrorCode e = requireHipFloat(context, tt, "Convolution::backward");
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, "Convolution::backward", &isDouble);
   if (e != VLE_Success) return e;
   if (!derOutput) return context.setError(VLE_IllegalArgument, "Convolution::backward: DEROUTPUT is required");
+  if (isDouble && derInputMult != 0)
+    return context.setError(VLE_Unsupported, "Convolution::backwardAccumulate: accumulation is implemented in single precision only");
   void* stream = context.getHipHelper().getStream();
   void* ws;
   size_t bytes;
@@ -137,9 +147,14 @@ ErrorCode Convolution::backwardAccumulate(Tensor& derInput, double derInputMult,
     mcn_conv_geom g = geometry(plain, derOutput, unit);
     if (derBias.getNumElements() != derOutput.getDepth())
       return context.setError(VLE_IllegalArgument, "Convolution::backward: DERBIASES has the wrong number of elements");
+    if (isDouble) {
+      rc = mcn_conv_backward_bias_f64(stream, &g, (double*)derBias.getMemory(), (double const*)derOutput.getMemory());
+      if (rc) return fromAbi(context, rc, "Convolution::backward");
+    } else {
     if (!scratch(context, g, MCN_CONV_BACKWARD_BIAS, &ws, &bytes)) return context.getLastError();
     rc = mcn_conv_backward_bias(stream, &g, (float*)derBias.getMemory(), (float const*)derOutput.getMemory(), ws, bytes);
     if (rc) return fromAbi(context, rc, "Convolution::backward");
+    }
   }
 
   if (derInput) {
@@ -151,10 +166,15 @@ ErrorCode Convolution::backwardAccumulate(Tensor& derInput, double derInputMult,
     if ((int)derOutput.getHeight() != oh || (int)derOutput.getWidth() != ow || derOutput.getDepth() != filter.getSize() ||
         derOutput.getSize() != derInput.getSize())
       return context.setError(VLE_IllegalArgument, "Convolution::backward: DEROUTPUT dimensions are incompatible with X and FILTERS");
-    if (!scratch(context, g, MCN_CONV_BACKWARD_DATA, &ws, &bytes)) return context.getLastError();
-    rc = mcn_conv_backward_data_packed(stream, &g, (float*)derInput.getMemory(), (float)derInputMult,
-                                       (float const*)filter.getMemory(), packedBackward, packedBackwardBytes,
-                                       (float const*)derOutput.getMemory(), ws, bytes);
+    if (isDouble) {
+      rc = mcn_conv_backward_data_f64(stream, &g, (double*)derInput.getMemory(), (double const*)filter.getMemory(),
+                                      (double const*)derOutput.getMemory());
+    } else {
+      if (!scratch(context, g, MCN_CONV_BACKWARD_DATA, &ws, &bytes)) return context.getLastError();
+      rc = mcn_conv_backward_data_packed(stream, &g, (float*)derInput.getMemory(), (float)derInputMult,
+                                         (float const*)filter.getMemory(), packedBackward, packedBackwardBytes,
+                                         (float const*)derOutput.getMemory(), ws, bytes);
+    }
     if (rc) return fromAbi(context, rc, "Convolution::backward");
   }
 
@@ -167,9 +187,14 @@ ErrorCode Convolution::backwardAccumulate(Tensor& derInput, double derInputMult,
     if ((int)derOutput.getHeight() != oh || (int)derOutput.getWidth() != ow || derOutput.getDepth() != derFilter.getSize() ||
         derOutput.getSize() != input.getSize())
       return context.setError(VLE_IllegalArgument, "Convolution::backward: DEROUTPUT dimensions are incompatible with X and FILTERS");
-    if (!scratch(context, g, MCN_CONV_BACKWARD_FILTER, &ws, &bytes)) return context.getLastError();
-    rc = mcn_conv_backward_filter(stream, &g, (float*)derFilter.getMemory(), (float const*)input.getMemory(),
-                                  (float const*)derOutput.getMemory(), ws, bytes);
+    if (isDouble) {
+      rc = mcn_conv_backward_filter_f64(stream, &g, (double*)derFilter.getMemory(), (double const*)input.getMemory(),
+                                        (double const*)derOutput.getMemory());
+    } else {
+      if (!scratch(context, g, MCN_CONV_BACKWARD_FILTER, &ws, &bytes)) return context.getLastError();
+      rc = mcn_conv_backward_filter(stream, &g, (float*)derFilter.getMemory(), (float const*)input.getMemory(),
+                                    (float const*)derOutput.getMemory(), ws, bytes);
+    }
     if (rc) return fromAbi(context, rc, "Convolution::backward");
   }
   return VLE_Success;

@@ -39,14 +39,18 @@ ErrorCode backwardAny(Pooling& op, char const* name, Tensor& derInput, Tensor co
                       int accumulate) {
   Context& context = op.context;
   tensor_type tt = findTensorType(derInput, input, derOutput);
-  ErrorCode e = requireHipFloat(context, tt, name);
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, name, &isDouble);
   if (e != VLE_Success) return e;
   if (!derInput || !derOutput || (op.method == Pooling::Max && !input))
     return context.setError(VLE_IllegalArgument, (std::string(name) + ": DERINPUT, INPUT and DEROUTPUT are required").c_str());
   mcn_pool_geom g = geometry(op, derInput);
   if ((e = checkOutput(context, name, g, derOutput, derInput)) != VLE_Success) return e;
-  int rc = mcn_pool_backward(context.getHipHelper().getStream(), &g, (float*)derInput.getMemory(),
-                             (float const*)input.getMemory(), (float const*)derOutput.getMemory(), accumulate);
+  int rc = isDouble ? mcn_pool_backward_f64(context.getHipHelper().getStream(), &g, (double*)derInput.getMemory(),
+                                            (double const*)input.getMemory(), (double const*)derOutput.getMemory(),
+                                            accumulate)
+                    : mcn_pool_backward(context.getHipHelper().getStream(), &g, (float*)derInput.getMemory(),
+                                        (float const*)input.getMemory(), (float const*)derOutput.getMemory(), accumulate);
   return fromAbi(context, rc, name);
 }
 
@@ -54,13 +58,16 @@ ErrorCode backwardAny(Pooling& op, char const* name, Tensor& derInput, Tensor co
 
 ErrorCode Pooling::forward(Tensor& output, Tensor const& input) {
   tensor_type tt = findTensorType(output, input);
-  ErrorCode e = requireHipFloat(context, tt, "Pooling::forward");
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, "Pooling::forward", &isDouble);
   if (e != VLE_Success) return e;
   if (!output || !input) return context.setError(VLE_IllegalArgument, "Pooling::forward: OUTPUT and INPUT are required");
   mcn_pool_geom g = geometry(*this, input);
   if ((e = checkOutput(context, "Pooling::forward", g, output, input)) != VLE_Success) return e;
-  int rc = mcn_pool_forward(context.getHipHelper().getStream(), &g, (float*)output.getMemory(),
-                            (float const*)input.getMemory());
+  int rc = isDouble ? mcn_pool_forward_f64(context.getHipHelper().getStream(), &g, (double*)output.getMemory(),
+                                           (double const*)input.getMemory())
+                    : mcn_pool_forward(context.getHipHelper().getStream(), &g, (float*)output.getMemory(),
+                                       (float const*)input.getMemory());
   return fromAbi(context, rc, "Pooling::forward");
 }
 

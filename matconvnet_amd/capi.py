@@ -84,6 +84,14 @@ PROTOTYPES = {
     "mcn_relu_backward": (_i, [_vp, _vp, _vp, _vp, _sz]),
     "mcn_add": (_i, [_vp, _vp, _vp, _vp, _sz]),
     "mcn_fill": (_i, [_vp, _vp, _f, _sz]),
+    "mcn_conv_forward_f64": (_i, [_vp, C.POINTER(ConvGeom), _vp, _d, _vp, _d, _vp, _vp]),
+    "mcn_conv_backward_data_f64": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp]),
+    "mcn_conv_backward_filter_f64": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp]),
+    "mcn_conv_backward_bias_f64": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp]),
+    "mcn_bnorm_forward_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
+    "mcn_bnorm_backward_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
+    "mcn_pool_forward_f64": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp]),
+    "mcn_pool_backward_f64": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp, _vp, _i]),
 }
 
 _lib = None
@@ -183,10 +191,11 @@ def _torch():
     return torch
 
 
-def to_device(a):
-    """numpy (H,W,C,N) array in any order -> contiguous float32 CUDA tensor of shape reversed(a.shape)."""
+def to_device(a, dtype=np.float32):
+    """numpy (H,W,C,N) array in any order -> contiguous CUDA tensor (float32, or float64 on request) of shape
+    reversed(a.shape)."""
     torch = _torch()
-    f = np.asfortranarray(a, dtype=np.float32)
+    f = np.asfortranarray(a, dtype=dtype)
     return torch.from_numpy(np.ascontiguousarray(f.T)).cuda()
 
 
@@ -196,13 +205,24 @@ def to_host(t, dtype=None):
     return np.asfortranarray(a, dtype=dtype or a.dtype)
 
 
-def empty(mshape, fill=None):
-    """Device buffer for a MATLAB-shaped array (H,W,C,N,...)."""
+def empty(mshape, fill=None, like=None):
+    """Device buffer for a MATLAB-shaped array (H,W,C,N,...), float32 or of the data type of `like`."""
     torch = _torch()
     shape = tuple(reversed([int(s) for s in mshape]))
+    dtype = like.dtype if like is not None else torch.float32
     if fill is None:
-        return torch.empty(shape, dtype=torch.float32, device="cuda")
-    return torch.full(shape, float(fill), dtype=torch.float32, device="cuda")
+        return torch.empty(shape, dtype=dtype, device="cuda")
+    return torch.full(shape, float(fill), dtype=dtype, device="cuda")
+
+
+def _is64(*tensors):
+    """True when the tensors are double precision (all of them: mixed types are refused, as
+    vl::impl::check_tensor_compatibility does, bits/data.hpp:260-266)."""
+    torch = _torch()
+    kinds = {t.dtype for t in tensors if t is not None}
+    if len(kinds) > 1:
+        raise TypeError("tensors of different data types: %s" % sorted(str(k) for k in kinds))
+    return kinds == {torch.float64}
 
 
 def ptr(t):
@@ -239,7 +259,10 @@ _ws = Workspace()
 def conv_forward(x, f, b, g, y=None, out_mult=0.0, in_mult=1.0, ws=None):
     ws = ws or _ws
     if y is None:
-        y = empty(conv_out_shape(g))
+        y = empty(conv_out_shape(g), like=x)
+    if _is64(x, f, b, y):
+        check(lib().mcn_conv_forward_f64(stream(), C.byref(g), ptr(y), out_mult, ptr(x), in_mult, ptr(f), ptr(b)))
+        return y
     wp, wn = ws.get(lib().mcn_conv_workspace_bytes(C.byref(g), CONV_FORWARD))
     check(lib().mcn_conv_forward(stream(), C.byref(g), ptr(y), out_mult, ptr(x), in_mult, ptr(f), ptr(b), wp, wn))
     return y
@@ -249,6 +272,17 @@ def conv_backward(x, f, dy, g, want=(True, True, True), ws=None):
     ws = ws or _ws
     L = lib()
     dx = df = db = None
+    if _is64(x, f, dy):
+        if want[0]:
+            dx = empty((g.H, g.W, g.C, g.N), like=dy)
+            check(L.mcn_conv_backward_data_f64(stream(), C.byref(g), ptr(dx), ptr(f), ptr(dy)))
+        if want[1]:
+            df = empty((g.FH, g.FW, g.FC, g.K), like=dy)
+            check(L.mcn_conv_backward_filter_f64(stream(), C.byref(g), ptr(df), ptr(x), ptr(dy)))
+        if want[2]:
+            db = empty((g.K,), like=dy)
+            check(L.mcn_conv_backward_bias_f64(stream(), C.byref(g), ptr(db), ptr(dy)))
+        return dx, df, db
     if want[0]:
         dx = empty((g.H, g.W, g.C, g.N))
         wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_DATA))
@@ -382,9 +416,13 @@ def _hwcn(t):
 def bnorm_forward(x, g, b, eps=1e-4, moments=None, ws=None):
     ws = ws or _ws
     H, W, Cc, N = _hwcn(x)
-    y = empty((H, W, Cc, N))
+    y = empty((H, W, Cc, N), like=x)
     given = moments is not None
-    mom = moments if given else empty((Cc, 2))
+    mom = moments if given else empty((Cc, 2), like=x)
+    if _is64(x, g, b, moments):
+        check(lib().mcn_bnorm_forward_f64(stream(), ptr(y), ptr(mom), ptr(x), ptr(g), ptr(b), H, W, Cc, N, eps, int(given),
+                                          None, 0))
+        return y, mom
     wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
     check(lib().mcn_bnorm_forward(stream(), ptr(y), ptr(mom), ptr(x), ptr(g), ptr(b), H, W, Cc, N, eps, int(given), wp, wn))
     return y, mom
@@ -404,11 +442,16 @@ def bnorm_forward_fused(x, g, b, residual=None, relu=False, eps=1e-4, ws=None):
 def bnorm_backward(x, g, dy, eps=1e-4, moments=None, ws=None, want_moments=True):
     ws = ws or _ws
     H, W, Cc, N = _hwcn(x)
-    dx = empty((H, W, Cc, N))
-    dg = empty((Cc,))
-    db = empty((Cc,))
+    dx = empty((H, W, Cc, N), like=x)
+    dg = empty((Cc,), like=x)
+    db = empty((Cc,), like=x)
     given = moments is not None
-    mom = moments if given else (empty((Cc, 2)) if want_moments else None)
+    mom = moments if given else (empty((Cc, 2), like=x) if want_moments else None)
+    if _is64(x, g, dy, moments):
+        wp, wn = (None, 0) if mom is not None else ws.get(2 * Cc * 8)
+        check(lib().mcn_bnorm_backward_f64(stream(), ptr(dx), ptr(dg), ptr(db), ptr(mom), ptr(x), ptr(g), ptr(dy),
+                                           H, W, Cc, N, eps, int(given), wp, wn))
+        return dx, dg, db, mom
     wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
     check(lib().mcn_bnorm_backward(stream(), ptr(dx), ptr(dg), ptr(db), ptr(mom), ptr(x), ptr(g), ptr(dy),
                                    H, W, Cc, N, eps, int(given), wp, wn))
@@ -441,8 +484,9 @@ def bnorm_backward_masked(x, g, dy, mask_source, moments, eps=1e-4, ws=None):
 
 
 def pool_forward(x, g):
-    y = empty(pool_out_shape(g))
-    check(lib().mcn_pool_forward(stream(), C.byref(g), ptr(y), ptr(x)))
+    y = empty(pool_out_shape(g), like=x)
+    fn = lib().mcn_pool_forward_f64 if _is64(x) else lib().mcn_pool_forward
+    check(fn(stream(), C.byref(g), ptr(y), ptr(x)))
     return y
 
 
@@ -450,8 +494,9 @@ def pool_backward(x, dy, g, dx=None):
     """dx given: accumulate into it (vl::nn::Pooling::backward contract); else a fresh write-only output."""
     acc = dx is not None
     if dx is None:
-        dx = empty((g.H, g.W, g.C, g.N))
-    check(lib().mcn_pool_backward(stream(), C.byref(g), ptr(dx), ptr(x), ptr(dy), int(acc)))
+        dx = empty((g.H, g.W, g.C, g.N), like=dy)
+    fn = lib().mcn_pool_backward_f64 if _is64(x, dy, dx) else lib().mcn_pool_backward
+    check(fn(stream(), C.byref(g), ptr(dx), ptr(x), ptr(dy), int(acc)))
     return dx
 
 

@@ -1,0 +1,495 @@
+// Double precision: the operators' VLDT_Double instantiation (matlab/src/bits/impl/dispatcher.hpp:60-98 switches on
+// the tensors' data type; every operator of the path is instantiated for float and double, e.g.
+// bits/nnconv.cu:444-469, bits/nnbnorm.cu:388-442, bits/nnpooling.cu:270-282).  These are the general kernels --
+// one accumulator per output element, any geometry -- not tuned ones: the measured configurations are all single
+// precision.  Results follow the reference's definitions; pooling keeps the order of its sequential loops, so its
+// results have the same bits as the CPU reference (this file is compiled without floating-point contraction and
+// uses fma() where a fused operation is meant).
+#include "conv_common.hpp"
+
+#include <algorithm>
+
+namespace mcn {
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------
+// convolution (bits/nnconv.cu:71-317 with bits/impl/im2row_cpu.cpp:52-230 folded in)
+// ---------------------------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void conv64_forward(double* __restrict__ y, double outMult, const double* __restrict__ x,
+                                                      double inMult, const double* __restrict__ f,
+                                                      const double* __restrict__ b, ConvP p, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int P = p.outH * p.outW;
+  size_t r = idx;
+  const int q = (int)(r % P);
+  r /= P;
+  const int k = (int)(r % p.K);
+  const int n = (int)(r / p.K);
+  const int ow = q / p.outH, oh = q - ow * p.outH;
+  const int g = k / p.Kg;
+  const double* xn = x + (size_t)p.H * p.W * ((size_t)p.C * n + (size_t)g * p.FC);
+  const double* fk = f + (size_t)p.FH * p.FW * p.FC * k;
+  double acc = 0.0;
+  for (int d = 0; d < p.FC; ++d)
+    for (int j = 0; j < p.FW; ++j) {
+      const int w = ow * p.sx + j * p.dx - p.pl;
+      if ((unsigned)w >= (unsigned)p.W) continue;
+      for (int i = 0; i < p.FH; ++i) {
+        const int h = oh * p.sy + i * p.dy - p.pt;
+        if ((unsigned)h >= (unsigned)p.H) continue;
+        acc = fma(xn[h + p.H * (w + (size_t)p.W * d)], fk[i + p.FH * (j + p.FW * d)], acc);
+      }
+    }
+  double r0 = inMult * acc;
+  if (outMult != 0.0) r0 = fma(outMult, y[idx], r0);
+  if (b) r0 += b[k];
+  y[idx] = r0;
+}
+
+__global__ __launch_bounds__(256) void conv64_backward_data(double* __restrict__ dx, const double* __restrict__ f,
+                                                            const double* __restrict__ dy, ConvP p, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int HW = p.H * p.W;
+  size_t r = idx;
+  const int q = (int)(r % HW);
+  r /= HW;
+  const int c = (int)(r % p.C);
+  const int n = (int)(r / p.C);
+  const int w = q / p.H, h = q - w * p.H;
+  const int g = c / p.FC, d = c - g * p.FC;
+  const int P = p.outH * p.outW;
+  double acc = 0.0;
+  for (int kk = 0; kk < p.Kg; ++kk) {
+    const int k = g * p.Kg + kk;
+    const double* dyk = dy + (size_t)P * ((size_t)p.K * n + k);
+    const double* fk = f + (size_t)p.FH * p.FW * ((size_t)p.FC * k + d);
+    for (int j = 0; j < p.FW; ++j) {
+      const int aw = w + p.pl - j * p.dx;
+      if (aw < 0 || aw % p.sx) continue;
+      const int ow = aw / p.sx;
+      if (ow >= p.outW) continue;
+      for (int i = 0; i < p.FH; ++i) {
+        const int ah = h + p.pt - i * p.dy;
+        if (ah < 0 || ah % p.sy) continue;
+        const int oh = ah / p.sy;
+        if (oh >= p.outH) continue;
+        acc = fma(dyk[oh + p.outH * ow], fk[i + p.FH * j], acc);
+      }
+    }
+  }
+  dx[idx] = acc;
+}
+
+// sum of the four wavefronts' values, in a fixed order, on thread 0
+__device__ __forceinline__ double block_sum(double v, double* lds) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const double s = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+  __syncthreads();
+  return s;
+}
+
+// one workgroup per filter element
+__global__ __launch_bounds__(256) void conv64_backward_filter(double* __restrict__ df, const double* __restrict__ x,
+                                                              const double* __restrict__ dy, ConvP p) {
+  __shared__ double lds[4];
+  size_t r = blockIdx.x;
+  const int i = (int)(r % p.FH);
+  r /= p.FH;
+  const int j = (int)(r % p.FW);
+  r /= p.FW;
+  const int d = (int)(r % p.FC);
+  const int k = (int)(r / p.FC);
+  const int g = k / p.Kg;
+  const int c = g * p.FC + d;
+  const int P = p.outH * p.outW;
+  const long long total = (long long)P * p.N;
+  double acc = 0.0;
+  for (long long m = threadIdx.x; m < total; m += 256) {
+    const int n = (int)(m / P);
+    const int q = (int)(m - (long long)n * P);
+    const int ow = q / p.outH, oh = q - ow * p.outH;
+    const int h = oh * p.sy + i * p.dy - p.pt;
+    const int w = ow * p.sx + j * p.dx - p.pl;
+    if ((unsigned)h < (unsigned)p.H && (unsigned)w < (unsigned)p.W)
+      acc = fma(x[h + p.H * (w + (size_t)p.W * (c + (size_t)p.C * n))], dy[q + (size_t)P * (k + (size_t)p.K * n)], acc);
+  }
+  const double s = block_sum(acc, lds);
+  if (threadIdx.x == 0) df[blockIdx.x] = s;
+}
+
+// one workgroup per filter: db[k] = sum over images and pixels of dy
+__global__ __launch_bounds__(256) void conv64_backward_bias(double* __restrict__ db, const double* __restrict__ dy, int P,
+                                                            int K, int N) {
+  __shared__ double lds[4];
+  const int k = blockIdx.x;
+  double acc = 0.0;
+  for (int n = 0; n < N; ++n) {
+    const double* src = dy + (size_t)P * (k + (size_t)K * n);
+    for (int i = threadIdx.x; i < P; i += 256) acc += src[i];
+  }
+  const double s = block_sum(acc, lds);
+  if (threadIdx.x == 0) db[k] = s;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// batch normalisation (bits/nnbnorm.cu:46-164: compute_moment, compute_ders, compute_ders_and_moments,
+// batch_normalize_forward / _backward)
+// ---------------------------------------------------------------------------------------------------------
+
+// One workgroup per channel.  DERS == false: sums of x and x*x, turned into (mean, sigma) in moments[c], moments[C + c].
+// DERS == true: sums of dy and x*dy (and, unless the moments are given, of x and x*x as well); writes dzdb, dzdg and
+// the moments.
+template <bool DERS, bool GIVEN>
+__global__ __launch_bounds__(256) void bnorm64_sums(double* __restrict__ moments, double* __restrict__ dG,
+                                                    double* __restrict__ dB, const double* __restrict__ x,
+                                                    const double* __restrict__ dy, int WH, int C, int N, double epsilon) {
+  __shared__ double lds[4];
+  const int c = blockIdx.x;
+  double sx = 0.0, sxx = 0.0, sd = 0.0, sxd = 0.0;
+  for (int n = 0; n < N; ++n) {
+    const size_t base = (size_t)WH * (c + (size_t)C * n);
+    for (int i = threadIdx.x; i < WH; i += 256) {
+      const double v = x[base + i];
+      if (!GIVEN) {
+        sx += v;
+        sxx = fma(v, v, sxx);
+      }
+      if (DERS) {
+        const double d = dy[base + i];
+        sd += d;
+        sxd = fma(v, d, sxd);
+      }
+    }
+  }
+  double mean, sigma;
+  const double mass = (double)WH * (double)N;
+  if (GIVEN) {
+    mean = moments[c];
+    sigma = moments[C + c];
+  } else {
+    sx = block_sum(sx, lds);
+    sxx = block_sum(sxx, lds);
+    mean = sx / mass;
+    sigma = sqrt(fmax(0.0, sxx / mass - mean * mean) + epsilon);  // sigma includes epsilon (bits/nnbnorm.cu:65-70)
+  }
+  if (DERS) {
+    sd = block_sum(sd, lds);
+    sxd = block_sum(sxd, lds);
+  }
+  if (threadIdx.x != 0) return;
+  if (!GIVEN) {
+    moments[c] = mean;
+    moments[C + c] = sigma;
+  }
+  if (DERS) {
+    dB[c] = sd;
+    dG[c] = (sxd - mean * sd) / sigma;  // bits/nnbnorm.cu:93-97,128-132
+  }
+}
+
+// y = (g/sigma)*(x - mean) + b, rounded as written  (bits/nnbnorm.cu:192-203)
+__global__ __launch_bounds__(256) void bnorm64_forward_apply(double* __restrict__ y, const double* __restrict__ x,
+                                                             const double* __restrict__ moments,
+                                                             const double* __restrict__ mult, const double* __restrict__ bias,
+                                                             int WH, int C, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int c = (int)((idx / WH) % C);
+  const double G = mult[c] / moments[C + c];
+  y[idx] = G * (x[idx] - moments[c]) + bias[c];
+}
+
+// dzdx = G1*(dzdy - dzdb/m) - G2*(x - mean),  G1 = g/sigma,  G2 = G1*dzdg/(m*sigma)  (bits/nnbnorm.cu:136-164)
+__global__ __launch_bounds__(256) void bnorm64_backward_apply(double* __restrict__ dx, const double* __restrict__ x,
+                                                              const double* __restrict__ dy,
+                                                              const double* __restrict__ moments,
+                                                              const double* __restrict__ mult, const double* __restrict__ dG,
+                                                              const double* __restrict__ dB, int WH, int C, double mass,
+                                                              size_t total) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int c = (int)((idx / WH) % C);
+  const double mean = moments[c], sigma = moments[C + c];
+  const double muz = dB[c] / mass;
+  const double G1 = mult[c] / sigma;
+  const double G2 = G1 * dG[c] / (mass * sigma);
+  dx[idx] = G1 * (dy[idx] - muz) - G2 * (x[idx] - mean);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// pooling (bits/nnpooling.cu:33-237)
+// ---------------------------------------------------------------------------------------------------------
+
+struct Pool64 {
+  int H, W, outH, outW;
+  int poolH, poolW, sy, sx, pt, pl;
+  int accumulate;
+};
+
+// one thread per output: window clipped to the image, columns (slow) then rows (fast); max: first element greater
+// than the running value, which starts at -inf (bits/nnpooling.cu:36-61); average: sum times T(1)/T(area) (:63-96)
+template <bool MAX>
+__global__ __launch_bounds__(256) void pool64_forward(double* __restrict__ y, const double* __restrict__ x, Pool64 p,
+                                                      size_t total) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int P = p.outH * p.outW;
+  const size_t plane = idx / P;
+  const int q = (int)(idx - plane * P);
+  const int ow = q / p.outH, oh = q - ow * p.outH;
+  int h1 = oh * p.sy - p.pt, w1 = ow * p.sx - p.pl;
+  const int h2 = min(h1 + p.poolH, p.H), w2 = min(w1 + p.poolW, p.W);
+  h1 = max(h1, 0);
+  w1 = max(w1, 0);
+  const double* xp = x + plane * (size_t)p.H * p.W;
+  if (MAX) {
+    double best = -__builtin_inf();
+    for (int w = w1; w < w2; ++w)
+      for (int h = h1; h < h2; ++h) {
+        const double v = xp[h + (size_t)p.H * w];
+        if (v > best) best = v;
+      }
+    y[idx] = best;
+  } else {
+    double acc = 0.0;
+    for (int w = w1; w < w2; ++w)
+      for (int h = h1; h < h2; ++h) acc += xp[h + (size_t)p.H * w];
+    y[idx] = acc * (1.0 / (double)((h2 - h1) * (w2 - w1)));
+  }
+}
+
+// One thread per input element: the outputs whose window holds it, columns ascending then rows ascending -- the
+// order in which the reference's loop over outputs adds to it (bits/nnpooling.cu:190-206) -- so the sum has the
+// same bits.  Max: an output counts when this element is its window's winner (first maximum in memory order).
+template <bool MAX>
+__global__ __launch_bounds__(256) void pool64_backward(double* __restrict__ dx, const double* __restrict__ x,
+                                                       const double* __restrict__ dy, Pool64 p, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int HW = p.H * p.W;
+  const size_t plane = idx / HW;
+  const int e = (int)(idx - plane * HW);
+  const int w = e / p.H, h = e - w * p.H;
+  const double* xp = x ? x + plane * (size_t)HW : nullptr;
+  const double* dyp = dy + plane * (size_t)p.outH * p.outW;
+  // outputs o with o*s - pad <= h < o*s - pad + pool
+  const int ohLo = max(0, (h + p.pt - p.poolH + p.sy) / p.sy), ohHi = min(p.outH - 1, (h + p.pt) / p.sy);
+  const int owLo = max(0, (w + p.pl - p.poolW + p.sx) / p.sx), owHi = min(p.outW - 1, (w + p.pl) / p.sx);
+  double acc = p.accumulate ? dx[idx] : 0.0;
+  for (int ow = owLo; ow <= owHi; ++ow)
+    for (int oh = ohLo; oh <= ohHi; ++oh) {
+      int h1 = oh * p.sy - p.pt, w1 = ow * p.sx - p.pl;
+      const int h2 = min(h1 + p.poolH, p.H), w2 = min(w1 + p.poolW, p.W);
+      h1 = max(h1, 0);
+      w1 = max(w1, 0);
+      if (h < h1 || h >= h2 || w < w1 || w >= w2) continue;
+      const double d = dyp[oh + (size_t)p.outH * ow];
+      if (MAX) {
+        double best = -__builtin_inf();
+        int at = -1;
+        for (int ww = w1; ww < w2; ++ww)
+          for (int hh = h1; hh < h2; ++hh) {
+            const double v = xp[hh + (size_t)p.H * ww];
+            if (v > best) {
+              best = v;
+              at = hh + p.H * ww;
+            }
+          }
+        if (at == e) acc += d;
+      } else {
+        acc += d * (1.0 / (double)((h2 - h1) * (w2 - w1)));
+      }
+    }
+  dx[idx] = acc;
+}
+
+int blocks_for(size_t total, const char* who, unsigned* blocks) {
+  const size_t b = (total + 255) / 256;
+  if (b >= (1ull << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
+  *blocks = (unsigned)b;
+  return MCN_SUCCESS;
+}
+
+}  // namespace
+}  // namespace mcn
+
+using namespace mcn;
+
+extern "C" {
+
+int mcn_conv_forward_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* y, double outMult, const double* x,
+                         double inMult, const double* filters, const double* bias) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_forward_f64", &p);
+  if (rc) return rc;
+  const size_t total = (size_t)p.outH * p.outW * p.K * p.N;
+  if (total == 0) return MCN_SUCCESS;
+  if (!y || !x || !filters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_forward_f64: null tensor");
+  unsigned blocks;
+  if ((rc = blocks_for(total, "mcn_conv_forward_f64", &blocks))) return rc;
+  KernelTimer timer("conv64_forward", as_stream(stream));
+  hipLaunchKernelGGL(conv64_forward, dim3(blocks), dim3(256), 0, as_stream(stream), y, outMult, x, inMult, filters, bias, p,
+                     total);
+  return check_launch("mcn_conv_forward_f64");
+}
+
+int mcn_conv_backward_data_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* derInput, const double* filters,
+                               const double* derOutput) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_data_f64", &p);
+  if (rc) return rc;
+  const size_t total = (size_t)p.H * p.W * p.C * p.N;
+  if (total == 0) return MCN_SUCCESS;
+  if (!derInput || !filters || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data_f64: null tensor");
+  unsigned blocks;
+  if ((rc = blocks_for(total, "mcn_conv_backward_data_f64", &blocks))) return rc;
+  KernelTimer timer("conv64_backward_data", as_stream(stream));
+  hipLaunchKernelGGL(conv64_backward_data, dim3(blocks), dim3(256), 0, as_stream(stream), derInput, filters, derOutput, p,
+                     total);
+  return check_launch("mcn_conv_backward_data_f64");
+}
+
+int mcn_conv_backward_filter_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* derFilters, const double* x,
+                                 const double* derOutput) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_filter_f64", &p);
+  if (rc) return rc;
+  if (!derFilters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_f64: null tensor");
+  const size_t total = (size_t)p.FH * p.FW * p.FC * p.K;
+  if ((size_t)p.outH * p.outW * p.N != 0 && (!x || !derOutput))
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_f64: null tensor");
+  KernelTimer timer("conv64_backward_filter", as_stream(stream));
+  hipLaunchKernelGGL(conv64_backward_filter, dim3((unsigned)total), dim3(256), 0, as_stream(stream), derFilters, x, derOutput,
+                     p);
+  return check_launch("mcn_conv_backward_filter_f64");
+}
+
+int mcn_conv_backward_bias_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* derBias, const double* derOutput) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_bias_f64", &p);
+  if (rc) return rc;
+  if (!derBias) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_bias_f64: null tensor");
+  if ((size_t)p.outH * p.outW * p.N != 0 && !derOutput)
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_bias_f64: null tensor");
+  KernelTimer timer("conv64_backward_bias", as_stream(stream));
+  hipLaunchKernelGGL(conv64_backward_bias, dim3((unsigned)p.K), dim3(256), 0, as_stream(stream), derBias, derOutput,
+                     p.outH * p.outW, p.K, p.N);
+  return check_launch("mcn_conv_backward_bias_f64");
+}
+
+int mcn_bnorm_forward_f64(mcn_stream_t stream, double* y, double* moments, const double* x, const double* multipliers,
+                          const double* biases, int H, int W, int C, int N, double epsilon, int givenMoments,
+                          void* workspace, size_t workspaceBytes) {
+  if (H < 0 || W < 0 || C < 0 || N < 0) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_f64: negative tensor extent");
+  if ((long long)H * W >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "mcn_bnorm_forward_f64: plane too large");
+  const size_t total = (size_t)H * W * C * N;
+  if (C == 0) return MCN_SUCCESS;
+  if ((total != 0 && (!y || !x)) || !multipliers || !biases) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_f64: null tensor");
+  if (givenMoments && !moments) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_f64: MOMENTS are required when given");
+  double* mom = moments;
+  if (!mom) {
+    if (!workspace || workspaceBytes < (size_t)2 * C * sizeof(double))
+      return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_f64: workspace too small (%zu < %zu bytes)", workspaceBytes,
+                  (size_t)2 * C * sizeof(double));
+    mom = (double*)workspace;
+  }
+  hipStream_t s = as_stream(stream);
+  if (!givenMoments) {
+    KernelTimer timer("bnorm64_sums", s);
+    hipLaunchKernelGGL((bnorm64_sums<false, false>), dim3((unsigned)C), dim3(256), 0, s, mom, nullptr, nullptr, x, nullptr,
+                       H * W, C, N, epsilon);
+    int rc = check_launch("mcn_bnorm_forward_f64");
+    if (rc) return rc;
+  }
+  if (total == 0) return MCN_SUCCESS;
+  unsigned blocks;
+  int rc = blocks_for(total, "mcn_bnorm_forward_f64", &blocks);
+  if (rc) return rc;
+  KernelTimer timer("bnorm64_forward_apply", s);
+  hipLaunchKernelGGL(bnorm64_forward_apply, dim3(blocks), dim3(256), 0, s, y, x, mom, multipliers, biases, H * W, C, total);
+  return check_launch("mcn_bnorm_forward_f64");
+}
+
+int mcn_bnorm_backward_f64(mcn_stream_t stream, double* derInput, double* derMultipliers, double* derBiases, double* moments,
+                           const double* x, const double* multipliers, const double* derOutput, int H, int W, int C, int N,
+                           double epsilon, int givenMoments, void* workspace, size_t workspaceBytes) {
+  if (H < 0 || W < 0 || C < 0 || N < 0) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_f64: negative tensor extent");
+  if ((long long)H * W >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "mcn_bnorm_backward_f64: plane too large");
+  const size_t total = (size_t)H * W * C * N;
+  if (C == 0) return MCN_SUCCESS;
+  if ((total != 0 && (!derInput || !x || !derOutput)) || !multipliers || !derMultipliers || !derBiases)
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_f64: null tensor");
+  if (givenMoments && !moments) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_f64: MOMENTS are required when given");
+  double* mom = moments;
+  if (!mom) {
+    if (!workspace || workspaceBytes < (size_t)2 * C * sizeof(double))
+      return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_f64: workspace too small (%zu < %zu bytes)", workspaceBytes,
+                  (size_t)2 * C * sizeof(double));
+    mom = (double*)workspace;
+  }
+  hipStream_t s = as_stream(stream);
+  {
+    KernelTimer timer("bnorm64_sums", s);
+    if (givenMoments)
+      hipLaunchKernelGGL((bnorm64_sums<true, true>), dim3((unsigned)C), dim3(256), 0, s, mom, derMultipliers, derBiases, x,
+                         derOutput, H * W, C, N, epsilon);
+    else
+      hipLaunchKernelGGL((bnorm64_sums<true, false>), dim3((unsigned)C), dim3(256), 0, s, mom, derMultipliers, derBiases, x,
+                         derOutput, H * W, C, N, epsilon);
+    int rc = check_launch("mcn_bnorm_backward_f64");
+    if (rc) return rc;
+  }
+  if (total == 0) return MCN_SUCCESS;
+  unsigned blocks;
+  int rc = blocks_for(total, "mcn_bnorm_backward_f64", &blocks);
+  if (rc) return rc;
+  KernelTimer timer("bnorm64_backward_apply", s);
+  hipLaunchKernelGGL(bnorm64_backward_apply, dim3(blocks), dim3(256), 0, s, derInput, x, derOutput, mom, multipliers,
+                     derMultipliers, derBiases, H * W, C, (double)H * W * (double)N, total);
+  return check_launch("mcn_bnorm_backward_f64");
+}
+
+int mcn_pool_forward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* y, const double* x) {
+  int oh = 0, ow = 0;
+  int rc = mcn_pool_output_size(g, &oh, &ow);
+  if (rc) return rc;
+  const size_t total = (size_t)oh * ow * g->C * g->N;
+  if (total == 0) return MCN_SUCCESS;
+  if (!y || !x) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_pool_forward_f64: null tensor");
+  Pool64 p = {g->H, g->W, oh, ow, g->poolH, g->poolW, g->strideY, g->strideX, g->padTop, g->padLeft, 0};
+  unsigned blocks;
+  if ((rc = blocks_for(total, "mcn_pool_forward_f64", &blocks))) return rc;
+  KernelTimer timer("pool64_forward", as_stream(stream));
+  if (g->method == MCN_POOL_MAX)
+    hipLaunchKernelGGL(pool64_forward<true>, dim3(blocks), dim3(256), 0, as_stream(stream), y, x, p, total);
+  else
+    hipLaunchKernelGGL(pool64_forward<false>, dim3(blocks), dim3(256), 0, as_stream(stream), y, x, p, total);
+  return check_launch("mcn_pool_forward_f64");
+}
+
+int mcn_pool_backward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* derInput, const double* x,
+                          const double* derOutput, int accumulate) {
+  int oh = 0, ow = 0;
+  int rc = mcn_pool_output_size(g, &oh, &ow);
+  if (rc) return rc;
+  const size_t total = (size_t)g->H * g->W * g->C * g->N;
+  if (total == 0) return MCN_SUCCESS;
+  const bool isMax = g->method == MCN_POOL_MAX;
+  if (!derInput || !derOutput || (isMax && !x)) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_pool_backward_f64: null tensor");
+  Pool64 p = {g->H, g->W, oh, ow, g->poolH, g->poolW, g->strideY, g->strideX, g->padTop, g->padLeft, accumulate ? 1 : 0};
+  unsigned blocks;
+  if ((rc = blocks_for(total, "mcn_pool_backward_f64", &blocks))) return rc;
+  KernelTimer timer("pool64_backward", as_stream(stream));
+  if (isMax)
+    hipLaunchKernelGGL(pool64_backward<true>, dim3(blocks), dim3(256), 0, as_stream(stream), derInput, x, derOutput, p, total);
+  else
+    hipLaunchKernelGGL(pool64_backward<false>, dim3(blocks), dim3(256), 0, as_stream(stream), derInput, x, derOutput, p, total);
+  return check_launch("mcn_pool_backward_f64");
+}
+
+}  // extern "C"
