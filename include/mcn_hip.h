@@ -345,6 +345,17 @@ MCN_API int mcn_bnorm_backward_f64(mcn_stream_t stream, double* derInput, double
 MCN_API int mcn_pool_forward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* y, const double* x);
 MCN_API int mcn_pool_backward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* derInput, const double* x,
                                   const double* derOutput, int accumulate);
+/* the companions in double: subsampling with bias (bits/nnsubsample.cu:31-216), the per-channel bias add of
+   ConvolutionTranspose (bits/nnconv.cu:369-371), vl_taccum (matlab/src/vl_taccummex.cu:48-113) */
+MCN_API int mcn_subsample_forward_f64(mcn_stream_t stream, double* y, const double* x, const double* bias, int H, int W,
+                                      int C, int N, int strideY, int strideX, int padTop, int padBottom, int padLeft,
+                                      int padRight);
+MCN_API int mcn_subsample_backward_f64(mcn_stream_t stream, double* derInput, const double* derOutput, int H, int W, int C,
+                                       int N, int strideY, int strideX, int padTop, int padBottom, int padLeft,
+                                       int padRight);
+MCN_API int mcn_bias_add_f64(mcn_stream_t stream, double* y, const double* bias, int H, int W, int C, int N);
+MCN_API int mcn_taccum_f64(mcn_stream_t stream, double* y, double alpha, const double* a, double beta, const double* b,
+                           size_t n);
 
 #ifdef __cplusplus
 }

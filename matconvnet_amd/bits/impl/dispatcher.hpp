@@ -1,9 +1,9 @@
 // Picks the back-end of an operator call from its tensor arguments.  Same rule as the reference
 // (matlab/src/bits/impl/dispatcher.hpp:30-53): the LAST non-null tensor argument decides device and
-// element type.  This library holds one back-end only -- the HIP device, single precision everywhere and double
-// precision for the three operators the reference instantiates for both (convolution, batch normalisation,
-// pooling); any other combination is reported as VLE_Unsupported with a message instead of silently running
-// elsewhere.
+// element type.  This library holds one back-end only -- the HIP device, single and double precision for the
+// operators the reference has (the calls it does not have -- fused, packed-ahead, accumulating -- are single
+// precision only); any other combination is reported as VLE_Unsupported with a message instead of silently
+// running elsewhere.
 #ifndef MCN_AMD_BITS_IMPL_DISPATCHER_HPP
 #define MCN_AMD_BITS_IMPL_DISPATCHER_HPP
 

@@ -214,7 +214,8 @@ ConvolutionTranspose::ConvolutionTranspose(Context& context, int upsampleY, int 
 
 ErrorCode ConvolutionTranspose::forward(Tensor& output, Tensor const& input, Tensor const& filter, Tensor const& bias) {
   tensor_type tt = findTensorType(output, input, filter, bias);
-  ErrorCode e = requireHipFloat(context, tt, "ConvolutionTranspose::forward");
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, "ConvolutionTranspose::forward", &isDouble);
   if (e != VLE_Success) return e;
   if (!output || !input || !filter)
     return context.setError(VLE_IllegalArgument, "ConvolutionTranspose::forward: OUTPUT, INPUT and FILTER are required");
@@ -225,8 +226,12 @@ ErrorCode ConvolutionTranspose::forward(Tensor& output, Tensor const& input, Ten
   e = opc.backward(output, null, null, null, filter, input);
   if (e != VLE_Success) return context.passError(e, "ConvolutionTranspose::forward");
   if (bias) {
-    int rc = mcn_bias_add(context.getHipHelper().getStream(), (float*)output.getMemory(), (float const*)bias.getMemory(),
-                          asInt(output.getHeight()), asInt(output.getWidth()), asInt(output.getDepth()), asInt(output.getSize()));
+    int rc = isDouble ? mcn_bias_add_f64(context.getHipHelper().getStream(), (double*)output.getMemory(),
+                                         (double const*)bias.getMemory(), asInt(output.getHeight()), asInt(output.getWidth()),
+                                         asInt(output.getDepth()), asInt(output.getSize()))
+                      : mcn_bias_add(context.getHipHelper().getStream(), (float*)output.getMemory(),
+                                     (float const*)bias.getMemory(), asInt(output.getHeight()), asInt(output.getWidth()),
+                                     asInt(output.getDepth()), asInt(output.getSize()));
     return fromAbi(context, rc, "ConvolutionTranspose::forward");
   }
   return VLE_Success;
@@ -235,7 +240,8 @@ ErrorCode ConvolutionTranspose::forward(Tensor& output, Tensor const& input, Ten
 ErrorCode ConvolutionTranspose::backward(Tensor& derData, Tensor& derFilter, Tensor& derBias, Tensor const& input,
                                          Tensor const& filter, Tensor const& derOutput) {
   tensor_type tt = findTensorType(derData, derFilter, derBias, input, filter, derOutput);
-  ErrorCode e = requireHipFloat(context, tt, "ConvolutionTranspose::backward");
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, "ConvolutionTranspose::backward", &isDouble);
   if (e != VLE_Success) return e;
   if (!derOutput) return context.setError(VLE_IllegalArgument, "ConvolutionTranspose::backward: DEROUTPUT is required");
   Convolution opc(context, upsampleY, upsampleX, cropTop, cropBottom, cropLeft, cropRight, 1, 1);

@@ -29,23 +29,30 @@ bool extentsMatch(Subsample const& op, Tensor const& big, Tensor const& small) {
 
 ErrorCode Subsample::forwardWithBias(Tensor& output, Tensor const& input, Tensor const& biases) {
   tensor_type tt = findTensorType(output, input, biases);
-  ErrorCode e = requireHipFloat(context, tt, "Subsample::forwardWithBias");
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, "Subsample::forwardWithBias", &isDouble);
   if (e != VLE_Success) return e;
   if (!output || !input) return context.setError(VLE_IllegalArgument, "Subsample::forwardWithBias: OUTPUT and INPUT are required");
   if (!extentsMatch(*this, input, output))
     return context.setError(VLE_IllegalArgument, "Subsample::forwardWithBias: OUTPUT dimensions are incompatible with INPUT");
   if (biases && biases.getNumElements() != input.getDepth())
     return context.setError(VLE_IllegalArgument, "Subsample::forwardWithBias: the number of elements of BIASES is not the DATA depth");
-  int rc = mcn_subsample_forward(context.getHipHelper().getStream(), (float*)output.getMemory(), (float const*)input.getMemory(),
-                                 (float const*)biases.getMemory(), asInt(input.getHeight()), asInt(input.getWidth()),
-                                 asInt(input.getDepth()), asInt(input.getSize()), strideY, strideX, padTop, padBottom, padLeft,
-                                 padRight);
+  int rc = isDouble
+               ? mcn_subsample_forward_f64(context.getHipHelper().getStream(), (double*)output.getMemory(),
+                                           (double const*)input.getMemory(), (double const*)biases.getMemory(),
+                                           asInt(input.getHeight()), asInt(input.getWidth()), asInt(input.getDepth()),
+                                           asInt(input.getSize()), strideY, strideX, padTop, padBottom, padLeft, padRight)
+               : mcn_subsample_forward(context.getHipHelper().getStream(), (float*)output.getMemory(),
+                                       (float const*)input.getMemory(), (float const*)biases.getMemory(),
+                                       asInt(input.getHeight()), asInt(input.getWidth()), asInt(input.getDepth()),
+                                       asInt(input.getSize()), strideY, strideX, padTop, padBottom, padLeft, padRight);
   return fromAbi(context, rc, "Subsample::forwardWithBias");
 }
 
 ErrorCode Subsample::backwardWithBias(Tensor& derInput, Tensor& derBiases, Tensor const& derOutput) {
   tensor_type tt = findTensorType(derInput, derBiases, derOutput);
-  ErrorCode e = requireHipFloat(context, tt, "Subsample::backwardWithBias");
+  bool isDouble;
+  ErrorCode e = requireHip(context, tt, "Subsample::backwardWithBias", &isDouble);
   if (e != VLE_Success) return e;
   if (!derOutput) return context.setError(VLE_IllegalArgument, "Subsample::backwardWithBias: DEROUTPUT is required");
   void* stream = context.getHipHelper().getStream();
@@ -53,9 +60,14 @@ ErrorCode Subsample::backwardWithBias(Tensor& derInput, Tensor& derBiases, Tenso
   if (derInput) {
     if (!extentsMatch(*this, derInput, derOutput))
       return context.setError(VLE_IllegalArgument, "Subsample::backwardWithBias: DEROUTPUT dimensions are incompatible with DERINPUT");
-    rc = mcn_subsample_backward(stream, (float*)derInput.getMemory(), (float const*)derOutput.getMemory(), asInt(derInput.getHeight()),
-                                asInt(derInput.getWidth()), asInt(derInput.getDepth()), asInt(derInput.getSize()), strideY, strideX,
-                                padTop, padBottom, padLeft, padRight);
+    rc = isDouble ? mcn_subsample_backward_f64(stream, (double*)derInput.getMemory(), (double const*)derOutput.getMemory(),
+                                               asInt(derInput.getHeight()), asInt(derInput.getWidth()),
+                                               asInt(derInput.getDepth()), asInt(derInput.getSize()), strideY, strideX,
+                                               padTop, padBottom, padLeft, padRight)
+                  : mcn_subsample_backward(stream, (float*)derInput.getMemory(), (float const*)derOutput.getMemory(),
+                                           asInt(derInput.getHeight()), asInt(derInput.getWidth()),
+                                           asInt(derInput.getDepth()), asInt(derInput.getSize()), strideY, strideX, padTop,
+                                           padBottom, padLeft, padRight);
     if (rc) return fromAbi(context, rc, "Subsample::backwardWithBias");
   }
   if (derBiases) {
@@ -66,6 +78,10 @@ ErrorCode Subsample::backwardWithBias(Tensor& derInput, Tensor& derBiases, Tenso
     g.H = asInt(derOutput.getHeight()); g.W = asInt(derOutput.getWidth()); g.C = asInt(derOutput.getDepth()); g.N = asInt(derOutput.getSize());
     g.FH = g.FW = 1; g.FC = g.C; g.K = g.C;
     g.strideY = g.strideX = 1; g.padTop = g.padBottom = g.padLeft = g.padRight = 0; g.dilateY = g.dilateX = 1;
+    if (isDouble) {
+      rc = mcn_conv_backward_bias_f64(stream, &g, (double*)derBiases.getMemory(), (double const*)derOutput.getMemory());
+      return fromAbi(context, rc, "Subsample::backwardWithBias");
+    }
     size_t bytes = mcn_conv_workspace_bytes(&g, MCN_CONV_BACKWARD_BIAS);
     void* ws = bytes ? context.getWorkspace(VLDT_GPU, bytes) : NULL;
     if (bytes && !ws) return context.getLastError();

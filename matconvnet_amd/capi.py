@@ -92,6 +92,10 @@ PROTOTYPES = {
     "mcn_bnorm_backward_f64": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_pool_forward_f64": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp]),
     "mcn_pool_backward_f64": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp, _vp, _i]),
+    "mcn_subsample_forward_f64": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i]),
+    "mcn_subsample_backward_f64": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i]),
+    "mcn_bias_add_f64": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "mcn_taccum_f64": (_i, [_vp, _vp, _d, _vp, _d, _vp, _sz]),
 }
 
 _lib = None

@@ -114,6 +114,17 @@ int launch(const char* who, mcn_stream_t stream, float* y, const float* a, const
   return check_launch(who);
 }
 
+// y = alpha*a + beta*b in double, each element with the roundings of the reference's scal + axpy pair:
+// t = fl(alpha*a), y = fl(t + fl(beta*b))  (this file is compiled without contraction)
+__global__ __launch_bounds__(256) void taccum64_kernel(double* __restrict__ y, double alpha, const double* __restrict__ a,
+                                                       double beta, const double* __restrict__ b, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    const double t = alpha * a[i];
+    const double u = beta * b[i];
+    y[i] = t + u;
+  }
+}
+
 }  // namespace
 }  // namespace mcn
 
@@ -132,6 +143,14 @@ int mcn_add(mcn_stream_t stream, float* y, const float* a, const float* b, size_
 }
 int mcn_taccum(mcn_stream_t stream, float* y, float alpha, const float* a, float beta, const float* b, size_t n) {
   return launch<OP_AXPBY>("mcn_taccum", stream, y, a, b, alpha, n, beta);
+}
+int mcn_taccum_f64(mcn_stream_t stream, double* y, double alpha, const double* a, double beta, const double* b, size_t n) {
+  if (n == 0) return MCN_SUCCESS;
+  if (!y || !a || !b) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_taccum_f64: null tensor");
+  const size_t blocks = std::min<size_t>((n + 255) / 256, 256u * 32u);
+  KernelTimer timer("taccum64_kernel", as_stream(stream));
+  hipLaunchKernelGGL(taccum64_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), y, alpha, a, beta, b, n);
+  return check_launch("mcn_taccum_f64");
 }
 int mcn_sgd_momentum(mcn_stream_t stream, float* value, float* state, const float* der, size_t chunks,
                      const unsigned short* chunkParam, const double* rates, double learningRate, double weightDecay,

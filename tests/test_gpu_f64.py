@@ -226,15 +226,41 @@ def test_front_end_double_tensors(vl, ob):
         assert bits_equal(_host(dxp), ob.pool_backward(x, dyp, og))
 
 
-def test_front_end_double_where_only_single_exists(vl):
-    """Operators without a double instantiation here say so (no silent conversion): vl_nnconv with empty filters
-    (subsampling with bias) and vl_nnconvt."""
+def test_front_end_double_companions(vl, ob):
+    """The other operators of the front-end in double: vl_nnconv with empty filters (subsampling with bias),
+    vl_nnconvt, vl_taccum."""
+    import torch
+    r = np.random.default_rng(2)
+    x = F(r.standard_normal((9, 8, 4, 2)), D)
+    b = r.standard_normal(4)
+    none = torch.empty((0,), dtype=torch.float64, device="cuda")
+    y = vl.vl_nnconv(_dev(x), none, _dev(b), "stride", [2, 3], "pad", [1, 0, 2, 1])
+    want = ob.subsample_forward(x, b, (2, 3), (1, 0, 2, 1))
+    assert y.dtype == torch.float64 and bits_equal(_host(y), want)
+    dy = F(r.standard_normal(want.shape), D)
+    dx, df, db = vl.vl_nnconv(_dev(x), none, _dev(b), _dev(dy), "stride", [2, 3], "pad", [1, 0, 2, 1])
+    wdx = ob.subsample_backward(x.shape, dy, (2, 3), (1, 0, 2, 1))
+    assert bits_equal(_host(dx), wdx) and rel_max(_host(db).ravel(), dy.sum(axis=(0, 1, 3))) < TOL and df.numel() == 0
+
+    f = F(r.standard_normal((3, 3, 5, 4)) * 0.3, D)   # FH x FW x K x C
+    bt = r.standard_normal(5)
+    yt = vl.vl_nnconvt(_dev(x), _dev(f), _dev(bt), "upsample", 2, "crop", [1, 0, 0, 1])
+    wt = ob.convt_forward(x, f, bt, 2, (1, 0, 0, 1))
+    assert yt.dtype == torch.float64 and tuple(reversed(yt.shape)) == wt.shape and rel_max(_host(yt), wt) < TOL
+    dyt = F(r.standard_normal(wt.shape), D)
+    dxt, dft, dbt = vl.vl_nnconvt(_dev(x), _dev(f), _dev(bt), _dev(dyt), "upsample", 2, "crop", [1, 0, 0, 1])
+    wdx, wdf, wdb = ob.convt_backward(x, f, dyt, 2, (1, 0, 0, 1))
+    assert rel_max(_host(dxt), wdx) < TOL and rel_max(_host(dft), wdf) < TOL and rel_max(_host(dbt).ravel(), wdb) < TOL
+
+    a, c = F(r.standard_normal((5, 4, 3, 2)), D), F(r.standard_normal((5, 4, 3, 2)), D)
+    got = vl.vl_taccum(0.9, _dev(a), -0.37, _dev(c))
+    assert got.dtype == torch.float64 and bits_equal(_host(got), ob.taccum(0.9, a, -0.37, c))
+
+
+def test_mixed_precision_is_refused_by_the_front_end(vl):
     import torch
     x = torch.zeros((2, 4, 8, 8), dtype=torch.float64, device="cuda")
-    b = torch.zeros((4,), dtype=torch.float64, device="cuda")
+    f = torch.zeros((5, 4, 3, 3), dtype=torch.float32, device="cuda")
     with pytest.raises(vl.VlError) as e:
-        vl.vl_nnconv(x, torch.empty((0,), dtype=torch.float64, device="cuda"), b, "stride", 2)
-    assert e.value.code == 1 and "single precision" in e.value.message
-    with pytest.raises(vl.VlError) as e:
-        vl.vl_nnconvt(x, torch.zeros((4, 3, 3, 3), dtype=torch.float64, device="cuda"), torch.zeros((3,), dtype=torch.float64, device="cuda"))
-    assert e.value.code == 1 and "single precision" in e.value.message
+        vl.vl_nnconv(x, f, torch.zeros((5,), device="cuda"))
+    assert e.value.message == "DATA and FILTERS do not have compatible formats."
