@@ -202,4 +202,9 @@ __device__ __forceinline__ void store_block(floatx16 acc, bufrsrc rsrc, unsigned
 int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, const float* wt, const float* bias,
                    const PixP& p, int* handled);
 
+// Products with at most four output channels (conv_few.hip): wt is the packed bank (tapMajor: its row order, see
+// conv_pack_weights).  Sets *handled when it took the work.
+int conv_few_launch(hipStream_t s, const char* who, float* out, const float* in, const float* wt, const float* bias,
+                    const PixP& p, bool tapMajor, int* handled);
+
 }  // namespace mcn

@@ -924,6 +924,12 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   p.rSplits = 1;
   p.stepsPerSplit = 0;
   p.partStride = 0;
+  // one to four output channels (the input gradient of a first layer): conv_few.hip
+  if (p.Cout <= 4) {
+    int handled = 0;
+    rc = conv_few_launch(s, who, out, in, wt, bias, p, ut, &handled);
+    if (rc || handled) return rc;
+  }
   // small filter banks: keep all the weights in LDS and stream the pixels past them (conv_ws.hip)
   if (ut) {
     int handled = 0;

@@ -504,3 +504,53 @@ def test_filter_gradients_with_one_deferred_sum(capi):
     assert sum(capi.lib().mcn_conv_backward_filter_partial_bytes(__import__("ctypes").byref(g)) > 0 for _, _, g in layers) >= 6
     for a, b_, case in zip(got, want, PACKED_CASES):
         assert torch.equal(a, b_), case
+
+
+FEW_CASES = [
+    # x, f, stride, pad, dilate        (backward-data has C output channels, forward K)
+    ((32, 32, 3, 5), (5, 5, 3, 32), 1, 2, 1),                # benchmark configuration 1: dzdx has 3 channels, 32 filters reduce
+    ((28, 28, 1, 4), (5, 5, 1, 20), 1, 0, 1),                # LeNet's first layer: one channel, 20 filters (not a multiple of 16)
+    ((30, 29, 3, 3), (7, 7, 3, 64), 2, 3, 1),                # a ResNet stem in small: strided (four stride classes)
+    ((17, 19, 4, 2), (3, 3, 4, 16), (1, 2), (1, 0, 2, 1), (2, 1)),   # four channels, dilation, one strided axis
+    ((12, 13, 2, 3), (3, 2, 2, 7), 1, 1, 1),                 # two channels, seven filters
+    ((14, 14, 16, 3), (3, 3, 16, 3), 1, 1, 1),               # forward with three filters (and backward-data with 16 channels)
+    ((9, 9, 32, 2), (1, 1, 32, 1), 1, 0, 1),                 # forward 1x1 with one filter
+    ((11, 12, 8, 2), (3, 3, 2, 8), 1, 1, 1),                 # four filter groups of two channels: dzdx per group has 2 channels
+    ((64, 64, 3, 2), (11, 11, 3, 48), 4, 0, 1),              # AlexNet-like first layer: 121 taps, stride 4
+]
+
+
+@pytest.mark.parametrize("xs,fs,stride,pad,dilate", FEW_CASES)
+def test_few_output_channels(capi, ob, xs, fs, stride, pad, dilate):
+    """Products with one to four output channels run a kernel of their own (no padding to 32-channel tiles): forward,
+    backward-data, accumulation into the output, bias; against the oracle, and against the tiled kernels."""
+    r = np.random.default_rng(sum(xs) * 3 + sum(fs))
+    x = F(r.standard_normal(xs))
+    f = F(r.standard_normal(fs) * 0.2)
+    b = r.standard_normal(fs[3]).astype(np.float32)
+    g = ob.conv_geom(xs, fs, stride, pad, dilate)
+    cg = capi.conv_geom(xs, fs, stride, pad, dilate)
+    xd, fd, bd = capi.to_device(x), capi.to_device(f), capi.to_device(b)
+    want = ob.conv_forward(x, f, b, g)
+    dy = F(r.standard_normal(want.shape))
+    base = F(r.standard_normal(want.shape))
+    dbase = F(r.standard_normal(xs))
+    wdx = ob.conv_backward(x, f, dy, g, want=(True, False, False))[0]
+    got = {}
+    for off in (0, 1):
+        capi.set_tunable("conv_no_few", off)
+        try:
+            capi.profile_begin("conv_few_mfma")
+            y = capi.conv_forward(xd, fd, bd, cg)
+            y2 = capi.conv_forward(xd, fd, bd, cg, y=capi.to_device(base), out_mult=0.5, in_mult=2.0)
+            dx, _, _ = capi.conv_backward(xd, fd, capi.to_device(dy), cg, want=(True, False, False))
+            dx2 = capi.conv_backward_data_acc(capi.to_device(dbase), 1.0, fd, capi.to_device(dy), cg)
+            launches, _ = capi.profile_end()
+        finally:
+            capi.set_tunable("conv_no_few", 0)
+        got[off] = launches
+        assert rel_max(capi.to_host(y), want) < 2e-4
+        assert rel_max(capi.to_host(y2), 0.5 * base.astype(np.float64) + 2.0 * (want.astype(np.float64) - b.reshape(1, 1, -1, 1)) + b.reshape(1, 1, -1, 1)) < 2e-4
+        assert rel_max(capi.to_host(dx), wdx) < 2e-4
+        assert rel_max(capi.to_host(dx2), dbase.astype(np.float64) + wdx) < 2e-4
+    assert got[0] >= 2 and got[1] == 0   # the kernel ran (at least the two products of the few-channel side)
