@@ -257,15 +257,15 @@ def bench_pool_bwd(capi, workloads, reps):
 
 def bench_resnet50(vlapi, batch, steps, warmup):
     """Whole ResNet-50 (224 x 224, 1000 classes; examples/imagenet/cnn_imagenet_init_resnet.m) through the same
-    operator classes: forward alone (training-mode batch normalisation), the training step forward + backward +
-    SGD update, and evaluation (stored moments; the mode of the reference's published 396 images/s,
+    operator classes: forward alone (training-mode batch normalisation), the training step forward + loss derivative
+    (softmax log-loss on random labels) + backward + SGD update, and evaluation (stored moments; the mode of the reference's published 396 images/s,
     doc/site/docs/pretrained.md:233, measured there on other hardware), images/s."""
     import torch
     net = vlapi.ResNet50(N=batch, eps=1e-5, image_size=224, classes=1000, fused=True, seed=11)
     try:
         r = np.random.default_rng(12)
         net.set("input", np.asfortranarray(r.standard_normal((224, 224, 3, batch), dtype=np.float32)))
-        net.set("dprediction", np.asfortranarray(r.standard_normal((1, 1, 1000, batch), dtype=np.float32)))
+        net.set("labels", np.asfortranarray(r.integers(1, 1001, (1, 1, 1, batch)).astype(np.float32)))
 
         def timed(fn):
             for _ in range(warmup):
@@ -281,6 +281,7 @@ def bench_resnet50(vlapi, batch, steps, warmup):
 
         def train():
             net.forward()
+            net.loss_derivative()
             net.backward()
             net.sgd_step(1e-3, 0.9, 1e-4)
 

@@ -320,6 +320,36 @@ MCN_API int mcn_sgd_momentum(mcn_stream_t stream, float* value, float* state, co
 MCN_API int mcn_fill(mcn_stream_t stream, float* y, float value, size_t n);
 
 /* ------------------------------------------------------------------------------------------------
+ * losses -- matlab/vl_nnloss.m:136-317 (MATLAB code on gpuArrays in the reference; the last layers of
+ * examples/imagenet/cnn_imagenet_init_resnet.m:128-139 are three of them: 'softmaxlog', 'classerror', 'topkerror').
+ * x is H x W x C x N.  Categorical losses take one label (a class number 1..C as a float; 0 = skip this instance)
+ * per image (nLabels == N) or per prediction vector (nLabels == H*W*N); attribute losses take one label (+1 / -1;
+ * 0 = skip) per element of x.  instanceWeights (may be NULL) multiply the terms; their nWeights values are
+ * broadcast over the labels by index (H*W values: one map for all images; 1: a scalar; as many as labels: one each).
+ * normalise != 0 divides by N, as the reference does for 4-D inputs.
+ * ---------------------------------------------------------------------------------------------- */
+enum {
+  MCN_LOSS_CLASSERROR = 0, MCN_LOSS_TOPKERROR = 1, MCN_LOSS_LOG = 2, MCN_LOSS_SOFTMAXLOG = 3, MCN_LOSS_MHINGE = 4,
+  MCN_LOSS_MSHINGE = 5, MCN_LOSS_BINARYERROR = 6, MCN_LOSS_BINARYLOG = 7, MCN_LOSS_LOGISTIC = 8, MCN_LOSS_HINGE = 9
+};
+typedef struct mcn_loss_geom {
+  int H, W, C, N;
+  int loss;          /* MCN_LOSS_* */
+  int topK;          /* 'topkerror' (reference default 5) */
+  int normalise;     /* reference default: true */
+  double threshold;  /* 'binaryerror' (reference default 0) */
+} mcn_loss_geom;
+MCN_API size_t mcn_loss_workspace_bytes(const mcn_loss_geom* g);
+/* y[0] (device) = sum over the instances of weight * loss term  (vl_nnloss.m:229-271) */
+MCN_API int mcn_loss_forward(mcn_stream_t stream, const mcn_loss_geom* g, float* y, const float* x, const float* labels,
+                             size_t nLabels, const float* instanceWeights, size_t nWeights, void* workspace,
+                             size_t workspaceBytes);
+/* dzdx (shape of x, fully overwritten) for the scalar derOutput = dz/dy  (vl_nnloss.m:273-316) */
+MCN_API int mcn_loss_backward(mcn_stream_t stream, const mcn_loss_geom* g, float* derInput, const float* x,
+                              const float* labels, size_t nLabels, const float* instanceWeights, size_t nWeights,
+                              double derOutput);
+
+/* ------------------------------------------------------------------------------------------------
  * double precision -- the operators' VLDT_Double instantiation (bits/impl/dispatcher.hpp:60-98 switches on the
  * tensors' data type; bits/nnconv.cu:444-469, bits/nnbnorm.cu:388-442, bits/nnpooling.cu:270-282 instantiate
  * every product for float and double).  Same arguments and meaning as the single-precision calls above; general

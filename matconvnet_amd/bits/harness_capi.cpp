@@ -246,6 +246,10 @@ int vlh_resnet50_pack(void* net) { return (int)((harness::ResNet50*)net)->pack()
 int vlh_resnet50_init(void* net, unsigned long long seed) { return (int)((harness::ResNet50*)net)->initParameters(seed); }
 int vlh_resnet50_forward(void* net) { return (int)((harness::ResNet50*)net)->forward(); }
 int vlh_resnet50_backward(void* net) { return (int)((harness::ResNet50*)net)->backward(); }
+int vlh_resnet50_loss_derivative(void* net, double derOutput) { return (int)((harness::ResNet50*)net)->lossDerivative(derOutput); }
+int vlh_resnet50_losses(void* net, double values[3]) {
+  return (int)((harness::ResNet50*)net)->losses(values, values + 1, values + 2);
+}
 int vlh_resnet50_sgd_step(void* net, double learningRate, double momentum, double weightDecay) {
   return (int)((harness::ResNet50*)net)->sgdStep(learningRate, momentum, weightDecay);
 }

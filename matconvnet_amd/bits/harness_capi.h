@@ -90,6 +90,11 @@ VLH_API int vlh_resnet50_backward(void* net);
    examples/cnn_train_dag.m:316-364 with the rates of cnn_imagenet_init_resnet.m:178-195; buffers "momentum.<parameter>"
    and "running.<moments>" hold the solver state */
 VLH_API int vlh_resnet50_sgd_step(void* net, double learningRate, double momentum, double weightDecay);
+/* the loss layers at the end of the network (cnn_imagenet_init_resnet.m:128-139) on buffers "prediction" and "labels"
+   (N class numbers 1..classes as floats, 0 = skip): _loss_derivative writes "dprediction" for vlh_resnet50_backward
+   (softmax log-loss normalised by N, times derOutput); _losses returns {that loss, top-1 error, top-5 error} */
+VLH_API int vlh_resnet50_loss_derivative(void* net, double derOutput);
+VLH_API int vlh_resnet50_losses(void* net, double values[3]);
 VLH_API size_t vlh_resnet50_parameters(void* net);
 /* records forward (training == 0) or a whole training step (forward, backward, SGD update with these rates) on the
    network's stream -- which must not be the default stream -- into a HIP graph; vlh_resnet50_replay launches it.  The

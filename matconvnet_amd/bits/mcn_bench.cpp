@@ -254,6 +254,14 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
       HIP_OK(hipMemcpy(p, host.data(), n * sizeof(float), hipMemcpyHostToDevice));
     }
   }
+  {
+    // one class number per image for the loss layers
+    size_t n = 0;
+    float* p = net.buffer("labels", &n);
+    std::vector<float> host(n);
+    for (size_t i = 0; i < n; ++i) host[i] = (float)(1 + (i * 37) % 1000);
+    HIP_OK(hipMemcpy(p, host.data(), n * sizeof(float), hipMemcpyHostToDevice));
+  }
   auto stop = [&] {
     std::fprintf(stderr, "resnet-50: %s\n", net.lastMessage().c_str());
     std::exit(3);
@@ -261,7 +269,8 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
   double tf = medianMs([&] { if (net.forward() != VLE_Success) stop(); }, warmup, iters);
   double t = medianMs([&] { if (net.forward() != VLE_Success || net.backward() != VLE_Success) stop(); }, warmup, iters);
   double ts = medianMs([&] {
-    if (net.forward() != VLE_Success || net.backward() != VLE_Success || net.sgdStep(1e-3, 0.9, 1e-4) != VLE_Success) stop();
+    if (net.forward() != VLE_Success || net.lossDerivative() != VLE_Success || net.backward() != VLE_Success ||
+        net.sgdStep(1e-3, 0.9, 1e-4) != VLE_Success) stop();
   }, warmup, iters);
   // the same training step and evaluation pass replayed from HIP graphs (recorded on a stream of the network's own)
   hipStream_t own = NULL;
@@ -285,7 +294,7 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
               "%8.2f ms %8.0f images/s, training step %8.2f ms %8.0f images/s\n", "resnet-50 224x224", te,
               N / (te * 1e-3), gf * N / te, teg, N / (teg * 1e-3), tsg, N / (tsg * 1e-3));
   std::printf("%-28s %8.2f ms forward  %8.0f images/s %6.1f TFLOP/s | %8.2f ms fwd+bwd %8.0f images/s %6.1f TFLOP/s | "
-              "%8.2f ms training step (with the SGD update of %.1f M parameters) %8.0f images/s "
+              "%8.2f ms training step (with the loss derivative and the SGD update of %.1f M parameters) %8.0f images/s "
               "(N = %d, %.2f GFLOP of convolution per image forward; %s)\n",
               "resnet-50 224x224", tf, N / (tf * 1e-3), gf * N / tf, t, N / (t * 1e-3), 3 * gf * N / t, ts,
               net.numParameters() * 1e-6, N / (ts * 1e-3), N, gf, fused ? "relu/sum folded into bnorm, filter banks packed once per update" : "layer by layer");

@@ -86,6 +86,7 @@ ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
 
   make("avg", TensorShape(1, 1, C, N)); make("davg", TensorShape(1, 1, C, N));
   make("prediction", TensorShape(1, 1, classes, N)); make("dprediction", TensorShape(1, 1, classes, N));
+  make("labels", TensorShape(1, 1, 1, N)); make("loss.terms", TensorShape(1, 1, 1, N)); make("loss.values", TensorShape(4, 1, 1, 1));
   flops += conv_flops(1, 1, 1, 1, C, classes);
   if (error == VLE_Success) buildArenas();
   setFused(true);
@@ -212,6 +213,54 @@ ErrorCode ResNet50::sgdStep(double learningRate, double momentum, double weightD
   const double rate = 0.3;
   ABI("moments", mcn_taccum(st, runningMoments, (float)(1.0 - rate), runningMoments, (float)rate, batchMoments, momentsCount));
   return pack();  // (the filters have changed)
+}
+
+namespace {
+mcn_loss_geom lossGeometry(Tensor const& prediction, int kind, int topK) {
+  mcn_loss_geom g;
+  g.H = g.W = 1;
+  g.C = (int)prediction.getDepth();
+  g.N = (int)prediction.getSize();
+  g.loss = kind;
+  g.topK = topK;
+  g.normalise = 1;
+  g.threshold = 0;
+  return g;
+}
+}  // namespace
+
+ErrorCode ResNet50::lossDerivative(double derOutput) {
+  if (error != VLE_Success) return error;
+  void* st = context.getHipHelper().getStream();
+  const mcn_loss_geom g = lossGeometry(slot("prediction"), MCN_LOSS_SOFTMAXLOG, 5);
+  ABI("loss", mcn_loss_backward(st, &g, (float*)slot("dprediction").getMemory(), (float const*)slot("prediction").getMemory(),
+                                (float const*)slot("labels").getMemory(), (size_t)g.N, NULL, 0, derOutput));
+  return VLE_Success;
+}
+
+ErrorCode ResNet50::losses(double* objective, double* top1Error, double* top5Error) {
+  if (error != VLE_Success) return error;
+  void* st = context.getHipHelper().getStream();
+  float* values = (float*)slot("loss.values").getMemory();
+  void* terms = slot("loss.terms").getMemory();
+  const size_t termBytes = slot("loss.terms").getNumElements() * sizeof(float);
+  const int kinds[3] = {MCN_LOSS_SOFTMAXLOG, MCN_LOSS_CLASSERROR, MCN_LOSS_TOPKERROR};
+  for (int k = 0; k < 3; ++k) {
+    const mcn_loss_geom g = lossGeometry(slot("prediction"), kinds[k], 5);
+    ABI("loss", mcn_loss_forward(st, &g, values + k, (float const*)slot("prediction").getMemory(),
+                                 (float const*)slot("labels").getMemory(), (size_t)g.N, NULL, 0, terms, termBytes));
+  }
+  float host[3] = {0, 0, 0};
+  if (hipMemcpyAsync(host, values, sizeof(host), hipMemcpyDeviceToHost, (hipStream_t)st) != hipSuccess ||
+      hipStreamSynchronize((hipStream_t)st) != hipSuccess) {
+    (void)hipGetLastError();
+    message = "cannot read the loss values back";
+    return VLE_Cuda;
+  }
+  if (objective) *objective = host[0];
+  if (top1Error) *top1Error = host[1];
+  if (top5Error) *top5Error = host[2];
+  return VLE_Success;
 }
 
 void ResNet50::dropGraph() {

@@ -52,6 +52,12 @@ class ResNet50 {
   ErrorCode setDeferred(bool on);
   ErrorCode forward();
   ErrorCode backward();
+  // The network's last layers (cnn_imagenet_init_resnet.m:128-139): from "prediction" and "labels" (one class number
+  // 1..classes per image, as floats; 0 = skip the image), lossDerivative() writes "dprediction" = the derivative of
+  // derOutput * (softmax log-loss, normalised by the batch size) -- what backward() starts from in training -- and
+  // losses() returns that loss and the top-1 / top-5 error rates of the batch (it waits for the stream).
+  ErrorCode lossDerivative(double derOutput = 1.0);
+  ErrorCode losses(double* objective, double* top1Error, double* top5Error);
   // one update of all parameters from the derivatives backward() left (numWorkers = 1), and of the moving averages of
   // the moments from those forward() left
   ErrorCode sgdStep(double learningRate, double momentum, double weightDecay);

@@ -29,6 +29,14 @@ class PoolGeom(C.Structure):
         "padTop", "padBottom", "padLeft", "padRight", "method")]
 
 
+class LossGeom(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("H", "W", "C", "N", "loss", "topK", "normalise")] + [("threshold", C.c_double)]
+
+
+LOSSES = ("classerror", "topkerror", "log", "softmaxlog", "mhinge", "mshinge", "binaryerror", "binarylog", "logistic",
+          "hinge")
+
+
 class McnError(RuntimeError):
     def __init__(self, code, message):
         super().__init__("mcn error %d: %s" % (code, message))
@@ -84,6 +92,9 @@ PROTOTYPES = {
     "mcn_relu_backward": (_i, [_vp, _vp, _vp, _vp, _sz]),
     "mcn_add": (_i, [_vp, _vp, _vp, _vp, _sz]),
     "mcn_fill": (_i, [_vp, _vp, _f, _sz]),
+    "mcn_loss_workspace_bytes": (_sz, [C.POINTER(LossGeom)]),
+    "mcn_loss_forward": (_i, [_vp, C.POINTER(LossGeom), _vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz]),
+    "mcn_loss_backward": (_i, [_vp, C.POINTER(LossGeom), _vp, _vp, _vp, _sz, _vp, _sz, _d]),
     "mcn_conv_forward_f64": (_i, [_vp, C.POINTER(ConvGeom), _vp, _d, _vp, _d, _vp, _vp]),
     "mcn_conv_backward_data_f64": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp]),
     "mcn_conv_backward_filter_f64": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp]),
@@ -501,6 +512,29 @@ def pool_backward(x, dy, g, dx=None):
         dx = empty((g.H, g.W, g.C, g.N), like=dy)
     fn = lib().mcn_pool_backward_f64 if _is64(x, dy, dx) else lib().mcn_pool_backward
     check(fn(stream(), C.byref(g), ptr(dx), ptr(x), ptr(dy), int(acc)))
+    return dx
+
+
+def loss_geom(xshape, loss="softmaxlog", top_k=5, normalise=True, threshold=0.0):
+    H, W, Cc, N = (list(xshape) + [1, 1, 1])[:4]
+    return LossGeom(H, W, Cc, N, LOSSES.index(loss.lower()), top_k, int(bool(normalise)), threshold)
+
+
+def loss_forward(x, c, g, instance_weights=None, ws=None):
+    """vl_nnloss(x, c, [], ...): the loss as a one-element device tensor."""
+    ws = ws or _ws
+    y = empty((1,))
+    wp, wn = ws.get(lib().mcn_loss_workspace_bytes(C.byref(g)))
+    check(lib().mcn_loss_forward(stream(), C.byref(g), ptr(y), ptr(x), ptr(c), c.numel(), ptr(instance_weights),
+                                 0 if instance_weights is None else instance_weights.numel(), wp, wn))
+    return y
+
+
+def loss_backward(x, c, dzdy, g, instance_weights=None):
+    """vl_nnloss(x, c, dzdy, ...): dzdx."""
+    dx = empty(tuple(reversed(x.shape)))
+    check(lib().mcn_loss_backward(stream(), C.byref(g), ptr(dx), ptr(x), ptr(c), c.numel(), ptr(instance_weights),
+                                  0 if instance_weights is None else instance_weights.numel(), float(dzdy)))
     return dx
 
 

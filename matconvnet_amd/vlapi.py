@@ -91,6 +91,8 @@ def lib():
         L.vlh_resnet50_forward.argtypes = [C.c_void_p]
         L.vlh_resnet50_backward.argtypes = [C.c_void_p]
         L.vlh_resnet50_sgd_step.argtypes = [C.c_void_p, C.c_double, C.c_double, C.c_double]
+        L.vlh_resnet50_loss_derivative.argtypes = [C.c_void_p, C.c_double]
+        L.vlh_resnet50_losses.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
         L.vlh_resnet50_parameters.argtypes = [C.c_void_p]
         L.vlh_resnet50_capture.argtypes = [C.c_void_p, C.c_int, C.c_double, C.c_double, C.c_double]
         L.vlh_resnet50_replay.argtypes = [C.c_void_p]
@@ -319,6 +321,16 @@ class ResNet50(_NamedBuffers):
 
     def sgd_step(self, learning_rate, momentum=0.9, weight_decay=1e-4):
         self._check(self.L.vlh_resnet50_sgd_step(self.h, learning_rate, momentum, weight_decay))
+
+    def loss_derivative(self, der_output=1.0):
+        """"dprediction" from "prediction" and "labels" (softmax log-loss normalised by the batch size)."""
+        self._check(self.L.vlh_resnet50_loss_derivative(self.h, der_output))
+
+    def losses(self):
+        """(softmax log-loss, top-1 error, top-5 error) of the batch, each normalised by the batch size."""
+        v = (C.c_double * 3)()
+        self._check(self.L.vlh_resnet50_losses(self.h, v))
+        return tuple(v)
 
     @property
     def parameters(self):

@@ -348,3 +348,39 @@ def test_image_size_must_be_a_multiple_of_32(vl):
     from matconvnet_amd.vlapi import VlError
     with pytest.raises(VlError, match="multiple of 32"):
         vl.ResNet50(N=1, image_size=100)
+
+
+def test_loss_layers_and_a_few_training_steps(vl, case):
+    """The network's last layers (softmax log-loss, top-1 / top-5 error; cnn_imagenet_init_resnet.m:128-139) on the
+    device: their values and the derivative the backward pass starts from against the numpy restatement of
+    vl_nnloss.m; then whole training steps (forward, loss derivative, backward, SGD) on one fixed batch lower that
+    batch's loss."""
+    from oracle import loss as ol
+    r = np.random.default_rng(31)
+    net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=True)
+    try:
+        _load(net, case)
+        labels = r.integers(1, CLASSES + 1, N).astype(np.float32)
+        labels[-1] = 0.0   # (a skipped image)
+        net.set("labels", np.asfortranarray(labels.reshape(1, 1, 1, N)))
+        net.forward()
+        net.loss_derivative()
+        pred = np.asfortranarray(net.get("prediction").reshape(1, 1, CLASSES, N, order="F"))
+        objective, top1, top5 = net.losses()
+        assert abs(objective - float(ol.vl_nnloss(pred, labels, None, loss="softmaxlog"))) < 1e-5 * max(1.0, abs(objective))
+        assert top1 == pytest.approx(float(ol.vl_nnloss(pred, labels, None, loss="classerror")), abs=1e-6)
+        assert top5 == pytest.approx(float(ol.vl_nnloss(pred, labels, None, loss="topkerror", top_k=5)), abs=1e-6)
+        want = ol.vl_nnloss(pred, labels, 1.0, loss="softmaxlog")
+        got = net.get("dprediction").reshape(1, 1, CLASSES, N, order="F")
+        assert rel_max(got, want) < 1e-5 and not got[..., -1].any()
+        first = objective
+        for _ in range(8):
+            net.forward()
+            net.loss_derivative()
+            net.backward()
+            net.sgd_step(0.05, 0.9, 1e-4)
+        net.forward()
+        last = net.losses()[0]
+        assert np.isfinite(last) and last < 0.7 * first, (first, last)
+    finally:
+        net.close()
