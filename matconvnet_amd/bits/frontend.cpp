@@ -5,6 +5,12 @@
 
 #include <cctype>
 #include <cstdio>
+#include <vector>
+
+#include <hip/hip_runtime_api.h>
+
+#include "../../include/mcn_hip.h"
+#include "hiphelper.hpp"
 
 #include "nnbnorm.hpp"
 #include "nnconv.hpp"
@@ -530,6 +536,106 @@ void taccum(Context& context, Allocator& allocator, int nout, Tensor* out, int n
   (void)nout;
 }
 
+// ------------------------------------------------------------------------------------------ vl_nnloss
+// matlab/vl_nnloss.m:129-317 (MATLAB code in the reference): (x, c [, dzdy], options)
+
+// A single-precision device copy of a numeric argument that may live on the host (labels and instance weights come
+// from the data loader there; the reference gathers the labels to the host, the kernels here want them on the device).
+Tensor onDeviceAsSingle(Context& context, Allocator& allocator, Arg const& a, char const* NAME) {
+  if (a.kind != Arg::Array) raise(VLE_IllegalArgument, std::string(NAME) + " is not a numeric array.");
+  Tensor const& t = a.tensor;
+  if (t.getDeviceType() == VLDT_GPU) {
+    if (t.getDataType() != VLDT_Float) raise(VLE_Unsupported, std::string(NAME) + ": only SINGLE arrays are supported on the device.");
+    return t;
+  }
+  const std::size_t n = t.getNumElements();
+  std::vector<float> host(n);
+  if (t.getDataType() == VLDT_Float) for (std::size_t i = 0; i < n; ++i) host[i] = ((float const*)t.getMemory())[i];
+  else if (t.getDataType() == VLDT_Double) for (std::size_t i = 0; i < n; ++i) host[i] = (float)((double const*)t.getMemory())[i];
+  else raise(VLE_IllegalArgument, std::string(NAME) + " is neither SINGLE nor DOUBLE.");
+  Tensor copy = newOutput(allocator, VLDT_GPU, VLDT_Float, t.getShape());
+  hipStream_t stream = (hipStream_t)context.getHipHelper().getStream();
+  if (n && (hipMemcpyAsync(copy.getMemory(), host.data(), n * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess ||
+            hipStreamSynchronize(stream) != hipSuccess)) {
+    (void)hipGetLastError();
+    raise(VLE_Cuda, std::string(NAME) + ": could not be copied to the device.");
+  }
+  return copy;
+}
+
+void nnloss(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in) {
+  enum { optLoss, optInstanceWeights, optClassWeights, optThreshold, optNormalise, optTopK };
+  static OptionSpec const specs[] = {{"loss", true, optLoss}, {"instanceWeights", true, optInstanceWeights},
+                                     {"classWeights", true, optClassWeights}, {"threshold", true, optThreshold},
+                                     {"normalise", true, optNormalise}, {"topK", true, optTopK}, {NULL, false, 0}};
+  static char const* const names[] = {"classerror", "topkerror", "log", "softmaxlog", "mhinge", "mshinge",
+                                      "binaryerror", "binarylog", "logistic", "hinge"};
+  if (nin < 2) raise(VLE_IllegalArgument, "There are less than two arguments.");
+  int next = 2;
+  Arg const* dzdy = NULL;
+  if (nin > 2 && in[2].kind != Arg::String) {   // (vl_nnloss.m:129-134)
+    dzdy = &in[2];
+    next = 3;
+  }
+  mcn_loss_geom g;
+  g.loss = MCN_LOSS_SOFTMAXLOG; g.topK = 5; g.normalise = 1; g.threshold = 0;   // (vl_nnloss.m:136-141)
+  Arg const* weights = NULL;
+  int opt;
+  Arg const* value = NULL;
+  auto scalar = [&](Arg const& a, char const* NAME) -> double {
+    if (!(isPlainMatrix(a) && a.tensor.getNumElements() == 1)) raise(VLE_IllegalArgument, std::string(NAME) + " is not a plain scalar.");
+    return values(a)[0];
+  };
+  while ((opt = nextOption(in, nin, specs, &next, &value)) >= 0) {
+    switch (opt) {
+      case optLoss: {
+        if (value->kind != Arg::String) raise(VLE_IllegalArgument, "LOSS is not a string.");
+        int k = 0;
+        for (; k < 10; ++k) if (sameTextNoCase(value->text, names[k])) break;
+        if (k == 10) raise(VLE_IllegalArgument, "Unknown loss '" + value->text + "'.");   // (vl_nnloss.m:199-200)
+        g.loss = k;
+        break;
+      }
+      case optInstanceWeights: if (!(value->kind == Arg::Array && value->tensor.getNumElements() == 0)) weights = value; break;
+      case optClassWeights:
+        if (!(value->kind == Arg::Array && value->tensor.getNumElements() == 0))
+          raise(VLE_Unsupported, "CLASSWEIGHTS are not used by vl_nnloss.");   // (parsed and never read by the reference)
+        break;
+      case optThreshold: g.threshold = scalar(*value, "THRESHOLD"); break;
+      case optNormalise: g.normalise = scalar(*value, "NORMALISE") != 0; break;
+      case optTopK: g.topK = (int)scalar(*value, "TOPK"); break;
+    }
+  }
+  Tensor x = dataTensor(in[0], "X", 4);
+  if (x.getDeviceType() != VLDT_GPU) raise(VLE_Unsupported, "vl_nnloss: X is on the CPU; this library implements the GPU (HIP, gfx950) device only");
+  if (x.getDataType() != VLDT_Float) raise(VLE_Unsupported, "vl_nnloss: only single precision is implemented on the HIP device");
+  g.H = (int)x.getHeight(); g.W = (int)x.getWidth(); g.C = (int)x.getDepth(); g.N = (int)x.getSize();
+  Tensor c = onDeviceAsSingle(context, allocator, in[1], "C");
+  Tensor w;
+  if (weights) w = onDeviceAsSingle(context, allocator, *weights, "INSTANCEWEIGHTS");
+  void* stream = context.getHipHelper().getStream();
+  const bool backMode = dzdy && !(dzdy->kind == Arg::Array && dzdy->tensor.getNumElements() == 0);
+  int rc;
+  if (!backMode) {
+    const std::size_t bytes = mcn_loss_workspace_bytes(&g);
+    void* ws = bytes ? context.getWorkspace(VLDT_GPU, bytes) : NULL;
+    if (bytes && !ws) failFromContext(context, context.getLastError());
+    std::size_t one[2] = {1, 1};
+    Tensor y = newOutput(allocator, VLDT_GPU, VLDT_Float, TensorShape(one, 2));
+    rc = mcn_loss_forward(stream, &g, (float*)y.getMemory(), (float const*)x.getMemory(), (float const*)c.getMemory(),
+                          c.getNumElements(), (float const*)w.getMemory(), w.getNumElements(), ws, bytes);
+    out[0] = y;
+  } else {
+    const double dz = scalar(*dzdy, "DZDY");
+    Tensor dzdx = newOutput(allocator, VLDT_GPU, VLDT_Float, in[0].tensor.getShape());
+    rc = mcn_loss_backward(stream, &g, (float*)dzdx.getMemory(), (float const*)x.getMemory(), (float const*)c.getMemory(),
+                           c.getNumElements(), (float const*)w.getMemory(), w.getNumElements(), dz);
+    out[0] = dzdx;
+  }
+  if (rc) raise(rc > 0 && rc <= (int)VLE_Interrupted ? (ErrorCode)rc : VLE_Unknown, mcn_last_error_message());
+  (void)nout;
+}
+
 typedef void (*Body)(Context&, Allocator&, int, Tensor*, int, Arg const*);
 
 ErrorCode guarded(Body body, Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
@@ -561,6 +667,9 @@ ErrorCode vl_nnpool(Context& context, Allocator& allocator, int nout, Tensor* ou
 }
 ErrorCode vl_taccum(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
   return guarded(taccum, context, allocator, nout, out, nin, in, message);
+}
+ErrorCode vl_nnloss(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
+  return guarded(nnloss, context, allocator, nout, out, nin, in, message);
 }
 
 } }  // namespace vl::frontend

@@ -48,6 +48,7 @@ class Allocator {
 //   vl_nnbnorm: forward [y, moments]    backward [dzdx, dzdg, dzdb, moments]
 //   vl_nnpool : forward [y]             backward [dzdx]
 //   vl_taccum : [alpha*a + beta*b]; nothing with 'InPlace' (a itself is updated)
+//   vl_nnloss : forward [y] (1 x 1 on the device)   backward [dzdx]
 ErrorCode vl_nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                     std::string& message);
 ErrorCode vl_nnconvt(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
@@ -57,6 +58,11 @@ ErrorCode vl_nnbnorm(Context& context, Allocator& allocator, int nout, Tensor* o
 ErrorCode vl_nnpool(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                     std::string& message);
 ErrorCode vl_taccum(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
+                    std::string& message);
+// vl_nnloss(x, c [, dzdy], 'loss', name, 'instanceWeights', w, 'normalise', tf, 'threshold', t, 'topK', k)
+// (matlab/vl_nnloss.m:129-142; a MATLAB function in the reference).  x: single, on the device.  c and the instance
+// weights: on the device (single) or host arrays (copied over).  dzdy: a host scalar, or empty for the forward mode.
+ErrorCode vl_nnloss(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                     std::string& message);
 
 } }  // namespace vl::frontend

@@ -205,6 +205,12 @@ def vl_nnpool(*args):
     return _call("vl_nnpool", 1, list(args))[0]
 
 
+def vl_nnloss(*args):
+    """vl_nnloss(x, c [, dzdy], 'loss', name, 'instanceWeights', w, 'normalise', tf, 'threshold', t, 'topK', k)
+    (matlab/vl_nnloss.m): the loss as a 1 x 1 device array, or dzdx when dzdy is given (a number)."""
+    return _call("vl_nnloss", 1, list(args))[0]
+
+
 def vl_taccum(*args):
     """vl_taccum(alpha, a, beta, b [, 'inplace']): alpha*a + beta*b (matlab/vl_taccum.m); with 'inplace', `a` itself
     is updated and returned."""

@@ -105,3 +105,36 @@ def test_argument_errors(capi):
     g.loss = 17
     with pytest.raises(capi.McnError):
         capi.loss_forward(x, capi.to_device(np.ones(4)), g)
+
+
+def test_front_end_vl_nnloss(vl):
+    """vl_nnloss with the reference's argument conventions (matlab/vl_nnloss.m:129-142): positional dzdy, options by
+    name without regard to case, labels and weights from the host or the device."""
+    import torch
+    r = np.random.default_rng(8)
+    shape = (4, 5, 3, 3)
+    x = F(r.standard_normal(shape))
+    c = r.integers(0, 4, (4, 5, 1, 3)).astype(np.float64)       # (zeros: skipped instances)
+    w = r.random((4, 5))
+    dev = lambda a, dt=np.float32: torch.from_numpy(np.ascontiguousarray(np.asfortranarray(a, dtype=dt).T)).cuda()
+    host = lambda a: torch.from_numpy(np.ascontiguousarray(np.asfortranarray(a, dtype=np.float64).T))
+    y = vl.vl_nnloss(dev(x), host(c))
+    assert tuple(y.shape) == (1, 1) and y.is_cuda
+    assert abs(float(y) - float(ol.vl_nnloss(x, c, None))) < 1e-5
+    y = vl.vl_nnloss(dev(x), dev(c), "LOSS", "mshinge", "instanceweights", host(w), "normalise", 0.0)
+    assert abs(float(y) - float(ol.vl_nnloss(x, c, None, loss="mshinge", instance_weights=w, normalise=False))) < 1e-5
+    y = vl.vl_nnloss(dev(x), host(c), torch.empty((0,), dtype=torch.float64), "loss", "topkerror", "topK", 2.0)
+    assert float(y) == float(ol.vl_nnloss(x, c, None, loss="topkerror", top_k=2))
+    dx = vl.vl_nnloss(dev(x), host(c), 0.7, "loss", "softmaxlog", "instanceWeights", dev(w))
+    want = ol.vl_nnloss(x, c, 0.7, loss="softmaxlog", instance_weights=w)
+    got = np.asfortranarray(dx.detach().cpu().numpy().T)
+    assert got.shape == want.shape and rel_max(got, want) < 1e-5
+    for args, message in [((dev(x), host(c), "loss", "bogus"), "Unknown loss 'bogus'."),
+                          ((dev(x), host(c), "frobnicate", 1.0), "Unknown option 'frobnicate'."),
+                          ((dev(x),), "There are less than two arguments.")]:
+        with pytest.raises(vl.VlError) as e:
+            vl.vl_nnloss(*args)
+        assert e.value.message == message, e.value.message
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnloss(dev(x, np.float64), host(c))
+    assert e.value.code == 1
