@@ -295,6 +295,11 @@ MCN_API int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float
 /* y = max(x, 0); dzdx = dzdy .* (x > 0)   (matlab/vl_nnrelu.m:43-48, leak = 0) */
 MCN_API int mcn_relu_forward(mcn_stream_t stream, float* y, const float* x, size_t n);
 MCN_API int mcn_relu_backward(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, size_t n);
+/* the same with a leak: y = x .* (leak + (1 - leak)*(x > 0)), dzdx = dzdy .* (leak + (1 - leak)*(x > 0))
+   (matlab/vl_nnrelu.m:49-55; leak = 0 takes the plain form above) */
+MCN_API int mcn_relu_forward_leaky(mcn_stream_t stream, float* y, const float* x, size_t n, double leak);
+MCN_API int mcn_relu_backward_leaky(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, size_t n,
+                                    double leak);
 /* y = a + b   (matlab/+dagnn/Sum.m:11-17; also the fan-out derivative sum of +dagnn/Layer.m:127-135) */
 MCN_API int mcn_add(mcn_stream_t stream, float* y, const float* a, const float* b, size_t n);
 /* y = alpha*a + beta*b, the momentum / weight update of SGD (matlab/src/vl_taccummex.cu:48-78: copy, BLAS scal, then

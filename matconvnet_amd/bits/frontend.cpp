@@ -636,6 +636,47 @@ void nnloss(Context& context, Allocator& allocator, int nout, Tensor* out, int n
   (void)nout;
 }
 
+// ------------------------------------------------------------------------------------------ vl_nnrelu
+// matlab/vl_nnrelu.m:33-55: (x [, dzdy], 'leak', value)
+
+void nnrelu(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in) {
+  enum { optLeak };
+  static OptionSpec const specs[] = {{"leak", true, optLeak}, {NULL, false, 0}};
+  if (nin < 1) raise(VLE_IllegalArgument, "There are no arguments.");
+  int next = 1;
+  Arg const* dzdyArg = NULL;
+  if (nin > 1 && in[1].kind != Arg::String) {
+    dzdyArg = &in[1];
+    next = 2;
+  }
+  double leak = 0;
+  int opt;
+  Arg const* value = NULL;
+  while ((opt = nextOption(in, nin, specs, &next, &value)) >= 0) {
+    if (!(isPlainMatrix(*value) && value->tensor.getNumElements() == 1)) raise(VLE_IllegalArgument, "LEAK is not a plain scalar.");
+    leak = values(*value)[0];
+  }
+  Tensor x = dataTensor(in[0], "X", 4);
+  if (x.getDeviceType() != VLDT_GPU) raise(VLE_Unsupported, "vl_nnrelu: X is on the CPU; this library implements the GPU (HIP, gfx950) device only");
+  if (x.getDataType() != VLDT_Float) raise(VLE_Unsupported, "vl_nnrelu: only single precision is implemented on the HIP device");
+  void* stream = context.getHipHelper().getStream();
+  Tensor y = newOutput(allocator, VLDT_GPU, VLDT_Float, in[0].tensor.getShape());
+  const bool backMode = dzdyArg && !(dzdyArg->kind == Arg::Array && dzdyArg->tensor.getNumElements() == 0);
+  int rc;
+  if (!backMode) {
+    rc = mcn_relu_forward_leaky(stream, (float*)y.getMemory(), (float const*)x.getMemory(), x.getNumElements(), leak);
+  } else {
+    Tensor dzdy = dataTensor(*dzdyArg, "DZDY", 4);
+    if (!areCompatible(x, dzdy)) raise(VLE_IllegalArgument, "X and DZDY do not have compatible formats.");
+    if (dzdy.getNumElements() != x.getNumElements()) raise(VLE_IllegalArgument, "X and DZDY do not have the same number of elements.");
+    rc = mcn_relu_backward_leaky(stream, (float*)y.getMemory(), (float const*)x.getMemory(), (float const*)dzdy.getMemory(),
+                                 x.getNumElements(), leak);
+  }
+  if (rc) raise(rc > 0 && rc <= (int)VLE_Interrupted ? (ErrorCode)rc : VLE_Unknown, mcn_last_error_message());
+  out[0] = y;
+  (void)nout;
+}
+
 typedef void (*Body)(Context&, Allocator&, int, Tensor*, int, Arg const*);
 
 ErrorCode guarded(Body body, Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
@@ -667,6 +708,9 @@ ErrorCode vl_nnpool(Context& context, Allocator& allocator, int nout, Tensor* ou
 }
 ErrorCode vl_taccum(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
   return guarded(taccum, context, allocator, nout, out, nin, in, message);
+}
+ErrorCode vl_nnrelu(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
+  return guarded(nnrelu, context, allocator, nout, out, nin, in, message);
 }
 ErrorCode vl_nnloss(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
   return guarded(nnloss, context, allocator, nout, out, nin, in, message);

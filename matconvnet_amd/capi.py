@@ -90,6 +90,8 @@ PROTOTYPES = {
     "mcn_pool_backward": (_i, [_vp, C.POINTER(PoolGeom), _vp, _vp, _vp, _i]),
     "mcn_relu_forward": (_i, [_vp, _vp, _vp, _sz]),
     "mcn_relu_backward": (_i, [_vp, _vp, _vp, _vp, _sz]),
+    "mcn_relu_forward_leaky": (_i, [_vp, _vp, _vp, _sz, _d]),
+    "mcn_relu_backward_leaky": (_i, [_vp, _vp, _vp, _vp, _sz, _d]),
     "mcn_add": (_i, [_vp, _vp, _vp, _vp, _sz]),
     "mcn_fill": (_i, [_vp, _vp, _f, _sz]),
     "mcn_loss_workspace_bytes": (_sz, [C.POINTER(LossGeom)]),
@@ -538,15 +540,21 @@ def loss_backward(x, c, dzdy, g, instance_weights=None):
     return dx
 
 
-def relu_forward(x):
+def relu_forward(x, leak=None):
     y = _torch().empty_like(x)
-    check(lib().mcn_relu_forward(stream(), ptr(y), ptr(x), x.numel()))
+    if leak is None:
+        check(lib().mcn_relu_forward(stream(), ptr(y), ptr(x), x.numel()))
+    else:
+        check(lib().mcn_relu_forward_leaky(stream(), ptr(y), ptr(x), x.numel(), float(leak)))
     return y
 
 
-def relu_backward(x, dy):
+def relu_backward(x, dy, leak=None):
     dx = _torch().empty_like(x)
-    check(lib().mcn_relu_backward(stream(), ptr(dx), ptr(x), ptr(dy), x.numel()))
+    if leak is None:
+        check(lib().mcn_relu_backward(stream(), ptr(dx), ptr(x), ptr(dy), x.numel()))
+    else:
+        check(lib().mcn_relu_backward_leaky(stream(), ptr(dx), ptr(x), ptr(dy), x.numel(), float(leak)))
     return dx
 
 

@@ -11,12 +11,12 @@
 namespace mcn {
 namespace {
 
-enum { OP_RELU_FWD, OP_RELU_BWD, OP_ADD, OP_FILL, OP_AXPBY };
+enum { OP_RELU_FWD, OP_RELU_BWD, OP_ADD, OP_FILL, OP_AXPBY, OP_LRELU_FWD, OP_LRELU_BWD };
 
 template <int OP>
 struct Reads {
   static constexpr bool a = OP != OP_FILL;
-  static constexpr bool b = OP == OP_RELU_BWD || OP == OP_ADD || OP == OP_AXPBY;
+  static constexpr bool b = OP == OP_RELU_BWD || OP == OP_ADD || OP == OP_AXPBY || OP == OP_LRELU_BWD;
 };
 
 template <int OP>
@@ -29,6 +29,10 @@ __device__ __forceinline__ float apply1(float a, float b, float k, float k2) {
     case OP_RELU_FWD: return a > 0.f ? a : 0.f;          // max(x, 0)
     case OP_RELU_BWD: return a > 0.f ? b : b * 0.f;      // dzdy .* (x > 0): keeps NaN/inf*0 semantics
     case OP_ADD: return a + b;
+    // leaky: x .* (leak + (1 - leak)*(x > 0)); k = single(leak), k2 = single(leak + (1 - leak)), the two values the
+    // factor takes (the reference forms it in double and the product in single, matlab/vl_nnrelu.m:49-55)
+    case OP_LRELU_FWD: return a * (a > 0.f ? k2 : k);
+    case OP_LRELU_BWD: return b * (a > 0.f ? k2 : k);
     default: return k;
   }
 }
@@ -134,6 +138,16 @@ extern "C" {
 
 int mcn_relu_forward(mcn_stream_t stream, float* y, const float* x, size_t n) {
   return launch<OP_RELU_FWD>("mcn_relu_forward", stream, y, x, nullptr, 0.f, n);
+}
+int mcn_relu_forward_leaky(mcn_stream_t stream, float* y, const float* x, size_t n, double leak) {
+  if (leak == 0) return launch<OP_RELU_FWD>("mcn_relu_forward_leaky", stream, y, x, nullptr, 0.f, n);
+  return launch<OP_LRELU_FWD>("mcn_relu_forward_leaky", stream, y, x, nullptr, (float)leak, n, (float)(leak + (1.0 - leak)));
+}
+int mcn_relu_backward_leaky(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, size_t n,
+                            double leak) {
+  if (leak == 0) return launch<OP_RELU_BWD>("mcn_relu_backward_leaky", stream, derInput, x, derOutput, 0.f, n);
+  return launch<OP_LRELU_BWD>("mcn_relu_backward_leaky", stream, derInput, x, derOutput, (float)leak, n,
+                              (float)(leak + (1.0 - leak)));
 }
 int mcn_relu_backward(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, size_t n) {
   return launch<OP_RELU_BWD>("mcn_relu_backward", stream, derInput, x, derOutput, 0.f, n);

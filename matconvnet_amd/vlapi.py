@@ -205,6 +205,11 @@ def vl_nnpool(*args):
     return _call("vl_nnpool", 1, list(args))[0]
 
 
+def vl_nnrelu(*args):
+    """vl_nnrelu(x [, dzdy], 'leak', value) (matlab/vl_nnrelu.m)."""
+    return _call("vl_nnrelu", 1, list(args))[0]
+
+
 def vl_nnloss(*args):
     """vl_nnloss(x, c [, dzdy], 'loss', name, 'instanceWeights', w, 'normalise', tf, 'threshold', t, 'topK', k)
     (matlab/vl_nnloss.m): the loss as a 1 x 1 device array, or dzdx when dzdy is given (a number)."""

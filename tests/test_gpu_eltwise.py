@@ -106,3 +106,35 @@ def test_sgd_momentum_arena_matches_the_reference_call_sequence(capi, ob, nester
     for off, c in zip(offsets, counts):
         pad[off:off + c] = False
     assert not got_v[pad].any() and not got_s[pad].any()
+
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+def test_leaky_relu(capi, ob, vl, n):
+    """vl_nnrelu with a leak (matlab/vl_nnrelu.m:49-55): y = x .* (leak + (1 - leak)*(x > 0)).  Pinned by what the
+    definition fixes: leak 0 is the plain ReLU bit for bit (the oracle's), leak 1 the identity, positive inputs pass
+    unchanged, negative ones come out as single(leak)*x exactly, and the derivative multiplies by the same factor."""
+    import torch
+    r = np.random.default_rng(n)
+    x = r.standard_normal(n).astype(np.float32)
+    x[::5] = 0.0
+    dy = r.standard_normal(n).astype(np.float32)
+    xd, dyd = capi.to_device(x), capi.to_device(dy)
+    assert bits_equal(capi.to_host(capi.relu_forward(xd, leak=0.0)), ob.relu_forward(x))
+    assert bits_equal(capi.to_host(capi.relu_backward(xd, dyd, leak=0.0)), ob.relu_backward(x, dy))
+    assert bits_equal(capi.to_host(capi.relu_forward(xd, leak=1.0)), x * np.float32(1))
+    for leak in (0.1, 0.01, 0.3):
+        y = capi.to_host(capi.relu_forward(xd, leak=leak))
+        dx = capi.to_host(capi.relu_backward(xd, dyd, leak=leak))
+        pos = x > 0
+        one = np.float32(leak + (1.0 - leak))
+        assert bits_equal(y[pos], x[pos] * one) and bits_equal(y[~pos], x[~pos] * np.float32(leak))
+        assert bits_equal(dx[pos], dy[pos] * one) and bits_equal(dx[~pos], dy[~pos] * np.float32(leak))
+        # through the front-end, options by name
+        yt = vl.vl_nnrelu(xd.reshape(1, 1, 1, n), "Leak", leak)
+        assert bits_equal(yt.cpu().numpy().ravel(), y)
+        dt = vl.vl_nnrelu(xd.reshape(1, 1, 1, n), dyd.reshape(1, 1, 1, n), "leak", leak)
+        assert bits_equal(dt.cpu().numpy().ravel(), dx)
+    assert bits_equal(vl.vl_nnrelu(xd.reshape(1, 1, 1, n)).cpu().numpy().ravel(), ob.relu_forward(x))
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnrelu(xd, "leek", 0.1)
+    assert e.value.message == "Unknown option 'leek'."
