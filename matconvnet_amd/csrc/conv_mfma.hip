@@ -760,7 +760,14 @@ int wgrad_splits(const ConvP& p, int* tilesOut) {
   const int BA = pick_channels_tile(p.K), BB = pick_rows_tile(p);
   const int tiles = ((p.K + BA - 1) / BA) * ((p.FH * p.FW * p.FC + BB - 1) / BB);
   int target = tunable("conv_wgrad_blocks", 0);
-  if (target <= 0) target = 512;
+  // two workgroups per CU; one when a workgroup's share of a 1x1 layer would be under ~10 MFLOP with several tiles
+  // to write (the partial banks then cost more than the idle half: 14x14 and 7x7 1x1 layers of ResNet-50 at 32
+  // images 46.6 -> 44.8 us, 54.6 -> 50.0 us), or when the whole bank is one tile
+  if (target <= 0) {
+    const double flops = 2.0 * p.outH * p.outW * p.N * (double)p.FH * p.FW * p.FC * p.K;
+    const bool small1x1 = p.FH * p.FW == 1 && flops < 5e9 && (tiles >= 4 || tiles == 1);
+    target = small1x1 && !tunable("conv_wgrad_no_small_rule", 0) ? 256 : 512;
+  }
   const long long chunks = ((long long)p.outH * p.outW * p.N + 31) / 32;
   long long s = std::max<long long>(1, target / tiles);
   s = std::min<long long>(s, std::max<long long>(1, chunks / 4));  // at least 4 reduction steps per split
