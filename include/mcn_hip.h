@@ -354,6 +354,12 @@ MCN_API int mcn_loss_backward(mcn_stream_t stream, const mcn_loss_geom* g, float
                               const float* labels, size_t nLabels, const float* instanceWeights, size_t nWeights,
                               double derOutput);
 
+/* softmax over the channels (matlab/vl_nnsoftmax.m:20-28; the 'prob' layer a deployed network ends with):
+   y = exp(x - max) / sum;  dzdx = y .* (dzdy - sum over the channels of dzdy .* y) */
+MCN_API int mcn_softmax_forward(mcn_stream_t stream, float* y, const float* x, int H, int W, int C, int N);
+MCN_API int mcn_softmax_backward(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, int H, int W,
+                                 int C, int N);
+
 /* ------------------------------------------------------------------------------------------------
  * double precision -- the operators' VLDT_Double instantiation (bits/impl/dispatcher.hpp:60-98 switches on the
  * tensors' data type; bits/nnconv.cu:444-469, bits/nnbnorm.cu:388-442, bits/nnpooling.cu:270-282 instantiate

@@ -677,6 +677,32 @@ void nnrelu(Context& context, Allocator& allocator, int nout, Tensor* out, int n
   (void)nout;
 }
 
+// ------------------------------------------------------------------------------------------ vl_nnsoftmax
+// matlab/vl_nnsoftmax.m:20-28: (x [, dzdy])
+
+void nnsoftmax(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in) {
+  if (nin < 1) raise(VLE_IllegalArgument, "There are no arguments.");
+  if (nin > 2) raise(VLE_IllegalArgument, "There are more than two arguments.");
+  Tensor x = dataTensor(in[0], "X", 4);
+  if (x.getDeviceType() != VLDT_GPU) raise(VLE_Unsupported, "vl_nnsoftmax: X is on the CPU; this library implements the GPU (HIP, gfx950) device only");
+  if (x.getDataType() != VLDT_Float) raise(VLE_Unsupported, "vl_nnsoftmax: only single precision is implemented on the HIP device");
+  void* stream = context.getHipHelper().getStream();
+  Tensor y = newOutput(allocator, VLDT_GPU, VLDT_Float, in[0].tensor.getShape());
+  const int H = (int)x.getHeight(), W = (int)x.getWidth(), C = (int)x.getDepth(), N = (int)x.getSize();
+  int rc;
+  if (nin < 2) {
+    rc = mcn_softmax_forward(stream, (float*)y.getMemory(), (float const*)x.getMemory(), H, W, C, N);
+  } else {
+    Tensor dzdy = dataTensor(in[1], "DZDY", 4);
+    if (!areCompatible(x, dzdy)) raise(VLE_IllegalArgument, "X and DZDY do not have compatible formats.");
+    if (dzdy.getNumElements() != x.getNumElements()) raise(VLE_IllegalArgument, "X and DZDY do not have the same number of elements.");
+    rc = mcn_softmax_backward(stream, (float*)y.getMemory(), (float const*)x.getMemory(), (float const*)dzdy.getMemory(), H, W, C, N);
+  }
+  if (rc) raise(rc > 0 && rc <= (int)VLE_Interrupted ? (ErrorCode)rc : VLE_Unknown, mcn_last_error_message());
+  out[0] = y;
+  (void)nout;
+}
+
 typedef void (*Body)(Context&, Allocator&, int, Tensor*, int, Arg const*);
 
 ErrorCode guarded(Body body, Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
@@ -708,6 +734,9 @@ ErrorCode vl_nnpool(Context& context, Allocator& allocator, int nout, Tensor* ou
 }
 ErrorCode vl_taccum(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
   return guarded(taccum, context, allocator, nout, out, nin, in, message);
+}
+ErrorCode vl_nnsoftmax(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
+  return guarded(nnsoftmax, context, allocator, nout, out, nin, in, message);
 }
 ErrorCode vl_nnrelu(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in, std::string& message) {
   return guarded(nnrelu, context, allocator, nout, out, nin, in, message);

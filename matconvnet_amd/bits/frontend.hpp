@@ -50,6 +50,7 @@ class Allocator {
 //   vl_taccum : [alpha*a + beta*b]; nothing with 'InPlace' (a itself is updated)
 //   vl_nnloss : forward [y] (1 x 1 on the device)   backward [dzdx]
 //   vl_nnrelu : forward [y]             backward [dzdx]
+//   vl_nnsoftmax: forward [y]           backward [dzdx]
 ErrorCode vl_nnconv(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                     std::string& message);
 ErrorCode vl_nnconvt(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
@@ -63,6 +64,9 @@ ErrorCode vl_taccum(Context& context, Allocator& allocator, int nout, Tensor* ou
 // vl_nnrelu(x [, dzdy], 'leak', value)  (matlab/vl_nnrelu.m:33-55; a MATLAB function in the reference)
 ErrorCode vl_nnrelu(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
                     std::string& message);
+// vl_nnsoftmax(x [, dzdy])  (matlab/vl_nnsoftmax.m:20-28; a MATLAB function in the reference)
+ErrorCode vl_nnsoftmax(Context& context, Allocator& allocator, int nout, Tensor* out, int nin, Arg const* in,
+                       std::string& message);
 // vl_nnloss(x, c [, dzdy], 'loss', name, 'instanceWeights', w, 'normalise', tf, 'threshold', t, 'topK', k)
 // (matlab/vl_nnloss.m:129-142; a MATLAB function in the reference).  x: single, on the device.  c and the instance
 // weights: on the device (single) or host arrays (copied over).  dzdy: a host scalar, or empty for the forward mode.

@@ -48,7 +48,7 @@ void fromTensor(Tensor const& t, vlh_arg* a) {
 
 // one context per front-end function, like the static vl::MexContext of each MEX file
 Context& contextOf(int which) {
-  static Context contexts[7];
+  static Context contexts[8];
   return contexts[which];
 }
 
@@ -95,7 +95,7 @@ int vlh_call(const char* function, int nout, vlh_arg* out, int nin, const vlh_ar
     g_message = "vlh_call: null argument";
     return VLE_IllegalArgument;
   }
-  int which = !std::strcmp(function, "vl_nnconv") ? 0 : !std::strcmp(function, "vl_nnbnorm") ? 1 : !std::strcmp(function, "vl_nnpool") ? 2 : !std::strcmp(function, "vl_nnconvt") ? 3 : !std::strcmp(function, "vl_taccum") ? 4 : !std::strcmp(function, "vl_nnloss") ? 5 : !std::strcmp(function, "vl_nnrelu") ? 6 : -1;
+  int which = !std::strcmp(function, "vl_nnconv") ? 0 : !std::strcmp(function, "vl_nnbnorm") ? 1 : !std::strcmp(function, "vl_nnpool") ? 2 : !std::strcmp(function, "vl_nnconvt") ? 3 : !std::strcmp(function, "vl_taccum") ? 4 : !std::strcmp(function, "vl_nnloss") ? 5 : !std::strcmp(function, "vl_nnrelu") ? 6 : !std::strcmp(function, "vl_nnsoftmax") ? 7 : -1;
   if (which < 0) {
     g_message = std::string("vlh_call: unknown function '") + function + "'";
     return VLE_IllegalArgument;
@@ -117,6 +117,7 @@ int vlh_call(const char* function, int nout, vlh_arg* out, int nin, const vlh_ar
   else if (which == 4) e = frontend::vl_taccum(context, allocator, nout, results, nin, a, g_message);
   else if (which == 5) e = frontend::vl_nnloss(context, allocator, nout, results, nin, a, g_message);
   else if (which == 6) e = frontend::vl_nnrelu(context, allocator, nout, results, nin, a, g_message);
+  else if (which == 7) e = frontend::vl_nnsoftmax(context, allocator, nout, results, nin, a, g_message);
   else e = frontend::vl_nnpool(context, allocator, nout, results, nin, a, g_message);
   for (int i = 0; i < 4; ++i) fromTensor(results[i], &out[i]);
   return (int)e;

@@ -94,6 +94,8 @@ PROTOTYPES = {
     "mcn_relu_backward_leaky": (_i, [_vp, _vp, _vp, _vp, _sz, _d]),
     "mcn_add": (_i, [_vp, _vp, _vp, _vp, _sz]),
     "mcn_fill": (_i, [_vp, _vp, _f, _sz]),
+    "mcn_softmax_forward": (_i, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "mcn_softmax_backward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     "mcn_loss_workspace_bytes": (_sz, [C.POINTER(LossGeom)]),
     "mcn_loss_forward": (_i, [_vp, C.POINTER(LossGeom), _vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz]),
     "mcn_loss_backward": (_i, [_vp, C.POINTER(LossGeom), _vp, _vp, _vp, _sz, _vp, _sz, _d]),
@@ -514,6 +516,20 @@ def pool_backward(x, dy, g, dx=None):
         dx = empty((g.H, g.W, g.C, g.N), like=dy)
     fn = lib().mcn_pool_backward_f64 if _is64(x, dy, dx) else lib().mcn_pool_backward
     check(fn(stream(), C.byref(g), ptr(dx), ptr(x), ptr(dy), int(acc)))
+    return dx
+
+
+def softmax_forward(x):
+    H, W, Cc, N = _hwcn(x)
+    y = _torch().empty_like(x)
+    check(lib().mcn_softmax_forward(stream(), ptr(y), ptr(x), H, W, Cc, N))
+    return y
+
+
+def softmax_backward(x, dzdy):
+    H, W, Cc, N = _hwcn(x)
+    dx = _torch().empty_like(x)
+    check(lib().mcn_softmax_backward(stream(), ptr(dx), ptr(x), ptr(dzdy), H, W, Cc, N))
     return dx
 
 

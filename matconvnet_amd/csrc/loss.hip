@@ -144,6 +144,33 @@ __global__ __launch_bounds__(256) void loss_categorical(float* __restrict__ out,
   }
 }
 
+// vl_nnsoftmax (matlab/vl_nnsoftmax.m:20-28): y = exp(x - max) / sum over the channels; with dzdy:
+// dzdx = y .* (dzdy - sum(dzdy .* y)).  One prediction vector per LANES lanes, like the losses.
+template <int LANES, bool BACKWARD>
+__global__ __launch_bounds__(256) void softmax_kernel(float* __restrict__ out, const float* __restrict__ x,
+                                                      const float* __restrict__ dzdy, int HW, int C, size_t items) {
+  const size_t item = ((size_t)blockIdx.x * 256 + threadIdx.x) / LANES;
+  const int lane = LANES > 1 ? (int)(threadIdx.x & (LANES - 1)) : 0;
+  if (item >= items) return;
+  const size_t n = item / HW, q = item - n * HW;
+  const size_t base = n * (size_t)HW * C + q;
+  float xmax = -__builtin_inff();
+  for (int c = lane; c < C; c += LANES) xmax = fmaxf(xmax, x[base + (size_t)c * HW]);
+  xmax = lanes_max<LANES>(xmax);
+  float sumex = 0.f;
+  for (int c = lane; c < C; c += LANES) sumex += expf(x[base + (size_t)c * HW] - xmax);
+  sumex = lanes_sum<LANES>(sumex);
+  float dot = 0.f;
+  if (BACKWARD) {
+    for (int c = lane; c < C; c += LANES) dot += dzdy[base + (size_t)c * HW] * (expf(x[base + (size_t)c * HW] - xmax) / sumex);
+    dot = lanes_sum<LANES>(dot);
+  }
+  for (int c = lane; c < C; c += LANES) {
+    const float y = expf(x[base + (size_t)c * HW] - xmax) / sumex;
+    out[base + (size_t)c * HW] = BACKWARD ? y * (dzdy[base + (size_t)c * HW] - dot) : y;
+  }
+}
+
 // attribute losses: one label per element
 template <bool BACKWARD>
 __global__ __launch_bounds__(256) void loss_binary(float* __restrict__ out, const float* __restrict__ x,
@@ -253,6 +280,28 @@ int launch_items(hipStream_t s, const char* who, float* out, const float* x, con
   return check_launch(who);
 }
 
+int softmax(const char* who, mcn_stream_t stream, float* out, const float* x, const float* dzdy, int H, int W, int C, int N) {
+  if (H < 0 || W < 0 || C < 0 || N < 0) return fail(MCN_ILLEGAL_ARGUMENT, "%s: negative tensor extent", who);
+  if ((long long)H * W >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: plane too large", who);
+  const size_t items = (size_t)H * W * N;
+  if (items == 0 || C == 0) return MCN_SUCCESS;
+  if (!out || !x) return fail(MCN_ILLEGAL_ARGUMENT, "%s: null tensor", who);
+  const bool wide = items < 16384;
+  const size_t blocks = ((wide ? items * 64 : items) + 255) / 256;
+  if (blocks >= (1ull << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
+  hipStream_t s = as_stream(stream);
+  KernelTimer timer("softmax_kernel", s);
+  const dim3 grid((unsigned)blocks), block(256);
+  if (dzdy) {
+    if (wide) hipLaunchKernelGGL((softmax_kernel<64, true>), grid, block, 0, s, out, x, dzdy, H * W, C, items);
+    else hipLaunchKernelGGL((softmax_kernel<1, true>), grid, block, 0, s, out, x, dzdy, H * W, C, items);
+  } else {
+    if (wide) hipLaunchKernelGGL((softmax_kernel<64, false>), grid, block, 0, s, out, x, dzdy, H * W, C, items);
+    else hipLaunchKernelGGL((softmax_kernel<1, false>), grid, block, 0, s, out, x, dzdy, H * W, C, items);
+  }
+  return check_launch(who);
+}
+
 }  // namespace
 }  // namespace mcn
 
@@ -297,6 +346,16 @@ int mcn_loss_backward(mcn_stream_t stream, const mcn_loss_geom* g, float* derInp
   if (!derInput || !x || !labels) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_loss_backward: null tensor");
   return launch_items<true>(as_stream(stream), "mcn_loss_backward", derInput, x, labels, instanceWeights, (float)derOutput, p,
                             items);
+}
+
+int mcn_softmax_forward(mcn_stream_t stream, float* y, const float* x, int H, int W, int C, int N) {
+  return softmax("mcn_softmax_forward", stream, y, x, nullptr, H, W, C, N);
+}
+
+int mcn_softmax_backward(mcn_stream_t stream, float* derInput, const float* x, const float* derOutput, int H, int W, int C,
+                         int N) {
+  if (!derOutput && (size_t)H * W * C * N != 0) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_softmax_backward: null tensor");
+  return softmax("mcn_softmax_backward", stream, derInput, x, derOutput, H, W, C, N);
 }
 
 }  // extern "C"

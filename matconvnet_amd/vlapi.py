@@ -210,6 +210,11 @@ def vl_nnrelu(*args):
     return _call("vl_nnrelu", 1, list(args))[0]
 
 
+def vl_nnsoftmax(*args):
+    """vl_nnsoftmax(x [, dzdy]) (matlab/vl_nnsoftmax.m)."""
+    return _call("vl_nnsoftmax", 1, list(args))[0]
+
+
 def vl_nnloss(*args):
     """vl_nnloss(x, c [, dzdy], 'loss', name, 'instanceWeights', w, 'normalise', tf, 'threshold', t, 'topK', k)
     (matlab/vl_nnloss.m): the loss as a 1 x 1 device array, or dzdx when dzdy is given (a number)."""

@@ -126,3 +126,15 @@ def vl_nnloss(x, c, dzdy=None, loss="softmaxlog", instance_weights=None, normali
     if normalise:                                                             # :313-315
         y = y / T(N)
     return np.asfortranarray(y)
+
+
+def vl_nnsoftmax(x, dzdy=None):
+    """matlab/vl_nnsoftmax.m:20-28, statement by statement.  Pinned by: rows sum to 1, shift invariance, the
+    derivative against a numerical one, sum over the channels of dzdx = 0 (tests/test_oracle_loss.py)."""
+    x = np.asarray(x)
+    e = np.exp(x - x.max(axis=2, keepdims=True))
+    y = e / e.sum(axis=2, keepdims=True, dtype=x.dtype)
+    if dzdy is None:
+        return np.asfortranarray(y.astype(x.dtype))
+    dzdy = np.asarray(dzdy, dtype=x.dtype)
+    return np.asfortranarray((y * (dzdy - (dzdy * y).sum(axis=2, keepdims=True, dtype=x.dtype))).astype(x.dtype))

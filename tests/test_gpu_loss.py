@@ -138,3 +138,30 @@ def test_front_end_vl_nnloss(vl):
     with pytest.raises(vl.VlError) as e:
         vl.vl_nnloss(dev(x, np.float64), host(c))
     assert e.value.code == 1
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1000, 32), (4, 5, 3, 3), (1, 1, 1, 4), (100, 90, 5, 2)])
+def test_softmax(capi, shape):
+    r = np.random.default_rng(9)
+    x = F(r.standard_normal(shape) * 3)
+    dzdy = F(r.standard_normal(shape))
+    xd = capi.to_device(x)
+    y = capi.to_host(capi.softmax_forward(xd)).reshape(shape, order="F")
+    assert rel_max(y, ol.vl_nnsoftmax(x)) < 1e-5 and np.abs(y.sum(axis=2) - 1).max() < 1e-5
+    dx = capi.to_host(capi.softmax_backward(xd, capi.to_device(dzdy))).reshape(shape, order="F")
+    want = ol.vl_nnsoftmax(x, dzdy)
+    assert (rel_max(dx, want) < 1e-5) if shape[2] > 1 else (np.abs(dx).max() < 1e-6)
+
+
+def test_front_end_vl_nnsoftmax(vl):
+    import torch
+    r = np.random.default_rng(10)
+    x, dzdy = F(r.standard_normal((3, 2, 7, 4))), F(r.standard_normal((3, 2, 7, 4)))
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a.T)).cuda()
+    y = vl.vl_nnsoftmax(dev(x))
+    assert rel_max(np.asfortranarray(y.cpu().numpy().T), ol.vl_nnsoftmax(x)) < 1e-5
+    dx = vl.vl_nnsoftmax(dev(x), dev(dzdy))
+    assert rel_max(np.asfortranarray(dx.cpu().numpy().T), ol.vl_nnsoftmax(x, dzdy)) < 1e-5
+    with pytest.raises(vl.VlError) as e:
+        vl.vl_nnsoftmax(dev(x), dev(dzdy[:, :, :3]))
+    assert e.value.message == "X and DZDY do not have the same number of elements."

@@ -126,3 +126,22 @@ def test_one_label_per_image_is_broadcast_over_the_pixels():
     full = np.broadcast_to(c.reshape(1, 1, 1, 4), (3, 2, 1, 4))
     assert float(ol.vl_nnloss(x, c, None)) == float(ol.vl_nnloss(x, full, None))
     assert np.array_equal(ol.vl_nnloss(x, c, 0.5), ol.vl_nnloss(x, full, 0.5))
+
+
+def test_softmax_properties_and_numerical_derivative():
+    r = np.random.default_rng(4)
+    x = r.standard_normal((3, 4, 6, 2))
+    y = ol.vl_nnsoftmax(x)
+    assert np.abs(y.sum(axis=2) - 1).max() < 1e-14 and (y > 0).all()
+    assert np.abs(ol.vl_nnsoftmax(x + 7.5) - y).max() < 1e-14
+    assert np.abs(ol.vl_nnsoftmax(np.zeros((1, 1, 5, 1))) - 0.2).max() < 1e-16
+    dzdy = r.standard_normal(x.shape)
+    dzdx = ol.vl_nnsoftmax(x, dzdy)
+    assert np.abs(dzdx.sum(axis=2)).max() < 1e-14
+    for _ in range(30):
+        i = tuple(int(r.integers(0, s)) for s in x.shape)
+        xp, xm = x.copy(), x.copy()
+        xp[i] += 1e-6
+        xm[i] -= 1e-6
+        num = ((ol.vl_nnsoftmax(xp) - ol.vl_nnsoftmax(xm)) / 2e-6 * dzdy).sum()
+        assert abs(num - dzdx[i]) < 1e-8
