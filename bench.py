@@ -309,7 +309,7 @@ def cpu_baseline(workloads):
     blocks.bottleneck(workloads.bottleneck_case(N=2))  # warm the threads and pages
     t0 = time.perf_counter()
     reps = 0
-    while reps < 1 or (time.perf_counter() - t0 < 8.0 and reps < 4):
+    while reps < 1 or (time.perf_counter() - t0 < 12.0 and reps < 20):   # about 12 s of CPU work
         blocks.bottleneck(w)
         reps += 1
     dt = (time.perf_counter() - t0) / reps
