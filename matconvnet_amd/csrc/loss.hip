@@ -91,6 +91,7 @@ __global__ __launch_bounds__(256) void loss_categorical(float* __restrict__ out,
   float qmax = -__builtin_inff();   // the same leaving the label's channel out (mshinge)
   int iq = 0x7fffffff;
   int above = 0;                    // channels ranked before the label's by a stable descending sort
+#pragma unroll 8
   for (int c = lane; c < p.C; c += LANES) {
     const float v = xv[(size_t)c * p.HW];
     if (v > xmax) { xmax = v; imax = c; }
@@ -102,6 +103,7 @@ __global__ __launch_bounds__(256) void loss_categorical(float* __restrict__ out,
   above = lanes_sum<LANES>(above);
   float sumex = 0.f;
   if (p.kind == MCN_LOSS_SOFTMAXLOG) {
+#pragma unroll 8
     for (int c = lane; c < p.C; c += LANES) sumex += expf(xv[(size_t)c * p.HW] - xmax);
     sumex = lanes_sum<LANES>(sumex);
   }
@@ -121,6 +123,7 @@ __global__ __launch_bounds__(256) void loss_categorical(float* __restrict__ out,
   }
   const float dz = dzdy * w;   // :275-277
   float* ov = out + n * (size_t)p.HW * p.C + q;
+#pragma unroll 8
   for (int c = lane; c < p.C; c += LANES) {
     float y = 0.f;
     switch (p.kind) {
@@ -155,16 +158,20 @@ __global__ __launch_bounds__(256) void softmax_kernel(float* __restrict__ out, c
   const size_t n = item / HW, q = item - n * HW;
   const size_t base = n * (size_t)HW * C + q;
   float xmax = -__builtin_inff();
+#pragma unroll 8
   for (int c = lane; c < C; c += LANES) xmax = fmaxf(xmax, x[base + (size_t)c * HW]);
   xmax = lanes_max<LANES>(xmax);
   float sumex = 0.f;
+#pragma unroll 8
   for (int c = lane; c < C; c += LANES) sumex += expf(x[base + (size_t)c * HW] - xmax);
   sumex = lanes_sum<LANES>(sumex);
   float dot = 0.f;
   if (BACKWARD) {
+#pragma unroll 8
     for (int c = lane; c < C; c += LANES) dot += dzdy[base + (size_t)c * HW] * (expf(x[base + (size_t)c * HW] - xmax) / sumex);
     dot = lanes_sum<LANES>(dot);
   }
+#pragma unroll 8
   for (int c = lane; c < C; c += LANES) {
     const float y = expf(x[base + (size_t)c * HW] - xmax) / sumex;
     out[base + (size_t)c * HW] = BACKWARD ? y * (dzdy[base + (size_t)c * HW] - dot) : y;
