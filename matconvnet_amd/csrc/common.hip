@@ -44,6 +44,7 @@ Tunable g_tunables[] = {
     {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels
     {"conv_pix_tile", 0},              // force a tile shape of the pixel-major MFMA kernel (0 = automatic)
     {"conv_no_uniform_tap", 0},        // 1: disable the uniform-tap variant of the pixel-major kernel
+    {"conv_wgrad_no_wide_rows", 0},    // 1: no 192-row filter-gradient tiles
     {"conv_wgrad_no_small_rule", 0},   // 1: always two filter-gradient workgroups per CU
     {"conv_wgrad_blocks", 0},          // target workgroups for filter-gradient split (0 = 2 per CU)
     {"conv_bias_blocks", 0},           // target workgroups for the bias-gradient reduction

@@ -554,3 +554,24 @@ def test_few_output_channels(capi, ob, xs, fs, stride, pad, dilate):
         assert rel_max(capi.to_host(dx), wdx) < 2e-4
         assert rel_max(capi.to_host(dx2), dbase.astype(np.float64) + wdx) < 2e-4
     assert got[0] >= 2 and got[1] == 0   # the kernel ran (at least the two products of the few-channel side)
+
+
+@pytest.mark.parametrize("xs,fs,stride,pad", [((30, 29, 3, 3), (7, 7, 3, 64), 2, 3), ((14, 15, 32, 2), (1, 5, 32, 40), 1, (0, 0, 2, 2)),
+                                               ((12, 12, 20, 2), (3, 3, 20, 64), 1, 1)])
+def test_filter_gradient_wide_row_tile(capi, ob, xs, fs, stride, pad):
+    """Filter volumes of 129...192 rows with up to 64 filters take one 192-row tile (a ResNet stem: 7x7x3 = 147 rows):
+    against the oracle, with that tile and with the 128-row tiles."""
+    r = np.random.default_rng(sum(xs) + sum(fs))
+    x = F(r.standard_normal(xs))
+    f = F(r.standard_normal(fs) * 0.1)
+    g = ob.conv_geom(xs, fs, stride, pad, 1)
+    cg = capi.conv_geom(xs, fs, stride, pad, 1)
+    dy = F(r.standard_normal(capi.conv_out_shape(cg)))
+    want = ob.conv_backward(x, f, dy, g, want=(False, True, False))[1]
+    for off in (0, 1):
+        capi.set_tunable("conv_wgrad_no_wide_rows", off)
+        try:
+            _, df, _ = capi.conv_backward(capi.to_device(x), capi.to_device(f), capi.to_device(dy), cg, want=(False, True, False))
+        finally:
+            capi.set_tunable("conv_wgrad_no_wide_rows", 0)
+        assert rel_max(capi.to_host(df), want) < 2e-4
