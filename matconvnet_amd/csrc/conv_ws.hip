@@ -351,8 +351,12 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
       const long long units = pixelBlocks * (p.coutPad / (32 * cand));
       const double balance = (double)units / (double)(((units + simds - 1) / simds) * simds);
       const double issue = cand == 4 ? 0.96 : (cand == 2 ? 0.94 : 0.90);
-      if (balance * issue > best) {
-        best = balance * issue;
+      // under four units per SIMD a wide unit no longer pays: the loads of a few long units per SIMD are hidden worse
+      // than those of many short ones (stride classes of 3x3 /2 128->128: 130 -> 118 us with the narrowest), so any
+      // shape that fills the SIMDs four deep wins over one that does not, and among those that do not the narrowest
+      const double score = units >= 4 * simds ? balance * issue : 0.01 / cand;
+      if (score > best) {
+        best = score;
         WA = cand;
       }
     }
