@@ -38,7 +38,7 @@ Tunable g_tunables[] = {
     {"conv_no_split", 0},              // 1: the tiled kernel never splits its reduction over workgroups
     {"conv_split_max_blocks", 512},    // ... it splits when the unsplit launch has at most this many workgroups,
     {"conv_split_target", 1024},       // aiming at this many workgroups in all,
-    {"conv_split_min_steps", 16},      // with at least this many 16-row steps left to each
+    {"conv_split_min_steps", 12},      // with at least this many 16-row steps left to each
     {"conv_split_force", 0},           // n > 0: exactly n splits (experiments)
     {"conv_no_fc_view", 0},            // 1: fully-connected layers are not recast as 1x1 layers
     {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels

@@ -850,14 +850,14 @@ PixPlan plan_pix(int Cout, long long M, int R) {
     static const int pxOf[8] = {0, 128, 256, 256, 128, 64, 64, 32}, baOf[8] = {0, 128, 64, 32, 64, 128, 64, 128};
     if (forced >= 1 && forced <= 7 && baOf[forced] == BA) { plan.shape = forced; px = pxOf[forced]; }
   }
-  // fewer than two workgroups per CU with a long reduction each: split it, down to 16 steps of 16 rows per
+  // fewer than two workgroups per CU with a long reduction each: split it, down to 12 steps of 16 rows per
   // workgroup, until about four workgroups per CU exist (values from a sweep over the 14x14 and 7x7 layers of
   // ResNet-50 at 32 images: 126 -> 89 us for 3x3x256x256)
   plan.splits = 1;
   const long long nb = blocks(px);
   const int nSteps = (R + 15) / 16;
   const int maxBlocks = tunable("conv_split_max_blocks", 512), target = tunable("conv_split_target", 1024),
-            minSteps = tunable("conv_split_min_steps", 16);
+            minSteps = tunable("conv_split_min_steps", 12);
   if (nb <= maxBlocks && nSteps >= 4 * minSteps && !tunable("conv_no_split", 0)) {
     long long want = (target + nb - 1) / nb;
     plan.splits = (int)std::max<long long>(1, std::min<long long>(want, nSteps / minSteps));

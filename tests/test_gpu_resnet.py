@@ -374,13 +374,13 @@ def test_loss_layers_and_a_few_training_steps(vl, case):
         got = net.get("dprediction").reshape(1, 1, CLASSES, N, order="F")
         assert rel_max(got, want) < 1e-5 and not got[..., -1].any()
         first = objective
-        for _ in range(8):
+        for _ in range(12):   # (a rate at which the trajectory is stable: at 0.05 the loss of this batch bounces)
             net.forward()
             net.loss_derivative()
             net.backward()
-            net.sgd_step(0.05, 0.9, 1e-4)
+            net.sgd_step(0.01, 0.9, 1e-4)
         net.forward()
         last = net.losses()[0]
-        assert np.isfinite(last) and last < 0.7 * first, (first, last)
+        assert np.isfinite(last) and last < 0.3 * first, (first, last)
     finally:
         net.close()
