@@ -34,6 +34,7 @@ Tunable g_tunables[] = {
     {"conv_ws_min_units", 0},          // least number of units for the weights-stationary kernel; 0 = one per two SIMDs
     {"conv_ws_max_slices", 8},         // most slices of output channels its bank may be cut into (1: whole banks only)
     {"conv_ws_sliced_strided", 0},     // 1: sliced banks also for strided gathers (slower than the tiled kernel)
+    {"conv_ws_fill", 4},               // units per SIMD from which its wide units are considered
     {"conv_ws_wa", 0},                 // 1, 2, 4: force its channels-per-wavefront (in units of 32); 0 = choose
     {"conv_no_split", 0},              // 1: the tiled kernel never splits its reduction over workgroups
     {"conv_split_max_blocks", 512},    // ... it splits when the unsplit launch has at most this many workgroups,

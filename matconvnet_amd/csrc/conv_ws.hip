@@ -354,7 +354,7 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
       // under four units per SIMD a wide unit no longer pays: the loads of a few long units per SIMD are hidden worse
       // than those of many short ones (stride classes of 3x3 /2 128->128: 130 -> 118 us with the narrowest), so any
       // shape that fills the SIMDs four deep wins over one that does not, and among those that do not the narrowest
-      const double score = units >= 4 * simds ? balance * issue : 0.01 / cand;
+      const double score = units >= tunable("conv_ws_fill", 4) * simds ? balance * issue : 0.01 / cand;
       if (score > best) {
         best = score;
         WA = cand;
