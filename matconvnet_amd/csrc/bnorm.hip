@@ -2,9 +2,10 @@
 //
 // Two launches per call:
 //   1. bnorm_sums  -- grid (channel, image-group).  Each workgroup streams its planes of x (and dzdy)
-//      once with 16-byte loads, keeps fp32 running sums per lane for one plane at a time, folds them into
-//      fp64 per plane, reduces across the wavefront with shuffles and across wavefronts through LDS, and
-//      writes one fp64 partial per (channel, group): sum x, sum x^2, sum x*dzdy, sum dzdy.
+//      once with 16-byte loads, widens every element to fp64 and keeps fp64 running sums per lane (the
+//      kernel waits on memory, the fp64 arithmetic is hidden), reduces across the wavefront with shuffles and
+//      across wavefronts through LDS, and writes one fp64 partial per (channel, group): sum x, sum x^2,
+//      sum x*dzdy, sum dzdy.
 //   2. bnorm_apply -- same grid.  Each workgroup re-reduces its channel's partials in a fixed order
 //      (deterministic), derives mean / sigma / dzdg / dzdb in fp64 exactly as the reference formulas
 //      (bits/nnbnorm.cu:101-164), and streams the elementwise result
@@ -13,9 +14,11 @@
 //   The apply pass can walk the planes in the reverse order of the sums pass so that it starts on the
 //   data most recently pulled through the caches.
 //
-// Accuracy: the reference sums ~1e5 terms sequentially in float; here at most one plane-slice per lane
-// is summed in fp32 and everything above is fp64, so results sit close to the reference's own
-// double-precision instantiation.
+// Accuracy: the reference sums ~1e5 terms sequentially in the data type.  Here every product and every sum is
+// fp64 (the inputs are float, so each product is exact), which puts the results next to the reference's own
+// double-precision instantiation run on the same float data -- also where the one-pass variance
+// E[x^2] - mean^2 cancels many digits (a constant channel, a channel with |mean| >> sigma), where a float
+// accumulation -- the reference's included -- keeps nothing of the variance.
 #include "mcn_internal.hpp"
 
 #include <algorithm>
@@ -39,13 +42,17 @@ __device__ __forceinline__ void image_range(const BnormP& p, int grp, int* n0, i
   *n1 = (int)(((long long)p.N * (grp + 1)) / p.groups);
 }
 
-// y = a*x + k with the rounding of the forward pass: the moments as stored (float), everything else in double,
-// the two coefficients rounded to float once.  Forward and the ReLU-masked backward both go through here, so
-// that "a*x + k > 0" decides the same way in both.
-__device__ __forceinline__ void forward_coefficients(double mean, double sigma, float mult, float bias, float* a, float* k) {
+// y = a*(x - s) + k with the rounding of the forward pass: the moments as stored (float), everything else in
+// double, the coefficients rounded to float once.  s is the mean rounded to float, taken off x first (as the
+// reference's (x - mean)*coef + b does, bits/nnbnorm.cu:190-199): with a channel whose mean is large against its
+// sigma, a*x and k would be two huge numbers that cancel.  k carries what the rounding of the mean left over.
+// Forward and the ReLU-masked backward both go through here, so that "a*(x - s) + k > 0" decides the same way in both.
+__device__ __forceinline__ void forward_coefficients(double mean, double sigma, float mult, float bias, float* a, float* k,
+                                                     float* s) {
   const double coef = (double)mult / sigma;
+  *s = (float)mean;
   *a = (float)coef;
-  *k = (float)((double)bias - coef * mean);
+  *k = (float)((double)bias - coef * (mean - (double)*s));
 }
 
 // Block-wide sum of NV doubles held per thread; result valid in thread 0.
@@ -75,23 +82,23 @@ __device__ __forceinline__ void block_sum(double (&v)[NV], double* lds /* [4][NV
 // passes that follow (this layer's apply pass, and whoever else consumes it).
 template <int MODE, bool VEC4, bool RELU, bool YMASK>
 __device__ __forceinline__ void sums_of_planes(double (&acc)[4], const float* __restrict__ x, const float* __restrict__ dy,
-                                               const BnormP& p, int c, int n0, int n1, float ra, float rk,
+                                               const BnormP& p, int c, int n0, int n1, float ra, float rk, float rs,
                                                const float* __restrict__ ymask, float* __restrict__ masked, double* lds) {
-  auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv, rk) > 0.f ? dv : 0.f) : dv; };
+  auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv - rs, rk) > 0.f ? dv : 0.f) : dv; };
   acc[0] = acc[1] = acc[2] = acc[3] = 0.0;
   const int shift = p.teamShift[VEC4 ? 1 : 0], TS = 1 << shift, teams = 256 >> shift;
   const int team = threadIdx.x >> shift, j0 = threadIdx.x & (TS - 1);
   for (int n = n0 + team; n < n1; n += teams) {
     const size_t base = (size_t)p.WH * (c + (size_t)p.C * n);
-    float sx = 0.f, sxx = 0.f, sxd = 0.f, sd = 0.f;
     if (VEC4) {
       const float4* x4 = (const float4*)(x + base);
       const float4* d4 = (const float4*)(MODE != 0 ? dy + base : x + base);
       for (int i = j0; i < p.WH / 4; i += TS) {
         const float4 a = x4[i];
+        const double ax = (double)a.x, ay = (double)a.y, az = (double)a.z, aw = (double)a.w;
         if (MODE != 1) {
-          sx += (a.x + a.y) + (a.z + a.w);
-          sxx += (a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w);
+          acc[0] += (ax + ay) + (az + aw);
+          acc[1] += fma(ax, ax, ay * ay) + fma(az, az, aw * aw);
         }
         if (MODE != 0) {
           float4 d = d4[i];
@@ -102,16 +109,18 @@ __device__ __forceinline__ void sums_of_planes(double (&acc)[4], const float* __
                             m.w > 0.f ? d.w : d.w * 0.f);
             ((float4*)(masked + base))[i] = d;
           }
-          sxd += (a.x * d.x + a.y * d.y) + (a.z * d.z + a.w * d.w);
-          sd += (d.x + d.y) + (d.z + d.w);
+          const double dx_ = (double)d.x, dy_ = (double)d.y, dz_ = (double)d.z, dw_ = (double)d.w;
+          acc[2] += fma(ax, dx_, ay * dy_) + fma(az, dz_, aw * dw_);
+          acc[3] += (dx_ + dy_) + (dz_ + dw_);
         }
       }
     } else {
       for (int i = j0; i < p.WH; i += TS) {
         const float a = x[base + i];
+        const double ad = (double)a;
         if (MODE != 1) {
-          sx += a;
-          sxx += a * a;
+          acc[0] += ad;
+          acc[1] = fma(ad, ad, acc[1]);
         }
         if (MODE != 0) {
           float d = gate(a, dy[base + i]);
@@ -119,15 +128,11 @@ __device__ __forceinline__ void sums_of_planes(double (&acc)[4], const float* __
             d = ymask[base + i] > 0.f ? d : d * 0.f;
             masked[base + i] = d;
           }
-          sxd += a * d;
-          sd += d;
+          acc[2] = fma(ad, (double)d, acc[2]);
+          acc[3] += (double)d;
         }
       }
     }
-    acc[0] += (double)sx;
-    acc[1] += (double)sxx;
-    acc[2] += (double)sxd;
-    acc[3] += (double)sd;
   }
   block_sum<4>(acc, lds);
 }
@@ -149,10 +154,10 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
   const int grp = logical - c * p.groups;
   int n0, n1;
   image_range(p, grp, &n0, &n1);
-  float ra = 0.f, rk = 0.f;
-  if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &ra, &rk);
+  float ra = 0.f, rk = 0.f, rs = 0.f;
+  if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &ra, &rk, &rs);
   double acc[4];
-  sums_of_planes<MODE, VEC4, RELU, YMASK>(acc, x, dy, p, c, n0, n1, ra, rk, ymask, masked, lds);
+  sums_of_planes<MODE, VEC4, RELU, YMASK>(acc, x, dy, p, c, n0, n1, ra, rk, rs, ymask, masked, lds);
   if (threadIdx.x == 0) {
     double* out = partials + ((size_t)c * p.groups + grp) * 4;
     out[0] = acc[0];
@@ -166,10 +171,10 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
 // planes, handed to every thread.  `lds`: 20 doubles.
 template <int MODE, bool VEC4, bool RELU, bool YMASK>
 __device__ __forceinline__ void own_totals(double (&tot)[4], const float* __restrict__ x, const float* __restrict__ dy,
-                                           const BnormP& p, int c, float ra, float rk, const float* __restrict__ ymask,
-                                           float* __restrict__ masked, double* lds) {
+                                           const BnormP& p, int c, float ra, float rk, float rs,
+                                           const float* __restrict__ ymask, float* __restrict__ masked, double* lds) {
   double acc[4];
-  sums_of_planes<MODE, VEC4, RELU, YMASK>(acc, x, dy, p, c, 0, p.N, ra, rk, ymask, masked, lds);
+  sums_of_planes<MODE, VEC4, RELU, YMASK>(acc, x, dy, p, c, 0, p.N, ra, rk, rs, ymask, masked, lds);
   if (threadIdx.x == 0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) lds[16 + i] = acc[i];
@@ -204,14 +209,15 @@ __device__ __forceinline__ void channel_totals(const double* __restrict__ partia
   for (int i = 0; i < 4; ++i) tot[i] = lds[i];
 }
 
-// out = a*in1 + b*in2 + k over this workgroup's planes (in2 optional)
-// RELU: in1 counts only where ra*in2 + rk > 0 (in1 = derivative after the ReLU, in2 = the layer's input)
+// out = a*(in1 - t) + b*(in2 - s) + k over this workgroup's planes (in2 optional)
+// RELU: in1 counts only where ra*(in2 - rs) + rk > 0 (in1 = derivative after the ReLU, in2 = the layer's input)
 template <bool TWO, bool VEC4, bool RELU = false>
 __device__ __forceinline__ void stream_planes(float* __restrict__ out, const float* __restrict__ in1,
-                                              const float* __restrict__ in2, float a, float b, float k,
-                                              const BnormP& p, int c, int n0, int n1, float ra = 0.f, float rk = 0.f) {
+                                              const float* __restrict__ in2, float a, float b, float k, float s,
+                                              float t, const BnormP& p, int c, int n0, int n1, float ra = 0.f, float rk = 0.f,
+                                              float rs = 0.f) {
   static_assert(!RELU || TWO, "the mask is computed from the second stream");
-  auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv, rk) > 0.f ? dv : 0.f) : dv; };
+  auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv - rs, rk) > 0.f ? dv : 0.f) : dv; };
   const int shift = p.teamShift[VEC4 ? 1 : 0], TS = 1 << shift, teams = 256 >> shift;
   const int team = threadIdx.x >> shift, j0 = threadIdx.x & (TS - 1);
   for (int nn = n0 + team; nn < n1; nn += teams) {
@@ -226,10 +232,10 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
         float4 r;
         if (TWO) {
           const float4 v = stream_load4(s2 + i);
-          r.x = fmaf(a, gate(v.x, u.x), fmaf(b, v.x, k));
-          r.y = fmaf(a, gate(v.y, u.y), fmaf(b, v.y, k));
-          r.z = fmaf(a, gate(v.z, u.z), fmaf(b, v.z, k));
-          r.w = fmaf(a, gate(v.w, u.w), fmaf(b, v.w, k));
+          r.x = fmaf(a, gate(v.x, u.x) - t, fmaf(b, v.x - s, k));
+          r.y = fmaf(a, gate(v.y, u.y) - t, fmaf(b, v.y - s, k));
+          r.z = fmaf(a, gate(v.z, u.z) - t, fmaf(b, v.z - s, k));
+          r.w = fmaf(a, gate(v.w, u.w) - t, fmaf(b, v.w - s, k));
         } else {
           r.x = fmaf(a, u.x, k);
           r.y = fmaf(a, u.y, k);
@@ -241,7 +247,7 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
     } else {
       for (int i = j0; i < p.WH; i += TS) {
         const float u = in1[base + i];
-        out[base + i] = TWO ? fmaf(a, gate(in2[base + i], u), fmaf(b, in2[base + i], k)) : fmaf(a, u, k);
+        out[base + i] = TWO ? fmaf(a, gate(in2[base + i], u) - t, fmaf(b, in2[base + i] - s, k)) : fmaf(a, u, k);
       }
     }
   }
@@ -273,9 +279,9 @@ __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ 
   const int grp = logical - c * p.groups;
   double tot[4];
   if (ONE) {
-    float sa = 0.f, sk = 0.f;
-    if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &sa, &sk);
-    own_totals<GIVEN ? 1 : 2, VEC4, RELU, ONE == 2>(tot, x, dy, p, c, sa, sk, ymask, masked, lds);
+    float sa = 0.f, sk = 0.f, ss = 0.f;
+    if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &sa, &sk, &ss);
+    own_totals<GIVEN ? 1 : 2, VEC4, RELU, ONE == 2>(tot, x, dy, p, c, sa, sk, ss, ymask, masked, lds);
     if (ONE == 2) dy = masked;
   } else {
     channel_totals(partials, p, c, lds, tot);
@@ -303,23 +309,29 @@ __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ 
       moments[c + p.C] = (float)sigma;
     }
   }
-  // dzdx = G1*(dy - muz) - G2*(x - mean) = G1*dy + (-G2)*x + (G2*mean - G1*muz)
+  // dzdx = G1*(dy - muz) - G2*(x - mean) = G1*(dy - t) + (-G2)*(x - s) + (G2*(mean - s) - G1*(muz - t)) with
+  // s = float(mean), t = float(muz): both means come off before anything is scaled, as in bits/nnbnorm.cu:148-160
+  // (scaled first, a channel whose mean is large against its spread would cancel two huge numbers); the constant
+  // carries what their rounding to float left over
   int n0, n1;
   image_range(p, grp, &n0, &n1);
-  float ra = 0.f, rk = 0.f;
-  if (RELU) forward_coefficients(mean, sigma, mult[c], bias[c], &ra, &rk);
-  stream_planes<true, VEC4, RELU>(dx, dy, x, (float)G1, (float)(-G2), (float)(G2 * mean - G1 * muz), p, c, n0, n1, ra, rk);
+  float ra = 0.f, rk = 0.f, rs = 0.f;
+  if (RELU) forward_coefficients(mean, sigma, mult[c], bias[c], &ra, &rk, &rs);
+  const float shift = (float)mean, shiftDy = (float)muz;
+  stream_planes<true, VEC4, RELU>(dx, dy, x, (float)G1, (float)(-G2),
+                                  (float)(G2 * (mean - (double)shift) - G1 * (muz - (double)shiftDy)), shift, shiftDy, p, c, n0,
+                                  n1, ra, rk, rs);
 }
 
-// out = act(a*in + k [+ res]) over this workgroup's planes: the forward apply with the element-wise layers
+// out = act(a*(in - s) + k [+ res]) over this workgroup's planes: the forward apply with the element-wise layers
 // that follow it folded in.  Each element goes through the same roundings as the separate kernels would
-// give it: fma, then add, then max.
+// give it: subtract, fma, then add, then max.
 template <bool RES, bool RELU, bool VEC4>
 __device__ __forceinline__ void stream_forward(float* __restrict__ out, const float* __restrict__ in,
-                                               const float* __restrict__ res, float a, float k, const BnormP& p,
-                                               int c, int n0, int n1) {
+                                               const float* __restrict__ res, float a, float k, float s,
+                                               const BnormP& p, int c, int n0, int n1) {
   auto one = [&](float u, float r) -> float {
-    float v = fmaf(a, u, k);
+    float v = fmaf(a, u - s, k);
     if (RES) v = v + r;
     if (RELU) v = v > 0.f ? v : 0.f;
     return v;
@@ -367,7 +379,7 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
     sigma = (double)moments[c + p.C];
   } else {
     double tot[4];
-    if (ONE) own_totals<0, VEC4, false, false>(tot, x, x, p, c, 0.f, 0.f, nullptr, nullptr, lds);
+    if (ONE) own_totals<0, VEC4, false, false>(tot, x, x, p, c, 0.f, 0.f, 0.f, nullptr, nullptr, lds);
     else channel_totals(partials, p, c, lds, tot);
     mean = tot[0] / p.mass;
     const double var = fmax(0.0, tot[1] / p.mass - mean * mean);
@@ -381,11 +393,11 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
     mean = (double)(float)mean;
     sigma = (double)(float)sigma;
   }
-  float a, k;
-  forward_coefficients(mean, sigma, mult[c], bias[c], &a, &k);
+  float a, k, shift;
+  forward_coefficients(mean, sigma, mult[c], bias[c], &a, &k, &shift);
   int n0, n1;
   image_range(p, grp, &n0, &n1);
-  stream_forward<RES, RELU, VEC4>(y, x, residual, a, k, p, c, n0, n1);
+  stream_forward<RES, RELU, VEC4>(y, x, residual, a, k, shift, p, c, n0, n1);
 }
 
 int image_groups(int WH, int N) {
@@ -578,24 +590,26 @@ int mcn_bnorm_backward_masked(mcn_stream_t stream, float* derInput, float* derMu
   return check_launch("mcn_bnorm_backward_masked");
 }
 
-int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases, float* moments,
-                       const float* x, const float* multipliers, const float* derOutput, int H, int W, int C,
-                       int N, double epsilon, int givenMoments, void* workspace, size_t workspaceBytes) {
+static int bnorm_backward_any(const char* who, mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
+                              float* moments, const float* x, const float* multipliers, const float* derOutput, int H,
+                              int W, int C, int N, double epsilon, int givenMoments, void* workspace,
+                              size_t workspaceBytes) {
   BnormP p;
-  int rc = setup("mcn_bnorm_backward", H, W, C, N, epsilon, &p);
+  int rc = setup(who, H, W, C, N, epsilon, &p);
   if (rc) return rc;
   if (C == 0) return MCN_SUCCESS;
-  if (!derMultipliers || !derBiases || !multipliers)
-    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward: null parameter tensor");
+  if (!derMultipliers || !derBiases || !multipliers) return fail(MCN_ILLEGAL_ARGUMENT, "%s: null parameter tensor", who);
   if ((size_t)p.WH * N == 0) {
     // nothing to sum over: the reference leaves dzdg = 0/sigma-related garbage; define zeros
     if ((rc = mcn_fill(stream, derMultipliers, 0.f, (size_t)C))) return rc;
     return mcn_fill(stream, derBiases, 0.f, (size_t)C);
   }
-  if (!derInput || !x || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward: null tensor");
-  if (givenMoments && !moments) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward: moments are required");
-  if (!workspace || workspaceBytes < mcn_bnorm_workspace_bytes(H, W, C, N))
-    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward: workspace too small");
+  if (!derInput || !x || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "%s: null tensor", who);
+  if (givenMoments && !moments) return fail(MCN_ILLEGAL_ARGUMENT, "%s: moments are required", who);
+  const size_t need = mcn_bnorm_workspace_bytes(H, W, C, N);
+  if (!workspace || workspaceBytes < need) {
+    return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small", who);
+  }
   hipStream_t s = as_stream(stream);
   const bool vec = (p.WH % 4 == 0) && aligned16(derInput) && aligned16(x) && aligned16(derOutput);
   const dim3 grid((unsigned)(C * p.groups)), block(256);
@@ -609,7 +623,7 @@ int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultiplie
       if (vec) hipLaunchKernelGGL((bnorm_backward_apply<false, true, false, 1>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
       else hipLaunchKernelGGL((bnorm_backward_apply<false, false, false, 1>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
     }
-    return check_launch("mcn_bnorm_backward");
+    return check_launch(who);
   }
   {
     KernelTimer timer("bnorm_sums", s);
@@ -621,7 +635,7 @@ int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultiplie
       else hipLaunchKernelGGL((bnorm_sums<2, false>), grid, block, 0, s, x, derOutput, partials, p);
     }
   }
-  if ((rc = check_launch("mcn_bnorm_backward(sums)"))) return rc;
+  if ((rc = check_launch(who))) return rc;
   KernelTimer timer("bnorm_backward_apply", s);
   if (givenMoments) {
     if (vec) hipLaunchKernelGGL((bnorm_backward_apply<true, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
@@ -630,7 +644,14 @@ int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultiplie
     if (vec) hipLaunchKernelGGL((bnorm_backward_apply<false, true>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
     else hipLaunchKernelGGL((bnorm_backward_apply<false, false>), grid, block, 0, s, derInput, derMultipliers, derBiases, moments, x, multipliers, derOutput, partials, p);
   }
-  return check_launch("mcn_bnorm_backward");
+  return check_launch(who);
+}
+
+int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases, float* moments,
+                       const float* x, const float* multipliers, const float* derOutput, int H, int W, int C,
+                       int N, double epsilon, int givenMoments, void* workspace, size_t workspaceBytes) {
+  return bnorm_backward_any("mcn_bnorm_backward", stream, derInput, derMultipliers, derBiases, moments, x, multipliers,
+                            derOutput, H, W, C, N, epsilon, givenMoments, workspace, workspaceBytes);
 }
 
 }  // extern "C"

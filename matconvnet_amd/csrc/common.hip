@@ -12,11 +12,13 @@ namespace mcn {
 
 namespace {
 thread_local char g_message[512] = "";
-std::mutex g_tunable_mutex;
 
+// Values are read on every launch (several per launch) from any thread and written only by experiments: relaxed
+// atomics, no lock; the table itself never changes.
 struct Tunable {
   const char* name;
-  int value;
+  std::atomic<int> value;
+  Tunable(const char* n, int v) : name(n), value(v) {}
 };
 // Defaults are the values chosen from on-device sweeps; see the per-kernel comments where each is read.
 Tunable g_tunables[] = {
@@ -102,10 +104,35 @@ KernelTimer::~KernelTimer() {
 }
 
 int tunable(const char* name, int fallback) {
-  std::lock_guard<std::mutex> lock(g_tunable_mutex);
   for (auto& t : g_tunables)
-    if (std::strcmp(t.name, name) == 0) return t.value;
+    if (std::strcmp(t.name, name) == 0) return t.value.load(std::memory_order_relaxed);
   return fallback;
+}
+
+int current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return -1;
+  }
+  return dev;
+}
+
+int device_compute_units() {
+  static std::atomic<int> cached[kMaxDevices];  // 0 = not asked yet
+  const int dev = current_device();
+  if (dev < 0) return -1;
+  if (dev < kMaxDevices) {
+    const int have = cached[dev].load(std::memory_order_relaxed);
+    if (have > 0) return have;
+  }
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+    (void)hipGetLastError();
+    return -1;
+  }
+  if (dev < kMaxDevices) cached[dev].store(cus, std::memory_order_relaxed);
+  return cus;
 }
 
 }  // namespace mcn
@@ -126,12 +153,7 @@ const char* mcn_error_name(int code) {
   }
 }
 
-int mcn_device_compute_units(void) {
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return -1;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
-  return cus;
-}
+int mcn_device_compute_units(void) { return mcn::device_compute_units(); }
 
 int mcn_profile_begin(const char* kernel_name) {
   if (!kernel_name || !*kernel_name) return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_profile_begin: empty kernel name");
@@ -163,10 +185,9 @@ int mcn_profile_end(int* launches, double* total_ms) {
 
 int mcn_set_tunable(const char* name, int value) {
   if (!name) return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_set_tunable: null name");
-  std::lock_guard<std::mutex> lock(mcn::g_tunable_mutex);
   for (auto& t : mcn::g_tunables)
     if (std::strcmp(t.name, name) == 0) {
-      t.value = value;
+      t.value.store(value, std::memory_order_relaxed);
       return MCN_SUCCESS;
     }
   return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_set_tunable: unknown tunable '%s'", name);
@@ -174,10 +195,9 @@ int mcn_set_tunable(const char* name, int value) {
 
 int mcn_get_tunable(const char* name, int* value) {
   if (!name || !value) return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_get_tunable: null argument");
-  std::lock_guard<std::mutex> lock(mcn::g_tunable_mutex);
   for (auto& t : mcn::g_tunables)
     if (std::strcmp(t.name, name) == 0) {
-      *value = t.value;
+      *value = t.value.load(std::memory_order_relaxed);
       return MCN_SUCCESS;
     }
   return mcn::fail(MCN_ILLEGAL_ARGUMENT, "mcn_get_tunable: unknown tunable '%s'", name);

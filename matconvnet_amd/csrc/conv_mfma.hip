@@ -25,6 +25,7 @@
 #include "conv_common.hpp"
 
 #include <algorithm>
+#include <atomic>
 
 namespace mcn {
 namespace {
@@ -815,14 +816,16 @@ template <int WA, int WB, int NWA, int NWB, bool UT>
 int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const float* dy, const WgP& p) {
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB, LD = 33;
   constexpr size_t lds = (size_t)2 * (BA + BB) * LD * sizeof(float) + BB * sizeof(int2);
-  static bool raised = false;  // one-time opt-in to more than 64 KB of LDS per workgroup
+  static std::atomic<bool> raisedOn[kMaxDevices];  // opt-in to more than 64 KB of LDS per workgroup, once per device
+  const int dev = current_device();
+  const bool raised = dev >= 0 && dev < kMaxDevices && raisedOn[dev].load(std::memory_order_acquire);
   if (lds > 64 * 1024 && !raised) {
     if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB, UT>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return fail(MCN_DEVICE_ERROR, "mcn_conv_backward_filter: cannot reserve %zu bytes of LDS", lds);
     }
-    raised = true;
+    if (dev >= 0 && dev < kMaxDevices) raisedOn[dev].store(true, std::memory_order_release);
   }
   KernelTimer timer("conv_wgrad_mfma", s);
   hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB, UT>), grid, dim3(256), lds, s, out, x, dy, p);

@@ -27,6 +27,7 @@
 #include "conv_common.hpp"
 
 #include <algorithm>
+#include <atomic>
 
 namespace mcn {
 namespace {
@@ -282,14 +283,21 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
 template <int WA, bool TAPS, int THREADS>
 int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, const float* in, const float* wt,
            const float* bias, const PixP& p, const WsP& w) {
-  static size_t raised = 0;  // largest dynamic LDS size this instantiation has been opted into
-  if (lds > 64 * 1024 && lds > raised) {
+  // largest dynamic LDS size this instantiation has been opted into, per device (concurrent callers may both opt in:
+  // the attribute call is idempotent, the atomic only keeps the bookkeeping whole)
+  static std::atomic<size_t> raised[kMaxDevices];
+  const int dev = current_device();
+  if (lds > 64 * 1024 && (dev < 0 || dev >= kMaxDevices || lds > raised[dev].load(std::memory_order_acquire))) {
     if (hipFuncSetAttribute((const void*)conv_ws_mfma<WA, TAPS, THREADS>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return fail(MCN_DEVICE_ERROR, "%s: cannot reserve %zu bytes of LDS", who, lds);
     }
-    raised = lds;
+    if (dev >= 0 && dev < kMaxDevices) {
+      size_t seen = raised[dev].load(std::memory_order_relaxed);
+      while (seen < lds && !raised[dev].compare_exchange_weak(seen, lds, std::memory_order_release)) {
+      }
+    }
   }
   KernelTimer timer("conv_ws_mfma", s);
   hipLaunchKernelGGL((conv_ws_mfma<WA, TAPS, THREADS>), dim3((unsigned)blocks), dim3(THREADS), lds, s, out, in, wt, bias, p, w);

@@ -22,6 +22,13 @@ int check_launch(const char* what);
 
 int tunable(const char* name, int fallback);
 
+// Ordinal of the current device (-1 on error) and its number of compute units (cached per device; -1 on error).
+// Per-device host state (function attributes already raised, addresses of device symbols) is kept in arrays of
+// kMaxDevices entries.
+constexpr int kMaxDevices = 64;
+int current_device();
+int device_compute_units();
+
 // Brackets one kernel launch with HIP events when live profiling of that kernel family is switched on
 // (mcn_profile_begin); costs one relaxed load otherwise.  Construct right before the launch, on its stream.
 class KernelTimer {

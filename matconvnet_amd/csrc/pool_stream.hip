@@ -356,7 +356,9 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   for (int i = 0; i < g->poolW; ++i) p.rankWpk |= (unsigned)((g->poolW - 1 - i) / g->strideX) << (4 * i);
 
   // widest tile whose LDS fits the budget and whose outputs and cells fit 4 per thread
-  const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024), 64 * 1024);
+  // (the kernel is not opted into more than 64 KB of LDS: the budget leaves room for the slots added below)
+  const size_t slotBytes = (4 + 256) * sizeof(float);
+  const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024), 64 * 1024 - (int)slotBytes);
   int TW = 0, maxOut = 0, maxCells = 0, maxC = 0;
   size_t lds = 0;
   for (int nT = 1; nT <= p.W; ++nT) {
@@ -403,15 +405,10 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   p.cellStepQ = 256 / p.H4;
   p.cellStepR = 256 % p.H4;
   const int opt = std::max((maxOut + 255) / 256, 1), xpt = std::max((maxCells + 255) / 256, 1);
-  lds += (4 + 256) * sizeof(float);  // the idle-lane cell and slots
+  lds += slotBytes;  // the idle-lane cell and slots
 
-  int cus = 256;
-  {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
-      cus = prop.multiProcessorCount;
-  }
+  int cus = device_compute_units();
+  if (cus <= 0) cus = 256;
   const int perCu = std::min(std::max(tunable("pool_blocks_per_cu", 3), 1), (int)std::max<size_t>((160 * 1024) / std::max<size_t>(lds, 1), 1));
   const int blocks = (int)std::min<long long>(p.totalTiles, (long long)cus * perCu);
   const dim3 grid((unsigned)blocks), block(256);

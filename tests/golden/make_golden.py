@@ -87,6 +87,42 @@ def bnorm_vectors():
     np.savez_compressed(os.path.join(HERE, "bnorm_golden.npz"), **out)
 
 
+def bnorm_edge_vectors():
+    """The corners of the one-pass variance (bits/nnbnorm.cu:64-70,118-132): a constant channel (variance 0 or, in
+    float, a rounding residue of either sign that max(0, .) clamps: sigma = sqrt(epsilon) or next to it), a channel with
+    mean 1e3 and standard deviation 1e-2 (E[x^2] - mean^2 cancels ten digits: the float instantiation keeps none of
+    the variance, the double one six digits), the same with mean 30 (seven digits cancel: float keeps a digit or two, double nine) and one element per channel (H = W = N = 1).  Float and double."""
+    r = np.random.default_rng(2027)
+    out = {}
+    k = 0
+    for kind, (H, W, C, N, eps) in (("constant", (6, 5, 3, 4, 1e-4)), ("constant", (8, 8, 2, 3, 1e-5)),
+                                    ("cancel", (8, 8, 3, 4, 1e-4)), ("cancel", (14, 14, 2, 6, 1e-5)),
+                                    ("cancel_mild", (8, 8, 3, 4, 1e-4)), ("cancel_mild", (14, 14, 2, 6, 1e-5)),
+                                    ("single", (1, 1, 4, 1, 1e-4))):
+        x64 = r.standard_normal((H, W, C, N)) * 1.5 + 0.25
+        if kind == "constant":
+            x64[:, :, 1, :] = 0.7          # (not representable in binary: sums and squares round)
+        if kind == "cancel":       # condition number mean^2/var = 1e10: float keeps nothing, double about six digits
+            x64[:, :, 0, :] = 1e3 + 1e-2 * r.standard_normal((H, W, N))
+        if kind == "cancel_mild":  # 1e7: float still keeps nothing, double nine digits
+            x64[:, :, 0, :] = 30.0 + 1e-2 * r.standard_normal((H, W, N))
+        g64 = r.uniform(0.5, 1.5, C)
+        b64 = 0.1 * r.standard_normal(C)
+        dy64 = r.standard_normal((H, W, C, N))
+        for dtype in (np.float32, np.float64):
+            x, g, b, dy = F(x64.astype(np.float32), dtype), g64.astype(np.float32).astype(dtype), \
+                b64.astype(np.float32).astype(dtype), F(dy64.astype(np.float32), dtype)
+            y, mom = ob.ref_bnorm_forward(x, g, b, eps)
+            dx, dg, db, mom2 = ob.ref_bnorm_backward(x, g, b, dy, eps)
+            for name, val in dict(x=x, g=g, b=b, dy=dy, y=y, mom=mom, dx=dx, dg=dg, db=db, mom2=mom2).items():
+                out["%s_%d" % (name, k)] = val
+            out["eps_%d" % k] = np.float64(eps)
+            out["kind_%d" % k] = np.array(kind)
+            k += 1
+    out["count"] = np.int32(k)
+    np.savez_compressed(os.path.join(HERE, "bnorm_edge_golden.npz"), **out)
+
+
 def im2row_vectors():
     r = np.random.default_rng(2026)
     out = {}
@@ -119,6 +155,7 @@ if __name__ == "__main__":
     assert ob.ref() is not None, "oracle/_ref did not build: is /root/reference present?"
     pool_vectors()
     bnorm_vectors()
+    bnorm_edge_vectors()
     im2row_vectors()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):

@@ -86,6 +86,56 @@ def test_golden_vectors_from_reference(capi):
     assert checked >= 4
 
 
+EDGE = os.path.join(os.path.dirname(__file__), "golden", "bnorm_edge_golden.npz")
+
+
+def test_edge_golden_vectors_from_reference(capi):
+    """The corners of the one-pass variance (bits/nnbnorm.cu:64-70,118-132), outputs of the compiled reference: a
+    constant channel (variance 0: the max(0, .) clamp, sigma = sqrt(epsilon)), a channel with standard deviation
+    1e-2 around a mean of 1e3 ('cancel': E[x^2] - mean^2 cancels ten digits) or of 30 ('cancel_mild': seven), one element
+    per channel.
+
+    The device result is compared with the reference's DOUBLE instantiation run on the same float data, at the usual
+    1e-5, on every output.  Why not the float one: in these corners the float instantiation is not a result to
+    match -- its sigma of the constant channel is a rounding residue (0.00341 for sqrt(1e-5) = 0.00316), its variance of
+    the large-mean channel is 0 or noise (sigma 0.0100 or 0.50 for 0.0140 and 0.0106), and which of these comes out
+    depends on the summation order.  The device kernels widen each float to double before squaring and summing, so they
+    keep what the double instantiation keeps.  The distance to the float instantiation is printed, not gated.
+    In the 'cancel' cases the double instantiation is itself only good to about six digits (its sigma is 5e-6 from the
+    two-pass value): any two summation orders differ by that much there, and the gate for those cases is 1e-4."""
+    z = np.load(EDGE)
+    checked = set()
+    for k in range(int(z["count"])):
+        if z["x_%d" % k].dtype != np.float64:
+            continue
+        kind = str(z["kind_%d" % k])
+        x, g, b, dy, eps = z["x_%d" % k], z["g_%d" % k], z["b_%d" % k], z["dy_%d" % k], float(z["eps_%d" % k])
+        xd, gd, bd, dyd = capi.to_device(x), capi.to_device(g), capi.to_device(b), capi.to_device(dy)
+        y, mom = [capi.to_host(t) for t in capi.bnorm_forward(xd, gd, bd, eps)]
+        dx, dg, db, mom2 = [capi.to_host(t) for t in capi.bnorm_backward(xd, gd, dyd, eps)]
+        errs = dict(y=rel_max(y, z["y_%d" % k]), mom=rel_max(mom, z["mom_%d" % k]), dx=rel_max(dx, z["dx_%d" % k]),
+                    dg=rel_max(dg, z["dg_%d" % k]), db=rel_max(db, z["db_%d" % k]), mom2=rel_max(mom2, z["mom2_%d" % k]))
+        # per channel as well: the corner channel must not hide behind a larger neighbour
+        sig, want_sig = mom2[:, 1].astype(np.float64), z["mom2_%d" % k][:, 1]
+        errs["sigma_per_channel"] = float(np.abs(sig / want_sig - 1).max())
+        for c in range(x.shape[2]):
+            errs["dx_c%d" % c] = rel_max(dx[:, :, c, :], z["dx_%d" % k][:, :, c, :]) if np.abs(z["dx_%d" % k][:, :, c, :]).max() > 0 else float(np.abs(dx[:, :, c, :]).max())
+        f = k - 1  # the float instantiation of the same case
+        assert str(z["kind_%d" % f]) == kind and z["x_%d" % f].dtype == np.float32
+        print("bnorm edge", kind, x.shape, "vs double:", {n: "%.1e" % v for n, v in errs.items()},
+              "| vs float: dx %.1e sigma %.1e" % (rel_max(dx, z["dx_%d" % f]), np.abs(sig / z["mom2_%d" % f][:, 1] - 1).max()))
+        # the forward output is normalised with the moments as they are stored, in float (so that a later pass given
+        # them reproduces it bit for bit; the reference's float instantiation does the same): the stored mean is within
+        # half an ulp of the double one, which moves y by up to that times |g|/sigma.  Only the 'cancel' kinds notice.
+        want_mom = z["mom2_%d" % k]
+        half_ulp = 0.5 * np.spacing(np.abs(want_mom[:, 0]).astype(np.float32)).astype(np.float64)
+        y_gate = max(TOL, 2 * float((half_ulp * np.abs(g) / want_mom[:, 1]).max()) / float(np.abs(z["y_%d" % k]).max()))
+        assert errs.pop("y") < y_gate, (kind, y_gate)
+        assert max(errs.values()) < (1e-4 if kind == "cancel" else TOL), (kind, errs)
+        checked.add(kind)
+    assert checked == {"constant", "cancel", "cancel_mild", "single"}
+
+
 def test_baseline_config_full_size(capi, ob):
     """benchmark configuration 2: 56x56x256x32, eps 1e-4, moments from the batch."""
     w = workloads.bnorm_case()

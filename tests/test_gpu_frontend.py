@@ -364,3 +364,36 @@ def test_residual_unit_against_oracle_and_across_modes(vl, ob, H, W, Cc, M, Cout
         assert bits_equal(outs["plain"][k], outs["fused"][k]), k
         assert bits_equal(outs["plain"][k], outs["overlap"][k]), k
         assert bits_equal(outs["plain"][k], outs["packed"][k]), k
+
+
+def test_timed_schedule_at_full_size_is_bit_identical_to_the_layer_by_layer_block(vl, ob):
+    """The schedule bench.py times -- N = 32 at 56x56, batch-norm folding (fused), filter banks packed ahead
+    (packed), one summing launch for the three filter gradients (deferred), stepped through `run` exactly as the
+    bench steps it -- against the layer-by-layer block on the same inputs, every output bit for bit.  The
+    layer-by-layer block is the one test_bottleneck_block_full_config_stage_by_stage checks against the oracle at
+    this size; at this size the planner picks other unit widths, split counts and summing job tables than at the
+    small batches of the tests above."""
+    N = 32
+    w = workloads.bottleneck_case()
+    assert w["x"].shape == (56, 56, 256, N)
+    shapes = dict(y=w["x"].shape, dzdx=w["x"].shape, df1=w["f1"].shape, df2=w["f2"].shape, df3=w["f3"].shape,
+                  dg1=(64,), db1=(64,), dg2=(64,), db2=(64,), dg3=(256,), db3=(256,), m1=(64, 2), m2=(64, 2), m3=(256, 2))
+    outs = {}
+    for mode in ("plain", "timed"):
+        timed = mode == "timed"
+        blk = vl.Bottleneck(N=N, eps=w["eps"], fused=timed, packed=timed, deferred=timed)
+        try:
+            _load(blk, w)
+            if timed:
+                blk.run(2)          # two whole steps, as bench.py's warm-up and timed region run them
+            else:
+                for _ in range(2):
+                    blk.forward()
+                    blk.backward()
+            torch.cuda.synchronize()
+            outs[mode] = {k: blk.get(k, v) for k, v in shapes.items()}
+        finally:
+            blk.close()
+    for k in shapes:
+        assert np.isfinite(outs["plain"][k]).all(), k
+        assert bits_equal(outs["plain"][k], outs["timed"][k]), k

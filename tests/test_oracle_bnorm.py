@@ -61,6 +61,49 @@ def test_oracle_matches_golden_vectors(ob):
         assert bits_equal(dxg, F(z["dxg_%d" % k], None)) and bits_equal(dgg, z["dgg_%d" % k]) and bits_equal(dbg, z["dbg_%d" % k])
 
 
+EDGE = os.path.join(os.path.dirname(__file__), "golden", "bnorm_edge_golden.npz")
+
+
+def test_oracle_matches_edge_golden_vectors(ob):
+    """Outputs of the compiled reference at the corners of its one-pass variance (bits/nnbnorm.cu:64-70,118-132):
+    a constant channel (the max(0, .) clamp, sigma = sqrt(epsilon) or a float rounding residue next to it), a channel
+    with mean 1e3 and standard deviation 1e-2 (the float instantiation loses the variance, the double one keeps it)
+    and one element per channel.  The oracle reproduces every bit, float and double."""
+    z = np.load(EDGE)
+    kinds = set()
+    for k in range(int(z["count"])):
+        x, g, b, dy, eps = F(z["x_%d" % k], None), z["g_%d" % k], z["b_%d" % k], F(z["dy_%d" % k], None), float(z["eps_%d" % k])
+        y, mom = ob.bnorm_forward(x, g, b, eps)
+        assert bits_equal(y, F(z["y_%d" % k], None)) and bits_equal(mom, F(z["mom_%d" % k], None))
+        dx, dg, db, mom2 = ob.bnorm_backward(x, g, dy, eps)
+        assert bits_equal(dx, F(z["dx_%d" % k], None)) and bits_equal(dg, z["dg_%d" % k])
+        assert bits_equal(db, z["db_%d" % k]) and bits_equal(mom2, F(z["mom2_%d" % k], None))
+        kinds.add(str(z["kind_%d" % k]))
+    assert kinds == {"constant", "cancel", "cancel_mild", "single"}
+
+
+def test_edge_golden_vectors_say_what_they_are_meant_to(ob):
+    """The double outputs obey the closed forms (sigma of a constant channel is sqrt(epsilon); the 'cancel' channel
+    has the two-pass variance); the float outputs of the same cases are off by what the one-pass formula loses in
+    float.  So the fixtures do sit in the regime they are named for."""
+    z = np.load(EDGE)
+    for k in range(int(z["count"])):
+        kind, x, eps, mom = str(z["kind_%d" % k]), z["x_%d" % k], float(z["eps_%d" % k]), z["mom2_%d" % k]
+        c = {"constant": 1, "cancel": 0, "cancel_mild": 0, "single": 0}[kind]
+        x64 = x[:, :, c, :].astype(np.float64)
+        sigma = np.sqrt(x64.var() + eps)
+        if x.dtype == np.float64:
+            # (ten digits cancel in the 'cancel' channel: the double instantiation itself keeps about six)
+            assert abs(mom[c, 1] - sigma) / sigma < (1e-4 if kind == "cancel" else 1e-7), (kind, mom[c, 1], sigma)
+            if kind in ("constant", "single"):
+                assert abs(mom[c, 1] - np.sqrt(eps)) / np.sqrt(eps) < 1e-6
+        elif kind in ("cancel", "cancel_mild"):
+            # float: nothing of the variance is left ('cancel'), or a digit or two ('cancel_mild')
+            assert abs(mom[c, 1] - sigma) / sigma > (0.2 if kind == "cancel" else 1e-3)
+        elif kind == "constant":
+            assert 1e-4 < abs(mom[c, 1] - sigma) / sigma < 0.2   # float: a rounding residue under the root
+
+
 @pytest.mark.parametrize("shape", SHAPES)
 def test_closed_form_and_torch_autograd_double(ob, shape):
     """y = g (x - mu)/sqrt(var + eps) + b with the biased variance; gradients from torch autograd of the
