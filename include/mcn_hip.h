@@ -272,6 +272,20 @@ MCN_API int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derM
                                int N, double epsilon, int givenMoments, void* workspace,
                                size_t workspaceBytes);
 
+/* mcn_bnorm_backward for callers that cannot allocate device memory and have no workspace to hand over (code under
+   HIP-graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+   arguments, meaning and bits as mcn_bnorm_backward without the workspace: the per-channel partial sums go to a device
+   array built into the library (MCN_BNORM_STATIC_SCRATCH_BYTES per device, held until the process ends).  The call
+   allocates and frees nothing; its first call on a device looks up that device's copy of the array (make that call
+   outside graph capture).  Shapes whose partial sums do not fit (mcn_bnorm_workspace_bytes(H,W,C,N) >
+   MCN_BNORM_STATIC_SCRATCH_BYTES) are rejected with MCN_UNSUPPORTED before anything is launched.  Every call on a
+   device uses the same array: two calls that overlap on one device (different streams, different threads) race;
+   calls on one stream are ordered and need nothing cleared between them. */
+#define MCN_BNORM_STATIC_SCRATCH_BYTES (1u << 20)
+MCN_API int mcn_bnorm_backward_static(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
+                                      float* moments, const float* x, const float* multipliers, const float* derOutput,
+                                      int H, int W, int C, int N, double epsilon, int givenMoments);
+
 /* ------------------------------------------------------------------------------------------------
  * pooling -- replaces PoolingForward/Backward<VLDT_GPU,T> (bits/nnpooling_gpu.cu:270-415).
  * ---------------------------------------------------------------------------------------------- */

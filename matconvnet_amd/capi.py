@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(HERE, "libmcn_hip.so")
 SUCCESS, UNSUPPORTED, DEVICE_ERROR, OUT_OF_MEMORY, OUT_OF_GPU_MEMORY, ILLEGAL_ARGUMENT, UNKNOWN = 0, 1, 2, 5, 6, 7, 8
 CONV_FORWARD, CONV_BACKWARD_DATA, CONV_BACKWARD_FILTER, CONV_BACKWARD_BIAS = 0, 1, 2, 3
 POOL_MAX, POOL_AVERAGE = 0, 1
+BNORM_STATIC_SCRATCH_BYTES = 1 << 20   # MCN_BNORM_STATIC_SCRATCH_BYTES
 
 
 class ConvGeom(C.Structure):
@@ -83,6 +84,7 @@ PROTOTYPES = {
     "mcn_bnorm_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_bnorm_forward_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _d, _i, _vp, _sz]),
     "mcn_bnorm_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i, _vp, _sz]),
+    "mcn_bnorm_backward_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _i]),
     "mcn_bnorm_backward_masked": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _vp, _sz]),
     "mcn_bnorm_backward_relu": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _vp, _sz]),
     "mcn_pool_output_size": (_i, [C.POINTER(PoolGeom), C.POINTER(_i), C.POINTER(_i)]),
@@ -474,6 +476,19 @@ def bnorm_backward(x, g, dy, eps=1e-4, moments=None, ws=None, want_moments=True)
     wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
     check(lib().mcn_bnorm_backward(stream(), ptr(dx), ptr(dg), ptr(db), ptr(mom), ptr(x), ptr(g), ptr(dy),
                                    H, W, Cc, N, eps, int(given), wp, wn))
+    return dx, dg, db, mom
+
+
+def bnorm_backward_static(x, g, dy, eps=1e-4, moments=None, out=None):
+    """mcn_bnorm_backward_static: the partial sums live in the library's own device array.  `out` = (dx, dg, db, mom)
+    allocated by the caller beforehand, so that the call itself is made with nothing allocated around it."""
+    H, W, Cc, N = _hwcn(x)
+    given = moments is not None
+    if out is None:
+        out = (empty((H, W, Cc, N)), empty((Cc,)), empty((Cc,)), moments if given else empty((Cc, 2)))
+    dx, dg, db, mom = out
+    check(lib().mcn_bnorm_backward_static(stream(), ptr(dx), ptr(dg), ptr(db), ptr(mom), ptr(x), ptr(g), ptr(dy),
+                                          H, W, Cc, N, eps, int(given)))
     return dx, dg, db, mom
 
 

@@ -22,9 +22,36 @@
 #include "mcn_internal.hpp"
 
 #include <algorithm>
+#include <atomic>
+
+// Partial sums of mcn_bnorm_backward_static, the entry point that allocates nothing: one copy per device, held
+// from the moment the library is loaded until the process ends.  In host code this name only identifies the
+// symbol; the address kernels are given is looked up once per device (static_scratch below).
+static __device__ __align__(256) unsigned char scratch[MCN_BNORM_STATIC_SCRATCH_BYTES];
 
 namespace mcn {
 namespace {
+
+// Device address of `scratch` on the current device (every device has its own copy at its own address).
+std::atomic<void*> g_scratch_address[kMaxDevices];
+
+int static_scratch(const char* who, void** address) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(MCN_DEVICE_ERROR, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+  if (device < 0 || device >= kMaxDevices) return fail(MCN_UNSUPPORTED, "%s: device ordinal %d is not supported", who, device);
+  void* p = g_scratch_address[device].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return fail(MCN_DEVICE_ERROR, "%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
+    }
+    g_scratch_address[device].store(p, std::memory_order_release);
+  }
+  *address = p;
+  return MCN_SUCCESS;
+}
 
 struct BnormP {
   int WH, C, N;
@@ -590,10 +617,12 @@ int mcn_bnorm_backward_masked(mcn_stream_t stream, float* derInput, float* derMu
   return check_launch("mcn_bnorm_backward_masked");
 }
 
+// Both forms of mcn_bnorm_backward.  staticScratch: the partial sums go to the library's own device array instead of a
+// workspace of the caller's.
 static int bnorm_backward_any(const char* who, mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
                               float* moments, const float* x, const float* multipliers, const float* derOutput, int H,
                               int W, int C, int N, double epsilon, int givenMoments, void* workspace,
-                              size_t workspaceBytes) {
+                              size_t workspaceBytes, bool staticScratch) {
   BnormP p;
   int rc = setup(who, H, W, C, N, epsilon, &p);
   if (rc) return rc;
@@ -607,7 +636,12 @@ static int bnorm_backward_any(const char* who, mcn_stream_t stream, float* derIn
   if (!derInput || !x || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "%s: null tensor", who);
   if (givenMoments && !moments) return fail(MCN_ILLEGAL_ARGUMENT, "%s: moments are required", who);
   const size_t need = mcn_bnorm_workspace_bytes(H, W, C, N);
-  if (!workspace || workspaceBytes < need) {
+  if (staticScratch) {
+    if (need > (size_t)MCN_BNORM_STATIC_SCRATCH_BYTES)
+      return fail(MCN_UNSUPPORTED, "%s: this shape needs %zu bytes of partial sums, the built-in scratch holds %zu; use "
+                  "mcn_bnorm_backward with a workspace", who, need, (size_t)MCN_BNORM_STATIC_SCRATCH_BYTES);
+    if ((rc = static_scratch(who, &workspace))) return rc;
+  } else if (!workspace || workspaceBytes < need) {
     return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small", who);
   }
   hipStream_t s = as_stream(stream);
@@ -651,7 +685,14 @@ int mcn_bnorm_backward(mcn_stream_t stream, float* derInput, float* derMultiplie
                        const float* x, const float* multipliers, const float* derOutput, int H, int W, int C,
                        int N, double epsilon, int givenMoments, void* workspace, size_t workspaceBytes) {
   return bnorm_backward_any("mcn_bnorm_backward", stream, derInput, derMultipliers, derBiases, moments, x, multipliers,
-                            derOutput, H, W, C, N, epsilon, givenMoments, workspace, workspaceBytes);
+                            derOutput, H, W, C, N, epsilon, givenMoments, workspace, workspaceBytes, false);
+}
+
+int mcn_bnorm_backward_static(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases, float* moments,
+                              const float* x, const float* multipliers, const float* derOutput, int H, int W, int C,
+                              int N, double epsilon, int givenMoments) {
+  return bnorm_backward_any("mcn_bnorm_backward_static", stream, derInput, derMultipliers, derBiases, moments, x,
+                            multipliers, derOutput, H, W, C, N, epsilon, givenMoments, nullptr, 0, true);
 }
 
 }  // extern "C"
