@@ -98,6 +98,19 @@ MCN_API int mcn_get_tunable(const char* name, int* value);
 MCN_API int mcn_profile_begin(const char* kernel_name);
 MCN_API int mcn_profile_end(int* launches, double* total_ms);
 
+/* Streaming yardstick (a measurement aid, not part of the reference interface): one launch of a plain kernel that
+   reads `bytes` from src (MCN_YARDSTICK_READ; dst = one float that is never written in practice), writes them to
+   dst (WRITE) or copies src to dst (COPY), with `width` bytes per access (4, 8, 16), `inFlight` accesses issued per
+   lane before the first is used (1, 2, 4, 8), `blocks` workgroups of 256 threads (0: one step each) and flags
+   (MCN_YARDSTICK_NONTEMPORAL: stores with the non-temporal hint; MCN_YARDSTICK_CHUNKED: every workgroup walks a
+   contiguous run of its own instead of sharing the array slab by slab).  Timed with mcn_profile_begin("yardstick").
+   The best of a sweep, with cold caches, is the measured ceiling the bandwidth-bound operators are reported
+   against beside the nominal 8 TB/s; the copy of known size scales the HBM byte counters. */
+enum { MCN_YARDSTICK_READ = 0, MCN_YARDSTICK_WRITE = 1, MCN_YARDSTICK_COPY = 2 };
+enum { MCN_YARDSTICK_NONTEMPORAL = 1, MCN_YARDSTICK_CHUNKED = 2 };
+MCN_API int mcn_hbm_yardstick(mcn_stream_t stream, void* dst, const void* src, size_t bytes, int mode, int width,
+                              int inFlight, int blocks, int flags);
+
 /* ------------------------------------------------------------------------------------------------
  * convolution -- replaces ConvolutionForward/Backward<VLDT_GPU,T> (bits/nnconv.cu:71-157,163-317),
  * i.e. im2row_gpu + cublasSgemm per image, and the cuDNN variant (bits/nnconv_cudnn.cu:40-540).
@@ -160,6 +173,24 @@ MCN_API int mcn_conv_forward_packed(mcn_stream_t stream, const mcn_conv_geom* g,
 MCN_API int mcn_conv_backward_data_packed(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, float derInputMult,
                                           const float* filters, const void* packed, size_t packedBytes,
                                           const float* derOutput, void* workspace, size_t workspaceBytes);
+
+/* Forward convolution that also sums its output per channel -- the first pass of a batch normalisation that
+   follows it (bits/nnbnorm.cu:46-71 sums x and x^2 over the tensor the convolution has just written), taken from
+   the accumulators while they are still in registers.  No counterpart in the reference, which runs the two layers
+   one after the other.
+     mcn_conv_forward_sums_groups   partial sums per channel the call below writes for this geometry; 0: this
+                                    geometry has no such form (banks that do not fit in local memory, filter groups):
+                                    use mcn_conv_forward and mcn_bnorm_forward
+     mcn_conv_forward_sums          y = conv(x, filters) (no bias, y overwritten; `packed` as in mcn_conv_forward_packed,
+                                    may be NULL) and sums[(k*groups + g)*2 + {0,1}] = partial sum of y and of y^2 over
+                                    the pixels partial g covers, channel k, in double; K*groups*16 bytes.  The
+                                    partials are deterministic (fixed by the launch shape); they are fp32 sums of at
+                                    most a few hundred values each, widened to double.
+   mcn_bnorm_forward_sums (below) takes them in place of its own summing pass. */
+MCN_API int mcn_conv_forward_sums_groups(const mcn_conv_geom* g);
+MCN_API int mcn_conv_forward_sums(mcn_stream_t stream, const mcn_conv_geom* g, float* y, const float* x, const float* filters,
+                                  const void* packed, size_t packedBytes, double* sums, size_t sumsBytes, void* workspace,
+                                  size_t workspaceBytes);
 
 /* dzdf: FH x FW x FC x K, fully overwritten  (bits/nnconv.cu:280-311: im2row::forward + gemm 't','n'
    accumulated over images) */
@@ -239,6 +270,13 @@ MCN_API int mcn_bnorm_forward_fused(mcn_stream_t stream, float* y, float* moment
                                     const float* multipliers, const float* biases, const float* residual,
                                     int relu, int H, int W, int C, int N, double epsilon, int givenMoments,
                                     void* workspace, size_t workspaceBytes);
+
+/* mcn_bnorm_forward_fused (moments from the batch) whose summing pass has been done already by the layer that
+   produced x: `sums` holds sumGroups partial sums of x and x^2 per channel as mcn_conv_forward_sums writes them.  Only
+   the output pass runs.  `moments` (may be NULL) receives the batch moments. */
+MCN_API int mcn_bnorm_forward_sums(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,
+                                   const float* biases, const float* residual, int relu, int H, int W, int C, int N,
+                                   double epsilon, const double* sums, int sumGroups);
 
 /* The derivative of "batch normalisation, then ReLU" in one go: derOutput is dz/d(ReLU output), and it counts only
    where the layer's own output g*(x - mean)/sigma + b was positive, which is recomputed from x and the moments the

@@ -14,7 +14,9 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
     : H(H), W(W), C(C), M(M), N(N), Cout(CoutArg > 0 ? CoutArg : C), stride(stride), Ho((H - 1) / stride + 1),
       Wo((W - 1) / stride + 1), adapter(adapter), epsilon(epsilon), context(shared ? *shared : ownContext),
       error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), testMode(false), packed(false), packedArena(NULL), packedJobs(NULL), packedBlocks(0), deferred(false), externalSums(false),
-      partialArena(NULL), sumJobsDevice(NULL), sumBlocks(0), sideStream(NULL) {
+      partialArena(NULL), sumJobsDevice(NULL), sumBlocks(0), epilogueSums(false), sumsBuffer(NULL), sumsBytes(0),
+      sideStream(NULL) {
+  for (int i = 0; i < 4; ++i) sumGroupsOf[i] = 0;
   for (int i = 0; i < 5; ++i) events[i] = NULL;
   if (!adapter && (Cout != C || stride != 1)) {
     error = VLE_IllegalArgument;
@@ -88,6 +90,7 @@ Bottleneck::~Bottleneck() {
   if (packedJobs) (void)hipFree(packedJobs);
   if (partialArena) (void)hipFree(partialArena);
   if (sumJobsDevice) (void)hipFree(sumJobsDevice);
+  if (sumsBuffer) (void)hipFree(sumsBuffer);
 }
 
 #define STEP(stage, call)                                   \
@@ -191,6 +194,32 @@ ErrorCode Bottleneck::setDeferred(bool on, bool external) {
   }
   deferred = true;
   externalSums = external;
+  return VLE_Success;
+}
+
+ErrorCode Bottleneck::setEpilogueSums(bool on) {
+  if (sumsBuffer) (void)hipFree(sumsBuffer);
+  sumsBuffer = NULL;
+  sumsBytes = 0;
+  epilogueSums = false;
+  for (int i = 0; i < 4; ++i) sumGroupsOf[i] = 0;
+  if (!on || error != VLE_Success) return error;
+  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),
+      cs(context, stride, stride, 0, 0, 0, 0, 1, 1);
+  struct Layer { nn::Convolution* op; char const* data; char const* filter; };
+  const Layer layers[4] = {{&c1, "x", "f1"}, {&c2, "r1", "f2"}, {&c1, "r2", "f3"}, {&cs, "x", "fs"}};
+  for (int l = 0; l < (adapter ? 4 : 3); ++l) {
+    sumGroupsOf[l] = layers[l].op->sumGroups(slot(layers[l].data).getShape(), slot(layers[l].filter).getShape());
+    const std::size_t bytes = (std::size_t)slot(layers[l].filter).getSize() * sumGroupsOf[l] * 2 * sizeof(double);
+    if (bytes > sumsBytes) sumsBytes = bytes;
+  }
+  if (sumsBytes && hipMalloc(&sumsBuffer, sumsBytes) != hipSuccess) {
+    (void)hipGetLastError();
+    sumsBuffer = NULL;
+    message = "cannot allocate the partial channel sums";
+    return VLE_OutOfGPUMemeory;
+  }
+  epilogueSums = true;
   return VLE_Success;
 }
 
@@ -302,6 +331,36 @@ ErrorCode Bottleneck::forward() {
     STEP("convs_fwd", cs.forward(slot("as"), 0, slot("x"), 1, slot("fs"), none));
     STEP("bns_fwd", bnForward("ns", ms, "as", "gs", "bs"));
     shortcut = "ns";
+  }
+  if (fused && epilogueSums && !testMode) {
+    // convolution + the channel sums of its output in one launch, then only the output pass of the batch normalisation
+    struct Stage {
+      nn::Convolution* op; int layer; char const* convStage; char const* bnStage;
+      char const* out; char const* in; char const* filter; char const* act; char const* moments; char const* g; char const* b;
+      char const* residual; int relu; int h, w, c;
+    };
+    const Stage stages[3] = {
+        {&c1, 0, "conv1_fwd", "bn1_fwd", "a1", "x", "f1", "r1", "m1", "g1", "b1", NULL, 1, H, W, M},
+        {&c2, 1, "conv2_fwd", "bn2_fwd", "a2", "r1", "f2", "r2", "m2", "g2", "b2", NULL, 1, Ho, Wo, M},
+        {&c3, 2, "conv3_fwd", "bn3_fwd", "a3", "r2", "f3", "y", "m3", "g3", "b3", shortcut, 1, Ho, Wo, Cout}};
+    for (int i = 0; i < 3; ++i) {
+      const Stage& sg = stages[i];
+      const int groups = sumGroupsOf[sg.layer];
+      float* residual = sg.residual ? buffer(sg.residual) : NULL;
+      if (groups > 0) {
+        STEP(sg.convStage, sg.op->forwardSums(slot(sg.out), slot(sg.in), slot(sg.filter), (double*)sumsBuffer, sumsBytes));
+        ABI(sg.bnStage, mcn_bnorm_forward_sums(st, buffer(sg.act), buffer(sg.moments), buffer(sg.out), buffer(sg.g), buffer(sg.b),
+                                               residual, sg.relu, sg.h, sg.w, sg.c, N, epsilon, (double const*)sumsBuffer, groups));
+      } else {
+        STEP(sg.convStage, sg.op->forward(slot(sg.out), 0, slot(sg.in), 1, slot(sg.filter), none));
+        const size_t wsBytes = mcn_bnorm_workspace_bytes(sg.h, sg.w, sg.c, N);
+        void* ws = context.getWorkspace(VLDT_GPU, wsBytes);
+        if (!ws) return fail(context.getLastError(), "workspace");
+        ABI(sg.bnStage, mcn_bnorm_forward_fused(st, buffer(sg.act), buffer(sg.moments), buffer(sg.out), buffer(sg.g), buffer(sg.b),
+                                                residual, sg.relu, sg.h, sg.w, sg.c, N, epsilon, 0, ws, wsBytes));
+      }
+    }
+    return VLE_Success;
   }
   if (fused) {
     const size_t wsMid = mcn_bnorm_workspace_bytes(H, W, M, N), wsOut = mcn_bnorm_workspace_bytes(Ho, Wo, Cout, N);

@@ -67,6 +67,11 @@ class Bottleneck {
   // setOverlap.
   ErrorCode setDeferred(bool on, bool external = false);
   std::vector<mcn_conv_reduce_job> const& reduceJobs() const { return sumJobs; }
+  // epilogue sums = true (fused mode, training): the forward convolutions also sum their output per channel
+  // (mcn_conv_forward_sums) and the batch normalisations that follow take those sums instead of reading the tensor
+  // in a summing pass of their own (mcn_bnorm_forward_sums).  The moments then come from a different summation order
+  // than the two-launch form's: same values to rounding (1e-7 relative), not the same bits.
+  ErrorCode setEpilogueSums(bool on);
   ErrorCode forward();
   ErrorCode backward();
 
@@ -108,6 +113,10 @@ class Bottleneck {
   void* sumJobsDevice;
   unsigned sumBlocks;
   std::vector<mcn_conv_reduce_job> sumJobs;
+  bool epilogueSums;
+  int sumGroupsOf[4];   // [convolution]: partial sums per channel its forward writes (0: it cannot)
+  void* sumsBuffer;     // the partial sums of the convolution that ran last
+  std::size_t sumsBytes;
   Context sideContext;
   void* sideStream;     // hipStream_t
   void* events[5];      // hipEvent_t: "derivative ready" for the convolutions, "second stream done"

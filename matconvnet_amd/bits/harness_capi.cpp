@@ -190,6 +190,7 @@ int vlh_bottleneck_set_overlap(void* block, int overlap) { return (int)((BlockHa
 int vlh_bottleneck_set_deferred(void* block, int deferred) {
   return (int)((BlockHandle*)block)->block->setDeferred(deferred != 0);
 }
+int vlh_bottleneck_set_epilogue_sums(void* block, int on) { return (int)((BlockHandle*)block)->block->setEpilogueSums(on != 0); }
 int vlh_bottleneck_set_packed(void* block, int packed) { return (int)((BlockHandle*)block)->block->setPacked(packed != 0); }
 int vlh_bottleneck_pack(void* block) { return (int)((BlockHandle*)block)->block->pack(); }
 int vlh_bottleneck_forward(void* block) { return (int)((BlockHandle*)block)->block->forward(); }

@@ -55,6 +55,8 @@ VLH_API int vlh_bottleneck_set_overlap(void* block, int overlap);
 /* deferred != 0: one launch sums the reduction splits of all the unit's filter gradients at the end of backward */
 VLH_API int vlh_bottleneck_set_deferred(void* block, int deferred);
 VLH_API int vlh_bottleneck_set_packed(void* block, int packed);
+/* the forward convolutions also sum their output per channel; the batch normalisations take those sums (fused mode) */
+VLH_API int vlh_bottleneck_set_epilogue_sums(void* block, int on);
 VLH_API int vlh_bottleneck_pack(void* block);
 VLH_API int vlh_bottleneck_forward(void* block);
 VLH_API int vlh_bottleneck_backward(void* block);

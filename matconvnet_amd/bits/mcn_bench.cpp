@@ -3,7 +3,7 @@
 // synthetic inputs, times them with HIP events and prints TFLOP/s, GB/s and images/s beside the
 // fraction of the MI355X rooflines (fp32 matrix 157.3 TFLOP/s, HBM 8 TB/s).
 //
-//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|resnet50] [--batch N]
+//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|yardstick|resnet50] [--batch N] [--config C]
 //
 // The bandwidth-bound operators (bnorm, pooling, copy) are timed over R independent sets of tensors used in
 // turn (default 4), so that no launch finds its inputs in the 256 MB memory-side cache because the previous
@@ -188,6 +188,55 @@ static void benchCopy(int warmup, int iters) {
               "copy 256 MiB", t * 1e3, 2.0 * n * 4 / t / 1e6, 100 * 2.0 * n * 4 / (t * 1e-3) / kPeakHbm, n * 4, n * 4, gRotate);
 }
 
+// Sweep of the plain streaming kernels (read-only, write-only, copy) over launch shapes: workgroups per compute
+// unit (0 = one step per workgroup, not persistent), 16-byte accesses in flight per lane, walk (slab by slab over the
+// whole chip, or one contiguous run per workgroup), store hint, access width.  256 MiB per stream, buffer sets used in
+// turn like the operators' measurements.  The best line of each mode is the measured ceiling of that traffic mix.
+// `fixed` >= 0: run only that one configuration (for counter runs): mode*1000 + perCu*100 + inFlight*10 + flags.
+static void benchYardstick(int warmup, int iters, int fixed) {
+  const size_t bytes = 256u << 20;
+  TensorSet a(TensorShape(bytes / 4, 1, 1, 1), gRotate), b(TensorShape(bytes / 4, 1, 1, 1), gRotate);
+  a.first().fill(1.f);
+  a.spread();
+  const int cus = mcn_device_compute_units();
+  char const* modeName[3] = {"read", "write", "copy"};
+  struct Best { double gbs; char text[160]; } best[3] = {{0, ""}, {0, ""}, {0, ""}};
+  const int perCuList[] = {0, 2, 4, 8, 16, 32};
+  for (int mode = 0; mode < 3; ++mode)
+    for (int width : {16, 4})
+      for (int perCu : perCuList)
+        for (int inFlight : {1, 2, 4, 8})
+          for (int flags = 0; flags < 4; ++flags) {
+            if (mode == MCN_YARDSTICK_READ && (flags & MCN_YARDSTICK_NONTEMPORAL)) continue;
+            if (perCu == 0 && (flags & MCN_YARDSTICK_CHUNKED)) continue;
+            if (width == 4 && (perCu == 2 || perCu == 32 || inFlight == 1)) continue;  // (a thinner sweep of the narrow accesses)
+            if (fixed >= 0 && (fixed != mode * 1000 + perCu * 100 + inFlight * 10 + flags || width != 16)) continue;
+            int turn = 0;
+            double t = medianMs([&] {
+              int rc = mcn_hbm_yardstick(NULL, b[turn].getMemory(), a[turn].getMemory(), bytes, mode, width, inFlight,
+                                         perCu * cus, flags);
+              if (rc) {
+                std::fprintf(stderr, "yardstick: %s\n", mcn_last_error_message());
+                std::exit(3);
+              }
+              ++turn;
+            }, warmup, iters);
+            const double moved = (mode == MCN_YARDSTICK_COPY ? 2.0 : 1.0) * bytes;
+            const double gbs = moved / t / 1e6;
+            char line[160];
+            std::snprintf(line, sizeof line, "%-5s width %2d B  workgroups/CU %2d  in flight %d  %-10s %-12s %8.1f us %7.0f GB/s (%4.1f%% of 8 TB/s)",
+                          modeName[mode], width, perCu, inFlight, (flags & MCN_YARDSTICK_CHUNKED) ? "chunked" : "slab-wise",
+                          (flags & MCN_YARDSTICK_NONTEMPORAL) ? "non-temporal" : "", t * 1e3, gbs, 100 * gbs * 1e9 / kPeakHbm);
+            std::printf("%s\n", line);
+            if (gbs > best[mode].gbs) {
+              best[mode].gbs = gbs;
+              std::strcpy(best[mode].text, line);
+            }
+          }
+  for (int mode = 0; mode < 3; ++mode)
+    if (best[mode].gbs > 0) std::printf("best %s\n", best[mode].text);
+}
+
 static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, bool packed = false) {
   const int H = 56, W = 56, C = 256, M = 64, N = 32;
   harness::Bottleneck block(H, W, C, M, N, 1e-5);
@@ -301,7 +350,7 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
 }
 
 int main(int argc, char** argv) {
-  int iters = 20, warmup = 3, batch = 32;
+  int iters = 20, warmup = 3, batch = 32, fixed = -1;
   std::string only;
   for (int i = 1; i < argc; ++i) {
     if (!std::strcmp(argv[i], "--iters") && i + 1 < argc) iters = std::atoi(argv[++i]);
@@ -309,8 +358,9 @@ int main(int argc, char** argv) {
     else if (!std::strcmp(argv[i], "--only") && i + 1 < argc) only = argv[++i];
     else if (!std::strcmp(argv[i], "--batch") && i + 1 < argc) batch = std::max(1, std::atoi(argv[++i]));
     else if (!std::strcmp(argv[i], "--rotate") && i + 1 < argc) gRotate = std::max(1, std::atoi(argv[++i]));
+    else if (!std::strcmp(argv[i], "--config") && i + 1 < argc) fixed = std::atoi(argv[++i]);
     else {
-      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|resnet50] [--batch N]\n");
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|yardstick|resnet50] [--batch N] [--config C]\n");
       return 1;
     }
   }
@@ -319,6 +369,7 @@ int main(int argc, char** argv) {
   std::printf("device: %s, %d CUs, %.0f MHz\n", prop.name, prop.multiProcessorCount, prop.clockRate / 1000.0);
   auto want = [&](char const* k) { return only.empty() || only == k; };
   if (only == "copy") benchCopy(warmup, iters);
+  if (only == "yardstick") benchYardstick(warmup, iters, fixed);
   if (only == "resnet50") {
     benchResNet(warmup, iters, batch, false);
     benchResNet(warmup, iters, batch, true);

@@ -70,6 +70,33 @@ ErrorCode Convolution::forward(Tensor& output, double outputMult, Tensor const& 
   return fromAbi(context, rc, "Convolution::forward");
 }
 
+int Convolution::sumGroups(TensorShape const& data, TensorShape const& filter) const {
+  mcn_conv_geom g = geometry(*this, data, filter);
+  return mcn_conv_forward_sums_groups(&g);
+}
+
+ErrorCode Convolution::forwardSums(Tensor& output, Tensor const& input, Tensor const& filter, double* sums,
+                                   std::size_t sumsBytes) {
+  tensor_type tt = findTensorType(output, input, filter);
+  ErrorCode e = requireHipFloat(context, tt, "Convolution::forwardSums");
+  if (e != VLE_Success) return e;
+  if (!output || !input || !filter)
+    return context.setError(VLE_IllegalArgument, "Convolution::forwardSums: OUTPUT, INPUT and FILTER are required");
+  mcn_conv_geom g = geometry(*this, input, filter);
+  int oh = 0, ow = 0;
+  int rc = mcn_conv_output_size(&g, &oh, &ow);
+  if (rc) return fromAbi(context, rc, "Convolution::forwardSums");
+  if ((int)output.getHeight() != oh || (int)output.getWidth() != ow || output.getDepth() != filter.getSize() ||
+      output.getSize() != input.getSize())
+    return context.setError(VLE_IllegalArgument, "Convolution::forwardSums: OUTPUT dimensions are incompatible with X and FILTERS");
+  void* ws;
+  size_t bytes;
+  if (!scratch(context, g, MCN_CONV_FORWARD, &ws, &bytes)) return context.getLastError();
+  rc = mcn_conv_forward_sums(context.getHipHelper().getStream(), &g, (float*)output.getMemory(), (float const*)input.getMemory(),
+                             (float const*)filter.getMemory(), packedForward, packedForwardBytes, sums, sumsBytes, ws, bytes);
+  return fromAbi(context, rc, "Convolution::forwardSums");
+}
+
 std::size_t Convolution::packedBytes(int product, TensorShape const& data, TensorShape const& filter) const {
   mcn_conv_geom g = geometry(*this, data, filter);
   return mcn_conv_packed_bytes(&g, product);

@@ -53,6 +53,14 @@ class Convolution {
   vl::ErrorCode backwardFilterPartial(vl::Tensor& derFilter, vl::Tensor const& input, vl::Tensor const& derOutput,
                                       void* partials, std::size_t bytes);
 
+  // Forward (no bias, output overwritten) that also sums the output and its square per channel in the same launch
+  // (mcn_conv_forward_sums): the summing pass of a batch normalisation that follows.  sumGroups: partial sums per
+  // channel for this geometry (0: no such form; use forward); sums: device buffer of K * sumGroups * 2 doubles.  Not
+  // part of the reference's class.
+  int sumGroups(vl::TensorShape const& data, vl::TensorShape const& filter) const;
+  vl::ErrorCode forwardSums(vl::Tensor& output, vl::Tensor const& input, vl::Tensor const& filter, double* sums,
+                            std::size_t sumsBytes);
+
   Context& context;
   int strideY;
   int strideX;

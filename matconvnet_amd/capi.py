@@ -55,9 +55,13 @@ PROTOTYPES = {
     "mcn_get_tunable": (_i, [C.c_char_p, C.POINTER(_i)]),
     "mcn_profile_begin": (_i, [C.c_char_p]),
     "mcn_profile_end": (_i, [C.POINTER(_i), C.POINTER(_d)]),
+    "mcn_hbm_yardstick": (_i, [_vp, _vp, _vp, _sz, _i, _i, _i, _i, _i]),
     "mcn_conv_output_size": (_i, [C.POINTER(ConvGeom), C.POINTER(_i), C.POINTER(_i)]),
     "mcn_conv_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _i]),
     "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),
+    "mcn_conv_forward_sums_groups": (_i, [C.POINTER(ConvGeom)]),
+    "mcn_conv_forward_sums": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz]),
+    "mcn_bnorm_forward_sums": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _d, _vp, _i]),
     "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_taccum": (_i, [_vp, _vp, C.c_float, _vp, C.c_float, _vp, _sz]),
     "mcn_conv_backward_filter_partial_bytes": (_sz, [_vp]),
@@ -287,6 +291,35 @@ def conv_forward(x, f, b, g, y=None, out_mult=0.0, in_mult=1.0, ws=None):
     wp, wn = ws.get(lib().mcn_conv_workspace_bytes(C.byref(g), CONV_FORWARD))
     check(lib().mcn_conv_forward(stream(), C.byref(g), ptr(y), out_mult, ptr(x), in_mult, ptr(f), ptr(b), wp, wn))
     return y
+
+
+def conv_forward_sums_groups(g):
+    """Partial sums per channel mcn_conv_forward_sums writes for this geometry; 0: no such form."""
+    return int(lib().mcn_conv_forward_sums_groups(C.byref(g)))
+
+
+def conv_forward_sums(x, f, g, packed=None, ws=None):
+    """y = conv(x, f) and, from the same launch, partial sums of y and y^2 per channel: (y, sums[K][groups][2] in double)."""
+    import torch
+    ws = ws or _ws
+    groups = conv_forward_sums_groups(g)
+    y = empty(conv_out_shape(g), like=x)
+    K = int(g.K)
+    sums = torch.zeros(max(K * groups * 2, 1), dtype=torch.float64, device="cuda")
+    wp, wn = ws.get(lib().mcn_conv_workspace_bytes(C.byref(g), CONV_FORWARD))
+    pk, pkn = (ptr(packed), packed.numel() * packed.element_size()) if packed is not None else (None, 0)
+    check(lib().mcn_conv_forward_sums(stream(), C.byref(g), ptr(y), ptr(x), ptr(f), pk, pkn, ptr(sums), sums.numel() * 8, wp, wn))
+    return y, sums.view(K, max(groups, 1), 2)
+
+
+def bnorm_forward_sums(x, g, b, sums, residual=None, relu=False, eps=1e-4):
+    """Batch normalisation (with optional shortcut sum and ReLU) that takes its channel sums from `sums`."""
+    H, W, Cc, N = _hwcn(x)
+    y = empty((H, W, Cc, N))
+    mom = empty((Cc, 2))
+    check(lib().mcn_bnorm_forward_sums(stream(), ptr(y), ptr(mom), ptr(x), ptr(g), ptr(b), ptr(residual), int(relu),
+                                       H, W, Cc, N, eps, ptr(sums), int(sums.shape[1])))
+    return y, mom
 
 
 def conv_backward(x, f, dy, g, want=(True, True, True), ws=None):

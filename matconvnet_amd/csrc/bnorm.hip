@@ -60,6 +60,8 @@ struct BnormP {
   int teamShift[2];  // log2 of the threads that share one plane, for scalar [0] and 16-byte [1] accesses: planes
                      // smaller than a workgroup's 256 accesses are walked several at a time, one per team
   int oneLaunch;     // groups == 1 and the apply kernels compute the sums themselves (small channels): no sums launch
+  int sumGroups, sumStride;  // the partial sums the apply kernels add up: sumGroups per channel, sumStride doubles each
+                             // (groups and 4 after a sums launch of this file; 2 when a convolution summed its output)
   double mass;       // WH * N
   double epsilon;
 };
@@ -212,28 +214,34 @@ __device__ __forceinline__ void own_totals(double (&tot)[4], const float* __rest
 }
 
 // Sum of a channel's partials in a fixed order: lane i owns groups i, i+64, ...; then a wave tree.
-// Every lane of wave 0 ends with the totals; other waves read them from LDS.
+// Every lane of wave 0 ends with the totals; other waves read them from LDS.  More than 64 partials (the sums a
+// convolution left, one per workgroup of its launch) are shared by all four wavefronts, thread i owning groups i,
+// i+256, ..., and the four wavefront sums are added in wavefront order: a quarter of the dependent loads.
+// `lds`: 20 doubles.
 __device__ __forceinline__ void channel_totals(const double* __restrict__ partials, const BnormP& p,
                                                int c, double* lds, double (&tot)[4]) {
-  if (threadIdx.x < kWave) {
+  const bool wide = p.sumGroups > kWave;
+  if (wide || threadIdx.x < kWave) {
     double v[4] = {0.0, 0.0, 0.0, 0.0};
-    for (int g = threadIdx.x; g < p.groups; g += kWave) {
-      const double* in = partials + ((size_t)c * p.groups + g) * 4;
+    for (int g = threadIdx.x; g < p.sumGroups; g += wide ? 256 : kWave) {
+      const double* in = partials + ((size_t)c * p.sumGroups + g) * p.sumStride;
       v[0] += in[0];
       v[1] += in[1];
-      v[2] += in[2];
-      v[3] += in[3];
+      if (p.sumStride == 4) {
+        v[2] += in[2];
+        v[3] += in[3];
+      }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = wave_sum(v[i]);
-    if (threadIdx.x == 0) {
+    if ((threadIdx.x & (kWave - 1)) == 0) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) lds[i] = v[i];
+      for (int i = 0; i < 4; ++i) lds[(threadIdx.x / kWave) * 4 + i] = v[i];
     }
   }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 4; ++i) tot[i] = lds[i];
+  for (int i = 0; i < 4; ++i) tot[i] = wide ? ((lds[i] + lds[4 + i]) + lds[8 + i]) + lds[12 + i] : lds[i];
 }
 
 // out = a*(in1 - t) + b*(in2 - s) + k over this workgroup's planes (in2 optional)
@@ -455,6 +463,8 @@ int setup(const char* who, int H, int W, int C, int N, double epsilon, BnormP* p
     while (shift < 8 && (1 << shift) < accesses) ++shift;
     p->teamShift[v] = shift;
   }
+  p->sumGroups = p->groups;
+  p->sumStride = 4;
   p->mass = (double)p->WH * (double)N;
   p->epsilon = epsilon;
   if ((long long)C * p->groups >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: too many channels", who);
@@ -526,6 +536,42 @@ int mcn_bnorm_forward_fused(mcn_stream_t stream, float* y, float* moments, const
 #undef MCN_BN_FWD_EPI
 #undef MCN_BN_FWD
   return check_launch("mcn_bnorm_forward");
+}
+
+int mcn_bnorm_forward_sums(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,
+                           const float* biases, const float* residual, int relu, int H, int W, int C, int N, double epsilon,
+                           const double* sums, int sumGroups) {
+  BnormP p;
+  int rc = setup("mcn_bnorm_forward_sums", H, W, C, N, epsilon, &p);
+  if (rc) return rc;
+  if ((size_t)p.WH * C * N == 0) return MCN_SUCCESS;
+  if (!y || !x || !multipliers || !biases || !sums) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_sums: null tensor");
+  if (sumGroups <= 0) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_sums: no partial sums");
+  if (p.oneLaunch) {  // (the grid of the two-launch form: the sums are there already)
+    p.oneLaunch = 0;
+    p.groups = image_groups(p.WH, N);
+  }
+  p.sumGroups = sumGroups;
+  p.sumStride = 2;
+  p.reverse = 0;
+  hipStream_t s = as_stream(stream);
+  const bool vec = (p.WH % 4 == 0) && aligned16(y) && aligned16(x) && (!residual || aligned16(residual));
+  const dim3 grid((unsigned)(C * p.groups)), block(256);
+  KernelTimer timer("bnorm_forward_apply", s);
+#define MCN_BN_SUMS(VECF, RESF, RELUF) \
+  hipLaunchKernelGGL((bnorm_forward_apply<false, VECF, RESF, RELUF>), grid, block, 0, s, y, moments, x, multipliers, biases, residual, sums, p)
+#define MCN_BN_SUMS_EPI(VECF)                              \
+  do {                                                     \
+    if (residual && relu) MCN_BN_SUMS(VECF, true, true);   \
+    else if (residual) MCN_BN_SUMS(VECF, true, false);     \
+    else if (relu) MCN_BN_SUMS(VECF, false, true);         \
+    else MCN_BN_SUMS(VECF, false, false);                  \
+  } while (0)
+  if (vec) MCN_BN_SUMS_EPI(true);
+  else MCN_BN_SUMS_EPI(false);
+#undef MCN_BN_SUMS_EPI
+#undef MCN_BN_SUMS
+  return check_launch("mcn_bnorm_forward_sums");
 }
 
 int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,

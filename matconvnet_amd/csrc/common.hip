@@ -24,7 +24,8 @@ struct Tunable {
 Tunable g_tunables[] = {
     {"pool_lds_bytes", 16 * 1024},     // LDS tile budget of the pooling-backward kernels
     {"pool_no_stream", 0},             // 1: max pooling skips the streaming kernel
-    {"pool_walk", 0},                  // streaming kernel's tile order: 0 round-robin, 1 contiguous runs, 2 round-robin per XCD
+    {"pool_walk", 0},                  // streaming kernel's tile order: 0 round-robin, 1 contiguous runs, 2 round-robin per XCD eighth, 3 planes round-robin over XCDs
+    {"pool_threads", 256},             // threads per workgroup of the streaming kernel (256; 512 and 1024 for 3x3 / 2 windows)
     {"pool_blocks_per_cu", 3},         // persistent workgroups per compute unit of the streaming kernel
     {"pool_forward_threads_k", 2048},  // threads (in 1024s) the four-rows-per-thread forward kernel aims at
     {"pool_force_gather", 0},          // 1: skip the ordered-pass kernel, use the general tiled gather

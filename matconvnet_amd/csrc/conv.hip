@@ -233,6 +233,34 @@ int mcn_conv_forward_packed(mcn_stream_t stream, const mcn_conv_geom* g, float* 
   return conv_forward_direct(as_stream(stream), p, y, outMult, x, inMult, filters, bias);
 }
 
+int mcn_conv_forward_sums_groups(const mcn_conv_geom* g) {
+  ConvP p;
+  if (conv_setup(g, "mcn_conv_forward_sums_groups", &p) || (size_t)p.outH * p.outW * p.K * p.N == 0) return 0;
+  if (tunable("conv_force_direct", 0) || !conv_mfma_forward_supported(p)) return 0;
+  int groups = 0;
+  float* dummy = nullptr;  // (nothing is touched when planning)
+  if (conv_forward_mfma(nullptr, p, dummy, 0.f, dummy, 1.f, dummy, nullptr, nullptr, 0, nullptr, nullptr, 0, &groups)) return 0;
+  return groups;
+}
+
+int mcn_conv_forward_sums(mcn_stream_t stream, const mcn_conv_geom* g, float* y, const float* x, const float* filters,
+                          const void* packed, size_t packedBytes, double* sums, size_t sumsBytes, void* workspace,
+                          size_t workspaceBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_forward_sums", &p);
+  if (rc) return rc;
+  if (!y || !x || !filters || !sums) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_forward_sums: null tensor");
+  const int groups = mcn_conv_forward_sums_groups(g);
+  if (groups <= 0) return fail(MCN_UNSUPPORTED, "mcn_conv_forward_sums: this geometry has no such form (ask mcn_conv_forward_sums_groups)");
+  if (sumsBytes < (size_t)p.K * groups * 2 * sizeof(double))
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_forward_sums: the buffer of partial sums is too small");
+  if (packed) {
+    PackCtx pk = {PackCtx::kUse, (char*)const_cast<void*>(packed), packedBytes, 0, nullptr};
+    return conv_forward_mfma(as_stream(stream), p, y, 0.f, x, 1.f, filters, nullptr, workspace, workspaceBytes, &pk, sums, groups);
+  }
+  return conv_forward_mfma(as_stream(stream), p, y, 0.f, x, 1.f, filters, nullptr, workspace, workspaceBytes, nullptr, sums, groups);
+}
+
 int mcn_conv_backward_data_packed(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, float derInputMult,
                                   const float* filters, const void* packed, size_t packedBytes, const float* derOutput,
                                   void* workspace, size_t workspaceBytes) {

@@ -77,8 +77,10 @@ bool conv_mfma_forward_supported(const ConvP& p);
 bool conv_mfma_backward_data_supported(const ConvP& p);
 bool conv_mfma_backward_filter_supported(const ConvP& p);
 size_t conv_mfma_workspace_bytes(const ConvP& p, int product);
+// stats / statGroups: also write per-channel partial sums of y and y^2 (see PixP::stats); statQuery: plan only
 int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
-                      const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk = nullptr);
+                      const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk = nullptr,
+                      double* stats = nullptr, int statGroups = 0, int* statQuery = nullptr);
 int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
                             void* ws, size_t wsBytes, PackCtx* pk = nullptr);
 int conv_pack_batch(hipStream_t s, const PackJob* deviceJobs, int nJobs, unsigned totalBlocks);
@@ -113,6 +115,12 @@ struct PixP {
   // (fully-connected layers above all), which would otherwise keep a handful of workgroups busy for a long time.
   int rSplits, stepsPerSplit;
   long long partStride;
+  // Per-channel sums of the produced tensor taken in the same launch (weights-stationary kernel only): where the
+  // partial sums go, and how many of them each channel gets.  statQuery (host only): no launch, just report that
+  // number (0: this product has no such form).
+  double* stats = nullptr;
+  int statGroups = 0;
+  int* statQuery = nullptr;
 };
 
 // the pixel's element offset inside its channel plane of the produced tensor
@@ -201,6 +209,8 @@ __device__ __forceinline__ void store_block(floatx16 acc, bufrsrc rsrc, unsigned
 // 16-channel-chunk order of conv_pack_weights.  Sets *handled when it took the work.
 int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, const float* wt, const float* bias,
                    const PixP& p, int* handled);
+// partial sums per channel it would write when asked to sum its output (PixP::stats); 0: it would not take `p` that way
+int conv_ws_stat_groups(const PixP& p);
 
 // Products with at most four output channels (conv_few.hip): wt is the packed bank (tapMajor: its row order, see
 // conv_pack_weights).  Sets *handled when it took the work.

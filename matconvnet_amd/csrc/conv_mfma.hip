@@ -883,6 +883,11 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   // uniform-tap variant: whole 16-row steps inside one tap, and 32-bit element offsets into the gathered tensor
   const long long inSpan = (long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW;  // elements from `in` to the end
   const bool ut = p.Cin % 16 == 0 && inSpan < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
+  if (p.statQuery) {  // (plan only: would this product also sum its output per channel, and into how many partials?)
+    *p.statQuery = ut && p.Cout > 4 && !bias && p.beta == 0.f ? conv_ws_stat_groups(p) : 0;
+    return MCN_SUCCESS;
+  }
+  if (p.stats && !(ut && p.Cout > 4)) return fail(MCN_UNSUPPORTED, "%s: this product cannot sum its output per channel", who);
   // The backward-data product of a 1x1 bank whose extents need no padding reads it as it is stored: rows = filters,
   // columns = the filters' channels, which is the packed order.
   const bool asStored = backward && taps.FH * taps.FW == 1 && rPad == p.R && p.coutPad == p.Cout && aligned16(f);
@@ -951,6 +956,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
     rc = conv_ws_launch(s, who, out, in, wt, bias, p, &handled);
     if (rc || handled) return rc;
   }
+  if (p.stats) return fail(MCN_UNSUPPORTED, "%s: this product cannot sum its output per channel", who);
   if (plan.splits > 1) {
     // every workgroup a slice of the reduction into its own partial tensor, then one pass to add them up
     float* partials = (float*)((char*)ws + align256(needW));
@@ -1075,8 +1081,12 @@ void dense_layout(PixP* q) {
 
 namespace {
 int forward_group(hipStream_t s, const ConvP& p, Wide wd, float* y, float outMult, const float* x, float inMult,
-                  const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk) {
+                  const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk, double* stats, int statGroups,
+                  int* statQuery) {
   PixP q;
+  q.stats = stats;
+  q.statGroups = statGroups;
+  q.statQuery = statQuery;
   q.IH = p.H; q.IW = p.W; q.Cin = p.C;
   q.OH = p.outH; q.OW = p.outW; q.Cout = p.K;
   q.N = p.N;
@@ -1102,14 +1112,22 @@ int conv_pack_batch(hipStream_t s, const PackJob* deviceJobs, int nJobs, unsigne
 }
 
 int conv_forward_mfma(hipStream_t s, const ConvP& original, float* y, float outMult, const float* x, float inMult,
-                      const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk) {
+                      const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk, double* stats, int statGroups,
+                      int* statQuery) {
   const ConvP p = fc_view(original);
   const ConvP g = group_view(p);
   const Wide wd = wide_of(p);
+  if ((stats || statQuery) && p.groups != 1) {
+    if (statQuery) {
+      *statQuery = 0;
+      return MCN_SUCCESS;
+    }
+    return fail(MCN_UNSUPPORTED, "mcn_conv_forward_sums: filter groups are not supported");
+  }
   const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
   for (int i = 0; i < p.groups; ++i) {
     int rc = forward_group(s, g, wd, y + i * p.Kg * Q, outMult, x + i * p.FC * HW, inMult, f + i * p.Kg * FV,
-                           b ? b + i * p.Kg : nullptr, ws, wsBytes, pk);
+                           b ? b + i * p.Kg : nullptr, ws, wsBytes, pk, stats, statGroups, statQuery);
     if (rc) return rc;
   }
   return MCN_SUCCESS;

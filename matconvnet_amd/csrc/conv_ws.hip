@@ -45,13 +45,32 @@ struct WsP {
   FastDiv byCB, byRow;  // byRow: 8 WA = 16-byte vectors per bank row of one channel block
 };
 
-template <int WA, bool TAPS, int THREADS>
+// STATS (WA = 1, one slice, no bias, beta = 0, every wavefront on one channel block for good): the kernel also sums what
+// it stores, and its square, per output channel -- the first pass of a batch normalisation that follows, taken from
+// the accumulators instead of re-reading the tensor.  Each lane keeps fp32 running sums of its pixels over the
+// wavefront's units (a few values each), the wavefront adds its lanes up once at the end, the wavefronts of a workgroup
+// that share a channel block add theirs through LDS in a fixed order, and the workgroup writes one fp64 partial per
+// channel (alpha must be 1): p.stats[(channel * p.statGroups + workgroup) * 2 + {0: sum, 1: sum of squares}].  Which
+// pixels a workgroup sums is fixed by the launch shape: same bits every run.
+// Sum over a row of 16 lanes, left in the row's lane 15: v += v shifted right by 1, 2, 4, 8 lanes inside the row (zeros
+// shift in), each a single vector add with a lane-shift modifier.
+__device__ __forceinline__ float row_sum16(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true));
+  return v;
+}
+
+template <int WA, bool TAPS, int THREADS, bool STATS = false>
 __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out, const float* __restrict__ in,
                                                         const float* __restrict__ wt, const float* __restrict__ bias,
                                                         PixP p, WsP w) {
+  static_assert(!STATS || WA == 1, "channel sums are kept for one 32-channel block per wavefront");
   extern __shared__ float smem[];
   float* wtL = smem;  // [chanBlocks][R][32 WA]
   constexpr int ROW = 32 * WA;                     // floats per bank row of one channel block
+  float* statsL = smem + (size_t)p.R * p.coutPad;  // STATS: [wavefront][2 rows of lanes][32 channels][2], behind the bank
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -91,6 +110,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
       for (int k = 0; k < 4; ++k)
         if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
     }
+    if (STATS) statsL[tid] = statsL[tid + THREADS] = 0.f;  // ([THREADS / 64][2 rows][32][2]: wavefronts without units leave zeros)
   }
   __syncthreads();
 
@@ -107,7 +127,52 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   // fetches 30 MB per launch through the fabric instead of 128 MB.  Without taps nothing is shared and spreading
   // neighbours over the XCDs measured 5% faster.)
   int unit = ((wave / sib) * nWg + wg) * sib + (wave % sib);
-  if (wave >= slots * sib || unit >= w.nUnits) return;
+  if (wave >= slots * sib) return;
+  // (STATS: sib = chanBlocks, so a wavefront's channel block is wave % sib for all its units)
+  float s1[STATS ? 16 : 1], s2[STATS ? 16 : 1];
+  auto write_stats = [&]() {
+    if (!STATS) return;
+    // the 32 lanes of a half-wave hold the same 16 channels for 32 different pixels.  Rows of 16 lanes are added up
+    // inside the vector unit (four shifted adds: lane 15 of a row ends with the row's sum), the two rows of a half meet
+    // in LDS.
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      s1[r] = row_sum16(s1[r]);
+      s2[r] = row_sum16(s2[r]);
+    }
+    if ((lane & 15) == 15) {
+      const int row = l32 >> 4;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c = 4 * kh + 8 * (r / 4) + r % 4;  // channel inside the block
+        statsL[((wave * 2 + row) * 32 + c) * 2] = s1[r];
+        statsL[((wave * 2 + row) * 32 + c) * 2 + 1] = s2[r];
+      }
+    }
+    __syncthreads();  // (wavefronts that had no units have left already: the barrier counts the others)
+    // wavefront b < sib adds up channel block b: slots in ascending order, lane = channel, in double
+    if (wave < sib && lane < 32) {
+      double t1 = 0.0, t2 = 0.0;
+      for (int j = 0; j < slots; ++j)
+        for (int row = 0; row < 2; ++row) {
+          t1 += (double)statsL[(((j * sib + wave) * 2 + row) * 32 + lane) * 2];
+          t2 += (double)statsL[(((j * sib + wave) * 2 + row) * 32 + lane) * 2 + 1];
+        }
+      const int c = wave * 32 + lane;
+      if (c < p.Cout) {
+        double* o = p.stats + ((size_t)c * p.statGroups + wg) * 2;
+        o[0] = t1;
+        o[1] = t2;
+      }
+    }
+  };
+  if (STATS) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s1[r] = s2[r] = 0.f;
+  }
+  // (STATS: wavefront b < sib writes the workgroup's partial of channel block b, so it stays to the end even without
+  // units; the host admits only launches in which every workgroup has units for its first wavefronts)
+  if (unit >= w.nUnits) return;
 
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, (int)w.inBytes, 0x00020000);
   const int planeBytes = IHW * 4;
@@ -247,6 +312,15 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
       for (int a = 0; a < WA; ++a)
         store_block(acc[a], orsrc, vo, (cbOut * ROW + a * 32) * plane, plane, p.alpha, p.beta,
                     bias ? bias + cbOut * ROW + a * 32 : nullptr, kh);
+      if (STATS) {
+        // what was stored is the accumulator itself (alpha = 1; lanes past the last pixel hold zeros: their loads
+        // fetched nothing)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          s1[r] += acc[0][r];
+          s2[r] = fmaf(acc[0][r], acc[0][r], s2[r]);
+        }
+      }
     } else if (mo < p.M) {
       int n, q;
       p.byQ.divmod(mo, &n, &q);
@@ -276,11 +350,12 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     aG = aLane;
     quadsLeft = quadsPerUnit;
   }
+  write_stats();
 #undef WS_STEP
 #undef WS_LOAD_NEXT
 }
 
-template <int WA, bool TAPS, int THREADS>
+template <int WA, bool TAPS, int THREADS, bool STATS = false>
 int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, const float* in, const float* wt,
            const float* bias, const PixP& p, const WsP& w) {
   // largest dynamic LDS size this instantiation has been opted into, per device (concurrent callers may both opt in:
@@ -288,7 +363,7 @@ int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, c
   static std::atomic<size_t> raised[kMaxDevices];
   const int dev = current_device();
   if (lds > 64 * 1024 && (dev < 0 || dev >= kMaxDevices || lds > raised[dev].load(std::memory_order_acquire))) {
-    if (hipFuncSetAttribute((const void*)conv_ws_mfma<WA, TAPS, THREADS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)conv_ws_mfma<WA, TAPS, THREADS, STATS>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return fail(MCN_DEVICE_ERROR, "%s: cannot reserve %zu bytes of LDS", who, lds);
@@ -300,7 +375,7 @@ int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, c
     }
   }
   KernelTimer timer("conv_ws_mfma", s);
-  hipLaunchKernelGGL((conv_ws_mfma<WA, TAPS, THREADS>), dim3((unsigned)blocks), dim3(THREADS), lds, s, out, in, wt, bias, p, w);
+  hipLaunchKernelGGL((conv_ws_mfma<WA, TAPS, THREADS, STATS>), dim3((unsigned)blocks), dim3(THREADS), lds, s, out, in, wt, bias, p, w);
   return check_launch(who);
 }
 
@@ -311,6 +386,13 @@ int dispatch(hipStream_t s, const char* who, int cus, bool twoFit, size_t lds, f
              const float* bias, const PixP& p, const WsP& w) {
   if constexpr (WA == 4) {
     return launch<WA, TAPS, 512>(s, who, cus, lds, out, in, wt, bias, p, w);
+  } else if constexpr (WA == 1) {
+    if (p.stats) {
+      if (twoFit) return launch<1, TAPS, 512, true>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
+      return launch<1, TAPS, 1024, true>(s, who, cus, lds, out, in, wt, bias, p, w);
+    }
+    if (twoFit) return launch<WA, TAPS, 512>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
+    return launch<WA, TAPS, 1024>(s, who, cus, lds, out, in, wt, bias, p, w);
   } else {
     if (twoFit) return launch<WA, TAPS, 512>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
     return launch<WA, TAPS, 1024>(s, who, cus, lds, out, in, wt, bias, p, w);
@@ -319,31 +401,40 @@ int dispatch(hipStream_t s, const char* who, int cus, bool twoFit, size_t lds, f
 
 }  // namespace
 
-int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, const float* wt, const float* bias,
-                   const PixP& p, int* handled) {
-  *handled = 0;
-  if (tunable("conv_no_ws", 0)) return MCN_SUCCESS;
-  if (p.Cin % (2 * kDepth) != 0 || p.R % (8 * kDepth) != 0 || p.T > kMaxTapsWs || p.coutPad % 32 != 0) return MCN_SUCCESS;
+namespace {
+
+// How the weights-stationary kernel would run `p`: unit width, slices, workgroups.  False: it does not take this
+// product.  wantStats: only shapes that can also sum their output per channel (see the kernel).
+struct WsPlan {
+  int WA, cus, statGroups;
+  bool taps, twoFit;
+  size_t lds;
+  WsP w;
+};
+
+bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
+  if (tunable("conv_no_ws", 0)) return false;
+  if (p.Cin % (2 * kDepth) != 0 || p.R % (8 * kDepth) != 0 || p.T > kMaxTapsWs || p.coutPad % 32 != 0) return false;
   // the bank, or the smallest power-of-two number of slices of it (each a multiple of 32 output channels), in 150 KB
-  const int maxSlices = std::max(1, tunable("conv_ws_max_slices", 8));
+  const int maxSlices = wantStats ? 1 : std::max(1, tunable("conv_ws_max_slices", 8));
   int slices = 1;
   while (slices <= maxSlices && ((size_t)p.R * (p.coutPad / slices) * sizeof(float) > 150 * 1024 || p.coutPad % (32 * slices) != 0)) {
-    if (p.coutPad % (32 * slices * 2) != 0) return MCN_SUCCESS;
+    if (p.coutPad % (32 * slices * 2) != 0) return false;
     slices *= 2;
   }
-  if (slices > maxSlices) return MCN_SUCCESS;
+  if (slices > maxSlices) return false;
   // every slice gathers all the pixels again: with a strided gather (half of each line fetched unused) the tiled
   // kernel, which gathers once, is the faster one
-  if (slices > 1 && (p.sy > 1 || p.sx > 1) && !tunable("conv_ws_sliced_strided", 0)) return MCN_SUCCESS;
+  if (slices > 1 && (p.sy > 1 || p.sx > 1) && !tunable("conv_ws_sliced_strided", 0)) return false;
   const int coutSlice = p.coutPad / slices;
   const size_t lds = (size_t)p.R * coutSlice * sizeof(float);
   // byte offsets into the gathered tensor must stay below the "outside" offset
   const long long inBytes = ((long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW) * 4;
-  if (inBytes >= (long long)kOutside) return MCN_SUCCESS;
+  if (inBytes >= (long long)kOutside) return false;
 
-  int cus = mcn_device_compute_units();
+  int cus = device_compute_units();
   if (cus <= 0) cus = 256;
-  if (cus % slices != 0) return MCN_SUCCESS;  // (every slice gets the same number of workgroups)
+  if (cus % slices != 0) return false;  // (every slice gets the same number of workgroups)
   const bool twoFit = lds <= 78 * 1024;  // two workgroups per CU fit the 160 KB
   const long long simds = (long long)cus * 4;
   const long long pixelBlocks = ((long long)p.M + 31) / 32;
@@ -351,7 +442,7 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
   // channels per wavefront: the widest unit that still spreads evenly over the SIMDs (wider units amortise the
   // pixel loads over more MFMAs; narrower ones balance better)
   const int minUnits = tunable("conv_ws_min_units", 0);
-  int WA = tunable("conv_ws_wa", 0);
+  int WA = wantStats ? 1 : tunable("conv_ws_wa", 0);
   if (WA != 1 && WA != 2 && WA != 4) {
     double best = 0;
     for (int cand : {4, 2, 1}) {
@@ -369,24 +460,64 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
       }
     }
   }
-  if (coutSlice % (32 * WA) != 0) return MCN_SUCCESS;
+  if (coutSlice % (32 * WA) != 0) return false;
   WsP w;
   w.slices = slices;
   w.chanBlocks = coutSlice / (32 * WA);
   const long long units = pixelBlocks * w.chanBlocks;  // per slice
   // too little work to occupy even half of the SIMDs: leave it to the tiled kernel, which can split its reduction
-  if (units >= (1ll << 30) || units * slices < (minUnits > 0 ? (long long)minUnits : simds / 2)) return MCN_SUCCESS;
+  if (units >= (1ll << 30) || units * slices < (minUnits > 0 ? (long long)minUnits : simds / 2)) return false;
   w.nUnits = (int)units;
   w.groups = p.R / (2 * kDepth);
   w.groupsPerTap = p.Cin / (2 * kDepth);
   w.inBytes = (unsigned)inBytes;
   w.byCB = FastDiv(w.chanBlocks);
   w.byRow = FastDiv(8 * WA);
-  const bool taps = !(p.T == 1 && p.dhBase == 0 && p.dwBase == 0 && p.sy == 1 && p.sx == 1 && p.IH == p.OH && p.IW == p.OW);
+  plan->WA = WA;
+  plan->cus = cus;
+  plan->taps = !(p.T == 1 && p.dhBase == 0 && p.dwBase == 0 && p.sy == 1 && p.sx == 1 && p.IH == p.OH && p.IW == p.OW);
+  plan->twoFit = twoFit;
+  plan->lds = lds;
+  plan->w = w;
+  plan->statGroups = 0;
+  if (wantStats) {
+    // every wavefront must stay on one channel block: the channel blocks sit side by side in a workgroup
+    const int wavesPerGroup = twoFit ? 8 : 16;
+    if (wavesPerGroup % w.chanBlocks != 0 || p.beta != 0.f || p.alpha != 1.f) return false;
+    const int nWg = twoFit ? cus * 2 : cus;
+    // the first wavefronts of every workgroup (slot 0) must have a unit: they write the workgroup's partials
+    if (units < (long long)nWg * w.chanBlocks) return false;
+    if (lds + (size_t)wavesPerGroup * 128 * sizeof(float) > 160 * 1024 / (twoFit ? 2 : 1)) return false;
+    plan->lds = lds + (size_t)wavesPerGroup * 128 * sizeof(float);
+    plan->statGroups = nWg;
+  }
+  return true;
+}
+
+}  // namespace
+
+int conv_ws_stat_groups(const PixP& p) {
+  WsPlan plan;
+  return plan_ws(p, true, &plan) ? plan.statGroups : 0;
+}
+
+int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, const float* wt, const float* bias,
+                   const PixP& p, int* handled) {
+  *handled = 0;
+  WsPlan plan;
+  const bool wantStats = p.stats != nullptr;
+  if (!plan_ws(p, wantStats, &plan) || (wantStats && (bias || plan.statGroups != p.statGroups))) {
+    if (wantStats) return fail(MCN_UNSUPPORTED, "%s: this product cannot sum its output per channel", who);
+    return MCN_SUCCESS;
+  }
+  const int WA = plan.WA, cus = plan.cus;
+  const bool twoFit = plan.twoFit;
+  const size_t lds = plan.lds;
+  const WsP& w = plan.w;
   int rc;
-  if (taps) rc = WA == 4 ? dispatch<4, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
-                 : (WA == 2 ? dispatch<2, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
-                            : dispatch<1, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w));
+  if (plan.taps) rc = WA == 4 ? dispatch<4, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
+                      : (WA == 2 ? dispatch<2, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
+                                 : dispatch<1, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w));
   else rc = WA == 4 ? dispatch<4, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
             : (WA == 2 ? dispatch<2, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
                        : dispatch<1, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w));

@@ -16,6 +16,7 @@
 #include "mcn_internal.hpp"
 
 #include <algorithm>
+#include <atomic>
 
 #pragma clang fp contract(off)
 
@@ -30,12 +31,13 @@ struct PoolS {
   int maxC;      // widest frame over the tiles of a plane, in columns
   int TW, tilesPerPlane, totalTiles;
   int accumulate;
-  int walk;  // 0: tiles dealt round-robin to workgroups; 1: one contiguous run each; 2: round-robin inside each XCD's eighth
+  int walk;  // 0: tiles dealt round-robin to workgroups; 1: one contiguous run each; 2: round-robin inside each XCD's eighth;
+             // 3: planes dealt round-robin to XCDs, a plane's tiles round-robin to that XCD's workgroups
   int KH, nPasses;
   unsigned rankHpk, rankWpk;  // 4 bits per window offset: (pool - 1 - offset) / stride
   FastDiv byTiles, bySx, byOutH, byH4, byBorder;  // byBorder: border rows per frame column (Hp - H)
-  int outStepQ, outStepR;    // 256 = outStepQ * outH + outStepR
-  int cellStepQ, cellStepR;  // 256 = cellStepQ * H4 + cellStepR
+  int outStepQ, outStepR;    // threads per workgroup = outStepQ * outH + outStepR
+  int cellStepQ, cellStepR;  // threads per workgroup = cellStepQ * H4 + cellStepR
 };
 
 // Uniform description of one tile: all rows of the image columns [w0, w0 + nW) of one plane.
@@ -73,17 +75,17 @@ __device__ __forceinline__ Tile tile_geometry(const PoolS& p, int tile, int pool
 }
 
 // Issues the global loads of tile g: this thread's cells of x and its outputs' dzdy.
-template <int OPT, int XPT>
+template <int OPT, int XPT, int T>
 __device__ __forceinline__ void prefetch_tile(v4f (&xr)[XPT], float (&dr)[OPT], const Tile& g, int tid) {
   // Lanes past the end re-read the last element instead of being masked off (their copies are never used):
   // a clamped index costs one instruction, a masked region four.
   if (g.nCells > 0) {
 #pragma unroll
-    for (int u = 0; u < XPT; ++u) xr[u] = ((const v4f*)g.xsrc)[min(tid + 256 * u, g.nCells - 1)];
+    for (int u = 0; u < XPT; ++u) xr[u] = ((const v4f*)g.xsrc)[min(tid + T * u, g.nCells - 1)];
   }
   if (g.nOut > 0) {
 #pragma unroll
-    for (int k = 0; k < OPT; ++k) dr[k] = g.dsrc[min(tid + 256 * k, g.nOut - 1)];
+    for (int k = 0; k < OPT; ++k) dr[k] = g.dsrc[min(tid + T * k, g.nOut - 1)];
   }
 }
 
@@ -99,8 +101,9 @@ __device__ __forceinline__ float hw_max(float a, float b) {
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // OPT outputs and XPT 16-byte cells of x per thread and tile; NP > 0: the number of passes, known at compile time.
-template <int PH, int PW, int NP, int OPT, int XPT>
-__global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restrict__ dx,
+// T threads per workgroup.
+template <int PH, int PW, int NP, int OPT, int XPT, int T>
+__global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict__ dx,
                                                                 const float* __restrict__ x,
                                                                 const float* __restrict__ dy, PoolS p) {
   extern __shared__ float smem[];
@@ -118,7 +121,7 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
   // 112x112x64x32 3x3/2 case, cold caches: 44 us, against 46.5 us when each XCD walks its own eighth of the
   // tiles that way and 50 us when every workgroup owns one contiguous run of tiles.
   const int G = (int)gridDim.x;
-  int t0, t1, step;
+  int t0, t1, step, zFirst = 0, zStep = 1;
   if (p.walk == 0) {
     t0 = blockIdx.x;
     t1 = p.totalTiles;
@@ -128,20 +131,31 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
     t0 = (int)(((long long)lb * p.totalTiles) / G);
     t1 = (int)(((long long)(lb + 1) * p.totalTiles) / G);
     step = 1;
-  } else {
+  } else if (p.walk == 2) {
     const int nx = min(kNumXcd, G);  // groups of workgroups; with 8 or more workgroups, one group per XCD
     const int xcd = blockIdx.x % nx, j = blockIdx.x / nx;
     step = G / nx + (xcd < G % nx ? 1 : 0);
     t0 = (int)(((long long)xcd * p.totalTiles) / nx) + j;
     t1 = (int)(((long long)(xcd + 1) * p.totalTiles) / nx);
+  } else {
+    // planes dealt round-robin to the XCDs (hardware deals workgroup b to XCD b mod 8): the tiles of one plane, which
+    // share their halo columns, meet in one L2, and the chip as a whole still covers one contiguous stretch.
+    // Here t counts the tiles of this XCD's planes zFirst, zFirst + zStep, ...
+    zStep = min(kNumXcd, G);
+    zFirst = blockIdx.x % zStep;
+    const int j = blockIdx.x / zStep;
+    const int planes = p.byTiles.div(p.totalTiles);
+    step = G / zStep + (zFirst < G % zStep ? 1 : 0);
+    t0 = j;
+    t1 = zFirst < planes ? ((planes - zFirst + zStep - 1) / zStep) * p.tilesPerPlane : 0;
   }
   if (t0 >= t1) return;
 
   // ---- once: accumulators at +0; the frame rows above and below the image at -inf (no tile writes them)
-  for (int i = tid; i < p.TW * p.H4; i += 256) ((float4*)acc)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = tid; i < p.TW * p.H4; i += T) ((float4*)acc)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
   {
     const int nb = p.Hp - p.H;
-    for (int i = tid; i < p.maxC * nb; i += 256) {
+    for (int i = tid; i < p.maxC * nb; i += T) {
       int c, k;
       p.byBorder.divmod(i, &c, &k);
       frame[c * p.Hp + (k < p.top ? k : k + p.H)] = -INFINITY;
@@ -149,7 +163,7 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
   }
 
   // ---- per-thread constants that no tile changes
-  // outputs o = tid + 256 k of a tile: tile-relative output column oCol, output row oRow
+  // outputs o = tid + T k of a tile: tile-relative output column oCol, output row oRow
   int oRow[OPT], oCol[OPT], orgOff[OPT], locBase[OPT];
   {
     int owr, oh;
@@ -168,7 +182,7 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
       }
     }
   }
-  // cells i = tid + 256 u of the tile's x: column i / H4 after the first present one, rows 4 (i % H4) ...
+  // cells i = tid + T u of the tile's x: column i / H4 after the first present one, rows 4 (i % H4) ...
   int cellDst[XPT];  // frame position when the first present column is frame column 0
   {
     int c, s;
@@ -193,9 +207,10 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
   {
     int z, tile;
     p.byTiles.divmod(t0, &z, &tile);
+    z = zFirst + zStep * z;
     cur = tile_geometry(p, tile, poolW, x + z * planeIn, dy + z * planeOut, dx + z * planeIn);
   }
-  prefetch_tile<OPT, XPT>(xr, dr, cur, tid);
+  prefetch_tile<OPT, XPT, T>(xr, dr, cur, tid);
 
   // The accumulators of a finished tile are written to memory at the start of the next iteration, so their
   // stores have a whole tile's worth of work to complete before this wave next waits on its memory counter.
@@ -213,25 +228,25 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
       const int colShift = (cur.ca - cur.cLo) * p.Hp;
 #pragma unroll
       for (int u = 0; u < XPT; ++u)
-        *(v4f*)(frame + (tid + 256 * u < cur.nCells ? cellDst[u] + colShift : trashCell)) = xr[u];
+        *(v4f*)(frame + (tid + T * u < cur.nCells ? cellDst[u] + colShift : trashCell)) = xr[u];
       // frame columns left / right of the image (first and last tiles of a plane only)
       if (cur.cLo < 0)
-        for (int r = tid; r < colShift; r += 256) frame[r] = -INFINITY;
+        for (int r = tid; r < colShift; r += T) frame[r] = -INFINITY;
       const int c0 = p.W - cur.cLo;
       if (cur.nC > c0)
-        for (int r = tid; r < (cur.nC - c0) * p.Hp; r += 256) frame[c0 * p.Hp + r] = -INFINITY;
+        for (int r = tid; r < (cur.nC - c0) * p.Hp; r += T) frame[c0 * p.Hp + r] = -INFINITY;
     }
     float dv[OPT];
 #pragma unroll
     for (int k = 0; k < OPT; ++k) dv[k] = dr[k];
     // ---- previous tile: stream its accumulators out, leaving +0 (or this tile's derInput when accumulating)
-    for (int i = tid; i < prevIn4; i += 256) {
+    for (int i = tid; i < prevIn4; i += T) {
       const float4 a = ((const float4*)acc)[i];
       ((float4*)acc)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
       stream_store4((float4*)prevOut + i, a);
     }
     if (p.accumulate)
-      for (int i = tid; i < nIn4; i += 256) ((float4*)acc)[i] = ((const float4*)cur.out)[i];
+      for (int i = tid; i < nIn4; i += T) ((float4*)acc)[i] = ((const float4*)cur.out)[i];
     lds_barrier();
 
     // ---- next tile's loads go out now and land while this tile is computed
@@ -239,8 +254,9 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
     if (t + step < t1) {
       int z, tile;
       p.byTiles.divmod(t + step, &z, &tile);
+      z = zFirst + zStep * z;
       nxt = tile_geometry(p, tile, poolW, x + z * planeIn, dy + z * planeOut, dx + z * planeIn);
-      prefetch_tile<OPT, XPT>(xr, dr, nxt, tid);
+      prefetch_tile<OPT, XPT, T>(xr, dr, nxt, tid);
     }
 
     // ---- winner of each owned output: first maximum of its window, scanning column by column
@@ -249,7 +265,7 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
     const float* org[OPT];
 #pragma unroll
     for (int k = 0; k < OPT; ++k) {
-      org[k] = frame + (tid + 256 * k < cur.nOut ? orgOff[k] : 0);  // idle lanes read a valid window
+      org[k] = frame + (tid + T * k < cur.nOut ? orgOff[k] : 0);  // idle lanes read a valid window
       best[k] = -INFINITY;
       code[k] = -1;
     }
@@ -288,7 +304,7 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
     for (int k = 0; k < OPT; ++k) {
       const int bj = code[k] >> 3, bi = code[k] & 7;
       const int w = oCol[k] * p.sx + bj + shift;  // tile-relative column of the winner
-      const bool ok = code[k] >= 0 && tid + 256 * k < cur.nOut && (unsigned)w < (unsigned)cur.nW;
+      const bool ok = code[k] >= 0 && tid + T * k < cur.nOut && (unsigned)w < (unsigned)cur.nW;
       const int ra = (int)((p.rankHpk >> (4 * bi)) & 15u), rb = (int)((p.rankWpk >> (4 * bj)) & 15u);
       rank[k] = (min(cur.owLo + oCol[k], rb) * p.KH + min(oRow[k], ra)) | (ok ? 0 : -1);  // -1: routes nothing
       loc[k] = locBase[k] + (shift + bj) * p.H + bi;
@@ -324,7 +340,25 @@ __global__ __launch_bounds__(256) void pool_max_backward_stream(float* __restric
     cur = nxt;
   }
   // ---- last tile
-  for (int i = tid; i < prevIn4; i += 256) stream_store4((float4*)prevOut + i, ((const float4*)acc)[i]);
+  for (int i = tid; i < prevIn4; i += T) stream_store4((float4*)prevOut + i, ((const float4*)acc)[i]);
+}
+
+// One instantiation: opts it into more than 64 KB of LDS when the tile needs that (once per device), then launches.
+template <int PH, int PW, int NP, int OPT, int XPT, int T>
+bool launch_stream(hipStream_t s, dim3 grid, size_t lds, float* dx, const float* x, const float* dy, const PoolS& p) {
+  static std::atomic<size_t> raised[kMaxDevices];
+  const int dev = current_device();
+  if (lds > 64 * 1024 && (dev < 0 || dev >= kMaxDevices || lds > raised[dev].load(std::memory_order_acquire))) {
+    if (hipFuncSetAttribute((const void*)pool_max_backward_stream<PH, PW, NP, OPT, XPT, T>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    if (dev >= 0 && dev < kMaxDevices) raised[dev].store(lds, std::memory_order_release);
+  }
+  KernelTimer timer("pool_backward_stream", s);
+  hipLaunchKernelGGL((pool_max_backward_stream<PH, PW, NP, OPT, XPT, T>), grid, dim3((unsigned)T), lds, s, dx, x, dy, p);
+  return true;
 }
 
 }  // namespace
@@ -356,9 +390,11 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   for (int i = 0; i < g->poolW; ++i) p.rankWpk |= (unsigned)((g->poolW - 1 - i) / g->strideX) << (4 * i);
 
   // widest tile whose LDS fits the budget and whose outputs and cells fit 4 per thread
-  // (the kernel is not opted into more than 64 KB of LDS: the budget leaves room for the slots added below)
-  const size_t slotBytes = (4 + 256) * sizeof(float);
-  const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024), 64 * 1024 - (int)slotBytes);
+  int threads = tunable("pool_threads", 256);
+  if (threads != 512 && threads != 1024) threads = 256;
+  if (threads != 256 && !(p.poolH == 3 && p.poolW == 3 && p.nPasses == 4)) threads = 256;  // (instantiated for 3x3 / 2 only)
+  const size_t slotBytes = (4 + (size_t)threads) * sizeof(float);
+  const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024), 150 * 1024) - slotBytes;
   int TW = 0, maxOut = 0, maxCells = 0, maxC = 0;
   size_t lds = 0;
   for (int nT = 1; nT <= p.W; ++nT) {
@@ -379,7 +415,7 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
     }
     worstC = std::max(worstC, p.poolW);  // idle lanes read the window at the frame origin
     const size_t need = ((size_t)cand * p.H + (size_t)worstC * p.Hp) * sizeof(float);
-    if (need <= budget && worstOut <= 4 * 256 && worstCells <= 4 * 256) {
+    if (need <= budget && worstOut <= 4 * threads && worstCells <= 4 * threads) {
       TW = cand;
       maxOut = worstOut;
       maxCells = worstCells;
@@ -400,21 +436,29 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   p.byOutH = FastDiv(p.outH);
   p.byH4 = FastDiv(p.H4);
   p.byBorder = FastDiv(std::max(p.Hp - p.H, 1));
-  p.outStepQ = 256 / p.outH;
-  p.outStepR = 256 % p.outH;
-  p.cellStepQ = 256 / p.H4;
-  p.cellStepR = 256 % p.H4;
-  const int opt = std::max((maxOut + 255) / 256, 1), xpt = std::max((maxCells + 255) / 256, 1);
+  p.outStepQ = threads / p.outH;
+  p.outStepR = threads % p.outH;
+  p.cellStepQ = threads / p.H4;
+  p.cellStepR = threads % p.H4;
+  const int opt = std::max((maxOut + threads - 1) / threads, 1), xpt = std::max((maxCells + threads - 1) / threads, 1);
   lds += slotBytes;  // the idle-lane cell and slots
 
   int cus = device_compute_units();
   if (cus <= 0) cus = 256;
   const int perCu = std::min(std::max(tunable("pool_blocks_per_cu", 3), 1), (int)std::max<size_t>((160 * 1024) / std::max<size_t>(lds, 1), 1));
-  const int blocks = (int)std::min<long long>(p.totalTiles, (long long)cus * perCu);
-  const dim3 grid((unsigned)blocks), block(256);
-  KernelTimer timer("pool_backward_stream", s);
-#define MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, XPTF) \
-  hipLaunchKernelGGL((pool_max_backward_stream<PHF, PWF, NPF, OPTF, XPTF>), grid, block, lds, s, derInput, x, derOutput, p)
+  const int blocks = tunable("pool_blocks_per_cu", 3) <= 0  // (experiments: one tile per workgroup)
+                         ? p.totalTiles
+                         : (int)std::min<long long>(p.totalTiles, (long long)cus * perCu);
+  const dim3 grid((unsigned)blocks), block((unsigned)threads);
+  bool launched = true;
+#define MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, TF) \
+  launched = launch_stream<PHF, PWF, NPF, OPTF, XPTF, TF>(s, grid, lds, derInput, x, derOutput, p)
+#define MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, XPTF)                                         \
+  do {                                                                                     \
+    if (threads == 256 || NPF != 4) MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, 256);      \
+    else if (threads == 512) MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, (NPF == 4 ? 512 : 256));  \
+    else MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, (NPF == 4 ? 1024 : 256));             \
+  } while (0)
 #define MCN_POOL_STREAM_XPT(PHF, PWF, NPF, OPTF)               \
   do {                                                         \
     if (xpt == 1) MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, 1);      \
@@ -438,7 +482,8 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
 #undef MCN_POOL_STREAM_OPT
 #undef MCN_POOL_STREAM_XPT
 #undef MCN_POOL_STREAM
-  return true;
+#undef MCN_POOL_STREAM_T
+  return launched;
 }
 
 }  // namespace mcn

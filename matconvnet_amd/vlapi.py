@@ -86,6 +86,7 @@ def lib():
         L.vlh_resnet50_set_packed.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_pack.argtypes = [C.c_void_p]
         L.vlh_bottleneck_set_packed.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_bottleneck_set_epilogue_sums.argtypes = [C.c_void_p, C.c_int]
         L.vlh_bottleneck_pack.argtypes = [C.c_void_p]
         L.vlh_resnet50_init.argtypes = [C.c_void_p, C.c_ulonglong]
         L.vlh_resnet50_forward.argtypes = [C.c_void_p]
@@ -368,7 +369,7 @@ class Bottleneck(_NamedBuffers):
     """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
 
     def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False, overlap=False, Cout=0, stride=1,
-                 adapter=False, packed=False, deferred=False):
+                 adapter=False, packed=False, deferred=False, epilogue_sums=False):
         """packed: the convolutions read filter banks packed ahead; `set` of a filter and every step of `run` refresh
         them with one launch (`pack`).  deferred: one launch at the end of backward sums the reduction splits of all
         the unit's filter gradients."""
@@ -386,6 +387,9 @@ class Bottleneck(_NamedBuffers):
             self.packed = True
         if deferred:
             self._check(self.L.vlh_bottleneck_set_deferred(self.h, 1))
+        if epilogue_sums:
+            # (fused mode: the forward convolutions sum their output per channel, batch normalisation takes the sums)
+            self._check(self.L.vlh_bottleneck_set_epilogue_sums(self.h, 1))
 
     def set(self, name, array):
         super().set(name, array)

@@ -575,3 +575,64 @@ def test_filter_gradient_wide_row_tile(capi, ob, xs, fs, stride, pad):
         finally:
             capi.set_tunable("conv_wgrad_no_wide_rows", 0)
         assert rel_max(capi.to_host(df), want) < 2e-4
+
+
+SUMMING = [  # x shape, filter shape, pad: the three convolutions of the bottleneck block, smaller batches
+    ((56, 56, 256, 8), (1, 1, 256, 64), 0),
+    ((56, 56, 64, 8), (3, 3, 64, 64), 1),
+    ((56, 56, 64, 12), (1, 1, 64, 256), 0),
+    ((28, 28, 256, 16), (1, 1, 256, 128), 0),     # four channel blocks side by side, one workgroup per compute unit
+]
+
+
+@pytest.mark.parametrize("xs,fs,pad", SUMMING)
+def test_conv_forward_with_channel_sums(capi, ob, xs, fs, pad):
+    """The convolution that also sums its output per channel (the first pass of a batch normalisation that
+    follows): y has the bits of the plain convolution, the partial sums add up to the sums of that y taken in
+    double, and batch normalisation from those sums is within 1e-5 of the reference's formula in double
+    (bits/nnbnorm.cu:46-71) applied to the same y."""
+    import torch
+    r = np.random.default_rng(3)
+    x = F(r.standard_normal(xs) + 0.3)
+    f = F(r.standard_normal(fs) * np.sqrt(2.0 / (fs[0] * fs[1] * fs[2])))
+    K = fs[3]
+    g = capi.conv_geom(xs, fs, 1, pad, 1)
+    groups = capi.conv_forward_sums_groups(g)
+    assert groups > 0
+    xd, fd = capi.to_device(x), capi.to_device(f)
+    want = capi.conv_forward(xd, fd, None, g)
+    for turn in range(2):  # (the second call finds the buffers of the first: nothing is carried over)
+        y, sums = capi.conv_forward_sums(xd, fd, g)
+        assert torch.equal(y, want)
+        yd = y.double()
+        s1, s2 = yd.sum(dim=(0, 2, 3)), (yd * yd).sum(dim=(0, 2, 3))
+        tot = sums.sum(dim=1)
+        assert float((tot[:, 0] - s1).abs().max() / s1.abs().max()) < 1e-6
+        assert float((tot[:, 1] - s2).abs().max() / s2.abs().max()) < 1e-6
+    gain = F(r.uniform(0.5, 1.5, K)).ravel()
+    bias = F(r.standard_normal(K) * 0.1).ravel()
+    res = F(r.standard_normal(capi.conv_out_shape(g)))
+    gd, bd, rd = capi.to_device(gain), capi.to_device(bias), capi.to_device(res)
+    y64 = F(capi.to_host(y), np.float64)
+    ref, mom = ob.bnorm_forward(y64, gain.astype(np.float64), bias.astype(np.float64), 1e-5)
+    for residual, relu in ((None, True), (rd, True), (rd, False), (None, False)):
+        out, m = capi.bnorm_forward_sums(y, gd, bd, sums, residual=residual, relu=relu, eps=1e-5)
+        w = ref + (res.astype(np.float64) if residual is not None else 0.0)
+        if relu:
+            w = np.maximum(w, 0.0)
+        assert rel_max(capi.to_host(out), w) <= 1e-5
+        assert rel_max(capi.to_host(m), mom) <= 1e-5
+    # against the two-launch form on the same tensor: same result to rounding
+    out2, m2 = capi.bnorm_forward_fused(y, gd, bd, residual=rd, relu=True, eps=1e-5)
+    out1, m1 = capi.bnorm_forward_sums(y, gd, bd, sums, residual=rd, relu=True, eps=1e-5)
+    assert rel_max(capi.to_host(out1), capi.to_host(out2)) <= 2e-6 and rel_max(capi.to_host(m1), capi.to_host(m2)) <= 1e-6
+
+
+def test_conv_forward_with_channel_sums_refuses_what_it_cannot_do(capi):
+    """Geometries the summing form does not cover report 0 groups, and the call says so instead of computing."""
+    g = capi.conv_geom((9, 9, 5, 2), (3, 3, 5, 7), 1, 1, 1)
+    assert capi.conv_forward_sums_groups(g) == 0
+    x, f = capi.empty((9, 9, 5, 2), fill=0.0), capi.empty((3, 3, 5, 7), fill=0.0)
+    with pytest.raises(capi.McnError) as e:
+        capi.conv_forward_sums(x, f, g)
+    assert "no such form" in str(e.value)
