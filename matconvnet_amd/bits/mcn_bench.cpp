@@ -3,7 +3,7 @@
 // synthetic inputs, times them with HIP events and prints TFLOP/s, GB/s and images/s beside the
 // fraction of the MI355X rooflines (fp32 matrix 157.3 TFLOP/s, HBM 8 TB/s).
 //
-//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|yardstick|resnet50] [--batch N] [--config C]
+//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...
 //
 // The bandwidth-bound operators (bnorm, pooling, copy) are timed over R independent sets of tensors used in
 // turn (default 4), so that no launch finds its inputs in the 256 MB memory-side cache because the previous
@@ -359,8 +359,17 @@ int main(int argc, char** argv) {
     else if (!std::strcmp(argv[i], "--batch") && i + 1 < argc) batch = std::max(1, std::atoi(argv[++i]));
     else if (!std::strcmp(argv[i], "--rotate") && i + 1 < argc) gRotate = std::max(1, std::atoi(argv[++i]));
     else if (!std::strcmp(argv[i], "--config") && i + 1 < argc) fixed = std::atoi(argv[++i]);
+    else if (!std::strcmp(argv[i], "--set") && i + 1 < argc && std::strchr(argv[i + 1], '=')) {
+      // a tunable of the back-end (mcn_set_tunable), as name=value
+      std::string kv = argv[++i];
+      const size_t eq = kv.find('=');
+      if (mcn_set_tunable(kv.substr(0, eq).c_str(), std::atoi(kv.c_str() + eq + 1)) != 0) {
+        std::fprintf(stderr, "mcn_bench: %s\n", mcn_last_error_message());
+        return 1;
+      }
+    }
     else {
-      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|yardstick|resnet50] [--batch N] [--config C]\n");
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...\n");
       return 1;
     }
   }
