@@ -212,6 +212,14 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
 // partial sums per channel it would write when asked to sum its output (PixP::stats); 0: it would not take `p` that way
 int conv_ws_stat_groups(const PixP& p);
 
+// Streamed-bank variant (conv_sb.hip) for banks too large for LDS, same packed order.  conv_sb_splits: the reduction
+// splits it would use for a product of these extents (0: it does not take them; depends on nothing else, so that the
+// workspace can be sized ahead); conv_sb_plan: the same, with the layout conditions checked.  conv_sb_launch: `p` laid
+// out as for the tiled kernel (with splits > 1: the partial tensors' dense layout, alpha = 1, beta = 0, no bias).
+int conv_sb_splits(int Cout, long long M, int R);
+bool conv_sb_plan(const PixP& p, int* splits);
+int conv_sb_launch(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, PixP p, int splits);
+
 // Products with at most four output channels (conv_few.hip): wt is the packed bank (tapMajor: its row order, see
 // conv_pack_weights).  Sets *handled when it took the work.
 int conv_few_launch(hipStream_t s, const char* who, float* out, const float* in, const float* wt, const float* bias,

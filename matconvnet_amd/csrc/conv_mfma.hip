@@ -915,7 +915,10 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
                        rPad, p.coutPad, backward, ut ? 1 : 0);
     return check_launch(who);
   }
-  const size_t need = plan.splits > 1 ? align256(needW) + (size_t)plan.splits * nOut * sizeof(float) : (slot || asStored ? 0 : needW);
+  int sbSplits = 1;
+  const bool sb = ut && p.Cout > 4 && !p.stats && conv_sb_plan(p, &sbSplits);
+  const int needSplits = std::max(plan.splits, sb ? sbSplits : 1);
+  const size_t need = needSplits > 1 ? align256(needW) + (size_t)needSplits * nOut * sizeof(float) : (slot || asStored ? 0 : needW);
   if (need && (!ws || wsBytes < need)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small (%zu < %zu bytes)", who, wsBytes, need);
   if (need && !aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
   float* wt = (float*)ws;
@@ -957,13 +960,18 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
     if (rc || handled) return rc;
   }
   if (p.stats) return fail(MCN_UNSUPPORTED, "%s: this product cannot sum its output per channel", who);
-  if (plan.splits > 1) {
+  // banks too large for LDS: stream them past pixels held in registers (conv_sb.hip)
+  if (sb && sbSplits == 1) {
+    rc = conv_sb_launch(s, out, in, wt, bias, p, 1);
+    return rc ? rc : check_launch(who);
+  }
+  if (sb || plan.splits > 1) {
     // every workgroup a slice of the reduction into its own partial tensor, then one pass to add them up
     float* partials = (float*)((char*)ws + align256(needW));
     PixP q = p;
     const int nSteps = rPad / 16;
     q.stepsPerSplit = (nSteps + plan.splits - 1) / plan.splits;
-    q.rSplits = (nSteps + q.stepsPerSplit - 1) / q.stepsPerSplit;
+    q.rSplits = sb ? sbSplits : (nSteps + q.stepsPerSplit - 1) / q.stepsPerSplit;
     q.partStride = (long long)nOut;
     q.alpha = 1.f;
     q.beta = 0.f;
@@ -975,8 +983,9 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
       const long long ob = (long long)nOut * 4;
       q.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
     }
-    launch_shape(s, plan.shape, partials, in, wt, nullptr, q, ut);
-    if ((rc = check_launch(who))) return rc;
+    if (sb) rc = conv_sb_launch(s, partials, in, wt, nullptr, q, sbSplits);
+    else launch_shape(s, plan.shape, partials, in, wt, nullptr, q, ut);
+    if (rc || (rc = check_launch(who))) return rc;
     p.rSplits = q.rSplits;
     p.partStride = q.partStride;
     KernelTimer timer("conv_pix_reduce", s);
@@ -1030,7 +1039,8 @@ size_t conv_mfma_workspace_bytes(const ConvP& original, int product) {
     const int BA = pick_channels_tile(Cout);
     const size_t needW = ((size_t)(R + 15) / 16 * 16) * (size_t)((Cout + BA - 1) / BA * BA) * sizeof(float);
     const PixPlan plan = plan_pix(Cout, M, R);
-    return plan.splits > 1 ? align256(needW) + (size_t)plan.splits * (size_t)M * Cout * sizeof(float) : needW;
+    const int splits = std::max(plan.splits, conv_sb_splits(Cout, M, R));  // (whichever kernel takes the product)
+    return splits > 1 ? align256(needW) + (size_t)splits * (size_t)M * Cout * sizeof(float) : needW;
   };
   switch (product) {
     case MCN_CONV_FORWARD: {
