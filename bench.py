@@ -57,8 +57,22 @@ def _sync():
     torch.cuda.synchronize()
 
 
+SPIN_UP_S = 0.03  # after a pause the device needs some 20 ms of work to come back to its full clock
+
+
+def spin_up(launch):
+    """Untimed calls of `launch` for SPIN_UP_S of device time: the per-operator rows are steady-state figures."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < SPIN_UP_S:
+        for _ in range(4):
+            launch()
+        _sync()
+
+
 def kernel_time(capi, kernel, launch, reps):
-    """Mean duration (s) of `kernel` over `reps` calls of `launch`, from HIP events bracketing each launch."""
+    """Mean duration (s) of `kernel` over `reps` calls of `launch`, from HIP events bracketing each launch (after
+    spin_up: see there)."""
+    spin_up(launch)
     capi.profile_begin(kernel)
     for _ in range(reps):
         launch()
@@ -66,11 +80,13 @@ def kernel_time(capi, kernel, launch, reps):
     return (ms / n) * 1e-3 if n else float("nan"), n
 
 
-def _time_block(blk, w, steps, warmup, layer_by_layer=False):
+def _load_block(blk, w):
     for k in ("x", "f1", "f2", "f3", "g1", "b1", "g2", "b2", "g3", "b3"):
         blk.set(k, w[k])
     blk.set("dzdy", w["dy"])
 
+
+def _time_block(blk, steps, warmup, layer_by_layer=False):
     def run(n):
         if layer_by_layer:
             for _ in range(n):
@@ -90,13 +106,12 @@ def _time_block(blk, w, steps, warmup, layer_by_layer=False):
 def bench_block(vlapi, capi, workloads, steps, warmup):
     w = workloads.bottleneck_case()
     N = w["x"].shape[3]
-    # The reference-interface-only schedule first: every layer a call of its own on vl::nn::Convolution / BatchNorm /
-    # ReLU / Sum, nothing folded, nothing packed ahead (what code written against the reference's classes gets unchanged).
-    blk = vlapi.Bottleneck(N=N, eps=w["eps"])
-    dt_plain = _time_block(blk, w, steps, warmup, layer_by_layer=True)
-    blk.close()
-    plain = dict(ms_per_step=dt_plain / steps * 1e3, images_per_s=N * steps / dt_plain,
-                 schedule="layer by layer through vl::nn::Convolution / BatchNorm / ReLU / Sum only")
+    # Both schedules are built and loaded first, so that no upload sits between the two measurements: after a pause the
+    # device takes some 20 ms of work to come back to its full clock (steps of 820 us falling to 755 us), which is the
+    # length of a measurement here.
+    # The reference-interface-only schedule: every layer a call of its own on vl::nn::Convolution / BatchNorm / ReLU /
+    # Sum, nothing folded, nothing packed ahead (what code written against the reference's classes gets unchanged).
+    plain_blk = vlapi.Bottleneck(N=N, eps=w["eps"])
     # The timed schedule: the same operator classes for the convolutions, and the library's folded batch-norm entry
     # points, which the reference does not have:
     # fused: ReLU / shortcut sum folded into batch normalisation; packed: the filter banks are re-laid for the matrix
@@ -104,7 +119,13 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
     # deferred: the sums over reduction splits that finish the three filter gradients run in one launch at the end;
     # epilogue_sums: the forward convolutions sum their output per channel, batch normalisation takes those sums
     blk = vlapi.Bottleneck(N=N, eps=w["eps"], fused=True, packed=True, deferred=True, epilogue_sums=True)
-    dt = _time_block(blk, w, steps, warmup)
+    _load_block(plain_blk, w)
+    _load_block(blk, w)
+    dt_plain = _time_block(plain_blk, steps, warmup, layer_by_layer=True)
+    dt = _time_block(blk, steps, warmup)
+    plain_blk.close()
+    plain = dict(ms_per_step=dt_plain / steps * 1e3, images_per_s=N * steps / dt_plain,
+                 schedule="layer by layer through vl::nn::Convolution / BatchNorm / ReLU / Sum only")
     # which kernel family dominates the step, and its live duration
     P = 56 * 56
     # per launch family per step.  The six forward + backward-data launches go to the weights-stationary kernel
@@ -170,7 +191,12 @@ def bench_conv_bwd(capi, workloads, reps):
     for fn in (data, filt, bias):
         fn()
     _sync()
-    t_data, _ = kernel_time(capi, "conv_pix_mfma", data, reps)
+    # backward-data goes to the streamed-bank kernel (conv_sb_mfma) when it takes the shape, else to the tiled one
+    data_kernel = "conv_sb_mfma"
+    t_data, n_data = kernel_time(capi, data_kernel, data, reps)
+    if n_data == 0:
+        data_kernel = "conv_pix_mfma"
+        t_data, _ = kernel_time(capi, data_kernel, data, reps)
     t_filt, _ = kernel_time(capi, "conv_wgrad_mfma", filt, reps)
     t_red, _ = kernel_time(capi, "conv_wgrad_reduce", filt, reps)
     # whole backward call (all launches incl. weight packing, partial-sum reduction and bias), wall clock
@@ -181,7 +207,7 @@ def bench_conv_bwd(capi, workloads, reps):
     _sync()
     t_all = (time.perf_counter() - t0) / reps
     out = []
-    for name, kern, t in (("conv backward-data", "conv_pix_mfma", t_data), ("conv backward-filter", "conv_wgrad_mfma", t_filt)):
+    for name, kern, t in (("conv backward-data", data_kernel, t_data), ("conv backward-filter", "conv_wgrad_mfma", t_filt)):
         out.append(dict(op=name, kernel=kern, workload="configs[4] 3x3x256x256 on 56x56x256x64", bound="mfma",
                         achieved=flops / t / 1e12, peak=PEAK_MFMA_FP32 / 1e12, unit="TFLOP/s", frac=flops / t / PEAK_MFMA_FP32,
                         avg_launch_us=t * 1e6, traffic=TRAFFIC.get("cfg5/" + kern)))
@@ -291,6 +317,7 @@ def _event_time(fn, reps, warm=2):
     import torch
     for _ in range(warm):
         fn()
+    spin_up(fn)
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     _sync()
     a.record()
@@ -318,7 +345,7 @@ def bench_hbm_ceiling(capi, reps):
     shapes = {"read": [(0, 4, 4, 0, 0), (0, 4, 8, 4, 0), (0, 16, 2, 4, 0), (0, 4, 4, 16, 0)],
               "write": [(1, 4, 2, 0, 1), (1, 16, 1, 0, 0), (1, 16, 1, 0, 1), (1, 4, 4, 0, 0)],
               "copy": [(2, 4, 4, 0, 1), (2, 4, 4, 0, 0), (2, 16, 1, 0, 0), (2, 16, 1, 4, 0)]}
-    for name, cands in shapes.items():
+    def sweep(cands, nb):
         best = None
         for mode, width, in_flight, per_cu, flags in cands:
             turn = [0]
@@ -326,16 +353,22 @@ def bench_hbm_ceiling(capi, reps):
             def call():
                 i = turn[0] % COLD_SETS
                 turn[0] += 1
-                capi.check(L.mcn_hbm_yardstick(st, capi.ptr(dst[i]), capi.ptr(src[i]), nbytes, mode, width, in_flight,
+                capi.check(L.mcn_hbm_yardstick(st, capi.ptr(dst[i]), capi.ptr(src[i]), nb, mode, width, in_flight,
                                                per_cu * cus, flags))
             for _ in range(COLD_SETS):
                 call()
             t, _ = kernel_time(capi, "yardstick_kernel", call, reps)
-            gbs = (2 if mode == 2 else 1) * nbytes / t / 1e9
+            gbs = (2 if mode == 2 else 1) * nb / t / 1e9
             if best is None or gbs > best["gbs"]:
                 best = dict(gbs=gbs, frac_of_peak=gbs * 1e9 / PEAK_HBM, us=t * 1e6, width_bytes=width, in_flight=in_flight,
-                            workgroups_per_cu=per_cu, non_temporal=bool(flags & 1))
-        out[name] = best
+                            workgroups_per_cu=per_cu, non_temporal=bool(flags & 1), bytes_per_stream=nb)
+        return best
+
+    for name, cands in shapes.items():
+        out[name] = sweep(cands, nbytes)
+    # the same copy kernels moving what one max-pooling backward launch moves (231 MB in all: launch ramp and tail
+    # weigh more on a 40 us kernel than on a 90 us one)
+    out["copy_231MB"] = sweep(shapes["copy"], 110 << 20)
     return out
 
 
@@ -492,6 +525,61 @@ def bench_resnet50(vlapi, batch, steps, warmup):
         net.close()
 
 
+def bench_resnet50_sections(capi, batch, reps):
+    """The convolutions of ResNet-50 (examples/imagenet/cnn_imagenet_init_resnet.m:52-134) section by section, each layer
+    shape timed on its own through the C ABI (whole call, events on the launch stream, one set of buffers reused) and
+    weighted by how often the network has it: TFLOP/s of the forward, backward-data and backward-filter products per
+    section.  Where the whole-network step loses against these figures is batch normalisation, pooling, the update and
+    cold caches between layers."""
+    import ctypes as C
+    import torch
+    L = capi.lib()
+    st = capi.stream()
+    layers = [("conv1", "stem 7x7 3->64 /2", 224, 3, 7, 64, 2, 3, 1)]
+    H, Cc = 56, 64
+    for s_, units in enumerate((3, 4, 6, 3)):
+        M, Co = 64 << s_, 256 << s_
+        stride = 2 if s_ >= 1 else 1
+        sec = "conv%d_x" % (s_ + 2)
+        layers.append((sec, "1x1 %d->%d" % (Cc, M), H, Cc, 1, M, 1, 0, 1))
+        layers.append((sec, "3x3 %d->%d /%d" % (M, M, stride), H, M, 3, M, stride, 1, 1))
+        layers.append((sec, "1x1 %d->%d /%d (shortcut)" % (Cc, Co, stride), H, Cc, 1, Co, stride, 0, 1))
+        H = (H - 1) // stride + 1
+        layers.append((sec, "1x1 %d->%d" % (M, Co), H, M, 1, Co, 1, 0, units))
+        layers.append((sec, "1x1 %d->%d" % (Co, M), H, Co, 1, M, 1, 0, units - 1))
+        layers.append((sec, "3x3 %d->%d" % (M, M), H, M, 3, M, 1, 1, units - 1))
+        Cc = Co
+    ws = capi.Workspace()
+    table = {}
+    for sec, _, Hh, Cin, fh, Cout, stride, pad, count in layers:
+        xs, fs = (Hh, Hh, Cin, batch), (fh, fh, Cin, Cout)
+        g = capi.conv_geom(xs, fs, stride, pad, 1)
+        ys = capi.conv_out_shape(g)
+        flops = 2.0 * ys[0] * ys[1] * batch * fh * fh * Cin * Cout
+        x = torch.randn(tuple(reversed(xs)), device="cuda")
+        f = torch.randn(tuple(reversed(fs)), device="cuda") * 0.05
+        dy = torch.randn(tuple(reversed(ys)), device="cuda")
+        dx, y, df = capi.empty(xs), capi.empty(ys), capi.empty(fs)
+        wp, wn = ws.get(max(L.mcn_conv_workspace_bytes(C.byref(g), k) for k in range(4)))
+        calls = (lambda: capi.check(L.mcn_conv_forward(st, C.byref(g), capi.ptr(y), 0.0, capi.ptr(x), 1.0, capi.ptr(f), None, wp, wn)),
+                 lambda: capi.check(L.mcn_conv_backward_data(st, C.byref(g), capi.ptr(dx), capi.ptr(f), capi.ptr(dy), wp, wn)),
+                 lambda: capi.check(L.mcn_conv_backward_filter(st, C.byref(g), capi.ptr(df), capi.ptr(x), capi.ptr(dy), wp, wn)))
+        row = table.setdefault(sec, dict(section=sec, gflop_per_pass=0.0, forward_us=0.0, backward_data_us=0.0, backward_filter_us=0.0))
+        row["gflop_per_pass"] += count * flops / 1e9
+        for key, fn in zip(("forward_us", "backward_data_us", "backward_filter_us"), calls):
+            if sec == "conv1" and key == "backward_data_us":
+                continue  # (nothing consumes the input gradient of the first layer: the network driver skips it)
+            row[key] += count * _event_time(fn, reps, warm=2) * 1e6
+        del x, f, dy, dx, y, df
+    out = []
+    for row in table.values():
+        for key in ("forward", "backward_data", "backward_filter"):
+            us = row[key + "_us"]
+            row[key + "_tflops"] = row["gflop_per_pass"] / us * 1e3 if us > 0 else None
+        out.append(row)
+    return out
+
+
 def cpu_baseline(workloads):
     """The CPU restatement of the reference path on this host: one forward+backward of the same block
     (same N = 32 inputs), GEMMs threaded like the reference's BLAS, everything else serial."""
@@ -610,6 +698,7 @@ def main():
     for row in bn_rows + pool_rows + forward_rows:
         if row["bound"] == "hbm":   # beside the fraction of the nominal 8 TB/s: of what a plain copy reaches here
             row["frac_of_measured_copy"] = row["achieved"] / ceiling["copy"]["gbs"]
+    pool_rows[0]["frac_of_measured_copy_of_same_size"] = pool_rows[0]["achieved"] / ceiling["copy_231MB"]["gbs"]
     line = {
         "metric": "ResNet-50-block fwd+bwd images/s; conv-bwd TFLOP/s; bnorm/pool-bwd GB/s",
         "value": images_per_s, "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -641,6 +730,7 @@ def main():
         # (64 is the reference's own sub-batch for this network: batchSize 256 in 4 sub-batches,
         # examples/imagenet/cnn_imagenet_init_resnet.m:170-171)
         "resnet50": [bench_resnet50(vlapi, b, max(3, args.steps // 10), 2) for b in (32, 64, 128)],
+        "resnet50_sections_batch32": bench_resnet50_sections(capi, 32, max(3, args.steps // 5)),
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(workloads)

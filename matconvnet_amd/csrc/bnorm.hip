@@ -144,21 +144,36 @@ __device__ __forceinline__ void sums_of_planes(double (&acc)[4], const float* __
         }
       }
     } else {
-      for (int i = j0; i < p.WH; i += TS) {
-        const float a = x[base + i];
-        const double ad = (double)a;
-        if (MODE != 1) {
-          acc[0] += ad;
-          acc[1] = fma(ad, ad, acc[1]);
+      // four scalar loads of each tensor in flight per thread (lanes past the plane's end re-read its last element and
+      // count it as zero)
+      for (int i = j0; i < p.WH; i += 4 * TS) {
+        float a[4], d[4], m[4];
+        bool in[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          in[u] = i + u * TS < p.WH;
+          const size_t at = base + (in[u] ? i + u * TS : p.WH - 1);
+          a[u] = x[at];
+          if (MODE != 0) d[u] = dy[at];
+          if (YMASK) m[u] = ymask[at];
         }
-        if (MODE != 0) {
-          float d = gate(a, dy[base + i]);
-          if (YMASK) {
-            d = ymask[base + i] > 0.f ? d : d * 0.f;
-            masked[base + i] = d;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const double ad = in[u] ? (double)a[u] : 0.0;
+          if (MODE != 1) {
+            acc[0] += ad;
+            acc[1] = fma(ad, ad, acc[1]);
           }
-          acc[2] = fma(ad, (double)d, acc[2]);
-          acc[3] += (double)d;
+          if (MODE != 0) {
+            float dv = gate(a[u], d[u]);
+            if (YMASK) {
+              dv = m[u] > 0.f ? dv : dv * 0.f;
+              if (in[u]) masked[base + i + u * TS] = dv;
+            }
+            const double dd = in[u] ? (double)dv : 0.0;
+            acc[2] = fma(ad, dd, acc[2]);
+            acc[3] += dd;
+          }
         }
       }
     }
@@ -711,7 +726,7 @@ static int bnorm_backward_any(const char* who, mcn_stream_t stream, float* derIn
       if (vec) hipLaunchKernelGGL((bnorm_sums<1, true>), grid, block, 0, s, x, derOutput, partials, p);
       else hipLaunchKernelGGL((bnorm_sums<1, false>), grid, block, 0, s, x, derOutput, partials, p);
     } else {
-      if (vec) hipLaunchKernelGGL((bnorm_sums<2, true>), grid, block, 0, s, x, derOutput, partials, p);
+      if (vec && !tunable("bnorm_sums_scalar", 0)) hipLaunchKernelGGL((bnorm_sums<2, true>), grid, block, 0, s, x, derOutput, partials, p);
       else hipLaunchKernelGGL((bnorm_sums<2, false>), grid, block, 0, s, x, derOutput, partials, p);
     }
   }

@@ -410,6 +410,7 @@ struct WgP {
   FastDiv byQ, byOH, byT, byFH, byTiles, byTilesK, byC;
   unsigned outBytes;     // size of the partial banks, or 0 when they do not fit a 2 GiB buffer descriptor
   int xImg, dyImg;       // elements between images of x and of dzdy (wider than C*H*W, K*OH*OW for a filter group)
+  unsigned xBytes, dyBytes;  // bytes from x / dzdy to the end of what this product reads (UT: both < 2 GiB)
 };
 
 // UT ("uniform tap"): rows are ordered tap-major (R' = c + C*t) and C is a multiple of 32, so each 32-row MFMA
@@ -477,12 +478,20 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   float pa[APT], pb[BPT];
   unsigned okA = 0, okB = 0;
 
-  // UT: per 32-row block its tap shift (uniform), per thread the constant offsets of its rows
+  // UT: per 32-row block its tap shift (uniform).  The loads are buffer loads: the per-lane offset is the pixel (plus one
+  // row for the upper half of the wavefront: thread group rg = 2 wave + half), the scalar offset is the row -- no
+  // address arithmetic per load in vector registers, and a pixel outside the image or past the split's end uses an
+  // offset beyond the tensor, for which the hardware returns 0 (no branches, no dummy reads).
   constexpr int NBLK = BB / 32;
-  int blkDh[NBLK], blkDw[NBLK];
-  int xOff[BPT], yOff[APT];
+  int blkDh[NBLK], blkDw[NBLK], blkShift[NBLK];
+  int xOffS[BPT], yOffS[APT];  // byte offsets of this wavefront's rows at half 0 (uniform: scalar registers)
   unsigned kPresent = 0;
+  const int waveU = __builtin_amdgcn_readfirstlane(wave);
+  const int half = rg & 1;
+  __amdgpu_buffer_rsrc_t xr, yr;
   if (UT) {
+    xr = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, (int)p.xBytes, 0x00020000);
+    yr = __builtin_amdgcn_make_buffer_rsrc((void*)dy, 0, (int)p.dyBytes, 0x00020000);
 #pragma unroll
     for (int jb = 0; jb < NBLK; ++jb) {
       const int Rb = r0 + 32 * jb;
@@ -493,13 +502,14 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
       blkDh[jb] = Rb < p.FV ? dh : -32768;  // absent block: never inside the image
       blkDw[jb] = dw;
 #pragma unroll
-      for (int e4 = 0; e4 < 4; ++e4) xOff[4 * jb + e4] = (cb + rg + 8 * e4) * HW + dh + p.H * dw;
+      for (int e4 = 0; e4 < 4; ++e4) xOffS[4 * jb + e4] = (cb + 2 * waveU + 8 * e4) * HW * 4;
+      blkShift[jb] = (dh + p.H * dw) * 4;  // (added to the lane's offset, and only where the shifted pixel is inside the image)
     }
 #pragma unroll
     for (int e = 0; e < APT; ++e) {
-      const int k = k0 + rg + 8 * e;
-      yOff[e] = (k < p.K ? k : 0) * Q;
-      kPresent |= k < p.K ? (1u << e) : 0u;
+      const int kE = k0 + 2 * waveU + 8 * e;  // (row of half 0; half 1 reads the row after it)
+      yOffS[e] = (kE < p.K ? kE : 0) * Q * 4;
+      kPresent |= kE + half < p.K ? (1u << e) : 0u;
     }
   }
 
@@ -513,26 +523,19 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
     p.byOH.divmod(q, &ow, &oh);
     const int ihB = oh * p.sy, iwB = ow * p.sx;
     if (UT) {
-      const int pixX = n * p.xImg + ihB + p.H * iwB;
-      const int pixY = n * p.dyImg + q;
+      const unsigned pixX = (unsigned)(n * p.xImg + ihB + p.H * iwB + half * HW) * 4u;
+      const unsigned pixY = valid ? (unsigned)(n * p.dyImg + q + half * Q) * 4u : kOutside;
 #pragma unroll
       for (int jb = 0; jb < NBLK; ++jb) {
         const bool ok = valid && (unsigned)(ihB + blkDh[jb]) < (unsigned)p.H && (unsigned)(iwB + blkDw[jb]) < (unsigned)p.W;
-        if (ok) {
+        const unsigned vo = ok ? pixX + (unsigned)blkShift[jb] : kOutside;
 #pragma unroll
-          for (int e4 = 0; e4 < 4; ++e4) pb[4 * jb + e4] = x[pixX + xOff[4 * jb + e4]];
-        } else {
-#pragma unroll
-          for (int e4 = 0; e4 < 4; ++e4) pb[4 * jb + e4] = 0.f;
-        }
+        for (int e4 = 0; e4 < 4; ++e4)
+          pb[4 * jb + e4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)vo, xOffS[4 * jb + e4], 0));
       }
-      if (valid) {
 #pragma unroll
-        for (int e = 0; e < APT; ++e) pa[e] = dy[pixY + yOff[e]];
-      } else {
-#pragma unroll
-        for (int e = 0; e < APT; ++e) pa[e] = 0.f;
-      }
+      for (int e = 0; e < APT; ++e)
+        pa[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(yr, (int)pixY, yOffS[e], 0));
       okA = kPresent;
       okB = 0xffffffffu;
       return;
@@ -747,8 +750,9 @@ Wide wide_of(const ConvP& p) { return Wide{p.C * p.H * p.W, p.K * p.outH * p.out
 // the tap-major variant of the filter-gradient kernel: 32-row blocks inside one tap, 32-bit element offsets
 // (takes the whole layer, not a group view: the offsets span the whole tensors)
 bool wgrad_uniform_tap(const ConvP& p) {
-  return p.FC % 32 == 0 && (long long)p.H * p.W * p.C * p.N < (1ll << 31) &&
-         (long long)p.outH * p.outW * p.K * p.N < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
+  // (byte offsets into x and dzdy stay below the "outside" offset of the buffer loads)
+  return p.FC % 32 == 0 && (long long)p.H * p.W * p.C * p.N < (1ll << 29) &&
+         (long long)p.outH * p.outW * p.K * p.N < (1ll << 29) && !tunable("conv_no_uniform_tap", 0);
 }
 
 // filter-volume rows per workgroup of the filter-gradient kernel: 128; 64 when the whole volume fits in 64 rows (a
@@ -1235,6 +1239,14 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
   q.sy = p.sy; q.sx = p.sx; q.pt = p.pt; q.pl = p.pl; q.dly = p.dy; q.dlx = p.dx;
   q.FV = p.FH * p.FW * p.FC;
   q.M = p.outH * p.outW * p.N;
+  {
+    // what the product reads of x and dzdy, from the group's first channel on (the uniform-tap test keeps both below
+    // 2 GiB; only that variant uses them)
+    const long long xb = ((long long)(p.N - 1) * wd.xImg + (long long)p.C * p.H * p.W) * 4;
+    const long long yb = ((long long)(p.N - 1) * wd.yImg + (long long)p.K * p.outH * p.outW) * 4;
+    q.xBytes = (unsigned)std::min<long long>(xb, 0x7fffffffll);
+    q.dyBytes = (unsigned)std::min<long long>(yb, 0x7fffffffll);
+  }
   int tiles = 0;
   q.splits = wgrad_splits(p, &tiles);
   const int chunks = (q.M + 31) / 32;

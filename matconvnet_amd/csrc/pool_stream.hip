@@ -31,6 +31,7 @@ struct PoolS {
   int maxC;      // widest frame over the tiles of a plane, in columns
   int TW, tilesPerPlane, totalTiles;
   int accumulate;
+  int ablate;  // (experiments only, wrong results: 1 skips the ordered passes, 2 the winner search too)
   int walk;  // 0: tiles dealt round-robin to workgroups; 1: one contiguous run each; 2: round-robin inside each XCD's eighth;
              // 3: planes dealt round-robin to XCDs, a plane's tiles round-robin to that XCD's workgroups
   int KH, nPasses;
@@ -117,9 +118,12 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
   const int poolH = PH > 0 ? PH : p.poolH, poolW = PW > 0 ? PW : p.poolW;
 
   // Tiles are dealt so that the workgroups running at any moment cover one contiguous stretch of each tensor
-  // (DRAM rows are used up while they are open): workgroup b takes tiles b, b + G, b + 2G, ...  Measured on the
-  // 112x112x64x32 3x3/2 case, cold caches: 44 us, against 46.5 us when each XCD walks its own eighth of the
-  // tiles that way and 50 us when every workgroup owns one contiguous run of tiles.
+  // (DRAM rows are used up while they are open) and so that the tiles of one plane, which read each other's border
+  // columns, sit behind one L2 (walk 3: planes round-robin over the XCDs, a plane's tiles round-robin over that XCD's
+  // workgroups).  Measured on the 112x112x64x32 3x3/2 case, cold caches: walk 3 fetches 128.6 MB per launch through the
+  // fabric (the tensors' 128.5 MB once) in 44 us; walk 0 (tiles round-robin over all workgroups) 153.5 MB in the same
+  // 44 us, 46.5 us when each XCD walks its own eighth of the tiles that way, 50 us when every workgroup owns one
+  // contiguous run of tiles.
   const int G = (int)gridDim.x;
   int t0, t1, step, zFirst = 0, zStep = 1;
   if (p.walk == 0) {
@@ -259,6 +263,7 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
       prefetch_tile<OPT, XPT, T>(xr, dr, nxt, tid);
     }
 
+    if (p.ablate < 2) {
     // ---- winner of each owned output: first maximum of its window, scanning column by column
     float best[OPT];
     int code[OPT];  // 8 * column offset + row offset of the winner, -1 when nothing beats -inf
@@ -312,7 +317,9 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
 
     // ---- ordered passes: in pass r the outputs of rank r add into their winner's accumulator
     // (a lane sitting out a pass adds into its private idle slot: a select instead of a masked region)
-    if (NP > 0) {
+    if (p.ablate >= 1) {
+      lds_barrier();
+    } else if (NP > 0) {
 #pragma unroll
       for (int r = 0; r < NP; ++r) {
         float a[OPT];
@@ -335,6 +342,7 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
         lds_barrier();
       }
     }
+    } else { lds_barrier(); }
     prevOut = cur.out;
     prevIn4 = nIn4;
     cur = nxt;
@@ -382,7 +390,8 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   const int rows = std::max(p.top + g->H, p.top - g->padTop + (outH - 1) * g->strideY + g->poolH);
   p.Hp = (rows + 3) & ~3;
   p.accumulate = accumulate ? 1 : 0;
-  p.walk = tunable("pool_walk", 0);
+  p.walk = tunable("pool_walk", 3);
+  p.ablate = tunable("pool_ablate", 0);
   p.KH = kh;
   p.nPasses = kh * kw;
   p.rankHpk = p.rankWpk = 0;
