@@ -117,8 +117,9 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
     # fused: ReLU / shortcut sum folded into batch normalisation; packed: the filter banks are re-laid for the matrix
     # kernels by ONE launch at the start of every step (as after an update of the filters) instead of one per product;
     # deferred: the sums over reduction splits that finish the three filter gradients run in one launch at the end;
-    # epilogue_sums: the forward convolutions sum their output per channel, batch normalisation takes those sums
-    blk = vlapi.Bottleneck(N=N, eps=w["eps"], fused=True, packed=True, deferred=True, epilogue_sums=True)
+    # epilogue_sums: the forward convolutions sum their output per channel, batch normalisation takes those sums;
+    # mask_bits: the unit's last ReLU leaves its mask as one bit per element for the backward pass
+    blk = vlapi.Bottleneck(N=N, eps=w["eps"], fused=True, packed=True, deferred=True, epilogue_sums=True, mask_bits=True)
     _load_block(plain_blk, w)
     _load_block(blk, w)
     dt_plain = _time_block(plain_blk, steps, warmup, layer_by_layer=True)
@@ -135,11 +136,11 @@ def bench_block(vlapi, capi, workloads, steps, warmup):
     conv_flops = {"conv_wgrad_mfma": 2.0 * P * N * (256 * 64 + 9 * 64 * 64 + 64 * 256)}
     eS, eB = 4.0 * P * 64 * N, 4.0 * P * 256 * N
     hbm_bytes = {  # algorithmic bytes per step of the memory-bound families (reads + writes once each)
-        # forward reads x; backward reads x and dzdy; bn3's backward also reads the block output (mask) and writes
-        # the masked derivative
-        "bnorm_sums": 2 * (eS + eS + eB) + 2 * eB,                # (the forward sums come from the convolutions)
-        "bnorm_forward_apply": 2 * eS + 2 * eS + 3 * eB,          # bn1, bn2 with ReLU; bn3 with shortcut sum and ReLU
-        "bnorm_backward_apply": 3 * (eS + eS + eB),
+        # backward sums read x and dzdy (the forward sums come from the convolutions); bn3's passes also read the last
+        # ReLU's mask, one bit per element
+        "bnorm_sums": 2 * (eS + eS + eB) + eB / 32,
+        "bnorm_forward_apply": 2 * eS + 2 * eS + 3 * eB + eB / 32,  # bn1, bn2 with ReLU; bn3 with shortcut sum, ReLU and its mask bits
+        "bnorm_backward_apply": 3 * (eS + eS + eB) + eB / 32,
         "eltwise_kernel": 0.0,                                    # (nothing left: every element-wise layer is folded)
     }
     fam = {}
@@ -301,7 +302,7 @@ def bench_pool_bwd(capi, workloads, reps):
                 call()
             _sync()
             t[label], _ = kernel_time(capi, "pool_backward", call, reps)
-        rows.append(dict(op=name, kernel="pool_max_backward_stream" if method == "max" else "pool_backward_passes",
+        rows.append(dict(op=name, kernel="pool_max_backward_stream" if method == "max" else "pool_backward_avg_tiles",
                          workload="configs[2] %s on %s" % (method, "x".join(map(str, shape))),
                          bound="hbm", achieved=nbytes / t["cold"] / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s",
                          frac=nbytes / t["cold"] / PEAK_HBM, avg_launch_us=t["cold"] * 1e6,
@@ -488,7 +489,7 @@ def bench_resnet50(vlapi, batch, steps, warmup):
     (softmax log-loss on random labels) + backward + SGD update, and evaluation (stored moments; the mode of the reference's published 396 images/s,
     doc/site/docs/pretrained.md:233, measured there on other hardware), images/s."""
     import torch
-    net = vlapi.ResNet50(N=batch, eps=1e-5, image_size=224, classes=1000, fused=True, seed=11)
+    net = vlapi.ResNet50(N=batch, eps=1e-5, image_size=224, classes=1000, fused=True, seed=11, channel_sums=True)
     try:
         r = np.random.default_rng(12)
         net.set("input", np.asfortranarray(r.standard_normal((224, 224, 3, batch), dtype=np.float32)))
@@ -706,11 +707,13 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "BASELINE configs[3]: ResNet-50 bottleneck fwd+bwd, 56x56, 256->64->64->256, N=32; timed schedule: "
                                "vl::nn::Convolution for the convolutions plus this library's folded batch-norm entry points (ReLU and "
-                               "shortcut sum folded in, channel sums taken by the forward convolutions, filter banks packed once per "
-                               "step, one summing launch for the three filter gradients); the reference-interface-only schedule is "
+                               "shortcut sum folded in, channel sums taken by the forward convolutions, the last ReLU's mask kept as bits, "
+                               "filter banks packed once per step, one summing launch for the three filter gradients); the "
+                               "reference-interface-only schedule is "
                                "`block_plain`",
                    "parity": "tests/test_gpu_frontend.py: this schedule at this size against the layer-by-layer block (moments 1e-6, "
-                             "other outputs 1e-4), the layer-by-layer block stage by stage against the oracle at the task's gates "
+                             "other outputs 1e-4; with and without the mask bits: same bits), the layer-by-layer block stage by "
+                             "stage against the oracle at the task's gates "
                              "(conv 2e-4, bnorm 1e-5); end-to-end block tests use 5e-4 (ReLU masks included)"},
         "block_plain": block_plain,
         "roofline": roof,

@@ -192,6 +192,20 @@ MCN_API int mcn_conv_forward_sums(mcn_stream_t stream, const mcn_conv_geom* g, f
                                   const void* packed, size_t packedBytes, double* sums, size_t sumsBytes, void* workspace,
                                   size_t workspaceBytes);
 
+/* dzdx = conv backward-data (as mcn_conv_backward_data_packed with derInputMult = 0) + the derivative that reaches x
+   along a second path, behind a ReLU: addend where its bit in maskBits is set (layout as mcn_bnorm_forward_sums_mask
+   writes it, over a tensor of dzdx's shape), else addend*0.  In a residual block: the identity shortcut's share of the
+   derivative, added in the epilogue of the first convolution's input gradient instead of being written out masked and
+   read back.  Bit-identical to mcn_relu_backward into dzdx followed by mcn_conv_backward_data_packed with
+   derInputMult = 1.  mcn_conv_backward_data_masked_add_supported: 1 when the geometry has this form (a filter bank that
+   fits in local memory, whole 32-channel blocks, planes of a multiple of 32 elements), else 0 and the call fails.
+   No counterpart in the reference. */
+MCN_API int mcn_conv_backward_data_masked_add_supported(const mcn_conv_geom* g);
+MCN_API int mcn_conv_backward_data_masked_add(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, const float* filters,
+                                              const void* packed, size_t packedBytes, const float* derOutput,
+                                              const float* addend, const unsigned* maskBits, void* workspace,
+                                              size_t workspaceBytes);
+
 /* dzdf: FH x FW x FC x K, fully overwritten  (bits/nnconv.cu:280-311: im2row::forward + gemm 't','n'
    accumulated over images) */
 MCN_API int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters,
@@ -301,6 +315,25 @@ MCN_API int mcn_bnorm_backward_masked(mcn_stream_t stream, float* derInput, floa
                                       const float* derOutput, const float* maskSource, float* maskedDerOutput,
                                       int H, int W, int C, int N, double epsilon, void* workspace,
                                       size_t workspaceBytes);
+
+/* The same, with the later ReLU's mask as one bit per element instead of a tensor of floats -- a thirty-second of the
+   bytes on each of the backward sweeps that need it, and no masked copy of the derivative written out.
+     mcn_bnorm_mask_bits_supported  1 when tensors of this shape can carry such a mask (planes of a multiple of 32
+                                    elements, large enough to be walked 16 bytes per lane), else 0
+     mcn_bnorm_forward_sums_mask    mcn_bnorm_forward_sums with the ReLU on, which also writes maskBits: bit e % 32 of
+                                    word e / 32 is set when element e of y (in memory order) is > 0; H*W*C*N/8 bytes
+     mcn_bnorm_backward_bits        mcn_bnorm_backward_masked reading maskBits where that reads maskSource; nothing else
+                                    is written (the other consumers of the masked derivative take derOutput and
+                                    maskBits themselves: mcn_conv_backward_data_masked_add).  Bit-identical to it.
+   No counterpart in the reference. */
+MCN_API int mcn_bnorm_mask_bits_supported(int H, int W, int C, int N);
+MCN_API int mcn_bnorm_forward_sums_mask(mcn_stream_t stream, float* y, unsigned* maskBits, float* moments, const float* x,
+                                        const float* multipliers, const float* biases, const float* residual, int H, int W,
+                                        int C, int N, double epsilon, const double* sums, int sumGroups);
+MCN_API int mcn_bnorm_backward_bits(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
+                                    const float* moments, const float* x, const float* multipliers, const float* derOutput,
+                                    const unsigned* maskBits, int H, int W, int C, int N, double epsilon, void* workspace,
+                                    size_t workspaceBytes);
 
 /* dzdx (H x W x C x N), dzdg (C), dzdb (C), all fully overwritten.  givenMoments == 0: BatchNorm::backward
    (bits/nnbnorm.cu:307-365), moments written if non-NULL.  givenMoments != 0: backwardWithMoment (:263-305). */

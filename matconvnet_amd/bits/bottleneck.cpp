@@ -14,7 +14,7 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
     : H(H), W(W), C(C), M(M), N(N), Cout(CoutArg > 0 ? CoutArg : C), stride(stride), Ho((H - 1) / stride + 1),
       Wo((W - 1) / stride + 1), adapter(adapter), epsilon(epsilon), context(shared ? *shared : ownContext),
       error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), testMode(false), packed(false), packedArena(NULL), packedJobs(NULL), packedBlocks(0), deferred(false), externalSums(false),
-      partialArena(NULL), sumJobsDevice(NULL), sumBlocks(0), epilogueSums(false), sumsBuffer(NULL), sumsBytes(0),
+      partialArena(NULL), sumJobsDevice(NULL), sumBlocks(0), epilogueSums(false), sumsBuffer(NULL), maskBits(NULL), sumsBytes(0),
       sideStream(NULL) {
   for (int i = 0; i < 4; ++i) sumGroupsOf[i] = 0;
   for (int i = 0; i < 5; ++i) events[i] = NULL;
@@ -91,6 +91,7 @@ Bottleneck::~Bottleneck() {
   if (partialArena) (void)hipFree(partialArena);
   if (sumJobsDevice) (void)hipFree(sumJobsDevice);
   if (sumsBuffer) (void)hipFree(sumsBuffer);
+  if (maskBits) (void)hipFree(maskBits);
 }
 
 #define STEP(stage, call)                                   \
@@ -202,6 +203,8 @@ ErrorCode Bottleneck::setEpilogueSums(bool on) {
   sumsBuffer = NULL;
   sumsBytes = 0;
   epilogueSums = false;
+  if (maskBits) (void)hipFree(maskBits);  // (the mask bits are written by the pass that takes the channel sums)
+  maskBits = NULL;
   for (int i = 0; i < 4; ++i) sumGroupsOf[i] = 0;
   if (!on || error != VLE_Success) return error;
   nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1), c2(context, stride, stride, 1, 1, 1, 1, 1, 1),
@@ -220,6 +223,25 @@ ErrorCode Bottleneck::setEpilogueSums(bool on) {
     return VLE_OutOfGPUMemeory;
   }
   epilogueSums = true;
+  return VLE_Success;
+}
+
+ErrorCode Bottleneck::setMaskBits(bool on) {
+  if (maskBits) (void)hipFree(maskBits);
+  maskBits = NULL;
+  if (!on || error != VLE_Success) return error;
+  // needs: the folded schedule with the third convolution's channel sums, an identity shortcut, planes of whole mask
+  // words, and a first convolution whose input gradient can take the second term
+  if (!fused || !epilogueSums || adapter || sumGroupsOf[2] <= 0 || !mcn_bnorm_mask_bits_supported(Ho, Wo, Cout, N)) return VLE_Success;
+  nn::Convolution c1(context, 1, 1, 0, 0, 0, 0, 1, 1);
+  if (!c1.maskedAddSupported(slot("x").getShape(), slot("f1").getShape())) return VLE_Success;
+  const std::size_t words = (slot("y").getNumElements() + 31) / 32;
+  if (hipMalloc((void**)&maskBits, words * sizeof(unsigned)) != hipSuccess) {
+    (void)hipGetLastError();
+    maskBits = NULL;
+    message = "cannot allocate the ReLU mask";
+    return VLE_OutOfGPUMemeory;
+  }
   return VLE_Success;
 }
 
@@ -349,6 +371,11 @@ ErrorCode Bottleneck::forward() {
       float* residual = sg.residual ? buffer(sg.residual) : NULL;
       if (groups > 0) {
         STEP(sg.convStage, sg.op->forwardSums(slot(sg.out), slot(sg.in), slot(sg.filter), (double*)sumsBuffer, sumsBytes));
+        if (i == 2 && maskBits)
+          ABI(sg.bnStage, mcn_bnorm_forward_sums_mask(st, buffer(sg.act), maskBits, buffer(sg.moments), buffer(sg.out), buffer(sg.g),
+                                                      buffer(sg.b), residual, sg.h, sg.w, sg.c, N, epsilon,
+                                                      (double const*)sumsBuffer, groups));
+        else
         ABI(sg.bnStage, mcn_bnorm_forward_sums(st, buffer(sg.act), buffer(sg.moments), buffer(sg.out), buffer(sg.g), buffer(sg.b),
                                                residual, sg.relu, sg.h, sg.w, sg.c, N, epsilon, (double const*)sumsBuffer, groups));
       } else {
@@ -423,20 +450,32 @@ ErrorCode Bottleneck::backward() {
       css(sideContext, stride, stride, 0, 0, 0, 0, 1, 1);
   Tensor none2, none3;
   // (k: the event of the two-stream schedule; 3 - k = the layer's place in {conv1, conv2, conv3, adapter} for k < 3)
+  // maskedAdd: the input gradient also takes the shortcut's share of the derivative, dzdy behind the unit's last ReLU
+  // (mask bits), in its epilogue (derInMult is then 0: nothing is accumulated onto)
   auto convBackward = [&](nn::Convolution& onMain, nn::Convolution& onSide, int k, Tensor& derIn, double derInMult,
-                          Tensor& derFilter, Tensor const& in, Tensor const& filter, Tensor const& derOut) -> ErrorCode {
+                          Tensor& derFilter, Tensor const& in, Tensor const& filter, Tensor const& derOut,
+                          bool maskedAdd = false) -> ErrorCode {
     const int layer = k == 3 ? 3 : 2 - k;
+    auto dataPart = [&]() -> ErrorCode {
+      if (maskedAdd) return onMain.backwardDataMaskedAdd(derIn, filter, derOut, buffer("dzdy"), maskBits);
+      return onMain.backwardAccumulate(derIn, derInMult, none2, none, in, filter, derOut);
+    };
     if (!overlap && deferred && partialBank[layer].bytes) {
-      ErrorCode ed = onMain.backwardAccumulate(derIn, derInMult, none2, none, in, filter, derOut);
+      ErrorCode ed = dataPart();
       if (ed != VLE_Success) return ed;
       return onMain.backwardFilterPartial(derFilter, in, derOut, (char*)partialArena + partialBank[layer].offset,
                                           partialBank[layer].bytes);
     }
-    if (!overlap) return onMain.backwardAccumulate(derIn, derInMult, derFilter, none, in, filter, derOut);
+    if (!overlap && !maskedAdd) return onMain.backwardAccumulate(derIn, derInMult, derFilter, none, in, filter, derOut);
+    if (!overlap) {
+      ErrorCode ed = dataPart();
+      if (ed != VLE_Success) return ed;
+      return onMain.backwardAccumulate(none3, 0, derFilter, none, in, filter, derOut);
+    }
     if (hipEventRecord((hipEvent_t)events[k], (hipStream_t)st) != hipSuccess ||
         hipStreamWaitEvent((hipStream_t)sideStream, (hipEvent_t)events[k], 0) != hipSuccess)
       return context.setError(VLE_Cuda, "cannot order the second stream");
-    ErrorCode e = onMain.backwardAccumulate(derIn, derInMult, none2, none, in, filter, derOut);
+    ErrorCode e = dataPart();
     if (e != VLE_Success) return e;
     e = onSide.backwardAccumulate(none3, 0, derFilter, none, in, filter, derOut);
     if (e != VLE_Success) context.setError(e, sideContext.getLastErrorMessage().c_str());
@@ -462,6 +501,10 @@ ErrorCode Bottleneck::backward() {
     // branch) in the summing pass of the batch-norm derivative
     wsBn = context.getWorkspace(VLDT_GPU, wsBnBytes);
     if (!wsBn) return fail(context.getLastError(), "workspace");
+    if (maskBits)  // (the mask as bits; the shortcut's share of the derivative is added by the first convolution below)
+      ABI("bn3_bwd", mcn_bnorm_backward_bits(st, buffer("da3"), buffer("dg3"), buffer("db3"), buffer("m3"), buffer("a3"),
+                                             buffer("g3"), buffer("dzdy"), maskBits, Ho, Wo, Cout, N, epsilon, wsBn, wsOut));
+    else
     ABI("bn3_bwd", mcn_bnorm_backward_masked(st, buffer("da3"), buffer("dg3"), buffer("db3"), buffer("m3"), buffer("a3"),
                                              buffer("g3"), buffer("dzdy"), buffer(mask3), buffer(dsName), Ho, Wo, Cout, N,
                                              epsilon, wsBn, wsOut));
@@ -506,7 +549,8 @@ ErrorCode Bottleneck::backward() {
     return VLE_Success;
   }
   if (fused) {
-    STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dzdx"), 1, slot("df1"), slot("x"), slot("f1"), slot("da1")));
+    if (maskBits) STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dzdx"), 0, slot("df1"), slot("x"), slot("f1"), slot("da1"), true));
+    else STEP("conv1_bwd", convBackward(c1, c1s, 2, slot("dzdx"), 1, slot("df1"), slot("x"), slot("f1"), slot("da1")));
     STEP("join", joinSide());
     return VLE_Success;
   }

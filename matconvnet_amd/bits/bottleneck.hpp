@@ -72,6 +72,13 @@ class Bottleneck {
   // in a summing pass of their own (mcn_bnorm_forward_sums).  The moments then come from a different summation order
   // than the two-launch form's: same values to rounding (1e-7 relative), not the same bits.
   ErrorCode setEpilogueSums(bool on);
+  // mask bits = true (with epilogue sums, identity shortcut): the unit's last ReLU leaves its mask as one bit per
+  // element (mcn_bnorm_forward_sums_mask); backward reads the bits instead of the unit's output
+  // (mcn_bnorm_backward_bits) and the shortcut's share of the derivative is added, masked, in the epilogue of the
+  // first convolution's input gradient (mcn_conv_backward_data_masked_add) instead of being written out and read
+  // back.  Same bits as without.  Stays off (returns success) where the shapes have no such form.
+  ErrorCode setMaskBits(bool on);
+  bool maskBitsOn() const { return maskBits != NULL; }
   ErrorCode forward();
   ErrorCode backward();
 
@@ -116,6 +123,7 @@ class Bottleneck {
   bool epilogueSums;
   int sumGroupsOf[4];   // [convolution]: partial sums per channel its forward writes (0: it cannot)
   void* sumsBuffer;     // the partial sums of the convolution that ran last
+  unsigned* maskBits;   // one bit per element of y: what the unit's last ReLU let through (setMaskBits)
   std::size_t sumsBytes;
   Context sideContext;
   void* sideStream;     // hipStream_t

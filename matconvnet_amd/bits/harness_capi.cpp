@@ -191,6 +191,8 @@ int vlh_bottleneck_set_deferred(void* block, int deferred) {
   return (int)((BlockHandle*)block)->block->setDeferred(deferred != 0);
 }
 int vlh_bottleneck_set_epilogue_sums(void* block, int on) { return (int)((BlockHandle*)block)->block->setEpilogueSums(on != 0); }
+int vlh_bottleneck_set_mask_bits(void* block, int on) { return (int)((BlockHandle*)block)->block->setMaskBits(on != 0); }
+int vlh_bottleneck_mask_bits_on(void* block) { return ((BlockHandle*)block)->block->maskBitsOn() ? 1 : 0; }
 int vlh_bottleneck_set_packed(void* block, int packed) { return (int)((BlockHandle*)block)->block->setPacked(packed != 0); }
 int vlh_bottleneck_pack(void* block) { return (int)((BlockHandle*)block)->block->pack(); }
 int vlh_bottleneck_forward(void* block) { return (int)((BlockHandle*)block)->block->forward(); }
@@ -245,6 +247,7 @@ int vlh_resnet50_set_stream(void* net, void* stream) { return (int)((harness::Re
 void vlh_resnet50_set_fused(void* net, int fused) { ((harness::ResNet50*)net)->setFused(fused != 0); }
 void vlh_resnet50_set_test_mode(void* net, int test) { ((harness::ResNet50*)net)->setTestMode(test != 0); }
 int vlh_resnet50_set_deferred(void* net, int deferred) { return (int)((harness::ResNet50*)net)->setDeferred(deferred != 0); }
+int vlh_resnet50_set_channel_sums(void* net, int on) { return (int)((harness::ResNet50*)net)->setChannelSums(on != 0); }
 int vlh_resnet50_set_packed(void* net, int packed) { return (int)((harness::ResNet50*)net)->setPacked(packed != 0); }
 int vlh_resnet50_pack(void* net) { return (int)((harness::ResNet50*)net)->pack(); }
 int vlh_resnet50_init(void* net, unsigned long long seed) { return (int)((harness::ResNet50*)net)->initParameters(seed); }

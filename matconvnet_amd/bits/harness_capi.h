@@ -57,6 +57,8 @@ VLH_API int vlh_bottleneck_set_deferred(void* block, int deferred);
 VLH_API int vlh_bottleneck_set_packed(void* block, int packed);
 /* the forward convolutions also sum their output per channel; the batch normalisations take those sums (fused mode) */
 VLH_API int vlh_bottleneck_set_epilogue_sums(void* block, int on);
+VLH_API int vlh_bottleneck_set_mask_bits(void* block, int on);
+VLH_API int vlh_bottleneck_mask_bits_on(void* block);  /* 1 when the shapes allowed it */
 VLH_API int vlh_bottleneck_pack(void* block);
 VLH_API int vlh_bottleneck_forward(void* block);
 VLH_API int vlh_bottleneck_backward(void* block);
@@ -83,6 +85,7 @@ VLH_API void vlh_resnet50_set_test_mode(void* net, int test);
 /* deferred != 0: the sums over reduction splits that finish the filter gradients run in ONE launch at the end of
    vlh_resnet50_backward instead of one per layer (same bits) */
 VLH_API int vlh_resnet50_set_deferred(void* net, int deferred);
+VLH_API int vlh_resnet50_set_channel_sums(void* net, int on);
 VLH_API int vlh_resnet50_set_packed(void* net, int packed);
 VLH_API int vlh_resnet50_pack(void* net);
 VLH_API int vlh_resnet50_init(void* net, unsigned long long seed);

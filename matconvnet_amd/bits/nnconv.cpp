@@ -97,6 +97,34 @@ ErrorCode Convolution::forwardSums(Tensor& output, Tensor const& input, Tensor c
   return fromAbi(context, rc, "Convolution::forwardSums");
 }
 
+bool Convolution::maskedAddSupported(TensorShape const& data, TensorShape const& filter) const {
+  mcn_conv_geom g = geometry(*this, data, filter);
+  return mcn_conv_backward_data_masked_add_supported(&g) != 0;
+}
+
+ErrorCode Convolution::backwardDataMaskedAdd(Tensor& derInput, Tensor const& filter, Tensor const& derOutput,
+                                             float const* addend, unsigned const* maskBits) {
+  tensor_type tt = findTensorType(derInput, filter, derOutput);
+  ErrorCode e = requireHipFloat(context, tt, "Convolution::backwardDataMaskedAdd");
+  if (e != VLE_Success) return e;
+  if (!derInput || !filter || !derOutput || !addend || !maskBits)
+    return context.setError(VLE_IllegalArgument, "Convolution::backwardDataMaskedAdd: DERINPUT, FILTER, DEROUTPUT, the addend and its mask are required");
+  mcn_conv_geom g = geometry(*this, derInput, filter);
+  int oh = 0, ow = 0;
+  int rc = mcn_conv_output_size(&g, &oh, &ow);
+  if (rc) return fromAbi(context, rc, "Convolution::backwardDataMaskedAdd");
+  if ((int)derOutput.getHeight() != oh || (int)derOutput.getWidth() != ow || derOutput.getDepth() != filter.getSize() ||
+      derOutput.getSize() != derInput.getSize())
+    return context.setError(VLE_IllegalArgument, "Convolution::backwardDataMaskedAdd: DEROUTPUT dimensions are incompatible with X and FILTERS");
+  void* ws;
+  size_t bytes;
+  if (!scratch(context, g, MCN_CONV_BACKWARD_DATA, &ws, &bytes)) return context.getLastError();
+  rc = mcn_conv_backward_data_masked_add(context.getHipHelper().getStream(), &g, (float*)derInput.getMemory(),
+                                         (float const*)filter.getMemory(), packedBackward, packedBackwardBytes,
+                                         (float const*)derOutput.getMemory(), addend, maskBits, ws, bytes);
+  return fromAbi(context, rc, "Convolution::backwardDataMaskedAdd");
+}
+
 std::size_t Convolution::packedBytes(int product, TensorShape const& data, TensorShape const& filter) const {
   mcn_conv_geom g = geometry(*this, data, filter);
   return mcn_conv_packed_bytes(&g, product);

@@ -61,6 +61,13 @@ class Convolution {
   vl::ErrorCode forwardSums(vl::Tensor& output, vl::Tensor const& input, vl::Tensor const& filter, double* sums,
                             std::size_t sumsBytes);
 
+  // DERINPUT = backward-data + a second term gated by one bit per element (mcn_conv_backward_data_masked_add): the
+  // derivative an identity shortcut brings to the same tensor from behind a ReLU.  maskedAddSupported: whether this
+  // geometry has that form.  Not part of the reference's class.
+  bool maskedAddSupported(vl::TensorShape const& data, vl::TensorShape const& filter) const;
+  vl::ErrorCode backwardDataMaskedAdd(vl::Tensor& derInput, vl::Tensor const& filter, vl::Tensor const& derOutput,
+                                      float const* addend, unsigned const* maskBits);
+
   Context& context;
   int strideY;
   int strideX;

@@ -315,6 +315,17 @@ ErrorCode ResNet50::setPacked(bool on) {
   return pack();
 }
 
+ErrorCode ResNet50::setChannelSums(bool on) {
+  if (error != VLE_Success) return error;
+  dropGraph();
+  for (std::size_t i = 0; i < units.size(); ++i)
+    if (units[i]->setEpilogueSums(on) != VLE_Success || units[i]->setMaskBits(on) != VLE_Success) {
+      message = units[i]->lastMessage();
+      return VLE_OutOfGPUMemeory;
+    }
+  return VLE_Success;
+}
+
 ErrorCode ResNet50::setDeferred(bool on) {
   if (error != VLE_Success) return error;
   dropGraph();

@@ -50,6 +50,11 @@ class ResNet50 {
   // deferred = true: backward() runs the matrix kernels of all filter gradients and sums their reduction splits in ONE
   // launch at its end instead of one per layer.  Same bits.
   ErrorCode setDeferred(bool on);
+  // channel sums = true (folded mode, training): in every unit the forward convolutions sum their own output per
+  // channel for the batch normalisation that follows, and units with an identity shortcut keep their last ReLU's mask
+  // as one bit per element, wherever the shapes have those forms (Bottleneck::setEpilogueSums, setMaskBits).  The
+  // moments then come from another summation order: same values to rounding, not the same bits.
+  ErrorCode setChannelSums(bool on);
   ErrorCode forward();
   ErrorCode backward();
   // The network's last layers (cnn_imagenet_init_resnet.m:128-139): from "prediction" and "labels" (one class number

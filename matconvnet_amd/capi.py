@@ -62,6 +62,11 @@ PROTOTYPES = {
     "mcn_conv_forward_sums_groups": (_i, [C.POINTER(ConvGeom)]),
     "mcn_conv_forward_sums": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz]),
     "mcn_bnorm_forward_sums": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _d, _vp, _i]),
+    "mcn_bnorm_mask_bits_supported": (_i, [_i, _i, _i, _i]),
+    "mcn_bnorm_forward_sums_mask": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _vp, _i]),
+    "mcn_bnorm_backward_bits": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _d, _vp, _sz]),
+    "mcn_conv_backward_data_masked_add_supported": (_i, [C.POINTER(ConvGeom)]),
+    "mcn_conv_backward_data_masked_add": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_data": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_taccum": (_i, [_vp, _vp, C.c_float, _vp, C.c_float, _vp, _sz]),
     "mcn_conv_backward_filter_partial_bytes": (_sz, [_vp]),
@@ -320,6 +325,38 @@ def bnorm_forward_sums(x, g, b, sums, residual=None, relu=False, eps=1e-4):
     check(lib().mcn_bnorm_forward_sums(stream(), ptr(y), ptr(mom), ptr(x), ptr(g), ptr(b), ptr(residual), int(relu),
                                        H, W, Cc, N, eps, ptr(sums), int(sums.shape[1])))
     return y, mom
+
+
+def bnorm_forward_sums_mask(x, g, b, sums, residual=None, eps=1e-4):
+    """mcn_bnorm_forward_sums with the ReLU on, which also writes one bit per element of y: (y, mask words, moments)."""
+    import torch
+    H, W, Cc, N = _hwcn(x)
+    y = empty((H, W, Cc, N))
+    mom = empty((Cc, 2))
+    bits = torch.zeros((H * W * Cc * N + 31) // 32, dtype=torch.int32, device="cuda")
+    check(lib().mcn_bnorm_forward_sums_mask(stream(), ptr(y), ptr(bits), ptr(mom), ptr(x), ptr(g), ptr(b), ptr(residual),
+                                            H, W, Cc, N, eps, ptr(sums), int(sums.shape[1])))
+    return y, bits, mom
+
+
+def bnorm_backward_bits(x, g, dy, bits, moments, eps=1e-4, ws=None):
+    ws = ws or _ws
+    H, W, Cc, N = _hwcn(x)
+    dx, dg, db = empty((H, W, Cc, N)), empty((Cc,)), empty((Cc,))
+    wp, wn = ws.get(lib().mcn_bnorm_workspace_bytes(H, W, Cc, N))
+    check(lib().mcn_bnorm_backward_bits(stream(), ptr(dx), ptr(dg), ptr(db), ptr(moments), ptr(x), ptr(g), ptr(dy), ptr(bits),
+                                        H, W, Cc, N, eps, wp, wn))
+    return dx, dg, db
+
+
+def conv_backward_data_masked_add(f, dy, g, addend, bits, packed=None, ws=None):
+    """dzdx = conv backward-data + (bit ? addend : addend*0)."""
+    ws = ws or _ws
+    dx = empty((g.H, g.W, g.C, g.N))
+    wp, wn = ws.get(lib().mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_DATA))
+    pk, pkn = (ptr(packed), packed.numel() * packed.element_size()) if packed is not None else (None, 0)
+    check(lib().mcn_conv_backward_data_masked_add(stream(), C.byref(g), ptr(dx), ptr(f), pk, pkn, ptr(dy), ptr(addend), ptr(bits), wp, wn))
+    return dx
 
 
 def conv_backward(x, f, dy, g, want=(True, True, True), ws=None):

@@ -84,6 +84,19 @@ __device__ __forceinline__ void forward_coefficients(double mean, double sigma, 
   *k = (float)((double)bias - coef * (mean - (double)*s));
 }
 
+// One bit per element of a tensor, in element order: bit e % 32 of word e / 32 says "the ReLU behind this element let
+// it through" (its output was > 0).  Written by the forward pass that applies that ReLU (stream_forward), read by the
+// backward passes instead of the ReLU's output: a thirty-second of the bytes.  Planes must be whole words (W*H a
+// multiple of 32).  The four bits of the 16-byte cell at element e (a multiple of 4):
+__device__ __forceinline__ unsigned mask_nibble(const unsigned* __restrict__ bits, size_t e) {
+  return (bits[e >> 5] >> (unsigned)(e & 31)) & 15u;
+}
+// dy where the bit is set, else dy*0 like mcn_relu_backward (a NaN or infinity stays visible)
+__device__ __forceinline__ float4 mask_by_nibble(float4 d, unsigned nb) {
+  return make_float4((nb & 1u) ? d.x : d.x * 0.f, (nb & 2u) ? d.y : d.y * 0.f, (nb & 4u) ? d.z : d.z * 0.f,
+                     (nb & 8u) ? d.w : d.w * 0.f);
+}
+
 // Block-wide sum of NV doubles held per thread; result valid in thread 0.
 template <int NV>
 __device__ __forceinline__ void block_sum(double (&v)[NV], double* lds /* [4][NV] */) {
@@ -109,10 +122,13 @@ __device__ __forceinline__ void block_sum(double (&v)[NV], double* lds /* [4][NV
 // YMASK (MODE 1 only): dy first passes the derivative of a ReLU whose *output* is ymask (dy counts where
 // ymask > 0, else dy*0 like mcn_relu_backward), and the masked derivative is also written to `masked` for the
 // passes that follow (this layer's apply pass, and whoever else consumes it).
-template <int MODE, bool VEC4, bool RELU, bool YMASK>
+// BITS (MODE 1, 16-byte accesses only): like YMASK, but the mask comes as one bit per element (`ymask` points at the
+// words, see mask_nibble) and nothing is written.
+template <int MODE, bool VEC4, bool RELU, bool YMASK, bool BITS = false>
 __device__ __forceinline__ void sums_of_planes(double (&acc)[4], const float* __restrict__ x, const float* __restrict__ dy,
                                                const BnormP& p, int c, int n0, int n1, float ra, float rk, float rs,
                                                const float* __restrict__ ymask, float* __restrict__ masked, double* lds) {
+  static_assert(!BITS || (VEC4 && MODE == 1 && !RELU && !YMASK), "the bit mask goes with 16-byte accesses and given moments");
   auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv - rs, rk) > 0.f ? dv : 0.f) : dv; };
   acc[0] = acc[1] = acc[2] = acc[3] = 0.0;
   const int shift = p.teamShift[VEC4 ? 1 : 0], TS = 1 << shift, teams = 256 >> shift;
@@ -138,6 +154,7 @@ __device__ __forceinline__ void sums_of_planes(double (&acc)[4], const float* __
                             m.w > 0.f ? d.w : d.w * 0.f);
             ((float4*)(masked + base))[i] = d;
           }
+          if (BITS) d = mask_by_nibble(d, mask_nibble((const unsigned*)ymask, base + 4 * (size_t)i));
           const double dx_ = (double)d.x, dy_ = (double)d.y, dz_ = (double)d.z, dw_ = (double)d.w;
           acc[2] += fma(ax, dx_, ay * dy_) + fma(az, dz_, aw * dw_);
           acc[3] += (dx_ + dy_) + (dz_ + dw_);
@@ -181,7 +198,7 @@ __device__ __forceinline__ void sums_of_planes(double (&acc)[4], const float* __
   block_sum<4>(acc, lds);
 }
 
-template <int MODE, bool VEC4, bool RELU = false, bool YMASK = false>
+template <int MODE, bool VEC4, bool RELU = false, bool YMASK = false, bool BITS = false>
 __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
                                                   const float* __restrict__ dy,
                                                   double* __restrict__ partials, BnormP p,
@@ -192,6 +209,7 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
                                                   float* __restrict__ masked = nullptr) {
   static_assert(!RELU || MODE == 1, "the ReLU mask needs the moments of the forward pass");
   static_assert(!YMASK || (MODE == 1 && !RELU), "one kind of mask at a time, with given moments");
+  static_assert(!BITS || !YMASK, "one kind of mask at a time");
   __shared__ double lds[16];
   const int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int c = logical / p.groups;
@@ -201,7 +219,7 @@ __global__ __launch_bounds__(256) void bnorm_sums(const float* __restrict__ x,
   float ra = 0.f, rk = 0.f, rs = 0.f;
   if (RELU) forward_coefficients((double)moments[c], (double)moments[c + p.C], mult[c], bias[c], &ra, &rk, &rs);
   double acc[4];
-  sums_of_planes<MODE, VEC4, RELU, YMASK>(acc, x, dy, p, c, n0, n1, ra, rk, rs, ymask, masked, lds);
+  sums_of_planes<MODE, VEC4, RELU, YMASK, BITS>(acc, x, dy, p, c, n0, n1, ra, rk, rs, ymask, masked, lds);
   if (threadIdx.x == 0) {
     double* out = partials + ((size_t)c * p.groups + grp) * 4;
     out[0] = acc[0];
@@ -261,12 +279,14 @@ __device__ __forceinline__ void channel_totals(const double* __restrict__ partia
 
 // out = a*(in1 - t) + b*(in2 - s) + k over this workgroup's planes (in2 optional)
 // RELU: in1 counts only where ra*(in2 - rs) + rk > 0 (in1 = derivative after the ReLU, in2 = the layer's input)
-template <bool TWO, bool VEC4, bool RELU = false>
+// BITS: in1 counts only where its bit is set (see mask_nibble), else as in1*0
+template <bool TWO, bool VEC4, bool RELU = false, bool BITS = false>
 __device__ __forceinline__ void stream_planes(float* __restrict__ out, const float* __restrict__ in1,
                                               const float* __restrict__ in2, float a, float b, float k, float s,
                                               float t, const BnormP& p, int c, int n0, int n1, float ra = 0.f, float rk = 0.f,
-                                              float rs = 0.f) {
+                                              float rs = 0.f, const unsigned* __restrict__ bits = nullptr) {
   static_assert(!RELU || TWO, "the mask is computed from the second stream");
+  static_assert(!BITS || (VEC4 && TWO && !RELU), "the bit mask goes with 16-byte accesses");
   auto gate = [&](float xv, float dv) -> float { return RELU ? (fmaf(ra, xv - rs, rk) > 0.f ? dv : 0.f) : dv; };
   const int shift = p.teamShift[VEC4 ? 1 : 0], TS = 1 << shift, teams = 256 >> shift;
   const int team = threadIdx.x >> shift, j0 = threadIdx.x & (TS - 1);
@@ -278,7 +298,8 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
       const float4* s2 = (const float4*)(TWO ? in2 + base : in1 + base);
       float4* o4 = (float4*)(out + base);
       for (int i = j0; i < p.WH / 4; i += TS) {
-        const float4 u = stream_load4(s1 + i);
+        float4 u = stream_load4(s1 + i);
+        if (BITS) u = mask_by_nibble(u, mask_nibble(bits, base + 4 * (size_t)i));
         float4 r;
         if (TWO) {
           const float4 v = stream_load4(s2 + i);
@@ -308,7 +329,8 @@ __device__ __forceinline__ void stream_planes(float* __restrict__ out, const flo
 // ONE: 0 = totals from the partials of a sums launch; 1 = this workgroup sums its channel itself first (oneLaunch);
 // 2 = the same with the mask of a later ReLU (dy = the raw derivative, ymask that ReLU's output, masked = where the
 // masked derivative goes: the apply pass then reads it back).
-template <bool GIVEN, bool VEC4, bool RELU = false, int ONE = 0>
+// BITS (GIVEN, ONE = 0): dy first passes a ReLU whose mask comes as one bit per element in `ymask` (see mask_nibble).
+template <bool GIVEN, bool VEC4, bool RELU = false, int ONE = 0, bool BITS = false>
 __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ dx,
                                                             float* __restrict__ dmult,
                                                             float* __restrict__ dbias,
@@ -322,6 +344,7 @@ __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ 
                                                             float* __restrict__ masked = nullptr) {
   static_assert(!RELU || GIVEN, "the ReLU mask needs the moments of the forward pass");
   static_assert(ONE != 2 || (GIVEN && !RELU), "one kind of mask at a time, with given moments");
+  static_assert(!BITS || (GIVEN && !RELU && ONE == 0 && VEC4), "the bit mask goes with given moments and a summing launch");
   __shared__ double lds[20];
   int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   if (p.reverse) logical = (int)gridDim.x - 1 - logical;
@@ -368,18 +391,21 @@ __global__ __launch_bounds__(256) void bnorm_backward_apply(float* __restrict__ 
   float ra = 0.f, rk = 0.f, rs = 0.f;
   if (RELU) forward_coefficients(mean, sigma, mult[c], bias[c], &ra, &rk, &rs);
   const float shift = (float)mean, shiftDy = (float)muz;
-  stream_planes<true, VEC4, RELU>(dx, dy, x, (float)G1, (float)(-G2),
-                                  (float)(G2 * (mean - (double)shift) - G1 * (muz - (double)shiftDy)), shift, shiftDy, p, c, n0,
-                                  n1, ra, rk, rs);
+  stream_planes<true, VEC4, RELU, BITS>(dx, dy, x, (float)G1, (float)(-G2),
+                                        (float)(G2 * (mean - (double)shift) - G1 * (muz - (double)shiftDy)), shift, shiftDy, p, c,
+                                        n0, n1, ra, rk, rs, (const unsigned*)ymask);
 }
 
 // out = act(a*(in - s) + k [+ res]) over this workgroup's planes: the forward apply with the element-wise layers
 // that follow it folded in.  Each element goes through the same roundings as the separate kernels would
 // give it: subtract, fma, then add, then max.
-template <bool RES, bool RELU, bool VEC4>
+// BITS: also writes which elements the ReLU let through, one bit each (see mask_nibble): eight neighbouring lanes hold
+// the 32 elements of one word (the host admits only planes of whole words walked by teams of at least 8 lanes).
+template <bool RES, bool RELU, bool VEC4, bool BITS = false>
 __device__ __forceinline__ void stream_forward(float* __restrict__ out, const float* __restrict__ in,
                                                const float* __restrict__ res, float a, float k, float s,
-                                               const BnormP& p, int c, int n0, int n1) {
+                                               const BnormP& p, int c, int n0, int n1, unsigned* __restrict__ bits = nullptr) {
+  static_assert(!BITS || (RELU && VEC4), "the bit mask is the ReLU's, written with 16-byte accesses");
   auto one = [&](float u, float r) -> float {
     float v = fmaf(a, u - s, k);
     if (RES) v = v + r;
@@ -399,7 +425,16 @@ __device__ __forceinline__ void stream_forward(float* __restrict__ out, const fl
         const float4 u = stream_load4(s1 + i);
         float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
         if (RES) r = stream_load4(s2 + i);
-        stream_store4(o4 + i, make_float4(one(u.x, r.x), one(u.y, r.y), one(u.z, r.z), one(u.w, r.w)));
+        const float4 v = make_float4(one(u.x, r.x), one(u.y, r.y), one(u.z, r.z), one(u.w, r.w));
+        stream_store4(o4 + i, v);
+        if (BITS) {
+          unsigned wd = ((v.x > 0.f ? 1u : 0u) | (v.y > 0.f ? 2u : 0u) | (v.z > 0.f ? 4u : 0u) | (v.w > 0.f ? 8u : 0u))
+                        << (4 * (threadIdx.x & 7));
+          wd |= (unsigned)__shfl_xor((int)wd, 1);
+          wd |= (unsigned)__shfl_xor((int)wd, 2);
+          wd |= (unsigned)__shfl_xor((int)wd, 4);
+          if ((threadIdx.x & 7) == 0) bits[(base + 4 * (size_t)i) >> 5] = wd;
+        }
       }
     } else {
       for (int i = j0; i < p.WH; i += TS) out[base + i] = one(in[base + i], RES ? res[base + i] : 0.f);
@@ -409,7 +444,7 @@ __device__ __forceinline__ void stream_forward(float* __restrict__ out, const fl
 
 // Forward apply: y = (g/sigma)*(x - mean) + b  (bits/nnbnorm.cu:190-199), optionally followed by "+ residual"
 // (matlab/+dagnn/Sum.m) and ReLU (matlab/vl_nnrelu.m) in the same pass.
-template <bool GIVEN, bool VEC4, bool RES, bool RELU, bool ONE = false>
+template <bool GIVEN, bool VEC4, bool RES, bool RELU, bool ONE = false, bool BITS = false>
 __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y,
                                                            float* __restrict__ moments,
                                                            const float* __restrict__ x,
@@ -417,7 +452,7 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
                                                            const float* __restrict__ bias,
                                                            const float* __restrict__ residual,
                                                            const double* __restrict__ partials,
-                                                           BnormP p) {
+                                                           BnormP p, unsigned* __restrict__ maskBits = nullptr) {
   __shared__ double lds[20];
   int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
   if (p.reverse) logical = (int)gridDim.x - 1 - logical;
@@ -447,7 +482,7 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
   forward_coefficients(mean, sigma, mult[c], bias[c], &a, &k, &shift);
   int n0, n1;
   image_range(p, grp, &n0, &n1);
-  stream_forward<RES, RELU, VEC4>(y, x, residual, a, k, shift, p, c, n0, n1);
+  stream_forward<RES, RELU, VEC4, BITS>(y, x, residual, a, k, shift, p, c, n0, n1, maskBits);
 }
 
 int image_groups(int WH, int N) {
@@ -553,15 +588,19 @@ int mcn_bnorm_forward_fused(mcn_stream_t stream, float* y, float* moments, const
   return check_launch("mcn_bnorm_forward");
 }
 
-int mcn_bnorm_forward_sums(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,
-                           const float* biases, const float* residual, int relu, int H, int W, int C, int N, double epsilon,
-                           const double* sums, int sumGroups) {
+// Planes of whole 32-bit words, walked 16 bytes per lane by teams of at least 8 lanes: what the one-bit-per-element
+// ReLU masks need (see mask_nibble).
+static bool mask_bits_fit(const BnormP& p) { return p.WH % 32 == 0 && p.teamShift[1] >= 3; }
+
+static int forward_from_sums(const char* who, mcn_stream_t stream, float* y, float* moments, const float* x,
+                             const float* multipliers, const float* biases, const float* residual, int relu, int H, int W,
+                             int C, int N, double epsilon, const double* sums, int sumGroups, unsigned* maskBits) {
   BnormP p;
-  int rc = setup("mcn_bnorm_forward_sums", H, W, C, N, epsilon, &p);
+  int rc = setup(who, H, W, C, N, epsilon, &p);
   if (rc) return rc;
   if ((size_t)p.WH * C * N == 0) return MCN_SUCCESS;
-  if (!y || !x || !multipliers || !biases || !sums) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_sums: null tensor");
-  if (sumGroups <= 0) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_sums: no partial sums");
+  if (!y || !x || !multipliers || !biases || !sums) return fail(MCN_ILLEGAL_ARGUMENT, "%s: null tensor", who);
+  if (sumGroups <= 0) return fail(MCN_ILLEGAL_ARGUMENT, "%s: no partial sums", who);
   if (p.oneLaunch) {  // (the grid of the two-launch form: the sums are there already)
     p.oneLaunch = 0;
     p.groups = image_groups(p.WH, N);
@@ -572,6 +611,14 @@ int mcn_bnorm_forward_sums(mcn_stream_t stream, float* y, float* moments, const 
   hipStream_t s = as_stream(stream);
   const bool vec = (p.WH % 4 == 0) && aligned16(y) && aligned16(x) && (!residual || aligned16(residual));
   const dim3 grid((unsigned)(C * p.groups)), block(256);
+  if (maskBits) {
+    if (!relu || !vec || !mask_bits_fit(p))
+      return fail(MCN_UNSUPPORTED, "%s: the bit mask needs a ReLU, 16-byte aligned tensors and planes of a multiple of 32 elements", who);
+    KernelTimer timer("bnorm_forward_apply", s);
+    if (residual) hipLaunchKernelGGL((bnorm_forward_apply<false, true, true, true, false, true>), grid, block, 0, s, y, moments, x, multipliers, biases, residual, sums, p, maskBits);
+    else hipLaunchKernelGGL((bnorm_forward_apply<false, true, false, true, false, true>), grid, block, 0, s, y, moments, x, multipliers, biases, residual, sums, p, maskBits);
+    return check_launch(who);
+  }
   KernelTimer timer("bnorm_forward_apply", s);
 #define MCN_BN_SUMS(VECF, RESF, RELUF) \
   hipLaunchKernelGGL((bnorm_forward_apply<false, VECF, RESF, RELUF>), grid, block, 0, s, y, moments, x, multipliers, biases, residual, sums, p)
@@ -586,7 +633,60 @@ int mcn_bnorm_forward_sums(mcn_stream_t stream, float* y, float* moments, const 
   else MCN_BN_SUMS_EPI(false);
 #undef MCN_BN_SUMS_EPI
 #undef MCN_BN_SUMS
-  return check_launch("mcn_bnorm_forward_sums");
+  return check_launch(who);
+}
+
+int mcn_bnorm_forward_sums(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,
+                           const float* biases, const float* residual, int relu, int H, int W, int C, int N, double epsilon,
+                           const double* sums, int sumGroups) {
+  return forward_from_sums("mcn_bnorm_forward_sums", stream, y, moments, x, multipliers, biases, residual, relu, H, W, C, N,
+                           epsilon, sums, sumGroups, nullptr);
+}
+
+int mcn_bnorm_mask_bits_supported(int H, int W, int C, int N) {
+  BnormP p;
+  if (setup("mcn_bnorm_mask_bits_supported", H, W, C, N, 1e-4, &p) || (size_t)p.WH * C * N == 0) return 0;
+  return mask_bits_fit(p) && !p.oneLaunch ? 1 : 0;
+}
+
+int mcn_bnorm_forward_sums_mask(mcn_stream_t stream, float* y, unsigned* maskBits, float* moments, const float* x,
+                                const float* multipliers, const float* biases, const float* residual, int H, int W, int C,
+                                int N, double epsilon, const double* sums, int sumGroups) {
+  if (!maskBits) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_forward_sums_mask: null mask");
+  return forward_from_sums("mcn_bnorm_forward_sums_mask", stream, y, moments, x, multipliers, biases, residual, 1, H, W, C, N,
+                           epsilon, sums, sumGroups, maskBits);
+}
+
+int mcn_bnorm_backward_bits(mcn_stream_t stream, float* derInput, float* derMultipliers, float* derBiases,
+                            const float* moments, const float* x, const float* multipliers, const float* derOutput,
+                            const unsigned* maskBits, int H, int W, int C, int N, double epsilon, void* workspace,
+                            size_t workspaceBytes) {
+  BnormP p;
+  int rc = setup("mcn_bnorm_backward_bits", H, W, C, N, epsilon, &p);
+  if (rc) return rc;
+  if ((size_t)p.WH * C * N == 0) return MCN_SUCCESS;
+  if (!derInput || !derMultipliers || !derBiases || !moments || !x || !multipliers || !derOutput || !maskBits)
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_bits: null tensor");
+  if (!mask_bits_fit(p) || p.oneLaunch || !aligned16(derInput) || !aligned16(x) || !aligned16(derOutput))
+    return fail(MCN_UNSUPPORTED, "mcn_bnorm_backward_bits: the bit mask needs 16-byte aligned tensors and planes of a multiple "
+                "of 32 elements (ask mcn_bnorm_mask_bits_supported)");
+  if (!workspace || workspaceBytes < mcn_bnorm_workspace_bytes(H, W, C, N))
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_bnorm_backward_bits: workspace too small");
+  hipStream_t s = as_stream(stream);
+  const dim3 grid((unsigned)(C * p.groups)), block(256);
+  double* partials = (double*)workspace;
+  float* mom = const_cast<float*>(moments);  // (the kernels only write moments when they are not given)
+  const float* bitsAsMask = (const float*)maskBits;
+  {
+    KernelTimer timer("bnorm_sums", s);
+    hipLaunchKernelGGL((bnorm_sums<1, true, false, false, true>), grid, block, 0, s, x, derOutput, partials, p, nullptr, nullptr,
+                       nullptr, bitsAsMask, nullptr);
+  }
+  if ((rc = check_launch("mcn_bnorm_backward_bits(sums)"))) return rc;
+  KernelTimer timer("bnorm_backward_apply", s);
+  hipLaunchKernelGGL((bnorm_backward_apply<true, true, false, 0, true>), grid, block, 0, s, derInput, derMultipliers, derBiases,
+                     mom, x, multipliers, derOutput, partials, p, nullptr, bitsAsMask, nullptr);
+  return check_launch("mcn_bnorm_backward_bits");
 }
 
 int mcn_bnorm_forward(mcn_stream_t stream, float* y, float* moments, const float* x, const float* multipliers,

@@ -33,6 +33,7 @@ Tunable g_tunables[] = {
     {"pool_no_stream", 0},             // 1: max pooling skips the streaming kernel
     {"pool_walk", 3},                  // streaming kernel's tile order: 0 round-robin, 1 contiguous runs, 2 round-robin per XCD eighth, 3 planes round-robin over XCDs
     {"bnorm_sums_scalar", 0},          // 1: the summing pass of batch-norm backward (moments from the batch) loads 4 bytes per lane, four in flight
+    {"pool_no_tiles", 0},              // 1: average pooling over windows that tile the plane skips its streaming kernel
     {"pool_ablate", 0},                // (experiments only, wrong results) 1: no ordered passes, 2: no winner search either
     {"pool_threads", 256},             // threads per workgroup of the streaming kernel (256; 512 and 1024 for 3x3 / 2 windows)
     {"pool_blocks_per_cu", 3},         // persistent workgroups per compute unit of the streaming kernel

@@ -279,6 +279,37 @@ int mcn_conv_backward_data_packed(mcn_stream_t stream, const mcn_conv_geom* g, f
   return conv_backward_data_direct(as_stream(stream), p, derInput, derInputMult, filters, derOutput);
 }
 
+int mcn_conv_backward_data_masked_add_supported(const mcn_conv_geom* g) {
+  ConvP p;
+  if (conv_setup(g, "mcn_conv_backward_data_masked_add_supported", &p) || (size_t)p.H * p.W * p.C * p.N == 0) return 0;
+  if (tunable("conv_force_direct", 0) || !conv_mfma_backward_data_supported(p)) return 0;
+  int ok = 0;
+  float* none = nullptr;  // (nothing is touched when planning)
+  if (conv_backward_data_mfma(nullptr, p, none, 0.f, none, none, nullptr, 0, nullptr, nullptr, nullptr, &ok)) return 0;
+  return ok;
+}
+
+int mcn_conv_backward_data_masked_add(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, const float* filters,
+                                      const void* packed, size_t packedBytes, const float* derOutput, const float* addend,
+                                      const unsigned* maskBits, void* workspace, size_t workspaceBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_data_masked_add", &p);
+  if (rc) return rc;
+  if ((size_t)p.H * p.W * p.C * p.N == 0) return MCN_SUCCESS;
+  if (!derInput || !filters || !derOutput || !addend || !maskBits)
+    return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data_masked_add: null tensor");
+  if (!mcn_conv_backward_data_masked_add_supported(g))
+    return fail(MCN_UNSUPPORTED, "mcn_conv_backward_data_masked_add: this geometry has no such form (ask "
+                "mcn_conv_backward_data_masked_add_supported)");
+  if (packed) {
+    PackCtx pk = {PackCtx::kUse, (char*)const_cast<void*>(packed), packedBytes, 0, nullptr};
+    return conv_backward_data_mfma(as_stream(stream), p, derInput, 0.f, filters, derOutput, workspace, workspaceBytes, &pk,
+                                   addend, maskBits);
+  }
+  return conv_backward_data_mfma(as_stream(stream), p, derInput, 0.f, filters, derOutput, workspace, workspaceBytes, nullptr,
+                                 addend, maskBits);
+}
+
 int mcn_conv_backward_data(mcn_stream_t stream, const mcn_conv_geom* g, float* derInput, const float* filters,
                            const float* derOutput, void* workspace, size_t workspaceBytes) {
   return mcn_conv_backward_data_acc(stream, g, derInput, 0.f, filters, derOutput, workspace, workspaceBytes);

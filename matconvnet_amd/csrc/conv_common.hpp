@@ -81,8 +81,10 @@ size_t conv_mfma_workspace_bytes(const ConvP& p, int product);
 int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
                       const float* f, const float* b, void* ws, size_t wsBytes, PackCtx* pk = nullptr,
                       double* stats = nullptr, int statGroups = 0, int* statQuery = nullptr);
+// addend / addBits: a masked second term added in the epilogue (see PixP::addend); addQuery: plan only
 int conv_backward_data_mfma(hipStream_t s, const ConvP& p, float* dx, float dxMult, const float* f, const float* dy,
-                            void* ws, size_t wsBytes, PackCtx* pk = nullptr);
+                            void* ws, size_t wsBytes, PackCtx* pk = nullptr, const float* addend = nullptr,
+                            const unsigned* addBits = nullptr, int* addQuery = nullptr);
 int conv_pack_batch(hipStream_t s, const PackJob* deviceJobs, int nJobs, unsigned totalBlocks);
 int conv_backward_filter_mfma(hipStream_t s, const ConvP& p, float* df, const float* x, const float* dy, void* ws,
                               size_t wsBytes, ReduceCtx* deferred = nullptr);
@@ -121,6 +123,13 @@ struct PixP {
   double* stats = nullptr;
   int statGroups = 0;
   int* statQuery = nullptr;
+  // A second term added in the epilogue (weights-stationary kernel only, dense whole 32-channel blocks, planes of a
+  // multiple of 32 elements, alpha = 1, beta = 0, no bias): out = acc + (bit ? addend : addend*0), addend a tensor of
+  // the produced tensor's layout, bit = bit e % 32 of word e / 32 of addBits for element e.  addQuery (host only): no
+  // launch, just report whether the product has this form.
+  const float* addend = nullptr;
+  const unsigned* addBits = nullptr;
+  int* addQuery = nullptr;
 };
 
 // the pixel's element offset inside its channel plane of the produced tensor
@@ -202,6 +211,33 @@ __device__ __forceinline__ void store_block(floatx16 acc, bufrsrc rsrc, unsigned
     store_block_as<false, true>(acc, rsrc, voffset, sblock, plane, alpha, beta, biasBlk, kh);
   } else {
     store_block_as<false, false>(acc, rsrc, voffset, sblock, plane, alpha, beta, biasBlk, kh);
+  }
+}
+
+// out = acc + (bit ? addend : addend*0): the block of store_block with a second term from a tensor of the same layout,
+// gated by one bit per element (see PixP::addend).  arsrc / brsrc: descriptors of the addend and of the bit words;
+// voffset and sblock as in store_block (plane bytes a multiple of 128, so a lane's bit position is the same for all 16
+// channels and the word offset splits into a lane part and a scalar part).
+__device__ __forceinline__ void store_block_masked_add(floatx16 acc, bufrsrc rsrc, bufrsrc arsrc, bufrsrc brsrc, unsigned voffset,
+                                                       int sblock, int plane) {
+  const __amdgpu_buffer_rsrc_t ar = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(((unsigned long long)(unsigned)arsrc.x) | ((unsigned long long)(unsigned)arsrc.y << 32)), 0, arsrc.z, arsrc.w);
+  const __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(((unsigned long long)(unsigned)brsrc.x) | ((unsigned long long)(unsigned)brsrc.y << 32)), 0, brsrc.z, brsrc.w);
+  const unsigned vword = voffset == kOutside ? kOutside : (voffset >> 7) << 2;  // byte offset of the lane's word at scalar offset 0
+  const unsigned bit = (voffset >> 2) & 31u;
+  float add[16];
+  unsigned wd[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int so = sblock + (8 * (r / 4) + r % 4) * plane;
+    add[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, (int)voffset, so, 0));
+    wd[r] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(br, (int)vword, so >> 5, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float term = ((wd[r] >> bit) & 1u) ? add[r] : add[r] * 0.f;
+    buffer_store_untracked(acc[r] + term, voffset, rsrc, sblock + (8 * (r / 4) + r % 4) * plane);
   }
 }
 

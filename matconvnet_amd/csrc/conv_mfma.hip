@@ -892,6 +892,19 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
     return MCN_SUCCESS;
   }
   if (p.stats && !(ut && p.Cout > 4)) return fail(MCN_UNSUPPORTED, "%s: this product cannot sum its output per channel", who);
+  {
+    const long long ob = ((long long)(p.N - 1) * p.outImg + (long long)p.Cout * p.outPlane) * 4;
+    p.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
+  }
+  if (p.addQuery) {  // (plan only: can this product add a masked second term in its epilogue?)
+    *p.addQuery = 0;
+    if (ut && p.Cout > 4) {
+      int handled = 0;
+      return conv_ws_launch(s, who, out, in, nullptr, bias, p, &handled);
+    }
+    return MCN_SUCCESS;
+  }
+  if (p.addend && !(ut && p.Cout > 4)) return fail(MCN_UNSUPPORTED, "%s: this product cannot add a masked second term in its epilogue", who);
   // The backward-data product of a 1x1 bank whose extents need no padding reads it as it is stored: rows = filters,
   // columns = the filters' channels, which is the packed order.
   const bool asStored = backward && taps.FH * taps.FW == 1 && rPad == p.R && p.coutPad == p.Cout && aligned16(f);
@@ -964,6 +977,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
     if (rc || handled) return rc;
   }
   if (p.stats) return fail(MCN_UNSUPPORTED, "%s: this product cannot sum its output per channel", who);
+  if (p.addend) return fail(MCN_UNSUPPORTED, "%s: this product cannot add a masked second term in its epilogue", who);
   // banks too large for LDS: stream them past pixels held in registers (conv_sb.hip)
   if (sb && sbSplits == 1) {
     rc = conv_sb_launch(s, out, in, wt, bias, p, 1);
@@ -1155,8 +1169,11 @@ int conv_forward_mfma(hipStream_t s, const ConvP& original, float* y, float outM
 // with a subset of the taps.  Classes no tap reaches (1x1 filters with stride 2: three of four) are zeros.
 namespace {
 int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float dxMult, const float* f, const float* dy,
-                        void* ws, size_t wsBytes, PackCtx* pk) {
+                        void* ws, size_t wsBytes, PackCtx* pk, const float* addend, const unsigned* addBits, int* addQuery) {
   PixP q;
+  q.addend = addend;
+  q.addBits = addBits;
+  q.addQuery = addQuery;
   q.IH = p.outH; q.IW = p.outW; q.Cin = p.K;
   q.N = p.N;
   q.Cout = p.C;
@@ -1202,8 +1219,19 @@ int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float
 }  // namespace
 
 int conv_backward_data_mfma(hipStream_t s, const ConvP& original, float* dx, float dxMult, const float* f, const float* dy,
-                            void* ws, size_t wsBytes, PackCtx* pk) {
+                            void* ws, size_t wsBytes, PackCtx* pk, const float* addend, const unsigned* addBits, int* addQuery) {
   const ConvP p = fc_view(original);
+  if (addend || addQuery) {
+    // the masked second term: one product over the whole tensor (no filter groups, no stride classes)
+    if (p.groups != 1 || p.sy != 1 || p.sx != 1 || dxMult != 0.f) {
+      if (addQuery) {
+        *addQuery = 0;
+        return MCN_SUCCESS;
+      }
+      return fail(MCN_UNSUPPORTED, "mcn_conv_backward_data_masked_add: not available for this geometry");
+    }
+    return backward_data_group(s, group_view(p), wide_of(p), dx, 0.f, f, dy, ws, wsBytes, pk, addend, addBits, addQuery);
+  }
   const bool compute = !pk || pk->mode == PackCtx::kUse;
   // stride classes no tap reaches get no launch: they are zeros (or keep what is there, when accumulating)
   bool anyEmpty = false;
@@ -1221,7 +1249,7 @@ int conv_backward_data_mfma(hipStream_t s, const ConvP& original, float* dx, flo
   const Wide wd = wide_of(p);
   const size_t FV = (size_t)p.FH * p.FW * p.FC, Q = (size_t)p.outH * p.outW, HW = (size_t)p.H * p.W;
   for (int i = 0; i < p.groups; ++i) {
-    int rc = backward_data_group(s, g, wd, dx + i * p.FC * HW, dxMult, f + i * p.Kg * FV, dy + i * p.Kg * Q, ws, wsBytes, pk);
+    int rc = backward_data_group(s, g, wd, dx + i * p.FC * HW, dxMult, f + i * p.Kg * FV, dy + i * p.Kg * Q, ws, wsBytes, pk, nullptr, nullptr, nullptr);
     if (rc) return rc;
   }
   return MCN_SUCCESS;

@@ -62,11 +62,14 @@ __device__ __forceinline__ float row_sum16(float v) {
   return v;
 }
 
-template <int WA, bool TAPS, int THREADS, bool STATS = false>
+// ADD (no bias, alpha = 1, beta = 0, whole channel blocks only): the epilogue adds a second term from another tensor,
+// gated by one bit per element (PixP::addend, store_block_masked_add).
+template <int WA, bool TAPS, int THREADS, bool STATS = false, bool ADD = false>
 __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out, const float* __restrict__ in,
                                                         const float* __restrict__ wt, const float* __restrict__ bias,
                                                         PixP p, WsP w) {
   static_assert(!STATS || WA == 1, "channel sums are kept for one 32-channel block per wavefront");
+  static_assert(!(STATS && ADD), "one extra at a time");
   extern __shared__ float smem[];
   float* wtL = smem;  // [chanBlocks][R][32 WA]
   constexpr int ROW = 32 * WA;                     // floats per bank row of one channel block
@@ -308,10 +311,16 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
       int n, q;
       p.byQ.divmod(mo < p.M ? mo : 0, &n, &q);
       const unsigned vo = mo < p.M ? (unsigned)(n * p.outImg + out_pixel_offset(p, q) + 4 * kh * p.outPlane) * 4u : kOutside;
+      if (ADD) {
+        const bufrsrc arsrc = make_bufrsrc(p.addend, p.outBytes), brsrc = make_bufrsrc(p.addBits, p.outBytes >> 5);
 #pragma unroll
-      for (int a = 0; a < WA; ++a)
-        store_block(acc[a], orsrc, vo, (cbOut * ROW + a * 32) * plane, plane, p.alpha, p.beta,
-                    bias ? bias + cbOut * ROW + a * 32 : nullptr, kh);
+        for (int a = 0; a < WA; ++a) store_block_masked_add(acc[a], orsrc, arsrc, brsrc, vo, (cbOut * ROW + a * 32) * plane, plane);
+      } else {
+#pragma unroll
+        for (int a = 0; a < WA; ++a)
+          store_block(acc[a], orsrc, vo, (cbOut * ROW + a * 32) * plane, plane, p.alpha, p.beta,
+                      bias ? bias + cbOut * ROW + a * 32 : nullptr, kh);
+      }
       if (STATS) {
         // what was stored is the accumulator itself (alpha = 1; lanes past the last pixel hold zeros: their loads
         // fetched nothing)
@@ -355,7 +364,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
 #undef WS_LOAD_NEXT
 }
 
-template <int WA, bool TAPS, int THREADS, bool STATS = false>
+template <int WA, bool TAPS, int THREADS, bool STATS = false, bool ADD = false>
 int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, const float* in, const float* wt,
            const float* bias, const PixP& p, const WsP& w) {
   // largest dynamic LDS size this instantiation has been opted into, per device (concurrent callers may both opt in:
@@ -363,7 +372,7 @@ int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, c
   static std::atomic<size_t> raised[kMaxDevices];
   const int dev = current_device();
   if (lds > 64 * 1024 && (dev < 0 || dev >= kMaxDevices || lds > raised[dev].load(std::memory_order_acquire))) {
-    if (hipFuncSetAttribute((const void*)conv_ws_mfma<WA, TAPS, THREADS, STATS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)conv_ws_mfma<WA, TAPS, THREADS, STATS, ADD>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return fail(MCN_DEVICE_ERROR, "%s: cannot reserve %zu bytes of LDS", who, lds);
@@ -375,7 +384,7 @@ int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, c
     }
   }
   KernelTimer timer("conv_ws_mfma", s);
-  hipLaunchKernelGGL((conv_ws_mfma<WA, TAPS, THREADS, STATS>), dim3((unsigned)blocks), dim3(THREADS), lds, s, out, in, wt, bias, p, w);
+  hipLaunchKernelGGL((conv_ws_mfma<WA, TAPS, THREADS, STATS, ADD>), dim3((unsigned)blocks), dim3(THREADS), lds, s, out, in, wt, bias, p, w);
   return check_launch(who);
 }
 
@@ -384,6 +393,11 @@ int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, c
 template <int WA, bool TAPS>
 int dispatch(hipStream_t s, const char* who, int cus, bool twoFit, size_t lds, float* out, const float* in, const float* wt,
              const float* bias, const PixP& p, const WsP& w) {
+  if (p.addend) {
+    if constexpr (WA == 4) return launch<WA, TAPS, 512, false, true>(s, who, cus, lds, out, in, wt, bias, p, w);
+    else if (twoFit) return launch<WA, TAPS, 512, false, true>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
+    else return launch<WA, TAPS, 1024, false, true>(s, who, cus, lds, out, in, wt, bias, p, w);
+  }
   if constexpr (WA == 4) {
     return launch<WA, TAPS, 512>(s, who, cus, lds, out, in, wt, bias, p, w);
   } else if constexpr (WA == 1) {
@@ -509,6 +523,18 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
   if (!plan_ws(p, wantStats, &plan) || (wantStats && (bias || plan.statGroups != p.statGroups))) {
     if (wantStats) return fail(MCN_UNSUPPORTED, "%s: this product cannot sum its output per channel", who);
     return MCN_SUCCESS;
+  }
+  if (p.addend || p.addQuery) {
+    // the second term of the epilogue: dense whole 32-channel blocks of a tensor a buffer descriptor covers, planes of
+    // whole 32-bit mask words
+    const bool fits = !wantStats && !bias && p.alpha == 1.f && p.beta == 0.f && p.dense && p.outBytes != 0 && p.Cout % 32 == 0 &&
+                      p.Cout == p.coutPad && p.outPlane % 32 == 0 && p.outImg % 32 == 0 && (p.addQuery || p.addBits);
+    if (p.addQuery) {
+      *p.addQuery = fits ? 1 : 0;
+      *handled = 1;
+      return MCN_SUCCESS;
+    }
+    if (!fits) return fail(MCN_UNSUPPORTED, "%s: this product cannot add a masked second term in its epilogue", who);
   }
   const int WA = plan.WA, cus = plan.cus;
   const bool twoFit = plan.twoFit;

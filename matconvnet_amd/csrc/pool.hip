@@ -109,6 +109,28 @@ __global__ __launch_bounds__(256) void pool_avg_backward_whole(float* __restrict
   dx[i] = (accumulate ? dx[i] : 0.0f) + v;  // (0 + v, as the general kernels' sum starts: -0 becomes +0)
 }
 
+// Average pooling whose windows tile the plane exactly (pool = stride, no padding, H = outH * poolH, W = outW *
+// poolW; H a multiple of 4): every input element lies in exactly one whole window, dx = [dx +] dy[its window] * (1 /
+// (poolH * poolW)).  One thread per 16 bytes of dx, in memory order: a plain streaming kernel (reads dzdy once -- the
+// poolH * poolW threads that share a window hit L1 -- and writes dx once).
+__global__ __launch_bounds__(256) void pool_backward_avg_tiles(float* __restrict__ dx, const float* __restrict__ dy, unsigned total4,
+                                                               int H4, int W, int outH, int outW, FastDiv byH4, FastDiv byW,
+                                                               FastDiv byPh, FastDiv byPw, int poolArea, int accumulate) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= total4) return;
+  int col, q, plane, w;
+  byH4.divmod((int)i, &col, &q);     // i = (plane * W + w) * H4 + q
+  byW.divmod(col, &plane, &w);
+  const float scale = 1.0f / (float)poolArea;  // as avg_scale: correctly rounded IEEE division
+  const float* src = dy + ((size_t)plane * outW + byPw.div(w)) * outH;
+  float v[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) v[r] = src[byPh.div(4 * q + r)] * scale;
+  float4 old = make_float4(0.f, 0.f, 0.f, 0.f);  // (0 + v, as the general kernels' sum starts: -0 becomes +0)
+  if (accumulate) old = ((const float4*)dx)[i];
+  stream_store4((float4*)dx + i, make_float4(old.x + v[0], old.y + v[1], old.z + v[2], old.w + v[3]));
+}
+
 // KH, KW: upper bounds on the number of output rows / columns covering one input element
 // (ceil(pool/stride)); 0 selects run-time loops.  With compile-time bounds the candidate loads are issued
 // together and the adds are predicated, which keeps the reference's addition order.
@@ -979,6 +1001,16 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
     KernelTimer timer("pool_avg_backward_whole", s);
     hipLaunchKernelGGL(pool_avg_backward_whole, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, derInput, derOutput,
                        (unsigned)total, (unsigned)(p.H * p.W), p.accumulate);
+    return check_launch("mcn_pool_backward");
+  }
+
+  // ---- average over windows that tile the plane exactly: one streaming pass in memory order
+  if (!isMax && p.poolH == p.sy && p.poolW == p.sx && p.pt == 0 && p.pl == 0 && p.H == p.outH * p.poolH && p.W == p.outW * p.poolW &&
+      vecIn && total / 4 < (1ull << 31) && !tunable("pool_force_gather", 0) && !tunable("pool_no_tiles", 0)) {
+    KernelTimer timer("pool_backward_avg_tiles", s);
+    hipLaunchKernelGGL(pool_backward_avg_tiles, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, s, derInput, derOutput,
+                       (unsigned)(total / 4), p.H / 4, p.W, p.outH, p.outW, FastDiv(p.H / 4), FastDiv(p.W), FastDiv(p.poolH),
+                       FastDiv(p.poolW), p.poolH * p.poolW, p.accumulate);
     return check_launch("mcn_pool_backward");
   }
 

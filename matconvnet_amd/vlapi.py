@@ -82,11 +82,14 @@ def lib():
         L.vlh_resnet50_set_test_mode.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_test_mode.restype = None
         L.vlh_resnet50_set_deferred.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_resnet50_set_channel_sums.argtypes = [C.c_void_p, C.c_int]
         L.vlh_bottleneck_set_deferred.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_packed.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_pack.argtypes = [C.c_void_p]
         L.vlh_bottleneck_set_packed.argtypes = [C.c_void_p, C.c_int]
         L.vlh_bottleneck_set_epilogue_sums.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_bottleneck_set_mask_bits.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_bottleneck_mask_bits_on.argtypes = [C.c_void_p]
         L.vlh_bottleneck_pack.argtypes = [C.c_void_p]
         L.vlh_resnet50_init.argtypes = [C.c_void_p, C.c_ulonglong]
         L.vlh_resnet50_forward.argtypes = [C.c_void_p]
@@ -265,7 +268,8 @@ class ResNet50(_NamedBuffers):
     the loss layers); buffers are owned by the C++ side and named "input", "prediction", "dprediction",
     "stem.f", "fc.f", "unit<i>.<name>", ..."""
 
-    def __init__(self, N=32, eps=1e-5, image_size=224, classes=1000, fused=True, seed=None, packed=True, deferred=False):
+    def __init__(self, N=32, eps=1e-5, image_size=224, classes=1000, fused=True, seed=None, packed=True, deferred=False,
+                 channel_sums=False):
         """packed: the convolutions read filter banks packed ahead, refreshed in one launch after every update (and by
         `set` of a parameter here); False: every call packs its own, as the plain operator calls do.
         deferred: the sums that finish the filter gradients run in one launch at the end of backward (off by
@@ -287,6 +291,10 @@ class ResNet50(_NamedBuffers):
             self.packed = True
         if deferred:
             self._check(self.L.vlh_resnet50_set_deferred(self.h, 1))
+        if channel_sums:
+            # (folded mode: the convolutions sum their output per channel for batch normalisation, identity units keep
+            # their last ReLU's mask as bits, wherever the shapes allow; moments equal to rounding, not bit for bit)
+            self._check(self.L.vlh_resnet50_set_channel_sums(self.h, 1))
         if seed is not None:
             self._check(self.L.vlh_resnet50_init(self.h, seed))
 
@@ -369,7 +377,7 @@ class Bottleneck(_NamedBuffers):
     """The ResNet-50 bottleneck block of the C++ harness (buffers owned by the C++ side)."""
 
     def __init__(self, H=56, W=56, Cc=256, M=64, N=32, eps=1e-5, fused=False, overlap=False, Cout=0, stride=1,
-                 adapter=False, packed=False, deferred=False, epilogue_sums=False):
+                 adapter=False, packed=False, deferred=False, epilogue_sums=False, mask_bits=False):
         """packed: the convolutions read filter banks packed ahead; `set` of a filter and every step of `run` refresh
         them with one launch (`pack`).  deferred: one launch at the end of backward sums the reduction splits of all
         the unit's filter gradients."""
@@ -390,6 +398,12 @@ class Bottleneck(_NamedBuffers):
         if epilogue_sums:
             # (fused mode: the forward convolutions sum their output per channel, batch normalisation takes the sums)
             self._check(self.L.vlh_bottleneck_set_epilogue_sums(self.h, 1))
+        self.mask_bits = False
+        if mask_bits:
+            # (with epilogue_sums, identity shortcut: the last ReLU's mask kept as one bit per element for backward;
+            # stays off where the shapes have no such form)
+            self._check(self.L.vlh_bottleneck_set_mask_bits(self.h, 1))
+            self.mask_bits = bool(self.L.vlh_bottleneck_mask_bits_on(self.h))
 
     def set(self, name, array):
         super().set(name, array)

@@ -197,3 +197,37 @@ def test_small_channels_in_one_launch_give_the_same_bits(capi, shape):
     assert len(outs[0]) == len(outs[1]) and len(outs[0]) >= 20
     for a, b_ in zip(*outs):
         assert bits_equal(a, b_)
+
+
+def test_relu_mask_as_bits_matches_the_float_mask_paths(capi, ob):
+    """The residual unit's last ReLU with its mask kept as one bit per element: the forward pass that writes the bits
+    gives the same y and moments as the one that does not, the bits say y > 0 element by element, and the batch-norm
+    derivative that reads them is bit-identical to the one that reads the ReLU's output (mcn_bnorm_backward_masked)."""
+    import torch
+    from util import bits_equal
+    H, W, Cc, N = 56, 56, 32, 6
+    assert capi.lib().mcn_bnorm_mask_bits_supported(H, W, Cc, N) == 1
+    assert capi.lib().mcn_bnorm_mask_bits_supported(14, 14, Cc, N) == 0      # planes of 196 elements: not whole words
+    r = np.random.default_rng(21)
+    x = capi.to_device(F(r.standard_normal((H, W, Cc, N)) * 1.5 + 0.2))
+    res = capi.to_device(F(r.standard_normal((H, W, Cc, N))))
+    dy = capi.to_device(F(r.standard_normal((H, W, Cc, N))))
+    g = capi.to_device(F(r.uniform(0.5, 1.5, Cc)).ravel())
+    b = capi.to_device(F(r.standard_normal(Cc) * 0.1).ravel())
+    # partial sums in the layout a summing convolution leaves them: [channel][group][2]
+    xd = x.double()
+    groups = 3
+    cuts = [0, 2, 4, N]
+    sums = torch.stack([torch.stack([xd[cuts[k]:cuts[k + 1]].sum(dim=(0, 2, 3)), (xd[cuts[k]:cuts[k + 1]] ** 2).sum(dim=(0, 2, 3))], dim=1)
+                        for k in range(groups)], dim=1).contiguous()
+    y0, m0 = capi.bnorm_forward_sums(x, g, b, sums, residual=res, relu=True, eps=1e-5)
+    y1, bits, m1 = capi.bnorm_forward_sums_mask(x, g, b, sums, residual=res, eps=1e-5)
+    assert torch.equal(y0, y1) and torch.equal(m0, m1)
+    want = (y1.reshape(-1) > 0).to(torch.int64).reshape(-1, 32)
+    weights = (1 << torch.arange(32, device="cuda", dtype=torch.int64))
+    words = (want * weights).sum(dim=1)
+    assert torch.equal(words, bits.to(torch.int64) & 0xffffffff)
+    got = capi.bnorm_backward_bits(x, g, dy, bits, m1, eps=1e-5)
+    ref = capi.bnorm_backward_masked(x, g, dy, y1, m1, eps=1e-5)
+    for a, c in zip(got, ref[:3]):
+        assert bits_equal(capi.to_host(a), capi.to_host(c))

@@ -636,3 +636,28 @@ def test_conv_forward_with_channel_sums_refuses_what_it_cannot_do(capi):
     with pytest.raises(capi.McnError) as e:
         capi.conv_forward_sums(x, f, g)
     assert "no such form" in str(e.value)
+
+
+def test_conv_backward_data_with_masked_second_term(capi):
+    """dzdx = backward-data + the shortcut's share of the derivative behind a ReLU, the mask as one bit per element:
+    bit-identical to writing the masked derivative into dzdx and accumulating the convolution's onto it."""
+    import torch
+    from util import bits_equal
+    r = np.random.default_rng(8)
+    xs, fs = (56, 56, 256, 4), (1, 1, 256, 64)
+    g = capi.conv_geom(xs, fs, 1, 0, 1)
+    assert capi.lib().mcn_conv_backward_data_masked_add_supported(g) == 1
+    f = capi.to_device(F(r.standard_normal(fs) * 0.1))
+    dy = capi.to_device(F(r.standard_normal((56, 56, 64, 4))))
+    addend = capi.to_device(F(r.standard_normal(xs)))
+    y = capi.to_device(F(r.standard_normal(xs)))   # the ReLU's output stands in for "what it let through"
+    keep = (y.reshape(-1) > 0).to(torch.int64).reshape(-1, 32)
+    words = (keep * (1 << torch.arange(32, device="cuda", dtype=torch.int64))).sum(dim=1)
+    bits = torch.where(words >= (1 << 31), words - (1 << 32), words).to(torch.int32)
+    want = capi.relu_backward(y, addend)            # addend where y > 0, else addend*0
+    want = capi.conv_backward_data_acc(want, 1.0, f, dy, g)
+    got = capi.conv_backward_data_masked_add(f, dy, g, addend, bits)
+    assert bits_equal(capi.to_host(got), capi.to_host(want))
+    # a geometry without this form says so
+    g2 = capi.conv_geom((9, 9, 5, 2), (3, 3, 5, 7), 1, 1, 1)
+    assert capi.lib().mcn_conv_backward_data_masked_add_supported(g2) == 0

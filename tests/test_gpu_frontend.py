@@ -448,3 +448,34 @@ def test_block_with_channel_sums_against_the_oracle(vl, ob):
     want = _oracle_bottleneck(ob, w, np.float64)
     errs = {k: rel_max(got[k], want[k]) for k in shapes}
     assert max(errs.values()) < 5e-4, errs
+
+
+def test_block_with_the_last_relu_mask_kept_as_bits(vl, ob):
+    """The benchmarked schedule with the unit's last ReLU mask kept as one bit per element (backward reads 3 MB of bits
+    instead of the 103 MB output; the shortcut's share of the derivative is added in the epilogue of the first
+    convolution's input gradient) against the same schedule without: every output bit for bit, at the benchmarked
+    size, two steps."""
+    N = 32
+    w = workloads.bottleneck_case()
+    shapes = dict(y=w["x"].shape, dzdx=w["x"].shape, df1=w["f1"].shape, df2=w["f2"].shape, df3=w["f3"].shape,
+                  dg1=(64,), db1=(64,), dg2=(64,), db2=(64,), dg3=(256,), db3=(256,), m1=(64, 2), m2=(64, 2), m3=(256, 2))
+    outs = {}
+    for bits in (False, True):
+        blk = vl.Bottleneck(N=N, eps=w["eps"], fused=True, packed=True, deferred=True, epilogue_sums=True, mask_bits=bits)
+        try:
+            assert blk.mask_bits == bits          # (this shape has the form: 56x56 planes are whole mask words)
+            _load(blk, w)
+            blk.run(2)
+            torch.cuda.synchronize()
+            outs[bits] = {k: blk.get(k, v) for k, v in shapes.items()}
+        finally:
+            blk.close()
+    for k in shapes:
+        assert np.isfinite(outs[True][k]).all(), k
+        assert bits_equal(outs[False][k], outs[True][k]), k
+    # a unit whose planes are not whole mask words keeps the float mask, silently
+    blk = vl.Bottleneck(H=14, W=14, Cc=256, M=64, N=4, eps=1e-5, fused=True, packed=True, deferred=True, epilogue_sums=True, mask_bits=True)
+    try:
+        assert blk.mask_bits is False
+    finally:
+        blk.close()

@@ -384,3 +384,50 @@ def test_loss_layers_and_a_few_training_steps(vl, case):
         assert np.isfinite(last) and last < 0.3 * first, (first, last)
     finally:
         net.close()
+
+
+def test_channel_sums_schedule_of_the_whole_network(vl):
+    """The network with the forward convolutions summing their own output per channel and the identity units keeping
+    their last ReLU's mask as bits (ResNet50(channel_sums=True); engaged by the 56x56 units at this size).  Forward:
+    against the folded schedule without, to rounding (the moments come from another summation order).  Backward: the
+    whole network's gradients are not continuous in rounding error (see test_stage_by_stage_against_oracle), so the
+    second unit -- identity shortcut, 56x56: both forms engaged -- is checked on the tensors the network actually gave
+    it: a stand-alone layer-by-layer unit run on the network's input and incoming derivative of that unit must give
+    the network's outputs of that unit.  And two runs give the same bits."""
+    B = 8
+    w = workloads.resnet50_case(seed=4, image_size=224, N=B, classes=10)
+    names = ("prediction", "unit0.y", "unit1.y", "unit2.dzdx", "unit1.dzdx") + tuple("unit1.d" + k for k in UNIT_PARAMS)
+    outs = []
+    for kw in (dict(), dict(channel_sums=True), dict(channel_sums=True)):
+        net = vl.ResNet50(N=B, eps=w["eps"], image_size=224, classes=10, fused=True, **kw)
+        try:
+            _load(net, w)
+            net.forward()
+            net.backward()
+            outs.append({k: net.get(k) for k in names})
+        finally:
+            net.close()
+    plain, sums, again = outs
+    for k in names:
+        assert np.isfinite(sums[k]).all(), k
+        assert bits_equal(sums[k], again[k]), k
+    for k, gate in (("unit0.y", 1e-5), ("unit1.y", 1e-5), ("prediction", 1e-4)):   # (fifty layers later: 1e-5 measured)
+        assert rel_max(sums[k], plain[k]) < gate, (k, rel_max(sums[k], plain[k]))
+    u = w["units"][1]
+    assert not u["adapter"]
+    shape = (56, 56, 256, B)
+    blk = vl.Bottleneck(H=56, W=56, Cc=256, M=64, N=B, eps=w["eps"])
+    try:
+        blk.set("x", sums["unit0.y"].reshape(shape, order="F"))
+        blk.set("dzdy", sums["unit2.dzdx"].reshape(shape, order="F"))
+        for k in UNIT_PARAMS:
+            blk.set(k, u[k])
+        blk.forward()
+        blk.backward()
+        assert rel_max(blk.get("y", shape).ravel(order="F"), sums["unit1.y"].ravel(order="F")) < 1e-5
+        errs = {"dzdx": rel_max(blk.get("dzdx", shape).ravel(order="F"), sums["unit1.dzdx"].ravel(order="F"))}
+        for k in UNIT_PARAMS:
+            errs["d" + k] = rel_max(blk.get("d" + k, np.shape(u[k])).ravel(order="F"), sums["unit1.d" + k].ravel(order="F"))
+        assert max(errs.values()) < 2e-4, errs
+    finally:
+        blk.close()
