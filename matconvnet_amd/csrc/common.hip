@@ -22,13 +22,14 @@ struct Tunable {
 };
 // Defaults are the values chosen from on-device sweeps; see the per-kernel comments where each is read.
 Tunable g_tunables[] = {
+    {"conv_wgrad_wide_rows_exact", 1}, // 192-row filter-gradient tiles for volumes they cover exactly and 128-row tiles do not
     {"conv_no_sb", 0},                 // 1: the streamed-bank kernel is not used (banks too large for LDS go to the tiled kernel)
     {"conv_sb_split", 0},              // 0: the streamed-bank kernel leaves products whose reduction it would split to the tiled kernel
-                                       // (3x3x256x256 on 14x14x256x32: 87 us tiled, 104 us here in 8 splits)
+                                       // (on their own, warm, the split products win 8-11% at 32 images; inside ResNet-50 the step loses 0.17 ms)
     {"conv_sb_slab", 32},              // reduction rows per slab of the bank in LDS (32 or 64) of the streamed-bank kernel
     {"conv_sb_occupancy", 2},          // wavefronts per SIMD the 128-channel streamed-bank kernel's registers are cut for (2 or 3)
-    {"conv_sb_fill", 3},               // workgroups per compute unit below which the streamed-bank kernel splits the reduction
-    {"conv_sb_min_pairs", 3},          // least pairs of 32-row slabs per split of the streamed-bank kernel
+    {"conv_sb_fill", 2},               // workgroups per compute unit below which the streamed-bank kernel splits the reduction
+    {"conv_sb_min_pairs", 6},          // least pairs of 32-row slabs per split of the streamed-bank kernel
     {"pool_lds_bytes", 16 * 1024},     // LDS tile budget of the pooling-backward kernels
     {"pool_no_stream", 0},             // 1: max pooling skips the streaming kernel
     {"pool_walk", 3},                  // streaming kernel's tile order: 0 round-robin, 1 contiguous runs, 2 round-robin per XCD eighth, 3 planes round-robin over XCDs

@@ -763,6 +763,9 @@ int pick_rows_tile(const ConvP& p) {
   const int FV = p.FH * p.FW * p.FC, BA = pick_channels_tile(p.K);
   if (FV <= 64 && BA >= 64) return 64;
   if (FV > 128 && FV <= 192 && BA == 64 && !tunable("conv_wgrad_no_wide_rows", 0)) return 192;
+  // a volume that 192-row tiles cover exactly and 128-row tiles do not (3x3x64 = 576 rows: three tiles instead of
+  // four and a half, and 48 instead of 32 MFMAs per wavefront between two barriers)
+  if (FV % 192 == 0 && FV % 128 != 0 && BA == 64 && tunable("conv_wgrad_wide_rows_exact", 1)) return 192;
   return 128;
 }
 

@@ -274,19 +274,24 @@ int conv_sb_splits(int Cout, long long M, int R) {
   if ((long long)R * coutPad * 4 >= (long long)kOutside) return 0;
   const long long tiles = ((M + 127) / 128) * (coutPad / BA);
   if (tiles >= (1ll << 30)) return 0;
-  // a long reduction over few tiles is split so that the launch fills the chip (three workgroups per compute unit)
+  // A long reduction over few tiles is split so that the launch fills the chip: two workgroups per compute unit, at
+  // least six pairs of slabs each.  Measured against the tiled kernel's own split reduction, forward, 32 images:
+  // 3x3x256x256 on 14x14: 99 -> 92 us, 3x3x512x512 on 7x7: 104 -> 93 us; with 64 images (196 tiles and more) the tiled
+  // kernel is the faster one (155 against 160 us), so products with more than half a tile per compute unit are left
+  // to it.  Inside the whole network (cold caches, the partial tensors' extra traffic) the split form loses: a ResNet-50
+  // training step at 32 images went 12.73 -> 12.90 ms, so it is off unless asked for (conv_sb_split).
   int cus = device_compute_units();
   if (cus <= 0) cus = 256;
   const int pairs = R / (2 * slab_rows(R));  // pairs of slabs: the unit a split is made of
-  const long long want = (long long)cus * std::max(1, tunable("conv_sb_fill", 3));
+  const long long want = (long long)cus * std::max(1, tunable("conv_sb_fill", 2));
   int s = 1;
   if (tiles < want) {
-    const int minPairs = std::max(1, tunable("conv_sb_min_pairs", 3));
+    const int minPairs = std::max(1, tunable("conv_sb_min_pairs", 6));
     s = (int)std::min<long long>((want + tiles - 1) / tiles, std::max(1, pairs / minPairs));
     const int per = (pairs + s - 1) / s;
     s = (pairs + per - 1) / per;
   }
-  if (s > 1 && !tunable("conv_sb_split", 0)) return 0;
+  if (s > 1 && (!tunable("conv_sb_split", 0) || 2 * tiles > cus)) return 0;
   return s;
 }
 

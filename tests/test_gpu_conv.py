@@ -35,6 +35,8 @@ CASES = [
     (6, 6, 32, 8, 6, 6, 32, 200, 1, 0, 1),                   # fully connected, 1152 rows: forward splits the reduction
     (4, 4, 16, 4, 4, 4, 16, 640, 1, 0, 1),                   # fully connected, 640 filters: backward-data splits it
     (13, 13, 2, 3, 13, 13, 2, 5, 1, 0, 1),                   # fully connected with 169 taps: only the 1x1 view fits the MFMA kernels
+    (20, 22, 64, 3, 3, 3, 64, 64, 1, 1, 1),                  # 576-row filter volume, 64 filters: 192-row filter-gradient tiles
+    (12, 12, 64, 2, 3, 3, 64, 40, (2, 1), (1, 0, 1, 1), 1),  # the same volume with a partial filter tile, strided
 ]
 
 
