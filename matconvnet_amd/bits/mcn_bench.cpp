@@ -3,7 +3,7 @@
 // synthetic inputs, times them with HIP events and prints TFLOP/s, GB/s and images/s beside the
 // fraction of the MI355X rooflines (fp32 matrix 157.3 TFLOP/s, HBM 8 TB/s).
 //
-//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...
+//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|blocktimed|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...
 //
 // The bandwidth-bound operators (bnorm, pooling, copy) are timed over R independent sets of tensors used in
 // turn (default 4), so that no launch finds its inputs in the 256 MB memory-side cache because the previous
@@ -237,7 +237,9 @@ static void benchYardstick(int warmup, int iters, int fixed) {
     if (best[mode].gbs > 0) std::printf("best %s\n", best[mode].text);
 }
 
-static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, bool packed = false) {
+// sums: (with packed) the forward convolutions sum their output per channel and the last ReLU's mask is kept as bits:
+// the schedule bench.py times
+static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, bool packed = false, bool sums = false) {
   const int H = 56, W = 56, C = 256, M = 64, N = 32;
   harness::Bottleneck block(H, W, C, M, N, 1e-5);
   block.setFused(fused);
@@ -266,6 +268,10 @@ static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, 
     std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
     std::exit(3);
   }
+  if (sums && (block.setEpilogueSums(true) != VLE_Success || block.setMaskBits(true) != VLE_Success)) {
+    std::fprintf(stderr, "bottleneck: %s\n", block.lastMessage().c_str());
+    std::exit(3);
+  }
   double t = medianMs([&] {
     // (packed: the banks are re-packed every step, as they would be after an update of the filters: one launch)
     if (block.pack() != VLE_Success || block.forward() != VLE_Success || block.backward() != VLE_Success) {
@@ -274,7 +280,8 @@ static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, 
     }
   }, warmup, iters);
   std::printf("%-28s %8.3f ms/step %9.0f images/s (fwd+bwd, N = %d, 41.93 GFLOP of convolution per step; %s)\n",
-              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, packed ? "folded, filter banks packed by one launch per step, filter gradients summed by one"
+              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, sums ? "folded, banks packed by one launch, filter gradients summed by one, channel sums from the convolutions, last mask as bits"
+                     : packed ? "folded, filter banks packed by one launch per step, filter gradients summed by one"
                      : (overlap ? "folded, filter gradients on a second stream" : (fused ? "relu/sum folded into bnorm" : "layer by layer")));
 }
 
@@ -288,7 +295,7 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
   }
   net.setFused(fused);
   // (the folded run also packs the filter banks ahead, once per update)
-  if (fused && net.setPacked(true) != VLE_Success) {
+  if (fused && (net.setPacked(true) != VLE_Success || net.setChannelSums(true) != VLE_Success)) {
     std::fprintf(stderr, "resnet-50: %s\n", net.lastMessage().c_str());
     std::exit(3);
   }
@@ -346,7 +353,7 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
               "%8.2f ms training step (with the loss derivative and the SGD update of %.1f M parameters) %8.0f images/s "
               "(N = %d, %.2f GFLOP of convolution per image forward; %s)\n",
               "resnet-50 224x224", tf, N / (tf * 1e-3), gf * N / tf, t, N / (t * 1e-3), 3 * gf * N / t, ts,
-              net.numParameters() * 1e-6, N / (ts * 1e-3), N, gf, fused ? "relu/sum folded into bnorm, filter banks packed once per update" : "layer by layer");
+              net.numParameters() * 1e-6, N / (ts * 1e-3), N, gf, fused ? "relu/sum folded into bnorm, filter banks packed once per update, channel sums from the convolutions and mask bits where the shapes allow" : "layer by layer");
 }
 
 int main(int argc, char** argv) {
@@ -369,7 +376,7 @@ int main(int argc, char** argv) {
       }
     }
     else {
-      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...\n");
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|blocktimed|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...\n");
       return 1;
     }
   }
@@ -392,7 +399,9 @@ int main(int argc, char** argv) {
     benchBlock(warmup, iters, true);
     benchBlock(warmup, iters, true, true);
     benchBlock(warmup, iters, true, false, true);
+    benchBlock(warmup, iters, true, false, true, true);
   }
+  if (only == "blocktimed") benchBlock(warmup, iters, true, false, true, true);
   if (want("conv5")) benchConv("conv 3x3x256x256 56x56 N=64", 56, 56, 256, 64, 3, 256, 1, warmup, iters);
   return 0;
 }
