@@ -318,11 +318,19 @@ ErrorCode ResNet50::setPacked(bool on) {
 ErrorCode ResNet50::setChannelSums(bool on) {
   if (error != VLE_Success) return error;
   dropGraph();
-  for (std::size_t i = 0; i < units.size(); ++i)
+  for (std::size_t i = 0; i < units.size(); ++i) {
     if (units[i]->setEpilogueSums(on) != VLE_Success || units[i]->setMaskBits(on) != VLE_Success) {
       message = units[i]->lastMessage();
       return VLE_OutOfGPUMemeory;
     }
+    // Only units that can also keep their mask as bits take the sums from their convolutions: elsewhere the summing
+    // convolution (one 32-channel block per wavefront, whole banks only) costs the forward pass more than the saved
+    // summing launches give back (forward 4.09 -> 4.28 ms at 32 images with all units, 7.53 -> 7.88 ms at 64).
+    if (on && !units[i]->maskBitsOn() && units[i]->setEpilogueSums(false) != VLE_Success) {
+      message = units[i]->lastMessage();
+      return VLE_OutOfGPUMemeory;
+    }
+  }
   return VLE_Success;
 }
 

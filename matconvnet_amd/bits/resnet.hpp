@@ -50,10 +50,10 @@ class ResNet50 {
   // deferred = true: backward() runs the matrix kernels of all filter gradients and sums their reduction splits in ONE
   // launch at its end instead of one per layer.  Same bits.
   ErrorCode setDeferred(bool on);
-  // channel sums = true (folded mode, training): in every unit the forward convolutions sum their own output per
-  // channel for the batch normalisation that follows, and units with an identity shortcut keep their last ReLU's mask
-  // as one bit per element, wherever the shapes have those forms (Bottleneck::setEpilogueSums, setMaskBits).  The
-  // moments then come from another summation order: same values to rounding, not the same bits.
+  // channel sums = true (folded mode, training): units with an identity shortcut whose planes are whole mask words
+  // (the 56x56 section) keep their last ReLU's mask as one bit per element, and their forward convolutions sum their
+  // own output per channel for the batch normalisation that follows (Bottleneck::setEpilogueSums, setMaskBits).  The
+  // moments of those units then come from another summation order: same values to rounding, not the same bits.
   ErrorCode setChannelSums(bool on);
   ErrorCode forward();
   ErrorCode backward();
