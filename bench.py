@@ -17,6 +17,7 @@ region.  `value` is images/s over exactly K steps.  The same line carries
   block_plain   the same block through the reference's operator interface only (layer by layer, no folded entry points),
   forward_rows  forward convolution / batch normalisation / pooling on the same shapes,
   latency_rows  BASELINE configs[0] (a 7 MB layer: a launch-latency case, not a roofline one),
+  double_rows   the untuned double-precision instantiation on reduced forms of the same configurations,
   hbm_ceiling   the best plain read / write / copy kernels of a small sweep, cold, timed in this run: every HBM-bound
                 row is also given as a fraction of that measured copy rate,
   cpu_baseline  the CPU restatement of the reference path (oracle/) timed on this machine's host cores: the block, and
@@ -483,6 +484,37 @@ def bench_conv_single(capi, workloads, reps):
     return rows, whole
 
 
+def bench_double(capi, workloads, reps):
+    """The double-precision instantiation (general one-accumulator-per-output kernels, no MFMA, no LDS: correct, not
+    tuned) on reduced forms of the graded configurations: measured so that its distance to the roofline is on record."""
+    import torch
+    rows = []
+    w = workloads.conv_single()
+    g = capi.conv_geom(w["x"].shape, w["f"].shape, w["stride"], w["pad"], w["dilate"])
+    x, f, dy = (capi.to_device(w[k], np.float64) for k in ("x", "f", "dy"))
+    flops = 3 * 2.0 * 32 * 32 * 100 * 75 * 32
+    t = _event_time(lambda: capi.conv_backward(x, f, dy, g), max(2, reps // 4), warm=1)
+    rows.append(dict(op="conv backward (dzdx, dzdf, dzdb), double", workload="configs[0] 5x5x3x32 on 32x32x3x100", call_us=t * 1e6,
+                     achieved=flops / t / 1e12, unit="TFLOP/s", peak=78.6, frac=flops / t / 78.6e12, bound="fp64 vector (no f64 MFMA used)"))
+    H, W, Cc, N = 56, 56, 256, 8
+    xb = torch.randn((N, Cc, W, H), device="cuda", dtype=torch.float64)
+    dyb = torch.randn((N, Cc, W, H), device="cuda", dtype=torch.float64)
+    gb = torch.rand(Cc, device="cuda", dtype=torch.float64) + 0.5
+    t = _event_time(lambda: capi.bnorm_backward(xb, gb, dyb, 1e-4), reps, warm=2)
+    nbytes = 5 * 8.0 * H * W * Cc * N
+    rows.append(dict(op="bnorm backward, double", workload="56x56x256x8 (configs[1] at a quarter of the batch)", call_us=t * 1e6,
+                     achieved=nbytes / t / 1e9, unit="GB/s", peak=PEAK_HBM / 1e9, frac=nbytes / t / PEAK_HBM, bound="hbm"))
+    shape = (112, 112, 64, 8)
+    gp = capi.pool_geom(shape, 3, 2, 1, "max")
+    xp = torch.randn(tuple(reversed(shape)), device="cuda", dtype=torch.float64)
+    dyp = torch.randn(tuple(reversed(capi.pool_out_shape(gp))), device="cuda", dtype=torch.float64)
+    t = _event_time(lambda: capi.pool_backward(xp, dyp, gp), reps, warm=2)
+    nbytes = 8.0 * (2 * np.prod(shape) + np.prod(capi.pool_out_shape(gp)))
+    rows.append(dict(op="max-pool backward, double", workload="112x112x64x8 (configs[2]a at a quarter of the batch)", call_us=t * 1e6,
+                     achieved=nbytes / t / 1e9, unit="GB/s", peak=PEAK_HBM / 1e9, frac=nbytes / t / PEAK_HBM, bound="hbm"))
+    return rows
+
+
 def bench_resnet50(vlapi, batch, steps, warmup):
     """Whole ResNet-50 (224 x 224, 1000 classes; examples/imagenet/cnn_imagenet_init_resnet.m) through the same
     operator classes: forward alone (training-mode batch normalisation), the training step forward + loss derivative
@@ -729,6 +761,7 @@ def main():
         "hbm_ceiling": ceiling,
         "forward_rows": forward_rows,
         "latency_rows": single_rows, "conv_single": single_whole,
+        "double_rows": bench_double(capi, workloads, max(4, args.steps // 2)),
         # beyond the headline block: the whole network the block comes from, per-image rates of whole training steps
         # (64 is the reference's own sub-batch for this network: batchSize 256 in 4 sub-batches,
         # examples/imagenet/cnn_imagenet_init_resnet.m:170-171)

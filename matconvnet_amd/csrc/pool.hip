@@ -825,12 +825,21 @@ __global__ __launch_bounds__(256) void pool_forward_quads(float* __restrict__ y,
     scan(acc, c, r0, n);
     return MAX ? acc : acc * (1.0f / (float)(n * (useA ? 3 : 2)));
   };
+  // The columns of the next pair of outputs are loaded before this pair is computed: twice the loads in flight per
+  // thread (the walk along the width is a chain of small dependent steps otherwise).
+  if (ow0 >= ow1) return;
+  float bn[ROWS], cn[ROWS];
   if (P3) {
     bool haveA = ow0 > 0;
     if (haveA) column(2 * ow0 - 1, a);
+    column(2 * ow0, b);
+    column(2 * ow0 + 1, c);
     for (int ow = ow0; ow < ow1; ++ow) {
-      column(2 * ow, b);
-      column(2 * ow + 1, c);
+      const bool more = ow + 1 < ow1;
+      if (more) {
+        column(2 * ow + 2, bn);
+        column(2 * ow + 3, cn);
+      }
       float2 r;
       // output row 2j: rows 4j-1 .. 4j+1 (without the first when it is above the plane); row 2j+1: rows 4j+1 .. 4j+3
       if (haveA) {
@@ -842,17 +851,31 @@ __global__ __launch_bounds__(256) void pool_forward_quads(float* __restrict__ y,
       }
       *(float2*)(yp + (size_t)ow * outH) = r;
 #pragma unroll
-      for (int k = 0; k < ROWS; ++k) a[k] = c[k];
+      for (int k = 0; k < ROWS; ++k) {
+        a[k] = c[k];
+        b[k] = bn[k];
+        c[k] = cn[k];
+      }
       haveA = true;
     }
   } else {
+    column(2 * ow0, b);
+    column(2 * ow0 + 1, c);
     for (int ow = ow0; ow < ow1; ++ow) {
-      column(2 * ow, b);
-      column(2 * ow + 1, c);
+      const bool more = ow + 1 < ow1;
+      if (more) {
+        column(2 * ow + 2, bn);
+        column(2 * ow + 3, cn);
+      }
       float2 r;
       r.x = output(false, 0, 2);
       r.y = output(false, 2, 2);
       *(float2*)(yp + (size_t)ow * outH) = r;
+#pragma unroll
+      for (int k = 0; k < ROWS; ++k) {
+        b[k] = bn[k];
+        c[k] = cn[k];
+      }
     }
   }
 }
