@@ -663,3 +663,41 @@ def test_conv_backward_data_with_masked_second_term(capi):
     # a geometry without this form says so
     g2 = capi.conv_geom((9, 9, 5, 2), (3, 3, 5, 7), 1, 1, 1)
     assert capi.lib().mcn_conv_backward_data_masked_add_supported(g2) == 0
+
+
+STREAMED = [  # H, W, C, N, FH, FW, FC, K, stride, pad, dilate: shapes the streamed-bank kernel takes when the others are off
+    (28, 28, 64, 4, 3, 3, 64, 128, 1, 1, 1),                 # 128-channel tiles, taps, padding
+    (20, 18, 128, 3, 1, 1, 128, 320, 1, 0, 1),               # no taps; 320 filters: a partial 128-channel tile at the end
+    (14, 14, 256, 4, 3, 3, 256, 256, 1, 1, 1),               # few tiles, long reduction: split into partial tensors
+    (16, 16, 64, 2, 3, 3, 64, 64, (2, 2), 1, 1),             # 64-channel tiles; strided: stride classes in backward-data
+    (12, 12, 128, 3, 3, 3, 128, 96, 1, (2, 0, 1, 1), (2, 1)),  # dilation, asymmetric padding, 96 filters in a 128 tile
+    (6, 6, 64, 8, 6, 6, 64, 200, 1, 0, 1),                   # fully connected: one pixel per image
+]
+
+
+@pytest.mark.parametrize("case", STREAMED)
+def test_streamed_bank_kernel_on_its_own(capi, ob, case):
+    """Forward and backward-data with the weights-stationary kernel switched off and the streamed-bank kernel's split
+    reduction on, so that conv_sb_mfma runs shapes the committed configurations would send elsewhere: against the
+    oracle at the convolution gate, and the launches are counted so that the test cannot pass on another kernel."""
+    H, W, C, N, FH, FW, FC, K, stride, pad, dilate = case
+    x, f, b = _tensors(case, seed=11)
+    g = capi.conv_geom(x.shape, f.shape, stride, pad, dilate)
+    og = ob.conv_geom(x.shape, f.shape, stride, pad, dilate)
+    want = ob.conv_forward(x, f, b, og)
+    dy = F(np.random.default_rng(12).standard_normal(want.shape))
+    wdx, _, _ = ob.conv_backward(x, f, dy, og, want=(True, False, False))
+    xd, fd, bd, dyd = capi.to_device(x), capi.to_device(f), capi.to_device(b), capi.to_device(dy)
+    capi.set_tunable("conv_no_ws", 1)
+    capi.set_tunable("conv_sb_split", 1)
+    try:
+        capi.profile_begin("conv_sb_mfma")
+        y = capi.to_host(capi.conv_forward(xd, fd, bd, g))
+        dx = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(True, False, False))[0])
+        launches, _ = capi.profile_end()
+    finally:
+        capi.set_tunable("conv_no_ws", 0)
+        capi.set_tunable("conv_sb_split", 0)
+    assert launches >= 1, launches   # (backward-data of 96 filters x 9 taps = 864 rows is not a multiple of 64: another kernel)
+    errs = dict(y=rel_max(y, want), dzdx=rel_max(dx, wdx))
+    assert max(errs.values()) <= TOL, errs
