@@ -81,6 +81,17 @@ def kernel_time(capi, kernel, launch, reps):
     return (ms / n) * 1e-3 if n else float("nan"), n
 
 
+def kernels_time_per_call(capi, pattern, launch, reps):
+    """Summed duration (s) per call of `launch` of every kernel whose name contains `pattern` (a product that takes
+    several launches), and their number per call."""
+    spin_up(launch)
+    capi.profile_begin(pattern)
+    for _ in range(reps):
+        launch()
+    n, ms = capi.profile_end()
+    return (ms / reps) * 1e-3 if n else float("nan"), n / reps
+
+
 def _load_block(blk, w):
     for k in ("x", "f1", "f2", "f3", "g1", "b1", "g2", "b2", "g3", "b3"):
         blk.set(k, w[k])
@@ -193,12 +204,16 @@ def bench_conv_bwd(capi, workloads, reps):
     for fn in (data, filt, bias):
         fn()
     _sync()
-    # backward-data goes to the streamed-bank kernel (conv_sb_mfma) when it takes the shape, else to the tiled one
+    # backward-data goes to the streamed-bank kernel when it takes the shape (conv_sb_mfma for the full rounds of
+    # resident workgroups, the same kernel once more for the left-over tiles with their reduction split, and
+    # conv_sb_tail_reduce: the row's time is the three together), else to the tiled one
     data_kernel = "conv_sb_mfma"
-    t_data, n_data = kernel_time(capi, data_kernel, data, reps)
+    t_data, n_data = kernels_time_per_call(capi, "conv_sb_", data, reps)
     if n_data == 0:
         data_kernel = "conv_pix_mfma"
         t_data, _ = kernel_time(capi, data_kernel, data, reps)
+    elif n_data > 1:
+        data_kernel = "conv_sb_mfma (%d launches: full rounds, left-over tiles split, their sum)" % round(n_data)
     t_filt, _ = kernel_time(capi, "conv_wgrad_mfma", filt, reps)
     t_red, _ = kernel_time(capi, "conv_wgrad_reduce", filt, reps)
     # whole backward call (all launches incl. weight packing, partial-sum reduction and bias), wall clock
@@ -212,7 +227,7 @@ def bench_conv_bwd(capi, workloads, reps):
     for name, kern, t in (("conv backward-data", data_kernel, t_data), ("conv backward-filter", "conv_wgrad_mfma", t_filt)):
         out.append(dict(op=name, kernel=kern, workload="configs[4] 3x3x256x256 on 56x56x256x64", bound="mfma",
                         achieved=flops / t / 1e12, peak=PEAK_MFMA_FP32 / 1e12, unit="TFLOP/s", frac=flops / t / PEAK_MFMA_FP32,
-                        avg_launch_us=t * 1e6, traffic=TRAFFIC.get("cfg5/" + kern)))
+                        avg_launch_us=t * 1e6, traffic=TRAFFIC.get("cfg5/" + kern.split(" ")[0])))
     whole = dict(tflops=2 * flops / t_all / 1e12, frac=2 * flops / t_all / PEAK_MFMA_FP32, ms=t_all * 1e3,
                  wgrad_reduce_us=t_red * 1e6)
     return out, whole

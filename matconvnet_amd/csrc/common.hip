@@ -29,6 +29,10 @@ Tunable g_tunables[] = {
     {"conv_sb_slab", 32},              // reduction rows per slab of the bank in LDS (32 or 64) of the streamed-bank kernel
     {"conv_sb_occupancy", 2},          // wavefronts per SIMD the 128-channel streamed-bank kernel's registers are cut for (2 or 3)
     {"conv_sb_fill", 2},               // workgroups per compute unit below which the streamed-bank kernel splits the reduction
+    {"conv_sb_tail", 1},               // streamed-bank kernel: the tiles of a partly filled last round get a launch of their own that splits their reduction
+    {"conv_sb_tail_slots", 0},         // resident workgroups per compute unit that plan assumes (0: the instantiation's own)
+    {"conv_sb_tail_min_pairs", 2},     // least pairs of slabs per split of a tail tile
+    {"conv_sb_tail_max_splits", 16},   // most splits of a tail tile
     {"conv_sb_min_pairs", 6},          // least pairs of 32-row slabs per split of the streamed-bank kernel
     {"pool_lds_bytes", 16 * 1024},     // LDS tile budget of the pooling-backward kernels
     {"pool_no_stream", 0},             // 1: max pooling skips the streaming kernel

@@ -259,9 +259,13 @@ int conv_ws_stat_groups(const PixP& p);
 // splits it would use for a product of these extents (0: it does not take them; depends on nothing else, so that the
 // workspace can be sized ahead); conv_sb_plan: the same, with the layout conditions checked.  conv_sb_launch: `p` laid
 // out as for the tiled kernel (with splits > 1: the partial tensors' dense layout, alpha = 1, beta = 0, no bias).
+// conv_sb_tail_bytes: scratch memory an unsplit launch of these extents wants for the tiles of its last, partly
+// filled round (0: none); conv_sb_launch takes it as tailWs (nullptr: every tile by one workgroup).
 int conv_sb_splits(int Cout, long long M, int R);
+size_t conv_sb_tail_bytes(int Cout, long long M, int R);
 bool conv_sb_plan(const PixP& p, int* splits);
-int conv_sb_launch(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, PixP p, int splits);
+int conv_sb_launch(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, PixP p, int splits,
+                   float* tailWs);
 
 // Products with at most four output channels (conv_few.hip): wt is the packed bank (tapMajor: its row order, see
 // conv_pack_weights).  Sets *handled when it took the work.

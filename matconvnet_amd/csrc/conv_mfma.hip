@@ -938,7 +938,9 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   int sbSplits = 1;
   const bool sb = ut && p.Cout > 4 && !p.stats && conv_sb_plan(p, &sbSplits);
   const int needSplits = std::max(plan.splits, sb ? sbSplits : 1);
-  const size_t need = needSplits > 1 ? align256(needW) + (size_t)needSplits * nOut * sizeof(float) : (slot || asStored ? 0 : needW);
+  const size_t tailBytes = sb && sbSplits == 1 ? conv_sb_tail_bytes(p.Cout, p.M, p.R) : 0;
+  const size_t needParts = std::max(needSplits > 1 ? (size_t)needSplits * nOut * sizeof(float) : (size_t)0, tailBytes);
+  const size_t need = needParts ? align256(needW) + needParts : (slot || asStored ? 0 : needW);
   if (need && (!ws || wsBytes < need)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small (%zu < %zu bytes)", who, wsBytes, need);
   if (need && !aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
   float* wt = (float*)ws;
@@ -983,7 +985,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   if (p.addend) return fail(MCN_UNSUPPORTED, "%s: this product cannot add a masked second term in its epilogue", who);
   // banks too large for LDS: stream them past pixels held in registers (conv_sb.hip)
   if (sb && sbSplits == 1) {
-    rc = conv_sb_launch(s, out, in, wt, bias, p, 1);
+    rc = conv_sb_launch(s, out, in, wt, bias, p, 1, tailBytes ? (float*)((char*)ws + align256(needW)) : nullptr);
     return rc ? rc : check_launch(who);
   }
   if (sb || plan.splits > 1) {
@@ -1004,7 +1006,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
       const long long ob = (long long)nOut * 4;
       q.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
     }
-    if (sb) rc = conv_sb_launch(s, partials, in, wt, nullptr, q, sbSplits);
+    if (sb) rc = conv_sb_launch(s, partials, in, wt, nullptr, q, sbSplits, nullptr);
     else launch_shape(s, plan.shape, partials, in, wt, nullptr, q, ut);
     if (rc || (rc = check_launch(who))) return rc;
     p.rSplits = q.rSplits;
@@ -1061,7 +1063,9 @@ size_t conv_mfma_workspace_bytes(const ConvP& original, int product) {
     const size_t needW = ((size_t)(R + 15) / 16 * 16) * (size_t)((Cout + BA - 1) / BA * BA) * sizeof(float);
     const PixPlan plan = plan_pix(Cout, M, R);
     const int splits = std::max(plan.splits, conv_sb_splits(Cout, M, R));  // (whichever kernel takes the product)
-    return splits > 1 ? align256(needW) + (size_t)splits * (size_t)M * Cout * sizeof(float) : needW;
+    const size_t parts = std::max(splits > 1 ? (size_t)splits * (size_t)M * Cout * sizeof(float) : (size_t)0,
+                                  conv_sb_tail_bytes(Cout, M, R));
+    return parts ? align256(needW) + parts : needW;
   };
   switch (product) {
     case MCN_CONV_FORWARD: {

@@ -19,6 +19,10 @@
 // Reduction order: the packed bank's (chunks of 16 channels, the taps inside a chunk), pairs of rows per MFMA,
 // sequential accumulation in fp32: the same sums in the same order as the tiled and the weights-stationary kernels.
 // A long reduction over few pixels is split like the tiled kernel's (partial tensors + conv_pix_reduce).
+// A launch whose tiles do not fill the chip's last round (3136 tiles on 768 resident workgroups: four rounds, then 64
+// workgroups alone on the chip for as long as a tile takes a wavefront that has its SIMD to itself) hands those last
+// tiles to a second launch that splits THEIR reduction over the whole chip (TAIL instantiation: partial tiles into the
+// workspace) and a small kernel that adds the partial tiles up in a fixed order (conv_sb_tail_reduce).
 #include "conv_common.hpp"
 
 #include <algorithm>
@@ -36,14 +40,18 @@ struct SbP {
   int groupsPerTap;   // Cin / 16
   unsigned inBytes;   // size of the gathered tensor
   unsigned wtBytes;   // size of the packed bank
+  int tileBase;       // TAIL: first tile of the tail (tiles are numbered pixel tile x tilesA + channel tile)
+  int tailTiles;      // TAIL: tiles of the tail; workgroup = (split, tile of the tail), split-major
 };
 
 // LDS-only barrier: waits for this wave's LDS traffic, not for the global loads in flight
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // kSlab: reduction rows per slab of the bank in LDS (32 or 64: two or four groups); OCC: wavefronts per SIMD the
-// register budget is cut for.
-template <int WA, bool TAPS, int kSlab, int OCC>
+// register budget is cut for.  TAIL: the launch covers tiles [tileBase, tileBase + tailTiles), each by several
+// workgroups that take a slice of the reduction each and leave their 32 WA x 128 sums, as they are, in a tile of
+// their own at out[(split * tailTiles + tile) * 32 WA * 128] (channel-major, 128 pixels per channel).
+template <int WA, bool TAPS, int kSlab, int OCC, bool TAIL = false>
 __global__ __launch_bounds__(256, OCC) void conv_sb_mfma(float* __restrict__ out, const float* __restrict__ in,
                                                     const float* __restrict__ wt, const float* __restrict__ bias,
                                                     PixP p, SbP w) {
@@ -60,7 +68,12 @@ __global__ __launch_bounds__(256, OCC) void conv_sb_mfma(float* __restrict__ out
   // neighbouring pixel tiles, whose taps reach into each other's columns, read the same pixels behind one L2)
   int logical = xcd_contiguous_id((int)blockIdx.x, (int)gridDim.x);
   int split = 0;
-  if (p.rSplits > 1) {  // (split-major: the workgroups of one split are neighbours)
+  if (TAIL) {
+    split = logical / w.tailTiles;
+    logical -= split * w.tailTiles;
+    out += ((size_t)split * w.tailTiles + logical) * (size_t)(CT * 128);
+    logical += w.tileBase;
+  } else if (p.rSplits > 1) {  // (split-major: the workgroups of one split are neighbours)
     const int tiles = (int)gridDim.x / p.rSplits;
     split = logical / tiles;
     logical -= split * tiles;
@@ -222,6 +235,13 @@ __global__ __launch_bounds__(256, OCC) void conv_sb_mfma(float* __restrict__ out
 
   // ---- epilogue: lane = pixel, register = channel
   const int coW = ca * CT;
+  if (TAIL) {  // (idle lanes and padding channels hold zeros: every load of theirs was outside its tensor)
+    const bufrsrc orsrc = make_bufrsrc(out, (unsigned)(CT * 128 * 4));
+    const unsigned vo = (unsigned)(wave * 32 + l32 + 4 * kh * 128) * 4u;
+#pragma unroll
+    for (int a = 0; a < WA; ++a) store_block(acc[a], orsrc, vo, a * 32 * 512, 512, 1.f, 0.f, nullptr, kh);
+    return;
+  }
   if (p.outBytes != 0 && coW + CT <= p.Cout) {
     const bufrsrc orsrc = make_bufrsrc(out, p.outBytes);
     const int plane = p.outPlane * 4;
@@ -251,9 +271,44 @@ __global__ __launch_bounds__(256, OCC) void conv_sb_mfma(float* __restrict__ out
     }
 }
 
+// out[tile of the tail] = alpha * (sum over the splits, in their order) (+ beta * out) (+ bias): one thread per
+// (tile, channel, pixel), pixels fastest
+__global__ __launch_bounds__(256) void conv_sb_tail_reduce(float* __restrict__ out, const float* __restrict__ partials,
+                                                           const float* __restrict__ bias, PixP p, int tileBase,
+                                                           int tailTiles, int splits, int tilesA, int CT) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  const int pxl = (int)(idx & 127);
+  const long long rest = idx >> 7;
+  const int c = (int)(rest % CT);
+  const int tl = (int)(rest / CT);
+  if (tl >= tailTiles) return;
+  const int tile = tileBase + tl;
+  const int mt = tile / tilesA, ca = tile - mt * tilesA;
+  const long long m = (long long)mt * 128 + pxl;
+  const int co = ca * CT + c;
+  if (m >= p.M || co >= p.Cout) return;
+  const size_t tileFloats = (size_t)CT * 128;
+  const float* src = partials + (size_t)tl * tileFloats + (size_t)c * 128 + pxl;
+  float sum = 0.f;
+  for (int k = 0; k < splits; ++k) sum += src[(size_t)k * tailTiles * tileFloats];
+  int n, q;
+  p.byQ.divmod((int)m, &n, &q);
+  float* o = out + (size_t)n * p.outImg + out_pixel_offset(p, q) + (size_t)co * p.outPlane;
+  float v = p.alpha * sum;
+  if (p.beta != 0.f) v = fmaf(p.beta, *o, v);
+  if (bias) v += bias[co];
+  *o = v;
+}
+
 template <int WA, int kSlab, int OCC>
 void launch(hipStream_t s, bool taps, unsigned blocks, float* out, const float* in, const float* wt, const float* bias,
             const PixP& p, const SbP& w) {
+  if (w.tailTiles > 0) {
+    KernelTimer timer("conv_sb_mfma_tail", s);
+    if (taps) hipLaunchKernelGGL((conv_sb_mfma<WA, true, kSlab, OCC, true>), dim3(blocks), dim3(256), 0, s, out, in, wt, bias, p, w);
+    else hipLaunchKernelGGL((conv_sb_mfma<WA, false, kSlab, OCC, true>), dim3(blocks), dim3(256), 0, s, out, in, wt, bias, p, w);
+    return;
+  }
   KernelTimer timer("conv_sb_mfma", s);
   if (taps) hipLaunchKernelGGL((conv_sb_mfma<WA, true, kSlab, OCC>), dim3(blocks), dim3(256), 0, s, out, in, wt, bias, p, w);
   else hipLaunchKernelGGL((conv_sb_mfma<WA, false, kSlab, OCC>), dim3(blocks), dim3(256), 0, s, out, in, wt, bias, p, w);
@@ -303,7 +358,46 @@ bool conv_sb_plan(const PixP& p, int* splits) {
   return inBytes < (long long)kOutside;
 }
 
-int conv_sb_launch(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, PixP p, int splits) {
+namespace {
+// The tail of a launch without reduction splits: the tiles left over after the last full round of resident
+// workgroups, and the reduction splits their own launch uses.  Depends on the extents only (workspace sizing).
+struct SbTail { int tiles, splits; size_t bytes; };
+SbTail sb_tail(int Cout, long long M, int R) {
+  SbTail t = {0, 0, 0};
+  if (!tunable("conv_sb_tail", 1)) return t;
+  const int CT = Cout > 64 ? 128 : 64;
+  const int coutPad = (Cout + CT - 1) / CT * CT;
+  const long long tilesAll = ((M + 127) / 128) * (coutPad / CT);
+  int cus = device_compute_units();
+  if (cus <= 0) cus = 256;
+  const int slab = slab_rows(R);
+  // resident workgroups per compute unit of the instantiation conv_sb_launch picks (registers: 160 with 128 channels)
+  const int asked = tunable("conv_sb_tail_slots", 0);
+  const int perCu = asked > 0 ? asked : CT == 128 ? 3 : slab == 64 ? 3 : 4;
+  const long long slots = (long long)cus * perCu;
+  if (tilesAll <= slots) return t;  // one round or less
+  const long long rem = tilesAll % slots;
+  if (rem == 0 || 2 * rem > slots) return t;  // a last round at least half full stays as it is
+  const int pairs = R / (2 * slab);
+  int s = (int)std::min<long long>(slots / rem, pairs / std::max(1, tunable("conv_sb_tail_min_pairs", 2)));
+  s = std::min(s, std::max(1, tunable("conv_sb_tail_max_splits", 16)));
+  if (s < 2) return t;
+  const int per = (pairs + s - 1) / s;
+  s = (pairs + per - 1) / per;
+  if (s < 2) return t;
+  t.tiles = (int)rem;
+  t.splits = s;
+  t.bytes = (size_t)s * (size_t)rem * CT * 128 * sizeof(float);
+  return t;
+}
+}  // namespace
+
+size_t conv_sb_tail_bytes(int Cout, long long M, int R) {
+  return conv_sb_splits(Cout, M, R) == 1 ? sb_tail(Cout, M, R).bytes : 0;
+}
+
+int conv_sb_launch(hipStream_t s, float* out, const float* in, const float* wt, const float* bias, PixP p, int splits,
+                   float* tailWs) {
   const int CT = p.coutPad % 128 == 0 && p.Cout > 64 ? 128 : 64;
   const int slab = slab_rows(p.R);
   SbP w;
@@ -315,18 +409,38 @@ int conv_sb_launch(hipStream_t s, float* out, const float* in, const float* wt, 
   w.groupsPerTap = p.Cin / (2 * kDepth);
   w.inBytes = (unsigned)(((long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW) * 4);
   w.wtBytes = (unsigned)((long long)p.R * p.coutPad * 4);
+  w.tileBase = 0;
+  w.tailTiles = 0;
   p.rSplits = splits;
-  const unsigned blocks = (unsigned)((long long)w.mTiles * w.tilesA * splits);
   const bool taps = !(p.T == 1 && p.dhBase == 0 && p.dwBase == 0 && p.sy == 1 && p.sx == 1 && p.IH == p.OH && p.IW == p.OW);
   const int occ = tunable("conv_sb_occupancy", 2);
-  if (CT == 128) {
-    if (slab == 64) launch<4, 64, 2>(s, taps, blocks, out, in, wt, bias, p, w);
-    else if (occ >= 3) launch<4, 32, 3>(s, taps, blocks, out, in, wt, bias, p, w);
-    else launch<4, 32, 2>(s, taps, blocks, out, in, wt, bias, p, w);
-  } else {
-    if (slab == 64) launch<2, 64, 3>(s, taps, blocks, out, in, wt, bias, p, w);
-    else launch<2, 32, 4>(s, taps, blocks, out, in, wt, bias, p, w);
+  auto dispatch = [&](unsigned blocks, float* o, const float* b, const SbP& ww) {
+    if (CT == 128) {
+      if (slab == 64) launch<4, 64, 2>(s, taps, blocks, o, in, wt, b, p, ww);
+      else if (occ >= 3) launch<4, 32, 3>(s, taps, blocks, o, in, wt, b, p, ww);
+      else launch<4, 32, 2>(s, taps, blocks, o, in, wt, b, p, ww);
+    } else {
+      if (slab == 64) launch<2, 64, 3>(s, taps, blocks, o, in, wt, b, p, ww);
+      else launch<2, 32, 4>(s, taps, blocks, o, in, wt, b, p, ww);
+    }
+  };
+  const long long tilesAll = (long long)w.mTiles * w.tilesA;
+  const SbTail tail = splits == 1 && tailWs ? sb_tail(p.Cout, p.M, p.R) : SbTail{0, 0, 0};
+  if (tail.tiles > 0 && CT == (p.Cout > 64 ? 128 : 64)) {
+    // full rounds as they are, then the left-over tiles with their reduction split over the whole chip
+    dispatch((unsigned)(tilesAll - tail.tiles), out, bias, w);
+    SbP wb = w;
+    wb.tileBase = (int)(tilesAll - tail.tiles);
+    wb.tailTiles = tail.tiles;
+    wb.slabsPerSplit = 2 * ((pairs + tail.splits - 1) / tail.splits);
+    dispatch((unsigned)((long long)tail.tiles * tail.splits), tailWs, nullptr, wb);
+    KernelTimer timer("conv_sb_tail_reduce", s);
+    const long long threads = (long long)tail.tiles * CT * 128;
+    hipLaunchKernelGGL(conv_sb_tail_reduce, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, out, tailWs, bias, p,
+                       wb.tileBase, tail.tiles, tail.splits, w.tilesA, CT);
+    return MCN_SUCCESS;
   }
+  dispatch((unsigned)(tilesAll * splits), out, bias, w);
   return MCN_SUCCESS;
 }
 

@@ -141,7 +141,7 @@ def main(src, dst):
         traffic["kernels"]["block/conv_ws_mfma"] = {"bytes": sum(ws_f) / len(ws_f) * fetch_unit + sum(ws_w) / len(ws_w) * write_unit,
                                                     "source": "profiles/bottleneck_block_56x56_N32_fwd_bwd.txt",
                                                     "note": "mean over the six launches of a step"}
-    put("cfg5/conv_sb_mfma", "conv5", "conv_sb_mfma")
+    put("cfg5/conv_sb_mfma", "conv5", ("conv_sb_mfma", "conv_sb_tail_reduce"), note="the product's launches together")
     put("cfg5/conv_pix_mfma", "conv5", "conv_pix_mfma")
     put("cfg5/conv_wgrad_mfma", "conv5", "conv_wgrad_mfma")
     put("cfg2/bnorm_sums", "bnorm", "bnorm_sums")

@@ -701,3 +701,45 @@ def test_streamed_bank_kernel_on_its_own(capi, ob, case):
     assert launches >= 1, launches   # (backward-data of 96 filters x 9 taps = 864 rows is not a multiple of 64: another kernel)
     errs = dict(y=rel_max(y, want), dzdx=rel_max(dx, wdx))
     assert max(errs.values()) <= TOL, errs
+
+
+TAILED = [  # shapes whose tiles leave a partly filled last round when one workgroup per compute unit is assumed
+    (40, 40, 64, 12, 3, 3, 64, 256, 1, 1, 1),   # forward: 300 tiles of 128 channels, 44 in the tail, three splits
+    (37, 41, 64, 13, 3, 3, 64, 200, 1, 1, 1),   # a last pixel tile of 9 pixels and a channel tile of 72 of 128 in the tail
+    (48, 48, 64, 16, 3, 3, 64, 64, 1, 1, 1),    # 64-channel tiles, forward and backward-data: 288 tiles, 32 in the tail
+]
+
+
+@pytest.mark.parametrize("case", TAILED)
+def test_streamed_bank_tail_tiles_split_their_reduction(capi, ob, case):
+    """The streamed-bank kernel gives the tiles of a partly filled last round a launch of their own that splits their
+    reduction, and a small kernel adds the partial tiles up.  With one resident workgroup per compute unit assumed,
+    shapes of a few hundred tiles take that path: forward (with bias) and backward-data against the oracle at the
+    convolution gate, the tail's launches counted."""
+    x, f, b = _tensors(case, seed=21)
+    stride, pad, dilate = case[8:]
+    g = capi.conv_geom(x.shape, f.shape, stride, pad, dilate)
+    og = ob.conv_geom(x.shape, f.shape, stride, pad, dilate)
+    want = ob.conv_forward(x, f, b, og)
+    dy = F(np.random.default_rng(22).standard_normal(want.shape))
+    wdx, _, _ = ob.conv_backward(x, f, dy, og, want=(True, False, False))
+    xd, fd, bd, dyd = capi.to_device(x), capi.to_device(f), capi.to_device(b), capi.to_device(dy)
+    capi.set_tunable("conv_no_ws", 1)
+    capi.set_tunable("conv_sb_tail_slots", 1)
+    try:
+        capi.profile_begin("conv_sb_tail_reduce")
+        y = capi.to_host(capi.conv_forward(xd, fd, bd, g))
+        dx = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(True, False, False))[0])
+        launches, _ = capi.profile_end()
+        # the same products with every tile by one workgroup: the tail only changes the order of a tile's partial sums
+        capi.set_tunable("conv_sb_tail", 0)
+        y1 = capi.to_host(capi.conv_forward(xd, fd, bd, g))
+        dx1 = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(True, False, False))[0])
+    finally:
+        capi.set_tunable("conv_no_ws", 0)
+        capi.set_tunable("conv_sb_tail_slots", 0)
+        capi.set_tunable("conv_sb_tail", 1)
+    assert launches >= 1, launches
+    errs = dict(y=rel_max(y, want), dzdx=rel_max(dx, wdx), y_whole=rel_max(y1, want), dzdx_whole=rel_max(dx1, wdx),
+                y_modes=rel_max(y, y1), dzdx_modes=rel_max(dx, dx1))
+    assert max(errs.values()) <= TOL, errs
