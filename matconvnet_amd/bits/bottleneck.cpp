@@ -1,4 +1,5 @@
 #include "bottleneck.hpp"
+#include <cstdlib>
 
 #include <hip/hip_runtime_api.h>
 
@@ -477,19 +478,24 @@ ErrorCode Bottleneck::backward() {
       return context.setError(VLE_Cuda, "cannot order the second stream");
     ErrorCode e = dataPart();
     if (e != VLE_Success) return e;
-    e = onSide.backwardAccumulate(none3, 0, derFilter, none, in, filter, derOut);
+    // (deferred: only the matrix kernel runs on the second stream, into the layer's partial banks; the sums over the
+    // splits of all layers follow the join, in one launch on the caller's stream)
+    if (deferred && partialBank[layer].bytes)
+      e = onSide.backwardFilterPartial(derFilter, in, derOut, (char*)partialArena + partialBank[layer].offset,
+                                       partialBank[layer].bytes);
+    else
+      e = onSide.backwardAccumulate(none3, 0, derFilter, none, in, filter, derOut);
     if (e != VLE_Success) context.setError(e, sideContext.getLastErrorMessage().c_str());
     return e;
   };
   auto joinSide = [&]() -> ErrorCode {
-    if (!overlap && deferred && !externalSums && !sumJobs.empty()) {
+    if (overlap && (hipEventRecord((hipEvent_t)events[4], (hipStream_t)sideStream) != hipSuccess ||
+                    hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)events[4], 0) != hipSuccess))
+      return context.setError(VLE_Cuda, "cannot join the second stream");
+    if (deferred && !externalSums && !sumJobs.empty()) {
       int rcSum = mcn_conv_reduce_batch(st, (mcn_conv_reduce_job const*)sumJobsDevice, (int)sumJobs.size(), sumBlocks);
       if (rcSum) return context.setError((ErrorCode)rcSum, mcn_last_error_message());
     }
-    if (!overlap) return VLE_Success;
-    if (hipEventRecord((hipEvent_t)events[4], (hipStream_t)sideStream) != hipSuccess ||
-        hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)events[4], 0) != hipSuccess)
-      return context.setError(VLE_Cuda, "cannot join the second stream");
     return VLE_Success;
   };
 

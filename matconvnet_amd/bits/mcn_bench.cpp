@@ -402,6 +402,7 @@ int main(int argc, char** argv) {
     benchBlock(warmup, iters, true, false, true, true);
   }
   if (only == "blocktimed") benchBlock(warmup, iters, true, false, true, true);
+  if (only == "blockoverlap") benchBlock(warmup, iters, true, true, true, true);
   if (want("conv5")) benchConv("conv 3x3x256x256 56x56 N=64", 56, 56, 256, 64, 3, 256, 1, warmup, iters);
   return 0;
 }

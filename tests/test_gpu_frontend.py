@@ -479,3 +479,28 @@ def test_block_with_the_last_relu_mask_kept_as_bits(vl, ob):
         assert blk.mask_bits is False
     finally:
         blk.close()
+
+
+def test_timed_schedule_with_filter_gradients_on_a_second_stream(vl, ob):
+    """The benchmarked schedule with the three filter-gradient matrix kernels on a second stream (they run beside the
+    batch-norm derivatives of the layer below; the sums over their reduction splits follow the join, in one launch)
+    against the same schedule on one stream: every output bit for bit, at the benchmarked size, three steps (the
+    second stream is joined at the end of each)."""
+    N = 32
+    w = workloads.bottleneck_case()
+    shapes = dict(y=w["x"].shape, dzdx=w["x"].shape, df1=w["f1"].shape, df2=w["f2"].shape, df3=w["f3"].shape,
+                  dg1=(64,), db1=(64,), dg2=(64,), db2=(64,), dg3=(256,), db3=(256,), m1=(64, 2), m2=(64, 2), m3=(256, 2))
+    outs = {}
+    for two in (False, True):
+        blk = vl.Bottleneck(N=N, eps=w["eps"], fused=True, overlap=two, packed=True, deferred=True, epilogue_sums=True,
+                            mask_bits=True)
+        try:
+            _load(blk, w)
+            blk.run(3)
+            torch.cuda.synchronize()
+            outs[two] = {k: blk.get(k, v) for k, v in shapes.items()}
+        finally:
+            blk.close()
+    for k in shapes:
+        assert np.isfinite(outs[True][k]).all(), k
+        assert bits_equal(outs[False][k], outs[True][k]), k
