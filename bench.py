@@ -549,7 +549,9 @@ def bench_resnet50(vlapi, batch, steps, warmup):
     (softmax log-loss on random labels) + backward + SGD update, and evaluation (stored moments; the mode of the reference's published 396 images/s,
     doc/site/docs/pretrained.md:233, measured there on other hardware), images/s."""
     import torch
-    net = vlapi.ResNet50(N=batch, eps=1e-5, image_size=224, classes=1000, fused=True, seed=11, channel_sums=True)
+    # (overlap: in backward the units' filter gradients run on a second stream beside the kernels that follow them on
+    # the network's stream -- same bits, tests/test_gpu_resnet.py; the one-stream step is reported beside it)
+    net = vlapi.ResNet50(N=batch, eps=1e-5, image_size=224, classes=1000, fused=True, seed=11, channel_sums=True, overlap=True)
     try:
         r = np.random.default_rng(12)
         net.set("input", np.asfortranarray(r.standard_normal((224, 224, 3, batch), dtype=np.float32)))
@@ -574,6 +576,9 @@ def bench_resnet50(vlapi, batch, steps, warmup):
             net.sgd_step(1e-3, 0.9, 1e-4)
 
         fwd_ms, step_ms = timed(net.forward), timed(train)
+        net.set_overlap(False)
+        one_stream_ms = timed(train)
+        net.set_overlap(True)
         net.set_test_mode(True)     # evaluation: batch normalisation with the moving averages of the steps above
         eval_ms = timed(net.forward)
         net.set_test_mode(False)
@@ -581,7 +586,8 @@ def bench_resnet50(vlapi, batch, steps, warmup):
         return {"batch": batch, "eval_ms": eval_ms, "eval_images_per_s": batch / eval_ms * 1e3,
                 "forward_ms": fwd_ms, "forward_images_per_s": batch / fwd_ms * 1e3,
                 "train_step_ms": step_ms, "train_images_per_s": batch / step_ms * 1e3,
-                "train_conv_tflops": 3 * flops / step_ms / 1e9, "parameters": net.parameters}
+                "train_conv_tflops": 3 * flops / step_ms / 1e9, "parameters": net.parameters,
+                "schedule": "filter gradients on a second stream", "train_step_ms_on_one_stream": one_stream_ms}
     finally:
         net.close()
 

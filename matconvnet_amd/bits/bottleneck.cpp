@@ -16,7 +16,7 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
       Wo((W - 1) / stride + 1), adapter(adapter), epsilon(epsilon), context(shared ? *shared : ownContext),
       error(VLE_Success), stageHook(NULL), hookUser(NULL), fused(false), overlap(false), testMode(false), packed(false), packedArena(NULL), packedJobs(NULL), packedBlocks(0), deferred(false), externalSums(false),
       partialArena(NULL), sumJobsDevice(NULL), sumBlocks(0), epilogueSums(false), sumsBuffer(NULL), maskBits(NULL), sumsBytes(0),
-      sideStream(NULL) {
+      sideStream(NULL), sideShared(false) {
   for (int i = 0; i < 4; ++i) sumGroupsOf[i] = 0;
   for (int i = 0; i < 5; ++i) events[i] = NULL;
   if (!adapter && (Cout != C || stride != 1)) {
@@ -53,15 +53,20 @@ Bottleneck::Bottleneck(int H, int W, int C, int M, int N, double epsilon, int Co
   }
 }
 
-ErrorCode Bottleneck::setOverlap(bool on) {
+ErrorCode Bottleneck::setOverlap(bool on, void* stream) {
+  if (on && sideStream && (stream ? sideStream != stream : sideShared)) {
+    message = "the second stream cannot be changed once set";
+    return VLE_IllegalArgument;
+  }
   if (on && !sideStream) {
-    hipStream_t st = NULL;
-    if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) {
+    hipStream_t st = (hipStream_t)stream;
+    if (!st && hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) {
       (void)hipGetLastError();
       message = "cannot create the second stream";
       return error = VLE_Cuda;
     }
     sideStream = st;
+    sideShared = stream != NULL;
     for (int i = 0; i < 5; ++i) {
       hipEvent_t e = NULL;
       if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
@@ -83,7 +88,7 @@ Bottleneck::~Bottleneck() {
     sideContext.clear();
     for (int i = 0; i < 5; ++i)
       if (events[i]) (void)hipEventDestroy((hipEvent_t)events[i]);
-    (void)hipStreamDestroy((hipStream_t)sideStream);
+    if (!sideShared) (void)hipStreamDestroy((hipStream_t)sideStream);
   }
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
@@ -489,8 +494,10 @@ ErrorCode Bottleneck::backward() {
     return e;
   };
   auto joinSide = [&]() -> ErrorCode {
-    if (overlap && (hipEventRecord((hipEvent_t)events[4], (hipStream_t)sideStream) != hipSuccess ||
-                    hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)events[4], 0) != hipSuccess))
+    // (a shared second stream is joined by its owner, unless this unit sums its own filter gradients right here)
+    if (overlap && (!sideShared || (deferred && !externalSums)) &&
+        (hipEventRecord((hipEvent_t)events[4], (hipStream_t)sideStream) != hipSuccess ||
+         hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)events[4], 0) != hipSuccess))
       return context.setError(VLE_Cuda, "cannot join the second stream");
     if (deferred && !externalSums && !sumJobs.empty()) {
       int rcSum = mcn_conv_reduce_batch(st, (mcn_conv_reduce_job const*)sumJobsDevice, (int)sumJobs.size(), sumBlocks);

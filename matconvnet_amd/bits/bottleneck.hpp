@@ -49,8 +49,11 @@ class Bottleneck {
   // overlap = true: in the backward pass each convolution's filter gradient runs on a second stream (with a
   // context and workspace of its own) beside the same layer's input gradient, which is all the following layers
   // wait for; the second stream is joined before backward() returns its work to the caller's stream.  Results are
-  // the same bits; only the schedule changes.
-  ErrorCode setOverlap(bool on);
+  // the same bits; only the schedule changes.  `stream`: a second stream of the caller's, shared by several units, in
+  // place of one of the unit's own; with it backward() does NOT join: the caller makes its stream wait for that
+  // second stream once, after the last unit (so a unit's last filter gradient also runs beside the next unit's
+  // first kernels), and before anything reads the filter gradients or rewrites the unit's activations.
+  ErrorCode setOverlap(bool on, void* stream = NULL);
   // test mode: batch normalisation uses the stored moments "rm1", "rm2", "rm3" ("rms") instead of the batch's
   // (matlab/+dagnn/BatchNorm.m:12-17); forward only
   void setTestMode(bool on) { testMode = on; }
@@ -127,6 +130,7 @@ class Bottleneck {
   std::size_t sumsBytes;
   Context sideContext;
   void* sideStream;     // hipStream_t
+  bool sideShared;      // the second stream is the caller's: not joined and not destroyed here
   void* events[5];      // hipEvent_t: "derivative ready" for the convolutions, "second stream done"
 };
 

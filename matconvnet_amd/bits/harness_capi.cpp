@@ -247,6 +247,7 @@ int vlh_resnet50_set_stream(void* net, void* stream) { return (int)((harness::Re
 void vlh_resnet50_set_fused(void* net, int fused) { ((harness::ResNet50*)net)->setFused(fused != 0); }
 void vlh_resnet50_set_test_mode(void* net, int test) { ((harness::ResNet50*)net)->setTestMode(test != 0); }
 int vlh_resnet50_set_deferred(void* net, int deferred) { return (int)((harness::ResNet50*)net)->setDeferred(deferred != 0); }
+int vlh_resnet50_set_overlap(void* net, int on) { return (int)((harness::ResNet50*)net)->setOverlap(on != 0); }
 int vlh_resnet50_set_channel_sums(void* net, int on) { return (int)((harness::ResNet50*)net)->setChannelSums(on != 0); }
 int vlh_resnet50_set_packed(void* net, int packed) { return (int)((harness::ResNet50*)net)->setPacked(packed != 0); }
 int vlh_resnet50_pack(void* net) { return (int)((harness::ResNet50*)net)->pack(); }

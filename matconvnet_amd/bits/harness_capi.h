@@ -85,6 +85,9 @@ VLH_API void vlh_resnet50_set_test_mode(void* net, int test);
 /* deferred != 0: the sums over reduction splits that finish the filter gradients run in ONE launch at the end of
    vlh_resnet50_backward instead of one per layer (same bits) */
 VLH_API int vlh_resnet50_set_deferred(void* net, int deferred);
+/* on != 0: the units' filter gradients run on a second stream beside the kernels that follow them, joined once at the end
+   of vlh_resnet50_backward (same bits) */
+VLH_API int vlh_resnet50_set_overlap(void* net, int on);
 VLH_API int vlh_resnet50_set_channel_sums(void* net, int on);
 VLH_API int vlh_resnet50_set_packed(void* net, int packed);
 VLH_API int vlh_resnet50_pack(void* net);

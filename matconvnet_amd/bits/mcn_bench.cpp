@@ -287,6 +287,8 @@ static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, 
 
 // Whole ResNet-50 (224 x 224 images, 1000 classes): forward alone (training-mode batch normalisation: moments are
 // computed, nothing is merged into the filters) and forward + backward.
+static bool gTwoStreams = false;  // --two-streams: the network's filter gradients on a second stream
+
 static void benchResNet(int warmup, int iters, int N, bool fused) {
   harness::ResNet50 net(N, 1e-5, 224, 1000);
   if (!net.ok() || net.initParameters(11) != VLE_Success) {
@@ -296,6 +298,10 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
   net.setFused(fused);
   // (the folded run also packs the filter banks ahead, once per update)
   if (fused && (net.setPacked(true) != VLE_Success || net.setChannelSums(true) != VLE_Success)) {
+    std::fprintf(stderr, "resnet-50: %s\n", net.lastMessage().c_str());
+    std::exit(3);
+  }
+  if (fused && gTwoStreams && net.setOverlap(true) != VLE_Success) {
     std::fprintf(stderr, "resnet-50: %s\n", net.lastMessage().c_str());
     std::exit(3);
   }
@@ -353,7 +359,8 @@ static void benchResNet(int warmup, int iters, int N, bool fused) {
               "%8.2f ms training step (with the loss derivative and the SGD update of %.1f M parameters) %8.0f images/s "
               "(N = %d, %.2f GFLOP of convolution per image forward; %s)\n",
               "resnet-50 224x224", tf, N / (tf * 1e-3), gf * N / tf, t, N / (t * 1e-3), 3 * gf * N / t, ts,
-              net.numParameters() * 1e-6, N / (ts * 1e-3), N, gf, fused ? "relu/sum folded into bnorm, filter banks packed once per update, channel sums from the convolutions and mask bits where the shapes allow" : "layer by layer");
+              net.numParameters() * 1e-6, N / (ts * 1e-3), N, gf, fused ? (gTwoStreams ? "relu/sum folded into bnorm, filter banks packed once per update, channel sums from the convolutions and mask bits where the shapes allow, filter gradients on a second stream"
+                                                   : "relu/sum folded into bnorm, filter banks packed once per update, channel sums from the convolutions and mask bits where the shapes allow") : "layer by layer");
 }
 
 int main(int argc, char** argv) {
@@ -366,6 +373,7 @@ int main(int argc, char** argv) {
     else if (!std::strcmp(argv[i], "--batch") && i + 1 < argc) batch = std::max(1, std::atoi(argv[++i]));
     else if (!std::strcmp(argv[i], "--rotate") && i + 1 < argc) gRotate = std::max(1, std::atoi(argv[++i]));
     else if (!std::strcmp(argv[i], "--config") && i + 1 < argc) fixed = std::atoi(argv[++i]);
+    else if (!std::strcmp(argv[i], "--two-streams")) gTwoStreams = true;
     else if (!std::strcmp(argv[i], "--set") && i + 1 < argc && std::strchr(argv[i + 1], '=')) {
       // a tunable of the back-end (mcn_set_tunable), as name=value
       std::string kv = argv[++i];
@@ -376,7 +384,7 @@ int main(int argc, char** argv) {
       }
     }
     else {
-      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|blocktimed|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...\n");
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|blocktimed|copy|yardstick|resnet50] [--batch N] [--config C] [--two-streams] [--set tunable=value]...\n");
       return 1;
     }
   }

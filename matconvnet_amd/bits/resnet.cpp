@@ -41,7 +41,7 @@ ResNet50::ResNet50(int N, double epsilon, int imageSize, int classes)
       momentsCount(0), parameterCount(0), deferred(false), partialArena(NULL), sumJobsDevice(NULL), stemPartialBytes(0),
       fcPartialBytes(0), sumJobCount(0), sumBlocks(0), packed(false), packedArena(NULL), packedJobs(NULL), stemBytes(0),
       fcForwardBytes(0), fcBackwardBytes(0), fcBackwardOffset(0), packedJobCount(0), packedBlocks(0), graph(NULL),
-      graphExec(NULL) {
+      graphExec(NULL), overlap(false), sideStream(NULL), sideDone(NULL) {
   if (S < 32 || S % 32 != 0) {
     error = VLE_IllegalArgument;
     message = "the image size must be a multiple of 32";
@@ -334,6 +334,31 @@ ErrorCode ResNet50::setChannelSums(bool on) {
   return VLE_Success;
 }
 
+ErrorCode ResNet50::setOverlap(bool on) {
+  if (error != VLE_Success) return error;
+  dropGraph();
+  if (on && !sideStream) {
+    hipStream_t st = NULL;
+    hipEvent_t ev = NULL;
+    if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      if (st) (void)hipStreamDestroy(st);
+      message = "cannot create the second stream";
+      return VLE_Cuda;
+    }
+    sideStream = st;
+    sideDone = ev;
+  }
+  for (std::size_t i = 0; i < units.size(); ++i)
+    if (units[i]->setOverlap(on, sideStream) != VLE_Success) {
+      message = units[i]->lastMessage();
+      return VLE_Cuda;
+    }
+  overlap = on;
+  return VLE_Success;
+}
+
 ErrorCode ResNet50::setDeferred(bool on) {
   if (error != VLE_Success) return error;
   dropGraph();
@@ -443,7 +468,10 @@ ErrorCode ResNet50::replay() {
 
 ResNet50::~ResNet50() {
   dropGraph();
+  if (sideStream) (void)hipStreamSynchronize((hipStream_t)sideStream);
   for (std::size_t i = 0; i < units.size(); ++i) delete units[i];
+  if (sideDone) (void)hipEventDestroy((hipEvent_t)sideDone);
+  if (sideStream) (void)hipStreamDestroy((hipStream_t)sideStream);
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
   void* arenas[] = {values, ders, state, batchMoments, runningMoments, chunkParam, rates, packedArena, packedJobs,
@@ -677,6 +705,12 @@ ErrorCode ResNet50::backward() {
     STEP("stem conv", stem.backwardFilterPartial(slot("stem.df"), slot("input"), slot("stem.da"), partialArena, stemPartialBytes));
   } else {
     STEP("stem conv", stem.backward(none, slot("stem.df"), none, slot("input"), slot("stem.f"), slot("stem.da")));
+  }
+  if (overlap && (hipEventRecord((hipEvent_t)sideDone, (hipStream_t)sideStream) != hipSuccess ||
+                  hipStreamWaitEvent((hipStream_t)st, (hipEvent_t)sideDone, 0) != hipSuccess)) {
+    (void)hipGetLastError();
+    message = "cannot join the second stream";
+    return error = VLE_Cuda;
   }
   if (deferred)  // the sums over the reduction splits of every filter gradient of the network
     ABI("filter sums", mcn_conv_reduce_batch(st, (mcn_conv_reduce_job const*)sumJobsDevice, sumJobCount, sumBlocks));

@@ -55,6 +55,11 @@ class ResNet50 {
   // own output per channel for the batch normalisation that follows (Bottleneck::setEpilogueSums, setMaskBits).  The
   // moments of those units then come from another summation order: same values to rounding, not the same bits.
   ErrorCode setChannelSums(bool on);
+  // overlap = true: in backward() the filter gradients of every unit run on a second stream of the network's, beside
+  // the kernels that follow them on the network's own stream (the batch-norm derivatives of the layer below, the next
+  // unit's first kernels); the network's stream waits for the second one once, at the end of backward() (before the
+  // sums over the reduction splits when those are deferred).  Same bits; only the schedule changes.
+  ErrorCode setOverlap(bool on);
   ErrorCode forward();
   ErrorCode backward();
   // The network's last layers (cnn_imagenet_init_resnet.m:128-139): from "prediction" and "labels" (one class number
@@ -113,6 +118,8 @@ class ResNet50 {
   int packedJobCount;
   unsigned packedBlocks;
   void *graph, *graphExec;      // hipGraph_t, hipGraphExec_t
+  bool overlap;
+  void *sideStream, *sideDone;  // hipStream_t, hipEvent_t: the second stream of setOverlap and "its work is done"
   void dropGraph();
 };
 

@@ -82,6 +82,7 @@ def lib():
         L.vlh_resnet50_set_test_mode.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_test_mode.restype = None
         L.vlh_resnet50_set_deferred.argtypes = [C.c_void_p, C.c_int]
+        L.vlh_resnet50_set_overlap.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_channel_sums.argtypes = [C.c_void_p, C.c_int]
         L.vlh_bottleneck_set_deferred.argtypes = [C.c_void_p, C.c_int]
         L.vlh_resnet50_set_packed.argtypes = [C.c_void_p, C.c_int]
@@ -269,7 +270,7 @@ class ResNet50(_NamedBuffers):
     "stem.f", "fc.f", "unit<i>.<name>", ..."""
 
     def __init__(self, N=32, eps=1e-5, image_size=224, classes=1000, fused=True, seed=None, packed=True, deferred=False,
-                 channel_sums=False):
+                 channel_sums=False, overlap=False):
         """packed: the convolutions read filter banks packed ahead, refreshed in one launch after every update (and by
         `set` of a parameter here); False: every call packs its own, as the plain operator calls do.
         deferred: the sums that finish the filter gradients run in one launch at the end of backward (off by
@@ -295,6 +296,9 @@ class ResNet50(_NamedBuffers):
             # (folded mode: the convolutions sum their output per channel for batch normalisation, identity units keep
             # their last ReLU's mask as bits, wherever the shapes allow; moments equal to rounding, not bit for bit)
             self._check(self.L.vlh_resnet50_set_channel_sums(self.h, 1))
+        if overlap:
+            # (backward: the units' filter gradients on a second stream beside the kernels that follow them; same bits)
+            self._check(self.L.vlh_resnet50_set_overlap(self.h, 1))
         if seed is not None:
             self._check(self.L.vlh_resnet50_init(self.h, seed))
 
@@ -326,6 +330,10 @@ class ResNet50(_NamedBuffers):
     def set_test_mode(self, on):
         """Batch normalisation with the moving averages ("running.*") instead of the batch's moments; forward only."""
         self.L.vlh_resnet50_set_test_mode(self.h, int(on))
+
+    def set_overlap(self, on):
+        """backward: the units' filter gradients on a second stream beside the kernels that follow them (same bits)."""
+        self._check(self.L.vlh_resnet50_set_overlap(self.h, int(on)))
 
     def _buf(self, name):
         n = C.c_size_t(0)

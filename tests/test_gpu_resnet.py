@@ -431,3 +431,39 @@ def test_channel_sums_schedule_of_the_whole_network(vl):
         assert max(errs.values()) < 2e-4, errs
     finally:
         blk.close()
+
+
+@pytest.mark.parametrize("deferred", [False, True])
+def test_filter_gradients_on_a_second_stream_change_no_bit(vl, case, deferred):
+    """backward() with every unit's filter gradients on a second stream of the network's (joined once, at the end)
+    against the one-stream schedule: gradients after two passes, parameters after two training steps, and the same
+    training step replayed three times from a HIP graph (the fork and the join are recorded with it)."""
+    import torch
+    lr, mom, wd = 0.002, 0.9, 1e-4
+    watch = _gradient_names(case) + ["stem.f", "unit0.f1", "unit3.f2", "unit3.fs", "unit15.f3", "fc.f", "momentum.unit7.f2"]
+    seen = {}
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for two in (False, True):
+            net = vl.ResNet50(N=N, eps=case["eps"], image_size=S, classes=CLASSES, fused=True, deferred=deferred, overlap=two)
+            try:
+                _load(net, case)
+                for _ in range(2):
+                    net.forward()
+                    net.backward()
+                    net.sgd_step(lr, mom, wd)
+                net.forward()
+                net.backward()
+                got = {k: net.get(k) for k in watch}
+                net.capture(True, lr, mom, wd)
+                for i in range(3):
+                    net.replay()
+                    torch.cuda.synchronize()
+                    got["replay%d" % i] = np.concatenate([net.get(k).ravel() for k in ("stem.f", "unit7.f2", "unit15.f3", "fc.f")])
+                seen[two] = got
+            finally:
+                net.close()
+    for k in seen[False]:
+        assert np.isfinite(seen[True][k]).all(), k
+        assert bits_equal(seen[False][k], seen[True][k]), k
+    assert not bits_equal(seen[True]["replay0"], seen[True]["replay2"])
