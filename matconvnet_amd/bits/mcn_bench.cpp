@@ -3,7 +3,7 @@
 // synthetic inputs, times them with HIP events and prints TFLOP/s, GB/s and images/s beside the
 // fraction of the MI355X rooflines (fp32 matrix 157.3 TFLOP/s, HBM 8 TB/s).
 //
-//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|blocktimed|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...
+//   mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|blocktimed|blockoverlap|copy|yardstick|resnet50] [--batch N] [--config C] [--set tunable=value]...
 //
 // The bandwidth-bound operators (bnorm, pooling, copy) are timed over R independent sets of tensors used in
 // turn (default 4), so that no launch finds its inputs in the 256 MB memory-side cache because the previous
@@ -280,7 +280,8 @@ static void benchBlock(int warmup, int iters, bool fused, bool overlap = false, 
     }
   }, warmup, iters);
   std::printf("%-28s %8.3f ms/step %9.0f images/s (fwd+bwd, N = %d, 41.93 GFLOP of convolution per step; %s)\n",
-              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, sums ? "folded, banks packed by one launch, filter gradients summed by one, channel sums from the convolutions, last mask as bits"
+              "resnet-50 bottleneck 56x56", t, N / (t * 1e-3), N, sums && overlap ? "folded, banks packed by one launch, filter gradients on a second stream and summed by one launch, channel sums from the convolutions, last mask as bits"
+                     : sums ? "folded, banks packed by one launch, filter gradients summed by one, channel sums from the convolutions, last mask as bits"
                      : packed ? "folded, filter banks packed by one launch per step, filter gradients summed by one"
                      : (overlap ? "folded, filter gradients on a second stream" : (fused ? "relu/sum folded into bnorm" : "layer by layer")));
 }
@@ -384,7 +385,7 @@ int main(int argc, char** argv) {
       }
     }
     else {
-      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|blocktimed|copy|yardstick|resnet50] [--batch N] [--config C] [--two-streams] [--set tunable=value]...\n");
+      std::fprintf(stderr, "usage: mcn_bench [--iters K] [--warmup W] [--rotate R] [--only conv5|conv1|bnorm|maxpool|avgpool|block|blocktimed|blockoverlap|copy|yardstick|resnet50] [--batch N] [--config C] [--two-streams] [--set tunable=value]...\n");
       return 1;
     }
   }
@@ -408,6 +409,7 @@ int main(int argc, char** argv) {
     benchBlock(warmup, iters, true, true);
     benchBlock(warmup, iters, true, false, true);
     benchBlock(warmup, iters, true, false, true, true);
+    benchBlock(warmup, iters, true, true, true, true);
   }
   if (only == "blocktimed") benchBlock(warmup, iters, true, false, true, true);
   if (only == "blockoverlap") benchBlock(warmup, iters, true, true, true, true);

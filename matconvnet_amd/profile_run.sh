@@ -25,6 +25,7 @@ for k in conv5 blocktimed; do
   echo "done counters $k"
 done
 timeout -s KILL 150 rocprofv3 --kernel-trace --stats -d "$O/kt_resnet50" -o kt -- $B --only resnet50 --batch 32 --iters 6 --warmup 2 > "$O/kt_resnet50.txt" 2>&1
+timeout -s KILL 150 $B --only resnet50 --batch 32 --iters 6 --warmup 2 --two-streams > "$O/resnet50_two_streams.txt" 2>&1
 echo "done resnet50"
 timeout -s KILL 300 $B --only yardstick --iters 8 --warmup 2 > "$O/yardstick.txt" 2>&1
 echo "done yardstick"

@@ -180,6 +180,8 @@ def main(src, dst):
          "layer and with ReLU / shortcut sums folded into batch normalisation.\n\ncommand: " + PRE +
          "  rocprofv3 --kernel-trace --stats -d gpurun_out/prof/kt_resnet50 -o kt -- ./matconvnet_amd/mcn_bench --only resnet50 --batch 32 --iters 6 --warmup 2\n\n"
          "program output under the trace:\n" + program_output(src + "/kt_resnet50.txt") +
+         "the same program untraced with the units' filter gradients on a second stream (./matconvnet_amd/mcn_bench --only resnet50 --batch 32\n"
+         " --iters 6 --warmup 2 --two-streams):\n" + program_output(src + "/resnet50_two_streams.txt") +
          "(the replays from HIP graphs at the end of each line are slowed by the tracer, which serialises the nodes of a graph; untraced they take\n"
          " the same time as the eager calls)\n\nall launches of the run:\n" + "\n".join(durations(src + "/kt_resnet50")) + "\n")
     write("resnet50_224x224_N32_training_step.txt", t)
