@@ -1,12 +1,12 @@
 #!/bin/bash
 # Collects the rocprofv3 data behind profiles/*.txt and profiles/traffic.json on an MI355X box, from the repository root:
-#     bash matconvnet_amd/profile_run.sh [output directory, default gpurun_out/prof]
+#     bash matconvnet_amd/profile_run.sh [output directory, default prof_out]
 # then  python3 -m matconvnet_amd.profile_summary <output directory> profiles
 # Kernel traces, FETCH_SIZE, WRITE_SIZE and the matrix-pipe counters each get a run of their own (rocprofv3 does not split
 # counters over passes), every run under a time limit.  mcn_bench is built by `python -m matconvnet_amd.build`.
 set -e
 R=$(pwd)
-O=${1:-gpurun_out/prof}
+O=${1:-prof_out}
 case "$O" in /*) ;; *) O=$R/$O ;; esac
 rm -rf "$O"; mkdir -p "$O"
 cd /tmp && export TMPDIR=/tmp && cd "$R"

@@ -83,8 +83,8 @@ def main(src, dst):
 
     write("bench_bottleneck_block_kernel_trace.txt",
           "Kernel trace of the default benchmark (ResNet-50 bottleneck fwd+bwd, N=32; then the per-operator configurations).\n"
-          "command: " + PRE + "  rocprofv3 --kernel-trace --stats -d gpurun_out/prof/bench -o bench -- python3 bench.py --steps 20 --warmup 5 --no-cpu-baseline\n"
-          "(all commands of this folder: bash matconvnet_amd/profile_run.sh; summaries: python3 -m matconvnet_amd.profile_summary gpurun_out/prof profiles)\n"
+          "command: " + PRE + "  rocprofv3 --kernel-trace --stats -d " + src + "/bench -o bench -- python3 bench.py --steps 20 --warmup 5 --no-cpu-baseline\n"
+          "(all commands of this folder: bash matconvnet_amd/profile_run.sh; summaries: python3 -m matconvnet_amd.profile_summary " + src + " profiles)\n"
           "Durations are per dispatch, from the profiler's kernel table (ns converted to us / ms).\n\n" + "\n".join(durations(src + "/bench")) + "\n")
 
     names = {"conv5": ("conv_vgg_3x3x256x256_N64_backward", "conv 3x3x256x256 on 56x56x256x64 (BASELINE configs[4]), backward data + filter + bias"),
@@ -98,9 +98,9 @@ def main(src, dst):
     per_kernel = {}
     for k, (fn, desc) in names.items():
         t = desc + "\n\ncommands: " + PRE
-        t += "  rocprofv3 --kernel-trace --stats -d gpurun_out/prof/kt_%s -o kt -- ./matconvnet_amd/mcn_bench --only %s --iters 12 --warmup 4\n" % (k, k)
-        t += "  rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof/fetch_%s -o pmc -- ./matconvnet_amd/mcn_bench --only %s --iters 8 --warmup 4\n" % (k, k)
-        t += "  rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof/write_%s -o pmc -- ./matconvnet_amd/mcn_bench --only %s --iters 8 --warmup 4\n" % (k, k)
+        t += "  rocprofv3 --kernel-trace --stats -d %s/kt_%s -o kt -- ./matconvnet_amd/mcn_bench --only %s --iters 12 --warmup 4\n" % (src, k, k)
+        t += "  rocprofv3 --pmc FETCH_SIZE -d %s/fetch_%s -o pmc -- ./matconvnet_amd/mcn_bench --only %s --iters 8 --warmup 4\n" % (src, k, k)
+        t += "  rocprofv3 --pmc WRITE_SIZE -d %s/write_%s -o pmc -- ./matconvnet_amd/mcn_bench --only %s --iters 8 --warmup 4\n" % (src, k, k)
         t += ("(mcn_bench is built from matconvnet_amd/bits/mcn_bench.cpp by `python -m matconvnet_amd.build`; the bandwidth-bound\n"
               " operators run COLD: mcn_bench cycles over 4 sets of tensors, --rotate 4 is its default)\n\n")
         t += "program output under the kernel trace:\n" + program_output("%s/kt_%s.txt" % (src, k)) + "\n"
@@ -157,7 +157,7 @@ def main(src, dst):
     t = ("Matrix-core utilisation counters of the convolution kernels (rocprofv3 --pmc, one pass).\n\ncommands: " + PRE)
     for k in ("conv5", "blocktimed"):
         t += ("  rocprofv3 --pmc SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_INSTS_LDS SQ_ACTIVE_INST_LDS "
-              "GRBM_GUI_ACTIVE -d gpurun_out/prof/sq_%s -o pmc -- ./matconvnet_amd/mcn_bench --only %s --iters 6 --warmup 3\n" % (k, k))
+              "GRBM_GUI_ACTIVE -d %s/sq_%s -o pmc -- ./matconvnet_amd/mcn_bench --only %s --iters 6 --warmup 3\n" % (src, k, k))
     t += ("\nReading: SQ_INSTS_MFMA counts v_mfma_f32_32x32x2_f32 instructions (4096 FLOP each); SQ_VALU_MFMA_BUSY_CYCLES is 64 cycles per\n"
           "such instruction, summed over the 1024 SIMDs; GRBM_GUI_ACTIVE is summed over the 8 XCDs.  Matrix-core utilisation of a launch =\n"
           "SQ_VALU_MFMA_BUSY_CYCLES / (1024 * GRBM_GUI_ACTIVE / 8).  (Durations under --pmc are longer than in the kernel trace: the counters\n"
@@ -178,7 +178,7 @@ def main(src, dst):
     # ---- whole network
     t = ("Whole ResNet-50 (224x224x3, 1000 classes, 32 images): kernel trace of forward, forward + backward and whole training steps, layer by\n"
          "layer and with ReLU / shortcut sums folded into batch normalisation.\n\ncommand: " + PRE +
-         "  rocprofv3 --kernel-trace --stats -d gpurun_out/prof/kt_resnet50 -o kt -- ./matconvnet_amd/mcn_bench --only resnet50 --batch 32 --iters 6 --warmup 2\n\n"
+         "  rocprofv3 --kernel-trace --stats -d " + src + "/kt_resnet50 -o kt -- ./matconvnet_amd/mcn_bench --only resnet50 --batch 32 --iters 6 --warmup 2\n\n"
          "program output under the trace:\n" + program_output(src + "/kt_resnet50.txt") +
          "the same program untraced with the units' filter gradients on a second stream (./matconvnet_amd/mcn_bench --only resnet50 --batch 32\n"
          " --iters 6 --warmup 2 --two-streams):\n" + program_output(src + "/resnet50_two_streams.txt") +
