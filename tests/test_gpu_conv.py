@@ -731,6 +731,11 @@ def test_streamed_bank_tail_tiles_split_their_reduction(capi, ob, case):
         y = capi.to_host(capi.conv_forward(xd, fd, bd, g))
         dx = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(True, False, False))[0])
         launches, _ = capi.profile_end()
+        # accumulating form through the same path: y = 2 conv(x) + bias + 0.5 y0 (the tail's summing kernel scales, adds
+        # the bias and accumulates like the matrix kernel's own epilogue)
+        y0 = F(np.random.default_rng(23).standard_normal(want.shape))
+        yacc = capi.to_host(capi.conv_forward(xd, fd, bd, g, y=capi.to_device(y0), out_mult=0.5, in_mult=2.0))
+        want_acc = 2.0 * (want - b.reshape(1, 1, -1, 1)) + b.reshape(1, 1, -1, 1) + 0.5 * y0
         # the same products with every tile by one workgroup: the tail only changes the order of a tile's partial sums
         capi.set_tunable("conv_sb_tail", 0)
         y1 = capi.to_host(capi.conv_forward(xd, fd, bd, g))
@@ -741,5 +746,5 @@ def test_streamed_bank_tail_tiles_split_their_reduction(capi, ob, case):
         capi.set_tunable("conv_sb_tail", 1)
     assert launches >= 1, launches
     errs = dict(y=rel_max(y, want), dzdx=rel_max(dx, wdx), y_whole=rel_max(y1, want), dzdx_whole=rel_max(dx1, wdx),
-                y_modes=rel_max(y, y1), dzdx_modes=rel_max(dx, dx1))
+                y_modes=rel_max(y, y1), dzdx_modes=rel_max(dx, dx1), y_accumulated=rel_max(yacc, want_acc))
     assert max(errs.values()) <= TOL, errs
