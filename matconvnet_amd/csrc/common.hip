@@ -37,6 +37,7 @@ Tunable g_tunables[] = {
     {"pool_lds_bytes", 16 * 1024},     // LDS tile budget of the pooling-backward kernels
     {"pool_no_stream", 0},             // 1: max pooling skips the streaming kernel
     {"pool_walk", 3},                  // streaming kernel's tile order: 0 round-robin, 1 contiguous runs, 2 round-robin per XCD eighth, 3 planes round-robin over XCDs
+    {"bnorm_walk", 1},                 // order of batch normalisation's workgroups: 1 by plane address (image-major), 0 channel-major and XCD by XCD, 2 by plane address and XCD by XCD
     {"bnorm_sums_scalar", 0},          // 1: the summing pass of batch-norm backward (moments from the batch) loads 4 bytes per lane, four in flight
     {"pool_no_tiles", 0},              // 1: average pooling over windows that tile the plane skips its streaming kernel
     {"pool_ablate", 0},                // (experiments only, wrong results) 1: no ordered passes, 2: no winner search either
