@@ -417,10 +417,16 @@ struct WgP {
 // block lies inside one tap.  A thread's sixteen patch rows then need four inside-the-image tests per step
 // instead of sixteen, and every load is a per-thread constant 32-bit offset from a per-step pixel offset.
 // The partial banks come out in R' order; conv_wgrad_reduce puts them back in MATLAB order.
-template <int WA, int WB, int NWA, int NWB, bool UT>
+// DIRECT (with UT, all filter rows of every tile present): the loads of a step go from global memory straight into LDS
+// (buffer loads with the LDS destination: no staging registers, no LDS write instructions, nothing to wait for
+// before the next step's MFMAs but the barrier).  A wavefront's load instruction fills 64 consecutive floats of LDS,
+// so a pair of rows (the two halves of the wavefront) lies side by side and pairs are 65 floats apart: row r, pixel p
+// at (r / 2) 65 + (r % 2) 32 + p -- the 32 rows a fragment read touches fall into 32 different banks.
+template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
 __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ out, const float* __restrict__ x,
                                                           const float* __restrict__ dy, WgP p) {
   static_assert(NWA * NWB == 4, "four wavefronts per workgroup");
+  static_assert(!DIRECT || UT, "loads into LDS go with the uniform-tap row order");
   constexpr int BA = WA * 32 * NWA;  // filters (k) per workgroup
   constexpr int BB = WB * 32 * NWB;  // filter-volume rows (R) per workgroup
   constexpr int BP = 32;             // pixels per reduction step
@@ -525,6 +531,24 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
     if (UT) {
       const unsigned pixX = (unsigned)(n * p.xImg + ihB + p.H * iwB + half * HW) * 4u;
       const unsigned pixY = valid ? (unsigned)(n * p.dyImg + q + half * Q) * 4u : kOutside;
+      if (DIRECT) {
+        typedef __attribute__((address_space(3))) void* lds_ptr;
+        float* Bd = Bs[step & 1];
+        float* Ad = As[step & 1];
+#pragma unroll
+        for (int jb = 0; jb < NBLK; ++jb) {
+          const bool ok = valid && (unsigned)(ihB + blkDh[jb]) < (unsigned)p.H && (unsigned)(iwB + blkDw[jb]) < (unsigned)p.W;
+          const unsigned vo = ok ? pixX + (unsigned)blkShift[jb] : kOutside;
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4)  // rows 32 jb + 2 wave + 8 e4 (+ half): pair 16 jb + wave + 4 e4
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (lds_ptr)(Bd + (16 * jb + waveU + 4 * e4) * 65), 4, (int)vo,
+                                                     xOffS[4 * jb + e4], 0, 0);
+        }
+#pragma unroll
+        for (int e = 0; e < APT; ++e)  // rows 2 wave + 8 e (+ half): pair wave + 4 e
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(yr, (lds_ptr)(Ad + (waveU + 4 * e) * 65), 4, (int)pixY, yOffS[e], 0, 0);
+        return;
+      }
 #pragma unroll
       for (int jb = 0; jb < NBLK; ++jb) {
         const bool ok = valid && (unsigned)(ihB + blkDh[jb]) < (unsigned)p.H && (unsigned)(iwB + blkDw[jb]) < (unsigned)p.W;
@@ -581,28 +605,32 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   __syncthreads();  // rowTab ready
   if (nSteps > 0) {
     fetch(0);
-    stash(0);
+    if (!DIRECT) stash(0);
   }
+  if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (this wavefront's loads into LDS have landed)
   __syncthreads();
 
+  // floats between the rows of consecutive 32-row blocks, and this lane's row inside its first block
+  constexpr int BLK = DIRECT ? 16 * 65 : 32 * LD;
+  const int laneRow = DIRECT ? (l32 >> 1) * 65 + (l32 & 1) * 32 : l32 * LD;
   for (int step = 0; step < nSteps; ++step) {
     const int buf = step & 1;
     if (step + 1 < nSteps) fetch(step + 1);
-    const float* Ab = As[buf] + (wa * WA * 32 + l32) * LD + kh;
-    const float* Bb = Bs[buf] + (wb * WB * 32 + l32) * LD + kh;
+    const float* Ab = As[buf] + wa * WA * BLK + laneRow + kh;
+    const float* Bb = Bs[buf] + wb * WB * BLK + laneRow + kh;
     float a[2][WA], b[2][WB];
 #pragma unroll
-    for (int ii = 0; ii < WA; ++ii) a[0][ii] = Ab[ii * 32 * LD];
+    for (int ii = 0; ii < WA; ++ii) a[0][ii] = Ab[ii * BLK];
 #pragma unroll
-    for (int jj = 0; jj < WB; ++jj) b[0][jj] = Bb[jj * 32 * LD];
+    for (int jj = 0; jj < WB; ++jj) b[0][jj] = Bb[jj * BLK];
 #pragma unroll
     for (int s = 0; s < BP / 2; ++s) {
       const int cur = s & 1, nxt = cur ^ 1;
       if (s + 1 < BP / 2) {
 #pragma unroll
-        for (int ii = 0; ii < WA; ++ii) a[nxt][ii] = Ab[ii * 32 * LD + 2 * s + 2];
+        for (int ii = 0; ii < WA; ++ii) a[nxt][ii] = Ab[ii * BLK + 2 * s + 2];
 #pragma unroll
-        for (int jj = 0; jj < WB; ++jj) b[nxt][jj] = Bb[jj * 32 * LD + 2 * s + 2];
+        for (int jj = 0; jj < WB; ++jj) b[nxt][jj] = Bb[jj * BLK + 2 * s + 2];
       }
       __builtin_amdgcn_sched_barrier(0);  // keep the look-ahead reads ahead of this pair's MFMAs
 #pragma unroll
@@ -611,7 +639,8 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
         for (int jj = 0; jj < WB; ++jj)
           acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][ii], b[cur][jj], acc[ii][jj], 0, 0, 0);
     }
-    if (step + 1 < nSteps) stash(buf ^ 1);
+    if (!DIRECT && step + 1 < nSteps) stash(buf ^ 1);
+    if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
 
@@ -819,7 +848,7 @@ void launch_shape(hipStream_t s, int shape, float* out, const float* in, const f
   }
 }
 
-template <int WA, int WB, int NWA, int NWB, bool UT>
+template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
 int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const float* dy, const WgP& p) {
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB, LD = 33;
   constexpr size_t lds = (size_t)2 * (BA + BB) * LD * sizeof(float) + BB * sizeof(int2);
@@ -827,7 +856,7 @@ int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const flo
   const int dev = current_device();
   const bool raised = dev >= 0 && dev < kMaxDevices && raisedOn[dev].load(std::memory_order_acquire);
   if (lds > 64 * 1024 && !raised) {
-    if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB, UT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB, UT, DIRECT>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return fail(MCN_DEVICE_ERROR, "mcn_conv_backward_filter: cannot reserve %zu bytes of LDS", lds);
@@ -835,7 +864,7 @@ int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const flo
     if (dev >= 0 && dev < kMaxDevices) raisedOn[dev].store(true, std::memory_order_release);
   }
   KernelTimer timer("conv_wgrad_mfma", s);
-  hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB, UT>), grid, dim3(256), lds, s, out, x, dy, p);
+  hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB, UT, DIRECT>), grid, dim3(256), lds, s, out, x, dy, p);
   return MCN_SUCCESS;
 }
 
@@ -1328,7 +1357,20 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
   const int BA = pick_channels_tile(p.K);
   int rc;
   const bool narrow = pick_rows_tile(p) == 64, wide = pick_rows_tile(p) == 192;
-  if (wide) {   // (BA == 64 by pick_rows_tile)
+  // Loads straight into LDS where they measured faster: 1x1 layers of every size (9-10 %: 44.5 -> 40.4 us for the
+  // 28x28, 14x14 and 7x7 layers of ResNet-50 at 32 images, 46 -> 41 us for 256 -> 64 on 56x56) and 3x3 layers of up to 64
+  // channels (78 -> 73 us); 3x3 layers of 128 channels show no difference, wider ones lose (3x3x256x256 on 56x56x256x64:
+  // 1.96 -> 2.09 ms -- in a long loop the register path is the faster one, what the direct path saves is start-up).
+  // (tunable 2: wherever the kernel has the form, for experiments)
+  const int directMode = tunable("conv_wgrad_direct", 1);
+  const bool direct = ut && p.K % BA == 0 && (directMode == 2 || (directMode == 1 && (q.T == 1 || p.C <= 64)));
+  if (direct && wide) {
+    rc = launch_wgrad<1, 3, 2, 2, true, true>(s, grid, target, x, dy, q);
+  } else if (direct && BA == 128) {
+    rc = narrow ? launch_wgrad<2, 1, 2, 2, true, true>(s, grid, target, x, dy, q) : launch_wgrad<2, 2, 2, 2, true, true>(s, grid, target, x, dy, q);
+  } else if (direct && BA == 64) {
+    rc = narrow ? launch_wgrad<1, 1, 2, 2, true, true>(s, grid, target, x, dy, q) : launch_wgrad<2, 1, 1, 4, true, true>(s, grid, target, x, dy, q);
+  } else if (wide) {   // (BA == 64 by pick_rows_tile)
     rc = ut ? launch_wgrad<1, 3, 2, 2, true>(s, grid, target, x, dy, q) : launch_wgrad<1, 3, 2, 2, false>(s, grid, target, x, dy, q);
   } else if (ut) {
     if (BA == 128) rc = narrow ? launch_wgrad<2, 1, 2, 2, true>(s, grid, target, x, dy, q) : launch_wgrad<2, 2, 2, 2, true>(s, grid, target, x, dy, q);
