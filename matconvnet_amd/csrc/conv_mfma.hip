@@ -531,24 +531,6 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
     if (UT) {
       const unsigned pixX = (unsigned)(n * p.xImg + ihB + p.H * iwB + half * HW) * 4u;
       const unsigned pixY = valid ? (unsigned)(n * p.dyImg + q + half * Q) * 4u : kOutside;
-      if (DIRECT) {
-        typedef __attribute__((address_space(3))) void* lds_ptr;
-        float* Bd = Bs[step & 1];
-        float* Ad = As[step & 1];
-#pragma unroll
-        for (int jb = 0; jb < NBLK; ++jb) {
-          const bool ok = valid && (unsigned)(ihB + blkDh[jb]) < (unsigned)p.H && (unsigned)(iwB + blkDw[jb]) < (unsigned)p.W;
-          const unsigned vo = ok ? pixX + (unsigned)blkShift[jb] : kOutside;
-#pragma unroll
-          for (int e4 = 0; e4 < 4; ++e4)  // rows 32 jb + 2 wave + 8 e4 (+ half): pair 16 jb + wave + 4 e4
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (lds_ptr)(Bd + (16 * jb + waveU + 4 * e4) * 65), 4, (int)vo,
-                                                     xOffS[4 * jb + e4], 0, 0);
-        }
-#pragma unroll
-        for (int e = 0; e < APT; ++e)  // rows 2 wave + 8 e (+ half): pair wave + 4 e
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(yr, (lds_ptr)(Ad + (waveU + 4 * e) * 65), 4, (int)pixY, yOffS[e], 0, 0);
-        return;
-      }
 #pragma unroll
       for (int jb = 0; jb < NBLK; ++jb) {
         const bool ok = valid && (unsigned)(ihB + blkDh[jb]) < (unsigned)p.H && (unsigned)(iwB + blkDw[jb]) < (unsigned)p.W;
@@ -589,6 +571,39 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
       okA |= ok ? (1u << e) : 0u;
     }
   };
+  // DIRECT: the loads of the next step are issued a few at a time between the MFMAs of the step in hand (all at once at
+  // the top of a step they hold up that wavefront's first MFMAs).  prep: the per-lane offsets of step `step` (nothing
+  // is fetched when !live: the instruction stream stays the same on the last step); issue(t): load t of the step.
+  constexpr int NLOADS = BPT + APT;
+  unsigned voX[NBLK], voY = kOutside;
+  float *Bd = Bs[0], *Ad = As[0];
+  auto prep = [&](int step, bool live) {
+    const int m = mBegin + step * BP + px;
+    const bool valid = live && m < mEnd;
+    int n, q, ow, oh;
+    p.byQ.divmod(valid ? m : mBegin, &n, &q);
+    p.byOH.divmod(q, &ow, &oh);
+    const int ihB = oh * p.sy, iwB = ow * p.sx;
+    const unsigned pixX = (unsigned)(n * p.xImg + ihB + p.H * iwB + half * HW) * 4u;
+#pragma unroll
+    for (int jb = 0; jb < NBLK; ++jb) {
+      const bool ok = valid && (unsigned)(ihB + blkDh[jb]) < (unsigned)p.H && (unsigned)(iwB + blkDw[jb]) < (unsigned)p.W;
+      voX[jb] = ok ? pixX + (unsigned)blkShift[jb] : kOutside;
+    }
+    voY = valid ? (unsigned)(n * p.dyImg + q + half * Q) * 4u : kOutside;
+    Bd = Bs[step & 1];
+    Ad = As[step & 1];
+  };
+  auto issue = [&](int t) {
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+    if (t < BPT) {  // x: rows 32 jb + 2 wave + 8 e4 (+ half) = pair 16 jb + wave + 4 e4
+      const int jb = t / 4, e4 = t % 4;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (lds_ptr)(Bd + (16 * jb + waveU + 4 * e4) * 65), 4, (int)voX[jb], xOffS[t], 0, 0);
+    } else {        // dzdy: rows 2 wave + 8 e (+ half) = pair wave + 4 e
+      const int e = t - BPT;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(yr, (lds_ptr)(Ad + (waveU + 4 * e) * 65), 4, (int)voY, yOffS[e], 0, 0);
+    }
+  };
   const bool allK = k0 + BA <= p.K;  // uniform: no filter row of this tile is absent
   auto stash = [&](int buf) {
 #pragma unroll
@@ -604,8 +619,14 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
 
   __syncthreads();  // rowTab ready
   if (nSteps > 0) {
-    fetch(0);
-    if (!DIRECT) stash(0);
+    if (DIRECT) {
+      prep(0, true);
+#pragma unroll
+      for (int t = 0; t < NLOADS; ++t) issue(t);
+    } else {
+      fetch(0);
+      stash(0);
+    }
   }
   if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (this wavefront's loads into LDS have landed)
   __syncthreads();
@@ -615,7 +636,8 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   const int laneRow = DIRECT ? (l32 >> 1) * 65 + (l32 & 1) * 32 : l32 * LD;
   for (int step = 0; step < nSteps; ++step) {
     const int buf = step & 1;
-    if (step + 1 < nSteps) fetch(step + 1);
+    if (DIRECT) prep(step + 1, step + 1 < nSteps);
+    else if (step + 1 < nSteps) fetch(step + 1);
     const float* Ab = As[buf] + wa * WA * BLK + laneRow + kh;
     const float* Bb = Bs[buf] + wb * WB * BLK + laneRow + kh;
     float a[2][WA], b[2][WB];
@@ -626,6 +648,10 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
 #pragma unroll
     for (int s = 0; s < BP / 2; ++s) {
       const int cur = s & 1, nxt = cur ^ 1;
+      if (DIRECT) {
+#pragma unroll
+        for (int t = s * NLOADS / (BP / 2); t < (s + 1) * NLOADS / (BP / 2); ++t) issue(t);
+      }
       if (s + 1 < BP / 2) {
 #pragma unroll
         for (int ii = 0; ii < WA; ++ii) a[nxt][ii] = Ab[ii * BLK + 2 * s + 2];
@@ -1357,13 +1383,11 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
   const int BA = pick_channels_tile(p.K);
   int rc;
   const bool narrow = pick_rows_tile(p) == 64, wide = pick_rows_tile(p) == 192;
-  // Loads straight into LDS where they measured faster: 1x1 layers of every size (9-10 %: 44.5 -> 40.4 us for the
-  // 28x28, 14x14 and 7x7 layers of ResNet-50 at 32 images, 46 -> 41 us for 256 -> 64 on 56x56) and 3x3 layers of up to 64
-  // channels (78 -> 73 us); 3x3 layers of 128 channels show no difference, wider ones lose (3x3x256x256 on 56x56x256x64:
-  // 1.96 -> 2.09 ms -- in a long loop the register path is the faster one, what the direct path saves is start-up).
-  // (tunable 2: wherever the kernel has the form, for experiments)
-  const int directMode = tunable("conv_wgrad_direct", 1);
-  const bool direct = ut && p.K % BA == 0 && (directMode == 2 || (directMode == 1 && (q.T == 1 || p.C <= 64)));
+  // Loads straight into LDS wherever the kernel has the form (uniform taps, whole filter tiles), issued a few at a time
+  // between the MFMAs: 12-18 % on every layer measured (1x1 layers of ResNet-50 at 32 images 44.3 -> 37.4 us, 3x3x64x64 on
+  // 56x56 78.8 -> 67.9 us, 3x3x256x256 on 56x56x256x64 1.95 -> 1.74 ms).  Issued all at once at the top of a step the same
+  // loads were a gain only for short launches and a loss for long ones (1.96 -> 2.09 ms).
+  const bool direct = ut && p.K % BA == 0 && tunable("conv_wgrad_direct", 1);
   if (direct && wide) {
     rc = launch_wgrad<1, 3, 2, 2, true, true>(s, grid, target, x, dy, q);
   } else if (direct && BA == 128) {
