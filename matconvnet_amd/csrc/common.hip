@@ -23,6 +23,7 @@ struct Tunable {
 // Defaults are the values chosen from on-device sweeps; see the per-kernel comments where each is read.
 Tunable g_tunables[] = {
     {"conv_wgrad_wide_rows_exact", 1}, // 192-row filter-gradient tiles for volumes they cover exactly and 128-row tiles do not
+    {"conv_pix_direct", 1},            // tiled kernel: the loads of a step go straight into LDS, a few at a time between the MFMAs (0: through registers)
     {"conv_wgrad_direct", 1},          // filter gradient: the loads of a step go straight into LDS, a few at a time between the MFMAs (0: through registers)
     {"conv_no_sb", 0},                 // 1: the streamed-bank kernel is not used (banks too large for LDS go to the tiled kernel)
     {"conv_sb_split", 0},              // 0: the streamed-bank kernel leaves products whose reduction it would split to the tiled kernel

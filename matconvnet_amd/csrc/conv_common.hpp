@@ -105,6 +105,8 @@ struct PixP {
   FastDiv byQ, byOH, byT;  // Q = OH*OW; T = taps
   int advC, advT;          // 16 = advC*T + advT (reduction rows per step)
   unsigned outBytes;       // bytes from `out` to the end of the produced tensor, or 0 when >= 2 GiB (no buffer descriptor)
+  // tiled kernel, loads straight into LDS: bytes of the gathered tensor and of the packed bank (both < 2 GiB), else 0
+  unsigned inBytes = 0, wtBytes = 0;
   // Where things lie, in elements.  The gathered tensor: image n, channel ci at in + n*inImg + ci*IH*IW.  The produced
   // tensor: pixel (oh, ow) of image n, channel co at out + n*outImg + co*outPlane + outOff + oh*outSH + ow*outSW.
   // A plain layer has inImg = Cin*IH*IW, outImg = Cout*OH*OW, outPlane = OH*OW, outOff = 0, outSH = 1, outSW = OH

@@ -152,11 +152,16 @@ __global__ __launch_bounds__(256) void conv_pix_reduce(float* __restrict__ out, 
 // thread, the step's base address is uniform (scalar registers), and every gathered row is a load at a
 // per-thread constant 32-bit offset from it.  This removes almost all vector-ALU work from the loop, and
 // vector-ALU work is what competes with the MFMAs for the SIMD.
-template <int WA, int WB, int NWA, int NWB, bool UT>
+// DIRECT (with UT; pixel tiles of at least 64, channel tiles of at least 64): the loads of a step go from global memory
+// straight into LDS (buffer loads with the LDS destination), a few at a time between the MFMAs of the step in hand: no
+// staging registers, no LDS write instructions.  Both tiles are laid out in LDS exactly as a wavefront's load delivers
+// them: 64 consecutive pixels of a row, or 64 consecutive 16-byte vectors of the bank's rows.
+template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
 __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out, const float* __restrict__ in,
                                                         const float* __restrict__ wt,
                                                         const float* __restrict__ bias, PixP p) {
   static_assert(NWA * NWB == 4, "four wavefronts per workgroup");
+  static_assert(!DIRECT || (UT && WB * 32 * NWB >= 64 && WA * 32 * NWA >= 64), "loads into LDS: uniform taps, tiles of 64 and more");
   constexpr int BA = WA * 32 * NWA;  // output channels per workgroup
   constexpr int BB = WB * 32 * NWB;  // pixels per workgroup
   constexpr int BK = 16;             // reduction rows per step
@@ -165,9 +170,18 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   constexpr int A4 = BK * BA / 4;    // float4s in a weight tile
   constexpr int APT = (A4 + 255) / 256;
 
-  __shared__ float As[2][BK * BA];
-  __shared__ float Bs[2][BK * BB];
-  __shared__ int2 tapTab[kMaxTaps];  // .x = dh + IH*dw, .y = (dh & 0xffff) | (dw << 16)
+  // DIRECT: loads run two steps ahead (they need no registers to wait in): three buffers, in dynamic LDS (with static
+  // arrays the compiler makes every LDS read wait for all loads in flight, whatever buffer they fill)
+  constexpr int NBUF = DIRECT ? 3 : 2;
+  extern __shared__ float smem[];
+  __shared__ float AsStatic[DIRECT ? 1 : 2][DIRECT ? 4 : BK * BA];
+  __shared__ float BsStatic[DIRECT ? 1 : 2][DIRECT ? 4 : BK * BB];
+  float* const AsBase = DIRECT ? smem : &AsStatic[0][0];
+  float* const BsBase = DIRECT ? smem + NBUF * BK * BA : &BsStatic[0][0];
+  auto As = [&](int b) -> float* { return AsBase + b * (BK * BA); };
+  auto Bs = [&](int b) -> float* { return BsBase + b * (BK * BB); };
+  __shared__ int2 tapStatic[DIRECT ? 1 : kMaxTaps];
+  int2* const tapTab = DIRECT ? (int2*)(smem + NBUF * BK * (BA + BB)) : tapStatic;  // .x = dh + IH*dw, .y = (dh & 0xffff) | (dw << 16)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -309,23 +323,92 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int e = 0; e < RPT; ++e) Bs[buf][(pg * RPT + e) * BB + mm] = (UT || ((okMask >> e) & 1u)) ? pb[e] : 0.f;
-    if (A4 % 256 == 0 || tid < A4) *(float4*)&As[buf][tid * 4] = pa0;
-    if (APT == 2) *(float4*)&As[buf][(tid + 256) * 4] = pa1;
+    for (int e = 0; e < RPT; ++e) Bs(buf)[(pg * RPT + e) * BB + mm] = (UT || ((okMask >> e) & 1u)) ? pb[e] : 0.f;
+    if (A4 % 256 == 0 || tid < A4) *(float4*)&As(buf)[tid * 4] = pa0;
+    if (APT == 2) *(float4*)&As(buf)[(tid + 256) * 4] = pa1;
+  };
+  // DIRECT: prep(step, live, buffer) works out the step's offsets (nothing is fetched when !live: the instruction stream
+  // stays the same on the last step); issue(t) is load t of the step: the thread group's RPT gathered rows, then the
+  // APT vectors of the bank.
+  constexpr int NLOADS = RPT + APT;
+  const int waveU = __builtin_amdgcn_readfirstlane(wave);
+  __amdgpu_buffer_rsrc_t inr, wtr;
+  unsigned voB = kOutside, voB0 = kOutside, voA[APT];
+  int sB = 0, sA = 0;
+  float *Bd = Bs(0), *Ad = As(0);
+  if (DIRECT) {
+    inr = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, (int)p.inBytes, 0x00020000);
+    wtr = __builtin_amdgcn_make_buffer_rsrc((void*)wt, 0, (int)p.wtBytes, 0x00020000);
+    // this lane's pixel, row 0 of its thread group, at tap shift 0
+    voB0 = mvalid ? (unsigned)((int)(inN - in) + pg * RPT * IHW) * 4u : kOutside;
+#pragma unroll
+    for (int j = 0; j < APT; ++j) {
+      const int idx = tid + 256 * j;
+      const int row = idx / (BA / 4), c4 = idx - row * (BA / 4);
+      voA[j] = (unsigned)(row * p.coutPad + c4 * 4) * 4u;
+    }
+  }
+  // (the tap's shift as scalars kept up to date by additions, not from the table in LDS: the compiler makes a table
+  // read wait for every load into LDS still in flight)
+  int tapRow = utTap % p.FH, dhL = p.dhBase + tapRow * p.dhStep, dwL = p.dwBase + (utTap / p.FH) * p.dwStep;
+  auto prep = [&](int step, bool live, int buf) {
+    const int ih = ihB + dhL, iw = iwB + dwL;
+    const bool ok = live && mvalid && (unsigned)ih < (unsigned)p.IH && (unsigned)iw < (unsigned)p.IW;
+    voB = ok ? voB0 + (unsigned)((dhL + p.IH * dwL) * 4) : kOutside;  // (the shift may be negative: it goes with the lane's offset)
+    sB = utCi * IHW * 4;
+    dhL += p.dhStep;
+    if (++tapRow == p.FH) {
+      tapRow = 0;
+      dhL = p.dhBase;
+      dwL += p.dwStep;
+    }
+    if (++utTap == p.T) {
+      utTap = 0;
+      dwL = p.dwBase;
+      utCi += BK;
+    }
+    sA = live ? (step * BK * p.coutPad + co0) * 4 : (int)kOutside;
+    Bd = Bs(buf);
+    Ad = As(buf);
+  };
+  auto issue = [&](int t) {
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+    if (t < RPT) {  // gathered row pg RPT + t: this wavefront's 64 pixels of it
+      const int pgU = (waveU * 64) / BB, mm0 = (waveU * 64) % BB;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(inr, (lds_ptr)(Bd + (pgU * RPT + t) * BB + mm0), 4, (int)voB, sB + t * IHW * 4, 0, 0);
+    } else {        // vectors 256 j + tid of the bank's 16 rows
+      const int j = t - RPT;
+      if (A4 % 256 == 0 || (256 * j + waveU * 64) < A4)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(wtr, (lds_ptr)(Ad + (256 * j + waveU * 64) * 4), 16, (int)voA[j], sA, 0, 0);
+    }
   };
 
   __syncthreads();  // tapTab ready
-  if (sBegin < sEnd) {
-    fetch(sBegin);
-    stash(0);
+  if (DIRECT) {
+    // two steps in flight before the loop (every wavefront issues NLOADS loads per step whether they fetch anything or
+    // not, so "all but the youngest NLOADS have landed" is a count the hardware can wait for)
+    prep(sBegin, sBegin < sEnd, 0);
+#pragma unroll
+    for (int t = 0; t < NLOADS; ++t) issue(t);
+    prep(sBegin + 1, sBegin + 1 < sEnd, 1);
+#pragma unroll
+    for (int t = 0; t < NLOADS; ++t) issue(t);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::"n"(NLOADS) : "memory");
+  } else {
+    if (sBegin < sEnd) {
+      fetch(sBegin);
+      stash(0);
+    }
+    __syncthreads();
   }
-  __syncthreads();
 
+  int buf = 0;  // (DIRECT: of three)
   for (int step = sBegin; step < sEnd; ++step) {
-    const int buf = (step - sBegin) & 1;
-    if (step + 1 < sEnd) fetch(step + 1);
-    const float* Ab = As[buf] + wa * WA * 32 + l32 + kh * BA;
-    const float* Bb = Bs[buf] + wb * WB * 32 + l32 + kh * BB;
+    if (!DIRECT) buf = (step - sBegin) & 1;
+    if (DIRECT) prep(step + 2, step + 2 < sEnd, buf >= 1 ? buf - 1 : 2);  // = (buf + 2) % 3
+    else if (step + 1 < sEnd) fetch(step + 1);
+    const float* Ab = As(buf) + wa * WA * 32 + l32 + kh * BA;
+    const float* Bb = Bs(buf) + wb * WB * 32 + l32 + kh * BB;
     // operand fragments are read one reduction pair ahead of the MFMAs that consume them
     float a[2][WA], b[2][WB];
 #pragma unroll
@@ -335,6 +418,10 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
 #pragma unroll
     for (int s = 0; s < BK / 2; ++s) {
       const int cur = s & 1, nxt = cur ^ 1;
+      if (DIRECT) {
+#pragma unroll
+        for (int t = s * NLOADS / (BK / 2); t < (s + 1) * NLOADS / (BK / 2); ++t) issue(t);
+      }
       if (s + 1 < BK / 2) {
 #pragma unroll
         for (int ii = 0; ii < WA; ++ii) a[nxt][ii] = Ab[(2 * s + 2) * BA + ii * 32];
@@ -348,8 +435,14 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
         for (int jj = 0; jj < WB; ++jj)
           acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][ii], b[cur][jj], acc[ii][jj], 0, 0, 0);
     }
-    if (step + 1 < sEnd) stash(buf ^ 1);
-    __syncthreads();
+    if (DIRECT) {
+      // the next step's loads (issued a step ago) have landed; this step's own may still be in flight
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::"n"(NLOADS) : "memory");
+      buf = buf == 2 ? 0 : buf + 1;
+    } else {
+      if (step + 1 < sEnd) stash(buf ^ 1);
+      __syncthreads();
+    }
   }
 
   // ---- epilogue: lane = pixel, register = channel
@@ -850,6 +943,13 @@ void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, con
   const int tilesA = (p.Cout + BA - 1) / BA;
   const dim3 grid((unsigned)(mTiles * tilesA * p.rSplits));
   KernelTimer timer("conv_pix_mfma", s);
+  if constexpr (BA >= 64 && BB >= 64) {
+    if (ut && p.inBytes != 0 && p.wtBytes != 0) {
+      hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB, true, true>), grid, dim3(256), 3 * 16 * (BA + BB) * sizeof(float) + kMaxTaps * sizeof(int2), s, out,
+                         in, wt, bias, p);
+      return;
+    }
+  }
   if (ut) hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB, true>), grid, dim3(256), 0, s, out, in, wt, bias, p);
   else hipLaunchKernelGGL((conv_pix_mfma<WA, WB, NWA, NWB, false>), grid, dim3(256), 0, s, out, in, wt, bias, p);
 }
@@ -1015,6 +1115,13 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   {
     const long long ob = ((long long)(p.N - 1) * p.outImg + (long long)p.Cout * p.outPlane) * 4;
     p.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
+  }
+  {
+    // (loads straight into LDS in the tiled kernel: both operands behind buffer descriptors of less than 2 GiB)
+    const long long ib = inSpan * 4, wb = (long long)rPad * p.coutPad * 4;
+    const bool direct = ut && ib < (1ll << 31) && wb < (1ll << 31) && tunable("conv_pix_direct", 1);
+    p.inBytes = direct ? (unsigned)ib : 0u;
+    p.wtBytes = direct ? (unsigned)wb : 0u;
   }
   p.byQ = FastDiv(p.OH * p.OW);
   p.byOH = FastDiv(p.OH);
