@@ -668,6 +668,7 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   // the top of a step they hold up that wavefront's first MFMAs).  prep: the per-lane offsets of step `step` (nothing
   // is fetched when !live: the instruction stream stays the same on the last step); issue(t): load t of the step.
   constexpr int NLOADS = BPT + APT;
+  constexpr int SPREAD = BP / 2;  // pairs of a step the loads are spread over (over the first 8 or 12 only: same times)
   unsigned voX[NBLK], voY = kOutside;
   float *Bd = Bs[0], *Ad = As[0];
   auto prep = [&](int step, bool live) {
@@ -741,9 +742,9 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
 #pragma unroll
     for (int s = 0; s < BP / 2; ++s) {
       const int cur = s & 1, nxt = cur ^ 1;
-      if (DIRECT) {
+      if (DIRECT && s < SPREAD) {
 #pragma unroll
-        for (int t = s * NLOADS / (BP / 2); t < (s + 1) * NLOADS / (BP / 2); ++t) issue(t);
+        for (int t = s * NLOADS / SPREAD; t < (s + 1) * NLOADS / SPREAD; ++t) issue(t);
       }
       if (s + 1 < BP / 2) {
 #pragma unroll
