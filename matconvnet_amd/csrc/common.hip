@@ -59,7 +59,7 @@ Tunable g_tunables[] = {
     {"conv_ws_wa", 0},                 // 1, 2, 4: force its channels-per-wavefront (in units of 32); 0 = choose
     {"conv_no_split", 0},              // 1: the tiled kernel never splits its reduction over workgroups
     {"conv_split_max_blocks", 512},    // ... it splits when the unsplit launch has at most this many workgroups,
-    {"conv_split_target", 1024},       // aiming at this many workgroups in all,
+    {"conv_split_most", 16},           // into at most this many parts (the count is chosen by a model of the time),
     {"conv_split_min_steps", 12},      // with at least this many 16-row steps left to each
     {"conv_split_force", 0},           // n > 0: exactly n splits (experiments)
     {"conv_no_fc_view", 0},            // 1: fully-connected layers are not recast as 1x1 layers

@@ -1017,16 +1017,29 @@ PixPlan plan_pix(int Cout, long long M, int R) {
     if (forced >= 1 && forced <= 7 && baOf[forced] == BA) { plan.shape = forced; px = pxOf[forced]; }
   }
   // fewer than two workgroups per CU with a long reduction each: split it, down to 12 steps of 16 rows per
-  // workgroup, until about four workgroups per CU exist (values from a sweep over the 14x14 and 7x7 layers of
-  // ResNet-50 at 32 images: 126 -> 89 us for 3x3x256x256)
+  // workgroup.  How many ways: the count with the least modelled time -- the busiest CU's workgroups (dealt evenly)
+  // times their steps at the rate that many resident workgroups reach, plus the partial results written and read
+  // back once per split.  What
+  // matters at these sizes is how the workgroups divide among the CUs (196 tiles on 256 CUs: 5 splits leave at most 4
+  // workgroups of 29 steps on a CU, 6 splits 5 of 24; 3x3x256x256 on 14x14x256x32 82 -> 76 us, 3x3x512x512 on
+  // 7x7x512x32 95 -> 84 us).
   plan.splits = 1;
   const long long nb = blocks(px);
   const int nSteps = (R + 15) / 16;
-  const int maxBlocks = tunable("conv_split_max_blocks", 512), target = tunable("conv_split_target", 1024),
-            minSteps = tunable("conv_split_min_steps", 12);
+  const int maxBlocks = tunable("conv_split_max_blocks", 512), minSteps = tunable("conv_split_min_steps", 12);
   if (nb <= maxBlocks && nSteps >= 4 * minSteps && !tunable("conv_no_split", 0)) {
-    long long want = (target + nb - 1) / nb;
-    plan.splits = (int)std::max<long long>(1, std::min<long long>(want, nSteps / minSteps));
+    const int cus = std::max(1, device_compute_units());
+    const double stepUs = 32.0 * BA * px / (157.3e6 / 256.0);           // one step of one tile on one CU
+    const double partUs = 2.0 * (double)M * Cout * sizeof(float) / 5e6;  // one split's partial results, out and back
+    double best = 0;
+    for (int s = 1; s <= std::min(nSteps / minSteps, tunable("conv_split_most", 16)); ++s) {
+      // (a CU's workgroups share its matrix pipes; with few of them the pipes wait for loads and barriers: rates measured
+      // on 3x3x256x256 over 14x14x256x32 with 1, 2, 3 and 4 workgroups to a CU)
+      static const double rate[5] = {0, 0.63, 0.80, 0.85, 0.88};
+      const long long perCu = (nb * s + cus - 1) / cus;
+      const double cost = (double)perCu * ((nSteps + s - 1) / s) * stepUs / rate[std::min<long long>(perCu, 4)] + (s > 1 ? s * partUs + 6.0 : 0.0);
+      if (s == 1 || cost < best) { best = cost; plan.splits = s; }
+    }
   }
   if (const int forcedSplits = tunable("conv_split_force", 0)) plan.splits = std::max(1, std::min(forcedSplits, nSteps));
   return plan;
