@@ -62,6 +62,7 @@ Tunable g_tunables[] = {
     {"conv_split_most", 16},           // into at most this many parts (the count is chosen by a model of the time),
     {"conv_split_min_steps", 12},      // with at least this many 16-row steps left to each
     {"conv_split_force", 0},           // n > 0: exactly n splits (experiments)
+    {"conv_pack_tiled", 1},            // forward banks are packed tile by tile through LDS (0: element by element)
     {"conv_no_fc_view", 0},            // 1: fully-connected layers are not recast as 1x1 layers
     {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels
     {"conv_pix_tile", 0},              // force a tile shape of the pixel-major MFMA kernel (0 = automatic)
