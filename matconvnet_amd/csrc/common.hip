@@ -62,6 +62,8 @@ Tunable g_tunables[] = {
     {"conv_split_most", 16},           // into at most this many parts (the count is chosen by a model of the time),
     {"conv_split_min_steps", 12},      // with at least this many 16-row steps left to each
     {"conv_split_force", 0},           // n > 0: exactly n splits (experiments)
+    {"conv_pix_multi", 1},             // the stride classes of a strided backward-data product share one launch where they can
+    {"conv_pix_multi_tiles", 4096},    // ... up to this many tiles in all (larger layers: a launch per class)
     {"conv_pack_tiled", 1},            // forward banks are packed tile by tile through LDS (0: element by element)
     {"conv_no_fc_view", 0},            // 1: fully-connected layers are not recast as 1x1 layers
     {"conv_force_direct", 0},          // 1: always use the direct (non-MFMA) convolution kernels

@@ -74,29 +74,32 @@ __device__ __forceinline__ void pack_element(float* __restrict__ wt, const float
 // Forward banks with every tap: wt[r][k] = f[v + FV*k], v = t + T*c the position in the filter volume and r = v or its
 // tap-major permutation.  Element by element (above) the lanes of a wavefront run along k and read f a whole filter
 // volume apart.  Here a workgroup moves a tile of 64 volume positions x 64 filters through LDS: the reads run along the
-// volume, the writes along the filters (all banks of ResNet-50 in one launch: 180 -> 95 us).
+// volume, the writes along the filters (all banks of ResNet-50 in one launch: 0.12 ms less per training step).
 __device__ __forceinline__ void pack_tile(float* __restrict__ wt, const float* __restrict__ f, int T, int Cin, int Cout,
                                           int rPad, int coutPad, int tapMajor, unsigned tile, float (*lds)[65]) {
   const unsigned tilesK = (unsigned)(coutPad + 63) / 64;
   const int v0 = (int)(tile / tilesK) * 64, k0 = (int)(tile % tilesK) * 64;
   const int FV = T * Cin;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-#pragma unroll 4
+  // (all 16 loads of a thread in flight at once: a small bank is a handful of tiles, and its packing is one round trip)
+  float got[16];
+#pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int k = k0 + w * 16 + i, v = v0 + lane;
-    lds[w * 16 + i][lane] = (k < Cout && v < FV) ? f[(size_t)FV * k + v] : 0.f;
+    got[i] = (k < Cout && v < FV) ? f[(size_t)FV * k + v] : 0.f;
   }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) lds[w * 16 + i][lane] = got[i];
   __syncthreads();
-#pragma unroll 4
+#pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int v = v0 + w * 16 + i;
-    if (v >= rPad) break;
     int r = v;
     if (tapMajor && v < FV) {
       const int ci = v / T, t = v - ci * T;
       r = (ci & 15) + 16 * (t + T * (ci >> 4));
     }
-    if (k0 + lane < coutPad) wt[(size_t)r * coutPad + k0 + lane] = lds[lane][w * 16 + i];
+    if (v < rPad && k0 + lane < coutPad) wt[(size_t)r * coutPad + k0 + lane] = lds[lane][w * 16 + i];
   }
 }
 
@@ -124,10 +127,12 @@ __global__ __launch_bounds__(256) void conv_pack_many(const PackJob* __restrict_
                     (size_t)(blockIdx.x - j.firstBlock) * 256 + threadIdx.x);
 }
 
-// tile by tile: forward banks of all taps; the flags for `tapMajor` and the workgroups of the launch
-int pack_flags(const TapSet& ts, int backward, bool tapMajor) {
+// tile by tile: forward banks of all taps -- in a launch of their own only from 32 tiles on (a small bank is packed
+// sooner by many workgroups of one element per thread than by a handful of tiles); the flags for `tapMajor`
+int pack_flags(const TapSet& ts, int backward, bool tapMajor, int rPad, int coutPad, bool batched) {
   const bool tiled = !backward && ts.nI == ts.FH && ts.nJ == ts.FW && ts.i0 == 0 && ts.j0 == 0 && ts.iStep == 1 &&
-                     ts.jStep == 1 && tunable("conv_pack_tiled", 1);
+                     ts.jStep == 1 && (batched || (long long)((rPad + 63) / 64) * ((coutPad + 63) / 64) >= 32) &&
+                     tunable("conv_pack_tiled", 1);
   return (tapMajor ? 1 : 0) | (tiled ? 2 : 0);
 }
 unsigned pack_blocks(int flags, int rPad, int coutPad) {
@@ -201,10 +206,11 @@ __global__ __launch_bounds__(256) void conv_pix_reduce(float* __restrict__ out, 
 // straight into LDS (buffer loads with the LDS destination), a few at a time between the MFMAs of the step in hand: no
 // staging registers, no LDS write instructions.  Both tiles are laid out in LDS exactly as a wavefront's load delivers
 // them: 64 consecutive pixels of a row, or 64 consecutive 16-byte vectors of the bank's rows.
-template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
-__global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out, const float* __restrict__ in,
-                                                        const float* __restrict__ wt,
-                                                        const float* __restrict__ bias, PixP p) {
+// (the kernel's body: workgroup `block` of the `blocks` that share the product `p`)
+template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT>
+__device__ __forceinline__ void pix_body(float* __restrict__ out, const float* __restrict__ in, const float* __restrict__ wt,
+                                         const float* __restrict__ bias, const PixP& p, const unsigned block,
+                                         const unsigned blocks) {
   static_assert(NWA * NWB == 4, "four wavefronts per workgroup");
   static_assert(!DIRECT || (UT && WB * 32 * NWB >= 64 && WA * 32 * NWA >= 64), "loads into LDS: uniform taps, tiles of 64 and more");
   constexpr int BA = WA * 32 * NWA;  // output channels per workgroup
@@ -234,10 +240,10 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
   const int wa = wave / NWB, wb = wave - wa * NWB;
 
   const int tilesA = (p.Cout + BA - 1) / BA;
-  int logical = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  int logical = xcd_contiguous_id(block, blocks);
   int split = 0;
   if (p.rSplits > 1) {  // (split-major: the workgroups of one split are neighbours)
-    const int tiles = (int)gridDim.x / p.rSplits;
+    const int tiles = (int)blocks / p.rSplits;
     split = logical / tiles;
     logical -= split * tiles;
     out += (size_t)split * p.partStride;
@@ -530,6 +536,34 @@ __global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out,
         }
       }
   }
+}
+
+template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
+__global__ __launch_bounds__(256, 2) void conv_pix_mfma(float* __restrict__ out, const float* __restrict__ in,
+                                                        const float* __restrict__ wt,
+                                                        const float* __restrict__ bias, PixP p) {
+  pix_body<WA, WB, NWA, NWB, UT, DIRECT>(out, in, wt, bias, p, blockIdx.x, gridDim.x);
+}
+
+// Up to four products over the same two tensors in one launch (the stride classes of a strided layer's backward-data
+// product: each a small product of its own, with its own taps, bank and sub-grid of the output).  Workgroups
+// [first[i], first[i + 1]) belong to product i; the longest reductions come first.  Always the form with uniform taps
+// and loads straight into LDS.
+constexpr int kMaxMulti = 4;
+struct PixMulti {
+  PixP p[kMaxMulti];
+  const float* wt[kMaxMulti];
+  unsigned first[kMaxMulti + 1];
+  int n;
+};
+
+template <int WA, int WB, int NWA, int NWB>
+__global__ __launch_bounds__(256, 2) void conv_pix_multi(float* __restrict__ out, const float* __restrict__ in, PixMulti m) {
+  int i = 0;
+#pragma unroll
+  for (int j = 1; j < kMaxMulti; ++j)
+    if (j < m.n && blockIdx.x >= m.first[j]) i = j;
+  pix_body<WA, WB, NWA, NWB, true, true>(out, in, m.wt[i], nullptr, m.p[i], blockIdx.x - m.first[i], m.first[i + 1] - m.first[i]);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1092,8 +1126,15 @@ PixPlan plan_pix(int Cout, long long M, int R) {
 
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
+// (run_pix with a PixCollect: the product is not launched but appended to a launch of several; wsUsed reports what its
+// bank, packed on the fly, takes of the workspace)
+struct PixCollect {
+  PixMulti m;
+  size_t wsUsed;
+};
+
 int run_pix(hipStream_t s, const char* who, float* out, const float* in, const float* f, const float* bias, PixP p,
-            const TapSet& taps, int backward, void* ws, size_t wsBytes, PackCtx* pk) {
+            const TapSet& taps, int backward, void* ws, size_t wsBytes, PackCtx* pk, PixCollect* collect = nullptr) {
   const int BA = pick_channels_tile(p.Cout);
   const int rPad = (p.R + 15) / 16 * 16;
   p.coutPad = (p.Cout + BA - 1) / BA * BA;
@@ -1137,14 +1178,14 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
       if (pk->jobs) {
         PackJob j;
         j.wt = slot; j.f = f; j.taps = taps;
-        j.Cin = p.Cin; j.Cout = p.Cout; j.rPad = rPad; j.coutPad = p.coutPad; j.backward = backward; j.tapMajor = pack_flags(taps, backward, ut);
+        j.Cin = p.Cin; j.Cout = p.Cout; j.rPad = rPad; j.coutPad = p.coutPad; j.backward = backward; j.tapMajor = pack_flags(taps, backward, ut, rPad, p.coutPad, true);
         j.firstBlock = 0; j.blocks = pack_blocks(j.tapMajor, rPad, p.coutPad);
         pk->jobs->push_back(j);
       }
       return MCN_SUCCESS;
     }
     KernelTimer timer("conv_pack_weights", s);
-    const int flags = pack_flags(taps, backward, ut);
+    const int flags = pack_flags(taps, backward, ut, rPad, p.coutPad, false);
     hipLaunchKernelGGL(conv_pack_weights, dim3(pack_blocks(flags, rPad, p.coutPad)), dim3(256), 0, s, slot, f, taps, p.Cin, p.Cout,
                        rPad, p.coutPad, backward, flags);
     return check_launch(who);
@@ -1154,7 +1195,8 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   const int needSplits = std::max(plan.splits, sb ? sbSplits : 1);
   const size_t tailBytes = sb && sbSplits == 1 ? conv_sb_tail_bytes(p.Cout, p.M, p.R) : 0;
   const size_t needParts = std::max(needSplits > 1 ? (size_t)needSplits * nOut * sizeof(float) : (size_t)0, tailBytes);
-  const size_t need = needParts ? align256(needW) + needParts : (slot || asStored ? 0 : needW);
+  const size_t need = needParts && !collect ? align256(needW) + needParts : (slot || asStored ? 0 : needW);
+  if (collect) collect->wsUsed = slot || asStored ? 0 : align256(needW);
   if (need && (!ws || wsBytes < need)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small (%zu < %zu bytes)", who, wsBytes, need);
   if (need && !aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
   float* wt = (float*)ws;
@@ -1165,7 +1207,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
     wt = slot;
   } else {
     KernelTimer timer("conv_pack_weights", s);
-    const int flags = pack_flags(taps, backward, ut);
+    const int flags = pack_flags(taps, backward, ut, rPad, p.coutPad, false);
     hipLaunchKernelGGL(conv_pack_weights, dim3(pack_blocks(flags, rPad, p.coutPad)), dim3(256), 0, s, wt, f, taps, p.Cin, p.Cout,
                        rPad, p.coutPad, backward, flags);
     rc = check_launch(who);
@@ -1191,6 +1233,13 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   p.rSplits = 1;
   p.stepsPerSplit = 0;
   p.partStride = 0;
+  if (collect) {
+    if (!p.inBytes || !p.wtBytes || collect->m.n >= kMaxMulti) return fail(MCN_UNSUPPORTED, "%s: product cannot join a launch of several", who);
+    collect->m.p[collect->m.n] = p;
+    collect->m.wt[collect->m.n] = wt;
+    ++collect->m.n;
+    return MCN_SUCCESS;
+  }
   // one to four output channels (the input gradient of a first layer): conv_few.hip
   if (p.Cout <= 4) {
     int handled = 0;
@@ -1269,6 +1318,54 @@ Axis stride_axis(int phase, int pad, int dil, int stride, int taps) {
   return a;
 }
 
+// The stride classes of a strided layer's backward-data product in ONE launch of the tiled kernel (conv_pix_multi) instead
+// of one launch each: every class is a quarter of the work with a launch's fixed costs to itself, and at network sizes
+// those costs are most of it (3x3 /2, 256 -> 256 onto 28x28x256x32: four launches and a fill, 121 us; one launch ...).
+// Whether a layer (one filter group of it) takes this path depends on its geometry only: 2...4 classes with taps,
+// channels in whole steps of 16, tiles of at least 64 channels, tensors within 32-bit byte offsets, not more tiles than
+// leave a launch per class short.  Returns the number of classes, 0 = one launch per class.
+int multi_classes(const ConvP& p, Wide wd, size_t* bankBytes) {
+  if (bankBytes) *bankBytes = 0;
+  if ((p.sy == 1 && p.sx == 1) || !tunable("conv_pix_multi", 1)) return 0;
+  if (p.K % 16 != 0 || tunable("conv_no_uniform_tap", 0) || !tunable("conv_pix_direct", 1)) return 0;
+  const long long inSpan = (long long)(p.N - 1) * wd.yImg + (long long)p.K * p.outH * p.outW;
+  if (inSpan * 4 >= (1ll << 31)) return 0;
+  const int BA = pick_channels_tile(p.C);
+  if (BA < 64) return 0;
+  const long long tilesA = (p.C + BA - 1) / BA, coutPad = tilesA * BA;
+  int n = 0;
+  long long tiles = 0;
+  size_t banks = 0;
+  for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
+    for (int ph = 0; ph < p.sy && ph < p.H; ++ph) {
+      const Axis ai = stride_axis(ph, p.pt, p.dy, p.sy, p.FH), aj = stride_axis(pw, p.pl, p.dx, p.sx, p.FW);
+      if (ai.count == 0 || aj.count == 0) continue;
+      ++n;
+      const long long M = (long long)((p.H - ph + p.sy - 1) / p.sy) * ((p.W - pw + p.sx - 1) / p.sx) * p.N;
+      const long long bank = (long long)ai.count * aj.count * p.K * coutPad * 4;  // (K a multiple of 16: no padded rows)
+      if (bank >= (1ll << 31)) return 0;
+      banks += align256((size_t)bank);
+      tiles += (M + 63) / 64 * tilesA;
+    }
+  if (n < 2 || n > kMaxMulti || tiles > tunable("conv_pix_multi_tiles", 4096)) return 0;
+  if (bankBytes) *bankBytes = banks;
+  return n;
+}
+
+template <int WA, int WB, int NWA, int NWB>
+void launch_multi(hipStream_t s, float* out, const float* in, PixMulti& m) {
+  constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB;
+  unsigned at = 0;
+  for (int i = 0; i < m.n; ++i) {
+    m.first[i] = at;
+    at += (unsigned)((((long long)m.p[i].M + BB - 1) / BB) * ((m.p[i].Cout + BA - 1) / BA));
+  }
+  for (int i = m.n; i <= kMaxMulti; ++i) m.first[i] = at;
+  KernelTimer timer("conv_pix_multi", s);
+  hipLaunchKernelGGL((conv_pix_multi<WA, WB, NWA, NWB>), dim3(at), dim3(256), 3 * 16 * (BA + BB) * sizeof(float) + kMaxTaps * sizeof(int2), s,
+                     out, in, m);
+}
+
 }  // namespace
 
 bool conv_mfma_forward_supported(const ConvP& p) { return common_ok(fc_view(p)); }
@@ -1296,6 +1393,9 @@ size_t conv_mfma_workspace_bytes(const ConvP& original, int product) {
     }
     case MCN_CONV_BACKWARD_DATA: {
       if (!conv_mfma_backward_data_supported(layer)) return 0;
+      // all classes in one launch: their banks side by side
+      size_t banks = 0;
+      if (multi_classes(p, wide_of(layer), &banks)) return banks;
       // the largest need of any stride class (one class, all taps, when the strides are 1)
       size_t need = 0;
       for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
@@ -1420,11 +1520,18 @@ int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float
     q.outImg = wd.xImg;
     return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, all_taps(p), 1, ws, wsBytes, pk);
   }
-  // one class at a time (the caller has dealt with the classes no tap reaches)
+  // one class at a time (the caller has dealt with the classes no tap reaches), or all of them in one launch: then the
+  // classes with the most taps go first (planning, packing and using the banks walk them in this same order)
+  const int together = multi_classes(p, wd, nullptr);
+  PixCollect batch;
+  batch.m.n = 0;
+  size_t wsAt = 0;
+  for (int most = together ? p.FH * p.FW : 0; most >= 0; --most)
   for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
     for (int ph = 0; ph < p.sy && ph < p.H; ++ph) {
       const Axis ai = stride_axis(ph, p.pt, p.dy, p.sy, p.FH), aj = stride_axis(pw, p.pl, p.dx, p.sx, p.FW);
       if (ai.count == 0 || aj.count == 0) continue;
+      if (together && ai.count * aj.count != most) continue;
       PixP c = q;
       c.OH = (p.H - ph + p.sy - 1) / p.sy;
       c.OW = (p.W - pw + p.sx - 1) / p.sx;
@@ -1440,9 +1547,31 @@ int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float
       t.FH = p.FH; t.FW = p.FW;
       t.i0 = ai.first; t.iStep = ai.step; t.nI = ai.count;
       t.j0 = aj.first; t.jStep = aj.step; t.nJ = aj.count;
-      int rc = run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, c, t, 1, ws, wsBytes, pk);
+      int rc;
+      if (together) {
+        batch.wsUsed = 0;
+        rc = run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, c, t, 1, ws ? (char*)ws + wsAt : nullptr,
+                     wsBytes > wsAt ? wsBytes - wsAt : 0, pk, &batch);
+        wsAt += batch.wsUsed;
+      } else {
+        rc = run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, c, t, 1, ws, wsBytes, pk);
+      }
       if (rc) return rc;
     }
+  if (together && batch.m.n > 0) {
+    // 128 x 64 tiles, or 64 channels x 128 or 64 pixels: the smaller ones while the larger would leave fewer than two
+    // tiles to a CU (the classes' reductions differ four to one in length: with few tiles the longest sets the time)
+    long long tiles128 = 0, tilesWide = 0;
+    for (int i = 0; i < batch.m.n; ++i) {
+      tiles128 += ((long long)batch.m.p[i].M + 127) / 128;
+      tilesWide += (((long long)batch.m.p[i].M + 63) / 64) * ((p.C + 127) / 128);
+    }
+    const int few = 2 * std::max(1, device_compute_units());
+    if (pick_channels_tile(p.C) == 128 && tilesWide >= few) launch_multi<2, 1, 2, 2>(s, dx, dy, batch.m);
+    else if (tiles128 >= 512) launch_multi<1, 2, 2, 2>(s, dx, dy, batch.m);
+    else launch_multi<1, 1, 2, 2>(s, dx, dy, batch.m);
+    return check_launch("mcn_conv_backward_data");
+  }
   return MCN_SUCCESS;
 }
 }  // namespace
