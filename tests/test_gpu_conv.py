@@ -748,3 +748,46 @@ def test_streamed_bank_tail_tiles_split_their_reduction(capi, ob, case):
     errs = dict(y=rel_max(y, want), dzdx=rel_max(dx, wdx), y_whole=rel_max(y1, want), dzdx_whole=rel_max(dx1, wdx),
                 y_modes=rel_max(y, y1), dzdx_modes=rel_max(dx, dx1), y_accumulated=rel_max(yacc, want_acc))
     assert max(errs.values()) <= TOL, errs
+
+
+STRIDED_TOGETHER = [  # strided layers whose backward-data classes share one launch of the tiled kernel
+    (28, 28, 128, 4, 3, 3, 128, 128, 2, 1, 1),           # 3x3 /2: four classes of 4, 2, 2 and 1 taps, 128-channel tiles
+    (19, 23, 64, 3, 3, 3, 64, 64, (2, 1), (1, 0, 2, 1), 1),   # stride along one axis only: two classes, 64-channel tiles
+    (21, 20, 48, 2, 5, 4, 48, 80, 2, (2, 1, 0, 3), (1, 2)),   # dilated columns, ragged tiles, 48 channels of a tile's 64
+    (17, 17, 128, 5, 2, 2, 64, 96, 2, 0, 1),             # two filter groups; every class a single tap
+]
+
+
+@pytest.mark.parametrize("case", STRIDED_TOGETHER)
+def test_stride_classes_of_backward_data_share_one_launch(capi, ob, case):
+    """The backward-data product of a strided layer falls into one product per stride class (bits/nnconv.cu:246-278 does
+    it as one GEMM and col2im).  Where the geometry allows, all classes run in one launch of the tiled kernel: against
+    the oracle at the convolution gate, overwriting and accumulating (dzdx = dzdx0 + ...), with the banks packed on the
+    fly and packed ahead, and against the one-launch-per-class path (the same products; a class may split its
+    reduction there, so equal to rounding, not bit for bit).  The shared launch is counted."""
+    from util import bits_equal
+    H, W, C, N, FH, FW, FC, K, stride, pad, dilate = case
+    r = np.random.default_rng(31)
+    x = F(r.standard_normal((H, W, C, N)))
+    f = F(r.standard_normal((FH, FW, FC, K)) / np.sqrt(FH * FW * FC))
+    g = capi.conv_geom(x.shape, f.shape, stride, pad, dilate)
+    og = ob.conv_geom(x.shape, f.shape, stride, pad, dilate)
+    dy = F(r.standard_normal(capi.conv_out_shape(g)))
+    wdx, _, _ = ob.conv_backward(x, f, dy, og, want=(True, False, False))
+    xd, fd, dyd = capi.to_device(x), capi.to_device(f), capi.to_device(dy)
+    capi.profile_begin("conv_pix_multi")
+    dx = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(True, False, False))[0])
+    launches, _ = capi.profile_end()
+    dx0 = F(r.standard_normal(x.shape))
+    acc = capi.to_host(capi.conv_backward_data_acc(capi.to_device(dx0), 1.0, fd, dyd, g))
+    packed = capi.conv_pack_filters(fd, g, capi.CONV_BACKWARD_DATA)
+    ahead = capi.to_host(capi.conv_backward_data_packed(capi.empty(x.shape), 0.0, fd, packed, dyd, g))
+    capi.set_tunable("conv_pix_multi", 0)
+    try:
+        apart = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(True, False, False))[0])
+    finally:
+        capi.set_tunable("conv_pix_multi", 1)
+    assert launches == (2 if FC != C else 1), launches  # (one per filter group)
+    assert bits_equal(dx, ahead)
+    errs = dict(dzdx=rel_max(dx, wdx), accumulated=rel_max(acc, wdx + dx0), apart=rel_max(apart, wdx), paths=rel_max(dx, apart))
+    assert max(errs.values()) <= TOL, errs
