@@ -594,6 +594,8 @@ struct WgP {
 // before the next step's MFMAs but the barrier).  A wavefront's load instruction fills 64 consecutive floats of LDS,
 // so a pair of rows (the two halves of the wavefront) lies side by side and pairs are 65 floats apart: row r, pixel p
 // at (r / 2) 65 + (r % 2) 32 + p -- the 32 rows a fragment read touches fall into 32 different banks.
+constexpr int wgrad_buffers(int BA, int BB, bool direct) { return direct && BA + BB <= 192 ? 3 : 2; }
+
 template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
 __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ out, const float* __restrict__ x,
                                                           const float* __restrict__ dy, WgP p) {
@@ -605,11 +607,14 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   constexpr int LD = BP + 1;         // padded LDS pitch: column reads hit 32 distinct banks
   constexpr int APT = BA / 8, BPT = BB / 8;
 
-  // dynamic LDS (the 128 x 128 configuration needs 67 KB, above the 64 KB static limit)
+  // dynamic LDS (the 128 x 128 configuration needs 67 KB, above the 64 KB static limit).  DIRECT tiles of up to 192
+  // rows take three buffers (two workgroups still fit a CU): their loads run two steps ahead, and the barrier at the
+  // end of a step waits only for the step before them
+  constexpr int NBUF = wgrad_buffers(BA, BB, DIRECT);
   extern __shared__ float smem[];
-  float(*As)[BA * LD] = (float(*)[BA * LD])smem;                  // [2][BA*LD]
-  float(*Bs)[BB * LD] = (float(*)[BB * LD])(smem + 2 * BA * LD);  // [2][BB*LD]
-  int2* rowTab = (int2*)(smem + 2 * (BA + BB) * LD);              // [BB] .x = c*H*W + dh + H*dw, .y = dh | dw << 16
+  float(*As)[BA * LD] = (float(*)[BA * LD])smem;                     // [NBUF][BA*LD]
+  float(*Bs)[BB * LD] = (float(*)[BB * LD])(smem + NBUF * BA * LD);  // [NBUF][BB*LD]
+  int2* rowTab = (int2*)(smem + NBUF * (BA + BB) * LD);              // [BB] .x = c*H*W + dh + H*dw, .y = dh | dw << 16
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -750,6 +755,7 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   constexpr int SPREAD = BP / 2;  // pairs of a step the loads are spread over (over the first 8 or 12 only: same times)
   unsigned voX[NBLK], voY = kOutside;
   float *Bd = Bs[0], *Ad = As[0];
+  int bufL = 0;  // the buffer the next prepared step loads into (steps take the buffers in turn)
   auto prep = [&](int step, bool live) {
     const int m = mBegin + step * BP + px;
     const bool valid = live && m < mEnd;
@@ -764,8 +770,9 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
       voX[jb] = ok ? pixX + (unsigned)blkShift[jb] : kOutside;
     }
     voY = valid ? (unsigned)(n * p.dyImg + q + half * Q) * 4u : kOutside;
-    Bd = Bs[step & 1];
-    Ad = As[step & 1];
+    Bd = Bs[bufL];
+    Ad = As[bufL];
+    bufL = bufL == NBUF - 1 ? 0 : bufL + 1;
   };
   auto issue = [&](int t) {
     typedef __attribute__((address_space(3))) void* lds_ptr;
@@ -796,20 +803,31 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
       prep(0, true);
 #pragma unroll
       for (int t = 0; t < NLOADS; ++t) issue(t);
+      if (NBUF == 3) {
+        prep(1, 1 < nSteps);
+#pragma unroll
+        for (int t = 0; t < NLOADS; ++t) issue(t);
+      }
     } else {
       fetch(0);
       stash(0);
     }
   }
-  if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (this wavefront's loads into LDS have landed)
-  __syncthreads();
+  // (this wavefront's loads into LDS for the first step have landed; with three buffers the second step's stay in flight:
+  // every wavefront issues NLOADS loads per step whether they fetch anything or not, so the count is exact)
+  if (DIRECT && NBUF == 3) {
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::"n"(NLOADS) : "memory");
+  } else {
+    if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
 
   // floats between the rows of consecutive 32-row blocks, and this lane's row inside its first block
   constexpr int BLK = DIRECT ? 16 * 65 : 32 * LD;
   const int laneRow = DIRECT ? (l32 >> 1) * 65 + (l32 & 1) * 32 : l32 * LD;
+  int buf = 0;
   for (int step = 0; step < nSteps; ++step) {
-    const int buf = step & 1;
-    if (DIRECT) prep(step + 1, step + 1 < nSteps);
+    if (DIRECT) prep(step + NBUF - 1, step + NBUF - 1 < nSteps);
     else if (step + 1 < nSteps) fetch(step + 1);
     const float* Ab = As[buf] + wa * WA * BLK + laneRow + kh;
     const float* Bb = Bs[buf] + wb * WB * BLK + laneRow + kh;
@@ -839,8 +857,14 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
           acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][ii], b[cur][jj], acc[ii][jj], 0, 0, 0);
     }
     if (!DIRECT && step + 1 < nSteps) stash(buf ^ 1);
-    if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    if (DIRECT && NBUF == 3) {
+      // the next step's loads (issued a step ago) have landed; this step's own may still be in flight
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::"n"(NLOADS) : "memory");
+    } else {
+      if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
+    buf = buf == NBUF - 1 ? 0 : buf + 1;
   }
 
   // ---- epilogue: lane = filter-volume row R (contiguous in dF), register = filter k
@@ -1057,7 +1081,7 @@ void launch_shape(hipStream_t s, int shape, float* out, const float* in, const f
 template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
 int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const float* dy, const WgP& p) {
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB, LD = 33;
-  constexpr size_t lds = (size_t)2 * (BA + BB) * LD * sizeof(float) + BB * sizeof(int2);
+  constexpr size_t lds = (size_t)wgrad_buffers(BA, BB, DIRECT) * (BA + BB) * LD * sizeof(float) + BB * sizeof(int2);
   static std::atomic<bool> raisedOn[kMaxDevices];  // opt-in to more than 64 KB of LDS per workgroup, once per device
   const int dev = current_device();
   const bool raised = dev >= 0 && dev < kMaxDevices && raisedOn[dev].load(std::memory_order_acquire);
