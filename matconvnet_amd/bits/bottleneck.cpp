@@ -77,6 +77,8 @@ ErrorCode Bottleneck::setOverlap(bool on, void* stream) {
       events[i] = e;
     }
     sideContext.getHipHelper().setStream(sideStream);
+    // (a stream of the unit's own: its launches run beside the caller's stream; a shared one is marked by its owner)
+    if (!sideShared) (void)mcn_stream_beside(sideStream, 1);
   }
   overlap = on;
   return VLE_Success;
@@ -88,7 +90,10 @@ Bottleneck::~Bottleneck() {
     sideContext.clear();
     for (int i = 0; i < 5; ++i)
       if (events[i]) (void)hipEventDestroy((hipEvent_t)events[i]);
-    if (!sideShared) (void)hipStreamDestroy((hipStream_t)sideStream);
+    if (!sideShared) {
+      (void)mcn_stream_beside(sideStream, 0);
+      (void)hipStreamDestroy((hipStream_t)sideStream);
+    }
   }
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());

@@ -349,6 +349,7 @@ ErrorCode ResNet50::setOverlap(bool on) {
     }
     sideStream = st;
     sideDone = ev;
+    (void)mcn_stream_beside(sideStream, 1);  // its launches run beside the main stream's: one workgroup slot per CU
   }
   for (std::size_t i = 0; i < units.size(); ++i)
     if (units[i]->setOverlap(on, sideStream) != VLE_Success) {
@@ -471,7 +472,10 @@ ResNet50::~ResNet50() {
   if (sideStream) (void)hipStreamSynchronize((hipStream_t)sideStream);
   for (std::size_t i = 0; i < units.size(); ++i) delete units[i];
   if (sideDone) (void)hipEventDestroy((hipEvent_t)sideDone);
-  if (sideStream) (void)hipStreamDestroy((hipStream_t)sideStream);
+  if (sideStream) {
+    (void)mcn_stream_beside(sideStream, 0);
+    (void)hipStreamDestroy((hipStream_t)sideStream);
+  }
   for (std::size_t i = 0; i < slots.size(); ++i)
     if (slots[i].owned && slots[i].tensor.getMemory()) (void)hipFree(slots[i].tensor.getMemory());
   void* arenas[] = {values, ders, state, batchMoments, runningMoments, chunkParam, rates, packedArena, packedJobs,

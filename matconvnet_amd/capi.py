@@ -52,6 +52,7 @@ PROTOTYPES = {
     "mcn_error_name": (C.c_char_p, [_i]),
     "mcn_device_compute_units": (_i, []),
     "mcn_set_tunable": (_i, [C.c_char_p, _i]),
+    "mcn_stream_beside": (_i, [_vp, _i]),
     "mcn_get_tunable": (_i, [C.c_char_p, C.POINTER(_i)]),
     "mcn_profile_begin": (_i, [C.c_char_p]),
     "mcn_profile_end": (_i, [C.POINTER(_i), C.POINTER(_d)]),

@@ -62,6 +62,8 @@ Tunable g_tunables[] = {
     {"conv_split_most", 16},           // into at most this many parts (the count is chosen by a model of the time),
     {"conv_split_min_steps", 12},      // with at least this many 16-row steps left to each
     {"conv_split_force", 0},           // n > 0: exactly n splits (experiments)
+    {"conv_wgrad_beside_kb", 84},      // local memory a filter-gradient launch asks for on a stream marked by mcn_stream_beside
+    {"conv_wgrad_deep", 1},            // filter gradients of at most one workgroup per CU load two steps ahead (three LDS buffers)
     {"conv_pix_multi", 1},             // the stride classes of a strided backward-data product share one launch where they can
     {"conv_pix_multi_tiles", 4096},    // ... up to this many tiles in all (larger layers: a launch per class)
     {"conv_pack_tiled", 1},            // forward banks are packed tile by tile through LDS (0: element by element)
@@ -131,6 +133,18 @@ int tunable(const char* name, int fallback) {
   return fallback;
 }
 
+namespace {
+constexpr int kMaxBeside = 16;
+std::atomic<void*> g_beside[kMaxBeside];
+}  // namespace
+
+bool stream_beside(hipStream_t s) {
+  if (!s) return false;
+  for (auto& slot : g_beside)
+    if (slot.load(std::memory_order_relaxed) == (void*)s) return true;
+  return false;
+}
+
 int current_device() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
@@ -162,6 +176,22 @@ int device_compute_units() {
 extern "C" {
 
 const char* mcn_last_error_message(void) { return mcn::g_message; }
+
+int mcn_stream_beside(mcn_stream_t stream, int on) {
+  using namespace mcn;
+  if (!stream) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_stream_beside: the null stream cannot be marked");
+  for (auto& slot : g_beside)
+    if (slot.load(std::memory_order_relaxed) == (void*)stream) {
+      if (!on) slot.store(nullptr, std::memory_order_relaxed);
+      return MCN_SUCCESS;
+    }
+  if (!on) return MCN_SUCCESS;
+  for (auto& slot : g_beside) {
+    void* expected = nullptr;
+    if (slot.compare_exchange_strong(expected, (void*)stream, std::memory_order_relaxed)) return MCN_SUCCESS;
+  }
+  return fail(MCN_UNSUPPORTED, "mcn_stream_beside: %d streams are marked already", kMaxBeside);
+}
 
 const char* mcn_error_name(int code) {
   switch (code) {

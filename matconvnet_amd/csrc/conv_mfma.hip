@@ -594,9 +594,11 @@ struct WgP {
 // before the next step's MFMAs but the barrier).  A wavefront's load instruction fills 64 consecutive floats of LDS,
 // so a pair of rows (the two halves of the wavefront) lies side by side and pairs are 65 floats apart: row r, pixel p
 // at (r / 2) 65 + (r % 2) 32 + p -- the 32 rows a fragment read touches fall into 32 different banks.
-constexpr int wgrad_buffers(int BA, int BB, bool direct) { return direct && BA + BB <= 192 ? 3 : 2; }
+// (LDS buffers of the filter-gradient kernel.  DEEP: three also for larger tiles -- one workgroup to a CU then, so only
+// for launches that have no more workgroups than CUs anyway)
+constexpr int wgrad_buffers(int BA, int BB, bool direct, bool deep) { return direct && (BA + BB <= 192 || deep) ? 3 : 2; }
 
-template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
+template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false, bool DEEP = false>
 __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ out, const float* __restrict__ x,
                                                           const float* __restrict__ dy, WgP p) {
   static_assert(NWA * NWB == 4, "four wavefronts per workgroup");
@@ -610,7 +612,7 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
   // dynamic LDS (the 128 x 128 configuration needs 67 KB, above the 64 KB static limit).  DIRECT tiles of up to 192
   // rows take three buffers (two workgroups still fit a CU): their loads run two steps ahead, and the barrier at the
   // end of a step waits only for the step before them
-  constexpr int NBUF = wgrad_buffers(BA, BB, DIRECT);
+  constexpr int NBUF = wgrad_buffers(BA, BB, DIRECT, DEEP);
   extern __shared__ float smem[];
   float(*As)[BA * LD] = (float(*)[BA * LD])smem;                     // [NBUF][BA*LD]
   float(*Bs)[BB * LD] = (float(*)[BB * LD])(smem + NBUF * BA * LD);  // [NBUF][BB*LD]
@@ -1078,23 +1080,39 @@ void launch_shape(hipStream_t s, int shape, float* out, const float* in, const f
   }
 }
 
-template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false>
+template <int WA, int WB, int NWA, int NWB, bool UT, bool DIRECT = false, bool DEEP = false>
 int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const float* dy, const WgP& p) {
   constexpr int BA = WA * 32 * NWA, BB = WB * 32 * NWB, LD = 33;
-  constexpr size_t lds = (size_t)wgrad_buffers(BA, BB, DIRECT) * (BA + BB) * LD * sizeof(float) + BB * sizeof(int2);
+  constexpr size_t lds = (size_t)wgrad_buffers(BA, BB, DIRECT, DEEP) * (BA + BB) * LD * sizeof(float) + BB * sizeof(int2);
   static std::atomic<bool> raisedOn[kMaxDevices];  // opt-in to more than 64 KB of LDS per workgroup, once per device
   const int dev = current_device();
   const bool raised = dev >= 0 && dev < kMaxDevices && raisedOn[dev].load(std::memory_order_acquire);
   if (lds > 64 * 1024 && !raised) {
-    if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB, UT, DIRECT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB, UT, DIRECT, DEEP>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return fail(MCN_DEVICE_ERROR, "mcn_conv_backward_filter: cannot reserve %zu bytes of LDS", lds);
     }
     if (dev >= 0 && dev < kMaxDevices) raisedOn[dev].store(true, std::memory_order_release);
   }
+  // On a stream marked as running beside another one the launch asks for more local memory than it uses, so that a CU
+  // holds one of its workgroups at a time and the other stream's kernels keep the rest of the CU.
+  size_t ldsAsk = lds;
+  if (stream_beside(s)) {
+    ldsAsk = std::max(lds, (size_t)std::min(std::max(tunable("conv_wgrad_beside_kb", 84), 0), 128) * 1024);
+    static std::atomic<bool> widened[kMaxDevices];
+    if (ldsAsk > 64 * 1024 && ldsAsk > lds && dev >= 0 && dev < kMaxDevices && !widened[dev].load(std::memory_order_acquire)) {
+      if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB, UT, DIRECT, DEEP>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              128 * 1024) != hipSuccess) {
+        (void)hipGetLastError();
+        ldsAsk = lds;  // (the launch goes ahead with what it needs)
+      } else {
+        widened[dev].store(true, std::memory_order_release);
+      }
+    }
+  }
   KernelTimer timer("conv_wgrad_mfma", s);
-  hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB, UT, DIRECT>), grid, dim3(256), lds, s, out, x, dy, p);
+  hipLaunchKernelGGL((conv_wgrad_mfma<WA, WB, NWA, NWB, UT, DIRECT, DEEP>), grid, dim3(256), ldsAsk, s, out, x, dy, p);
   return MCN_SUCCESS;
 }
 
@@ -1711,7 +1729,11 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
   if (direct && wide) {
     rc = launch_wgrad<1, 3, 2, 2, true, true>(s, grid, target, x, dy, q);
   } else if (direct && BA == 128) {
-    rc = narrow ? launch_wgrad<2, 1, 2, 2, true, true>(s, grid, target, x, dy, q) : launch_wgrad<2, 2, 2, 2, true, true>(s, grid, target, x, dy, q);
+    // (128 x 128 tiles with no more workgroups than CUs: three buffers, which leave room for one workgroup on a CU)
+    const bool deep = !narrow && (long long)tiles * q.splits <= device_compute_units() && tunable("conv_wgrad_deep", 1);
+    rc = narrow ? launch_wgrad<2, 1, 2, 2, true, true>(s, grid, target, x, dy, q)
+                : (deep ? launch_wgrad<2, 2, 2, 2, true, true, true>(s, grid, target, x, dy, q)
+                        : launch_wgrad<2, 2, 2, 2, true, true>(s, grid, target, x, dy, q));
   } else if (direct && BA == 64) {
     rc = narrow ? launch_wgrad<1, 1, 2, 2, true, true>(s, grid, target, x, dy, q) : launch_wgrad<2, 1, 1, 4, true, true>(s, grid, target, x, dy, q);
   } else if (wide) {   // (BA == 64 by pick_rows_tile)

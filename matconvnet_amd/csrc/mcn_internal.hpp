@@ -28,6 +28,7 @@ int tunable(const char* name, int fallback);
 constexpr int kMaxDevices = 64;
 int current_device();
 int device_compute_units();
+bool stream_beside(hipStream_t s);  // marked by mcn_stream_beside: its launches take one workgroup slot per CU
 
 // Brackets one kernel launch with HIP events when live profiling of that kernel family is switched on
 // (mcn_profile_begin); costs one relaxed load otherwise.  Construct right before the launch, on its stream.

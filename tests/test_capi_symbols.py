@@ -42,3 +42,24 @@ def test_host_side_validation_needs_no_gpu():
         raise AssertionError("stride 0 accepted")
     except capi.McnError as e:
         assert e.code == capi.ILLEGAL_ARGUMENT and "STRIDE" in e.message
+
+
+def test_marking_streams_as_running_beside_another_is_host_bookkeeping():
+    """mcn_stream_beside keeps a table of at most 16 stream handles (no GPU call): the null stream is refused, marking
+    twice and unmarking an unmarked handle are harmless, the seventeenth distinct handle is refused until one is freed."""
+    import ctypes as C
+    from matconvnet_amd import capi
+    L = capi.lib()
+    handles = [C.c_void_p(0x1000 + 16 * i) for i in range(17)]  # (stand-ins: the table only compares handles)
+    try:
+        assert L.mcn_stream_beside(None, 1) == capi.ILLEGAL_ARGUMENT
+        for h in handles[:16]:
+            assert L.mcn_stream_beside(h, 1) == 0
+        assert L.mcn_stream_beside(handles[3], 1) == 0          # already marked
+        assert L.mcn_stream_beside(handles[16], 1) != 0         # table full
+        assert L.mcn_stream_beside(handles[5], 0) == 0
+        assert L.mcn_stream_beside(handles[16], 1) == 0         # a slot is free again
+        assert L.mcn_stream_beside(handles[5], 0) == 0          # not marked: nothing to do
+    finally:
+        for h in handles:
+            L.mcn_stream_beside(h, 0)

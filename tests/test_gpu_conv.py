@@ -791,3 +791,35 @@ def test_stride_classes_of_backward_data_share_one_launch(capi, ob, case):
     assert bits_equal(dx, ahead)
     errs = dict(dzdx=rel_max(dx, wdx), accumulated=rel_max(acc, wdx + dx0), apart=rel_max(apart, wdx), paths=rel_max(dx, apart))
     assert max(errs.values()) <= TOL, errs
+
+
+def test_filter_gradient_on_a_stream_marked_as_beside_another(capi, ob):
+    """mcn_stream_beside: filter-gradient launches on a marked stream ask for more local memory than they use (one
+    workgroup to a compute unit).  Nothing else changes: same bits as on an unmarked stream, for a tile shape of every
+    kind (128 x 128 with two and with three buffers, 192 rows, 64 x 64), and the oracle's values at the convolution gate."""
+    import ctypes as C
+    import torch
+    from util import bits_equal
+    side = torch.cuda.Stream()
+    L = capi.lib()
+    cases = [(14, 14, 256, 8, 1, 1, 256, 256, 1, 0, 1), (28, 28, 128, 4, 3, 3, 128, 128, 1, 1, 1),
+             (28, 28, 64, 4, 1, 1, 64, 256, 1, 0, 1), (20, 20, 64, 4, 1, 1, 64, 64, 1, 0, 1)]
+    capi.check(L.mcn_stream_beside(C.c_void_p(side.cuda_stream), 1))
+    try:
+        for case in cases:
+            x, f, _ = _tensors(case, seed=41)
+            stride, pad, dilate = case[8:]
+            g = capi.conv_geom(x.shape, f.shape, stride, pad, dilate)
+            og = ob.conv_geom(x.shape, f.shape, stride, pad, dilate)
+            dy = F(np.random.default_rng(42).standard_normal(capi.conv_out_shape(g)))
+            _, wdf, _ = ob.conv_backward(x, f, dy, og, want=(False, True, False))
+            xd, fd, dyd = capi.to_device(x), capi.to_device(f), capi.to_device(dy)
+            plain = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(False, True, False))[1])
+            torch.cuda.synchronize()
+            with torch.cuda.stream(side):
+                beside = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(False, True, False))[1])
+            side.synchronize()
+            assert bits_equal(plain, beside), case
+            assert rel_max(plain, wdf) <= TOL, case
+    finally:
+        capi.check(L.mcn_stream_beside(C.c_void_p(side.cuda_stream), 0))
