@@ -1562,18 +1562,18 @@ int backward_data_group(hipStream_t s, const ConvP& p, Wide wd, float* dx, float
     q.outImg = wd.xImg;
     return run_pix(s, "mcn_conv_backward_data", dx, dy, f, nullptr, q, all_taps(p), 1, ws, wsBytes, pk);
   }
-  // one class at a time (the caller has dealt with the classes no tap reaches), or all of them in one launch: then the
-  // classes with the most taps go first (planning, packing and using the banks walk them in this same order)
+  // one class at a time (the caller has dealt with the classes no tap reaches), or all of them in one launch.  Either way
+  // the classes with the most taps go first: in a shared launch the longest workgroups should start first, and planning,
+  // packing and using the banks must walk the classes in one order whichever way the launches go.
   const int together = multi_classes(p, wd, nullptr);
   PixCollect batch;
   batch.m.n = 0;
   size_t wsAt = 0;
-  for (int most = together ? p.FH * p.FW : 0; most >= 0; --most)
+  for (int most = p.FH * p.FW; most >= 1; --most)
   for (int pw = 0; pw < p.sx && pw < p.W; ++pw)
     for (int ph = 0; ph < p.sy && ph < p.H; ++ph) {
       const Axis ai = stride_axis(ph, p.pt, p.dy, p.sy, p.FH), aj = stride_axis(pw, p.pl, p.dx, p.sx, p.FW);
-      if (ai.count == 0 || aj.count == 0) continue;
-      if (together && ai.count * aj.count != most) continue;
+      if (ai.count * aj.count != most) continue;
       PixP c = q;
       c.OH = (p.H - ph + p.sy - 1) / p.sy;
       c.OW = (p.W - pw + p.sx - 1) / p.sx;

@@ -764,7 +764,8 @@ def test_stride_classes_of_backward_data_share_one_launch(capi, ob, case):
     it as one GEMM and col2im).  Where the geometry allows, all classes run in one launch of the tiled kernel: against
     the oracle at the convolution gate, overwriting and accumulating (dzdx = dzdx0 + ...), with the banks packed on the
     fly and packed ahead, and against the one-launch-per-class path (the same products; a class may split its
-    reduction there, so equal to rounding, not bit for bit).  The shared launch is counted."""
+    reduction there, so equal to rounding, not bit for bit; the banks packed ahead serve both paths).  The shared launch
+    is counted."""
     from util import bits_equal
     H, W, C, N, FH, FW, FC, K, stride, pad, dilate = case
     r = np.random.default_rng(31)
@@ -785,10 +786,13 @@ def test_stride_classes_of_backward_data_share_one_launch(capi, ob, case):
     capi.set_tunable("conv_pix_multi", 0)
     try:
         apart = capi.to_host(capi.conv_backward(xd, fd, dyd, g, want=(True, False, False))[0])
+        # (the banks packed ahead lie in one order whichever way the launches go)
+        apart_ahead = capi.to_host(capi.conv_backward_data_packed(capi.empty(x.shape), 0.0, fd, packed, dyd, g))
     finally:
         capi.set_tunable("conv_pix_multi", 1)
     assert launches == (2 if FC != C else 1), launches  # (one per filter group)
     assert bits_equal(dx, ahead)
+    assert bits_equal(apart, apart_ahead)
     errs = dict(dzdx=rel_max(dx, wdx), accumulated=rel_max(acc, wdx + dx0), apart=rel_max(apart, wdx), paths=rel_max(dx, apart))
     assert max(errs.values()) <= TOL, errs
 
