@@ -63,6 +63,7 @@ Tunable g_tunables[] = {
     {"conv_split_min_steps", 12},      // with at least this many 16-row steps left to each
     {"conv_split_force", 0},           // n > 0: exactly n splits (experiments)
     {"conv_wgrad_beside_kb", 84},      // local memory a filter-gradient launch asks for on a stream marked by mcn_stream_beside
+    {"conv_ws_deep_copy", 1},
     {"conv_wgrad_deep", 1},            // filter gradients of at most one workgroup per CU load two steps ahead (three LDS buffers)
     {"conv_pix_multi", 1},             // the stride classes of a strided backward-data product share one launch where they can
     {"conv_pix_multi_tiles", 4096},    // ... up to this many tiles in all (larger layers: a launch per class)

@@ -42,6 +42,7 @@ struct WsP {
   int groups;        // R / (2 kDepth)
   int groupsPerTap;  // Cin / (2 kDepth)
   unsigned inBytes;  // size of the gathered tensor
+  int deepCopy;
   FastDiv byCB, byRow;  // byRow: 8 WA = 16-byte vectors per bank row of one channel block
 };
 
@@ -97,17 +98,42 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     const int n4 = perBlock * w.chanBlocks;
     // (four vectors in flight per thread: one at a time, every round trip to L2 would be paid in full; the empty
     // asm keeps the compiler from sinking each load into the branch that guards its store)
-    for (int i0 = tid; i0 < n4; i0 += 4 * THREADS) {
+    auto fetch = [&](int i) -> v4f {
+      i = min(i, n4 - 1);
+      const int cbk = i / perBlock;  // (one-time code: a plain division)
+      const int rem = i - cbk * perBlock;
+      int r, c4;
+      w.byRow.divmod(rem, &r, &c4);
+      return *(const v4f*)(wt + (size_t)r * p.coutPad + (cbBase + cbk) * ROW + c4 * 4);
+    };
+    int i0 = tid;
+    // As many vectors in flight per thread as the bank has for it, up to twelve (a 147 KB bank is nine per thread at
+    // 1024 threads: one round trip to L2 instead of three, 80.1 -> 78.3 us on 3x3x64x64 over 56x56x64x32); a pass never
+    // asks for more than four vectors beyond the bank's end (those re-read its last vector, all threads the same one,
+    // which costs more than it looks: a pass of twelve over a bank of eight per thread lost 1-1.5 us)
+    for (; w.deepCopy && i0 + 8 * THREADS < n4; i0 += 12 * THREADS) {
+      v4f v[12];
+#pragma unroll
+      for (int k = 0; k < 12; ++k) v[k] = fetch(i0 + k * THREADS);
+      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
+                   "+v"(v[9]), "+v"(v[10]), "+v"(v[11]));
+#pragma unroll
+      for (int k = 0; k < 12; ++k)
+        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
+    }
+    for (; w.deepCopy && i0 + 4 * THREADS < n4; i0 += 8 * THREADS) {
+      v4f v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = fetch(i0 + k * THREADS);
+      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
+    }
+    for (; i0 < n4; i0 += 4 * THREADS) {
       v4f v[4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int i = min(i0 + k * THREADS, n4 - 1);
-        const int cbk = i / perBlock;  // (one-time code: a plain division)
-        const int rem = i - cbk * perBlock;
-        int r, c4;
-        w.byRow.divmod(rem, &r, &c4);
-        v[k] = *(const v4f*)(wt + (size_t)r * p.coutPad + (cbBase + cbk) * ROW + c4 * 4);
-      }
+      for (int k = 0; k < 4; ++k) v[k] = fetch(i0 + k * THREADS);
       asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
 #pragma unroll
       for (int k = 0; k < 4; ++k)
@@ -485,6 +511,7 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
   w.groups = p.R / (2 * kDepth);
   w.groupsPerTap = p.Cin / (2 * kDepth);
   w.inBytes = (unsigned)inBytes;
+  w.deepCopy = tunable("conv_ws_deep_copy", 1);
   w.byCB = FastDiv(w.chanBlocks);
   w.byRow = FastDiv(8 * WA);
   plan->WA = WA;
