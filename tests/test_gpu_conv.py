@@ -442,6 +442,8 @@ PACKED_CASES = [  # (H, W, C, N, FH, FW, K, stride, pad, dilate, groups)
     (10, 10, 32, 2, 3, 3, 32, 1, 1, 1, 2),      # two filter groups
     (6, 6, 16, 4, 6, 6, 40, 1, 0, 1, 1),        # fully connected
     (14, 14, 256, 4, 3, 3, 256, 1, 1, 1, 1),    # split reduction
+    (13, 13, 48, 2, 3, 3, 100, 1, 1, 1, 1),     # bank tiles of the packing kernel ragged both ways (432 rows, 100 of 128 filters)
+    (20, 20, 64, 2, 3, 3, 128, 2, 1, 1, 1),     # 3x3 /2: four stride classes in one launch, their banks side by side
 ]
 
 
