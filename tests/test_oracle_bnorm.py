@@ -154,7 +154,7 @@ def test_given_moments_equal_batch_moments(ob):
     assert rel_max(dx2, dx) < 1e-12 and rel_max(dg2, dg) < 1e-12 and rel_max(db2, db) < 1e-13
 
 
-def test_survey_sanity_value(ob):
+def test_known_moments_of_a_four_by_four_ramp(ob):
     # 4x4 ramp, C = N = 1, g = 2, eps = 1e-4: moments = (8.5, 4.60978)
     x = F(np.arange(1, 17, dtype=np.float32).reshape(4, 4, 1, 1, order="F"))
     _, mom = ob.bnorm_forward(x, np.array([2], np.float32), np.array([0], np.float32), 1e-4)

@@ -216,7 +216,7 @@ def test_filter_groups_equal_block_diagonal_dense(ob):
         assert rel_max(dfg[:, :, :, 3 * gi:3 * gi + 3], dfd[:, :, 2 * gi:2 * gi + 2, 3 * gi:3 * gi + 3]) < 1e-13
 
 
-def test_survey_sanity_values(ob):
+def test_known_derivatives_of_a_four_by_four_ramp(ob):
     # 4x4 ramp, 3x3 ones filter, pad 1, dzdy = ones
     x = F(np.arange(1, 17, dtype=np.float32).reshape(4, 4, 1, 1, order="F"))
     f = F(np.ones((3, 3, 1, 1)))

@@ -131,7 +131,7 @@ def test_max_backward_brute_force_tiny(ob, mode):
     assert bits_equal(ob.pool_backward(x, dy, g)[:, :, 0, 0].copy(), want)
 
 
-def test_survey_tie_example(ob):
+def test_ties_go_to_the_first_maximum_in_memory_order(ob):
     # 2x2 stride-2 max pooling of columns [1 1 1 1],[2 2 2 2],[3 3 3 3],[4 4 4 4]: winners at offsets 4,6,12,14
     x = F(np.tile(np.array([1, 2, 3, 4], np.float32), (4, 1)).reshape(4, 4, 1, 1))
     g = ob.pool_geom(x.shape, 2, 2, 0, "max")
