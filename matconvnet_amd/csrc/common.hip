@@ -37,12 +37,16 @@ Tunable g_tunables[] = {
     {"conv_sb_tail_max_splits", 16},   // most splits of a tail tile
     {"conv_sb_min_pairs", 6},          // least pairs of 32-row slabs per split of the streamed-bank kernel
     {"pool_lds_bytes", 16 * 1024},     // LDS tile budget of the pooling-backward kernels
+    {"pool_no_pairs", 0},              // 1: max pooling skips the kernel for 3x3 windows at stride 2, padding 1
+    {"pool_pairs_per_cu", 0},          // its persistent workgroups per compute unit (0: as many as fit)
+    {"pool_pairs_cols", 0},            // n > 0: its tiles are n output columns wide (0: chosen)
+    {"pool_pairs_stages", 3},          // 2 or 3 stages of a tile's operands in LDS (1 or 2 tiles in flight per workgroup)
+    {"pool_pairs_static", 0},          // 1: the workgroups of a compute unit take equal shares of its tiles
     {"pool_no_stream", 0},             // 1: max pooling skips the streaming kernel
     {"pool_walk", 3},                  // streaming kernel's tile order: 0 round-robin, 1 contiguous runs, 2 round-robin per XCD eighth, 3 planes round-robin over XCDs
     {"bnorm_walk", 1},                 // order of batch normalisation's workgroups: 1 by plane address (image-major), 0 channel-major and XCD by XCD, 2 by plane address and XCD by XCD
     {"bnorm_sums_scalar", 0},          // 1: the summing pass of batch-norm backward (moments from the batch) loads 4 bytes per lane, four in flight
     {"pool_no_tiles", 0},              // 1: average pooling over windows that tile the plane skips its streaming kernel
-    {"pool_ablate", 0},                // (experiments only, wrong results) 1: no ordered passes, 2: no winner search either
     {"pool_threads", 256},             // threads per workgroup of the streaming kernel (256; 512 and 1024 for 3x3 / 2 windows)
     {"pool_blocks_per_cu", 3},         // persistent workgroups per compute unit of the streaming kernel
     {"pool_forward_threads_k", 2048},  // threads (in 1024s) the four-rows-per-thread forward kernel aims at
@@ -181,16 +185,21 @@ const char* mcn_last_error_message(void) { return mcn::g_message; }
 int mcn_stream_beside(mcn_stream_t stream, int on) {
   using namespace mcn;
   if (!stream) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_stream_beside: the null stream cannot be marked");
+  // (not a hot path: marking and unmarking are serialised, so a stream holds at most one slot and unmarking frees it)
+  static std::mutex mutex;
+  std::lock_guard<std::mutex> lock(mutex);
+  bool marked = false;
   for (auto& slot : g_beside)
     if (slot.load(std::memory_order_relaxed) == (void*)stream) {
-      if (!on) slot.store(nullptr, std::memory_order_relaxed);
+      if (!on) slot.store(nullptr, std::memory_order_relaxed);  // (every slot that holds it)
+      marked = true;
+    }
+  if (!on || marked) return MCN_SUCCESS;
+  for (auto& slot : g_beside)
+    if (slot.load(std::memory_order_relaxed) == nullptr) {
+      slot.store((void*)stream, std::memory_order_relaxed);
       return MCN_SUCCESS;
     }
-  if (!on) return MCN_SUCCESS;
-  for (auto& slot : g_beside) {
-    void* expected = nullptr;
-    if (slot.compare_exchange_strong(expected, (void*)stream, std::memory_order_relaxed)) return MCN_SUCCESS;
-  }
   return fail(MCN_UNSUPPORTED, "mcn_stream_beside: %d streams are marked already", kMaxBeside);
 }
 

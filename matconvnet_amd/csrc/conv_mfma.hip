@@ -1194,15 +1194,15 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   // uniform-tap variant: whole 16-row steps inside one tap, and 32-bit element offsets into the gathered tensor
   const long long inSpan = (long long)(p.N - 1) * p.inImg + (long long)p.Cin * p.IH * p.IW;  // elements from `in` to the end
   const bool ut = p.Cin % 16 == 0 && inSpan < (1ll << 31) && !tunable("conv_no_uniform_tap", 0);
+  {
+    const long long ob = ((long long)(p.N - 1) * p.outImg + (long long)p.Cout * p.outPlane) * 4;
+    p.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
+  }
   if (p.statQuery) {  // (plan only: would this product also sum its output per channel, and into how many partials?)
     *p.statQuery = ut && p.Cout > 4 && !bias && p.beta == 0.f ? conv_ws_stat_groups(p) : 0;
     return MCN_SUCCESS;
   }
   if (p.stats && !(ut && p.Cout > 4)) return fail(MCN_UNSUPPORTED, "%s: this product cannot sum its output per channel", who);
-  {
-    const long long ob = ((long long)(p.N - 1) * p.outImg + (long long)p.Cout * p.outPlane) * 4;
-    p.outBytes = ob < (1ll << 31) ? (unsigned)ob : 0u;
-  }
   if (p.addQuery) {  // (plan only: can this product add a masked second term in its epilogue?)
     *p.addQuery = 0;
     if (ut && p.Cout > 4) {
@@ -1244,11 +1244,15 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   const bool sb = ut && p.Cout > 4 && !p.stats && conv_sb_plan(p, &sbSplits);
   const int needSplits = std::max(plan.splits, sb ? sbSplits : 1);
   const size_t tailBytes = sb && sbSplits == 1 ? conv_sb_tail_bytes(p.Cout, p.M, p.R) : 0;
-  const size_t needParts = std::max(needSplits > 1 ? (size_t)needSplits * nOut * sizeof(float) : (size_t)0, tailBytes);
+  // The partial tensors of a split reduction must fit; the scratch for the left-over tiles of the streamed-bank kernel is
+  // taken when the workspace has room for it and done without otherwise (every tile by one workgroup): a workspace
+  // sized before a tunable changed, or fixed for a captured graph, stays valid.
+  const size_t needParts = needSplits > 1 ? (size_t)needSplits * nOut * sizeof(float) : (size_t)0;
   const size_t need = needParts && !collect ? align256(needW) + needParts : (slot || asStored ? 0 : needW);
   if (collect) collect->wsUsed = slot || asStored ? 0 : align256(needW);
   if (need && (!ws || wsBytes < need)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace too small (%zu < %zu bytes)", who, wsBytes, need);
   if (need && !aligned16(ws)) return fail(MCN_ILLEGAL_ARGUMENT, "%s: workspace must be 16-byte aligned", who);
+  const bool haveTail = tailBytes && ws && aligned16(ws) && wsBytes >= align256(needW) + tailBytes;
   float* wt = (float*)ws;
   int rc = MCN_SUCCESS;
   if (asStored) {
@@ -1306,7 +1310,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   if (p.addend) return fail(MCN_UNSUPPORTED, "%s: this product cannot add a masked second term in its epilogue", who);
   // banks too large for LDS: stream them past pixels held in registers (conv_sb.hip)
   if (sb && sbSplits == 1) {
-    rc = conv_sb_launch(s, out, in, wt, bias, p, 1, tailBytes ? (float*)((char*)ws + align256(needW)) : nullptr);
+    rc = conv_sb_launch(s, out, in, wt, bias, p, 1, haveTail ? (float*)((char*)ws + align256(needW)) : nullptr);
     return rc ? rc : check_launch(who);
   }
   if (sb || plan.splits > 1) {

@@ -522,6 +522,9 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
   plan->w = w;
   plan->statGroups = 0;
   if (wantStats) {
+    // the sums are taken where whole 32-channel blocks are stored through the output's buffer descriptor: every block
+    // must be whole (no padded channels) and the output under 2 GiB, or some channels' sums would stay zero
+    if (p.Cout != p.coutPad || p.Cout % 32 != 0 || p.outBytes == 0) return false;
     // every wavefront must stay on one channel block: the channel blocks sit side by side in a workgroup
     const int wavesPerGroup = twoFit ? 8 : 16;
     if (wavesPerGroup % w.chanBlocks != 0 || p.beta != 0.f || p.alpha != 1.f) return false;

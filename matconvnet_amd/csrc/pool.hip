@@ -25,6 +25,8 @@
 
 namespace mcn {
 
+bool pool_max_backward_pairs_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, float* derInput,
+                                    const float* x, const float* derOutput, int accumulate);  // pool_pairs.hip
 bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, float* derInput,
                                      const float* x, const float* derOutput, int accumulate);  // pool_stream.hip
 
@@ -1013,6 +1015,9 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
   const int passes = isMax ? kh * kw : p.poolH * p.poolW;
   const bool vecIn = (p.H % 4 == 0) && aligned16(derInput);
 
+  // ---- max pooling, 3x3 windows at stride 2 with padding 1 in front, plane height a multiple of 4
+  if (isMax && pool_max_backward_pairs_launch(s, g, p.outH, p.outW, derInput, x, derOutput, accumulate))
+    return check_launch("mcn_pool_backward");
   // ---- max pooling, plane height a multiple of 4: streaming kernel
   if (isMax && pool_max_backward_stream_launch(s, g, p.outH, p.outW, derInput, x, derOutput, accumulate))
     return check_launch("mcn_pool_backward");

@@ -31,7 +31,6 @@ struct PoolS {
   int maxC;      // widest frame over the tiles of a plane, in columns
   int TW, tilesPerPlane, totalTiles;
   int accumulate;
-  int ablate;  // (experiments only, wrong results: 1 skips the ordered passes, 2 the winner search too)
   int walk;  // 0: tiles dealt round-robin to workgroups; 1: one contiguous run each; 2: round-robin inside each XCD's eighth;
              // 3: planes dealt round-robin to XCDs, a plane's tiles round-robin to that XCD's workgroups
   int KH, nPasses;
@@ -263,7 +262,6 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
       prefetch_tile<OPT, XPT, T>(xr, dr, nxt, tid);
     }
 
-    if (p.ablate < 2) {
     // ---- winner of each owned output: first maximum of its window, scanning column by column
     float best[OPT];
     int code[OPT];  // 8 * column offset + row offset of the winner, -1 when nothing beats -inf
@@ -317,9 +315,7 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
 
     // ---- ordered passes: in pass r the outputs of rank r add into their winner's accumulator
     // (a lane sitting out a pass adds into its private idle slot: a select instead of a masked region)
-    if (p.ablate >= 1) {
-      lds_barrier();
-    } else if (NP > 0) {
+    if (NP > 0) {
 #pragma unroll
       for (int r = 0; r < NP; ++r) {
         float a[OPT];
@@ -342,7 +338,6 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
         lds_barrier();
       }
     }
-    } else { lds_barrier(); }
     prevOut = cur.out;
     prevIn4 = nIn4;
     cur = nxt;
@@ -391,7 +386,6 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   p.Hp = (rows + 3) & ~3;
   p.accumulate = accumulate ? 1 : 0;
   p.walk = tunable("pool_walk", 3);
-  p.ablate = tunable("pool_ablate", 0);
   p.KH = kh;
   p.nPasses = kh * kw;
   p.rankHpk = p.rankWpk = 0;

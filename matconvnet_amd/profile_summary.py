@@ -146,7 +146,7 @@ def main(src, dst):
     put("cfg5/conv_wgrad_mfma", "conv5", "conv_wgrad_mfma")
     put("cfg2/bnorm_sums", "bnorm", "bnorm_sums")
     put("cfg2/bnorm_backward_apply", "bnorm", "bnorm_backward_apply")
-    put("cfg3a/pool", "maxpool", "pool_max_backward_stream")
+    put("cfg3a/pool", "maxpool", "pool_max_backward_pairs")
     put("cfg3b/pool", "avgpool", "pool_backward_avg_tiles")
     with open(os.path.join(dst, "traffic.json"), "w") as f:
         json.dump(traffic, f, indent=1, sort_keys=True)

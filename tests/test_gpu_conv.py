@@ -642,6 +642,34 @@ def test_conv_forward_with_channel_sums_refuses_what_it_cannot_do(capi):
     assert "no such form" in str(e.value)
 
 
+@pytest.mark.parametrize("K", [48, 80, 96])
+def test_conv_forward_with_channel_sums_and_filter_counts_off_the_32_grid(capi, K):
+    """Filter counts that leave a partial 32-channel block (48, 80) have no summing form -- the kernel sums where whole
+    blocks are stored -- and say so; a count it does take (96) gives the sums of every channel, the last block included."""
+    import torch
+    xs, fs = (56, 56, 64, 8), (1, 1, 64, K)
+    g = capi.conv_geom(xs, fs, 1, 0, 1)
+    groups = capi.conv_forward_sums_groups(g)
+    r = np.random.default_rng(K)
+    xd = capi.to_device(F(r.standard_normal(xs) + 0.3))
+    fd = capi.to_device(F(r.standard_normal(fs) * 0.2))
+    if K % 32 != 0:
+        assert groups == 0
+        with pytest.raises(capi.McnError) as e:
+            capi.conv_forward_sums(xd, fd, g)
+        assert "no such form" in str(e.value)
+        return
+    assert groups > 0
+    y, sums = capi.conv_forward_sums(xd, fd, g)
+    assert torch.equal(y, capi.conv_forward(xd, fd, None, g))
+    yd = y.double()
+    s1, s2 = yd.sum(dim=(0, 2, 3)), (yd * yd).sum(dim=(0, 2, 3))
+    tot = sums.sum(dim=1)
+    assert float((tot[:, 0] - s1).abs().max() / s1.abs().max()) < 1e-6
+    assert float((tot[:, 1] - s2).abs().max() / s2.abs().max()) < 1e-6
+    assert float(tot[:, 1].min()) > 0.0
+
+
 def test_conv_backward_data_with_masked_second_term(capi):
     """dzdx = backward-data + the shortcut's share of the derivative behind a ReLU, the mask as one bit per element:
     bit-identical to writing the masked derivative into dzdx and accumulating the convolution's onto it."""

@@ -36,8 +36,13 @@ def test_static_scratch_entry_point_matches_the_workspace_one(capi, given):
         for t in out[:3]:
             t.fill_(float("nan"))
         torch.cuda.synchronize()
+        # the call's defining property: device memory in use is the same before and after it (the first call on a device
+        # also looks the array's address up, which allocates nothing either)
+        free_before, _ = torch.cuda.mem_get_info()
         got = capi.bnorm_backward_static(x, g, dy, 1e-4, moments=mom_in, out=out)
         torch.cuda.synchronize()
+        free_after, _ = torch.cuda.mem_get_info()
+        assert free_after == free_before, (shape, free_before - free_after)
         for name, a, b in zip(("dzdx", "dzdg", "dzdb", "moments"), got, want):
             assert bits_equal(capi.to_host(a), capi.to_host(b)), (shape, name)
 
