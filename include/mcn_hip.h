@@ -246,6 +246,14 @@ MCN_API int mcn_conv_reduce_batch(mcn_stream_t stream, const mcn_conv_reduce_job
 MCN_API int mcn_conv_backward_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* derBias,
                                    const float* derOutput, void* workspace, size_t workspaceBytes);
 
+/* dzdf and dzdb by one call: what vl::nn::Convolution::backward computes when both DERFILTERS and DERBIASES are asked
+   for (bits/nnconv.cu:230-244,280-311).  For first layers (at most four input channels, a filter volume of at most 159
+   elements, 32 or 64 filters) one pass over x and dzdy gives both; other layers run the two products above one after
+   the other.  Workspace: the larger of mcn_conv_workspace_bytes for MCN_CONV_BACKWARD_FILTER and
+   MCN_CONV_BACKWARD_BIAS.  Same results as the two separate calls to rounding (another summation order). */
+MCN_API int mcn_conv_backward_filter_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters, float* derBias,
+                                          const float* x, const float* derOutput, void* workspace, size_t workspaceBytes);
+
 /* ------------------------------------------------------------------------------------------------
  * subsampling with bias -- vl_nnconv with empty FILTERS (the identity filter bank, vl_nnconv.cu:316-321,432-441):
  * replaces Subsample::forwardWithBias / backwardWithBias (bits/nnsubsample.cu:31-216, nnsubsample_gpu.cu).

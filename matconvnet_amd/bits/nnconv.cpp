@@ -3,6 +3,8 @@
 // implicit-GEMM kernel over the whole batch.
 #include "nnconv.hpp"
 
+#include <algorithm>
+
 #include "impl/dispatcher.hpp"
 
 using namespace vl;
@@ -28,8 +30,9 @@ mcn_conv_geom geometry(Convolution const& op, TensorShape const& data, TensorSha
 }
 
 // Scratch from the context, sized by the back-end; NULL with an error recorded when it cannot be had.
-bool scratch(Context& context, mcn_conv_geom const& g, int product, void** ws, size_t* bytes) {
+bool scratch(Context& context, mcn_conv_geom const& g, int product, void** ws, size_t* bytes, int alsoProduct = -1) {
   *bytes = mcn_conv_workspace_bytes(&g, product);
+  if (alsoProduct >= 0) *bytes = std::max(*bytes, mcn_conv_workspace_bytes(&g, alsoProduct));
   *ws = NULL;
   if (*bytes == 0) return true;
   *ws = context.getWorkspace(VLDT_GPU, *bytes);
@@ -195,13 +198,16 @@ ErrorCode Convolution::backwardAccumulate(Tensor& derInput, double derInputMult,
   size_t bytes;
   int rc;
 
-  if (derBias) {
+  // DERBIASES together with DERFILTER in single precision: one call below gives both (first layers take them from the
+  // same pass over DEROUTPUT)
+  const bool biasWithFilter = derBias && derFilter && !isDouble;
+  if (derBias && derBias.getNumElements() != derOutput.getDepth())
+    return context.setError(VLE_IllegalArgument, "Convolution::backward: DERBIASES has the wrong number of elements");
+  if (derBias && !biasWithFilter) {
     // only the extent of DEROUTPUT matters: describe it as a 1x1 convolution over itself
     TensorShape unit(1, 1, derOutput.getDepth(), derOutput.getDepth());
     Convolution plain(context, 1, 1, 0, 0, 0, 0, 1, 1);
     mcn_conv_geom g = geometry(plain, derOutput, unit);
-    if (derBias.getNumElements() != derOutput.getDepth())
-      return context.setError(VLE_IllegalArgument, "Convolution::backward: DERBIASES has the wrong number of elements");
     if (isDouble) {
       rc = mcn_conv_backward_bias_f64(stream, &g, (double*)derBias.getMemory(), (double const*)derOutput.getMemory());
       if (rc) return fromAbi(context, rc, "Convolution::backward");
@@ -246,9 +252,14 @@ ErrorCode Convolution::backwardAccumulate(Tensor& derInput, double derInputMult,
       rc = mcn_conv_backward_filter_f64(stream, &g, (double*)derFilter.getMemory(), (double const*)input.getMemory(),
                                         (double const*)derOutput.getMemory());
     } else {
-      if (!scratch(context, g, MCN_CONV_BACKWARD_FILTER, &ws, &bytes)) return context.getLastError();
-      rc = mcn_conv_backward_filter(stream, &g, (float*)derFilter.getMemory(), (float const*)input.getMemory(),
-                                    (float const*)derOutput.getMemory(), ws, bytes);
+      if (!scratch(context, g, MCN_CONV_BACKWARD_FILTER, &ws, &bytes, biasWithFilter ? MCN_CONV_BACKWARD_BIAS : -1))
+        return context.getLastError();
+      if (biasWithFilter)
+        rc = mcn_conv_backward_filter_bias(stream, &g, (float*)derFilter.getMemory(), (float*)derBias.getMemory(),
+                                           (float const*)input.getMemory(), (float const*)derOutput.getMemory(), ws, bytes);
+      else
+        rc = mcn_conv_backward_filter(stream, &g, (float*)derFilter.getMemory(), (float const*)input.getMemory(),
+                                      (float const*)derOutput.getMemory(), ws, bytes);
     }
     if (rc) return fromAbi(context, rc, "Convolution::backward");
   }

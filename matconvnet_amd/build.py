@@ -19,7 +19,7 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibilit
 # files whose results are compared bit for bit with sequential CPU loops: no FMA contraction at all
 NO_CONTRACT = {"pool.hip", "pool_stream.hip", "pool_pairs.hip", "eltwise.hip", "subsample.hip", "f64.hip", "loss.hip"}
 
-HIP_SOURCES = ["common.hip", "pool.hip", "pool_stream.hip", "pool_pairs.hip", "bnorm.hip", "eltwise.hip", "subsample.hip", "conv.hip", "conv_direct.hip", "conv_mfma.hip", "conv_ws.hip", "conv_sb.hip", "conv_few.hip", "f64.hip", "loss.hip", "yardstick.hip"]
+HIP_SOURCES = ["common.hip", "pool.hip", "pool_stream.hip", "pool_pairs.hip", "bnorm.hip", "eltwise.hip", "subsample.hip", "conv.hip", "conv_direct.hip", "conv_mfma.hip", "conv_ws.hip", "conv_sb.hip", "conv_few.hip", "conv_first.hip", "f64.hip", "loss.hip", "yardstick.hip"]
 
 
 def _run(cmd, quiet_pattern="packed-fp32-ops"):

@@ -86,6 +86,7 @@ PROTOTYPES = {
     "mcn_conv_backward_data_acc": (_i, [_vp, C.POINTER(ConvGeom), _vp, C.c_float, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_filter": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _sz]),
     "mcn_conv_backward_bias": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _sz]),
+    "mcn_conv_backward_filter_bias": (_i, [_vp, C.POINTER(ConvGeom), _vp, _vp, _vp, _vp, _vp, _sz]),
     "mcn_subsample_output_size": (_i, [_i, _i, _i, _i, _i, _i, _i, _i, C.POINTER(_i), C.POINTER(_i)]),
     "mcn_subsample_forward": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i]),
     "mcn_subsample_backward": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i]),
@@ -388,6 +389,17 @@ def conv_backward(x, f, dy, g, want=(True, True, True), ws=None):
         wp, wn = ws.get(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_BIAS))
         check(L.mcn_conv_backward_bias(stream(), C.byref(g), ptr(db), ptr(dy), wp, wn))
     return dx, df, db
+
+
+def conv_backward_filter_bias(x, dy, g, ws=None):
+    """(dzdf, dzdb) by one call (include/mcn_hip.h: mcn_conv_backward_filter_bias)."""
+    ws = ws or _ws
+    L = lib()
+    df, db = empty((g.FH, g.FW, g.FC, g.K)), empty((g.K,))
+    need = max(L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_FILTER), L.mcn_conv_workspace_bytes(C.byref(g), CONV_BACKWARD_BIAS))
+    wp, wn = ws.get(need)
+    check(L.mcn_conv_backward_filter_bias(stream(), C.byref(g), ptr(df), ptr(db), ptr(x), ptr(dy), wp, wn))
+    return df, db
 
 
 def conv_backward_data_acc(dx, mult, f, dy, g, ws=None):

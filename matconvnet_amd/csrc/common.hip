@@ -55,6 +55,10 @@ Tunable g_tunables[] = {
     {"bnorm_one_launch_elems", 8192},  // channels of at most this many elements (and >= 128 of them): sums and apply in one launch
     {"bnorm_reverse_apply", 1},        // second bnorm pass walks planes in reverse (cache reuse)
     {"conv_no_ws", 0},                 // 1: never use the weights-stationary kernel
+    {"conv_first_per_cu", 0},          // > 0: workgroups per compute unit of the first-layer filter gradient (else by its registers)
+    {"conv_first_max_wg", 0},          // > 0: at most this many workgroups in the first-layer filter gradient
+    {"conv_no_first", 0},              // 1: never use the filter-gradient kernel for first layers (few input channels)
+    {"conv_first_no_vec", 0},          // 1: the first-layer filter gradient stages its tiles 4 bytes per lane always
     {"conv_no_few", 0},                // 1: never use the kernel for products with at most four output channels
     {"conv_ws_min_units", 0},          // least number of units for the weights-stationary kernel; 0 = one per two SIMDs
     {"conv_ws_max_slices", 8},         // most slices of output channels its bank may be cut into (1: whole banks only)

@@ -114,7 +114,9 @@ size_t mcn_conv_workspace_bytes(const mcn_conv_geom* g, int product) {
   if (conv_setup(g, "mcn_conv_workspace_bytes", &p)) return 0;
   if (p.N == 0) return 0;
   if (product == MCN_CONV_BACKWARD_BIAS) return (size_t)p.K * bias_groups(p) * sizeof(double);
-  return conv_mfma_workspace_bytes(p, product);
+  size_t bytes = conv_mfma_workspace_bytes(p, product);
+  if (product == MCN_CONV_BACKWARD_FILTER && conv_first_backward_filter_supported(p)) bytes = std::max(bytes, conv_first_workspace_bytes(p));
+  return bytes;
 }
 
 int mcn_conv_forward(mcn_stream_t stream, const mcn_conv_geom* g, float* y, float outMult, const float* x,
@@ -324,6 +326,8 @@ int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float*
   const size_t nf = (size_t)p.FH * p.FW * p.FC * p.K;
   if ((size_t)p.outH * p.outW * p.N == 0) return mcn_fill(stream, derFilters, 0.f, nf);
   if (!x || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter: null tensor");
+  if (!tunable("conv_force_direct", 0) && conv_first_backward_filter_supported(p))
+    return conv_first_backward_filter(as_stream(stream), p, derFilters, nullptr, x, derOutput, workspace, workspaceBytes);
   if (!tunable("conv_force_direct", 0) && conv_mfma_backward_filter_supported(p))
     return conv_backward_filter_mfma(as_stream(stream), p, derFilters, x, derOutput, workspace, workspaceBytes);
   return conv_backward_filter_direct(as_stream(stream), p, derFilters, x, derOutput);
@@ -332,7 +336,9 @@ int mcn_conv_backward_filter(mcn_stream_t stream, const mcn_conv_geom* g, float*
 namespace {
 static_assert(sizeof(ReduceJob) == sizeof(mcn_conv_reduce_job), "a device array of mcn_conv_reduce_job is read as ReduceJob[]");
 bool deferred_available(const ConvP& p) {
-  return !tunable("conv_force_direct", 0) && conv_mfma_backward_filter_supported(p) && (size_t)p.outH * p.outW * p.N != 0;
+  // (first layers have a kernel of their own, which sums its partial banks itself: no deferred form)
+  return !tunable("conv_force_direct", 0) && !conv_first_backward_filter_supported(p) && conv_mfma_backward_filter_supported(p) &&
+         (size_t)p.outH * p.outW * p.N != 0;
 }
 }  // namespace
 
@@ -390,6 +396,22 @@ unsigned mcn_conv_reduce_layout(mcn_conv_reduce_job* jobs, int nJobs) {
 int mcn_conv_reduce_batch(mcn_stream_t stream, const mcn_conv_reduce_job* deviceJobs, int nJobs, unsigned totalBlocks) {
   if (nJobs > 0 && !deviceJobs) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_reduce_batch: null argument");
   return conv_reduce_batch(as_stream(stream), (const ReduceJob*)deviceJobs, nJobs, totalBlocks);
+}
+
+int mcn_conv_backward_filter_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* derFilters, float* derBias,
+                                  const float* x, const float* derOutput, void* workspace, size_t workspaceBytes) {
+  ConvP p;
+  int rc = conv_setup(g, "mcn_conv_backward_filter_bias", &p);
+  if (rc) return rc;
+  if (!derFilters || !derBias) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_bias: null tensor");
+  // a first layer: one pass gives both (the bias gradient is the column of the product that multiplies a row of ones)
+  if ((size_t)p.outH * p.outW * p.N != 0 && x && derOutput && !tunable("conv_force_direct", 0) &&
+      conv_first_backward_filter_supported(p))
+    return conv_first_backward_filter(as_stream(stream), p, derFilters, derBias, x, derOutput, workspace, workspaceBytes);
+  // otherwise the two products one after the other, through the same workspace
+  rc = mcn_conv_backward_filter(stream, g, derFilters, x, derOutput, workspace, workspaceBytes);
+  if (rc) return rc;
+  return mcn_conv_backward_bias(stream, g, derBias, derOutput, workspace, workspaceBytes);
 }
 
 int mcn_conv_backward_bias(mcn_stream_t stream, const mcn_conv_geom* g, float* derBias, const float* derOutput,

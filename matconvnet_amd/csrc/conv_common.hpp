@@ -76,6 +76,12 @@ struct ReduceCtx {
 bool conv_mfma_forward_supported(const ConvP& p);
 bool conv_mfma_backward_data_supported(const ConvP& p);
 bool conv_mfma_backward_filter_supported(const ConvP& p);
+// first layers (few input channels, 32 or 64 filters): filter gradient and, from the same pass, bias gradient
+// (conv_first.hip); dB may be null
+bool conv_first_backward_filter_supported(const ConvP& p);
+size_t conv_first_workspace_bytes(const ConvP& p);
+int conv_first_backward_filter(hipStream_t s, const ConvP& p, float* dF, float* dB, const float* x, const float* dy, void* ws,
+                               size_t wsBytes);
 size_t conv_mfma_workspace_bytes(const ConvP& p, int product);
 // stats / statGroups: also write per-channel partial sums of y and y^2 (see PixP::stats); statQuery: plan only
 int conv_forward_mfma(hipStream_t s, const ConvP& p, float* y, float outMult, const float* x, float inMult,
@@ -202,6 +208,9 @@ __device__ __forceinline__ void store_block_as(floatx16 acc, bufrsrc rsrc, unsig
     for (int r = 0; r < 16; ++r) buffer_store_untracked(acc[r], voffset, rsrc, sblock + (8 * (r / 4) + r % 4) * plane);
     return;
   }
+  // (alpha made opaque here: left visible, the compiler forms the sixteen products before it tests alpha == 1 and the
+  // plain product above pays for them as well)
+  asm volatile("" : "+s"(alpha));
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     float v = alpha * acc[r];

@@ -350,10 +350,12 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
       if (STATS) {
         // what was stored is the accumulator itself (alpha = 1; lanes past the last pixel hold zeros: their loads
         // fetched nothing)
+        // (as instructions that update the sums where they are: the compiler put the results into fresh registers and
+        // copied all 32 back at the end of every unit)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          s1[r] += acc[0][r];
-          s2[r] = fmaf(acc[0][r], acc[0][r], s2[r]);
+          asm("v_add_f32 %0, %0, %1" : "+v"(s1[r]) : "v"(acc[0][r]));
+          asm("v_fmac_f32 %0, %1, %1" : "+v"(s2[r]) : "v"(acc[0][r]));
         }
       }
     } else if (mo < p.M) {
@@ -522,9 +524,10 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
   plan->w = w;
   plan->statGroups = 0;
   if (wantStats) {
-    // the sums are taken where whole 32-channel blocks are stored through the output's buffer descriptor: every block
-    // must be whole (no padded channels) and the output under 2 GiB, or some channels' sums would stay zero
-    if (p.Cout != p.coutPad || p.Cout % 32 != 0 || p.outBytes == 0) return false;
+    // the sums are taken where whole 32-channel blocks are stored through the output's buffer descriptor: no block
+    // may be partial (a block of padding only has nothing to sum) and the output must be under 2 GiB, or some
+    // channels' sums would stay zero
+    if (p.Cout % 32 != 0 || p.outBytes == 0) return false;
     // every wavefront must stay on one channel block: the channel blocks sit side by side in a workgroup
     const int wavesPerGroup = twoFit ? 8 : 16;
     if (wavesPerGroup % w.chanBlocks != 0 || p.beta != 0.f || p.alpha != 1.f) return false;

@@ -40,6 +40,50 @@ CASES = [
 ]
 
 
+# first layers: few input channels, 32 or 64 filters (the filter gradient takes a kernel of its own, which also gives
+# the bias gradient): H, W, C, N, FH, FW, FC, K, stride, pad, dilate
+FIRST_LAYERS = [
+    (32, 32, 3, 5, 5, 5, 3, 32, 1, 2, 1),                     # BASELINE configs[0] at a smaller batch
+    (64, 64, 3, 3, 7, 7, 3, 64, 2, 3, 1),                     # the ResNet stem's geometry on a smaller image
+    (30, 31, 1, 3, 3, 3, 1, 32, (1, 2), (1, 0, 2, 1), 1),     # one channel, rectangular stride, asymmetric padding
+    (17, 16, 4, 2, 5, 3, 4, 64, 1, (0, 1, 1, 0), 1),          # four channels, odd output height
+    (150, 20, 2, 2, 3, 3, 2, 32, (3, 1), 1, 1),               # tall planes: more than one tile per column
+    (9, 40, 3, 2, 2, 2, 3, 64, 1, 0, 1),                      # short planes, even filter
+]
+
+
+@pytest.mark.parametrize("case", FIRST_LAYERS)
+def test_first_layer_filter_and_bias_gradients(capi, ob, case):
+    """Filter gradient of first layers against the oracle, alone and together with the bias gradient
+    (mcn_conv_backward_filter_bias: one pass gives both), and the same call on a layer that is no first layer."""
+    x, f, b = _tensors(case)
+    og = ob.conv_geom(x.shape, f.shape, *case[8:])
+    dy = F(np.random.default_rng(6).standard_normal(ob.conv_out_shape(og)))
+    _check(capi, ob, x, f, b, dy, *case[8:])
+    g = capi.conv_geom(x.shape, f.shape, *case[8:])
+    _, wdf, wdb = ob.conv_backward(x, f, dy, og)
+    df, db = capi.conv_backward_filter_bias(capi.to_device(x), capi.to_device(dy), g)
+    assert rel_max(capi.to_host(df), wdf) <= TOL and rel_max(capi.to_host(db), wdb) <= TOL
+    # three workgroups walk all the tiles, each staging its next tile during the product
+    capi.set_tunable("conv_first_max_wg", 3)
+    try:
+        df, db = capi.conv_backward_filter_bias(capi.to_device(x), capi.to_device(dy), g)
+    finally:
+        capi.set_tunable("conv_first_max_wg", 0)
+    assert rel_max(capi.to_host(df), wdf) <= TOL and rel_max(capi.to_host(db), wdb) <= TOL
+
+
+def test_filter_and_bias_gradients_by_one_call_on_any_layer(capi, ob):
+    case = CASES[9]
+    x, f, b = _tensors(case)
+    og = ob.conv_geom(x.shape, f.shape, *case[8:])
+    dy = F(np.random.default_rng(6).standard_normal(ob.conv_out_shape(og)))
+    g = capi.conv_geom(x.shape, f.shape, *case[8:])
+    _, wdf, wdb = ob.conv_backward(x, f, dy, og)
+    df, db = capi.conv_backward_filter_bias(capi.to_device(x), capi.to_device(dy), g)
+    assert rel_max(capi.to_host(df), wdf) <= TOL and rel_max(capi.to_host(db), wdb) <= TOL
+
+
 def _tensors(case, seed=5):
     H, W, C, N, FH, FW, FC, K, stride, pad, dilate = case
     r = np.random.default_rng(seed)
