@@ -481,6 +481,48 @@ def test_block_with_the_last_relu_mask_kept_as_bits(vl, ob):
         blk.close()
 
 
+def test_timed_schedule_batch_norm_stages_against_the_double_oracle_at_full_size(vl, ob):
+    """The batch-norm stages of the benchmarked schedule (moments from the convolutions' own channel sums, ReLU and the
+    shortcut sum folded into the output pass, the last mask as bits) at N = 32, each against the oracle in double on
+    the stage's OWN inputs -- the block's buffers -- at 1e-5: the moments, what the output pass writes, and the three
+    derivatives of every stage.  (A mask is what the forward pass wrote: r > 0.)"""
+    N = 32
+    w = workloads.bottleneck_case()
+    blk = vl.Bottleneck(N=N, eps=w["eps"], fused=True, packed=True, deferred=True, epilogue_sums=True, mask_bits=True)
+    try:
+        _load(blk, w)
+        blk.run(1)
+        torch.cuda.synchronize()
+        big, small = (56, 56, 256, N), (56, 56, 64, N)
+        shp = dict(a1=small, r1=small, a2=small, r2=small, a3=big, y=big, m1=(64, 2), m2=(64, 2), m3=(256, 2),
+                   da3=big, dr2=small, da2=small, dr1=small, da1=small,
+                   dg1=(64,), db1=(64,), dg2=(64,), db2=(64,), dg3=(256,), db3=(256,))
+        G = {k: blk.get(k, v) for k, v in shp.items()}
+    finally:
+        blk.close()
+    x, dy, eps = w["x"], w["dy"], w["eps"]
+    d = lambda a: F(a, np.float64) if a.ndim > 1 else a.astype(np.float64)
+    errs = {}
+    # forward: moments and the written output (ReLU, and for the last stage the shortcut sum, included)
+    for a, r, m, gk, bk, add in [("a1", "r1", "m1", "g1", "b1", None), ("a2", "r2", "m2", "g2", "b2", None),
+                                 ("a3", "y", "m3", "g3", "b3", x)]:
+        wy, wm = ob.bnorm_forward(d(G[a]), d(w[gk]), d(w[bk]), eps)
+        if add is not None:
+            wy = wy + d(add)
+        errs[m] = rel_max(G[m], wm)
+        errs[r] = rel_max(G[r], np.maximum(wy, 0))
+    # backward: the derivative that enters each stage, masked by what the forward pass wrote
+    for da, dg, db, a, m, gk, dz, r in [("da3", "dg3", "db3", "a3", "m3", "g3", dy, "y"),
+                                        ("da2", "dg2", "db2", "a2", "m2", "g2", G["dr2"], "r2"),
+                                        ("da1", "dg1", "db1", "a1", "m1", "g1", G["dr1"], "r1")]:
+        dn = d(dz) * (G[r] > 0)
+        wdx, wdg, wdb, _ = ob.bnorm_backward(d(G[a]), d(w[gk]), dn, eps, moments=d(G[m]))
+        errs[da], errs[dg], errs[db] = rel_max(G[da], wdx), rel_max(G[dg], wdg), rel_max(G[db], wdb)
+    print("timed schedule, batch-norm stages at N=32:", {k: "%.1e" % v for k, v in errs.items()})
+    for k, v in errs.items():
+        assert v <= 1e-5, (k, v)
+
+
 def test_timed_schedule_with_filter_gradients_on_a_second_stream(vl, ob):
     """The benchmarked schedule with the three filter-gradient matrix kernels on a second stream (they run beside the
     batch-norm derivatives of the layer below; the sums over their reduction splits follow the join, in one launch)
