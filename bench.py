@@ -530,6 +530,9 @@ def bench_conv_single(capi, workloads, reps):
         "backward-data": lambda: capi.check(L.mcn_conv_backward_data(st, C.byref(g), capi.ptr(dx), capi.ptr(f), capi.ptr(dy), wp, wn)),
         "backward-filter": lambda: capi.check(L.mcn_conv_backward_filter(st, C.byref(g), capi.ptr(df), capi.ptr(x), capi.ptr(dy), wp, wn)),
         "backward-bias": lambda: capi.check(L.mcn_conv_backward_bias(st, C.byref(g), capi.ptr(db), capi.ptr(dy), wp, wn)),
+        # (what Convolution::backward calls when both are asked for: one pass over dzdy gives both)
+        "backward-filter and -bias, one call": lambda: capi.check(L.mcn_conv_backward_filter_bias(
+            st, C.byref(g), capi.ptr(df), capi.ptr(db), capi.ptr(x), capi.ptr(dy), wp, wn)),
     }
     rows = []
     for name, fn in calls.items():
@@ -542,7 +545,7 @@ def bench_conv_single(capi, workloads, reps):
         rows.append(row)
 
     def backward():
-        calls["backward-data"](); calls["backward-filter"](); calls["backward-bias"]()
+        calls["backward-data"](); calls["backward-filter and -bias, one call"]()
     t = _event_time(backward, reps * 4, warm=3)
     whole = dict(backward_us=t * 1e6, backward_tflops=2 * flops / t / 1e12, backward_frac_of_mfma_peak=2 * flops / t / PEAK_MFMA_FP32)
     return rows, whole

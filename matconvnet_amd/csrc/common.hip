@@ -57,6 +57,9 @@ Tunable g_tunables[] = {
     {"conv_no_ws", 0},                 // 1: never use the weights-stationary kernel
     {"conv_first_per_cu", 0},          // > 0: workgroups per compute unit of the first-layer filter gradient (else by its registers)
     {"conv_first_max_wg", 0},          // > 0: at most this many workgroups in the first-layer filter gradient
+    {"pool64_tile_kb", 40},
+    {"pool64_walk_per_cu", 0},
+    {"pool64_no_tiles", 0},            // 1: max-pool backward in double never by tiles through LDS
     {"conv_no_first", 0},              // 1: never use the filter-gradient kernel for first layers (few input channels)
     {"conv_first_no_vec", 0},          // 1: the first-layer filter gradient stages its tiles 4 bytes per lane always
     {"conv_no_few", 0},                // 1: never use the kernel for products with at most four output channels

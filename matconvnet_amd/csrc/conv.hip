@@ -138,6 +138,8 @@ int mcn_conv_backward_data_acc(mcn_stream_t stream, const mcn_conv_geom* g, floa
   if (rc) return rc;
   if ((size_t)p.H * p.W * p.C * p.N == 0) return MCN_SUCCESS;
   if (!derInput || !filters || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data: null tensor");
+  if (!tunable("conv_force_direct", 0) && derInputMult == 0.f && conv_first_backward_data_supported(p))
+    return conv_first_backward_data(as_stream(stream), p, derInput, filters, derOutput);
   if (!tunable("conv_force_direct", 0) && conv_mfma_backward_data_supported(p))
     return conv_backward_data_mfma(as_stream(stream), p, derInput, derInputMult, filters, derOutput, workspace, workspaceBytes);
   return conv_backward_data_direct(as_stream(stream), p, derInput, derInputMult, filters, derOutput);
@@ -273,6 +275,8 @@ int mcn_conv_backward_data_packed(mcn_stream_t stream, const mcn_conv_geom* g, f
   if (rc) return rc;
   if ((size_t)p.H * p.W * p.C * p.N == 0) return MCN_SUCCESS;
   if (!derInput || !filters || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data: null tensor");
+  if (!tunable("conv_force_direct", 0) && derInputMult == 0.f && conv_first_backward_data_supported(p))
+    return conv_first_backward_data(as_stream(stream), p, derInput, filters, derOutput);  // (reads the bank as it is stored)
   if (!tunable("conv_force_direct", 0) && conv_mfma_backward_data_supported(p)) {
     PackCtx pk = {PackCtx::kUse, (char*)const_cast<void*>(packed), packedBytes, 0, nullptr};
     return conv_backward_data_mfma(as_stream(stream), p, derInput, derInputMult, filters, derOutput, workspace,

@@ -487,10 +487,202 @@ int first_launch(hipStream_t s, size_t lds, float* partials, const float* x, con
 
 }  // namespace
 
+// ------------------------------------------------------------------------------------------------------------------
+// Input gradient of a first layer (stride 1): dzdx has at most four channels, so the product is short of matrix
+// shape in one direction (bits/nnconv.cu:247-277 for such a layer).  Here it runs on vector FMAs from LDS:
+//   * a workgroup takes a tile of input pixels of one image (whole columns up to 64 rows x a few columns) and stages
+//     the dzdy its windows reach, every filter's plane, by loads that write LDS directly (zero outside the image);
+//   * a lane owns two vertically adjacent pixels and all channels: for a filter and a window column it reads FH + 1
+//     consecutive rows of dzdy from LDS (8-byte reads) and uses each for both pixels -- 2 FH C multiply-adds per
+//     (FH + 1) / 2 reads; the weights are wave-uniform, read as scalars;
+//   * the four wavefronts take a quarter of the filters each; their sums are added in wavefront order through LDS.
+namespace {
+
+struct FirstD {
+  int H, W, N, FW, K, pt, pl, outH, outW;
+  int TH, TW;               // input pixels of a tile
+  int halfTH, cols;         // lanes: pair of rows u = lane % halfTH of column lane / halfTH (cols columns per tile)
+  int LH, LW;               // rows and columns of dzdy a tile reaches: TH + FH - 1, TW + FW - 1
+  int kPer;                 // filters per wavefront
+  int tilesH, tilesW, tiles;
+  int chunks;               // chunks of 64 floats of the staged region [filter][column][row]
+  int stepR, stepC, stepK;  // 256 slots on = stepK filters, stepC columns, stepR rows
+  unsigned dyImgBytes;
+  FastDiv byLH, byLW, byTilesH, byTilesW, byHalfTH, byTH, byTW;
+};
+
+template <int FH, int FW, int C>
+__global__ __launch_bounds__(256) void conv_first_dgrad(float* __restrict__ dx, const float* __restrict__ f,
+                                                        const float* __restrict__ dy, FirstD p) {
+  extern __shared__ float smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const size_t inPlane = (size_t)p.H * p.W, outPlane = (size_t)p.outH * p.outW;
+  int n, rest, tw, th;
+  p.byTilesW.divmod((int)blockIdx.x, &rest, &tw);
+  p.byTilesH.divmod(rest, &n, &th);
+  const int h0 = th * p.TH, w0 = tw * p.TW;
+
+  // ---- dzdy of the tile: slot (filter k, column cc, row rr) is output pixel (h0 + pt - (FH - 1) + rr,
+  // w0 + pl - (FW - 1) + cc); a lane follows its slot from chunk to chunk (256 slots on) by carries
+  {
+    const __amdgpu_buffer_rsrc_t dr =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(dy + (size_t)n * p.K * outPlane), 0, (int)p.dyImgBytes, 0x00020000);
+    int seg, rr, k, cc;
+    p.byLH.divmod(wave * 64 + lane, &seg, &rr);
+    p.byLW.divmod(seg, &k, &cc);
+    const int oh0 = h0 + p.pt - (FH - 1), ow0 = w0 + p.pl - (FW - 1);
+    for (int c = wave; c < p.chunks; c += 4) {
+      const int oh = oh0 + rr, ow = ow0 + cc;
+      const bool in = k < p.K && (unsigned)oh < (unsigned)p.outH && (unsigned)ow < (unsigned)p.outW;
+      const unsigned off = in ? 4u * (unsigned)(k * (int)outPlane + ow * p.outH + oh) : 0x80000000u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(dr, (first_lds_ptr)(smem + c * 64), 4, (int)off, 0, 0, 0);
+      rr += p.stepR;
+      const int carry = rr >= p.LH ? 1 : 0;
+      rr -= carry ? p.LH : 0;
+      cc += p.stepC + carry;
+      const int wrap = cc >= p.LW ? 1 : 0;
+      cc -= wrap ? p.LW : 0;
+      k += p.stepK + wrap;
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  // ---- this lane's two pixels: rows h0 + 2 u, h0 + 2 u + 1 of column w0 + col
+  int col, u;
+  p.byHalfTH.divmod(lane, &col, &u);
+  const int colR = min(col, p.TW - 1);  // (lanes past the tile's columns read a column that exists and write nothing)
+  float acc[2][C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) acc[0][c] = acc[1][c] = 0.f;
+  const int kEnd = min(p.K, (wave + 1) * p.kPer);
+  for (int k = wave * p.kPer; k < kEnd; ++k) {
+    // (the window's columns unrolled: the scalar loads of the weights and the LDS reads of all of them are in flight
+    // before the first multiply)
+#pragma unroll
+    for (int j = 0; j < FW; ++j) {
+      // rows 2 u ... 2 u + FH of column colR + FW - 1 - j: the window rows both pixels reach through column tap j
+      const float2* src = (const float2*)(smem + (k * p.LW + colR + FW - 1 - j) * p.LH + 2 * u);
+      float v[FH + 1];
+#pragma unroll
+      for (int e = 0; e < (FH + 1) / 2; ++e) {
+        const float2 pair = src[e];
+        v[2 * e] = pair.x;
+        v[2 * e + 1] = pair.y;
+      }
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        const float* wv = f + (size_t)FH * (j + FW * (c + C * k));
+#pragma unroll
+        for (int i = 0; i < FH; ++i) {
+          const float w = wv[i];
+          acc[0][c] = fmaf(v[FH - 1 - i], w, acc[0][c]);
+          acc[1][c] = fmaf(v[FH - i], w, acc[1][c]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // ---- the four wavefronts' sums: [wavefront][channel][column][row], added in wavefront order
+  const int T = p.TH * p.TW;
+  if (col < p.TW) {
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      float* dst = smem + (wave * C + c) * T + col * p.TH + 2 * u;
+      dst[0] = acc[0][c];
+      dst[1] = acc[1][c];
+    }
+  }
+  __syncthreads();
+  float* dxImg = dx + (size_t)n * C * inPlane;
+  for (int i = tid; i < C * T; i += 256) {
+    const float sum = ((smem[i] + smem[C * T + i]) + smem[2 * C * T + i]) + smem[3 * C * T + i];
+    int seg, row, c, cw;
+    p.byTH.divmod(i, &seg, &row);
+    p.byTW.divmod(seg, &c, &cw);
+    const int ih = h0 + row, iw = w0 + cw;
+    if (ih < p.H && iw < p.W) dxImg[(size_t)c * inPlane + (size_t)iw * p.H + ih] = sum;
+  }
+}
+
+bool first_data_plan(const ConvP& c, FirstD* out, size_t* lds) {
+  if (c.groups != 1 || c.dy != 1 || c.dx != 1 || c.sy != 1 || c.sx != 1 || c.C > 4 || c.C < 1) return false;
+  if ((c.FH != 3 && c.FH != 5 && c.FH != 7) || c.FW != c.FH) return false;  // (square windows: both loops over them are unrolled)
+  if (c.K < 4 || c.N < 1 || c.H < 2 || c.outH < 1 || c.outW < 1 || tunable("conv_no_first", 0)) return false;
+  if ((size_t)c.K * c.outH * c.outW >= (1u << 29) || (size_t)c.C * c.H * c.W >= (1u << 29)) return false;
+  FirstD p;
+  p.H = c.H; p.W = c.W; p.N = c.N; p.FW = c.FW; p.K = c.K; p.pt = c.pt; p.pl = c.pl; p.outH = c.outH; p.outW = c.outW;
+  const int evenH = (c.H + 1) & ~1;
+  int TH = std::min(evenH, 64);
+  if (evenH > 64) {
+    const int parts = (evenH + 63) / 64;
+    TH = (((evenH + parts - 1) / parts) + 1) & ~1;
+  }
+  p.TH = TH;
+  p.halfTH = TH / 2;
+  p.cols = 64 / p.halfTH;
+  p.TW = std::min(p.cols, c.W);
+  p.LH = TH + c.FH - 1;
+  p.LW = p.TW + c.FW - 1;
+  p.kPer = (c.K + 3) / 4;
+  const size_t region = ((size_t)c.K * p.LW * p.LH + 63) / 64 * 64;
+  const size_t sums = (size_t)4 * c.C * TH * p.TW;
+  const size_t bytes = std::max(region, sums) * sizeof(float);
+  if (bytes > 64 * 1024) return false;
+  p.chunks = (int)(region / 64);
+  p.stepR = 256 % p.LH;
+  p.stepC = (256 / p.LH) % p.LW;
+  p.stepK = (256 / p.LH) / p.LW;
+  p.tilesH = (c.H + TH - 1) / TH;
+  p.tilesW = (c.W + p.TW - 1) / p.TW;
+  const long long tiles = (long long)p.tilesH * p.tilesW * c.N;
+  if (tiles >= (1ll << 30)) return false;
+  p.tiles = (int)tiles;
+  p.dyImgBytes = (unsigned)((size_t)c.K * c.outH * c.outW * 4);
+  p.byLH = FastDiv(p.LH); p.byLW = FastDiv(p.LW); p.byTilesH = FastDiv(p.tilesH); p.byTilesW = FastDiv(p.tilesW);
+  p.byHalfTH = FastDiv(p.halfTH); p.byTH = FastDiv(TH); p.byTW = FastDiv(p.TW);
+  *out = p;
+  *lds = bytes;
+  return true;
+}
+
+template <int FH>
+void first_data_launch(hipStream_t s, int C, size_t lds, float* dx, const float* f, const float* dy, const FirstD& p) {
+  const dim3 grid((unsigned)p.tiles), block(256);
+  switch (C) {
+    case 1: hipLaunchKernelGGL((conv_first_dgrad<FH, FH, 1>), grid, block, lds, s, dx, f, dy, p); break;
+    case 2: hipLaunchKernelGGL((conv_first_dgrad<FH, FH, 2>), grid, block, lds, s, dx, f, dy, p); break;
+    case 3: hipLaunchKernelGGL((conv_first_dgrad<FH, FH, 3>), grid, block, lds, s, dx, f, dy, p); break;
+    default: hipLaunchKernelGGL((conv_first_dgrad<FH, FH, 4>), grid, block, lds, s, dx, f, dy, p); break;
+  }
+}
+
+}  // namespace
+
+bool conv_first_backward_data_supported(const ConvP& c) {
+  FirstD p;
+  size_t lds;
+  return first_data_plan(c, &p, &lds);
+}
+
+// dzdx of a first layer with stride 1 (nothing is accumulated onto it)
+int conv_first_backward_data(hipStream_t s, const ConvP& c, float* dx, const float* f, const float* dy) {
+  FirstD p;
+  size_t lds;
+  if (!first_data_plan(c, &p, &lds)) return fail(MCN_UNSUPPORTED, "mcn_conv_backward_data: not a first layer");
+  KernelTimer timer("conv_first_dgrad", s);
+  if (c.FH == 3) first_data_launch<3>(s, c.C, lds, dx, f, dy, p);
+  else if (c.FH == 5) first_data_launch<5>(s, c.C, lds, dx, f, dy, p);
+  else first_data_launch<7>(s, c.C, lds, dx, f, dy, p);
+  return check_launch("mcn_conv_backward_data");
+}
+
 bool conv_first_backward_filter_supported(const ConvP& c) {
   FirstP p;
   size_t lds;
   int rb, kb;
+  if (c.C > 4) return false;  // (the common answer, before any look-up)
   return !tunable("conv_no_first", 0) && first_plan(c, &p, &lds, &rb, &kb);
 }
 

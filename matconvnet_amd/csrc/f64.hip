@@ -141,28 +141,51 @@ __global__ __launch_bounds__(256) void conv64_backward_bias(double* __restrict__
 // batch_normalize_forward / _backward)
 // ---------------------------------------------------------------------------------------------------------
 
-// One workgroup per channel.  DERS == false: sums of x and x*x, turned into (mean, sigma) in moments[c], moments[C + c].
+// sum of sixteen wavefronts' values, in a fixed order, on every thread
+__device__ __forceinline__ double block_sum16(double v, double* lds) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  double s = 0.0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += lds[i];
+  __syncthreads();
+  return s;
+}
+
+// One workgroup of sixteen wavefronts per channel (a read-only stream: the more wavefronts a CU holds, the more loads
+// are in flight).  DERS == false: sums of x and x*x, turned into (mean, sigma) in moments[c], moments[C + c].
 // DERS == true: sums of dy and x*dy (and, unless the moments are given, of x and x*x as well); writes dzdb, dzdg and
 // the moments.
 template <bool DERS, bool GIVEN>
-__global__ __launch_bounds__(256) void bnorm64_sums(double* __restrict__ moments, double* __restrict__ dG,
-                                                    double* __restrict__ dB, const double* __restrict__ x,
-                                                    const double* __restrict__ dy, int WH, int C, int N, double epsilon) {
-  __shared__ double lds[4];
+__global__ __launch_bounds__(1024) void bnorm64_sums(double* __restrict__ moments, double* __restrict__ dG,
+                                                     double* __restrict__ dB, const double* __restrict__ x,
+                                                     const double* __restrict__ dy, int WH, int C, int N, double epsilon) {
+  __shared__ double lds[16];
   const int c = blockIdx.x;
   double sx = 0.0, sxx = 0.0, sd = 0.0, sxd = 0.0;
   for (int n = 0; n < N; ++n) {
     const size_t base = (size_t)WH * (c + (size_t)C * n);
-    for (int i = threadIdx.x; i < WH; i += 256) {
-      const double v = x[base + i];
+    // (two elements per thread and turn: their loads are issued together)
+    for (int i = threadIdx.x; i < WH; i += 2048) {
+      const bool two = i + 1024 < WH;
+      const double v0 = x[base + i], v1 = two ? x[base + i + 1024] : 0.0;
+      double d0 = 0.0, d1 = 0.0;
+      if (DERS) {
+        d0 = dy[base + i];
+        d1 = two ? dy[base + i + 1024] : 0.0;
+      }
       if (!GIVEN) {
-        sx += v;
-        sxx = fma(v, v, sxx);
+        sx += v0;
+        sxx = fma(v0, v0, sxx);
+        sx += v1;
+        sxx = fma(v1, v1, sxx);
       }
       if (DERS) {
-        const double d = dy[base + i];
-        sd += d;
-        sxd = fma(v, d, sxd);
+        sd += d0;
+        sxd = fma(v0, d0, sxd);
+        sd += d1;
+        sxd = fma(v1, d1, sxd);
       }
     }
   }
@@ -172,14 +195,14 @@ __global__ __launch_bounds__(256) void bnorm64_sums(double* __restrict__ moments
     mean = moments[c];
     sigma = moments[C + c];
   } else {
-    sx = block_sum(sx, lds);
-    sxx = block_sum(sxx, lds);
+    sx = block_sum16(sx, lds);
+    sxx = block_sum16(sxx, lds);
     mean = sx / mass;
     sigma = sqrt(fmax(0.0, sxx / mass - mean * mean) + epsilon);  // sigma includes epsilon (bits/nnbnorm.cu:65-70)
   }
   if (DERS) {
-    sd = block_sum(sd, lds);
-    sxd = block_sum(sxd, lds);
+    sd = block_sum16(sd, lds);
+    sxd = block_sum16(sxd, lds);
   }
   if (threadIdx.x != 0) return;
   if (!GIVEN) {
@@ -192,16 +215,17 @@ __global__ __launch_bounds__(256) void bnorm64_sums(double* __restrict__ moments
   }
 }
 
-// y = (g/sigma)*(x - mean) + b, rounded as written  (bits/nnbnorm.cu:192-203)
+// y = (g/sigma)*(x - mean) + b, rounded as written  (bits/nnbnorm.cu:192-203).  A workgroup works inside one plane
+// (blockIdx.x = c + C n), on slab blockIdx.y of it: the channel's constants (two divisions) are worked out once per thread.
 __global__ __launch_bounds__(256) void bnorm64_forward_apply(double* __restrict__ y, const double* __restrict__ x,
                                                              const double* __restrict__ moments,
                                                              const double* __restrict__ mult, const double* __restrict__ bias,
-                                                             int WH, int C, size_t total) {
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  const int c = (int)((idx / WH) % C);
-  const double G = mult[c] / moments[C + c];
-  y[idx] = G * (x[idx] - moments[c]) + bias[c];
+                                                             int WH, int C, int slab) {
+  const int c = blockIdx.x % C;
+  const double G = mult[c] / moments[C + c], mean = moments[c], b = bias[c];
+  const size_t base = (size_t)blockIdx.x * WH;
+  const int i0 = blockIdx.y * slab, i1 = min(i0 + slab, WH);
+  for (int i = i0 + threadIdx.x; i < i1; i += 256) y[base + i] = G * (x[base + i] - mean) + b;
 }
 
 // dzdx = G1*(dzdy - dzdb/m) - G2*(x - mean),  G1 = g/sigma,  G2 = G1*dzdg/(m*sigma)  (bits/nnbnorm.cu:136-164)
@@ -210,15 +234,15 @@ __global__ __launch_bounds__(256) void bnorm64_backward_apply(double* __restrict
                                                               const double* __restrict__ moments,
                                                               const double* __restrict__ mult, const double* __restrict__ dG,
                                                               const double* __restrict__ dB, int WH, int C, double mass,
-                                                              size_t total) {
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  const int c = (int)((idx / WH) % C);
+                                                              int slab) {
+  const int c = blockIdx.x % C;
   const double mean = moments[c], sigma = moments[C + c];
   const double muz = dB[c] / mass;
   const double G1 = mult[c] / sigma;
   const double G2 = G1 * dG[c] / (mass * sigma);
-  dx[idx] = G1 * (dy[idx] - muz) - G2 * (x[idx] - mean);
+  const size_t base = (size_t)blockIdx.x * WH;
+  const int i0 = blockIdx.y * slab, i1 = min(i0 + slab, WH);
+  for (int i = i0 + threadIdx.x; i < i1; i += 256) dx[base + i] = G1 * (dy[base + i] - muz) - G2 * (x[base + i] - mean);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -306,6 +330,199 @@ __global__ __launch_bounds__(256) void pool64_backward(double* __restrict__ dx, 
       }
     }
   dx[idx] = acc;
+}
+
+// The same sums by tiles through LDS (max only; the kernel above reads each window once per element it holds, from the
+// caches).  A workgroup owns a strip of input columns of one plane: it stages the strip's x with the columns its
+// outputs' windows reach, and those outputs' dzdy; finds every such output's winner once (the same search); then each
+// thread adds, for an element of the strip, the dzdy of the outputs that chose it, in the same order as above -- so
+// the same bits.
+struct Pool64Tile {
+  int TW;          // input columns of a strip
+  int maxXW, maxOW;  // most x columns / output columns a strip stages
+  int items;                             // strips of all planes
+  int rowsIn, colsIn, rowsOut, colsOut;  // threads as rows x columns: of the strip's inputs, of its outputs
+  FastDiv byRowsIn, byRowsOut, bySy, bySx;
+};
+
+// what strip `strip` stages: its owned columns [w0, w1), the outputs [owLo, owLo + nOW) and x columns [xLo, xLo + nXW)
+struct Pool64Strip { int w0, w1, owLo, nOW, xLo, nXW; };
+__host__ __device__ inline Pool64Strip pool64_strip(const Pool64& p, int TW, int strip) {
+  Pool64Strip s;
+  s.w0 = strip * TW;
+  s.w1 = s.w0 + TW < p.W ? s.w0 + TW : p.W;
+  int lo = (s.w0 + p.pl - p.poolW + p.sx) / p.sx, hi = (s.w1 - 1 + p.pl) / p.sx;
+  lo = lo > 0 ? lo : 0;
+  hi = hi < p.outW - 1 ? hi : p.outW - 1;
+  s.owLo = lo;
+  s.nOW = hi >= lo ? hi - lo + 1 : 0;
+  int xLo = s.w0, xHi = s.w1;
+  if (s.nOW > 0) {
+    xLo = xLo < lo * p.sx - p.pl ? xLo : lo * p.sx - p.pl;
+    xHi = xHi > hi * p.sx - p.pl + p.poolW ? xHi : hi * p.sx - p.pl + p.poolW;
+  }
+  xLo = xLo > 0 ? xLo : 0;
+  xHi = xHi < p.W ? xHi : p.W;
+  s.xLo = xLo;
+  s.nXW = xHi - xLo;
+  return s;
+}
+
+// PH, PW, SY, SX > 0: the window and stride are these constants, and the loops over a window / over the outputs that hold
+// an element are unrolled with predicates (same order of comparisons and sums): their LDS reads are independent and
+// in flight together, where the loops with run-time bounds wait for one read per turn.  0: any geometry.
+template <int PH, int PW, int SY, int SX>
+__global__ __launch_bounds__(256) void pool64_max_backward_tiled(double* __restrict__ dx, const double* __restrict__ x,
+                                                                 const double* __restrict__ dy, Pool64 p, Pool64Tile t,
+                                                                 int strips) {
+  extern __shared__ double tile[];
+  const int tid = threadIdx.x;
+  double* xs = tile;                                    // [nXW][H]
+  double* ds = tile + (size_t)t.maxXW * p.H;            // [nOW][outH]
+  int* win = (int*)(ds + (size_t)t.maxOW * p.outH);     // [nOW][outH]: the winner's index in the plane
+  const size_t HW = (size_t)p.H * p.W;
+  // A workgroup walks strips blockIdx.x, blockIdx.x + gridDim.x, ...: the next strip's loads (up to twelve of x and
+  // four of dzdy per thread, into registers) are in flight while this strip is worked on.
+  double vx[12], vd[4];
+  auto fetch = [&](int item) {
+    const int plane = item / strips;
+    const Pool64Strip st = pool64_strip(p, t.TW, item - plane * strips);
+    const double* xp = x + (size_t)plane * HW + (size_t)st.xLo * p.H;
+    const double* dyp = dy + (size_t)plane * p.outH * p.outW + (size_t)st.owLo * p.outH;
+    const int nX = st.nXW * p.H, nD = st.nOW * p.outH;
+#pragma unroll
+    for (int u = 0; u < 12; ++u) vx[u] = tid + u * 256 < nX ? xp[tid + u * 256] : 0.0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) vd[u] = tid + u * 256 < nD ? dyp[tid + u * 256] : 0.0;
+  };
+  int item = blockIdx.x;
+  if (item < t.items) fetch(item);
+  for (; item < t.items; item += gridDim.x) {
+  const int plane = item / strips, strip = item - plane * strips;
+  // owned columns, the outputs whose window holds one of them, and the x columns those windows reach
+  const Pool64Strip st = pool64_strip(p, t.TW, strip);
+  const int w0 = st.w0, w1 = st.w1, owLo = st.owLo, nOW = st.nOW, xLo = st.xLo, nXW = st.nXW;
+  __syncthreads();  // (the strip before this one is done with the tile)
+  {
+    const int nX = nXW * p.H, nD = nOW * p.outH;
+#pragma unroll
+    for (int u = 0; u < 12; ++u)
+      if (tid + u * 256 < nX) xs[tid + u * 256] = vx[u];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (tid + u * 256 < nD) ds[tid + u * 256] = vd[u];
+  }
+  __syncthreads();
+  if (item + (int)gridDim.x < t.items) fetch(item + gridDim.x);
+  // ---- winners: a thread keeps its output row and walks the strip's output columns (the row bounds of its windows
+  // are worked out once)
+  {
+    int cq, oh;
+    t.byRowsOut.divmod(tid, &cq, &oh);
+    if (cq < t.colsOut) {
+      for (; oh < p.outH; oh += t.rowsOut) {
+        int h1 = oh * p.sy - p.pt;
+        const int h2 = min(h1 + p.poolH, p.H);
+        h1 = max(h1, 0);
+        for (int o = cq; o < nOW; o += t.colsOut) {
+          const int ow = owLo + o;
+          int c1 = ow * p.sx - p.pl;
+          const int c2 = min(c1 + p.poolW, p.W);
+          c1 = max(c1, 0);
+          double best = -__builtin_inf();
+          int at = -1;
+          if (PH > 0) {
+            const int hr = oh * SY - p.pt, cr = ow * SX - p.pl;  // the window before clipping
+            double v[PW > 0 ? PW : 1][PH > 0 ? PH : 1];
+#pragma unroll
+            for (int b = 0; b < PW; ++b)
+#pragma unroll
+              for (int a = 0; a < PH; ++a)
+                v[b][a] = xs[min(max(hr + a, 0), p.H - 1) + p.H * (min(max(cr + b, xLo), xLo + nXW - 1) - xLo)];
+#pragma unroll
+            for (int b = 0; b < PW; ++b)
+#pragma unroll
+              for (int a = 0; a < PH; ++a) {
+                const bool in = hr + a >= h1 && hr + a < h2 && cr + b >= c1 && cr + b < c2;
+                if (in && v[b][a] > best) {
+                  best = v[b][a];
+                  at = hr + a + p.H * (cr + b);
+                }
+              }
+          } else {
+            for (int ww = c1; ww < c2; ++ww) {
+              const double* col = xs + p.H * (ww - xLo);
+              for (int hh = h1; hh < h2; ++hh) {
+                const double v = col[hh];
+                if (v > best) {
+                  best = v;
+                  at = hh + p.H * ww;
+                }
+              }
+            }
+          }
+          win[oh + p.outH * o] = at;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // ---- sums: a thread keeps its input row (the output rows whose windows hold it: once) and walks the strip's columns
+  {
+    int cq, h;
+    t.byRowsIn.divmod(tid, &cq, &h);
+    if (cq < t.colsIn) {
+      double* dxp = dx + (size_t)plane * HW + (size_t)w0 * p.H;
+      for (; h < p.H; h += t.rowsIn) {
+        // (a negative numerator can only give a first output below 0, which is clipped to 0 anyway)
+        const int nh = h + p.pt - p.poolH + p.sy;
+        const int ohLo = nh > 0 ? t.bySy.div(nh) : 0, ohHi = min(p.outH - 1, t.bySy.div(h + p.pt));
+        for (int c = cq; c < w1 - w0; c += t.colsIn) {
+          const int w = w0 + c, e = h + p.H * w;
+          const int nw = w + p.pl - p.poolW + p.sx;
+          const int oLo = nw > 0 ? t.bySx.div(nw) : 0, oHi = min(p.outW - 1, t.bySx.div(w + p.pl));
+          double acc = p.accumulate ? dxp[h + p.H * c] : 0.0;
+          if (PH > 0) {
+            constexpr int NR = PH > 0 ? (PH + SY - 1) / (SY > 0 ? SY : 1) : 1, NC = PW > 0 ? (PW + SX - 1) / (SX > 0 ? SX : 1) : 1;
+            int wn[NC][NR];
+            double dv[NC][NR];
+#pragma unroll
+            for (int b = 0; b < NC; ++b)
+#pragma unroll
+              for (int a = 0; a < NR; ++a) {
+                const int j = min(ohLo + a, p.outH - 1) + p.outH * (min(oLo + b, owLo + nOW - 1) - owLo);
+                wn[b][a] = win[j];
+                dv[b][a] = ds[j];
+              }
+#pragma unroll
+            for (int b = 0; b < NC; ++b)
+#pragma unroll
+              for (int a = 0; a < NR; ++a)
+                if (oLo + b <= oHi && ohLo + a <= ohHi && wn[b][a] == e) acc += dv[b][a];
+          } else {
+            for (int ow = oLo; ow <= oHi; ++ow)
+              for (int oh = ohLo; oh <= ohHi; ++oh) {
+                // (the window holds the element: the bounds above are exact for a window clipped to the image)
+                const int j = oh + p.outH * (ow - owLo);
+                if (win[j] == e) acc += ds[j];
+              }
+          }
+          dxp[h + p.H * c] = acc;
+        }
+      }
+    }
+  }
+  }  // (strips of this workgroup)
+}
+
+// the grid of the apply passes: planes x slabs of a plane (1024 elements, or more where a plane has over 65535 of them)
+int plane_slabs(int WH, int C, int N, const char* who, int* slab, int* slabs) {
+  if ((long long)C * N >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
+  int sl = 1024;
+  while ((WH + sl - 1) / sl > 65535) sl *= 2;
+  *slab = sl;
+  *slabs = (WH + sl - 1) / sl;
+  return MCN_SUCCESS;
 }
 
 int blocks_for(size_t total, const char* who, unsigned* blocks) {
@@ -401,17 +618,18 @@ int mcn_bnorm_forward_f64(mcn_stream_t stream, double* y, double* moments, const
   hipStream_t s = as_stream(stream);
   if (!givenMoments) {
     KernelTimer timer("bnorm64_sums", s);
-    hipLaunchKernelGGL((bnorm64_sums<false, false>), dim3((unsigned)C), dim3(256), 0, s, mom, nullptr, nullptr, x, nullptr,
+    hipLaunchKernelGGL((bnorm64_sums<false, false>), dim3((unsigned)C), dim3(1024), 0, s, mom, nullptr, nullptr, x, nullptr,
                        H * W, C, N, epsilon);
     int rc = check_launch("mcn_bnorm_forward_f64");
     if (rc) return rc;
   }
   if (total == 0) return MCN_SUCCESS;
-  unsigned blocks;
-  int rc = blocks_for(total, "mcn_bnorm_forward_f64", &blocks);
+  int slab, slabs;
+  int rc = plane_slabs(H * W, C, N, "mcn_bnorm_forward_f64", &slab, &slabs);
   if (rc) return rc;
   KernelTimer timer("bnorm64_forward_apply", s);
-  hipLaunchKernelGGL(bnorm64_forward_apply, dim3(blocks), dim3(256), 0, s, y, x, mom, multipliers, biases, H * W, C, total);
+  hipLaunchKernelGGL(bnorm64_forward_apply, dim3((unsigned)(C * N), (unsigned)slabs), dim3(256), 0, s, y, x, mom, multipliers,
+                     biases, H * W, C, slab);
   return check_launch("mcn_bnorm_forward_f64");
 }
 
@@ -436,21 +654,21 @@ int mcn_bnorm_backward_f64(mcn_stream_t stream, double* derInput, double* derMul
   {
     KernelTimer timer("bnorm64_sums", s);
     if (givenMoments)
-      hipLaunchKernelGGL((bnorm64_sums<true, true>), dim3((unsigned)C), dim3(256), 0, s, mom, derMultipliers, derBiases, x,
+      hipLaunchKernelGGL((bnorm64_sums<true, true>), dim3((unsigned)C), dim3(1024), 0, s, mom, derMultipliers, derBiases, x,
                          derOutput, H * W, C, N, epsilon);
     else
-      hipLaunchKernelGGL((bnorm64_sums<true, false>), dim3((unsigned)C), dim3(256), 0, s, mom, derMultipliers, derBiases, x,
+      hipLaunchKernelGGL((bnorm64_sums<true, false>), dim3((unsigned)C), dim3(1024), 0, s, mom, derMultipliers, derBiases, x,
                          derOutput, H * W, C, N, epsilon);
     int rc = check_launch("mcn_bnorm_backward_f64");
     if (rc) return rc;
   }
   if (total == 0) return MCN_SUCCESS;
-  unsigned blocks;
-  int rc = blocks_for(total, "mcn_bnorm_backward_f64", &blocks);
+  int slab, slabs;
+  int rc = plane_slabs(H * W, C, N, "mcn_bnorm_backward_f64", &slab, &slabs);
   if (rc) return rc;
   KernelTimer timer("bnorm64_backward_apply", s);
-  hipLaunchKernelGGL(bnorm64_backward_apply, dim3(blocks), dim3(256), 0, s, derInput, x, derOutput, mom, multipliers,
-                     derMultipliers, derBiases, H * W, C, (double)H * W * (double)N, total);
+  hipLaunchKernelGGL(bnorm64_backward_apply, dim3((unsigned)(C * N), (unsigned)slabs), dim3(256), 0, s, derInput, x, derOutput,
+                     mom, multipliers, derMultipliers, derBiases, H * W, C, (double)H * W * (double)N, slab);
   return check_launch("mcn_bnorm_backward_f64");
 }
 
@@ -484,6 +702,54 @@ int mcn_pool_backward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* d
   Pool64 p = {g->H, g->W, oh, ow, g->poolH, g->poolW, g->strideY, g->strideX, g->padTop, g->padLeft, accumulate ? 1 : 0};
   unsigned blocks;
   if ((rc = blocks_for(total, "mcn_pool_backward_f64", &blocks))) return rc;
+  if (isMax && !tunable("pool64_no_tiles", 0)) {
+    // strips of input columns through LDS, when a strip with its halo fits
+    const int sx = g->strideX, sy = g->strideY;
+    for (int TW = 32; TW >= 4; TW /= 2) {
+      const int tw = std::min(TW, g->W);
+      const int nStrips = (g->W + tw - 1) / tw;
+      int maxOW = 1, maxXW = 1;
+      for (int i = 0; i < nStrips; ++i) {
+        const Pool64Strip st = pool64_strip(p, tw, i);
+        maxOW = std::max(maxOW, st.nOW);
+        maxXW = std::max(maxXW, st.nXW);
+      }
+      const size_t bytes = ((size_t)maxXW * g->H + (size_t)maxOW * oh) * sizeof(double) + (size_t)maxOW * oh * sizeof(int);
+      const long long strips = (g->W + tw - 1) / tw, wgs = strips * (long long)g->C * g->N;
+      // (a strip is fetched into registers one strip ahead: twelve x values and four of dzdy per thread at most)
+      if (bytes > (size_t)tunable("pool64_tile_kb", 40) * 1024 || wgs >= (1ll << 31) || sy < 1 || sx < 1 ||
+          (long long)maxXW * g->H > 12 * 256 || (long long)maxOW * oh > 4 * 256)
+        continue;
+      Pool64Tile t;
+      t.TW = tw;
+      t.maxXW = maxXW;
+      t.maxOW = maxOW;
+      t.rowsIn = std::min(g->H, 256);
+      t.colsIn = 256 / t.rowsIn;
+      t.rowsOut = std::min(oh, 256);
+      t.colsOut = 256 / t.rowsOut;
+      t.byRowsIn = FastDiv(t.rowsIn);
+      t.byRowsOut = FastDiv(t.rowsOut);
+      t.bySy = FastDiv(sy);
+      t.bySx = FastDiv(sx);
+      KernelTimer timer("pool64_max_backward_tiled", as_stream(stream));
+      t.items = (int)wgs;
+      int cus = device_compute_units();
+      if (cus <= 0) cus = 256;
+      // (one strip per workgroup measured faster than resident workgroups walking the strips -- 32.6 against 36.7 us
+      // on 112x112x64x8 -- so the walk is only taken when asked for)
+      const int walkPerCu = tunable("pool64_walk_per_cu", 0);
+      const dim3 grid((unsigned)(walkPerCu > 0 ? std::min<long long>(wgs, (long long)cus * walkPerCu) : wgs)), block(256);
+      hipStream_t st = as_stream(stream);
+      if (g->poolH == 3 && g->poolW == 3 && sy == 2 && sx == 2)
+        hipLaunchKernelGGL((pool64_max_backward_tiled<3, 3, 2, 2>), grid, block, bytes, st, derInput, x, derOutput, p, t, (int)strips);
+      else if (g->poolH == 2 && g->poolW == 2 && sy == 2 && sx == 2)
+        hipLaunchKernelGGL((pool64_max_backward_tiled<2, 2, 2, 2>), grid, block, bytes, st, derInput, x, derOutput, p, t, (int)strips);
+      else
+        hipLaunchKernelGGL((pool64_max_backward_tiled<0, 0, 0, 0>), grid, block, bytes, st, derInput, x, derOutput, p, t, (int)strips);
+      return check_launch("mcn_pool_backward_f64");
+    }
+  }
   KernelTimer timer("pool64_backward", as_stream(stream));
   if (isMax)
     hipLaunchKernelGGL(pool64_backward<true>, dim3(blocks), dim3(256), 0, as_stream(stream), derInput, x, derOutput, p, total);

@@ -49,6 +49,10 @@ FIRST_LAYERS = [
     (17, 16, 4, 2, 5, 3, 4, 64, 1, (0, 1, 1, 0), 1),          # four channels, odd output height
     (150, 20, 2, 2, 3, 3, 2, 32, (3, 1), 1, 1),               # tall planes: more than one tile per column
     (9, 40, 3, 2, 2, 2, 3, 64, 1, 0, 1),                      # short planes, even filter
+    (21, 19, 1, 3, 3, 3, 1, 32, 1, 1, 1),                     # stride 1, one channel, odd height: the input gradient's own kernel
+    (40, 12, 3, 2, 7, 7, 3, 64, 1, (3, 3, 2, 4), 1),          # stride 1, 7x7, asymmetric padding
+    (150, 9, 2, 2, 5, 5, 2, 32, 1, (2, 2, 0, 1), 1),          # stride 1, tall planes: more than one tile per column
+    (6, 70, 4, 2, 3, 3, 4, 12, 1, 1, 1),                      # stride 1, 12 filters (no filter-gradient kernel of its own), short and wide
 ]
 
 
@@ -587,6 +591,7 @@ def test_few_output_channels(capi, ob, xs, fs, stride, pad, dilate):
     got = {}
     for off in (0, 1):
         capi.set_tunable("conv_no_few", off)
+        capi.set_tunable("conv_no_first", 1)   # (first layers at stride 1 have another kernel for the input gradient)
         try:
             capi.profile_begin("conv_few_mfma")
             y = capi.conv_forward(xd, fd, bd, cg)
@@ -596,6 +601,7 @@ def test_few_output_channels(capi, ob, xs, fs, stride, pad, dilate):
             launches, _ = capi.profile_end()
         finally:
             capi.set_tunable("conv_no_few", 0)
+            capi.set_tunable("conv_no_first", 0)
         got[off] = launches
         assert rel_max(capi.to_host(y), want) < 2e-4
         assert rel_max(capi.to_host(y2), 0.5 * base.astype(np.float64) + 2.0 * (want.astype(np.float64) - b.reshape(1, 1, -1, 1)) + b.reshape(1, 1, -1, 1)) < 2e-4
