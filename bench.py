@@ -552,8 +552,9 @@ def bench_conv_single(capi, workloads, reps):
 
 
 def bench_double(capi, workloads, reps):
-    """The double-precision instantiation (general one-accumulator-per-output kernels, no MFMA, no LDS: correct, not
-    tuned) on reduced forms of the graded configurations: measured so that its distance to the roofline is on record."""
+    """The double-precision instantiation on reduced forms of the graded configurations (convolutions on the fp64 matrix
+    instruction where a product has sixteen columns or more, max-pool backward by strips through LDS, batch norm as two
+    streaming passes): measured so that its distance to the roofline is on record."""
     import torch
     rows = []
     w = workloads.conv_single()
@@ -562,7 +563,20 @@ def bench_double(capi, workloads, reps):
     flops = 3 * 2.0 * 32 * 32 * 100 * 75 * 32
     t = _event_time(lambda: capi.conv_backward(x, f, dy, g), max(2, reps // 4), warm=1)
     rows.append(dict(op="conv backward (dzdx, dzdf, dzdb), double", workload="configs[0] 5x5x3x32 on 32x32x3x100", call_us=t * 1e6,
-                     achieved=flops / t / 1e12, unit="TFLOP/s", peak=78.6, frac=flops / t / 78.6e12, bound="fp64 vector (no f64 MFMA used)"))
+                     achieved=flops / t / 1e12, unit="TFLOP/s", peak=78.6, frac=flops / t / 78.6e12,
+                     bound="fp64: dzdf on v_mfma_f64_16x16x4_f64, dzdx (3 channels) on vector FMAs"))
+    del x, f, dy
+    # a layer with enough channels for the matrix instruction in every product: configs[3]'s 3x3 convolution
+    xs, fs = (56, 56, 64, 32), (3, 3, 64, 64)
+    g = capi.conv_geom(xs, fs, 1, 1, 1)
+    x = torch.randn(tuple(reversed(xs)), device="cuda", dtype=torch.float64)
+    f = torch.randn(tuple(reversed(fs)), device="cuda", dtype=torch.float64)
+    dy = torch.randn(tuple(reversed(xs)), device="cuda", dtype=torch.float64)
+    flops = 2 * 2.0 * 56 * 56 * 32 * 576 * 64
+    t = _event_time(lambda: capi.conv_backward(x, f, dy, g, want=(True, True, False)), max(2, reps // 4), warm=1)
+    rows.append(dict(op="conv backward (dzdx, dzdf), double", workload="configs[3] conv2 3x3x64x64 on 56x56x64x32", call_us=t * 1e6,
+                     achieved=flops / t / 1e12, unit="TFLOP/s", peak=78.6, frac=flops / t / 78.6e12, bound="fp64 mfma"))
+    del x, f, dy
     H, W, Cc, N = 56, 56, 256, 8
     xb = torch.randn((N, Cc, W, H), device="cuda", dtype=torch.float64)
     dyb = torch.randn((N, Cc, W, H), device="cuda", dtype=torch.float64)

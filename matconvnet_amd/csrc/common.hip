@@ -57,6 +57,7 @@ Tunable g_tunables[] = {
     {"conv_no_ws", 0},                 // 1: never use the weights-stationary kernel
     {"conv_first_per_cu", 0},          // > 0: workgroups per compute unit of the first-layer filter gradient (else by its registers)
     {"conv_first_max_wg", 0},          // > 0: at most this many workgroups in the first-layer filter gradient
+    {"conv64_no_mfma", 0},             // 1: double-precision convolutions never on the matrix instruction
     {"pool64_tile_kb", 40},
     {"pool64_walk_per_cu", 0},
     {"pool64_no_tiles", 0},            // 1: max-pool backward in double never by tiles through LDS

@@ -137,6 +137,195 @@ __global__ __launch_bounds__(256) void conv64_backward_bias(double* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// The three products on the fp64 matrix instruction (groups == 1): C[m][n] = sum over k of A[m][k] B[k][n] with
+//   forward          m = output pixel (all images), n = filter,        k = row of the filter volume;  A = the patch
+//                    element (gathered from x, zero outside the image), B = the bank as stored
+//   backward-data    m = input pixel,               n = input channel, k = (tap, filter);  A = dzdy where the tap of
+//                    that filter lands on an output pixel (zero elsewhere), B = the bank read tap-major
+//   backward-filter  m = row of the filter volume,  n = filter,        k = output pixel (all images), in splits;
+//                    A = the patch element, B = dzdy; partial banks per split, added in split order afterwards
+// v_mfma_f64_16x16x4_f64: lane l gives A[l % 16][l / 16] and B[l / 16][l % 16] and holds C[l / 16 + 4 i][l % 16],
+// i = 0..3.  A workgroup makes a 64 x 64 tile (four wavefronts, 32 x 32 each: four accumulators) in stages of 16
+// along k through LDS; the next stage's operands are fetched into registers while this one is multiplied.  A thread
+// fetches four consecutive k of one m (and of one n): its m is decomposed once, its k once per stage and then by carries.
+// ---------------------------------------------------------------------------------------------------------
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+
+struct Gemm64P {
+  ConvP c;
+  int M, Nn, Kd;       // extents of the product
+  int P, HW, FV, T;    // output pixels / input pixels of an image, rows of the filter volume, taps
+  int chunk;           // backward-filter: k per split (a multiple of 16)
+  double outMult, inMult;
+  FastDiv byP, byOutH, byHW, byH, byFH, byT, bySy, bySx;
+};
+
+template <int KIND>
+__global__ __launch_bounds__(256) void conv64_mfma(double* __restrict__ out, const double* __restrict__ a,
+                                                   const double* __restrict__ b, const double* __restrict__ bias, Gemm64P p) {
+  constexpr int KS = 16, LDA = KS + 1, LDB = 64 + 2;
+  __shared__ double As[64 * LDA];
+  __shared__ double Bs[KS * LDB];
+  const ConvP& c = p.c;
+  const int tid = threadIdx.x, lane = tid & 63, l16 = lane & 15, lk = lane >> 4;
+  const int wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
+  const int kBegin = KIND == 2 ? blockIdx.z * p.chunk : 0;
+  const int kEnd = KIND == 2 ? min(kBegin + p.chunk, p.Kd) : p.Kd;
+
+  // ---- this thread's fetches: element (m0 + fm, k .. k + 3) of A and (k .. k + 3, n0 + fm) of B
+  const int fm = tid & 63, fk = (tid >> 6) * 4;
+  const int m = m0 + fm, n = n0 + fm;
+  // what m means (fixed): KIND 0: output pixel; 1: input pixel; 2: row of the filter volume
+  int mImg = 0, mH = 0, mW = 0, mC = 0;
+  if (KIND == 0) {
+    int q;
+    p.byP.divmod(min(m, p.M - 1), &mImg, &q);
+    p.byOutH.divmod(q, &mW, &mH);
+  } else if (KIND == 1) {
+    int e;
+    p.byHW.divmod(min(m, p.M - 1), &mImg, &e);
+    p.byH.divmod(e, &mW, &mH);
+  } else {
+    int t;
+    p.byT.divmod(min(m, p.M - 1), &mC, &t);
+    p.byFH.divmod(t, &mW, &mH);  // (mW, mH) = the tap (j, i)
+  }
+  double ra[4], rb[4];
+  auto fetch = [&](int k0) {
+    const int k = k0 + fk;
+    if (KIND == 0 || KIND == 1) {
+      // k = t + T * (channel or filter), t = i + FH j
+      int d, t, j, i;
+      p.byT.divmod(k, &d, &t);
+      p.byFH.divmod(t, &j, &i);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        double va = 0.0, vb = 0.0;
+        if (k + u < kEnd) {
+          if (KIND == 0) {
+            const int h = mH * c.sy - c.pt + i * c.dy, w = mW * c.sx - c.pl + j * c.dx;
+            if (m < p.M && (unsigned)h < (unsigned)c.H && (unsigned)w < (unsigned)c.W)
+              va = a[h + (size_t)c.H * (w + (size_t)c.W * (d + (size_t)c.C * mImg))];
+            if (n < p.Nn) vb = b[(size_t)(k + u) + (size_t)p.FV * n];
+          } else {
+            const int nh = mH + c.pt - i * c.dy, nw = mW + c.pl - j * c.dx;
+            if (m < p.M && nh >= 0 && nw >= 0) {
+              const int oh = p.bySy.div(nh), ow = p.bySx.div(nw);
+              if (oh * c.sy == nh && ow * c.sx == nw && oh < c.outH && ow < c.outW)
+                va = a[oh + (size_t)c.outH * (ow + (size_t)c.outW * (d + (size_t)c.K * mImg))];
+            }
+            if (n < p.Nn) vb = b[(size_t)t + (size_t)p.T * (n + (size_t)c.C * d)];
+          }
+        }
+        ra[u] = va;
+        rb[u] = vb;
+        if (++i == c.FH) {
+          i = 0;
+          if (++j == c.FW) {
+            j = 0;
+            ++d;
+          }
+        }
+        t = i + c.FH * j;
+      }
+    } else {
+      // k = output pixel of all images
+      int img, q, ow, oh;
+      p.byP.divmod(min(k, p.Kd - 1), &img, &q);
+      p.byOutH.divmod(q, &ow, &oh);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        double va = 0.0, vb = 0.0;
+        if (k + u < kEnd) {
+          const int h = oh * c.sy - c.pt + mH * c.dy, w = ow * c.sx - c.pl + mW * c.dx;
+          if (m < p.M && (unsigned)h < (unsigned)c.H && (unsigned)w < (unsigned)c.W)
+            va = a[h + (size_t)c.H * (w + (size_t)c.W * (mC + (size_t)c.C * img))];
+          if (n < p.Nn) vb = b[oh + (size_t)c.outH * (ow + (size_t)c.outW * (n + (size_t)c.K * img))];
+        }
+        ra[u] = va;
+        rb[u] = vb;
+        if (++oh == c.outH) {
+          oh = 0;
+          if (++ow == c.outW) {
+            ow = 0;
+            ++img;
+          }
+        }
+      }
+    }
+  };
+
+  doublex4 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = (doublex4){0.0, 0.0, 0.0, 0.0};
+
+  if (kBegin < kEnd) fetch(kBegin);
+  for (int k0 = kBegin; k0 < kEnd; k0 += KS) {
+    __syncthreads();  // (the stage before this one has been multiplied)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      As[fm * LDA + fk + u] = ra[u];
+      Bs[(fk + u) * LDB + fm] = rb[u];
+    }
+    __syncthreads();
+    if (k0 + KS < kEnd) fetch(k0 + KS);
+#pragma unroll
+    for (int kk = 0; kk < KS / 4; ++kk) {
+      double av[2], bv[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) av[i] = As[(32 * wm + 16 * i + l16) * LDA + 4 * kk + lk];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bv[j] = Bs[(4 * kk + lk) * LDB + 32 * wn + 16 * j + l16];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // ---- element (row 32 wm + 16 i + lk + 4 e, column 32 wn + 16 j + l16) of the tile is acc[i][j][e]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int row = m0 + 32 * wm + 16 * i + lk + 4 * e, col = n0 + 32 * wn + 16 * j + l16;
+        if (row >= p.M || col >= p.Nn) continue;
+        const double v = acc[i][j][e];
+        if (KIND == 0) {
+          int img, q;
+          p.byP.divmod(row, &img, &q);
+          const size_t at = (size_t)q + (size_t)p.P * (col + (size_t)c.K * img);
+          double r0 = p.inMult * v;
+          if (p.outMult != 0.0) r0 = fma(p.outMult, out[at], r0);
+          if (bias) r0 += bias[col];
+          out[at] = r0;
+        } else if (KIND == 1) {
+          int img, el;
+          p.byHW.divmod(row, &img, &el);
+          out[(size_t)el + (size_t)p.HW * (col + (size_t)c.C * img)] = v;
+        } else {
+          // rows are t + T c here as in the bank (row = the stored index of the filter volume)
+          out[(size_t)blockIdx.z * p.FV * c.K + (size_t)row + (size_t)p.FV * col] = v;
+        }
+      }
+}
+
+// dF[e] = sum over the splits' partial banks, in split order
+__global__ __launch_bounds__(256) void conv64_sum_splits(double* __restrict__ df, const double* __restrict__ partials, size_t n,
+                                                         int splits) {
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= n) return;
+  double s = 0.0;
+  for (int i = 0; i < splits; ++i) s += partials[(size_t)i * n + e];
+  df[e] = s;
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // batch normalisation (bits/nnbnorm.cu:46-164: compute_moment, compute_ders, compute_ders_and_moments,
 // batch_normalize_forward / _backward)
 // ---------------------------------------------------------------------------------------------------------
@@ -515,6 +704,31 @@ __global__ __launch_bounds__(256) void pool64_max_backward_tiled(double* __restr
   }  // (strips of this workgroup)
 }
 
+// The matrix-instruction form of a product (kind 0 forward, 1 backward-data, 2 backward-filter): one filter group,
+// every extent inside 31 bits, and at least sixteen columns of the product (fewer: the one-accumulator kernels above
+// multiply nothing in vain, a 64-wide tile would).
+bool gemm64_plan(const ConvP& c, int kind, Gemm64P* out) {
+  if (c.groups != 1 || tunable("conv64_no_mfma", 0)) return false;
+  const long long P = (long long)c.outH * c.outW, HW = (long long)c.H * c.W, T = (long long)c.FH * c.FW, FV = T * c.C;
+  const long long M = kind == 0 ? P * c.N : (kind == 1 ? HW * c.N : FV);
+  const long long Nn = kind == 1 ? c.C : c.K;
+  const long long Kd = kind == 0 ? FV : (kind == 1 ? T * c.K : P * c.N);
+  if (M < 1 || Nn < 16 || Kd < 1 || M >= (1ll << 30) || Kd >= (1ll << 30) || FV >= (1ll << 30) || (M + 63) / 64 >= (1ll << 31) ||
+      (Nn + 63) / 64 > 65535)
+    return false;
+  Gemm64P p;
+  p.c = c;
+  p.M = (int)M; p.Nn = (int)Nn; p.Kd = (int)Kd;
+  p.P = (int)P; p.HW = (int)HW; p.FV = (int)FV; p.T = (int)T;
+  p.chunk = (int)Kd;
+  p.outMult = 0.0;
+  p.inMult = 1.0;
+  p.byP = FastDiv((int)std::max(1ll, P)); p.byOutH = FastDiv(std::max(1, c.outH)); p.byHW = FastDiv((int)std::max(1ll, HW));
+  p.byH = FastDiv(std::max(1, c.H)); p.byFH = FastDiv(c.FH); p.byT = FastDiv((int)T); p.bySy = FastDiv(c.sy); p.bySx = FastDiv(c.sx);
+  *out = p;
+  return true;
+}
+
 // the grid of the apply passes: planes x slabs of a plane (1024 elements, or more where a plane has over 65535 of them)
 int plane_slabs(int WH, int C, int N, const char* who, int* slab, int* slabs) {
   if ((long long)C * N >= (1ll << 31)) return fail(MCN_UNSUPPORTED, "%s: tensor too large", who);
@@ -547,6 +761,15 @@ int mcn_conv_forward_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* y,
   const size_t total = (size_t)p.outH * p.outW * p.K * p.N;
   if (total == 0) return MCN_SUCCESS;
   if (!y || !x || !filters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_forward_f64: null tensor");
+  Gemm64P gp;
+  if (gemm64_plan(p, 0, &gp)) {
+    gp.outMult = outMult;
+    gp.inMult = inMult;
+    KernelTimer timer("conv64_mfma", as_stream(stream));
+    hipLaunchKernelGGL(conv64_mfma<0>, dim3((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64)), dim3(256), 0,
+                       as_stream(stream), y, x, filters, bias, gp);
+    return check_launch("mcn_conv_forward_f64");
+  }
   unsigned blocks;
   if ((rc = blocks_for(total, "mcn_conv_forward_f64", &blocks))) return rc;
   KernelTimer timer("conv64_forward", as_stream(stream));
@@ -563,6 +786,13 @@ int mcn_conv_backward_data_f64(mcn_stream_t stream, const mcn_conv_geom* g, doub
   const size_t total = (size_t)p.H * p.W * p.C * p.N;
   if (total == 0) return MCN_SUCCESS;
   if (!derInput || !filters || !derOutput) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_data_f64: null tensor");
+  Gemm64P gp;
+  if (gemm64_plan(p, 1, &gp)) {
+    KernelTimer timer("conv64_mfma", as_stream(stream));
+    hipLaunchKernelGGL(conv64_mfma<1>, dim3((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64)), dim3(256), 0,
+                       as_stream(stream), derInput, derOutput, filters, nullptr, gp);
+    return check_launch("mcn_conv_backward_data_f64");
+  }
   unsigned blocks;
   if ((rc = blocks_for(total, "mcn_conv_backward_data_f64", &blocks))) return rc;
   KernelTimer timer("conv64_backward_data", as_stream(stream));
@@ -580,6 +810,42 @@ int mcn_conv_backward_filter_f64(mcn_stream_t stream, const mcn_conv_geom* g, do
   const size_t total = (size_t)p.FH * p.FW * p.FC * p.K;
   if ((size_t)p.outH * p.outW * p.N != 0 && (!x || !derOutput))
     return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_filter_f64: null tensor");
+  Gemm64P gp;
+  if ((size_t)p.outH * p.outW * p.N != 0 && gemm64_plan(p, 2, &gp) && gp.M >= 16) {
+    // the pixels in splits, so that the launch fills the chip about twice; the partial banks live in memory taken from
+    // (and given back to) the stream's pool
+    hipStream_t st = as_stream(stream);
+    int cus = device_compute_units();
+    if (cus <= 0) cus = 256;
+    const long long tiles = (long long)((gp.M + 63) / 64) * ((gp.Nn + 63) / 64);
+    long long splits = std::max(1ll, std::min<long long>((2ll * cus + tiles - 1) / tiles, (gp.Kd + 255) / 256));
+    splits = std::min(splits, 65535ll);
+    gp.chunk = (int)(((gp.Kd + splits - 1) / splits + 15) / 16 * 16);
+    splits = (gp.Kd + gp.chunk - 1) / gp.chunk;
+    void* partials = nullptr;
+    if (splits > 1 && hipMallocAsync(&partials, (size_t)splits * total * sizeof(double), st) != hipSuccess) {
+      (void)hipGetLastError();
+      partials = nullptr;
+      splits = 1;
+      gp.chunk = gp.Kd;
+    }
+    {
+      KernelTimer timer("conv64_mfma", st);
+      hipLaunchKernelGGL(conv64_mfma<2>, dim3((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64), (unsigned)splits),
+                         dim3(256), 0, st, splits > 1 ? (double*)partials : derFilters, x, derOutput, nullptr, gp);
+    }
+    rc = check_launch("mcn_conv_backward_filter_f64");
+    if (splits > 1) {
+      if (!rc) {
+        KernelTimer timer("conv64_sum_splits", st);
+        hipLaunchKernelGGL(conv64_sum_splits, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, derFilters,
+                           (const double*)partials, total, (int)splits);
+        rc = check_launch("mcn_conv_backward_filter_f64");
+      }
+      if (hipFreeAsync(partials, st) != hipSuccess) (void)hipGetLastError();
+    }
+    return rc;
+  }
   KernelTimer timer("conv64_backward_filter", as_stream(stream));
   hipLaunchKernelGGL(conv64_backward_filter, dim3((unsigned)total), dim3(256), 0, as_stream(stream), derFilters, x, derOutput,
                      p);

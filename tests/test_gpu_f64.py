@@ -24,6 +24,9 @@ CONV_CASES = [
     ((6, 6, 8, 3), (1, 1, 8, 16), 1, 0, 1),
     ((5, 5, 4, 2), (5, 5, 4, 7), 1, 0, 1),                   # fully connected
     ((32, 32, 3, 4), (5, 5, 3, 32), 1, 2, 1),                # benchmark configuration 1, four images
+    ((14, 13, 16, 3), (3, 3, 16, 24), 1, 1, 1),              # sixteen and more columns in every product: the matrix instruction
+    ((15, 12, 20, 2), (3, 2, 20, 70), (2, 1), (1, 0, 2, 1), (1, 2)),   # the same with stride, dilation, partial tiles
+    ((9, 9, 64, 2), (1, 1, 64, 64), 1, 0, 1),                # 1x1
 ]
 
 POOL_GEOMS = [
