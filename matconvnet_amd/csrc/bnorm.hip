@@ -510,7 +510,7 @@ __global__ __launch_bounds__(256) void bnorm_forward_apply(float* __restrict__ y
 
 int image_groups(int WH, int N) {
   // one plane per workgroup unless planes are small; then enough planes to own ~bnorm_block_elems
-  const int want = std::max(tunable("bnorm_block_elems", 4096), 1);
+  const int want = 4096;
   const int perBlock = std::max(1, want / std::max(WH, 1));
   return std::max(1, (N + perBlock - 1) / perBlock);
 }
@@ -529,8 +529,8 @@ int setup(const char* who, int H, int W, int C, int N, double epsilon, BnormP* p
     p->groups = 1;
     p->oneLaunch = 1;
   }
-  p->reverse = tunable("bnorm_reverse_apply", 1) ? 1 : 0;
-  p->walk = tunable("bnorm_walk", 1);
+  p->reverse = 1;
+  p->walk = 1;
   for (int v = 0; v < 2; ++v) {
     const int accesses = v ? p->WH / 4 : p->WH;  // per plane
     int shift = 4;                               // teams of 16 ... 256 threads
@@ -850,7 +850,7 @@ static int bnorm_backward_any(const char* who, mcn_stream_t stream, float* derIn
       if (vec) hipLaunchKernelGGL((bnorm_sums<1, true>), grid, block, 0, s, x, derOutput, partials, p);
       else hipLaunchKernelGGL((bnorm_sums<1, false>), grid, block, 0, s, x, derOutput, partials, p);
     } else {
-      if (vec && !tunable("bnorm_sums_scalar", 0)) hipLaunchKernelGGL((bnorm_sums<2, true>), grid, block, 0, s, x, derOutput, partials, p);
+      if (vec) hipLaunchKernelGGL((bnorm_sums<2, true>), grid, block, 0, s, x, derOutput, partials, p);
       else hipLaunchKernelGGL((bnorm_sums<2, false>), grid, block, 0, s, x, derOutput, partials, p);
     }
   }

@@ -85,8 +85,7 @@ __global__ __launch_bounds__(256) void conv_bias_finish(float* __restrict__ db, 
 }
 
 int bias_groups(const ConvP& p) {
-  int target = tunable("conv_bias_blocks", 0);
-  if (target <= 0) target = 2048;
+  const int target = 2048;
   const int P = p.outH * p.outW;
   const int perBlock = std::max(1, 4096 / std::max(P, 1));  // at least ~4096 elements per workgroup
   const int maxGroups = std::max(1, (p.N + perBlock - 1) / perBlock);

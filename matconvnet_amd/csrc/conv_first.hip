@@ -371,7 +371,7 @@ bool first_plan(const ConvP& c, FirstP* out, size_t* lds, int* rb, int* kb) {
   p.H = c.H; p.W = c.W; p.Cin = c.C; p.N = c.N; p.FH = c.FH; p.FW = c.FW; p.K = c.K; p.R = R;
   p.sy = c.sy; p.sx = c.sx; p.pt = c.pt; p.pl = c.pl; p.outH = c.outH; p.outW = c.outW;
   // 16 bytes per lane when every group of four rows is whole: in the planes and in the tiles
-  const int vec = (c.outH % 4 == 0 && c.H % 4 == 0 && !tunable("conv_first_no_vec", 0)) ? 1 : 0;
+  const int vec = (c.outH % 4 == 0 && c.H % 4 == 0) ? 1 : 0;
   p.vec = vec;
   // tile: whole columns of the output up to 64 rows (even; a multiple of four for 16-byte loads), and some columns:
   // at most 256 pixels, and two buffers for each of the workgroups that share a compute unit (as many as the
@@ -415,8 +415,7 @@ bool first_plan(const ConvP& c, FirstP* out, size_t* lds, int* rb, int* kb) {
     const long long atOnce = cap > 0 ? cap : (long long)cus * std::min<size_t>(4, (160 * 1024) / (one + 1024));
     if (floats(TW) * sizeof(float) <= 38 * 1024 && tiles <= atOnce) walk = false;
   }
-  const int asked = tunable("conv_first_per_cu", 0);
-  const int perCu = asked > 0 ? std::min(4, asked) : first_waves(c.K / 32, (R + 1 + 31) / 32);
+  const int perCu = first_waves(c.K / 32, (R + 1 + 31) / 32);
   if (walk) {
     const size_t budget = (160 * 1024 / perCu - 1024) / 2;
     TW = widest(budget);

@@ -131,8 +131,7 @@ __global__ __launch_bounds__(256) void conv_pack_many(const PackJob* __restrict_
 // sooner by many workgroups of one element per thread than by a handful of tiles); the flags for `tapMajor`
 int pack_flags(const TapSet& ts, int backward, bool tapMajor, int rPad, int coutPad, bool batched) {
   const bool tiled = !backward && ts.nI == ts.FH && ts.nJ == ts.FW && ts.i0 == 0 && ts.j0 == 0 && ts.iStep == 1 &&
-                     ts.jStep == 1 && (batched || (long long)((rPad + 63) / 64) * ((coutPad + 63) / 64) >= 32) &&
-                     tunable("conv_pack_tiled", 1);
+                     ts.jStep == 1 && (batched || (long long)((rPad + 63) / 64) * ((coutPad + 63) / 64) >= 32);
   return (tapMajor ? 1 : 0) | (tiled ? 2 : 0);
 }
 unsigned pack_blocks(int flags, int rPad, int coutPad) {
@@ -993,8 +992,7 @@ ConvP group_view(const ConvP& p) {
 // backward-data product uses one.
 ConvP fc_view(const ConvP& p) {
   if (!(p.groups == 1 && p.FH == p.H && p.FW == p.W && p.pt == 0 && p.pl == 0 && p.outH == 1 && p.outW == 1 &&
-        p.dy == 1 && p.dx == 1) || (p.H == 1 && p.W == 1) || (long long)p.H * p.W * p.C >= (1ll << 31) ||
-      tunable("conv_no_fc_view", 0))
+        p.dy == 1 && p.dx == 1) || (p.H == 1 && p.W == 1) || (long long)p.H * p.W * p.C >= (1ll << 31))
     return p;
   ConvP v = p;
   v.C = v.FC = p.H * p.W * p.C;
@@ -1027,22 +1025,19 @@ int pick_rows_tile(const ConvP& p) {
   if (FV > 128 && FV <= 192 && BA == 64 && !tunable("conv_wgrad_no_wide_rows", 0)) return 192;
   // a volume that 192-row tiles cover exactly and 128-row tiles do not (3x3x64 = 576 rows: three tiles instead of
   // four and a half, and 48 instead of 32 MFMAs per wavefront between two barriers)
-  if (FV % 192 == 0 && FV % 128 != 0 && BA == 64 && tunable("conv_wgrad_wide_rows_exact", 1)) return 192;
+  if (FV % 192 == 0 && FV % 128 != 0 && BA == 64) return 192;
   return 128;
 }
 
 int wgrad_splits(const ConvP& p, int* tilesOut) {
   const int BA = pick_channels_tile(p.K), BB = pick_rows_tile(p);
   const int tiles = ((p.K + BA - 1) / BA) * ((p.FH * p.FW * p.FC + BB - 1) / BB);
-  int target = tunable("conv_wgrad_blocks", 0);
   // two workgroups per CU; one when a workgroup's share of a 1x1 layer would be under ~10 MFLOP with several tiles
   // to write (the partial banks then cost more than the idle half: 14x14 and 7x7 1x1 layers of ResNet-50 at 32
   // images 46.6 -> 44.8 us, 54.6 -> 50.0 us), or when the whole bank is one tile
-  if (target <= 0) {
-    const double flops = 2.0 * p.outH * p.outW * p.N * (double)p.FH * p.FW * p.FC * p.K;
-    const bool small1x1 = p.FH * p.FW == 1 && flops < 5e9 && (tiles >= 4 || tiles == 1);
-    target = small1x1 && !tunable("conv_wgrad_no_small_rule", 0) ? 256 : 512;
-  }
+  const double flops = 2.0 * p.outH * p.outW * p.N * (double)p.FH * p.FW * p.FC * p.K;
+  const bool small1x1 = p.FH * p.FW == 1 && flops < 5e9 && (tiles >= 4 || tiles == 1);
+  const int target = small1x1 ? 256 : 512;
   const long long chunks = ((long long)p.outH * p.outW * p.N + 31) / 32;
   long long s = std::max<long long>(1, target / tiles);
   s = std::min<long long>(s, std::max<long long>(1, chunks / 4));  // at least 4 reduction steps per split
@@ -1072,8 +1067,6 @@ void launch_pix(hipStream_t s, float* out, const float* in, const float* wt, con
 void launch_shape(hipStream_t s, int shape, float* out, const float* in, const float* wt, const float* bias, const PixP& p,
                   bool ut) {
   const int BA = pick_channels_tile(p.Cout);
-  const int forced = tunable("conv_pix_tile", 0);
-  if (forced) shape = forced;
   if ((shape == 1 || shape == 5 || shape == 7) && BA != 128) shape = BA == 64 ? 2 : 3;
   if ((shape == 2 || shape == 4 || shape == 6) && BA != 64) shape = BA == 128 ? 1 : 3;
   if (shape == 3 && BA != 32) shape = BA == 128 ? 1 : 2;
@@ -1107,7 +1100,7 @@ int launch_wgrad(hipStream_t s, dim3 grid, float* out, const float* x, const flo
   // holds one of its workgroups at a time and the other stream's kernels keep the rest of the CU.
   size_t ldsAsk = lds;
   if (stream_beside(s)) {
-    ldsAsk = std::max(lds, (size_t)std::min(std::max(tunable("conv_wgrad_beside_kb", 84), 0), 128) * 1024);
+    ldsAsk = std::max(lds, (size_t)84 * 1024);
     static std::atomic<bool> widened[kMaxDevices];
     if (ldsAsk > 64 * 1024 && ldsAsk > lds && dev >= 0 && dev < kMaxDevices && !widened[dev].load(std::memory_order_acquire)) {
       if (hipFuncSetAttribute((const void*)conv_wgrad_mfma<WA, WB, NWA, NWB, UT, DIRECT, DEEP>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1141,10 +1134,6 @@ PixPlan plan_pix(int Cout, long long M, int R) {
   if (BA == 128) { plan.shape = M <= 32 ? 7 : (blocks(128) >= 2048 ? 1 : 5); px = plan.shape == 7 ? 32 : (plan.shape == 1 ? 128 : 64); }
   else if (BA == 64) { plan.shape = blocks(256) >= 2048 ? 2 : (blocks(128) >= 2048 ? 4 : 6); px = plan.shape == 2 ? 256 : (plan.shape == 4 ? 128 : 64); }
   else { plan.shape = 3; px = 256; }
-  if (const int forced = tunable("conv_pix_tile", 0)) {  // (experiments: a shape that fits the channel tile)
-    static const int pxOf[8] = {0, 128, 256, 256, 128, 64, 64, 32}, baOf[8] = {0, 128, 64, 32, 64, 128, 64, 128};
-    if (forced >= 1 && forced <= 7 && baOf[forced] == BA) { plan.shape = forced; px = pxOf[forced]; }
-  }
   // fewer than two workgroups per CU with a long reduction each: split it, down to 12 steps of 16 rows per
   // workgroup.  How many ways: the count with the least modelled time -- the busiest CU's workgroups (dealt evenly)
   // times their steps at the rate that many resident workgroups reach, plus the partial results written and read
@@ -1155,13 +1144,13 @@ PixPlan plan_pix(int Cout, long long M, int R) {
   plan.splits = 1;
   const long long nb = blocks(px);
   const int nSteps = (R + 15) / 16;
-  const int maxBlocks = tunable("conv_split_max_blocks", 512), minSteps = tunable("conv_split_min_steps", 12);
+  const int maxBlocks = 512, minSteps = 12;
   if (nb <= maxBlocks && nSteps >= 4 * minSteps && !tunable("conv_no_split", 0)) {
     const int cus = std::max(1, device_compute_units());
     const double stepUs = 32.0 * BA * px / (157.3e6 / 256.0);           // one step of one tile on one CU
     const double partUs = 2.0 * (double)M * Cout * sizeof(float) / 5e6;  // one split's partial results, out and back
     double best = 0;
-    for (int s = 1; s <= std::min(nSteps / minSteps, tunable("conv_split_most", 16)); ++s) {
+    for (int s = 1; s <= std::min(nSteps / minSteps, 16); ++s) {
       // (a CU's workgroups share its matrix pipes; with few of them the pipes wait for loads and barriers: rates measured
       // on 3x3x256x256 over 14x14x256x32 with 1, 2, 3 and 4 workgroups to a CU)
       static const double rate[5] = {0, 0.63, 0.80, 0.85, 0.88};
@@ -1170,7 +1159,6 @@ PixPlan plan_pix(int Cout, long long M, int R) {
       if (s == 1 || cost < best) { best = cost; plan.splits = s; }
     }
   }
-  if (const int forcedSplits = tunable("conv_split_force", 0)) plan.splits = std::max(1, std::min(forcedSplits, nSteps));
   return plan;
 }
 
@@ -1275,7 +1263,7 @@ int run_pix(hipStream_t s, const char* who, float* out, const float* in, const f
   {
     // (loads straight into LDS in the tiled kernel: both operands behind buffer descriptors of less than 2 GiB)
     const long long ib = inSpan * 4, wb = (long long)rPad * p.coutPad * 4;
-    const bool direct = ut && ib < (1ll << 31) && wb < (1ll << 31) && tunable("conv_pix_direct", 1);
+    const bool direct = ut && ib < (1ll << 31) && wb < (1ll << 31);
     p.inBytes = direct ? (unsigned)ib : 0u;
     p.wtBytes = direct ? (unsigned)wb : 0u;
   }
@@ -1381,7 +1369,7 @@ Axis stride_axis(int phase, int pad, int dil, int stride, int taps) {
 int multi_classes(const ConvP& p, Wide wd, size_t* bankBytes) {
   if (bankBytes) *bankBytes = 0;
   if ((p.sy == 1 && p.sx == 1) || !tunable("conv_pix_multi", 1)) return 0;
-  if (p.K % 16 != 0 || tunable("conv_no_uniform_tap", 0) || !tunable("conv_pix_direct", 1)) return 0;
+  if (p.K % 16 != 0 || tunable("conv_no_uniform_tap", 0)) return 0;
   const long long inSpan = (long long)(p.N - 1) * wd.yImg + (long long)p.K * p.outH * p.outW;
   if (inSpan * 4 >= (1ll << 31)) return 0;
   const int BA = pick_channels_tile(p.C);
@@ -1401,7 +1389,7 @@ int multi_classes(const ConvP& p, Wide wd, size_t* bankBytes) {
       banks += align256((size_t)bank);
       tiles += (M + 63) / 64 * tilesA;
     }
-  if (n < 2 || n > kMaxMulti || tiles > tunable("conv_pix_multi_tiles", 4096)) return 0;
+  if (n < 2 || n > kMaxMulti || tiles > 4096) return 0;
   if (bankBytes) *bankBytes = banks;
   return n;
 }
@@ -1737,12 +1725,12 @@ int backward_filter_group(hipStream_t s, const ConvP& p, Wide wd, bool ut, float
   // between the MFMAs: 12-18 % on every layer measured (1x1 layers of ResNet-50 at 32 images 44.3 -> 37.4 us, 3x3x64x64 on
   // 56x56 78.8 -> 67.9 us, 3x3x256x256 on 56x56x256x64 1.95 -> 1.74 ms).  Issued all at once at the top of a step the same
   // loads were a gain only for short launches and a loss for long ones (1.96 -> 2.09 ms).
-  const bool direct = ut && p.K % BA == 0 && tunable("conv_wgrad_direct", 1);
+  const bool direct = ut && p.K % BA == 0;
   if (direct && wide) {
     rc = launch_wgrad<1, 3, 2, 2, true, true>(s, grid, target, x, dy, q);
   } else if (direct && BA == 128) {
     // (128 x 128 tiles with no more workgroups than CUs: three buffers, which leave room for one workgroup on a CU)
-    const bool deep = !narrow && (long long)tiles * q.splits <= device_compute_units() && tunable("conv_wgrad_deep", 1);
+    const bool deep = !narrow && (long long)tiles * q.splits <= device_compute_units();
     rc = narrow ? launch_wgrad<2, 1, 2, 2, true, true>(s, grid, target, x, dy, q)
                 : (deep ? launch_wgrad<2, 2, 2, 2, true, true, true>(s, grid, target, x, dy, q)
                         : launch_wgrad<2, 2, 2, 2, true, true>(s, grid, target, x, dy, q));

@@ -318,12 +318,12 @@ void launch(hipStream_t s, bool taps, unsigned blocks, float* out, const float* 
 
 // rows per slab of the bank in LDS for a reduction of R rows (a turn of the kernel's loop is two slabs)
 static int slab_rows(int R) {
-  const int want = tunable("conv_sb_slab", 32);
-  return want == 64 && R % 128 == 0 ? 64 : 32;
+  (void)R;
+  return 32;  // (64-row slabs, possible when R is a multiple of 128, measured no faster)
 }
 
 int conv_sb_splits(int Cout, long long M, int R) {
-  if (tunable("conv_no_sb", 0) || R % 64 != 0 || Cout <= 32) return 0;
+  if (R % 64 != 0 || Cout <= 32) return 0;
   const int BA = Cout > 64 ? 128 : 64;
   const int coutPad = (Cout + BA - 1) / BA * BA;
   if ((long long)R * coutPad * 4 >= (long long)kOutside) return 0;
@@ -338,10 +338,10 @@ int conv_sb_splits(int Cout, long long M, int R) {
   int cus = device_compute_units();
   if (cus <= 0) cus = 256;
   const int pairs = R / (2 * slab_rows(R));  // pairs of slabs: the unit a split is made of
-  const long long want = (long long)cus * std::max(1, tunable("conv_sb_fill", 2));
+  const long long want = (long long)cus * 2;
   int s = 1;
   if (tiles < want) {
-    const int minPairs = std::max(1, tunable("conv_sb_min_pairs", 6));
+    const int minPairs = 6;
     s = (int)std::min<long long>((want + tiles - 1) / tiles, std::max(1, pairs / minPairs));
     const int per = (pairs + s - 1) / s;
     s = (pairs + per - 1) / per;
@@ -379,8 +379,8 @@ SbTail sb_tail(int Cout, long long M, int R) {
   const long long rem = tilesAll % slots;
   if (rem == 0 || 2 * rem > slots) return t;  // a last round at least half full stays as it is
   const int pairs = R / (2 * slab);
-  int s = (int)std::min<long long>(slots / rem, pairs / std::max(1, tunable("conv_sb_tail_min_pairs", 2)));
-  s = std::min(s, std::max(1, tunable("conv_sb_tail_max_splits", 16)));
+  int s = (int)std::min<long long>(slots / rem, pairs / 2);
+  s = std::min(s, 16);
   if (s < 2) return t;
   const int per = (pairs + s - 1) / s;
   s = (pairs + per - 1) / per;
@@ -413,7 +413,7 @@ int conv_sb_launch(hipStream_t s, float* out, const float* in, const float* wt, 
   w.tailTiles = 0;
   p.rSplits = splits;
   const bool taps = !(p.T == 1 && p.dhBase == 0 && p.dwBase == 0 && p.sy == 1 && p.sx == 1 && p.IH == p.OH && p.IW == p.OW);
-  const int occ = tunable("conv_sb_occupancy", 2);
+  const int occ = 2;  // (wavefronts per SIMD the 128-channel kernel's registers are cut for; 3 measured slower)
   auto dispatch = [&](unsigned blocks, float* o, const float* b, const SbP& ww) {
     if (CT == 128) {
       if (slab == 64) launch<4, 64, 2>(s, taps, blocks, o, in, wt, b, p, ww);

@@ -458,7 +458,7 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
   if (tunable("conv_no_ws", 0)) return false;
   if (p.Cin % (2 * kDepth) != 0 || p.R % (8 * kDepth) != 0 || p.T > kMaxTapsWs || p.coutPad % 32 != 0) return false;
   // the bank, or the smallest power-of-two number of slices of it (each a multiple of 32 output channels), in 150 KB
-  const int maxSlices = wantStats ? 1 : std::max(1, tunable("conv_ws_max_slices", 8));
+  const int maxSlices = wantStats ? 1 : 8;
   int slices = 1;
   while (slices <= maxSlices && ((size_t)p.R * (p.coutPad / slices) * sizeof(float) > 150 * 1024 || p.coutPad % (32 * slices) != 0)) {
     if (p.coutPad % (32 * slices * 2) != 0) return false;
@@ -495,7 +495,7 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
       // under four units per SIMD a wide unit no longer pays: the loads of a few long units per SIMD are hidden worse
       // than those of many short ones (stride classes of 3x3 /2 128->128: 130 -> 118 us with the narrowest), so any
       // shape that fills the SIMDs four deep wins over one that does not, and among those that do not the narrowest
-      const double score = units >= tunable("conv_ws_fill", 4) * simds ? balance * issue : 0.01 / cand;
+      const double score = units >= 4 * simds ? balance * issue : 0.01 / cand;
       if (score > best) {
         best = score;
         WA = cand;
@@ -513,7 +513,7 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
   w.groups = p.R / (2 * kDepth);
   w.groupsPerTap = p.Cin / (2 * kDepth);
   w.inBytes = (unsigned)inBytes;
-  w.deepCopy = tunable("conv_ws_deep_copy", 1);
+  w.deepCopy = 1;
   w.byCB = FastDiv(w.chanBlocks);
   w.byRow = FastDiv(8 * WA);
   plan->WA = WA;

@@ -983,7 +983,7 @@ int mcn_pool_backward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* d
       const size_t bytes = ((size_t)maxXW * g->H + (size_t)maxOW * oh) * sizeof(double) + (size_t)maxOW * oh * sizeof(int);
       const long long strips = (g->W + tw - 1) / tw, wgs = strips * (long long)g->C * g->N;
       // (a strip is fetched into registers one strip ahead: twelve x values and four of dzdy per thread at most)
-      if (bytes > (size_t)tunable("pool64_tile_kb", 40) * 1024 || wgs >= (1ll << 31) || sy < 1 || sx < 1 ||
+      if (bytes > (size_t)40 * 1024 || wgs >= (1ll << 31) || sy < 1 || sx < 1 ||
           (long long)maxXW * g->H > 12 * 256 || (long long)maxOW * oh > 4 * 256)
         continue;
       Pool64Tile t;
@@ -1000,12 +1000,9 @@ int mcn_pool_backward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* d
       t.bySx = FastDiv(sx);
       KernelTimer timer("pool64_max_backward_tiled", as_stream(stream));
       t.items = (int)wgs;
-      int cus = device_compute_units();
-      if (cus <= 0) cus = 256;
-      // (one strip per workgroup measured faster than resident workgroups walking the strips -- 32.6 against 36.7 us
-      // on 112x112x64x8 -- so the walk is only taken when asked for)
-      const int walkPerCu = tunable("pool64_walk_per_cu", 0);
-      const dim3 grid((unsigned)(walkPerCu > 0 ? std::min<long long>(wgs, (long long)cus * walkPerCu) : wgs)), block(256);
+      // (one strip per workgroup: resident workgroups walking the strips with the next strip's loads in flight
+      // measured slower, 36.7 against 32.6 us on 112x112x64x8; the kernel's loop serves either launch)
+      const dim3 grid((unsigned)wgs), block(256);
       hipStream_t st = as_stream(stream);
       if (g->poolH == 3 && g->poolW == 3 && sy == 2 && sx == 2)
         hipLaunchKernelGGL((pool64_max_backward_tiled<3, 3, 2, 2>), grid, block, bytes, st, derInput, x, derOutput, p, t, (int)strips);

@@ -969,7 +969,7 @@ int mcn_pool_forward(mcn_stream_t stream, const mcn_pool_geom* g, float* y, cons
       const size_t planes = (size_t)g->C * g->N;
       // many short walks beat few long ones (measured: 2 output columns per thread 26 us, 14 per thread 32 us on
       // 112x112x64x32): enough threads for 8 wavefronts per SIMD, each with at least two output columns
-      const size_t wantThreads = (size_t)std::max(tunable("pool_forward_threads_k", 2048), 1) * 1024;
+      const size_t wantThreads = (size_t)2048 * 1024;
       int segments = (int)std::min<size_t>(std::max<size_t>(1, (wantThreads + planes * quads - 1) / (planes * quads)),
                                            (size_t)std::max(1, p.outW / 2));
       const int owPerSegment = (p.outW + segments - 1) / segments;
@@ -1034,7 +1034,7 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
 
   // ---- average over windows that tile the plane exactly: one streaming pass in memory order
   if (!isMax && p.poolH == p.sy && p.poolW == p.sx && p.pt == 0 && p.pl == 0 && p.H == p.outH * p.poolH && p.W == p.outW * p.poolW &&
-      vecIn && total / 4 < (1ull << 31) && !tunable("pool_force_gather", 0) && !tunable("pool_no_tiles", 0)) {
+      vecIn && total / 4 < (1ull << 31) && !tunable("pool_force_gather", 0)) {
     KernelTimer timer("pool_backward_avg_tiles", s);
     hipLaunchKernelGGL(pool_backward_avg_tiles, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, s, derInput, derOutput,
                        (unsigned)(total / 4), p.H / 4, p.W, p.outH, p.outW, FastDiv(p.H / 4), FastDiv(p.W), FastDiv(p.poolH),

@@ -481,8 +481,8 @@ bool pool_max_backward_pairs_launch(hipStream_t s, const mcn_pool_geom* g, int o
   unsigned blocks = 0;
   size_t lds = 0;
   int nl = 0;
-  if (!pair_plan(g, outH, outW, device_compute_units(), tunable("pool_pairs_per_cu", 0), tunable("pool_pairs_cols", 0),
-                 tunable("pool_pairs_stages", 3), !tunable("pool_pairs_static", 0), &p, &blocks, &lds, &nl))
+  // (as many workgroups per compute unit as fit, tile width chosen, three stages, weighted shares)
+  if (!pair_plan(g, outH, outW, device_compute_units(), 0, 0, 3, true, &p, &blocks, &lds, &nl))
     return false;
   typedef void (*Kernel)(float*, const float*, const float*, PairP);
   static const Kernel kernels[2][4] = {

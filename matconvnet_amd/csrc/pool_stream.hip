@@ -373,7 +373,7 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   if (g->poolH > 8 || g->poolW > 8) return false;
   const int kh = (g->poolH + g->strideY - 1) / g->strideY, kw = (g->poolW + g->strideX - 1) / g->strideX;
   if (kh * kw > 4) return false;  // windows overlapping more than 2 x 2 outputs: the ordered-pass kernel of pool.hip is faster
-  if (tunable("pool_force_gather", 0) || tunable("pool_no_stream", 0)) return false;
+  if (tunable("pool_force_gather", 0)) return false;
   const size_t planes = (size_t)g->C * g->N;
 
   PoolS p;
@@ -385,7 +385,7 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   const int rows = std::max(p.top + g->H, p.top - g->padTop + (outH - 1) * g->strideY + g->poolH);
   p.Hp = (rows + 3) & ~3;
   p.accumulate = accumulate ? 1 : 0;
-  p.walk = tunable("pool_walk", 3);
+  p.walk = 3;
   p.KH = kh;
   p.nPasses = kh * kw;
   p.rankHpk = p.rankWpk = 0;
@@ -393,9 +393,7 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   for (int i = 0; i < g->poolW; ++i) p.rankWpk |= (unsigned)((g->poolW - 1 - i) / g->strideX) << (4 * i);
 
   // widest tile whose LDS fits the budget and whose outputs and cells fit 4 per thread
-  int threads = tunable("pool_threads", 256);
-  if (threads != 512 && threads != 1024) threads = 256;
-  if (threads != 256 && !(p.poolH == 3 && p.poolW == 3 && p.nPasses == 4)) threads = 256;  // (instantiated for 3x3 / 2 only)
+  const int threads = 256;  // (512 and 1024 threads measured no faster on 3x3 / 2 windows)
   const size_t slotBytes = (4 + (size_t)threads) * sizeof(float);
   const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024), 150 * 1024) - slotBytes;
   int TW = 0, maxOut = 0, maxCells = 0, maxC = 0;
@@ -448,20 +446,13 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
 
   int cus = device_compute_units();
   if (cus <= 0) cus = 256;
-  const int perCu = std::min(std::max(tunable("pool_blocks_per_cu", 3), 1), (int)std::max<size_t>((160 * 1024) / std::max<size_t>(lds, 1), 1));
-  const int blocks = tunable("pool_blocks_per_cu", 3) <= 0  // (experiments: one tile per workgroup)
-                         ? p.totalTiles
-                         : (int)std::min<long long>(p.totalTiles, (long long)cus * perCu);
-  const dim3 grid((unsigned)blocks), block((unsigned)threads);
+  const int perCu = std::min(3, (int)std::max<size_t>((160 * 1024) / std::max<size_t>(lds, 1), 1));
+  const int blocks = (int)std::min<long long>(p.totalTiles, (long long)cus * perCu);
+  const dim3 grid((unsigned)blocks);
   bool launched = true;
 #define MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, TF) \
   launched = launch_stream<PHF, PWF, NPF, OPTF, XPTF, TF>(s, grid, lds, derInput, x, derOutput, p)
-#define MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, XPTF)                                         \
-  do {                                                                                     \
-    if (threads == 256 || NPF != 4) MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, 256);      \
-    else if (threads == 512) MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, (NPF == 4 ? 512 : 256));  \
-    else MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, (NPF == 4 ? 1024 : 256));             \
-  } while (0)
+#define MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, XPTF) MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, 256)
 #define MCN_POOL_STREAM_XPT(PHF, PWF, NPF, OPTF)               \
   do {                                                         \
     if (xpt == 1) MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, 1);      \

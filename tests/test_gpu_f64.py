@@ -173,6 +173,20 @@ def test_pooling_bit_exact(capi, ob, geom, method, mode):
     assert bits_equal(got, want), count_bit_mismatches(got, want)
 
 
+@pytest.mark.parametrize("switch", ["conv64_no_mfma", "pool64_no_tiles"])
+def test_general_double_kernels_stay_checked(capi, ob, switch):
+    """With the matrix-instruction convolutions / the LDS strips of max-pool backward switched off, the one-accumulator
+    kernels serve the same shapes: against the oracle as above."""
+    capi.set_tunable(switch, 1)
+    try:
+        if switch == "conv64_no_mfma":
+            test_convolution(capi, ob, (14, 13, 16, 3), (3, 3, 16, 24), 1, 1, 1, True)
+        else:
+            test_pooling_bit_exact(capi, ob, (28, 28, 5, 3, 3, 2, 1), "max", "ties")
+    finally:
+        capi.set_tunable(switch, 0)
+
+
 def test_mixed_precision_is_refused(capi):
     """All tensors of a call are single or all are double (bits/data.hpp:260-266)."""
     x = capi.to_device(np.zeros((4, 4, 1, 1)), D)

@@ -207,6 +207,18 @@ def test_baseline_max_pool_full_size_bit_exact(capi, ob, ties):
     assert np.isclose(got.astype(np.float64).sum(), w["dy"].astype(np.float64).sum(), rtol=1e-6)
 
 
+def test_baseline_max_pool_by_the_streaming_kernel_as_well(capi, ob):
+    """The same configuration through the general streaming kernel (the 3x3 / stride 2 / pad 1 kernel switched off): the
+    same bits, so both kernels stay checked at the benchmarked size."""
+    w = workloads.pool_max_case(ties=True)
+    capi.set_tunable("pool_no_pairs", 1)
+    try:
+        got, want = _run(capi, ob, w["x"], w["dy"], w["x"].shape, w["pool"], w["stride"], w["pad"], "max")
+    finally:
+        capi.set_tunable("pool_no_pairs", 0)
+    assert bits_equal(got, want), count_bit_mismatches(got, want)
+
+
 def test_baseline_avg_pool_full_size_bit_exact(capi, ob):
     """benchmark configuration 3b: 56x56x256x32, 2x2 stride 2."""
     w = workloads.pool_avg_case()
