@@ -367,7 +367,7 @@ def bench_pool_bwd(capi, workloads, reps):
                 call()
             _sync()
             t[label], _ = kernel_time(capi, "pool_backward", call, reps)
-        rows.append(dict(op=name, kernel="pool_max_backward_pairs" if method == "max" else "pool_backward_avg_tiles",
+        rows.append(dict(op=name, kernel="pool_max_backward_stream" if method == "max" else "pool_backward_avg_tiles",
                          workload="configs[2] %s on %s" % (method, "x".join(map(str, shape))),
                          bound="hbm", achieved=nbytes / t["cold"] / 1e9, peak=PEAK_HBM / 1e9, unit="GB/s",
                          frac=nbytes / t["cold"] / PEAK_HBM, avg_launch_us=t["cold"] * 1e6,

@@ -108,16 +108,17 @@ static void check(Context& ctx, ErrorCode e, char const* what) {
   }
 }
 
-static void benchConv(char const* name, int H, int W, int C, int N, int F, int K, int pad, int warmup, int iters) {
+static void benchConv(char const* name, int H, int W, int C, int N, int F, int K, int pad, int warmup, int iters, int stride = 1) {
   Context ctx;
-  DeviceTensor x(TensorShape(H, W, C, N)), f(TensorShape(F, F, C, K)), dy(TensorShape(H, W, K, N));
+  const int OH = (H + 2 * pad - F) / stride + 1, OW = (W + 2 * pad - F) / stride + 1;
+  DeviceTensor x(TensorShape(H, W, C, N)), f(TensorShape(F, F, C, K)), dy(TensorShape(OH, OW, K, N));
   DeviceTensor dx(TensorShape(H, W, C, N)), df(TensorShape(F, F, C, K)), db(TensorShape(K, 1, 1, 1));
   x.randn(1);
   f.randn(2, std::sqrt(2.f / (F * F * C)));
   dy.randn(3);
-  nn::Convolution op(ctx, 1, 1, pad, pad, pad, pad, 1, 1);
+  nn::Convolution op(ctx, stride, stride, pad, pad, pad, pad, 1, 1);
   Tensor none;
-  const double flops = 2.0 * H * W * (double)F * F * C * K * N;
+  const double flops = 2.0 * OH * OW * (double)F * F * C * K * N;
   double tData = medianMs([&] { check(ctx, op.backward(dx.view, none, none, none, f.view, dy.view), name); }, warmup, iters);
   double tFilt = medianMs([&] { check(ctx, op.backward(none, df.view, none, x.view, none, dy.view), name); }, warmup, iters);
   double tBias = medianMs([&] { check(ctx, op.backward(none, none, db.view, none, none, dy.view), name); }, warmup, iters);
@@ -400,6 +401,7 @@ int main(int argc, char** argv) {
     benchResNet(warmup, iters, batch, true);
   }
   if (want("conv1")) benchConv("conv 5x5x3x32 on 32x32x3x100", 32, 32, 3, 100, 5, 32, 2, warmup, iters);
+  if (only == "stem") benchConv("conv 7x7x3x64 /2 on 224x224x3x32", 224, 224, 3, 32, 7, 64, 3, warmup, iters, 2);
   if (want("bnorm")) benchBnorm(warmup, iters);
   if (want("maxpool")) benchPool(true, warmup, iters);
   if (want("avgpool")) benchPool(false, warmup, iters);

@@ -27,7 +27,8 @@ Tunable g_tunables[] = {
     {"conv_sb_tail", 1},               // streamed-bank kernel: the tiles of a partly filled last round get a launch of their own that splits their reduction
     {"conv_sb_tail_slots", 0},         // resident workgroups per compute unit that plan assumes (0: the instantiation's own)
     {"pool_lds_bytes", 16 * 1024},     // LDS tile budget of the pooling-backward kernels
-    {"pool_no_pairs", 0},              // 1: max pooling skips the kernel for 3x3 windows at stride 2, padding 1
+    {"pool_pairs", 0},                 // 1: max pooling backward over 3x3 windows at stride 2, padding 1 by the kernel with direct-to-LDS
+                                       // loads and one winner table (pool_pairs.hip) instead of the streaming kernel (equal to 2% slower)
     {"pool_force_gather", 0},          // 1: skip the ordered-pass kernel, use the general tiled gather
     {"bnorm_one_launch_elems", 8192},  // channels of at most this many elements (and >= 128 of them): sums and apply in one launch
     {"conv_no_ws", 0},                 // 1: never use the weights-stationary kernel

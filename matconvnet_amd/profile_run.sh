@@ -19,6 +19,10 @@ for k in copy bnorm maxpool avgpool conv5 blocktimed; do
   timeout -s KILL 90 rocprofv3 --pmc WRITE_SIZE -d "$O/write_$k" -o pmc -- $B --only $k --iters 8 --warmup 4 > "$O/write_$k.txt" 2>&1
   echo "done $k"
 done
+for k in conv1 stem; do
+  timeout -s KILL 90 rocprofv3 --kernel-trace --stats -d "$O/kt_$k" -o kt -- $B --only $k --iters 12 --warmup 4 > "$O/kt_$k.txt" 2>&1
+  echo "done $k"
+done
 timeout -s KILL 90 rocprofv3 --kernel-trace --stats -d "$O/kt_block" -o kt -- $B --only block --iters 12 --warmup 4 > "$O/kt_block.txt" 2>&1
 for k in conv5 blocktimed; do
   timeout -s KILL 90 rocprofv3 --pmc SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_INSTS_LDS SQ_ACTIVE_INST_LDS GRBM_GUI_ACTIVE -d "$O/sq_$k" -o pmc -- $B --only $k --iters 6 --warmup 3 > "$O/sq_$k.txt" 2>&1

@@ -95,6 +95,16 @@ def main(src, dst):
                             "(ReLU / shortcut sum folded into batch normalisation, banks packed by one launch, filter gradients summed by one, channel sums "
                             "from the convolutions, last ReLU mask as bits)"),
              "copy": ("copy_256MiB_counter_yardstick", "plain streaming copy (ReLU of positive data): reads 268435456 B, writes 268435456 B per launch; yardstick for FETCH_SIZE / WRITE_SIZE")}
+    # first layers (kernel traces only: latency-sized launches)
+    first = "first layers (three input channels): kernel traces of their backward products\n\ncommands: " + PRE
+    for k in ("conv1", "stem"):
+        first += "  rocprofv3 --kernel-trace --stats -d %s/kt_%s -o kt -- ./matconvnet_amd/mcn_bench --only %s --iters 12 --warmup 4\n" % (src, k, k)
+    for k, title in (("conv1", "BASELINE configs[0]: 5x5x3x32 on 32x32x3x100, stride 1, pad 2"),
+                     ("stem", "a ResNet stem: 7x7x3x64 on 224x224x3x32, stride 2, pad 3")):
+        first += "\n" + title + "\nprogram output under the kernel trace:\n" + program_output("%s/kt_%s.txt" % (src, k)) + "\nkernel durations:\n"
+        first += "\n".join(durations("%s/kt_%s" % (src, k))) + "\n"
+    write("conv_first_layers_backward.txt", first)
+
     per_kernel = {}
     for k, (fn, desc) in names.items():
         t = desc + "\n\ncommands: " + PRE
@@ -146,7 +156,7 @@ def main(src, dst):
     put("cfg5/conv_wgrad_mfma", "conv5", "conv_wgrad_mfma")
     put("cfg2/bnorm_sums", "bnorm", "bnorm_sums")
     put("cfg2/bnorm_backward_apply", "bnorm", "bnorm_backward_apply")
-    put("cfg3a/pool", "maxpool", "pool_max_backward_pairs")
+    put("cfg3a/pool", "maxpool", "pool_max_backward_stream")
     put("cfg3b/pool", "avgpool", "pool_backward_avg_tiles")
     with open(os.path.join(dst, "traffic.json"), "w") as f:
         json.dump(traffic, f, indent=1, sort_keys=True)

@@ -207,15 +207,40 @@ def test_baseline_max_pool_full_size_bit_exact(capi, ob, ties):
     assert np.isclose(got.astype(np.float64).sum(), w["dy"].astype(np.float64).sum(), rtol=1e-6)
 
 
-def test_baseline_max_pool_by_the_streaming_kernel_as_well(capi, ob):
-    """The same configuration through the general streaming kernel (the 3x3 / stride 2 / pad 1 kernel switched off): the
-    same bits, so both kernels stay checked at the benchmarked size."""
-    w = workloads.pool_max_case(ties=True)
-    capi.set_tunable("pool_no_pairs", 1)
+@pytest.mark.parametrize("shape,pad", [((224, 8, 2, 1), 1), ((8, 224, 2, 1), 1), ((16, 16, 3, 2), 1), ((112, 30, 2, 2), 1),
+                                       ((40, 41, 1, 9), (1, 0, 1, 0)), ((8, 6, 70, 1), (1, 0, 1, 0))])
+@pytest.mark.parametrize("mode", ["ties", "special", "normal"])
+def test_table_kernel_small_planes(capi, ob, shape, pad, mode):
+    """The kernel for 3x3 / stride 2 / padding 1 (`pool_pairs` = 1) on small planes: tall, wide, one column behind the
+    last window (odd width), fewer planes than XCDs and more than workgroups; ties, NaN and infinities; bit-exact."""
+    og = ob.pool_geom(shape, 3, 2, pad, "max")
+    x = _inputs(shape, 21, mode)
+    dy = F(np.random.default_rng(22).standard_normal(ob.pool_out_shape(og)))
+    capi.set_tunable("pool_pairs", 1)
     try:
-        got, want = _run(capi, ob, w["x"], w["dy"], w["x"].shape, w["pool"], w["stride"], w["pad"], "max")
+        capi.profile_begin("pool_backward_pairs")
+        got, want = _run(capi, ob, x, dy, shape, 3, 2, pad, "max")
+        launches, _ = capi.profile_end()
     finally:
-        capi.set_tunable("pool_no_pairs", 0)
+        capi.set_tunable("pool_pairs", 0)
+    assert launches >= 1
+    assert bits_equal(got, want), count_bit_mismatches(got, want)
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_baseline_max_pool_by_the_table_kernel_as_well(capi, ob, ties):
+    """The same configuration through the kernel for 3x3 windows at stride 2 behind one row and column of padding (tiles
+    by direct-to-LDS loads, one winner table, sums in registers; switched on by `pool_pairs`): the same bits, and the
+    launches counted, so both kernels stay checked at the benchmarked size."""
+    w = workloads.pool_max_case(ties=ties)
+    capi.set_tunable("pool_pairs", 1)
+    try:
+        capi.profile_begin("pool_backward_pairs")
+        got, want = _run(capi, ob, w["x"], w["dy"], w["x"].shape, w["pool"], w["stride"], w["pad"], "max")
+        launches, _ = capi.profile_end()
+    finally:
+        capi.set_tunable("pool_pairs", 0)
+    assert launches >= 1
     assert bits_equal(got, want), count_bit_mismatches(got, want)
 
 
