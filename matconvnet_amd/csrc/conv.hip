@@ -125,6 +125,8 @@ int mcn_conv_forward(mcn_stream_t stream, const mcn_conv_geom* g, float* y, floa
   if (rc) return rc;
   if ((size_t)p.outH * p.outW * p.K * p.N == 0) return MCN_SUCCESS;
   if (!y || !x || !filters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_forward: null tensor");
+  if (!tunable("conv_force_direct", 0) && outMult == 0.f && inMult == 1.f && conv_first_forward_supported(p))
+    return conv_first_forward(as_stream(stream), p, y, x, filters, bias);
   if (!tunable("conv_force_direct", 0) && conv_mfma_forward_supported(p))
     return conv_forward_mfma(as_stream(stream), p, y, outMult, x, inMult, filters, bias, workspace, workspaceBytes);
   return conv_forward_direct(as_stream(stream), p, y, outMult, x, inMult, filters, bias);
@@ -229,6 +231,8 @@ int mcn_conv_forward_packed(mcn_stream_t stream, const mcn_conv_geom* g, float* 
   if (rc) return rc;
   if ((size_t)p.outH * p.outW * p.K * p.N == 0) return MCN_SUCCESS;
   if (!y || !x || !filters) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_forward: null tensor");
+  if (!tunable("conv_force_direct", 0) && outMult == 0.f && inMult == 1.f && conv_first_forward_supported(p))
+    return conv_first_forward(as_stream(stream), p, y, x, filters, bias);  // (reads the bank as it is stored)
   if (!tunable("conv_force_direct", 0) && conv_mfma_forward_supported(p)) {
     PackCtx pk = {PackCtx::kUse, (char*)const_cast<void*>(packed), packedBytes, 0, nullptr};
     return conv_forward_mfma(as_stream(stream), p, y, outMult, x, inMult, filters, bias, workspace, workspaceBytes, &pk);

@@ -80,7 +80,9 @@ bool conv_mfma_backward_filter_supported(const ConvP& p);
 // (conv_first.hip); dB may be null
 bool conv_first_backward_filter_supported(const ConvP& p);
 size_t conv_first_workspace_bytes(const ConvP& p);
-// (and their input gradient at stride 1, on vector FMAs: at most four channels come out)
+// (their forward product; and their input gradient at stride 1, on vector FMAs: at most four channels come out)
+bool conv_first_forward_supported(const ConvP& p);
+int conv_first_forward(hipStream_t s, const ConvP& p, float* y, const float* x, const float* f, const float* bias);
 bool conv_first_backward_data_supported(const ConvP& p);
 int conv_first_backward_data(hipStream_t s, const ConvP& p, float* dx, const float* f, const float* dy);
 int conv_first_backward_filter(hipStream_t s, const ConvP& p, float* dF, float* dB, const float* x, const float* dy, void* ws,

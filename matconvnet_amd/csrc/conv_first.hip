@@ -677,6 +677,285 @@ int conv_first_backward_data(hipStream_t s, const ConvP& c, float* dx, const flo
   return check_launch("mcn_conv_backward_data");
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// Forward product of a first layer (bits/nnconv.cu:126-161 for such a layer): y[k][pixel] = sum over the rows r of the
+// filter volume of w[k][r] patch[r][pixel] + b[k], on v_mfma_f32_32x32x2_f32 with 32 filters as rows, 32 output pixels
+// as columns and two rows of the volume per instruction.
+//   * A workgroup keeps the whole bank in LDS, [row][filter] (staged once), and walks tiles of TH x TW output pixels of
+//     one image; a tile's input pixels are staged as in the filter-gradient kernel above (direct-to-LDS loads, zero
+//     outside the image), and a patch element is again "offset of the row inside the window + offset of the pixel
+//     inside the tile": one LDS read per operand.
+//   * Its four wavefronts are WK groups of 32 filters x WP groups of pixel blocks; a wavefront holds up to eight blocks
+//     of 32 pixels in its accumulators (started at the bias), so a weight read from LDS feeds up to eight instructions.
+//   * The tile of x is small next to the arithmetic it feeds (every staged pixel meets all filters), so one buffer and
+//     the compiler's own waits are enough here: the loads of a tile are a tenth of its matrix instructions.
+namespace {
+
+struct FirstF {
+  int H, W, Cin, N, FH, FW, K, R;
+  int sy, sx, pt, pl, outH, outW;
+  int TH, TW, T;
+  int tilesH, tilesW, tiles, nWg;
+  int XW, XHl, xShift, XHs;   // columns of x a tile reads; LDS pitch of a column; rows before the window's first; slots per column
+  int vec;                    // 16 bytes per lane
+  int xChunks;                // chunks of 64 slots of the x region
+  int steps;                  // pairs of rows of the filter volume
+  int WP, bpw;                // pixel groups of wavefronts; blocks of 32 pixels per wavefront
+  int xStepR, xStepC, xStepD;
+  unsigned xImgBytes;
+  int wFloats, tabFloats;     // floats of the bank in LDS and of the row table (whole chunks of 64)
+  FastDiv byXHs, byXW, byTilesH, byTilesW, byTH, byRows, byFH, byFW;
+};
+
+// BPW: blocks of 32 pixels per wavefront (a constant, so that a step's LDS reads are issued together, ahead of its
+// matrix instructions)
+template <int BPW>
+__global__ __launch_bounds__(256, 2) void conv_first_fwd(float* __restrict__ y, const float* __restrict__ x,
+                                                         const float* __restrict__ f, const float* __restrict__ bias, FirstF p) {
+  extern __shared__ float smem[];
+  const int KP = p.K + 1;                             // (pitch of a row of the bank: staging writes it down the columns)
+  float* wT = smem;                                   // [2 steps + 2][K + 1]: rows past the volume's last are zero
+  int* rowTab = (int*)(smem + p.wFloats);             // [2 steps + 4]: offset of a row of the volume inside a pixel's window
+  float* xT = smem + p.wFloats + p.tabFloats;         // [channel][column][row]
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, kh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wp = wave % p.WP, wk = wave / p.WP;
+  const size_t inPlane = (size_t)p.H * p.W, outPlane = (size_t)p.outH * p.outW;
+
+  // the bank: read along the rows of a filter (consecutive addresses for consecutive threads), eight loads in flight
+  // per thread; written transposed (the LDS writes of a wavefront collide, once per workgroup)
+  {
+    const int rows = 2 * p.steps + 2, total = rows * p.K;
+    for (int base = tid; base < total; base += 8 * 256) {
+      float v[8];
+      int at[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int idx = base + u * 256;
+        int k, r;
+        p.byRows.divmod(min(idx, total - 1), &k, &r);
+        at[u] = idx < total ? r * KP + k : -1;
+        v[u] = (idx < total && r < p.R) ? f[(size_t)r + (size_t)p.R * k] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (at[u] >= 0) wT[at[u]] = v[u];
+    }
+  }
+  for (int r = tid; r < 2 * p.steps + 4; r += 256) {
+    int jd, i, d, j;
+    p.byFH.divmod(r, &jd, &i);   // r = i + FH (j + FW d)
+    p.byFW.divmod(jd, &d, &j);
+    rowTab[r] = r < p.R ? p.xShift + (d * p.XW + j) * p.XHl + i : 0;
+  }
+  // this lane's pixels: block wp + WP j of the tile, pixel 32 block + l32 = (column w, row h) of the tile
+  int pixOff[BPW], pixWH[BPW];
+#pragma unroll
+  for (int j = 0; j < BPW; ++j) {
+    const int pix = min(32 * (wp + p.WP * j) + l32, p.T - 1);
+    int w, h;
+    p.byTH.divmod(pix, &w, &h);
+    pixOff[j] = w * p.sx * p.XHl + h * p.sy;
+    pixWH[j] = (32 * (wp + p.WP * j) + l32 < p.T) ? (w | (h << 16)) : 0x7fff7fff;  // (past the tile: never inside the output)
+  }
+  float bv[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) bv[v] = bias ? bias[wk * 32 + 8 * (v / 4) + 4 * kh + v % 4] : 0.f;
+  int xr0, xc0, xd0;
+  {
+    int seg;
+    p.byXHs.divmod(wave * 64 + lane, &seg, &xr0);
+    p.byXW.divmod(seg, &xd0, &xc0);
+  }
+
+  for (int t = blockIdx.x; t < p.tiles; t += p.nWg) {
+    int n, rest, tw, th;
+    p.byTilesW.divmod(t, &rest, &tw);
+    p.byTilesH.divmod(rest, &n, &th);
+    const int h0 = th * p.TH, w0 = tw * p.TW;
+    __syncthreads();  // (the tile before this one has been multiplied; the first time: the bank is in place)
+    {
+      const __amdgpu_buffer_rsrc_t xr =
+          __builtin_amdgcn_make_buffer_rsrc((void*)(x + (size_t)n * p.Cin * inPlane), 0, (int)p.xImgBytes, 0x00020000);
+      const int row0 = h0 * p.sy - p.pt - p.xShift, col0 = w0 * p.sx - p.pl;
+      int rr = xr0, cc = xc0, d = xd0;
+      for (int c = wave; c < p.xChunks; c += 4) {
+        const int row = row0 + (p.vec ? 4 * rr : rr), col = col0 + cc;
+        const bool in = d < p.Cin && (unsigned)row < (unsigned)p.H && (unsigned)col < (unsigned)p.W;
+        const unsigned off = in ? 4u * (unsigned)(d * (int)inPlane + col * p.H + row) : 0x80000000u;
+        if (p.vec) __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (first_lds_ptr)(xT + c * 256), 16, (int)off, 0, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (first_lds_ptr)(xT + c * 64), 4, (int)off, 0, 0, 0);
+        rr += p.xStepR;
+        const int carry = rr >= p.XHs ? 1 : 0;
+        rr -= carry ? p.XHs : 0;
+        cc += p.xStepC + carry;
+        const int wrap = cc >= p.XW ? 1 : 0;
+        cc -= wrap ? p.XW : 0;
+        d += p.xStepD + wrap;
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    floatx16 acc[BPW];
+#pragma unroll
+    for (int j = 0; j < BPW; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[j][v] = bv[v];
+    // rows 2 s + kh of the volume, s = 0, 1, ...; the operands of step s + 1 are read while step s multiplies (the
+    // row's offset inside the window comes from a table, read two steps ahead)
+    const float* aPtr = wT + kh * KP + wk * 32 + l32;
+    float aNext = aPtr[0];
+    float bNext[BPW];
+    {
+      const int off = rowTab[kh];
+#pragma unroll
+      for (int j = 0; j < BPW; ++j) bNext[j] = xT[off + pixOff[j]];
+    }
+    int offAfter = rowTab[2 + kh];
+    for (int s = 0; s < p.steps; ++s) {
+      const float a = aNext;
+      float b[BPW];
+#pragma unroll
+      for (int j = 0; j < BPW; ++j) b[j] = bNext[j];
+      // (past the last step: the table and the bank have two more rows, of zeros)
+      aNext = aPtr[2 * (s + 1) * KP];
+#pragma unroll
+      for (int j = 0; j < BPW; ++j) bNext[j] = xT[offAfter + pixOff[j]];
+      offAfter = rowTab[2 * (s + 2) + kh];
+      if (s == p.steps - 1 && (p.R & 1)) {
+        // the row past an odd volume's last: its weight is zero, and so must its patch be (x may hold infinities)
+#pragma unroll
+        for (int j = 0; j < BPW; ++j) b[j] = kh ? 0.f : b[j];
+      }
+#pragma unroll
+      for (int j = 0; j < BPW; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[j], acc[j], 0, 0, 0);
+    }
+    // register v of lane (l32, kh) of block j: filter wk 32 + 8 (v / 4) + 4 kh + v % 4, the lane's pixel of the block
+    float* yImg = y + (size_t)n * p.K * outPlane;
+#pragma unroll
+    for (int j = 0; j < BPW; ++j) {
+      const int ow = w0 + (pixWH[j] & 0xffff), oh = h0 + (pixWH[j] >> 16);
+      if (ow < p.outW && oh < p.outH) {
+        float* dst = yImg + (size_t)ow * p.outH + oh;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[(size_t)(wk * 32 + 8 * (v / 4) + 4 * kh + v % 4) * outPlane] = acc[j][v];
+      }
+    }
+  }
+}
+
+bool first_fwd_plan(const ConvP& c, FirstF* out, size_t* lds) {
+  if (c.groups != 1 || c.dy != 1 || c.dx != 1 || c.C > 4 || c.C < 1 || c.FH < 2) return false;
+  const int R = c.FH * c.FW * c.C;
+  // (small volumes are all output: 3x3x3x64 on 224x224x3x32 writes 411 MB for 5.5 GFLOP, and the general kernel's
+  // stores are the better ones: 152 against 162 us)
+  if (R < 48 || R + 1 > 160 || (c.K != 32 && c.K != 64) || tunable("conv_no_first", 0)) return false;
+  if (c.outH < 1 || c.outW < 1 || c.N < 1) return false;
+  if ((size_t)c.K * c.outH * c.outW >= (1u << 29) || (size_t)c.C * c.H * c.W >= (1u << 29)) return false;
+  FirstF p;
+  p.H = c.H; p.W = c.W; p.Cin = c.C; p.N = c.N; p.FH = c.FH; p.FW = c.FW; p.K = c.K; p.R = R;
+  p.sy = c.sy; p.sx = c.sx; p.pt = c.pt; p.pl = c.pl; p.outH = c.outH; p.outW = c.outW;
+  p.steps = (R + 1) / 2;
+  p.vec = c.H % 4 == 0 ? 1 : 0;  // (whole groups of four rows are inside the image or outside)
+  const int WK = c.K / 32;
+  p.WP = 4 / WK;
+  // rows of a tile: whole columns up to 64 rows, in equal parts (a multiple of four rows when x is staged 16 bytes
+  // per lane: the window's first row must keep its place inside a group of four from tile to tile)
+  const int unit = p.vec ? 4 : 1;
+  int TH = (std::min(c.outH, 64) + unit - 1) / unit * unit;
+  if (c.outH > 64) {
+    const int parts = (c.outH + 63) / 64;
+    TH = ((c.outH + parts - 1) / parts + unit - 1) / unit * unit;
+  }
+  const int shift = p.vec ? ((c.pt % 4) == 0 ? 0 : 4 - c.pt % 4) : 0;
+  const int XH = (TH - 1) * c.sy + c.FH;
+  const int XHl = p.vec ? (shift + XH + 3) / 4 * 4 : XH;
+  p.tabFloats = (2 * p.steps + 4 + 63) / 64 * 64;
+  p.wFloats = ((2 * p.steps + 2) * (c.K + 1) + 63) / 64 * 64;
+  const size_t wFloats = (size_t)p.wFloats + p.tabFloats;
+  auto x_floats = [&](int tw) {
+    const size_t XW = (size_t)(tw - 1) * c.sx + c.FW;
+    return p.vec ? ((size_t)c.C * XW * (XHl / 4) + 63) / 64 * 256 : ((size_t)c.C * XW * XH + 63) / 64 * 64;
+  };
+  int cus = device_compute_units();
+  if (cus <= 0) cus = 256;
+  const int perCu = 2;  // (one workgroup per compute unit: 122 against 105 us on a ResNet stem)
+  const size_t budget = 160 * 1024 / perCu - 1024;
+  // columns of a tile: among those that fit (LDS; eight blocks of 32 pixels per wavefront), the width with the
+  // shortest longest walk -- tiles per workgroup x blocks per wavefront, and half a block's time per tile besides
+  const int tilesH = (c.outH + TH - 1) / TH;
+  long long best = -1;
+  int TW = 0;
+  for (int tw = std::min(c.outW, 32 * 8 * p.WP / TH); tw >= 1; --tw) {
+    if ((wFloats + x_floats(tw)) * sizeof(float) > budget) continue;
+    const long long tiles = (long long)tilesH * ((c.outW + tw - 1) / tw) * c.N;
+    const long long nWg = std::min<long long>(tiles, (long long)cus * perCu);
+    const int blocks = (TH * tw + 31) / 32, bpw = (blocks + p.WP - 1) / p.WP;
+    const long long cost = ((tiles + nWg - 1) / nWg) * (2 * bpw + 1);
+    if (best < 0 || cost < best) {
+      best = cost;
+      TW = tw;
+    }
+  }
+  if (TW < 1) return false;
+  p.TH = TH; p.TW = TW; p.T = TH * TW;
+  p.bpw = ((p.T + 31) / 32 + p.WP - 1) / p.WP;
+  if (p.bpw > 8) return false;
+  p.tilesH = tilesH;
+  p.tilesW = (c.outW + TW - 1) / TW;
+  const long long tiles = (long long)p.tilesH * p.tilesW * c.N;
+  if (tiles >= (1ll << 30)) return false;
+  p.tiles = (int)tiles;
+  p.nWg = (int)std::min<long long>(tiles, (long long)cus * perCu);
+  p.XW = (TW - 1) * c.sx + c.FW;
+  p.XHl = XHl;
+  p.xShift = shift;
+  p.XHs = p.vec ? XHl / 4 : XH;
+  p.xChunks = (int)(x_floats(TW) / (p.vec ? 256 : 64));
+  p.xStepR = 256 % p.XHs;
+  p.xStepC = (256 / p.XHs) % p.XW;
+  p.xStepD = (256 / p.XHs) / p.XW;
+  p.xImgBytes = (unsigned)((size_t)c.C * c.H * c.W * 4);
+  p.byXHs = FastDiv(p.XHs); p.byXW = FastDiv(p.XW); p.byTilesH = FastDiv(p.tilesH); p.byTilesW = FastDiv(p.tilesW);
+  p.byTH = FastDiv(TH); p.byRows = FastDiv(2 * p.steps + 2); p.byFH = FastDiv(c.FH); p.byFW = FastDiv(c.FW);
+  *lds = (wFloats + x_floats(TW)) * sizeof(float);
+  *out = p;
+  return true;
+}
+
+}  // namespace
+
+bool conv_first_forward_supported(const ConvP& c) {
+  if (c.C > 4) return false;
+  FirstF p;
+  size_t lds;
+  return first_fwd_plan(c, &p, &lds);
+}
+
+// y = conv(x, f) + bias of a first layer (nothing is accumulated onto y)
+int conv_first_forward(hipStream_t s, const ConvP& c, float* y, const float* x, const float* f, const float* bias) {
+  FirstF p;
+  size_t lds;
+  if (!first_fwd_plan(c, &p, &lds)) return fail(MCN_UNSUPPORTED, "mcn_conv_forward: not a first layer");
+  typedef void (*Kernel)(float*, const float*, const float*, const float*, FirstF);
+  static const Kernel kernels[8] = {conv_first_fwd<1>, conv_first_fwd<2>, conv_first_fwd<3>, conv_first_fwd<4>,
+                                    conv_first_fwd<5>, conv_first_fwd<6>, conv_first_fwd<7>, conv_first_fwd<8>};
+  const Kernel kernel = kernels[p.bpw - 1];
+  static std::atomic<size_t> raised[kMaxDevices][8];
+  const int dev = current_device();
+  if (lds > 64 * 1024 && (dev < 0 || dev >= kMaxDevices || lds > raised[dev][p.bpw - 1].load(std::memory_order_acquire))) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(MCN_UNSUPPORTED, "mcn_conv_forward: %zu bytes of LDS refused", lds);
+    }
+    if (dev >= 0 && dev < kMaxDevices) raised[dev][p.bpw - 1].store(lds, std::memory_order_release);
+  }
+  KernelTimer timer("conv_first_fwd", s);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)p.nWg), dim3(256), lds, s, y, x, f, bias, p);
+  return check_launch("mcn_conv_forward");
+}
+
 bool conv_first_backward_filter_supported(const ConvP& c) {
   FirstP p;
   size_t lds;
