@@ -1,3 +1,7 @@
+// Kernels for first layers (one to four input channels, 32 or 64 filters): the filter gradient with the bias gradient
+// from the same pass (this comment), the input gradient at stride 1 and the forward product (further down, each with
+// a comment of its own).
+//
 // Filter gradient (and, from the same pass, bias gradient) of first layers: few input channels, a filter volume of at
 // most 160 rows (5x5x3 = 75, 7x7x3 = 147), 32 or 64 filters -- bits/nnconv.cu:230-244,280-311 for such a layer.
 //
@@ -722,15 +726,15 @@ __global__ __launch_bounds__(256, 2) void conv_first_fwd(float* __restrict__ y, 
   const int wp = wave % p.WP, wk = wave / p.WP;
   const size_t inPlane = (size_t)p.H * p.W, outPlane = (size_t)p.outH * p.outW;
 
-  // the bank: read along the rows of a filter (consecutive addresses for consecutive threads), eight loads in flight
-  // per thread; written transposed (the LDS writes of a wavefront collide, once per workgroup)
+  // the bank: read along the rows of a filter (consecutive addresses for consecutive threads), twenty loads in flight
+  // per thread; written transposed
   {
     const int rows = 2 * p.steps + 2, total = rows * p.K;
-    for (int base = tid; base < total; base += 8 * 256) {
-      float v[8];
-      int at[8];
+    for (int base = tid; base < total; base += 20 * 256) {
+      float v[20];
+      int at[20];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < 20; ++u) {
         const int idx = base + u * 256;
         int k, r;
         p.byRows.divmod(min(idx, total - 1), &k, &r);
@@ -738,7 +742,7 @@ __global__ __launch_bounds__(256, 2) void conv_first_fwd(float* __restrict__ y, 
         v[u] = (idx < total && r < p.R) ? f[(size_t)r + (size_t)p.R * k] : 0.f;
       }
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < 20; ++u)
         if (at[u] >= 0) wT[at[u]] = v[u];
     }
   }
