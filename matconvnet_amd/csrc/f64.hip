@@ -10,6 +10,10 @@
 #include <algorithm>
 
 namespace mcn {
+
+bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, double* derInput,
+                                     const double* x, const double* derOutput, int accumulate);  // pool_stream.hip
+
 namespace {
 
 // ---------------------------------------------------------------------------------------------------------
@@ -968,6 +972,11 @@ int mcn_pool_backward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* d
   Pool64 p = {g->H, g->W, oh, ow, g->poolH, g->poolW, g->strideY, g->strideX, g->padTop, g->padLeft, accumulate ? 1 : 0};
   unsigned blocks;
   if ((rc = blocks_for(total, "mcn_pool_backward_f64", &blocks))) return rc;
+  // the streaming kernel of single precision, for the shapes it takes (columns of whole 16-byte cells, windows over at
+  // most 2 x 2 outputs); same bits as the kernels below
+  if (isMax && !tunable("pool64_no_tiles", 0) &&
+      pool_max_backward_stream_launch(as_stream(stream), g, oh, ow, derInput, x, derOutput, accumulate))
+    return check_launch("mcn_pool_backward_f64");
   if (isMax && !tunable("pool64_no_tiles", 0)) {
     // strips of input columns through LDS, when a strip with its halo fits
     const int sx = g->strideX, sy = g->strideY;

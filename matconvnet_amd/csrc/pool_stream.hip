@@ -1,7 +1,8 @@
-// Max-pooling backward, streaming form (the fast path for planes whose height is a multiple of 4).
+// Max-pooling backward, streaming form (the fast path for planes whose columns are whole 16-byte cells: heights that
+// are a multiple of 4 in single precision, of 2 in double).
 //
-// Same arithmetic and visiting order as the ordered-pass kernel of pool.hip -- one fp32 accumulator per input
-// element, every output adds its dzdy to the first maximum of its window, outputs reach an accumulator in
+// Same arithmetic and visiting order as the ordered-pass kernel of pool.hip -- one accumulator of the data type per
+// input element, every output adds its dzdy to the first maximum of its window, outputs reach an accumulator in
 // ascending (output column, output row) order (bits/nnpooling.cu:33-66,190-206) -- organised so that HBM
 // never waits for the arithmetic:
 //   * persistent workgroups: workgroup b of G takes tiles b, b + G, ... (a tile = all rows of TW columns of one
@@ -23,11 +24,22 @@
 namespace mcn {
 namespace {
 
+// A 16-byte cell of the data type: four floats or two doubles.
+template <typename E> struct Cell;
+template <> struct Cell<float> {
+  typedef float vec __attribute__((ext_vector_type(4)));
+  static constexpr int n = 4;
+};
+template <> struct Cell<double> {
+  typedef double vec __attribute__((ext_vector_type(2)));
+  static constexpr int n = 2;
+};
+
 struct PoolS {
   int H, W, outH, outW, sy, sx, pt, pl, poolH, poolW;
-  int H4;        // H / 4
-  int top;       // frame row of image row 0: the padding rounded up to a multiple of 4
-  int Hp;        // frame pitch in floats (multiple of 4)
+  int H4;        // cells per column: H / (elements per cell)
+  int top;       // frame row of image row 0: the padding rounded up to whole cells
+  int Hp;        // frame pitch in elements (whole cells)
   int maxC;      // widest frame over the tiles of a plane, in columns
   int TW, tilesPerPlane, totalTiles;
   int accumulate;
@@ -41,20 +53,22 @@ struct PoolS {
 };
 
 // Uniform description of one tile: all rows of the image columns [w0, w0 + nW) of one plane.
+template <typename E>
 struct Tile {
   int w0, nW;          // owned columns
   int owLo, nOut;      // first output column whose window touches the tile; outputs touching it
   int cLo, nC;         // frame column 0 is image column cLo (may be negative: padding); frame columns
   int ca;              // first image column present in the frame
   int nCells;          // 16-byte cells of x to load: columns [ca, cb) x H/4
-  const float* xsrc;   // x at (row 0, column ca)
-  const float* dsrc;   // dzdy at (row 0, column owLo)
-  float* out;          // dzdx at (row 0, column w0)
+  const E* xsrc;       // x at (row 0, column ca)
+  const E* dsrc;       // dzdy at (row 0, column owLo)
+  E* out;              // dzdx at (row 0, column w0)
 };
 
-__device__ __forceinline__ Tile tile_geometry(const PoolS& p, int tile, int poolW, const float* xPlane,
-                                              const float* dyPlane, float* dxPlane) {
-  Tile g;
+template <typename E>
+__device__ __forceinline__ Tile<E> tile_geometry(const PoolS& p, int tile, int poolW, const E* xPlane, const E* dyPlane,
+                                                 E* dxPlane) {
+  Tile<E> g;
   g.w0 = tile * p.TW;
   const int w1 = min(g.w0 + p.TW, p.W);
   g.nW = w1 - g.w0;
@@ -75,13 +89,13 @@ __device__ __forceinline__ Tile tile_geometry(const PoolS& p, int tile, int pool
 }
 
 // Issues the global loads of tile g: this thread's cells of x and its outputs' dzdy.
-template <int OPT, int XPT, int T>
-__device__ __forceinline__ void prefetch_tile(v4f (&xr)[XPT], float (&dr)[OPT], const Tile& g, int tid) {
+template <typename E, int OPT, int XPT, int T>
+__device__ __forceinline__ void prefetch_tile(typename Cell<E>::vec (&xr)[XPT], E (&dr)[OPT], const Tile<E>& g, int tid) {
   // Lanes past the end re-read the last element instead of being masked off (their copies are never used):
   // a clamped index costs one instruction, a masked region four.
   if (g.nCells > 0) {
 #pragma unroll
-    for (int u = 0; u < XPT; ++u) xr[u] = ((const v4f*)g.xsrc)[min(tid + T * u, g.nCells - 1)];
+    for (int u = 0; u < XPT; ++u) xr[u] = ((const typename Cell<E>::vec*)g.xsrc)[min(tid + T * u, g.nCells - 1)];
   }
   if (g.nOut > 0) {
 #pragma unroll
@@ -96,23 +110,41 @@ __device__ __forceinline__ float hw_max(float a, float b) {
   asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
   return r;
 }
+__device__ __forceinline__ double hw_max(double a, double b) {
+  double r;
+  asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// a finished cell of accumulators on its way out: written once, not read again by this launch
+template <typename V>
+__device__ __forceinline__ void stream_store_cell(V* p, const V v) {
+#if MCN_NT_STORE
+  __builtin_nontemporal_store(v, p);
+#else
+  *p = v;
+#endif
+}
 
 // LDS-only barrier: waits for this wave's LDS traffic, not for the global loads of the next tile in flight
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // OPT outputs and XPT 16-byte cells of x per thread and tile; NP > 0: the number of passes, known at compile time.
 // T threads per workgroup.
-template <int PH, int PW, int NP, int OPT, int XPT, int T>
-__global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict__ dx,
-                                                                const float* __restrict__ x,
-                                                                const float* __restrict__ dy, PoolS p) {
-  extern __shared__ float smem[];
-  float* acc = smem;                 // [TW * H] accumulators, all +0 between tiles
-  float* frame = smem + p.TW * p.H;  // [maxC * Hp] x inside its -inf frame; frame row r = image row r - top
-  // after the frame: one 16-byte cell that swallows the staging writes of idle lanes, and one float per lane
+template <typename E, int PH, int PW, int NP, int OPT, int XPT, int T>
+__global__ __launch_bounds__(T) void pool_max_backward_stream(E* __restrict__ dx, const E* __restrict__ x,
+                                                                const E* __restrict__ dy, PoolS p) {
+  typedef typename Cell<E>::vec vec;
+  constexpr int VE = Cell<E>::n;
+  const E minusInf = -(E)INFINITY;
+  const vec zeroCell = (vec)(E)0;
+  extern __shared__ __align__(16) unsigned char smemBytes[];
+  E* acc = (E*)smemBytes;        // [TW * H] accumulators, all +0 between tiles
+  E* frame = acc + p.TW * p.H;   // [maxC * Hp] x inside its -inf frame; frame row r = image row r - top
+  // after the frame: one 16-byte cell that swallows the staging writes of idle lanes, and one element per lane
   // that swallows the additions of lanes sitting out a pass
   const int trashCell = p.maxC * p.Hp;                      // relative to frame
-  const int idleAcc = p.TW * p.H + p.maxC * p.Hp + 4 + threadIdx.x;  // relative to acc
+  const int idleAcc = p.TW * p.H + p.maxC * p.Hp + VE + threadIdx.x;  // relative to acc
   const int tid = threadIdx.x;
   const int poolH = PH > 0 ? PH : p.poolH, poolW = PW > 0 ? PW : p.poolW;
 
@@ -155,13 +187,13 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
   if (t0 >= t1) return;
 
   // ---- once: accumulators at +0; the frame rows above and below the image at -inf (no tile writes them)
-  for (int i = tid; i < p.TW * p.H4; i += T) ((float4*)acc)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = tid; i < p.TW * p.H4; i += T) ((vec*)acc)[i] = zeroCell;
   {
     const int nb = p.Hp - p.H;
     for (int i = tid; i < p.maxC * nb; i += T) {
       int c, k;
       p.byBorder.divmod(i, &c, &k);
-      frame[c * p.Hp + (k < p.top ? k : k + p.H)] = -INFINITY;
+      frame[c * p.Hp + (k < p.top ? k : k + p.H)] = minusInf;
     }
   }
 
@@ -185,14 +217,14 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
       }
     }
   }
-  // cells i = tid + T u of the tile's x: column i / H4 after the first present one, rows 4 (i % H4) ...
+  // cells i = tid + T u of the tile's x: column i / H4 after the first present one, rows VE (i % H4) ...
   int cellDst[XPT];  // frame position when the first present column is frame column 0
   {
     int c, s;
     p.byH4.divmod(tid, &c, &s);
 #pragma unroll
     for (int u = 0; u < XPT; ++u) {
-      cellDst[u] = c * p.Hp + p.top + 4 * s;
+      cellDst[u] = c * p.Hp + p.top + VE * s;
       c += p.cellStepQ;
       s += p.cellStepR;
       if (s >= p.H4) {
@@ -204,20 +236,20 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
 
   // ---- walk the tiles t0, t0 + step, ... < t1
   const size_t planeIn = (size_t)p.H * p.W, planeOut = (size_t)p.outH * p.outW;
-  v4f xr[XPT];  // native vectors: these stay in registers under conditional assignment
-  float dr[OPT];
-  Tile cur;
+  vec xr[XPT];  // native vectors: these stay in registers under conditional assignment
+  E dr[OPT];
+  Tile<E> cur;
   {
     int z, tile;
     p.byTiles.divmod(t0, &z, &tile);
     z = zFirst + zStep * z;
     cur = tile_geometry(p, tile, poolW, x + z * planeIn, dy + z * planeOut, dx + z * planeIn);
   }
-  prefetch_tile<OPT, XPT, T>(xr, dr, cur, tid);
+  prefetch_tile<E, OPT, XPT, T>(xr, dr, cur, tid);
 
   // The accumulators of a finished tile are written to memory at the start of the next iteration, so their
   // stores have a whole tile's worth of work to complete before this wave next waits on its memory counter.
-  float* prevOut = dx;
+  E* prevOut = dx;
   int prevIn4 = 0;
 
   for (int t = t0; t < t1; t += step) {
@@ -231,49 +263,49 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
       const int colShift = (cur.ca - cur.cLo) * p.Hp;
 #pragma unroll
       for (int u = 0; u < XPT; ++u)
-        *(v4f*)(frame + (tid + T * u < cur.nCells ? cellDst[u] + colShift : trashCell)) = xr[u];
+        *(vec*)(frame + (tid + T * u < cur.nCells ? cellDst[u] + colShift : trashCell)) = xr[u];
       // frame columns left / right of the image (first and last tiles of a plane only)
       if (cur.cLo < 0)
-        for (int r = tid; r < colShift; r += T) frame[r] = -INFINITY;
+        for (int r = tid; r < colShift; r += T) frame[r] = minusInf;
       const int c0 = p.W - cur.cLo;
       if (cur.nC > c0)
-        for (int r = tid; r < (cur.nC - c0) * p.Hp; r += T) frame[c0 * p.Hp + r] = -INFINITY;
+        for (int r = tid; r < (cur.nC - c0) * p.Hp; r += T) frame[c0 * p.Hp + r] = minusInf;
     }
-    float dv[OPT];
+    E dv[OPT];
 #pragma unroll
     for (int k = 0; k < OPT; ++k) dv[k] = dr[k];
     // ---- previous tile: stream its accumulators out, leaving +0 (or this tile's derInput when accumulating)
     for (int i = tid; i < prevIn4; i += T) {
-      const float4 a = ((const float4*)acc)[i];
-      ((float4*)acc)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-      stream_store4((float4*)prevOut + i, a);
+      const vec a = ((const vec*)acc)[i];
+      ((vec*)acc)[i] = zeroCell;
+      stream_store_cell((vec*)prevOut + i, a);
     }
     if (p.accumulate)
-      for (int i = tid; i < nIn4; i += T) ((float4*)acc)[i] = ((const float4*)cur.out)[i];
+      for (int i = tid; i < nIn4; i += T) ((vec*)acc)[i] = ((const vec*)cur.out)[i];
     lds_barrier();
 
     // ---- next tile's loads go out now and land while this tile is computed
-    Tile nxt = cur;
+    Tile<E> nxt = cur;
     if (t + step < t1) {
       int z, tile;
       p.byTiles.divmod(t + step, &z, &tile);
       z = zFirst + zStep * z;
       nxt = tile_geometry(p, tile, poolW, x + z * planeIn, dy + z * planeOut, dx + z * planeIn);
-      prefetch_tile<OPT, XPT, T>(xr, dr, nxt, tid);
+      prefetch_tile<E, OPT, XPT, T>(xr, dr, nxt, tid);
     }
 
     // ---- winner of each owned output: first maximum of its window, scanning column by column
-    float best[OPT];
+    E best[OPT];
     int code[OPT];  // 8 * column offset + row offset of the winner, -1 when nothing beats -inf
-    const float* org[OPT];
+    const E* org[OPT];
 #pragma unroll
     for (int k = 0; k < OPT; ++k) {
       org[k] = frame + (tid + T * k < cur.nOut ? orgOff[k] : 0);  // idle lanes read a valid window
-      best[k] = -INFINITY;
+      best[k] = minusInf;
       code[k] = -1;
     }
     if (PH > 0 && PW > 0) {
-      float v[OPT][PW > 0 ? PW : 1][PH > 0 ? PH : 1];
+      E v[OPT][PW > 0 ? PW : 1][PH > 0 ? PH : 1];
 #pragma unroll
       for (int k = 0; k < OPT; ++k)
 #pragma unroll
@@ -295,7 +327,7 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
         for (int i = 0; i < poolH; ++i)
 #pragma unroll
           for (int k = 0; k < OPT; ++k) {
-            const float v = org[k][j * p.Hp + i];
+            const E v = org[k][j * p.Hp + i];
             code[k] = v > best[k] ? (8 * j + i) : code[k];
             best[k] = hw_max(best[k], v);
           }
@@ -318,7 +350,7 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
     if (NP > 0) {
 #pragma unroll
       for (int r = 0; r < NP; ++r) {
-        float a[OPT];
+        E a[OPT];
         int at[OPT];
 #pragma unroll
         for (int k = 0; k < OPT; ++k) {
@@ -343,16 +375,16 @@ __global__ __launch_bounds__(T) void pool_max_backward_stream(float* __restrict_
     cur = nxt;
   }
   // ---- last tile
-  for (int i = tid; i < prevIn4; i += T) stream_store4((float4*)prevOut + i, ((const float4*)acc)[i]);
+  for (int i = tid; i < prevIn4; i += T) stream_store_cell((vec*)prevOut + i, ((const vec*)acc)[i]);
 }
 
 // One instantiation: opts it into more than 64 KB of LDS when the tile needs that (once per device), then launches.
-template <int PH, int PW, int NP, int OPT, int XPT, int T>
-bool launch_stream(hipStream_t s, dim3 grid, size_t lds, float* dx, const float* x, const float* dy, const PoolS& p) {
+template <typename E, int PH, int PW, int NP, int OPT, int XPT, int T>
+bool launch_stream(hipStream_t s, dim3 grid, size_t lds, E* dx, const E* x, const E* dy, const PoolS& p) {
   static std::atomic<size_t> raised[kMaxDevices];
   const int dev = current_device();
   if (lds > 64 * 1024 && (dev < 0 || dev >= kMaxDevices || lds > raised[dev].load(std::memory_order_acquire))) {
-    if (hipFuncSetAttribute((const void*)pool_max_backward_stream<PH, PW, NP, OPT, XPT, T>,
+    if (hipFuncSetAttribute((const void*)pool_max_backward_stream<E, PH, PW, NP, OPT, XPT, T>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
       (void)hipGetLastError();
       return false;
@@ -360,16 +392,16 @@ bool launch_stream(hipStream_t s, dim3 grid, size_t lds, float* dx, const float*
     if (dev >= 0 && dev < kMaxDevices) raised[dev].store(lds, std::memory_order_release);
   }
   KernelTimer timer("pool_backward_stream", s);
-  hipLaunchKernelGGL((pool_max_backward_stream<PH, PW, NP, OPT, XPT, T>), grid, dim3((unsigned)T), lds, s, dx, x, dy, p);
+  hipLaunchKernelGGL((pool_max_backward_stream<E, PH, PW, NP, OPT, XPT, T>), grid, dim3((unsigned)T), lds, s, dx, x, dy, p);
   return true;
 }
 
-}  // namespace
-
 // Launches the streaming kernel when the problem fits it.  Returns true when the work was enqueued.
-bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, float* derInput,
-                                     const float* x, const float* derOutput, int accumulate) {
-  if (g->H % 4 != 0 || !aligned16(derInput) || !aligned16(x)) return false;
+template <typename E>
+bool stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, E* derInput, const E* x,
+                   const E* derOutput, int accumulate) {
+  constexpr int VE = Cell<E>::n;
+  if (g->H % VE != 0 || !aligned16(derInput) || !aligned16(x)) return false;
   if (g->poolH > 8 || g->poolW > 8) return false;
   const int kh = (g->poolH + g->strideY - 1) / g->strideY, kw = (g->poolW + g->strideX - 1) / g->strideX;
   if (kh * kw > 4) return false;  // windows overlapping more than 2 x 2 outputs: the ordered-pass kernel of pool.hip is faster
@@ -380,10 +412,10 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   p.H = g->H; p.W = g->W; p.outH = outH; p.outW = outW;
   p.sy = g->strideY; p.sx = g->strideX; p.pt = g->padTop; p.pl = g->padLeft;
   p.poolH = g->poolH; p.poolW = g->poolW;
-  p.H4 = g->H / 4;
-  p.top = (g->padTop + 3) & ~3;
+  p.H4 = g->H / VE;
+  p.top = (g->padTop + VE - 1) & ~(VE - 1);
   const int rows = std::max(p.top + g->H, p.top - g->padTop + (outH - 1) * g->strideY + g->poolH);
-  p.Hp = (rows + 3) & ~3;
+  p.Hp = (rows + VE - 1) & ~(VE - 1);
   p.accumulate = accumulate ? 1 : 0;
   p.walk = 3;
   p.KH = kh;
@@ -394,8 +426,10 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
 
   // widest tile whose LDS fits the budget and whose outputs and cells fit 4 per thread
   const int threads = 256;  // (512 and 1024 threads measured no faster on 3x3 / 2 windows)
-  const size_t slotBytes = (4 + (size_t)threads) * sizeof(float);
-  const size_t budget = (size_t)std::min(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024), 150 * 1024) - slotBytes;
+  // (the budget is for single precision; double precision takes the same tiles in twice the bytes)
+  const size_t slotBytes = (VE + (size_t)threads) * sizeof(E), scale = sizeof(E) / sizeof(float);
+  const size_t budget =
+      std::min<size_t>(std::max(tunable("pool_lds_bytes", 16 * 1024), 1024) * scale, 150 * 1024) - slotBytes;
   int TW = 0, maxOut = 0, maxCells = 0, maxC = 0;
   size_t lds = 0;
   for (int nT = 1; nT <= p.W; ++nT) {
@@ -415,7 +449,7 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
       worstC = std::max(worstC, nC);
     }
     worstC = std::max(worstC, p.poolW);  // idle lanes read the window at the frame origin
-    const size_t need = ((size_t)cand * p.H + (size_t)worstC * p.Hp) * sizeof(float);
+    const size_t need = ((size_t)cand * p.H + (size_t)worstC * p.Hp) * sizeof(E);
     if (need <= budget && worstOut <= 4 * threads && worstCells <= 4 * threads) {
       TW = cand;
       maxOut = worstOut;
@@ -451,7 +485,7 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
   const dim3 grid((unsigned)blocks);
   bool launched = true;
 #define MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, TF) \
-  launched = launch_stream<PHF, PWF, NPF, OPTF, XPTF, TF>(s, grid, lds, derInput, x, derOutput, p)
+  launched = launch_stream<E, PHF, PWF, NPF, OPTF, XPTF, TF>(s, grid, lds, derInput, x, derOutput, p)
 #define MCN_POOL_STREAM(PHF, PWF, NPF, OPTF, XPTF) MCN_POOL_STREAM_T(PHF, PWF, NPF, OPTF, XPTF, 256)
 #define MCN_POOL_STREAM_XPT(PHF, PWF, NPF, OPTF)               \
   do {                                                         \
@@ -478,6 +512,17 @@ bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int 
 #undef MCN_POOL_STREAM
 #undef MCN_POOL_STREAM_T
   return launched;
+}
+
+}  // namespace
+
+bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, float* derInput,
+                                     const float* x, const float* derOutput, int accumulate) {
+  return stream_launch<float>(s, g, outH, outW, derInput, x, derOutput, accumulate);
+}
+bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, double* derInput,
+                                     const double* x, const double* derOutput, int accumulate) {
+  return stream_launch<double>(s, g, outH, outW, derInput, x, derOutput, accumulate);
 }
 
 }  // namespace mcn

@@ -187,6 +187,20 @@ def test_general_double_kernels_stay_checked(capi, ob, switch):
         capi.set_tunable(switch, 0)
 
 
+@pytest.mark.parametrize("geom", [(112, 112, 3, 2, 3, 2, (0, 1, 0, 1)), (56, 40, 4, 2, 2, 2, 0), (30, 17, 2, 3, 3, 2, 1),
+                                  (64, 64, 2, 2, (3, 2), (2, 2), (1, 1, 0, 0)), (6, 5, 3, 2, 3, 1, 1)])
+@pytest.mark.parametrize("mode", ["ties", "special"])
+def test_max_pool_backward_streaming_and_strips(capi, ob, geom, mode):
+    """Heights of whole 16-byte cells take single precision's streaming kernel (several tiles per plane, the frame's
+    borders, ties and non-finite values); with that kernel switched off the same shapes go through the LDS strips."""
+    test_pooling_bit_exact(capi, ob, geom, "max", mode)
+    capi.set_tunable("pool_force_gather", 1)
+    try:
+        test_pooling_bit_exact(capi, ob, geom, "max", mode)
+    finally:
+        capi.set_tunable("pool_force_gather", 0)
+
+
 def test_mixed_precision_is_refused(capi):
     """All tensors of a call are single or all are double (bits/data.hpp:260-266)."""
     x = capi.to_device(np.zeros((4, 4, 1, 1)), D)
