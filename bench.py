@@ -553,8 +553,8 @@ def bench_conv_single(capi, workloads, reps):
 
 def bench_double(capi, workloads, reps):
     """The double-precision instantiation on reduced forms of the graded configurations (convolutions on the fp64 matrix
-    instruction where a product has sixteen columns or more, max-pool backward by strips through LDS, batch norm as two
-    streaming passes): measured so that its distance to the roofline is on record."""
+    instruction where a product has sixteen columns or more, the pooling derivatives on single precision's streaming
+    kernels instantiated for double, batch norm as two streaming passes): measured so that its distance to the roofline is on record."""
     import torch
     rows = []
     w = workloads.conv_single()
@@ -592,6 +592,15 @@ def bench_double(capi, workloads, reps):
     t = _event_time(lambda: capi.pool_backward(xp, dyp, gp), reps, warm=2)
     nbytes = 8.0 * (2 * np.prod(shape) + np.prod(capi.pool_out_shape(gp)))
     rows.append(dict(op="max-pool backward, double", workload="112x112x64x8 (configs[2]a at a quarter of the batch)", call_us=t * 1e6,
+                     achieved=nbytes / t / 1e9, unit="GB/s", peak=PEAK_HBM / 1e9, frac=nbytes / t / PEAK_HBM, bound="hbm"))
+    del xp, dyp
+    shape = (56, 56, 256, 8)
+    gp = capi.pool_geom(shape, 2, 2, 0, "avg")
+    xp = torch.empty(tuple(reversed(shape)), device="cuda", dtype=torch.float64)
+    dyp = torch.randn(tuple(reversed(capi.pool_out_shape(gp))), device="cuda", dtype=torch.float64)
+    t = _event_time(lambda: capi.pool_backward(xp, dyp, gp), reps, warm=2)
+    nbytes = 8.0 * (np.prod(shape) + np.prod(capi.pool_out_shape(gp)))
+    rows.append(dict(op="avg-pool backward, double", workload="56x56x256x8 (configs[2]b at a quarter of the batch)", call_us=t * 1e6,
                      achieved=nbytes / t / 1e9, unit="GB/s", peak=PEAK_HBM / 1e9, frac=nbytes / t / PEAK_HBM, bound="hbm"))
     return rows
 

@@ -13,6 +13,8 @@ namespace mcn {
 
 bool pool_max_backward_stream_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, double* derInput,
                                      const double* x, const double* derOutput, int accumulate);  // pool_stream.hip
+bool pool_avg_backward_tiles_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, double* derInput,
+                                    const double* derOutput, int accumulate);  // pool.hip
 
 namespace {
 
@@ -976,6 +978,10 @@ int mcn_pool_backward_f64(mcn_stream_t stream, const mcn_pool_geom* g, double* d
   // most 2 x 2 outputs); same bits as the kernels below
   if (isMax && !tunable("pool64_no_tiles", 0) &&
       pool_max_backward_stream_launch(as_stream(stream), g, oh, ow, derInput, x, derOutput, accumulate))
+    return check_launch("mcn_pool_backward_f64");
+  // averages over windows that tile the plane exactly: single precision's streaming pass in memory order
+  if (!isMax && !tunable("pool64_no_tiles", 0) &&
+      pool_avg_backward_tiles_launch(as_stream(stream), g, oh, ow, derInput, derOutput, accumulate))
     return check_launch("mcn_pool_backward_f64");
   if (isMax && !tunable("pool64_no_tiles", 0)) {
     // strips of input columns through LDS, when a strip with its halo fits

@@ -115,22 +115,49 @@ __global__ __launch_bounds__(256) void pool_avg_backward_whole(float* __restrict
 // poolW; H a multiple of 4): every input element lies in exactly one whole window, dx = [dx +] dy[its window] * (1 /
 // (poolH * poolW)).  One thread per 16 bytes of dx, in memory order: a plain streaming kernel (reads dzdy once -- the
 // poolH * poolW threads that share a window hit L1 -- and writes dx once).
-__global__ __launch_bounds__(256) void pool_backward_avg_tiles(float* __restrict__ dx, const float* __restrict__ dy, unsigned total4,
+// E: float or double; a thread's 16 bytes are VE = 4 or 2 elements (H4 = H / VE cells per column).
+template <typename E>
+__global__ __launch_bounds__(256) void pool_backward_avg_tiles(E* __restrict__ dx, const E* __restrict__ dy, unsigned total4,
                                                                int H4, int W, int outH, int outW, FastDiv byH4, FastDiv byW,
                                                                FastDiv byPh, FastDiv byPw, int poolArea, int accumulate) {
+  constexpr int VE = 16 / sizeof(E);
+  typedef E vec __attribute__((ext_vector_type(VE)));
   const unsigned i = blockIdx.x * 256u + threadIdx.x;
   if (i >= total4) return;
   int col, q, plane, w;
   byH4.divmod((int)i, &col, &q);     // i = (plane * W + w) * H4 + q
   byW.divmod(col, &plane, &w);
-  const float scale = 1.0f / (float)poolArea;  // as avg_scale: correctly rounded IEEE division
-  const float* src = dy + ((size_t)plane * outW + byPw.div(w)) * outH;
-  float v[4];
+  const E scale = (E)1 / (E)poolArea;  // as avg_scale: correctly rounded IEEE division
+  const E* src = dy + ((size_t)plane * outW + byPw.div(w)) * outH;
+  E v[VE];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) v[r] = src[byPh.div(4 * q + r)] * scale;
-  float4 old = make_float4(0.f, 0.f, 0.f, 0.f);  // (0 + v, as the general kernels' sum starts: -0 becomes +0)
-  if (accumulate) old = ((const float4*)dx)[i];
-  stream_store4((float4*)dx + i, make_float4(old.x + v[0], old.y + v[1], old.z + v[2], old.w + v[3]));
+  for (int r = 0; r < VE; ++r) v[r] = src[byPh.div(VE * q + r)] * scale;
+  vec out = (vec)(E)0;  // (0 + v, as the general kernels' sum starts: -0 becomes +0)
+  if (accumulate) out = ((const vec*)dx)[i];
+#pragma unroll
+  for (int r = 0; r < VE; ++r) out[r] = out[r] + v[r];
+#if MCN_NT_STORE
+  __builtin_nontemporal_store(out, (vec*)dx + i);
+#else
+  ((vec*)dx)[i] = out;
+#endif
+}
+
+// Launches it when the windows tile the plane exactly and its columns are whole 16-byte cells; false otherwise.
+template <typename E>
+bool avg_tiles_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, E* derInput, const E* derOutput,
+                      int accumulate) {
+  constexpr int VE = 16 / sizeof(E);
+  const size_t total = (size_t)g->C * g->N * g->H * g->W;
+  if (g->method == MCN_POOL_MAX || g->poolH != g->strideY || g->poolW != g->strideX || g->padTop != 0 || g->padLeft != 0 ||
+      g->H != outH * g->poolH || g->W != outW * g->poolW || g->H % VE != 0 || !aligned16(derInput) ||
+      total / VE >= (1ull << 31) || tunable("pool_force_gather", 0))
+    return false;
+  KernelTimer timer("pool_backward_avg_tiles", s);
+  hipLaunchKernelGGL(pool_backward_avg_tiles<E>, dim3((unsigned)((total / VE + 255) / 256)), dim3(256), 0, s, derInput,
+                     derOutput, (unsigned)(total / VE), g->H / VE, g->W, outH, outW, FastDiv(g->H / VE), FastDiv(g->W),
+                     FastDiv(g->poolH), FastDiv(g->poolW), g->poolH * g->poolW, accumulate ? 1 : 0);
+  return true;
 }
 
 // KH, KW: upper bounds on the number of output rows / columns covering one input element
@@ -937,6 +964,13 @@ size_t tile_lds_bytes(const PoolP& p, bool isMax, bool useFlags, int TW) {
 }
 
 }  // namespace
+
+// the double-precision entry of the kernel above (f64.hip)
+bool pool_avg_backward_tiles_launch(hipStream_t s, const mcn_pool_geom* g, int outH, int outW, double* derInput,
+                                    const double* derOutput, int accumulate) {
+  return avg_tiles_launch<double>(s, g, outH, outW, derInput, derOutput, accumulate);
+}
+
 }  // namespace mcn
 
 using namespace mcn;
@@ -1033,14 +1067,7 @@ int mcn_pool_backward(mcn_stream_t stream, const mcn_pool_geom* g, float* derInp
   }
 
   // ---- average over windows that tile the plane exactly: one streaming pass in memory order
-  if (!isMax && p.poolH == p.sy && p.poolW == p.sx && p.pt == 0 && p.pl == 0 && p.H == p.outH * p.poolH && p.W == p.outW * p.poolW &&
-      vecIn && total / 4 < (1ull << 31) && !tunable("pool_force_gather", 0)) {
-    KernelTimer timer("pool_backward_avg_tiles", s);
-    hipLaunchKernelGGL(pool_backward_avg_tiles, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, s, derInput, derOutput,
-                       (unsigned)(total / 4), p.H / 4, p.W, p.outH, p.outW, FastDiv(p.H / 4), FastDiv(p.W), FastDiv(p.poolH),
-                       FastDiv(p.poolW), p.poolH * p.poolW, p.accumulate);
-    return check_launch("mcn_pool_backward");
-  }
+  if (avg_tiles_launch<float>(s, g, p.outH, p.outW, derInput, derOutput, accumulate)) return check_launch("mcn_pool_backward");
 
   // ---- ordered passes.  Widest tile whose LDS fits the budget and whose outputs fit 4 per thread.
   if (passes <= 16 && p.poolH <= 8 && p.poolW <= 8 && !tunable("pool_force_gather", 0)) {

@@ -201,6 +201,18 @@ def test_max_pool_backward_streaming_and_strips(capi, ob, geom, mode):
         capi.set_tunable("pool_force_gather", 0)
 
 
+@pytest.mark.parametrize("geom", [(56, 56, 5, 2, 2, 2, 0), (8, 12, 3, 2, (2, 3), (2, 3), 0), (12, 9, 2, 3, (6, 3), (6, 3), 0)])
+def test_average_pooling_over_exact_tiles(capi, ob, geom):
+    """Windows that tile the plane exactly, columns of whole 16-byte cells: the streaming pass in memory order; with it
+    switched off, the one-thread-per-element kernel.  Same bits either way."""
+    test_pooling_bit_exact(capi, ob, geom, "avg", "normal")
+    capi.set_tunable("pool64_no_tiles", 1)
+    try:
+        test_pooling_bit_exact(capi, ob, geom, "avg", "normal")
+    finally:
+        capi.set_tunable("pool64_no_tiles", 0)
+
+
 def test_mixed_precision_is_refused(capi):
     """All tensors of a call are single or all are double (bits/data.hpp:260-266)."""
     x = capi.to_device(np.zeros((4, 4, 1, 1)), D)
