@@ -54,6 +54,8 @@ __global__ __launch_bounds__(256) void conv64_forward(double* __restrict__ y, do
   y[idx] = r0;
 }
 
+// UNIT: strides of 1 (every tap position is an output pixel: no divisions in the loops)
+template <bool UNIT>
 __global__ __launch_bounds__(256) void conv64_backward_data(double* __restrict__ dx, const double* __restrict__ f,
                                                             const double* __restrict__ dy, ConvP p, size_t total) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -74,13 +76,13 @@ __global__ __launch_bounds__(256) void conv64_backward_data(double* __restrict__
     const double* fk = f + (size_t)p.FH * p.FW * ((size_t)p.FC * k + d);
     for (int j = 0; j < p.FW; ++j) {
       const int aw = w + p.pl - j * p.dx;
-      if (aw < 0 || aw % p.sx) continue;
-      const int ow = aw / p.sx;
+      if (aw < 0 || (!UNIT && aw % p.sx)) continue;
+      const int ow = UNIT ? aw : aw / p.sx;
       if (ow >= p.outW) continue;
       for (int i = 0; i < p.FH; ++i) {
         const int ah = h + p.pt - i * p.dy;
-        if (ah < 0 || ah % p.sy) continue;
-        const int oh = ah / p.sy;
+        if (ah < 0 || (!UNIT && ah % p.sy)) continue;
+        const int oh = UNIT ? ah : ah / p.sy;
         if (oh >= p.outH) continue;
         acc = fma(dyk[oh + p.outH * ow], fk[i + p.FH * j], acc);
       }
@@ -89,12 +91,91 @@ __global__ __launch_bounds__(256) void conv64_backward_data(double* __restrict__
   dx[idx] = acc;
 }
 
+// The same sums for a layer with at most four input channels (one filter group, strides and dilations of 1: a first
+// layer): a thread owns one input pixel and all its channels, so a dzdy value is loaded once for all of them and the
+// channels' sums are independent chains; the taps that land on an output pixel are a range worked out up front, so
+// the loops carry no tests.  Each sum runs over (filter, column tap, row tap) ascending, as above: same bits.
+// FHW > 0: a square window of that size, its loops unrolled -- the loads of a filter's whole window are in flight
+// together, where the loops with run-time bounds (FHW == 0) wait for one load per turn.  A tap off the output
+// contributes 0 * weight there (the reference adds nothing: the same unless that weight is not finite).
+template <int CC, int FHW>
+__global__ __launch_bounds__(256) void conv64_backward_data_few(double* __restrict__ dx, const double* __restrict__ f,
+                                                                const double* __restrict__ dy, ConvP p, size_t pixels) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= pixels) return;
+  const int FH = FHW > 0 ? FHW : p.FH, FW = FHW > 0 ? FHW : p.FW;
+  const int HW = p.H * p.W, P = p.outH * p.outW, T = FH * FW;
+  const size_t n = idx / HW;
+  const int q = (int)(idx - n * HW);
+  const int w = q / p.H, h = q - w * p.H;
+  const int iLo = max(0, h + p.pt - (p.outH - 1)), iHi = min(FH - 1, h + p.pt);
+  const int jLo = max(0, w + p.pl - (p.outW - 1)), jHi = min(FW - 1, w + p.pl);
+  double acc[CC];
+#pragma unroll
+  for (int c = 0; c < CC; ++c) acc[c] = 0.0;
+  const double* dy0 = dy + (size_t)P * p.K * n + (size_t)p.outH * (w + p.pl) + (h + p.pt);  // tap (0, 0) of filter 0
+  if (FHW > 0) {
+    // a tap that lands off the output reads the nearest tap that does not (a real value) and counts as zero: the loop
+    // body is straight-line code (with a test per tap the compiler branches around every load and multiply)
+    int rowOff[FHW > 0 ? FHW : 1], colOff[FHW > 0 ? FHW : 1];
+#pragma unroll
+    for (int i = 0; i < FHW; ++i) {
+      rowOff[i] = -min(max(i, iLo), iHi);
+      colOff[i] = -p.outH * min(max(i, jLo), jHi);
+    }
+#pragma unroll 2
+    for (int k = 0; k < p.K; ++k) {
+      const double* dyk = dy0 + (size_t)P * k;
+      const double* fk = f + (size_t)T * CC * k;
+      double v[FHW > 0 ? FHW : 1][FHW > 0 ? FHW : 1];
+#pragma unroll
+      for (int j = 0; j < FHW; ++j)
+#pragma unroll
+        for (int i = 0; i < FHW; ++i) {
+          const double got = dyk[colOff[j] + rowOff[i]];
+          v[j][i] = (j >= jLo && j <= jHi && i >= iLo && i <= iHi) ? got : 0.0;
+        }
+#pragma unroll
+      for (int j = 0; j < FHW; ++j)
+#pragma unroll
+        for (int i = 0; i < FHW; ++i)
+#pragma unroll
+          for (int c = 0; c < CC; ++c) acc[c] = fma(v[j][i], fk[i + FHW * j + T * c], acc[c]);
+    }
+  } else {
+    for (int k = 0; k < p.K; ++k) {
+      const double* dyk = dy0 + (size_t)P * k;
+      const double* fk = f + (size_t)T * CC * k;
+      for (int j = jLo; j <= jHi; ++j)
+        for (int i = iLo; i <= iHi; ++i) {
+          const double v = dyk[-(p.outH * j + i)];
+#pragma unroll
+          for (int c = 0; c < CC; ++c) acc[c] = fma(v, fk[i + FH * j + T * c], acc[c]);
+        }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < CC; ++c) dx[(size_t)q + (size_t)HW * (c + (size_t)CC * n)] = acc[c];
+}
+
 // sum of the four wavefronts' values, in a fixed order, on thread 0
 __device__ __forceinline__ double block_sum(double v, double* lds) {
   v = wave_sum(v);
   if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
   __syncthreads();
   const double s = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+  __syncthreads();
+  return s;
+}
+
+// sum of sixteen wavefronts' values, in a fixed order, on every thread
+__device__ __forceinline__ double block_sum16(double v, double* lds) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  double s = 0.0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += lds[i];
   __syncthreads();
   return s;
 }
@@ -128,17 +209,37 @@ __global__ __launch_bounds__(256) void conv64_backward_filter(double* __restrict
   if (threadIdx.x == 0) df[blockIdx.x] = s;
 }
 
-// one workgroup per filter: db[k] = sum over images and pixels of dy
-__global__ __launch_bounds__(256) void conv64_backward_bias(double* __restrict__ db, const double* __restrict__ dy, int P,
-                                                            int K, int N) {
-  __shared__ double lds[4];
+// one workgroup of sixteen wavefronts per filter: db[k] = sum over images and pixels of dy.  A thread walks the
+// filter's N * P values 1024 apart -- (image, pixel) advanced by carries -- four at a time, so four loads are in
+// flight per thread: with few filters the launch is a few workgroups, each of which has to keep its CU's memory path
+// busy alone.
+__global__ __launch_bounds__(1024) void conv64_backward_bias(double* __restrict__ db, const double* __restrict__ dy, int P,
+                                                             int K, int N) {
+  __shared__ double lds[16];
   const int k = blockIdx.x;
-  double acc = 0.0;
-  for (int n = 0; n < N; ++n) {
-    const double* src = dy + (size_t)P * (k + (size_t)K * n);
-    for (int i = threadIdx.x; i < P; i += 256) acc += src[i];
+  if (P <= 0 || N <= 0) {  // (an empty output: the sum of nothing)
+    if (threadIdx.x == 0) db[k] = 0.0;
+    return;
   }
-  const double s = block_sum(acc, lds);
+  const int stepN = 1024 / P, stepI = 1024 - stepN * P;  // 1024 values on: stepN images and stepI pixels
+  int n = (int)threadIdx.x / P, i = (int)threadIdx.x - n * P;
+  double a[4] = {0.0, 0.0, 0.0, 0.0};
+  while (n < N) {
+    double v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      v[u] = n < N ? dy[(size_t)P * (k + (size_t)K * n) + i] : 0.0;
+      i += stepI;
+      n += stepN;
+      if (i >= P) {
+        i -= P;
+        ++n;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) a[u] += v[u];
+  }
+  const double s = block_sum16((a[0] + a[1]) + (a[2] + a[3]), lds);
   if (threadIdx.x == 0) db[k] = s;
 }
 
@@ -321,32 +422,41 @@ __global__ __launch_bounds__(256) void conv64_mfma(double* __restrict__ out, con
       }
 }
 
-// dF[e] = sum over the splits' partial banks, in split order
+// dF[e] = sum over the splits' partial banks, in a fixed order: a workgroup owns 16 consecutive elements; thread
+// (e, g) adds the splits g, g + 16, g + 32, ... (eight loads in flight), and the sixteen sums of an element are added
+// in order of g.  (One thread per element walking all the splits waits for one load at a time: 256 splits of a
+// 2400-element bank took 65 us that way.)
 __global__ __launch_bounds__(256) void conv64_sum_splits(double* __restrict__ df, const double* __restrict__ partials, size_t n,
                                                          int splits) {
-  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= n) return;
+  __shared__ double part[16][17];
+  const int le = threadIdx.x & 15, g = threadIdx.x >> 4;
+  const size_t e = (size_t)blockIdx.x * 16 + le;
   double s = 0.0;
-  for (int i = 0; i < splits; ++i) s += partials[(size_t)i * n + e];
-  df[e] = s;
+  if (e < n) {
+    int i = g;
+    for (; i + 112 < splits; i += 128) {
+      double v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = partials[(size_t)(i + 16 * u) * n + e];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; i < splits; i += 16) s += partials[(size_t)i * n + e];
+  }
+  part[g][le] = s;
+  __syncthreads();
+  if (g == 0 && e < n) {
+    double t = part[0][le];
+#pragma unroll
+    for (int k = 1; k < 16; ++k) t += part[k][le];
+    df[e] = t;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------------
 // batch normalisation (bits/nnbnorm.cu:46-164: compute_moment, compute_ders, compute_ders_and_moments,
 // batch_normalize_forward / _backward)
 // ---------------------------------------------------------------------------------------------------------
-
-// sum of sixteen wavefronts' values, in a fixed order, on every thread
-__device__ __forceinline__ double block_sum16(double v, double* lds) {
-  v = wave_sum(v);
-  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
-  __syncthreads();
-  double s = 0.0;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) s += lds[i];
-  __syncthreads();
-  return s;
-}
 
 // One workgroup of sixteen wavefronts per channel (a read-only stream: the more wavefronts a CU holds, the more loads
 // are in flight).  DERS == false: sums of x and x*x, turned into (mean, sigma) in moments[c], moments[C + c].
@@ -800,10 +910,37 @@ int mcn_conv_backward_data_f64(mcn_stream_t stream, const mcn_conv_geom* g, doub
     return check_launch("mcn_conv_backward_data_f64");
   }
   unsigned blocks;
+  if (p.groups == 1 && p.C <= 4 && p.sy == 1 && p.sx == 1 && p.dy == 1 && p.dx == 1 && !tunable("conv64_no_mfma", 0)) {
+    const size_t pixels = total / p.C;
+    if ((rc = blocks_for(pixels, "mcn_conv_backward_data_f64", &blocks))) return rc;
+    KernelTimer timer("conv64_backward_data_few", as_stream(stream));
+    hipStream_t st = as_stream(stream);
+    const int sq = p.FH == p.FW && (p.FH == 3 || p.FH == 5 || p.FH == 7) ? p.FH : 0;
+#define MCN_FEW64(CCF, FHF) \
+  hipLaunchKernelGGL((conv64_backward_data_few<CCF, FHF>), dim3(blocks), dim3(256), 0, st, derInput, filters, derOutput, p, pixels)
+#define MCN_FEW64_C(FHF)            \
+  do {                              \
+    if (p.C == 1) MCN_FEW64(1, FHF); \
+    else if (p.C == 2) MCN_FEW64(2, FHF); \
+    else if (p.C == 3) MCN_FEW64(3, FHF); \
+    else MCN_FEW64(4, FHF);          \
+  } while (0)
+    if (sq == 3) MCN_FEW64_C(3);
+    else if (sq == 5) MCN_FEW64_C(5);
+    else if (sq == 7) MCN_FEW64_C(7);
+    else MCN_FEW64_C(0);
+#undef MCN_FEW64_C
+#undef MCN_FEW64
+    return check_launch("mcn_conv_backward_data_f64");
+  }
   if ((rc = blocks_for(total, "mcn_conv_backward_data_f64", &blocks))) return rc;
   KernelTimer timer("conv64_backward_data", as_stream(stream));
-  hipLaunchKernelGGL(conv64_backward_data, dim3(blocks), dim3(256), 0, as_stream(stream), derInput, filters, derOutput, p,
-                     total);
+  if (p.sy == 1 && p.sx == 1)
+    hipLaunchKernelGGL(conv64_backward_data<true>, dim3(blocks), dim3(256), 0, as_stream(stream), derInput, filters, derOutput,
+                       p, total);
+  else
+    hipLaunchKernelGGL(conv64_backward_data<false>, dim3(blocks), dim3(256), 0, as_stream(stream), derInput, filters, derOutput,
+                       p, total);
   return check_launch("mcn_conv_backward_data_f64");
 }
 
@@ -844,7 +981,7 @@ int mcn_conv_backward_filter_f64(mcn_stream_t stream, const mcn_conv_geom* g, do
     if (splits > 1) {
       if (!rc) {
         KernelTimer timer("conv64_sum_splits", st);
-        hipLaunchKernelGGL(conv64_sum_splits, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, derFilters,
+        hipLaunchKernelGGL(conv64_sum_splits, dim3((unsigned)((total + 15) / 16)), dim3(256), 0, st, derFilters,
                            (const double*)partials, total, (int)splits);
         rc = check_launch("mcn_conv_backward_filter_f64");
       }
@@ -866,7 +1003,7 @@ int mcn_conv_backward_bias_f64(mcn_stream_t stream, const mcn_conv_geom* g, doub
   if ((size_t)p.outH * p.outW * p.N != 0 && !derOutput)
     return fail(MCN_ILLEGAL_ARGUMENT, "mcn_conv_backward_bias_f64: null tensor");
   KernelTimer timer("conv64_backward_bias", as_stream(stream));
-  hipLaunchKernelGGL(conv64_backward_bias, dim3((unsigned)p.K), dim3(256), 0, as_stream(stream), derBias, derOutput,
+  hipLaunchKernelGGL(conv64_backward_bias, dim3((unsigned)p.K), dim3(1024), 0, as_stream(stream), derBias, derOutput,
                      p.outH * p.outW, p.K, p.N);
   return check_launch("mcn_conv_backward_bias_f64");
 }

@@ -27,6 +27,10 @@ CONV_CASES = [
     ((14, 13, 16, 3), (3, 3, 16, 24), 1, 1, 1),              # sixteen and more columns in every product: the matrix instruction
     ((15, 12, 20, 2), (3, 2, 20, 70), (2, 1), (1, 0, 2, 1), (1, 2)),   # the same with stride, dilation, partial tiles
     ((9, 9, 64, 2), (1, 1, 64, 64), 1, 0, 1),                # 1x1
+    ((7, 9, 1, 2), (3, 2, 1, 5), 1, (2, 0, 1, 1), 1),        # one, two and four input channels, uneven padding: the
+    ((6, 5, 2, 3), (2, 3, 2, 4), 1, (1, 1, 2, 0), 1),        # pixel-per-thread input gradient of first layers
+    ((10, 6, 4, 2), (5, 3, 4, 6), 1, (0, 4, 2, 1), 1),
+    ((16, 15, 3, 2), (7, 7, 3, 8), 1, 3, 1), ((9, 11, 4, 2), (3, 3, 4, 5), 1, (1, 2, 0, 1), 1),   # square windows: unrolled
 ]
 
 POOL_GEOMS = [
