@@ -92,57 +92,6 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   const int nWg = (int)gridDim.x / w.slices;
   const int cbBase = slice * w.chanBlocks;                         // first channel block of the slice
 
-  // ---- once per workgroup: the bank, re-laid by channel block
-  {
-    const int perBlock = p.R * (ROW / 4);  // 16-byte vectors per channel block
-    const int n4 = perBlock * w.chanBlocks;
-    // (four vectors in flight per thread: one at a time, every round trip to L2 would be paid in full; the empty
-    // asm keeps the compiler from sinking each load into the branch that guards its store)
-    auto fetch = [&](int i) -> v4f {
-      i = min(i, n4 - 1);
-      const int cbk = i / perBlock;  // (one-time code: a plain division)
-      const int rem = i - cbk * perBlock;
-      int r, c4;
-      w.byRow.divmod(rem, &r, &c4);
-      return *(const v4f*)(wt + (size_t)r * p.coutPad + (cbBase + cbk) * ROW + c4 * 4);
-    };
-    int i0 = tid;
-    // As many vectors in flight per thread as the bank has for it, up to twelve (a 147 KB bank is nine per thread at
-    // 1024 threads: one round trip to L2 instead of three, 80.1 -> 78.3 us on 3x3x64x64 over 56x56x64x32); a pass never
-    // asks for more than four vectors beyond the bank's end (those re-read its last vector, all threads the same one,
-    // which costs more than it looks: a pass of twelve over a bank of eight per thread lost 1-1.5 us)
-    for (; w.deepCopy && i0 + 8 * THREADS < n4; i0 += 12 * THREADS) {
-      v4f v[12];
-#pragma unroll
-      for (int k = 0; k < 12; ++k) v[k] = fetch(i0 + k * THREADS);
-      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
-                   "+v"(v[9]), "+v"(v[10]), "+v"(v[11]));
-#pragma unroll
-      for (int k = 0; k < 12; ++k)
-        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
-    }
-    for (; w.deepCopy && i0 + 4 * THREADS < n4; i0 += 8 * THREADS) {
-      v4f v[8];
-#pragma unroll
-      for (int k = 0; k < 8; ++k) v[k] = fetch(i0 + k * THREADS);
-      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
-#pragma unroll
-      for (int k = 0; k < 8; ++k)
-        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
-    }
-    for (; i0 < n4; i0 += 4 * THREADS) {
-      v4f v[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) v[k] = fetch(i0 + k * THREADS);
-      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
-#pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
-    }
-    if (STATS) statsL[tid] = statsL[tid + THREADS] = 0.f;  // ([THREADS / 64][2 rows][32][2]: wavefronts without units leave zeros)
-  }
-  __syncthreads();
-
   // ---- units of this wavefront.  The channel blocks of one pixel block go to neighbouring wavefronts of one
   // workgroup, which reach them at about the same time.  Pixel blocks are dealt slot-major (slot = wavefront /
   // channel blocks), so that consecutive pixel blocks sit on different CUs and every SIMD of the chip gets the
@@ -156,53 +105,6 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   // fetches 30 MB per launch through the fabric instead of 128 MB.  Without taps nothing is shared and spreading
   // neighbours over the XCDs measured 5% faster.)
   int unit = ((wave / sib) * nWg + wg) * sib + (wave % sib);
-  if (wave >= slots * sib) return;
-  // (STATS: sib = chanBlocks, so a wavefront's channel block is wave % sib for all its units)
-  float s1[STATS ? 16 : 1], s2[STATS ? 16 : 1];
-  auto write_stats = [&]() {
-    if (!STATS) return;
-    // the 32 lanes of a half-wave hold the same 16 channels for 32 different pixels.  Rows of 16 lanes are added up
-    // inside the vector unit (four shifted adds: lane 15 of a row ends with the row's sum), the two rows of a half meet
-    // in LDS.
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      s1[r] = row_sum16(s1[r]);
-      s2[r] = row_sum16(s2[r]);
-    }
-    if ((lane & 15) == 15) {
-      const int row = l32 >> 4;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int c = 4 * kh + 8 * (r / 4) + r % 4;  // channel inside the block
-        statsL[((wave * 2 + row) * 32 + c) * 2] = s1[r];
-        statsL[((wave * 2 + row) * 32 + c) * 2 + 1] = s2[r];
-      }
-    }
-    __syncthreads();  // (wavefronts that had no units have left already: the barrier counts the others)
-    // wavefront b < sib adds up channel block b: slots in ascending order, lane = channel, in double
-    if (wave < sib && lane < 32) {
-      double t1 = 0.0, t2 = 0.0;
-      for (int j = 0; j < slots; ++j)
-        for (int row = 0; row < 2; ++row) {
-          t1 += (double)statsL[(((j * sib + wave) * 2 + row) * 32 + lane) * 2];
-          t2 += (double)statsL[(((j * sib + wave) * 2 + row) * 32 + lane) * 2 + 1];
-        }
-      const int c = wave * 32 + lane;
-      if (c < p.Cout) {
-        double* o = p.stats + ((size_t)c * p.statGroups + wg) * 2;
-        o[0] = t1;
-        o[1] = t2;
-      }
-    }
-  };
-  if (STATS) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) s1[r] = s2[r] = 0.f;
-  }
-  // (STATS: wavefront b < sib writes the workgroup's partial of channel block b, so it stays to the end even without
-  // units; the host admits only launches in which every workgroup has units for its first wavefronts)
-  if (unit >= w.nUnits) return;
-
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, (int)w.inBytes, 0x00020000);
   const int planeBytes = IHW * 4;
 
@@ -294,15 +196,121 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_) asm volatile("" : "+v"(acc[a_])::"memory");                 \
   }
 
-  setup_next(unit);
-  voff = voffN;
-  ihB = ihBN;
-  iwB = iwBN;
-  setup_next(unit + unitStep);
-  voTap = tap_offset(dhL, dwL);
-  WS_LOAD_NEXT(b0);
-  WS_LOAD_NEXT(b1);
-  WS_LOAD_NEXT(b2);
+  // The stream's first three groups go out before the bank is copied: they land while the copy runs, instead of the
+  // whole chip asking for its first pixels at once after it (the loads return in order, so the copy's own waits cover
+  // them; block step 0.711 -> 0.700 ms.  Only the first group ahead of the copy and the other two behind it, so that
+  // the bank does not queue behind 24 loads: 0.708 -> 0.702).  Wavefronts without units issue nothing and leave after
+  // the barrier.
+  const bool mine = wave < slots * sib && unit < w.nUnits;
+  if (mine) {
+    setup_next(unit);
+    voff = voffN;
+    ihB = ihBN;
+    iwB = iwBN;
+    setup_next(unit + unitStep);
+    voTap = tap_offset(dhL, dwL);
+    WS_LOAD_NEXT(b0);
+    WS_LOAD_NEXT(b1);
+    WS_LOAD_NEXT(b2);
+  }
+
+  // ---- once per workgroup: the bank, re-laid by channel block
+  {
+    const int perBlock = p.R * (ROW / 4);  // 16-byte vectors per channel block
+    const int n4 = perBlock * w.chanBlocks;
+    // (four vectors in flight per thread: one at a time, every round trip to L2 would be paid in full; the empty
+    // asm keeps the compiler from sinking each load into the branch that guards its store)
+    auto fetch = [&](int i) -> v4f {
+      i = min(i, n4 - 1);
+      const int cbk = i / perBlock;  // (one-time code: a plain division)
+      const int rem = i - cbk * perBlock;
+      int r, c4;
+      w.byRow.divmod(rem, &r, &c4);
+      return *(const v4f*)(wt + (size_t)r * p.coutPad + (cbBase + cbk) * ROW + c4 * 4);
+    };
+    int i0 = tid;
+    // As many vectors in flight per thread as the bank has for it, up to twelve (a 147 KB bank is nine per thread at
+    // 1024 threads: one round trip to L2 instead of three, 80.1 -> 78.3 us on 3x3x64x64 over 56x56x64x32); a pass never
+    // asks for more than four vectors beyond the bank's end (those re-read its last vector, all threads the same one,
+    // which costs more than it looks: a pass of twelve over a bank of eight per thread lost 1-1.5 us)
+    for (; w.deepCopy && i0 + 8 * THREADS < n4; i0 += 12 * THREADS) {
+      v4f v[12];
+#pragma unroll
+      for (int k = 0; k < 12; ++k) v[k] = fetch(i0 + k * THREADS);
+      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
+                   "+v"(v[9]), "+v"(v[10]), "+v"(v[11]));
+#pragma unroll
+      for (int k = 0; k < 12; ++k)
+        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
+    }
+    for (; w.deepCopy && i0 + 4 * THREADS < n4; i0 += 8 * THREADS) {
+      v4f v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = fetch(i0 + k * THREADS);
+      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
+    }
+    for (; i0 < n4; i0 += 4 * THREADS) {
+      v4f v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) v[k] = fetch(i0 + k * THREADS);
+      asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (i0 + k * THREADS < n4) ((v4f*)wtL)[i0 + k * THREADS] = v[k];
+    }
+    if (STATS) statsL[tid] = statsL[tid + THREADS] = 0.f;  // ([THREADS / 64][2 rows][32][2]: wavefronts without units leave zeros)
+  }
+  __syncthreads();
+
+  if (wave >= slots * sib) return;
+  // (STATS: sib = chanBlocks, so a wavefront's channel block is wave % sib for all its units)
+  float s1[STATS ? 16 : 1], s2[STATS ? 16 : 1];
+  auto write_stats = [&]() {
+    if (!STATS) return;
+    // the 32 lanes of a half-wave hold the same 16 channels for 32 different pixels.  Rows of 16 lanes are added up
+    // inside the vector unit (four shifted adds: lane 15 of a row ends with the row's sum), the two rows of a half meet
+    // in LDS.
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      s1[r] = row_sum16(s1[r]);
+      s2[r] = row_sum16(s2[r]);
+    }
+    if ((lane & 15) == 15) {
+      const int row = l32 >> 4;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c = 4 * kh + 8 * (r / 4) + r % 4;  // channel inside the block
+        statsL[((wave * 2 + row) * 32 + c) * 2] = s1[r];
+        statsL[((wave * 2 + row) * 32 + c) * 2 + 1] = s2[r];
+      }
+    }
+    __syncthreads();  // (wavefronts that had no units have left already: the barrier counts the others)
+    // wavefront b < sib adds up channel block b: slots in ascending order, lane = channel, in double
+    if (wave < sib && lane < 32) {
+      double t1 = 0.0, t2 = 0.0;
+      for (int j = 0; j < slots; ++j)
+        for (int row = 0; row < 2; ++row) {
+          t1 += (double)statsL[(((j * sib + wave) * 2 + row) * 32 + lane) * 2];
+          t2 += (double)statsL[(((j * sib + wave) * 2 + row) * 32 + lane) * 2 + 1];
+        }
+      const int c = wave * 32 + lane;
+      if (c < p.Cout) {
+        double* o = p.stats + ((size_t)c * p.statGroups + wg) * 2;
+        o[0] = t1;
+        o[1] = t2;
+      }
+    }
+  };
+  if (STATS) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s1[r] = s2[r] = 0.f;
+  }
+  // (STATS: wavefront b < sib writes the workgroup's partial of channel block b, so it stays to the end even without
+  // units; the host admits only launches in which every workgroup has units for its first wavefronts)
+  if (unit >= w.nUnits) return;
 
   const bufrsrc orsrc = make_bufrsrc(out, p.outBytes);
   const int plane = p.outPlane * 4;
