@@ -4,7 +4,7 @@
 // The tiled kernel of conv_mfma.hip stages both operands through LDS with a barrier per 16 reduction rows; with
 // short reductions (R = 64 ... 576) and 64-channel tiles its workgroups spend most of their time waiting for the
 // one step of loads they have in flight.  Here
-//   * a persistent workgroup copies the bank into LDS once (up to 150 KB; one or two workgroups per CU), laid out
+//   * a persistent workgroup copies the bank into LDS once (up to 150 KB; one workgroup per CU), laid out
 //     [channel block][R][32 WA] so that every weight-fragment read is "lane base + immediate";
 //   * each wavefront then works alone, with no barriers: it takes units of 32 pixels x (32 WA) output channels;
 //     the pixel operand of v_mfma_f32_32x32x2_f32 is exactly "lane = pixel (l32), half = reduction row (kh)", so it
@@ -424,29 +424,19 @@ int launch(hipStream_t s, const char* who, int blocks, size_t lds, float* out, c
   return check_launch(who);
 }
 
-// Wavefronts per CU: 16 (4 per SIMD, 128 registers each) for the narrow units; 8 for WA = 4, whose 64 accumulator
-// registers plus operands need more than 128.
+// One workgroup per CU: sixteen wavefronts (4 per SIMD, 128 registers each) for the narrow units; eight for WA = 4,
+// whose 64 accumulator registers plus operands need more than 128.  (Banks of up to 78 KB used to get two workgroups of
+// eight wavefronts per CU; one of sixteen copies the bank once per CU instead of twice and measured 1.5-2 us faster per
+// launch on the 1x1 layers of a 56x56x256x32 bottleneck, 42-48 us each.)
 template <int WA, bool TAPS>
-int dispatch(hipStream_t s, const char* who, int cus, bool twoFit, size_t lds, float* out, const float* in, const float* wt,
+int dispatch(hipStream_t s, const char* who, int cus, size_t lds, float* out, const float* in, const float* wt,
              const float* bias, const PixP& p, const WsP& w) {
-  if (p.addend) {
-    if constexpr (WA == 4) return launch<WA, TAPS, 512, false, true>(s, who, cus, lds, out, in, wt, bias, p, w);
-    else if (twoFit) return launch<WA, TAPS, 512, false, true>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
-    else return launch<WA, TAPS, 1024, false, true>(s, who, cus, lds, out, in, wt, bias, p, w);
+  constexpr int THREADS = WA == 4 ? 512 : 1024;
+  if (p.addend) return launch<WA, TAPS, THREADS, false, true>(s, who, cus, lds, out, in, wt, bias, p, w);
+  if constexpr (WA == 1) {
+    if (p.stats) return launch<1, TAPS, 1024, true>(s, who, cus, lds, out, in, wt, bias, p, w);
   }
-  if constexpr (WA == 4) {
-    return launch<WA, TAPS, 512>(s, who, cus, lds, out, in, wt, bias, p, w);
-  } else if constexpr (WA == 1) {
-    if (p.stats) {
-      if (twoFit) return launch<1, TAPS, 512, true>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
-      return launch<1, TAPS, 1024, true>(s, who, cus, lds, out, in, wt, bias, p, w);
-    }
-    if (twoFit) return launch<WA, TAPS, 512>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
-    return launch<WA, TAPS, 1024>(s, who, cus, lds, out, in, wt, bias, p, w);
-  } else {
-    if (twoFit) return launch<WA, TAPS, 512>(s, who, cus * 2, lds, out, in, wt, bias, p, w);
-    return launch<WA, TAPS, 1024>(s, who, cus, lds, out, in, wt, bias, p, w);
-  }
+  return launch<WA, TAPS, THREADS>(s, who, cus, lds, out, in, wt, bias, p, w);
 }
 
 }  // namespace
@@ -457,7 +447,7 @@ namespace {
 // product.  wantStats: only shapes that can also sum their output per channel (see the kernel).
 struct WsPlan {
   int WA, cus, statGroups;
-  bool taps, twoFit;
+  bool taps;
   size_t lds;
   WsP w;
 };
@@ -485,7 +475,6 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
   int cus = device_compute_units();
   if (cus <= 0) cus = 256;
   if (cus % slices != 0) return false;  // (every slice gets the same number of workgroups)
-  const bool twoFit = lds <= 78 * 1024;  // two workgroups per CU fit the 160 KB
   const long long simds = (long long)cus * 4;
   const long long pixelBlocks = ((long long)p.M + 31) / 32;
 
@@ -527,7 +516,6 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
   plan->WA = WA;
   plan->cus = cus;
   plan->taps = !(p.T == 1 && p.dhBase == 0 && p.dwBase == 0 && p.sy == 1 && p.sx == 1 && p.IH == p.OH && p.IW == p.OW);
-  plan->twoFit = twoFit;
   plan->lds = lds;
   plan->w = w;
   plan->statGroups = 0;
@@ -537,12 +525,12 @@ bool plan_ws(const PixP& p, bool wantStats, WsPlan* plan) {
     // channels' sums would stay zero
     if (p.Cout % 32 != 0 || p.outBytes == 0) return false;
     // every wavefront must stay on one channel block: the channel blocks sit side by side in a workgroup
-    const int wavesPerGroup = twoFit ? 8 : 16;
+    const int wavesPerGroup = 16;
     if (wavesPerGroup % w.chanBlocks != 0 || p.beta != 0.f || p.alpha != 1.f) return false;
-    const int nWg = twoFit ? cus * 2 : cus;
+    const int nWg = cus;
     // the first wavefronts of every workgroup (slot 0) must have a unit: they write the workgroup's partials
     if (units < (long long)nWg * w.chanBlocks) return false;
-    if (lds + (size_t)wavesPerGroup * 128 * sizeof(float) > 160 * 1024 / (twoFit ? 2 : 1)) return false;
+    if (lds + (size_t)wavesPerGroup * 128 * sizeof(float) > 160 * 1024) return false;
     plan->lds = lds + (size_t)wavesPerGroup * 128 * sizeof(float);
     plan->statGroups = nWg;
   }
@@ -578,16 +566,15 @@ int conv_ws_launch(hipStream_t s, const char* who, float* out, const float* in, 
     if (!fits) return fail(MCN_UNSUPPORTED, "%s: this product cannot add a masked second term in its epilogue", who);
   }
   const int WA = plan.WA, cus = plan.cus;
-  const bool twoFit = plan.twoFit;
   const size_t lds = plan.lds;
   const WsP& w = plan.w;
   int rc;
-  if (plan.taps) rc = WA == 4 ? dispatch<4, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
-                      : (WA == 2 ? dispatch<2, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
-                                 : dispatch<1, true>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w));
-  else rc = WA == 4 ? dispatch<4, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
-            : (WA == 2 ? dispatch<2, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w)
-                       : dispatch<1, false>(s, who, cus, twoFit, lds, out, in, wt, bias, p, w));
+  if (plan.taps) rc = WA == 4 ? dispatch<4, true>(s, who, cus, lds, out, in, wt, bias, p, w)
+                      : (WA == 2 ? dispatch<2, true>(s, who, cus, lds, out, in, wt, bias, p, w)
+                                 : dispatch<1, true>(s, who, cus, lds, out, in, wt, bias, p, w));
+  else rc = WA == 4 ? dispatch<4, false>(s, who, cus, lds, out, in, wt, bias, p, w)
+            : (WA == 2 ? dispatch<2, false>(s, who, cus, lds, out, in, wt, bias, p, w)
+                       : dispatch<1, false>(s, who, cus, lds, out, in, wt, bias, p, w));
   *handled = 1;
   return rc;
 }
