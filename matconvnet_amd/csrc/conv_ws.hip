@@ -340,11 +340,17 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     // ---- stores of the finished unit (the next unit's first three groups are already in flight)
     const int mo = pb * 32 + l32;
     const int cbOut = cbBase + cb;  // the channel block's place in the whole bank
-    if (p.outBytes != 0 && (cbOut + 1) * ROW <= p.Cout) {
+    // (STATS and ADD launches have a descriptor-covered output whose channel blocks are whole or padding only, by
+    // contract: they always take this branch -- a block of padding stores to the "outside" offset, i.e. nothing, and
+    // adds zeros to the sums -- so the test is known at compile time, the other branch is gone, and with it the copies
+    // of the thirty-two running sums that the compiler made where the two branches met, every unit)
+    const bool whole = (cbOut + 1) * ROW <= p.Cout;
+    if ((STATS || ADD) || (p.outBytes != 0 && whole)) {
       // whole channel blocks inside the tensor: straight-line stores through a buffer descriptor
       int n, q;
       p.byQ.divmod(mo < p.M ? mo : 0, &n, &q);
-      const unsigned vo = mo < p.M ? (unsigned)(n * p.outImg + out_pixel_offset(p, q) + 4 * kh * p.outPlane) * 4u : kOutside;
+      const unsigned vo =
+          mo < p.M && whole ? (unsigned)(n * p.outImg + out_pixel_offset(p, q) + 4 * kh * p.outPlane) * 4u : kOutside;
       if (ADD) {
         const bufrsrc arsrc = make_bufrsrc(p.addend, p.outBytes), brsrc = make_bufrsrc(p.addBits, p.outBytes >> 5);
 #pragma unroll
