@@ -22,6 +22,8 @@ region.  `value` is images/s over exactly K steps.  The same line carries
   double_rows   the untuned double-precision instantiation on reduced forms of the same configurations,
   hbm_ceiling   the best plain read / write / copy kernels of a small sweep, cold, timed in this run: every HBM-bound
                 row is also given as a fraction of that measured copy rate,
+  mfma_ceiling  the matrix pipe alone (a stream of dependent matrix instructions on every SIMD), timed in this run: every
+                matrix-bound row is also given as a fraction of it,
   cpu_baseline  the CPU restatement of the reference path (oracle/) timed on this machine's host cores: the block, and
                 one leg per configuration (`per_config`).
 One GPU only: nothing here shards.
@@ -438,6 +440,29 @@ def bench_hbm_ceiling(capi, reps):
     return out
 
 
+def bench_mfma_ceiling(capi, reps):
+    """The matrix pipe alone (mcn_mfma_yardstick: four wavefronts per SIMD, each a dependent chain of matrix instructions
+    and nothing else), timed in this run: what the chip reaches of its nominal peak at the clock it holds under such a
+    stream.  Every matrix-bound row is also given as a fraction of that."""
+    import ctypes as C
+    import torch
+    L = capi.lib()
+    st = capi.stream()
+    sink = torch.zeros(4, device="cuda")
+    out = {}
+    for name, is_double, peak, iters in (("fp32", 0, PEAK_MFMA_FP32, 2000), ("fp64", 1, 78.6e12, 1000)):
+        flop = C.c_double(0.0)
+
+        def call():
+            capi.check(L.mcn_mfma_yardstick(st, capi.ptr(sink), iters, is_double, C.byref(flop)))
+        for _ in range(3):
+            call()
+        t, _ = kernel_time(capi, "mfma_yardstick_kernel", call, reps)
+        out[name] = dict(tflops=flop.value / t / 1e12, frac_of_peak=flop.value / t / peak, us=t * 1e6,
+                         instruction="v_mfma_f64_16x16x4_f64" if is_double else "v_mfma_f32_32x32x2_f32")
+    return out
+
+
 def bench_forward(capi, reps):
     """Forward kernels on the graded shapes: convolution (the three layers of the block, configs[3], and configs[4]),
     batch normalisation (configs[1], moments from the batch) and pooling (configs[2]).  Convolutions: whole call, events
@@ -823,12 +848,17 @@ def main():
     bn_rows, bn_whole = bench_bnorm_bwd(capi, workloads, args.steps)
     pool_rows = bench_pool_bwd(capi, workloads, args.steps)
     ceiling = bench_hbm_ceiling(capi, max(8, args.steps // 2))
+    mfma_ceiling = bench_mfma_ceiling(capi, 5)
     forward_rows = bench_forward(capi, max(5, args.steps // 2))
     single_rows, single_whole = bench_conv_single(capi, workloads, args.steps)
     for row in bn_rows + pool_rows + forward_rows:
         if row["bound"] == "hbm":   # beside the fraction of the nominal 8 TB/s: of what a plain copy reaches here
             row["frac_of_measured_copy"] = row["achieved"] / ceiling["copy"]["gbs"]
     pool_rows[0]["frac_of_measured_copy_of_same_size"] = pool_rows[0]["achieved"] / ceiling["copy_231MB"]["gbs"]
+    for row in conv_rows + forward_rows:
+        if row["bound"] == "mfma":  # beside the fraction of the nominal 157.3 TFLOP/s: of what the matrix pipe reaches alone
+            row["frac_of_measured_mfma"] = row["achieved"] / mfma_ceiling["fp32"]["tflops"]
+    roof["frac_of_measured_mfma"] = roof["achieved"] / mfma_ceiling["fp32"]["tflops"]
     graded = conv_rows + bn_rows + pool_rows
     # the per-operator figures once more inside `roofline`, in short form (fraction of the nominal roof, achieved, mean
     # launch time): records that keep `roofline` whole and only the names of the other keys still carry them
@@ -871,6 +901,7 @@ def main():
     # ---- the graded per-operator figures last: the end of the line is what a truncating record keeps
     line.update({
         "hbm_ceiling": ceiling,
+        "mfma_ceiling": mfma_ceiling,
         "block_plain": block_plain,
         "block_two_streams": block_two_streams,
         "conv_bwd_tflops": conv_whole["tflops"], "conv_bwd_frac_of_mfma_peak": conv_whole["frac"], "conv_bwd_ms": conv_whole["ms"],

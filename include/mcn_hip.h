@@ -120,6 +120,14 @@ enum { MCN_YARDSTICK_NONTEMPORAL = 1, MCN_YARDSTICK_CHUNKED = 2 };
 MCN_API int mcn_hbm_yardstick(mcn_stream_t stream, void* dst, const void* src, size_t bytes, int mode, int width,
                               int inFlight, int blocks, int flags);
 
+/* Matrix-pipe yardstick (no counterpart in the reference): one workgroup of sixteen wavefronts per CU, every wavefront a
+   dependent chain of `iters` x 8 v_mfma_f32_32x32x2_f32 (isDouble: `iters` x 16 v_mfma_f64_16x16x4_f64) and nothing
+   else; *flop receives the floating-point operations of the launch.  Timed with
+   mcn_profile_begin("mfma_yardstick"): what it reaches is the measured ceiling the matrix-bound kernels are reported
+   against beside the nominal peak (the chip does not hold its nominal clock under such a stream).  sink: one float
+   of device memory, never written in practice. */
+MCN_API int mcn_mfma_yardstick(mcn_stream_t stream, void* sink, int iters, int isDouble, double* flop);
+
 /* ------------------------------------------------------------------------------------------------
  * convolution -- replaces ConvolutionForward/Backward<VLDT_GPU,T> (bits/nnconv.cu:71-157,163-317),
  * i.e. im2row_gpu + cublasSgemm per image, and the cuDNN variant (bits/nnconv_cudnn.cu:40-540).

@@ -57,6 +57,7 @@ PROTOTYPES = {
     "mcn_profile_begin": (_i, [C.c_char_p]),
     "mcn_profile_end": (_i, [C.POINTER(_i), C.POINTER(_d)]),
     "mcn_hbm_yardstick": (_i, [_vp, _vp, _vp, _sz, _i, _i, _i, _i, _i]),
+    "mcn_mfma_yardstick": (_i, [_vp, _vp, _i, _i, C.POINTER(_d)]),
     "mcn_conv_output_size": (_i, [C.POINTER(ConvGeom), C.POINTER(_i), C.POINTER(_i)]),
     "mcn_conv_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _i]),
     "mcn_conv_forward": (_i, [_vp, C.POINTER(ConvGeom), _vp, _f, _vp, _f, _vp, _vp, _vp, _sz]),

@@ -103,10 +103,53 @@ int launch_mode(hipStream_t s, int mode, int blocks, int unroll, bool nt, bool c
   }
 }
 
+// Matrix-pipe yardstick: every SIMD of the chip gets four wavefronts, each a dependent chain of matrix instructions on
+// its own accumulator (what a convolution's inner loop is once its operands are in registers), and nothing else.
+// What it reaches is the ceiling the matrix-bound kernels are reported against beside the nominal peak: the chip does
+// not hold its nominal clock under such a stream.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+
+template <bool F64>
+__global__ __launch_bounds__(1024) void mfma_yardstick_kernel(float* __restrict__ sink, int iters) {
+  const float a = (float)(threadIdx.x & 63) * 0.001f, b = 1.0f;
+  float total = 0.f;
+  if (F64) {
+    doublex4 acc = {0.0, 0.0, 0.0, 0.0};
+    for (int i = 0; i < iters; ++i)
+#pragma unroll
+      for (int u = 0; u < 16; ++u) acc = __builtin_amdgcn_mfma_f64_16x16x4f64((double)a, (double)b, acc, 0, 0, 0);
+    total = (float)((acc[0] + acc[1]) + (acc[2] + acc[3]));
+  } else {
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int i = 0; i < iters; ++i)
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) total += acc[r];
+  }
+  if (total == -12345.678f) *sink = total;  // (cannot happen: the chains must be computed all the same)
+}
+
 }  // namespace
 }  // namespace mcn
 
 using namespace mcn;
+
+extern "C" int mcn_mfma_yardstick(mcn_stream_t stream, void* sink, int iters, int isDouble, double* flop) {
+  if (!sink || iters < 1 || iters > (1 << 20)) return fail(MCN_ILLEGAL_ARGUMENT, "mcn_mfma_yardstick: null sink or iteration count out of range");
+  int cus = device_compute_units();
+  if (cus <= 0) cus = 256;
+  hipStream_t s = as_stream(stream);
+  KernelTimer timer("mfma_yardstick_kernel", s);
+  if (isDouble) hipLaunchKernelGGL(mfma_yardstick_kernel<true>, dim3((unsigned)cus), dim3(1024), 0, s, (float*)sink, iters);
+  else hipLaunchKernelGGL(mfma_yardstick_kernel<false>, dim3((unsigned)cus), dim3(1024), 0, s, (float*)sink, iters);
+  // wavefronts x instructions x FLOP per instruction (32x32x2: 4096; 16x16x4: 2048)
+  if (flop) *flop = (double)cus * 16.0 * (double)iters * (isDouble ? 16.0 * 2048.0 : 8.0 * 4096.0);
+  return check_launch("mcn_mfma_yardstick");
+}
 
 extern "C" int mcn_hbm_yardstick(mcn_stream_t stream, void* dst, const void* src, size_t bytes, int mode, int width,
                                  int inFlight, int blocks, int flags) {

@@ -138,3 +138,25 @@ def test_leaky_relu(capi, ob, vl, n):
     with pytest.raises(vl.VlError) as e:
         vl.vl_nnrelu(xd, "leek", 0.1)
     assert e.value.message == "Unknown option 'leek'."
+
+
+def test_yardsticks_run_and_report_their_work(capi):
+    """The measurement helpers of the bench line: the streaming copy moves what it says (the copy is checked), the
+    matrix-pipe stream reports its floating-point operations and rejects a senseless iteration count."""
+    import ctypes as C
+    import torch
+    L = capi.lib()
+    src = torch.arange(1 << 16, device="cuda", dtype=torch.float32)
+    dst = torch.zeros_like(src)
+    capi.check(L.mcn_hbm_yardstick(capi.stream(), capi.ptr(dst), capi.ptr(src), src.numel() * 4, 2, 16, 2, 0, 0))
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+    sink = torch.zeros(4, device="cuda")
+    flop = C.c_double(0.0)
+    cus = int(L.mcn_device_compute_units())
+    for is_double, per_wave in ((0, 8 * 4096.0), (1, 16 * 2048.0)):
+        capi.check(L.mcn_mfma_yardstick(capi.stream(), capi.ptr(sink), 3, is_double, C.byref(flop)))
+        torch.cuda.synchronize()
+        assert flop.value == cus * 16 * 3 * per_wave
+    assert float(sink.abs().sum()) == 0.0   # (the sink is never written)
+    assert L.mcn_mfma_yardstick(capi.stream(), capi.ptr(sink), 0, 0, C.byref(flop)) != 0
