@@ -267,9 +267,14 @@ struct Gemm64P {
   FastDiv byP, byOutH, byHW, byH, byFH, byT, bySy, bySx;
 };
 
-template <int KIND>
-__global__ __launch_bounds__(256) void conv64_mfma(double* __restrict__ out, const double* __restrict__ a,
-                                                   const double* __restrict__ b, const double* __restrict__ bias, Gemm64P p) {
+// FAST: strides and dilations of 1 and every tensor under 2^31 elements -- offsets are 32-bit sums of a part that
+// depends on m (or n) alone and a part that depends on k alone, the latter advanced by carries; every load is issued
+// (from offset 0 where its element does not exist) and what does not exist is zeroed afterwards, so the eight loads
+// of a stage are in flight together.  (The general form spends 2.4 times the matrix instructions' cycles on 64-bit
+// address arithmetic.)
+template <int KIND, bool FAST>
+__global__ __launch_bounds__(256, 2) void conv64_mfma(double* __restrict__ out, const double* __restrict__ a,
+                                                      const double* __restrict__ b, const double* __restrict__ bias, Gemm64P p) {
   constexpr int KS = 16, LDA = KS + 1, LDB = 64 + 2;
   __shared__ double As[64 * LDA];
   __shared__ double Bs[KS * LDB];
@@ -299,9 +304,103 @@ __global__ __launch_bounds__(256) void conv64_mfma(double* __restrict__ out, con
     p.byFH.divmod(t, &mW, &mH);  // (mW, mH) = the tap (j, i)
   }
   double ra[4], rb[4];
+  unsigned okMask = 0;  // FAST: bit u: ra[u] exists, bit 4 + u: rb[u] exists
+  // FAST: the parts of the offsets that m and n fix
+  int baseA = 0, baseB = 0;
+  if (FAST) {
+    if (KIND == 0) {
+      baseA = (mH - c.pt) + c.H * ((mW - c.pl) + c.W * c.C * mImg);
+      baseB = p.FV * min(n, p.Nn - 1);
+    } else if (KIND == 1) {
+      baseA = (mH + c.pt) + c.outH * ((mW + c.pl) + c.outW * c.K * mImg);
+      baseB = p.T * min(n, p.Nn - 1);
+    } else {
+      baseA = (mH - c.pt) + c.H * ((mW - c.pl) + c.W * mC);
+      baseB = p.P * min(n, p.Nn - 1);
+    }
+  }
   auto fetch = [&](int k0) {
     const int k = k0 + fk;
-    if (KIND == 0 || KIND == 1) {
+    if (FAST && (KIND == 0 || KIND == 1)) {
+      int d, t, j, i;
+      p.byT.divmod(k, &d, &t);
+      p.byFH.divmod(t, &j, &i);
+      // the parts that k fixes: KIND 0: x at (i, j, d) and the bank row k; KIND 1: dzdy at (-i, -j, d) and the bank
+      // at (t, d)
+      int offA = KIND == 0 ? i + c.H * (j + c.W * d) : p.P * d - c.outH * j - i;
+      int offB = KIND == 0 ? k : t + p.T * c.C * d;
+      const int rowStep = KIND == 0 ? c.H - c.FH : c.FH - c.outH;           // a column on, back to the first row
+      const int volStep = KIND == 0 ? p.HW - c.H * c.FW : p.P + c.outH * c.FW;  // a channel (filter) on, back to the first column
+      double la[4], lb[4];
+      bool okA[4], okB[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int h = KIND == 0 ? mH - c.pt + i : mH + c.pt - i, w = KIND == 0 ? mW - c.pl + j : mW + c.pl - j;
+        const bool inK = k + u < kEnd;
+        okA[u] = inK && m < p.M && (unsigned)h < (unsigned)(KIND == 0 ? c.H : c.outH) &&
+                 (unsigned)w < (unsigned)(KIND == 0 ? c.W : c.outW);
+        okB[u] = inK && n < p.Nn;
+        la[u] = a[okA[u] ? baseA + offA : 0];
+        lb[u] = b[okB[u] ? baseB + offB : 0];
+        offA += KIND == 0 ? 1 : -1;
+        offB += 1;
+        if (++i == c.FH) {
+          i = 0;
+          offA += rowStep;
+          if (++j == c.FW) {
+            j = 0;
+            offA += volStep;
+            if (KIND == 1) offB += p.T * c.C - p.T;
+          }
+        }
+      }
+      // (what does not exist is zeroed where the stage is written to LDS: a select here would wait for the loads
+      // before this stage's matrix instructions)
+      okMask = 0;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        ra[u] = la[u];
+        rb[u] = lb[u];
+        okMask |= (okA[u] ? 1u : 0u) << u | (okB[u] ? 16u : 0u) << u;
+      }
+    } else if (FAST) {
+      // k = output pixel of all images; x at (oh, ow, img) shifted by the tap, dzdy at pixel q of image img
+      int img, q, ow, oh;
+      p.byP.divmod(min(k, p.Kd - 1), &img, &q);
+      p.byOutH.divmod(q, &ow, &oh);
+      int offA = oh + c.H * ow + p.HW * c.C * img, offB = q + p.P * c.K * img;
+      double la[4], lb[4];
+      bool okA[4], okB[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int h = oh - c.pt + mH, w = ow - c.pl + mW;
+        const bool inK = k + u < kEnd;
+        okA[u] = inK && m < p.M && (unsigned)h < (unsigned)c.H && (unsigned)w < (unsigned)c.W;
+        okB[u] = inK && n < p.Nn;
+        la[u] = a[okA[u] ? baseA + offA : 0];
+        lb[u] = b[okB[u] ? baseB + offB : 0];
+        offA += 1;
+        offB += 1;
+        if (++oh == c.outH) {
+          oh = 0;
+          offA += c.H - c.outH;
+          if (++ow == c.outW) {
+            ow = 0;
+            offA += p.HW * c.C - c.H * c.outW;
+            offB += p.P * c.K - p.P;
+          }
+        }
+      }
+      // (what does not exist is zeroed where the stage is written to LDS: a select here would wait for the loads
+      // before this stage's matrix instructions)
+      okMask = 0;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        ra[u] = la[u];
+        rb[u] = lb[u];
+        okMask |= (okA[u] ? 1u : 0u) << u | (okB[u] ? 16u : 0u) << u;
+      }
+    } else if (KIND == 0 || KIND == 1) {
       // k = t + T * (channel or filter), t = i + FH j
       int d, t, j, i;
       p.byT.divmod(k, &d, &t);
@@ -374,8 +473,8 @@ __global__ __launch_bounds__(256) void conv64_mfma(double* __restrict__ out, con
     __syncthreads();  // (the stage before this one has been multiplied)
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      As[fm * LDA + fk + u] = ra[u];
-      Bs[(fk + u) * LDB + fm] = rb[u];
+      As[fm * LDA + fk + u] = !FAST || (okMask >> u & 1u) ? ra[u] : 0.0;
+      Bs[(fk + u) * LDB + fm] = !FAST || (okMask >> (4 + u) & 1u) ? rb[u] : 0.0;
     }
     __syncthreads();
     if (k0 + KS < kEnd) fetch(k0 + KS);
@@ -823,6 +922,13 @@ __global__ __launch_bounds__(256) void pool64_max_backward_tiled(double* __restr
 // The matrix-instruction form of a product (kind 0 forward, 1 backward-data, 2 backward-filter): one filter group,
 // every extent inside 31 bits, and at least sixteen columns of the product (fewer: the one-accumulator kernels above
 // multiply nothing in vain, a 64-wide tile would).
+// unit strides and dilations, every tensor under 2^31 elements: the matrix kernels' 32-bit offsets (FAST)
+bool gemm64_fast(const ConvP& c) {
+  const long long lim = 1ll << 31;
+  return c.sy == 1 && c.sx == 1 && c.dy == 1 && c.dx == 1 && (long long)c.H * c.W * c.C * c.N < lim &&
+         (long long)c.outH * c.outW * c.K * c.N < lim && (long long)c.FH * c.FW * c.FC * c.K < lim;
+}
+
 bool gemm64_plan(const ConvP& c, int kind, Gemm64P* out) {
   if (c.groups != 1 || tunable("conv64_no_mfma", 0)) return false;
   const long long P = (long long)c.outH * c.outW, HW = (long long)c.H * c.W, T = (long long)c.FH * c.FW, FV = T * c.C;
@@ -882,8 +988,9 @@ int mcn_conv_forward_f64(mcn_stream_t stream, const mcn_conv_geom* g, double* y,
     gp.outMult = outMult;
     gp.inMult = inMult;
     KernelTimer timer("conv64_mfma", as_stream(stream));
-    hipLaunchKernelGGL(conv64_mfma<0>, dim3((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64)), dim3(256), 0,
-                       as_stream(stream), y, x, filters, bias, gp);
+    const dim3 grid((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64));
+    if (gemm64_fast(p)) hipLaunchKernelGGL((conv64_mfma<0, true>), grid, dim3(256), 0, as_stream(stream), y, x, filters, bias, gp);
+    else hipLaunchKernelGGL((conv64_mfma<0, false>), grid, dim3(256), 0, as_stream(stream), y, x, filters, bias, gp);
     return check_launch("mcn_conv_forward_f64");
   }
   unsigned blocks;
@@ -905,8 +1012,11 @@ int mcn_conv_backward_data_f64(mcn_stream_t stream, const mcn_conv_geom* g, doub
   Gemm64P gp;
   if (gemm64_plan(p, 1, &gp)) {
     KernelTimer timer("conv64_mfma", as_stream(stream));
-    hipLaunchKernelGGL(conv64_mfma<1>, dim3((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64)), dim3(256), 0,
-                       as_stream(stream), derInput, derOutput, filters, nullptr, gp);
+    const dim3 grid((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64));
+    if (gemm64_fast(p))
+      hipLaunchKernelGGL((conv64_mfma<1, true>), grid, dim3(256), 0, as_stream(stream), derInput, derOutput, filters, nullptr, gp);
+    else
+      hipLaunchKernelGGL((conv64_mfma<1, false>), grid, dim3(256), 0, as_stream(stream), derInput, derOutput, filters, nullptr, gp);
     return check_launch("mcn_conv_backward_data_f64");
   }
   unsigned blocks;
@@ -974,8 +1084,10 @@ int mcn_conv_backward_filter_f64(mcn_stream_t stream, const mcn_conv_geom* g, do
     }
     {
       KernelTimer timer("conv64_mfma", st);
-      hipLaunchKernelGGL(conv64_mfma<2>, dim3((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64), (unsigned)splits),
-                         dim3(256), 0, st, splits > 1 ? (double*)partials : derFilters, x, derOutput, nullptr, gp);
+      const dim3 grid((unsigned)((gp.M + 63) / 64), (unsigned)((gp.Nn + 63) / 64), (unsigned)splits);
+      double* target = splits > 1 ? (double*)partials : derFilters;
+      if (gemm64_fast(p)) hipLaunchKernelGGL((conv64_mfma<2, true>), grid, dim3(256), 0, st, target, x, derOutput, nullptr, gp);
+      else hipLaunchKernelGGL((conv64_mfma<2, false>), grid, dim3(256), 0, st, target, x, derOutput, nullptr, gp);
     }
     rc = check_launch("mcn_conv_backward_filter_f64");
     if (splits > 1) {
