@@ -36,7 +36,7 @@ struct FewP {
 };
 
 template <int kTapGroup>
-__global__ __launch_bounds__(256) void conv_few_mfma(float* __restrict__ out, const float* __restrict__ in,
+__global__ __launch_bounds__(256, 2) void conv_few_mfma(float* __restrict__ out, const float* __restrict__ in,
                                                      const float* __restrict__ wt, const float* __restrict__ bias, PixP p,
                                                      FewP w) {
   extern __shared__ float lds[];
