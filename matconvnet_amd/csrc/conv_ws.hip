@@ -177,7 +177,7 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
 
   // multiplies the stream's oldest group (operands CUR, group G of the unit in hand) after putting one more
   // group in flight into FREE
-#define WS_STEP(G, CUR, FREE)                                                                                     \
+#define WS_STEP_C(G, CUR, FREE, ZEROC)                                                                            \
   {                                                                                                               \
     WS_LOAD_NEXT(FREE);                                                                                           \
     const float* aG_ = aG + (G) * (2 * kDepth * ROW);                                                             \
@@ -188,13 +188,15 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
         _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_) av_[d_][a_] = aG_[(2 * (h_ * HALF_ + d_)) * ROW + a_ * 32]; \
       _Pragma("unroll") for (int d_ = 0; d_ < HALF_; ++d_)                                                        \
         _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_)                                                         \
-          acc[a_] = __builtin_amdgcn_mfma_f32_32x32x2f32(av_[d_][a_], CUR[h_ * HALF_ + d_], acc[a_], 0, 0, 0);    \
+          acc[a_] = __builtin_amdgcn_mfma_f32_32x32x2f32(av_[d_][a_], CUR[h_ * HALF_ + d_],                     \
+                                                         (ZEROC) && h_ == 0 && d_ == 0 ? zero16 : acc[a_], 0, 0, 0); \
     }                                                                                                             \
     /* Pins the step's MFMAs before the next step's loads.  Left free, the compiler lifts those loads over the */ \
     /* last MFMA, which still reads a register of the buffer they fill; the load then gets a fresh register    */ \
     /* and the loop copies it back at its end, after waiting for every load in flight.                         */ \
     _Pragma("unroll") for (int a_ = 0; a_ < WA; ++a_) asm volatile("" : "+v"(acc[a_])::"memory");                 \
   }
+#define WS_STEP(G, CUR, FREE) WS_STEP_C(G, CUR, FREE, false)
 
   // The stream's first three groups go out before the bank is copied: they land while the copy runs, instead of the
   // whole chip asking for its first pixels at once after it (the loads return in order, so the copy's own waits cover
@@ -315,11 +317,10 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   const bufrsrc orsrc = make_bufrsrc(out, p.outBytes);
   const int plane = p.outPlane * 4;
 
-  floatx16 acc[WA];
+  floatx16 acc[WA];  // (written whole by a unit's first matrix instructions)
+  floatx16 zero16;
 #pragma unroll
-  for (int a = 0; a < WA; ++a)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
+  for (int r = 0; r < 16; ++r) zero16[r] = 0.f;
   int pb, cb;
   w.byCB.divmod(unit, &pb, &cb);  // unit = pixel block * chanBlocks + channel block
   const float* aLane = wtL + (size_t)cb * p.R * ROW + kh * ROW + l32;
@@ -328,14 +329,21 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
   // One flat loop over this wavefront's whole stream, four groups per turn (the host admits only reductions of
   // a multiple of 4 groups, so a unit ends at the end of a turn with the four buffers back in place).
   const int quadsPerUnit = w.groups >> 2;
-  int quadsLeft = quadsPerUnit;
   while (true) {
-    WS_STEP(0, b0, b3)
+    // a unit's first matrix instruction takes zero as its addend (an operand of the instruction: no sixteen moves per
+    // accumulator and unit to clear it); the unit's other turns of four groups follow in a loop of their own
+    WS_STEP_C(0, b0, b3, true)
     WS_STEP(1, b1, b0)
     WS_STEP(2, b2, b1)
     WS_STEP(3, b3, b2)
     aG += 4 * (2 * kDepth * ROW);
-    if (--quadsLeft != 0) continue;
+    for (int quadsLeft = quadsPerUnit - 1; quadsLeft != 0; --quadsLeft) {
+      WS_STEP(0, b0, b3)
+      WS_STEP(1, b1, b0)
+      WS_STEP(2, b2, b1)
+      WS_STEP(3, b3, b2)
+      aG += 4 * (2 * kDepth * ROW);
+    }
 
     // ---- stores of the finished unit (the next unit's first three groups are already in flight)
     const int mo = pb * 32 + l32;
@@ -392,17 +400,13 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     unit += unitStep;
     if (unit >= w.nUnits) break;
     setup_next(unit + unitStep);  // (the loader is already inside `unit`)
-#pragma unroll
-    for (int a = 0; a < WA; ++a)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
     w.byCB.divmod(unit, &pb, &cb);
     aLane = wtL + (size_t)cb * p.R * ROW + kh * ROW + l32;
     aG = aLane;
-    quadsLeft = quadsPerUnit;
   }
   write_stats();
 #undef WS_STEP
+#undef WS_STEP_C
 #undef WS_LOAD_NEXT
 }
 
