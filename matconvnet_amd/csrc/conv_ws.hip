@@ -125,6 +125,12 @@ __global__ __launch_bounds__(THREADS) void conv_ws_mfma(float* __restrict__ out,
     const bool mvalid = u < w.nUnits && m < p.M;
     int n, q, ow, oh;
     p.byQ.divmod(mvalid ? m : 0, &n, &q);
+    if (!TAPS) {
+      // (one tap at shift 0, unit strides, output plane = input plane: the pixel's place in its image is q itself)
+      ihBN = iwBN = 0;
+      voffN = mvalid ? (unsigned)(n * p.inImg + q + kh * IHW) * 4u : kOutside;
+      return;
+    }
     p.byOH.divmod(q, &ow, &oh);
     ihBN = mvalid ? oh * p.sy : -0x40000000;  // (an idle lane fails every "row inside the image" test)
     iwBN = ow * p.sx;
